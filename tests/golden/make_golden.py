@@ -1,0 +1,184 @@
+"""Writes tests/golden/*.npz by running the reference's own quantizer / autograd code on CPU.
+
+Run once, in the build container only (the reference checkout does not exist on GPU boxes):
+
+    python tests/golden/make_golden.py [/root/reference]
+
+Why an import and not only closed forms: the results recorded here depend on the exact
+sequence of per-op roundings of eager PyTorch (bf16-per-op mode differs from an ideal
+round-to-nearest E2M1 conversion in ~1 % of elements), on torch's CPU random stream for the
+stochastic-rounding quantizer, and on the wiring of the autograd function -- none of which a
+closed form fixes bit for bit.  The fixtures are data only: inputs, the uniform draws that the
+reference consumed, and its outputs.  bf16 tensors are stored as their uint16 bit patterns.
+"""
+from __future__ import annotations
+
+import os
+import sys
+from types import SimpleNamespace
+
+import numpy as np
+import torch
+
+REF = sys.argv[1] if len(sys.argv) > 1 else "/root/reference"
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.dont_write_bytecode = True
+sys.path.insert(0, os.path.join(REF, "src", "Metis"))
+
+from Metis import quant as rq  # noqa: E402
+from Metis import bitlinear as rb  # noqa: E402
+
+
+def bits(t: torch.Tensor) -> np.ndarray:
+    """bf16 -> uint16 patterns; fp32 stays fp32."""
+    if t.dtype == torch.bfloat16:
+        return t.contiguous().view(torch.int16).numpy().view(np.uint16).copy()
+    return t.contiguous().numpy().copy()
+
+
+def planted_input(seed: int, rows: int, cols: int) -> torch.Tensor:
+    """bf16 test tensor with outlier channels, exact ties, a zero block, tiny and huge blocks."""
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(rows, cols, generator=g)
+    x[:, 5] *= 20.0                                   # outlier channel
+    x[:, cols - 3] *= 20.0
+    x = x.bfloat16()
+    x[1, 0:16] = 0.0                                  # all-zero block
+    x[2, 16:32] = torch.tensor([6.0, 0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0,
+                                -0.25, -0.75, -1.25, -1.75, -2.5, -3.5, -5.0, -6.0]).bfloat16()  # scalar=1: every midpoint
+    x[3, 32:48] = (torch.randn(16, generator=g) * 1e-12).bfloat16()   # scalar dominated by 1e-9
+    x[4, 48:64] = (torch.randn(16, generator=g) * 1e-4).bfloat16()    # small block -> subnormal E4M3 scale
+    x[5, 0:16] = (torch.randn(16, generator=g) * 3e4).bfloat16()      # huge block sets the tensor scale
+    x[6, 64:80] = torch.tensor([3.0, 0.125, 0.375, 0.625, 0.875, 1.25, 1.75, 2.5,
+                                -3.0, -0.125, -0.375, -0.625, -0.875, -1.25, -1.75, -2.5]).bfloat16()  # scalar=.5 midpoints
+    x[7, 80:96] = -0.0
+    return x
+
+
+def golden_rne(out: dict):
+    x = planted_input(11, 64, 256)
+    out["rne_x"] = bits(x)
+    for tag, xin in (("p32", x.float()), ("pb16", x)):
+        q = rq.Cast2NVFp4e2m1BlockNOSR
+        out[f"rne_qdq_{tag}"] = bits(q.quantize_dequantize(xin.clone()))
+        s = q.get_scalar(xin.clone())
+        out[f"rne_scalar_{tag}"] = bits(s)
+        xq = q.quant(xin.clone(), s)
+        out[f"rne_quant_{tag}"] = bits(xq)
+        s_arg = s.clone()
+        out[f"rne_rquant_{tag}"] = bits(q.rquant(xq, s_arg))
+        out[f"rne_scalar_after_rquant_{tag}"] = bits(s_arg)      # reference mutates its argument
+    # a 3-D activation-shaped case (batch, tokens, hidden)
+    g = torch.Generator().manual_seed(12)
+    x3 = (torch.randn(2, 24, 128, generator=g) * 0.7).bfloat16()
+    out["rne3d_x"] = bits(x3)
+    out["rne3d_qdq_p32"] = bits(rq.Cast2NVFp4e2m1BlockNOSR.quantize_dequantize(x3.float()))
+    out["rne3d_qdq_pb16"] = bits(rq.Cast2NVFp4e2m1BlockNOSR.quantize_dequantize(x3))
+    # weight-like magnitudes (N(0, 0.02^2)): the 1e-9 term perturbs every scalar
+    g = torch.Generator().manual_seed(13)
+    w = (torch.randn(48, 192, generator=g) * 0.02).bfloat16()
+    out["rnew_x"] = bits(w)
+    out["rnew_qdq_p32"] = bits(rq.Cast2NVFp4e2m1BlockNOSR.quantize_dequantize(w.float()))
+    out["rnew_qdq_pb16"] = bits(rq.Cast2NVFp4e2m1BlockNOSR.quantize_dequantize(w))
+
+
+def golden_sr(out: dict):
+    x = planted_input(21, 32, 128)
+    out["sr_x"] = bits(x)
+    for tag, xin in (("p32", x.float()), ("pb16", x)):
+        q = rq.Cast2NVFp4e2m1Block
+        s = q.get_scalar(xin.clone())
+        blocks_shape = (xin.shape[0], 1, xin.shape[1] // 16, 16)
+        torch.manual_seed(2004)
+        u = torch.rand(blocks_shape, dtype=xin.dtype)            # the draw rand_like will make
+        torch.manual_seed(2004)
+        xq = q.quant(xin.clone(), s)
+        out[f"sr_noise_{tag}"] = bits(u.reshape(xin.shape))
+        out[f"sr_quant_{tag}"] = bits(xq)
+        out[f"sr_rquant_{tag}"] = bits(q.rquant(xq, s.clone()))
+
+
+def _configure(fwd_in, fwd_w, bwd_g, dtype):
+    F = rb.LinearLowbitFunction
+    F.q_forward_input = rq.quant_func[fwd_in]
+    F.q_forward_weight = rq.quant_func[fwd_w]
+    F.q_backward_input = rq.quant_func[bwd_g]
+    F.q_backward_weight = rq.quant_func[bwd_g]
+    F.q_backward_outputgrad = rq.quant_func[bwd_g]
+    F.enable_activation_svd = False
+    F.enable_backward_svd = False
+    F.enable_nv_recipe = False
+    F.compute_dtype = dtype
+    F.metis_mode = "mean"
+
+
+def golden_linear(out: dict):
+    """LinearLowbit forward + backward (direct FP4 path) and a hand-assembled BitLinear forward."""
+    g = torch.Generator().manual_seed(31)
+    B, T, K, N, r = 2, 16, 64, 48, 8
+    x = torch.randn(B, T, K, generator=g).bfloat16().float()
+    w = (torch.randn(N, K, generator=g) * 0.05).bfloat16().float()
+    b = (torch.randn(N, generator=g) * 0.1).bfloat16().float()
+    dy = (torch.randn(B, T, N, generator=g) * 1e-3).bfloat16().float()
+    args = SimpleNamespace(device="cpu", cache_quantized_weight=False, forward_svd_rank=r)
+    _configure("nvfp4e2m1bnosr", "nvfp4e2m1bnosr", "nvfp4e2m1b", torch.float32)
+
+    layer = rb.LinearLowbit(K, N, bias=True, args=args)
+    with torch.no_grad():
+        layer.weight.copy_(w)
+        layer.bias.copy_(b)
+    xr = x.clone().requires_grad_(True)
+    y = layer(xr)
+    torch.manual_seed(2005)
+    u = torch.rand((B * T, 1, N // 16, 16), dtype=torch.float32)
+    torch.manual_seed(2005)
+    y.backward(dy)
+    out["lin_x"], out["lin_w"], out["lin_b"], out["lin_dy"] = bits(x), bits(w), bits(b), bits(dy)
+    out["lin_y"] = bits(y.detach())
+    out["lin_noise_dy"] = bits(u.reshape(B, T, N))
+    out["lin_gx"] = bits(xr.grad)
+    out["lin_gw"] = bits(layer.weight.grad)
+    out["lin_gb"] = bits(layer.bias.grad)
+
+    # BitLinear assembled by hand (split() needs a GPU): low-rank branch + residual branch
+    bl = rb.BitLinear.__new__(rb.BitLinear)
+    torch.nn.Module.__init__(bl)
+    bl.args = args
+    bl.is_svd_quant = True
+    bl.mean_cache = {}
+    bl.activation_group = None
+    bl._merged_rollout_weight_cache = None
+    bl.layer_name = "golden.layer"
+    bl.vlinear = rb.LinearLowbit(K, r, bias=False, args=args)
+    bl.ulinear = torch.nn.Linear(r, N, bias=False)
+    bl.warmup_linear = rb.LinearLowbit(K, N, bias=True, args=args)
+    U, S, Vh = torch.linalg.svd(w, full_matrices=False)
+    with torch.no_grad():
+        bl.vlinear.weight.copy_(Vh[:r])
+        bl.ulinear.weight.copy_(U[:, :r])
+        bl.s = torch.nn.Parameter(S[:r].clone())
+        bl.warmup_linear.weight.copy_(w - (U[:, :r] * S[:r]) @ Vh[:r])
+        bl.warmup_linear.bias.copy_(b)
+    _configure("nvfp4e2m1bnosr", "nvfp4e2m1bnosr", "nvfp4e2m1b", torch.float32)
+    with torch.no_grad():
+        yb = bl(x)
+    out["bl_v"] = bits(bl.vlinear.weight.detach())
+    out["bl_u"] = bits(bl.ulinear.weight.detach())
+    out["bl_s"] = bits(bl.s.detach())
+    out["bl_res"] = bits(bl.warmup_linear.weight.detach())
+    out["bl_y"] = bits(yb)
+
+
+def main():
+    torch.set_num_threads(1)
+    out: dict = {}
+    golden_rne(out)
+    golden_sr(out)
+    golden_linear(out)
+    path = os.path.join(HERE, "metis_reference_golden.npz")
+    np.savez_compressed(path, **out)
+    print(f"wrote {path}: {len(out)} arrays, {os.path.getsize(path)} bytes; torch {torch.__version__}")
+
+
+if __name__ == "__main__":
+    main()

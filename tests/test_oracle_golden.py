@@ -1,0 +1,95 @@
+"""The oracle (torch restatement and C restatement) against vectors the reference itself produced.
+
+Fixtures: tests/golden/metis_reference_golden.npz, written by tests/golden/make_golden.py.
+Everything here is bit-exact (atol = rtol = 0).
+"""
+import pytest
+import torch
+
+from oracle import c_oracle as C
+from oracle import metis_oracle as O
+from helpers import same_bits, t
+
+MODES = [("p32", 0), ("pb16", 1)]
+
+
+def _inp(x_bf16, tag):
+    return x_bf16.float() if tag == "p32" else x_bf16
+
+
+@pytest.mark.parametrize("tag,mode", MODES)
+@pytest.mark.parametrize("case", ["rne", "rne3d", "rnew"])
+def test_fused_qdq_matches_reference(golden, case, tag, mode):
+    x = t(golden[f"{case}_x"])
+    want = t(golden[f"{case}_qdq_{tag}"])
+    got = O.nvfp4_qdq(_inp(x, tag))
+    assert same_bits(got, want)
+    # packed integers -> dequant reproduces the reference output too
+    codes, scales, unit, ncl = O.nvfp4_pack(_inp(x, tag))
+    assert ncl == 0
+    assert same_bits(O.nvfp4_unpack_dequant(codes, scales, unit, want.dtype).reshape(want.shape), want)
+    # C restatement: same integers, same dequantized values
+    c_codes, c_scales, c_unit, _ = C.nvfp4_pack(x.reshape(-1, x.shape[-1]).contiguous(), mode)
+    assert torch.equal(c_codes, codes) and torch.equal(c_scales, scales) and c_unit == float(unit)
+    ob, of = C.nvfp4_dequant(c_codes, c_scales, c_unit, mode)
+    assert same_bits((of if mode == 0 else ob).reshape(want.shape), want)
+
+
+@pytest.mark.parametrize("tag,mode", MODES)
+def test_three_call_form_matches_reference(golden, tag, mode):
+    x = _inp(t(golden["rne_x"]), tag)
+    s = O.get_scalar(x)
+    assert same_bits(s, t(golden[f"rne_scalar_{tag}"]))
+    xq = O.quant(x, s)
+    assert same_bits(xq, t(golden[f"rne_quant_{tag}"]))
+    s_arg = s.clone()
+    out = O.rquant(xq, s_arg)
+    assert same_bits(out, t(golden[f"rne_rquant_{tag}"]))
+    assert same_bits(s_arg, t(golden[f"rne_scalar_after_rquant_{tag}"]))   # in-place side effect
+    assert same_bits(out, t(golden[f"rne_qdq_{tag}"]))                     # reference test 17-26
+
+
+@pytest.mark.parametrize("tag,mode", MODES)
+def test_stochastic_rounding_with_shared_noise_matches_reference(golden, tag, mode):
+    x_b = t(golden["sr_x"])
+    x = _inp(x_b, tag)
+    u = t(golden[f"sr_noise_{tag}"])
+    s = O.get_scalar(x)
+    xq = O.quant(x, s, noise=u)
+    assert same_bits(xq, t(golden[f"sr_quant_{tag}"]))
+    want = t(golden[f"sr_rquant_{tag}"])
+    assert same_bits(O.rquant(xq, s.clone()), want)
+    assert same_bits(O.nvfp4_qdq(x, noise=u), want)
+    # packed form: identical wherever the reference stayed on the E2M1 grid (r <= 7)
+    codes, scales, unit, ncl = O.nvfp4_pack(x, noise=u)
+    deq = O.nvfp4_unpack_dequant(codes, scales, unit, want.dtype)
+    off_grid = (t(golden[f"sr_quant_{tag}"]).abs() > 6)
+    assert int(off_grid.sum()) == ncl
+    assert torch.equal(deq[~off_grid], want[~off_grid])
+    c_codes, c_scales, c_unit, c_ncl = C.nvfp4_pack(x_b.contiguous(), mode, u.contiguous())
+    assert torch.equal(c_codes, codes) and torch.equal(c_scales, scales) and c_ncl == ncl
+
+
+def test_linear_forward_backward_matches_reference(golden):
+    """bitlinear.py:407-513 in fp32: RNE on x and w forward, SR on dY backward (shared noise)."""
+    x, w, b, dy = (t(golden[k]) for k in ("lin_x", "lin_w", "lin_b", "lin_dy"))
+    xq, wq = O.nvfp4_qdq(x), O.nvfp4_qdq(w)
+    y = O.linear_forward(xq, wq, b)
+    assert same_bits(y, t(golden["lin_y"]))
+    dyq = O.nvfp4_qdq(dy, noise=t(golden["lin_noise_dy"]))
+    gx, gw = O.linear_backward(dyq, xq, wq)
+    assert same_bits(gx, t(golden["lin_gx"]))
+    assert same_bits(gw, t(golden["lin_gw"]))
+    assert same_bits(dy.sum(dim=(0, 1)), t(golden["lin_gb"]))
+
+
+def test_bitlinear_forward_matches_reference(golden):
+    """bitlinear.py:736-769 with quantized X and V in the rank-r branch (current reference file)."""
+    x, b = t(golden["lin_x"]), t(golden["lin_b"])
+    v, u, s, res = (t(golden[k]) for k in ("bl_v", "bl_u", "bl_s", "bl_res"))
+    xq = O.nvfp4_qdq(x)
+    y = torch.matmul(xq, O.nvfp4_qdq(v).T)
+    y = torch.mul(s, y)
+    y = torch.matmul(y, u.T)
+    y = y + O.linear_forward(xq, O.nvfp4_qdq(res), b)
+    assert same_bits(y, t(golden["bl_y"]))
