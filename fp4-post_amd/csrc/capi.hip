@@ -1,0 +1,114 @@
+// extern "C" surface of libmetis_hip.so (declared in include/metis_hip.h).
+#include "metis_host.h"
+
+namespace metis {
+int device_cus()
+{
+    static int cached[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+}  // namespace metis
+
+using namespace metis;
+
+extern "C" {
+
+int metis_version(void) { return (0 << 16) | (1 << 8) | 0; }
+
+const char* metis_error_string(int code)
+{
+    switch (code) {
+        case METIS_OK: return "ok";
+        case METIS_E_ARG: return "invalid argument (null/misaligned pointer, negative size, unknown mode or dtype)";
+        case METIS_E_SHAPE: return "NVFP4 block shape (1, 16) does not divide the blocked dimension";
+        case METIS_E_WORKSPACE: return "workspace missing, misaligned or too small";
+        case METIS_E_LAUNCH: return "HIP runtime rejected a kernel launch";
+        case METIS_E_DEVICE: return "unsupported device";
+        default: return "unknown error code";
+    }
+}
+
+size_t metis_nvfp4_workspace_bytes(int64_t rows, int64_t cols)
+{
+    if (rows < 0 || cols < 0) return 0;
+    return workspace_bytes(rows, cols);
+}
+
+int metis_nvfp4_quant_row(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, void* codes, void* scales,
+                          float* unit, void* workspace, size_t workspace_bytes, void* stream)
+{
+    return quantize(x, rows, cols, ld, mode, false, false, nullptr, 0, 0, codes, scales, unit, workspace,
+                    workspace_bytes, (hipStream_t)stream);
+}
+
+int metis_nvfp4_quant_col(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, void* codes, void* scales,
+                          float* unit, void* workspace, size_t workspace_bytes, void* stream)
+{
+    return quantize(x, rows, cols, ld, mode, false, true, nullptr, 0, 0, codes, scales, unit, workspace,
+                    workspace_bytes, (hipStream_t)stream);
+}
+
+int metis_nvfp4_quant_sr_row(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, const void* noise,
+                             uint64_t seed, uint64_t offset, void* codes, void* scales, float* unit, void* workspace,
+                             size_t workspace_bytes, void* stream)
+{
+    return quantize(x, rows, cols, ld, mode, true, false, noise, seed, offset, codes, scales, unit, workspace,
+                    workspace_bytes, (hipStream_t)stream);
+}
+
+int metis_nvfp4_quant_sr_col(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, const void* noise,
+                             uint64_t seed, uint64_t offset, void* codes, void* scales, float* unit, void* workspace,
+                             size_t workspace_bytes, void* stream)
+{
+    return quantize(x, rows, cols, ld, mode, true, true, noise, seed, offset, codes, scales, unit, workspace,
+                    workspace_bytes, (hipStream_t)stream);
+}
+
+int metis_nvfp4_dequant(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, int mode,
+                        void* out, int out_dtype, void* stream)
+{
+    return dequantize(codes, scales, unit, rows, cols, mode, out, out_dtype, (hipStream_t)stream);
+}
+
+int metis_rmsnorm_nvfp4_quant(const void* x, const void* gamma, float eps, int64_t rows, int64_t cols, int mode,
+                              void* normed, void* codes, void* scales, float* unit, void* workspace,
+                              size_t workspace_bytes, void* stream)
+{
+    return rmsnorm_quantize(x, gamma, eps, rows, cols, mode, normed, codes, scales, unit, workspace, workspace_bytes,
+                            (hipStream_t)stream);
+}
+
+int metis_linear_fwd(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes,
+                     const void* b_scales, const float* b_unit, int64_t M, int64_t N, int64_t K, const void* t,
+                     const void* u, int64_t r, const void* bias, void* out, int out_dtype, void* stream)
+{
+    return gemm_nvfp4(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype,
+                      (hipStream_t)stream);
+}
+
+int metis_linear_dgrad(const void* dy_codes, const void* dy_scales, const float* dy_unit, const void* wt_codes,
+                       const void* wt_scales, const float* wt_unit, int64_t L, int64_t N, int64_t K, void* grad_input,
+                       int out_dtype, void* stream)
+{
+    // grad_input[L,K] = dY[L,N] . W[N,K]: contraction over N, both operands blocked along N
+    return gemm_nvfp4(dy_codes, dy_scales, dy_unit, wt_codes, wt_scales, wt_unit, L, K, N, nullptr, nullptr, 0, nullptr,
+                      grad_input, out_dtype, (hipStream_t)stream);
+}
+
+int metis_linear_wgrad(const void* dyt_codes, const void* dyt_scales, const float* dyt_unit, const void* xt_codes,
+                       const void* xt_scales, const float* xt_unit, int64_t L, int64_t N, int64_t K, void* grad_weight,
+                       int out_dtype, void* stream)
+{
+    // grad_weight[N,K] = dY^T[N,L] . X[L,K]: contraction over L, both operands blocked along L
+    return gemm_nvfp4(dyt_codes, dyt_scales, dyt_unit, xt_codes, xt_scales, xt_unit, N, K, L, nullptr, nullptr, 0,
+                      nullptr, grad_weight, out_dtype, (hipStream_t)stream);
+}
+
+}  // extern "C"

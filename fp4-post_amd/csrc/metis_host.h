@@ -1,0 +1,57 @@
+// Host-side declarations shared by the translation units of libmetis_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/metis_hip.h"
+
+namespace metis {
+
+// Caller-supplied scratch, carved as:
+//   [0, 16 KiB)        one partial maximum (uint32 bit pattern) per workgroup of phase 1
+//   [16 KiB, +256 B)   reserved for grid-wide synchronisation words (zero when idle)
+//   [16 KiB + 256, ..) one bf16 block maximum per block of 16
+struct Workspace {
+    uint32_t* gmax;
+    uint32_t* sync;
+    uint16_t* amax;
+};
+constexpr size_t kWsGmaxBytes = 4096 * 4;
+constexpr size_t kWsSyncBytes = 256;
+
+inline size_t workspace_bytes(int64_t rows, int64_t cols)
+{
+    const size_t nblocks = (size_t)((rows * cols + 15) / 16);
+    return kWsGmaxBytes + kWsSyncBytes + ((nblocks * 2 + 255) / 256) * 256;
+}
+
+inline int carve_workspace(void* p, size_t bytes, int64_t rows, int64_t cols, Workspace* ws)
+{
+    if (!p || ((uintptr_t)p % 256) || bytes < workspace_bytes(rows, cols)) return METIS_E_WORKSPACE;
+    char* c = static_cast<char*>(p);
+    ws->gmax = reinterpret_cast<uint32_t*>(c);
+    ws->sync = reinterpret_cast<uint32_t*>(c + kWsGmaxBytes);
+    ws->amax = reinterpret_cast<uint16_t*>(c + kWsGmaxBytes + kWsSyncBytes);
+    return METIS_OK;
+}
+
+// compute units of the current device (cached per device ordinal)
+int device_cus();
+
+// phase 2 of the quantizer (tensor unit + E4M3 bytes from parked block maxima); nvfp4_quant.hip
+int launch_scales(int mode, const Workspace& ws, uint32_t ngroups, void* scales, float* unit, uint32_t nblocks,
+                  hipStream_t st);
+
+int quantize(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, bool sr, bool col, const void* noise,
+             uint64_t seed, uint64_t offset, void* codes, void* scales, float* unit, void* workspace,
+             size_t workspace_bytes, hipStream_t st);
+int dequantize(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, int mode, void* out,
+               int out_dtype, hipStream_t st);
+int rmsnorm_quantize(const void* x, const void* gamma, float eps, int64_t rows, int64_t cols, int mode, void* normed,
+                     void* codes, void* scales, float* unit, void* workspace, size_t workspace_bytes, hipStream_t st);
+int gemm_nvfp4(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes, const void* b_scales,
+               const float* b_unit, int64_t M, int64_t N, int64_t K, const void* t, const void* u, int64_t r,
+               const void* bias, void* out, int out_dtype, hipStream_t st);
+
+}  // namespace metis

@@ -1,0 +1,112 @@
+// Per-block NVFP4 encoding shared by the quantizer kernels (plain and RMSNorm-fused).
+#pragma once
+#include "metis_device.h"
+
+namespace metis {
+
+// ---------------------------------------------------------------------------------------------
+// E2M1 codes of one block.  v: the 16 elements, s: raw block scalar, u: uniform draws (SR only).
+// Packed as two dwords, element 2j in the low nibble of byte j.
+// ---------------------------------------------------------------------------------------------
+template <int MODE, bool SR>
+__device__ __forceinline__ uint2 encode_literal(const float (&v)[kBlock], float s, const float (&u)[kBlock])
+{
+    const float h = rd<MODE>(s / 2.0f);
+    uint32_t w[2] = {0u, 0u};
+#pragma unroll
+    for (int j = 0; j < kBlock; ++j) {
+        float r = code_literal<MODE, SR>(fabsf(v[j]), h, SR ? u[j] : 0.0f);
+        uint32_t code = (uint32_t)fminf(fmaxf(r, 0.0f), 7.0f);      // SR may reach 8: clamp to the grid
+        code |= (v[j] < 0.0f) ? 8u : 0u;
+        w[j >> 3] |= code << (4 * (j & 7));
+    }
+    return make_uint2(w[0], w[1]);
+}
+
+// Round-to-nearest, binary32 arithmetic.  The reference's compress/round/expand sequence equals
+// a round-to-nearest-even conversion of q = RN(|x|/h) onto the E2M1 grid for every binary32 q
+// except q = 5+1ulp, 7-1ulp and 10+1ulp (exhaustive host check), where its second rounding lands
+// on a tie.  The hardware FP4 converter does the RNE conversion two elements at a time; a block
+// whose scalar could produce one of the three exceptional quotients from a bf16 input takes
+// the literal path instead.
+__device__ __forceinline__ bool may_hit_exception(float s)
+{
+    const float h = 0.5f * s;
+    const float t5 = 5.0f * h, t7 = 7.0f * h;                 // 10h shares t5's significand
+    const uint32_t b5 = __float_as_uint(t5), b7 = __float_as_uint(t7);
+    // a bf16 X with RN(X/h) = 5+ulp lies 0..4 binary32 steps above RN(5h); with RN(X/h) = 7-ulp,
+    // 0..4 steps below RN(7h).  Zero steps only counts when the product was inexact.
+    bool c5 = ((b5 + 4u) & 0xffffu) < 4u;
+    bool c7 = ((b7 - 1u) & 0xffffu) < 4u;
+    bool z5 = ((b5 & 0xffffu) == 0u) && (fmaf(5.0f, h, -t5) != 0.0f);
+    bool z7 = ((b7 & 0xffffu) == 0u) && (fmaf(7.0f, h, -t7) != 0.0f);
+    return c5 | c7 | z5 | z7;
+}
+
+__device__ __forceinline__ uint2 encode_rne_p32(const float (&v)[kBlock], float s)
+{
+    if (may_hit_exception(s)) {
+        const float none[kBlock] = {};
+        return encode_literal<0, false>(v, s, none);
+    }
+    const float rs = 1.0f / s;                                // correctly rounded
+    uint32_t lo = 0u, hi = 0u;
+    // code = E2M1(x / s): x/s = (|x| / (s/2)) / 2 exactly, sign carried by the quotient
+    lo = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(lo, div_by(v[0], s, rs), div_by(v[1], s, rs), 1.0f, 0);
+    lo = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(lo, div_by(v[2], s, rs), div_by(v[3], s, rs), 1.0f, 1);
+    lo = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(lo, div_by(v[4], s, rs), div_by(v[5], s, rs), 1.0f, 2);
+    lo = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(lo, div_by(v[6], s, rs), div_by(v[7], s, rs), 1.0f, 3);
+    hi = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(hi, div_by(v[8], s, rs), div_by(v[9], s, rs), 1.0f, 0);
+    hi = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(hi, div_by(v[10], s, rs), div_by(v[11], s, rs), 1.0f, 1);
+    hi = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(hi, div_by(v[12], s, rs), div_by(v[13], s, rs), 1.0f, 2);
+    hi = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(hi, div_by(v[14], s, rs), div_by(v[15], s, rs), 1.0f, 3);
+    return make_uint2(lo, hi);
+}
+
+template <int MODE, bool SR>
+__device__ __forceinline__ uint2 encode_block(const float (&v)[kBlock], float s, const float (&u)[kBlock])
+{
+    if constexpr (MODE == 0 && !SR) return encode_rne_p32(v, s);
+    else return encode_literal<MODE, SR>(v, s, u);
+}
+
+__device__ __forceinline__ float block_amax(const float (&v)[kBlock])
+{
+    float m = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kBlock; j += 2) m = fmaxf(m, fmaxf(fabsf(v[j]), fabsf(v[j + 1])));
+    return m;
+}
+
+__device__ __forceinline__ void unpack16(const uint4 a, const uint4 b, float (&v)[kBlock])
+{
+    const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) { v[2 * j] = bf16_lo(w[j]); v[2 * j + 1] = bf16_hi(w[j]); }
+}
+
+// uniform draws for output block `ob` (16 consecutive elements of the packed orientation)
+template <int MODE>
+__device__ __forceinline__ void philox16(uint64_t seed, uint64_t offset, int64_t ob, float (&u)[kBlock])
+{
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        uint4 r = Philox::draw(offset + (uint64_t)ob * 4u + g, seed);
+        u[4 * g + 0] = uniform_from_bits<MODE>(r.x);
+        u[4 * g + 1] = uniform_from_bits<MODE>(r.y);
+        u[4 * g + 2] = uniform_from_bits<MODE>(r.z);
+        u[4 * g + 3] = uniform_from_bits<MODE>(r.w);
+    }
+}
+
+// publish the workgroup's maximum block-maximum (non-negative floats order like their bit patterns)
+__device__ __forceinline__ void publish_group_max(float m, uint32_t* ws_gmax)
+{
+    __shared__ float smax[4];
+    m = wave_max(m);
+    if ((threadIdx.x & 63) == 0) smax[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) ws_gmax[blockIdx.x] = __float_as_uint(fmaxf(fmaxf(smax[0], smax[1]), fmaxf(smax[2], smax[3])));
+}
+
+}  // namespace metis

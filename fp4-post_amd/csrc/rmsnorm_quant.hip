@@ -1,0 +1,109 @@
+// Fused RMSNorm -> NVFP4 quantization for gfx950: one HBM read of the hidden states.
+//
+// RMSNorm: src/Metis/models/llama.py:23-31 with a bf16 weight (binary32 x * rsqrt(mean(x^2)+eps),
+// rounded to bf16, times gamma, rounded to bf16).  The quantizer then runs on those bf16 values
+// exactly as nvfp4_quant.hip does (src/Metis/Metis/quant.py:6-36); the reference reaches it via
+// LinearLowbitFunction.quantize_input (src/Metis/Metis/bitlinear.py:371-393).
+//
+// One workgroup of 256 threads owns a row at a time; thread t holds blocks t, t+256, ... of the
+// row in registers, so the row is read once.  The sum of squares is reduced across lanes with
+// DPP shuffles and across the four waves through LDS.
+#include "metis_device.h"
+#include "metis_host.h"
+#include "nvfp4_encode.h"
+
+namespace metis {
+
+template <int MODE, int NBT, bool WRITE_NORMED>
+__global__ __launch_bounds__(256) void rmsnorm_quant_kernel(const uint16_t* __restrict__ x,
+                                                            const uint16_t* __restrict__ gamma, float eps,
+                                                            uint32_t rows, uint32_t cols, uint16_t* __restrict__ normed,
+                                                            uint2* __restrict__ codes, uint16_t* __restrict__ ws_amax,
+                                                            uint32_t* __restrict__ ws_gmax)
+{
+    __shared__ float part[2][4];
+    const uint32_t nbpr = cols / kBlock;
+    const float inv_is_div = (float)cols;                     // mean = sum / cols (a division, as torch.mean)
+    float gmax = 0.0f;
+    uint32_t parity = 0;
+    for (uint32_t row = blockIdx.x; row < rows; row += gridDim.x, parity ^= 1u) {
+        float v[NBT][kBlock];
+        float ss = 0.0f;
+#pragma unroll
+        for (int k = 0; k < NBT; ++k) {
+            const uint32_t cb = threadIdx.x + k * 256u;
+            if (cb < nbpr) {
+                const uint4* p = reinterpret_cast<const uint4*>(x + (int64_t)row * cols + (int64_t)cb * kBlock);
+                unpack16(p[0], p[1], v[k]);
+#pragma unroll
+                for (int j = 0; j < kBlock; ++j) ss += v[k][j] * v[k][j];
+            }
+        }
+        ss = wave_sum(ss);
+        if ((threadIdx.x & 63) == 0) part[parity][threadIdx.x >> 6] = ss;
+        __syncthreads();                                      // the other parity is free again after this barrier
+        const float total = (part[parity][0] + part[parity][1]) + (part[parity][2] + part[parity][3]);
+        const float rstd = 1.0f / sqrtf(total / inv_is_div + eps);
+#pragma unroll
+        for (int k = 0; k < NBT; ++k) {
+            const uint32_t cb = threadIdx.x + k * 256u;
+            if (cb < nbpr) {
+                const uint4* g = reinterpret_cast<const uint4*>(gamma + (int64_t)cb * kBlock);
+                float gm[kBlock], n[kBlock];
+                unpack16(g[0], g[1], gm);
+#pragma unroll
+                for (int j = 0; j < kBlock; ++j) n[j] = rb(rb(v[k][j] * rstd) * gm[j]);
+                const uint32_t ob = row * nbpr + cb;
+                if (WRITE_NORMED) {
+                    uint32_t w[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        w[j] = (__float_as_uint(n[2 * j]) >> 16) | (__float_as_uint(n[2 * j + 1]) & 0xffff0000u);
+                    uint4* o = reinterpret_cast<uint4*>(normed + (int64_t)ob * kBlock);
+                    o[0] = make_uint4(w[0], w[1], w[2], w[3]);
+                    o[1] = make_uint4(w[4], w[5], w[6], w[7]);
+                }
+                const float am = block_amax(n);
+                gmax = fmaxf(gmax, am);
+                ws_amax[ob] = (uint16_t)(__float_as_uint(am) >> 16);
+                const float none[kBlock] = {};
+                codes[ob] = encode_block<MODE, false>(n, block_scalar<MODE>(am), none);
+            }
+        }
+    }
+    publish_group_max(gmax, ws_gmax);
+}
+
+int rmsnorm_quantize(const void* x, const void* gamma, float eps, int64_t rows, int64_t cols, int mode, void* normed,
+                     void* codes, void* scales, float* unit, void* workspace, size_t workspace_bytes, hipStream_t st)
+{
+    if (!x || !gamma || !codes || !scales || !unit || rows < 0 || cols < 0) return METIS_E_ARG;
+    if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) return METIS_E_ARG;
+    if (cols % kBlock) return METIS_E_SHAPE;
+    if (cols > 256 * kBlock * 4) return METIS_E_ARG;          // a row is held in registers: at most 16384 columns
+    if (rows * cols / kBlock >= (int64_t)1 << 31) return METIS_E_ARG;
+    if (((uintptr_t)x % 16) || ((uintptr_t)gamma % 16) || ((uintptr_t)codes % 8) || ((uintptr_t)scales % 4) ||
+        (normed && ((uintptr_t)normed % 16)))
+        return METIS_E_ARG;
+    Workspace ws;
+    int rc = carve_workspace(workspace, workspace_bytes, rows, cols, &ws);
+    if (rc != METIS_OK) return rc;
+    if (rows == 0 || cols == 0) return METIS_OK;
+    int64_t g = rows;
+    const int64_t cap = (int64_t)device_cus() * 8;
+    if (g > cap) g = cap;
+    if (g > kMaxGroups) g = kMaxGroups;
+    const int nbt = (int)((cols / kBlock + 255) / 256);
+#define METIS_R(M, NBT, W) hipLaunchKernelGGL((rmsnorm_quant_kernel<M, NBT, W>), dim3((int)g), dim3(256), 0, st, \
+        (const uint16_t*)x, (const uint16_t*)gamma, eps, (uint32_t)rows, (uint32_t)cols, (uint16_t*)normed, (uint2*)codes, \
+        ws.amax, ws.gmax)
+#define METIS_RN(M, W) do { if (nbt <= 1) METIS_R(M, 1, W); else if (nbt == 2) METIS_R(M, 2, W); else METIS_R(M, 4, W); } while (0)
+    if (mode == 0) { if (normed) METIS_RN(0, true); else METIS_RN(0, false); }
+    else { if (normed) METIS_RN(1, true); else METIS_RN(1, false); }
+#undef METIS_RN
+#undef METIS_R
+    if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
+    return launch_scales(mode, ws, (uint32_t)g, scales, unit, (uint32_t)(rows * cols / kBlock), st);
+}
+
+}  // namespace metis

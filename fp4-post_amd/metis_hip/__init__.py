@@ -1,0 +1,12 @@
+"""metis_hip: the Metis NVFP4 hot path on MI355X (gfx950) behind the reference's Python interface.
+
+    from metis_hip import quant_func, LinearLowbitFunction, LinearLowbit, BitLinear
+    from metis_hip import MetisArgs, replace_linear_with_metis, replace_model_with_metis
+
+Compute goes through libmetis_hip.so (hand-written HIP kernels, C ABI in include/metis_hip.h).
+"""
+from . import ops
+from ._lib import MODE_P32, MODE_PB16, MetisHipError
+from .ops import PackedNVFP4
+
+__all__ = ["ops", "PackedNVFP4", "MODE_P32", "MODE_PB16", "MetisHipError"]

@@ -1,0 +1,69 @@
+"""ctypes binding of libmetis_hip.so (the C ABI declared in include/metis_hip.h).
+
+The product path has no CPU or PyTorch fallback: if the shared library is missing or a call
+returns an error code, an exception is raised.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmetis_hip.so")
+
+OK, E_ARG, E_SHAPE, E_WORKSPACE, E_LAUNCH, E_DEVICE = 0, -1, -2, -3, -4, -5
+MODE_P32, MODE_PB16 = 0, 1
+DTYPE_BF16, DTYPE_F32 = 0, 1
+
+_vp, _i64, _i32, _u64, _f32, _sz = (ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_uint64,
+                                    ctypes.c_float, ctypes.c_size_t)
+
+# name -> (restype, argtypes); must list every symbol include/metis_hip.h declares
+SIGNATURES = {
+    "metis_version": (_i32, []),
+    "metis_error_string": (ctypes.c_char_p, [_i32]),
+    "metis_nvfp4_workspace_bytes": (_sz, [_i64, _i64]),
+    "metis_nvfp4_quant_row": (_i32, [_vp, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "metis_nvfp4_quant_col": (_i32, [_vp, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "metis_nvfp4_quant_sr_row": (_i32, [_vp, _i64, _i64, _i64, _i32, _vp, _u64, _u64, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "metis_nvfp4_quant_sr_col": (_i32, [_vp, _i64, _i64, _i64, _i32, _vp, _u64, _u64, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "metis_nvfp4_dequant": (_i32, [_vp, _vp, _vp, _i64, _i64, _i32, _vp, _i32, _vp]),
+    "metis_rmsnorm_nvfp4_quant": (_i32, [_vp, _vp, _f32, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "metis_linear_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _i32, _vp]),
+    "metis_linear_dgrad": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i32, _vp]),
+    "metis_linear_wgrad": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i32, _vp]),
+}
+
+_lib = None
+
+
+class MetisHipError(RuntimeError):
+    pass
+
+
+def load():
+    """Load the library once; raises MetisHipError if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise MetisHipError(
+                f"{LIB_PATH} not found: build it with `make -C fp4-post_amd/csrc` "
+                "(or __graft_entry__.build()); there is no fallback path"
+            )
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = lib
+    return _lib
+
+
+def check(rc: int, what: str, shape=None):
+    """Map a return code to the exception the reference raises for the same condition."""
+    if rc == OK:
+        return
+    msg = load().metis_error_string(rc).decode()
+    if rc == E_SHAPE:
+        # quant.py:400-403 raises ValueError for a last dim that 16 does not divide
+        raise ValueError(f"NVFP4 block shape (1, 16) does not divide tensor shape {tuple(shape) if shape is not None else '?'}")
+    raise MetisHipError(f"{what}: {msg} (code {rc})")

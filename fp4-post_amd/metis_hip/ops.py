@@ -1,0 +1,184 @@
+"""Tensor-level entry points over the C ABI: quantize, dequantize, fused norm+quant, GEMMs.
+
+All functions take CUDA (ROCm) tensors, enqueue on torch's current stream and return tensors;
+PyTorch is used only to own device memory and streams.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from . import _lib
+from ._lib import DTYPE_BF16, DTYPE_F32, MODE_P32, MODE_PB16, check, load
+
+BLOCK = 16
+_workspaces: dict = {}
+
+
+@dataclass
+class PackedNVFP4:
+    """NVFP4 tensor: value[i, k] = e2m1(codes) * e4m3(scales[i, k // 16]) * unit.
+
+    `codes` [rows, cols/2] uint8 (element 2j in the low nibble), `scales` [rows, cols/16] uint8
+    (float8_e4m3fn bytes), `unit` float32[1] on the device.  (rows, cols) is the logical shape in
+    the packed orientation: for column-blocked packing of x[R, C] it is (C, R).
+    """
+    codes: torch.Tensor
+    scales: torch.Tensor
+    unit: torch.Tensor
+    rows: int
+    cols: int
+    mode: int = MODE_P32
+
+    def dequantize(self, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+        return dequantize(self, dtype)
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _workspace(rows: int, cols: int, device: torch.device) -> torch.Tensor:
+    need = load().metis_nvfp4_workspace_bytes(rows, cols)
+    key = (device.index, _stream())
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < need:
+        ws = torch.zeros(max(need, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def _as_2d_bf16(x: torch.Tensor) -> torch.Tensor:
+    if not x.is_cuda:
+        raise _lib.MetisHipError("metis_hip ops need a ROCm device tensor; there is no CPU path")
+    if x.dtype != torch.bfloat16:
+        # P32 parity is defined on bf16-valued inputs; a wider tensor must already hold bf16 values
+        xb = x.to(torch.bfloat16)
+        x = xb
+    x2 = x.reshape(-1, x.shape[-1])
+    return x2 if x2.is_contiguous() else x2.contiguous()
+
+
+def quantize(x: torch.Tensor, mode: int = MODE_P32, *, col: bool = False, sr: bool = False,
+             noise: torch.Tensor | None = None, seed: int = 0, offset: int = 0) -> PackedNVFP4:
+    """NVFP4-quantize x (flattened to [R, C]).
+
+    col=False: blocks of 16 along C -> PackedNVFP4 of shape (R, C).
+    col=True : blocks of 16 along R, written transposed -> shape (C, R).
+    sr=True  : stochastic rounding; `noise` (same shape as x, float32 for P32 / bf16 for PB16)
+               overrides the internal Philox stream keyed by (seed, offset).
+    """
+    x2 = _as_2d_bf16(x)
+    rows, cols = x2.shape
+    blocked = rows if col else cols
+    if blocked % BLOCK:
+        raise ValueError(f"NVFP4 block shape (1, 16) does not divide tensor shape {tuple(x.shape)}")
+    prow, pcol = (cols, rows) if col else (rows, cols)
+    dev = x2.device
+    codes = torch.empty(prow, pcol // 2, dtype=torch.uint8, device=dev)
+    scales = torch.empty(prow, pcol // BLOCK, dtype=torch.uint8, device=dev)
+    unit = torch.empty(1, dtype=torch.float32, device=dev)
+    ws = _workspace(rows, cols, dev)
+    L = load()
+    if sr:
+        nz = None
+        if noise is not None:
+            want = torch.bfloat16 if mode == MODE_PB16 else torch.float32
+            nz = noise.reshape(rows, cols).to(want).contiguous()
+        fn = L.metis_nvfp4_quant_sr_col if col else L.metis_nvfp4_quant_sr_row
+        rc = fn(x2.data_ptr(), rows, cols, x2.stride(0), mode, None if nz is None else nz.data_ptr(),
+                seed & (2 ** 64 - 1), offset, codes.data_ptr(), scales.data_ptr(), unit.data_ptr(),
+                ws.data_ptr(), ws.numel(), _stream())
+    else:
+        fn = L.metis_nvfp4_quant_col if col else L.metis_nvfp4_quant_row
+        rc = fn(x2.data_ptr(), rows, cols, x2.stride(0), mode, codes.data_ptr(), scales.data_ptr(),
+                unit.data_ptr(), ws.data_ptr(), ws.numel(), _stream())
+    check(rc, "metis_nvfp4_quant", x.shape)
+    return PackedNVFP4(codes, scales, unit, prow, pcol, mode)
+
+
+def dequantize(p: PackedNVFP4, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    if dtype not in (torch.bfloat16, torch.float32):
+        raise ValueError("dequantize: dtype must be bfloat16 or float32")
+    out = torch.empty(p.rows, p.cols, dtype=dtype, device=p.codes.device)
+    rc = load().metis_nvfp4_dequant(p.codes.data_ptr(), p.scales.data_ptr(), p.unit.data_ptr(), p.rows, p.cols,
+                                    p.mode, out.data_ptr(), DTYPE_F32 if dtype == torch.float32 else DTYPE_BF16,
+                                    _stream())
+    check(rc, "metis_nvfp4_dequant", (p.rows, p.cols))
+    return out
+
+
+def rmsnorm_quantize(x: torch.Tensor, gamma: torch.Tensor, eps: float, mode: int = MODE_P32,
+                     want_normed: bool = True):
+    """Fused RMSNorm -> NVFP4.  Returns (normed bf16 or None, PackedNVFP4)."""
+    x2 = _as_2d_bf16(x)
+    rows, cols = x2.shape
+    if cols % BLOCK:
+        raise ValueError(f"NVFP4 block shape (1, 16) does not divide tensor shape {tuple(x.shape)}")
+    g = gamma.to(device=x2.device, dtype=torch.bfloat16).contiguous()
+    dev = x2.device
+    normed = torch.empty(rows, cols, dtype=torch.bfloat16, device=dev) if want_normed else None
+    codes = torch.empty(rows, cols // 2, dtype=torch.uint8, device=dev)
+    scales = torch.empty(rows, cols // BLOCK, dtype=torch.uint8, device=dev)
+    unit = torch.empty(1, dtype=torch.float32, device=dev)
+    ws = _workspace(rows, cols, dev)
+    rc = load().metis_rmsnorm_nvfp4_quant(x2.data_ptr(), g.data_ptr(), float(eps), rows, cols, mode,
+                                          None if normed is None else normed.data_ptr(), codes.data_ptr(),
+                                          scales.data_ptr(), unit.data_ptr(), ws.data_ptr(), ws.numel(), _stream())
+    check(rc, "metis_rmsnorm_nvfp4_quant", x.shape)
+    if normed is not None:
+        normed = normed.reshape(x.shape)
+    return normed, PackedNVFP4(codes, scales, unit, rows, cols, mode)
+
+
+def linear_fwd(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None, u: torch.Tensor | None = None,
+               bias: torch.Tensor | None = None, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """out[M, N] = deq(a)[M, K] . deq(b)[N, K]^T (+ t[M, r] . u[N, r]^T) (+ bias[N])."""
+    if a.cols != b.cols:
+        raise ValueError(f"contraction mismatch: {a.cols} vs {b.cols}")
+    M, N, K = a.rows, b.rows, a.cols
+    dev = a.codes.device
+    r = 0
+    if t is not None:
+        t = t.to(torch.bfloat16).contiguous()
+        u = u.to(torch.bfloat16).contiguous()
+        r = t.shape[1]
+        if t.shape != (M, r) or u.shape != (N, r):
+            raise ValueError("low-rank operands must be t[M, r], u[N, r]")
+    if bias is not None:
+        bias = bias.to(torch.bfloat16).contiguous()
+    out = torch.empty(M, N, dtype=out_dtype, device=dev)
+    rc = load().metis_linear_fwd(a.codes.data_ptr(), a.scales.data_ptr(), a.unit.data_ptr(), b.codes.data_ptr(),
+                                 b.scales.data_ptr(), b.unit.data_ptr(), M, N, K,
+                                 None if t is None else t.data_ptr(), None if u is None else u.data_ptr(), r,
+                                 None if bias is None else bias.data_ptr(), out.data_ptr(),
+                                 DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16, _stream())
+    check(rc, "metis_linear_fwd", (M, N, K))
+    return out
+
+
+def linear_dgrad(dy: PackedNVFP4, wt: PackedNVFP4, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """grad_input[L, K] from dY packed along N [L, N] and W packed along N (column-blocked) [K, N]."""
+    if dy.cols != wt.cols:
+        raise ValueError(f"contraction mismatch: {dy.cols} vs {wt.cols}")
+    L, N, K = dy.rows, dy.cols, wt.rows
+    out = torch.empty(L, K, dtype=out_dtype, device=dy.codes.device)
+    rc = load().metis_linear_dgrad(dy.codes.data_ptr(), dy.scales.data_ptr(), dy.unit.data_ptr(), wt.codes.data_ptr(),
+                                   wt.scales.data_ptr(), wt.unit.data_ptr(), L, N, K, out.data_ptr(),
+                                   DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16, _stream())
+    check(rc, "metis_linear_dgrad", (L, N, K))
+    return out
+
+
+def linear_wgrad(dyt: PackedNVFP4, xt: PackedNVFP4, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """grad_weight[N, K] from dY and X both packed along tokens: dyt [N, L], xt [K, L]."""
+    if dyt.cols != xt.cols:
+        raise ValueError(f"contraction mismatch: {dyt.cols} vs {xt.cols}")
+    N, L, K = dyt.rows, dyt.cols, xt.rows
+    out = torch.empty(N, K, dtype=out_dtype, device=dyt.codes.device)
+    rc = load().metis_linear_wgrad(dyt.codes.data_ptr(), dyt.scales.data_ptr(), dyt.unit.data_ptr(),
+                                   xt.codes.data_ptr(), xt.scales.data_ptr(), xt.unit.data_ptr(), L, N, K,
+                                   out.data_ptr(), DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16, _stream())
+    check(rc, "metis_linear_wgrad", (L, N, K))
+    return out

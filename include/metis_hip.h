@@ -1,0 +1,172 @@
+/*
+ * metis_hip.h -- C ABI of libmetis_hip.so: the Metis NVFP4 hot path as HIP kernels for gfx950.
+ *
+ * The reference implements this path as eager PyTorch code with no native entry points, so each
+ * function below names the Python function whose arithmetic it replaces (paths relative to the
+ * reference checkout).  A binding needs nothing but device pointers, sizes and a stream.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless stated otherwise; `stream` is a hipStream_t
+ *     passed as void* (NULL = the default stream)
+ *   - tensors are row-major; bf16 tensors are 16-bit patterns
+ *   - functions enqueue work on `stream` and return immediately; they never allocate, free or
+ *     synchronise.  Scratch memory comes from the caller (`workspace`), must be 256-byte
+ *     aligned, zero-filled once when it is allocated, and may be reused by later calls on the
+ *     same stream (calls that share a workspace must not overlap in time)
+ *   - return value: METIS_OK or a negative METIS_E_* code; nothing is written on error
+ *   - `mode` selects which arithmetic of the reference is reproduced bit for bit:
+ *       METIS_MODE_P32  binary32 arithmetic on the bf16-valued input (reference run with
+ *                       compute_dtype=float32, src/Metis/Metis/bitlinear.py:70,377)
+ *       METIS_MODE_PB16 every eager op rounded to bf16 (compute_dtype=bfloat16,
+ *                       src/grpo/grpo.py:204-205)
+ *
+ * NVFP4 layout produced / consumed (the reference never materialises it; these are the integers
+ * its arithmetic passes through, src/Metis/Metis/quant.py:19-31)
+ *   codes  uint8 [rows, cols/2]   element 2j in the low nibble of byte j;
+ *                                 nibble = (x < 0) << 3 | r, r in 0..7 the E2M1 magnitude code
+ *   scales uint8 [rows, cols/16]  float8_e4m3fn byte of (block scalar / unit)
+ *   unit   float                  max(block scalar) / 448   (bf16-valued in METIS_MODE_PB16)
+ *   value of an element = e2m1(r) * sign * e4m3(scale) * unit,  e2m1 = {0,.5,1,1.5,2,3,4,6}
+ */
+#ifndef METIS_HIP_H
+#define METIS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define METIS_OK 0
+#define METIS_E_ARG (-1)       /* null pointer, negative size, unknown mode/dtype             */
+#define METIS_E_SHAPE (-2)     /* block of 16 does not divide the blocked dimension -> ValueError
+                                  in the reference (src/Metis/Metis/quant.py:400-403)          */
+#define METIS_E_WORKSPACE (-3) /* workspace missing, misaligned or too small                   */
+#define METIS_E_LAUNCH (-4)    /* the HIP runtime rejected a launch                             */
+#define METIS_E_DEVICE (-5)    /* not a gfx950 device / required feature missing               */
+
+#define METIS_MODE_P32 0
+#define METIS_MODE_PB16 1
+
+#define METIS_DTYPE_BF16 0
+#define METIS_DTYPE_F32 1
+
+/* Library version, (major << 16) | (minor << 8) | patch.  No reference counterpart. */
+int metis_version(void);
+
+/* Static text for a return code.  Host pointer, never NULL. */
+const char *metis_error_string(int code);
+
+/* Bytes of workspace the quantizer entry points need for a [rows, cols] tensor. */
+size_t metis_nvfp4_workspace_bytes(int64_t rows, int64_t cols);
+
+/*
+ * NVFP4 round-to-nearest quantizer, blocks of 16 along the last dimension.
+ * Replaces Cast2NVFp4e2m1BlockNOSR.quantize_dequantize -> _nvfp4_nosr_quantize_dequantize
+ * (src/Metis/Metis/quant.py:6-36, 392-433) up to the dequantisation, i.e. it emits the packed
+ * integers; metis_nvfp4_dequant() completes the round trip.
+ *   x      bf16 [rows, cols], row stride `ld` elements (ld >= cols)
+ *   codes  uint8 [rows, cols/2]; scales uint8 [rows, cols/16]; unit float[1]
+ * METIS_E_SHAPE when cols % 16 != 0.
+ */
+int metis_nvfp4_quant_row(const void *x, int64_t rows, int64_t cols, int64_t ld, int mode,
+                          void *codes, void *scales, float *unit, void *workspace,
+                          size_t workspace_bytes, void *stream);
+
+/*
+ * Same quantizer with blocks of 16 along dimension 0 (tokens), written transposed: the operand
+ * layout of a GEMM that contracts over tokens.  Equals metis_nvfp4_quant_row applied to x^T.
+ * The reference quantizes dY along its last dimension only (src/Metis/Metis/bitlinear.py:
+ * 395-405, 488-492), which a block-scaled GEMM cannot contract over tokens.
+ *   x      bf16 [rows, cols], row stride ld
+ *   codes  uint8 [cols, rows/2]; scales uint8 [cols, rows/16]; unit float[1]
+ * METIS_E_SHAPE when rows % 16 != 0.
+ */
+int metis_nvfp4_quant_col(const void *x, int64_t rows, int64_t cols, int64_t ld, int mode,
+                          void *codes, void *scales, float *unit, void *workspace,
+                          size_t workspace_bytes, void *stream);
+
+/*
+ * NVFP4 stochastic-rounding quantizer: Cast2NVFp4e2m1Block.get_scalar/quant
+ * (src/Metis/Metis/quant.py:273-308) with the element rule of Cast2Fp4e2m1Random.quant
+ * (137-147): compress, add (u - 0.5), round.
+ *   noise  NULL -> u is drawn from Philox4x32-10 keyed by (seed, offset + element index);
+ *          else the uniform draws in [0,1) to use, same shape as x: float32 in METIS_MODE_P32,
+ *          bf16 in METIS_MODE_PB16 (what torch.rand_like yields for that dtype)
+ * A draw that rounds the block maximum up to r = 8 (possible in the reference, which then
+ * returns the off-grid value 8 * scalar) is clamped to r = 7.
+ */
+int metis_nvfp4_quant_sr_row(const void *x, int64_t rows, int64_t cols, int64_t ld, int mode,
+                             const void *noise, uint64_t seed, uint64_t offset, void *codes,
+                             void *scales, float *unit, void *workspace, size_t workspace_bytes,
+                             void *stream);
+
+/* Column-blocked stochastic rounding: metis_nvfp4_quant_sr_row of x^T; `noise`, when given, is
+ * indexed like x (noise[r, c] belongs to x[r, c]) and the Philox counter is the index in x^T. */
+int metis_nvfp4_quant_sr_col(const void *x, int64_t rows, int64_t cols, int64_t ld, int mode,
+                             const void *noise, uint64_t seed, uint64_t offset, void *codes,
+                             void *scales, float *unit, void *workspace, size_t workspace_bytes,
+                             void *stream);
+
+/*
+ * Dequantize packed NVFP4: the last three multiplications of the reference,
+ * out = ((v * sign) / 2) * (e4m3 * unit)  (src/Metis/Metis/quant.py:23-24, 32-35; rquant 470-548).
+ *   out    [rows, cols] of out_dtype (METIS_DTYPE_BF16 or METIS_DTYPE_F32); in METIS_MODE_P32 a
+ *          bf16 output is the binary32 result rounded once
+ */
+int metis_nvfp4_dequant(const void *codes, const void *scales, const float *unit, int64_t rows,
+                        int64_t cols, int mode, void *out, int out_dtype, void *stream);
+
+/*
+ * Fused RMSNorm -> NVFP4 quantization of the normed activations: one read of the hidden states.
+ * RMSNorm follows src/Metis/models/llama.py:23-31 with a bf16 weight (binary32 normalisation,
+ * rounded to bf16, times gamma, rounded to bf16); the quantizer is metis_nvfp4_quant_row applied
+ * to the bf16 normed values.  The reference has no fused op: it runs the norm, then quantizes
+ * in LinearLowbitFunction.quantize_input (src/Metis/Metis/bitlinear.py:371-393).
+ *   x      bf16 [rows, cols]; gamma bf16 [cols]
+ *   normed bf16 [rows, cols] (may be NULL when only the packed form is wanted)
+ */
+int metis_rmsnorm_nvfp4_quant(const void *x, const void *gamma, float eps, int64_t rows,
+                              int64_t cols, int mode, void *normed, void *codes, void *scales,
+                              float *unit, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Block-scaled NVFP4 GEMM with an optional bf16 low-rank extension and bias:
+ *   out[M,N] = ua*ub * sum_k deq(A)[m,k] * deq(B)[n,k]  +  sum_j T[m,j] * U[n,j]  +  bias[n]
+ * A (M x K) and B (N x K) are packed NVFP4 with blocks of 16 along K; *ua, *ub are their units.
+ * Products of E2M1 and E4M3 values are exact in bf16, accumulation is binary32 (MFMA).
+ * Replaces torch.matmul(input_, quantized_weight.T) (+ bias) in LinearLowbitFunction.forward
+ * (src/Metis/Metis/bitlinear.py:435-438) and, with T = (X V^T) * s and U, the sum of the two
+ * branches in BitLinear.forward (src/Metis/Metis/bitlinear.py:752-760).
+ *   t      bf16 [M, r] row stride r, u bf16 [N, r]; r % 32 == 0 or r == 0 (t, u NULL)
+ *   bias   bf16 [N] or NULL
+ *   out    [M, N] of out_dtype
+ */
+int metis_linear_fwd(const void *a_codes, const void *a_scales, const float *a_unit,
+                     const void *b_codes, const void *b_scales, const float *b_unit, int64_t M,
+                     int64_t N, int64_t K, const void *t, const void *u, int64_t r,
+                     const void *bias, void *out, int out_dtype, void *stream);
+
+/*
+ * grad_input[L,K] = deq(dY)[L,N] . deq(W)[N,K]   (src/Metis/Metis/bitlinear.py:507-508)
+ *   dy_* : dY packed with blocks along N (metis_nvfp4_quant_sr_row of dY [L,N])
+ *   wt_* : W packed with blocks along N  (metis_nvfp4_quant_col of W [N,K] -> [K, N/2])
+ */
+int metis_linear_dgrad(const void *dy_codes, const void *dy_scales, const float *dy_unit,
+                       const void *wt_codes, const void *wt_scales, const float *wt_unit, int64_t L,
+                       int64_t N, int64_t K, void *grad_input, int out_dtype, void *stream);
+
+/*
+ * grad_weight[N,K] = deq(dY)^T[N,L] . deq(X)[L,K]  in binary32 (src/Metis/Metis/bitlinear.py:502-510)
+ *   dyt_* : dY packed with blocks along L (metis_nvfp4_quant_sr_col of dY [L,N] -> [N, L/2])
+ *   xt_*  : X  packed with blocks along L (metis_nvfp4_quant_sr_col of X  [L,K] -> [K, L/2])
+ */
+int metis_linear_wgrad(const void *dyt_codes, const void *dyt_scales, const float *dyt_unit,
+                       const void *xt_codes, const void *xt_scales, const float *xt_unit, int64_t L,
+                       int64_t N, int64_t K, void *grad_weight, int out_dtype, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* METIS_HIP_H */

@@ -1,0 +1,234 @@
+"""GPU parity of the NVFP4 quantizer kernels, called through the C ABI, against the CPU oracle.
+
+Bar: bit-exact codes, E4M3 scale bytes and unit in both parity modes; dequantized output equal
+to the reference's own golden QDQ output.
+"""
+import numpy as np
+import pytest
+import torch
+
+from helpers import same_bits, synthetic_activation, t
+
+pytestmark = pytest.mark.gpu
+
+MODES = [("p32", 0), ("pb16", 1)]
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from metis_hip import ops as _ops
+    assert torch.cuda.is_available(), "GPU tests need a ROCm device"
+    return _ops
+
+
+def _oracle_in(x_bf16, mode):
+    return x_bf16.float() if mode == 0 else x_bf16
+
+
+def _check_packed(p, codes, scales, unit, what=""):
+    torch.cuda.synchronize()
+    assert torch.equal(p.codes.cpu(), codes), f"codes differ {what}: {(p.codes.cpu() != codes).sum().item()} bytes"
+    assert torch.equal(p.scales.cpu(), scales), f"scales differ {what}: {(p.scales.cpu() != scales).sum().item()} bytes"
+    assert float(p.unit.cpu()) == float(unit), f"unit differs {what}: {float(p.unit.cpu())} vs {float(unit)}"
+
+
+@pytest.mark.parametrize("tag,mode", MODES)
+@pytest.mark.parametrize("case", ["rne", "rne3d", "rnew"])
+def test_rne_against_reference_golden(ops, golden, case, tag, mode):
+    """deq(pack(x)) == the reference's quantize_dequantize(x) on the reference's own vectors."""
+    from oracle import metis_oracle as O
+    x = t(golden[f"{case}_x"])
+    want = t(golden[f"{case}_qdq_{tag}"])
+    p = ops.quantize(x.cuda(), mode)
+    codes, scales, unit, _ = O.nvfp4_pack(_oracle_in(x, mode))
+    _check_packed(p, codes, scales, unit, case)
+    got = ops.dequantize(p, want.dtype).cpu().reshape(want.shape)
+    assert same_bits(got, want)
+    if mode == 0:   # "stored as bf16": one rounding of the binary32 result
+        assert same_bits(ops.dequantize(p, torch.bfloat16).cpu().reshape(want.shape), want.bfloat16())
+
+
+@pytest.mark.parametrize("tag,mode", MODES)
+@pytest.mark.parametrize("shape", [(256, 512), (1, 16), (37, 48), (3, 5, 64), (1000, 1536)])
+def test_rne_row_seeded(ops, shape, tag, mode):
+    from oracle import metis_oracle as O
+    x = synthetic_activation(100 + sum(shape), int(np.prod(shape[:-1])), shape[-1]).reshape(shape)
+    x.view(-1)[::97] = 0
+    p = ops.quantize(x.cuda(), mode)
+    codes, scales, unit, _ = O.nvfp4_pack(_oracle_in(x, mode))
+    _check_packed(p, codes, scales, unit, str(shape))
+
+
+@pytest.mark.parametrize("tag,mode", MODES)
+def test_rne_all_bf16_magnitudes_and_exact_ties(ops, tag, mode):
+    """Every finite bf16 magnitude against block scalars that make ties exact."""
+    from oracle import c_oracle as C
+    pat = torch.arange(0, 0x7F80, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    n = (pat.numel() // 15) * 15
+    for amax in (6.0, 3.0, 0.75, 448.0, 0.0283203125, 3.0e-5, 2.984375, 1.5e30):
+        am = torch.tensor(amax).bfloat16()
+        body = pat[:n].reshape(-1, 15)
+        body = torch.where(body.float() <= am.float(), body, torch.zeros_like(body))
+        x = torch.cat([am.expand(body.shape[0], 1), body], dim=1).contiguous()
+        x[1::2] = -x[1::2]
+        p = ops.quantize(x.cuda(), mode)
+        cc, cs, cu, _ = C.nvfp4_pack(x, mode)
+        _check_packed(p, cc, cs, cu, f"amax={amax}")
+
+
+def test_rne_p32_exception_quotients(ops):
+    """Blocks built so that |x| / (scalar/2) rounds to 5+1ulp, 7-1ulp, 10+1ulp: the three quotients
+    where the reference's compress/round sequence differs from a plain RNE conversion."""
+    from oracle import c_oracle as C
+    import struct
+    rows = []
+    g = torch.Generator().manual_seed(9)
+    found = 0
+    # search block maxima whose scalar h = s/2 puts a bf16 value right next to 5h / 7h / 10h
+    cand = torch.arange(0x3C00, 0x4400, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).float()
+    s = cand / 6 + 1e-9
+    h = s / 2
+    for mult, delta in ((5.0, 1), (7.0, -1), (10.0, 1)):
+        tgt = torch.tensor(mult)
+        tq = torch.nextafter(tgt, tgt + delta)                       # the exceptional quotient
+        xs = (tq * h).bfloat16()                                     # nearest bf16 to q*h
+        q = xs.float() / h
+        hit = (q == tq) & (xs.float() <= cand)
+        for i in hit.nonzero().flatten().tolist()[:8]:
+            blk = torch.zeros(16)
+            blk[0] = cand[i]
+            blk[1] = xs[i].float()
+            blk[2] = -xs[i].float()
+            rows.append(blk)
+            found += 1
+    assert found >= 3, "test construction failed to reach the exceptional quotients"
+    x = torch.stack(rows).bfloat16().contiguous()
+    p = ops.quantize(x.cuda(), 0)
+    cc, cs, cu, _ = C.nvfp4_pack(x, 0)
+    _check_packed(p, cc, cs, cu, "exception quotients")
+
+
+@pytest.mark.parametrize("tag,mode", MODES)
+@pytest.mark.parametrize("shape", [(64, 96), (256, 512), (48, 1000)])
+def test_rne_col(ops, shape, tag, mode):
+    from oracle import metis_oracle as O
+    x = synthetic_activation(200 + shape[0], *shape)
+    p = ops.quantize(x.cuda(), mode, col=True)
+    codes, scales, unit, _ = O.nvfp4_pack_col(_oracle_in(x, mode))
+    assert (p.rows, p.cols) == (shape[1], shape[0])
+    _check_packed(p, codes, scales, unit, str(shape))
+
+
+@pytest.mark.parametrize("tag,mode", MODES)
+@pytest.mark.parametrize("col", [False, True])
+def test_sr_explicit_noise(ops, golden, tag, mode, col):
+    from oracle import metis_oracle as O
+    x = t(golden["sr_x"])
+    u = t(golden[f"sr_noise_{tag}"])
+    p = ops.quantize(x.cuda(), mode, col=col, sr=True, noise=u.cuda())
+    xin = _oracle_in(x, mode)
+    codes, scales, unit, ncl = (O.nvfp4_pack_col if col else O.nvfp4_pack)(xin, u)
+    _check_packed(p, codes, scales, unit, f"sr col={col}")
+    if not col:
+        # against the reference's own SR output wherever it stayed on the E2M1 grid
+        want = t(golden[f"sr_rquant_{tag}"])
+        on_grid = t(golden[f"sr_quant_{tag}"]).abs() <= 6
+        got = ops.dequantize(p, want.dtype).cpu()
+        assert torch.equal(got[on_grid], want[on_grid]) and int((~on_grid).sum()) == ncl
+
+
+@pytest.mark.parametrize("tag,mode", MODES)
+@pytest.mark.parametrize("col", [False, True])
+def test_sr_internal_philox_stream(ops, tag, mode, col):
+    """The device draws Philox4x32-10(counter = offset + e/4, key = seed), word e%4, for packed element e."""
+    from oracle import metis_oracle as O
+    from philox_ref import uniform_for_elements
+    x = synthetic_activation(300, 64, 128)
+    seed, offset = 0x1234_5678_9ABC_DEF0, 77
+    p = ops.quantize(x.cuda(), mode, col=col, sr=True, seed=seed, offset=offset)
+    u = torch.from_numpy(uniform_for_elements(x.numel(), seed, offset, bf16=(mode == 1)))
+    xin = _oracle_in(x, mode)
+    if col:
+        u_as_x = u.reshape(128, 64).t().contiguous()               # draws are indexed in the packed orientation
+        codes, scales, unit, _ = O.nvfp4_pack_col(xin, u_as_x.to(xin.dtype))
+    else:
+        codes, scales, unit, _ = O.nvfp4_pack(xin, u.reshape(64, 128).to(xin.dtype))
+    _check_packed(p, codes, scales, unit, f"philox col={col}")
+
+
+def test_sr_is_unbiased(ops):
+    """E[deq(SR(x))] = x for values inside the grid: mean over 4096 independent draws."""
+    vals = torch.tensor([0.1, 0.3, 0.6, 0.9, 1.2, 1.7, 2.3, 2.9, 3.4, 4.4, 5.1, 5.8, -0.2, -1.1, -2.6, 6.0])
+    x = vals.bfloat16().repeat(4096, 1).contiguous()              # block max 6 -> scalar 1 + 1e-9
+    p = ops.quantize(x.cuda(), 0, sr=True, seed=42)
+    deq = ops.dequantize(p, torch.float32).cpu()
+    mean = deq.mean(0)
+    step = torch.tensor([0.5] * 4 + [0.5] * 3 + [1.0] * 2 + [2.0] * 3 + [0.5, 0.5, 1.0, 2.0])
+    sigma = step / 2 / (4096 ** 0.5)
+    assert bool(((mean - x[0].float()).abs() <= 5 * sigma + 1e-6).all()), (mean, x[0])
+    assert bool((deq[:, :15].std(0) > 0).all())                      # every off-grid value rounds both ways
+    assert float(deq[:, 15].std()) == 0.0                            # the block maximum sits on the grid
+    # different seeds give different streams, same seed the same codes
+    p2 = ops.quantize(x.cuda(), 0, sr=True, seed=42)
+    p3 = ops.quantize(x.cuda(), 0, sr=True, seed=43)
+    assert torch.equal(p.codes, p2.codes) and not torch.equal(p.codes, p3.codes)
+
+
+def test_errors_and_edges(ops):
+    with pytest.raises(ValueError):
+        ops.quantize(torch.zeros(4, 24, dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(ValueError):
+        ops.quantize(torch.zeros(24, 32, dtype=torch.bfloat16, device="cuda"), col=True)
+    p = ops.quantize(torch.zeros(0, 32, dtype=torch.bfloat16, device="cuda"))
+    assert p.codes.shape == (0, 16) and p.scales.shape == (0, 2)
+    # all-zero tensor: scalar = 1e-9 everywhere, scale byte 0x7E, codes 0
+    z = ops.quantize(torch.zeros(8, 64, dtype=torch.bfloat16, device="cuda"))
+    torch.cuda.synchronize()
+    assert int(z.codes.sum()) == 0 and bool((z.scales == 0x7E).all())
+    assert float(z.unit.cpu()) == float(torch.tensor(1e-9) / 448)
+    # strided rows (ld > cols)
+    from oracle import metis_oracle as O
+    base = synthetic_activation(5, 32, 256)
+    view = base[:, 64:192]
+    from metis_hip import _lib
+    L = _lib.load()
+    xd = base.cuda()
+    codes = torch.empty(32, 64, dtype=torch.uint8, device="cuda")
+    scales = torch.empty(32, 8, dtype=torch.uint8, device="cuda")
+    unit = torch.empty(1, dtype=torch.float32, device="cuda")
+    ws = torch.zeros(L.metis_nvfp4_workspace_bytes(32, 128), dtype=torch.uint8, device="cuda")
+    rc = L.metis_nvfp4_quant_row(xd.data_ptr() + 64 * 2, 32, 128, 256, 0, codes.data_ptr(), scales.data_ptr(),
+                                 unit.data_ptr(), ws.data_ptr(), ws.numel(), None)
+    assert rc == 0
+    oc, os_, ou, _ = O.nvfp4_pack(view.float().contiguous())
+    torch.cuda.synchronize()
+    assert torch.equal(codes.cpu(), oc) and torch.equal(scales.cpu(), os_) and float(unit.cpu()) == float(ou)
+    # error codes straight from the C ABI
+    assert L.metis_nvfp4_quant_row(None, 1, 16, 16, 0, codes.data_ptr(), scales.data_ptr(), unit.data_ptr(),
+                                   ws.data_ptr(), ws.numel(), None) == _lib.E_ARG
+    assert L.metis_nvfp4_quant_row(xd.data_ptr(), 32, 128, 256, 0, codes.data_ptr(), scales.data_ptr(),
+                                   unit.data_ptr(), ws.data_ptr(), 16, None) == _lib.E_WORKSPACE
+    assert L.metis_nvfp4_quant_row(xd.data_ptr(), 32, 24, 256, 0, codes.data_ptr(), scales.data_ptr(),
+                                   unit.data_ptr(), ws.data_ptr(), ws.numel(), None) == _lib.E_SHAPE
+
+
+@pytest.mark.parametrize("tag,mode", MODES)
+def test_full_size_config1(ops, tag, mode):
+    """bf16 [8192, 4096], 0.1 % outlier channels: bit-exact against the C restatement, plus the
+    size-independent properties (idempotence of QDQ on its own output, odd symmetry)."""
+    from oracle import c_oracle as C
+    x = synthetic_activation(1001, 8192, 4096)
+    xd = x.cuda()
+    p = ops.quantize(xd, mode)
+    cc, cs, cu, _ = C.nvfp4_pack(x, mode)
+    _check_packed(p, cc, cs, cu, "config 1")
+    deq = ops.dequantize(p, torch.bfloat16)
+    ob, of = C.nvfp4_dequant(cc, cs, cu, mode)
+    assert same_bits(deq.cpu(), ob)
+    pn = ops.quantize(-xd, mode)
+    torch.cuda.synchronize()
+    assert torch.equal(pn.scales, p.scales) and torch.equal(pn.unit, p.unit)
+    nz = (xd != 0)
+    flip = torch.where(nz, 8, 0).to(torch.uint8)
+    flip = flip[:, 0::2] | (flip[:, 1::2] << 4)
+    assert torch.equal(pn.codes, p.codes ^ flip)
