@@ -184,16 +184,17 @@ int quantize(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, bo
              uint64_t seed, uint64_t offset, void* codes, void* scales, float* unit, void* workspace,
              size_t workspace_bytes, hipStream_t st)
 {
-    if (!x || !codes || !scales || !unit || rows < 0 || cols < 0 || ld < cols) return METIS_E_ARG;
+    if (rows < 0 || cols < 0 || ld < cols) return METIS_E_ARG;
     if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) return METIS_E_ARG;
     if ((col ? rows : cols) % kBlock) return METIS_E_SHAPE;
+    if (rows == 0 || cols == 0) return METIS_OK;              // nothing to read or write, unit untouched
+    if (!x || !codes || !scales || !unit) return METIS_E_ARG;
     if (rows * cols / kBlock >= (int64_t)1 << 31) return METIS_E_ARG;
     if (!col && ((ld % 8) || ((uintptr_t)x % 16))) return METIS_E_ARG;     // 16-byte vector loads
     if (((uintptr_t)codes % 8) || ((uintptr_t)scales % 4)) return METIS_E_ARG;
     Workspace ws;
     int rc = carve_workspace(workspace, workspace_bytes, rows, cols, &ws);
     if (rc != METIS_OK) return rc;
-    if (rows == 0 || cols == 0) return METIS_OK;
 #define METIS_Q(M, S, C) return launch_quant<M, S, C>(x, rows, cols, ld, noise, seed, offset, codes, scales, unit, ws, st)
     if (mode == 0) {
         if (!sr) { if (!col) METIS_Q(0, false, false); else METIS_Q(0, false, true); }
@@ -208,10 +209,12 @@ int quantize(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, bo
 int dequantize(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, int mode, void* out,
                int out_dtype, hipStream_t st)
 {
-    if (!codes || !scales || !unit || !out || rows < 0 || cols < 0) return METIS_E_ARG;
+    if (rows < 0 || cols < 0) return METIS_E_ARG;
     if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) return METIS_E_ARG;
     if (out_dtype != METIS_DTYPE_BF16 && out_dtype != METIS_DTYPE_F32) return METIS_E_ARG;
     if (cols % kBlock) return METIS_E_SHAPE;
+    if (rows == 0 || cols == 0) return METIS_OK;
+    if (!codes || !scales || !unit || !out) return METIS_E_ARG;
     if (((uintptr_t)codes % 4) || ((uintptr_t)out % 16)) return METIS_E_ARG;
     const int64_t noct = rows * cols / 8;
     if (noct == 0) return METIS_OK;

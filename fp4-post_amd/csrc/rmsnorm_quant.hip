@@ -77,9 +77,11 @@ __global__ __launch_bounds__(256) void rmsnorm_quant_kernel(const uint16_t* __re
 int rmsnorm_quantize(const void* x, const void* gamma, float eps, int64_t rows, int64_t cols, int mode, void* normed,
                      void* codes, void* scales, float* unit, void* workspace, size_t workspace_bytes, hipStream_t st)
 {
-    if (!x || !gamma || !codes || !scales || !unit || rows < 0 || cols < 0) return METIS_E_ARG;
+    if (rows < 0 || cols < 0) return METIS_E_ARG;
     if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) return METIS_E_ARG;
     if (cols % kBlock) return METIS_E_SHAPE;
+    if (rows == 0 || cols == 0) return METIS_OK;
+    if (!x || !gamma || !codes || !scales || !unit) return METIS_E_ARG;
     if (cols > 256 * kBlock * 4) return METIS_E_ARG;          // a row is held in registers: at most 16384 columns
     if (rows * cols / kBlock >= (int64_t)1 << 31) return METIS_E_ARG;
     if (((uintptr_t)x % 16) || ((uintptr_t)gamma % 16) || ((uintptr_t)codes % 8) || ((uintptr_t)scales % 4) ||
@@ -88,7 +90,6 @@ int rmsnorm_quantize(const void* x, const void* gamma, float eps, int64_t rows, 
     Workspace ws;
     int rc = carve_workspace(workspace, workspace_bytes, rows, cols, &ws);
     if (rc != METIS_OK) return rc;
-    if (rows == 0 || cols == 0) return METIS_OK;
     int64_t g = rows;
     const int64_t cap = (int64_t)device_cus() * 8;
     if (g > cap) g = cap;

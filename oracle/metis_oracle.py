@@ -214,8 +214,10 @@ def metis_forward(x: torch.Tensor, v: torch.Tensor, s: torch.Tensor, u: torch.Te
     y = ulinear(s * vlinear(x)) + warmup_linear(x)
       = ((x . v^T) * s) . u^T  +  QDQ(x) . QDQ(w_res)^T + bias
     x [M,K] bf16, v [r,K], s [r], u [N,r], w_res [N,K] (all bf16).
-    The low-rank branch runs in bf16 on the raw x (each matmul rounds to bf16); with
-    ``quantized_lowrank`` it consumes QDQ(x) and QDQ(v) as the current reference file does
+    Default (north-star) variant: the low-rank operands are bf16 -- t = bf16(bf16(x . v^T) * s) is
+    the stored rank-r activation -- and both branches are ACCUMULATED IN FP32 and summed before
+    the single rounding of the output to bf16.  With ``quantized_lowrank`` the rank-r branch
+    consumes QDQ(x) and QDQ(v) in dtype D as the current reference file does
     (bitlinear.py:752, 863-871).  The residual branch is computed in fp32 (p32) or bf16.
     Returns bf16 [M,N].
     """
@@ -230,8 +232,8 @@ def metis_forward(x: torch.Tensor, v: torch.Tensor, s: torch.Tensor, u: torch.Te
     else:
         t = torch.matmul(x, v.T)
         t = s * t
-        low = torch.matmul(t, u.T)
-    return (low.to(D) + res).to(torch.bfloat16)
+        low = torch.matmul(t.float(), u.float().T)
+    return (low.float() + res.float()).to(torch.bfloat16)
 
 
 def linear_backward(dyq: torch.Tensor, xq: torch.Tensor, wq: torch.Tensor):
