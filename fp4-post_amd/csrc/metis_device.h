@@ -47,17 +47,32 @@ template <int MODE> __device__ __forceinline__ float block_scalar(float amax)
     return rd<MODE>(rd<MODE>(div6(amax)) + 1e-9f);
 }
 
-// x / s correctly rounded, given rs = RN(1/s): product, then two exact-remainder corrections.
-// After the second correction the value before the final rounding is within 2^-69 of x/s,
-// far below the 2^-49 spacing that separates x/s from any rounding breakpoint when x has
-// 8 significant bits, so the result is RN(x/s).
-__device__ __forceinline__ float div_by(float x, float s, float rs)
+// x / s for a bf16-valued x (8 significant bits), given rs within 1 ulp of 1/s: product, exact
+// remainder, one correction.  Before its final rounding the value is within 2^-44 (relative) of
+// x/s, so the result is a faithful rounding of x/s and is RN(x/s) whenever x/s is exactly
+// representable (all exact ties).  It can differ from RN(x/s) only when x/s lies within 2^-44 of
+// a midpoint between two binary32 numbers; near an E2M1 decision threshold W (k/4, k in
+// {1,3,5,7,10,14,20}) that requires the low 20 bits of the significand of s to be a non-zero
+// value within 64 of 0 modulo 2^20 -- see near_threshold_hazard() -- because x - W*s is a multiple
+// of ulp(s)/4 while the half-ulp offset of the midpoint is s * 2^(E_W-24).
+__device__ __forceinline__ float div3(float x, float s, float rs)
 {
     float w = x * rs;
     float e = fmaf(-s, w, x);
-    w = fmaf(e, rs, w);
-    e = fmaf(-s, w, x);
     return fmaf(e, rs, w);
+}
+__device__ __forceinline__ bool near_threshold_hazard(float s)
+{
+    const uint32_t t = __float_as_uint(s) & 0xfffffu;
+    return (t != 0u) & (((t + 64u) & 0xfffffu) <= 128u);
+}
+
+// max(acc, |a|, |b|) in one instruction, without the NaN canonicalisation that fmaxf adds
+__device__ __forceinline__ float amax3(float acc, float a, float b)
+{
+    float r;
+    asm("v_max3_f32 %0, %1, |%2|, |%3|" : "=v"(r) : "v"(acc), "v"(a), "v"(b));
+    return r;
 }
 
 // float8_e4m3fn byte of a non-negative binary32 value (round to nearest even; > 464 -> 0x7F).

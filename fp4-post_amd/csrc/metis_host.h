@@ -10,15 +10,15 @@ namespace metis {
 
 // Caller-supplied scratch, carved as:
 //   [0, 16 KiB)        one partial maximum (uint32 bit pattern) per workgroup of phase 1
-//   [16 KiB, +256 B)   reserved for grid-wide synchronisation words (zero when idle)
-//   [16 KiB + 256, ..) one bf16 block maximum per block of 16
+//   [16 KiB, +65 KiB)  grid-wide reduction words of the single-launch quantizer (zero when idle)
+//   [81 KiB, ..)       one bf16 block maximum per block of 16
 struct Workspace {
     uint32_t* gmax;
     uint32_t* sync;
     uint16_t* amax;
 };
 constexpr size_t kWsGmaxBytes = 4096 * 4;
-constexpr size_t kWsSyncBytes = 256;
+constexpr size_t kWsSyncBytes = 260 * 256;     // 1 + 64 + 64 + 128 words of the grid reduction, 256 bytes apart
 
 inline size_t workspace_bytes(int64_t rows, int64_t cols)
 {

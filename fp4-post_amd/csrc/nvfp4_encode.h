@@ -26,9 +26,10 @@ __device__ __forceinline__ uint2 encode_literal(const float (&v)[kBlock], float 
 // Round-to-nearest, binary32 arithmetic.  The reference's compress/round/expand sequence equals
 // a round-to-nearest-even conversion of q = RN(|x|/h) onto the E2M1 grid for every binary32 q
 // except q = 5+1ulp, 7-1ulp and 10+1ulp (exhaustive host check), where its second rounding lands
-// on a tie.  The hardware FP4 converter does the RNE conversion two elements at a time; a block
-// whose scalar could produce one of the three exceptional quotients from a bf16 input takes
-// the literal path instead.
+// on a tie.  The hardware FP4 converter does the RNE conversion two elements at a time on the
+// quotient x/s from div3(); a block whose scalar could produce one of the three exceptional
+// quotients from a bf16 input, or for which div3() is not provably decisive at a threshold,
+// takes the literal path instead.
 __device__ __forceinline__ bool may_hit_exception(float s)
 {
     const float h = 0.5f * s;
@@ -45,21 +46,21 @@ __device__ __forceinline__ bool may_hit_exception(float s)
 
 __device__ __forceinline__ uint2 encode_rne_p32(const float (&v)[kBlock], float s)
 {
-    if (may_hit_exception(s)) {
+    if (may_hit_exception(s) || near_threshold_hazard(s)) {   // ~1e-4 of blocks
         const float none[kBlock] = {};
         return encode_literal<0, false>(v, s, none);
     }
-    const float rs = 1.0f / s;                                // correctly rounded
+    const float rs = __builtin_amdgcn_rcpf(s);                // 1 ulp
     uint32_t lo = 0u, hi = 0u;
     // code = E2M1(x / s): x/s = (|x| / (s/2)) / 2 exactly, sign carried by the quotient
-    lo = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(lo, div_by(v[0], s, rs), div_by(v[1], s, rs), 1.0f, 0);
-    lo = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(lo, div_by(v[2], s, rs), div_by(v[3], s, rs), 1.0f, 1);
-    lo = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(lo, div_by(v[4], s, rs), div_by(v[5], s, rs), 1.0f, 2);
-    lo = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(lo, div_by(v[6], s, rs), div_by(v[7], s, rs), 1.0f, 3);
-    hi = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(hi, div_by(v[8], s, rs), div_by(v[9], s, rs), 1.0f, 0);
-    hi = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(hi, div_by(v[10], s, rs), div_by(v[11], s, rs), 1.0f, 1);
-    hi = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(hi, div_by(v[12], s, rs), div_by(v[13], s, rs), 1.0f, 2);
-    hi = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(hi, div_by(v[14], s, rs), div_by(v[15], s, rs), 1.0f, 3);
+    lo = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(lo, div3(v[0], s, rs), div3(v[1], s, rs), 1.0f, 0);
+    lo = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(lo, div3(v[2], s, rs), div3(v[3], s, rs), 1.0f, 1);
+    lo = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(lo, div3(v[4], s, rs), div3(v[5], s, rs), 1.0f, 2);
+    lo = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(lo, div3(v[6], s, rs), div3(v[7], s, rs), 1.0f, 3);
+    hi = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(hi, div3(v[8], s, rs), div3(v[9], s, rs), 1.0f, 0);
+    hi = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(hi, div3(v[10], s, rs), div3(v[11], s, rs), 1.0f, 1);
+    hi = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(hi, div3(v[12], s, rs), div3(v[13], s, rs), 1.0f, 2);
+    hi = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(hi, div3(v[14], s, rs), div3(v[15], s, rs), 1.0f, 3);
     return make_uint2(lo, hi);
 }
 
@@ -74,8 +75,24 @@ __device__ __forceinline__ float block_amax(const float (&v)[kBlock])
 {
     float m = 0.0f;
 #pragma unroll
-    for (int j = 0; j < kBlock; j += 2) m = fmaxf(m, fmaxf(fabsf(v[j]), fabsf(v[j + 1])));
+    for (int j = 0; j < kBlock; j += 2) m = amax3(m, v[j], v[j + 1]);
     return m;
+}
+
+// maximum magnitude of the 16 packed bf16 values, computed on the bit patterns (two per dword)
+typedef unsigned short ushort2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float block_amax_packed(const uint4 a, const uint4 b)
+{
+    const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    ushort2_t m[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) m[j] = __builtin_bit_cast(ushort2_t, w[j] & 0x7fff7fffu);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) m[j] = __builtin_elementwise_max(m[j], m[j + 4]);
+    m[0] = __builtin_elementwise_max(__builtin_elementwise_max(m[0], m[1]), __builtin_elementwise_max(m[2], m[3]));
+    const uint32_t r = __builtin_bit_cast(uint32_t, m[0]);
+    const uint32_t hi = r >> 16, lo = r & 0xffffu;
+    return __uint_as_float((hi > lo ? hi : lo) << 16);
 }
 
 __device__ __forceinline__ void unpack16(const uint4 a, const uint4 b, float (&v)[kBlock])

@@ -12,6 +12,8 @@
 #include "metis_device.h"
 #include "metis_host.h"
 #include "nvfp4_encode.h"
+#include <stdio.h>
+#include <stdlib.h>
 
 namespace metis {
 
@@ -30,6 +32,33 @@ __global__ __launch_bounds__(256) void quant_codes_kernel(
     float gmax = 0.0f;
     const uint32_t nbpr = cols / kBlock;      // row layout: blocks per row
     const uint32_t nbc = rows / kBlock;       // column layout: blocks per column
+    if constexpr (!COL && !SR) {
+        // Round-to-nearest rows: software-pipelined, the next block's 32 bytes are in flight while the
+        // current block is encoded.
+        const uint32_t step = gridDim.x * 256u;
+        uint32_t i = blockIdx.x * 256u + threadIdx.x;
+        uint4 c0 = make_uint4(0u, 0u, 0u, 0u), c1 = c0;
+        auto src = [&](uint32_t blk) {
+            const uint32_t row = blk / nbpr, cb = blk - row * nbpr;
+            return reinterpret_cast<const uint4*>(x + (int64_t)row * ld + (int64_t)cb * kBlock);
+        };
+        if (i < nblocks) { const uint4* p = src(i); c0 = p[0]; c1 = p[1]; }
+        while (i < nblocks) {
+            const uint32_t nxt = i + step;
+            uint4 n0 = c0, n1 = c1;
+            if (nxt < nblocks) { const uint4* p = src(nxt); n0 = p[0]; n1 = p[1]; }
+            float v[kBlock];
+            const float none[kBlock] = {};
+            unpack16(c0, c1, v);
+            const float am = block_amax(v);
+            gmax = fmaxf(gmax, am);
+            ws_amax[i] = (uint16_t)(__float_as_uint(am) >> 16);
+            codes[i] = encode_block<MODE, false>(v, block_scalar<MODE>(am), none);
+            c0 = n0; c1 = n1; i = nxt;
+        }
+        publish_group_max(gmax, ws_gmax);
+        return;
+    }
     for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < nblocks; i += gridDim.x * 256u) {
         float v[kBlock], u[kBlock] = {};
         uint32_t ob;
@@ -78,6 +107,11 @@ __global__ __launch_bounds__(256) void quant_scales_kernel(const uint16_t* __res
                                                            uint32_t nblocks)
 {
     __shared__ float smax[4];
+    const uint32_t nquads = (nblocks + 3u) / 4u;
+    uint32_t q = blockIdx.x * 256u + threadIdx.x;
+    // first quad of parked maxima is requested before the reduction so that both round trips overlap
+    uint2 a = make_uint2(0u, 0u);
+    if (q < nquads && q * 4u + 4u <= nblocks) a = *reinterpret_cast<const uint2*>(ws_amax + q * 4u);
     float m = 0.0f;
     for (uint32_t g = threadIdx.x; g < ngroups; g += 256u) m = fmaxf(m, __uint_as_float(ws_gmax[g]));
     m = wave_max(m);
@@ -88,11 +122,10 @@ __global__ __launch_bounds__(256) void quant_scales_kernel(const uint16_t* __res
     const float unit = rd<MODE>(block_scalar<MODE>(amax) / 448.0f);
     if (blockIdx.x == 0 && threadIdx.x == 0) *unit_out = unit;
 
-    const uint32_t nquads = (nblocks + 3u) / 4u;
-    for (uint32_t q = blockIdx.x * 256u + threadIdx.x; q < nquads; q += gridDim.x * 256u) {
+    for (; q < nquads; q += gridDim.x * 256u) {
         const uint32_t base = q * 4u;
         if (base + 4u <= nblocks) {
-            const uint2 a = *reinterpret_cast<const uint2*>(ws_amax + base);
+            if (q >= gridDim.x * 256u) a = *reinterpret_cast<const uint2*>(ws_amax + base);
             const float t0 = rd<MODE>(block_scalar<MODE>(bf16_lo(a.x)) / unit);
             const float t1 = rd<MODE>(block_scalar<MODE>(bf16_hi(a.x)) / unit);
             const float t2 = rd<MODE>(block_scalar<MODE>(bf16_lo(a.y)) / unit);
@@ -106,6 +139,151 @@ __global__ __launch_bounds__(256) void quant_scales_kernel(const uint16_t* __res
                 scales[k] = (uint8_t)e4m3_byte(rd<MODE>(s / unit));
             }
         }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Single-launch variant for round-to-nearest row quantization: both phases in one cooperative
+// kernel.  Each thread keeps the maxima of its (at most NB) blocks in registers across a grid-wide
+// reduction, so neither the parked maxima nor a second launch are needed.
+//
+// Grid-wide maximum without a stall: workgroups ARRIVE as soon as their block maxima are known,
+// compute and store their codes while the reduction propagates, and only then WAIT for it.
+// Device-scope atomics to one address serialise at ~11 ns each on this part, so arrivals go
+// through a two-level tree: workgroup b uses group j = b % 64 (sub-counter, maximum slot and poll
+// flag of its own, 256 bytes apart), the last arriver of a group bumps the top counter, and the
+// last group folds the 64 maxima and publishes {generation + 1, maximum} to the 64 flags.
+// All traffic is relaxed device-scope atomics whose completion is waited for where order matters;
+// no cache write-back or invalidate is involved.  Counters are restored to zero and the slots of
+// the other generation parity are cleared on the way, so the words only need zero-filling once.
+// The wait is bounded: after kSpinLimit polls a workgroup raises the time-out word and carries
+// on, so every wave always exits.
+// ---------------------------------------------------------------------------------------------
+constexpr uint32_t kSpinLimit = 1u << 20;
+constexpr uint32_t kGroups = 64;
+// word offsets inside the synchronisation area (uint32 units; 64 words = 256 bytes apart)
+__device__ __forceinline__ uint32_t* sync_top(uint32_t* s) { return s; }
+__device__ __forceinline__ uint32_t* sync_timeout(uint32_t* s) { return s + 32; }
+__device__ __forceinline__ uint32_t* sync_sub(uint32_t* s, uint32_t j) { return s + 64u * (1u + j); }
+__device__ __forceinline__ uint64_t* sync_flag(uint32_t* s, uint32_t j) { return reinterpret_cast<uint64_t*>(s + 64u * (65u + j)); }
+__device__ __forceinline__ uint32_t* sync_slot(uint32_t* s, uint32_t parity, uint32_t j) { return s + 64u * (129u + parity * 64u + j); }
+
+#define METIS_AT_LOAD(p) __hip_atomic_load((p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+#define METIS_AT_STORE(p, v) __hip_atomic_store((p), (v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+#define METIS_AT_ADD(p, v) __hip_atomic_fetch_add((p), (v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+#define METIS_AT_MAX(p, v) __hip_atomic_fetch_max((p), (v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+#define METIS_AT_XCHG(p, v) __hip_atomic_exchange((p), (v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+
+struct GridMaxState {
+    float wave_part[4];
+    uint32_t gen;
+    float result;
+};
+
+// Called by every thread of every workgroup, once.  Publishes the workgroup maximum and arrives.
+__device__ __forceinline__ void grid_max_arrive(float thread_max, uint32_t* sync, GridMaxState& sh)
+{
+    float m = wave_max(thread_max);
+    if ((threadIdx.x & 63) == 0) sh.wave_part[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        const uint32_t lane = threadIdx.x;
+        const uint32_t j = blockIdx.x % kGroups;
+        const uint32_t ngroups = gridDim.x < kGroups ? gridDim.x : kGroups;
+        uint32_t gen = 0u, finalize = 0u;
+        if (lane == 0) {
+            gen = (uint32_t)METIS_AT_LOAD(sync_flag(sync, j));     // low word: generation left by the previous call
+            m = fmaxf(fmaxf(sh.wave_part[0], sh.wave_part[1]), fmaxf(sh.wave_part[2], sh.wave_part[3]));
+            uint32_t o = METIS_AT_MAX(sync_slot(sync, gen & 1u, j), __float_as_uint(m));
+            asm volatile("s_waitcnt vmcnt(0)" ::"v"(o) : "memory");   // maximum in place before arriving
+            const uint32_t members = (gridDim.x + kGroups - 1u - j) / kGroups;
+            o = METIS_AT_ADD(sync_sub(sync, j), 1u);
+            if (o == members - 1u) {
+                METIS_AT_STORE(sync_sub(sync, j), 0u);             // restored for the next call (ordered by kernel end)
+                o = METIS_AT_ADD(sync_top(sync), 1u);
+                if (o == ngroups - 1u) {
+                    METIS_AT_STORE(sync_top(sync), 0u);
+                    finalize = 1u;
+                }
+            }
+            sh.gen = gen;
+        }
+        gen = __builtin_amdgcn_readfirstlane(gen);
+        finalize = __builtin_amdgcn_readfirstlane(finalize);
+        if (finalize) {                                            // wave 0 of the very last arriver
+            uint32_t v = lane < ngroups ? METIS_AT_LOAD(sync_slot(sync, gen & 1u, lane)) : 0u;
+            v = __float_as_uint(wave_max(__uint_as_float(v)));
+            METIS_AT_STORE(sync_slot(sync, (gen + 1u) & 1u, lane), 0u);
+            METIS_AT_STORE(sync_flag(sync, lane), ((uint64_t)v << 32) | (uint64_t)(gen + 1u));
+        }
+    }
+}
+
+// Called by every thread after grid_max_arrive(); returns the tensor-wide maximum.
+__device__ __forceinline__ float grid_max_wait(uint32_t* sync, GridMaxState& sh)
+{
+    if (threadIdx.x == 0) {
+        const uint32_t j = blockIdx.x % kGroups;
+        const uint32_t want = sh.gen + 1u;
+        uint64_t f = METIS_AT_LOAD(sync_flag(sync, j));
+        uint32_t polls = 0;
+        while ((uint32_t)f != want) {
+            if (++polls > kSpinLimit) {
+                METIS_AT_STORE(sync_timeout(sync), 1u);
+                break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+            f = METIS_AT_LOAD(sync_flag(sync, j));
+        }
+        sh.result = __uint_as_float((uint32_t)(f >> 32));
+    }
+    __syncthreads();
+    return sh.result;
+}
+
+template <int MODE, int NB>
+__global__ __launch_bounds__(256) void quant_fused_kernel(const uint16_t* __restrict__ x, uint2* __restrict__ codes,
+                                                          uint8_t* __restrict__ scales, float* __restrict__ unit_out,
+                                                          uint32_t* __restrict__ sync, uint32_t nblocks,
+                                                          uint32_t dbg)
+{
+    __shared__ GridMaxState sh;
+    const uint32_t stride = gridDim.x * 256u;
+    const uint32_t i0 = blockIdx.x * 256u + threadIdx.x;
+    uint4 raw[NB][2];
+#pragma unroll
+    for (int k = 0; k < NB; ++k) {                            // all loads in flight first
+        const uint32_t i = i0 + k * stride;
+        if (i < nblocks) {
+            const uint4* p = reinterpret_cast<const uint4*>(x) + 2 * (size_t)i;
+            raw[k][0] = p[0];
+            raw[k][1] = p[1];
+        } else {
+            raw[k][0] = raw[k][1] = make_uint4(0u, 0u, 0u, 0u);
+        }
+    }
+    // phase A: codes of each block as its data arrives (memory and VALU work overlap), then arrive
+    float am[NB];
+    float gmax = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NB; ++k) {
+        const uint32_t i = i0 + k * stride;
+        float v[kBlock];
+        const float none[kBlock] = {};
+        unpack16(raw[k][0], raw[k][1], v);
+        am[k] = block_amax(v);
+        gmax = fmaxf(gmax, am[k]);
+        if (i < nblocks) codes[i] = (dbg & 4u) ? make_uint2(raw[k][0].x ^ raw[k][1].y, raw[k][0].z) : encode_block<MODE, false>(v, block_scalar<MODE>(am[k]), none);
+    }
+    if (!(dbg & 1u)) grid_max_arrive(gmax, sync, sh);
+    // phase C: tensor unit and scale bytes
+    const float amax = (dbg & 2u) ? 6.0f : grid_max_wait(sync, sh);
+    const float unit = rd<MODE>(block_scalar<MODE>(amax) / 448.0f);          // quant.py:21-22
+    if (i0 == 0) *unit_out = unit;
+#pragma unroll
+    for (int k = 0; k < NB; ++k) {
+        const uint32_t i = i0 + k * stride;
+        if (i < nblocks) scales[i] = (uint8_t)e4m3_byte(rd<MODE>(block_scalar<MODE>(am[k]) / unit));   // quant.py:23
     }
 }
 
@@ -169,6 +347,63 @@ int launch_scales(int mode, const Workspace& ws, uint32_t ngroups, void* scales,
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 
+// Co-resident workgroups of the fused kernel on the current device (0 = cooperative launch unavailable).
+template <int MODE, int NB>
+static int fused_capacity()
+{
+    static int cached[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    if (cached[dev] == 0) {
+        int coop = 0, per_cu = 0;
+        if (hipDeviceGetAttribute(&coop, hipDeviceAttributeCooperativeLaunch, dev) != hipSuccess || !coop) cached[dev] = -1;
+        else if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, quant_fused_kernel<MODE, NB>, 256, 0) != hipSuccess ||
+                 per_cu <= 0)
+            cached[dev] = -1;
+        else
+            cached[dev] = per_cu * device_cus();
+    }
+    return cached[dev] < 0 ? 0 : cached[dev];
+}
+
+template <int MODE, int NB>
+static int try_fused(const void* x, void* codes, void* scales, float* unit, const Workspace& ws, uint32_t nblocks,
+                     hipStream_t st)
+{
+    int cap = fused_capacity<MODE, NB>();
+    if (cap > kMaxGroups) cap = kMaxGroups;
+    const int64_t need = ((int64_t)nblocks + 256 * NB - 1) / (256 * NB);
+    if (getenv("METIS_DEBUG")) fprintf(stderr, "[metis] fused NB=%d cap=%d need=%ld\n", NB, cap, (long)need);
+    if (cap <= 0 || need > cap) return 1;                      // does not fit: caller picks another path
+    const uint16_t* xp = (const uint16_t*)x;
+    uint2* cp = (uint2*)codes;
+    uint8_t* sp = (uint8_t*)scales;
+    uint32_t* sy = ws.sync;
+    uint32_t dbg = getenv("METIS_DBG_FLAGS") ? (uint32_t)atoi(getenv("METIS_DBG_FLAGS")) : 0u;
+    void* args[] = {&xp, &cp, &sp, &unit, &sy, &nblocks, &dbg};
+    hipError_t e = getenv("METIS_COOP")
+                       ? hipLaunchCooperativeKernel((const void*)quant_fused_kernel<MODE, NB>, dim3((unsigned)need),
+                                                    dim3(256), args, 0, st)
+                       : hipLaunchKernel((const void*)quant_fused_kernel<MODE, NB>, dim3((unsigned)need), dim3(256), args, 0, st);
+    if (e != hipSuccess) {
+        if (getenv("METIS_DEBUG")) fprintf(stderr, "[metis] cooperative launch failed: %s\n", hipGetErrorString(e));
+        (void)hipGetLastError();
+        return 1;
+    }
+    return METIS_OK;
+}
+
+template <int MODE>
+static int launch_fused(const void* x, void* codes, void* scales, float* unit, const Workspace& ws, uint32_t nblocks,
+                        hipStream_t st)
+{
+    int rc = try_fused<MODE, 1>(x, codes, scales, unit, ws, nblocks, st);
+    if (rc == 1) rc = try_fused<MODE, 2>(x, codes, scales, unit, ws, nblocks, st);
+    if (rc == 1) rc = try_fused<MODE, 4>(x, codes, scales, unit, ws, nblocks, st);
+    if (rc == 1) rc = try_fused<MODE, 8>(x, codes, scales, unit, ws, nblocks, st);
+    return rc;
+}
+
 template <int MODE, bool SR, bool COL>
 static int launch_quant(const void* x, int64_t rows, int64_t cols, int64_t ld, const void* noise, uint64_t seed,
                         uint64_t offset, void* codes, void* scales, float* unit, const Workspace& ws, hipStream_t st)
@@ -195,6 +430,12 @@ int quantize(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, bo
     Workspace ws;
     int rc = carve_workspace(workspace, workspace_bytes, rows, cols, &ws);
     if (rc != METIS_OK) return rc;
+    if (!sr && !col && ld == cols && getenv("METIS_FUSED_QUANT")) {   // opt-in single-launch path; falls through when it does not fit
+        const uint32_t nblocks = (uint32_t)(rows * cols / kBlock);
+        rc = mode == 0 ? launch_fused<0>(x, codes, scales, unit, ws, nblocks, st)
+                       : launch_fused<1>(x, codes, scales, unit, ws, nblocks, st);
+        if (rc != 1) return rc;
+    }
 #define METIS_Q(M, S, C) return launch_quant<M, S, C>(x, rows, cols, ld, noise, seed, offset, codes, scales, unit, ws, st)
     if (mode == 0) {
         if (!sr) { if (!col) METIS_Q(0, false, false); else METIS_Q(0, false, true); }
