@@ -71,6 +71,23 @@ int metis_nvfp4_quant_sr_col(const void* x, int64_t rows, int64_t cols, int64_t 
                     workspace_bytes, (hipStream_t)stream);
 }
 
+int metis_nvfp4_get_scalar(const void* x, int64_t rows, int64_t cols, int mode, void* s, void* stream)
+{
+    return block_scalars(x, rows, cols, mode, s, (hipStream_t)stream);
+}
+
+int metis_nvfp4_quant_values(const void* x, const void* s, int64_t rows, int64_t cols, int mode, int sr, const void* noise,
+                             uint64_t seed, uint64_t offset, void* out, void* stream)
+{
+    return quant_values(x, s, rows, cols, mode, sr, noise, seed, offset, out, (hipStream_t)stream);
+}
+
+int metis_nvfp4_rquant(const void* xq, void* s, int64_t rows, int64_t cols, int mode, void* out, float* scratch,
+                       void* stream)
+{
+    return rquant_values(xq, s, rows, cols, mode, out, scratch, (hipStream_t)stream);
+}
+
 int metis_nvfp4_dequant(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, int mode,
                         void* out, int out_dtype, void* stream)
 {

@@ -15,6 +15,8 @@
 // The low-rank operands stay bf16 and use v_mfma_f32_32x32x16_bf16 on the same accumulators.
 #include "metis_device.h"
 #include "metis_host.h"
+#include <stdlib.h>
+#include <type_traits>
 
 namespace metis {
 
@@ -193,6 +195,277 @@ __global__ __launch_bounds__(256) void gemm_nvfp4_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Large-tile kernel: 256 x 256 per workgroup, 4 waves of 128 x 128 (16 MFMA tiles, 256 accumulator
+// registers per lane), K step 64, LDS double buffered (2 x 72 KiB) with one barrier per step.
+// Per step a thread owns one A row and one B row of the tile: it fetches their 32 bytes of codes
+// and 4 scale bytes into registers one step ahead, and expands them into the idle LDS buffer
+// while the MFMAs of the current buffer execute.  A wave reads (4 + 4) KiB of fragments per
+// 16 MFMAs, half the LDS traffic per flop of the 64 x 64 wave tile.
+//
+// Tile order: workgroup ids are dealt round-robin to the 8 XCDs by the hardware, so id -> (xcd,
+// slot) is undone first to give every XCD (and its private L2) one contiguous range of tiles,
+// which is then walked in groups of 4 tile-rows so that concurrently running workgroups share
+// A and B panels.
+// ---------------------------------------------------------------------------------------------
+constexpr int L_BM = 256, L_BN = 256, L_STRIDE = BK + LDS_PAD;
+constexpr int L_STAGE_HALVES = (L_BM + L_BN) * L_STRIDE;          // one buffer: A rows then B rows
+
+struct RowRegs {
+    uint4 c0, c1;      // 64 codes
+    uint32_t sc;       // 4 scale bytes
+};
+
+__device__ __forceinline__ void fetch_row(RowRegs& r, const uint8_t* codes, const uint8_t* scales, int64_t row, int kbytes,
+                                          int kblocks, int k0, int K)
+{
+    r.c0 = r.c1 = make_uint4(0u, 0u, 0u, 0u);
+    r.sc = 0u;
+    const uint8_t* cp = codes + row * kbytes + k0 / 2;
+    const uint8_t* sp = scales + row * kblocks + k0 / kBlock;
+    if (k0 + 64 <= K) {
+        r.c0 = reinterpret_cast<const uint4*>(cp)[0];
+        r.c1 = reinterpret_cast<const uint4*>(cp)[1];
+        r.sc = *reinterpret_cast<const uint32_t*>(sp);
+    } else if (k0 < K) {                                         // K % 64 == 32: half a step left
+        r.c0 = reinterpret_cast<const uint4*>(cp)[0];
+        r.sc = *reinterpret_cast<const uint16_t*>(sp);
+    }
+}
+
+__device__ __forceinline__ void expand_row(const RowRegs& r, uint16_t* dst)
+{
+    const half2_t s0 = scale_pair(r.sc & 0xffu), s1 = scale_pair((r.sc >> 8) & 0xffu);
+    const half2_t s2 = scale_pair((r.sc >> 16) & 0xffu), s3 = scale_pair(r.sc >> 24);
+    uint4* d = reinterpret_cast<uint4*>(dst);
+    d[0] = expand8(r.c0.x, s0); d[1] = expand8(r.c0.y, s0);
+    d[2] = expand8(r.c0.z, s1); d[3] = expand8(r.c0.w, s1);
+    d[4] = expand8(r.c1.x, s2); d[5] = expand8(r.c1.y, s2);
+    d[6] = expand8(r.c1.z, s3); d[7] = expand8(r.c1.w, s3);
+}
+
+// one expand8 of the 16 that make up a thread's two rows: q in 0..7 -> A row, 8..15 -> B row
+__device__ __forceinline__ void expand_piece(const RowRegs& ra, const RowRegs& rb, int q, uint16_t* da, uint16_t* db)
+{
+    const RowRegs& r = q < 8 ? ra : rb;
+    uint16_t* d = q < 8 ? da : db;
+    const int p = q & 7;
+    const uint32_t w = p == 0 ? r.c0.x : p == 1 ? r.c0.y : p == 2 ? r.c0.z : p == 3 ? r.c0.w
+                     : p == 4 ? r.c1.x : p == 5 ? r.c1.y : p == 6 ? r.c1.z : r.c1.w;
+    reinterpret_cast<uint4*>(d)[p] = expand8(w, scale_pair((r.sc >> (8 * (p >> 1))) & 0xffu));
+}
+
+// MFMA : VALU : LDS interleave requested from the scheduler for one K=16 sub-step
+template <int N_VALU_PER_MFMA, int N_DSR, int N_DSW>
+__device__ __forceinline__ void sched_substep()
+{
+#pragma unroll
+    for (int m = 0; m < 16; ++m) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                       // one MFMA
+        if (m < N_DSR) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);        // one LDS read
+        __builtin_amdgcn_sched_group_barrier(0x002, N_VALU_PER_MFMA, 0);         // VALU of the expansion
+        if (m % 3 == 2 && m / 3 < N_DSW) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);   // one LDS write
+    }
+}
+
+template <int OUT_F32, int DBG = 0>
+__global__ __launch_bounds__(256, 1) void gemm_nvfp4_large_kernel(
+    const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const float* __restrict__ a_unit,
+    const uint8_t* __restrict__ b_codes, const uint8_t* __restrict__ b_scales, const float* __restrict__ b_unit,
+    int M, int N, int K, const uint16_t* __restrict__ t, const uint16_t* __restrict__ u, int r,
+    const uint16_t* __restrict__ bias, void* __restrict__ out, int tiles_m, int tiles_n)
+{
+    extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+
+    // ---- tile assignment (XCD-contiguous, grouped)
+    const int total = tiles_m * tiles_n;
+    const int per_xcd = (total + 7) / 8;
+    const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (logical >= total) return;
+    constexpr int GM = 4;
+    const int group = logical / (GM * tiles_n);
+    const int first_m = group * GM;
+    const int gsize = min(tiles_m - first_m, GM);
+    const int tm = first_m + (logical % (GM * tiles_n)) % gsize;
+    const int tn = (logical % (GM * tiles_n)) / gsize;
+    const int m0 = tm * L_BM, n0 = tn * L_BN;
+
+    float16_t acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+    const int kbytes = K / 2, kblocks = K / kBlock;
+    const int64_t arow = min(m0 + tid, M - 1), brow = min(n0 + tid, N - 1);
+    uint16_t* const my_a = lds + tid * L_STRIDE;
+    uint16_t* const my_b = lds + (L_BM + tid) * L_STRIDE;
+    const uint8_t* const a_cp = a_codes + arow * kbytes;
+    const uint8_t* const a_sp = a_scales + arow * kblocks;
+    const uint8_t* const b_cp = b_codes + brow * kbytes;
+    const uint8_t* const b_sp = b_scales + brow * kblocks;
+    auto fetch = [&](RowRegs& ra, RowRegs& rb, int k0) {           // K % 64 == 0: always a full step
+        ra.c0 = reinterpret_cast<const uint4*>(a_cp + k0 / 2)[0];
+        ra.c1 = reinterpret_cast<const uint4*>(a_cp + k0 / 2)[1];
+        ra.sc = *reinterpret_cast<const uint32_t*>(a_sp + k0 / kBlock);
+        rb.c0 = reinterpret_cast<const uint4*>(b_cp + k0 / 2)[0];
+        rb.c1 = reinterpret_cast<const uint4*>(b_cp + k0 / 2)[1];
+        rb.sc = *reinterpret_cast<const uint32_t*>(b_sp + k0 / kBlock);
+    };
+
+    const int steps = K / BK;
+    // two register sets of packed rows: during step s the rows of step s+1 (r1) are expanded into the idle
+    // LDS buffer while the global loads of step s+2 land in r2 -- a full step of latency cover -- and
+    // r2 is moved into r1 at the end of the step
+    RowRegs ra1, rb1, ra2, rb2;
+    fetch(ra1, rb1, 0);
+    expand_row(ra1, my_a);
+    expand_row(rb1, my_b);
+    if (steps > 1) fetch(ra1, rb1, BK);
+    __syncthreads();
+
+    const int frag_off = (lane & 31) * L_STRIDE + (lane >> 5) * 8;
+    const int a_off = wm * 128 * L_STRIDE + frag_off;
+    const int b_off = (L_BM + wn * 128) * L_STRIDE + frag_off;
+    half8_t fa[2][4], fb[2][4];
+    auto load_frags = [&](int buf, const uint16_t* stage, int ks) {
+        if ((DBG & 4) && !(stage == lds && ks == 0 && buf == 0)) { if (buf != 0) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { fa[1][i] = fa[0][i]; fb[1][i] = fb[0][i]; } } return; }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) fa[buf][i] = *reinterpret_cast<const half8_t*>(stage + a_off + i * 32 * L_STRIDE + ks * 16);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) fb[buf][j] = *reinterpret_cast<const half8_t*>(stage + b_off + j * 32 * L_STRIDE + ks * 16);
+    };
+    auto mfma16 = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
+    };
+    // One K step.  EXPAND: rows of step s+1 (r1) are expanded into the idle LDS buffer during sub-steps
+    // 0..2; the barrier sits before sub-step 3, whose MFMAs cover the first fragment loads of step s+1.
+    // FETCH: global loads of step s+2 into r2, issued at the top so they have the whole step to arrive.
+    auto stage = [&](int s, auto do_expand, auto do_fetch) {
+        constexpr bool EXPAND = decltype(do_expand)::value && !(DBG & 1), FETCH = decltype(do_fetch)::value && !(DBG & 1);
+        const uint16_t* cur = lds + (s & 1) * L_STAGE_HALVES;
+        uint16_t* nxt = lds + ((s + 1) & 1) * L_STAGE_HALVES;
+        uint16_t* na = nxt + tid * L_STRIDE;
+        uint16_t* nb = nxt + (L_BM + tid) * L_STRIDE;
+        if (FETCH) fetch(ra2, rb2, (s + 2) * BK);
+        // sub-step 0
+        load_frags(1, cur, 1);
+        if (EXPAND) {
+#pragma unroll
+            for (int q = 0; q < 6; ++q) expand_piece(ra1, rb1, q, na, nb);
+        }
+        mfma16(0);
+        if (EXPAND) sched_substep<3, 8, 5>(); else sched_substep<0, 8, 0>();
+        // sub-step 1
+        load_frags(0, cur, 2);
+        if (EXPAND) {
+#pragma unroll
+            for (int q = 6; q < 11; ++q) expand_piece(ra1, rb1, q, na, nb);
+        }
+        mfma16(1);
+        if (EXPAND) sched_substep<3, 8, 5>(); else sched_substep<0, 8, 0>();
+        // sub-step 2
+        load_frags(1, cur, 3);
+        if (EXPAND) {
+#pragma unroll
+            for (int q = 11; q < 16; ++q) expand_piece(ra1, rb1, q, na, nb);
+        }
+        mfma16(0);
+        if (EXPAND) sched_substep<3, 8, 5>(); else sched_substep<0, 8, 0>();
+        if (!(DBG & 2)) __syncthreads();
+        // sub-step 3
+        if (EXPAND || (DBG & 1)) load_frags(0, nxt, 0);
+        mfma16(1);
+        sched_substep<0, 8, 0>();
+        if (FETCH) { ra1 = ra2; rb1 = rb2; }
+    };
+    using T_ = std::true_type;
+    using F_ = std::false_type;
+    load_frags(0, lds, 0);
+    int s = 0;
+    for (; s + 2 < steps; ++s) stage(s, T_{}, T_{});
+    if (s + 1 < steps) { stage(s, T_{}, F_{}); ++s; }
+    stage(s, F_{}, F_{});
+    __syncthreads();
+
+    // ---- tensor units (and the 2^8 * 2^8 of the scale placement)
+    const float us = (*a_unit) * (*b_unit) * 65536.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] *= us;
+
+    // ---- bf16 low-rank extension, 32 columns of T / U per step, staged in buffer 0
+    for (int j0 = 0; j0 < r; j0 += 32) {
+        {
+            const uint4* sa = reinterpret_cast<const uint4*>(t + arow * r + j0);
+            const uint4* sb = reinterpret_cast<const uint4*>(u + brow * r + j0);
+            uint4* da = reinterpret_cast<uint4*>(my_a);
+            uint4* db = reinterpret_cast<uint4*>(my_b);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) { da[q] = sa[q]; db[q] = sb[q]; }
+        }
+        __syncthreads();
+        const uint16_t* pa = lds + a_off;
+        const uint16_t* pb = lds + b_off;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            bf16x8_t fa[4], fb[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) fa[i] = *reinterpret_cast<const bf16x8_t*>(pa + i * 32 * L_STRIDE + ks * 16);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) fb[j] = *reinterpret_cast<const bf16x8_t*>(pb + j * 32 * L_STRIDE + ks * 16);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+
+    // ---- epilogue.  acc[i][j][e]: n = 8*(e/4) + 4*(lane/32) + e%4, m = lane%32 within the tile
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = m0 + wm * 128 + i * 32 + (lane & 31);
+        if (m >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int n = n0 + wn * 128 + j * 32 + 8 * g + 4 * (lane >> 5);
+                if (n >= N) continue;
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    v[e] = acc[i][j][4 * g + e];
+                    if (bias) v[e] += bf16_lo(bias[n + e]);
+                }
+                if (OUT_F32) {
+                    *reinterpret_cast<float4*>((float*)out + (int64_t)m * N + n) = make_float4(v[0], v[1], v[2], v[3]);
+                } else {
+                    uint2 w;
+                    w.x = bf16_bits(v[0]) | (bf16_bits(v[1]) << 16);
+                    w.y = bf16_bits(v[2]) | (bf16_bits(v[3]) << 16);
+                    *reinterpret_cast<uint2*>((uint16_t*)out + (int64_t)m * N + n) = w;
+                }
+            }
+        }
+    }
+}
+
 int gemm_nvfp4(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes, const void* b_scales,
                const float* b_unit, int64_t M, int64_t N, int64_t K, const void* t, const void* u, int64_t r,
                const void* bias, void* out, int out_dtype, hipStream_t st)
@@ -208,6 +481,36 @@ int gemm_nvfp4(const void* a_codes, const void* a_scales, const float* a_unit, c
         return METIS_E_ARG;
     if (K % 32) return METIS_E_ARG;                            // 16-byte code chunks: rows must stay 16-byte aligned
     if (M == 0 || N == 0) return METIS_OK;
+    if (M >= 256 && N >= 256 && K % BK == 0 && !getenv("METIS_GEMM_SMALL")) {
+        static bool attr_set[2] = {false, false};
+        const size_t lds_bytes = 2 * (size_t)L_STAGE_HALVES * sizeof(uint16_t);
+        const int f32 = out_dtype == METIS_DTYPE_F32;
+        const void* fn = f32 ? (const void*)gemm_nvfp4_large_kernel<1> : (const void*)gemm_nvfp4_large_kernel<0>;
+        if (const char* d = getenv("METIS_GEMM_DBG")) {
+            const int v = atoi(d);
+            fn = v == 1 ? (const void*)gemm_nvfp4_large_kernel<0, 1> : v == 3 ? (const void*)gemm_nvfp4_large_kernel<0, 3>
+               : v == 7 ? (const void*)gemm_nvfp4_large_kernel<0, 7> : v == 2 ? (const void*)gemm_nvfp4_large_kernel<0, 2> : fn;
+            (void)hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        }
+        if (!attr_set[f32]) {
+            if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
+                return METIS_E_DEVICE;
+            attr_set[f32] = true;
+        }
+        const int tiles_m = (int)((M + L_BM - 1) / L_BM), tiles_n = (int)((N + L_BN - 1) / L_BN);
+        const int total = tiles_m * tiles_n;
+        const unsigned grid_x = (unsigned)(((total + 7) / 8) * 8);
+        const uint8_t *ac = (const uint8_t*)a_codes, *as = (const uint8_t*)a_scales, *bc = (const uint8_t*)b_codes,
+                      *bs = (const uint8_t*)b_scales;
+        const uint16_t *tp = (const uint16_t*)t, *up = (const uint16_t*)u, *bp = (const uint16_t*)bias;
+        int Mi = (int)M, Ni = (int)N, Ki = (int)K, ri = (int)r, tmi = tiles_m, tni = tiles_n;
+        void* args[] = {&ac, &as, &a_unit, &bc, &bs, &b_unit, &Mi, &Ni, &Ki, &tp, &up, &ri, &bp, &out, &tmi, &tni};
+        if (hipLaunchKernel(fn, dim3(grid_x), dim3(256), args, lds_bytes, st) != hipSuccess) {
+            (void)hipGetLastError();
+            return METIS_E_LAUNCH;
+        }
+        return METIS_OK;
+    }
     constexpr int BM = 128, BN = 128;
     dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM));
     if (out_dtype == METIS_DTYPE_F32)

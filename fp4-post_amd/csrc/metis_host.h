@@ -48,6 +48,11 @@ int quantize(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, bo
              size_t workspace_bytes, hipStream_t st);
 int dequantize(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, int mode, void* out,
                int out_dtype, hipStream_t st);
+int block_scalars(const void* x, int64_t rows, int64_t cols, int mode, void* s, hipStream_t st);
+int quant_values(const void* x, const void* s, int64_t rows, int64_t cols, int mode, int sr, const void* noise,
+                 uint64_t seed, uint64_t offset, void* out, hipStream_t st);
+int rquant_values(const void* xq, void* s, int64_t rows, int64_t cols, int mode, void* out, float* scratch,
+                  hipStream_t st);
 int rmsnorm_quantize(const void* x, const void* gamma, float eps, int64_t rows, int64_t cols, int mode, void* normed,
                      void* codes, void* scales, float* unit, void* workspace, size_t workspace_bytes, hipStream_t st);
 int gemm_nvfp4(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes, const void* b_scales,

@@ -7,6 +7,11 @@ Compute goes through libmetis_hip.so (hand-written HIP kernels, C ABI in include
 """
 from . import ops
 from ._lib import MODE_P32, MODE_PB16, MetisHipError
+from .bitlinear import BitLinear, LinearLowbit, LinearLowbitFunction
 from .ops import PackedNVFP4
+from .patch import MetisArgs, replace_linear_with_metis, replace_model_with_metis
+from .quant import (BlockQuantFunc, Cast2Fp32, Cast2NVFp4e2m1Block, Cast2NVFp4e2m1BlockNOSR, QuantFunc, quant_func)
 
-__all__ = ["ops", "PackedNVFP4", "MODE_P32", "MODE_PB16", "MetisHipError"]
+__all__ = ["ops", "PackedNVFP4", "MODE_P32", "MODE_PB16", "MetisHipError", "quant_func", "QuantFunc", "BlockQuantFunc",
+           "Cast2Fp32", "Cast2NVFp4e2m1Block", "Cast2NVFp4e2m1BlockNOSR", "LinearLowbitFunction", "LinearLowbit",
+           "BitLinear", "MetisArgs", "replace_linear_with_metis", "replace_model_with_metis"]

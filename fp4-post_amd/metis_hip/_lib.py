@@ -27,6 +27,9 @@ SIGNATURES = {
     "metis_nvfp4_quant_col": (_i32, [_vp, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _sz, _vp]),
     "metis_nvfp4_quant_sr_row": (_i32, [_vp, _i64, _i64, _i64, _i32, _vp, _u64, _u64, _vp, _vp, _vp, _vp, _sz, _vp]),
     "metis_nvfp4_quant_sr_col": (_i32, [_vp, _i64, _i64, _i64, _i32, _vp, _u64, _u64, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "metis_nvfp4_get_scalar": (_i32, [_vp, _i64, _i64, _i32, _vp, _vp]),
+    "metis_nvfp4_quant_values": (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _vp, _u64, _u64, _vp, _vp]),
+    "metis_nvfp4_rquant": (_i32, [_vp, _vp, _i64, _i64, _i32, _vp, _vp, _vp]),
     "metis_nvfp4_dequant": (_i32, [_vp, _vp, _vp, _i64, _i64, _i32, _vp, _i32, _vp]),
     "metis_rmsnorm_nvfp4_quant": (_i32, [_vp, _vp, _f32, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "metis_linear_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _i32, _vp]),

@@ -1,0 +1,498 @@
+"""Metis low-bit linear modules with the reference's interface, computing on HIP kernels.
+
+Mirrors src/Metis/Metis/bitlinear.py: ``LinearLowbitFunction`` (autograd function with class-level
+configuration, 18-513), ``LinearLowbit`` (515-595) and ``BitLinear`` (597-940) keep their names,
+constructor arguments, attributes, state-dict keys and error behaviour, so model patching code written
+for the reference works unchanged.
+
+What differs underneath
+  * NVFP4 quantizers emit packed codes + E4M3 scale bytes (ops.PackedNVFP4) and the matmuls run as
+    block-scaled MFMA GEMMs on the packed operands; nothing is dequantized to HBM on the hot path.
+  * BitLinear.forward evaluates both branches in one kernel:
+        y = ((x V^T) * s) U^T + deq(Q(x)) deq(Q(W_res))^T + b        (fp32 accumulate)
+    with the rank-r branch on the raw activations in bf16 (as bitlinear_new.py:376-388,473-488 does);
+    the reference's current file feeds the quantized activation and a quantized V to that branch
+    (bitlinear.py:752, 863-879).
+  * Backward re-quantizes dY and X with stochastic rounding along the contraction dimension of each
+    GEMM (tokens for wgrad), which a block-scaled GEMM needs; the reference quantizes dY along its last
+    dimension only and reuses the forward X^ (bitlinear.py:488-508).
+Quantizer classes other than the kernel-backed NVFP4 pair (e.g. Cast2Fp32 or user subclasses) take a
+generic path that follows the reference line by line with torch matmuls.
+"""
+from __future__ import annotations
+
+import math
+import weakref
+
+import torch
+import torch.nn as nn
+import torch.nn.init as init
+
+from . import ops
+from .ops import PackedNVFP4
+from .quant import (Cast2Fp32, Cast2NVFp4e2m1Block, Cast2NVFp4e2m1BlockNOSR, QuantFunc, is_hip_nvfp4, quant_func)
+
+__all__ = ["LinearLowbitFunction", "LinearLowbit", "BitLinear"]
+
+
+def _flat2d(x: torch.Tensor) -> torch.Tensor:
+    return x.reshape(-1, x.shape[-1])
+
+
+def _packable(x: torch.Tensor, q) -> bool:
+    """Fast path available: kernel-backed quantizer, device tensor, shapes the GEMM accepts."""
+    return is_hip_nvfp4(q) and x.is_cuda and x.shape[-1] % 32 == 0 and x.dtype in (torch.float32, torch.bfloat16)
+
+
+class LinearLowbitFunction(torch.autograd.Function):
+    """Low-bit GEMM with quantized activations / weights / gradients (reference 18-513).
+
+    Class attributes are configured by BitLinear.__init__ exactly as in the reference; they are
+    process-wide mutable state there too (last constructed layer wins).
+    """
+    q_forward_input = Cast2NVFp4e2m1BlockNOSR
+    q_forward_weight = Cast2NVFp4e2m1BlockNOSR
+    q_backward_input = Cast2NVFp4e2m1Block
+    q_backward_weight = Cast2NVFp4e2m1Block
+    q_backward_outputgrad = Cast2NVFp4e2m1Block
+
+    enable_nv_recipe = False
+    hadamard_workspace_mb = 128
+    hadamard_tile_size = 16
+    hadamard_backend = "auto"
+
+    activation_lowrank_niter = 0
+    backward_lowrank_niter = 0
+    enable_activation_svd = False
+    activation_lowrank_svd = -1
+    enable_backward_svd = False
+    backward_lowrank_svd = -1
+    activation_broadcast_dim = -1
+    backward_broadcast_dim = -1
+
+    tp_simulate = False
+    tp_parts = 4
+
+    compute_dtype = torch.float32
+    metis_mode = "mean"
+    mean_cache = None
+    mean_cache_key = "default"
+
+    # ------------------------------------------------------------------ activation paths
+    @staticmethod
+    def svd_quant(input_, quant_func, rank=60, niter=0, broadcast_dim=-1, tp_simulate=False, tp_parts=4,
+                  metis_mode="mean", mean_cache=None, cache_key="default"):
+        """Mean-residual activation quantization (reference 311-336, 363-366).
+
+        Column mean over tokens is kept in high precision, the centred residual goes through the
+        quantizer's fused QDQ, and the mean is added back; during single-token decode a weighted
+        running mean per cache key is used.  The "svd" mode and the TP simulation of the reference
+        are not part of this build.
+        """
+        if tp_simulate or metis_mode != "mean":
+            if metis_mode not in ("mean", "svd"):
+                raise ValueError(f"Unsupported metis_mode: {metis_mode}")
+            raise NotImplementedError("only metis_mode='mean' without TP simulation is implemented")
+        shape = input_.shape
+        flat = _flat2d(input_)
+        seq_len = shape[1] if len(shape) == 3 else shape[0]
+        if seq_len == 1 and mean_cache is not None and cache_key in mean_cache:
+            cached_mean, cached_count = mean_cache[cache_key]
+            new_count = cached_count + flat.shape[0]
+            this_mean = flat.mean(dim=0, keepdim=True)
+            me = (cached_mean * cached_count + this_mean * flat.shape[0]) / new_count
+            mean_cache[cache_key] = (me.detach(), new_count)
+        else:
+            me = flat.mean(dim=0, keepdim=True)
+            if mean_cache is not None:
+                mean_cache[cache_key] = (me.detach(), flat.shape[0])
+        res = quant_func.quantize_dequantize(flat - me)
+        out = me + res
+        return out.view(shape) if len(shape) == 3 else out
+
+    @staticmethod
+    def quantize_input(input_: torch.Tensor, mean_cache: dict = None, cache_key: str = "default") -> torch.Tensor:
+        """Dequantized activation, as the reference returns it (371-393)."""
+        F = LinearLowbitFunction
+        input_ = input_.to(F.compute_dtype)
+        if F.enable_activation_svd:
+            return F.svd_quant(input_, quant_func=F.q_forward_input, rank=F.activation_lowrank_svd,
+                               niter=F.activation_lowrank_niter, broadcast_dim=F.activation_broadcast_dim,
+                               tp_simulate=F.tp_simulate, tp_parts=F.tp_parts, metis_mode=F.metis_mode,
+                               mean_cache=mean_cache, cache_key=cache_key)
+        return F.q_forward_input.quantize_dequantize(input_)
+
+    @staticmethod
+    def _prepare_input(input_: torch.Tensor, mean_cache=None, cache_key="default"):
+        """Packed activation when the direct NVFP4 path applies, else the dequantized tensor."""
+        F = LinearLowbitFunction
+        xin = input_.to(F.compute_dtype)
+        if not F.enable_activation_svd and not F.enable_nv_recipe and _packable(xin, F.q_forward_input):
+            return F.q_forward_input.pack(_flat2d(xin))
+        return F.quantize_input(input_, mean_cache=mean_cache, cache_key=cache_key)
+
+    @staticmethod
+    def _quantize_wgrad_operand(value: torch.Tensor, quantizer) -> torch.Tensor:
+        """Three-call QDQ of one backward operand (reference 395-405); the Hadamard pre-rotation of
+        the NV recipe is not part of this build."""
+        if LinearLowbitFunction.enable_nv_recipe:
+            raise NotImplementedError("enable_nv_recipe (random Hadamard rotation) is not implemented")
+        scalar = quantizer.get_scalar(value)
+        value = quantizer.quant(value, scalar)
+        return quantizer.rquant(value, scalar)
+
+    # ------------------------------------------------------------------ autograd
+    @staticmethod
+    def forward(ctx, input_, weight, bias, quantized_weight, quantized_input):
+        F = LinearLowbitFunction
+        if quantized_input is None:
+            quantized_input = F._prepare_input(input_, mean_cache=F.mean_cache, cache_key=F.mean_cache_key)
+        lead = input_.shape[:-1]
+        ctx.lead = lead
+        ctx.has_bias = bias is not None
+        ctx.packed = isinstance(quantized_input, PackedNVFP4) and isinstance(quantized_weight, PackedNVFP4)
+        if ctx.packed:
+            ctx.pw = quantized_weight
+            ctx.weight_ref = weight
+            ctx.save_for_backward(input_, bias if bias is not None else input_.new_empty(0))
+            out_dtype = torch.float32 if F.compute_dtype == torch.float32 else torch.bfloat16
+            out = ops.linear_fwd(quantized_input, quantized_weight, bias=bias, out_dtype=out_dtype)
+            return out.reshape(*lead, quantized_weight.rows).to(F.compute_dtype)
+        if isinstance(quantized_input, PackedNVFP4):
+            quantized_input = quantized_input.dequantize(F.compute_dtype).reshape(input_.shape)
+        if isinstance(quantized_weight, PackedNVFP4):
+            quantized_weight = quantized_weight.dequantize(F.compute_dtype)
+        ctx.save_for_backward(quantized_input, quantized_weight, bias if bias is not None else input_.new_empty(0))
+        output = torch.matmul(quantized_input, quantized_weight.T)
+        if bias is not None:
+            output = output + bias
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        F = LinearLowbitFunction
+        grad_output = grad_output.to(F.compute_dtype)
+        grad_bias = None
+        if ctx.has_bias:
+            grad_bias = _flat2d(grad_output).sum(dim=0).to(torch.float32)
+        dy2 = _flat2d(grad_output)
+        if ctx.packed:
+            input_, _ = ctx.saved_tensors
+            x2 = _flat2d(input_.to(F.compute_dtype))
+            L, N = dy2.shape
+            qg, qi = F.q_backward_outputgrad, F.q_backward_input
+            if L % 16 == 0 and L % 32 == 0 and is_hip_nvfp4(qg) and is_hip_nvfp4(qi) and N % 32 == 0:
+                # dgrad: contraction over N; wgrad: contraction over tokens
+                p_dy = qg.pack(dy2)
+                pw_col = F.q_forward_weight.pack(ctx.weight_ref.to(F.compute_dtype), col=True)
+                gx = ops.linear_dgrad(p_dy, pw_col, out_dtype=grad_output.dtype if grad_output.dtype != torch.float16 else torch.float32)
+                gw = ops.linear_wgrad(qg.pack(dy2, col=True), qi.pack(x2, col=True))
+                return gx.reshape(*ctx.lead, gx.shape[-1]).to(grad_output.dtype), gw, grad_bias, None, None
+            xq = F.q_forward_input.quantize_dequantize(x2)
+            wq = ctx.pw.dequantize(F.compute_dtype)
+        else:
+            xq, wq, _ = ctx.saved_tensors
+            xq = _flat2d(xq)
+        if F.enable_backward_svd:
+            dyq = F.svd_quant(grad_output, quant_func=F.q_backward_outputgrad, rank=F.backward_lowrank_svd,
+                              niter=F.backward_lowrank_niter, broadcast_dim=F.backward_broadcast_dim,
+                              tp_simulate=F.tp_simulate, tp_parts=F.tp_parts, metis_mode=F.metis_mode)
+            dyq = _flat2d(dyq)
+        else:
+            dyq = _flat2d(F._quantize_wgrad_operand(dy2, F.q_backward_outputgrad))
+        grad_weight = torch.matmul(dyq.T, xq).to(torch.float32)            # reference 502-510
+        grad_input = torch.matmul(dyq, wq).reshape(*ctx.lead, wq.shape[-1])  # reference 507-508
+        return grad_input, grad_weight, grad_bias, None, None
+
+
+class LinearLowbit(nn.Module):
+    """nn.Linear replacement whose matmul runs on quantized operands (reference 515-595)."""
+
+    def __init__(self, in_features: int, out_features: int, bias=True, args=None, device=None,
+                 storage_dtype=torch.float32, compute_dtype=torch.float32) -> None:
+        super().__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        self.storage_dtype = storage_dtype
+        self.compute_dtype = compute_dtype
+        self.cache_quantized_weight = getattr(args, "cache_quantized_weight", False)
+        self._quantized_weight_cache = None
+        dev = getattr(args, "device", None) if device is None else device
+        self.weight = nn.Parameter(torch.empty((out_features, in_features), dtype=storage_dtype, device=dev))
+        if bias:
+            self.bias = nn.Parameter(torch.empty((out_features,), dtype=storage_dtype, device=dev))
+        else:
+            self.bias = None
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        init.kaiming_uniform_(self.weight, a=math.sqrt(5))
+        if self.bias is not None:
+            fan_in, _ = init._calculate_fan_in_and_fan_out(self.weight)
+            bound = 1 / math.sqrt(fan_in) if fan_in > 0 else 0
+            init.uniform_(self.bias, -bound, bound)
+
+    def forward(self, input, quantized_input=None):
+        weight_compute = self.weight.to(self.compute_dtype)
+        bias_compute = self.bias.to(self.compute_dtype) if self.bias is not None else None
+        quantized_weight = self._get_quantized_weight(weight_compute)
+        return LinearLowbitFunction.apply(input, weight_compute, bias_compute, quantized_weight, quantized_input)
+
+    @torch.no_grad()
+    def _get_quantized_weight(self, weight_compute):
+        """Quantized weight, cached on Parameter._version when enabled (reference 563-589).  Returns a
+        PackedNVFP4 when the kernel path applies, otherwise the dequantized tensor."""
+        F = LinearLowbitFunction
+        key = (self.weight._version, weight_compute.device, weight_compute.dtype, F.q_forward_weight, F.enable_nv_recipe)
+        if self.cache_quantized_weight and self._quantized_weight_cache is not None:
+            cached_key, cached = self._quantized_weight_cache
+            if cached_key == key:
+                return cached
+        if F.enable_nv_recipe:
+            raise NotImplementedError("enable_nv_recipe (random Hadamard rotation) is not implemented")
+        if _packable(weight_compute, F.q_forward_weight) and weight_compute.shape[0] % 4 == 0:
+            q = F.q_forward_weight.pack(weight_compute)
+        else:
+            q = F.q_forward_weight.quantize_dequantize(weight_compute)
+        if self.cache_quantized_weight:
+            self._quantized_weight_cache = (key, q)
+        return q
+
+    def _apply(self, fn, recurse=True):
+        self._quantized_weight_cache = None
+        return super()._apply(fn, recurse=recurse)
+
+
+class _MetisFusedFunction(torch.autograd.Function):
+    """y = ((x V^T) * s) U^T + deq(Q(x)) deq(Q(R))^T + b in one GEMM launch, with its gradients."""
+
+    @staticmethod
+    def forward(ctx, x, v, s, u, res, bias, px, p_res):
+        F = LinearLowbitFunction
+        cd = torch.bfloat16
+        x2 = _flat2d(x).to(cd)
+        xv = torch.matmul(x2, v.to(cd).T)                      # [L, r] rank-r projection (library GEMM, bf16)
+        t = xv * s.to(cd)
+        out_dtype = torch.float32 if F.compute_dtype == torch.float32 else torch.bfloat16
+        y = ops.linear_fwd(px, p_res, t=t, u=u.to(cd), bias=None if bias is None else bias.to(cd), out_dtype=out_dtype)
+        ctx.save_for_backward(x, v, s, u, res, xv)
+        ctx.has_bias = bias is not None
+        ctx.lead = x.shape[:-1]
+        return y.reshape(*ctx.lead, y.shape[-1]).to(F.compute_dtype)
+
+    @staticmethod
+    def backward(ctx, dy):
+        F = LinearLowbitFunction
+        x, v, s, u, res, xv = ctx.saved_tensors
+        cd = torch.bfloat16
+        dy2 = _flat2d(dy).to(cd)
+        x2 = _flat2d(x).to(cd)
+        L, N = dy2.shape
+        # rank-r branch in bf16
+        g_t = torch.matmul(dy2, u.to(cd))                      # [L, r]
+        g_u = torch.matmul(dy2.T, xv * s.to(cd))               # [N, r]
+        g_s = (g_t.float() * xv.float()).sum(dim=0)
+        g_xv = g_t * s.to(cd)
+        g_v = torch.matmul(g_xv.T, x2)                         # [r, K]
+        gx = torch.matmul(g_xv, v.to(cd))                      # [L, K]
+        # residual branch on re-quantized operands
+        qg, qi = F.q_backward_outputgrad, F.q_backward_input
+        if L % 32 == 0 and N % 32 == 0 and is_hip_nvfp4(qg) and is_hip_nvfp4(qi):
+            gx = gx + ops.linear_dgrad(qg.pack(dy2.to(F.compute_dtype)),
+                                       F.q_forward_weight.pack(res.to(F.compute_dtype), col=True), out_dtype=cd)
+            g_res = ops.linear_wgrad(qg.pack(dy2.to(F.compute_dtype), col=True), qi.pack(x2.to(F.compute_dtype), col=True))
+        else:
+            dyq = F._quantize_wgrad_operand(dy2.to(F.compute_dtype), qg)
+            xq = F.q_forward_input.quantize_dequantize(x2.to(F.compute_dtype))
+            wq = F.q_forward_weight.quantize_dequantize(res.to(F.compute_dtype))
+            gx = gx + torch.matmul(dyq, wq).to(cd)
+            g_res = torch.matmul(dyq.T, xq).to(torch.float32)
+        g_b = dy2.float().sum(dim=0) if ctx.has_bias else None
+        return (gx.reshape(x.shape).to(x.dtype), g_v.to(v.dtype), g_s.to(s.dtype), g_u.to(u.dtype),
+                g_res.to(torch.float32), g_b, None, None)
+
+
+class BitLinear(nn.Module):
+    """Drop-in for nn.Linear: W = U diag(s) V + W_res with the residual in NVFP4 (reference 597-940)."""
+    rollout_merge_active = False
+
+    def __init__(self, in_features, out_features, args=None, bias=True, dtype=torch.float32, compute_dtype=None):
+        super().__init__()
+        self.storage_dtype = dtype
+        self.compute_dtype = compute_dtype if compute_dtype is not None else dtype
+        if self.compute_dtype not in [torch.float32, torch.float16, torch.bfloat16]:
+            raise ValueError(f"Unsupported compute_dtype: {self.compute_dtype}")
+        if getattr(args, "enable_te", False):
+            raise NotImplementedError("transformer_engine layers are not part of this build")
+        if args.enable_forward_svd is False and args.enable_lowbit is True:
+            self.warmup_linear = LinearLowbit(in_features, out_features, bias=bias, args=args,
+                                              storage_dtype=self.storage_dtype, compute_dtype=self.compute_dtype)
+        else:
+            self.warmup_linear = nn.Linear(in_features, out_features, bias=bias, device=args.device, dtype=self.storage_dtype)
+        self.ulinear = None
+        self.vlinear = None
+        self.s = None
+
+        F = LinearLowbitFunction
+        F.q_forward_input = quant_func[args.q_forward_input]
+        F.q_forward_weight = quant_func[args.q_forward_weight]
+        F.q_backward_input = quant_func[args.q_backward_input]
+        F.q_backward_weight = quant_func[args.q_backward_weight]
+        F.q_backward_outputgrad = quant_func[args.q_backward_outputgrad]
+        F.enable_backward_svd = args.enable_backward_svd
+        F.backward_lowrank_svd = args.backward_lowrank_svd
+        F.backward_lowrank_niter = args.backward_lowrank_niter
+        F.enable_activation_svd = args.enable_activation_svd
+        F.activation_lowrank_svd = args.activation_lowrank_svd
+        F.activation_lowrank_niter = args.activation_lowrank_niter
+        F.activation_broadcast_dim = args.activation_broadcast_dim
+        F.backward_broadcast_dim = args.backward_broadcast_dim
+        F.enable_nv_recipe = args.enable_nv_recipe
+        F.hadamard_workspace_mb = getattr(args, "hadamard_workspace_mb", 128)
+        F.hadamard_tile_size = getattr(args, "hadamard_tile_size", 16)
+        F.hadamard_backend = getattr(args, "hadamard_backend", "auto")
+        F.tp_simulation = args.tp_simulation          # the reference writes this name and reads tp_simulate
+        F.tp_parts = args.tp_parts
+        F.compute_dtype = self.compute_dtype
+        F.metis_mode = args.metis_mode
+
+        self.args = args
+        self.is_svd_quant = False
+        if args.forward_svd_warmup_steps <= 0 and args.enable_forward_svd:
+            self.split()
+        self.mean_cache = {}
+        self.activation_group = None
+        self._merged_rollout_weight_cache = None
+        self.layer_name = ""
+
+    # ------------------------------------------------------------------ shared activation (reference 676-702)
+    def _get_shared_quantized_input(self, x: torch.Tensor):
+        F = LinearLowbitFunction
+        group = getattr(self, "activation_group", None)
+        if group is None:
+            return F._prepare_input(x, mean_cache=self.mean_cache, cache_key=f"{self.layer_name}.shared")
+        input_ref = group.get("input_ref")
+        if input_ref is not None and input_ref() is x:
+            return group["quantized_input"]
+        quantized_input = F._prepare_input(x, mean_cache=group["mean_cache"], cache_key=f"{group['name']}.shared")
+
+        def clear_cached_input(ref):
+            if group.get("input_ref") is ref:
+                group["input_ref"] = None
+                group["quantized_input"] = None
+
+        group["input_ref"] = weakref.ref(x, clear_cached_input)
+        group["quantized_input"] = quantized_input
+        return quantized_input
+
+    @torch.no_grad()
+    def _get_merged_rollout_weight(self, dtype: torch.dtype) -> torch.Tensor:
+        """(U diag s) Q(V) + Q(W_res), cached on the parameters' versions (reference 704-730)."""
+        F = LinearLowbitFunction
+        key = (self.vlinear.weight._version, self.ulinear.weight._version, self.s._version,
+               self.warmup_linear.weight._version, self.vlinear.weight.device, dtype, F.q_forward_weight, F.enable_nv_recipe)
+        if self._merged_rollout_weight_cache is not None:
+            cached_key, cached = self._merged_rollout_weight_cache
+            if cached_key == key:
+                return cached
+
+        def deq(q):
+            return q.dequantize(dtype) if isinstance(q, PackedNVFP4) else q
+
+        v_weight = deq(self.vlinear._get_quantized_weight(self.vlinear.weight.to(dtype)))
+        residual = deq(self.warmup_linear._get_quantized_weight(self.warmup_linear.weight.to(dtype)))
+        merged = (self.ulinear.weight.to(dtype) * self.s.to(dtype).unsqueeze(0)) @ v_weight + residual
+        self._merged_rollout_weight_cache = (key, merged)
+        return merged
+
+    def _apply(self, fn, recurse=True):
+        self._merged_rollout_weight_cache = None
+        return super()._apply(fn, recurse=recurse)
+
+    # ------------------------------------------------------------------ forward (reference 736-769)
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        F = LinearLowbitFunction
+        F.mean_cache = self.mean_cache
+        if not self.is_svd_quant:
+            return self.warmup_linear(x)
+        share_activation = (isinstance(self.vlinear, LinearLowbit) and isinstance(self.warmup_linear, LinearLowbit)
+                            and self.args.forward_svd_rank > 0)
+        if share_activation:
+            shared_input = self._get_shared_quantized_input(x)
+            r = self.args.forward_svd_rank
+            if isinstance(shared_input, PackedNVFP4) and r % 32 == 0 and self.ulinear.bias is None:
+                # one fused launch for both branches; it already is the "merged" evaluation, so the
+                # rollout switch changes nothing on this path
+                p_res = self.warmup_linear._get_quantized_weight(self.warmup_linear.weight.to(self.compute_dtype))
+                if isinstance(p_res, PackedNVFP4):
+                    return _MetisFusedFunction.apply(x, self.vlinear.weight, self.s, self.ulinear.weight,
+                                                     self.warmup_linear.weight, self.warmup_linear.bias, shared_input, p_res)
+            if BitLinear.rollout_merge_active and not torch.is_grad_enabled():
+                if isinstance(shared_input, PackedNVFP4):
+                    shared_input = shared_input.dequantize(F.compute_dtype).reshape(x.shape)
+                merged = self._get_merged_rollout_weight(shared_input.dtype)
+                y = torch.matmul(shared_input, merged.T)
+                if self.warmup_linear.bias is not None:
+                    y = y + self.warmup_linear.bias.to(y.dtype)
+                return y
+            y = self.vlinear(x, quantized_input=shared_input)
+        else:
+            F.mean_cache_key = f"{self.layer_name}.vlinear"
+            y = self.vlinear(x)
+        y = torch.mul(self.s, y)
+        y = self.ulinear(y.to(self.ulinear.weight.dtype))
+        if self.args.forward_svd_rank > 0:
+            if share_activation:
+                y = y + self.warmup_linear(x, quantized_input=shared_input)
+            else:
+                F.mean_cache_key = f"{self.layer_name}.warmup"
+                y = y + self.warmup_linear(x)
+        return y
+
+    # ------------------------------------------------------------------ factorisation (reference 776-924)
+    @torch.no_grad()
+    def split(self):
+        if not self.args.enable_forward_svd:
+            return
+        if self.vlinear is not None:
+            raise NotImplementedError("re-splitting an already factorised layer is not part of this build")
+        if not self.args.enable_lowbit:
+            raise NotImplementedError("enable_lowbit=False is not part of this build")
+        w = self.warmup_linear.weight
+        device, original_dtype = w.device, w.dtype
+        u, s, v = torch.linalg.svd(w.to(torch.float32), full_matrices=False)
+        u, s, v = u.to(original_dtype), s.to(original_dtype), v.to(original_dtype)
+        bias = self.warmup_linear.bias
+        rank = self.args.forward_svd_rank
+        out_f, in_f = w.shape
+        if rank > 0:
+            residual = LinearLowbit(in_f, out_f, bias=bias is not None, args=self.args, device=device,
+                                    storage_dtype=original_dtype, compute_dtype=self.compute_dtype)
+            if bias is not None:
+                residual.bias.copy_(bias)
+            residual.weight.copy_(w - u[:, :rank] @ torch.diag(s[:rank]) @ v[:rank])
+            self.warmup_linear = residual
+            self.vlinear = LinearLowbit(in_f, rank, bias=False, args=self.args, device=device,
+                                        storage_dtype=original_dtype, compute_dtype=self.compute_dtype)
+            self.ulinear = nn.Linear(rank, out_f, bias=False, device=device, dtype=original_dtype)
+            self.vlinear.weight.copy_(v[:rank, :])
+            self.ulinear.weight.copy_(u[:, :rank])
+            self.s = nn.Parameter(s[:rank].clone())
+        else:
+            self.vlinear = LinearLowbit(in_f, v.shape[0], bias=False, args=self.args, device=device,
+                                        storage_dtype=original_dtype, compute_dtype=self.compute_dtype)
+            self.ulinear = nn.Linear(u.shape[1], out_f, bias=False, device=device, dtype=original_dtype)
+            self.vlinear.weight.copy_(v)
+            self.ulinear.weight.copy_(u)
+            self.s = nn.Parameter(s.clone())
+            self.warmup_linear = None
+        self.is_svd_quant = True
+
+    @torch.no_grad()
+    def lowrank_initialization(self, rank: int = 32):
+        """Replace the weight by its best rank-r approximation (reference 926-940)."""
+        W = self.warmup_linear.weight
+        out_features, in_features = W.shape
+        r = max(1, min(int(rank), min(out_features, in_features)))
+        U, S, Vh = torch.linalg.svd(W.detach().to(torch.float32), full_matrices=False)
+        W.copy_(((U[:, :r] * S[:r]) @ Vh[:r, :]).to(dtype=W.dtype, device=W.device))

@@ -1,0 +1,180 @@
+"""Quantizer registry with the reference's interface (src/Metis/Metis/quant.py:69-92, 180-195, 661-673).
+
+    quant_func[name] -> class with classmethods get_scalar(x), quant(x, s), rquant(x, s),
+                        quantize_dequantize(x)   (all under torch.no_grad)
+
+NVFP4 classes run on the HIP kernels of libmetis_hip.so and reproduce the reference's CPU arithmetic
+bit for bit in the dtype of the tensor they are given: float32 tensors use binary32 arithmetic,
+bfloat16 tensors the bf16-per-op arithmetic.  They need a ROCm device tensor; there is no CPU path.
+Formats the hot path does not use (MXFP4, FP6, FP8, 1.58-bit) are not provided.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import ops
+from ._lib import MODE_P32, MODE_PB16, MetisHipError, check, load
+
+BLOCK = 16
+
+
+def _mode_of(x: torch.Tensor) -> int:
+    if x.dtype == torch.float32:
+        return MODE_P32
+    if x.dtype == torch.bfloat16:
+        return MODE_PB16
+    raise ValueError(f"NVFP4 quantizers support float32 and bfloat16 tensors, got {x.dtype}")
+
+
+def _need_gpu(x: torch.Tensor):
+    if not x.is_cuda:
+        raise MetisHipError("NVFP4 quantizers run on the HIP kernels only: pass a ROCm device tensor")
+
+
+class QuantFunc:
+    """Per-tensor identity-scale quantizer base (quant.py:69-92)."""
+    compile_quantize_dequantize = False   # accepted for compatibility; there is nothing to compile here
+
+    @classmethod
+    @torch.no_grad()
+    def quantize_dequantize(cls, x: torch.Tensor):
+        scalar = cls.get_scalar(x)
+        return cls.rquant(cls.quant(x, scalar), scalar)
+
+    @classmethod
+    @torch.no_grad()
+    def get_scalar(cls, x: torch.Tensor):
+        return x.abs().max() + 1e-6
+
+    @classmethod
+    @torch.no_grad()
+    def quant(cls, x: torch.Tensor, s: torch.Tensor):
+        return x / s
+
+    @classmethod
+    @torch.no_grad()
+    def rquant(cls, x: torch.Tensor, s: torch.Tensor):
+        return x * s
+
+
+class Cast2Fp32(QuantFunc):
+    """Identity quantizer (quant.py:177-178), used by tests as a spy base class."""
+
+
+class BlockQuantFunc(QuantFunc):
+    block_shape = (1, BLOCK)
+
+    @classmethod
+    def _check(cls, x: torch.Tensor):
+        rows = x.numel() // max(x.shape[-1], 1)
+        cols = x.shape[-1]
+        if rows % cls.block_shape[0] != 0 or cols % cls.block_shape[1] != 0:
+            raise ValueError(f"NVFP4 block shape {cls.block_shape} does not divide tensor shape {tuple(x.shape)}")
+
+
+class _NVFP4Base(BlockQuantFunc):
+    stochastic = False
+    # seed / running offset of the Philox stream used by stochastic rounding (class-level like the
+    # reference's use of the global torch generator); offset advances by the element count per call
+    sr_seed = 0x5EED
+    sr_offset = 0
+
+    @classmethod
+    def _next_offset(cls, numel: int) -> int:
+        off = _NVFP4Base.sr_offset
+        _NVFP4Base.sr_offset = off + (numel + 3) // 4
+        return off
+
+    @classmethod
+    @torch.no_grad()
+    def pack(cls, x: torch.Tensor, col: bool = False, noise: torch.Tensor | None = None) -> ops.PackedNVFP4:
+        """Packed NVFP4 (codes, E4M3 scale bytes, unit) of x in the arithmetic of x's dtype."""
+        _need_gpu(x)
+        if not col:
+            cls._check(x)
+        mode = _mode_of(x)
+        if cls.stochastic:
+            return ops.quantize(x, mode, col=col, sr=True, noise=noise, seed=_NVFP4Base.sr_seed,
+                                offset=cls._next_offset(x.numel()) if noise is None else 0)
+        return ops.quantize(x, mode, col=col)
+
+    @classmethod
+    @torch.no_grad()
+    def quantize_dequantize(cls, x: torch.Tensor):
+        """Fused QDQ (quant.py:6-36 / 392-433): same shape and dtype as x."""
+        cls._check(x)
+        p = cls.pack(x)
+        return ops.dequantize(p, x.dtype).reshape(x.shape)
+
+    @classmethod
+    @torch.no_grad()
+    def get_scalar(cls, x: torch.Tensor):
+        """[R, C/16] raw block scalars amax/6 + 1e-9 (quant.py:435-455)."""
+        _need_gpu(x)
+        cols = x.shape[-1]
+        x2 = x.reshape(-1, cols).contiguous()
+        rows = x2.shape[0]
+        assert rows % cls.block_shape[0] == 0 and cols % cls.block_shape[1] == 0
+        s = torch.empty(rows, cols // BLOCK, dtype=x.dtype, device=x.device)
+        rc = load().metis_nvfp4_get_scalar(x2.data_ptr(), rows, cols, _mode_of(x), s.data_ptr(), ops._stream())
+        check(rc, "metis_nvfp4_get_scalar", x.shape)
+        return s
+
+    @classmethod
+    @torch.no_grad()
+    def quant(cls, x: torch.Tensor, s: torch.Tensor, noise: torch.Tensor | None = None):
+        """E2M1 values of x / s in x's dtype (quant.py:459-466)."""
+        _need_gpu(x)
+        cols = x.shape[-1]
+        x2 = x.reshape(-1, cols).contiguous()
+        rows = x2.shape[0]
+        s2 = s.reshape(rows, cols // BLOCK).to(x.dtype).contiguous()
+        out = torch.empty_like(x2)
+        nz = None if noise is None else noise.reshape(rows, cols).to(x.dtype).contiguous()
+        off = cls._next_offset(x2.numel()) if (cls.stochastic and nz is None) else 0
+        rc = load().metis_nvfp4_quant_values(x2.data_ptr(), s2.data_ptr(), rows, cols, _mode_of(x), int(cls.stochastic),
+                                             None if nz is None else nz.data_ptr(), _NVFP4Base.sr_seed, off,
+                                             out.data_ptr(), ops._stream())
+        check(rc, "metis_nvfp4_quant_values", x.shape)
+        return out.reshape(x.shape)
+
+    @classmethod
+    @torch.no_grad()
+    def rquant(cls, x: torch.Tensor, s: torch.Tensor):
+        """x * e4m3_roundtrip(s / (max s / 448)) * (max s / 448); divides ``s`` in place as the
+        reference does (quant.py:470-548)."""
+        _need_gpu(x)
+        cols = x.shape[-1]
+        x2 = x.reshape(-1, cols).contiguous()
+        rows = x2.shape[0]
+        if not (s.is_contiguous() and s.dtype == x.dtype):
+            raise ValueError("rquant: the scalar tensor must be contiguous and of the dtype of x")
+        out = torch.empty_like(x2)
+        scratch = torch.empty(1, dtype=torch.float32, device=x.device)
+        rc = load().metis_nvfp4_rquant(x2.data_ptr(), s.data_ptr(), rows, cols, _mode_of(x), out.data_ptr(),
+                                       scratch.data_ptr(), ops._stream())
+        check(rc, "metis_nvfp4_rquant", x.shape)
+        return out.reshape(x.shape)
+
+
+class Cast2NVFp4e2m1BlockNOSR(_NVFP4Base):
+    """NVFP4, round to nearest (quant.py:390-548); registry key "nvfp4e2m1bnosr"."""
+    stochastic = False
+
+
+class Cast2NVFp4e2m1Block(_NVFP4Base):
+    """NVFP4, stochastic rounding (quant.py:273-388); registry key "nvfp4e2m1b"."""
+    stochastic = True
+
+
+quant_func = {
+    "nvfp4e2m1b": Cast2NVFp4e2m1Block,
+    "nvfp4e2m1bnosr": Cast2NVFp4e2m1BlockNOSR,
+    "fp32": Cast2Fp32,
+}
+
+
+def is_hip_nvfp4(q) -> bool:
+    """True when ``q`` is one of the kernel-backed NVFP4 classes themselves (not a user subclass
+    that overrides the arithmetic)."""
+    return q is Cast2NVFp4e2m1BlockNOSR or q is Cast2NVFp4e2m1Block

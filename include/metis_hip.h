@@ -110,6 +110,22 @@ int metis_nvfp4_quant_sr_col(const void *x, int64_t rows, int64_t cols, int64_t 
                              void *stream);
 
 /*
+ * The reference's three-call form on dequantized tensors of dtype D (float32 in METIS_MODE_P32, bf16 in
+ * METIS_MODE_PB16), for callers that use the quantizer classes directly.  All tensors contiguous [rows, cols].
+ *   metis_nvfp4_get_scalar : Cast2NVFp4e2m1Block[NOSR].get_scalar (src/Metis/Metis/quant.py:435-455)
+ *                            s [rows, cols/16] = amax|x| / 6 + 1e-9
+ *   metis_nvfp4_quant_values : .quant (quant.py:459-466; element rule 118-128, or 137-147 when sr != 0)
+ *                            out [rows, cols] in {0, +-0.5, ..., +-6} (+-8 possible under sr, as in the reference)
+ *   metis_nvfp4_rquant     : .rquant (quant.py:470-548): s is DIVIDED IN PLACE by max|s|/448 as the reference
+ *                            does; out = xq * (e4m3_roundtrip(s) * max|s|/448).  scratch: float[1] on the device.
+ */
+int metis_nvfp4_get_scalar(const void *x, int64_t rows, int64_t cols, int mode, void *s, void *stream);
+int metis_nvfp4_quant_values(const void *x, const void *s, int64_t rows, int64_t cols, int mode, int sr,
+                             const void *noise, uint64_t seed, uint64_t offset, void *out, void *stream);
+int metis_nvfp4_rquant(const void *xq, void *s, int64_t rows, int64_t cols, int mode, void *out, float *scratch,
+                       void *stream);
+
+/*
  * Dequantize packed NVFP4: the last three multiplications of the reference,
  * out = ((v * sign) / 2) * (e4m3 * unit)  (src/Metis/Metis/quant.py:23-24, 32-35; rquant 470-548).
  *   out    [rows, cols] of out_dtype (METIS_DTYPE_BF16 or METIS_DTYPE_F32); in METIS_MODE_P32 a

@@ -1,0 +1,259 @@
+"""GPU tests of the drop-in Python surface: registry classes against the reference's golden vectors
+(bit-exact), LinearLowbit / BitLinear forward against the oracle (<= 2e-3 relative Frobenius, P32),
+backward wiring, and patching of a Hugging Face Qwen2 decoder layer."""
+import pytest
+import torch
+
+from helpers import rel_fro, same_bits, synthetic_activation, t
+
+pytestmark = pytest.mark.gpu
+
+TOL = 2e-3
+
+
+@pytest.fixture(autouse=True)
+def _config():
+    from metis_hip import BitLinear, LinearLowbitFunction as F, quant_func
+    F.q_forward_input = quant_func["nvfp4e2m1bnosr"]
+    F.q_forward_weight = quant_func["nvfp4e2m1bnosr"]
+    F.q_backward_input = quant_func["nvfp4e2m1b"]
+    F.q_backward_weight = quant_func["nvfp4e2m1b"]
+    F.q_backward_outputgrad = quant_func["nvfp4e2m1b"]
+    F.enable_activation_svd = False
+    F.enable_backward_svd = False
+    F.enable_nv_recipe = False
+    F.compute_dtype = torch.float32
+    yield
+    BitLinear.rollout_merge_active = False
+
+
+@pytest.mark.parametrize("tag", ["p32", "pb16"])
+def test_three_call_and_fused_against_reference_golden(golden, tag):
+    from metis_hip import quant_func
+    q = quant_func["nvfp4e2m1bnosr"]
+    xb = t(golden["rne_x"])
+    x = (xb.float() if tag == "p32" else xb).cuda()
+    s = q.get_scalar(x)
+    assert same_bits(s.cpu(), t(golden[f"rne_scalar_{tag}"]))
+    xq = q.quant(x, s)
+    assert same_bits(xq.cpu(), t(golden[f"rne_quant_{tag}"]))
+    s_arg = s.clone()
+    out = q.rquant(xq, s_arg)
+    assert same_bits(out.cpu(), t(golden[f"rne_rquant_{tag}"]))
+    assert same_bits(s_arg.cpu(), t(golden[f"rne_scalar_after_rquant_{tag}"]))      # in-place side effect
+    fused = q.quantize_dequantize(x)
+    assert same_bits(fused.cpu(), t(golden[f"rne_qdq_{tag}"])) and same_bits(fused.cpu(), out.cpu())
+    x3 = t(golden["rne3d_x"])
+    x3 = (x3.float() if tag == "p32" else x3).cuda()
+    assert same_bits(q.quantize_dequantize(x3).cpu(), t(golden[f"rne3d_qdq_{tag}"]))
+
+
+@pytest.mark.parametrize("tag", ["p32", "pb16"])
+def test_stochastic_three_call_against_reference_golden(golden, tag):
+    from metis_hip import quant_func
+    q = quant_func["nvfp4e2m1b"]
+    xb = t(golden["sr_x"])
+    x = (xb.float() if tag == "p32" else xb).cuda()
+    u = t(golden[f"sr_noise_{tag}"]).cuda()
+    s = q.get_scalar(x)
+    xq = q.quant(x, s, noise=u)
+    assert same_bits(xq.cpu(), t(golden[f"sr_quant_{tag}"]))                        # incl. the off-grid +-8
+    assert same_bits(q.rquant(xq, s.clone()).cpu(), t(golden[f"sr_rquant_{tag}"]))
+
+
+def test_linear_lowbit_forward_backward_against_reference_golden(golden):
+    """LinearLowbit (fp32 compute) on the reference's own input: forward within tolerance of its
+    output; backward with the generic three-call path and the reference's recorded noise is exact
+    up to the GEMM's summation order."""
+    from types import SimpleNamespace
+    from metis_hip import LinearLowbit, LinearLowbitFunction as F, quant_func
+    x, w, b, dy = (t(golden[k]) for k in ("lin_x", "lin_w", "lin_b", "lin_dy"))
+    args = SimpleNamespace(device="cuda", cache_quantized_weight=False)
+    layer = LinearLowbit(64, 48, bias=True, args=args)
+    with torch.no_grad():
+        layer.weight.copy_(w)
+        layer.bias.copy_(b)
+    xr = x.cuda().requires_grad_(True)
+    y = layer(xr)
+    assert y.shape == (2, 16, 48) and y.dtype == torch.float32
+    assert rel_fro(y.detach().cpu(), t(golden["lin_y"])) <= 1e-5
+    y.backward(dy.cuda())
+    # packed backward uses its own stochastic stream and token-blocked operands: FP4-noise level agreement
+    assert rel_fro(xr.grad.cpu(), t(golden["lin_gx"])) < 0.2
+    assert rel_fro(layer.weight.grad.cpu(), t(golden["lin_gw"])) < 0.35
+    assert same_bits(layer.bias.grad.cpu(), t(golden["lin_gb"]))
+    assert layer.weight.grad.dtype == torch.float32
+    # reference-style backward: dY through the three-call SR quantizer with the reference's noise
+    q = quant_func["nvfp4e2m1b"]
+    dyd = dy.cuda()
+    s = q.get_scalar(dyd)
+    dyq = q.rquant(q.quant(dyd, s, noise=t(golden["lin_noise_dy"]).cuda()), s).reshape(-1, 48)
+    xq = quant_func["nvfp4e2m1bnosr"].quantize_dequantize(x.cuda()).reshape(-1, 64)
+    wq = quant_func["nvfp4e2m1bnosr"].quantize_dequantize(w.cuda())
+    assert rel_fro((dyq.T @ xq).cpu(), t(golden["lin_gw"])) <= 1e-5
+    assert rel_fro((dyq @ wq).reshape(2, 16, 64).cpu(), t(golden["lin_gx"])) <= 1e-5
+
+
+def _make_bitlinear(K, N, r, bias, dtype, compute_dtype, seed=0):
+    from metis_hip import BitLinear, MetisArgs
+    g = torch.Generator().manual_seed(seed)
+    w = torch.randn(N, K, generator=g) * 0.02
+    a = torch.linalg.qr(torch.randn(N, 8, generator=g))[0]
+    b = torch.linalg.qr(torch.randn(K, 8, generator=g))[0]
+    w = w + (a * 3.0) @ b.T
+    args = MetisArgs.direct_fp4(forward_svd_rank=r)
+    layer = BitLinear(K, N, args=args, bias=bias, dtype=dtype, compute_dtype=compute_dtype).cuda()
+    with torch.no_grad():
+        layer.warmup_linear.weight.copy_(w)
+        if bias:
+            layer.warmup_linear.bias.copy_(torch.randn(N, generator=g) * 0.1)
+    layer.split()
+    return layer, w
+
+
+@pytest.mark.parametrize("bias", [False, True])
+def test_bitlinear_fused_forward_against_oracle(bias):
+    """P32 (compute_dtype=float32, the reference's default): <= 2e-3, bf16 vs bf16."""
+    from oracle import metis_oracle as O
+    K, N, r, L = 256, 192, 32, 128
+    layer, w = _make_bitlinear(K, N, r, bias, torch.bfloat16, torch.float32)
+    assert layer.is_svd_quant and layer.vlinear.weight.shape == (r, K)
+    x = synthetic_activation(50, L, K).reshape(2, L // 2, K)
+    y = layer(x.cuda())
+    assert y.shape == (2, L // 2, N) and y.dtype == torch.float32
+    want = O.metis_forward(x.reshape(L, K), layer.vlinear.weight.detach().cpu(), layer.s.detach().cpu(),
+                           layer.ulinear.weight.detach().cpu(), layer.warmup_linear.weight.detach().cpu(),
+                           None if not bias else layer.warmup_linear.bias.detach().cpu(), p32=True)
+    assert rel_fro(y.detach().cpu().reshape(L, N).bfloat16(), want) <= TOL
+    # and close to the unquantized layer it replaces (FP4 noise on the residual only)
+    dense = x.reshape(L, K).float() @ w.T
+    if bias:
+        dense = dense + layer.warmup_linear.bias.detach().cpu().float()
+    assert rel_fro(y.detach().cpu().reshape(L, N).float(), dense) < 0.05
+
+
+def test_bitlinear_fused_forward_bf16_compute():
+    """compute_dtype=bfloat16: operands are packed with the bf16-per-op arithmetic (bit-exact codes,
+    see test_gpu_quant); the GEMM keeps exact products and fp32 accumulation, so against the
+    reference's all-bf16 matmuls only FP4-level agreement is asserted (no 2e-3 claim in this mode)."""
+    from oracle import metis_oracle as O
+    K, N, r, L = 256, 192, 32, 128
+    layer, w = _make_bitlinear(K, N, r, True, torch.bfloat16, torch.bfloat16)
+    x = synthetic_activation(50, L, K).reshape(2, L // 2, K)
+    y = layer(x.cuda())
+    assert y.dtype == torch.bfloat16
+    want = O.metis_forward(x.reshape(L, K), layer.vlinear.weight.detach().cpu(), layer.s.detach().cpu(),
+                           layer.ulinear.weight.detach().cpu(), layer.warmup_linear.weight.detach().cpu(),
+                           layer.warmup_linear.bias.detach().cpu(), p32=False)
+    assert rel_fro(y.detach().cpu().reshape(L, N), want) < 2e-2
+
+
+def test_bitlinear_backward_reaches_every_parameter_and_matches_dense_gradients():
+    K, N, r, L = 256, 192, 32, 128
+    layer, w = _make_bitlinear(K, N, r, True, torch.bfloat16, torch.bfloat16, seed=3)
+    x = synthetic_activation(51, L, K).reshape(2, L // 2, K).cuda().requires_grad_(True)
+    g = torch.Generator().manual_seed(4)
+    dy = (torch.randn(2, L // 2, N, generator=g) * 1e-2).bfloat16().cuda()
+    layer(x).backward(dy)
+    for p in (layer.vlinear.weight, layer.ulinear.weight, layer.s, layer.warmup_linear.weight, layer.warmup_linear.bias):
+        assert p.grad is not None and bool(torch.isfinite(p.grad).all())
+    # dense reference gradients of y = x W^T + b
+    gx_dense = dy.reshape(L, N).float().cpu() @ w
+    assert rel_fro(x.grad.reshape(L, K).float().cpu(), gx_dense) < 0.1
+    gw_dense = dy.reshape(L, N).float().cpu().T @ x.detach().reshape(L, K).float().cpu()
+    assert rel_fro(layer.warmup_linear.weight.grad.float().cpu(), gw_dense) < 0.3      # both operands in FP4 with SR
+    assert rel_fro(layer.ulinear.weight.grad.float().cpu(),
+                   gw_dense @ (layer.vlinear.weight.detach().float().cpu().T * layer.s.detach().float().cpu())) < 0.05
+    torch.testing.assert_close(layer.warmup_linear.bias.grad.float().cpu(), dy.reshape(L, N).float().sum(0).cpu(),
+                               rtol=2e-2, atol=1e-3)
+
+
+def test_shared_activation_is_quantized_once_per_group():
+    from metis_hip import LinearLowbitFunction as F, quant_func
+    calls = {"n": 0}
+    base = quant_func["nvfp4e2m1bnosr"]
+    orig = base.pack.__func__
+
+    def counting(cls, x, col=False, noise=None):
+        if not col and tuple(x.shape) == (96, 256):      # the activation, not the [N, 256] weights
+            calls["n"] += 1
+        return orig(cls, x, col, noise)
+
+    base.pack = classmethod(counting)
+    try:
+        q, _ = _make_bitlinear(256, 128, 32, False, torch.bfloat16, torch.bfloat16, seed=5)
+        k, _ = _make_bitlinear(256, 64, 32, False, torch.bfloat16, torch.bfloat16, seed=6)
+        group = {"name": "l0.qkv", "mean_cache": {}, "input_ref": None, "quantized_input": None}
+        q.activation_group = k.activation_group = group
+        calls["n"] = 0
+        x = synthetic_activation(52, 96, 256).cuda()
+        q(x), k(x)
+        assert calls["n"] == 1                       # one activation quantization for the group
+        q(synthetic_activation(53, 96, 256).cuda())
+        assert calls["n"] == 2
+    finally:
+        base.pack = classmethod(orig)
+
+
+def test_rollout_switch_on_the_fused_path_and_merged_weight_helper():
+    """The fused launch already evaluates both branches at once, so the rollout switch leaves the
+    output unchanged; the merged-weight helper keeps the reference's definition
+    (U diag s) Q(V) + Q(W_res) and its cache semantics (reference 704-730)."""
+    from metis_hip import BitLinear
+    layer, _ = _make_bitlinear(256, 128, 32, True, torch.bfloat16, torch.float32, seed=7)
+    x = synthetic_activation(54, 64, 256).float().cuda()
+    with torch.no_grad():
+        BitLinear.rollout_merge_active = False
+        expected = layer(x)
+        BitLinear.rollout_merge_active = True
+        actual = layer(x)
+        first = layer._get_merged_rollout_weight(torch.float32)
+        second = layer._get_merged_rollout_weight(torch.float32)
+        from metis_hip import quant_func
+        q = quant_func["nvfp4e2m1bnosr"]
+        want = (layer.ulinear.weight.float() * layer.s.float()) @ q.quantize_dequantize(layer.vlinear.weight.float()) \
+            + q.quantize_dequantize(layer.warmup_linear.weight.float())
+        layer.s.add_(0.1)
+        updated = layer._get_merged_rollout_weight(torch.float32)
+    assert torch.equal(actual, expected)
+    assert first is second and updated is not first
+    assert rel_fro(first.cpu(), want.cpu()) < 1e-6
+
+
+def test_patch_qwen2_decoder_layer():
+    """A randomly initialised Hugging Face Qwen2 decoder layer with every projection replaced."""
+    transformers = pytest.importorskip("transformers")
+    from transformers.models.qwen2.modeling_qwen2 import Qwen2Config, Qwen2DecoderLayer, Qwen2RotaryEmbedding
+    from metis_hip import BitLinear, MetisArgs, replace_model_with_metis
+    torch.manual_seed(0)
+    cfg = Qwen2Config(hidden_size=256, intermediate_size=512, num_attention_heads=4, num_key_value_heads=2,
+                      num_hidden_layers=1, vocab_size=128, max_position_embeddings=256)
+    cfg._attn_implementation = "eager"
+    layer = Qwen2DecoderLayer(cfg, layer_idx=0).to(torch.bfloat16).cuda()
+    for p in layer.parameters():
+        if p.dim() == 2:
+            torch.nn.init.normal_(p, std=0.02)
+    holder = torch.nn.ModuleDict({"layer": layer})
+    x = torch.randn(2, 64, 256, device="cuda", dtype=torch.bfloat16)
+    pos = torch.arange(64, device="cuda").unsqueeze(0).expand(2, -1)
+    rope = Qwen2RotaryEmbedding(cfg).cuda()
+    pe = rope(x, pos)
+
+    def run(m, inp):
+        out = m(inp, position_embeddings=pe, attention_mask=None, position_ids=pos)
+        return out[0] if isinstance(out, tuple) else out
+
+    with torch.no_grad():
+        ref = run(layer, x)
+    replace_model_with_metis(holder, MetisArgs.direct_fp4(forward_svd_rank=32))
+    names = [n for n, m in holder.named_modules() if isinstance(m, BitLinear)]
+    assert len(names) == 7
+    attn = holder["layer"].self_attn
+    assert attn.q_proj.activation_group is attn.k_proj.activation_group is attn.v_proj.activation_group
+    xr = x.clone().requires_grad_(True)
+    out = run(holder["layer"], xr)
+    assert out.shape == ref.shape and bool(torch.isfinite(out).all())
+    assert rel_fro(out.detach().float().cpu(), ref.float().cpu()) < 0.1
+    out.float().square().mean().backward()
+    assert xr.grad is not None and bool(torch.isfinite(xr.grad).all())
+    assert attn.q_proj.warmup_linear.weight.grad is not None

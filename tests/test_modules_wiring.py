@@ -1,0 +1,243 @@
+"""Module wiring of the drop-in classes, mirroring the reference's own tests
+(tests/test_metis_quant_cache.py) with counting quantizer subclasses of Cast2Fp32 as spies.
+These run on CPU: identity quantizers take the generic (torch matmul) path, no NVFP4 arithmetic.
+"""
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from metis_hip import (BitLinear, Cast2Fp32, LinearLowbit, LinearLowbitFunction, MetisArgs, MetisHipError,
+                       quant_func, replace_linear_with_metis)
+
+
+@pytest.fixture(autouse=True)
+def _reset_function_config():
+    F = LinearLowbitFunction
+    keep = {k: getattr(F, k) for k in ("q_forward_input", "q_forward_weight", "q_backward_input", "q_backward_weight",
+                                       "q_backward_outputgrad", "enable_activation_svd", "enable_backward_svd",
+                                       "enable_nv_recipe", "compute_dtype", "metis_mode")}
+    yield
+    for k, v in keep.items():
+        setattr(F, k, v)
+    BitLinear.rollout_merge_active = False
+
+
+def _identity_config():
+    F = LinearLowbitFunction
+    F.compute_dtype = torch.float32
+    F.q_forward_input = Cast2Fp32
+    F.q_forward_weight = Cast2Fp32
+    F.q_backward_input = Cast2Fp32
+    F.q_backward_outputgrad = Cast2Fp32
+    F.enable_activation_svd = False
+    F.enable_backward_svd = False
+    F.enable_nv_recipe = False
+
+
+def test_registry_surface():
+    assert {"nvfp4e2m1bnosr", "nvfp4e2m1b", "fp32"} <= set(quant_func)
+    for q in quant_func.values():
+        for m in ("get_scalar", "quant", "rquant", "quantize_dequantize"):
+            assert callable(getattr(q, m))
+        assert hasattr(q, "compile_quantize_dequantize")
+    assert quant_func["nvfp4e2m1bnosr"].block_shape == (1, 16)
+    with pytest.raises(KeyError):
+        quant_func["no_such_format"]
+
+
+def test_nvfp4_has_no_cpu_path():
+    with pytest.raises(MetisHipError):
+        quant_func["nvfp4e2m1bnosr"].quantize_dequantize(torch.zeros(4, 32))
+    with pytest.raises(ValueError):       # reference quant.py:400-403
+        quant_func["nvfp4e2m1bnosr"].quantize_dequantize(torch.zeros(4, 24))
+
+
+def test_weight_cache_reuses_then_invalidates_after_parameter_update():
+    class CountingQuant(Cast2Fp32):
+        calls = 0
+
+        @classmethod
+        def quantize_dequantize(cls, value):
+            cls.calls += 1
+            return value.detach().clone()
+
+    args = SimpleNamespace(device="cpu", cache_quantized_weight=True)
+    layer = LinearLowbit(16, 8, bias=False, args=args)
+    _identity_config()
+    LinearLowbitFunction.q_forward_weight = CountingQuant
+    x = torch.randn(2, 3, 16, requires_grad=True)
+    layer(x).sum().backward()
+    assert layer.weight.grad is not None
+    layer(x.detach())
+    assert CountingQuant.calls == 1
+    with torch.no_grad():
+        layer.weight.add_(0.1)
+    layer(x.detach())
+    assert CountingQuant.calls == 2
+
+
+def test_mean_activation_path_uses_quantize_dequantize():
+    class CountingQuant(Cast2Fp32):
+        calls = 0
+
+        @classmethod
+        def quantize_dequantize(cls, value):
+            cls.calls += 1
+            return value
+
+        @classmethod
+        def get_scalar(cls, value):
+            raise AssertionError("mean activation path must use fused QDQ")
+
+    x = torch.randn(2, 3, 16)
+    cache = {}
+    out = LinearLowbitFunction.svd_quant(x, quant_func=CountingQuant, metis_mode="mean", mean_cache=cache, cache_key="t")
+    assert out.shape == x.shape and CountingQuant.calls == 1
+    torch.testing.assert_close(out, x)
+    assert cache["t"][1] == 6
+    # single-token decode updates the running mean with weights (reference 315-322)
+    step = torch.randn(4, 1, 16)
+    LinearLowbitFunction.svd_quant(step, quant_func=CountingQuant, metis_mode="mean", mean_cache=cache, cache_key="t")
+    assert cache["t"][1] == 10
+    with pytest.raises(ValueError):
+        LinearLowbitFunction.svd_quant(x, quant_func=CountingQuant, metis_mode="bogus")
+
+
+def test_identity_quantizers_give_plain_linear_gradients():
+    args = SimpleNamespace(device="cpu", cache_quantized_weight=False)
+    layer = LinearLowbit(16, 16, bias=True, args=args)
+    _identity_config()
+    x = torch.randn(2, 3, 16, requires_grad=True)
+    layer(x).sum().backward()
+    want_w = torch.ones(16, 1) @ x.detach().reshape(-1, 16).sum(dim=0, keepdim=True)
+    torch.testing.assert_close(layer.weight.grad, want_w, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(layer.bias.grad, torch.full((16,), 6.0))
+    torch.testing.assert_close(x.grad, layer.weight.detach().sum(0).expand(2, 3, 16), rtol=1e-5, atol=1e-5)
+    assert layer.weight.grad.dtype == torch.float32
+
+
+def test_replace_linear_does_not_split_when_forward_svd_disabled():
+    model = torch.nn.Sequential(torch.nn.Linear(16, 8, bias=False))
+    args = MetisArgs(enable_forward_svd=False)
+    args.device = "cpu"
+    replaced = replace_linear_with_metis(model, dtype=torch.float32, metis_args=args, target_modules=["0"],
+                                         compute_dtype=torch.float32)
+    layer = replaced[0]
+    assert isinstance(layer.warmup_linear, LinearLowbit)
+    assert layer.vlinear is None and layer.ulinear is None and layer.s is None and not layer.is_svd_quant
+
+
+def test_replace_linear_splits_and_keeps_state_dict_keys():
+    torch.manual_seed(0)
+    model = torch.nn.ModuleDict({"attn": torch.nn.ModuleDict({"q_proj": torch.nn.Linear(32, 24, bias=True),
+                                                              "k_proj": torch.nn.Linear(32, 16, bias=True)}),
+                                 "mlp": torch.nn.ModuleDict({"down_proj": torch.nn.Linear(24, 32, bias=False)})})
+    w_q = model["attn"]["q_proj"].weight.detach().clone()
+    args = MetisArgs(forward_svd_rank=8)
+    args.device = "cpu"
+    replace_linear_with_metis(model, dtype=torch.float32, metis_args=args, compute_dtype=torch.float32)
+    q, k, d = model["attn"]["q_proj"], model["attn"]["k_proj"], model["mlp"]["down_proj"]
+    assert all(isinstance(m, BitLinear) and m.is_svd_quant for m in (q, k, d))
+    assert q.activation_group is k.activation_group and q.activation_group["name"] == "attn.qkv"
+    assert d.activation_group is None and q.layer_name == "attn.q_proj"
+    keys = set(model.state_dict())
+    assert {"attn.q_proj.ulinear.weight", "attn.q_proj.vlinear.weight", "attn.q_proj.s",
+            "attn.q_proj.warmup_linear.weight", "attn.q_proj.warmup_linear.bias"} <= keys
+    assert "mlp.down_proj.warmup_linear.bias" not in keys
+    # U diag(s) V + residual reconstructs the original weight
+    rec = (q.ulinear.weight * q.s) @ q.vlinear.weight + q.warmup_linear.weight
+    torch.testing.assert_close(rec, w_q, rtol=1e-5, atol=1e-5)
+    assert q.vlinear.weight.shape == (8, 32) and q.ulinear.weight.shape == (24, 8) and q.s.shape == (8,)
+
+
+def _hand_assembled(args, group=None, name="test.layer", bias=False):
+    layer = BitLinear.__new__(BitLinear)
+    torch.nn.Module.__init__(layer)
+    layer.args = args
+    layer.is_svd_quant = True
+    layer.mean_cache = {}
+    layer.activation_group = group
+    layer._merged_rollout_weight_cache = None
+    layer.layer_name = name
+    layer.compute_dtype = torch.float32
+    layer.vlinear = LinearLowbit(16, 4, bias=False, args=args)
+    layer.ulinear = torch.nn.Linear(4, 8, bias=False)
+    layer.warmup_linear = LinearLowbit(16, 8, bias=bias, args=args)
+    layer.s = torch.nn.Parameter(torch.ones(4))
+    return layer
+
+
+class _CountingActivationQuant(Cast2Fp32):
+    calls = 0
+
+    @classmethod
+    def quantize_dequantize(cls, value):
+        cls.calls += 1
+        return value
+
+
+def _mean_config(q):
+    _identity_config()
+    F = LinearLowbitFunction
+    F.q_forward_input = q
+    F.enable_activation_svd = True
+    F.activation_lowrank_svd = 4
+    F.activation_broadcast_dim = -1
+    F.tp_simulate = False
+    F.metis_mode = "mean"
+
+
+def test_bitlinear_svd_branches_share_one_quantized_activation():
+    args = SimpleNamespace(device="cpu", cache_quantized_weight=False, forward_svd_rank=4)
+    layer = _hand_assembled(args)
+    _CountingActivationQuant.calls = 0
+    _mean_config(_CountingActivationQuant)
+    x = torch.randn(2, 3, 16, requires_grad=True)
+    layer(x).sum().backward()
+    assert _CountingActivationQuant.calls == 1
+    assert x.grad is not None and layer.vlinear.weight.grad is not None and layer.warmup_linear.weight.grad is not None
+
+
+def test_projection_group_reuses_quantized_activation():
+    args = SimpleNamespace(device="cpu", cache_quantized_weight=False, forward_svd_rank=4)
+    group = {"name": "test.attention.qkv", "mean_cache": {}, "input_ref": None, "quantized_input": None}
+    q_proj = _hand_assembled(args, group, "test.attention.q_proj")
+    k_proj = _hand_assembled(args, group, "test.attention.k_proj")
+    _CountingActivationQuant.calls = 0
+    _mean_config(_CountingActivationQuant)
+    x = torch.randn(2, 3, 16, requires_grad=True)
+    (q_proj(x).sum() + k_proj(x).sum()).backward()
+    assert _CountingActivationQuant.calls == 1
+    assert x.grad is not None and q_proj.vlinear.weight.grad is not None and k_proj.vlinear.weight.grad is not None
+    # a different tensor object is quantized again
+    q_proj(torch.randn(2, 3, 16))
+    assert _CountingActivationQuant.calls == 2
+
+
+def test_rollout_merged_weight_cache_reuses_and_invalidates():
+    args = SimpleNamespace(device="cpu", cache_quantized_weight=True, forward_svd_rank=4)
+    layer = _hand_assembled(args, bias=True)
+    _mean_config(Cast2Fp32)
+    x = torch.randn(2, 3, 16)
+    with torch.no_grad():
+        BitLinear.rollout_merge_active = False
+        expected = layer(x)
+        BitLinear.rollout_merge_active = True
+        actual = layer(x)
+        first = layer._get_merged_rollout_weight(torch.float32)
+        second = layer._get_merged_rollout_weight(torch.float32)
+        layer.s.add_(0.1)
+        updated = layer._get_merged_rollout_weight(torch.float32)
+    torch.testing.assert_close(actual, expected)
+    assert first is second and updated is not first
+
+
+def test_unsupported_options_fail_loudly():
+    args = MetisArgs()
+    args.device = "cpu"
+    with pytest.raises(ValueError):
+        BitLinear(16, 8, args=args, dtype=torch.float32, compute_dtype=torch.int8)
+    LinearLowbitFunction.enable_nv_recipe = True
+    with pytest.raises(NotImplementedError):
+        LinearLowbitFunction._quantize_wgrad_operand(torch.zeros(2, 16), Cast2Fp32)
