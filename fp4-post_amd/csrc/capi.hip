@@ -110,6 +110,18 @@ int metis_linear_fwd(const void* a_codes, const void* a_scales, const float* a_u
                       (hipStream_t)stream);
 }
 
+int metis_nvfp4_expand_f16(const void* codes, const void* scales, int64_t rows, int64_t cols, void* out, void* stream)
+{
+    return expand_f16(codes, scales, rows, cols, out, (hipStream_t)stream);
+}
+
+int metis_linear_fwd_expanded(const void* a_exp, const float* a_unit, const void* b_exp, const float* b_unit, int64_t M,
+                              int64_t N, int64_t K, const void* t, const void* u, int64_t r, const void* bias, void* out,
+                              int out_dtype, void* stream)
+{
+    return gemm_expanded(a_exp, a_unit, b_exp, b_unit, M, N, K, t, u, r, bias, out, out_dtype, (hipStream_t)stream);
+}
+
 int metis_linear_dgrad(const void* dy_codes, const void* dy_scales, const float* dy_unit, const void* wt_codes,
                        const void* wt_scales, const float* wt_unit, int64_t L, int64_t N, int64_t K, void* grad_input,
                        int out_dtype, void* stream)

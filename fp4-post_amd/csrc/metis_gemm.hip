@@ -196,12 +196,13 @@ __global__ __launch_bounds__(256) void gemm_nvfp4_kernel(
 }
 
 // ---------------------------------------------------------------------------------------------
-// Large-tile kernel: 256 x 256 per workgroup, 4 waves of 128 x 128 (16 MFMA tiles, 256 accumulator
-// registers per lane), K step 64, LDS double buffered (2 x 72 KiB) with one barrier per step.
-// Per step a thread owns one A row and one B row of the tile: it fetches their 32 bytes of codes
-// and 4 scale bytes into registers one step ahead, and expands them into the idle LDS buffer
-// while the MFMAs of the current buffer execute.  A wave reads (4 + 4) KiB of fragments per
-// 16 MFMAs, half the LDS traffic per flop of the 64 x 64 wave tile.
+// Large-tile kernel: 256 x 256 per workgroup, K step 64, LDS double buffered (2 x 72 KiB) with one
+// barrier per step.  Two wave layouts:
+//   4 waves (2 x 2), 128 x 128 per wave: 16 MFMA tiles, 256 accumulator registers per lane
+//   8 waves (2 x 4), 128 x  64 per wave:  8 MFMA tiles, two waves per SIMD
+// Each thread owns one (8 waves) or two (4 waves) rows of the 512-row A|B tile per step: it fetches
+// their 32 bytes of codes and 4 scale bytes into registers a full step ahead and expands them into
+// the idle LDS buffer between the MFMAs of the current buffer.
 //
 // Tile order: workgroup ids are dealt round-robin to the 8 XCDs by the hardware, so id -> (xcd,
 // slot) is undone first to give every XCD (and its private L2) one contiguous range of tiles,
@@ -216,23 +217,6 @@ struct RowRegs {
     uint32_t sc;       // 4 scale bytes
 };
 
-__device__ __forceinline__ void fetch_row(RowRegs& r, const uint8_t* codes, const uint8_t* scales, int64_t row, int kbytes,
-                                          int kblocks, int k0, int K)
-{
-    r.c0 = r.c1 = make_uint4(0u, 0u, 0u, 0u);
-    r.sc = 0u;
-    const uint8_t* cp = codes + row * kbytes + k0 / 2;
-    const uint8_t* sp = scales + row * kblocks + k0 / kBlock;
-    if (k0 + 64 <= K) {
-        r.c0 = reinterpret_cast<const uint4*>(cp)[0];
-        r.c1 = reinterpret_cast<const uint4*>(cp)[1];
-        r.sc = *reinterpret_cast<const uint32_t*>(sp);
-    } else if (k0 < K) {                                         // K % 64 == 32: half a step left
-        r.c0 = reinterpret_cast<const uint4*>(cp)[0];
-        r.sc = *reinterpret_cast<const uint16_t*>(sp);
-    }
-}
-
 __device__ __forceinline__ void expand_row(const RowRegs& r, uint16_t* dst)
 {
     const half2_t s0 = scale_pair(r.sc & 0xffu), s1 = scale_pair((r.sc >> 8) & 0xffu);
@@ -244,40 +228,43 @@ __device__ __forceinline__ void expand_row(const RowRegs& r, uint16_t* dst)
     d[6] = expand8(r.c1.z, s3); d[7] = expand8(r.c1.w, s3);
 }
 
-// one expand8 of the 16 that make up a thread's two rows: q in 0..7 -> A row, 8..15 -> B row
-__device__ __forceinline__ void expand_piece(const RowRegs& ra, const RowRegs& rb, int q, uint16_t* da, uint16_t* db)
+// one expand8 (8 elements) of a row: p in 0..7
+__device__ __forceinline__ void expand_piece(const RowRegs& r, int p, uint16_t* d)
 {
-    const RowRegs& r = q < 8 ? ra : rb;
-    uint16_t* d = q < 8 ? da : db;
-    const int p = q & 7;
     const uint32_t w = p == 0 ? r.c0.x : p == 1 ? r.c0.y : p == 2 ? r.c0.z : p == 3 ? r.c0.w
                      : p == 4 ? r.c1.x : p == 5 ? r.c1.y : p == 6 ? r.c1.z : r.c1.w;
     reinterpret_cast<uint4*>(d)[p] = expand8(w, scale_pair((r.sc >> (8 * (p >> 1))) & 0xffu));
 }
 
-// MFMA : VALU : LDS interleave requested from the scheduler for one K=16 sub-step
-template <int N_VALU_PER_MFMA, int N_DSR, int N_DSW>
+// MFMA : VALU : LDS interleave requested from the scheduler for one K=16 sub-step of N_MFMA MFMAs
+template <int N_MFMA, int N_VALU_PER_MFMA, int N_DSR, int N_DSW>
 __device__ __forceinline__ void sched_substep()
 {
 #pragma unroll
-    for (int m = 0; m < 16; ++m) {
+    for (int m = 0; m < N_MFMA; ++m) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                       // one MFMA
         if (m < N_DSR) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);        // one LDS read
-        __builtin_amdgcn_sched_group_barrier(0x002, N_VALU_PER_MFMA, 0);         // VALU of the expansion
-        if (m % 3 == 2 && m / 3 < N_DSW) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);   // one LDS write
+        if (N_VALU_PER_MFMA) __builtin_amdgcn_sched_group_barrier(0x002, N_VALU_PER_MFMA, 0);   // expansion VALU
+        if (m < N_DSW) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);        // one LDS write
     }
 }
 
-template <int OUT_F32, int DBG = 0>
-__global__ __launch_bounds__(256, 1) void gemm_nvfp4_large_kernel(
+template <int OUT_F32, int WN_WAVES, int DBG = 0>
+__global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_nvfp4_large_kernel(
     const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const float* __restrict__ a_unit,
     const uint8_t* __restrict__ b_codes, const uint8_t* __restrict__ b_scales, const float* __restrict__ b_unit,
     int M, int N, int K, const uint16_t* __restrict__ t, const uint16_t* __restrict__ u, int r,
     const uint16_t* __restrict__ bias, void* __restrict__ out, int tiles_m, int tiles_n)
 {
     extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+    constexpr int TM = 4;                            // 32-tall MFMA tiles per wave along m
+    constexpr int TN = 8 / WN_WAVES;                 // 32-wide MFMA tiles per wave along n: 4 or 2
+    constexpr int WTN = 256 / WN_WAVES;              // wave tile width: 128 or 64
+    constexpr int NTHREADS = 128 * WN_WAVES;
+    constexpr int RPT = 512 / NTHREADS;              // A|B tile rows expanded by one thread: 2 or 1
+    constexpr int PIECES = 8 * RPT;                  // expand8 pieces per thread per step
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WN_WAVES, wn = wave % WN_WAVES;
 
     // ---- tile assignment (XCD-contiguous, grouped)
     const int total = tiles_m * tiles_n;
@@ -292,62 +279,67 @@ __global__ __launch_bounds__(256, 1) void gemm_nvfp4_large_kernel(
     const int tn = (logical % (GM * tiles_n)) / gsize;
     const int m0 = tm * L_BM, n0 = tn * L_BN;
 
-    float16_t acc[4][4];
+    float16_t acc[TM][TN];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
+    // ---- rows of the A|B tile this thread stages: tile row q*NTHREADS + tid (0..255 = A, 256..511 = B)
     const int kbytes = K / 2, kblocks = K / kBlock;
-    const int64_t arow = min(m0 + tid, M - 1), brow = min(n0 + tid, N - 1);
-    uint16_t* const my_a = lds + tid * L_STRIDE;
-    uint16_t* const my_b = lds + (L_BM + tid) * L_STRIDE;
-    const uint8_t* const a_cp = a_codes + arow * kbytes;
-    const uint8_t* const a_sp = a_scales + arow * kblocks;
-    const uint8_t* const b_cp = b_codes + brow * kbytes;
-    const uint8_t* const b_sp = b_scales + brow * kblocks;
-    auto fetch = [&](RowRegs& ra, RowRegs& rb, int k0) {           // K % 64 == 0: always a full step
-        ra.c0 = reinterpret_cast<const uint4*>(a_cp + k0 / 2)[0];
-        ra.c1 = reinterpret_cast<const uint4*>(a_cp + k0 / 2)[1];
-        ra.sc = *reinterpret_cast<const uint32_t*>(a_sp + k0 / kBlock);
-        rb.c0 = reinterpret_cast<const uint4*>(b_cp + k0 / 2)[0];
-        rb.c1 = reinterpret_cast<const uint4*>(b_cp + k0 / 2)[1];
-        rb.sc = *reinterpret_cast<const uint32_t*>(b_sp + k0 / kBlock);
+    const uint8_t* cp[RPT];
+    const uint8_t* sp[RPT];
+    int lds_row[RPT];
+#pragma unroll
+    for (int q = 0; q < RPT; ++q) {
+        const int trow = q * NTHREADS + tid;
+        const bool is_a = trow < L_BM;
+        const int64_t grow = is_a ? min(m0 + trow, M - 1) : min(n0 + trow - L_BM, N - 1);
+        cp[q] = (is_a ? a_codes : b_codes) + grow * kbytes;
+        sp[q] = (is_a ? a_scales : b_scales) + grow * kblocks;
+        lds_row[q] = trow * L_STRIDE;
+    }
+    auto fetch = [&](RowRegs (&rr)[RPT], int k0) {               // K % 64 == 0: always a full step
+#pragma unroll
+        for (int q = 0; q < RPT; ++q) {
+            rr[q].c0 = reinterpret_cast<const uint4*>(cp[q] + k0 / 2)[0];
+            rr[q].c1 = reinterpret_cast<const uint4*>(cp[q] + k0 / 2)[1];
+            rr[q].sc = *reinterpret_cast<const uint32_t*>(sp[q] + k0 / kBlock);
+        }
     };
 
     const int steps = K / BK;
-    // two register sets of packed rows: during step s the rows of step s+1 (r1) are expanded into the idle
-    // LDS buffer while the global loads of step s+2 land in r2 -- a full step of latency cover -- and
-    // r2 is moved into r1 at the end of the step
-    RowRegs ra1, rb1, ra2, rb2;
-    fetch(ra1, rb1, 0);
-    expand_row(ra1, my_a);
-    expand_row(rb1, my_b);
-    if (steps > 1) fetch(ra1, rb1, BK);
+    // r1: rows of step s+1, expanded during step s; r2: rows of step s+2, in flight during step s
+    RowRegs r1[RPT], r2[RPT];
+    fetch(r1, 0);
+#pragma unroll
+    for (int q = 0; q < RPT; ++q) expand_row(r1[q], lds + lds_row[q]);
+    if (steps > 1) fetch(r1, BK);
     __syncthreads();
 
     const int frag_off = (lane & 31) * L_STRIDE + (lane >> 5) * 8;
     const int a_off = wm * 128 * L_STRIDE + frag_off;
-    const int b_off = (L_BM + wn * 128) * L_STRIDE + frag_off;
-    half8_t fa[2][4], fb[2][4];
+    const int b_off = (L_BM + wn * WTN) * L_STRIDE + frag_off;
+    half8_t fa[2][TM], fb[2][TN];
     auto load_frags = [&](int buf, const uint16_t* stage, int ks) {
-        if ((DBG & 4) && !(stage == lds && ks == 0 && buf == 0)) { if (buf != 0) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) { fa[1][i] = fa[0][i]; fb[1][i] = fb[0][i]; } } return; }
+        for (int i = 0; i < TM; ++i) fa[buf][i] = *reinterpret_cast<const half8_t*>(stage + a_off + i * 32 * L_STRIDE + ks * 16);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) fa[buf][i] = *reinterpret_cast<const half8_t*>(stage + a_off + i * 32 * L_STRIDE + ks * 16);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) fb[buf][j] = *reinterpret_cast<const half8_t*>(stage + b_off + j * 32 * L_STRIDE + ks * 16);
+        for (int j = 0; j < TN; ++j) fb[buf][j] = *reinterpret_cast<const half8_t*>(stage + b_off + j * 32 * L_STRIDE + ks * 16);
     };
-    auto mfma16 = [&](int buf) {
+    auto mfmas = [&](int buf) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+            for (int j = 0; j < TN; ++j)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
     };
+    constexpr int NM = TM * TN, NF = TM + TN;
+    // pieces expanded in sub-steps 0, 1, 2 (all before the barrier)
+    constexpr int P0 = (PIECES + 2) / 3, P1 = (PIECES - P0 + 1) / 2, P2 = PIECES - P0 - P1;
+    constexpr int VPM = (P0 * 9 + NM - 1) / NM;       // VALU ops to slot behind each MFMA
     // One K step.  EXPAND: rows of step s+1 (r1) are expanded into the idle LDS buffer during sub-steps
     // 0..2; the barrier sits before sub-step 3, whose MFMAs cover the first fragment loads of step s+1.
     // FETCH: global loads of step s+2 into r2, issued at the top so they have the whole step to arrive.
@@ -355,39 +347,31 @@ __global__ __launch_bounds__(256, 1) void gemm_nvfp4_large_kernel(
         constexpr bool EXPAND = decltype(do_expand)::value && !(DBG & 1), FETCH = decltype(do_fetch)::value && !(DBG & 1);
         const uint16_t* cur = lds + (s & 1) * L_STAGE_HALVES;
         uint16_t* nxt = lds + ((s + 1) & 1) * L_STAGE_HALVES;
-        uint16_t* na = nxt + tid * L_STRIDE;
-        uint16_t* nb = nxt + (L_BM + tid) * L_STRIDE;
-        if (FETCH) fetch(ra2, rb2, (s + 2) * BK);
-        // sub-step 0
+        if (FETCH) fetch(r2, (s + 2) * BK);
+        auto pieces = [&](int from, int to) {
+#pragma unroll
+            for (int p = from; p < to; ++p) expand_piece(r1[p / 8], p % 8, nxt + lds_row[p / 8]);
+        };
         load_frags(1, cur, 1);
-        if (EXPAND) {
-#pragma unroll
-            for (int q = 0; q < 6; ++q) expand_piece(ra1, rb1, q, na, nb);
-        }
-        mfma16(0);
-        if (EXPAND) sched_substep<3, 8, 5>(); else sched_substep<0, 8, 0>();
-        // sub-step 1
+        if (EXPAND) pieces(0, P0);
+        mfmas(0);
+        if (!(DBG & 8)) { if (EXPAND) sched_substep<NM, VPM, NF, P0>(); else sched_substep<NM, 0, NF, 0>(); }
         load_frags(0, cur, 2);
-        if (EXPAND) {
-#pragma unroll
-            for (int q = 6; q < 11; ++q) expand_piece(ra1, rb1, q, na, nb);
-        }
-        mfma16(1);
-        if (EXPAND) sched_substep<3, 8, 5>(); else sched_substep<0, 8, 0>();
-        // sub-step 2
+        if (EXPAND) pieces(P0, P0 + P1);
+        mfmas(1);
+        if (!(DBG & 8)) { if (EXPAND) sched_substep<NM, VPM, NF, P1>(); else sched_substep<NM, 0, NF, 0>(); }
         load_frags(1, cur, 3);
-        if (EXPAND) {
-#pragma unroll
-            for (int q = 11; q < 16; ++q) expand_piece(ra1, rb1, q, na, nb);
-        }
-        mfma16(0);
-        if (EXPAND) sched_substep<3, 8, 5>(); else sched_substep<0, 8, 0>();
+        if (EXPAND) pieces(P0 + P1, PIECES);
+        mfmas(0);
+        if (!(DBG & 8)) { if (EXPAND) sched_substep<NM, VPM, NF, P2>(); else sched_substep<NM, 0, NF, 0>(); }
         if (!(DBG & 2)) __syncthreads();
-        // sub-step 3
         if (EXPAND || (DBG & 1)) load_frags(0, nxt, 0);
-        mfma16(1);
-        sched_substep<0, 8, 0>();
-        if (FETCH) { ra1 = ra2; rb1 = rb2; }
+        mfmas(1);
+        if (!(DBG & 8)) sched_substep<NM, 0, NF, 0>();
+        if (FETCH) {
+#pragma unroll
+            for (int q = 0; q < RPT; ++q) r1[q] = r2[q];
+        }
     };
     using T_ = std::true_type;
     using F_ = std::false_type;
@@ -401,51 +385,51 @@ __global__ __launch_bounds__(256, 1) void gemm_nvfp4_large_kernel(
     // ---- tensor units (and the 2^8 * 2^8 of the scale placement)
     const float us = (*a_unit) * (*b_unit) * 65536.0f;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] *= us;
 
     // ---- bf16 low-rank extension, 32 columns of T / U per step, staged in buffer 0
     for (int j0 = 0; j0 < r; j0 += 32) {
-        {
-            const uint4* sa = reinterpret_cast<const uint4*>(t + arow * r + j0);
-            const uint4* sb = reinterpret_cast<const uint4*>(u + brow * r + j0);
-            uint4* da = reinterpret_cast<uint4*>(my_a);
-            uint4* db = reinterpret_cast<uint4*>(my_b);
 #pragma unroll
-            for (int q = 0; q < 4; ++q) { da[q] = sa[q]; db[q] = sb[q]; }
+        for (int q = 0; q < RPT; ++q) {
+            const int trow = q * NTHREADS + tid;
+            const bool is_a = trow < L_BM;
+            const int64_t grow = is_a ? min(m0 + trow, M - 1) : min(n0 + trow - L_BM, N - 1);
+            const uint4* src = reinterpret_cast<const uint4*>((is_a ? t : u) + grow * r + j0);
+            uint4* dst = reinterpret_cast<uint4*>(lds + lds_row[q]);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) dst[c] = src[c];
         }
         __syncthreads();
-        const uint16_t* pa = lds + a_off;
-        const uint16_t* pb = lds + b_off;
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
-            bf16x8_t fa[4], fb[4];
+            bf16x8_t ga[TM], gb[TN];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) fa[i] = *reinterpret_cast<const bf16x8_t*>(pa + i * 32 * L_STRIDE + ks * 16);
+            for (int i = 0; i < TM; ++i) ga[i] = *reinterpret_cast<const bf16x8_t*>(lds + a_off + i * 32 * L_STRIDE + ks * 16);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) fb[j] = *reinterpret_cast<const bf16x8_t*>(pb + j * 32 * L_STRIDE + ks * 16);
+            for (int j = 0; j < TN; ++j) gb[j] = *reinterpret_cast<const bf16x8_t*>(lds + b_off + j * 32 * L_STRIDE + ks * 16);
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gb[j], ga[i], acc[i][j], 0, 0, 0);
         }
         __syncthreads();
     }
 
     // ---- epilogue.  acc[i][j][e]: n = 8*(e/4) + 4*(lane/32) + e%4, m = lane%32 within the tile
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < TM; ++i) {
         const int m = m0 + wm * 128 + i * 32 + (lane & 31);
         if (m >= M) continue;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < TN; ++j) {
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                const int n = n0 + wn * 128 + j * 32 + 8 * g + 4 * (lane >> 5);
+                const int n = n0 + wn * WTN + j * 32 + 8 * g + 4 * (lane >> 5);
                 if (n >= N) continue;
                 float v[4];
 #pragma unroll
@@ -466,6 +450,283 @@ __global__ __launch_bounds__(256, 1) void gemm_nvfp4_large_kernel(
     }
 }
 
+template <int WN_WAVES>
+static int launch_large(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes,
+                        const void* b_scales, const float* b_unit, int64_t M, int64_t N, int64_t K, const void* t,
+                        const void* u, int64_t r, const void* bias, void* out, int out_dtype, hipStream_t st)
+{
+    static bool attr_set[2] = {false, false};
+    const size_t lds_bytes = 2 * (size_t)L_STAGE_HALVES * sizeof(uint16_t);
+    const int f32 = out_dtype == METIS_DTYPE_F32;
+    const void* fn = f32 ? (const void*)gemm_nvfp4_large_kernel<1, WN_WAVES> : (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES>;
+    if (const char* d = getenv("METIS_GEMM_DBG")) {
+        const int v = atoi(d);
+        fn = v == 1 ? (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 1> : v == 8 ? (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 8>
+           : v == 7 ? (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 7> : fn;
+        (void)hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    }
+    if (!attr_set[f32]) {
+        if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
+            return METIS_E_DEVICE;
+        attr_set[f32] = true;
+    }
+    const int tiles_m = (int)((M + L_BM - 1) / L_BM), tiles_n = (int)((N + L_BN - 1) / L_BN);
+    const int total = tiles_m * tiles_n;
+    const unsigned grid_x = (unsigned)(((total + 7) / 8) * 8);
+    const uint8_t *ac = (const uint8_t*)a_codes, *as = (const uint8_t*)a_scales, *bc = (const uint8_t*)b_codes,
+                  *bs = (const uint8_t*)b_scales;
+    const uint16_t *tp = (const uint16_t*)t, *up = (const uint16_t*)u, *bp = (const uint16_t*)bias;
+    int Mi = (int)M, Ni = (int)N, Ki = (int)K, ri = (int)r, tmi = tiles_m, tni = tiles_n;
+    void* args[] = {&ac, &as, &a_unit, &bc, &bs, &b_unit, &Mi, &Ni, &Ki, &tp, &up, &ri, &bp, &out, &tmi, &tni};
+    if (hipLaunchKernel(fn, dim3(grid_x), dim3(128 * WN_WAVES), args, lds_bytes, st) != hipSuccess) {
+        (void)hipGetLastError();
+        return METIS_E_LAUNCH;
+    }
+    return METIS_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Expansion of a packed tensor to binary16: value = e2m1(code) * e4m3(scale) * 2^-8, exact.
+// One thread per 8 elements (one dword of codes -> 16 bytes).  HBM-bound: 0.5625 B read, 2 B written
+// per element.  The expanded tensor is what gemm_f16_large_kernel consumes; it is derived data that
+// callers may cache next to the packed weight (the reference caches the dequantized weight the
+// same way, src/Metis/Metis/bitlinear.py:563-589).
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void expand_f16_kernel(const uint32_t* __restrict__ codes, const uint8_t* __restrict__ scales,
+                                                         uint4* __restrict__ out, int64_t noct)
+{
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < noct; i += (int64_t)gridDim.x * 256)
+        out[i] = expand8(codes[i], scale_pair(scales[i >> 1]));
+}
+
+int expand_f16(const void* codes, const void* scales, int64_t rows, int64_t cols, void* out, hipStream_t st)
+{
+    if (rows < 0 || cols < 0) return METIS_E_ARG;
+    if (cols % kBlock) return METIS_E_SHAPE;
+    const int64_t noct = rows * cols / 8;
+    if (noct == 0) return METIS_OK;
+    if (!codes || !scales || !out || ((uintptr_t)codes % 4) || ((uintptr_t)out % 16)) return METIS_E_ARG;
+    int64_t g = (noct + 255) / 256;
+    const int64_t cap = (int64_t)device_cus() * 16;
+    if (g > cap) g = cap;
+    hipLaunchKernelGGL(expand_f16_kernel, dim3((int)g), dim3(256), 0, st, (const uint32_t*)codes, (const uint8_t*)scales,
+                       (uint4*)out, noct);
+    return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
+}
+
+// ---------------------------------------------------------------------------------------------
+// GEMM on expanded operands: same tile (256 x 256, 8 waves of 128 x 64, K step 64), same epilogue, but
+// the inner loop is MFMA + LDS reads only.  Operand tiles go HBM/L2 -> LDS directly
+// (global_load_lds_dwordx4, no registers, no VALU), one full step ahead, into a double buffer of
+// 2 x 64 KiB.  LDS rows are 128 bytes with the 16-byte chunk index XOR-ed by (row & 7): the 8
+// lanes of one LDS access phase hit 8 different chunk columns, so fragment reads are conflict
+// free without padding (a direct load fills 1 KiB of contiguous LDS, which rules padding out).
+// ---------------------------------------------------------------------------------------------
+constexpr int X_STAGE_BYTES = (L_BM + L_BN) * BK * 2;             // 64 KiB: 512 rows x 128 B
+
+template <int OUT_F32>
+__global__ __launch_bounds__(512, 1) void gemm_f16_large_kernel(
+    const uint16_t* __restrict__ a_exp, const float* __restrict__ a_unit, const uint16_t* __restrict__ b_exp,
+    const float* __restrict__ b_unit, int M, int N, int K, const uint16_t* __restrict__ t, const uint16_t* __restrict__ u,
+    int r, const uint16_t* __restrict__ bias, void* __restrict__ out, int tiles_m, int tiles_n)
+{
+    extern __shared__ __attribute__((aligned(1024))) uint8_t xlds[];
+    constexpr int TM = 4, TN = 2, WTN = 64;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 2, wn = wave & 3;
+
+    const int total = tiles_m * tiles_n;
+    const int per_xcd = (total + 7) / 8;
+    const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (logical >= total) return;
+    constexpr int GM = 4;
+    const int group = logical / (GM * tiles_n);
+    const int first_m = group * GM;
+    const int gsize = min(tiles_m - first_m, GM);
+    const int tm = first_m + (logical % (GM * tiles_n)) % gsize;
+    const int tn = (logical % (GM * tiles_n)) / gsize;
+    const int m0 = tm * L_BM, n0 = tn * L_BN;
+
+    float16_t acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+    // ---- async staging: instruction j of wave w fills LDS rows (j*8 + w)*8 .. +7 (1 KiB); lane -> (row, chunk)
+    const uint8_t* src[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int trow = (j * 8 + wave) * 8 + (lane >> 3);          // row of the A|B tile, 0..511
+        const int chunk = (lane & 7) ^ (trow & 7);                  // logical 16-byte chunk that belongs at this slot
+        const bool is_a = trow < L_BM;
+        const int64_t grow = is_a ? min(m0 + trow, M - 1) : min(n0 + trow - L_BM, N - 1);
+        src[j] = reinterpret_cast<const uint8_t*>((is_a ? a_exp : b_exp) + grow * K) + chunk * 16;
+    }
+    auto stage_in = [&](int buf, int k0) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)(src[j] + (int64_t)k0 * 2),
+                                             (void __attribute__((address_space(3)))*)(xlds + buf * X_STAGE_BYTES + (j * 8 + wave) * 1024),
+                                             16, 0, 0);
+    };
+
+    const int steps = K / BK;
+    stage_in(0, 0);
+    if (steps > 1) {
+        stage_in(1, BK);
+        __builtin_amdgcn_s_waitcnt(0x0F78);                         // vmcnt(8): the first step has landed, the second may fly
+    } else {
+        __builtin_amdgcn_s_waitcnt(0x0F70);                         // vmcnt(0)
+    }
+    __syncthreads();
+
+    // fragment addressing: row = base + (lane & 31), chunk = 2*ks + (lane >> 5), slot = chunk ^ (row & 7)
+    const int frow = lane & 31, fhi = lane >> 5;
+    int a_row_off[TM], b_row_off[TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) a_row_off[i] = (wm * 128 + i * 32 + frow) * 128;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) b_row_off[j] = (L_BM + wn * WTN + j * 32 + frow) * 128;
+    const int sw = frow & 7;                                        // (row & 7): tile bases are multiples of 32
+    half8_t fa[2][TM], fb[2][TN];
+    auto load_frags = [&](int fbuf, int buf, int ks) {
+        const int slot = ((2 * ks + fhi) ^ sw) * 16;
+        const uint8_t* base = xlds + buf * X_STAGE_BYTES + slot;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[fbuf][i] = *reinterpret_cast<const half8_t*>(base + a_row_off[i]);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb[fbuf][j] = *reinterpret_cast<const half8_t*>(base + b_row_off[j]);
+    };
+    auto mfmas = [&](int fbuf) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[fbuf][j], fa[fbuf][i], acc[i][j], 0, 0, 0);
+    };
+
+    load_frags(0, 0, 0);
+    for (int s = 0; s < steps; ++s) {
+        const int buf = s & 1;
+        load_frags(1, buf, 1);
+        mfmas(0);
+        load_frags(0, buf, 2);
+        mfmas(1);
+        load_frags(1, buf, 3);
+        mfmas(0);
+        // every wave has issued its last reads of `buf`; the loads of step s+1 (issued one step ago) must have landed
+        __builtin_amdgcn_s_waitcnt(0x0070);                         // vmcnt(0), lgkmcnt(0)
+        __syncthreads();
+        if (s + 2 < steps) stage_in(buf, (s + 2) * BK);             // refill the buffer just released
+        if (s + 1 < steps) load_frags(0, buf ^ 1, 0);
+        mfmas(1);
+    }
+    __syncthreads();
+
+    const float us = (*a_unit) * (*b_unit) * 65536.0f;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] *= us;
+
+    // ---- bf16 low-rank extension, 32 columns per step: rows staged through registers, padded 144-byte rows
+    uint16_t* plds = reinterpret_cast<uint16_t*>(xlds);
+    for (int j0 = 0; j0 < r; j0 += 32) {
+        {
+            const bool is_a = tid < L_BM;
+            const int64_t grow = is_a ? min(m0 + tid, M - 1) : min(n0 + tid - L_BM, N - 1);
+            const uint4* sp = reinterpret_cast<const uint4*>((is_a ? t : u) + grow * r + j0);
+            uint4* dp = reinterpret_cast<uint4*>(plds + tid * L_STRIDE);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) dp[c] = sp[c];
+        }
+        __syncthreads();
+        const int foff = frow * L_STRIDE + fhi * 8;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            bf16x8_t ga[TM], gb[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) ga[i] = *reinterpret_cast<const bf16x8_t*>(plds + (wm * 128 + i * 32) * L_STRIDE + foff + ks * 16);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) gb[j] = *reinterpret_cast<const bf16x8_t*>(plds + (L_BM + wn * WTN + j * 32) * L_STRIDE + foff + ks * 16);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gb[j], ga[i], acc[i][j], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        const int m = m0 + wm * 128 + i * 32 + (lane & 31);
+        if (m >= M) continue;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int n = n0 + wn * WTN + j * 32 + 8 * g + 4 * (lane >> 5);
+                if (n >= N) continue;
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    v[e] = acc[i][j][4 * g + e];
+                    if (bias) v[e] += bf16_lo(bias[n + e]);
+                }
+                if (OUT_F32) {
+                    *reinterpret_cast<float4*>((float*)out + (int64_t)m * N + n) = make_float4(v[0], v[1], v[2], v[3]);
+                } else {
+                    uint2 w;
+                    w.x = bf16_bits(v[0]) | (bf16_bits(v[1]) << 16);
+                    w.y = bf16_bits(v[2]) | (bf16_bits(v[3]) << 16);
+                    *reinterpret_cast<uint2*>((uint16_t*)out + (int64_t)m * N + n) = w;
+                }
+            }
+        }
+    }
+}
+
+int gemm_expanded(const void* a_exp, const float* a_unit, const void* b_exp, const float* b_unit, int64_t M, int64_t N,
+                  int64_t K, const void* t, const void* u, int64_t r, const void* bias, void* out, int out_dtype,
+                  hipStream_t st)
+{
+    if (M < 0 || N < 0 || K < 0 || r < 0) return METIS_E_ARG;
+    if (out_dtype != METIS_DTYPE_BF16 && out_dtype != METIS_DTYPE_F32) return METIS_E_ARG;
+    if (K % kBlock) return METIS_E_SHAPE;
+    if (K % BK || K == 0 || N % 4 || r % 32 || (r > 0 && (!t || !u))) return METIS_E_ARG;
+    if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return METIS_E_ARG;
+    if (M == 0 || N == 0) return METIS_OK;
+    if (!a_exp || !a_unit || !b_exp || !b_unit || !out) return METIS_E_ARG;
+    if (((uintptr_t)a_exp % 16) || ((uintptr_t)b_exp % 16) || ((uintptr_t)out % 16)) return METIS_E_ARG;
+    static bool attr_set[2] = {false, false};
+    const size_t lds_bytes = 2 * (size_t)X_STAGE_BYTES;
+    const int f32 = out_dtype == METIS_DTYPE_F32;
+    const void* fn = f32 ? (const void*)gemm_f16_large_kernel<1> : (const void*)gemm_f16_large_kernel<0>;
+    if (!attr_set[f32]) {
+        if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
+            return METIS_E_DEVICE;
+        attr_set[f32] = true;
+    }
+    const int tiles_m = (int)((M + L_BM - 1) / L_BM), tiles_n = (int)((N + L_BN - 1) / L_BN);
+    const int total = tiles_m * tiles_n;
+    const unsigned grid_x = (unsigned)(((total + 7) / 8) * 8);
+    const uint16_t *ae = (const uint16_t*)a_exp, *be = (const uint16_t*)b_exp, *tp = (const uint16_t*)t,
+                   *up = (const uint16_t*)u, *bp = (const uint16_t*)bias;
+    int Mi = (int)M, Ni = (int)N, Ki = (int)K, ri = (int)r, tmi = tiles_m, tni = tiles_n;
+    void* args[] = {&ae, &a_unit, &be, &b_unit, &Mi, &Ni, &Ki, &tp, &up, &ri, &bp, &out, &tmi, &tni};
+    if (hipLaunchKernel(fn, dim3(grid_x), dim3(512), args, lds_bytes, st) != hipSuccess) {
+        (void)hipGetLastError();
+        return METIS_E_LAUNCH;
+    }
+    return METIS_OK;
+}
+
 int gemm_nvfp4(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes, const void* b_scales,
                const float* b_unit, int64_t M, int64_t N, int64_t K, const void* t, const void* u, int64_t r,
                const void* bias, void* out, int out_dtype, hipStream_t st)
@@ -482,34 +743,9 @@ int gemm_nvfp4(const void* a_codes, const void* a_scales, const float* a_unit, c
     if (K % 32) return METIS_E_ARG;                            // 16-byte code chunks: rows must stay 16-byte aligned
     if (M == 0 || N == 0) return METIS_OK;
     if (M >= 256 && N >= 256 && K % BK == 0 && !getenv("METIS_GEMM_SMALL")) {
-        static bool attr_set[2] = {false, false};
-        const size_t lds_bytes = 2 * (size_t)L_STAGE_HALVES * sizeof(uint16_t);
-        const int f32 = out_dtype == METIS_DTYPE_F32;
-        const void* fn = f32 ? (const void*)gemm_nvfp4_large_kernel<1> : (const void*)gemm_nvfp4_large_kernel<0>;
-        if (const char* d = getenv("METIS_GEMM_DBG")) {
-            const int v = atoi(d);
-            fn = v == 1 ? (const void*)gemm_nvfp4_large_kernel<0, 1> : v == 3 ? (const void*)gemm_nvfp4_large_kernel<0, 3>
-               : v == 7 ? (const void*)gemm_nvfp4_large_kernel<0, 7> : v == 2 ? (const void*)gemm_nvfp4_large_kernel<0, 2> : fn;
-            (void)hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-        }
-        if (!attr_set[f32]) {
-            if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
-                return METIS_E_DEVICE;
-            attr_set[f32] = true;
-        }
-        const int tiles_m = (int)((M + L_BM - 1) / L_BM), tiles_n = (int)((N + L_BN - 1) / L_BN);
-        const int total = tiles_m * tiles_n;
-        const unsigned grid_x = (unsigned)(((total + 7) / 8) * 8);
-        const uint8_t *ac = (const uint8_t*)a_codes, *as = (const uint8_t*)a_scales, *bc = (const uint8_t*)b_codes,
-                      *bs = (const uint8_t*)b_scales;
-        const uint16_t *tp = (const uint16_t*)t, *up = (const uint16_t*)u, *bp = (const uint16_t*)bias;
-        int Mi = (int)M, Ni = (int)N, Ki = (int)K, ri = (int)r, tmi = tiles_m, tni = tiles_n;
-        void* args[] = {&ac, &as, &a_unit, &bc, &bs, &b_unit, &Mi, &Ni, &Ki, &tp, &up, &ri, &bp, &out, &tmi, &tni};
-        if (hipLaunchKernel(fn, dim3(grid_x), dim3(256), args, lds_bytes, st) != hipSuccess) {
-            (void)hipGetLastError();
-            return METIS_E_LAUNCH;
-        }
-        return METIS_OK;
+        if (getenv("METIS_GEMM_W4"))
+            return launch_large<2>(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st);
+        return launch_large<4>(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st);
     }
     constexpr int BM = 128, BN = 128;
     dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM));

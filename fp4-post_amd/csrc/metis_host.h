@@ -59,4 +59,9 @@ int gemm_nvfp4(const void* a_codes, const void* a_scales, const float* a_unit, c
                const float* b_unit, int64_t M, int64_t N, int64_t K, const void* t, const void* u, int64_t r,
                const void* bias, void* out, int out_dtype, hipStream_t st);
 
+int expand_f16(const void* codes, const void* scales, int64_t rows, int64_t cols, void* out, hipStream_t st);
+int gemm_expanded(const void* a_exp, const float* a_unit, const void* b_exp, const float* b_unit, int64_t M, int64_t N,
+                  int64_t K, const void* t, const void* u, int64_t r, const void* bias, void* out, int out_dtype,
+                  hipStream_t st);
+
 }  // namespace metis

@@ -165,6 +165,21 @@ int metis_linear_fwd(const void *a_codes, const void *a_scales, const float *a_u
                      const void *bias, void *out, int out_dtype, void *stream);
 
 /*
+ * Expanded operands for compute-bound shapes.  metis_nvfp4_expand_f16 writes, for a packed tensor,
+ *   out[i,k] = e2m1(code) * e4m3(scale) * 2^-8   as binary16 [rows, cols]   (exact; unit not applied)
+ * and metis_linear_fwd_expanded computes the same result as metis_linear_fwd from two such tensors and
+ * the two units (it multiplies the accumulators by unit_a * unit_b * 2^16).  The inner loop then is MFMA
+ * and LDS reads only; the expansion costs 2 B/element of HBM and can be cached with a weight, as the
+ * reference caches its dequantized weight (src/Metis/Metis/bitlinear.py:563-589).
+ * Limits: K % 64 == 0, N % 4 == 0, r % 32 == 0.
+ */
+int metis_nvfp4_expand_f16(const void *codes, const void *scales, int64_t rows, int64_t cols, void *out,
+                           void *stream);
+int metis_linear_fwd_expanded(const void *a_exp, const float *a_unit, const void *b_exp, const float *b_unit,
+                              int64_t M, int64_t N, int64_t K, const void *t, const void *u, int64_t r,
+                              const void *bias, void *out, int out_dtype, void *stream);
+
+/*
  * grad_input[L,K] = deq(dY)[L,N] . deq(W)[N,K]   (src/Metis/Metis/bitlinear.py:507-508)
  *   dy_* : dY packed with blocks along N (metis_nvfp4_quant_sr_row of dY [L,N])
  *   wt_* : W packed with blocks along N  (metis_nvfp4_quant_col of W [N,K] -> [K, N/2])

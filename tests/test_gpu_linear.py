@@ -98,3 +98,22 @@ def test_dgrad_and_wgrad():
     # and both stay close to the unquantized gradients (FP4 noise level, not a parity bar)
     assert rel_fro(gx.cpu(), dy.double() @ w.double()) < 0.25
     assert rel_fro(gw.cpu(), dy.double().T @ x.double()) < 0.25
+
+
+def test_expanded_path_is_bit_identical_to_packed_path():
+    """metis_linear_fwd_expanded on exact f16 expansions == metis_linear_fwd on packed operands."""
+    from metis_hip import ops
+    M, N, K, r = 512, 768, 1024, 64
+    x = synthetic_activation(40, M, K)
+    w = _weights(41, N, K)
+    g = torch.Generator().manual_seed(42)
+    t = torch.randn(M, r, generator=g).bfloat16().cuda()
+    u = torch.randn(N, r, generator=g).bfloat16().cuda()
+    bias = torch.randn(N, generator=g).bfloat16().cuda()
+    px, pw = ops.quantize(x.cuda()), ops.quantize(w.cuda())
+    a = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, out_dtype=torch.float32, expanded=False)
+    b = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, out_dtype=torch.float32, expanded=True)
+    assert torch.equal(a, b)
+    # the expansion itself: e2m1 * e4m3 * 2^-8, exact
+    e = ops.expand(px).float() * 256.0 * px.unit
+    assert rel_fro(e.cpu(), ops.dequantize(px, torch.float32).cpu()) < 1e-6
