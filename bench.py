@@ -29,6 +29,11 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_PEAK_TFLOPS = 2516.6      # dense bf16/fp16 MFMA: 256 CU x 4096 flop/clk x 2.4 GHz
 QUANT_BYTES_PER_ELT = 2.5625   # 2 B read + 0.5 B codes + 1/16 B scale
 NORMQ_BYTES_PER_ELT = 4.5625   # + 2 B normed
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this workload, scaled by what the
+# same counters read for a 64 MiB copy (x2.0 reads, x1.0 writes); summary in profiles/hbm_traffic_pmc_config1_2_3.md
+TRAFFIC_GEMM_C3 = 661.3e6
+TRAFFIC_QUANT_C1 = 94.7e6
+TRAFFIC_NORMQ_C2 = 323.6e6
 
 
 def outlier_activation(torch, seed, rows, cols, device):
@@ -79,7 +84,7 @@ def cpu_baseline_linear(torch, x, v, s, u, res, budget_rows=2048):
     xs = x[:budget_rows].cpu()
     vc, sc, uc, rc = v.cpu(), s.cpu(), u.cpu(), res.cpu()
     reps, dt = 0, 0.0
-    while dt < 10.0 and reps < 8:                      # about 10-30 s of CPU work
+    while dt < 12.0 and reps < 64:                      # about 10-30 s of CPU work
         t0 = time.perf_counter()
         O.metis_forward(xs, vc, sc, uc, rc, None, p32=True)
         dt += time.perf_counter() - t0
@@ -221,17 +226,17 @@ def main():
                    "parity_mode": "P32", "parity_rel_fro_256_rows": err},
         "roofline": {"bound": "mfma", "kernel": "gemm_nvfp4_large_kernel", "achieved": round(gemm_tflops, 2),
                      "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(gemm_tflops / MFMA_PEAK_TFLOPS, 4),
-                     "traffic": None, "kernel_ms": round(gemm_ms, 4)},
+                     "traffic": TRAFFIC_GEMM_C3, "kernel_ms": round(gemm_ms, 4)},
         "quant": {"workload": "config 1: NVFP4 RNE quantize bf16 [8192,4096] (P32), codes+scales+unit",
                   "value": round(q_gbs, 1), "unit": "GB/s", "us_per_call": round(q_ms * 1e3, 2),
                   "roofline": {"bound": "hbm", "kernel": "quant_codes_kernel+quant_scales_kernel",
                                "achieved": round(q_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                               "frac": round(q_gbs / HBM_PEAK_GBS, 4), "traffic": None}},
+                               "frac": round(q_gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_QUANT_C1}},
         "rmsnorm_quant": {"workload": "config 2: fused RMSNorm->NVFP4 bf16 [16384,4096] (P32), normed+codes+scales",
                           "value": round(n_gbs, 1), "unit": "GB/s", "us_per_call": round(n_ms * 1e3, 2),
                           "roofline": {"bound": "hbm", "kernel": "rmsnorm_quant_kernel+quant_scales_kernel",
                                        "achieved": round(n_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                                       "frac": round(n_gbs / HBM_PEAK_GBS, 4), "traffic": None}},
+                                       "frac": round(n_gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_NORMQ_C2}},
     }
     if not args.no_cpu_baseline:
         torch_threads = torch.get_num_threads()

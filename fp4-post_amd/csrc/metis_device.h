@@ -17,18 +17,12 @@ constexpr int kMaxGroups = 4096;      // upper bound on workgroups that publish 
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
 
-// binary32 -> bf16 round-to-nearest-even, result widened back to binary32 (finite inputs).
-__device__ __forceinline__ float rb(float f)
+// binary32 -> bf16 round-to-nearest-even (hardware convert), result widened back to binary32.
+__device__ __forceinline__ uint32_t bf16_bits(float f)
 {
-    uint32_t u = __float_as_uint(f);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return __uint_as_float(u & 0xffff0000u);
+    return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)f);
 }
-__device__ __forceinline__ uint32_t bf16_bits(float f)   // RNE, finite inputs
-{
-    uint32_t u = __float_as_uint(f);
-    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-}
+__device__ __forceinline__ float rb(float f) { return __uint_as_float(bf16_bits(f) << 16); }
 template <int MODE> __device__ __forceinline__ float rd(float v) { return MODE ? rb(v) : v; }
 
 // a / 6 correctly rounded for every bf16-valued a (exhaustively checked on the host):

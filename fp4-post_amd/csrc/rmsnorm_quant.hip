@@ -26,6 +26,12 @@ __global__ __launch_bounds__(256) void rmsnorm_quant_kernel(const uint16_t* __re
     const float inv_is_div = (float)cols;                     // mean = sum / cols (a division, as torch.mean)
     float gmax = 0.0f;
     uint32_t parity = 0;
+    // gamma of the thread's first block stays in registers for every row (all of it when cols <= 4096)
+    float g0[kBlock] = {};
+    if (threadIdx.x < nbpr) {
+        const uint4* g = reinterpret_cast<const uint4*>(gamma + (int64_t)threadIdx.x * kBlock);
+        unpack16(g[0], g[1], g0);
+    }
     for (uint32_t row = blockIdx.x; row < rows; row += gridDim.x, parity ^= 1u) {
         float v[NBT][kBlock];
         float ss = 0.0f;
@@ -36,7 +42,7 @@ __global__ __launch_bounds__(256) void rmsnorm_quant_kernel(const uint16_t* __re
                 const uint4* p = reinterpret_cast<const uint4*>(x + (int64_t)row * cols + (int64_t)cb * kBlock);
                 unpack16(p[0], p[1], v[k]);
 #pragma unroll
-                for (int j = 0; j < kBlock; ++j) ss += v[k][j] * v[k][j];
+                for (int j = 0; j < kBlock; ++j) ss = fmaf(v[k][j], v[k][j], ss);
             }
         }
         ss = wave_sum(ss);
@@ -48,9 +54,14 @@ __global__ __launch_bounds__(256) void rmsnorm_quant_kernel(const uint16_t* __re
         for (int k = 0; k < NBT; ++k) {
             const uint32_t cb = threadIdx.x + k * 256u;
             if (cb < nbpr) {
-                const uint4* g = reinterpret_cast<const uint4*>(gamma + (int64_t)cb * kBlock);
                 float gm[kBlock], n[kBlock];
-                unpack16(g[0], g[1], gm);
+                if (k == 0) {
+#pragma unroll
+                    for (int j = 0; j < kBlock; ++j) gm[j] = g0[j];
+                } else {
+                    const uint4* g = reinterpret_cast<const uint4*>(gamma + (int64_t)cb * kBlock);
+                    unpack16(g[0], g[1], gm);
+                }
 #pragma unroll
                 for (int j = 0; j < kBlock; ++j) n[j] = rb(rb(v[k][j] * rstd) * gm[j]);
                 const uint32_t ob = row * nbpr + cb;
