@@ -420,6 +420,44 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_nvfp4_large_kernel(
         __syncthreads();
     }
 
+    // ---- epilogue, bf16 output with N % 8 == 0: each wave transposes its tile through its own slice of the
+    //      (now idle) LDS so that a store instruction writes 8 rows x 128 contiguous bytes instead of 32 rows x 16
+    if constexpr (!OUT_F32 && WN_WAVES == 4 && !(DBG & 32)) {
+        if ((N & 7) == 0) {
+            constexpr int CROW = 64 + 8;                              // halves per staged row (144 bytes: conflict-free)
+            uint16_t* cw = lds + wave * (128 * CROW);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const int nl = j * 32 + 8 * g + 4 * (lane >> 5);
+                        float v[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            v[e] = acc[i][j][4 * g + e];
+                            if (bias) v[e] += bf16_lo(bias[min(n0 + wn * WTN + nl + e, N - 1)]);
+                        }
+                        uint2 w;
+                        w.x = bf16_bits(v[0]) | (bf16_bits(v[1]) << 16);
+                        w.y = bf16_bits(v[2]) | (bf16_bits(v[3]) << 16);
+                        *reinterpret_cast<uint2*>(cw + (i * 32 + (lane & 31)) * CROW + nl) = w;
+                    }
+            // same wave reads back what it wrote: no workgroup barrier needed, only the wave's own LDS writes
+            __builtin_amdgcn_s_waitcnt(0xC07F);                       // lgkmcnt(0)
+            const int rsub = lane >> 3, chunk = lane & 7;
+            const int n = n0 + wn * WTN + chunk * 8;
+#pragma unroll
+            for (int it = 0; it < 16; ++it) {
+                const int ml = it * 8 + rsub;
+                const int m = m0 + wm * 128 + ml;
+                const uint4 w = *reinterpret_cast<const uint4*>(cw + ml * CROW + chunk * 8);
+                if (m < M && n < N) *reinterpret_cast<uint4*>((uint16_t*)out + (int64_t)m * N + n) = w;
+            }
+            return;
+        }
+    }
     // ---- epilogue.  acc[i][j][e]: n = 8*(e/4) + 4*(lane/32) + e%4, m = lane%32 within the tile
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
@@ -437,6 +475,7 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_nvfp4_large_kernel(
                     v[e] = acc[i][j][4 * g + e];
                     if (bias) v[e] += bf16_lo(bias[n + e]);
                 }
+                if ((DBG & 16) && v[0] != 12345.678f) continue;
                 if (OUT_F32) {
                     *reinterpret_cast<float4*>((float*)out + (int64_t)m * N + n) = make_float4(v[0], v[1], v[2], v[3]);
                 } else {
@@ -462,7 +501,7 @@ static int launch_large(const void* a_codes, const void* a_scales, const float* 
     if (const char* d = getenv("METIS_GEMM_DBG")) {
         const int v = atoi(d);
         fn = v == 1 ? (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 1> : v == 8 ? (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 8>
-           : v == 7 ? (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 7> : fn;
+           : v == 7 ? (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 7> : v == 16 ? (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 16> : v == 32 ? (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 32> : fn;
         (void)hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     }
     if (!attr_set[f32]) {

@@ -38,7 +38,9 @@ __global__ __launch_bounds__(256) void quant_codes_kernel(
         const uint32_t step = gridDim.x * 256u;
         uint32_t i = blockIdx.x * 256u + threadIdx.x;
         uint4 c0 = make_uint4(0u, 0u, 0u, 0u), c1 = c0;
+        const bool contiguous = ld == (int64_t)cols;            // uniform: no per-block integer division then
         auto src = [&](uint32_t blk) {
+            if (contiguous) return reinterpret_cast<const uint4*>(x) + 2 * (size_t)blk;
             const uint32_t row = blk / nbpr, cb = blk - row * nbpr;
             return reinterpret_cast<const uint4*>(x + (int64_t)row * ld + (int64_t)cb * kBlock);
         };
