@@ -18,7 +18,7 @@ struct Workspace {
     uint16_t* amax;
 };
 constexpr size_t kWsGmaxBytes = 4096 * 4;
-constexpr size_t kWsSyncBytes = 260 * 256;     // 1 + 64 + 64 + 128 words of the grid reduction, 256 bytes apart
+constexpr size_t kWsSyncBytes = 260 * 256;     // 1 KiB header + 4096 member words + 64 x 64 group-maximum copies, 8 bytes each
 
 inline size_t workspace_bytes(int64_t rows, int64_t cols)
 {

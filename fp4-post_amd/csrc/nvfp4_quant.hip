@@ -109,11 +109,12 @@ __global__ __launch_bounds__(256) void quant_scales_kernel(const uint16_t* __res
                                                            uint32_t nblocks)
 {
     __shared__ float smax[4];
-    const uint32_t nquads = (nblocks + 3u) / 4u;
+    const uint32_t nocts = nblocks / 8u;
+    const uint32_t step = gridDim.x * 256u;
     uint32_t q = blockIdx.x * 256u + threadIdx.x;
-    // first quad of parked maxima is requested before the reduction so that both round trips overlap
-    uint2 a = make_uint2(0u, 0u);
-    if (q < nquads && q * 4u + 4u <= nblocks) a = *reinterpret_cast<const uint2*>(ws_amax + q * 4u);
+    // first eight parked maxima are requested before the reduction so that both round trips overlap
+    uint4 a = make_uint4(0u, 0u, 0u, 0u);
+    if (q < nocts) a = reinterpret_cast<const uint4*>(ws_amax)[q];
     float m = 0.0f;
     for (uint32_t g = threadIdx.x; g < ngroups; g += 256u) m = fmaxf(m, __uint_as_float(ws_gmax[g]));
     m = wave_max(m);
@@ -124,162 +125,165 @@ __global__ __launch_bounds__(256) void quant_scales_kernel(const uint16_t* __res
     const float unit = rd<MODE>(block_scalar<MODE>(amax) / 448.0f);
     if (blockIdx.x == 0 && threadIdx.x == 0) *unit_out = unit;
 
-    for (; q < nquads; q += gridDim.x * 256u) {
-        const uint32_t base = q * 4u;
-        if (base + 4u <= nblocks) {
-            if (q >= gridDim.x * 256u) a = *reinterpret_cast<const uint2*>(ws_amax + base);
-            const float t0 = rd<MODE>(block_scalar<MODE>(bf16_lo(a.x)) / unit);
-            const float t1 = rd<MODE>(block_scalar<MODE>(bf16_hi(a.x)) / unit);
-            const float t2 = rd<MODE>(block_scalar<MODE>(bf16_lo(a.y)) / unit);
-            const float t3 = rd<MODE>(block_scalar<MODE>(bf16_hi(a.y)) / unit);
-            int w = __builtin_amdgcn_cvt_pk_fp8_f32(t0, t1, 0, false);
-            w = __builtin_amdgcn_cvt_pk_fp8_f32(t2, t3, w, true);
-            *reinterpret_cast<uint32_t*>(scales + base) = (uint32_t)w;
-        } else {
-            for (uint32_t k = base; k < nblocks; ++k) {
-                const float s = block_scalar<MODE>(__uint_as_float((uint32_t)ws_amax[k] << 16));
-                scales[k] = (uint8_t)e4m3_byte(rd<MODE>(s / unit));
-            }
-        }
+    auto four_bytes = [&](uint32_t w0, uint32_t w1) {
+        const float t0 = rd<MODE>(block_scalar<MODE>(bf16_lo(w0)) / unit);
+        const float t1 = rd<MODE>(block_scalar<MODE>(bf16_hi(w0)) / unit);
+        const float t2 = rd<MODE>(block_scalar<MODE>(bf16_lo(w1)) / unit);
+        const float t3 = rd<MODE>(block_scalar<MODE>(bf16_hi(w1)) / unit);
+        const int w = __builtin_amdgcn_cvt_pk_fp8_f32(t0, t1, 0, false);
+        return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(t2, t3, w, true);
+    };
+    while (q < nocts) {
+        const uint32_t nxt = q + step;
+        uint4 n = a;
+        if (nxt < nocts) n = reinterpret_cast<const uint4*>(ws_amax)[nxt];
+        uint2 o;
+        o.x = four_bytes(a.x, a.y);
+        o.y = four_bytes(a.z, a.w);
+        reinterpret_cast<uint2*>(scales)[q] = o;
+        a = n; q = nxt;
+    }
+    // ragged tail (block count not a multiple of eight)
+    for (uint32_t k = nocts * 8u + blockIdx.x * 256u + threadIdx.x; k < nblocks; k += step) {
+        const float s = block_scalar<MODE>(__uint_as_float((uint32_t)ws_amax[k] << 16));
+        scales[k] = (uint8_t)e4m3_byte(rd<MODE>(s / unit));
     }
 }
 
 // ---------------------------------------------------------------------------------------------
-// Single-launch variant for round-to-nearest row quantization: both phases in one cooperative
-// kernel.  Each thread keeps the maxima of its (at most NB) blocks in registers across a grid-wide
-// reduction, so neither the parked maxima nor a second launch are needed.
+// Single-launch variant for round-to-nearest row quantization (opt-in): both phases in one kernel
+// whose workgroups are all resident at once.  Each thread keeps the maxima of its (at most NB)
+// blocks in registers across a grid-wide reduction, so neither the parked maxima nor a second
+// launch are needed.
 //
-// Grid-wide maximum without a stall: workgroups ARRIVE as soon as their block maxima are known,
-// compute and store their codes while the reduction propagates, and only then WAIT for it.
-// Device-scope atomics to one address serialise at ~11 ns each on this part, so arrivals go
-// through a two-level tree: workgroup b uses group j = b % 64 (sub-counter, maximum slot and poll
-// flag of its own, 256 bytes apart), the last arriver of a group bumps the top counter, and the
-// last group folds the 64 maxima and publishes {generation + 1, maximum} to the 64 flags.
-// All traffic is relaxed device-scope atomics whose completion is waited for where order matters;
-// no cache write-back or invalidate is involved.  Counters are restored to zero and the slots of
-// the other generation parity are cleared on the way, so the words only need zero-filling once.
-// The wait is bounded: after kSpinLimit polls a workgroup raises the time-out word and carries
-// on, so every wave always exits.
+// Grid-wide maximum from tagged words, no read-modify-write traffic at all.  A call's tag is the
+// 48-bit generation counter of the workspace plus one.  Workgroup b belongs to group j = b % 64
+// as member b / 64 and publishes {tag, its maximum as bf16} as ONE 64-bit store to its own word.
+// Wave 0 of member 0 polls the (at most 64) words of its group with one load per lane until all
+// carry the tag, folds them and stores {tag, group maximum} into a private copy for each of the
+// 64 groups; wave 0 of every workgroup polls its group's copy of the 64 group maxima the same way.
+// Tag and value share a word, so no ordering between locations is needed: relaxed device-scope
+// loads and stores only, and no line is polled by more than one group's members.
+// Workgroup 0 advances the generation counter once its own wait is over, by which time every
+// workgroup has read it.  The words only need zero-filling once.  The wait is bounded: after
+// kSpinLimit polls a workgroup raises the time-out word and carries on, so every wave always exits.
 // ---------------------------------------------------------------------------------------------
 constexpr uint32_t kSpinLimit = 1u << 20;
-constexpr uint32_t kGroups = 64;
-// word offsets inside the synchronisation area (uint32 units; 64 words = 256 bytes apart)
-__device__ __forceinline__ uint32_t* sync_top(uint32_t* s) { return s; }
+constexpr uint32_t kGroups = 64;                 // groups, and the most members a group can have
+constexpr int kFusedMaxGrid = kGroups * kGroups;
+// locations inside the synchronisation area (uint32 units)
+__device__ __forceinline__ uint64_t* sync_generation(uint32_t* s) { return reinterpret_cast<uint64_t*>(s); }
 __device__ __forceinline__ uint32_t* sync_timeout(uint32_t* s) { return s + 32; }
-__device__ __forceinline__ uint32_t* sync_sub(uint32_t* s, uint32_t j) { return s + 64u * (1u + j); }
-__device__ __forceinline__ uint64_t* sync_flag(uint32_t* s, uint32_t j) { return reinterpret_cast<uint64_t*>(s + 64u * (65u + j)); }
-__device__ __forceinline__ uint32_t* sync_slot(uint32_t* s, uint32_t parity, uint32_t j) { return s + 64u * (129u + parity * 64u + j); }
+__device__ __forceinline__ uint64_t* sync_member(uint32_t* s, uint32_t j, uint32_t m)
+{
+    return reinterpret_cast<uint64_t*>(s + 256) + j * kGroups + m;
+}
+// group maxima as seen by reader group g: a private copy per group so that no line has more than
+// a group's worth of pollers (device-scope accesses to one line are served one after another)
+__device__ __forceinline__ uint64_t* sync_copy(uint32_t* s, uint32_t g, uint32_t j)
+{
+    return reinterpret_cast<uint64_t*>(s + 256 + 2 * kGroups * kGroups) + g * kGroups + j;
+}
 
 #define METIS_AT_LOAD(p) __hip_atomic_load((p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
 #define METIS_AT_STORE(p, v) __hip_atomic_store((p), (v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-#define METIS_AT_ADD(p, v) __hip_atomic_fetch_add((p), (v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-#define METIS_AT_MAX(p, v) __hip_atomic_fetch_max((p), (v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-#define METIS_AT_XCHG(p, v) __hip_atomic_exchange((p), (v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
 
 struct GridMaxState {
     float wave_part[4];
-    uint32_t gen;
     float result;
 };
 
-// Called by every thread of every workgroup, once.  Publishes the workgroup maximum and arrives.
-__device__ __forceinline__ void grid_max_arrive(float thread_max, uint32_t* sync, GridMaxState& sh)
+// Wave 0 of every workgroup, at kernel start: the tag of this call (other waves get 0, unused).
+__device__ __forceinline__ uint64_t grid_max_begin(uint32_t* sync)
 {
-    float m = wave_max(thread_max);
+    return threadIdx.x < 64 ? METIS_AT_LOAD(sync_generation(sync)) + 1u : 0u;
+}
+
+// Called by every thread of every workgroup, once: publishes the workgroup maximum (a bf16 value).
+__device__ __forceinline__ void grid_max_arrive(float thread_max, uint64_t tag, uint32_t* sync, GridMaxState& sh)
+{
+    const float m = wave_max(thread_max);
     if ((threadIdx.x & 63) == 0) sh.wave_part[threadIdx.x >> 6] = m;
     __syncthreads();
-    if (threadIdx.x < 64) {
-        const uint32_t lane = threadIdx.x;
-        const uint32_t j = blockIdx.x % kGroups;
-        const uint32_t ngroups = gridDim.x < kGroups ? gridDim.x : kGroups;
-        uint32_t gen = 0u, finalize = 0u;
-        if (lane == 0) {
-            gen = (uint32_t)METIS_AT_LOAD(sync_flag(sync, j));     // low word: generation left by the previous call
-            m = fmaxf(fmaxf(sh.wave_part[0], sh.wave_part[1]), fmaxf(sh.wave_part[2], sh.wave_part[3]));
-            uint32_t o = METIS_AT_MAX(sync_slot(sync, gen & 1u, j), __float_as_uint(m));
-            asm volatile("s_waitcnt vmcnt(0)" ::"v"(o) : "memory");   // maximum in place before arriving
-            const uint32_t members = (gridDim.x + kGroups - 1u - j) / kGroups;
-            o = METIS_AT_ADD(sync_sub(sync, j), 1u);
-            if (o == members - 1u) {
-                METIS_AT_STORE(sync_sub(sync, j), 0u);             // restored for the next call (ordered by kernel end)
-                o = METIS_AT_ADD(sync_top(sync), 1u);
-                if (o == ngroups - 1u) {
-                    METIS_AT_STORE(sync_top(sync), 0u);
-                    finalize = 1u;
-                }
-            }
-            sh.gen = gen;
-        }
-        gen = __builtin_amdgcn_readfirstlane(gen);
-        finalize = __builtin_amdgcn_readfirstlane(finalize);
-        if (finalize) {                                            // wave 0 of the very last arriver
-            uint32_t v = lane < ngroups ? METIS_AT_LOAD(sync_slot(sync, gen & 1u, lane)) : 0u;
-            v = __float_as_uint(wave_max(__uint_as_float(v)));
-            METIS_AT_STORE(sync_slot(sync, (gen + 1u) & 1u, lane), 0u);
-            METIS_AT_STORE(sync_flag(sync, lane), ((uint64_t)v << 32) | (uint64_t)(gen + 1u));
-        }
+    if (threadIdx.x == 0) {
+        const float g = fmaxf(fmaxf(sh.wave_part[0], sh.wave_part[1]), fmaxf(sh.wave_part[2], sh.wave_part[3]));
+        METIS_AT_STORE(sync_member(sync, blockIdx.x % kGroups, blockIdx.x / kGroups), (tag << 16) | (uint64_t)(__float_as_uint(g) >> 16));
     }
 }
 
-// Called by every thread after grid_max_arrive(); returns the tensor-wide maximum.
-__device__ __forceinline__ float grid_max_wait(uint32_t* sync, GridMaxState& sh)
+// Wave-wide: polls one word per lane (lanes >= count are idle) until all carry the tag; returns the
+// maximum of the bf16 payloads.
+__device__ __forceinline__ float poll_tagged_max(const uint64_t* words, uint32_t count, uint64_t tag, uint32_t* sync)
 {
-    if (threadIdx.x == 0) {
-        const uint32_t j = blockIdx.x % kGroups;
-        const uint32_t want = sh.gen + 1u;
-        uint64_t f = METIS_AT_LOAD(sync_flag(sync, j));
-        uint32_t polls = 0;
-        while ((uint32_t)f != want) {
-            if (++polls > kSpinLimit) {
-                METIS_AT_STORE(sync_timeout(sync), 1u);
-                break;
-            }
-            __builtin_amdgcn_s_sleep(1);
-            f = METIS_AT_LOAD(sync_flag(sync, j));
+    const uint32_t lane = threadIdx.x & 63u;
+    uint64_t w = tag << 16;
+    uint32_t polls = 0;
+    for (;;) {
+        if (lane < count) w = METIS_AT_LOAD(words + lane);
+        if (__builtin_amdgcn_ballot_w64((w >> 16) != tag) == 0ull) break;
+        if (++polls > kSpinLimit) {
+            if (lane == 0) METIS_AT_STORE(sync_timeout(sync), 1u);
+            break;
         }
-        sh.result = __uint_as_float((uint32_t)(f >> 32));
+        __builtin_amdgcn_s_sleep(1);
+    }
+    return wave_max(__uint_as_float(((uint32_t)w & 0xffffu) << 16));
+}
+
+// Called by every thread after grid_max_arrive(); returns the tensor-wide maximum.
+__device__ __forceinline__ float grid_max_wait(uint64_t tag, uint32_t* sync, GridMaxState& sh)
+{
+    if (threadIdx.x < 64) {
+        const uint32_t j = blockIdx.x % kGroups;
+        const uint32_t ngroups = gridDim.x < kGroups ? gridDim.x : kGroups;
+        const uint32_t members = (gridDim.x + kGroups - 1u - j) / kGroups;
+        if (blockIdx.x < kGroups) {                               // member 0 folds its group and tells every group
+            const float gm = poll_tagged_max(sync_member(sync, j, 0), members, tag, sync);
+            if (threadIdx.x < ngroups) METIS_AT_STORE(sync_copy(sync, threadIdx.x, j), (tag << 16) | (uint64_t)(__float_as_uint(gm) >> 16));
+        }
+        const float all = poll_tagged_max(sync_copy(sync, j, 0), ngroups, tag, sync);
+        if (threadIdx.x == 0) {
+            sh.result = all;
+            if (blockIdx.x == 0) METIS_AT_STORE(sync_generation(sync), tag);
+        }
     }
     __syncthreads();
     return sh.result;
 }
 
+// One block in flight ahead of the one being encoded (as in phase 1 of the two-launch path), block
+// maxima kept in registers, and the arrival placed before the encoding of the thread's last block
+// so that part of the reduction latency is covered.
 template <int MODE, int NB>
 __global__ __launch_bounds__(256) void quant_fused_kernel(const uint16_t* __restrict__ x, uint2* __restrict__ codes,
-                                                          uint8_t* __restrict__ scales, float* __restrict__ unit_out,
-                                                          uint32_t* __restrict__ sync, uint32_t nblocks,
-                                                          uint32_t dbg)
+                                                               uint8_t* __restrict__ scales, float* __restrict__ unit_out,
+                                                               uint32_t* __restrict__ sync, uint32_t nblocks,
+                                                               uint32_t dbg)
 {
     __shared__ GridMaxState sh;
+    const uint64_t tag = grid_max_begin(sync);
     const uint32_t stride = gridDim.x * 256u;
     const uint32_t i0 = blockIdx.x * 256u + threadIdx.x;
-    uint4 raw[NB][2];
-#pragma unroll
-    for (int k = 0; k < NB; ++k) {                            // all loads in flight first
-        const uint32_t i = i0 + k * stride;
-        if (i < nblocks) {
-            const uint4* p = reinterpret_cast<const uint4*>(x) + 2 * (size_t)i;
-            raw[k][0] = p[0];
-            raw[k][1] = p[1];
-        } else {
-            raw[k][0] = raw[k][1] = make_uint4(0u, 0u, 0u, 0u);
-        }
-    }
-    // phase A: codes of each block as its data arrives (memory and VALU work overlap), then arrive
+    const uint4* xp = reinterpret_cast<const uint4*>(x);
+    uint4 c0 = make_uint4(0u, 0u, 0u, 0u), c1 = c0;
+    if (i0 < nblocks) { c0 = xp[2 * (size_t)i0]; c1 = xp[2 * (size_t)i0 + 1]; }
     float am[NB];
     float gmax = 0.0f;
 #pragma unroll
     for (int k = 0; k < NB; ++k) {
         const uint32_t i = i0 + k * stride;
+        uint4 n0 = make_uint4(0u, 0u, 0u, 0u), n1 = n0;
+        if (k + 1 < NB && i + stride < nblocks) { n0 = xp[2 * (size_t)(i + stride)]; n1 = xp[2 * (size_t)(i + stride) + 1]; }
         float v[kBlock];
         const float none[kBlock] = {};
-        unpack16(raw[k][0], raw[k][1], v);
+        unpack16(c0, c1, v);
         am[k] = block_amax(v);
         gmax = fmaxf(gmax, am[k]);
-        if (i < nblocks) codes[i] = (dbg & 4u) ? make_uint2(raw[k][0].x ^ raw[k][1].y, raw[k][0].z) : encode_block<MODE, false>(v, block_scalar<MODE>(am[k]), none);
+        if (k == NB - 1 && !(dbg & 1u)) grid_max_arrive(gmax, tag, sync, sh);
+        if (i < nblocks) codes[i] = encode_block<MODE, false>(v, block_scalar<MODE>(am[k]), none);
+        c0 = n0; c1 = n1;
     }
-    if (!(dbg & 1u)) grid_max_arrive(gmax, sync, sh);
-    // phase C: tensor unit and scale bytes
-    const float amax = (dbg & 2u) ? 6.0f : grid_max_wait(sync, sh);
+    const float amax = (dbg & 2u) ? 6.0f : grid_max_wait(tag, sync, sh);
     const float unit = rd<MODE>(block_scalar<MODE>(amax) / 448.0f);          // quant.py:21-22
     if (i0 == 0) *unit_out = unit;
 #pragma unroll
@@ -339,7 +343,7 @@ static int grid_for(uint32_t work_items)
 int launch_scales(int mode, const Workspace& ws, uint32_t ngroups, void* scales, float* unit, uint32_t nblocks,
                   hipStream_t st)
 {
-    const int g2 = grid_for((nblocks + 3) / 4);
+    const int g2 = grid_for((nblocks + 7) / 8);
     if (mode == 0)
         hipLaunchKernelGGL((quant_scales_kernel<0>), dim3(g2), dim3(256), 0, st, ws.amax, ws.gmax, ngroups,
                            (uint8_t*)scales, unit, nblocks);
@@ -349,7 +353,7 @@ int launch_scales(int mode, const Workspace& ws, uint32_t ngroups, void* scales,
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 
-// Co-resident workgroups of the fused kernel on the current device (0 = cooperative launch unavailable).
+// Co-resident workgroups of the single-launch kernel on the current device (0 = unknown).
 template <int MODE, int NB>
 static int fused_capacity()
 {
@@ -357,13 +361,9 @@ static int fused_capacity()
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
     if (cached[dev] == 0) {
-        int coop = 0, per_cu = 0;
-        if (hipDeviceGetAttribute(&coop, hipDeviceAttributeCooperativeLaunch, dev) != hipSuccess || !coop) cached[dev] = -1;
-        else if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, quant_fused_kernel<MODE, NB>, 256, 0) != hipSuccess ||
-                 per_cu <= 0)
-            cached[dev] = -1;
-        else
-            cached[dev] = per_cu * device_cus();
+        int per_cu = 0;
+        const hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, quant_fused_kernel<MODE, NB>, 256, 0);
+        cached[dev] = (e != hipSuccess || per_cu <= 0) ? -1 : per_cu * device_cus();
     }
     return cached[dev] < 0 ? 0 : cached[dev];
 }
@@ -373,26 +373,13 @@ static int try_fused(const void* x, void* codes, void* scales, float* unit, cons
                      hipStream_t st)
 {
     int cap = fused_capacity<MODE, NB>();
-    if (cap > kMaxGroups) cap = kMaxGroups;
+    if (cap > kFusedMaxGrid) cap = kFusedMaxGrid;
     const int64_t need = ((int64_t)nblocks + 256 * NB - 1) / (256 * NB);
-    if (getenv("METIS_DEBUG")) fprintf(stderr, "[metis] fused NB=%d cap=%d need=%ld\n", NB, cap, (long)need);
     if (cap <= 0 || need > cap) return 1;                      // does not fit: caller picks another path
-    const uint16_t* xp = (const uint16_t*)x;
-    uint2* cp = (uint2*)codes;
-    uint8_t* sp = (uint8_t*)scales;
-    uint32_t* sy = ws.sync;
     uint32_t dbg = getenv("METIS_DBG_FLAGS") ? (uint32_t)atoi(getenv("METIS_DBG_FLAGS")) : 0u;
-    void* args[] = {&xp, &cp, &sp, &unit, &sy, &nblocks, &dbg};
-    hipError_t e = getenv("METIS_COOP")
-                       ? hipLaunchCooperativeKernel((const void*)quant_fused_kernel<MODE, NB>, dim3((unsigned)need),
-                                                    dim3(256), args, 0, st)
-                       : hipLaunchKernel((const void*)quant_fused_kernel<MODE, NB>, dim3((unsigned)need), dim3(256), args, 0, st);
-    if (e != hipSuccess) {
-        if (getenv("METIS_DEBUG")) fprintf(stderr, "[metis] cooperative launch failed: %s\n", hipGetErrorString(e));
-        (void)hipGetLastError();
-        return 1;
-    }
-    return METIS_OK;
+    hipLaunchKernelGGL((quant_fused_kernel<MODE, NB>), dim3((unsigned)need), dim3(256), 0, st, (const uint16_t*)x,
+                       (uint2*)codes, (uint8_t*)scales, unit, ws.sync, nblocks, dbg);
+    return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 
 template <int MODE>
@@ -428,7 +415,7 @@ int quantize(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, bo
     if (!x || !codes || !scales || !unit) return METIS_E_ARG;
     if (rows * cols / kBlock >= (int64_t)1 << 31) return METIS_E_ARG;
     if (!col && ((ld % 8) || ((uintptr_t)x % 16))) return METIS_E_ARG;     // 16-byte vector loads
-    if (((uintptr_t)codes % 8) || ((uintptr_t)scales % 4)) return METIS_E_ARG;
+    if (((uintptr_t)codes % 8) || ((uintptr_t)scales % 8)) return METIS_E_ARG;
     Workspace ws;
     int rc = carve_workspace(workspace, workspace_bytes, rows, cols, &ws);
     if (rc != METIS_OK) return rc;

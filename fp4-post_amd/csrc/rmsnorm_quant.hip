@@ -95,7 +95,7 @@ int rmsnorm_quantize(const void* x, const void* gamma, float eps, int64_t rows, 
     if (!x || !gamma || !codes || !scales || !unit) return METIS_E_ARG;
     if (cols > 256 * kBlock * 4) return METIS_E_ARG;          // a row is held in registers: at most 16384 columns
     if (rows * cols / kBlock >= (int64_t)1 << 31) return METIS_E_ARG;
-    if (((uintptr_t)x % 16) || ((uintptr_t)gamma % 16) || ((uintptr_t)codes % 8) || ((uintptr_t)scales % 4) ||
+    if (((uintptr_t)x % 16) || ((uintptr_t)gamma % 16) || ((uintptr_t)codes % 8) || ((uintptr_t)scales % 8) ||
         (normed && ((uintptr_t)normed % 16)))
         return METIS_E_ARG;
     Workspace ws;

@@ -232,3 +232,20 @@ def test_full_size_config1(ops, tag, mode):
     flip = torch.where(nz, 8, 0).to(torch.uint8)
     flip = flip[:, 0::2] | (flip[:, 1::2] << 4)
     assert torch.equal(pn.codes, p.codes ^ flip)
+
+
+@pytest.mark.parametrize("tag,mode", MODES)
+def test_single_launch_variant_matches_two_launch_path(ops, monkeypatch, tag, mode):
+    """The opt-in single-launch kernel (grid-wide reduction through tagged words) gives the same
+    bytes as the default two-launch path, call after call on one workspace (the generation tag
+    advances each time) and across sizes that change the number of groups and members."""
+    shapes = [(8192, 4096), (16, 16), (64, 256), (4096, 1536), (16384, 4096), (1000, 48), (8192, 4096), (2, 32)]
+    for k, (r, c) in enumerate(shapes):
+        x = synthetic_activation(300 + k, r, c).cuda()
+        monkeypatch.delenv("METIS_FUSED_QUANT", raising=False)
+        ref = ops.quantize(x, mode)
+        monkeypatch.setenv("METIS_FUSED_QUANT", "1")
+        for rep in range(3):
+            got = ops.quantize(x, mode)
+            _check_packed(got, ref.codes.cpu(), ref.scales.cpu(), ref.unit.cpu(), f"shape {r}x{c} rep {rep} {tag}")
+    monkeypatch.delenv("METIS_FUSED_QUANT", raising=False)
