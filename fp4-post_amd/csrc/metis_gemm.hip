@@ -525,6 +525,178 @@ static int launch_large(const void* a_codes, const void* a_scales, const float* 
 }
 
 // ---------------------------------------------------------------------------------------------
+// Skinny kernel for M <= 64 (decode steps, tiny batches): HBM-bound on the packed weight bytes.
+// No LDS in the main loop and no barriers: a workgroup owns 32 output columns, its eight waves
+// split K between them, and every wave streams its slice of the 32 weight rows straight from
+// global memory into MFMA operands (the activations, at most 64 rows, come from L2).
+//
+// Lane l holds weight row n0 + l % 32; per iteration the two half-waves cover 64*C consecutive
+// elements of K, lane group l / 32 taking a contiguous run of 32*C elements (16*C bytes of codes,
+// 2*C scale bytes), so that with C = 4 the two lanes of a row consume one whole 128-byte line.
+// A contraction may visit K in any order as long as both operands agree: the m-th MFMA of an
+// iteration multiplies elements [8m, 8m+8) of every lane's run, and the activation rows are
+// fetched with the same mapping.  Partial sums of the eight waves meet in LDS at the end.
+// ---------------------------------------------------------------------------------------------
+template <int C>
+struct RunRegs {
+    uint4 c[C];                  // 32*C codes
+    uint32_t sc[(C + 1) / 2];    // 2*C scale bytes
+};
+
+template <int C>
+__device__ __forceinline__ void load_run(RunRegs<C>& r, const uint8_t* codes, const uint8_t* scales)
+{
+#pragma unroll
+    for (int c = 0; c < C; ++c) r.c[c] = reinterpret_cast<const uint4*>(codes)[c];
+    if constexpr (C == 1) r.sc[0] = *reinterpret_cast<const uint16_t*>(scales);
+    else if constexpr (C == 2) r.sc[0] = *reinterpret_cast<const uint32_t*>(scales);
+    else {
+        const uint2 w = *reinterpret_cast<const uint2*>(scales);
+        r.sc[0] = w.x; r.sc[1] = w.y;
+    }
+}
+
+// MFMA operand m (8 elements) of a run
+template <int C>
+__device__ __forceinline__ half8_t run_operand(const RunRegs<C>& r, int m)
+{
+    const uint4 q = r.c[m >> 2];
+    const uint32_t w = (m & 3) == 0 ? q.x : (m & 3) == 1 ? q.y : (m & 3) == 2 ? q.z : q.w;
+    const uint32_t byte = (r.sc[m >> 3] >> (8 * ((m >> 1) & 3))) & 0xffu;
+    return __builtin_bit_cast(half8_t, expand8(w, scale_pair(byte)));
+}
+
+template <int TM, int C, int WAVES, int OUT_F32>
+__global__ __launch_bounds__(64 * WAVES) void gemm_nvfp4_skinny_kernel(
+    const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const float* __restrict__ a_unit,
+    const uint8_t* __restrict__ b_codes, const uint8_t* __restrict__ b_scales, const float* __restrict__ b_unit,
+    int M, int N, int K, const uint16_t* __restrict__ t, const uint16_t* __restrict__ u, int r,
+    const uint16_t* __restrict__ bias, void* __restrict__ out)
+{
+    __shared__ float red[WAVES][TM * 16][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, hi = lane >> 5;
+    const int n0 = blockIdx.x * 32, m0 = blockIdx.y * 32 * TM;
+    const int kbytes = K / 2, kblocks = K / kBlock;
+    const int nrow = min(n0 + (lane & 31), N - 1);
+    const uint8_t* bc = b_codes + (int64_t)nrow * kbytes + hi * 16 * C;
+    const uint8_t* bs = b_scales + (int64_t)nrow * kblocks + hi * 2 * C;
+    const uint8_t *ac[TM], *as[TM];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        const int mrow = min(m0 + i * 32 + (lane & 31), M - 1);
+        ac[i] = a_codes + (int64_t)mrow * kbytes + hi * 16 * C;
+        as[i] = a_scales + (int64_t)mrow * kblocks + hi * 2 * C;
+    }
+    float16_t acc[TM];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][e] = 0.0f;
+
+    const int iters = K / (64 * C);
+    const int it1 = (wave + 1) * iters / WAVES;
+    for (int it = wave * iters / WAVES; it < it1; ++it) {
+        RunRegs<C> rb;
+        load_run<C>(rb, bc + (int64_t)it * 32 * C, bs + it * 4 * C);
+        RunRegs<C> ra[TM];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) load_run<C>(ra[i], ac[i] + (int64_t)it * 32 * C, as[i] + it * 4 * C);
+#pragma unroll
+        for (int m = 0; m < 4 * C; ++m) {
+            const half8_t fb = run_operand<C>(rb, m);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb, run_operand<C>(ra[i], m), acc[i], 0, 0, 0);
+        }
+    }
+    // tensor units (and the 2^8 * 2^8 of the scale placement)
+    const float us = (*a_unit) * (*b_unit) * 65536.0f;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][e] *= us;
+    // bf16 low-rank extension: slices of 32 columns dealt to the waves
+    for (int j0 = wave * 32; j0 < r; j0 += WAVES * 32) {
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const int j = j0 + q * 16 + hi * 8;
+            const bf16x8_t fu = *reinterpret_cast<const bf16x8_t*>(u + (int64_t)nrow * r + j);
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const int mrow = min(m0 + i * 32 + (lane & 31), M - 1);
+                const bf16x8_t ft = *reinterpret_cast<const bf16x8_t*>(t + (int64_t)mrow * r + j);
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fu, ft, acc[i], 0, 0, 0);
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) red[wave][i * 16 + e][lane] = acc[i][e];
+    __syncthreads();
+    // acc[i][e] of lane l: m = 32 i + l % 32, n = 8 (e / 4) + 4 (l / 32) + e % 4.  One (i, e / 4, l) per thread.
+    for (int id = threadIdx.x; id < TM * 256; id += 64 * WAVES) {
+        const int l = id & 63, g = (id >> 6) & 3, i = id >> 8;
+        const int m = m0 + i * 32 + (l & 31), n = n0 + 8 * g + 4 * (l >> 5);
+        float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] += red[w][i * 16 + 4 * g + e][l];
+        if (m >= M || n >= N) continue;                        // N % 4 == 0 is required
+        if (bias)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] += bf16_lo(bias[n + e]);
+        if (OUT_F32) {
+            *reinterpret_cast<float4*>((float*)out + (int64_t)m * N + n) = make_float4(v[0], v[1], v[2], v[3]);
+        } else {
+            uint2 w;
+            w.x = bf16_bits(v[0]) | (bf16_bits(v[1]) << 16);
+            w.y = bf16_bits(v[2]) | (bf16_bits(v[3]) << 16);
+            *reinterpret_cast<uint2*>((uint16_t*)out + (int64_t)m * N + n) = w;
+        }
+    }
+}
+
+template <int TM, int C, int WAVES>
+static int launch_skinny(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes,
+                         const void* b_scales, const float* b_unit, int64_t M, int64_t N, int64_t K, const void* t,
+                         const void* u, int64_t r, const void* bias, void* out, int out_dtype, hipStream_t st)
+{
+    const dim3 grid((unsigned)((N + 31) / 32), (unsigned)((M + 32 * TM - 1) / (32 * TM))), block(64 * WAVES);
+#define METIS_SK(F) hipLaunchKernelGGL((gemm_nvfp4_skinny_kernel<TM, C, WAVES, F>), grid, block, 0, st, (const uint8_t*)a_codes, \
+                                       (const uint8_t*)a_scales, a_unit, (const uint8_t*)b_codes, (const uint8_t*)b_scales,   \
+                                       b_unit, (int)M, (int)N, (int)K, (const uint16_t*)t, (const uint16_t*)u, (int)r,        \
+                                       (const uint16_t*)bias, out)
+    if (out_dtype == METIS_DTYPE_F32) METIS_SK(1); else METIS_SK(0);
+#undef METIS_SK
+    return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
+}
+
+// Shape heuristics from measurements at 3584/4608/18944-wide projections: wide runs whenever alignment
+// allows; two row tiles per wave when M > 32 unless that leaves fewer workgroups than half the CUs (then the
+// row tiles go to separate workgroups); four waves per workgroup only when there are plenty of
+// workgroups anyway.
+static int gemm_skinny(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes,
+                       const void* b_scales, const float* b_unit, int64_t M, int64_t N, int64_t K, const void* t,
+                       const void* u, int64_t r, const void* bias, void* out, int out_dtype, hipStream_t st)
+{
+    const bool al8 = ((uintptr_t)a_scales % 8) == 0 && ((uintptr_t)b_scales % 8) == 0;
+    const int c = (K % 256 == 0 && al8) ? 4 : 1;
+    const int64_t tiles_n = (N + 31) / 32;
+    const int tm = (M <= 32 || tiles_n < device_cus() / 2) ? 1 : 2;
+    const int waves = (tm == 1 && M <= 32 && tiles_n >= 2 * device_cus()) ? 4 : 8;
+#define METIS_SKL(TM, C, W) return launch_skinny<TM, C, W>(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st)
+    if (tm == 1) {
+        if (waves == 4) { if (c == 4) METIS_SKL(1, 4, 4); else METIS_SKL(1, 1, 4); }
+        else { if (c == 4) METIS_SKL(1, 4, 8); else METIS_SKL(1, 1, 8); }
+    } else {
+        if (c == 4) METIS_SKL(2, 4, 8); else METIS_SKL(2, 1, 8);
+    }
+#undef METIS_SKL
+}
+
+// ---------------------------------------------------------------------------------------------
 // Expansion of a packed tensor to binary16: value = e2m1(code) * e4m3(scale) * 2^-8, exact.
 // One thread per 8 elements (one dword of codes -> 16 bytes).  HBM-bound: 0.5625 B read, 2 B written
 // per element.  The expanded tensor is what gemm_f16_large_kernel consumes; it is derived data that
@@ -777,7 +949,7 @@ int gemm_nvfp4(const void* a_codes, const void* a_scales, const float* a_unit, c
     if (N % 4 || r % 32 || (r > 0 && (!t || !u))) return METIS_E_ARG;
     if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return METIS_E_ARG;
     if (((uintptr_t)a_codes % 16) || ((uintptr_t)b_codes % 16) || ((uintptr_t)a_scales % 2) || ((uintptr_t)b_scales % 2) ||
-        ((uintptr_t)out % 16))
+        ((uintptr_t)out % 16) || ((uintptr_t)t % 16) || ((uintptr_t)u % 16))
         return METIS_E_ARG;
     if (K % 32) return METIS_E_ARG;                            // 16-byte code chunks: rows must stay 16-byte aligned
     if (M == 0 || N == 0) return METIS_OK;
@@ -786,6 +958,8 @@ int gemm_nvfp4(const void* a_codes, const void* a_scales, const float* a_unit, c
             return launch_large<2>(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st);
         return launch_large<4>(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st);
     }
+    if (M <= 64 && K % 64 == 0 && !getenv("METIS_GEMM_SMALL"))
+        return gemm_skinny(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st);
     constexpr int BM = 128, BN = 128;
     dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM));
     if (out_dtype == METIS_DTYPE_F32)

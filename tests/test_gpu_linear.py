@@ -20,7 +20,10 @@ def _weights(seed, n, k, scale=0.02):
 
 
 @pytest.mark.parametrize("M,N,K", [(128, 128, 64), (256, 384, 512), (100, 132, 96), (1, 64, 32), (64, 3584, 1536),
-                                   (300, 260, 4096)])
+                                   (300, 260, 4096),
+                                   # skinny path (M <= 64): narrow and wide runs, ragged N, one and two row tiles
+                                   (7, 100, 64), (33, 96, 320), (32, 2052, 768), (1, 3584, 3584), (64, 4736, 3584),
+                                   (16, 1536, 8960)])
 def test_gemm_against_fp64_of_dequantized_operands(M, N, K):
     from metis_hip import ops
     x = synthetic_activation(10 + M, M, K)
@@ -53,7 +56,8 @@ def test_gemm_tiny_blocks_with_subnormal_scales():
     assert rel_fro(out.cpu(), want.cpu()) <= 1e-5
 
 
-@pytest.mark.parametrize("M,N,K,r", [(128, 256, 256, 32), (200, 192, 512, 64)])
+@pytest.mark.parametrize("M,N,K,r", [(128, 256, 256, 32), (200, 192, 512, 64), (48, 260, 256, 64), (5, 96, 192, 32),
+                                     (64, 512, 1024, 320)])
 def test_metis_forward_with_lowrank_extension_and_bias(M, N, K, r):
     """out = (X V^T * s) U^T + QDQ(X) QDQ(R)^T + b against the op-for-op oracle (P32)."""
     from metis_hip import ops
@@ -117,3 +121,30 @@ def test_expanded_path_is_bit_identical_to_packed_path():
     # the expansion itself: e2m1 * e4m3 * 2^-8, exact
     e = ops.expand(px).float() * 256.0 * px.unit
     assert rel_fro(e.cpu(), ops.dequantize(px, torch.float32).cpu()) < 1e-6
+
+
+@pytest.mark.parametrize("M,N,K,r", [(64, 4736, 3584, 64), (17, 2052, 2048, 0), (1, 4608, 3584, 32), (40, 1536, 8960, 64),
+                                     (64, 18944, 3584, 64)])
+def test_decode_shapes_with_lowrank_and_bias(M, N, K, r):
+    """M <= 64 runs on the skinny kernel (waves split K, partial sums meet in LDS); every layout the shape
+    heuristics can pick is covered: one or two row tiles per wave, row tiles in separate workgroups,
+    four or eight waves."""
+    from metis_hip import ops
+    g = torch.Generator().manual_seed(77)
+    x = synthetic_activation(40 + M, M, K).cuda()
+    w = _weights(41 + N, N, K).cuda()
+    t = u = None
+    if r:
+        t = torch.randn(M, r, generator=g).bfloat16().cuda()
+        u = torch.randn(N, r, generator=g).bfloat16().cuda()
+    bias = (torch.randn(N, generator=g) * 0.1).bfloat16().cuda()
+    px, pw = ops.quantize(x), ops.quantize(w)
+    got = ops.linear_fwd(px, pw, t=t, u=u, bias=bias)
+    got32 = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, out_dtype=torch.float32)
+    want = ops.dequantize(px, torch.float32).double() @ ops.dequantize(pw, torch.float32).double().T
+    if r:
+        want = want + t.double() @ u.double().T
+    want = want + bias.double()
+    torch.cuda.synchronize()
+    assert rel_fro(got32.cpu(), want.cpu()) <= 1e-5
+    assert rel_fro(got.cpu(), want.cpu().bfloat16()) <= TOL
