@@ -115,6 +115,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-decode", action="store_true", help="skip the config-5 decode-layer leg")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures the one-GPU hot path only: this build has no multi-GPU path "
@@ -208,6 +209,53 @@ def main():
     n_bytes = h.numel() * NORMQ_BYTES_PER_ELT
     n_gbs = n_bytes / (n_ms * 1e-3) / 1e9
 
+    # ------------------------------------------------------------------ config 5, decode step: the seven
+    # projections of one Qwen2.5-7B decoder layer at M = 64 rows (rank 64), packed weights streamed once
+    dec = None
+    if not args.no_decode:
+        shapes = [(3584, 3584), (512, 3584), (512, 3584), (3584, 3584), (18944, 3584), (18944, 3584), (3584, 18944)]
+        gd = torch.Generator().manual_seed(1005)
+        ws_, acts, lows = [], {}, []
+        for (n_, k_) in shapes:
+            ws_.append(ops.quantize((torch.randn(n_, k_, generator=gd) * 0.02).bfloat16().to(dev)))
+            if k_ not in acts:
+                acts[k_] = ops.quantize(torch.randn(64, k_, generator=gd).bfloat16().to(dev))
+            lows.append((torch.randn(64, 64, generator=gd).bfloat16().to(dev), torch.randn(n_, 64, generator=gd).bfloat16().to(dev)))
+        outs = [torch.empty(64, n_, dtype=torch.bfloat16, device=dev) for (n_, _) in shapes]
+
+        def layer():
+            s_ = torch.cuda.current_stream().cuda_stream
+            for pw_, (n_, k_), (t_, u_), o_ in zip(ws_, shapes, lows, outs):
+                a_ = acts[k_]
+                rc = L.metis_linear_fwd(a_.codes.data_ptr(), a_.scales.data_ptr(), a_.unit.data_ptr(), pw_.codes.data_ptr(),
+                                        pw_.scales.data_ptr(), pw_.unit.data_ptr(), 64, n_, k_, t_.data_ptr(), u_.data_ptr(), 64,
+                                        None, o_.data_ptr(), 0, s_)
+                assert rc == 0
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            layer()
+            torch.cuda.synchronize()
+            with torch.cuda.graph(graph, stream=side):
+                for _ in range(10):
+                    layer()
+        graph.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(10):
+            graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        d_us = e0.elapsed_time(e1) / 100 * 1e3
+        d_bytes = sum(n_ * k_ for n_, k_ in shapes) * (0.5 + 1.0 / 16)
+        d_flops = sum(2.0 * 64 * n_ * k_ for n_, k_ in shapes)
+        dec = {"workload": "config 5 decode: 7 projections of a Qwen2.5-7B layer, M=64, r=64, packed weights (graph replay)",
+               "us_per_layer": round(d_us, 1), "tflops": round(d_flops / d_us / 1e6, 1),
+               "roofline": {"bound": "hbm", "kernel": "gemm_nvfp4_skinny_kernel", "achieved": round(d_bytes / d_us / 1e3, 1),
+                            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(d_bytes / d_us / 1e3 / HBM_PEAK_GBS, 4),
+                            "traffic": None}}
+
     line = {
         "metric": "Metis NVFP4 linear TFLOP/s at 8192x4096x14336 (rank 64)",
         "value": round(value, 2),
@@ -238,6 +286,8 @@ def main():
                                        "achieved": round(n_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                        "frac": round(n_gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_NORMQ_C2}},
     }
+    if dec is not None:
+        line["decode_layer"] = dec
     if not args.no_cpu_baseline:
         torch_threads = torch.get_num_threads()
         cpu_tflops, cpu_dt, cpu_reps = cpu_baseline_linear(torch, x, v, s, u, res)

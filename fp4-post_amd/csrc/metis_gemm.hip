@@ -525,7 +525,8 @@ static int launch_large(const void* a_codes, const void* a_scales, const float* 
 }
 
 // ---------------------------------------------------------------------------------------------
-// Skinny kernel for M <= 64 (decode steps, tiny batches): HBM-bound on the packed weight bytes.
+// Skinny kernel for M <= 64 per workgroup row (decode steps, small batches): HBM-bound on the packed
+// weight bytes; taller inputs below 256 rows take one grid row per 64 rows.
 // No LDS in the main loop and no barriers: a workgroup owns 32 output columns, its eight waves
 // split K between them, and every wave streams its slice of the 32 weight rows straight from
 // global memory into MFMA operands (the activations, at most 64 rows, come from L2).
@@ -958,7 +959,7 @@ int gemm_nvfp4(const void* a_codes, const void* a_scales, const float* a_unit, c
             return launch_large<2>(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st);
         return launch_large<4>(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st);
     }
-    if (M <= 64 && K % 64 == 0 && !getenv("METIS_GEMM_SMALL"))
+    if (M < 256 && K % 64 == 0 && !getenv("METIS_GEMM_SMALL"))    // up to four 64-row passes over the weights beat a mostly empty 256-row tile
         return gemm_skinny(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st);
     constexpr int BM = 128, BN = 128;
     dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM));
