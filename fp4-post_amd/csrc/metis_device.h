@@ -23,6 +23,14 @@ __device__ __forceinline__ uint32_t bf16_bits(float f)
     return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)f);
 }
 __device__ __forceinline__ float rb(float f) { return __uint_as_float(bf16_bits(f) << 16); }
+// two roundings to bf16 at once, packed (first argument in the low half): one v_cvt_pk_bf16_f32
+typedef float metis_float2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 metis_bf16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t rb_pair(float lo, float hi)
+{
+    const metis_float2_t f = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, metis_bf16x2_t));
+}
 template <int MODE> __device__ __forceinline__ float rd(float v) { return MODE ? rb(v) : v; }
 
 // a / 6 correctly rounded for every bf16-valued a (exhaustively checked on the host):

@@ -32,6 +32,20 @@ __global__ __launch_bounds__(256) void rmsnorm_quant_kernel(const uint16_t* __re
         const uint4* g = reinterpret_cast<const uint4*>(gamma + (int64_t)threadIdx.x * kBlock);
         unpack16(g[0], g[1], g0);
     }
+    // the next row's bytes are requested before the current row is reduced and encoded
+    uint4 raw[NBT][2];
+    auto request = [&](uint32_t row) {
+#pragma unroll
+        for (int k = 0; k < NBT; ++k) {
+            const uint32_t cb = threadIdx.x + k * 256u;
+            if (cb < nbpr) {
+                const uint4* p = reinterpret_cast<const uint4*>(x + (int64_t)row * cols + (int64_t)cb * kBlock);
+                raw[k][0] = p[0];
+                raw[k][1] = p[1];
+            }
+        }
+    };
+    if (blockIdx.x < rows) request(blockIdx.x);
     for (uint32_t row = blockIdx.x; row < rows; row += gridDim.x, parity ^= 1u) {
         float v[NBT][kBlock];
         float ss = 0.0f;
@@ -39,12 +53,12 @@ __global__ __launch_bounds__(256) void rmsnorm_quant_kernel(const uint16_t* __re
         for (int k = 0; k < NBT; ++k) {
             const uint32_t cb = threadIdx.x + k * 256u;
             if (cb < nbpr) {
-                const uint4* p = reinterpret_cast<const uint4*>(x + (int64_t)row * cols + (int64_t)cb * kBlock);
-                unpack16(p[0], p[1], v[k]);
+                unpack16(raw[k][0], raw[k][1], v[k]);
 #pragma unroll
                 for (int j = 0; j < kBlock; ++j) ss = fmaf(v[k][j], v[k][j], ss);
             }
         }
+        if (row + gridDim.x < rows) request(row + gridDim.x);
         ss = wave_sum(ss);
         if ((threadIdx.x & 63) == 0) part[parity][threadIdx.x >> 6] = ss;
         __syncthreads();                                      // the other parity is free again after this barrier
@@ -62,14 +76,17 @@ __global__ __launch_bounds__(256) void rmsnorm_quant_kernel(const uint16_t* __re
                     const uint4* g = reinterpret_cast<const uint4*>(gamma + (int64_t)cb * kBlock);
                     unpack16(g[0], g[1], gm);
                 }
+                // bf16(bf16(x * rstd) * gamma), two elements per conversion; the packed pairs are the normed output
+                uint32_t w[8];
 #pragma unroll
-                for (int j = 0; j < kBlock; ++j) n[j] = rb(rb(v[k][j] * rstd) * gm[j]);
+                for (int j = 0; j < 8; ++j) {
+                    const uint32_t h = rb_pair(v[k][2 * j] * rstd, v[k][2 * j + 1] * rstd);
+                    w[j] = rb_pair(bf16_lo(h) * gm[2 * j], bf16_hi(h) * gm[2 * j + 1]);
+                    n[2 * j] = bf16_lo(w[j]);
+                    n[2 * j + 1] = bf16_hi(w[j]);
+                }
                 const uint32_t ob = row * nbpr + cb;
                 if (WRITE_NORMED) {
-                    uint32_t w[8];
-#pragma unroll
-                    for (int j = 0; j < 8; ++j)
-                        w[j] = (__float_as_uint(n[2 * j]) >> 16) | (__float_as_uint(n[2 * j + 1]) & 0xffff0000u);
                     uint4* o = reinterpret_cast<uint4*>(normed + (int64_t)ob * kBlock);
                     o[0] = make_uint4(w[0], w[1], w[2], w[3]);
                     o[1] = make_uint4(w[4], w[5], w[6], w[7]);
