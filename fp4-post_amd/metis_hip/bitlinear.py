@@ -126,9 +126,9 @@ class LinearLowbitFunction(torch.autograd.Function):
     def _prepare_input(input_: torch.Tensor, mean_cache=None, cache_key="default"):
         """Packed activation when the direct NVFP4 path applies, else the dequantized tensor."""
         F = LinearLowbitFunction
-        xin = input_.to(F.compute_dtype)
-        if not F.enable_activation_svd and not F.enable_nv_recipe and _packable(xin, F.q_forward_input):
-            return F.q_forward_input.pack(_flat2d(xin))
+        if not F.enable_activation_svd and not F.enable_nv_recipe and _packable(input_, F.q_forward_input):
+            # the kernels read bf16 values and take the arithmetic as a mode: no upcast copy of a bf16 tensor
+            return F.q_forward_input.pack(_flat2d(input_), arith=F.compute_dtype)
         return F.quantize_input(input_, mean_cache=mean_cache, cache_key=cache_key)
 
     @staticmethod
@@ -171,26 +171,34 @@ class LinearLowbitFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output):
         F = LinearLowbitFunction
-        grad_output = grad_output.to(F.compute_dtype)
         grad_bias = None
         if ctx.has_bias:
-            grad_bias = _flat2d(grad_output).sum(dim=0).to(torch.float32)
-        dy2 = _flat2d(grad_output)
+            grad_bias = _flat2d(grad_output).to(F.compute_dtype).sum(dim=0).to(torch.float32)
         if ctx.packed:
             input_, _ = ctx.saved_tensors
-            x2 = _flat2d(input_.to(F.compute_dtype))
-            L, N = dy2.shape
+            L, N = _flat2d(grad_output).shape
             qg, qi = F.q_backward_outputgrad, F.q_backward_input
-            if L % 16 == 0 and L % 32 == 0 and is_hip_nvfp4(qg) and is_hip_nvfp4(qi) and N % 32 == 0:
-                # dgrad: contraction over N; wgrad: contraction over tokens
-                p_dy = qg.pack(dy2)
-                pw_col = F.q_forward_weight.pack(ctx.weight_ref.to(F.compute_dtype), col=True)
-                gx = ops.linear_dgrad(p_dy, pw_col, out_dtype=grad_output.dtype if grad_output.dtype != torch.float16 else torch.float32)
-                gw = ops.linear_wgrad(qg.pack(dy2, col=True), qi.pack(x2, col=True))
-                return gx.reshape(*ctx.lead, gx.shape[-1]).to(grad_output.dtype), gw, grad_bias, None, None
+            if (L % 32 == 0 and is_hip_nvfp4(qg) and is_hip_nvfp4(qi) and N % 32 == 0
+                    and grad_output.dtype in (torch.float32, torch.bfloat16)):
+                # dgrad: contraction over N; wgrad: contraction over tokens.  Operands are packed straight from the
+                # tensors autograd hands over, in compute_dtype arithmetic (no upcast copies of bf16 tensors).
+                dy2, x2, cd = _flat2d(grad_output), _flat2d(input_), F.compute_dtype
+                p_dy = qg.pack(dy2, arith=cd)
+                pw_col = ctx.pw.transposed                    # lives as long as the (possibly cached) packed weight
+                if pw_col is None:
+                    pw_col = ctx.pw.transposed = F.q_forward_weight.pack(ctx.weight_ref, col=True, arith=cd)
+                gx_dtype = input_.dtype if input_.dtype in (torch.float32, torch.bfloat16) else torch.float32
+                gx = ops.linear_dgrad(p_dy, pw_col, out_dtype=gx_dtype)
+                gw = ops.linear_wgrad(qg.pack(dy2, col=True, arith=cd), qi.pack(x2, col=True, arith=cd))
+                return gx.reshape(*ctx.lead, gx.shape[-1]), gw, grad_bias, None, None
+            grad_output = grad_output.to(F.compute_dtype)
+            dy2 = _flat2d(grad_output)
+            x2 = _flat2d(input_.to(F.compute_dtype))
             xq = F.q_forward_input.quantize_dequantize(x2)
             wq = ctx.pw.dequantize(F.compute_dtype)
         else:
+            grad_output = grad_output.to(F.compute_dtype)
+            dy2 = _flat2d(grad_output)
             xq, wq, _ = ctx.saved_tensors
             xq = _flat2d(xq)
         if F.enable_backward_svd:
@@ -233,17 +241,23 @@ class LinearLowbit(nn.Module):
             init.uniform_(self.bias, -bound, bound)
 
     def forward(self, input, quantized_input=None):
-        weight_compute = self.weight.to(self.compute_dtype)
+        F = LinearLowbitFunction
         bias_compute = self.bias.to(self.compute_dtype) if self.bias is not None else None
+        if not F.enable_nv_recipe and _packable(self.weight, F.q_forward_weight) and self.weight.shape[0] % 4 == 0:
+            # kernel path: packed straight from the stored parameter in compute_dtype arithmetic, so a cache hit
+            # costs no pass over the weight at all
+            quantized_weight = self._get_quantized_weight(self.weight, arith=self.compute_dtype)
+            return F.apply(input, self.weight, bias_compute, quantized_weight, quantized_input)
+        weight_compute = self.weight.to(self.compute_dtype)
         quantized_weight = self._get_quantized_weight(weight_compute)
-        return LinearLowbitFunction.apply(input, weight_compute, bias_compute, quantized_weight, quantized_input)
+        return F.apply(input, weight_compute, bias_compute, quantized_weight, quantized_input)
 
     @torch.no_grad()
-    def _get_quantized_weight(self, weight_compute):
+    def _get_quantized_weight(self, weight_compute, arith=None):
         """Quantized weight, cached on Parameter._version when enabled (reference 563-589).  Returns a
         PackedNVFP4 when the kernel path applies, otherwise the dequantized tensor."""
         F = LinearLowbitFunction
-        key = (self.weight._version, weight_compute.device, weight_compute.dtype, F.q_forward_weight, F.enable_nv_recipe)
+        key = (self.weight._version, weight_compute.device, arith or weight_compute.dtype, F.q_forward_weight, F.enable_nv_recipe)
         if self.cache_quantized_weight and self._quantized_weight_cache is not None:
             cached_key, cached = self._quantized_weight_cache
             if cached_key == key:
@@ -251,7 +265,7 @@ class LinearLowbit(nn.Module):
         if F.enable_nv_recipe:
             raise NotImplementedError("enable_nv_recipe (random Hadamard rotation) is not implemented")
         if _packable(weight_compute, F.q_forward_weight) and weight_compute.shape[0] % 4 == 0:
-            q = F.q_forward_weight.pack(weight_compute)
+            q = F.q_forward_weight.pack(weight_compute, arith=arith)
         else:
             q = F.q_forward_weight.quantize_dequantize(weight_compute)
         if self.cache_quantized_weight:
@@ -276,6 +290,7 @@ class _MetisFusedFunction(torch.autograd.Function):
         out_dtype = torch.float32 if F.compute_dtype == torch.float32 else torch.bfloat16
         y = ops.linear_fwd(px, p_res, t=t, u=u.to(cd), bias=None if bias is None else bias.to(cd), out_dtype=out_dtype)
         ctx.save_for_backward(x, v, s, u, res, xv)
+        ctx.p_res = p_res
         ctx.has_bias = bias is not None
         ctx.lead = x.shape[:-1]
         return y.reshape(*ctx.lead, y.shape[-1]).to(F.compute_dtype)
@@ -298,9 +313,12 @@ class _MetisFusedFunction(torch.autograd.Function):
         # residual branch on re-quantized operands
         qg, qi = F.q_backward_outputgrad, F.q_backward_input
         if L % 32 == 0 and N % 32 == 0 and is_hip_nvfp4(qg) and is_hip_nvfp4(qi):
-            gx = gx + ops.linear_dgrad(qg.pack(dy2.to(F.compute_dtype)),
-                                       F.q_forward_weight.pack(res.to(F.compute_dtype), col=True), out_dtype=cd)
-            g_res = ops.linear_wgrad(qg.pack(dy2.to(F.compute_dtype), col=True), qi.pack(x2.to(F.compute_dtype), col=True))
+            ar = F.compute_dtype                               # arithmetic of the quantizers; the tensors stay bf16
+            p_res_col = ctx.p_res.transposed                   # lives as long as the (cached) packed residual
+            if p_res_col is None:
+                p_res_col = ctx.p_res.transposed = F.q_forward_weight.pack(res, col=True, arith=ar)
+            gx = gx + ops.linear_dgrad(qg.pack(dy2, arith=ar), p_res_col, out_dtype=cd)
+            g_res = ops.linear_wgrad(qg.pack(dy2, col=True, arith=ar), qi.pack(x2, col=True, arith=ar))
         else:
             dyq = F._quantize_wgrad_operand(dy2.to(F.compute_dtype), qg)
             xq = F.q_forward_input.quantize_dequantize(x2.to(F.compute_dtype))
@@ -423,7 +441,11 @@ class BitLinear(nn.Module):
             if isinstance(shared_input, PackedNVFP4) and r % 32 == 0 and self.ulinear.bias is None:
                 # one fused launch for both branches; it already is the "merged" evaluation, so the
                 # rollout switch changes nothing on this path
-                p_res = self.warmup_linear._get_quantized_weight(self.warmup_linear.weight.to(self.compute_dtype))
+                wl = self.warmup_linear
+                if not F.enable_nv_recipe and _packable(wl.weight, F.q_forward_weight) and wl.weight.shape[0] % 4 == 0:
+                    p_res = wl._get_quantized_weight(wl.weight, arith=self.compute_dtype)   # cache hit: no pass over W
+                else:
+                    p_res = wl._get_quantized_weight(wl.weight.to(self.compute_dtype))
                 if isinstance(p_res, PackedNVFP4):
                     return _MetisFusedFunction.apply(x, self.vlinear.weight, self.s, self.ulinear.weight,
                                                      self.warmup_linear.weight, self.warmup_linear.bias, shared_input, p_res)

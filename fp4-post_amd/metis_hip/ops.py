@@ -31,6 +31,7 @@ class PackedNVFP4:
     cols: int
     mode: int = MODE_P32
     expanded: torch.Tensor | None = None      # cached exact f16 expansion e2m1 * e4m3 * 2^-8, see expand()
+    transposed: "PackedNVFP4 | None" = None   # cached column-blocked packing of the same source tensor (dgrad operand)
 
     def dequantize(self, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
         return dequantize(self, dtype)

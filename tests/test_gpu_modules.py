@@ -174,10 +174,10 @@ def test_shared_activation_is_quantized_once_per_group():
     base = quant_func["nvfp4e2m1bnosr"]
     orig = base.pack.__func__
 
-    def counting(cls, x, col=False, noise=None):
+    def counting(cls, x, col=False, noise=None, arith=None):
         if not col and tuple(x.shape) == (96, 256):      # the activation, not the [N, 256] weights
             calls["n"] += 1
-        return orig(cls, x, col, noise)
+        return orig(cls, x, col, noise, arith)
 
     base.pack = classmethod(counting)
     try:
