@@ -18,12 +18,10 @@
 namespace metis {
 
 // ---------------------------------------------------------------------------------------------
-// Phase 1: codes + parked block maxima + per-workgroup maximum.  One block of 16 per thread per
-// iteration.  Row layout: thread i <-> block i (32 contiguous bytes, two 16-byte loads).
-// Column layout: thread i <-> (block-row b = i / cols, column c = i % cols) so that a wave reads
-// 64 consecutive columns of each of the 16 rows.
+// Phase 1, row-blocked: codes + parked block maxima + per-workgroup maximum.  One block of 16 per
+// thread per iteration: thread i <-> block i (32 contiguous bytes, two 16-byte loads).
 // ---------------------------------------------------------------------------------------------
-template <int MODE, bool SR, bool COL>
+template <int MODE, bool SR>
 __global__ __launch_bounds__(256) void quant_codes_kernel(
     const uint16_t* __restrict__ x, uint32_t rows, uint32_t cols, int64_t ld, const void* __restrict__ noise,
     uint64_t seed, uint64_t offset, uint2* __restrict__ codes, uint16_t* __restrict__ ws_amax,
@@ -31,8 +29,7 @@ __global__ __launch_bounds__(256) void quant_codes_kernel(
 {
     float gmax = 0.0f;
     const uint32_t nbpr = cols / kBlock;      // row layout: blocks per row
-    const uint32_t nbc = rows / kBlock;       // column layout: blocks per column
-    if constexpr (!COL && !SR) {
+    if constexpr (!SR) {
         // Round-to-nearest rows: software-pipelined, the next block's 32 bytes are in flight while the
         // current block is encoded.
         const uint32_t step = gridDim.x * 256u;
@@ -63,37 +60,88 @@ __global__ __launch_bounds__(256) void quant_codes_kernel(
     }
     for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < nblocks; i += gridDim.x * 256u) {
         float v[kBlock], u[kBlock] = {};
-        uint32_t ob;
-        if constexpr (!COL) {
-            ob = i;
-            const uint32_t row = i / nbpr, cb = i - row * nbpr;
-            const uint4* p = reinterpret_cast<const uint4*>(x + (int64_t)row * ld + (int64_t)cb * kBlock);
-            unpack16(p[0], p[1], v);
-            if (SR && noise) {
+        const uint32_t row = i / nbpr, cb = i - row * nbpr;
+        const uint4* p = reinterpret_cast<const uint4*>(x + (int64_t)row * ld + (int64_t)cb * kBlock);
+        unpack16(p[0], p[1], v);
+        if (SR && noise) {
 #pragma unroll
-                for (int j = 0; j < kBlock; ++j) {
-                    int64_t e = (int64_t)i * kBlock + j;
-                    u[j] = MODE ? bf16_lo(((const uint16_t*)noise)[e]) : ((const float*)noise)[e];
-                }
+            for (int j = 0; j < kBlock; ++j) {
+                int64_t e = (int64_t)i * kBlock + j;
+                u[j] = MODE ? bf16_lo(((const uint16_t*)noise)[e]) : ((const float*)noise)[e];
             }
-        } else {
-            const uint32_t b = i / cols, c = i - b * cols;
-            ob = c * nbc + b;
+        }
+        if (SR && !noise) philox16<MODE>(seed, offset, i, u);
+        const float am = block_amax(v);
+        gmax = fmaxf(gmax, am);
+        ws_amax[i] = (uint16_t)(__float_as_uint(am) >> 16);          // am is a bf16 value
+        codes[i] = encode_block<MODE, SR>(v, block_scalar<MODE>(am), u);
+    }
+    publish_group_max(gmax, ws_gmax);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Phase 1, column-blocked: blocks run down 16 consecutive rows of one column and the packed tensor
+// is stored transposed ([cols, rows/2] codes, [cols, rows/16] scales).  A workgroup owns a tile of
+// 256 rows x 64 columns: thread t encodes blocks 4g..4g+3 (g = t / 64) of column t % 64, every load
+// instruction reading 64 consecutive columns of one row.  Codes and block maxima are transposed
+// through LDS so that they leave as 32-byte (8-byte) pieces of the 128 (32) contiguous bytes each
+// column owns in the tile, instead of one scattered 8-byte and 2-byte store per lane.
+// ---------------------------------------------------------------------------------------------
+constexpr int kColTileBlocks = 16, kColTileCols = 64;
+template <int MODE, bool SR>
+__global__ __launch_bounds__(256) void quant_codes_col_kernel(
+    const uint16_t* __restrict__ x, uint32_t rows, uint32_t cols, int64_t ld, const void* __restrict__ noise,
+    uint64_t seed, uint64_t offset, uint2* __restrict__ codes, uint16_t* __restrict__ ws_amax,
+    uint32_t* __restrict__ ws_gmax, uint32_t tiles_c, uint32_t tiles_total)
+{
+    __shared__ uint2 s_codes[kColTileCols][kColTileBlocks + 1];
+    __shared__ uint16_t s_amax[kColTileCols][kColTileBlocks + 2];
+    const uint32_t nbc = rows / kBlock;                       // blocks per column
+    const uint32_t cl = threadIdx.x & 63u, g = threadIdx.x >> 6;
+    float gmax = 0.0f;
+    for (uint32_t tile = blockIdx.x; tile < tiles_total; tile += gridDim.x) {
+        const uint32_t tr = tile / tiles_c, tc = tile - tr * tiles_c;
+        const uint32_t c = tc * kColTileCols + cl;
+#pragma unroll 1
+        for (uint32_t k = 0; k < 4u; ++k) {
+            const uint32_t bl = g * 4u + k, b = tr * kColTileBlocks + bl;
+            uint2 packed = make_uint2(0u, 0u);
+            float am = 0.0f;
+            if (c < cols && b < nbc) {
+                float v[kBlock], u[kBlock] = {};
 #pragma unroll
-            for (int j = 0; j < kBlock; ++j) v[j] = bf16_lo(x[(int64_t)(b * kBlock + j) * ld + c]);
-            if (SR && noise) {
+                for (int j = 0; j < kBlock; ++j) v[j] = bf16_lo(x[(int64_t)(b * kBlock + j) * ld + c]);
+                if (SR && noise) {
 #pragma unroll
-                for (int j = 0; j < kBlock; ++j) {
-                    int64_t e = (int64_t)(b * kBlock + j) * cols + c;
-                    u[j] = MODE ? bf16_lo(((const uint16_t*)noise)[e]) : ((const float*)noise)[e];
+                    for (int j = 0; j < kBlock; ++j) {
+                        int64_t e = (int64_t)(b * kBlock + j) * cols + c;
+                        u[j] = MODE ? bf16_lo(((const uint16_t*)noise)[e]) : ((const float*)noise)[e];
+                    }
+                }
+                if (SR && !noise) philox16<MODE>(seed, offset, (int64_t)c * nbc + b, u);
+                am = block_amax(v);
+                gmax = fmaxf(gmax, am);
+                packed = encode_block<MODE, SR>(v, block_scalar<MODE>(am), u);
+            }
+            s_codes[cl][bl] = packed;
+            s_amax[cl][bl] = (uint16_t)(__float_as_uint(am) >> 16);
+        }
+        __syncthreads();
+        {   // column t / 4, blocks 4 (t % 4) .. +3 of the tile: 32 contiguous bytes of codes, 8 of maxima
+            const uint32_t oc = threadIdx.x >> 2, part = threadIdx.x & 3u;
+            const uint32_t c2 = tc * kColTileCols + oc, b0 = tr * kColTileBlocks + part * 4u;
+            if (c2 < cols) {
+#pragma unroll
+                for (uint32_t i = 0; i < 4u; ++i) {
+                    if (b0 + i < nbc) {
+                        const int64_t ob = (int64_t)c2 * nbc + b0 + i;
+                        codes[ob] = s_codes[oc][part * 4u + i];
+                        ws_amax[ob] = s_amax[oc][part * 4u + i];
+                    }
                 }
             }
         }
-        if (SR && !noise) philox16<MODE>(seed, offset, ob, u);
-        const float am = block_amax(v);
-        gmax = fmaxf(gmax, am);
-        ws_amax[ob] = (uint16_t)(__float_as_uint(am) >> 16);          // am is a bf16 value
-        codes[ob] = encode_block<MODE, SR>(v, block_scalar<MODE>(am), u);
+        __syncthreads();
     }
     publish_group_max(gmax, ws_gmax);
 }
@@ -398,10 +446,24 @@ static int launch_quant(const void* x, int64_t rows, int64_t cols, int64_t ld, c
                         uint64_t offset, void* codes, void* scales, float* unit, const Workspace& ws, hipStream_t st)
 {
     const uint32_t nblocks = (uint32_t)(rows * cols / kBlock);
-    const int g1 = grid_for(nblocks);
-    hipLaunchKernelGGL((quant_codes_kernel<MODE, SR, COL>), dim3(g1), dim3(256), 0, st, (const uint16_t*)x,
-                       (uint32_t)rows, (uint32_t)cols, ld, noise, seed, offset, (uint2*)codes, ws.amax, ws.gmax, nblocks);
-    return launch_scales(MODE, ws, (uint32_t)g1, scales, unit, nblocks, st);
+    if constexpr (COL) {
+        const uint32_t tiles_r = (uint32_t)((rows / kBlock + kColTileBlocks - 1) / kColTileBlocks);
+        const uint32_t tiles_c = (uint32_t)((cols + kColTileCols - 1) / kColTileCols);
+        const int64_t tiles = (int64_t)tiles_r * tiles_c;
+        int64_t g = tiles;
+        const int64_t cap = (int64_t)device_cus() * 8;
+        if (g > cap) g = cap;
+        if (g > kMaxGroups) g = kMaxGroups;
+        hipLaunchKernelGGL((quant_codes_col_kernel<MODE, SR>), dim3((unsigned)g), dim3(256), 0, st, (const uint16_t*)x,
+                           (uint32_t)rows, (uint32_t)cols, ld, noise, seed, offset, (uint2*)codes, ws.amax, ws.gmax, tiles_c,
+                           (uint32_t)tiles);
+        return launch_scales(MODE, ws, (uint32_t)g, scales, unit, nblocks, st);
+    } else {
+        const int g1 = grid_for(nblocks);
+        hipLaunchKernelGGL((quant_codes_kernel<MODE, SR>), dim3(g1), dim3(256), 0, st, (const uint16_t*)x, (uint32_t)rows,
+                           (uint32_t)cols, ld, noise, seed, offset, (uint2*)codes, ws.amax, ws.gmax, nblocks);
+        return launch_scales(MODE, ws, (uint32_t)g1, scales, unit, nblocks, st);
+    }
 }
 
 int quantize(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, bool sr, bool col, const void* noise,
