@@ -249,3 +249,21 @@ def test_single_launch_variant_matches_two_launch_path(ops, monkeypatch, tag, mo
             got = ops.quantize(x, mode)
             _check_packed(got, ref.codes.cpu(), ref.scales.cpu(), ref.unit.cpu(), f"shape {r}x{c} rep {rep} {tag}")
     monkeypatch.delenv("METIS_FUSED_QUANT", raising=False)
+
+
+@pytest.mark.parametrize("tag,mode", MODES)
+def test_signed_zeros_and_negatives_that_round_to_zero(ops, tag, mode):
+    """The reference's sign comes from sign(x): -0.0 has no sign (nibble 0), a negative value whose
+    magnitude rounds to zero keeps it (nibble 8).  Both sit next to ordinary values in every block."""
+    from oracle import metis_oracle as O
+    x = synthetic_activation(61, 64, 256)
+    x[:, 0::7] = -0.0
+    x[:, 1::7] = 0.0
+    x[:, 2::7] = -1e-4
+    x[:, 3::7] = 1e-4
+    x[3] = 0.0
+    x[4] = -0.0
+    codes, scales, unit, _ = O.nvfp4_pack(_oracle_in(x, mode))
+    _check_packed(ops.quantize(x.cuda(), mode), codes, scales, unit, tag)
+    ct, st, ut, _ = O.nvfp4_pack_col(_oracle_in(x, mode))
+    _check_packed(ops.quantize(x.cuda(), mode, col=True), ct, st, ut, tag + " col")
