@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
 
-Headline (BASELINE.json): Metis NVFP4 linear TFLOP/s at 8192x4096x14336, rank 64 (config 3).
+Headline: Metis NVFP4 linear TFLOP/s at 8192x4096x14336, rank 64 (config 3).
 One step = one pass of the forward hot path over one batch that is already resident in HBM:
     NVFP4-quantize X (RNE)  ->  T = (X V^T) * s in bf16  ->  fused GEMM
     out = deq(Q(X)) deq(Q(W - U S V^T))^T + T U^T      (fp32 accumulate, bf16 store)

@@ -355,19 +355,19 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_nvfp4_large_kernel(
         load_frags(1, cur, 1);
         if (EXPAND) pieces(0, P0);
         mfmas(0);
-        if (!(DBG & 8)) { if (EXPAND) sched_substep<NM, VPM, NF, P0>(); else sched_substep<NM, 0, NF, 0>(); }
+        if (EXPAND) sched_substep<NM, VPM, NF, P0>(); else sched_substep<NM, 0, NF, 0>();
         load_frags(0, cur, 2);
         if (EXPAND) pieces(P0, P0 + P1);
         mfmas(1);
-        if (!(DBG & 8)) { if (EXPAND) sched_substep<NM, VPM, NF, P1>(); else sched_substep<NM, 0, NF, 0>(); }
+        if (EXPAND) sched_substep<NM, VPM, NF, P1>(); else sched_substep<NM, 0, NF, 0>();
         load_frags(1, cur, 3);
         if (EXPAND) pieces(P0 + P1, PIECES);
         mfmas(0);
-        if (!(DBG & 8)) { if (EXPAND) sched_substep<NM, VPM, NF, P2>(); else sched_substep<NM, 0, NF, 0>(); }
+        if (EXPAND) sched_substep<NM, VPM, NF, P2>(); else sched_substep<NM, 0, NF, 0>();
         if (!(DBG & 2)) __syncthreads();
         if (EXPAND || (DBG & 1)) load_frags(0, nxt, 0);
         mfmas(1);
-        if (!(DBG & 8)) sched_substep<NM, 0, NF, 0>();
+        sched_substep<NM, 0, NF, 0>();
         if (FETCH) {
 #pragma unroll
             for (int q = 0; q < RPT; ++q) r1[q] = r2[q];
@@ -422,7 +422,7 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_nvfp4_large_kernel(
 
     // ---- epilogue, bf16 output with N % 8 == 0: each wave transposes its tile through its own slice of the
     //      (now idle) LDS so that a store instruction writes 8 rows x 128 contiguous bytes instead of 32 rows x 16
-    if constexpr (!OUT_F32 && WN_WAVES == 4 && !(DBG & 32)) {
+    if constexpr (!OUT_F32 && WN_WAVES == 4) {
         if ((N & 7) == 0) {
             constexpr int CROW = 64 + 8;                              // halves per staged row (144 bytes: conflict-free)
             uint16_t* cw = lds + wave * (128 * CROW);
@@ -475,7 +475,6 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_nvfp4_large_kernel(
                     v[e] = acc[i][j][4 * g + e];
                     if (bias) v[e] += bf16_lo(bias[n + e]);
                 }
-                if ((DBG & 16) && v[0] != 12345.678f) continue;
                 if (OUT_F32) {
                     *reinterpret_cast<float4*>((float*)out + (int64_t)m * N + n) = make_float4(v[0], v[1], v[2], v[3]);
                 } else {
@@ -498,11 +497,12 @@ static int launch_large(const void* a_codes, const void* a_scales, const float* 
     const size_t lds_bytes = 2 * (size_t)L_STAGE_HALVES * sizeof(uint16_t);
     const int f32 = out_dtype == METIS_DTYPE_F32;
     const void* fn = f32 ? (const void*)gemm_nvfp4_large_kernel<1, WN_WAVES> : (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES>;
-    if (const char* d = getenv("METIS_GEMM_DBG")) {
-        const int v = atoi(d);
-        fn = v == 1 ? (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 1> : v == 8 ? (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 8>
-           : v == 7 ? (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 7> : v == 16 ? (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 16> : v == 32 ? (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 32> : fn;
-        (void)hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (const char* d = getenv("METIS_GEMM_DBG")) {            // measurement switches, results are meaningless:
+        const int v = atoi(d);                                 // 1 = no operand fetch/expansion, 7 = also no barriers
+        if (v == 1 || v == 7) {
+            fn = v == 1 ? (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 1> : (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 7>;
+            (void)hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        }
     }
     if (!attr_set[f32]) {
         if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)

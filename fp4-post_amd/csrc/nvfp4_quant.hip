@@ -304,9 +304,8 @@ __device__ __forceinline__ float grid_max_wait(uint64_t tag, uint32_t* sync, Gri
 // so that part of the reduction latency is covered.
 template <int MODE, int NB>
 __global__ __launch_bounds__(256) void quant_fused_kernel(const uint16_t* __restrict__ x, uint2* __restrict__ codes,
-                                                               uint8_t* __restrict__ scales, float* __restrict__ unit_out,
-                                                               uint32_t* __restrict__ sync, uint32_t nblocks,
-                                                               uint32_t dbg)
+                                                          uint8_t* __restrict__ scales, float* __restrict__ unit_out,
+                                                          uint32_t* __restrict__ sync, uint32_t nblocks)
 {
     __shared__ GridMaxState sh;
     const uint64_t tag = grid_max_begin(sync);
@@ -327,11 +326,11 @@ __global__ __launch_bounds__(256) void quant_fused_kernel(const uint16_t* __rest
         unpack16(c0, c1, v);
         am[k] = block_amax(v);
         gmax = fmaxf(gmax, am[k]);
-        if (k == NB - 1 && !(dbg & 1u)) grid_max_arrive(gmax, tag, sync, sh);
+        if (k == NB - 1) grid_max_arrive(gmax, tag, sync, sh);
         if (i < nblocks) codes[i] = encode_block<MODE, false>(v, block_scalar<MODE>(am[k]), none);
         c0 = n0; c1 = n1;
     }
-    const float amax = (dbg & 2u) ? 6.0f : grid_max_wait(tag, sync, sh);
+    const float amax = grid_max_wait(tag, sync, sh);
     const float unit = rd<MODE>(block_scalar<MODE>(amax) / 448.0f);          // quant.py:21-22
     if (i0 == 0) *unit_out = unit;
 #pragma unroll
@@ -424,9 +423,8 @@ static int try_fused(const void* x, void* codes, void* scales, float* unit, cons
     if (cap > kFusedMaxGrid) cap = kFusedMaxGrid;
     const int64_t need = ((int64_t)nblocks + 256 * NB - 1) / (256 * NB);
     if (cap <= 0 || need > cap) return 1;                      // does not fit: caller picks another path
-    uint32_t dbg = getenv("METIS_DBG_FLAGS") ? (uint32_t)atoi(getenv("METIS_DBG_FLAGS")) : 0u;
     hipLaunchKernelGGL((quant_fused_kernel<MODE, NB>), dim3((unsigned)need), dim3(256), 0, st, (const uint16_t*)x,
-                       (uint2*)codes, (uint8_t*)scales, unit, ws.sync, nblocks, dbg);
+                       (uint2*)codes, (uint8_t*)scales, unit, ws.sync, nblocks);
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 
