@@ -79,6 +79,74 @@ class LinearLowbitFunction(torch.autograd.Function):
     mean_cache_key = "default"
 
     # ------------------------------------------------------------------ activation paths
+    # ------------------------------------------------------------------ tiled random Hadamard rotation
+    _hadamard_cache: dict = {}
+    _hadamard_sign_cache: dict = {}
+
+    @staticmethod
+    def _get_hadamard(size: int, device, dtype) -> torch.Tensor:
+        """Sylvester Hadamard matrix H_size (entries +-1), cached per (size, device, dtype); reference 75-96."""
+        F = LinearLowbitFunction
+        key = (int(size), device, dtype)
+        if key not in F._hadamard_cache:
+            if size <= 0 or size & (size - 1):
+                raise ValueError(f"Hadamard block size must be a power of two, got {size}")
+            h = torch.ones((1, 1), device=device, dtype=dtype)
+            while h.shape[0] < size:
+                h = torch.cat((torch.cat((h, h), dim=1), torch.cat((h, -h), dim=1)), dim=0)
+            F._hadamard_cache[key] = h
+        return F._hadamard_cache[key]
+
+    @staticmethod
+    def _get_hadamard_sign(size: int, device, dtype) -> torch.Tensor:
+        """The one +-1 vector shared by every tile of a given size: CPU generator seeded with
+        1729 + size, so it is the same vector the reference draws (reference 98-111)."""
+        F = LinearLowbitFunction
+        key = (int(size), device, dtype)
+        if key not in F._hadamard_sign_cache:
+            gen = torch.Generator(device="cpu")
+            gen.manual_seed(1729 + size)
+            bits = torch.randint(0, 2, (size,), generator=gen, dtype=torch.int8)
+            F._hadamard_sign_cache[key] = (bits * 2 - 1).to(device=device, dtype=dtype)
+        return F._hadamard_sign_cache[key]
+
+    @staticmethod
+    def _apply_hadamard_blocks(value: torch.Tensor, inverse: bool = False) -> torch.Tensor:
+        """Rotate every tile of `hadamard_tile_size` consecutive elements of the last dimension:
+        forward (x * S) H, inverse (y H) / d * S (reference 125-211).  All tiles go through one
+        small GEMM per row chunk, in binary32 for 16-bit inputs; chunks are sized so that the
+        binary32 workspace stays within `hadamard_workspace_mb`."""
+        F = LinearLowbitFunction
+        dim = value.shape[-1]
+        if dim <= 1 or value.numel() == 0:
+            return value
+        tile = int(F.hadamard_tile_size)
+        if tile <= 0 or tile & (tile - 1):
+            raise ValueError(f"Hadamard tile size must be a positive power of two, got {tile}")
+        if dim % tile:
+            raise ValueError(f"RHT tile size {tile} must divide hidden dimension {dim}; "
+                             "set --metis_hadamard_tile_size to a compatible power of two")
+        if F.hadamard_backend not in {"auto", "dao_cuda", "torch_gemm"}:
+            raise ValueError(f"Unsupported Hadamard backend: {F.hadamard_backend}")
+        if F.hadamard_backend == "dao_cuda":
+            raise RuntimeError("Hadamard backend dao_cuda was requested but fast_hadamard_transform is unavailable "
+                               "in this build; use 'auto' or 'torch_gemm'")
+        work_dtype = torch.float32 if value.dtype in (torch.float16, torch.bfloat16) else value.dtype
+        h = F._get_hadamard(tile, value.device, work_dtype)
+        signs = F._get_hadamard_sign(tile, value.device, work_dtype)
+        tiles = value.reshape(-1, tile)
+        out = torch.empty_like(tiles)
+        budget = max(1, int(F.hadamard_workspace_mb)) * 1024 * 1024
+        chunk = max(1, budget // (8 * tile * torch.empty((), dtype=work_dtype).element_size()))
+        for r0 in range(0, tiles.shape[0], chunk):
+            work = tiles[r0:r0 + chunk].to(work_dtype)
+            if inverse:
+                rotated = torch.mm(work, h).mul_(1.0 / tile).mul_(signs)
+            else:
+                rotated = torch.mm(work * signs, h)
+            out[r0:r0 + chunk].copy_(rotated)
+        return out.reshape(value.shape)
+
     @staticmethod
     def svd_quant(input_, quant_func, rank=60, niter=0, broadcast_dim=-1, tp_simulate=False, tp_parts=4,
                   metis_mode="mean", mean_cache=None, cache_key="default"):
@@ -133,13 +201,17 @@ class LinearLowbitFunction(torch.autograd.Function):
 
     @staticmethod
     def _quantize_wgrad_operand(value: torch.Tensor, quantizer) -> torch.Tensor:
-        """Three-call QDQ of one backward operand (reference 395-405); the Hadamard pre-rotation of
-        the NV recipe is not part of this build."""
-        if LinearLowbitFunction.enable_nv_recipe:
-            raise NotImplementedError("enable_nv_recipe (random Hadamard rotation) is not implemented")
+        """Three-call QDQ of one backward operand, between a tiled random Hadamard rotation and its
+        inverse under the NV recipe (reference 395-405)."""
+        F = LinearLowbitFunction
+        if F.enable_nv_recipe:
+            value = F._apply_hadamard_blocks(value, inverse=False)
         scalar = quantizer.get_scalar(value)
         value = quantizer.quant(value, scalar)
-        return quantizer.rquant(value, scalar)
+        value = quantizer.rquant(value, scalar)
+        if F.enable_nv_recipe:
+            value = F._apply_hadamard_blocks(value, inverse=True)
+        return value
 
     # ------------------------------------------------------------------ autograd
     @staticmethod
@@ -208,6 +280,8 @@ class LinearLowbitFunction(torch.autograd.Function):
             dyq = _flat2d(dyq)
         else:
             dyq = _flat2d(F._quantize_wgrad_operand(dy2, F.q_backward_outputgrad))
+        if F.enable_nv_recipe:                                             # reference 495-501: only the two wgrad operands
+            xq = _flat2d(F._quantize_wgrad_operand(xq, F.q_backward_input))
         grad_weight = torch.matmul(dyq.T, xq).to(torch.float32)            # reference 502-510
         grad_input = torch.matmul(dyq, wq).reshape(*ctx.lead, wq.shape[-1])  # reference 507-508
         return grad_input, grad_weight, grad_bias, None, None
@@ -262,9 +336,10 @@ class LinearLowbit(nn.Module):
             cached_key, cached = self._quantized_weight_cache
             if cached_key == key:
                 return cached
-        if F.enable_nv_recipe:
-            raise NotImplementedError("enable_nv_recipe (random Hadamard rotation) is not implemented")
-        if _packable(weight_compute, F.q_forward_weight) and weight_compute.shape[0] % 4 == 0:
+        if F.enable_nv_recipe:                                             # reference 577-585
+            q = F._apply_hadamard_blocks(weight_compute, inverse=False)
+            q = F._apply_hadamard_blocks(F.q_forward_weight.quantize_dequantize(q), inverse=True)
+        elif _packable(weight_compute, F.q_forward_weight) and weight_compute.shape[0] % 4 == 0:
             q = F.q_forward_weight.pack(weight_compute, arith=arith)
         else:
             q = F.q_forward_weight.quantize_dequantize(weight_compute)

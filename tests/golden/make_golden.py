@@ -169,6 +169,39 @@ def golden_linear(out: dict):
     out["bl_y"] = bits(yb)
 
 
+def golden_hadamard(out: dict):
+    """Tiled random Hadamard rotation of the NV recipe (bitlinear.py:75-211, 395-405, 495-501, 577-585):
+    the rotation itself, a rotated wgrad operand through the NVFP4 quantizer, and LinearLowbit forward +
+    backward with round-to-nearest quantizers everywhere (no random draws involved)."""
+    F = rb.LinearLowbitFunction
+    g = torch.Generator().manual_seed(41)
+    x = torch.randn(6, 48, generator=g).bfloat16().float()
+    F.hadamard_tile_size, F.hadamard_backend, F.hadamard_workspace_mb = 16, "torch_gemm", 128
+    out["had_x"] = bits(x)
+    out["had_sign16"] = bits(F._get_hadamard_sign(16, torch.device("cpu"), torch.float32))
+    out["had_fwd"] = bits(F._apply_hadamard_blocks(x, inverse=False))
+    out["had_inv"] = bits(F._apply_hadamard_blocks(x, inverse=True))
+    out["had_fwd_bf16"] = bits(F._apply_hadamard_blocks(x.bfloat16(), inverse=False))
+    _configure("nvfp4e2m1bnosr", "nvfp4e2m1bnosr", "nvfp4e2m1bnosr", torch.float32)
+    F.enable_nv_recipe = True
+    try:
+        out["had_wgrad_operand_p32"] = bits(F._quantize_wgrad_operand(x.clone(), rq.Cast2NVFp4e2m1BlockNOSR))
+        B, T, K, N = 2, 16, 64, 48
+        xl = torch.randn(B, T, K, generator=g).bfloat16().float()
+        w = (torch.randn(N, K, generator=g) * 0.05).bfloat16().float()
+        dy = (torch.randn(B, T, N, generator=g) * 1e-3).bfloat16().float()
+        layer = rb.LinearLowbit(K, N, bias=False, args=SimpleNamespace(device="cpu", cache_quantized_weight=False))
+        with torch.no_grad():
+            layer.weight.copy_(w)
+        xr = xl.clone().requires_grad_(True)
+        y = layer(xr)
+        y.backward(dy)
+        out["had_lin_x"], out["had_lin_w"], out["had_lin_dy"] = bits(xl), bits(w), bits(dy)
+        out["had_lin_y"], out["had_lin_gx"], out["had_lin_gw"] = bits(y.detach()), bits(xr.grad), bits(layer.weight.grad)
+    finally:
+        F.enable_nv_recipe = False
+
+
 def main():
     torch.set_num_threads(1)
     out: dict = {}
@@ -178,6 +211,11 @@ def main():
     path = os.path.join(HERE, "metis_reference_golden.npz")
     np.savez_compressed(path, **out)
     print(f"wrote {path}: {len(out)} arrays, {os.path.getsize(path)} bytes; torch {torch.__version__}")
+    had: dict = {}
+    golden_hadamard(had)
+    path = os.path.join(HERE, "metis_reference_hadamard.npz")
+    np.savez_compressed(path, **had)
+    print(f"wrote {path}: {len(had)} arrays, {os.path.getsize(path)} bytes")
 
 
 if __name__ == "__main__":

@@ -257,3 +257,42 @@ def test_patch_qwen2_decoder_layer():
     out.float().square().mean().backward()
     assert xr.grad is not None and bool(torch.isfinite(xr.grad).all())
     assert attn.q_proj.warmup_linear.weight.grad is not None
+
+
+def test_nv_recipe_against_reference_vectors():
+    """NV recipe (tiled random Hadamard rotation around the wgrad operands and the weight QDQ), all
+    quantizers round-to-nearest: rotated wgrad operand, LinearLowbit forward and both gradients against
+    what the reference computed on CPU.  The rotation is a 16-term binary32 GEMM whose summation order
+    differs between devices, so an element now and then lands on the other side of an FP4 rounding
+    boundary: agreement is checked in the Frobenius norm and as a fraction of identical elements."""
+    import os
+    from types import SimpleNamespace
+
+    import numpy as np
+
+    from metis_hip import LinearLowbit, LinearLowbitFunction as F, quant_func
+    g = dict(np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "metis_reference_hadamard.npz")))
+    nosr = quant_func["nvfp4e2m1bnosr"]
+    F.q_backward_input = F.q_backward_weight = F.q_backward_outputgrad = nosr
+    F.hadamard_tile_size, F.hadamard_backend = 16, "torch_gemm"
+    F.enable_nv_recipe = True
+    try:
+        x = t(g["had_x"]).cuda()
+        torch.testing.assert_close(F._apply_hadamard_blocks(x).cpu(), t(g["had_fwd"]), rtol=1e-6, atol=1e-6)
+        got = F._quantize_wgrad_operand(x.clone(), nosr).cpu()
+        want = t(g["had_wgrad_operand_p32"])
+        assert rel_fro(got, want) <= 2e-2
+        assert float((got - want).abs().le(1e-6).float().mean()) > 0.9
+
+        layer = LinearLowbit(64, 48, bias=False, args=SimpleNamespace(device="cuda", cache_quantized_weight=False))
+        with torch.no_grad():
+            layer.weight.copy_(t(g["had_lin_w"]))
+        xr = t(g["had_lin_x"]).cuda().requires_grad_(True)
+        y = layer(xr)
+        y.backward(t(g["had_lin_dy"]).cuda())
+        assert rel_fro(y.detach().cpu(), t(g["had_lin_y"])) <= 2e-2
+        assert rel_fro(xr.grad.cpu(), t(g["had_lin_gx"])) <= 2e-2
+        assert rel_fro(layer.weight.grad.cpu(), t(g["had_lin_gw"])) <= 2e-2
+        assert layer.weight.grad.dtype == torch.float32
+    finally:
+        F.enable_nv_recipe = False

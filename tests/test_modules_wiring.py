@@ -238,6 +238,71 @@ def test_unsupported_options_fail_loudly():
     args.device = "cpu"
     with pytest.raises(ValueError):
         BitLinear(16, 8, args=args, dtype=torch.float32, compute_dtype=torch.int8)
-    LinearLowbitFunction.enable_nv_recipe = True
     with pytest.raises(NotImplementedError):
-        LinearLowbitFunction._quantize_wgrad_operand(torch.zeros(2, 16), Cast2Fp32)
+        LinearLowbitFunction.svd_quant(torch.zeros(2, 16), Cast2Fp32, metis_mode="svd")
+    LinearLowbitFunction.hadamard_backend = "dao_cuda"          # the optional CUDA extension is not part of this build
+    try:
+        with pytest.raises(RuntimeError):
+            LinearLowbitFunction._apply_hadamard_blocks(torch.zeros(2, 16))
+    finally:
+        LinearLowbitFunction.hadamard_backend = "auto"
+
+
+# ----------------------------------------------------------------------------- NV recipe: tiled random Hadamard rotation
+def _hadamard_golden():
+    import os
+    import numpy as np
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "metis_reference_hadamard.npz")
+    return np.load(path)
+
+
+def test_hadamard_rotation_matches_the_reference_vectors():
+    g = _hadamard_golden()
+    F = LinearLowbitFunction
+    x = torch.from_numpy(g["had_x"])
+    assert torch.equal(F._get_hadamard_sign(16, torch.device("cpu"), torch.float32), torch.from_numpy(g["had_sign16"]))
+    torch.testing.assert_close(F._apply_hadamard_blocks(x), torch.from_numpy(g["had_fwd"]), rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(F._apply_hadamard_blocks(x, inverse=True), torch.from_numpy(g["had_inv"]), rtol=1e-6, atol=1e-6)
+    want_bf16 = torch.from_numpy(g["had_fwd_bf16"].view("int16")).view(torch.bfloat16)
+    got_bf16 = F._apply_hadamard_blocks(x.bfloat16())
+    assert got_bf16.dtype == torch.bfloat16
+    torch.testing.assert_close(got_bf16.float(), want_bf16.float(), rtol=1e-2, atol=1e-2)
+    with pytest.raises(ValueError):
+        F._apply_hadamard_blocks(torch.zeros(2, 24))              # 16 does not divide 24 (reference 143-147)
+
+
+def test_hadamard_roundtrip_non_power_of_two_hidden_size_and_small_workspace():
+    """Reference tests/test_metis_quant_cache.py:101-122."""
+    F = LinearLowbitFunction
+    x = torch.randn(2, 3, 1536, generator=torch.Generator().manual_seed(3))
+    torch.testing.assert_close(F._apply_hadamard_blocks(F._apply_hadamard_blocks(x), inverse=True), x, rtol=1e-5, atol=1e-5)
+    x = torch.randn(64, 1536, generator=torch.Generator().manual_seed(4))
+    keep = F.hadamard_workspace_mb
+    F.hadamard_workspace_mb = 1
+    try:
+        back = F._apply_hadamard_blocks(F._apply_hadamard_blocks(x), inverse=True)
+    finally:
+        F.hadamard_workspace_mb = keep
+    torch.testing.assert_close(back, x, rtol=1e-5, atol=1e-5)
+
+
+def test_direct_forward_path_is_untouched_by_the_nv_recipe():
+    """Reference tests/test_metis_quant_cache.py:125-135."""
+    _identity_config()
+    LinearLowbitFunction.enable_nv_recipe = True
+    x = torch.randn(2, 3, 1536, generator=torch.Generator().manual_seed(5))
+    torch.testing.assert_close(LinearLowbitFunction.quantize_input(x), x, rtol=1e-5, atol=1e-5)
+
+
+def test_nv_recipe_rotates_only_the_wgrad_operands():
+    """Reference tests/test_metis_quant_cache.py:138-160: with identity quantizers the rotations cancel
+    and the weight gradient is the plain one."""
+    _identity_config()
+    layer = LinearLowbit(16, 16, bias=False, args=SimpleNamespace(device="cpu", cache_quantized_weight=False))
+    LinearLowbitFunction.enable_nv_recipe = True
+    LinearLowbitFunction.hadamard_backend = "torch_gemm"
+    LinearLowbitFunction.hadamard_tile_size = 16
+    x = torch.randn(2, 3, 16, generator=torch.Generator().manual_seed(6), requires_grad=True)
+    layer(x).sum().backward()
+    expected = torch.ones(16, 1) @ x.detach().reshape(-1, 16).sum(dim=0, keepdim=True)
+    torch.testing.assert_close(layer.weight.grad, expected, rtol=1e-5, atol=1e-5)
