@@ -150,33 +150,62 @@ class LinearLowbitFunction(torch.autograd.Function):
     @staticmethod
     def svd_quant(input_, quant_func, rank=60, niter=0, broadcast_dim=-1, tp_simulate=False, tp_parts=4,
                   metis_mode="mean", mean_cache=None, cache_key="default"):
-        """Mean-residual activation quantization (reference 311-336, 363-366).
+        """Low-rank (or mean) part kept in high precision + quantized residual (reference 213-369).
 
-        Column mean over tokens is kept in high precision, the centred residual goes through the
-        quantizer's fused QDQ, and the mean is added back; during single-token decode a weighted
-        running mean per cache key is used.  The "svd" mode and the TP simulation of the reference
-        are not part of this build.
+        "mean": the column mean over tokens stays in high precision, the centred residual goes through
+        the quantizer's fused QDQ and the mean is added back; single-token decode calls use a weighted
+        running mean per cache key (311-336).  "svd": a randomized rank-`rank` SVD of the (optionally
+        broadcast-sliced) input, U and V through the three-call QDQ, S untouched, residual through the
+        fused QDQ (243-309).  With tp_simulate the last dimension is cut into tp_parts chunks that are
+        treated independently in "svd" style and concatenated (338-360).
         """
-        if tp_simulate or metis_mode != "mean":
-            if metis_mode not in ("mean", "svd"):
-                raise ValueError(f"Unsupported metis_mode: {metis_mode}")
-            raise NotImplementedError("only metis_mode='mean' without TP simulation is implemented")
-        shape = input_.shape
-        flat = _flat2d(input_)
-        seq_len = shape[1] if len(shape) == 3 else shape[0]
-        if seq_len == 1 and mean_cache is not None and cache_key in mean_cache:
-            cached_mean, cached_count = mean_cache[cache_key]
-            new_count = cached_count + flat.shape[0]
-            this_mean = flat.mean(dim=0, keepdim=True)
-            me = (cached_mean * cached_count + this_mean * flat.shape[0]) / new_count
-            mean_cache[cache_key] = (me.detach(), new_count)
-        else:
-            me = flat.mean(dim=0, keepdim=True)
-            if mean_cache is not None:
-                mean_cache[cache_key] = (me.detach(), flat.shape[0])
-        res = quant_func.quantize_dequantize(flat - me)
-        out = me + res
-        return out.view(shape) if len(shape) == 3 else out
+        F = LinearLowbitFunction
+
+        def lowrank_single(chunk):
+            picked = broadcast_dim >= 0
+            rep = chunk.select(broadcast_dim, 0) if picked else chunk
+            shape = rep.shape
+            rep2 = rep.reshape(-1, shape[-1]) if len(shape) == 3 else rep
+            flat = chunk.reshape(-1, shape[-1]) if len(shape) == 3 else chunk
+            dtype = rep2.dtype
+            with torch.amp.autocast(rep2.device.type, enabled=False):
+                ug, sg, vg = torch.svd_lowrank(rep2.to(torch.float32), q=rank, niter=niter)
+            ug, sg, vg = ug.to(dtype), sg.to(dtype), vg.to(dtype).T
+            us, vs = quant_func.get_scalar(ug), quant_func.get_scalar(vg)
+            ug = quant_func.rquant(quant_func.quant(ug, us), us)
+            vg = quant_func.rquant(quant_func.quant(vg, vs), vs)
+            ker = ug @ torch.diag(sg) @ vg
+            if picked:
+                ker = ker.unsqueeze(broadcast_dim)
+            out = ker + quant_func.quantize_dequantize(flat - ker)
+            return out.view(shape[0], shape[1], -1) if len(shape) == 3 else out
+
+        def mean_single(x):
+            shape = x.shape
+            flat = _flat2d(x)
+            seq_len = shape[1] if len(shape) == 3 else shape[0]
+            if seq_len == 1 and mean_cache is not None and cache_key in mean_cache:
+                cached_mean, cached_count = mean_cache[cache_key]
+                new_count = cached_count + flat.shape[0]
+                this_mean = flat.mean(dim=0, keepdim=True)
+                me = (cached_mean * cached_count + this_mean * flat.shape[0]) / new_count
+                mean_cache[cache_key] = (me.detach(), new_count)
+            else:
+                me = flat.mean(dim=0, keepdim=True)
+                if mean_cache is not None:
+                    mean_cache[cache_key] = (me.detach(), flat.shape[0])
+            out = me + quant_func.quantize_dequantize(flat - me)
+            return out.view(shape) if len(shape) == 3 else out
+
+        if tp_simulate:
+            width, parts = input_.shape[-1], max(1, int(tp_parts))
+            edges = [(width * p) // parts for p in range(parts + 1)]
+            return torch.cat([lowrank_single(input_[..., a:b]) for a, b in zip(edges, edges[1:]) if b > a], dim=-1)
+        if metis_mode == "svd":
+            return lowrank_single(input_)
+        if metis_mode == "mean":
+            return mean_single(input_)
+        raise ValueError(f"Unsupported metis_mode: {metis_mode}")
 
     @staticmethod
     def quantize_input(input_: torch.Tensor, mean_cache: dict = None, cache_key: str = "default") -> torch.Tensor:

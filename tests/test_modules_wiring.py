@@ -238,8 +238,8 @@ def test_unsupported_options_fail_loudly():
     args.device = "cpu"
     with pytest.raises(ValueError):
         BitLinear(16, 8, args=args, dtype=torch.float32, compute_dtype=torch.int8)
-    with pytest.raises(NotImplementedError):
-        LinearLowbitFunction.svd_quant(torch.zeros(2, 16), Cast2Fp32, metis_mode="svd")
+    with pytest.raises(ValueError):                             # reference bitlinear.py:368
+        LinearLowbitFunction.svd_quant(torch.zeros(2, 16), Cast2Fp32, metis_mode="no_such_mode")
     LinearLowbitFunction.hadamard_backend = "dao_cuda"          # the optional CUDA extension is not part of this build
     try:
         with pytest.raises(RuntimeError):
@@ -306,3 +306,21 @@ def test_nv_recipe_rotates_only_the_wgrad_operands():
     layer(x).sum().backward()
     expected = torch.ones(16, 1) @ x.detach().reshape(-1, 16).sum(dim=0, keepdim=True)
     torch.testing.assert_close(layer.weight.grad, expected, rtol=1e-5, atol=1e-5)
+
+
+def test_svd_mode_and_tp_simulation_reassemble_the_input_with_identity_quantizers():
+    """With identity quantizers, low-rank part + residual is the input again, whatever the rank, for 2-D
+    and 3-D inputs, with a broadcast slice, and chunk by chunk under the TP simulation (reference 243-360)."""
+    F = LinearLowbitFunction
+    g = torch.Generator().manual_seed(8)
+    x2 = torch.randn(48, 64, generator=g)
+    x3 = torch.randn(2, 24, 64, generator=g)
+    for x in (x2, x3):
+        out = F.svd_quant(x, Cast2Fp32, rank=16, niter=1, metis_mode="svd")
+        assert out.shape == x.shape
+        torch.testing.assert_close(out, x, rtol=1e-5, atol=1e-5)
+        out = F.svd_quant(x, Cast2Fp32, rank=16, niter=1, tp_simulate=True, tp_parts=3, metis_mode="svd")
+        assert out.shape == x.shape
+        torch.testing.assert_close(out, x, rtol=1e-5, atol=1e-5)
+    out = F.svd_quant(x3, Cast2Fp32, rank=8, niter=0, broadcast_dim=0, metis_mode="svd")
+    torch.testing.assert_close(out, x3, rtol=1e-5, atol=1e-5)
