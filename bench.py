@@ -31,9 +31,9 @@ QUANT_BYTES_PER_ELT = 2.5625   # 2 B read + 0.5 B codes + 1/16 B scale
 NORMQ_BYTES_PER_ELT = 4.5625   # + 2 B normed
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this workload, scaled by what the
 # same counters read for a 64 MiB copy (x2.0 reads, x1.0 writes); summary in profiles/hbm_traffic_pmc_config1_2_3.md
-TRAFFIC_GEMM_C3 = 661.3e6
-TRAFFIC_QUANT_C1 = 94.7e6
-TRAFFIC_NORMQ_C2 = 323.6e6
+TRAFFIC_GEMM_C3 = 653.6e6
+TRAFFIC_QUANT_C1 = 94.8e6
+TRAFFIC_NORMQ_C2 = 324.0e6
 
 
 def outlier_activation(torch, seed, rows, cols, device):
