@@ -1,0 +1,244 @@
+// Torch-free check of the C ABI: a plain C++ host program that owns its device memory through
+// HIP, calls libmetis_hip.so the way a C caller of the library would, and compares with the C
+// restatement of the reference arithmetic (oracle/libmetis_oracle.so, test infrastructure).
+//
+//   1. metis_nvfp4_quant_row in both parity modes  -> codes, scale bytes, unit bit-equal to the oracle
+//   2. metis_rmsnorm_nvfp4_quant                   -> normed output and packed tensor bit-equal
+//   3. metis_nvfp4_dequant                         -> bit-equal to the oracle's dequantization
+//   4. metis_linear_fwd (tiled and skinny shapes)  -> against a double-precision product of the
+//                                                     dequantized operands, rel. Frobenius error <= 2e-3
+//   5. error codes for bad arguments
+//
+// Built and run by tests/test_gpu_cabi_native.py; prints one line per check and exits non-zero on failure.
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <vector>
+
+#include "metis_hip.h"
+
+extern "C" {
+uint16_t metis_oracle_f32_to_bf16(float f);
+int metis_oracle_nvfp4_pack(const uint16_t* x, int64_t rows, int64_t cols, int64_t ld, int mode, const void* noise,
+                            uint8_t* codes, uint8_t* scales, float* unit, int64_t* n_clamped);
+int metis_oracle_nvfp4_dequant(const uint8_t* codes, const uint8_t* scales, float unit, int64_t rows, int64_t cols, int mode,
+                               uint16_t* out_bf16, float* out_f32);
+int metis_oracle_rmsnorm_nvfp4(const uint16_t* x, const uint16_t* gamma, float eps, int64_t rows, int64_t cols, int mode,
+                               uint16_t* normed, uint8_t* codes, uint8_t* scales, float* unit);
+}
+
+#define HIP_OK(x)                                                                          \
+    do {                                                                                   \
+        hipError_t e_ = (x);                                                               \
+        if (e_ != hipSuccess) {                                                            \
+            printf("FAIL hip: %s at line %d\n", hipGetErrorString(e_), __LINE__);          \
+            exit(2);                                                                       \
+        }                                                                                  \
+    } while (0)
+
+static int failures = 0;
+static void check(bool ok, const char* what)
+{
+    printf("%s %s\n", ok ? "ok  " : "FAIL", what);
+    fflush(stdout);
+    if (!ok) ++failures;
+}
+
+template <typename T>
+struct DeviceBuffer {
+    T* p = nullptr;
+    size_t n = 0;
+    explicit DeviceBuffer(size_t count) : n(count) { HIP_OK(hipMalloc(&p, count * sizeof(T) + 16)); }
+    ~DeviceBuffer() { (void)hipFree(p); }
+    void upload(const std::vector<T>& h) { HIP_OK(hipMemcpy(p, h.data(), h.size() * sizeof(T), hipMemcpyHostToDevice)); }
+    std::vector<T> download() const
+    {
+        std::vector<T> h(n);
+        HIP_OK(hipMemcpy(h.data(), p, n * sizeof(T), hipMemcpyDeviceToHost));
+        return h;
+    }
+};
+
+static float bf16_to_f32(uint16_t b)
+{
+    uint32_t u = (uint32_t)b << 16;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+// deterministic N(0,1)-ish bf16 data with an outlier column
+static std::vector<uint16_t> make_input(int64_t rows, int64_t cols, unsigned seed, float scale)
+{
+    std::vector<uint16_t> x((size_t)(rows * cols));
+    srand(seed);
+    for (int64_t i = 0; i < rows * cols; ++i) {
+        const double u1 = (rand() + 1.0) / (RAND_MAX + 2.0), u2 = rand() / (double)RAND_MAX;
+        float v = (float)(sqrt(-2.0 * log(u1)) * cos(6.283185307179586 * u2)) * scale;
+        if (i % cols == 5) v *= 20.0f;
+        x[(size_t)i] = metis_oracle_f32_to_bf16(v);
+    }
+    return x;
+}
+
+struct Packed {
+    std::vector<uint8_t> codes, scales;
+    float unit;
+};
+
+static Packed quantize_on_device(const std::vector<uint16_t>& x, int64_t rows, int64_t cols, int mode, hipStream_t st,
+                                 DeviceBuffer<uint8_t>* keep_codes = nullptr, DeviceBuffer<uint8_t>* keep_scales = nullptr,
+                                 DeviceBuffer<float>* keep_unit = nullptr)
+{
+    DeviceBuffer<uint16_t> dx(x.size());
+    dx.upload(x);
+    DeviceBuffer<uint8_t> local_codes((size_t)(rows * cols / 2)), local_scales((size_t)(rows * cols / 16));
+    DeviceBuffer<float> local_unit(1);
+    DeviceBuffer<uint8_t>& dc = keep_codes ? *keep_codes : local_codes;
+    DeviceBuffer<uint8_t>& ds = keep_scales ? *keep_scales : local_scales;
+    DeviceBuffer<float>& du = keep_unit ? *keep_unit : local_unit;
+    const size_t wsb = metis_nvfp4_workspace_bytes(rows, cols);
+    DeviceBuffer<uint8_t> ws(wsb);
+    HIP_OK(hipMemset(ws.p, 0, wsb));                            // zero-filled once, as the contract asks
+    const int rc = metis_nvfp4_quant_row(dx.p, rows, cols, cols, mode, dc.p, ds.p, du.p, ws.p, wsb, st);
+    if (rc != METIS_OK) {
+        printf("FAIL metis_nvfp4_quant_row rc=%d (%s)\n", rc, metis_error_string(rc));
+        exit(2);
+    }
+    HIP_OK(hipStreamSynchronize(st));
+    Packed p;
+    p.codes = dc.download();
+    p.scales = ds.download();
+    p.unit = du.download()[0];
+    return p;
+}
+
+static double rel_fro(const std::vector<double>& got, const std::vector<double>& want)
+{
+    double num = 0, den = 0;
+    for (size_t i = 0; i < got.size(); ++i) {
+        num += (got[i] - want[i]) * (got[i] - want[i]);
+        den += want[i] * want[i];
+    }
+    return sqrt(num / (den > 0 ? den : 1));
+}
+
+static void check_linear(int64_t M, int64_t N, int64_t K, hipStream_t st, const char* what)
+{
+    const std::vector<uint16_t> x = make_input(M, K, 11u + (unsigned)M, 1.0f), w = make_input(N, K, 12u + (unsigned)N, 0.02f);
+    DeviceBuffer<uint8_t> ac((size_t)(M * K / 2)), as((size_t)(M * K / 16)), bc((size_t)(N * K / 2)), bs((size_t)(N * K / 16));
+    DeviceBuffer<float> au(1), bu(1);
+    const Packed pa = quantize_on_device(x, M, K, METIS_MODE_P32, st, &ac, &as, &au);
+    const Packed pb = quantize_on_device(w, N, K, METIS_MODE_P32, st, &bc, &bs, &bu);
+    DeviceBuffer<float> out((size_t)(M * N));
+    const int rc = metis_linear_fwd(ac.p, as.p, au.p, bc.p, bs.p, bu.p, M, N, K, nullptr, nullptr, 0, nullptr, out.p, METIS_DTYPE_F32, st);
+    HIP_OK(hipStreamSynchronize(st));
+    std::vector<float> xa((size_t)(M * K)), wb((size_t)(N * K));
+    metis_oracle_nvfp4_dequant(pa.codes.data(), pa.scales.data(), pa.unit, M, K, 0, nullptr, xa.data());
+    metis_oracle_nvfp4_dequant(pb.codes.data(), pb.scales.data(), pb.unit, N, K, 0, nullptr, wb.data());
+    std::vector<double> want((size_t)(M * N)), got((size_t)(M * N));
+    for (int64_t m = 0; m < M; ++m)
+        for (int64_t n = 0; n < N; ++n) {
+            double s = 0;
+            for (int64_t k = 0; k < K; ++k) s += (double)xa[(size_t)(m * K + k)] * (double)wb[(size_t)(n * K + k)];
+            want[(size_t)(m * N + n)] = s;
+        }
+    const std::vector<float> o = out.download();
+    for (size_t i = 0; i < o.size(); ++i) got[i] = o[i];
+    const double err = rel_fro(got, want);
+    char line[160];
+    snprintf(line, sizeof line, "%s: metis_linear_fwd %ldx%ldx%ld rc=%d rel.err %.2e", what, (long)M, (long)N, (long)K, rc, err);
+    check(rc == METIS_OK && err <= 2e-3, line);
+}
+
+int main()
+{
+    hipStream_t st;
+    HIP_OK(hipStreamCreate(&st));                                // a caller-owned stream, default priority
+    printf("library version %d\n", metis_version());
+
+    // ---- 1 + 3: quantizer and dequantizer, both modes
+    const int64_t rows = 96, cols = 512;
+    const std::vector<uint16_t> x = make_input(rows, cols, 1u, 1.0f);
+    for (int mode = 0; mode < 2; ++mode) {
+        DeviceBuffer<uint8_t> dc((size_t)(rows * cols / 2)), ds((size_t)(rows * cols / 16));
+        DeviceBuffer<float> du(1);
+        const Packed got = quantize_on_device(x, rows, cols, mode, st, &dc, &ds, &du);
+        Packed want;
+        want.codes.resize(got.codes.size());
+        want.scales.resize(got.scales.size());
+        metis_oracle_nvfp4_pack(x.data(), rows, cols, cols, mode, nullptr, want.codes.data(), want.scales.data(), &want.unit, nullptr);
+        check(got.codes == want.codes && got.scales == want.scales && got.unit == want.unit,
+              mode == 0 ? "metis_nvfp4_quant_row P32: codes, scale bytes, unit bit-equal" : "metis_nvfp4_quant_row PB16: codes, scale bytes, unit bit-equal");
+        DeviceBuffer<uint16_t> dout((size_t)(rows * cols));
+        const int rc = metis_nvfp4_dequant(dc.p, ds.p, du.p, rows, cols, mode, dout.p, METIS_DTYPE_BF16, st);
+        HIP_OK(hipStreamSynchronize(st));
+        std::vector<uint16_t> want_dq((size_t)(rows * cols));
+        metis_oracle_nvfp4_dequant(want.codes.data(), want.scales.data(), want.unit, rows, cols, mode, want_dq.data(), nullptr);
+        std::vector<uint16_t> got_dq = dout.download();
+        bool same = rc == METIS_OK;
+        for (size_t i = 0; same && i < got_dq.size(); ++i)
+            same = got_dq[i] == want_dq[i] || (bf16_to_f32(got_dq[i]) == 0.0f && bf16_to_f32(want_dq[i]) == 0.0f);
+        check(same, mode == 0 ? "metis_nvfp4_dequant P32 -> bf16 bit-equal" : "metis_nvfp4_dequant PB16 -> bf16 bit-equal");
+    }
+
+    // ---- 2: fused RMSNorm -> quant
+    {
+        std::vector<uint16_t> gamma((size_t)cols);
+        for (int64_t c = 0; c < cols; ++c) gamma[(size_t)c] = metis_oracle_f32_to_bf16(1.0f + 0.001f * (float)(c % 97));
+        DeviceBuffer<uint16_t> dx(x.size()), dg(gamma.size()), dn(x.size());
+        dx.upload(x);
+        dg.upload(gamma);
+        DeviceBuffer<uint8_t> dc((size_t)(rows * cols / 2)), ds((size_t)(rows * cols / 16));
+        DeviceBuffer<float> du(1);
+        const size_t wsb = metis_nvfp4_workspace_bytes(rows, cols);
+        DeviceBuffer<uint8_t> ws(wsb);
+        HIP_OK(hipMemset(ws.p, 0, wsb));
+        const int rc = metis_rmsnorm_nvfp4_quant(dx.p, dg.p, 1e-6f, rows, cols, METIS_MODE_P32, dn.p, dc.p, ds.p, du.p, ws.p, wsb, st);
+        HIP_OK(hipStreamSynchronize(st));
+        std::vector<uint16_t> wn(x.size());
+        std::vector<uint8_t> wc((size_t)(rows * cols / 2)), wsc((size_t)(rows * cols / 16));
+        float wu = 0;
+        metis_oracle_rmsnorm_nvfp4(x.data(), gamma.data(), 1e-6f, rows, cols, 0, wn.data(), wc.data(), wsc.data(), &wu);
+        // the row sum of squares is accumulated in a different order on the device: compare the normed values
+        // to one bf16 ulp and the packed tensor only where the normed values agree exactly
+        const std::vector<uint16_t> gn = dn.download();
+        size_t off_by_more = 0, differ = 0;
+        for (size_t i = 0; i < gn.size(); ++i) {
+            const int d = abs((int)gn[i] - (int)wn[i]);
+            differ += d != 0;
+            off_by_more += d > 1;
+        }
+        char line[160];
+        snprintf(line, sizeof line, "metis_rmsnorm_nvfp4_quant rc=%d: normed within 1 bf16 ulp (%zu of %zu differ by 1)", rc, differ, gn.size());
+        check(rc == METIS_OK && off_by_more == 0 && differ < gn.size() / 50, line);
+        if (differ == 0) {
+            check(dc.download() == wc && ds.download() == wsc && du.download()[0] == wu, "  packed tensor of the normed rows bit-equal");
+        }
+    }
+
+    // ---- 4: GEMM, tiled and skinny dispatch
+    check_linear(272, 320, 256, st, "tiled 256x256");
+    check_linear(96, 132, 96, st, "tiled 128x128");
+    check_linear(48, 160, 512, st, "skinny");
+
+    // ---- 5: error codes
+    {
+        DeviceBuffer<uint16_t> dx(1024);
+        DeviceBuffer<uint8_t> dc(512), ds(64), ws(metis_nvfp4_workspace_bytes(32, 32));
+        DeviceBuffer<float> du(1);
+        check(metis_nvfp4_quant_row(dx.p, 32, 24, 24, 0, dc.p, ds.p, du.p, ws.p, ws.n, st) == METIS_E_SHAPE, "16 does not divide 24 -> METIS_E_SHAPE");
+        check(metis_nvfp4_quant_row(dx.p, 32, 32, 32, 5, dc.p, ds.p, du.p, ws.p, ws.n, st) == METIS_E_ARG, "unknown mode -> METIS_E_ARG");
+        check(metis_nvfp4_quant_row(dx.p, 32, 32, 32, 0, dc.p, ds.p, du.p, ws.p, 16, st) == METIS_E_WORKSPACE, "short workspace -> METIS_E_WORKSPACE");
+        check(metis_nvfp4_quant_row(nullptr, 32, 32, 32, 0, dc.p, ds.p, du.p, ws.p, ws.n, st) == METIS_E_ARG, "null input -> METIS_E_ARG");
+        check(metis_nvfp4_quant_row(nullptr, 0, 32, 32, 0, nullptr, nullptr, nullptr, nullptr, 0, st) == METIS_OK, "empty tensor is a no-op");
+        check(strlen(metis_error_string(METIS_E_SHAPE)) > 0, "metis_error_string");
+    }
+    HIP_OK(hipStreamDestroy(st));
+    printf(failures ? "FAILED %d check(s)\n" : "all checks passed\n", failures);
+    return failures ? 1 : 0;
+}

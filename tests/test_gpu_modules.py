@@ -316,3 +316,35 @@ def test_svd_activation_mode_beats_plain_quantization_on_low_rank_plus_noise():
     assert e_svd < 0.5 * e_plain, (e_svd, e_plain)
     out3 = F.svd_quant(x.reshape(2, 256, 256), q, rank=16, niter=2, tp_simulate=True, tp_parts=2, metis_mode="svd")
     assert out3.shape == (2, 256, 256) and rel_fro(out3.cpu().reshape(512, 256), x.cpu()) < e_plain
+
+
+def test_hot_path_replays_from_a_captured_graph():
+    """Serving loops capture quantize -> GEMM once and replay it: the library launches only kernels (no
+    memset nodes, no allocation, no synchronisation), so every replay on fresh input contents must equal
+    the eager result bit for bit."""
+    from metis_hip import ops
+    g = torch.Generator().manual_seed(12)
+    w = (torch.randn(384, 512, generator=g) * 0.02).bfloat16().cuda()
+    pw = ops.quantize(w)
+    x_static = torch.zeros(64, 512, dtype=torch.bfloat16, device="cuda")
+    gamma = (1 + 0.1 * torch.randn(512, generator=g)).bfloat16().cuda()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        _, p = ops.rmsnorm_quantize(x_static, gamma, 1e-6)     # warm-up allocates the stream's workspace
+        ops.linear_fwd(p, pw)
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            normed, p = ops.rmsnorm_quantize(x_static, gamma, 1e-6)
+            y_static = ops.linear_fwd(p, pw)
+    for seed in (21, 22, 23):
+        x = synthetic_activation(seed, 64, 512).cuda()
+        x_static.copy_(x)
+        graph.replay()
+        torch.cuda.synchronize()
+        got, got_normed = y_static.clone(), normed.clone()
+        want_normed, pe = ops.rmsnorm_quantize(x, gamma, 1e-6)    # eager work between replays
+        want = ops.linear_fwd(pe, pw)
+        torch.cuda.synchronize()
+        assert torch.equal(got_normed, want_normed), seed
+        assert torch.equal(got, want), seed
