@@ -148,3 +148,21 @@ def test_decode_shapes_with_lowrank_and_bias(M, N, K, r):
     torch.cuda.synchronize()
     assert rel_fro(got32.cpu(), want.cpu()) <= 1e-5
     assert rel_fro(got.cpu(), want.cpu().bfloat16()) <= TOL
+
+
+def test_output_offsets_beyond_32_bits():
+    """2.2 G output elements: element offsets m * N + n pass 2^31.  Activation rows repeat with period 256,
+    so output rows must repeat too; one period is checked against the double-precision product."""
+    from metis_hip import ops
+    M, N, K = 49152, 45056, 64
+    base = synthetic_activation(81, 256, K).cuda()
+    w = _weights(82, N, K).cuda()
+    px, pw = ops.quantize(base.repeat(M // 256, 1)), ops.quantize(w)
+    out = ops.linear_fwd(px, pw)
+    assert out.numel() > 2 ** 31
+    want = ops.dequantize(ops.quantize(base), torch.float32).double() @ ops.dequantize(pw, torch.float32).double().T
+    torch.cuda.synchronize()
+    assert rel_fro(out[:256].cpu(), want.cpu().bfloat16()) <= TOL
+    first = out[:256]
+    for rep in (1, 95, 191):
+        assert torch.equal(out[rep * 256:(rep + 1) * 256], first), rep

@@ -267,3 +267,29 @@ def test_signed_zeros_and_negatives_that_round_to_zero(ops, tag, mode):
     _check_packed(ops.quantize(x.cuda(), mode), codes, scales, unit, tag)
     ct, st, ut, _ = O.nvfp4_pack_col(_oracle_in(x, mode))
     _check_packed(ops.quantize(x.cuda(), mode, col=True), ct, st, ut, tag + " col")
+
+
+def test_offsets_beyond_32_bits(ops):
+    """2.4 GB input, 75 M blocks: byte offsets pass 2^31 and 2^32.  The tensor is a 1024-row pattern
+    repeated 36 times, so every repetition must carry the pattern's own codes and scale bytes (the
+    tensor-wide unit is the same) -- checked against the oracle on the pattern."""
+    from oracle import metis_oracle as O
+    pat = synthetic_activation(71, 1024, 32768)
+    codes, scales, unit, _ = O.nvfp4_pack(pat.float())
+    x = pat.cuda().repeat(36, 1)
+    assert x.numel() * 2 > 2 ** 31
+    p = ops.quantize(x, 0)
+    torch.cuda.synchronize()
+    assert float(p.unit.cpu()) == float(unit)
+    cd, sd = codes.cuda(), scales.cuda()
+    for rep in (0, 17, 35):
+        assert torch.equal(p.codes[rep * 1024:(rep + 1) * 1024], cd), rep
+        assert torch.equal(p.scales[rep * 1024:(rep + 1) * 1024], sd), rep
+    assert torch.equal(p.codes.view(36, -1), cd.view(1, -1).expand(36, -1))
+    del p
+    pc = ops.quantize(x, 0, col=True)                         # [32768, 36864 / 2]: blocks run down the repeated rows
+    ct, st, ut, _ = O.nvfp4_pack_col(pat.float())
+    torch.cuda.synchronize()
+    assert float(pc.unit.cpu()) == float(ut)
+    assert torch.equal(pc.codes.view(32768, 36, -1), ct.cuda().view(32768, 1, -1).expand(-1, 36, -1))
+    assert torch.equal(pc.scales.view(32768, 36, -1), st.cuda().view(32768, 1, -1).expand(-1, 36, -1))
