@@ -2,6 +2,7 @@
 (tests/test_metis_quant_cache.py) with counting quantizer subclasses of Cast2Fp32 as spies.
 These run on CPU: identity quantizers take the generic (torch matmul) path, no NVFP4 arithmetic.
 """
+from collections import OrderedDict as OrderedDictCompat
 from types import SimpleNamespace
 
 import pytest
@@ -324,3 +325,36 @@ def test_svd_mode_and_tp_simulation_reassemble_the_input_with_identity_quantizer
         torch.testing.assert_close(out, x, rtol=1e-5, atol=1e-5)
     out = F.svd_quant(x3, Cast2Fp32, rank=8, niter=0, broadcast_dim=0, metis_mode="svd")
     torch.testing.assert_close(out, x3, rtol=1e-5, atol=1e-5)
+
+
+def test_merge_tool_restores_plain_linear_weights(tmp_path):
+    """Patched-and-split model -> state dict -> merge tool -> loads into the unpatched architecture with
+    the original weights (reference tools/convert_bitlinear_to_standard.py:80-172)."""
+    from metis_hip.tools.merge_state_dict import main as merge_main, merge_bitlinear_state_dict
+    torch.manual_seed(11)
+
+    def make():
+        return torch.nn.Sequential(OrderedDictCompat([("q_proj", torch.nn.Linear(64, 48, bias=True)),
+                                                     ("act", torch.nn.ReLU()),
+                                                     ("o_proj", torch.nn.Linear(48, 32, bias=False))]))
+    plain = make()
+    reference_weights = {k: v.clone() for k, v in plain.state_dict().items()}
+    args = MetisArgs(forward_svd_rank=16)
+    args.device = "cpu"
+    replace_linear_with_metis(plain, dtype=torch.float32, metis_args=args, target_modules=["q_proj", "o_proj"],
+                              compute_dtype=torch.float32)
+    sd = plain.state_dict()
+    assert "q_proj.ulinear.weight" in sd and "o_proj.s" in sd and "q_proj.warmup_linear.bias" in sd
+    merged = merge_bitlinear_state_dict(sd)
+    assert set(merged) == set(reference_weights)
+    for k, w in reference_weights.items():
+        torch.testing.assert_close(merged[k], w, rtol=1e-5, atol=1e-5)
+    fresh = make()
+    fresh.load_state_dict(merged)                                # strict: exactly the plain architecture's keys
+    # file round trip and dtype cast
+    from safetensors.torch import load_file, save_file
+    src, dst = tmp_path / "in.safetensors", tmp_path / "out.safetensors"
+    save_file({k: v.contiguous() for k, v in sd.items()}, str(src))
+    merge_main([str(src), str(dst), "--dtype", "bf16"])
+    back = load_file(str(dst))
+    assert set(back) == set(reference_weights) and all(t.dtype == torch.bfloat16 for t in back.values())
