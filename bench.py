@@ -256,6 +256,33 @@ def main():
                             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(d_bytes / d_us / 1e3 / HBM_PEAK_GBS, 4),
                             "traffic": None}}
 
+    # ------------------------------------------------------------------ config 4: one QAT projection, forward +
+    # dgrad + wgrad through the module path (L = 4096 tokens, gate/up shape 1536 -> 8960, bf16 tensors)
+    qat = None
+    if not args.no_decode:
+        from metis_hip import LinearLowbit, LinearLowbitFunction, MetisArgs
+        LinearLowbitFunction.compute_dtype = torch.float32
+        margs = MetisArgs.direct_fp4()
+        margs.cache_quantized_weight = True
+        lin = LinearLowbit(1536, 8960, bias=False, args=margs, device=dev, storage_dtype=torch.bfloat16,
+                           compute_dtype=torch.float32)
+        xq_ = torch.randn(1, 4096, 1536, generator=torch.Generator().manual_seed(1004)).bfloat16().to(dev).requires_grad_(True)
+        dy_ = (torch.randn(1, 4096, 8960, generator=torch.Generator().manual_seed(2004)) * 1e-3).bfloat16().to(dev)
+
+        def qat_step(ev):
+            if ev is not None:
+                ev[0].record()
+            y_ = lin(xq_)
+            y_.backward(dy_.to(y_.dtype))
+            if ev is not None:
+                ev[1].record()
+            lin.weight.grad = None
+            xq_.grad = None
+        _, qat_ms = time_region(torch, qat_step, 10, 3)
+        qat = {"workload": "config 4: LinearLowbit 1536->8960, L=4096, forward + dgrad + wgrad incl. RNE/SR quantization "
+                           "of X, dY (row and column blocked) through the Python module path (P32 arithmetic)",
+               "us_per_step": round(qat_ms * 1e3, 1), "tflops": round(3 * 2.0 * 4096 * 1536 * 8960 / (qat_ms * 1e-3) / 1e12, 1)}
+
     line = {
         "metric": "Metis NVFP4 linear TFLOP/s at 8192x4096x14336 (rank 64)",
         "value": round(value, 2),
@@ -288,6 +315,8 @@ def main():
     }
     if dec is not None:
         line["decode_layer"] = dec
+    if qat is not None:
+        line["qat_projection"] = qat
     if not args.no_cpu_baseline:
         torch_threads = torch.get_num_threads()
         cpu_tflops, cpu_dt, cpu_reps = cpu_baseline_linear(torch, x, v, s, u, res)

@@ -46,7 +46,8 @@ def _workspace(rows: int, cols: int, device: torch.device) -> torch.Tensor:
     key = (device.index, _stream())
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < need:
-        ws = torch.zeros(max(need, 1 << 20), dtype=torch.uint8, device=device)
+        # zero-filled once by a fill kernel (not a memset, which must not be recorded into a captured graph)
+        ws = torch.empty(max(need, 1 << 20), dtype=torch.uint8, device=device).fill_(0)
         _workspaces[key] = ws
     return ws
 
