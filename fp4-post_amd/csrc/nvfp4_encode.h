@@ -100,6 +100,64 @@ __device__ __forceinline__ uint2 encode_rne_pb16(const float (&v)[kBlock], float
     return make_uint2(w[0] | sg[0], w[1] | sg[1]);
 }
 
+// One v_cvt_scalef32_sr_pk_fp4_f32: converts (q0, q1) / 2^MODE with stochastic rounding into byte `byte` of w
+// and keeps w's other bytes.  Written as assembly because the compiler builtin of this ROCm release does not
+// tie the previous value of the destination to the instruction (the other bytes came back undefined); the
+// leading s_nop covers the wait state a partial (op_sel) write needs before the register is read again.
+template <int MODE>
+__device__ __forceinline__ void sr_convert_pair(uint32_t& w, float q0, float q1, uint32_t bits, int byte)
+{
+    typedef float pair_t __attribute__((ext_vector_type(2)));
+    const pair_t q = {q0, q1};
+#define METIS_SR_CVT(SCALE, SEL) asm("s_nop 0\n\tv_cvt_scalef32_sr_pk_fp4_f32 %0, %1, %2, " SCALE SEL : "+v"(w) : "v"(q), "v"(bits))
+    if (MODE == 0) {
+        if (byte == 0) METIS_SR_CVT("1.0", "");
+        else if (byte == 1) METIS_SR_CVT("1.0", " op_sel:[0,0,1,0]");
+        else if (byte == 2) METIS_SR_CVT("1.0", " op_sel:[0,0,0,1]");
+        else METIS_SR_CVT("1.0", " op_sel:[0,0,1,1]");
+    } else {
+        if (byte == 0) METIS_SR_CVT("2.0", "");
+        else if (byte == 1) METIS_SR_CVT("2.0", " op_sel:[0,0,1,0]");
+        else if (byte == 2) METIS_SR_CVT("2.0", " op_sel:[0,0,0,1]");
+        else METIS_SR_CVT("2.0", " op_sel:[0,0,1,1]");
+    }
+#undef METIS_SR_CVT
+}
+
+// Stochastic rounding with the library's own random stream.  The reference adds U(-1/2, 1/2) to the
+// compressed quotient and rounds to nearest (src/Metis/Metis/quant.py:137-147); compress is linear
+// between neighbouring grid points, so this is plain stochastic rounding onto the E2M1 grid:
+// P(up) = (q - lo) / (hi - lo).  The hardware converter v_cvt_scalef32_sr_pk_fp4_f32 does exactly
+// that from 32 random bits per element pair (measured on hardware: unbiased over 2^20 seeds for
+// every grid interval, saturating at 6, sign kept, the two elements of a pair read the random
+// word one bit apart).  One Philox4x32-10 draw serves a block: counter = offset + output block,
+// pair p (elements 2p, 2p+1) takes word p % 4, rotated by 16 bits for p >= 4 (the converter only
+// looks at the top 13 bits).  Scale bytes and unit do not depend on the rounding mode.
+template <int MODE>
+__device__ __forceinline__ uint2 encode_sr_hardware(const float (&v)[kBlock], float s, uint64_t seed, uint64_t offset,
+                                                    int64_t ob)
+{
+    const uint4 r = Philox::draw(offset + (uint64_t)ob, seed);
+    const uint32_t word[4] = {r.x, r.y, r.z, r.w};
+    // MODE 0: x / s in binary32 (div3 is a faithful rounding of the quotient).  MODE 1: bf16(x / h), h = s / 2.
+    const float d = MODE ? 0.5f * s : s;
+    const float rd_ = __builtin_amdgcn_rcpf(d);
+    uint32_t w[2] = {0u, 0u};
+#pragma unroll
+    for (int j = 0; j < kBlock; j += 2) {
+        const int p = j >> 1;
+        const uint32_t bits = p < 4 ? word[p] : __builtin_amdgcn_alignbit(word[p & 3], word[p & 3], 16);
+        float q0 = div3(v[j], d, rd_), q1 = div3(v[j + 1], d, rd_);
+        if (MODE) {
+            const uint32_t qq = rb_pair(q0, q1);
+            q0 = bf16_lo(qq);
+            q1 = bf16_hi(qq);
+        }
+        sr_convert_pair<MODE>(w[p >> 2], q0, q1, bits, p & 3);
+    }
+    return make_uint2(w[0], w[1]);
+}
+
 template <int MODE, bool SR>
 __device__ __forceinline__ uint2 encode_block(const float (&v)[kBlock], float s, const float (&u)[kBlock])
 {
@@ -137,20 +195,6 @@ __device__ __forceinline__ void unpack16(const uint4 a, const uint4 b, float (&v
     const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
 #pragma unroll
     for (int j = 0; j < 8; ++j) { v[2 * j] = bf16_lo(w[j]); v[2 * j + 1] = bf16_hi(w[j]); }
-}
-
-// uniform draws for output block `ob` (16 consecutive elements of the packed orientation)
-template <int MODE>
-__device__ __forceinline__ void philox16(uint64_t seed, uint64_t offset, int64_t ob, float (&u)[kBlock])
-{
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-        uint4 r = Philox::draw(offset + (uint64_t)ob * 4u + g, seed);
-        u[4 * g + 0] = uniform_from_bits<MODE>(r.x);
-        u[4 * g + 1] = uniform_from_bits<MODE>(r.y);
-        u[4 * g + 2] = uniform_from_bits<MODE>(r.z);
-        u[4 * g + 3] = uniform_from_bits<MODE>(r.w);
-    }
 }
 
 // publish the workgroup's maximum block-maximum (non-negative floats order like their bit patterns)

@@ -70,11 +70,12 @@ __global__ __launch_bounds__(256) void quant_codes_kernel(
                 u[j] = MODE ? bf16_lo(((const uint16_t*)noise)[e]) : ((const float*)noise)[e];
             }
         }
-        if (SR && !noise) philox16<MODE>(seed, offset, i, u);
         const float am = block_amax(v);
         gmax = fmaxf(gmax, am);
         ws_amax[i] = (uint16_t)(__float_as_uint(am) >> 16);          // am is a bf16 value
-        codes[i] = encode_block<MODE, SR>(v, block_scalar<MODE>(am), u);
+        // caller-supplied noise: the reference's literal sequence; own stream: hardware stochastic rounding
+        codes[i] = (SR && !noise) ? encode_sr_hardware<MODE>(v, block_scalar<MODE>(am), seed, offset, i)
+                                  : encode_block<MODE, SR>(v, block_scalar<MODE>(am), u);
     }
     publish_group_max(gmax, ws_gmax);
 }
@@ -118,10 +119,10 @@ __global__ __launch_bounds__(256) void quant_codes_col_kernel(
                         u[j] = MODE ? bf16_lo(((const uint16_t*)noise)[e]) : ((const float*)noise)[e];
                     }
                 }
-                if (SR && !noise) philox16<MODE>(seed, offset, (int64_t)c * nbc + b, u);
                 am = block_amax(v);
                 gmax = fmaxf(gmax, am);
-                packed = encode_block<MODE, SR>(v, block_scalar<MODE>(am), u);
+                packed = (SR && !noise) ? encode_sr_hardware<MODE>(v, block_scalar<MODE>(am), seed, offset, (int64_t)c * nbc + b)
+                                        : encode_block<MODE, SR>(v, block_scalar<MODE>(am), u);
             }
             s_codes[cl][bl] = packed;
             s_amax[cl][bl] = (uint16_t)(__float_as_uint(am) >> 16);

@@ -139,28 +139,80 @@ def test_sr_explicit_noise(ops, golden, tag, mode, col):
 
 @pytest.mark.parametrize("tag,mode", MODES)
 @pytest.mark.parametrize("col", [False, True])
-def test_sr_internal_philox_stream(ops, tag, mode, col):
-    """The device draws Philox4x32-10(counter = offset + e/4, key = seed), word e%4, for packed element e."""
+def test_sr_internal_stream_properties(ops, tag, mode, col):
+    """With its own random stream the library rounds stochastically in hardware, one Philox draw per
+    output block.  What must hold whatever the draws: scale bytes and unit are those of the
+    round-to-nearest pack (bit-exact against the oracle); every code is one of the two grid neighbours
+    of the exact quotient with the sign of x; the result is a function of (seed, offset) only; and since
+    the stream is indexed by output block, column packing equals row packing of the transpose."""
+    from oracle import metis_oracle as O
+    x = synthetic_activation(300, 64, 128)
+    x.view(-1)[::53] = 0
+    seed, offset = 0x1234_5678_9ABC_DEF0, 77
+    xd = x.cuda()
+    p = ops.quantize(xd, mode, col=col, sr=True, seed=seed, offset=offset)
+    xin = _oracle_in(x, mode)
+    xt = xin.t().contiguous() if col else xin
+    _, scales, unit, _ = O.nvfp4_pack(xt)
+    torch.cuda.synchronize()
+    assert torch.equal(p.scales.cpu(), scales) and float(p.unit.cpu()) == float(unit)
+    # bracket: code magnitude in {floor, ceil} of the quotient on the grid {0,1,2,3,4,6,8,12} (units of s/2)
+    scalar = O.block_scalars(xt).double().reshape(xt.shape[0], -1, 1)
+    q = (xt.double().abs().reshape(xt.shape[0], -1, 16) / (scalar / 2)).reshape(xt.shape)
+    grid = torch.tensor([0, 1, 2, 3, 4, 6, 8, 12], dtype=torch.float64)
+    nib = torch.stack((p.codes.cpu() & 0xF, p.codes.cpu() >> 4), dim=-1).reshape(xt.shape)
+    mag = grid[(nib & 7).long()]
+    lo = grid[(torch.bucketize(q * (1 - 1e-2), grid, right=True) - 1).clamp(0, 7)]
+    hi = grid[torch.bucketize(q * (1 + 1e-2), grid).clamp(0, 7)]
+    assert bool(((mag >= lo) & (mag <= hi)).all())
+    nonzero = xt.float() != 0
+    assert bool((((nib & 8) != 0) == (xt.float() < 0))[nonzero].all())
+    assert bool((nib[~nonzero] == 0).all())
+    assert float((mag != grid[(torch.bucketize(q, grid) - 0).clamp(0, 7)]).double().mean()) > 0.05   # it does round both ways
+    # determinism and sensitivity
+    again = ops.quantize(xd, mode, col=col, sr=True, seed=seed, offset=offset)
+    other_seed = ops.quantize(xd, mode, col=col, sr=True, seed=seed + 1, offset=offset)
+    other_off = ops.quantize(xd, mode, col=col, sr=True, seed=seed, offset=offset + 1)
+    assert torch.equal(p.codes, again.codes)
+    assert not torch.equal(p.codes, other_seed.codes) and not torch.equal(p.codes, other_off.codes)
+    if col:
+        as_rows = ops.quantize(xd.t().contiguous(), mode, sr=True, seed=seed, offset=offset)
+        assert torch.equal(p.codes, as_rows.codes) and torch.equal(p.scales, as_rows.scales)
+
+
+@pytest.mark.parametrize("tag,mode", MODES)
+def test_three_call_quant_draws_the_documented_philox_stream(tag, mode):
+    """quant() without caller noise draws Philox4x32-10(counter = offset + e/4, key = seed), word e % 4, for
+    element e; with the same draws fed to the oracle as explicit noise the values agree bit for bit.  This
+    pins the device generator to the host implementation checked against the published known answers."""
+    from metis_hip import quant_func
+    from metis_hip.quant import _NVFP4Base
     from oracle import metis_oracle as O
     from philox_ref import uniform_for_elements
-    x = synthetic_activation(300, 64, 128)
-    seed, offset = 0x1234_5678_9ABC_DEF0, 77
-    p = ops.quantize(x.cuda(), mode, col=col, sr=True, seed=seed, offset=offset)
-    u = torch.from_numpy(uniform_for_elements(x.numel(), seed, offset, bf16=(mode == 1)))
+    q = quant_func["nvfp4e2m1b"]
+    x = synthetic_activation(301, 32, 128)
     xin = _oracle_in(x, mode)
-    if col:
-        u_as_x = u.reshape(128, 64).t().contiguous()               # draws are indexed in the packed orientation
-        codes, scales, unit, _ = O.nvfp4_pack_col(xin, u_as_x.to(xin.dtype))
-    else:
-        codes, scales, unit, _ = O.nvfp4_pack(xin, u.reshape(64, 128).to(xin.dtype))
-    _check_packed(p, codes, scales, unit, f"philox col={col}")
+    keep = (_NVFP4Base.sr_seed, _NVFP4Base.sr_offset)
+    _NVFP4Base.sr_seed, _NVFP4Base.sr_offset = 0x0BAD_CAFE_1234_5678, 1000
+    try:
+        xd = xin.cuda()
+        s = q.get_scalar(xd)
+        got = q.quant(xd, s)
+    finally:
+        _NVFP4Base.sr_seed, _NVFP4Base.sr_offset = keep
+    u = torch.from_numpy(uniform_for_elements(x.numel(), 0x0BAD_CAFE_1234_5678, 1000, bf16=(mode == 1))).reshape(32, 128)
+    want = O.quant(xin, O.get_scalar(xin), noise=u.to(xin.dtype))
+    torch.cuda.synchronize()
+    clamped = want.abs() > 6                                       # the reference's off-grid 8: kept by quant()
+    assert same_bits(got.cpu(), want) or bool((got.cpu() == want)[~clamped].all())
 
 
-def test_sr_is_unbiased(ops):
+@pytest.mark.parametrize("tag,mode", MODES)
+def test_sr_is_unbiased(ops, tag, mode):
     """E[deq(SR(x))] = x for values inside the grid: mean over 4096 independent draws."""
     vals = torch.tensor([0.1, 0.3, 0.6, 0.9, 1.2, 1.7, 2.3, 2.9, 3.4, 4.4, 5.1, 5.8, -0.2, -1.1, -2.6, 6.0])
     x = vals.bfloat16().repeat(4096, 1).contiguous()              # block max 6 -> scalar 1 + 1e-9
-    p = ops.quantize(x.cuda(), 0, sr=True, seed=42)
+    p = ops.quantize(x.cuda(), mode, sr=True, seed=42)
     deq = ops.dequantize(p, torch.float32).cpu()
     mean = deq.mean(0)
     step = torch.tensor([0.5] * 4 + [0.5] * 3 + [1.0] * 2 + [2.0] * 3 + [0.5, 0.5, 1.0, 2.0])
@@ -169,8 +221,8 @@ def test_sr_is_unbiased(ops):
     assert bool((deq[:, :15].std(0) > 0).all())                      # every off-grid value rounds both ways
     assert float(deq[:, 15].std()) == 0.0                            # the block maximum sits on the grid
     # different seeds give different streams, same seed the same codes
-    p2 = ops.quantize(x.cuda(), 0, sr=True, seed=42)
-    p3 = ops.quantize(x.cuda(), 0, sr=True, seed=43)
+    p2 = ops.quantize(x.cuda(), mode, sr=True, seed=42)
+    p3 = ops.quantize(x.cuda(), mode, sr=True, seed=43)
     assert torch.equal(p.codes, p2.codes) and not torch.equal(p.codes, p3.codes)
 
 
