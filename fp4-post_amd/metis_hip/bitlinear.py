@@ -283,7 +283,9 @@ class LinearLowbitFunction(torch.autograd.Function):
                     and grad_output.dtype in (torch.float32, torch.bfloat16)):
                 # dgrad: contraction over N; wgrad: contraction over tokens.  Operands are packed straight from the
                 # tensors autograd hands over, in compute_dtype arithmetic (no upcast copies of bf16 tensors).
-                dy2, x2, cd = _flat2d(grad_output), _flat2d(input_), F.compute_dtype
+                cd = F.compute_dtype
+                # the kernels read bf16 values: one rounding pass per tensor, shared by its row and column packing
+                dy2, x2 = _flat2d(grad_output).to(torch.bfloat16), _flat2d(input_).to(torch.bfloat16)
                 p_dy = qg.pack(dy2, arith=cd)
                 pw_col = ctx.pw.transposed                    # lives as long as the (possibly cached) packed weight
                 if pw_col is None:
