@@ -488,26 +488,34 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_nvfp4_large_kernel(
     }
 }
 
+// Dynamic LDS above 64 KiB has to be allowed per kernel function and per device: done once for each pair.
+static int allow_dynamic_lds(const void* fn, size_t bytes, bool (&done)[64])
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return METIS_E_DEVICE;
+    if (!done[dev]) {
+        if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess) return METIS_E_DEVICE;
+        done[dev] = true;
+    }
+    return METIS_OK;
+}
+
 template <int WN_WAVES>
 static int launch_large(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes,
                         const void* b_scales, const float* b_unit, int64_t M, int64_t N, int64_t K, const void* t,
                         const void* u, int64_t r, const void* bias, void* out, int out_dtype, hipStream_t st)
 {
-    static bool attr_set[2] = {false, false};
+    static bool attr_set[2][64] = {};
     const size_t lds_bytes = 2 * (size_t)L_STAGE_HALVES * sizeof(uint16_t);
     const int f32 = out_dtype == METIS_DTYPE_F32;
     const void* fn = f32 ? (const void*)gemm_nvfp4_large_kernel<1, WN_WAVES> : (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES>;
-    if (const char* d = getenv("METIS_GEMM_DBG")) {            // measurement switches, results are meaningless:
-        const int v = atoi(d);                                 // 1 = no operand fetch/expansion, 7 = also no barriers
-        if (v == 1 || v == 7) {
-            fn = v == 1 ? (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 1> : (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 7>;
-            (void)hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-        }
-    }
-    if (!attr_set[f32]) {
-        if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
-            return METIS_E_DEVICE;
-        attr_set[f32] = true;
+    const char* d = getenv("METIS_GEMM_DBG");                  // measurement switches, results are meaningless:
+    const int v = d ? atoi(d) : 0;                             // 1 = no operand fetch/expansion, 7 = also no barriers
+    if (v == 1 || v == 7) {
+        fn = v == 1 ? (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 1> : (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 7>;
+        if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess) return METIS_E_DEVICE;
+    } else if (const int rc = allow_dynamic_lds(fn, lds_bytes, attr_set[f32])) {
+        return rc;
     }
     const int tiles_m = (int)((M + L_BM - 1) / L_BM), tiles_n = (int)((N + L_BN - 1) / L_BN);
     const int total = tiles_m * tiles_n;
@@ -916,15 +924,11 @@ int gemm_expanded(const void* a_exp, const float* a_unit, const void* b_exp, con
     if (M == 0 || N == 0) return METIS_OK;
     if (!a_exp || !a_unit || !b_exp || !b_unit || !out) return METIS_E_ARG;
     if (((uintptr_t)a_exp % 16) || ((uintptr_t)b_exp % 16) || ((uintptr_t)out % 16)) return METIS_E_ARG;
-    static bool attr_set[2] = {false, false};
+    static bool attr_set[2][64] = {};
     const size_t lds_bytes = 2 * (size_t)X_STAGE_BYTES;
     const int f32 = out_dtype == METIS_DTYPE_F32;
     const void* fn = f32 ? (const void*)gemm_f16_large_kernel<1> : (const void*)gemm_f16_large_kernel<0>;
-    if (!attr_set[f32]) {
-        if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
-            return METIS_E_DEVICE;
-        attr_set[f32] = true;
-    }
+    if (const int rc = allow_dynamic_lds(fn, lds_bytes, attr_set[f32])) return rc;
     const int tiles_m = (int)((M + L_BM - 1) / L_BM), tiles_n = (int)((N + L_BN - 1) / L_BN);
     const int total = tiles_m * tiles_n;
     const unsigned grid_x = (unsigned)(((total + 7) / 8) * 8);
