@@ -10,8 +10,9 @@ from ._lib import MODE_P32, MODE_PB16, MetisHipError
 from .bitlinear import BitLinear, LinearLowbit, LinearLowbitFunction
 from .ops import PackedNVFP4
 from .patch import MetisArgs, replace_linear_with_metis, replace_model_with_metis
-from .quant import (BlockQuantFunc, Cast2Fp32, Cast2NVFp4e2m1Block, Cast2NVFp4e2m1BlockNOSR, QuantFunc, quant_func)
+from .quant import (BlockQuantFunc, Cast2Fp32, Cast2NVFp4e2m1Block, Cast2NVFp4e2m1BlockNOSR, QuantFunc,
+                    nvfp4_nosr_qdq_compile_status, quant_func)
 
-__all__ = ["ops", "PackedNVFP4", "MODE_P32", "MODE_PB16", "MetisHipError", "quant_func", "QuantFunc", "BlockQuantFunc",
+__all__ = ["nvfp4_nosr_qdq_compile_status", "ops", "PackedNVFP4", "MODE_P32", "MODE_PB16", "MetisHipError", "quant_func", "QuantFunc", "BlockQuantFunc",
            "Cast2Fp32", "Cast2NVFp4e2m1Block", "Cast2NVFp4e2m1BlockNOSR", "LinearLowbitFunction", "LinearLowbit",
            "BitLinear", "MetisArgs", "replace_linear_with_metis", "replace_model_with_metis"]

@@ -176,6 +176,14 @@ quant_func = {
 }
 
 
+def nvfp4_nosr_qdq_compile_status() -> str:
+    """The reference validates a torch.compile'd fused QDQ against the eager one before using it and reports
+    "validated" / "not validated" / "disabled: ..." (quant.py:61-66).  Here the fused QDQ is a hand-written
+    kernel whichever way `compile_quantize_dequantize` is set, checked bit for bit by the test-suite: the
+    answer callers branch on is always "validated"."""
+    return "validated"
+
+
 def is_hip_nvfp4(q) -> bool:
     """True when ``q`` is one of the kernel-backed NVFP4 classes themselves (not a user subclass
     that overrides the arithmetic)."""

@@ -348,3 +348,20 @@ def test_hot_path_replays_from_a_captured_graph():
         torch.cuda.synchronize()
         assert torch.equal(got_normed, want_normed), seed
         assert torch.equal(got, want), seed
+
+
+def test_compile_flag_is_accepted_and_changes_nothing():
+    """Reference tests/test_metis_quant_cache.py:30-42: the flag that selects the torch.compile'd QDQ there
+    selects the same kernel here; results are identical at atol 0 and the status helper says so."""
+    from metis_hip import nvfp4_nosr_qdq_compile_status, quant_func
+    q = quant_func["nvfp4e2m1bnosr"]
+    x = synthetic_activation(90, 8 * 16, 128).reshape(8, 16, 128).cuda()
+    q.compile_quantize_dequantize = False
+    expected = q.quantize_dequantize(x)
+    q.compile_quantize_dequantize = True
+    try:
+        actual = q.quantize_dequantize(x)
+    finally:
+        q.compile_quantize_dequantize = False
+    assert same_bits(actual, expected)
+    assert nvfp4_nosr_qdq_compile_status() == "validated"
