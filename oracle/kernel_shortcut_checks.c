@@ -8,6 +8,8 @@
  *   pb16        every op rounded to bf16: all (h, x) pairs of positive bf16 values with x/h in
  *               [0.05, 13.2]: literal sequence  vs  q = bf16(div3(x, h)), three q values nudged
  *               onto their tie, round-to-nearest-even onto the grid.
+ *   div6        amax / 6 by a constant reciprocal and one correction: every finite non-negative bf16 value
+ *               against the correctly rounded quotient (the block scalar, quant.py:19).
  *   p32 ITERS   binary32 arithmetic: for ITERS block scalars (realistic, random, and adversarially
  *               close to decision thresholds) and the bf16 inputs around every threshold:
  *               literal sequence  vs  round-to-nearest-even of div3(x, s), for blocks the kernel's
@@ -161,10 +163,25 @@ static long check_p32(long iters)
     return bad;
 }
 
+static long check_div6(void)
+{
+    long n = 0, bad = 0;
+    for (uint32_t p = 0; p < 0x7f80; ++p) {
+        const float a = bits_f(p << 16), c = 0x1.555556p-3f;
+        const float q = a * c;
+        const float r = fmaf(-6.0f, q, a);
+        n++;
+        if (f_bits(fmaf(r, c, q)) != f_bits(a / 6.0f)) bad++;
+    }
+    printf("div6: cases %ld mismatches %ld\n", n, bad);
+    return bad;
+}
+
 int main(int argc, char** argv)
 {
+    if (argc >= 2 && !strcmp(argv[1], "div6")) return check_div6() ? 1 : 0;
     if (argc >= 2 && !strcmp(argv[1], "pb16")) return check_pb16() ? 1 : 0;
     if (argc >= 3 && !strcmp(argv[1], "p32")) return check_p32(atol(argv[2])) ? 1 : 0;
-    fprintf(stderr, "usage: %s pb16 | p32 ITERS\n", argv[0]);
+    fprintf(stderr, "usage: %s div6 | pb16 | p32 ITERS\n", argv[0]);
     return 2;
 }

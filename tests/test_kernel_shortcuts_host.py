@@ -14,7 +14,8 @@ BIN = os.path.join(ROOT, "oracle", "kernel_shortcut_checks")
 
 
 def _run(*args):
-    if not os.path.exists(BIN):
+    src = os.path.join(ROOT, "oracle", "kernel_shortcut_checks.c")
+    if not os.path.exists(BIN) or os.path.getmtime(BIN) < os.path.getmtime(src):
         subprocess.run(["make", "-C", os.path.join(ROOT, "oracle"), "kernel_shortcut_checks"], check=True,
                        capture_output=True)
     env = dict(os.environ, OMP_NUM_THREADS=str(min(8, os.cpu_count() or 1)))
@@ -22,6 +23,10 @@ def _run(*args):
     assert out.returncode == 0, out.stdout + out.stderr
     assert "mismatches 0" in out.stdout, out.stdout
     return out.stdout
+
+
+def test_block_scalar_division_by_six_is_correctly_rounded_for_every_bf16_value():
+    assert "cases 32640" in _run("div6")
 
 
 def test_bf16_mode_shortcut_is_exact_for_every_bf16_pair():
