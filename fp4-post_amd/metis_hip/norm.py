@@ -1,0 +1,114 @@
+"""RMSNorm fused with the NVFP4 quantization of its output, wired into a projection group.
+
+The reference has no fused norm: it runs the model's RMSNorm (src/Metis/models/llama.py:23-31; the
+Hugging Face Qwen2/Llama classes compute the same thing) and then the first projection of a
+{q,k,v} or {gate,up} group quantizes the normed tensor once for the whole group
+(src/Metis/Metis/bitlinear.py:676-702).  `FusedRMSNormQuant` replaces the norm module in front of
+such a group: one kernel reads the hidden states once and writes the normed bf16 tensor and its
+packed NVFP4 form, and the packed tensor is left in the group's cache under the identity of the
+normed tensor, which is exactly what the group's first projection would have put there.
+"""
+from __future__ import annotations
+
+import weakref
+
+import torch
+from torch import nn
+
+from . import ops
+from ._lib import MODE_P32, MODE_PB16
+from .bitlinear import BitLinear, LinearLowbitFunction
+from .quant import is_hip_nvfp4
+
+
+class _NormedWithGrad(torch.autograd.Function):
+    """Carries the kernel's normed output into autograd: forward hands the precomputed tensor through,
+    backward is the RMSNorm gradient in binary32."""
+
+    @staticmethod
+    def forward(ctx, x, weight, normed, eps):
+        ctx.save_for_backward(x, weight)
+        ctx.eps = eps
+        return normed.view_as(normed)
+
+    @staticmethod
+    def backward(ctx, g):
+        x, weight = ctx.saved_tensors
+        xf, gf = x.float(), g.float()
+        rstd = torch.rsqrt(xf.pow(2).mean(dim=-1, keepdim=True) + ctx.eps)
+        xhat = xf * rstd
+        g_weight = (gf * xhat.to(x.dtype).float()).reshape(-1, x.shape[-1]).sum(dim=0).to(weight.dtype)
+        gh = gf * weight.float()
+        g_x = (rstd * (gh - xhat * (gh * xhat).mean(dim=-1, keepdim=True))).to(x.dtype)
+        return g_x, g_weight, None, None
+
+
+class FusedRMSNormQuant(nn.Module):
+    """Drop-in for an RMSNorm module (`weight`, `variance_epsilon`) whose output feeds a projection group."""
+
+    def __init__(self, weight: nn.Parameter, eps: float, group: dict):
+        super().__init__()
+        self.weight = weight
+        self.variance_epsilon = eps
+        self.group = group
+
+    @classmethod
+    def from_norm(cls, norm: nn.Module, group: dict) -> "FusedRMSNormQuant":
+        eps = getattr(norm, "variance_epsilon", None)
+        if eps is None:
+            eps = getattr(norm, "eps", 1e-6)
+        return cls(norm.weight, float(eps), group)
+
+    def extra_repr(self):
+        return f"{tuple(self.weight.shape)}, eps={self.variance_epsilon}, group={self.group['name']}"
+
+    def _plain(self, x):
+        dtype = x.dtype
+        h = x.to(torch.float32)
+        h = h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + self.variance_epsilon)
+        return self.weight * h.to(dtype)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        F = LinearLowbitFunction
+        cols = x.shape[-1]
+        fused = (x.is_cuda and x.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16 and cols % 32 == 0
+                 and cols <= 16384 and is_hip_nvfp4(F.q_forward_input) and not F.enable_activation_svd
+                 and not F.enable_nv_recipe)
+        if not fused:
+            return self._plain(x)
+        mode = MODE_P32 if F.compute_dtype == torch.float32 else MODE_PB16
+        with torch.no_grad():
+            normed, packed = ops.rmsnorm_quantize(x, self.weight, self.variance_epsilon, mode)
+        normed = normed.reshape(x.shape)
+        out = _NormedWithGrad.apply(x, self.weight, normed, self.variance_epsilon) if torch.is_grad_enabled() and (
+            x.requires_grad or self.weight.requires_grad) else normed
+        group = self.group
+
+        def clear(ref):
+            if group.get("input_ref") is ref:
+                group["input_ref"] = None
+                group["quantized_input"] = None
+
+        group["input_ref"] = weakref.ref(out, clear)
+        group["quantized_input"] = packed
+        return out
+
+
+def fuse_rmsnorm_into_groups(model: nn.Module) -> int:
+    """Replace `input_layernorm` / `post_attention_layernorm` of every decoder layer whose q/k/v or
+    gate/up projections are BitLinear layers sharing an activation group.  Returns the number of norms
+    replaced.  Layers with other layouts are left alone."""
+    replaced = 0
+    for layer in model.modules():
+        for norm_name, path in (("input_layernorm", ("self_attn", "q_proj")), ("post_attention_layernorm", ("mlp", "gate_proj"))):
+            norm = getattr(layer, norm_name, None)
+            owner = getattr(layer, path[0], None)
+            proj = getattr(owner, path[1], None) if owner is not None else None
+            if norm is None or isinstance(norm, FusedRMSNormQuant) or not isinstance(proj, BitLinear):
+                continue
+            group = getattr(proj, "activation_group", None)
+            if group is None or not hasattr(norm, "weight") or norm.weight.dim() != 1:
+                continue
+            setattr(layer, norm_name, FusedRMSNormQuant.from_norm(norm, group))
+            replaced += 1
+    return replaced

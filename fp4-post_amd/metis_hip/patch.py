@@ -102,9 +102,14 @@ def replace_linear_with_metis(model, dtype, metis_args, target_modules=None, com
     return model
 
 
-def replace_model_with_metis(model, metis_args=None):
-    """bf16 storage and compute, default targets (reference grpo.py:199-215)."""
+def replace_model_with_metis(model, metis_args=None, fuse_norms: bool = False):
+    """bf16 storage and compute, default targets (reference grpo.py:199-215).  fuse_norms additionally
+    replaces the RMSNorm in front of every q/k/v and gate/up group by the fused norm+quant module."""
     if metis_args is None:
         metis_args = MetisArgs()
-    return replace_linear_with_metis(model=model, dtype=torch.bfloat16, metis_args=metis_args,
-                                     target_modules=list(DEFAULT_TARGETS), compute_dtype=torch.bfloat16)
+    model = replace_linear_with_metis(model=model, dtype=torch.bfloat16, metis_args=metis_args,
+                                      target_modules=list(DEFAULT_TARGETS), compute_dtype=torch.bfloat16)
+    if fuse_norms:
+        from .norm import fuse_rmsnorm_into_groups
+        fuse_rmsnorm_into_groups(model)
+    return model

@@ -365,3 +365,73 @@ def test_compile_flag_is_accepted_and_changes_nothing():
         q.compile_quantize_dequantize = False
     assert same_bits(actual, expected)
     assert nvfp4_nosr_qdq_compile_status() == "validated"
+
+
+def test_fused_rmsnorm_feeds_the_projection_groups_of_a_qwen2_layer():
+    """The RMSNorm in front of {q,k,v} and {gate,up} is replaced by the fused norm+quant module: the
+    groups find their packed activation already cached (no quantizer launch for the normed tensors),
+    the layer output and the gradients agree with the unfused patched layer, and norm weights get
+    gradients."""
+    pytest.importorskip("transformers")
+    from transformers.models.qwen2.modeling_qwen2 import Qwen2Config, Qwen2DecoderLayer, Qwen2RotaryEmbedding
+    from metis_hip import FusedRMSNormQuant, MetisArgs, fuse_rmsnorm_into_groups, quant_func, replace_model_with_metis
+    torch.manual_seed(0)
+    cfg = Qwen2Config(hidden_size=256, intermediate_size=512, num_attention_heads=4, num_key_value_heads=2,
+                      num_hidden_layers=1, vocab_size=128, max_position_embeddings=256)
+    cfg._attn_implementation = "eager"
+    layer = Qwen2DecoderLayer(cfg, layer_idx=0).to(torch.bfloat16).cuda()
+    for p in layer.parameters():
+        if p.dim() == 2:
+            torch.nn.init.normal_(p, std=0.02)
+        else:
+            torch.nn.init.normal_(p, mean=1.0, std=0.1)
+    holder = torch.nn.ModuleDict({"layer": layer})
+    replace_model_with_metis(holder, MetisArgs.direct_fp4(forward_svd_rank=32))
+    x = torch.randn(2, 64, 256, device="cuda", dtype=torch.bfloat16)
+    pos = torch.arange(64, device="cuda").unsqueeze(0).expand(2, -1)
+    pe = Qwen2RotaryEmbedding(cfg).cuda()(x, pos)
+
+    def run(inp):
+        out = holder["layer"](inp, position_embeddings=pe, attention_mask=None, position_ids=pos)
+        return out[0] if isinstance(out, tuple) else out
+
+    def grads():
+        xr = x.clone().requires_grad_(True)
+        for p in holder.parameters():
+            p.grad = None
+        out = run(xr)
+        out.float().square().mean().backward()
+        lyr = holder["layer"]
+        return (out.detach().float().cpu(), xr.grad.float().cpu(), lyr.input_layernorm.weight.grad.float().cpu(),
+                lyr.post_attention_layernorm.weight.grad.float().cpu())
+
+    plain = grads()
+    assert fuse_rmsnorm_into_groups(holder) == 2
+    lyr = holder["layer"]
+    assert isinstance(lyr.input_layernorm, FusedRMSNormQuant) and isinstance(lyr.post_attention_layernorm, FusedRMSNormQuant)
+    assert lyr.input_layernorm.group is lyr.self_attn.q_proj.activation_group
+    assert lyr.post_attention_layernorm.group is lyr.mlp.gate_proj.activation_group
+    assert fuse_rmsnorm_into_groups(holder) == 0                       # idempotent
+    fused = grads()
+    assert rel_fro(fused[0], plain[0]) < 2e-2                              # a bf16 ulp of the norm here and there
+    assert rel_fro(fused[1], plain[1]) < 0.25                              # backward re-draws its stochastic rounding
+    assert rel_fro(fused[2], plain[2]) < 0.25 and rel_fro(fused[3], plain[3]) < 0.25
+    # the normed tensors are never quantized by the projections: only o_proj's and down_proj's inputs are
+    base = quant_func["nvfp4e2m1bnosr"]
+    orig = base.pack.__func__
+    seen = []
+
+    def spy(cls, t_, col=False, noise=None, arith=None):
+        if not col:
+            seen.append(tuple(t_.shape))
+        return orig(cls, t_, col, noise, arith)
+
+    base.pack = classmethod(spy)
+    try:
+        with torch.no_grad():
+            run(x)
+    finally:
+        base.pack = classmethod(orig)
+    # q/k/v and gate/up inputs came packed from the norms: the only row quantizations left are o_proj's input
+    # (attention output, also [128, 256]) and down_proj's (the MLP activation)
+    assert sorted(seen) == [(128, 256), (128, 512)], seen
