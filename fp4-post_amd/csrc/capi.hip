@@ -140,4 +140,31 @@ int metis_linear_wgrad(const void* dyt_codes, const void* dyt_scales, const floa
                       nullptr, grad_weight, out_dtype, (hipStream_t)stream);
 }
 
+size_t metis_linear_workspace_bytes(int64_t M, int64_t N, int64_t K) { return gemm_workspace_bytes(M, N, K); }
+
+int metis_linear_fwd_ws(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes,
+                        const void* b_scales, const float* b_unit, int64_t M, int64_t N, int64_t K, const void* t,
+                        const void* u, int64_t r, const void* bias, void* out, int out_dtype, void* workspace,
+                        size_t workspace_bytes, void* stream)
+{
+    return gemm_nvfp4(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype,
+                      (hipStream_t)stream, workspace, workspace_bytes);
+}
+
+int metis_linear_dgrad_ws(const void* dy_codes, const void* dy_scales, const float* dy_unit, const void* wt_codes,
+                          const void* wt_scales, const float* wt_unit, int64_t L, int64_t N, int64_t K, void* grad_input,
+                          int out_dtype, void* workspace, size_t workspace_bytes, void* stream)
+{
+    return gemm_nvfp4(dy_codes, dy_scales, dy_unit, wt_codes, wt_scales, wt_unit, L, K, N, nullptr, nullptr, 0, nullptr,
+                      grad_input, out_dtype, (hipStream_t)stream, workspace, workspace_bytes);
+}
+
+int metis_linear_wgrad_ws(const void* dyt_codes, const void* dyt_scales, const float* dyt_unit, const void* xt_codes,
+                          const void* xt_scales, const float* xt_unit, int64_t L, int64_t N, int64_t K, void* grad_weight,
+                          int out_dtype, void* workspace, size_t workspace_bytes, void* stream)
+{
+    return gemm_nvfp4(dyt_codes, dyt_scales, dyt_unit, xt_codes, xt_scales, xt_unit, N, K, L, nullptr, nullptr, 0,
+                      nullptr, grad_weight, out_dtype, (hipStream_t)stream, workspace, workspace_bytes);
+}
+
 }  // extern "C"

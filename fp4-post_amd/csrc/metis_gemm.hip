@@ -249,12 +249,29 @@ __device__ __forceinline__ void sched_substep()
     }
 }
 
-template <int OUT_F32, int WN_WAVES, int DBG = 0>
+// logical tile number -> origin of its 256 x 256 tile: groups of 4 tile-rows, walked column by column
+__device__ __forceinline__ void tile_origin(int logical, int tiles_m, int tiles_n, int& m0, int& n0)
+{
+    constexpr int GM = 4;
+    const int group = logical / (GM * tiles_n);
+    const int first_m = group * GM;
+    const int gsize = min(tiles_m - first_m, GM);
+    const int tm = first_m + (logical % (GM * tiles_n)) % gsize;
+    const int tn = (logical % (GM * tiles_n)) / gsize;
+    m0 = tm * L_BM;
+    n0 = tn * L_BN;
+}
+
+// SPLIT: the grid holds nsplit workgroups per tile, each contracting its own range of K steps; workgroup
+// `logical_all` leaves its binary32 tile (units applied; low-rank term and bias in split 0 only) in
+// ws[logical_all][65536], ordered as the accumulator registers lie, for gemm_splitk_reduce_kernel.
+template <int OUT_F32, int WN_WAVES, int DBG = 0, int SPLIT = 0>
 __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_nvfp4_large_kernel(
     const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const float* __restrict__ a_unit,
     const uint8_t* __restrict__ b_codes, const uint8_t* __restrict__ b_scales, const float* __restrict__ b_unit,
     int M, int N, int K, const uint16_t* __restrict__ t, const uint16_t* __restrict__ u, int r,
-    const uint16_t* __restrict__ bias, void* __restrict__ out, int tiles_m, int tiles_n)
+    const uint16_t* __restrict__ bias, void* __restrict__ out, int tiles_m, int tiles_n, float* __restrict__ ws,
+    int nsplit)
 {
     extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
     constexpr int TM = 4;                            // 32-tall MFMA tiles per wave along m
@@ -268,16 +285,16 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_nvfp4_large_kernel(
 
     // ---- tile assignment (XCD-contiguous, grouped)
     const int total = tiles_m * tiles_n;
-    const int per_xcd = (total + 7) / 8;
-    const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if (logical >= total) return;
-    constexpr int GM = 4;
-    const int group = logical / (GM * tiles_n);
-    const int first_m = group * GM;
-    const int gsize = min(tiles_m - first_m, GM);
-    const int tm = first_m + (logical % (GM * tiles_n)) % gsize;
-    const int tn = (logical % (GM * tiles_n)) / gsize;
-    const int m0 = tm * L_BM, n0 = tn * L_BN;
+    const int total_all = SPLIT ? total * nsplit : total;
+    const int per_xcd = (total_all + 7) / 8;
+    const int logical_all = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (logical_all >= total_all) return;
+    const int split = SPLIT ? logical_all / total : 0;           // consecutive workgroups of an XCD share a K range
+    int m0, n0;
+    tile_origin(SPLIT ? logical_all % total : logical_all, tiles_m, tiles_n, m0, n0);
+    const int steps_all = K / BK;
+    const int step_begin = SPLIT ? (int)((int64_t)split * steps_all / nsplit) : 0;
+    const int step_end = SPLIT ? (int)((int64_t)(split + 1) * steps_all / nsplit) : steps_all;
 
     float16_t acc[TM][TN];
 #pragma unroll
@@ -297,8 +314,8 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_nvfp4_large_kernel(
         const int trow = q * NTHREADS + tid;
         const bool is_a = trow < L_BM;
         const int64_t grow = is_a ? min(m0 + trow, M - 1) : min(n0 + trow - L_BM, N - 1);
-        cp[q] = (is_a ? a_codes : b_codes) + grow * kbytes;
-        sp[q] = (is_a ? a_scales : b_scales) + grow * kblocks;
+        cp[q] = (is_a ? a_codes : b_codes) + grow * kbytes + step_begin * (BK / 2);
+        sp[q] = (is_a ? a_scales : b_scales) + grow * kblocks + step_begin * (BK / kBlock);
         lds_row[q] = trow * L_STRIDE;
     }
     auto fetch = [&](RowRegs (&rr)[RPT], int k0) {               // K % 64 == 0: always a full step
@@ -310,7 +327,7 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_nvfp4_large_kernel(
         }
     };
 
-    const int steps = K / BK;
+    const int steps = step_end - step_begin;                     // >= 1: the host never asks for more splits than steps
     // r1: rows of step s+1, expanded during step s; r2: rows of step s+2, in flight during step s
     RowRegs r1[RPT], r2[RPT];
     fetch(r1, 0);
@@ -391,6 +408,10 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_nvfp4_large_kernel(
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] *= us;
 
+    if (SPLIT && split) {                                        // the low-rank term and the bias enter once
+        r = 0;
+        bias = nullptr;
+    }
     // ---- bf16 low-rank extension, 32 columns of T / U per step, staged in buffer 0
     for (int j0 = 0; j0 < r; j0 += 32) {
 #pragma unroll
@@ -420,6 +441,25 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_nvfp4_large_kernel(
         __syncthreads();
     }
 
+    if constexpr (SPLIT != 0) {
+        float* wt = ws + (size_t)logical_all * (L_BM * L_BN) + tid * 4;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int n = n0 + wn * WTN + j * 32 + 8 * g + 4 * (lane >> 5);
+                    float v[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        v[e] = acc[i][j][4 * g + e];
+                        if (bias) v[e] += bf16_lo(bias[min(n + e, N - 1)]);
+                    }
+                    *reinterpret_cast<float4*>(wt + ((i * TN + j) * 4 + g) * (NTHREADS * 4)) = make_float4(v[0], v[1], v[2], v[3]);
+                }
+        return;
+    }
     // ---- epilogue, bf16 output with N % 8 == 0: each wave transposes its tile through its own slice of the
     //      (now idle) LDS so that a store instruction writes 8 rows x 128 contiguous bytes instead of 32 rows x 16
     if constexpr (!OUT_F32 && WN_WAVES == 4) {
@@ -488,6 +528,104 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_nvfp4_large_kernel(
     }
 }
 
+// Sums the nsplit partial tiles of gemm_nvfp4_large_kernel<.., SPLIT = 1> (8 waves) and writes the output.
+// One wave per 32 x 64 piece (tile, wave of the GEMM, 32-row slab i): its lanes read what the same lanes of
+// the GEMM wrote, 1 KiB per instruction, and add the splits in ascending order.
+template <int OUT_F32>
+__global__ __launch_bounds__(64) void gemm_splitk_reduce_kernel(const float* __restrict__ ws, int nsplit, int M, int N,
+                                                                int tiles_m, int tiles_n, void* __restrict__ out)
+{
+    constexpr int TN = 2, WTN = 64, NTHREADS = 512, TILE = L_BM * L_BN;
+    __shared__ __attribute__((aligned(16))) uint16_t cw[32 * 72];
+    const int total = tiles_m * tiles_n;
+    const int tile = blockIdx.x >> 5, wave = (blockIdx.x >> 2) & 7, i = blockIdx.x & 3;
+    const int lane = threadIdx.x, tid = wave * 64 + lane;
+    const int wm = wave / 4, wn = wave % 4;
+    int m0, n0;
+    tile_origin(tile, tiles_m, tiles_n, m0, n0);
+    const int mbase = m0 + wm * 128 + i * 32, nbase = n0 + wn * WTN;
+    if (mbase >= M || nbase >= N) return;
+
+    float4 v[TN][4];
+    const float* src = ws + (size_t)tile * TILE + (size_t)(i * TN * 4) * (NTHREADS * 4) + tid * 4;
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) v[j][g] = *reinterpret_cast<const float4*>(src + (j * 4 + g) * (NTHREADS * 4));
+    for (int z = 1; z < nsplit; ++z) {
+        const float* sz = src + (size_t)z * total * TILE;
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const float4 p = *reinterpret_cast<const float4*>(sz + (j * 4 + g) * (NTHREADS * 4));
+                v[j][g].x += p.x; v[j][g].y += p.y; v[j][g].z += p.z; v[j][g].w += p.w;
+            }
+    }
+
+    if (!OUT_F32 && (N & 7) == 0) {
+        // 32 x 64 bf16 through LDS: a store instruction then writes 8 rows x 128 contiguous bytes
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                uint2 w;
+                w.x = bf16_bits(v[j][g].x) | (bf16_bits(v[j][g].y) << 16);
+                w.y = bf16_bits(v[j][g].z) | (bf16_bits(v[j][g].w) << 16);
+                *reinterpret_cast<uint2*>(cw + (lane & 31) * 72 + j * 32 + 8 * g + 4 * (lane >> 5)) = w;
+            }
+        __syncthreads();
+        const int rsub = lane >> 3, chunk = lane & 7;
+        const int n = nbase + chunk * 8;
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            const int ml = it * 8 + rsub;
+            const uint4 w = *reinterpret_cast<const uint4*>(cw + ml * 72 + chunk * 8);
+            if (mbase + ml < M && n < N) *reinterpret_cast<uint4*>((uint16_t*)out + (int64_t)(mbase + ml) * N + n) = w;
+        }
+        return;
+    }
+    const int m = mbase + (lane & 31);
+    if (m >= M) return;
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int n = nbase + j * 32 + 8 * g + 4 * (lane >> 5);
+            if (n >= N) continue;                                  // N % 4 == 0
+            if (OUT_F32) {
+                *reinterpret_cast<float4*>((float*)out + (int64_t)m * N + n) = v[j][g];
+            } else {
+                uint2 w;
+                w.x = bf16_bits(v[j][g].x) | (bf16_bits(v[j][g].y) << 16);
+                w.y = bf16_bits(v[j][g].z) | (bf16_bits(v[j][g].w) << 16);
+                *reinterpret_cast<uint2*>((uint16_t*)out + (int64_t)m * N + n) = w;
+            }
+        }
+}
+
+// Splits of K for a tiled GEMM that would leave more than half of the compute units without a tile:
+// as many as fill the device once, at least 8 K steps (512 elements) each, at most 16.  1 = do not split.
+static int split_factor(int64_t M, int64_t N, int64_t K)
+{
+    if (M < L_BM || N < L_BN || K % BK) return 1;
+    const int64_t tiles = ((M + L_BM - 1) / L_BM) * ((N + L_BN - 1) / L_BN);
+    const int cus = device_cus();
+    if (cus <= 0 || tiles * 2 > cus) return 1;
+    int64_t s = cus / tiles;
+    if (s > K / BK / 8) s = K / BK / 8;
+    if (s > 16) s = 16;
+    return s < 1 ? 1 : (int)s;
+}
+
+size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K)
+{
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    const int s = split_factor(M, N, K);
+    if (s <= 1) return 0;
+    return (size_t)s * (size_t)(((M + L_BM - 1) / L_BM) * ((N + L_BN - 1) / L_BN)) * L_BM * L_BN * sizeof(float);
+}
+
 // Dynamic LDS above 64 KiB has to be allowed per kernel function and per device: done once for each pair.
 static int allow_dynamic_lds(const void* fn, size_t bytes, bool (&done)[64])
 {
@@ -503,31 +641,44 @@ static int allow_dynamic_lds(const void* fn, size_t bytes, bool (&done)[64])
 template <int WN_WAVES>
 static int launch_large(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes,
                         const void* b_scales, const float* b_unit, int64_t M, int64_t N, int64_t K, const void* t,
-                        const void* u, int64_t r, const void* bias, void* out, int out_dtype, hipStream_t st)
+                        const void* u, int64_t r, const void* bias, void* out, int out_dtype, hipStream_t st,
+                        float* ws = nullptr, int nsplit = 1)
 {
-    static bool attr_set[2][64] = {};
+    static bool attr_set[3][64] = {};
     const size_t lds_bytes = 2 * (size_t)L_STAGE_HALVES * sizeof(uint16_t);
+    const bool split = WN_WAVES == 4 && ws && nsplit > 1;
     const int f32 = out_dtype == METIS_DTYPE_F32;
-    const void* fn = f32 ? (const void*)gemm_nvfp4_large_kernel<1, WN_WAVES> : (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES>;
+    const void* fn = split ? (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 0, WN_WAVES == 4>
+                   : f32   ? (const void*)gemm_nvfp4_large_kernel<1, WN_WAVES>
+                           : (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES>;
     const char* d = getenv("METIS_GEMM_DBG");                  // measurement switches, results are meaningless:
     const int v = d ? atoi(d) : 0;                             // 1 = no operand fetch/expansion, 7 = also no barriers
     if (v == 1 || v == 7) {
         fn = v == 1 ? (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 1> : (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 7>;
         if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess) return METIS_E_DEVICE;
-    } else if (const int rc = allow_dynamic_lds(fn, lds_bytes, attr_set[f32])) {
+    } else if (const int rc = allow_dynamic_lds(fn, lds_bytes, attr_set[split ? 2 : f32])) {
         return rc;
     }
     const int tiles_m = (int)((M + L_BM - 1) / L_BM), tiles_n = (int)((N + L_BN - 1) / L_BN);
     const int total = tiles_m * tiles_n;
-    const unsigned grid_x = (unsigned)(((total + 7) / 8) * 8);
+    if (!split) nsplit = 1;
+    const unsigned grid_x = (unsigned)(((total * nsplit + 7) / 8) * 8);
     const uint8_t *ac = (const uint8_t*)a_codes, *as = (const uint8_t*)a_scales, *bc = (const uint8_t*)b_codes,
                   *bs = (const uint8_t*)b_scales;
     const uint16_t *tp = (const uint16_t*)t, *up = (const uint16_t*)u, *bp = (const uint16_t*)bias;
     int Mi = (int)M, Ni = (int)N, Ki = (int)K, ri = (int)r, tmi = tiles_m, tni = tiles_n;
-    void* args[] = {&ac, &as, &a_unit, &bc, &bs, &b_unit, &Mi, &Ni, &Ki, &tp, &up, &ri, &bp, &out, &tmi, &tni};
+    void* args[] = {&ac, &as, &a_unit, &bc, &bs, &b_unit, &Mi, &Ni, &Ki, &tp, &up, &ri, &bp, &out, &tmi, &tni, &ws, &nsplit};
     if (hipLaunchKernel(fn, dim3(grid_x), dim3(128 * WN_WAVES), args, lds_bytes, st) != hipSuccess) {
         (void)hipGetLastError();
         return METIS_E_LAUNCH;
+    }
+    if (split) {
+        const dim3 rgrid((unsigned)total * 32u);
+        if (f32)
+            hipLaunchKernelGGL(gemm_splitk_reduce_kernel<1>, rgrid, dim3(64), 0, st, ws, nsplit, Mi, Ni, tmi, tni, out);
+        else
+            hipLaunchKernelGGL(gemm_splitk_reduce_kernel<0>, rgrid, dim3(64), 0, st, ws, nsplit, Mi, Ni, tmi, tni, out);
+        if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
     }
     return METIS_OK;
 }
@@ -945,7 +1096,7 @@ int gemm_expanded(const void* a_exp, const float* a_unit, const void* b_exp, con
 
 int gemm_nvfp4(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes, const void* b_scales,
                const float* b_unit, int64_t M, int64_t N, int64_t K, const void* t, const void* u, int64_t r,
-               const void* bias, void* out, int out_dtype, hipStream_t st)
+               const void* bias, void* out, int out_dtype, hipStream_t st, void* workspace, size_t workspace_bytes)
 {
     if (!a_codes || !a_scales || !a_unit || !b_codes || !b_scales || !b_unit || !out) return METIS_E_ARG;
     if (M < 0 || N < 0 || K < 0 || r < 0) return METIS_E_ARG;
@@ -961,7 +1112,13 @@ int gemm_nvfp4(const void* a_codes, const void* a_scales, const float* a_unit, c
     if (M >= 256 && N >= 256 && K % BK == 0 && !getenv("METIS_GEMM_SMALL")) {
         if (getenv("METIS_GEMM_W4"))
             return launch_large<2>(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st);
-        return launch_large<4>(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st);
+        int nsplit = 1;
+        if (workspace && !getenv("METIS_GEMM_NOSPLIT")) {
+            nsplit = split_factor(M, N, K);
+            if (nsplit > 1 && (((uintptr_t)workspace % 16) || workspace_bytes < gemm_workspace_bytes(M, N, K))) return METIS_E_WORKSPACE;
+        }
+        return launch_large<4>(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st,
+                               (float*)workspace, nsplit);
     }
     if (M < 256 && K % 64 == 0 && !getenv("METIS_GEMM_SMALL"))    // up to four 64-row passes over the weights beat a mostly empty 256-row tile
         return gemm_skinny(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st);

@@ -57,7 +57,10 @@ int rmsnorm_quantize(const void* x, const void* gamma, float eps, int64_t rows, 
                      void* codes, void* scales, float* unit, void* workspace, size_t workspace_bytes, hipStream_t st);
 int gemm_nvfp4(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes, const void* b_scales,
                const float* b_unit, int64_t M, int64_t N, int64_t K, const void* t, const void* u, int64_t r,
-               const void* bias, void* out, int out_dtype, hipStream_t st);
+               const void* bias, void* out, int out_dtype, hipStream_t st, void* workspace = nullptr,
+               size_t workspace_bytes = 0);
+// bytes of split-K scratch gemm_nvfp4 can use for this shape on the current device (0: it would not split)
+size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 int expand_f16(const void* codes, const void* scales, int64_t rows, int64_t cols, void* out, hipStream_t st);
 int gemm_expanded(const void* a_exp, const float* a_unit, const void* b_exp, const float* b_unit, int64_t M, int64_t N,

@@ -37,6 +37,10 @@ SIGNATURES = {
     "metis_linear_fwd_expanded": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _i32, _vp]),
     "metis_linear_dgrad": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i32, _vp]),
     "metis_linear_wgrad": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i32, _vp]),
+    "metis_linear_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "metis_linear_fwd_ws": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _i32, _vp, _sz, _vp]),
+    "metis_linear_dgrad_ws": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i32, _vp, _sz, _vp]),
+    "metis_linear_wgrad_ws": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i32, _vp, _sz, _vp]),
 }
 
 _lib = None

@@ -148,6 +148,17 @@ def rmsnorm_quantize(x: torch.Tensor, gamma: torch.Tensor, eps: float, mode: int
     return normed, PackedNVFP4(codes, scales, unit, rows, cols, mode)
 
 
+def _gemm_workspace(M: int, N: int, K: int, device: torch.device) -> torch.Tensor | None:
+    """Split-K scratch for an M x N output contracted over K, or None when the shape is not split.
+
+    Taken from torch's caching allocator per call (stream-ordered, so overlapping streams and captured
+    graphs each get their own) rather than cached here."""
+    if M < 256 or N < 256:
+        return None
+    need = load().metis_linear_workspace_bytes(M, N, K)
+    return torch.empty(need, dtype=torch.uint8, device=device) if need else None
+
+
 def linear_fwd(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None, u: torch.Tensor | None = None,
                bias: torch.Tensor | None = None, out_dtype: torch.dtype = torch.bfloat16,
                expanded: bool | None = None) -> torch.Tensor:
@@ -183,6 +194,13 @@ def linear_fwd(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None,
                                               tp, up, r, bp, out.data_ptr(), dt, _stream())
         check(rc, "metis_linear_fwd_expanded", (M, N, K))
         return out
+    ws = _gemm_workspace(M, N, K, dev)
+    if ws is not None:
+        rc = load().metis_linear_fwd_ws(a.codes.data_ptr(), a.scales.data_ptr(), a.unit.data_ptr(), b.codes.data_ptr(),
+                                        b.scales.data_ptr(), b.unit.data_ptr(), M, N, K, tp, up, r, bp, out.data_ptr(), dt,
+                                        ws.data_ptr(), ws.numel(), _stream())
+        check(rc, "metis_linear_fwd_ws", (M, N, K))
+        return out
     rc = load().metis_linear_fwd(a.codes.data_ptr(), a.scales.data_ptr(), a.unit.data_ptr(), b.codes.data_ptr(),
                                  b.scales.data_ptr(), b.unit.data_ptr(), M, N, K, tp, up, r, bp, out.data_ptr(), dt, _stream())
     check(rc, "metis_linear_fwd", (M, N, K))
@@ -195,9 +213,16 @@ def linear_dgrad(dy: PackedNVFP4, wt: PackedNVFP4, out_dtype: torch.dtype = torc
         raise ValueError(f"contraction mismatch: {dy.cols} vs {wt.cols}")
     L, N, K = dy.rows, dy.cols, wt.rows
     out = torch.empty(L, K, dtype=out_dtype, device=dy.codes.device)
+    dt = DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16
+    ws = _gemm_workspace(L, K, N, out.device)
+    if ws is not None:
+        rc = load().metis_linear_dgrad_ws(dy.codes.data_ptr(), dy.scales.data_ptr(), dy.unit.data_ptr(), wt.codes.data_ptr(),
+                                          wt.scales.data_ptr(), wt.unit.data_ptr(), L, N, K, out.data_ptr(), dt,
+                                          ws.data_ptr(), ws.numel(), _stream())
+        check(rc, "metis_linear_dgrad_ws", (L, N, K))
+        return out
     rc = load().metis_linear_dgrad(dy.codes.data_ptr(), dy.scales.data_ptr(), dy.unit.data_ptr(), wt.codes.data_ptr(),
-                                   wt.scales.data_ptr(), wt.unit.data_ptr(), L, N, K, out.data_ptr(),
-                                   DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16, _stream())
+                                   wt.scales.data_ptr(), wt.unit.data_ptr(), L, N, K, out.data_ptr(), dt, _stream())
     check(rc, "metis_linear_dgrad", (L, N, K))
     return out
 
@@ -208,8 +233,16 @@ def linear_wgrad(dyt: PackedNVFP4, xt: PackedNVFP4, out_dtype: torch.dtype = tor
         raise ValueError(f"contraction mismatch: {dyt.cols} vs {xt.cols}")
     N, L, K = dyt.rows, dyt.cols, xt.rows
     out = torch.empty(N, K, dtype=out_dtype, device=dyt.codes.device)
+    dt = DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16
+    ws = _gemm_workspace(N, K, L, out.device)
+    if ws is not None:
+        rc = load().metis_linear_wgrad_ws(dyt.codes.data_ptr(), dyt.scales.data_ptr(), dyt.unit.data_ptr(),
+                                          xt.codes.data_ptr(), xt.scales.data_ptr(), xt.unit.data_ptr(), L, N, K,
+                                          out.data_ptr(), dt, ws.data_ptr(), ws.numel(), _stream())
+        check(rc, "metis_linear_wgrad_ws", (L, N, K))
+        return out
     rc = load().metis_linear_wgrad(dyt.codes.data_ptr(), dyt.scales.data_ptr(), dyt.unit.data_ptr(),
                                    xt.codes.data_ptr(), xt.scales.data_ptr(), xt.unit.data_ptr(), L, N, K,
-                                   out.data_ptr(), DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16, _stream())
+                                   out.data_ptr(), dt, _stream())
     check(rc, "metis_linear_wgrad", (L, N, K))
     return out

@@ -203,6 +203,38 @@ int metis_linear_wgrad(const void *dyt_codes, const void *dyt_scales, const floa
                        const void *xt_codes, const void *xt_scales, const float *xt_unit, int64_t L,
                        int64_t N, int64_t K, void *grad_weight, int out_dtype, void *stream);
 
+/*
+ * The three contractions above with caller-supplied scratch for splitting K.  A shape whose 256 x 256
+ * output tiles number at most half the compute units of the device (a few hundred to a few thousand
+ * rows against a long contraction: short prefill batches, the down projection, dgrad of a narrow layer)
+ * leaves most of the device idle in the plain entry points; here up to 16 workgroups share a tile, each
+ * contracts its own range of K into a binary32 partial tile in the workspace, and a second kernel adds
+ * the partials in ascending order of K and writes the output.  The order of the binary32 additions
+ * differs from the unsplit kernels'; the exact products and the result's tolerance do not.
+ *
+ * metis_linear_workspace_bytes(M, N, K) is what the call needs for an M x N output contracted over K on
+ * the CURRENT device (dgrad: L, K, N; wgrad: N, K, L); 0 means the shape is not split and workspace may
+ * be NULL.  A workspace that is too small or not 16-byte aligned is METIS_E_WORKSPACE; workspace == NULL
+ * always selects the unsplit kernels.  The workspace needs no initialisation and carries nothing
+ * between calls; calls that overlap in time need separate workspaces.
+ * No counterpart in the reference, whose matmuls go to the vendor library
+ * (src/Metis/Metis/bitlinear.py:435-438,502-510).
+ */
+size_t metis_linear_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int metis_linear_fwd_ws(const void *a_codes, const void *a_scales, const float *a_unit,
+                        const void *b_codes, const void *b_scales, const float *b_unit, int64_t M,
+                        int64_t N, int64_t K, const void *t, const void *u, int64_t r,
+                        const void *bias, void *out, int out_dtype, void *workspace,
+                        size_t workspace_bytes, void *stream);
+int metis_linear_dgrad_ws(const void *dy_codes, const void *dy_scales, const float *dy_unit,
+                          const void *wt_codes, const void *wt_scales, const float *wt_unit,
+                          int64_t L, int64_t N, int64_t K, void *grad_input, int out_dtype,
+                          void *workspace, size_t workspace_bytes, void *stream);
+int metis_linear_wgrad_ws(const void *dyt_codes, const void *dyt_scales, const float *dyt_unit,
+                          const void *xt_codes, const void *xt_scales, const float *xt_unit,
+                          int64_t L, int64_t N, int64_t K, void *grad_weight, int out_dtype,
+                          void *workspace, size_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

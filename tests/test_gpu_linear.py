@@ -104,9 +104,11 @@ def test_dgrad_and_wgrad():
     assert rel_fro(gw.cpu(), dy.double().T @ x.double()) < 0.25
 
 
-def test_expanded_path_is_bit_identical_to_packed_path():
-    """metis_linear_fwd_expanded on exact f16 expansions == metis_linear_fwd on packed operands."""
+def test_expanded_path_is_bit_identical_to_packed_path(monkeypatch):
+    """metis_linear_fwd_expanded on exact f16 expansions == metis_linear_fwd on packed operands
+    (with K unsplit: splitting changes the order of the binary32 additions)."""
     from metis_hip import ops
+    monkeypatch.setenv("METIS_GEMM_NOSPLIT", "1")
     M, N, K, r = 512, 768, 1024, 64
     x = synthetic_activation(40, M, K)
     w = _weights(41, N, K)
@@ -148,6 +150,74 @@ def test_decode_shapes_with_lowrank_and_bias(M, N, K, r):
     torch.cuda.synchronize()
     assert rel_fro(got32.cpu(), want.cpu()) <= 1e-5
     assert rel_fro(got.cpu(), want.cpu().bfloat16()) <= TOL
+
+
+@pytest.mark.parametrize("M,N,K,r", [(256, 512, 4096, 64), (300, 260, 4096, 0), (512, 3584, 2048, 32), (1024, 1536, 4160, 64),
+                                     (260, 776, 18944, 0)])
+def test_split_k_shapes(M, N, K, r, monkeypatch):
+    """Few output tiles and a long contraction: up to 16 workgroups share a tile, partial tiles meet in a
+    caller-supplied workspace.  Covers ragged M and N (N % 8 != 0 takes the plain stores), step counts that
+    do not divide by the number of splits, the low-rank term and the bias (which must enter exactly once)."""
+    from metis_hip import _lib, ops
+    assert _lib.load().metis_linear_workspace_bytes(M, N, K) > 0
+    g = torch.Generator().manual_seed(91)
+    x = synthetic_activation(50 + M, M, K).cuda()
+    w = _weights(51 + N, N, K).cuda()
+    t = u = None
+    if r:
+        t = torch.randn(M, r, generator=g).bfloat16().cuda()
+        u = torch.randn(N, r, generator=g).bfloat16().cuda()
+    bias = (torch.randn(N, generator=g) * 0.1).bfloat16().cuda()
+    px, pw = ops.quantize(x), ops.quantize(w)
+    got = ops.linear_fwd(px, pw, t=t, u=u, bias=bias)
+    got32 = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, out_dtype=torch.float32)
+    want = ops.dequantize(px, torch.float32).double() @ ops.dequantize(pw, torch.float32).double().T
+    if r:
+        want = want + t.double() @ u.double().T
+    want = want + bias.double()
+    torch.cuda.synchronize()
+    assert rel_fro(got32.cpu(), want.cpu()) <= 1e-5
+    assert rel_fro(got.cpu(), want.cpu().bfloat16()) <= TOL
+    # and against the unsplit kernel on the same operands
+    monkeypatch.setenv("METIS_GEMM_NOSPLIT", "1")
+    whole32 = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, out_dtype=torch.float32)
+    torch.cuda.synchronize()
+    assert rel_fro(got32.cpu(), whole32.cpu()) <= 1e-5
+
+
+def test_split_k_dgrad_wgrad_and_workspace_errors():
+    from metis_hip import _lib, ops
+    L, N, K = 512, 2048, 512
+    lib = _lib.load()
+    assert lib.metis_linear_workspace_bytes(L, K, N) > 0       # dgrad: L x K contracted over N
+    g = torch.Generator().manual_seed(92)
+    dy = (torch.randn(L, N, generator=g) * 1e-3).bfloat16().cuda()
+    w = _weights(93, N, K).cuda()
+    p_dy, p_wt = ops.quantize(dy, sr=True, seed=5), ops.quantize(w, col=True)
+    gx = ops.linear_dgrad(p_dy, p_wt, out_dtype=torch.float32)
+    want = ops.dequantize(p_dy, torch.float32).double() @ ops.dequantize(p_wt, torch.float32).double().T
+    assert rel_fro(gx.cpu(), want.cpu()) <= 1e-5
+    # wgrad: N x K contracted over L
+    L2, N2, K2 = 4096, 256, 512
+    assert lib.metis_linear_workspace_bytes(N2, K2, L2) > 0
+    dy2 = (torch.randn(L2, N2, generator=g) * 1e-3).bfloat16().cuda()
+    x2 = synthetic_activation(94, L2, K2).cuda()
+    p_dyt, p_xt = ops.quantize(dy2, col=True, sr=True, seed=6), ops.quantize(x2, col=True, sr=True, seed=7)
+    gw = ops.linear_wgrad(p_dyt, p_xt)
+    want = ops.dequantize(p_dyt, torch.float32).double() @ ops.dequantize(p_xt, torch.float32).double().T
+    assert gw.dtype == torch.float32 and rel_fro(gw.cpu(), want.cpu()) <= 1e-5
+    # a workspace that is too small or misaligned is refused; none at all selects the unsplit kernel
+    need = lib.metis_linear_workspace_bytes(L, K, N)
+    ws = torch.empty(need + 16, dtype=torch.uint8, device="cuda")
+    out = torch.empty(L, K, dtype=torch.float32, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    args = (p_dy.codes.data_ptr(), p_dy.scales.data_ptr(), p_dy.unit.data_ptr(), p_wt.codes.data_ptr(),
+            p_wt.scales.data_ptr(), p_wt.unit.data_ptr(), L, N, K, out.data_ptr(), _lib.DTYPE_F32)
+    assert lib.metis_linear_dgrad_ws(*args, ws.data_ptr(), need - 1, st) == _lib.E_WORKSPACE
+    assert lib.metis_linear_dgrad_ws(*args, ws.data_ptr() + 4, need, st) == _lib.E_WORKSPACE
+    assert lib.metis_linear_dgrad_ws(*args, None, 0, st) == 0
+    torch.cuda.synchronize()
+    assert rel_fro(out.cpu(), gx.cpu()) <= 1e-5
 
 
 def test_output_offsets_beyond_32_bits():
