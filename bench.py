@@ -297,6 +297,31 @@ def main():
         except Exception as exc:  # an optional leg must not cost the headline line
             qat = {"workload": "config 4 projection", "error": f"{type(exc).__name__}: {exc}"[:300]}
 
+    # ------------------------------------------------------------------ a tile-starved shape: 1024-token prefill
+    # through the Qwen2.5-7B down projection (56 output tiles on 256 CUs; K split through a workspace)
+    prefill = None
+    if not args.no_decode:
+        try:
+            gp = torch.Generator().manual_seed(1005)
+            xp = ops.quantize(outlier_activation(torch, 1006, 1024, 18944, dev))
+            wp = ops.quantize((torch.randn(3584, 18944, generator=gp) * 0.02).bfloat16().to(dev))
+            tp_ = torch.randn(1024, 64, generator=gp).bfloat16().to(dev)
+            up_ = torch.randn(3584, 64, generator=gp).bfloat16().to(dev)
+
+            def prefill_step(ev):
+                if ev is not None:
+                    ev[0].record()
+                ops.linear_fwd(xp, wp, t=tp_, u=up_)
+                if ev is not None:
+                    ev[1].record()
+            _, pf_ms = time_region(torch, prefill_step, 20, 5)
+            prefill = {"workload": "1024-token prefill, Qwen2.5-7B down projection 18944->3584, r=64, packed operands "
+                                   "(split-K GEMM + reduce)",
+                       "us_per_call": round(pf_ms * 1e3, 1),
+                       "tflops": round(2.0 * 1024 * 3584 * (18944 + 64) / (pf_ms * 1e-3) / 1e12, 1)}
+        except Exception as exc:  # an optional leg must not cost the headline line
+            prefill = {"workload": "short prefill projection", "error": f"{type(exc).__name__}: {exc}"[:300]}
+
     line = {
         "metric": "Metis NVFP4 linear TFLOP/s at 8192x4096x14336 (rank 64)",
         "value": round(value, 2),
@@ -333,6 +358,8 @@ def main():
         line["decode_layer"] = dec
     if qat is not None:
         line["qat_projection"] = qat
+    if prefill is not None:
+        line["short_prefill_projection"] = prefill
     if not args.no_cpu_baseline:
         torch_threads = torch.get_num_threads()
         cpu_tflops, cpu_dt, cpu_reps = cpu_baseline_linear(torch, x, v, s, u, res)
