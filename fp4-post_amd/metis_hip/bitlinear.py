@@ -292,7 +292,9 @@ class LinearLowbitFunction(torch.autograd.Function):
                     pw_col = ctx.pw.transposed = F.q_forward_weight.pack(ctx.weight_ref, col=True, arith=cd)
                 gx_dtype = input_.dtype if input_.dtype in (torch.float32, torch.bfloat16) else torch.float32
                 gx = ops.linear_dgrad(p_dy, pw_col, out_dtype=gx_dtype)
-                gw = ops.linear_wgrad(qg.pack(dy2, col=True, arith=cd), qi.pack(x2, col=True, arith=cd))
+                # autograd rounds the gradient to the parameter's dtype anyway: let the GEMM epilogue do that rounding
+                gw_dtype = torch.bfloat16 if ctx.weight_ref.dtype == torch.bfloat16 else torch.float32
+                gw = ops.linear_wgrad(qg.pack(dy2, col=True, arith=cd), qi.pack(x2, col=True, arith=cd), out_dtype=gw_dtype)
                 return gx.reshape(*ctx.lead, gx.shape[-1]), gw, grad_bias, None, None
             grad_output = grad_output.to(F.compute_dtype)
             dy2 = _flat2d(grad_output)
@@ -424,7 +426,9 @@ class _MetisFusedFunction(torch.autograd.Function):
             if p_res_col is None:
                 p_res_col = ctx.p_res.transposed = F.q_forward_weight.pack(res, col=True, arith=ar)
             gx = gx + ops.linear_dgrad(qg.pack(dy2, arith=ar), p_res_col, out_dtype=cd)
-            g_res = ops.linear_wgrad(qg.pack(dy2, col=True, arith=ar), qi.pack(x2, col=True, arith=ar))
+            # autograd rounds to the parameter's dtype anyway: let the GEMM epilogue do that rounding
+            g_res = ops.linear_wgrad(qg.pack(dy2, col=True, arith=ar), qi.pack(x2, col=True, arith=ar),
+                                     out_dtype=torch.bfloat16 if res.dtype == torch.bfloat16 else torch.float32)
         else:
             dyq = F._quantize_wgrad_operand(dy2.to(F.compute_dtype), qg)
             xq = F.q_forward_input.quantize_dequantize(x2.to(F.compute_dtype))
@@ -433,7 +437,7 @@ class _MetisFusedFunction(torch.autograd.Function):
             g_res = torch.matmul(dyq.T, xq).to(torch.float32)
         g_b = dy2.float().sum(dim=0) if ctx.has_bias else None
         return (gx.reshape(x.shape).to(x.dtype), g_v.to(v.dtype), g_s.to(s.dtype), g_u.to(u.dtype),
-                g_res.to(torch.float32), g_b, None, None)
+                g_res, g_b, None, None)
 
 
 class BitLinear(nn.Module):
