@@ -11,7 +11,7 @@ namespace metis {
 // Caller-supplied scratch, carved as:
 //   [0, 16 KiB)        one partial maximum (uint32 bit pattern) per workgroup of phase 1
 //   [16 KiB, +65 KiB)  grid-wide reduction words of the single-launch quantizer (zero when idle)
-//   [81 KiB, ..)       one bf16 block maximum per block of 16
+//   [81 KiB, ..)       one block maximum per block of 16: bf16 for bf16 input, binary32 for binary32 input
 struct Workspace {
     uint32_t* gmax;
     uint32_t* sync;
@@ -23,7 +23,7 @@ constexpr size_t kWsSyncBytes = 260 * 256;     // 1 KiB header + 4096 member wor
 inline size_t workspace_bytes(int64_t rows, int64_t cols)
 {
     const size_t nblocks = (size_t)((rows * cols + 15) / 16);
-    return kWsGmaxBytes + kWsSyncBytes + ((nblocks * 2 + 255) / 256) * 256;
+    return kWsGmaxBytes + kWsSyncBytes + ((nblocks * 4 + 255) / 256) * 256;
 }
 
 inline int carve_workspace(void* p, size_t bytes, int64_t rows, int64_t cols, Workspace* ws)

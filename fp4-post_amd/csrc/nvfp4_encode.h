@@ -133,7 +133,8 @@ __device__ __forceinline__ void sr_convert_pair(uint32_t& w, float q0, float q1,
 // word one bit apart).  One Philox4x32-10 draw serves a block: counter = offset + output block,
 // pair p (elements 2p, 2p+1) takes word p % 4, rotated by 16 bits for p >= 4 (the converter only
 // looks at the top 13 bits).  Scale bytes and unit do not depend on the rounding mode.
-template <int MODE>
+// IEEE_DIV: the input need not be bf16-valued, so the quotient comes from a correctly rounded division.
+template <int MODE, bool IEEE_DIV = false>
 __device__ __forceinline__ uint2 encode_sr_hardware(const float (&v)[kBlock], float s, uint64_t seed, uint64_t offset,
                                                     int64_t ob)
 {
@@ -147,7 +148,7 @@ __device__ __forceinline__ uint2 encode_sr_hardware(const float (&v)[kBlock], fl
     for (int j = 0; j < kBlock; j += 2) {
         const int p = j >> 1;
         const uint32_t bits = p < 4 ? word[p] : __builtin_amdgcn_alignbit(word[p & 3], word[p & 3], 16);
-        float q0 = div3(v[j], d, rd_), q1 = div3(v[j + 1], d, rd_);
+        float q0 = IEEE_DIV ? v[j] / d : div3(v[j], d, rd_), q1 = IEEE_DIV ? v[j + 1] / d : div3(v[j + 1], d, rd_);
         if (MODE) {
             const uint32_t qq = rb_pair(q0, q1);
             q0 = bf16_lo(qq);

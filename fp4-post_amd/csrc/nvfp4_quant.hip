@@ -14,6 +14,7 @@
 #include "nvfp4_encode.h"
 #include <stdio.h>
 #include <stdlib.h>
+#include <type_traits>
 
 namespace metis {
 
@@ -21,15 +22,23 @@ namespace metis {
 // Phase 1, row-blocked: codes + parked block maxima + per-workgroup maximum.  One block of 16 per
 // thread per iteration: thread i <-> block i (32 contiguous bytes, two 16-byte loads).
 // ---------------------------------------------------------------------------------------------
-template <int MODE, bool SR>
+// F32IN (binary32 arithmetic only): x holds binary32 values that need not be bf16 values.  The short cuts
+// of the bf16 path (div6, div3, the guarded hardware conversion) are proven for bf16 inputs only, so these
+// instantiations use IEEE divisions and the literal encoder, and park the block maxima as binary32.
+__device__ __forceinline__ float block_scalar_ieee(float amax) { return amax / 6.0f + 1e-9f; }
+
+template <int MODE, bool SR, bool F32IN = false>
 __global__ __launch_bounds__(256) void quant_codes_kernel(
-    const uint16_t* __restrict__ x, uint32_t rows, uint32_t cols, int64_t ld, const void* __restrict__ noise,
-    uint64_t seed, uint64_t offset, uint2* __restrict__ codes, uint16_t* __restrict__ ws_amax,
+    const void* __restrict__ xv, uint32_t rows, uint32_t cols, int64_t ld, const void* __restrict__ noise,
+    uint64_t seed, uint64_t offset, uint2* __restrict__ codes, void* __restrict__ ws_amax_v,
     uint32_t* __restrict__ ws_gmax, uint32_t nblocks)
 {
+    static_assert(!F32IN || MODE == 0, "binary32 input implies binary32 arithmetic");
+    const uint16_t* __restrict__ x = static_cast<const uint16_t*>(xv);
+    uint16_t* __restrict__ ws_amax = static_cast<uint16_t*>(ws_amax_v);
     float gmax = 0.0f;
     const uint32_t nbpr = cols / kBlock;      // row layout: blocks per row
-    if constexpr (!SR) {
+    if constexpr (!SR && !F32IN) {
         // Round-to-nearest rows: software-pipelined, the next block's 32 bytes are in flight while the
         // current block is encoded.
         const uint32_t step = gridDim.x * 256u;
@@ -61,8 +70,17 @@ __global__ __launch_bounds__(256) void quant_codes_kernel(
     for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < nblocks; i += gridDim.x * 256u) {
         float v[kBlock], u[kBlock] = {};
         const uint32_t row = i / nbpr, cb = i - row * nbpr;
-        const uint4* p = reinterpret_cast<const uint4*>(x + (int64_t)row * ld + (int64_t)cb * kBlock);
-        unpack16(p[0], p[1], v);
+        if constexpr (F32IN) {
+            const float4* p = reinterpret_cast<const float4*>(static_cast<const float*>(xv) + (int64_t)row * ld + (int64_t)cb * kBlock);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const float4 f = p[c];
+                v[4 * c] = f.x; v[4 * c + 1] = f.y; v[4 * c + 2] = f.z; v[4 * c + 3] = f.w;
+            }
+        } else {
+            const uint4* p = reinterpret_cast<const uint4*>(x + (int64_t)row * ld + (int64_t)cb * kBlock);
+            unpack16(p[0], p[1], v);
+        }
         if (SR && noise) {
 #pragma unroll
             for (int j = 0; j < kBlock; ++j) {
@@ -72,10 +90,16 @@ __global__ __launch_bounds__(256) void quant_codes_kernel(
         }
         const float am = block_amax(v);
         gmax = fmaxf(gmax, am);
-        ws_amax[i] = (uint16_t)(__float_as_uint(am) >> 16);          // am is a bf16 value
-        // caller-supplied noise: the reference's literal sequence; own stream: hardware stochastic rounding
-        codes[i] = (SR && !noise) ? encode_sr_hardware<MODE>(v, block_scalar<MODE>(am), seed, offset, i)
-                                  : encode_block<MODE, SR>(v, block_scalar<MODE>(am), u);
+        if constexpr (F32IN) {
+            static_cast<float*>(ws_amax_v)[i] = am;
+            const float sc = block_scalar_ieee(am);
+            codes[i] = (SR && !noise) ? encode_sr_hardware<0, true>(v, sc, seed, offset, i) : encode_literal<0, SR>(v, sc, u);
+        } else {
+            ws_amax[i] = (uint16_t)(__float_as_uint(am) >> 16);      // am is a bf16 value
+            // caller-supplied noise: the reference's literal sequence; own stream: hardware stochastic rounding
+            codes[i] = (SR && !noise) ? encode_sr_hardware<MODE>(v, block_scalar<MODE>(am), seed, offset, i)
+                                      : encode_block<MODE, SR>(v, block_scalar<MODE>(am), u);
+        }
     }
     publish_group_max(gmax, ws_gmax);
 }
@@ -89,14 +113,18 @@ __global__ __launch_bounds__(256) void quant_codes_kernel(
 // column owns in the tile, instead of one scattered 8-byte and 2-byte store per lane.
 // ---------------------------------------------------------------------------------------------
 constexpr int kColTileBlocks = 16, kColTileCols = 64;
-template <int MODE, bool SR>
+template <int MODE, bool SR, bool F32IN = false>
 __global__ __launch_bounds__(256) void quant_codes_col_kernel(
-    const uint16_t* __restrict__ x, uint32_t rows, uint32_t cols, int64_t ld, const void* __restrict__ noise,
-    uint64_t seed, uint64_t offset, uint2* __restrict__ codes, uint16_t* __restrict__ ws_amax,
+    const void* __restrict__ xv, uint32_t rows, uint32_t cols, int64_t ld, const void* __restrict__ noise,
+    uint64_t seed, uint64_t offset, uint2* __restrict__ codes, void* __restrict__ ws_amax_v,
     uint32_t* __restrict__ ws_gmax, uint32_t tiles_c, uint32_t tiles_total)
 {
+    static_assert(!F32IN || MODE == 0, "binary32 input implies binary32 arithmetic");
+    using amax_t = typename std::conditional<F32IN, float, uint16_t>::type;   // parked block maximum
+    const uint16_t* __restrict__ x = static_cast<const uint16_t*>(xv);
+    amax_t* __restrict__ ws_amax = static_cast<amax_t*>(ws_amax_v);
     __shared__ uint2 s_codes[kColTileCols][kColTileBlocks + 1];
-    __shared__ uint16_t s_amax[kColTileCols][kColTileBlocks + 2];
+    __shared__ amax_t s_amax[kColTileCols][kColTileBlocks + 2];
     const uint32_t nbc = rows / kBlock;                       // blocks per column
     const uint32_t cl = threadIdx.x & 63u, g = threadIdx.x >> 6;
     float gmax = 0.0f;
@@ -111,7 +139,9 @@ __global__ __launch_bounds__(256) void quant_codes_col_kernel(
             if (c < cols && b < nbc) {
                 float v[kBlock], u[kBlock] = {};
 #pragma unroll
-                for (int j = 0; j < kBlock; ++j) v[j] = bf16_lo(x[(int64_t)(b * kBlock + j) * ld + c]);
+                for (int j = 0; j < kBlock; ++j)
+                    v[j] = F32IN ? static_cast<const float*>(xv)[(int64_t)(b * kBlock + j) * ld + c]
+                                 : bf16_lo(x[(int64_t)(b * kBlock + j) * ld + c]);
                 if (SR && noise) {
 #pragma unroll
                     for (int j = 0; j < kBlock; ++j) {
@@ -121,11 +151,18 @@ __global__ __launch_bounds__(256) void quant_codes_col_kernel(
                 }
                 am = block_amax(v);
                 gmax = fmaxf(gmax, am);
-                packed = (SR && !noise) ? encode_sr_hardware<MODE>(v, block_scalar<MODE>(am), seed, offset, (int64_t)c * nbc + b)
-                                        : encode_block<MODE, SR>(v, block_scalar<MODE>(am), u);
+                if constexpr (F32IN) {
+                    const float sc = block_scalar_ieee(am);
+                    packed = (SR && !noise) ? encode_sr_hardware<0, true>(v, sc, seed, offset, (int64_t)c * nbc + b)
+                                            : encode_literal<0, SR>(v, sc, u);
+                } else {
+                    packed = (SR && !noise) ? encode_sr_hardware<MODE>(v, block_scalar<MODE>(am), seed, offset, (int64_t)c * nbc + b)
+                                            : encode_block<MODE, SR>(v, block_scalar<MODE>(am), u);
+                }
             }
             s_codes[cl][bl] = packed;
-            s_amax[cl][bl] = (uint16_t)(__float_as_uint(am) >> 16);
+            if constexpr (F32IN) s_amax[cl][bl] = am;
+            else s_amax[cl][bl] = (uint16_t)(__float_as_uint(am) >> 16);
         }
         __syncthreads();
         {   // column t / 4, blocks 4 (t % 4) .. +3 of the tile: 32 contiguous bytes of codes, 8 of maxima
@@ -197,6 +234,32 @@ __global__ __launch_bounds__(256) void quant_scales_kernel(const uint16_t* __res
         const float s = block_scalar<MODE>(__uint_as_float((uint32_t)ws_amax[k] << 16));
         scales[k] = (uint8_t)e4m3_byte(rd<MODE>(s / unit));
     }
+}
+
+// Phase 2 for parked binary32 maxima (binary32 input): IEEE divisions, four blocks per thread.
+__global__ __launch_bounds__(256) void quant_scales_f32_kernel(const float* __restrict__ ws_amax,
+                                                               const uint32_t* __restrict__ ws_gmax, uint32_t ngroups,
+                                                               uint8_t* __restrict__ scales, float* __restrict__ unit_out,
+                                                               uint32_t nblocks)
+{
+    __shared__ float smax[4];
+    float m = 0.0f;
+    for (uint32_t g = threadIdx.x; g < ngroups; g += 256u) m = fmaxf(m, __uint_as_float(ws_gmax[g]));
+    m = wave_max(m);
+    if ((threadIdx.x & 63) == 0) smax[threadIdx.x >> 6] = m;
+    __syncthreads();
+    const float amax = fmaxf(fmaxf(smax[0], smax[1]), fmaxf(smax[2], smax[3]));
+    const float unit = block_scalar_ieee(amax) / 448.0f;      // the scalar map is monotone: max of scalars = scalar of max
+    if (blockIdx.x == 0 && threadIdx.x == 0) *unit_out = unit;
+    const uint32_t nquads = nblocks / 4u, step = gridDim.x * 256u;
+    for (uint32_t q = blockIdx.x * 256u + threadIdx.x; q < nquads; q += step) {
+        const float4 a = reinterpret_cast<const float4*>(ws_amax)[q];
+        const int w = __builtin_amdgcn_cvt_pk_fp8_f32(block_scalar_ieee(a.x) / unit, block_scalar_ieee(a.y) / unit, 0, false);
+        reinterpret_cast<uint32_t*>(scales)[q] =
+            (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(block_scalar_ieee(a.z) / unit, block_scalar_ieee(a.w) / unit, w, true);
+    }
+    for (uint32_t k = nquads * 4u + blockIdx.x * 256u + threadIdx.x; k < nblocks; k += step)
+        scales[k] = (uint8_t)e4m3_byte(block_scalar_ieee(ws_amax[k]) / unit);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -392,7 +455,10 @@ int launch_scales(int mode, const Workspace& ws, uint32_t ngroups, void* scales,
                   hipStream_t st)
 {
     const int g2 = grid_for((nblocks + 7) / 8);
-    if (mode == 0)
+    if (mode == METIS_MODE_P32_F32)
+        hipLaunchKernelGGL(quant_scales_f32_kernel, dim3(g2), dim3(256), 0, st, (const float*)ws.amax, ws.gmax, ngroups,
+                           (uint8_t*)scales, unit, nblocks);
+    else if (mode == 0)
         hipLaunchKernelGGL((quant_scales_kernel<0>), dim3(g2), dim3(256), 0, st, ws.amax, ws.gmax, ngroups,
                            (uint8_t*)scales, unit, nblocks);
     else
@@ -440,7 +506,7 @@ static int launch_fused(const void* x, void* codes, void* scales, float* unit, c
     return rc;
 }
 
-template <int MODE, bool SR, bool COL>
+template <int MODE, bool SR, bool COL, bool F32IN = false>
 static int launch_quant(const void* x, int64_t rows, int64_t cols, int64_t ld, const void* noise, uint64_t seed,
                         uint64_t offset, void* codes, void* scales, float* unit, const Workspace& ws, hipStream_t st)
 {
@@ -453,15 +519,15 @@ static int launch_quant(const void* x, int64_t rows, int64_t cols, int64_t ld, c
         const int64_t cap = (int64_t)device_cus() * 8;
         if (g > cap) g = cap;
         if (g > kMaxGroups) g = kMaxGroups;
-        hipLaunchKernelGGL((quant_codes_col_kernel<MODE, SR>), dim3((unsigned)g), dim3(256), 0, st, (const uint16_t*)x,
-                           (uint32_t)rows, (uint32_t)cols, ld, noise, seed, offset, (uint2*)codes, ws.amax, ws.gmax, tiles_c,
+        hipLaunchKernelGGL((quant_codes_col_kernel<MODE, SR, F32IN>), dim3((unsigned)g), dim3(256), 0, st, x,
+                           (uint32_t)rows, (uint32_t)cols, ld, noise, seed, offset, (uint2*)codes, (void*)ws.amax, ws.gmax, tiles_c,
                            (uint32_t)tiles);
-        return launch_scales(MODE, ws, (uint32_t)g, scales, unit, nblocks, st);
+        return launch_scales(F32IN ? METIS_MODE_P32_F32 : MODE, ws, (uint32_t)g, scales, unit, nblocks, st);
     } else {
         const int g1 = grid_for(nblocks);
-        hipLaunchKernelGGL((quant_codes_kernel<MODE, SR>), dim3(g1), dim3(256), 0, st, (const uint16_t*)x, (uint32_t)rows,
-                           (uint32_t)cols, ld, noise, seed, offset, (uint2*)codes, ws.amax, ws.gmax, nblocks);
-        return launch_scales(MODE, ws, (uint32_t)g1, scales, unit, nblocks, st);
+        hipLaunchKernelGGL((quant_codes_kernel<MODE, SR, F32IN>), dim3(g1), dim3(256), 0, st, x, (uint32_t)rows,
+                           (uint32_t)cols, ld, noise, seed, offset, (uint2*)codes, (void*)ws.amax, ws.gmax, nblocks);
+        return launch_scales(F32IN ? METIS_MODE_P32_F32 : MODE, ws, (uint32_t)g1, scales, unit, nblocks, st);
     }
 }
 
@@ -470,23 +536,31 @@ int quantize(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, bo
              size_t workspace_bytes, hipStream_t st)
 {
     if (rows < 0 || cols < 0 || ld < cols) return METIS_E_ARG;
-    if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) return METIS_E_ARG;
+    if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16 && mode != METIS_MODE_P32_F32) return METIS_E_ARG;
+    const bool f32in = mode == METIS_MODE_P32_F32;
     if ((col ? rows : cols) % kBlock) return METIS_E_SHAPE;
     if (rows == 0 || cols == 0) return METIS_OK;              // nothing to read or write, unit untouched
     if (!x || !codes || !scales || !unit) return METIS_E_ARG;
     if (rows * cols / kBlock >= (int64_t)1 << 31) return METIS_E_ARG;
-    if (!col && ((ld % 8) || ((uintptr_t)x % 16))) return METIS_E_ARG;     // 16-byte vector loads
+    if (!col && ((ld % (f32in ? 4 : 8)) || ((uintptr_t)x % 16))) return METIS_E_ARG;     // 16-byte vector loads
+    if (col && f32in && ((uintptr_t)x % 4)) return METIS_E_ARG;
     if (((uintptr_t)codes % 8) || ((uintptr_t)scales % 8)) return METIS_E_ARG;
     Workspace ws;
     int rc = carve_workspace(workspace, workspace_bytes, rows, cols, &ws);
     if (rc != METIS_OK) return rc;
-    if (!sr && !col && ld == cols && getenv("METIS_FUSED_QUANT")) {   // opt-in single-launch path; falls through when it does not fit
+    if (!sr && !col && !f32in && ld == cols && getenv("METIS_FUSED_QUANT")) {   // opt-in single-launch path; falls through when it does not fit
         const uint32_t nblocks = (uint32_t)(rows * cols / kBlock);
         rc = mode == 0 ? launch_fused<0>(x, codes, scales, unit, ws, nblocks, st)
                        : launch_fused<1>(x, codes, scales, unit, ws, nblocks, st);
         if (rc != 1) return rc;
     }
 #define METIS_Q(M, S, C) return launch_quant<M, S, C>(x, rows, cols, ld, noise, seed, offset, codes, scales, unit, ws, st)
+#define METIS_QF(S, C) return launch_quant<0, S, C, true>(x, rows, cols, ld, noise, seed, offset, codes, scales, unit, ws, st)
+    if (f32in) {
+        if (!sr) { if (!col) METIS_QF(false, false); else METIS_QF(false, true); }
+        else { if (!col) METIS_QF(true, false); else METIS_QF(true, true); }
+    }
+#undef METIS_QF
     if (mode == 0) {
         if (!sr) { if (!col) METIS_Q(0, false, false); else METIS_Q(0, false, true); }
         else { if (!col) METIS_Q(0, true, false); else METIS_Q(0, true, true); }
@@ -501,6 +575,7 @@ int dequantize(const void* codes, const void* scales, const float* unit, int64_t
                int out_dtype, hipStream_t st)
 {
     if (rows < 0 || cols < 0) return METIS_E_ARG;
+    if (mode == METIS_MODE_P32_F32) mode = METIS_MODE_P32;     // same arithmetic, the packed format does not know its source
     if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) return METIS_E_ARG;
     if (out_dtype != METIS_DTYPE_BF16 && out_dtype != METIS_DTYPE_F32) return METIS_E_ARG;
     if (cols % kBlock) return METIS_E_SHAPE;

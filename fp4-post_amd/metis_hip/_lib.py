@@ -13,6 +13,7 @@ LIB_PATH = os.path.join(_HERE, "libmetis_hip.so")
 
 OK, E_ARG, E_SHAPE, E_WORKSPACE, E_LAUNCH, E_DEVICE = 0, -1, -2, -3, -4, -5
 MODE_P32, MODE_PB16 = 0, 1
+MODE_P32_F32 = 2      # quantizer entry points only: binary32 arithmetic on a binary32 tensor
 DTYPE_BF16, DTYPE_F32 = 0, 1
 
 _vp, _i64, _i32, _u64, _f32, _sz = (ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_uint64,

@@ -284,8 +284,12 @@ class LinearLowbitFunction(torch.autograd.Function):
                 # dgrad: contraction over N; wgrad: contraction over tokens.  Operands are packed straight from the
                 # tensors autograd hands over, in compute_dtype arithmetic (no upcast copies of bf16 tensors).
                 cd = F.compute_dtype
-                # the kernels read bf16 values: one rounding pass per tensor, shared by its row and column packing
-                dy2, x2 = _flat2d(grad_output).to(torch.bfloat16), _flat2d(input_).to(torch.bfloat16)
+                # binary32 arithmetic quantizes the tensors as they are (binary32 gradients need not be bf16 values);
+                # bf16 arithmetic casts to the compute dtype first, as the reference does (453): one pass per tensor,
+                # shared by its row and column packing
+                dy2, x2 = _flat2d(grad_output), _flat2d(input_)
+                if cd != torch.float32:
+                    dy2, x2 = dy2.to(torch.bfloat16), x2.to(torch.bfloat16)
                 p_dy = qg.pack(dy2, arith=cd)
                 pw_col = ctx.pw.transposed                    # lives as long as the (possibly cached) packed weight
                 if pw_col is None:
@@ -421,13 +425,15 @@ class _MetisFusedFunction(torch.autograd.Function):
         # residual branch on re-quantized operands
         qg, qi = F.q_backward_outputgrad, F.q_backward_input
         if L % 32 == 0 and N % 32 == 0 and is_hip_nvfp4(qg) and is_hip_nvfp4(qi):
-            ar = F.compute_dtype                               # arithmetic of the quantizers; the tensors stay bf16
+            ar = F.compute_dtype                               # arithmetic of the quantizers
             p_res_col = ctx.p_res.transposed                   # lives as long as the (cached) packed residual
             if p_res_col is None:
                 p_res_col = ctx.p_res.transposed = F.q_forward_weight.pack(res, col=True, arith=ar)
-            gx = gx + ops.linear_dgrad(qg.pack(dy2, arith=ar), p_res_col, out_dtype=cd)
+            # binary32 arithmetic quantizes the tensors autograd handed over, not their bf16 roundings
+            dyq, xq_src = (_flat2d(dy), _flat2d(x)) if ar == torch.float32 else (dy2, x2)
+            gx = gx + ops.linear_dgrad(qg.pack(dyq, arith=ar), p_res_col, out_dtype=cd)
             # autograd rounds to the parameter's dtype anyway: let the GEMM epilogue do that rounding
-            g_res = ops.linear_wgrad(qg.pack(dy2, col=True, arith=ar), qi.pack(x2, col=True, arith=ar),
+            g_res = ops.linear_wgrad(qg.pack(dyq, col=True, arith=ar), qi.pack(xq_src, col=True, arith=ar),
                                      out_dtype=torch.bfloat16 if res.dtype == torch.bfloat16 else torch.float32)
         else:
             dyq = F._quantize_wgrad_operand(dy2.to(F.compute_dtype), qg)

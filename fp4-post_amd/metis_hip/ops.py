@@ -56,11 +56,21 @@ def _as_2d_bf16(x: torch.Tensor) -> torch.Tensor:
     if not x.is_cuda:
         raise _lib.MetisHipError("metis_hip ops need a ROCm device tensor; there is no CPU path")
     if x.dtype != torch.bfloat16:
-        # P32 parity is defined on bf16-valued inputs; a wider tensor must already hold bf16 values
-        xb = x.to(torch.bfloat16)
-        x = xb
+        x = x.to(torch.bfloat16)
     x2 = x.reshape(-1, x.shape[-1])
     return x2 if x2.is_contiguous() else x2.contiguous()
+
+
+def _as_2d_for_quant(x: torch.Tensor, mode: int) -> tuple[torch.Tensor, int]:
+    """(2-D contiguous tensor, kernel mode).  bf16 tensors go to the bf16 kernels.  In binary32 arithmetic any
+    other dtype is quantized from its binary32 values (they need not be bf16 values); in bf16 arithmetic the
+    tensor is first cast to bf16, as the reference casts to its compute dtype."""
+    if mode == MODE_P32 and x.dtype != torch.bfloat16:
+        if not x.is_cuda:
+            raise _lib.MetisHipError("metis_hip ops need a ROCm device tensor; there is no CPU path")
+        x2 = x.to(torch.float32).reshape(-1, x.shape[-1])
+        return (x2 if x2.is_contiguous() else x2.contiguous()), _lib.MODE_P32_F32
+    return _as_2d_bf16(x), mode
 
 
 def quantize(x: torch.Tensor, mode: int = MODE_P32, *, col: bool = False, sr: bool = False,
@@ -72,7 +82,7 @@ def quantize(x: torch.Tensor, mode: int = MODE_P32, *, col: bool = False, sr: bo
     sr=True  : stochastic rounding; `noise` (same shape as x, float32 for P32 / bf16 for PB16)
                overrides the internal Philox stream keyed by (seed, offset).
     """
-    x2 = _as_2d_bf16(x)
+    x2, kmode = _as_2d_for_quant(x, mode)
     rows, cols = x2.shape
     blocked = rows if col else cols
     if blocked % BLOCK:
@@ -90,12 +100,12 @@ def quantize(x: torch.Tensor, mode: int = MODE_P32, *, col: bool = False, sr: bo
             want = torch.bfloat16 if mode == MODE_PB16 else torch.float32
             nz = noise.reshape(rows, cols).to(want).contiguous()
         fn = L.metis_nvfp4_quant_sr_col if col else L.metis_nvfp4_quant_sr_row
-        rc = fn(x2.data_ptr(), rows, cols, x2.stride(0), mode, None if nz is None else nz.data_ptr(),
+        rc = fn(x2.data_ptr(), rows, cols, x2.stride(0), kmode, None if nz is None else nz.data_ptr(),
                 seed & (2 ** 64 - 1), offset, codes.data_ptr(), scales.data_ptr(), unit.data_ptr(),
                 ws.data_ptr(), ws.numel(), _stream())
     else:
         fn = L.metis_nvfp4_quant_col if col else L.metis_nvfp4_quant_row
-        rc = fn(x2.data_ptr(), rows, cols, x2.stride(0), mode, codes.data_ptr(), scales.data_ptr(),
+        rc = fn(x2.data_ptr(), rows, cols, x2.stride(0), kmode, codes.data_ptr(), scales.data_ptr(),
                 unit.data_ptr(), ws.data_ptr(), ws.numel(), _stream())
     check(rc, "metis_nvfp4_quant", x.shape)
     return PackedNVFP4(codes, scales, unit, prow, pcol, mode)

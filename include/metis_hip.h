@@ -19,6 +19,12 @@
  *                       compute_dtype=float32, src/Metis/Metis/bitlinear.py:70,377)
  *       METIS_MODE_PB16 every eager op rounded to bf16 (compute_dtype=bfloat16,
  *                       src/grpo/grpo.py:204-205)
+ *       METIS_MODE_P32_F32  (metis_nvfp4_quant_* only) binary32 arithmetic on a binary32 tensor whose
+ *                       values need not be bf16 values: gradients and activations downstream of a
+ *                       layer that ran with compute_dtype=float32 (src/dpo/run_dpo_metis.py:134;
+ *                       the forward returns binary32, src/Metis/Metis/bitlinear.py:435-441).  x is
+ *                       float [rows, cols] (row stride ld % 4 == 0), noise float; the packed result
+ *                       is an ordinary METIS_MODE_P32 tensor.
  *
  * NVFP4 layout produced / consumed (the reference never materialises it; these are the integers
  * its arithmetic passes through, src/Metis/Metis/quant.py:19-31)
@@ -48,6 +54,7 @@ extern "C" {
 
 #define METIS_MODE_P32 0
 #define METIS_MODE_PB16 1
+#define METIS_MODE_P32_F32 2   /* quantizer entry points only: METIS_MODE_P32 with x (and noise) binary32 */
 
 #define METIS_DTYPE_BF16 0
 #define METIS_DTYPE_F32 1

@@ -51,8 +51,9 @@ def _p(t):
 
 
 def nvfp4_pack(x_bf16: torch.Tensor, mode: int, noise: torch.Tensor | None = None):
-    """-> (codes u8 [R,C/2], scales u8 [R,C/16], unit float, n_clamped)."""
-    assert x_bf16.dtype == torch.bfloat16 and x_bf16.is_contiguous()
+    """-> (codes u8 [R,C/2], scales u8 [R,C/16], unit float, n_clamped).  mode 2: binary32 arithmetic on a
+    float32 tensor whose values need not be bf16 values."""
+    assert x_bf16.is_contiguous() and x_bf16.dtype == (torch.float32 if mode == 2 else torch.bfloat16)
     x2 = x_bf16.reshape(-1, x_bf16.shape[-1])
     rows, cols = x2.shape
     if cols % 16:
@@ -62,7 +63,7 @@ def nvfp4_pack(x_bf16: torch.Tensor, mode: int, noise: torch.Tensor | None = Non
     unit = torch.zeros(1, dtype=torch.float32)
     ncl = torch.zeros(1, dtype=torch.int64)
     if noise is not None:
-        want = torch.bfloat16 if mode else torch.float32
+        want = torch.bfloat16 if mode == 1 else torch.float32
         assert noise.dtype == want and noise.is_contiguous() and noise.numel() == x2.numel()
     rc = lib().metis_oracle_nvfp4_pack(_p(x2), rows, cols, cols, mode, _p(noise), _p(codes),
                                        _p(scales), _p(unit), _p(ncl))

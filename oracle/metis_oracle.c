@@ -102,7 +102,7 @@ static inline float block_scalar(float amax, int mode)
 }
 
 /*
- * Pack a [rows, cols] bf16 tensor (row stride ld elements) into NVFP4.
+ * Pack a [rows, cols] bf16 tensor (binary32 in mode 2; row stride ld elements) into NVFP4.
  *   codes  [rows, cols/2]  element 2j in the low nibble of byte j; nibble = (x<0)<<3 | r
  *   scales [rows, cols/16] float8_e4m3fn byte of scalar/unit
  *   unit   = max(scalar)/448 (bf16-valued in mode 1)
@@ -111,10 +111,17 @@ static inline float block_scalar(float amax, int mode)
  *   n_clamped (optional) counts SR elements whose r rounded to 8 and were clamped to 7
  * Returns 0, or -1 when 16 does not divide cols.
  */
-int metis_oracle_nvfp4_pack(const uint16_t *x, int64_t rows, int64_t cols, int64_t ld, int mode,
+int metis_oracle_nvfp4_pack(const void *xin, int64_t rows, int64_t cols, int64_t ld, int mode,
                             const void *noise, uint8_t *codes, uint8_t *scales, float *unit,
                             int64_t *n_clamped)
 {
+    /* mode 2: the arithmetic of mode 0 on a binary32 tensor (the reference run with compute_dtype=float32 on
+     * values that are not bf16 values, e.g. gradients: bitlinear.py:453) */
+    const int f32in = mode == 2;
+    if (f32in) mode = 0;
+    const uint16_t *x = (const uint16_t *)xin;
+    const float *xf = (const float *)xin;
+#define LDX(i) (f32in ? xf[i] : bf16_f32(x[i]))
     if (cols % BLK) return -1;
     const int64_t nb = cols / BLK;
     float smax = 0.0f;
@@ -124,7 +131,7 @@ int metis_oracle_nvfp4_pack(const uint16_t *x, int64_t rows, int64_t cols, int64
         for (int64_t b = 0; b < nb; ++b) {
             float am = 0.0f;
             for (int j = 0; j < BLK; ++j) {
-                float a = fabsf(bf16_f32(x[r * ld + b * BLK + j]));
+                float a = fabsf(LDX(r * ld + b * BLK + j));
                 am = a > am ? a : am;
             }
             float s = fabsf(block_scalar(am, mode));
@@ -137,10 +144,10 @@ int metis_oracle_nvfp4_pack(const uint16_t *x, int64_t rows, int64_t cols, int64
 #pragma omp parallel for reduction(+ : clamped) schedule(static)
     for (int64_t r = 0; r < rows; ++r) {
         for (int64_t b = 0; b < nb; ++b) {
-            const uint16_t *xb = x + r * ld + b * BLK;
+            const int64_t xb = r * ld + b * BLK;
             float am = 0.0f;
             for (int j = 0; j < BLK; ++j) {
-                float a = fabsf(bf16_f32(xb[j]));
+                float a = fabsf(LDX(xb + j));
                 am = a > am ? a : am;
             }
             const float s = block_scalar(am, mode);
@@ -148,7 +155,7 @@ int metis_oracle_nvfp4_pack(const uint16_t *x, int64_t rows, int64_t cols, int64
             const float h = RD(mode, s / 2.0f);
             uint8_t nib[BLK];
             for (int j = 0; j < BLK; ++j) {
-                float xv = bf16_f32(xb[j]);
+                float xv = LDX(xb + j);
                 float u = 0.0f;
                 if (noise) {
                     int64_t idx = r * cols + b * BLK + j;
@@ -166,6 +173,7 @@ int metis_oracle_nvfp4_pack(const uint16_t *x, int64_t rows, int64_t cols, int64
     }
     if (n_clamped) *n_clamped = clamped;
     return 0;
+#undef LDX
 }
 
 /*

@@ -23,7 +23,7 @@
 
 extern "C" {
 uint16_t metis_oracle_f32_to_bf16(float f);
-int metis_oracle_nvfp4_pack(const uint16_t* x, int64_t rows, int64_t cols, int64_t ld, int mode, const void* noise,
+int metis_oracle_nvfp4_pack(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, const void* noise,
                             uint8_t* codes, uint8_t* scales, float* unit, int64_t* n_clamped);
 int metis_oracle_nvfp4_dequant(const uint8_t* codes, const uint8_t* scales, float unit, int64_t rows, int64_t cols, int mode,
                                uint16_t* out_bf16, float* out_f32);

@@ -345,3 +345,122 @@ def test_offsets_beyond_32_bits(ops):
     assert float(pc.unit.cpu()) == float(ut)
     assert torch.equal(pc.codes.view(32768, 36, -1), ct.cuda().view(32768, 1, -1).expand(-1, 36, -1))
     assert torch.equal(pc.scales.view(32768, 36, -1), st.cuda().view(32768, 1, -1).expand(-1, 36, -1))
+
+
+# ---------------------------------------------------------------------------------------------
+# binary32 tensors whose values are not bf16 values (binary32 arithmetic only): gradients and
+# activations downstream of a layer that ran with compute_dtype=float32
+# ---------------------------------------------------------------------------------------------
+def _f32_valued(seed, rows, cols):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(rows, cols, generator=g) * torch.exp(torch.randn(rows, 1, generator=g))
+    x.view(-1)[::211] *= 37.0                                    # outliers
+    x.view(-1)[::97] = 0
+    x.view(-1)[5::389] = -0.0
+    assert not torch.equal(x, x.bfloat16().float())
+    return x
+
+
+@pytest.mark.parametrize("shape", [(256, 512), (1, 16), (37, 48), (1000, 1536)])
+def test_f32_input_rne_row(ops, shape):
+    from oracle import c_oracle as C, metis_oracle as O
+    x = _f32_valued(400 + shape[0], *shape)
+    p = ops.quantize(x.cuda(), 0)
+    codes, scales, unit, _ = O.nvfp4_pack(x)                    # torch restatement of the reference
+    _check_packed(p, codes, scales, unit, str(shape))
+    cc, cs, cu, _ = C.nvfp4_pack(x, 2)                          # C restatement
+    _check_packed(p, cc, cs, cu, f"C {shape}")
+    assert p.mode == 0
+    want = O.nvfp4_qdq(x)
+    assert same_bits(ops.dequantize(p, torch.float32).cpu(), want)
+
+
+@pytest.mark.parametrize("shape", [(64, 96), (256, 512), (48, 1000)])
+def test_f32_input_rne_col(ops, shape):
+    from oracle import metis_oracle as O
+    x = _f32_valued(410 + shape[0], *shape)
+    p = ops.quantize(x.cuda(), 0, col=True)
+    codes, scales, unit, _ = O.nvfp4_pack_col(x)
+    assert (p.rows, p.cols) == (shape[1], shape[0])
+    _check_packed(p, codes, scales, unit, str(shape))
+
+
+def test_f32_input_ties_and_their_neighbours(ops):
+    """Block scalar 1 (maximum 6; 1e-9 is below half an ulp), so |x| / 0.5 is exact: every rounding
+    threshold of the element rule, its binary32 neighbours on both sides, and the three quotients where
+    the rule's second rounding matters (5, 7, 10 and their neighbours)."""
+    from oracle import c_oracle as C, metis_oracle as O
+    ties = torch.tensor([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0])
+    vals = torch.cat([ties, torch.nextafter(ties, torch.zeros(())), torch.nextafter(ties, torch.full((), 9.0))])
+    vals = torch.cat([vals, -vals])
+    rows = []
+    for i in range(0, vals.numel(), 15):
+        chunk = vals[i:i + 15]
+        rows.append(torch.cat([torch.tensor([6.0]), chunk, torch.zeros(15 - chunk.numel())]))
+    x = torch.stack(rows).contiguous()
+    p = ops.quantize(x.cuda(), 0)
+    codes, scales, unit, _ = O.nvfp4_pack(x)
+    _check_packed(p, codes, scales, unit, "ties")
+    cc, cs, cu, _ = C.nvfp4_pack(x, 2)
+    _check_packed(p, cc, cs, cu, "ties C")
+
+
+@pytest.mark.parametrize("col", [False, True])
+def test_f32_input_sr_explicit_noise(ops, col):
+    from oracle import metis_oracle as O
+    x = _f32_valued(420, 128, 256)
+    u = torch.rand(128, 256, generator=torch.Generator().manual_seed(421))
+    p = ops.quantize(x.cuda(), 0, col=col, sr=True, noise=u.cuda())
+    codes, scales, unit, _ = (O.nvfp4_pack_col if col else O.nvfp4_pack)(x, u)
+    _check_packed(p, codes, scales, unit, f"sr col={col}")
+
+
+@pytest.mark.parametrize("col", [False, True])
+def test_f32_input_sr_internal_stream(ops, col):
+    """Own random stream: scale bytes and unit bit-exact, every code a grid neighbour of the exact quotient,
+    a function of (seed, offset) only, unbiased in the mean."""
+    from oracle import metis_oracle as O
+    x = _f32_valued(430, 64, 128)
+    xd = x.cuda()
+    p = ops.quantize(xd, 0, col=col, sr=True, seed=99, offset=5)
+    xt = x.t().contiguous() if col else x
+    _, scales, unit, _ = O.nvfp4_pack(xt)
+    torch.cuda.synchronize()
+    assert torch.equal(p.scales.cpu(), scales) and float(p.unit.cpu()) == float(unit)
+    scalar = O.block_scalars(xt).double().reshape(xt.shape[0], -1, 1)
+    q = (xt.double().abs().reshape(xt.shape[0], -1, 16) / (scalar / 2)).reshape(xt.shape)
+    grid = torch.tensor([0, 1, 2, 3, 4, 6, 8, 12], dtype=torch.float64)
+    nib = torch.stack((p.codes.cpu() & 0xF, p.codes.cpu() >> 4), dim=-1).reshape(xt.shape)
+    mag = grid[(nib & 7).long()]
+    lo = grid[(torch.bucketize(q * (1 - 1e-6), grid, right=True) - 1).clamp(0, 7)]
+    hi = grid[torch.bucketize(q * (1 + 1e-6), grid).clamp(0, 7)]
+    assert bool(((mag >= lo) & (mag <= hi)).all())
+    assert bool((((nib & 8) != 0) == (xt < 0))[xt != 0].all())
+    again = ops.quantize(xd, 0, col=col, sr=True, seed=99, offset=5)
+    assert torch.equal(p.codes, again.codes)
+    # unbiased: mean over many seeds of the dequantized value approaches x
+    acc = torch.zeros_like(xt, dtype=torch.float64)
+    n = 256
+    for sd in range(n):
+        acc += ops.dequantize(ops.quantize(xd, 0, col=col, sr=True, seed=1000 + sd), torch.float32).cpu().double()
+    step = (scalar / 2 * 4).expand(-1, -1, 16).reshape(xt.shape)     # widest grid interval in units of x
+    assert float(((acc / n - xt.double()).abs() / step).max()) < 0.2
+
+
+def test_f32_input_argument_checks():
+    from metis_hip import _lib
+    lib = _lib.load()
+    x = torch.zeros(16, 64, dtype=torch.float32, device="cuda")
+    codes = torch.empty(16, 32, dtype=torch.uint8, device="cuda")
+    scales = torch.empty(16, 4, dtype=torch.uint8, device="cuda")
+    unit = torch.empty(1, dtype=torch.float32, device="cuda")
+    need = lib.metis_nvfp4_workspace_bytes(16, 64)
+    ws = torch.zeros(need, dtype=torch.uint8, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    call = lambda ptr, ld, mode: lib.metis_nvfp4_quant_row(ptr, 16, 64, ld, mode, codes.data_ptr(), scales.data_ptr(),
+                                                           unit.data_ptr(), ws.data_ptr(), need, st)
+    assert call(x.data_ptr(), 64, 2) == 0
+    assert call(x.data_ptr(), 66, 2) == _lib.E_ARG               # rows must stay 16-byte aligned
+    assert call(x.data_ptr() + 4, 64, 2) == _lib.E_ARG
+    assert call(x.data_ptr(), 64, 3) == _lib.E_ARG               # unknown mode
+    torch.cuda.synchronize()

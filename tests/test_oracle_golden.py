@@ -93,3 +93,21 @@ def test_bitlinear_forward_matches_reference(golden):
     y = torch.matmul(y, u.T)
     y = y + O.linear_forward(xq, O.nvfp4_qdq(res), b)
     assert same_bits(y, t(golden["bl_y"]))
+
+
+def test_c_oracle_binary32_input_mode_matches_torch_restatement():
+    """Mode 2 of the C oracle (binary32 arithmetic on values that are not bf16 values) against the torch
+    restatement, which the reference's golden vectors pin; on bf16-valued data it equals mode 0."""
+    import torch
+    from oracle import c_oracle as C, metis_oracle as O
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(64, 256, generator=g) * torch.exp(torch.randn(64, 1, generator=g))
+    x.view(-1)[::53] = 0
+    u = torch.rand(64, 256, generator=g)
+    for noise in (None, u):
+        codes, scales, unit, _ = O.nvfp4_pack(x, noise)
+        cc, cs, cu, _ = C.nvfp4_pack(x, 2, noise)
+        assert torch.equal(cc, codes) and torch.equal(cs, scales) and cu == float(unit)
+    xb = x.bfloat16()
+    a, b = C.nvfp4_pack(xb, 0), C.nvfp4_pack(xb.float(), 2)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1]) and a[2] == b[2]
