@@ -4,6 +4,11 @@ device-to-device copy of known size that calibrates the FETCH_SIZE / WRITE_SIZE 
     rocprofv3 --kernel-trace --stats -- python3 fp4-post_amd/metis_hip/tools/profile_workload.py
     rocprofv3 --pmc FETCH_SIZE       -- python3 fp4-post_amd/metis_hip/tools/profile_workload.py
     rocprofv3 --pmc WRITE_SIZE       -- python3 fp4-post_amd/metis_hip/tools/profile_workload.py
+
+`--extra` adds the other kernels of the library at representative shapes: bf16-arithmetic, stochastic-rounding,
+column-blocked and binary32-input quantizers, the skinny (decode) GEMM and the split-K GEMM with its reduction.
+
+    rocprofv3 --kernel-trace --stats -- python3 fp4-post_amd/metis_hip/tools/profile_workload.py --extra
 """
 import os
 import sys
@@ -33,5 +38,27 @@ def main(reps: int = 5):
     torch.cuda.synchronize()
 
 
+def extra(reps: int = 5):
+    g = torch.Generator().manual_seed(1002)
+    xf = torch.randn(8192, 4096, generator=g).cuda()                    # binary32, not bf16-valued
+    x = xf.bfloat16()
+    dec = torch.randn(64, 18944, generator=g).bfloat16().cuda()         # decode step: 64 tokens
+    pre = torch.randn(1024, 18944, generator=g).bfloat16().cuda()       # short prefill
+    w_up = ops.quantize((torch.randn(18944, 3584, generator=g) * 0.02).bfloat16().cuda())
+    w_down = ops.quantize((torch.randn(3584, 18944, generator=g) * 0.02).bfloat16().cuda())
+    p_dec_up, p_dec_down, p_pre = ops.quantize(dec[:, :3584].contiguous()), ops.quantize(dec), ops.quantize(pre)
+    for i in range(reps):
+        ops.quantize(x, 1)                                              # bf16 arithmetic, round to nearest
+        ops.quantize(x, 0, col=True)                                    # column-blocked
+        ops.quantize(x, 0, sr=True, seed=i)                             # stochastic rounding, own stream
+        ops.quantize(x, 0, sr=True, col=True, seed=i)
+        ops.quantize(xf, 0)                                             # binary32 input
+        ops.quantize(xf, 0, sr=True, col=True, seed=i)
+        ops.linear_fwd(p_dec_up, w_up)                                  # skinny: 64 x 18944 x 3584
+        ops.linear_fwd(p_dec_down, w_down)                              # skinny: 64 x 3584 x 18944
+        ops.linear_fwd(p_pre, w_down)                                   # split-K: 1024 x 3584 x 18944
+    torch.cuda.synchronize()
+
+
 if __name__ == "__main__":
-    main()
+    extra() if "--extra" in sys.argv[1:] else main()
