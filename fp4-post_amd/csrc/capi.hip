@@ -140,6 +140,30 @@ int metis_linear_wgrad(const void* dyt_codes, const void* dyt_scales, const floa
                       nullptr, grad_weight, out_dtype, (hipStream_t)stream);
 }
 
+int metis_nvfp4_quant_centered(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, const void* center,
+                               int sr, int col, const void* noise, uint64_t seed, uint64_t offset, void* codes,
+                               void* scales, float* unit, void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (!center) return METIS_E_ARG;
+    return quantize(x, rows, cols, ld, mode, sr != 0, col != 0, sr ? noise : nullptr, seed, offset, codes, scales, unit,
+                    workspace, workspace_bytes, (hipStream_t)stream, center);
+}
+
+int metis_nvfp4_matvec(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols,
+                       const float* v, float alpha, float* out, void* split, int64_t split_ld, int split_col, void* stream)
+{
+    return packed_gemv(codes, scales, unit, rows, cols, v, alpha, out, split, split_ld, split_col, (hipStream_t)stream);
+}
+
+int metis_linear_fwd_f32bias(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes,
+                             const void* b_scales, const float* b_unit, int64_t M, int64_t N, int64_t K, const void* t,
+                             const void* u, int64_t r, const float* bias, void* out, int out_dtype, void* workspace,
+                             size_t workspace_bytes, void* stream)
+{
+    return gemm_nvfp4(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype,
+                      (hipStream_t)stream, workspace, workspace_bytes, 1);
+}
+
 size_t metis_linear_workspace_bytes(int64_t M, int64_t N, int64_t K) { return gemm_workspace_bytes(M, N, K); }
 
 int metis_linear_fwd_ws(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes,

@@ -42,6 +42,11 @@ __device__ __forceinline__ uint4 expand8(uint32_t codes, half2_t sc)
     r.w = __builtin_bit_cast(uint32_t, h3);
     return r;
 }
+// bias[n]: bf16, or binary32 when bias_f32 is set (a bias that already carries a rank-one term, see nvfp4_gemv.hip)
+__device__ __forceinline__ float bias_value(const uint16_t* bias, int bias_f32, int n)
+{
+    return bias_f32 ? reinterpret_cast<const float*>(bias)[n] : bf16_lo(bias[n]);
+}
 __device__ __forceinline__ half2_t scale_pair(uint32_t byte)
 {
     const uint32_t h = (byte & 0x7fu) << 7;
@@ -54,7 +59,7 @@ __global__ __launch_bounds__(256) void gemm_nvfp4_kernel(
     const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const float* __restrict__ a_unit,
     const uint8_t* __restrict__ b_codes, const uint8_t* __restrict__ b_scales, const float* __restrict__ b_unit,
     int M, int N, int K, const uint16_t* __restrict__ t, const uint16_t* __restrict__ u, int r,
-    const uint16_t* __restrict__ bias, void* __restrict__ out)
+    const uint16_t* __restrict__ bias, void* __restrict__ out, int bias_f32)
 {
     constexpr int WM = BM / 2, WN = BN / 2;          // wave tile
     constexpr int TM = WM / 32, TN = WN / 32;        // 32x32 MFMA tiles per wave
@@ -180,7 +185,7 @@ __global__ __launch_bounds__(256) void gemm_nvfp4_kernel(
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     v[e] = acc[i][j][4 * g + e];
-                    if (bias) v[e] += bf16_lo(bias[n + e]);
+                    if (bias) v[e] += bias_value(bias, bias_f32, n + e);
                 }
                 if (OUT_F32) {
                     *reinterpret_cast<float4*>((float*)out + (int64_t)m * N + n) = make_float4(v[0], v[1], v[2], v[3]);
@@ -271,7 +276,7 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_nvfp4_large_kernel(
     const uint8_t* __restrict__ b_codes, const uint8_t* __restrict__ b_scales, const float* __restrict__ b_unit,
     int M, int N, int K, const uint16_t* __restrict__ t, const uint16_t* __restrict__ u, int r,
     const uint16_t* __restrict__ bias, void* __restrict__ out, int tiles_m, int tiles_n, float* __restrict__ ws,
-    int nsplit)
+    int nsplit, int bias_f32)
 {
     extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
     constexpr int TM = 4;                            // 32-tall MFMA tiles per wave along m
@@ -454,7 +459,7 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_nvfp4_large_kernel(
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         v[e] = acc[i][j][4 * g + e];
-                        if (bias) v[e] += bf16_lo(bias[min(n + e, N - 1)]);
+                        if (bias) v[e] += bias_value(bias, bias_f32, min(n + e, N - 1));
                     }
                     *reinterpret_cast<float4*>(wt + ((i * TN + j) * 4 + g) * (NTHREADS * 4)) = make_float4(v[0], v[1], v[2], v[3]);
                 }
@@ -477,7 +482,7 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_nvfp4_large_kernel(
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
                             v[e] = acc[i][j][4 * g + e];
-                            if (bias) v[e] += bf16_lo(bias[min(n0 + wn * WTN + nl + e, N - 1)]);
+                            if (bias) v[e] += bias_value(bias, bias_f32, min(n0 + wn * WTN + nl + e, N - 1));
                         }
                         uint2 w;
                         w.x = bf16_bits(v[0]) | (bf16_bits(v[1]) << 16);
@@ -513,7 +518,7 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_nvfp4_large_kernel(
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     v[e] = acc[i][j][4 * g + e];
-                    if (bias) v[e] += bf16_lo(bias[n + e]);
+                    if (bias) v[e] += bias_value(bias, bias_f32, n + e);
                 }
                 if (OUT_F32) {
                     *reinterpret_cast<float4*>((float*)out + (int64_t)m * N + n) = make_float4(v[0], v[1], v[2], v[3]);
@@ -642,7 +647,7 @@ template <int WN_WAVES>
 static int launch_large(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes,
                         const void* b_scales, const float* b_unit, int64_t M, int64_t N, int64_t K, const void* t,
                         const void* u, int64_t r, const void* bias, void* out, int out_dtype, hipStream_t st,
-                        float* ws = nullptr, int nsplit = 1)
+                        int bias_f32 = 0, float* ws = nullptr, int nsplit = 1)
 {
     static bool attr_set[3][64] = {};
     const size_t lds_bytes = 2 * (size_t)L_STAGE_HALVES * sizeof(uint16_t);
@@ -667,7 +672,7 @@ static int launch_large(const void* a_codes, const void* a_scales, const float* 
                   *bs = (const uint8_t*)b_scales;
     const uint16_t *tp = (const uint16_t*)t, *up = (const uint16_t*)u, *bp = (const uint16_t*)bias;
     int Mi = (int)M, Ni = (int)N, Ki = (int)K, ri = (int)r, tmi = tiles_m, tni = tiles_n;
-    void* args[] = {&ac, &as, &a_unit, &bc, &bs, &b_unit, &Mi, &Ni, &Ki, &tp, &up, &ri, &bp, &out, &tmi, &tni, &ws, &nsplit};
+    void* args[] = {&ac, &as, &a_unit, &bc, &bs, &b_unit, &Mi, &Ni, &Ki, &tp, &up, &ri, &bp, &out, &tmi, &tni, &ws, &nsplit, &bias_f32};
     if (hipLaunchKernel(fn, dim3(grid_x), dim3(128 * WN_WAVES), args, lds_bytes, st) != hipSuccess) {
         (void)hipGetLastError();
         return METIS_E_LAUNCH;
@@ -731,7 +736,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nvfp4_skinny_kernel(
     const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const float* __restrict__ a_unit,
     const uint8_t* __restrict__ b_codes, const uint8_t* __restrict__ b_scales, const float* __restrict__ b_unit,
     int M, int N, int K, const uint16_t* __restrict__ t, const uint16_t* __restrict__ u, int r,
-    const uint16_t* __restrict__ bias, void* __restrict__ out)
+    const uint16_t* __restrict__ bias, void* __restrict__ out, int bias_f32)
 {
     __shared__ float red[WAVES][TM * 16][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, hi = lane >> 5;
@@ -806,7 +811,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nvfp4_skinny_kernel(
         if (m >= M || n >= N) continue;                        // N % 4 == 0 is required
         if (bias)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] += bf16_lo(bias[n + e]);
+            for (int e = 0; e < 4; ++e) v[e] += bias_value(bias, bias_f32, n + e);
         if (OUT_F32) {
             *reinterpret_cast<float4*>((float*)out + (int64_t)m * N + n) = make_float4(v[0], v[1], v[2], v[3]);
         } else {
@@ -821,13 +826,13 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nvfp4_skinny_kernel(
 template <int TM, int C, int WAVES>
 static int launch_skinny(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes,
                          const void* b_scales, const float* b_unit, int64_t M, int64_t N, int64_t K, const void* t,
-                         const void* u, int64_t r, const void* bias, void* out, int out_dtype, hipStream_t st)
+                         const void* u, int64_t r, const void* bias, void* out, int out_dtype, hipStream_t st, int bias_f32)
 {
     const dim3 grid((unsigned)((N + 31) / 32), (unsigned)((M + 32 * TM - 1) / (32 * TM))), block(64 * WAVES);
 #define METIS_SK(F) hipLaunchKernelGGL((gemm_nvfp4_skinny_kernel<TM, C, WAVES, F>), grid, block, 0, st, (const uint8_t*)a_codes, \
                                        (const uint8_t*)a_scales, a_unit, (const uint8_t*)b_codes, (const uint8_t*)b_scales,   \
                                        b_unit, (int)M, (int)N, (int)K, (const uint16_t*)t, (const uint16_t*)u, (int)r,        \
-                                       (const uint16_t*)bias, out)
+                                       (const uint16_t*)bias, out, bias_f32)
     if (out_dtype == METIS_DTYPE_F32) METIS_SK(1); else METIS_SK(0);
 #undef METIS_SK
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
@@ -839,14 +844,14 @@ static int launch_skinny(const void* a_codes, const void* a_scales, const float*
 // workgroups anyway.
 static int gemm_skinny(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes,
                        const void* b_scales, const float* b_unit, int64_t M, int64_t N, int64_t K, const void* t,
-                       const void* u, int64_t r, const void* bias, void* out, int out_dtype, hipStream_t st)
+                       const void* u, int64_t r, const void* bias, void* out, int out_dtype, hipStream_t st, int bias_f32)
 {
     const bool al8 = ((uintptr_t)a_scales % 8) == 0 && ((uintptr_t)b_scales % 8) == 0;
     const int c = (K % 256 == 0 && al8) ? 4 : 1;
     const int64_t tiles_n = (N + 31) / 32;
     const int tm = (M <= 32 || tiles_n < device_cus() / 2) ? 1 : 2;
     const int waves = (tm == 1 && M <= 32 && tiles_n >= 2 * device_cus()) ? 4 : 8;
-#define METIS_SKL(TM, C, W) return launch_skinny<TM, C, W>(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st)
+#define METIS_SKL(TM, C, W) return launch_skinny<TM, C, W>(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st, bias_f32)
     if (tm == 1) {
         if (waves == 4) { if (c == 4) METIS_SKL(1, 4, 4); else METIS_SKL(1, 1, 4); }
         else { if (c == 4) METIS_SKL(1, 4, 8); else METIS_SKL(1, 1, 8); }
@@ -1096,7 +1101,8 @@ int gemm_expanded(const void* a_exp, const float* a_unit, const void* b_exp, con
 
 int gemm_nvfp4(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes, const void* b_scales,
                const float* b_unit, int64_t M, int64_t N, int64_t K, const void* t, const void* u, int64_t r,
-               const void* bias, void* out, int out_dtype, hipStream_t st, void* workspace, size_t workspace_bytes)
+               const void* bias, void* out, int out_dtype, hipStream_t st, void* workspace, size_t workspace_bytes,
+               int bias_f32)
 {
     if (!a_codes || !a_scales || !a_unit || !b_codes || !b_scales || !b_unit || !out) return METIS_E_ARG;
     if (M < 0 || N < 0 || K < 0 || r < 0) return METIS_E_ARG;
@@ -1105,33 +1111,33 @@ int gemm_nvfp4(const void* a_codes, const void* a_scales, const float* a_unit, c
     if (N % 4 || r % 32 || (r > 0 && (!t || !u))) return METIS_E_ARG;
     if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return METIS_E_ARG;
     if (((uintptr_t)a_codes % 16) || ((uintptr_t)b_codes % 16) || ((uintptr_t)a_scales % 2) || ((uintptr_t)b_scales % 2) ||
-        ((uintptr_t)out % 16) || ((uintptr_t)t % 16) || ((uintptr_t)u % 16))
+        ((uintptr_t)out % 16) || ((uintptr_t)t % 16) || ((uintptr_t)u % 16) || ((uintptr_t)bias % (bias_f32 ? 4 : 2)))
         return METIS_E_ARG;
     if (K % 32) return METIS_E_ARG;                            // 16-byte code chunks: rows must stay 16-byte aligned
     if (M == 0 || N == 0) return METIS_OK;
     if (M >= 256 && N >= 256 && K % BK == 0 && !getenv("METIS_GEMM_SMALL")) {
         if (getenv("METIS_GEMM_W4"))
-            return launch_large<2>(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st);
+            return launch_large<2>(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st, bias_f32);
         int nsplit = 1;
         if (workspace && !getenv("METIS_GEMM_NOSPLIT")) {
             nsplit = split_factor(M, N, K);
             if (nsplit > 1 && (((uintptr_t)workspace % 16) || workspace_bytes < gemm_workspace_bytes(M, N, K))) return METIS_E_WORKSPACE;
         }
         return launch_large<4>(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st,
-                               (float*)workspace, nsplit);
+                               bias_f32, (float*)workspace, nsplit);
     }
     if (M < 256 && K % 64 == 0 && !getenv("METIS_GEMM_SMALL"))    // up to four 64-row passes over the weights beat a mostly empty 256-row tile
-        return gemm_skinny(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st);
+        return gemm_skinny(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st, bias_f32);
     constexpr int BM = 128, BN = 128;
     dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM));
     if (out_dtype == METIS_DTYPE_F32)
         hipLaunchKernelGGL((gemm_nvfp4_kernel<BM, BN, 1>), grid, dim3(256), 0, st, (const uint8_t*)a_codes,
                            (const uint8_t*)a_scales, a_unit, (const uint8_t*)b_codes, (const uint8_t*)b_scales, b_unit,
-                           (int)M, (int)N, (int)K, (const uint16_t*)t, (const uint16_t*)u, (int)r, (const uint16_t*)bias, out);
+                           (int)M, (int)N, (int)K, (const uint16_t*)t, (const uint16_t*)u, (int)r, (const uint16_t*)bias, out, bias_f32);
     else
         hipLaunchKernelGGL((gemm_nvfp4_kernel<BM, BN, 0>), grid, dim3(256), 0, st, (const uint8_t*)a_codes,
                            (const uint8_t*)a_scales, a_unit, (const uint8_t*)b_codes, (const uint8_t*)b_scales, b_unit,
-                           (int)M, (int)N, (int)K, (const uint16_t*)t, (const uint16_t*)u, (int)r, (const uint16_t*)bias, out);
+                           (int)M, (int)N, (int)K, (const uint16_t*)t, (const uint16_t*)u, (int)r, (const uint16_t*)bias, out, bias_f32);
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 

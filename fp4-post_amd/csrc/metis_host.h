@@ -45,7 +45,7 @@ int launch_scales(int mode, const Workspace& ws, uint32_t ngroups, void* scales,
 
 int quantize(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, bool sr, bool col, const void* noise,
              uint64_t seed, uint64_t offset, void* codes, void* scales, float* unit, void* workspace,
-             size_t workspace_bytes, hipStream_t st);
+             size_t workspace_bytes, hipStream_t st, const void* center = nullptr);
 int dequantize(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, int mode, void* out,
                int out_dtype, hipStream_t st);
 int block_scalars(const void* x, int64_t rows, int64_t cols, int mode, void* s, hipStream_t st);
@@ -58,7 +58,10 @@ int rmsnorm_quantize(const void* x, const void* gamma, float eps, int64_t rows, 
 int gemm_nvfp4(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes, const void* b_scales,
                const float* b_unit, int64_t M, int64_t N, int64_t K, const void* t, const void* u, int64_t r,
                const void* bias, void* out, int out_dtype, hipStream_t st, void* workspace = nullptr,
-               size_t workspace_bytes = 0);
+               size_t workspace_bytes = 0, int bias_f32 = 0);
+// y = alpha * unit * deq(codes, scales) . v  (v == NULL: all ones); nvfp4_gemv.hip
+int packed_gemv(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, const float* v,
+                float alpha, float* out32, void* split, int64_t split_ld, int split_col, hipStream_t st);
 // bytes of split-K scratch gemm_nvfp4 can use for this shape on the current device (0: it would not split)
 size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 

@@ -22,23 +22,29 @@ namespace metis {
 // Phase 1, row-blocked: codes + parked block maxima + per-workgroup maximum.  One block of 16 per
 // thread per iteration: thread i <-> block i (32 contiguous bytes, two 16-byte loads).
 // ---------------------------------------------------------------------------------------------
-// F32IN (binary32 arithmetic only): x holds binary32 values that need not be bf16 values.  The short cuts
-// of the bf16 path (div6, div3, the guarded hardware conversion) are proven for bf16 inputs only, so these
+// WIDE (binary32 arithmetic only): the values to encode are binary32 values that need not be bf16 values,
+// because the input tensor is binary32 (in_f32) and/or a binary32 centre is subtracted first.  The short cuts
+// of the bf16 path (div6, div3, the guarded hardware conversion) are proven for bf16 values only, so these
 // instantiations use IEEE divisions and the literal encoder, and park the block maxima as binary32.
+//
+// center (optional): one value per column, subtracted before anything else: x - center rounded to the
+// arithmetic's dtype, the centred residual of the reference's mean mode (src/Metis/Metis/bitlinear.py:
+// 330-333).  binary32 [cols] in binary32 arithmetic (always WIDE then), bf16 [cols] in bf16 arithmetic.
 __device__ __forceinline__ float block_scalar_ieee(float amax) { return amax / 6.0f + 1e-9f; }
 
-template <int MODE, bool SR, bool F32IN = false>
+template <int MODE, bool SR, bool WIDE = false>
 __global__ __launch_bounds__(256) void quant_codes_kernel(
     const void* __restrict__ xv, uint32_t rows, uint32_t cols, int64_t ld, const void* __restrict__ noise,
     uint64_t seed, uint64_t offset, uint2* __restrict__ codes, void* __restrict__ ws_amax_v,
-    uint32_t* __restrict__ ws_gmax, uint32_t nblocks)
+    uint32_t* __restrict__ ws_gmax, uint32_t nblocks, int in_f32, const void* __restrict__ center)
 {
-    static_assert(!F32IN || MODE == 0, "binary32 input implies binary32 arithmetic");
+    static_assert(!WIDE || MODE == 0, "binary32 values imply binary32 arithmetic");
     const uint16_t* __restrict__ x = static_cast<const uint16_t*>(xv);
     uint16_t* __restrict__ ws_amax = static_cast<uint16_t*>(ws_amax_v);
     float gmax = 0.0f;
     const uint32_t nbpr = cols / kBlock;      // row layout: blocks per row
-    if constexpr (!SR && !F32IN) {
+    if constexpr (!SR && !WIDE) {
+      if (!center) {
         // Round-to-nearest rows: software-pipelined, the next block's 32 bytes are in flight while the
         // current block is encoded.
         const uint32_t step = gridDim.x * 256u;
@@ -66,11 +72,12 @@ __global__ __launch_bounds__(256) void quant_codes_kernel(
         }
         publish_group_max(gmax, ws_gmax);
         return;
+      }
     }
     for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < nblocks; i += gridDim.x * 256u) {
         float v[kBlock], u[kBlock] = {};
         const uint32_t row = i / nbpr, cb = i - row * nbpr;
-        if constexpr (F32IN) {
+        if (WIDE && in_f32) {
             const float4* p = reinterpret_cast<const float4*>(static_cast<const float*>(xv) + (int64_t)row * ld + (int64_t)cb * kBlock);
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
@@ -81,6 +88,22 @@ __global__ __launch_bounds__(256) void quant_codes_kernel(
             const uint4* p = reinterpret_cast<const uint4*>(x + (int64_t)row * ld + (int64_t)cb * kBlock);
             unpack16(p[0], p[1], v);
         }
+        if (center) {
+            if constexpr (MODE == 0) {
+                const float4* cp = reinterpret_cast<const float4*>(static_cast<const float*>(center) + (size_t)cb * kBlock);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const float4 f = cp[c];
+                    v[4 * c] -= f.x; v[4 * c + 1] -= f.y; v[4 * c + 2] -= f.z; v[4 * c + 3] -= f.w;
+                }
+            } else {
+                const uint4* cp = reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(center) + (size_t)cb * kBlock);
+                float cv[kBlock];
+                unpack16(cp[0], cp[1], cv);
+#pragma unroll
+                for (int j = 0; j < kBlock; ++j) v[j] = rb(v[j] - cv[j]);
+            }
+        }
         if (SR && noise) {
 #pragma unroll
             for (int j = 0; j < kBlock; ++j) {
@@ -90,7 +113,7 @@ __global__ __launch_bounds__(256) void quant_codes_kernel(
         }
         const float am = block_amax(v);
         gmax = fmaxf(gmax, am);
-        if constexpr (F32IN) {
+        if constexpr (WIDE) {
             static_cast<float*>(ws_amax_v)[i] = am;
             const float sc = block_scalar_ieee(am);
             codes[i] = (SR && !noise) ? encode_sr_hardware<0, true>(v, sc, seed, offset, i) : encode_literal<0, SR>(v, sc, u);
@@ -113,14 +136,14 @@ __global__ __launch_bounds__(256) void quant_codes_kernel(
 // column owns in the tile, instead of one scattered 8-byte and 2-byte store per lane.
 // ---------------------------------------------------------------------------------------------
 constexpr int kColTileBlocks = 16, kColTileCols = 64;
-template <int MODE, bool SR, bool F32IN = false>
+template <int MODE, bool SR, bool WIDE = false>
 __global__ __launch_bounds__(256) void quant_codes_col_kernel(
     const void* __restrict__ xv, uint32_t rows, uint32_t cols, int64_t ld, const void* __restrict__ noise,
     uint64_t seed, uint64_t offset, uint2* __restrict__ codes, void* __restrict__ ws_amax_v,
-    uint32_t* __restrict__ ws_gmax, uint32_t tiles_c, uint32_t tiles_total)
+    uint32_t* __restrict__ ws_gmax, uint32_t tiles_c, uint32_t tiles_total, int in_f32, const void* __restrict__ center)
 {
-    static_assert(!F32IN || MODE == 0, "binary32 input implies binary32 arithmetic");
-    using amax_t = typename std::conditional<F32IN, float, uint16_t>::type;   // parked block maximum
+    static_assert(!WIDE || MODE == 0, "binary32 values imply binary32 arithmetic");
+    using amax_t = typename std::conditional<WIDE, float, uint16_t>::type;   // parked block maximum
     const uint16_t* __restrict__ x = static_cast<const uint16_t*>(xv);
     amax_t* __restrict__ ws_amax = static_cast<amax_t*>(ws_amax_v);
     __shared__ uint2 s_codes[kColTileCols][kColTileBlocks + 1];
@@ -140,8 +163,19 @@ __global__ __launch_bounds__(256) void quant_codes_col_kernel(
                 float v[kBlock], u[kBlock] = {};
 #pragma unroll
                 for (int j = 0; j < kBlock; ++j)
-                    v[j] = F32IN ? static_cast<const float*>(xv)[(int64_t)(b * kBlock + j) * ld + c]
-                                 : bf16_lo(x[(int64_t)(b * kBlock + j) * ld + c]);
+                    v[j] = (WIDE && in_f32) ? static_cast<const float*>(xv)[(int64_t)(b * kBlock + j) * ld + c]
+                                            : bf16_lo(x[(int64_t)(b * kBlock + j) * ld + c]);
+                if (center) {                                  // one centre per column: the same for the whole block
+                    if constexpr (MODE == 0) {
+                        const float cen = static_cast<const float*>(center)[c];
+#pragma unroll
+                        for (int j = 0; j < kBlock; ++j) v[j] -= cen;
+                    } else {
+                        const float cen = bf16_lo(static_cast<const uint16_t*>(center)[c]);
+#pragma unroll
+                        for (int j = 0; j < kBlock; ++j) v[j] = rb(v[j] - cen);
+                    }
+                }
                 if (SR && noise) {
 #pragma unroll
                     for (int j = 0; j < kBlock; ++j) {
@@ -151,7 +185,7 @@ __global__ __launch_bounds__(256) void quant_codes_col_kernel(
                 }
                 am = block_amax(v);
                 gmax = fmaxf(gmax, am);
-                if constexpr (F32IN) {
+                if constexpr (WIDE) {
                     const float sc = block_scalar_ieee(am);
                     packed = (SR && !noise) ? encode_sr_hardware<0, true>(v, sc, seed, offset, (int64_t)c * nbc + b)
                                             : encode_literal<0, SR>(v, sc, u);
@@ -161,7 +195,7 @@ __global__ __launch_bounds__(256) void quant_codes_col_kernel(
                 }
             }
             s_codes[cl][bl] = packed;
-            if constexpr (F32IN) s_amax[cl][bl] = am;
+            if constexpr (WIDE) s_amax[cl][bl] = am;
             else s_amax[cl][bl] = (uint16_t)(__float_as_uint(am) >> 16);
         }
         __syncthreads();
@@ -506,9 +540,10 @@ static int launch_fused(const void* x, void* codes, void* scales, float* unit, c
     return rc;
 }
 
-template <int MODE, bool SR, bool COL, bool F32IN = false>
+template <int MODE, bool SR, bool COL, bool WIDE = false>
 static int launch_quant(const void* x, int64_t rows, int64_t cols, int64_t ld, const void* noise, uint64_t seed,
-                        uint64_t offset, void* codes, void* scales, float* unit, const Workspace& ws, hipStream_t st)
+                        uint64_t offset, void* codes, void* scales, float* unit, const Workspace& ws, hipStream_t st,
+                        int in_f32 = 0, const void* center = nullptr)
 {
     const uint32_t nblocks = (uint32_t)(rows * cols / kBlock);
     if constexpr (COL) {
@@ -519,21 +554,21 @@ static int launch_quant(const void* x, int64_t rows, int64_t cols, int64_t ld, c
         const int64_t cap = (int64_t)device_cus() * 8;
         if (g > cap) g = cap;
         if (g > kMaxGroups) g = kMaxGroups;
-        hipLaunchKernelGGL((quant_codes_col_kernel<MODE, SR, F32IN>), dim3((unsigned)g), dim3(256), 0, st, x,
+        hipLaunchKernelGGL((quant_codes_col_kernel<MODE, SR, WIDE>), dim3((unsigned)g), dim3(256), 0, st, x,
                            (uint32_t)rows, (uint32_t)cols, ld, noise, seed, offset, (uint2*)codes, (void*)ws.amax, ws.gmax, tiles_c,
-                           (uint32_t)tiles);
-        return launch_scales(F32IN ? METIS_MODE_P32_F32 : MODE, ws, (uint32_t)g, scales, unit, nblocks, st);
+                           (uint32_t)tiles, in_f32, center);
+        return launch_scales(WIDE ? METIS_MODE_P32_F32 : MODE, ws, (uint32_t)g, scales, unit, nblocks, st);
     } else {
         const int g1 = grid_for(nblocks);
-        hipLaunchKernelGGL((quant_codes_kernel<MODE, SR, F32IN>), dim3(g1), dim3(256), 0, st, x, (uint32_t)rows,
-                           (uint32_t)cols, ld, noise, seed, offset, (uint2*)codes, (void*)ws.amax, ws.gmax, nblocks);
-        return launch_scales(F32IN ? METIS_MODE_P32_F32 : MODE, ws, (uint32_t)g1, scales, unit, nblocks, st);
+        hipLaunchKernelGGL((quant_codes_kernel<MODE, SR, WIDE>), dim3(g1), dim3(256), 0, st, x, (uint32_t)rows,
+                           (uint32_t)cols, ld, noise, seed, offset, (uint2*)codes, (void*)ws.amax, ws.gmax, nblocks, in_f32, center);
+        return launch_scales(WIDE ? METIS_MODE_P32_F32 : MODE, ws, (uint32_t)g1, scales, unit, nblocks, st);
     }
 }
 
 int quantize(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, bool sr, bool col, const void* noise,
              uint64_t seed, uint64_t offset, void* codes, void* scales, float* unit, void* workspace,
-             size_t workspace_bytes, hipStream_t st)
+             size_t workspace_bytes, hipStream_t st, const void* center)
 {
     if (rows < 0 || cols < 0 || ld < cols) return METIS_E_ARG;
     if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16 && mode != METIS_MODE_P32_F32) return METIS_E_ARG;
@@ -544,19 +579,21 @@ int quantize(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, bo
     if (rows * cols / kBlock >= (int64_t)1 << 31) return METIS_E_ARG;
     if (!col && ((ld % (f32in ? 4 : 8)) || ((uintptr_t)x % 16))) return METIS_E_ARG;     // 16-byte vector loads
     if (col && f32in && ((uintptr_t)x % 4)) return METIS_E_ARG;
+    if (center && ((uintptr_t)center % 16)) return METIS_E_ARG;
+    const bool wide = f32in || (center && mode == METIS_MODE_P32);   // a binary32 centre leaves binary32 residuals
     if (((uintptr_t)codes % 8) || ((uintptr_t)scales % 8)) return METIS_E_ARG;
     Workspace ws;
     int rc = carve_workspace(workspace, workspace_bytes, rows, cols, &ws);
     if (rc != METIS_OK) return rc;
-    if (!sr && !col && !f32in && ld == cols && getenv("METIS_FUSED_QUANT")) {   // opt-in single-launch path; falls through when it does not fit
+    if (!sr && !col && !wide && !center && ld == cols && getenv("METIS_FUSED_QUANT")) {   // opt-in single-launch path; falls through when it does not fit
         const uint32_t nblocks = (uint32_t)(rows * cols / kBlock);
         rc = mode == 0 ? launch_fused<0>(x, codes, scales, unit, ws, nblocks, st)
                        : launch_fused<1>(x, codes, scales, unit, ws, nblocks, st);
         if (rc != 1) return rc;
     }
-#define METIS_Q(M, S, C) return launch_quant<M, S, C>(x, rows, cols, ld, noise, seed, offset, codes, scales, unit, ws, st)
-#define METIS_QF(S, C) return launch_quant<0, S, C, true>(x, rows, cols, ld, noise, seed, offset, codes, scales, unit, ws, st)
-    if (f32in) {
+#define METIS_Q(M, S, C) return launch_quant<M, S, C>(x, rows, cols, ld, noise, seed, offset, codes, scales, unit, ws, st, 0, center)
+#define METIS_QF(S, C) return launch_quant<0, S, C, true>(x, rows, cols, ld, noise, seed, offset, codes, scales, unit, ws, st, f32in, center)
+    if (wide) {
         if (!sr) { if (!col) METIS_QF(false, false); else METIS_QF(false, true); }
         else { if (!col) METIS_QF(true, false); else METIS_QF(true, true); }
     }

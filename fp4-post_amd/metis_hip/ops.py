@@ -74,13 +74,16 @@ def _as_2d_for_quant(x: torch.Tensor, mode: int) -> tuple[torch.Tensor, int]:
 
 
 def quantize(x: torch.Tensor, mode: int = MODE_P32, *, col: bool = False, sr: bool = False,
-             noise: torch.Tensor | None = None, seed: int = 0, offset: int = 0) -> PackedNVFP4:
+             noise: torch.Tensor | None = None, seed: int = 0, offset: int = 0,
+             center: torch.Tensor | None = None) -> PackedNVFP4:
     """NVFP4-quantize x (flattened to [R, C]).
 
     col=False: blocks of 16 along C -> PackedNVFP4 of shape (R, C).
     col=True : blocks of 16 along R, written transposed -> shape (C, R).
     sr=True  : stochastic rounding; `noise` (same shape as x, float32 for P32 / bf16 for PB16)
                overrides the internal Philox stream keyed by (seed, offset).
+    center   : [C] vector subtracted from every row first (the reference's mean mode), in the arithmetic's
+               dtype: the packed tensor is that of x - center.
     """
     x2, kmode = _as_2d_for_quant(x, mode)
     rows, cols = x2.shape
@@ -94,6 +97,19 @@ def quantize(x: torch.Tensor, mode: int = MODE_P32, *, col: bool = False, sr: bo
     unit = torch.empty(1, dtype=torch.float32, device=dev)
     ws = _workspace(rows, cols, dev)
     L = load()
+    if center is not None:
+        cen = center.reshape(-1).to(device=dev, dtype=torch.bfloat16 if mode == MODE_PB16 else torch.float32).contiguous()
+        if cen.numel() != cols:
+            raise ValueError(f"center must have one value per column ({cols}), got {cen.numel()}")
+        nz = None
+        if sr and noise is not None:
+            nz = noise.reshape(rows, cols).to(torch.bfloat16 if mode == MODE_PB16 else torch.float32).contiguous()
+        rc = L.metis_nvfp4_quant_centered(x2.data_ptr(), rows, cols, x2.stride(0), kmode, cen.data_ptr(), int(sr), int(col),
+                                          None if nz is None else nz.data_ptr(), seed & (2 ** 64 - 1), offset,
+                                          codes.data_ptr(), scales.data_ptr(), unit.data_ptr(), ws.data_ptr(), ws.numel(),
+                                          _stream())
+        check(rc, "metis_nvfp4_quant_centered", x.shape)
+        return PackedNVFP4(codes, scales, unit, prow, pcol, mode)
     if sr:
         nz = None
         if noise is not None:
@@ -119,6 +135,33 @@ def dequantize(p: PackedNVFP4, dtype: torch.dtype = torch.bfloat16) -> torch.Ten
                                     p.mode, out.data_ptr(), DTYPE_F32 if dtype == torch.float32 else DTYPE_BF16,
                                     _stream())
     check(rc, "metis_nvfp4_dequant", (p.rows, p.cols))
+    return out
+
+
+def matvec(p: PackedNVFP4, v: torch.Tensor | None = None, alpha: float = 1.0, *, out: torch.Tensor | None = None,
+           split: torch.Tensor | None = None, split_col: int = 0) -> torch.Tensor | None:
+    """y[i] = alpha * sum_k deq(p)[i, k] * v[k] in binary32 (v=None: all ones, i.e. row sums of deq(p)).
+
+    Returns y as float32 [rows] (written into `out` when given).  With `split` (a bf16 matrix with at least
+    split_col + 3 columns) y is also stored as three bf16 terms hi + mid + lo in columns split_col..+2 of
+    its rows; with split given and out=None nothing else is allocated and None is returned."""
+    dev = p.codes.device
+    vp = None
+    if v is not None:
+        v = v.reshape(-1).to(device=dev, dtype=torch.float32).contiguous()
+        if v.numel() != p.cols:
+            raise ValueError(f"vector length {v.numel()} does not match the packed tensor's {p.cols} columns")
+        vp = v.data_ptr()
+    if out is None and split is None:
+        out = torch.empty(p.rows, dtype=torch.float32, device=dev)
+    sp, sld = None, 0
+    if split is not None:
+        if split.dtype != torch.bfloat16 or split.dim() != 2 or split.shape[0] != p.rows or split.stride(1) != 1:
+            raise ValueError("split must be a bf16 matrix with one row per packed row and unit column stride")
+        sp, sld = split.data_ptr(), split.stride(0)
+    rc = load().metis_nvfp4_matvec(p.codes.data_ptr(), p.scales.data_ptr(), p.unit.data_ptr(), p.rows, p.cols, vp,
+                                   float(alpha), None if out is None else out.data_ptr(), sp, sld, int(split_col), _stream())
+    check(rc, "metis_nvfp4_matvec", (p.rows, p.cols))
     return out
 
 
@@ -187,8 +230,9 @@ def linear_fwd(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None,
         r = t.shape[1]
         if t.shape != (M, r) or u.shape != (N, r):
             raise ValueError("low-rank operands must be t[M, r], u[N, r]")
+    bias_f32 = bias is not None and bias.dtype == torch.float32     # e.g. bias + W^ me of the mean mode
     if bias is not None:
-        bias = bias.to(torch.bfloat16).contiguous()
+        bias = bias.contiguous() if bias_f32 else bias.to(torch.bfloat16).contiguous()
     out = torch.empty(M, N, dtype=out_dtype, device=dev)
     dt = DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16
     tp = None if t is None else t.data_ptr()
@@ -198,6 +242,8 @@ def linear_fwd(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None,
         # measured on MI355X: the packed kernel (expansion inside the K loop, 16 KiB/step of operand traffic)
         # is within 5 % of the expanded one at 8192x4096x14336 and faster on smaller shapes, so it is the default
         expanded = False
+    if expanded and bias_f32:
+        raise ValueError("the expanded-operand path takes a bf16 bias")
     if expanded:
         ae, be = expand(a), expand(b)
         rc = load().metis_linear_fwd_expanded(ae.data_ptr(), a.unit.data_ptr(), be.data_ptr(), b.unit.data_ptr(), M, N, K,
@@ -205,6 +251,12 @@ def linear_fwd(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None,
         check(rc, "metis_linear_fwd_expanded", (M, N, K))
         return out
     ws = _gemm_workspace(M, N, K, dev)
+    if bias_f32:
+        rc = load().metis_linear_fwd_f32bias(a.codes.data_ptr(), a.scales.data_ptr(), a.unit.data_ptr(), b.codes.data_ptr(),
+                                             b.scales.data_ptr(), b.unit.data_ptr(), M, N, K, tp, up, r, bp, out.data_ptr(), dt,
+                                             None if ws is None else ws.data_ptr(), 0 if ws is None else ws.numel(), _stream())
+        check(rc, "metis_linear_fwd_f32bias", (M, N, K))
+        return out
     if ws is not None:
         rc = load().metis_linear_fwd_ws(a.codes.data_ptr(), a.scales.data_ptr(), a.unit.data_ptr(), b.codes.data_ptr(),
                                         b.scales.data_ptr(), b.unit.data_ptr(), M, N, K, tp, up, r, bp, out.data_ptr(), dt,

@@ -242,6 +242,51 @@ int metis_linear_wgrad_ws(const void *dyt_codes, const void *dyt_scales, const f
                           int64_t L, int64_t N, int64_t K, void *grad_weight, int out_dtype,
                           void *workspace, size_t workspace_bytes, void *stream);
 
+/*
+ * Mean mode: X^ = 1 me^T + QDQ(X - me), the column mean over tokens kept in high precision and only the
+ * centred residual quantized (LinearLowbitFunction.svd_quant with metis_mode="mean",
+ * src/Metis/Metis/bitlinear.py:311-336; the default of the reference's MetisArgs, src/grpo/grpo.py:66).
+ * A matmul with X^ splits into a GEMM on the packed residual and rank-one terms:
+ *     X^ W^T = QDQ(X - me) W^T + 1 (W^ me)^T
+ * Three entry points provide the pieces.
+ *
+ * metis_nvfp4_quant_centered: the quantizers above applied to x - center, the subtraction rounded to the
+ * dtype of the mode exactly as the reference's `input_flat - me`.
+ *   center  one value per column of x: float [cols] in METIS_MODE_P32 / METIS_MODE_P32_F32 (the residual is
+ *           then a binary32 value and is encoded by the literal element rule), bf16 [cols] in
+ *           METIS_MODE_PB16; 16-byte aligned
+ *   sr, col  0/1: stochastic rounding (noise / seed / offset as in metis_nvfp4_quant_sr_row), column-blocked
+ *           and transposed output (as metis_nvfp4_quant_col; the centre still belongs to the columns of x)
+ */
+int metis_nvfp4_quant_centered(const void *x, int64_t rows, int64_t cols, int64_t ld, int mode,
+                               const void *center, int sr, int col, const void *noise, uint64_t seed,
+                               uint64_t offset, void *codes, void *scales, float *unit,
+                               void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * y[i] = alpha * sum_k deq(P)[i, k] * v[k] for a packed [rows, cols] tensor P, binary32 accumulation.
+ *   v      float [cols], 16-byte aligned, or NULL for all ones (row sums of the dequantized tensor)
+ *   out    float [rows] or NULL
+ *   split  bf16 matrix with row stride split_ld, or NULL: y[i] is also written as three bf16 terms
+ *          hi + mid + lo (exact to binary32 precision) into columns split_col .. split_col + 2 of row i,
+ *          the form in which a rank-one term enters the t / u operands of metis_linear_fwd
+ * With P a packed weight and v the mean this is W^ me (forward) or W^T^ me_dy (dgrad); with v = NULL and P
+ * a column-blocked residual it is the column sum the weight gradient's rank-one terms need.
+ */
+int metis_nvfp4_matvec(const void *codes, const void *scales, const float *unit, int64_t rows,
+                       int64_t cols, const float *v, float alpha, float *out, void *split,
+                       int64_t split_ld, int split_col, void *stream);
+
+/*
+ * metis_linear_fwd_ws with a binary32 bias [N]: the place for bias + W^ me, which a bf16 bias would round
+ * to 8 bits.  workspace may be NULL (no split-K).
+ */
+int metis_linear_fwd_f32bias(const void *a_codes, const void *a_scales, const float *a_unit,
+                             const void *b_codes, const void *b_scales, const float *b_unit,
+                             int64_t M, int64_t N, int64_t K, const void *t, const void *u,
+                             int64_t r, const float *bias, void *out, int out_dtype,
+                             void *workspace, size_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
