@@ -29,7 +29,7 @@ import torch.nn as nn
 import torch.nn.init as init
 
 from . import ops
-from .ops import PackedNVFP4
+from .ops import CenteredNVFP4, PackedNVFP4
 from .quant import (Cast2Fp32, Cast2NVFp4e2m1Block, Cast2NVFp4e2m1BlockNOSR, QuantFunc, is_hip_nvfp4, quant_func)
 
 __all__ = ["LinearLowbitFunction", "LinearLowbit", "BitLinear"]
@@ -220,13 +220,98 @@ class LinearLowbitFunction(torch.autograd.Function):
         return F.q_forward_input.quantize_dequantize(input_)
 
     @staticmethod
-    def _prepare_input(input_: torch.Tensor, mean_cache=None, cache_key="default"):
-        """Packed activation when the direct NVFP4 path applies, else the dequantized tensor."""
+    def _token_mean(input_: torch.Tensor, mean_cache=None, cache_key="default") -> torch.Tensor:
+        """Column mean over tokens in the compute dtype ([C]); single-token decode calls update a weighted
+        running mean per cache key instead (reference 311-329).  The cache holds ([1, C] mean, count) as the
+        reference's does."""
+        cd = LinearLowbitFunction.compute_dtype
+        flat = _flat2d(input_)
+        rows = flat.shape[0]
+        if cd == torch.float32:
+            this_mean = flat.mean(dim=0, keepdim=True, dtype=torch.float32)       # no binary32 copy of a bf16 tensor
+        else:
+            this_mean = flat.to(cd).mean(dim=0, keepdim=True)
+        seq_len = input_.shape[1] if input_.dim() == 3 else input_.shape[0]
+        if seq_len == 1 and mean_cache is not None and cache_key in mean_cache:
+            cached_mean, cached_count = mean_cache[cache_key]
+            new_count = cached_count + rows
+            me = (cached_mean * cached_count + this_mean * rows) / new_count
+            mean_cache[cache_key] = (me.detach(), new_count)
+        else:
+            me = this_mean
+            if mean_cache is not None:
+                mean_cache[cache_key] = (me.detach(), rows)
+        return me.reshape(-1)
+
+    @staticmethod
+    def _mean_mode_packable() -> bool:
         F = LinearLowbitFunction
-        if not F.enable_activation_svd and not F.enable_nv_recipe and _packable(input_, F.q_forward_input):
-            # the kernels read bf16 values and take the arithmetic as a mode: no upcast copy of a bf16 tensor
-            return F.q_forward_input.pack(_flat2d(input_), arith=F.compute_dtype)
+        return F.metis_mode == "mean" and not F.tp_simulate and not F.enable_nv_recipe
+
+    @staticmethod
+    def _prepare_input(input_: torch.Tensor, mean_cache=None, cache_key="default"):
+        """Packed activation when a kernel path applies (direct: PackedNVFP4; mean mode: CenteredNVFP4), else
+        the dequantized tensor."""
+        F = LinearLowbitFunction
+        if not F.enable_nv_recipe and _packable(input_, F.q_forward_input):
+            if not F.enable_activation_svd:
+                # the kernels read bf16 values and take the arithmetic as a mode: no upcast copy of a bf16 tensor
+                return F.q_forward_input.pack(_flat2d(input_), arith=F.compute_dtype)
+            if F._mean_mode_packable():
+                # mean + QDQ(x - mean) (reference 311-336) without materialising either: the subtraction happens
+                # inside the quantizer and the mean's contribution to a matmul is a rank-one term
+                me = F._token_mean(input_, mean_cache=mean_cache, cache_key=cache_key)
+                return CenteredNVFP4(F.q_forward_input.pack(_flat2d(input_), arith=F.compute_dtype, center=me), me)
         return F.quantize_input(input_, mean_cache=mean_cache, cache_key=cache_key)
+
+    @staticmethod
+    def _packed_grads(dy2, x2, pw_col, center_x, gx_dtype, gw_dtype):
+        """(grad_input [L, K], grad_weight [N, K]) on packed operands.  dgrad contracts over N, wgrad over tokens.
+
+        Direct mode: dY^ = SR-Q(dY).  Mean mode (enable_backward_svd): dY^ = 1 me_dy^T + SR-Q(dY - me_dy)
+        (reference 462-474 with 311-336).  The saved activation enters the weight gradient as
+        1 center_x^T + SR-Q(X - center_x) along tokens (center_x None: plain SR-Q(X)).  The means contribute
+        rank-one terms:
+            gX = R_dy W^ + 1 (W^^T me_dy)^T
+            gW = R_dy^T R_x + (sum_l R_dy) center_x^T + me_dy (sum_l R_x + L center_x)^T
+        """
+        F = LinearLowbitFunction
+        cd = F.compute_dtype
+        qg, qi = F.q_backward_outputgrad, F.q_backward_input
+        me_dy = F._token_mean(dy2) if F.enable_backward_svd else None
+        p_dy = qg.pack(dy2, arith=cd, center=me_dy)
+        if me_dy is None:
+            gx = ops.linear_dgrad(p_dy, pw_col, out_dtype=gx_dtype)
+        else:
+            gx = ops.linear_fwd(p_dy, pw_col, bias=ops.matvec(pw_col, me_dy), out_dtype=gx_dtype)
+        p_dyt = qg.pack(dy2, col=True, arith=cd, center=me_dy)
+        p_xt = qi.pack(x2, col=True, arith=cd, center=center_x)
+        if me_dy is None and center_x is None:
+            # autograd rounds the gradient to the parameter's dtype anyway: let the GEMM epilogue do that rounding
+            return gx, ops.linear_wgrad(p_dyt, p_xt, out_dtype=gw_dtype)
+        gw = ops.linear_wgrad(p_dyt, p_xt, out_dtype=torch.float32)
+        left, right = [], []
+        if center_x is not None:
+            left.append(ops.matvec(p_dyt))
+            right.append(center_x.float())
+        if me_dy is not None:
+            tail = ops.matvec(p_xt)
+            if center_x is not None:
+                tail = tail + float(dy2.shape[0]) * center_x.float()
+            left.append(me_dy.float())
+            right.append(tail)
+        gw.addmm_(torch.stack(left, dim=1), torch.stack(right, dim=0))
+        return gx, gw
+
+    @staticmethod
+    def _packed_backward_applies(L: int, N: int, grad_output: torch.Tensor) -> bool:
+        F = LinearLowbitFunction
+        if not (L % 32 == 0 and N % 32 == 0 and is_hip_nvfp4(F.q_backward_outputgrad) and is_hip_nvfp4(F.q_backward_input)
+                and grad_output.dtype in (torch.float32, torch.bfloat16)):
+            return False
+        if not F.enable_backward_svd:
+            return True
+        return F.backward_lowrank_svd > 0 and F._mean_mode_packable()
 
     @staticmethod
     def _quantize_wgrad_operand(value: torch.Tensor, quantizer) -> torch.Tensor:
@@ -251,15 +336,22 @@ class LinearLowbitFunction(torch.autograd.Function):
         lead = input_.shape[:-1]
         ctx.lead = lead
         ctx.has_bias = bias is not None
-        ctx.packed = isinstance(quantized_input, PackedNVFP4) and isinstance(quantized_weight, PackedNVFP4)
+        ctx.packed = isinstance(quantized_input, (PackedNVFP4, CenteredNVFP4)) and isinstance(quantized_weight, PackedNVFP4)
         if ctx.packed:
             ctx.pw = quantized_weight
             ctx.weight_ref = weight
             ctx.save_for_backward(input_, bias if bias is not None else input_.new_empty(0))
+            ctx.center = None
+            if isinstance(quantized_input, CenteredNVFP4):
+                # (1 me^T + R) W^^T = R W^^T + 1 (W^ me)^T: the mean's term rides in a binary32 bias
+                ctx.center = quantized_input.mean
+                w_mean = ops.matvec(quantized_weight, quantized_input.mean)
+                bias = w_mean if bias is None else w_mean + bias.float()
+                quantized_input = quantized_input.residual
             out_dtype = torch.float32 if F.compute_dtype == torch.float32 else torch.bfloat16
             out = ops.linear_fwd(quantized_input, quantized_weight, bias=bias, out_dtype=out_dtype)
             return out.reshape(*lead, quantized_weight.rows).to(F.compute_dtype)
-        if isinstance(quantized_input, PackedNVFP4):
+        if isinstance(quantized_input, (PackedNVFP4, CenteredNVFP4)):
             quantized_input = quantized_input.dequantize(F.compute_dtype).reshape(input_.shape)
         if isinstance(quantized_weight, PackedNVFP4):
             quantized_weight = quantized_weight.dequantize(F.compute_dtype)
@@ -278,9 +370,7 @@ class LinearLowbitFunction(torch.autograd.Function):
         if ctx.packed:
             input_, _ = ctx.saved_tensors
             L, N = _flat2d(grad_output).shape
-            qg, qi = F.q_backward_outputgrad, F.q_backward_input
-            if (L % 32 == 0 and is_hip_nvfp4(qg) and is_hip_nvfp4(qi) and N % 32 == 0
-                    and grad_output.dtype in (torch.float32, torch.bfloat16)):
+            if F._packed_backward_applies(L, N, grad_output):
                 # dgrad: contraction over N; wgrad: contraction over tokens.  Operands are packed straight from the
                 # tensors autograd hands over, in compute_dtype arithmetic (no upcast copies of bf16 tensors).
                 cd = F.compute_dtype
@@ -290,20 +380,20 @@ class LinearLowbitFunction(torch.autograd.Function):
                 dy2, x2 = _flat2d(grad_output), _flat2d(input_)
                 if cd != torch.float32:
                     dy2, x2 = dy2.to(torch.bfloat16), x2.to(torch.bfloat16)
-                p_dy = qg.pack(dy2, arith=cd)
                 pw_col = ctx.pw.transposed                    # lives as long as the (possibly cached) packed weight
                 if pw_col is None:
                     pw_col = ctx.pw.transposed = F.q_forward_weight.pack(ctx.weight_ref, col=True, arith=cd)
                 gx_dtype = input_.dtype if input_.dtype in (torch.float32, torch.bfloat16) else torch.float32
-                gx = ops.linear_dgrad(p_dy, pw_col, out_dtype=gx_dtype)
-                # autograd rounds the gradient to the parameter's dtype anyway: let the GEMM epilogue do that rounding
                 gw_dtype = torch.bfloat16 if ctx.weight_ref.dtype == torch.bfloat16 else torch.float32
-                gw = ops.linear_wgrad(qg.pack(dy2, col=True, arith=cd), qi.pack(x2, col=True, arith=cd), out_dtype=gw_dtype)
+                gx, gw = F._packed_grads(dy2, x2, pw_col, ctx.center, gx_dtype, gw_dtype)
                 return gx.reshape(*ctx.lead, gx.shape[-1]), gw, grad_bias, None, None
             grad_output = grad_output.to(F.compute_dtype)
             dy2 = _flat2d(grad_output)
             x2 = _flat2d(input_.to(F.compute_dtype))
-            xq = F.q_forward_input.quantize_dequantize(x2)
+            if ctx.center is not None:
+                xq = ctx.center.to(F.compute_dtype) + F.q_forward_input.quantize_dequantize(x2 - ctx.center.to(F.compute_dtype))
+            else:
+                xq = F.q_forward_input.quantize_dequantize(x2)
             wq = ctx.pw.dequantize(F.compute_dtype)
         else:
             grad_output = grad_output.to(F.compute_dtype)
@@ -400,7 +490,15 @@ class _MetisFusedFunction(torch.autograd.Function):
         xv = torch.matmul(x2, v.to(cd).T)                      # [L, r] rank-r projection (library GEMM, bf16)
         t = xv * s.to(cd)
         out_dtype = torch.float32 if F.compute_dtype == torch.float32 else torch.bfloat16
-        y = ops.linear_fwd(px, p_res, t=t, u=u.to(cd), bias=None if bias is None else bias.to(cd), out_dtype=out_dtype)
+        ctx.center = None
+        gemm_bias = None if bias is None else bias.to(cd)
+        if isinstance(px, CenteredNVFP4):
+            # mean mode: the residual branch sees 1 me^T + R, whose mean term rides in a binary32 bias
+            ctx.center = px.mean
+            w_mean = ops.matvec(p_res, px.mean)
+            gemm_bias = w_mean if bias is None else w_mean + bias.float()
+            px = px.residual
+        y = ops.linear_fwd(px, p_res, t=t, u=u.to(cd), bias=gemm_bias, out_dtype=out_dtype)
         ctx.save_for_backward(x, v, s, u, res, xv)
         ctx.p_res = p_res
         ctx.has_bias = bias is not None
@@ -423,21 +521,29 @@ class _MetisFusedFunction(torch.autograd.Function):
         g_v = torch.matmul(g_xv.T, x2)                         # [r, K]
         gx = torch.matmul(g_xv, v.to(cd))                      # [L, K]
         # residual branch on re-quantized operands
-        qg, qi = F.q_backward_outputgrad, F.q_backward_input
-        if L % 32 == 0 and N % 32 == 0 and is_hip_nvfp4(qg) and is_hip_nvfp4(qi):
+        qg = F.q_backward_outputgrad
+        if F._packed_backward_applies(L, N, dy2):
             ar = F.compute_dtype                               # arithmetic of the quantizers
             p_res_col = ctx.p_res.transposed                   # lives as long as the (cached) packed residual
             if p_res_col is None:
                 p_res_col = ctx.p_res.transposed = F.q_forward_weight.pack(res, col=True, arith=ar)
             # binary32 arithmetic quantizes the tensors autograd handed over, not their bf16 roundings
             dyq, xq_src = (_flat2d(dy), _flat2d(x)) if ar == torch.float32 else (dy2, x2)
-            gx = gx + ops.linear_dgrad(qg.pack(dyq, arith=ar), p_res_col, out_dtype=cd)
-            # autograd rounds to the parameter's dtype anyway: let the GEMM epilogue do that rounding
-            g_res = ops.linear_wgrad(qg.pack(dyq, col=True, arith=ar), qi.pack(xq_src, col=True, arith=ar),
-                                     out_dtype=torch.bfloat16 if res.dtype == torch.bfloat16 else torch.float32)
+            g_res_gx, g_res = F._packed_grads(dyq, xq_src, p_res_col, ctx.center, cd,
+                                              torch.bfloat16 if res.dtype == torch.bfloat16 else torch.float32)
+            gx = gx + g_res_gx
         else:
-            dyq = F._quantize_wgrad_operand(dy2.to(F.compute_dtype), qg)
-            xq = F.q_forward_input.quantize_dequantize(x2.to(F.compute_dtype))
+            cdt = F.compute_dtype
+            if F.enable_backward_svd:
+                dyq = _flat2d(F.svd_quant(dy2.to(cdt), quant_func=qg, rank=F.backward_lowrank_svd, niter=F.backward_lowrank_niter,
+                                          broadcast_dim=F.backward_broadcast_dim, tp_simulate=F.tp_simulate,
+                                          tp_parts=F.tp_parts, metis_mode=F.metis_mode))
+            else:
+                dyq = F._quantize_wgrad_operand(dy2.to(cdt), qg)
+            if ctx.center is not None:
+                xq = ctx.center.to(cdt) + F.q_forward_input.quantize_dequantize(x2.to(cdt) - ctx.center.to(cdt))
+            else:
+                xq = F.q_forward_input.quantize_dequantize(x2.to(cdt))
             wq = F.q_forward_weight.quantize_dequantize(res.to(F.compute_dtype))
             gx = gx + torch.matmul(dyq, wq).to(cd)
             g_res = torch.matmul(dyq.T, xq).to(torch.float32)
@@ -554,7 +660,7 @@ class BitLinear(nn.Module):
         if share_activation:
             shared_input = self._get_shared_quantized_input(x)
             r = self.args.forward_svd_rank
-            if isinstance(shared_input, PackedNVFP4) and r % 32 == 0 and self.ulinear.bias is None:
+            if isinstance(shared_input, (PackedNVFP4, CenteredNVFP4)) and r % 32 == 0 and self.ulinear.bias is None:
                 # one fused launch for both branches; it already is the "merged" evaluation, so the
                 # rollout switch changes nothing on this path
                 wl = self.warmup_linear
@@ -566,7 +672,7 @@ class BitLinear(nn.Module):
                     return _MetisFusedFunction.apply(x, self.vlinear.weight, self.s, self.ulinear.weight,
                                                      self.warmup_linear.weight, self.warmup_linear.bias, shared_input, p_res)
             if BitLinear.rollout_merge_active and not torch.is_grad_enabled():
-                if isinstance(shared_input, PackedNVFP4):
+                if isinstance(shared_input, (PackedNVFP4, CenteredNVFP4)):
                     shared_input = shared_input.dequantize(F.compute_dtype).reshape(x.shape)
                 merged = self._get_merged_rollout_weight(shared_input.dtype)
                 y = torch.matmul(shared_input, merged.T)

@@ -37,6 +37,26 @@ class PackedNVFP4:
         return dequantize(self, dtype)
 
 
+@dataclass
+class CenteredNVFP4:
+    """Mean-mode activation: value[i, k] = mean[k] + deq(residual)[i, k] (the column mean over tokens stays in
+    high precision, only the centred residual is NVFP4).  `mean` is float32 [cols] in binary32 arithmetic,
+    bf16 [cols] in bf16 arithmetic."""
+    residual: PackedNVFP4
+    mean: torch.Tensor
+
+    @property
+    def rows(self) -> int:
+        return self.residual.rows
+
+    @property
+    def cols(self) -> int:
+        return self.residual.cols
+
+    def dequantize(self, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+        return self.mean.to(dtype).unsqueeze(0) + dequantize(self.residual, dtype)
+
+
 def _stream() -> int:
     return torch.cuda.current_stream().cuda_stream
 

@@ -88,17 +88,18 @@ class _NVFP4Base(BlockQuantFunc):
     @classmethod
     @torch.no_grad()
     def pack(cls, x: torch.Tensor, col: bool = False, noise: torch.Tensor | None = None,
-             arith: torch.dtype | None = None) -> ops.PackedNVFP4:
+             arith: torch.dtype | None = None, center: torch.Tensor | None = None) -> ops.PackedNVFP4:
         """Packed NVFP4 (codes, E4M3 scale bytes, unit) of x in the arithmetic of x's dtype, or of `arith`
-        when given: a bf16 tensor packed with arith=float32 gives what x.float() would, without the copy."""
+        when given: a bf16 tensor packed with arith=float32 gives what x.float() would, without the copy.
+        center: per-column vector subtracted first (mean mode): the packed tensor is that of x - center."""
         _need_gpu(x)
         if not col:
             cls._check(x)
         mode = _mode_of(x) if arith is None else (MODE_P32 if arith == torch.float32 else MODE_PB16)
         if cls.stochastic:
             return ops.quantize(x, mode, col=col, sr=True, noise=noise, seed=_NVFP4Base.sr_seed,
-                                offset=cls._next_offset(x.numel()) if noise is None else 0)
-        return ops.quantize(x, mode, col=col)
+                                offset=cls._next_offset(x.numel()) if noise is None else 0, center=center)
+        return ops.quantize(x, mode, col=col, center=center)
 
     @classmethod
     @torch.no_grad()

@@ -1,6 +1,8 @@
 """GPU parity of the pieces of the mean mode (column mean kept in high precision, centred residual in
 NVFP4): centred quantizers bit-exact against the oracle on x - me, the packed matrix-vector product and
 the binary32 bias of the GEMM against double precision."""
+import dataclasses
+
 import pytest
 import torch
 
@@ -104,3 +106,125 @@ def test_gemm_binary32_bias(M, N, K):
     want = ops.dequantize(px, torch.float32).double() @ ops.dequantize(pw, torch.float32).double().T + bias.double()
     torch.cuda.synchronize()
     assert rel_fro(got.cpu(), want.cpu()) <= 1e-6
+
+
+# ---------------------------------------------------------------------------------------------
+# module path: reference defaults (metis_mode="mean", activation and backward "svd" switches on)
+# ---------------------------------------------------------------------------------------------
+def _mean_args(rank=32):
+    from metis_hip import MetisArgs
+    args = MetisArgs(forward_svd_rank=rank, cache_quantized_weight=True)      # the reference's defaults: mean mode
+    assert args.metis_mode == "mean" and args.enable_activation_svd and args.enable_backward_svd
+    return args
+
+
+def _oracle_mean_qdq(x32):
+    from oracle import metis_oracle as O
+    me = x32.mean(dim=0, keepdim=True)
+    return me + O.nvfp4_qdq(x32 - me)
+
+
+def test_linear_lowbit_mean_mode_forward_runs_packed_and_matches_oracle(monkeypatch):
+    """LinearLowbit under the reference's default arguments: mean + QDQ(x - mean) against QDQ(W), on the
+    packed kernels (no dequantized activation or weight is ever formed)."""
+    from metis_hip import BitLinear, LinearLowbitFunction as F, ops
+    from oracle import metis_oracle as O
+    K, N, L = 256, 192, 128
+    args = _mean_args()
+    args.enable_forward_svd = False                                # keep the plain quantized linear, no factorisation
+    layer = BitLinear(K, N, args=args, bias=True, dtype=torch.bfloat16, compute_dtype=torch.float32).cuda()
+    lin = layer.warmup_linear
+    calls = []
+    real = ops.dequantize
+    monkeypatch.setattr(ops, "dequantize", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+    x = _offset_activation(600, L, K).reshape(2, L // 2, K)
+    y = lin(x.cuda())
+    assert not calls and y.dtype == torch.float32
+    w = lin.weight.detach().cpu().float()
+    want = _oracle_mean_qdq(x.reshape(L, K).float()).double() @ O.nvfp4_qdq(w).double().T + lin.bias.detach().cpu().double()
+    assert rel_fro(y.detach().cpu().reshape(L, N).double(), want) <= 1e-4
+    # removing the mean matters on this input: plain quantization of x is visibly worse against the dense product
+    dense = x.reshape(L, K).double() @ w.double().T + lin.bias.detach().cpu().double()
+    plain = O.nvfp4_qdq(x.reshape(L, K).float()).double() @ O.nvfp4_qdq(w).double().T + lin.bias.detach().cpu().double()
+    assert rel_fro(y.detach().cpu().reshape(L, N).double(), dense) < rel_fro(plain, dense)
+
+
+@pytest.mark.parametrize("compute", [torch.float32, torch.bfloat16])
+def test_packed_grads_mean_mode_decomposition(compute):
+    """The rank-one bookkeeping of the mean mode, made deterministic with round-to-nearest quantizers:
+    gX = (1 me_dy^T + R_dy) W^, gW = (1 me_dy^T + R_dy)^T (1 me_x^T + R_x), evaluated in double precision
+    from the same packed residuals."""
+    from metis_hip import LinearLowbitFunction as F, ops, quant_func
+    L, N, K = 256, 192, 320
+    g = torch.Generator().manual_seed(610)
+    x = _offset_activation(611, L, K).cuda()
+    dy = ((torch.randn(L, N, generator=g) + 0.7 * torch.randn(1, N, generator=g)) * 1e-2).bfloat16().cuda()
+    w = (torch.randn(N, K, generator=g) * 0.02).bfloat16().cuda()
+    keep = (F.q_backward_outputgrad, F.q_backward_input, F.enable_backward_svd, F.compute_dtype, F.metis_mode,
+            F.backward_lowrank_svd, F.tp_simulate, F.enable_nv_recipe)
+    rne = quant_func["nvfp4e2m1bnosr"]
+    try:
+        F.q_backward_outputgrad, F.q_backward_input, F.enable_backward_svd, F.compute_dtype = rne, rne, True, compute
+        F.metis_mode, F.backward_lowrank_svd, F.tp_simulate, F.enable_nv_recipe = "mean", 64, False, False
+        me_x = F._token_mean(x)
+        pw_col = rne.pack(w, col=True, arith=compute)
+        gx, gw = F._packed_grads(dy, x, pw_col, me_x, torch.float32, torch.float32)
+        me_dy = F._token_mean(dy)
+        # exact operand values code * e4m3 * unit (what the GEMM multiplies), also for tensors packed in bf16 arithmetic
+        d = lambda p: ops.dequantize(dataclasses.replace(p, mode=0), torch.float32).double()
+        dy_hat = me_dy.double() + d(rne.pack(dy, arith=compute, center=me_dy))
+        want_gx = dy_hat @ d(pw_col).t()                                   # [L, N] x [N, K]: pw_col is W^T packed as [K, N]
+        dyt_hat = me_dy.double().unsqueeze(1) + d(rne.pack(dy, col=True, arith=compute, center=me_dy))     # [N, L]
+        xt_hat = me_x.double().unsqueeze(1) + d(rne.pack(x, col=True, arith=compute, center=me_x))         # [K, L]
+        want_gw = dyt_hat @ xt_hat.t()
+    finally:
+        (F.q_backward_outputgrad, F.q_backward_input, F.enable_backward_svd, F.compute_dtype, F.metis_mode,
+         F.backward_lowrank_svd, F.tp_simulate, F.enable_nv_recipe) = keep
+    torch.cuda.synchronize()
+    assert rel_fro(gx.cpu().double(), want_gx.cpu()) <= 1e-5
+    assert rel_fro(gw.cpu().double(), want_gw.cpu()) <= 1e-5
+
+
+def test_bitlinear_mean_mode_forward_backward_and_decode_running_mean():
+    """Split BitLinear under the reference's defaults: forward against the formula with mean-mode
+    activations, gradients at FP4 noise level of the dense ones, and the single-token running mean."""
+    from metis_hip import BitLinear, LinearLowbitFunction as F
+    from oracle import metis_oracle as O
+    K, N, r, L = 256, 192, 32, 128
+    g = torch.Generator().manual_seed(620)
+    w = torch.randn(N, K, generator=g) * 0.02 + (torch.linalg.qr(torch.randn(N, 8, generator=g))[0] * 3.0) @ torch.linalg.qr(torch.randn(K, 8, generator=g))[0].T
+    layer = BitLinear(K, N, args=_mean_args(r), bias=True, dtype=torch.bfloat16, compute_dtype=torch.float32).cuda()
+    with torch.no_grad():
+        layer.warmup_linear.weight.copy_(w)
+    layer.split()
+    x = _offset_activation(621, L, K).reshape(2, L // 2, K).cuda().requires_grad_(True)
+    y = layer(x)
+    xf = x.detach().cpu().reshape(L, K).float()
+    v, s, u = (t.detach().cpu().float() for t in (layer.vlinear.weight, layer.s, layer.ulinear.weight))
+    res, b = layer.warmup_linear.weight.detach().cpu().float(), layer.warmup_linear.bias.detach().cpu().float()
+    low = ((xf.bfloat16() @ v.bfloat16().T) * s.bfloat16()).float() @ u.bfloat16().float().T        # bf16 rank-r branch
+    want = low.double() + _oracle_mean_qdq(xf).double() @ O.nvfp4_qdq(res).double().T + b.double()
+    assert rel_fro(y.detach().cpu().reshape(L, N).double(), want) <= 2e-3
+    dy = ((torch.randn(2, L // 2, N, generator=g) + 0.5) * 1e-2).bfloat16().cuda()
+    y.backward(dy.to(y.dtype))
+    dyf = dy.reshape(L, N).float().cpu()
+    assert rel_fro(x.grad.reshape(L, K).float().cpu(), dyf @ w) < 0.1
+    assert rel_fro(layer.warmup_linear.weight.grad.float().cpu(), dyf.T @ xf) < 0.3
+    for p in (layer.vlinear.weight, layer.ulinear.weight, layer.s, layer.warmup_linear.weight, layer.warmup_linear.bias):
+        assert p.grad is not None and bool(torch.isfinite(p.grad).all())
+    # decode: single-token calls fold into the cached mean with their row counts (reference 316-323)
+    key = f"{layer.layer_name}.shared"
+    cached, count = layer.mean_cache[key]
+    assert count == L
+    step = _offset_activation(622, 4, K).reshape(4, 1, K).cuda()
+    with torch.no_grad():
+        y1 = layer(step)
+    me2, count2 = layer.mean_cache[key]
+    assert count2 == L + 4
+    want_me = (cached * L + step.reshape(4, K).float().mean(dim=0, keepdim=True) * 4) / (L + 4)
+    assert torch.allclose(me2, want_me, rtol=1e-6, atol=1e-7)
+    sf = step.reshape(4, K).float().cpu()
+    mec = want_me.cpu()
+    low1 = ((sf.bfloat16() @ v.bfloat16().T) * s.bfloat16()).float() @ u.bfloat16().float().T
+    want1 = low1.double() + (mec + O.nvfp4_qdq(sf - mec)).double() @ O.nvfp4_qdq(res).double().T + b.double()
+    assert rel_fro(y1.cpu().reshape(4, N).double(), want1) <= 2e-3
