@@ -99,4 +99,89 @@ int packed_gemv(const void* codes, const void* scales, const float* unit, int64_
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Column mean over rows (tokens): me[c] = (sum_r x[r, c]) / rows, binary32 accumulation, the `input_flat.mean(dim=0)`
+// of the reference's mean mode (src/Metis/Metis/bitlinear.py:326).  HBM-bound: one read of x.
+// Phase 1: a workgroup sums a slab of rows for a strip of 256 columns (thread = 4 adjacent columns, the four
+// waves take every fourth row) and leaves one partial row in the workspace; phase 2 adds the partial rows in
+// a fixed order, divides and rounds to the output dtype.  No atomics: the result does not depend on timing.
+// ---------------------------------------------------------------------------------------------
+constexpr int kMeanMaxSlabs = 64;
+
+template <bool IN_F32>
+__global__ __launch_bounds__(256) void column_sum_kernel(const void* __restrict__ xv, uint32_t rows, uint32_t cols, int64_t ld,
+                                                         float* __restrict__ partial, uint32_t rows_per_slab)
+{
+    __shared__ float4 part[4][64];
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t c = (blockIdx.x * 64u + lane) * 4u;
+    const uint32_t r0 = blockIdx.y * rows_per_slab, r1 = min(r0 + rows_per_slab, rows);
+    float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (c < cols) {                                            // cols % 4 == 0: a thread's four columns exist together
+#pragma unroll 4
+        for (uint32_t r = r0 + wave; r < r1; r += 4u) {
+            if (IN_F32) {
+                const float4 f = *reinterpret_cast<const float4*>(static_cast<const float*>(xv) + (int64_t)r * ld + c);
+                acc.x += f.x; acc.y += f.y; acc.z += f.z; acc.w += f.w;
+            } else {
+                const uint2 w = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(xv) + (int64_t)r * ld + c);
+                acc.x += bf16_lo(w.x); acc.y += bf16_hi(w.x); acc.z += bf16_lo(w.y); acc.w += bf16_hi(w.y);
+            }
+        }
+    }
+    part[wave][lane] = acc;
+    __syncthreads();
+    if (wave == 0 && c < cols) {
+        const float4 a = part[0][lane], b = part[1][lane], d = part[2][lane], e = part[3][lane];
+        *reinterpret_cast<float4*>(partial + (size_t)blockIdx.y * cols + c) =
+            make_float4((a.x + b.x) + (d.x + e.x), (a.y + b.y) + (d.y + e.y), (a.z + b.z) + (d.z + e.z), (a.w + b.w) + (d.w + e.w));
+    }
+}
+
+template <bool OUT_BF16>
+__global__ __launch_bounds__(256) void column_mean_finish_kernel(const float* __restrict__ partial, uint32_t slabs, uint32_t cols,
+                                                                 float count, void* __restrict__ out)
+{
+    const uint32_t c = blockIdx.x * 256u + threadIdx.x;
+    if (c >= cols) return;
+    float s = 0.0f;
+    for (uint32_t k = 0; k < slabs; ++k) s += partial[(size_t)k * cols + c];
+    const float m = s / count;
+    if (OUT_BF16) static_cast<uint16_t*>(out)[c] = (uint16_t)bf16_bits(m);
+    else static_cast<float*>(out)[c] = m;
+}
+
+size_t column_mean_workspace_bytes(int64_t cols) { return cols > 0 ? (size_t)kMeanMaxSlabs * (size_t)cols * sizeof(float) : 0; }
+
+int column_mean(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_f32, void* out, int out_bf16, void* workspace,
+                size_t workspace_bytes, hipStream_t st)
+{
+    if (rows <= 0 || cols <= 0 || ld < cols) return METIS_E_ARG;
+    if (cols % 4 || ld % 4) return METIS_E_SHAPE;
+    if (!x || !out) return METIS_E_ARG;
+    if (rows > INT32_MAX || cols > INT32_MAX) return METIS_E_ARG;
+    if (((uintptr_t)x % (in_f32 ? 16 : 8)) || ((uintptr_t)out % 4)) return METIS_E_ARG;
+    if (!workspace || ((uintptr_t)workspace % 16) || workspace_bytes < column_mean_workspace_bytes(cols)) return METIS_E_WORKSPACE;
+    const uint32_t strips = (uint32_t)((cols + 255) / 256);
+    // enough workgroups to fill the device about eight times over, at least 16 rows each, at most kMeanMaxSlabs slabs
+    int64_t slabs = (8 * (int64_t)device_cus() + strips - 1) / strips;
+    if (slabs > (rows + 15) / 16) slabs = (rows + 15) / 16;
+    if (slabs > kMeanMaxSlabs) slabs = kMeanMaxSlabs;
+    if (slabs < 1) slabs = 1;
+    const uint32_t rows_per_slab = (uint32_t)((rows + slabs - 1) / slabs);
+    slabs = (rows + rows_per_slab - 1) / rows_per_slab;
+    float* partial = static_cast<float*>(workspace);
+    const dim3 grid(strips, (unsigned)slabs);
+    if (in_f32)
+        hipLaunchKernelGGL(column_sum_kernel<true>, grid, dim3(256), 0, st, x, (uint32_t)rows, (uint32_t)cols, ld, partial, rows_per_slab);
+    else
+        hipLaunchKernelGGL(column_sum_kernel<false>, grid, dim3(256), 0, st, x, (uint32_t)rows, (uint32_t)cols, ld, partial, rows_per_slab);
+    const dim3 g2((unsigned)((cols + 255) / 256));
+    if (out_bf16)
+        hipLaunchKernelGGL(column_mean_finish_kernel<true>, g2, dim3(256), 0, st, partial, (uint32_t)slabs, (uint32_t)cols, (float)rows, out);
+    else
+        hipLaunchKernelGGL(column_mean_finish_kernel<false>, g2, dim3(256), 0, st, partial, (uint32_t)slabs, (uint32_t)cols, (float)rows, out);
+    return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
+}
+
 }  // namespace metis

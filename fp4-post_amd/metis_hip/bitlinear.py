@@ -227,8 +227,13 @@ class LinearLowbitFunction(torch.autograd.Function):
         cd = LinearLowbitFunction.compute_dtype
         flat = _flat2d(input_)
         rows = flat.shape[0]
-        if cd == torch.float32:
-            this_mean = flat.mean(dim=0, keepdim=True, dtype=torch.float32)       # no binary32 copy of a bf16 tensor
+        if flat.is_cuda and flat.dtype in (torch.float32, torch.bfloat16) and flat.shape[1] % 4 == 0 and \
+                cd in (torch.float32, torch.bfloat16):
+            # one pass over the tensor; a bf16 tensor is read as it is in either arithmetic
+            src = flat if (cd == torch.float32 or flat.dtype == torch.bfloat16) else flat.to(cd)
+            this_mean = ops.column_mean(src, out_dtype=cd).unsqueeze(0)
+        elif cd == torch.float32:
+            this_mean = flat.mean(dim=0, keepdim=True, dtype=torch.float32)
         else:
             this_mean = flat.to(cd).mean(dim=0, keepdim=True)
         seq_len = input_.shape[1] if input_.dim() == 3 else input_.shape[0]

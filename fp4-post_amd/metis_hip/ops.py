@@ -158,6 +158,26 @@ def dequantize(p: PackedNVFP4, dtype: torch.dtype = torch.bfloat16) -> torch.Ten
     return out
 
 
+def column_mean(x: torch.Tensor, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """Mean over the rows of x flattened to [R, C] -> [C] (binary32 accumulation; bf16 or float32 in and out)."""
+    if not x.is_cuda:
+        raise _lib.MetisHipError("metis_hip ops need a ROCm device tensor; there is no CPU path")
+    if x.dtype not in (torch.bfloat16, torch.float32) or out_dtype not in (torch.bfloat16, torch.float32):
+        raise ValueError("column_mean: bfloat16 or float32 tensors only")
+    x2 = x.reshape(-1, x.shape[-1])
+    if not x2.is_contiguous():
+        x2 = x2.contiguous()
+    rows, cols = x2.shape
+    out = torch.empty(cols, dtype=out_dtype, device=x2.device)
+    L = load()
+    ws = torch.empty(L.metis_column_mean_workspace_bytes(cols), dtype=torch.uint8, device=x2.device)
+    rc = L.metis_column_mean(x2.data_ptr(), rows, cols, x2.stride(0), DTYPE_F32 if x2.dtype == torch.float32 else DTYPE_BF16,
+                             out.data_ptr(), DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16, ws.data_ptr(),
+                             ws.numel(), _stream())
+    check(rc, "metis_column_mean", x.shape)
+    return out
+
+
 def matvec(p: PackedNVFP4, v: torch.Tensor | None = None, alpha: float = 1.0, *, out: torch.Tensor | None = None,
            split: torch.Tensor | None = None, split_col: int = 0) -> torch.Tensor | None:
     """y[i] = alpha * sum_k deq(p)[i, k] * v[k] in binary32 (v=None: all ones, i.e. row sums of deq(p)).

@@ -264,6 +264,17 @@ int metis_nvfp4_quant_centered(const void *x, int64_t rows, int64_t cols, int64_
                                void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * me[c] = (sum_r x[r, c]) / rows: the column mean over tokens of the mean mode (`input_flat.mean(dim=0)`,
+ * src/Metis/Metis/bitlinear.py:326), binary32 accumulation in a fixed order (slabs of rows, then slabs).
+ *   x      [rows, cols] of x_dtype (METIS_DTYPE_BF16 / METIS_DTYPE_F32), row stride ld; cols % 4 == 0, ld % 4 == 0
+ *   out    [cols] of out_dtype (float for binary32 arithmetic, bf16 for bf16 arithmetic)
+ *   workspace  metis_column_mean_workspace_bytes(cols) bytes, 16-byte aligned, no initialisation needed
+ */
+size_t metis_column_mean_workspace_bytes(int64_t cols);
+int metis_column_mean(const void *x, int64_t rows, int64_t cols, int64_t ld, int x_dtype, void *out,
+                      int out_dtype, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * y[i] = alpha * sum_k deq(P)[i, k] * v[k] for a packed [rows, cols] tensor P, binary32 accumulation.
  *   v      float [cols], 16-byte aligned, or NULL for all ones (row sums of the dequantized tensor)
  *   out    float [rows] or NULL

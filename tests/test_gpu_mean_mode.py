@@ -228,3 +228,23 @@ def test_bitlinear_mean_mode_forward_backward_and_decode_running_mean():
     low1 = ((sf.bfloat16() @ v.bfloat16().T) * s.bfloat16()).float() @ u.bfloat16().float().T
     want1 = low1.double() + (mec + O.nvfp4_qdq(sf - mec)).double() @ O.nvfp4_qdq(res).double().T + b.double()
     assert rel_fro(y1.cpu().reshape(4, N).double(), want1) <= 2e-3
+
+
+@pytest.mark.parametrize("rows,cols,dtype", [(4096, 8960, torch.float32), (128, 256, torch.bfloat16), (1, 64, torch.float32),
+                                             (1000, 1540, torch.bfloat16), (17, 4, torch.float32)])
+def test_column_mean(rows, cols, dtype):
+    from metis_hip import ops
+    g = torch.Generator().manual_seed(rows)
+    x = (torch.randn(rows, cols, generator=g) + 2.0 * torch.randn(1, cols, generator=g)).to(dtype)
+    want = x.double().mean(dim=0)
+    got32 = ops.column_mean(x.cuda(), torch.float32).cpu()
+    assert float((got32.double() - want).abs().max()) <= 1e-6 * float(want.abs().max() + 1)
+    got16 = ops.column_mean(x.cuda(), torch.bfloat16).cpu()
+    assert got16.dtype == torch.bfloat16 and float((got16.double() - want).abs().max()) <= 2 ** -8 * float(want.abs().max() + 1)
+    # a strided view (row stride > cols)
+    wide = torch.zeros(rows, cols + 8, dtype=dtype)
+    wide[:, :cols] = x
+    xs = wide.cuda()[:, :cols]
+    if not xs.is_contiguous():
+        again = ops.column_mean(xs, torch.float32).cpu()
+        assert torch.equal(again, got32)
