@@ -133,8 +133,10 @@ __device__ __forceinline__ void sr_convert_pair(uint32_t& w, float q0, float q1,
 // word one bit apart).  One Philox4x32-10 draw serves a block: counter = offset + output block,
 // pair p (elements 2p, 2p+1) takes word p % 4, rotated by 16 bits for p >= 4 (the converter only
 // looks at the top 13 bits).  Scale bytes and unit do not depend on the rounding mode.
-// IEEE_DIV: the input need not be bf16-valued, so the quotient comes from a correctly rounded division.
-template <int MODE, bool IEEE_DIV = false>
+// WIDE_VALUES: the input need not be bf16-valued, which div3's exactness argument assumes; the quotient is then
+// x * rcp(s), within 2 ulp of x / s.  Stochastic rounding does not need more: the probability of rounding up
+// moves by 1e-7 of a grid interval, and a quotient that lands above 6 saturates in the converter either way.
+template <int MODE, bool WIDE_VALUES = false>
 __device__ __forceinline__ uint2 encode_sr_hardware(const float (&v)[kBlock], float s, uint64_t seed, uint64_t offset,
                                                     int64_t ob)
 {
@@ -148,7 +150,9 @@ __device__ __forceinline__ uint2 encode_sr_hardware(const float (&v)[kBlock], fl
     for (int j = 0; j < kBlock; j += 2) {
         const int p = j >> 1;
         const uint32_t bits = p < 4 ? word[p] : __builtin_amdgcn_alignbit(word[p & 3], word[p & 3], 16);
-        float q0 = IEEE_DIV ? v[j] / d : div3(v[j], d, rd_), q1 = IEEE_DIV ? v[j + 1] / d : div3(v[j + 1], d, rd_);
+        // "+ 0.0f" turns a -0.0 quotient into +0.0, as div3 does: the reference's sign(x) is 0 for x = -0.0
+        float q0 = WIDE_VALUES ? v[j] * rd_ + 0.0f : div3(v[j], d, rd_);
+        float q1 = WIDE_VALUES ? v[j + 1] * rd_ + 0.0f : div3(v[j + 1], d, rd_);
         if (MODE) {
             const uint32_t qq = rb_pair(q0, q1);
             q0 = bf16_lo(qq);

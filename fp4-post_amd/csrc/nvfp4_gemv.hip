@@ -139,13 +139,18 @@ __global__ __launch_bounds__(256) void column_sum_kernel(const void* __restrict_
 }
 
 template <bool OUT_BF16>
-__global__ __launch_bounds__(256) void column_mean_finish_kernel(const float* __restrict__ partial, uint32_t slabs, uint32_t cols,
+__global__ __launch_bounds__(64) void column_mean_finish_kernel(const float* __restrict__ partial, uint32_t slabs, uint32_t cols,
                                                                  float count, void* __restrict__ out)
 {
-    const uint32_t c = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t c = blockIdx.x * 64u + threadIdx.x;
     if (c >= cols) return;
+    // all loads first (independent, at most kMeanMaxSlabs of them), then the additions in slab order
+    float v[kMeanMaxSlabs];
+#pragma unroll
+    for (uint32_t k = 0; k < (uint32_t)kMeanMaxSlabs; ++k) v[k] = k < slabs ? partial[(size_t)k * cols + c] : 0.0f;
     float s = 0.0f;
-    for (uint32_t k = 0; k < slabs; ++k) s += partial[(size_t)k * cols + c];
+#pragma unroll
+    for (uint32_t k = 0; k < (uint32_t)kMeanMaxSlabs; ++k) s += v[k];
     const float m = s / count;
     if (OUT_BF16) static_cast<uint16_t*>(out)[c] = (uint16_t)bf16_bits(m);
     else static_cast<float*>(out)[c] = m;
@@ -176,11 +181,11 @@ int column_mean(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_f3
         hipLaunchKernelGGL(column_sum_kernel<true>, grid, dim3(256), 0, st, x, (uint32_t)rows, (uint32_t)cols, ld, partial, rows_per_slab);
     else
         hipLaunchKernelGGL(column_sum_kernel<false>, grid, dim3(256), 0, st, x, (uint32_t)rows, (uint32_t)cols, ld, partial, rows_per_slab);
-    const dim3 g2((unsigned)((cols + 255) / 256));
+    const dim3 g2((unsigned)((cols + 63) / 64));
     if (out_bf16)
-        hipLaunchKernelGGL(column_mean_finish_kernel<true>, g2, dim3(256), 0, st, partial, (uint32_t)slabs, (uint32_t)cols, (float)rows, out);
+        hipLaunchKernelGGL(column_mean_finish_kernel<true>, g2, dim3(64), 0, st, partial, (uint32_t)slabs, (uint32_t)cols, (float)rows, out);
     else
-        hipLaunchKernelGGL(column_mean_finish_kernel<false>, g2, dim3(256), 0, st, partial, (uint32_t)slabs, (uint32_t)cols, (float)rows, out);
+        hipLaunchKernelGGL(column_mean_finish_kernel<false>, g2, dim3(64), 0, st, partial, (uint32_t)slabs, (uint32_t)cols, (float)rows, out);
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 

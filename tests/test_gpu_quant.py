@@ -436,6 +436,7 @@ def test_f32_input_sr_internal_stream(ops, col):
     hi = grid[torch.bucketize(q * (1 + 1e-6), grid).clamp(0, 7)]
     assert bool(((mag >= lo) & (mag <= hi)).all())
     assert bool((((nib & 8) != 0) == (xt < 0))[xt != 0].all())
+    assert bool((nib[xt == 0] == 0).all())                          # +0.0 and -0.0 both give the all-zero nibble
     again = ops.quantize(xd, 0, col=col, sr=True, seed=99, offset=5)
     assert torch.equal(p.codes, again.codes)
     # unbiased: mean over many seeds of the dequantized value approaches x
