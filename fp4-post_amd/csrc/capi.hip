@@ -166,6 +166,19 @@ int metis_nvfp4_matvec(const void* codes, const void* scales, const float* unit,
     return packed_gemv(codes, scales, unit, rows, cols, v, alpha, out, split, split_ld, split_col, (hipStream_t)stream);
 }
 
+int metis_nvfp4_matvec_affine(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols,
+                              const float* v, float alpha, const float* z, float beta, float* out, void* stream)
+{
+    if (!out) return METIS_E_ARG;
+    return packed_gemv(codes, scales, unit, rows, cols, v, alpha, out, nullptr, 0, 0, (hipStream_t)stream, z, beta);
+}
+
+int metis_rank_one_operands(const float* a1, const float* b1, const float* a2, const float* b2, int64_t n, int64_t k,
+                            void* t, void* u, void* stream)
+{
+    return rank_one_operands(a1, b1, a2, b2, n, k, t, u, (hipStream_t)stream);
+}
+
 int metis_linear_fwd_f32bias(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes,
                              const void* b_scales, const float* b_unit, int64_t M, int64_t N, int64_t K, const void* t,
                              const void* u, int64_t r, const float* bias, void* out, int out_dtype, void* workspace,

@@ -61,7 +61,11 @@ int gemm_nvfp4(const void* a_codes, const void* a_scales, const float* a_unit, c
                size_t workspace_bytes = 0, int bias_f32 = 0);
 // y = alpha * unit * deq(codes, scales) . v  (v == NULL: all ones); nvfp4_gemv.hip
 int packed_gemv(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, const float* v,
-                float alpha, float* out32, void* split, int64_t split_ld, int split_col, hipStream_t st);
+                float alpha, float* out32, void* split, int64_t split_ld, int split_col, hipStream_t st,
+                const float* z = nullptr, float beta = 0.0f);
+// T [n, 32], U [k, 32] (bf16) with T U^T = a1 b1^T + a2 b2^T to binary32 precision; nvfp4_gemv.hip
+int rank_one_operands(const float* a1, const float* b1, const float* a2, const float* b2, int64_t n, int64_t k, void* T, void* U,
+                      hipStream_t st);
 // bytes of split-K scratch gemm_nvfp4 can use for this shape on the current device (0: it would not split)
 size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 

@@ -19,7 +19,8 @@ typedef float float2_t __attribute__((ext_vector_type(2)));
 __global__ __launch_bounds__(256) void packed_gemv_kernel(const uint2* __restrict__ codes, const uint8_t* __restrict__ scales,
                                                           const float* __restrict__ unit, uint32_t rows, uint32_t nblocks_row,
                                                           const float* __restrict__ v, float alpha, float* __restrict__ out32,
-                                                          uint16_t* __restrict__ split, int64_t split_ld, int split_col)
+                                                          uint16_t* __restrict__ split, int64_t split_ld, int split_col,
+                                                          const float* __restrict__ z, float beta)
 {
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6);
@@ -68,7 +69,8 @@ __global__ __launch_bounds__(256) void packed_gemv_kernel(const uint2* __restric
     }
     acc = wave_sum(acc);
     if (lane == 0) {
-        const float y = acc * (*unit) * alpha;
+        float y = acc * (*unit) * alpha;
+        if (z) y = fmaf(beta, z[row], y);
         if (out32) out32[row] = y;
         if (split) {
             uint16_t* d = split + (int64_t)row * split_ld + split_col;
@@ -84,18 +86,76 @@ __global__ __launch_bounds__(256) void packed_gemv_kernel(const uint2* __restric
 }
 
 int packed_gemv(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, const float* v,
-                float alpha, float* out32, void* split, int64_t split_ld, int split_col, hipStream_t st)
+                float alpha, float* out32, void* split, int64_t split_ld, int split_col, hipStream_t st, const float* z,
+                float beta)
 {
     if (rows < 0 || cols < 0) return METIS_E_ARG;
     if (cols % kBlock) return METIS_E_SHAPE;
     if (rows == 0) return METIS_OK;
     if (!codes || !scales || !unit || (!out32 && !split)) return METIS_E_ARG;
     if (rows > INT32_MAX || cols / kBlock > INT32_MAX) return METIS_E_ARG;
-    if (((uintptr_t)codes % 8) || ((uintptr_t)v % 16) || ((uintptr_t)out32 % 4) || ((uintptr_t)split % 2)) return METIS_E_ARG;
+    if (((uintptr_t)codes % 8) || ((uintptr_t)v % 16) || ((uintptr_t)out32 % 4) || ((uintptr_t)split % 2) || ((uintptr_t)z % 4)) return METIS_E_ARG;
     if (split && (split_col < 0 || split_ld < (int64_t)split_col + 3)) return METIS_E_ARG;
     hipLaunchKernelGGL(packed_gemv_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, (const uint2*)codes,
                        (const uint8_t*)scales, unit, (uint32_t)rows, (uint32_t)(cols / kBlock), v, alpha, out32,
-                       (uint16_t*)split, split_ld, split_col);
+                       (uint16_t*)split, split_ld, split_col, z, beta);
+    return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Rank-one terms for the low-rank extension of the GEMM:  T [n, 32], U [k, 32] (bf16) with
+//     T U^T = a1 b1^T + a2 b2^T      to binary32 precision,
+// each binary32 factor split into three bf16 terms x = h + m + l and the six leading cross products kept:
+// T columns (h, h, h, m, m, l) against U columns (h, m, l, h, m, h) per term; the other 20 columns are zero.
+// The weight gradient of the mean mode carries two such terms (bitlinear.py:311-336 applied to both operands).
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ void split3(float x, uint32_t (&p)[3])
+{
+    p[0] = bf16_bits(x);
+    const float r1 = x - __uint_as_float(p[0] << 16);
+    p[1] = bf16_bits(r1);
+    p[2] = bf16_bits(r1 - __uint_as_float(p[1] << 16));
+}
+
+__global__ __launch_bounds__(256) void rank_one_operands_kernel(const float* __restrict__ a1, const float* __restrict__ b1,
+                                                                const float* __restrict__ a2, const float* __restrict__ b2,
+                                                                uint32_t n, uint32_t k, uint16_t* __restrict__ T,
+                                                                uint16_t* __restrict__ U)
+{
+    const uint32_t row = blockIdx.x * 256u + threadIdx.x;
+    for (int side = 0; side < 2; ++side) {
+        const uint32_t limit = side ? k : n;
+        if (row >= limit) continue;
+        uint32_t h[16] = {};                                    // 32 bf16 values, two per word
+        const float* src[2] = {side ? b1 : a1, side ? b2 : a2};
+#pragma unroll
+        for (int term = 0; term < 2; ++term) {
+            if (!src[term]) continue;
+            uint32_t p[3];
+            split3(src[term][row], p);
+            // six columns of this term, as three words
+            const uint32_t left[3] = {p[0] | (p[0] << 16), p[0] | (p[1] << 16), p[1] | (p[2] << 16)};      // h h | h m | m l
+            const uint32_t right[3] = {p[0] | (p[1] << 16), p[2] | (p[0] << 16), p[1] | (p[0] << 16)};     // h m | l h | m h
+#pragma unroll
+            for (int w = 0; w < 3; ++w) h[term * 3 + w] = side ? right[w] : left[w];
+        }
+        uint4* dst = reinterpret_cast<uint4*>((side ? U : T) + (size_t)row * 32);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) dst[q] = make_uint4(h[4 * q], h[4 * q + 1], h[4 * q + 2], h[4 * q + 3]);
+    }
+}
+
+int rank_one_operands(const float* a1, const float* b1, const float* a2, const float* b2, int64_t n, int64_t k, void* T, void* U,
+                      hipStream_t st)
+{
+    if (n <= 0 || k <= 0 || n > INT32_MAX || k > INT32_MAX) return METIS_E_ARG;
+    if (!T || !U || !a1 != !b1 || !a2 != !b2) return METIS_E_ARG;
+    if (((uintptr_t)T % 16) || ((uintptr_t)U % 16) || ((uintptr_t)a1 % 4) || ((uintptr_t)b1 % 4) || ((uintptr_t)a2 % 4) ||
+        ((uintptr_t)b2 % 4))
+        return METIS_E_ARG;
+    const int64_t m = n > k ? n : k;
+    hipLaunchKernelGGL(rank_one_operands_kernel, dim3((unsigned)((m + 255) / 256)), dim3(256), 0, st, a1, b1, a2, b2, (uint32_t)n,
+                       (uint32_t)k, (uint16_t*)T, (uint16_t*)U);
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 

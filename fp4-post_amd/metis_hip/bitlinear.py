@@ -294,19 +294,15 @@ class LinearLowbitFunction(torch.autograd.Function):
         if me_dy is None and center_x is None:
             # autograd rounds the gradient to the parameter's dtype anyway: let the GEMM epilogue do that rounding
             return gx, ops.linear_wgrad(p_dyt, p_xt, out_dtype=gw_dtype)
-        gw = ops.linear_wgrad(p_dyt, p_xt, out_dtype=torch.float32)
-        left, right = [], []
+        # the rank-one terms ride in the GEMM's low-rank operands (three bf16 terms per factor: binary32 precision)
+        first = second = None
         if center_x is not None:
-            left.append(ops.matvec(p_dyt))
-            right.append(center_x.float())
+            first = (ops.matvec(p_dyt), center_x)
         if me_dy is not None:
-            tail = ops.matvec(p_xt)
-            if center_x is not None:
-                tail = tail + float(dy2.shape[0]) * center_x.float()
-            left.append(me_dy.float())
-            right.append(tail)
-        gw.addmm_(torch.stack(left, dim=1), torch.stack(right, dim=0))
-        return gx, gw
+            tail = ops.matvec(p_xt) if center_x is None else ops.matvec(p_xt, z=center_x, beta=float(dy2.shape[0]))
+            second = (me_dy, tail)
+        t, u = ops.rank_one_operands(p_dyt.rows, p_xt.rows, first or second, second if first else None)
+        return gx, ops.linear_fwd(p_dyt, p_xt, t=t, u=u, out_dtype=gw_dtype)
 
     @staticmethod
     def _packed_backward_applies(L: int, N: int, grad_output: torch.Tensor) -> bool:

@@ -179,8 +179,9 @@ def column_mean(x: torch.Tensor, out_dtype: torch.dtype = torch.float32) -> torc
 
 
 def matvec(p: PackedNVFP4, v: torch.Tensor | None = None, alpha: float = 1.0, *, out: torch.Tensor | None = None,
-           split: torch.Tensor | None = None, split_col: int = 0) -> torch.Tensor | None:
-    """y[i] = alpha * sum_k deq(p)[i, k] * v[k] in binary32 (v=None: all ones, i.e. row sums of deq(p)).
+           split: torch.Tensor | None = None, split_col: int = 0, z: torch.Tensor | None = None,
+           beta: float = 0.0) -> torch.Tensor | None:
+    """y[i] = alpha * sum_k deq(p)[i, k] * v[k] (+ beta * z[i]) in binary32 (v=None: all ones, i.e. row sums).
 
     Returns y as float32 [rows] (written into `out` when given).  With `split` (a bf16 matrix with at least
     split_col + 3 columns) y is also stored as three bf16 terms hi + mid + lo in columns split_col..+2 of
@@ -192,8 +193,18 @@ def matvec(p: PackedNVFP4, v: torch.Tensor | None = None, alpha: float = 1.0, *,
         if v.numel() != p.cols:
             raise ValueError(f"vector length {v.numel()} does not match the packed tensor's {p.cols} columns")
         vp = v.data_ptr()
-    if out is None and split is None:
+    if out is None and (split is None or z is not None):
         out = torch.empty(p.rows, dtype=torch.float32, device=dev)
+    if z is not None:
+        if split is not None:
+            raise ValueError("matvec: the affine tail and the split output are separate entry points")
+        z = z.reshape(-1).to(device=dev, dtype=torch.float32).contiguous()
+        if z.numel() != p.rows:
+            raise ValueError(f"z must have one value per packed row ({p.rows}), got {z.numel()}")
+        rc = load().metis_nvfp4_matvec_affine(p.codes.data_ptr(), p.scales.data_ptr(), p.unit.data_ptr(), p.rows, p.cols, vp,
+                                              float(alpha), z.data_ptr(), float(beta), out.data_ptr(), _stream())
+        check(rc, "metis_nvfp4_matvec_affine", (p.rows, p.cols))
+        return out
     sp, sld = None, 0
     if split is not None:
         if split.dtype != torch.bfloat16 or split.dim() != 2 or split.shape[0] != p.rows or split.stride(1) != 1:
@@ -203,6 +214,30 @@ def matvec(p: PackedNVFP4, v: torch.Tensor | None = None, alpha: float = 1.0, *,
                                    float(alpha), None if out is None else out.data_ptr(), sp, sld, int(split_col), _stream())
     check(rc, "metis_nvfp4_matvec", (p.rows, p.cols))
     return out
+
+
+def rank_one_operands(n: int, k: int, first: tuple | None, second: tuple | None = None):
+    """(t [n, 32], u [k, 32]) bf16 with t u^T = a1 b1^T (+ a2 b2^T) to binary32 precision; first = (a1 [n], b1 [k]),
+    second = (a2, b2) or None.  They go into linear_fwd as its low-rank operands."""
+    pairs = [pr for pr in (first, second) if pr is not None]
+    if not pairs:
+        raise ValueError("rank_one_operands: at least one (a, b) pair")
+    dev = pairs[0][0].device
+    ptrs, keep = [], []
+    for a, b in pairs:
+        a = a.reshape(-1).to(torch.float32).contiguous()
+        b = b.reshape(-1).to(torch.float32).contiguous()
+        if a.numel() != n or b.numel() != k:
+            raise ValueError("rank_one_operands: a must have n values and b must have k")
+        keep += [a, b]
+        ptrs += [a.data_ptr(), b.data_ptr()]
+    while len(ptrs) < 4:
+        ptrs.append(None)
+    t = torch.empty(n, 32, dtype=torch.bfloat16, device=dev)
+    u = torch.empty(k, 32, dtype=torch.bfloat16, device=dev)
+    rc = load().metis_rank_one_operands(ptrs[0], ptrs[1], ptrs[2], ptrs[3], n, k, t.data_ptr(), u.data_ptr(), _stream())
+    check(rc, "metis_rank_one_operands", (n, k))
+    return t, u
 
 
 def expand(p: PackedNVFP4) -> torch.Tensor:

@@ -288,6 +288,22 @@ int metis_nvfp4_matvec(const void *codes, const void *scales, const float *unit,
                        int64_t cols, const float *v, float alpha, float *out, void *split,
                        int64_t split_ld, int split_col, void *stream);
 
+/* metis_nvfp4_matvec with an affine tail: out[i] = alpha * sum_k deq(P)[i, k] * v[k] + beta * z[i]  (z float [rows]). */
+int metis_nvfp4_matvec_affine(const void *codes, const void *scales, const float *unit, int64_t rows,
+                              int64_t cols, const float *v, float alpha, const float *z, float beta,
+                              float *out, void *stream);
+
+/*
+ * Low-rank operands that carry up to two rank-one terms at binary32 precision:
+ *     t [n, 32], u [k, 32] (bf16, row stride 32)  with  t u^T = a1 b1^T + a2 b2^T
+ * (each factor split into three bf16 terms, the six leading cross products kept; unused columns zero).
+ * a1, a2 float [n]; b1, b2 float [k]; a pair may be NULL together.  The weight gradient of the mean mode,
+ *     (1 me_dy^T + R_dy)^T (1 me_x^T + R_x) = R_dy^T R_x + (sum_l R_dy) me_x^T + me_dy (sum_l R_x + L me_x)^T,
+ * is then one metis_linear_fwd call on the packed residuals with these t and u.
+ */
+int metis_rank_one_operands(const float *a1, const float *b1, const float *a2, const float *b2,
+                            int64_t n, int64_t k, void *t, void *u, void *stream);
+
 /*
  * metis_linear_fwd_ws with a binary32 bias [N]: the place for bias + W^ me, which a bf16 bias would round
  * to 8 bits.  workspace may be NULL (no split-K).

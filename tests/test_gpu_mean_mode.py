@@ -248,3 +248,23 @@ def test_column_mean(rows, cols, dtype):
     if not xs.is_contiguous():
         again = ops.column_mean(xs, torch.float32).cpu()
         assert torch.equal(again, got32)
+
+
+def test_rank_one_operands_reach_binary32_precision():
+    from metis_hip import ops
+    g = torch.Generator().manual_seed(700)
+    n, k = 300, 200
+    a1, b1, a2, b2 = (torch.randn(m, generator=g).cuda() * s for m, s in ((n, 3.0), (k, 0.01), (n, 1e-3), (k, 50.0)))
+    t, u = ops.rank_one_operands(n, k, (a1, b1), (a2, b2))
+    got = t.double() @ u.double().T
+    want = torch.outer(a1.double(), b1.double()) + torch.outer(a2.double(), b2.double())
+    assert rel_fro(got.cpu(), want.cpu()) <= 2e-7
+    t, u = ops.rank_one_operands(n, k, (a1, b1))
+    assert rel_fro((t.double() @ u.double().T).cpu(), torch.outer(a1.double(), b1.double()).cpu()) <= 2e-7
+    assert int((t[:, 6:] != 0).sum()) == 0 and int((u[:, 6:] != 0).sum()) == 0
+    # the affine tail of the matrix-vector product
+    w = (torch.randn(n, 64, generator=g) * 0.1).bfloat16().cuda()
+    p = ops.quantize(w)
+    y = ops.matvec(p, z=a1, beta=7.0)
+    want = ops.dequantize(p, torch.float32).double().sum(dim=1) + 7.0 * a1.double()
+    assert rel_fro(y.cpu().double(), want.cpu()) <= 1e-6
