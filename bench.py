@@ -296,6 +296,31 @@ def main():
                    "us_per_step": round(qat_ms * 1e3, 1), "tflops": round(3 * 2.0 * 4096 * 1536 * 8960 / (qat_ms * 1e-3) / 1e12, 1)}
         except Exception as exc:  # an optional leg must not cost the headline line
             qat = {"workload": "config 4 projection", "error": f"{type(exc).__name__}: {exc}"[:300]}
+        # the same projection under the reference's default arguments: mean mode for activations and gradients
+        try:
+            from metis_hip import BitLinear
+            mean_args = MetisArgs(cache_quantized_weight=True)
+            mean_args.enable_forward_svd = False
+            mlin = BitLinear(1536, 8960, args=mean_args, bias=False, dtype=torch.bfloat16, compute_dtype=torch.float32).to(dev).warmup_linear
+
+            def mean_step(ev):
+                if ev is not None:
+                    ev[0].record()
+                y_ = mlin(xq_)
+                y_.backward(dy_.to(y_.dtype))
+                if ev is not None:
+                    ev[1].record()
+                mlin.weight.grad = None
+                xq_.grad = None
+            _, mean_ms = time_region(torch, mean_step, 10, 3)
+            qat["mean_mode"] = {"workload": "same projection, metis_mode=mean for activations and output gradients (column "
+                                            "mean + centred NVFP4 residual, rank-one terms inside the GEMMs)",
+                                "us_per_step": round(mean_ms * 1e3, 1)}
+            LinearLowbitFunction.enable_activation_svd = False     # class-level switches: back to the direct mode
+            LinearLowbitFunction.enable_backward_svd = False
+        except Exception as exc:
+            if isinstance(qat, dict):
+                qat["mean_mode"] = {"error": f"{type(exc).__name__}: {exc}"[:300]}
 
     # ------------------------------------------------------------------ a tile-starved shape: 1024-token prefill
     # through the Qwen2.5-7B down projection (56 output tiles on 256 CUs; K split through a workspace)

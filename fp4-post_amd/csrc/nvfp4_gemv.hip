@@ -16,71 +16,96 @@ typedef float float2_t __attribute__((ext_vector_type(2)));
 // out32 (optional): y as binary32.  split (optional): y as three bf16 terms hi + mid + lo (exact to binary32
 // precision) in columns split_col .. split_col + 2 of a bf16 matrix with row stride split_ld: the form in which a
 // rank-one term enters the low-rank extension of the GEMM.
+// A wave owns R consecutive rows and walks the blocks of 16 columns lane by lane; the 16 values of v a lane
+// needs for a block are loaded once and used for all R rows (R = 4 for tall matrices: a quarter of the L1 traffic).
+__device__ __forceinline__ float block_dot(const uint2 c, const float (&w)[kBlock])
+{
+    float part = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float2_t lo = j == 0 ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 0)
+                          : j == 1 ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 1)
+                          : j == 2 ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 2)
+                                   : __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 3);
+        const float2_t hi = j == 0 ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 0)
+                          : j == 1 ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 1)
+                          : j == 2 ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 2)
+                                   : __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 3);
+        part = fmaf(lo[0], w[2 * j], part);
+        part = fmaf(lo[1], w[2 * j + 1], part);
+        part = fmaf(hi[0], w[8 + 2 * j], part);
+        part = fmaf(hi[1], w[8 + 2 * j + 1], part);
+    }
+    return part;
+}
+
+// R = 0: four rows per WORKGROUP, its four waves interleaved over the blocks (few, long rows).
+template <int R>
 __global__ __launch_bounds__(256) void packed_gemv_kernel(const uint2* __restrict__ codes, const uint8_t* __restrict__ scales,
                                                           const float* __restrict__ unit, uint32_t rows, uint32_t nblocks_row,
                                                           const float* __restrict__ v, float alpha, float* __restrict__ out32,
                                                           uint16_t* __restrict__ split, int64_t split_ld, int split_col,
                                                           const float* __restrict__ z, float beta)
 {
-    const uint32_t lane = threadIdx.x & 63u;
-    const uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6);
-    if (row >= rows) return;
-    const uint2* crow = codes + (size_t)row * nblocks_row;
-    const uint8_t* srow = scales + (size_t)row * nblocks_row;
-    float acc = 0.0f;
-    for (uint32_t b = lane; b < nblocks_row; b += 64u) {
-        const uint2 c = crow[b];
-        const float sc = __builtin_amdgcn_cvt_f32_fp8((int)srow[b], 0);
-        float part = 0.0f;
+    constexpr int RR = R ? R : 4;                               // rows per wave (R == 0: per workgroup)
+    __shared__ float wave_part[4][4];
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t row0 = R ? (blockIdx.x * 4u + wave) * R : blockIdx.x * 4u;
+    if (row0 >= rows) return;                                   // uniform per workgroup when R == 0
+    float acc[RR];
+#pragma unroll
+    for (int r = 0; r < RR; ++r) acc[r] = 0.0f;
+    for (uint32_t b = R ? lane : threadIdx.x; b < nblocks_row; b += R ? 64u : 256u) {
+        float w[kBlock];
         if (v) {
             const float4* vp = reinterpret_cast<const float4*>(v + (size_t)b * kBlock);
-            const float4 v0 = vp[0], v1 = vp[1], v2 = vp[2], v3 = vp[3];
-            const float w[kBlock] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w, v2.x, v2.y, v2.z, v2.w, v3.x, v3.y, v3.z, v3.w};
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const float2_t lo = j == 0 ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 0)
-                                  : j == 1 ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 1)
-                                  : j == 2 ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 2)
-                                           : __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 3);
-                const float2_t hi = j == 0 ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 0)
-                                  : j == 1 ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 1)
-                                  : j == 2 ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 2)
-                                           : __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 3);
-                part = fmaf(lo[0], w[2 * j], part);
-                part = fmaf(lo[1], w[2 * j + 1], part);
-                part = fmaf(hi[0], w[8 + 2 * j], part);
-                part = fmaf(hi[1], w[8 + 2 * j + 1], part);
+            for (int q = 0; q < 4; ++q) {
+                const float4 f = vp[q];
+                w[4 * q] = f.x; w[4 * q + 1] = f.y; w[4 * q + 2] = f.z; w[4 * q + 3] = f.w;
             }
         } else {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const float2_t lo = j == 0 ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 0)
-                                  : j == 1 ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 1)
-                                  : j == 2 ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 2)
-                                           : __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 3);
-                const float2_t hi = j == 0 ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 0)
-                                  : j == 1 ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 1)
-                                  : j == 2 ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 2)
-                                           : __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 3);
-                part += (lo[0] + lo[1]) + (hi[0] + hi[1]);      // E2M1 values: exact sums
-            }
+            for (int j = 0; j < kBlock; ++j) w[j] = 1.0f;
         }
-        acc = fmaf(part, sc, acc);
+#pragma unroll
+        for (int r = 0; r < RR; ++r) {
+            const uint32_t row = min(row0 + r, rows - 1);
+            const uint2 c = codes[(size_t)row * nblocks_row + b];
+            const float sc = __builtin_amdgcn_cvt_f32_fp8((int)scales[(size_t)row * nblocks_row + b], 0);
+            acc[r] = fmaf(block_dot(c, w), sc, acc[r]);
+        }
     }
-    acc = wave_sum(acc);
+#pragma unroll
+    for (int r = 0; r < RR; ++r) acc[r] = wave_sum(acc[r]);
+    if (R == 0) {                                               // fold the four waves
+        if (lane == 0) {
+#pragma unroll
+            for (int r = 0; r < RR; ++r) wave_part[wave][r] = acc[r];
+        }
+        __syncthreads();
+        if (wave != 0) return;
+#pragma unroll
+        for (int r = 0; r < RR; ++r) acc[r] = (wave_part[0][r] + wave_part[1][r]) + (wave_part[2][r] + wave_part[3][r]);
+    }
     if (lane == 0) {
-        float y = acc * (*unit) * alpha;
-        if (z) y = fmaf(beta, z[row], y);
-        if (out32) out32[row] = y;
-        if (split) {
-            uint16_t* d = split + (int64_t)row * split_ld + split_col;
-            const uint32_t h = bf16_bits(y);
-            const float r1 = y - __uint_as_float(h << 16);
-            const uint32_t m = bf16_bits(r1);
-            const float r2 = r1 - __uint_as_float(m << 16);
-            d[0] = (uint16_t)h;
-            d[1] = (uint16_t)m;
-            d[2] = (uint16_t)bf16_bits(r2);
+#pragma unroll
+        for (int r = 0; r < RR; ++r) {
+            const uint32_t row = row0 + r;
+            if (row >= rows) break;
+            float y = acc[r] * (*unit) * alpha;
+            if (z) y = fmaf(beta, z[row], y);
+            if (out32) out32[row] = y;
+            if (split) {
+                uint16_t* d = split + (int64_t)row * split_ld + split_col;
+                const uint32_t h = bf16_bits(y);
+                const float r1 = y - __uint_as_float(h << 16);
+                const uint32_t m = bf16_bits(r1);
+                const float r2 = r1 - __uint_as_float(m << 16);
+                d[0] = (uint16_t)h;
+                d[1] = (uint16_t)m;
+                d[2] = (uint16_t)bf16_bits(r2);
+            }
         }
     }
 }
@@ -96,9 +121,19 @@ int packed_gemv(const void* codes, const void* scales, const float* unit, int64_
     if (rows > INT32_MAX || cols / kBlock > INT32_MAX) return METIS_E_ARG;
     if (((uintptr_t)codes % 8) || ((uintptr_t)v % 16) || ((uintptr_t)out32 % 4) || ((uintptr_t)split % 2) || ((uintptr_t)z % 4)) return METIS_E_ARG;
     if (split && (split_col < 0 || split_ld < (int64_t)split_col + 3)) return METIS_E_ARG;
-    hipLaunchKernelGGL(packed_gemv_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, (const uint2*)codes,
-                       (const uint8_t*)scales, unit, (uint32_t)rows, (uint32_t)(cols / kBlock), v, alpha, out32,
-                       (uint16_t*)split, split_ld, split_col, z, beta);
+    // four rows per wave once that still leaves every CU a few workgroups
+    if (rows >= (int64_t)device_cus() * 64)
+        hipLaunchKernelGGL(packed_gemv_kernel<4>, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st, (const uint2*)codes,
+                           (const uint8_t*)scales, unit, (uint32_t)rows, (uint32_t)(cols / kBlock), v, alpha, out32,
+                           (uint16_t*)split, split_ld, split_col, z, beta);
+    else if (rows < (int64_t)device_cus() * 16 && cols >= 4096)    // few long rows: a workgroup per row
+        hipLaunchKernelGGL(packed_gemv_kernel<0>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, (const uint2*)codes,
+                           (const uint8_t*)scales, unit, (uint32_t)rows, (uint32_t)(cols / kBlock), v, alpha, out32,
+                           (uint16_t*)split, split_ld, split_col, z, beta);
+    else
+        hipLaunchKernelGGL(packed_gemv_kernel<1>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, (const uint2*)codes,
+                           (const uint8_t*)scales, unit, (uint32_t)rows, (uint32_t)(cols / kBlock), v, alpha, out32,
+                           (uint16_t*)split, split_ld, split_col, z, beta);
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 

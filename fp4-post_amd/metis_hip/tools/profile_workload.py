@@ -6,7 +6,8 @@ device-to-device copy of known size that calibrates the FETCH_SIZE / WRITE_SIZE 
     rocprofv3 --pmc WRITE_SIZE       -- python3 fp4-post_amd/metis_hip/tools/profile_workload.py
 
 `--extra` adds the other kernels of the library at representative shapes: bf16-arithmetic, stochastic-rounding,
-column-blocked and binary32-input quantizers, the skinny (decode) GEMM and the split-K GEMM with its reduction.
+column-blocked and binary32-input quantizers, the skinny (decode) GEMM, the split-K GEMM with its reduction and
+the kernels of the mean mode.
 
     rocprofv3 --kernel-trace --stats -- python3 fp4-post_amd/metis_hip/tools/profile_workload.py --extra
 """
@@ -57,6 +58,14 @@ def extra(reps: int = 5):
         ops.linear_fwd(p_dec_up, w_up)                                  # skinny: 64 x 18944 x 3584
         ops.linear_fwd(p_dec_down, w_down)                              # skinny: 64 x 3584 x 18944
         ops.linear_fwd(p_pre, w_down)                                   # split-K: 1024 x 3584 x 18944
+        # mean mode: column mean, centred quantizers, packed weight x mean, rank-one operands
+        me = ops.column_mean(x, torch.float32)
+        ops.column_mean(xf, torch.float32)
+        ops.quantize(x, 0, center=me)                                   # binary32 arithmetic: literal element rule
+        ops.quantize(x, 1, center=me.bfloat16())                        # bf16 arithmetic: hardware converter
+        ops.quantize(xf, 0, sr=True, col=True, seed=i, center=me)
+        wm = ops.matvec(w_up, me[:3584])
+        ops.rank_one_operands(18944, 3584, (wm, me[:3584]), (wm, me[:3584]))
     torch.cuda.synchronize()
 
 

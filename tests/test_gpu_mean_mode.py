@@ -71,7 +71,7 @@ def test_centered_quant_own_stream_and_errors():
         ops.quantize(x, 0, center=me[:-1])
 
 
-@pytest.mark.parametrize("rows,cols", [(192, 256), (1000, 48), (3584, 18944), (5, 16)])
+@pytest.mark.parametrize("rows,cols", [(192, 256), (1000, 48), (3584, 18944), (5, 16), (18944, 3584), (16387, 32), (1001, 4096)])
 def test_packed_matvec(rows, cols):
     from metis_hip import ops
     g = torch.Generator().manual_seed(rows + cols)

@@ -105,6 +105,33 @@ def test_mean_activation_path_uses_quantize_dequantize():
         LinearLowbitFunction.svd_quant(x, quant_func=CountingQuant, metis_mode="bogus")
 
 
+@pytest.mark.parametrize("cd", [torch.float32, torch.bfloat16])
+def test_token_mean_of_the_packed_mean_mode_follows_the_reference_bookkeeping(cd):
+    """The helper the packed mean mode uses gives the generic path's mean and cache entries: plain mean and
+    row count for a prefill call, weighted running mean for single-token calls (reference 311-329)."""
+    F = LinearLowbitFunction
+    keep = F.compute_dtype
+    F.compute_dtype = cd
+    try:
+        g = torch.Generator().manual_seed(1)
+        x = (torch.randn(2, 3, 16, generator=g) + 2.0).to(cd)
+        a, b = {}, {}
+        me = F._token_mean(x, mean_cache=a, cache_key="k")
+        F.svd_quant(x, quant_func=Cast2Fp32, metis_mode="mean", mean_cache=b, cache_key="k")
+        assert me.shape == (16,) and me.dtype == cd and a["k"][1] == b["k"][1] == 6
+        torch.testing.assert_close(a["k"][0], b["k"][0])
+        step = (torch.randn(4, 1, 16, generator=g) - 1.0).to(cd)
+        me2 = F._token_mean(step, mean_cache=a, cache_key="k")
+        F.svd_quant(step, quant_func=Cast2Fp32, metis_mode="mean", mean_cache=b, cache_key="k")
+        assert a["k"][1] == b["k"][1] == 10
+        torch.testing.assert_close(a["k"][0], b["k"][0])
+        torch.testing.assert_close(me2, a["k"][0].reshape(-1))
+        # without a cache: the plain mean, nothing stored
+        torch.testing.assert_close(F._token_mean(x.reshape(6, 16)), x.reshape(6, 16).float().mean(dim=0).to(cd))
+    finally:
+        F.compute_dtype = keep
+
+
 def test_identity_quantizers_give_plain_linear_gradients():
     args = SimpleNamespace(device="cpu", cache_quantized_weight=False)
     layer = LinearLowbit(16, 16, bias=True, args=args)
