@@ -64,6 +64,49 @@ __device__ __forceinline__ uint2 encode_rne_p32(const float (&v)[kBlock], float 
     return make_uint2(lo, hi);
 }
 
+// Round-to-nearest, binary32 arithmetic, on binary32 VALUES (inputs that are not bf16 values: a binary32
+// tensor, or a bf16 tensor minus a binary32 centre).  The block-level guards of encode_rne_p32 reason about
+// bf16 inputs and do not apply; here every quotient is tested instead.  div3 is a faithful quotient for any
+// binary32 x (its remainder step is exact), so it is within 1 ulp of RN(x/s); the reference's code can differ
+// from the round-to-nearest-even conversion of div3 only if a decision threshold, or one of the three
+// exceptional quotients next to 2.5, 3.5 and 5, lies within that distance.  Every threshold has zero low 20
+// significand bits, so a quotient whose low 20 bits are within 4 of 0 (mod 2^20) sends the block to the literal
+// sequence: about 1e-4 of blocks.  Quotients below 0.125 encode as 0 and quotients above 5.5 as 7 either way and
+// are never flagged (zeros are common, and every block's maximum has a quotient just below 6).  Checked on the host against the literal sequence on 9e8 cases around every threshold.
+__device__ __forceinline__ uint2 encode_rne_wide(const float (&v)[kBlock], float s)
+{
+    const float rs = __builtin_amdgcn_rcpf(s);                // 1 ulp
+    // the quotients are converted as they are formed (nothing but the two packed words stays live); the rare
+    // flagged block is redone literally afterwards
+    // all in vector integer ops (no compares): magnitudes outside [0.125, 5.5] are clamped to patterns that never flag,
+    // bits 3..19 of (pattern + 4) are zero exactly for a flagged quotient, and the minimum over the block is kept
+    uint32_t lo = 0u, hi = 0u, least = 0xffffffffu;
+    auto quot = [&](int j) {
+        const float q = div3(v[j], s, rs);
+        uint32_t a = __float_as_uint(q) & 0x7fffffffu;
+        a = a < 0x3e000010u ? 0x3e000010u : a;                 // below 0.125: code 0 either way
+        a = a > 0x40b00010u ? 0x40b00010u : a;                 // above 5.5: code 7 (every block maximum sits at 6)
+        const uint32_t m = ((a + 4u) >> 3) & 0x1ffffu;
+        least = m < least ? m : least;
+        return q;
+    };
+    lo = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(lo, quot(0), quot(1), 1.0f, 0);
+    lo = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(lo, quot(2), quot(3), 1.0f, 1);
+    lo = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(lo, quot(4), quot(5), 1.0f, 2);
+    lo = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(lo, quot(6), quot(7), 1.0f, 3);
+    hi = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(hi, quot(8), quot(9), 1.0f, 0);
+    hi = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(hi, quot(10), quot(11), 1.0f, 1);
+    hi = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(hi, quot(12), quot(13), 1.0f, 2);
+    hi = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(hi, quot(14), quot(15), 1.0f, 3);
+    const bool flagged = least == 0u;
+    if (__builtin_amdgcn_ballot_w64(flagged) != 0ull) {        // wave-uniform: a real branch around the long sequence
+        const float none[kBlock] = {};
+        const uint2 lit = encode_literal<0, false>(v, s, none);
+        if (flagged) { lo = lit.x; hi = lit.y; }
+    }
+    return make_uint2(lo, hi);
+}
+
 // Round-to-nearest, every op rounded to bf16.  With q = bf16(RN(|x| / h)) the reference's
 // compress/round/expand sequence is a function of the bf16 value q alone, and over all bf16 q in
 // [0, 13] it equals the round-to-nearest-even conversion onto the E2M1 grid except at q = 5+1ulp,

@@ -24,8 +24,9 @@ namespace metis {
 // ---------------------------------------------------------------------------------------------
 // WIDE (binary32 arithmetic only): the values to encode are binary32 values that need not be bf16 values,
 // because the input tensor is binary32 (in_f32) and/or a binary32 centre is subtracted first.  The short cuts
-// of the bf16 path (div6, div3, the guarded hardware conversion) are proven for bf16 values only, so these
-// instantiations use IEEE divisions and the literal encoder, and park the block maxima as binary32.
+// of the bf16 path (div6, the block-level guards of the hardware conversion) are proven for bf16 values only, so
+// these instantiations take the block scalar by IEEE division, test every quotient before trusting the hardware
+// conversion (encode_rne_wide), and park the block maxima as binary32.
 //
 // center (optional): one value per column, subtracted before anything else: x - center rounded to the
 // arithmetic's dtype, the centred residual of the reference's mean mode (src/Metis/Metis/bitlinear.py:
@@ -116,7 +117,8 @@ __global__ __launch_bounds__(256) void quant_codes_kernel(
         if constexpr (WIDE) {
             static_cast<float*>(ws_amax_v)[i] = am;
             const float sc = block_scalar_ieee(am);
-            codes[i] = (SR && !noise) ? encode_sr_hardware<0, true>(v, sc, seed, offset, i) : encode_literal<0, SR>(v, sc, u);
+            if constexpr (SR) codes[i] = !noise ? encode_sr_hardware<0, true>(v, sc, seed, offset, i) : encode_literal<0, true>(v, sc, u);
+            else codes[i] = encode_rne_wide(v, sc);
         } else {
             ws_amax[i] = (uint16_t)(__float_as_uint(am) >> 16);      // am is a bf16 value
             // caller-supplied noise: the reference's literal sequence; own stream: hardware stochastic rounding
@@ -187,8 +189,9 @@ __global__ __launch_bounds__(256) void quant_codes_col_kernel(
                 gmax = fmaxf(gmax, am);
                 if constexpr (WIDE) {
                     const float sc = block_scalar_ieee(am);
-                    packed = (SR && !noise) ? encode_sr_hardware<0, true>(v, sc, seed, offset, (int64_t)c * nbc + b)
-                                            : encode_literal<0, SR>(v, sc, u);
+                    if constexpr (SR) packed = !noise ? encode_sr_hardware<0, true>(v, sc, seed, offset, (int64_t)c * nbc + b)
+                                                      : encode_literal<0, true>(v, sc, u);
+                    else packed = encode_rne_wide(v, sc);
                 } else {
                     packed = (SR && !noise) ? encode_sr_hardware<MODE>(v, block_scalar<MODE>(am), seed, offset, (int64_t)c * nbc + b)
                                             : encode_block<MODE, SR>(v, block_scalar<MODE>(am), u);

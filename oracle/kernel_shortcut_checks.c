@@ -15,6 +15,11 @@
  *               literal sequence  vs  round-to-nearest-even of div3(x, s), for blocks the kernel's
  *               two guards do not send to the literal path.
  *
+ *   wide ITERS  binary32 arithmetic on binary32 values (not bf16 values): for ITERS block maxima of any
+ *               significand, inputs anywhere below the maximum and the binary32 neighbours of every
+ *               threshold: literal sequence  vs  round-to-nearest-even of div3(x, s), for quotients the
+ *               kernel's per-element test does not send to the literal path.
+ *
  * Exit status 0 and a final line "mismatches 0" mean the shortcut is exact on the domain covered.
  */
 #include <math.h>
@@ -163,6 +168,53 @@ static long check_p32(long iters)
     return bad;
 }
 
+/* ---- binary32 arithmetic on binary32 VALUES (inputs that are not bf16 values): the block-level guards above do not
+ * apply, the kernel tests every quotient instead: a quotient within 4 ulp of a value whose low 20 significand bits
+ * are zero (every decision threshold is such a value) sends the block to the literal path. */
+static int quotient_hazard(float q)
+{
+    uint32_t a = f_bits(q) & 0x7fffffffu;
+    if (a < 0x3e000010u) a = 0x3e000010u;                         /* below 0.125 the code is 0 either way */
+    if (a > 0x40b00010u) a = 0x40b00010u;                         /* above 5.5 it is 7 (every block maximum sits at 6) */
+    return ((a + 4u) & 0xfffffu) < 8u;
+}
+static long check_wide(long iters)
+{
+    static const float W[7] = {0.25f, 0.75f, 1.25f, 1.75f, 2.5f, 3.5f, 5.0f};
+    long n = 0, bad = 0, guarded = 0;
+#pragma omp parallel for reduction(+ : n, bad, guarded) schedule(dynamic, 1024)
+    for (long it = 0; it < iters; ++it) {
+        unsigned seed = 99991u + 104729u * (unsigned)it + (unsigned)(it >> 18);
+        const uint32_t r1 = rand_r(&seed), r2 = rand_r(&seed), r3 = rand_r(&seed), r4 = rand_r(&seed);
+        /* a binary32 block maximum of any significand, and its scalar */
+        const float amax = bits_f(((uint32_t)(90 + r2 % 70) << 23) | ((r1 ^ (r3 << 9)) & 0x7fffff));
+        const float s = amax / 6.0f + 1e-9f;
+        const float rs0 = 1.0f / s;
+        for (int k = 0; k < 24; ++k) {
+            float x;
+            if (k < 8) {                                           /* anywhere below the maximum */
+                const uint32_t rr = rand_r(&seed);
+                x = amax * ((float)(rr & 0xffffff) / 16777216.0f);
+            } else if (k < 22) {                                   /* binary32 neighbours of threshold * s */
+                const float c = W[(k - 8) % 7] * s;
+                x = bits_f(f_bits(c) + (int)(r4 >> (k - 8) & 15) - 8);
+            } else {
+                x = k == 22 ? amax : bits_f(f_bits(amax) - 1u);
+            }
+            if (!(x <= amax)) continue;
+            const int want = literal_p32(x, s);
+            for (int pert = -1; pert <= 1; ++pert) {
+                const float q = div3(x, s, bits_f(f_bits(rs0) + pert));
+                if (quotient_hazard(q)) { guarded++; continue; }
+                n++;
+                if (rne_grid(2.0f * q) != want) bad++;
+            }
+        }
+    }
+    printf("wide: cases %ld (quotients sent to the literal path: %ld) mismatches %ld\n", n, guarded, bad);
+    return bad;
+}
+
 static long check_div6(void)
 {
     long n = 0, bad = 0;
@@ -182,6 +234,7 @@ int main(int argc, char** argv)
     if (argc >= 2 && !strcmp(argv[1], "div6")) return check_div6() ? 1 : 0;
     if (argc >= 2 && !strcmp(argv[1], "pb16")) return check_pb16() ? 1 : 0;
     if (argc >= 3 && !strcmp(argv[1], "p32")) return check_p32(atol(argv[2])) ? 1 : 0;
-    fprintf(stderr, "usage: %s div6 | pb16 | p32 ITERS\n", argv[0]);
+    if (argc >= 3 && !strcmp(argv[1], "wide")) return check_wide(atol(argv[2])) ? 1 : 0;
+    fprintf(stderr, "usage: %s div6 | pb16 | p32 ITERS | wide ITERS\n", argv[0]);
     return 2;
 }

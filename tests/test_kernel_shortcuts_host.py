@@ -42,6 +42,14 @@ def test_binary32_mode_shortcut_is_exact_outside_its_guards():
     assert 0 < guarded < 2_000_000 // 4            # the guards fire, but mostly on the adversarial families
 
 
+def test_binary32_values_shortcut_is_exact_outside_its_per_quotient_test():
+    """Inputs that are not bf16 values (binary32 tensors, centred residuals): div3 + round-to-nearest-even
+    against the literal sequence for every quotient the kernel's low-bits test does not flag."""
+    text = _run("wide", "3000000")
+    assert int(text.split("cases")[1].split()[0]) > 100_000_000
+    assert int(text.split("literal path:")[1].split(")")[0]) > 0
+
+
 def test_bf16_mode_reference_differs_from_rne_at_exactly_three_quotients():
     """Pins the three constants of the device code against the op-for-op torch restatement: over every
     bf16 q in [0, 13] compress/round (quant.py:28-31 in bf16) equals round-to-nearest-even onto the grid
