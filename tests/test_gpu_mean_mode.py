@@ -268,3 +268,58 @@ def test_rank_one_operands_reach_binary32_precision():
     y = ops.matvec(p, z=a1, beta=7.0)
     want = ops.dequantize(p, torch.float32).double().sum(dim=1) + 7.0 * a1.double()
     assert rel_fro(y.cpu().double(), want.cpu()) <= 1e-6
+
+
+def test_qwen2_decoder_layer_under_the_reference_default_arguments(monkeypatch):
+    """A Hugging Face Qwen2 decoder layer patched with MetisArgs() as the reference constructs it (mean mode for
+    activations and output gradients): every projection runs on the packed kernels, and the result stays close to
+    the same layer evaluated on dequantized tensors and torch matmuls (the generic path)."""
+    pytest.importorskip("transformers")
+    from transformers.models.qwen2.modeling_qwen2 import Qwen2Config, Qwen2DecoderLayer, Qwen2RotaryEmbedding
+    from metis_hip import BitLinear, LinearLowbitFunction as F, MetisArgs, ops, replace_model_with_metis
+    torch.manual_seed(0)
+    cfg = Qwen2Config(hidden_size=256, intermediate_size=512, num_attention_heads=4, num_key_value_heads=2,
+                      num_hidden_layers=1, vocab_size=128, max_position_embeddings=256)
+    cfg._attn_implementation = "eager"
+    layer = Qwen2DecoderLayer(cfg, layer_idx=0).to(torch.bfloat16).cuda()
+    for p in layer.parameters():
+        if p.dim() == 2:
+            torch.nn.init.normal_(p, std=0.02)
+    holder = torch.nn.ModuleDict({"layer": layer})
+    x = (torch.randn(2, 64, 256, device="cuda") + 1.5 * torch.randn(1, 1, 256, device="cuda")).bfloat16()
+    pos = torch.arange(64, device="cuda").unsqueeze(0).expand(2, -1)
+    pe = Qwen2RotaryEmbedding(cfg).cuda()(x, pos)
+
+    def run(inp):
+        out = holder["layer"](inp, position_embeddings=pe, attention_mask=None, position_ids=pos)
+        return out[0] if isinstance(out, tuple) else out
+
+    args = MetisArgs(forward_svd_rank=32)
+    assert args.metis_mode == "mean" and args.enable_activation_svd and args.enable_backward_svd
+    replace_model_with_metis(holder, args)
+    assert sum(isinstance(m, BitLinear) and m.is_svd_quant for m in holder.modules()) == 7
+    centred = []
+    real = ops.quantize
+    monkeypatch.setattr(ops, "quantize", lambda *a, **k: (centred.append(k.get("center") is not None), real(*a, **k))[1])
+    xr = x.clone().requires_grad_(True)
+    out = run(xr)
+    n_fwd = sum(centred)
+    assert n_fwd == 4                                              # q/k/v share one, o, gate/up share one, down
+    out.float().square().mean().backward()
+    assert sum(centred) > n_fwd                                    # gradients are centred too
+    gx_packed = xr.grad.detach().float().cpu()
+    assert bool(torch.isfinite(gx_packed).all())
+    # generic evaluation of the same modules
+    monkeypatch.setattr(F, "_mean_mode_packable", staticmethod(lambda: False))
+    for m in holder.modules():
+        if isinstance(m, BitLinear):
+            m.mean_cache.clear()
+            if m.activation_group is not None:
+                m.activation_group["mean_cache"].clear()
+    xg = x.clone().requires_grad_(True)
+    ref = run(xg)
+    # not the same formula to the last bit: the fused launch feeds the rank-r branch the raw bf16 activation, the
+    # generic evaluation feeds it the quantized one (both documented variants), so agreement is at FP4-noise level
+    assert rel_fro(out.detach().float().cpu(), ref.detach().float().cpu()) <= 2e-2
+    ref.float().square().mean().backward()
+    assert rel_fro(gx_packed, xg.grad.detach().float().cpu()) < 0.2      # both carry independent stochastic rounding
