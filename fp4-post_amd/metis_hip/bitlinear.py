@@ -556,6 +556,10 @@ class _MetisFusedFunction(torch.autograd.Function):
 class BitLinear(nn.Module):
     """Drop-in for nn.Linear: W = U diag(s) V + W_res with the residual in NVFP4 (reference 597-940)."""
     rollout_merge_active = False
+    # False (default): the rank-r branch sees the raw activation and bf16 V, U, s and is folded into the residual
+    # GEMM's launch.  True: it consumes the quantized activation and the quantized V through their own GEMM, as the
+    # reference's current file does (752, 863-879): two packed GEMMs and a dense rank-r GEMM per call.
+    quantized_lowrank_branch = False
 
     def __init__(self, in_features, out_features, args=None, bias=True, dtype=torch.float32, compute_dtype=None):
         super().__init__()
@@ -661,7 +665,8 @@ class BitLinear(nn.Module):
         if share_activation:
             shared_input = self._get_shared_quantized_input(x)
             r = self.args.forward_svd_rank
-            if isinstance(shared_input, (PackedNVFP4, CenteredNVFP4)) and r % 32 == 0 and self.ulinear.bias is None:
+            if (isinstance(shared_input, (PackedNVFP4, CenteredNVFP4)) and r % 32 == 0 and self.ulinear.bias is None
+                    and not BitLinear.quantized_lowrank_branch):
                 # one fused launch for both branches; it already is the "merged" evaluation, so the
                 # rollout switch changes nothing on this path
                 wl = self.warmup_linear
@@ -685,7 +690,13 @@ class BitLinear(nn.Module):
             F.mean_cache_key = f"{self.layer_name}.vlinear"
             y = self.vlinear(x)
         y = torch.mul(self.s, y)
-        y = self.ulinear(y.to(self.ulinear.weight.dtype))
+        if y.dtype == self.ulinear.weight.dtype:
+            y = self.ulinear(y)
+        else:
+            # the reference builds ulinear without a dtype (binary32, 872-876), so with compute_dtype=float32 this
+            # matmul runs in binary32; here U is stored in the layer's dtype and widened for the product
+            ub = self.ulinear.bias
+            y = torch.nn.functional.linear(y, self.ulinear.weight.to(y.dtype), None if ub is None else ub.to(y.dtype))
         if self.args.forward_svd_rank > 0:
             if share_activation:
                 y = y + self.warmup_linear(x, quantized_input=shared_input)

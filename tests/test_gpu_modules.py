@@ -132,6 +132,24 @@ def test_bitlinear_fused_forward_against_oracle(bias):
     assert rel_fro(y.detach().cpu().reshape(L, N).float(), dense) < 0.05
 
 
+def test_bitlinear_quantized_lowrank_branch_switch(monkeypatch):
+    """BitLinear.quantized_lowrank_branch = True evaluates the reference's current formula, rank-r branch on
+    Q(x) and Q(V) (bitlinear.py:752, 863-879), still on packed operands: <= 2e-3 against the oracle's variant."""
+    from metis_hip import BitLinear
+    from oracle import metis_oracle as O
+    K, N, r, L = 256, 192, 32, 128
+    layer, w = _make_bitlinear(K, N, r, True, torch.bfloat16, torch.float32)
+    monkeypatch.setattr(BitLinear, "quantized_lowrank_branch", True)
+    x = synthetic_activation(50, L, K).reshape(2, L // 2, K)
+    y = layer(x.cuda())
+    want = O.metis_forward(x.reshape(L, K), layer.vlinear.weight.detach().cpu(), layer.s.detach().cpu(),
+                           layer.ulinear.weight.detach().cpu(), layer.warmup_linear.weight.detach().cpu(),
+                           layer.warmup_linear.bias.detach().cpu(), p32=True, quantized_lowrank=True)
+    assert rel_fro(y.detach().cpu().reshape(L, N).bfloat16(), want) <= TOL
+    y.float().square().mean().backward()
+    assert layer.vlinear.weight.grad is not None and layer.warmup_linear.weight.grad is not None
+
+
 def test_bitlinear_fused_forward_bf16_compute():
     """compute_dtype=bfloat16: operands are packed with the bf16-per-op arithmetic (bit-exact codes,
     see test_gpu_quant); the GEMM keeps exact products and fp32 accumulation, so against the
