@@ -160,6 +160,15 @@ int metis_column_mean(const void* x, int64_t rows, int64_t cols, int64_t ld, int
                        workspace_bytes, (hipStream_t)stream);
 }
 
+int metis_column_sum(const void* x, int64_t rows, int64_t cols, int64_t ld, int x_dtype, void* out, int out_dtype,
+                     void* workspace, size_t workspace_bytes, void* stream)
+{
+    if ((x_dtype != METIS_DTYPE_BF16 && x_dtype != METIS_DTYPE_F32) || (out_dtype != METIS_DTYPE_BF16 && out_dtype != METIS_DTYPE_F32))
+        return METIS_E_ARG;
+    return column_mean(x, rows, cols, ld, x_dtype == METIS_DTYPE_F32, out, out_dtype == METIS_DTYPE_BF16, workspace,
+                       workspace_bytes, (hipStream_t)stream, true);
+}
+
 int metis_nvfp4_matvec(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols,
                        const float* v, float alpha, float* out, void* split, int64_t split_ld, int split_col, void* stream)
 {

@@ -72,7 +72,7 @@ size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 // me[c] = mean over rows of x[:, c] (binary32 accumulation); nvfp4_gemv.hip
 size_t column_mean_workspace_bytes(int64_t cols);
 int column_mean(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_f32, void* out, int out_bf16, void* workspace,
-                size_t workspace_bytes, hipStream_t st);
+                size_t workspace_bytes, hipStream_t st, bool sum_only = false);
 
 int expand_f16(const void* codes, const void* scales, int64_t rows, int64_t cols, void* out, hipStream_t st);
 int gemm_expanded(const void* a_exp, const float* a_unit, const void* b_exp, const float* b_unit, int64_t M, int64_t N,

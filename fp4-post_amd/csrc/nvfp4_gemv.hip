@@ -254,7 +254,7 @@ __global__ __launch_bounds__(64) void column_mean_finish_kernel(const float* __r
 size_t column_mean_workspace_bytes(int64_t cols) { return cols > 0 ? (size_t)kMeanMaxSlabs * (size_t)cols * sizeof(float) : 0; }
 
 int column_mean(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_f32, void* out, int out_bf16, void* workspace,
-                size_t workspace_bytes, hipStream_t st)
+                size_t workspace_bytes, hipStream_t st, bool sum_only)
 {
     if (rows <= 0 || cols <= 0 || ld < cols) return METIS_E_ARG;
     if (cols % 4 || ld % 4) return METIS_E_SHAPE;
@@ -278,9 +278,9 @@ int column_mean(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_f3
         hipLaunchKernelGGL(column_sum_kernel<false>, grid, dim3(256), 0, st, x, (uint32_t)rows, (uint32_t)cols, ld, partial, rows_per_slab);
     const dim3 g2((unsigned)((cols + 63) / 64));
     if (out_bf16)
-        hipLaunchKernelGGL(column_mean_finish_kernel<true>, g2, dim3(64), 0, st, partial, (uint32_t)slabs, (uint32_t)cols, (float)rows, out);
+        hipLaunchKernelGGL(column_mean_finish_kernel<true>, g2, dim3(64), 0, st, partial, (uint32_t)slabs, (uint32_t)cols, sum_only ? 1.0f : (float)rows, out);
     else
-        hipLaunchKernelGGL(column_mean_finish_kernel<false>, g2, dim3(64), 0, st, partial, (uint32_t)slabs, (uint32_t)cols, (float)rows, out);
+        hipLaunchKernelGGL(column_mean_finish_kernel<false>, g2, dim3(64), 0, st, partial, (uint32_t)slabs, (uint32_t)cols, sum_only ? 1.0f : (float)rows, out);
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 

@@ -44,6 +44,16 @@ def _packable(x: torch.Tensor, q) -> bool:
     return is_hip_nvfp4(q) and x.is_cuda and x.shape[-1] % 32 == 0 and x.dtype in (torch.float32, torch.bfloat16)
 
 
+def _token_sum(flat: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """Sum over tokens of a [L, N] gradient with the result in `dtype` (the bias gradient, reference 455): one pass of the
+    library's column reduction on the device, torch elsewhere."""
+    if flat.is_cuda and flat.dtype in (torch.float32, torch.bfloat16) and dtype in (torch.float32, torch.bfloat16) \
+            and flat.shape[1] % 4 == 0 and flat.shape[0] > 0:
+        src = flat if (dtype == torch.float32 or flat.dtype == torch.bfloat16) else flat.to(dtype)
+        return ops.column_sum(src, out_dtype=dtype)
+    return flat.to(dtype).sum(dim=0)
+
+
 class LinearLowbitFunction(torch.autograd.Function):
     """Low-bit GEMM with quantized activations / weights / gradients (reference 18-513).
 
@@ -367,7 +377,7 @@ class LinearLowbitFunction(torch.autograd.Function):
         F = LinearLowbitFunction
         grad_bias = None
         if ctx.has_bias:
-            grad_bias = _flat2d(grad_output).to(F.compute_dtype).sum(dim=0).to(torch.float32)
+            grad_bias = _token_sum(_flat2d(grad_output), F.compute_dtype).to(torch.float32)
         if ctx.packed:
             input_, _ = ctx.saved_tensors
             L, N = _flat2d(grad_output).shape
@@ -548,7 +558,7 @@ class _MetisFusedFunction(torch.autograd.Function):
             wq = F.q_forward_weight.quantize_dequantize(res.to(F.compute_dtype))
             gx = gx + torch.matmul(dyq, wq).to(cd)
             g_res = torch.matmul(dyq.T, xq).to(torch.float32)
-        g_b = dy2.float().sum(dim=0) if ctx.has_bias else None
+        g_b = _token_sum(dy2, torch.float32) if ctx.has_bias else None
         return (gx.reshape(x.shape).to(x.dtype), g_v.to(v.dtype), g_s.to(s.dtype), g_u.to(u.dtype),
                 g_res, g_b, None, None)
 

@@ -158,7 +158,12 @@ def dequantize(p: PackedNVFP4, dtype: torch.dtype = torch.bfloat16) -> torch.Ten
     return out
 
 
-def column_mean(x: torch.Tensor, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+def column_sum(x: torch.Tensor, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """Sum over the rows of x flattened to [R, C] -> [C] (binary32 accumulation; bf16 or float32 in and out)."""
+    return column_mean(x, out_dtype, _sum_only=True)
+
+
+def column_mean(x: torch.Tensor, out_dtype: torch.dtype = torch.float32, _sum_only: bool = False) -> torch.Tensor:
     """Mean over the rows of x flattened to [R, C] -> [C] (binary32 accumulation; bf16 or float32 in and out)."""
     if not x.is_cuda:
         raise _lib.MetisHipError("metis_hip ops need a ROCm device tensor; there is no CPU path")
@@ -171,10 +176,10 @@ def column_mean(x: torch.Tensor, out_dtype: torch.dtype = torch.float32) -> torc
     out = torch.empty(cols, dtype=out_dtype, device=x2.device)
     L = load()
     ws = torch.empty(L.metis_column_mean_workspace_bytes(cols), dtype=torch.uint8, device=x2.device)
-    rc = L.metis_column_mean(x2.data_ptr(), rows, cols, x2.stride(0), DTYPE_F32 if x2.dtype == torch.float32 else DTYPE_BF16,
-                             out.data_ptr(), DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16, ws.data_ptr(),
-                             ws.numel(), _stream())
-    check(rc, "metis_column_mean", x.shape)
+    fn = L.metis_column_sum if _sum_only else L.metis_column_mean
+    rc = fn(x2.data_ptr(), rows, cols, x2.stride(0), DTYPE_F32 if x2.dtype == torch.float32 else DTYPE_BF16,
+            out.data_ptr(), DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16, ws.data_ptr(), ws.numel(), _stream())
+    check(rc, "metis_column_sum" if _sum_only else "metis_column_mean", x.shape)
     return out
 
 

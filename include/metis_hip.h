@@ -273,6 +273,10 @@ int metis_nvfp4_quant_centered(const void *x, int64_t rows, int64_t cols, int64_
 size_t metis_column_mean_workspace_bytes(int64_t cols);
 int metis_column_mean(const void *x, int64_t rows, int64_t cols, int64_t ld, int x_dtype, void *out,
                       int out_dtype, void *workspace, size_t workspace_bytes, void *stream);
+/* Same reduction without the division: out[c] = sum_r x[r, c], the bias gradient grad_output.sum(dim=(0, 1))
+ * of LinearLowbitFunction.backward (src/Metis/Metis/bitlinear.py:455).  Same arguments and workspace. */
+int metis_column_sum(const void *x, int64_t rows, int64_t cols, int64_t ld, int x_dtype, void *out,
+                     int out_dtype, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
  * y[i] = alpha * sum_k deq(P)[i, k] * v[k] for a packed [rows, cols] tensor P, binary32 accumulation.

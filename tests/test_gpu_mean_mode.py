@@ -239,6 +239,8 @@ def test_column_mean(rows, cols, dtype):
     want = x.double().mean(dim=0)
     got32 = ops.column_mean(x.cuda(), torch.float32).cpu()
     assert float((got32.double() - want).abs().max()) <= 1e-6 * float(want.abs().max() + 1)
+    total = ops.column_sum(x.cuda(), torch.float32).cpu()
+    assert float((total.double() - want * rows).abs().max()) <= 2e-6 * float((want * rows).abs().max() + rows)
     got16 = ops.column_mean(x.cuda(), torch.bfloat16).cpu()
     assert got16.dtype == torch.bfloat16 and float((got16.double() - want).abs().max()) <= 2 ** -8 * float(want.abs().max() + 1)
     # a strided view (row stride > cols)
