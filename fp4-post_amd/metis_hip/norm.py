@@ -37,7 +37,11 @@ class _NormedWithGrad(torch.autograd.Function):
         xf, gf = x.float(), g.float()
         rstd = torch.rsqrt(xf.pow(2).mean(dim=-1, keepdim=True) + ctx.eps)
         xhat = xf * rstd
-        g_weight = (gf * xhat.to(x.dtype).float()).reshape(-1, x.shape[-1]).sum(dim=0).to(weight.dtype)
+        prod = (gf * xhat.to(x.dtype).float()).reshape(-1, x.shape[-1])
+        if prod.is_cuda and prod.shape[1] % 4 == 0:
+            g_weight = ops.column_sum(prod, torch.float32).to(weight.dtype)     # torch's reduction over dim 0 is ~8x slower
+        else:
+            g_weight = prod.sum(dim=0).to(weight.dtype)
         gh = gf * weight.float()
         g_x = (rstd * (gh - xhat * (gh * xhat).mean(dim=-1, keepdim=True))).to(x.dtype)
         return g_x, g_weight, None, None
