@@ -280,7 +280,7 @@ class LinearLowbitFunction(torch.autograd.Function):
         return F.quantize_input(input_, mean_cache=mean_cache, cache_key=cache_key)
 
     @staticmethod
-    def _packed_grads(dy2, x2, pw_col, center_x, gx_dtype, gw_dtype):
+    def _packed_grads(dy2, x2, pw_col, center_x, gx_dtype, gw_dtype, gx_lowrank=None):
         """(grad_input [L, K], grad_weight [N, K]) on packed operands.  dgrad contracts over N, wgrad over tokens.
 
         Direct mode: dY^ = SR-Q(dY).  Mean mode (enable_backward_svd): dY^ = 1 me_dy^T + SR-Q(dY - me_dy)
@@ -289,16 +289,19 @@ class LinearLowbitFunction(torch.autograd.Function):
         rank-one terms:
             gX = R_dy W^ + 1 (W^^T me_dy)^T
             gW = R_dy^T R_x + (sum_l R_dy) center_x^T + me_dy (sum_l R_x + L center_x)^T
+        gx_lowrank = (t [L, r], u [K, r]) adds t u^T to grad_input inside the same launch (the rank-r branch's share).
         """
         F = LinearLowbitFunction
         cd = F.compute_dtype
         qg, qi = F.q_backward_outputgrad, F.q_backward_input
         me_dy = F._token_mean(dy2) if F.enable_backward_svd else None
         p_dy = qg.pack(dy2, arith=cd, center=me_dy)
-        if me_dy is None:
+        if me_dy is None and gx_lowrank is None:
             gx = ops.linear_dgrad(p_dy, pw_col, out_dtype=gx_dtype)
         else:
-            gx = ops.linear_fwd(p_dy, pw_col, bias=ops.matvec(pw_col, me_dy), out_dtype=gx_dtype)
+            lt, lu = gx_lowrank if gx_lowrank is not None else (None, None)
+            gx = ops.linear_fwd(p_dy, pw_col, t=lt, u=lu, bias=None if me_dy is None else ops.matvec(pw_col, me_dy),
+                                out_dtype=gx_dtype)
         p_dyt = qg.pack(dy2, col=True, arith=cd, center=me_dy)
         p_xt = qi.pack(x2, col=True, arith=cd, center=center_x)
         if me_dy is None and center_x is None:
@@ -530,7 +533,6 @@ class _MetisFusedFunction(torch.autograd.Function):
         g_s = (g_t.float() * xv.float()).sum(dim=0)
         g_xv = g_t * s.to(cd)
         g_v = torch.matmul(g_xv.T, x2)                         # [r, K]
-        gx = torch.matmul(g_xv, v.to(cd))                      # [L, K]
         # residual branch on re-quantized operands
         qg = F.q_backward_outputgrad
         if F._packed_backward_applies(L, N, dy2):
@@ -540,10 +542,12 @@ class _MetisFusedFunction(torch.autograd.Function):
                 p_res_col = ctx.p_res.transposed = F.q_forward_weight.pack(res, col=True, arith=ar)
             # binary32 arithmetic quantizes the tensors autograd handed over, not their bf16 roundings
             dyq, xq_src = (_flat2d(dy), _flat2d(x)) if ar == torch.float32 else (dy2, x2)
-            g_res_gx, g_res = F._packed_grads(dyq, xq_src, p_res_col, ctx.center, cd,
-                                              torch.bfloat16 if res.dtype == torch.bfloat16 else torch.float32)
-            gx = gx + g_res_gx
+            # the rank-r branch's share of grad_input, g_xv V, rides in the dgrad launch as its low-rank extension
+            gx, g_res = F._packed_grads(dyq, xq_src, p_res_col, ctx.center, cd,
+                                        torch.bfloat16 if res.dtype == torch.bfloat16 else torch.float32,
+                                        gx_lowrank=(g_xv, v.to(cd).T.contiguous()))
         else:
+            gx = torch.matmul(g_xv, v.to(cd))                  # [L, K]
             cdt = F.compute_dtype
             if F.enable_backward_svd:
                 dyq = _flat2d(F.svd_quant(dy2.to(cdt), quant_func=qg, rank=F.backward_lowrank_svd, niter=F.backward_lowrank_niter,
