@@ -197,6 +197,14 @@ int metis_linear_fwd_f32bias(const void* a_codes, const void* a_scales, const fl
                       (hipStream_t)stream, workspace, workspace_bytes, 1);
 }
 
+int metis_linear_fwd_grouped(const void* a_codes, const void* a_scales, const float* a_unit, int64_t M, int64_t K,
+                             const metis_linear_member* members, int count, int out_dtype, void* stream)
+{
+    static_assert(sizeof(metis_linear_member) == sizeof(GemmMember), "member layouts must agree");
+    return gemm_nvfp4_grouped(a_codes, a_scales, a_unit, M, K, reinterpret_cast<const GemmMember*>(members), count, out_dtype,
+                              (hipStream_t)stream);
+}
+
 size_t metis_linear_workspace_bytes(int64_t M, int64_t N, int64_t K) { return gemm_workspace_bytes(M, N, K); }
 
 int metis_linear_fwd_ws(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes,

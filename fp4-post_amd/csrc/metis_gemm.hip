@@ -732,15 +732,15 @@ __device__ __forceinline__ half8_t run_operand(const RunRegs<C>& r, int m)
 }
 
 template <int TM, int C, int WAVES, int OUT_F32>
-__global__ __launch_bounds__(64 * WAVES) void gemm_nvfp4_skinny_kernel(
+__device__ __forceinline__ void skinny_tile(
     const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const float* __restrict__ a_unit,
     const uint8_t* __restrict__ b_codes, const uint8_t* __restrict__ b_scales, const float* __restrict__ b_unit,
     int M, int N, int K, const uint16_t* __restrict__ t, const uint16_t* __restrict__ u, int r,
-    const uint16_t* __restrict__ bias, void* __restrict__ out, int bias_f32)
+    const uint16_t* __restrict__ bias, void* __restrict__ out, int bias_f32, int n0)
 {
     __shared__ float red[WAVES][TM * 16][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, hi = lane >> 5;
-    const int n0 = blockIdx.x * 32, m0 = blockIdx.y * 32 * TM;
+    const int m0 = blockIdx.y * 32 * TM;
     const int kbytes = K / 2, kblocks = K / kBlock;
     const int nrow = min(n0 + (lane & 31), N - 1);
     const uint8_t* bc = b_codes + (int64_t)nrow * kbytes + hi * 16 * C;
@@ -823,6 +823,55 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nvfp4_skinny_kernel(
     }
 }
 
+template <int TM, int C, int WAVES, int OUT_F32>
+__global__ __launch_bounds__(64 * WAVES) void gemm_nvfp4_skinny_kernel(
+    const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const float* __restrict__ a_unit,
+    const uint8_t* __restrict__ b_codes, const uint8_t* __restrict__ b_scales, const float* __restrict__ b_unit,
+    int M, int N, int K, const uint16_t* __restrict__ t, const uint16_t* __restrict__ u, int r,
+    const uint16_t* __restrict__ bias, void* __restrict__ out, int bias_f32)
+{
+    skinny_tile<TM, C, WAVES, OUT_F32>(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, bias_f32,
+                                       (int)blockIdx.x * 32);
+}
+
+// Several weight matrices against ONE packed activation in one launch (q/k/v, gate/up): the column tiles of the
+// members are laid end to end along grid x.  A decode-sized k or v projection alone is 16 workgroups and costs a
+// whole launch latency; next to q it is free.
+constexpr int kMaxGroupMembers = 4;
+struct SkinnyMember {
+    const uint8_t* b_codes;
+    const uint8_t* b_scales;
+    const float* b_unit;
+    const uint16_t* t;
+    const uint16_t* u;
+    const uint16_t* bias;
+    void* out;
+    int N, r, tile_end, bias_f32;
+};
+struct SkinnyGroup {
+    SkinnyMember m[kMaxGroupMembers];
+    int count;
+};
+
+template <int TM, int C, int WAVES, int OUT_F32>
+__global__ __launch_bounds__(64 * WAVES) void gemm_nvfp4_skinny_grouped_kernel(
+    const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const float* __restrict__ a_unit, int M, int K,
+    const SkinnyGroup grp)
+{
+    const int tile = (int)blockIdx.x;
+    int g = 0, start = 0;
+#pragma unroll
+    for (int i = 0; i + 1 < kMaxGroupMembers; ++i)
+        if (i + 1 < grp.count && tile >= grp.m[i].tile_end) { g = i + 1; start = grp.m[i].tile_end; }
+    // select with a uniform chain of compares rather than a dynamic index into the kernel arguments
+    SkinnyMember mm = grp.m[0];
+#pragma unroll
+    for (int i = 1; i < kMaxGroupMembers; ++i)
+        if (g == i) mm = grp.m[i];
+    skinny_tile<TM, C, WAVES, OUT_F32>(a_codes, a_scales, a_unit, mm.b_codes, mm.b_scales, mm.b_unit, M, mm.N, K, mm.t, mm.u, mm.r,
+                                       mm.bias, mm.out, mm.bias_f32, (tile - start) * 32);
+}
+
 template <int TM, int C, int WAVES>
 static int launch_skinny(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes,
                          const void* b_scales, const float* b_unit, int64_t M, int64_t N, int64_t K, const void* t,
@@ -859,6 +908,72 @@ static int gemm_skinny(const void* a_codes, const void* a_scales, const float* a
         if (c == 4) METIS_SKL(2, 4, 8); else METIS_SKL(2, 1, 8);
     }
 #undef METIS_SKL
+}
+
+template <int TM, int C, int WAVES>
+static int launch_skinny_grouped(const void* a_codes, const void* a_scales, const float* a_unit, int64_t M, int64_t K,
+                                 const SkinnyGroup& grp, int tiles, int out_dtype, hipStream_t st)
+{
+    const dim3 grid((unsigned)tiles, (unsigned)((M + 32 * TM - 1) / (32 * TM))), block(64 * WAVES);
+    if (out_dtype == METIS_DTYPE_F32)
+        hipLaunchKernelGGL((gemm_nvfp4_skinny_grouped_kernel<TM, C, WAVES, 1>), grid, block, 0, st, (const uint8_t*)a_codes,
+                           (const uint8_t*)a_scales, a_unit, (int)M, (int)K, grp);
+    else
+        hipLaunchKernelGGL((gemm_nvfp4_skinny_grouped_kernel<TM, C, WAVES, 0>), grid, block, 0, st, (const uint8_t*)a_codes,
+                           (const uint8_t*)a_scales, a_unit, (int)M, (int)K, grp);
+    return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
+}
+
+// One activation against up to four weight matrices.  Shapes the skinny kernel does not take fall back to one
+// gemm_nvfp4 call per member (same results either way).
+int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a_unit, int64_t M, int64_t K,
+                       const GemmMember* members, int count, int out_dtype, hipStream_t st)
+{
+    if (!members || count < 1) return METIS_E_ARG;
+    bool skinny = M > 0 && M < 256 && K % 64 == 0 && count <= kMaxGroupMembers && !getenv("METIS_GEMM_SMALL") &&
+                  a_codes && a_scales && a_unit && !((uintptr_t)a_codes % 16) && !((uintptr_t)a_scales % 2) && K <= INT32_MAX &&
+                  (out_dtype == METIS_DTYPE_BF16 || out_dtype == METIS_DTYPE_F32);
+    bool al8 = ((uintptr_t)a_scales % 8) == 0;
+    int64_t tiles = 0;
+    for (int i = 0; i < count && skinny; ++i) {
+        const GemmMember& g = members[i];
+        if (!g.b_codes || !g.b_scales || !g.b_unit || !g.out || g.N <= 0 || g.N > INT32_MAX || g.N % 4 || g.r < 0 || g.r % 32 ||
+            (g.r > 0 && (!g.t || !g.u)) || ((uintptr_t)g.b_codes % 16) || ((uintptr_t)g.b_scales % 2) || ((uintptr_t)g.out % 16) ||
+            ((uintptr_t)g.t % 16) || ((uintptr_t)g.u % 16) || ((uintptr_t)g.bias % 2))
+            skinny = false;
+        al8 = al8 && ((uintptr_t)g.b_scales % 8) == 0;
+        tiles += (g.N + 31) / 32;
+    }
+    if (!skinny || tiles > INT32_MAX) {
+        for (int i = 0; i < count; ++i) {
+            const GemmMember& g = members[i];
+            const int rc = gemm_nvfp4(a_codes, a_scales, a_unit, g.b_codes, g.b_scales, g.b_unit, M, g.N, K, g.t, g.u, g.r, g.bias,
+                                      g.out, out_dtype, st);
+            if (rc != METIS_OK) return rc;
+        }
+        return METIS_OK;
+    }
+    SkinnyGroup grp = {};
+    grp.count = count;
+    int end = 0;
+    for (int i = 0; i < count; ++i) {
+        const GemmMember& g = members[i];
+        end += (int)((g.N + 31) / 32);
+        grp.m[i] = SkinnyMember{(const uint8_t*)g.b_codes, (const uint8_t*)g.b_scales, g.b_unit, (const uint16_t*)g.t,
+                                (const uint16_t*)g.u, (const uint16_t*)g.bias, g.out, (int)g.N, (int)g.r, end, 0};
+    }
+    // same shape heuristics as gemm_skinny, on the joint column count
+    const int c = (K % 256 == 0 && al8) ? 4 : 1;
+    const int tm = (M <= 32 || tiles < device_cus() / 2) ? 1 : 2;
+    const int waves = (tm == 1 && M <= 32 && tiles >= 2 * device_cus()) ? 4 : 8;
+#define METIS_SKG(TM, C, W) return launch_skinny_grouped<TM, C, W>(a_codes, a_scales, a_unit, M, K, grp, (int)tiles, out_dtype, st)
+    if (tm == 1) {
+        if (waves == 4) { if (c == 4) METIS_SKG(1, 4, 4); else METIS_SKG(1, 1, 4); }
+        else { if (c == 4) METIS_SKG(1, 4, 8); else METIS_SKG(1, 1, 8); }
+    } else {
+        if (c == 4) METIS_SKG(2, 4, 8); else METIS_SKG(2, 1, 8);
+    }
+#undef METIS_SKG
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -66,6 +66,20 @@ int packed_gemv(const void* codes, const void* scales, const float* unit, int64_
 // T [n, 32], U [k, 32] (bf16) with T U^T = a1 b1^T + a2 b2^T to binary32 precision; nvfp4_gemv.hip
 int rank_one_operands(const float* a1, const float* b1, const float* a2, const float* b2, int64_t n, int64_t k, void* T, void* U,
                       hipStream_t st);
+// one weight matrix of a grouped GEMM (layout shared with metis_linear_member of the C ABI)
+struct GemmMember {
+    const void* b_codes;
+    const void* b_scales;
+    const float* b_unit;
+    const void* t;
+    const void* u;
+    int64_t r;
+    const void* bias;
+    void* out;
+    int64_t N;
+};
+int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a_unit, int64_t M, int64_t K,
+                       const GemmMember* members, int count, int out_dtype, hipStream_t st);
 // bytes of split-K scratch gemm_nvfp4 can use for this shape on the current device (0: it would not split)
 size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 

@@ -12,6 +12,13 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmetis_hip.so")
 
 OK, E_ARG, E_SHAPE, E_WORKSPACE, E_LAUNCH, E_DEVICE = 0, -1, -2, -3, -4, -5
+class LinearMember(ctypes.Structure):
+    """metis_linear_member of include/metis_hip.h: one weight matrix of a grouped GEMM."""
+    _fields_ = [("b_codes", ctypes.c_void_p), ("b_scales", ctypes.c_void_p), ("b_unit", ctypes.c_void_p),
+                ("t", ctypes.c_void_p), ("u", ctypes.c_void_p), ("r", ctypes.c_int64), ("bias", ctypes.c_void_p),
+                ("out", ctypes.c_void_p), ("N", ctypes.c_int64)]
+
+
 MODE_P32, MODE_PB16 = 0, 1
 MODE_P32_F32 = 2      # quantizer entry points only: binary32 arithmetic on a binary32 tensor
 DTYPE_BF16, DTYPE_F32 = 0, 1
@@ -46,6 +53,7 @@ SIGNATURES = {
     "metis_column_sum": (_i32, [_vp, _i64, _i64, _i64, _i32, _vp, _i32, _vp, _sz, _vp]),
     "metis_nvfp4_matvec": (_i32, [_vp, _vp, _vp, _i64, _i64, _vp, _f32, _vp, _vp, _i64, _i32, _vp]),
     "metis_linear_fwd_f32bias": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _i32, _vp, _sz, _vp]),
+    "metis_linear_fwd_grouped": (_i32, [_vp, _vp, _vp, _i64, _i64, _vp, _i32, _i32, _vp]),
     "metis_linear_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "metis_linear_fwd_ws": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _i32, _vp, _sz, _vp]),
     "metis_linear_dgrad_ws": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i32, _vp, _sz, _vp]),

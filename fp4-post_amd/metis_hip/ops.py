@@ -349,6 +349,38 @@ def linear_fwd(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None,
     return out
 
 
+def linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.bfloat16) -> list[torch.Tensor]:
+    """[linear_fwd(a, b, t=t, u=u, bias=bias) for (b, t, u, bias) in members] in one call: a projection group
+    (q/k/v, gate/up) that shares one packed activation.  Decode-sized batches run as a single launch."""
+    import ctypes
+    M, K = a.rows, a.cols
+    dev = a.codes.device
+    arr = (_lib.LinearMember * len(members))()
+    outs, keep = [], []
+    for i, (b, t, u, bias) in enumerate(members):
+        if b.cols != K:
+            raise ValueError(f"contraction mismatch: {K} vs {b.cols}")
+        r = 0
+        if t is not None:
+            t, u = t.to(torch.bfloat16).contiguous(), u.to(torch.bfloat16).contiguous()
+            r = t.shape[1]
+            if t.shape != (M, r) or u.shape != (b.rows, r):
+                raise ValueError("low-rank operands must be t[M, r], u[N, r]")
+        if bias is not None:
+            bias = bias.to(torch.bfloat16).contiguous()
+        out = torch.empty(M, b.rows, dtype=out_dtype, device=dev)
+        keep += [t, u, bias]
+        outs.append(out)
+        arr[i] = _lib.LinearMember(b.codes.data_ptr(), b.scales.data_ptr(), b.unit.data_ptr(),
+                                   None if t is None else t.data_ptr(), None if u is None else u.data_ptr(), r,
+                                   None if bias is None else bias.data_ptr(), out.data_ptr(), b.rows)
+    rc = load().metis_linear_fwd_grouped(a.codes.data_ptr(), a.scales.data_ptr(), a.unit.data_ptr(), M, K,
+                                         ctypes.cast(arr, ctypes.c_void_p), len(members),
+                                         DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16, _stream())
+    check(rc, "metis_linear_fwd_grouped", (M, K, [m[0].rows for m in members]))
+    return outs
+
+
 def linear_dgrad(dy: PackedNVFP4, wt: PackedNVFP4, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     """grad_input[L, K] from dY packed along N [L, N] and W packed along N (column-blocked) [K, N]."""
     if dy.cols != wt.cols:

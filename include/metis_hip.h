@@ -243,6 +243,28 @@ int metis_linear_wgrad_ws(const void *dyt_codes, const void *dyt_scales, const f
                           void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * One packed activation against several weight matrices in one call: the q/k/v (gate/up) projections of a
+ * decoder layer, which the reference quantizes the activation once for (BitLinear._get_shared_quantized_input,
+ * src/Metis/Metis/bitlinear.py:676-702) and then multiplies one by one.  Result i equals
+ * metis_linear_fwd(a, members[i].b_*, M, members[i].N, K, members[i].t, .u, .r, .bias, members[i].out).
+ * For decode-sized M (< 256, K % 64 == 0, count <= 4) all members share one launch, so a narrow k or v projection
+ * no longer costs a launch latency of its own; other shapes run member by member.
+ *   members  HOST array of `count` descriptors holding device pointers (bias bf16 [N] or NULL)
+ */
+typedef struct metis_linear_member {
+    const void *b_codes, *b_scales;
+    const float *b_unit;
+    const void *t, *u;
+    int64_t r;
+    const void *bias;
+    void *out;
+    int64_t N;
+} metis_linear_member;
+int metis_linear_fwd_grouped(const void *a_codes, const void *a_scales, const float *a_unit, int64_t M,
+                             int64_t K, const metis_linear_member *members, int count, int out_dtype,
+                             void *stream);
+
+/*
  * Mean mode: X^ = 1 me^T + QDQ(X - me), the column mean over tokens kept in high precision and only the
  * centred residual quantized (LinearLowbitFunction.svd_quant with metis_mode="mean",
  * src/Metis/Metis/bitlinear.py:311-336; the default of the reference's MetisArgs, src/grpo/grpo.py:66).

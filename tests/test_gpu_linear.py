@@ -236,3 +236,27 @@ def test_output_offsets_beyond_32_bits():
     first = out[:256]
     for rep in (1, 95, 191):
         assert torch.equal(out[rep * 256:(rep + 1) * 256], first), rep
+
+
+@pytest.mark.parametrize("M,K,Ns,r", [(64, 3584, (3584, 512, 512), 64), (1, 1024, (256, 96), 0), (40, 3584, (18944, 18944), 32),
+                                      (64, 320, (100, 36, 64, 2052), 32), (300, 512, (384, 260), 32)])
+def test_grouped_projections_equal_member_by_member_calls(M, K, Ns, r):
+    """A projection group against one packed activation: bit-identical to calling linear_fwd per member (the
+    decode-sized cases run as one launch, the last one falls back to a call per member)."""
+    from metis_hip import ops
+    g = torch.Generator().manual_seed(M + K)
+    px = ops.quantize(synthetic_activation(60 + M, M, K).cuda())
+    members = []
+    for i, N in enumerate(Ns):
+        pw = ops.quantize(_weights(61 + i, N, K).cuda())
+        t = u = None
+        if r and i != 1:                                        # one member without a low-rank term
+            t = torch.randn(M, r, generator=g).bfloat16().cuda()
+            u = torch.randn(N, r, generator=g).bfloat16().cuda()
+        bias = (torch.randn(N, generator=g) * 0.1).bfloat16().cuda() if i % 2 == 0 else None
+        members.append((pw, t, u, bias))
+    for dt in (torch.bfloat16, torch.float32):
+        got = ops.linear_fwd_grouped(px, members, out_dtype=dt)
+        for (pw, t, u, bias), y in zip(members, got):
+            want = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, out_dtype=dt)
+            assert torch.equal(y, want)
