@@ -7,8 +7,8 @@
 //
 // Two-phase structure forced by the arithmetic: the codes depend only on the block's own raw
 // scalar (quant.py:27), the scale bytes on the tensor-wide maximum (quant.py:21-23).  Phase 1
-// writes codes, parks each block's maximum as bf16 (2 B per block) and publishes one partial
-// maximum per workgroup; phase 2 turns the parked maxima into E4M3 bytes.
+// writes codes, parks each block's maximum (2 B per block as bf16; 4 B as binary32 for data that is not
+// bf16-valued) and publishes one partial maximum per workgroup; phase 2 turns the parked maxima into E4M3 bytes.
 #include "metis_device.h"
 #include "metis_host.h"
 #include "nvfp4_encode.h"
