@@ -260,3 +260,31 @@ def test_grouped_projections_equal_member_by_member_calls(M, K, Ns, r):
         for (pw, t, u, bias), y in zip(members, got):
             want = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, out_dtype=dt)
             assert torch.equal(y, want)
+
+
+def test_config3_full_size_forward_on_row_and_column_slices():
+    """8192 x 4096 x 14336 with r = 64 and bias: the full launch is checked on three row slabs and one column slab
+    against the double-precision product of the dequantized operands (the slabs straddle tile and XCD boundaries),
+    and on linearity in the low-rank term: out(t) - out(0) == t u^T."""
+    from metis_hip import ops
+    M, K, N, r = 8192, 4096, 14336, 64
+    g = torch.Generator().manual_seed(1003)
+    x = synthetic_activation(1003, M, K).cuda()
+    w = (torch.randn(N, K, generator=g) * 0.02).bfloat16().cuda()
+    t = torch.randn(M, r, generator=g).bfloat16().cuda()
+    u = (torch.randn(N, r, generator=g) * 0.1).bfloat16().cuda()
+    bias = (torch.randn(N, generator=g) * 0.1).bfloat16().cuda()
+    px, pw = ops.quantize(x), ops.quantize(w)
+    out = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, out_dtype=torch.float32)
+    xq, wq = ops.dequantize(px, torch.float32).double(), ops.dequantize(pw, torch.float32).double()
+    for r0 in (0, 4000, M - 100):
+        want = xq[r0:r0 + 100] @ wq.T + t[r0:r0 + 100].double() @ u.double().T + bias.double()
+        assert rel_fro(out[r0:r0 + 100].cpu(), want.cpu()) <= 1e-5
+    c0 = 7100
+    want = xq @ wq[c0:c0 + 100].T + t.double() @ u[c0:c0 + 100].double().T + bias[c0:c0 + 100].double()
+    assert rel_fro(out[:, c0:c0 + 100].cpu(), want.cpu()) <= 1e-5
+    plain = ops.linear_fwd(px, pw, bias=bias, out_dtype=torch.float32)
+    low = (out - plain)[::37].double()
+    assert rel_fro(low.cpu(), (t[::37].double() @ u.double().T).cpu()) <= 1e-4
+    got16 = ops.linear_fwd(px, pw, t=t, u=u, bias=bias)
+    assert rel_fro(got16[::53].float().cpu(), out[::53].bfloat16().float().cpu()) <= 1e-6     # the bf16 store is one rounding
