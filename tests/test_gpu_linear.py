@@ -288,3 +288,27 @@ def test_config3_full_size_forward_on_row_and_column_slices():
     assert rel_fro(low.cpu(), (t[::37].double() @ u.double().T).cpu()) <= 1e-4
     got16 = ops.linear_fwd(px, pw, t=t, u=u, bias=bias)
     assert rel_fro(got16[::53].float().cpu(), out[::53].bfloat16().float().cpu()) <= 1e-6     # the bf16 store is one rounding
+
+
+def test_config4_full_size_dgrad_and_wgrad():
+    """L = 4096 tokens, 1536 -> 8960 projection: dgrad (split-K: 96 output tiles) and wgrad (210 tiles) on operands
+    re-quantized along their contraction, against double precision on row slabs."""
+    from metis_hip import ops
+    L, K, N = 4096, 1536, 8960
+    g = torch.Generator().manual_seed(1004)
+    x = synthetic_activation(1004, L, K).cuda()
+    w = (torch.randn(N, K, generator=g) * 0.02).bfloat16().cuda()
+    dy = (torch.randn(L, N, generator=torch.Generator().manual_seed(2004)) * 1e-3).bfloat16().cuda()
+    p_dy, p_wt = ops.quantize(dy, sr=True, seed=2004), ops.quantize(w, col=True)
+    gx = ops.linear_dgrad(p_dy, p_wt, out_dtype=torch.float32)
+    dq, wq = ops.dequantize(p_dy, torch.float32).double(), ops.dequantize(p_wt, torch.float32).double()      # [L, N], [K, N]
+    for r0 in (0, 2000, L - 64):
+        assert rel_fro(gx[r0:r0 + 64].cpu(), (dq[r0:r0 + 64] @ wq.T).cpu()) <= 1e-5
+    p_dyt, p_xt = ops.quantize(dy, col=True, sr=True, seed=2005), ops.quantize(x, col=True, sr=True, seed=2006)
+    gw = ops.linear_wgrad(p_dyt, p_xt)
+    dtq, xtq = ops.dequantize(p_dyt, torch.float32).double(), ops.dequantize(p_xt, torch.float32).double()   # [N, L], [K, L]
+    for r0 in (0, 5000, N - 64):
+        assert rel_fro(gw[r0:r0 + 64].cpu(), (dtq[r0:r0 + 64] @ xtq.T).cpu()) <= 1e-5
+    # stochastic rounding keeps the gradients unbiased estimates of the dense ones: FP4 noise level, not a parity bar
+    assert rel_fro(gx.cpu(), (dy.double() @ w.double()).cpu()) < 0.2
+    assert rel_fro(gw.cpu(), (dy.double().T @ x.double()).cpu()) < 0.3
