@@ -30,9 +30,11 @@ def test_fused_rmsnorm_quant(rows, cols, mode):
     torch.cuda.synchronize()
     want = O.rmsnorm(x, gamma, 1e-6)
     assert rel_fro(normed.cpu(), want) <= TOL
-    # elementwise: at most one bf16 ulp apart anywhere
+    # elementwise: the row sum is taken in a different order, so rstd may differ in its last bit; a flip of the first
+    # bf16 rounding (x * rstd) can carry through the multiplication by gamma and its rounding: at most two bf16 ulps
     d = (normed.cpu().float() - want.float()).abs()
-    assert bool((d <= want.float().abs() * 2.0 ** -7 + 1e-30).all())
+    assert bool((d <= want.float().abs() * 2.0 ** -6 + 1e-30).all())
+    assert float((d > 0).float().mean()) < 0.01                  # and that is rare
     mine = normed.cpu()
     codes, scales, unit, _ = O.nvfp4_pack(mine.float() if mode == 0 else mine)
     assert torch.equal(p.codes.cpu(), codes) and torch.equal(p.scales.cpu(), scales)
