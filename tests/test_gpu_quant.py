@@ -465,3 +465,27 @@ def test_f32_input_argument_checks():
     assert call(x.data_ptr() + 4, 64, 2) == _lib.E_ARG
     assert call(x.data_ptr(), 64, 3) == _lib.E_ARG               # unknown mode
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("tag,mode", MODES + [("f32", 2)])
+def test_col_quant_large_ragged_tensors(ops, tag, mode):
+    """A tensor of many tiles, ragged in both directions (rows not a multiple of the 256-row tile, columns not a
+    multiple of the 64-column tile), plain, centred and with the library's own stochastic rounding."""
+    from oracle import metis_oracle as O
+    rows, cols = 4096 + 48, 8192 + 6
+    g = torch.Generator().manual_seed(77)
+    x = torch.randn(rows, cols, generator=g) * torch.exp(torch.randn(rows, 1, generator=g))
+    x.view(-1)[::101] = 0
+    xin = x if mode == 2 else x.bfloat16()
+    arith = xin if mode == 1 else xin.float()
+    p = ops.quantize(xin.cuda(), 1 if mode == 1 else 0, col=True)
+    codes, scales, unit, _ = O.nvfp4_pack_col(arith)
+    _check_packed(p, codes, scales, unit, f"wide col {tag}")
+    me = arith.mean(dim=0)
+    p = ops.quantize(xin.cuda(), 1 if mode == 1 else 0, col=True, center=me.cuda())
+    codes, scales, unit, _ = O.nvfp4_pack_col(arith - me)
+    _check_packed(p, codes, scales, unit, f"wide col centred {tag}")
+    # own-stream stochastic rounding is indexed by output block: equal to row packing of the transpose
+    a = ops.quantize(xin.cuda(), 1 if mode == 1 else 0, col=True, sr=True, seed=5, offset=9)
+    b = ops.quantize(xin.cuda().t().contiguous(), 1 if mode == 1 else 0, sr=True, seed=5, offset=9)
+    assert torch.equal(a.codes, b.codes) and torch.equal(a.scales, b.scales)
