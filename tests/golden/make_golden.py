@@ -202,6 +202,50 @@ def golden_hadamard(out: dict):
         F.enable_nv_recipe = False
 
 
+def golden_mean_mode(out: dict):
+    """Mean mode (bitlinear.py:311-336): column mean over tokens kept, centred residual through the fused QDQ; a
+    prefill call, then a single-token decode call on the same cache (weighted running mean), in binary32 and in
+    bf16; and LinearLowbit forward + backward with the mode on for activations and output gradients
+    (round-to-nearest quantizers everywhere, so no random draws are involved)."""
+    F = rb.LinearLowbitFunction
+    g = torch.Generator().manual_seed(51)
+    q = rq.Cast2NVFp4e2m1BlockNOSR
+    x = (torch.randn(2, 24, 64, generator=g) + 2.0 * torch.randn(1, 1, 64, generator=g)).bfloat16()
+    step = (torch.randn(4, 1, 64, generator=g) + 1.0).bfloat16()
+    out["mean_x"], out["mean_step"] = bits(x), bits(step)
+    for tag, cast in (("p32", torch.float32), ("pb16", torch.bfloat16)):
+        cache = {}
+        out[f"mean_out_{tag}"] = bits(F.svd_quant(x.to(cast), quant_func=q, metis_mode="mean", mean_cache=cache, cache_key="k"))
+        out[f"mean_cache_{tag}"] = bits(cache["k"][0])
+        out[f"mean_step_out_{tag}"] = bits(F.svd_quant(step.to(cast), quant_func=q, metis_mode="mean", mean_cache=cache, cache_key="k"))
+        out[f"mean_step_cache_{tag}"] = bits(cache["k"][0])
+        out[f"mean_step_count_{tag}"] = np.array([cache["k"][1]], dtype=np.int64)
+    _configure("nvfp4e2m1bnosr", "nvfp4e2m1bnosr", "nvfp4e2m1bnosr", torch.float32)
+    F.enable_activation_svd, F.enable_backward_svd = True, True
+    F.activation_lowrank_svd = F.backward_lowrank_svd = 8
+    F.activation_lowrank_niter, F.backward_lowrank_niter = 0, 0
+    F.activation_broadcast_dim, F.backward_broadcast_dim = 0, -1
+    F.tp_simulate = False
+    try:
+        B, T, K, N = 2, 16, 64, 48
+        xl = (torch.randn(B, T, K, generator=g) + 1.5 * torch.randn(1, 1, K, generator=g)).bfloat16().float()
+        w = (torch.randn(N, K, generator=g) * 0.05).bfloat16().float()
+        b = (torch.randn(N, generator=g) * 0.1).bfloat16().float()
+        dy = ((torch.randn(B, T, N, generator=g) + 0.5 * torch.randn(1, 1, N, generator=g)) * 1e-3).bfloat16().float()
+        layer = rb.LinearLowbit(K, N, bias=True, args=SimpleNamespace(device="cpu", cache_quantized_weight=False))
+        with torch.no_grad():
+            layer.weight.copy_(w)
+            layer.bias.copy_(b)
+        xr = xl.clone().requires_grad_(True)
+        y = layer(xr)
+        y.backward(dy)
+        out["mean_lin_x"], out["mean_lin_w"], out["mean_lin_b"], out["mean_lin_dy"] = bits(xl), bits(w), bits(b), bits(dy)
+        out["mean_lin_y"], out["mean_lin_gx"] = bits(y.detach()), bits(xr.grad)
+        out["mean_lin_gw"], out["mean_lin_gb"] = bits(layer.weight.grad), bits(layer.bias.grad)
+    finally:
+        F.enable_activation_svd, F.enable_backward_svd = False, False
+
+
 def main():
     torch.set_num_threads(1)
     out: dict = {}
@@ -216,6 +260,11 @@ def main():
     path = os.path.join(HERE, "metis_reference_hadamard.npz")
     np.savez_compressed(path, **had)
     print(f"wrote {path}: {len(had)} arrays, {os.path.getsize(path)} bytes")
+    mm: dict = {}
+    golden_mean_mode(mm)
+    path = os.path.join(HERE, "metis_reference_mean_mode.npz")
+    np.savez_compressed(path, **mm)
+    print(f"wrote {path}: {len(mm)} arrays, {os.path.getsize(path)} bytes")
 
 
 if __name__ == "__main__":

@@ -325,3 +325,73 @@ def test_qwen2_decoder_layer_under_the_reference_default_arguments(monkeypatch):
     assert rel_fro(out.detach().float().cpu(), ref.detach().float().cpu()) <= 2e-2
     ref.float().square().mean().backward()
     assert rel_fro(gx_packed, xg.grad.detach().float().cpu()) < 0.2      # both carry independent stochastic rounding
+
+
+def _mean_golden():
+    import os
+    import numpy as np
+    return dict(np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "metis_reference_mean_mode.npz")))
+
+
+@pytest.mark.parametrize("tag,cd", [("p32", torch.float32), ("pb16", torch.bfloat16)])
+def test_mean_mode_against_reference_vectors(tag, cd):
+    """The reference's own svd_quant(metis_mode="mean") outputs (prefill, then a decode call on the same cache)
+    against the packed path (centred quantizer + mean vector) and against the generic path."""
+    from helpers import t
+    from metis_hip import CenteredNVFP4, LinearLowbitFunction as F, quant_func
+    g = _mean_golden()
+    keep = (F.compute_dtype, F.enable_activation_svd, F.metis_mode, F.tp_simulate, F.enable_nv_recipe, F.q_forward_input)
+    F.compute_dtype, F.enable_activation_svd, F.metis_mode, F.tp_simulate, F.enable_nv_recipe = cd, True, "mean", False, False
+    F.q_forward_input = quant_func["nvfp4e2m1bnosr"]
+    try:
+        x, step = t(g["mean_x"]).cuda(), t(g["mean_step"]).cuda()
+        for path in ("packed", "generic"):
+            cache = {}
+            if path == "packed":
+                a = F._prepare_input(x, mean_cache=cache, cache_key="k")
+                assert isinstance(a, CenteredNVFP4)
+                got = a.dequantize(cd).reshape(x.shape)
+                b = F._prepare_input(step, mean_cache=cache, cache_key="k")
+                got_step = b.dequantize(cd).reshape(step.shape)
+            else:
+                got = F.svd_quant(x.to(cd), quant_func=F.q_forward_input, metis_mode="mean", mean_cache=cache, cache_key="k")
+                got_step = F.svd_quant(step.to(cd), quant_func=F.q_forward_input, metis_mode="mean", mean_cache=cache, cache_key="k")
+            want, want_step = t(g[f"mean_out_{tag}"]), t(g[f"mean_step_out_{tag}"])
+            # the column mean is summed in another order than torch's CPU reduction; a last-bit difference of the mean
+            # shifts every output by that much (and can move single codes), so the comparison is a tolerance: a few
+            # binary32 ulps, or one bf16 ulp of the mean in bf16 arithmetic
+            tol = 1e-6 if cd == torch.float32 else 4e-3
+            assert rel_fro(got.cpu().float(), want.float()) <= tol, path
+            assert rel_fro(got_step.cpu().float(), want_step.float()) <= tol, path
+            assert cache["k"][1] == int(g[f"mean_step_count_{tag}"][0])
+            torch.testing.assert_close(cache["k"][0].cpu().float().reshape(-1), t(g[f"mean_step_cache_{tag}"]).float().reshape(-1),
+                                       rtol=1e-6 if cd == torch.float32 else 2 ** -7, atol=1e-7)
+    finally:
+        F.compute_dtype, F.enable_activation_svd, F.metis_mode, F.tp_simulate, F.enable_nv_recipe, F.q_forward_input = keep
+
+
+def test_mean_mode_linear_against_reference_vectors(monkeypatch):
+    """LinearLowbit with the mean mode on for activations and output gradients, round-to-nearest quantizers everywhere:
+    forward against the reference's output on both paths; backward of the generic path (which follows the reference's
+    operand choice: dY blocked along its last dimension, the saved forward activation) against the reference's gradients."""
+    from helpers import t
+    from metis_hip import BitLinear, LinearLowbitFunction as F, MetisArgs, quant_func
+    g = _mean_golden()
+    x, w, b, dy = (t(g[k]) for k in ("mean_lin_x", "mean_lin_w", "mean_lin_b", "mean_lin_dy"))
+    args = MetisArgs(cache_quantized_weight=False)
+    args.enable_forward_svd = False
+    args.q_backward_input = args.q_backward_weight = args.q_backward_outputgrad = "nvfp4e2m1bnosr"
+    lin = BitLinear(64, 48, args=args, bias=True, dtype=torch.float32, compute_dtype=torch.float32).cuda().warmup_linear
+    with torch.no_grad():
+        lin.weight.copy_(w)
+        lin.bias.copy_(b)
+    y = lin(x.cuda())                                             # packed path
+    assert rel_fro(y.detach().cpu(), t(g["mean_lin_y"])) <= 1e-5
+    monkeypatch.setattr(F, "_mean_mode_packable", staticmethod(lambda: False))
+    xr = x.cuda().requires_grad_(True)
+    y2 = lin(xr)                                                  # generic path
+    assert rel_fro(y2.detach().cpu(), t(g["mean_lin_y"])) <= 1e-5
+    y2.backward(dy.cuda())
+    assert rel_fro(xr.grad.cpu(), t(g["mean_lin_gx"])) <= 1e-5
+    assert rel_fro(lin.weight.grad.cpu(), t(g["mean_lin_gw"])) <= 1e-5
+    assert rel_fro(lin.bias.grad.cpu(), t(g["mean_lin_gb"])) <= 1e-5

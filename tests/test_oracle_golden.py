@@ -111,3 +111,26 @@ def test_c_oracle_binary32_input_mode_matches_torch_restatement():
     xb = x.bfloat16()
     a, b = C.nvfp4_pack(xb, 0), C.nvfp4_pack(xb.float(), 2)
     assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1]) and a[2] == b[2]
+
+
+@pytest.mark.parametrize("tag,dt", [("p32", "float32"), ("pb16", "bfloat16")])
+def test_mean_mode_formula_matches_reference(tag, dt):
+    """mean + QDQ(x - mean) with the oracle's QDQ reproduces the reference's svd_quant(metis_mode="mean") output bit
+    for bit, for a prefill call and for the single-token decode call that updates the weighted running mean."""
+    import os
+    import numpy as np
+    import torch
+    from helpers import same_bits, t
+    from oracle import metis_oracle as O
+    g = dict(np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "metis_reference_mean_mode.npz")))
+    D = getattr(torch, dt)
+    x = t(g["mean_x"]).to(D).reshape(-1, 64)
+    me = x.mean(dim=0, keepdim=True)
+    assert same_bits(me, t(g[f"mean_cache_{tag}"]))
+    assert same_bits((me + O.nvfp4_qdq(x - me)).reshape(2, 24, 64), t(g[f"mean_out_{tag}"]))
+    step = t(g["mean_step"]).to(D).reshape(-1, 64)
+    count = x.shape[0]
+    me2 = (me * count + step.mean(dim=0, keepdim=True) * step.shape[0]) / (count + step.shape[0])
+    assert int(g[f"mean_step_count_{tag}"][0]) == count + step.shape[0]
+    assert same_bits(me2, t(g[f"mean_step_cache_{tag}"]))
+    assert same_bits((me2 + O.nvfp4_qdq(step - me2)).reshape(4, 1, 64), t(g[f"mean_step_out_{tag}"]))
