@@ -57,7 +57,14 @@ class CenteredNVFP4:
         return self.mean.to(dtype).unsqueeze(0) + dequantize(self.residual, dtype)
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> int:
+    """Handle of torch's current stream on the current device (the raw getter skips the Stream object: this is
+    called several times per layer)."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
