@@ -939,7 +939,7 @@ int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a
         const GemmMember& g = members[i];
         if (!g.b_codes || !g.b_scales || !g.b_unit || !g.out || g.N <= 0 || g.N > INT32_MAX || g.N % 4 || g.r < 0 || g.r % 32 ||
             (g.r > 0 && (!g.t || !g.u)) || ((uintptr_t)g.b_codes % 16) || ((uintptr_t)g.b_scales % 2) || ((uintptr_t)g.out % 16) ||
-            ((uintptr_t)g.t % 16) || ((uintptr_t)g.u % 16) || ((uintptr_t)g.bias % 2))
+            ((uintptr_t)g.t % 16) || ((uintptr_t)g.u % 16) || ((uintptr_t)g.bias % (g.bias_is_f32 ? 4 : 2)))
             skinny = false;
         al8 = al8 && ((uintptr_t)g.b_scales % 8) == 0;
         tiles += (g.N + 31) / 32;
@@ -948,7 +948,7 @@ int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a
         for (int i = 0; i < count; ++i) {
             const GemmMember& g = members[i];
             const int rc = gemm_nvfp4(a_codes, a_scales, a_unit, g.b_codes, g.b_scales, g.b_unit, M, g.N, K, g.t, g.u, g.r, g.bias,
-                                      g.out, out_dtype, st);
+                                      g.out, out_dtype, st, nullptr, 0, g.bias_is_f32 != 0);
             if (rc != METIS_OK) return rc;
         }
         return METIS_OK;
@@ -960,7 +960,7 @@ int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a
         const GemmMember& g = members[i];
         end += (int)((g.N + 31) / 32);
         grp.m[i] = SkinnyMember{(const uint8_t*)g.b_codes, (const uint8_t*)g.b_scales, g.b_unit, (const uint16_t*)g.t,
-                                (const uint16_t*)g.u, (const uint16_t*)g.bias, g.out, (int)g.N, (int)g.r, end, 0};
+                                (const uint16_t*)g.u, (const uint16_t*)g.bias, g.out, (int)g.N, (int)g.r, end, g.bias_is_f32 != 0};
     }
     // same shape heuristics as gemm_skinny, on the joint column count
     const int c = (K % 256 == 0 && al8) ? 4 : 1;

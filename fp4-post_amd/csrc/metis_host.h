@@ -77,6 +77,7 @@ struct GemmMember {
     const void* bias;
     void* out;
     int64_t N;
+    int64_t bias_is_f32;
 };
 int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a_unit, int64_t M, int64_t K,
                        const GemmMember* members, int count, int out_dtype, hipStream_t st);

@@ -16,7 +16,7 @@ class LinearMember(ctypes.Structure):
     """metis_linear_member of include/metis_hip.h: one weight matrix of a grouped GEMM."""
     _fields_ = [("b_codes", ctypes.c_void_p), ("b_scales", ctypes.c_void_p), ("b_unit", ctypes.c_void_p),
                 ("t", ctypes.c_void_p), ("u", ctypes.c_void_p), ("r", ctypes.c_int64), ("bias", ctypes.c_void_p),
-                ("out", ctypes.c_void_p), ("N", ctypes.c_int64)]
+                ("out", ctypes.c_void_p), ("N", ctypes.c_int64), ("bias_is_f32", ctypes.c_int64)]
 
 
 MODE_P32, MODE_PB16 = 0, 1

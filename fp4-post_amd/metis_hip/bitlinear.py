@@ -668,12 +668,88 @@ class BitLinear(nn.Module):
         self._merged_rollout_weight_cache = None
         return super()._apply(fn, recurse=recurse)
 
+    # ------------------------------------------------------------------ projection group in one launch (inference)
+    grouped_inference = True      # q/k/v and gate/up of a decode-sized batch as one GEMM launch when autograd is off
+
+    def _packed_residual(self):
+        """Packed residual weight for the fused launch, or None when the kernel path does not apply."""
+        F = LinearLowbitFunction
+        wl = self.warmup_linear
+        if not F.enable_nv_recipe and _packable(wl.weight, F.q_forward_weight) and wl.weight.shape[0] % 4 == 0:
+            p_res = wl._get_quantized_weight(wl.weight, arith=self.compute_dtype)       # cache hit: no pass over W
+        else:
+            p_res = wl._get_quantized_weight(wl.weight.to(self.compute_dtype))
+        return p_res if isinstance(p_res, PackedNVFP4) else None
+
+    def _fusable(self) -> bool:
+        r = self.args.forward_svd_rank
+        return (self.is_svd_quant and isinstance(self.vlinear, LinearLowbit) and isinstance(self.warmup_linear, LinearLowbit)
+                and r > 0 and r % 32 == 0 and self.ulinear.bias is None and not BitLinear.quantized_lowrank_branch)
+
+    def _forward_group(self, x: torch.Tensor, shared_input):
+        """All members of this layer's projection group on the shared activation in one call (no autograd):
+        {id(member): output}, or None when the group does not qualify.  The siblings pick their result up when they
+        are called with the same tensor object."""
+        F = LinearLowbitFunction
+        group = self.activation_group
+        members = group["members"]
+        rows = x.numel() // max(x.shape[-1], 1)
+        if rows >= 256 or not all(m._fusable() and m.compute_dtype == self.compute_dtype for m in members):
+            return None
+        packed = [m._packed_residual() for m in members]
+        if any(p is None for p in packed):
+            return None
+        cd = torch.bfloat16
+        x2 = _flat2d(x).to(cd)
+        # one product for every member's rank-r projection: V of all members stacked, cached on their versions
+        key = tuple((m.vlinear.weight._version, m.s._version) for m in members) + (x2.device,)
+        cached = group.get("stacked_v")
+        if cached is None or cached[0] != key:
+            cached = (key, torch.cat([m.vlinear.weight.to(cd) for m in members], dim=0),
+                      torch.cat([m.s.to(cd) for m in members], dim=0))
+            group["stacked_v"] = cached
+        t_all = torch.matmul(x2, cached[1].T) * cached[2]
+        centre = shared_input.mean if isinstance(shared_input, CenteredNVFP4) else None
+        px = shared_input.residual if centre is not None else shared_input
+        calls, c0 = [], 0
+        for m, p_res in zip(members, packed):
+            r = m.args.forward_svd_rank
+            bias = m.warmup_linear.bias
+            if centre is not None:                              # mean mode: bias + W^ me in binary32
+                w_mean = ops.matvec(p_res, centre)
+                bias = w_mean if bias is None else w_mean + bias.float()
+            elif bias is not None:
+                bias = bias.to(cd)
+            calls.append((p_res, t_all[:, c0:c0 + r].contiguous(), m.ulinear.weight.to(cd), bias))
+            c0 += r
+        out_dtype = torch.float32 if F.compute_dtype == torch.float32 else torch.bfloat16
+        outs = ops.linear_fwd_grouped(px, calls, out_dtype=out_dtype)
+        lead = x.shape[:-1]
+        return {id(m): y.reshape(*lead, y.shape[-1]).to(F.compute_dtype) for m, y in zip(members, outs)}
+
     # ------------------------------------------------------------------ forward (reference 736-769)
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         F = LinearLowbitFunction
         F.mean_cache = self.mean_cache
         if not self.is_svd_quant:
             return self.warmup_linear(x)
+        group = self.activation_group
+        if (BitLinear.grouped_inference and group is not None and not torch.is_grad_enabled() and len(group.get("members", ())) > 1
+                and x.is_cuda and self._fusable()):
+            ready = group.get("grouped_outputs")
+            if ready is not None and ready[0]() is x and id(self) in ready[1]:
+                return ready[1].pop(id(self))
+            shared_input = self._get_shared_quantized_input(x)
+            if isinstance(shared_input, (PackedNVFP4, CenteredNVFP4)):
+                outs = self._forward_group(x, shared_input)
+                if outs is not None:
+                    mine = outs.pop(id(self))
+
+                    def drop(ref, group=group):
+                        if group.get("grouped_outputs") is not None and group["grouped_outputs"][0] is ref:
+                            group["grouped_outputs"] = None
+                    group["grouped_outputs"] = (weakref.ref(x, drop), outs)
+                    return mine
         share_activation = (isinstance(self.vlinear, LinearLowbit) and isinstance(self.warmup_linear, LinearLowbit)
                             and self.args.forward_svd_rank > 0)
         if share_activation:
@@ -683,12 +759,8 @@ class BitLinear(nn.Module):
                     and not BitLinear.quantized_lowrank_branch):
                 # one fused launch for both branches; it already is the "merged" evaluation, so the
                 # rollout switch changes nothing on this path
-                wl = self.warmup_linear
-                if not F.enable_nv_recipe and _packable(wl.weight, F.q_forward_weight) and wl.weight.shape[0] % 4 == 0:
-                    p_res = wl._get_quantized_weight(wl.weight, arith=self.compute_dtype)   # cache hit: no pass over W
-                else:
-                    p_res = wl._get_quantized_weight(wl.weight.to(self.compute_dtype))
-                if isinstance(p_res, PackedNVFP4):
+                p_res = self._packed_residual()
+                if p_res is not None:
                     return _MetisFusedFunction.apply(x, self.vlinear.weight, self.s, self.ulinear.weight,
                                                      self.warmup_linear.weight, self.warmup_linear.bias, shared_input, p_res)
             if BitLinear.rollout_merge_active and not torch.is_grad_enabled():

@@ -373,14 +373,15 @@ def linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.b
             r = t.shape[1]
             if t.shape != (M, r) or u.shape != (b.rows, r):
                 raise ValueError("low-rank operands must be t[M, r], u[N, r]")
+        bias_f32 = bias is not None and bias.dtype == torch.float32
         if bias is not None:
-            bias = bias.to(torch.bfloat16).contiguous()
+            bias = bias.contiguous() if bias_f32 else bias.to(torch.bfloat16).contiguous()
         out = torch.empty(M, b.rows, dtype=out_dtype, device=dev)
         keep += [t, u, bias]
         outs.append(out)
         arr[i] = _lib.LinearMember(b.codes.data_ptr(), b.scales.data_ptr(), b.unit.data_ptr(),
                                    None if t is None else t.data_ptr(), None if u is None else u.data_ptr(), r,
-                                   None if bias is None else bias.data_ptr(), out.data_ptr(), b.rows)
+                                   None if bias is None else bias.data_ptr(), out.data_ptr(), b.rows, int(bias_f32))
     rc = load().metis_linear_fwd_grouped(a.codes.data_ptr(), a.scales.data_ptr(), a.unit.data_ptr(), M, K,
                                          ctypes.cast(arr, ctypes.c_void_p), len(members),
                                          DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16, _stream())

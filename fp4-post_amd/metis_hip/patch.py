@@ -95,7 +95,8 @@ def replace_linear_with_metis(model, dtype, metis_args, target_modules=None, com
             group_name = None
         if group_name is not None:
             new_layer.activation_group = activation_groups.setdefault(
-                group_name, {"name": group_name, "mean_cache": {}, "input_ref": None, "quantized_input": None})
+                group_name, {"name": group_name, "mean_cache": {}, "input_ref": None, "quantized_input": None, "members": []})
+            new_layer.activation_group["members"].append(new_layer)
         if metis_args.enable_forward_svd:
             new_layer.split()
         setattr(parent, leaf, new_layer)

@@ -249,7 +249,7 @@ int metis_linear_wgrad_ws(const void *dyt_codes, const void *dyt_scales, const f
  * metis_linear_fwd(a, members[i].b_*, M, members[i].N, K, members[i].t, .u, .r, .bias, members[i].out).
  * For decode-sized M (< 256, K % 64 == 0, count <= 4) all members share one launch, so a narrow k or v projection
  * no longer costs a launch latency of its own; other shapes run member by member.
- *   members  HOST array of `count` descriptors holding device pointers (bias bf16 [N] or NULL)
+ *   members  HOST array of `count` descriptors holding device pointers (bias [N] or NULL)
  */
 typedef struct metis_linear_member {
     const void *b_codes, *b_scales;
@@ -259,6 +259,7 @@ typedef struct metis_linear_member {
     const void *bias;
     void *out;
     int64_t N;
+    int64_t bias_is_f32; /* 0: bias is bf16 [N]; 1: binary32 [N] (metis_linear_fwd_f32bias) */
 } metis_linear_member;
 int metis_linear_fwd_grouped(const void *a_codes, const void *a_scales, const float *a_unit, int64_t M,
                              int64_t K, const metis_linear_member *members, int count, int out_dtype,

@@ -453,3 +453,59 @@ def test_fused_rmsnorm_feeds_the_projection_groups_of_a_qwen2_layer():
     # q/k/v and gate/up inputs came packed from the norms: the only row quantizations left are o_proj's input
     # (attention output, also [128, 256]) and down_proj's (the MLP activation)
     assert sorted(seen) == [(128, 256), (128, 512)], seen
+
+
+@pytest.mark.parametrize("mean_mode", [False, True])
+def test_projection_groups_run_as_one_launch_without_autograd(mean_mode, monkeypatch):
+    """Decode-sized batch through a patched Qwen2 decoder layer with autograd off: q/k/v and gate/up each take one
+    grouped GEMM call (the first member evaluates the group, its siblings pick their results up), o and down one
+    plain call each; the layer output equals the member-by-member evaluation up to bf16 roundings of the stacked
+    rank-r product."""
+    pytest.importorskip("transformers")
+    from transformers.models.qwen2.modeling_qwen2 import Qwen2Config, Qwen2DecoderLayer, Qwen2RotaryEmbedding
+    from metis_hip import BitLinear, MetisArgs, ops, replace_model_with_metis
+    torch.manual_seed(0)
+    cfg = Qwen2Config(hidden_size=256, intermediate_size=512, num_attention_heads=4, num_key_value_heads=2,
+                      num_hidden_layers=1, vocab_size=128, max_position_embeddings=256)
+    cfg._attn_implementation = "eager"
+    layer = Qwen2DecoderLayer(cfg, layer_idx=0).to(torch.bfloat16).cuda()
+    for p in layer.parameters():
+        if p.dim() == 2:
+            torch.nn.init.normal_(p, std=0.02)
+    holder = torch.nn.ModuleDict({"layer": layer})
+    args = MetisArgs(forward_svd_rank=32, cache_quantized_weight=True) if mean_mode else MetisArgs.direct_fp4(forward_svd_rank=32)
+    replace_model_with_metis(holder, args)
+    x = (torch.randn(64, 1, 256, device="cuda") + 0.5).bfloat16()
+    pos = torch.zeros(64, 1, dtype=torch.long, device="cuda")
+    pe = Qwen2RotaryEmbedding(cfg).cuda()(x, pos)
+
+    def run():
+        with torch.no_grad():
+            out = holder["layer"](x, position_embeddings=pe, attention_mask=None, position_ids=pos)
+        return out[0] if isinstance(out, tuple) else out
+
+    def reset_means():
+        for m in holder.modules():
+            if isinstance(m, BitLinear):
+                m.mean_cache.clear()
+                if m.activation_group is not None:
+                    m.activation_group["mean_cache"].clear()
+
+    calls = {"grouped": 0, "plain": 0}
+    real_g, real_p = ops.linear_fwd_grouped, ops.linear_fwd
+    monkeypatch.setattr(ops, "linear_fwd_grouped", lambda *a, **k: (calls.__setitem__("grouped", calls["grouped"] + 1), real_g(*a, **k))[1])
+    monkeypatch.setattr(ops, "linear_fwd", lambda *a, **k: (calls.__setitem__("plain", calls["plain"] + 1), real_p(*a, **k))[1])
+    reset_means()
+    got = run()
+    assert calls == {"grouped": 2, "plain": 2}
+    monkeypatch.setattr(BitLinear, "grouped_inference", False)
+    calls.update(grouped=0, plain=0)
+    reset_means()
+    want = run()
+    assert calls == {"grouped": 0, "plain": 7}
+    assert rel_fro(got.float().cpu(), want.float().cpu()) <= 2e-3
+    # with autograd on the group is evaluated member by member (each needs its own graph)
+    monkeypatch.setattr(BitLinear, "grouped_inference", True)
+    calls.update(grouped=0, plain=0)
+    out = holder["layer"](x.clone().requires_grad_(True), position_embeddings=pe, attention_mask=None, position_ids=pos)
+    assert calls["grouped"] == 0
