@@ -240,7 +240,7 @@ def main():
                 for j, i_ in enumerate(idx):
                     arr[j] = _ml.LinearMember(ws_[i_].codes.data_ptr(), ws_[i_].scales.data_ptr(), ws_[i_].unit.data_ptr(),
                                               lows[i_][0].data_ptr(), lows[i_][1].data_ptr(), 64, None, outs[i_].data_ptr(),
-                                              shapes[i_][0], 0)
+                                              shapes[i_][0], 0, 0)
                 return arr
             # projection groups share their activation: q/k/v in one call, o, gate/up in one call, down
             calls = [(3584, member_array([0, 1, 2])), (3584, member_array([3])), (3584, member_array([4, 5])),

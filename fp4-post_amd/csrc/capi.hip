@@ -205,6 +205,14 @@ int metis_linear_fwd_grouped(const void* a_codes, const void* a_scales, const fl
                               (hipStream_t)stream);
 }
 
+size_t metis_lowrank_project_workspace_bytes(int64_t M, int64_t R, int64_t K) { return lowrank_small_workspace_bytes(M, R, K); }
+
+int metis_lowrank_project(const void* x, int64_t ldx, const void* v, int64_t M, int64_t R, int64_t K, const void* s, void* xv,
+                          void* t, void* workspace, size_t workspace_bytes, void* stream)
+{
+    return lowrank_small(x, ldx, v, M, R, K, s, xv, t, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
 size_t metis_linear_workspace_bytes(int64_t M, int64_t N, int64_t K) { return gemm_workspace_bytes(M, N, K); }
 
 int metis_linear_fwd_ws(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes,

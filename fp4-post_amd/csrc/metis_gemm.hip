@@ -736,7 +736,7 @@ __device__ __forceinline__ void skinny_tile(
     const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const float* __restrict__ a_unit,
     const uint8_t* __restrict__ b_codes, const uint8_t* __restrict__ b_scales, const float* __restrict__ b_unit,
     int M, int N, int K, const uint16_t* __restrict__ t, const uint16_t* __restrict__ u, int r,
-    const uint16_t* __restrict__ bias, void* __restrict__ out, int bias_f32, int n0)
+    const uint16_t* __restrict__ bias, void* __restrict__ out, int bias_f32, int n0, int ldt)
 {
     __shared__ float red[WAVES][TM * 16][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, hi = lane >> 5;
@@ -789,7 +789,7 @@ __device__ __forceinline__ void skinny_tile(
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
                 const int mrow = min(m0 + i * 32 + (lane & 31), M - 1);
-                const bf16x8_t ft = *reinterpret_cast<const bf16x8_t*>(t + (int64_t)mrow * r + j);
+                const bf16x8_t ft = *reinterpret_cast<const bf16x8_t*>(t + (int64_t)mrow * ldt + j);
                 acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fu, ft, acc[i], 0, 0, 0);
             }
         }
@@ -831,7 +831,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nvfp4_skinny_kernel(
     const uint16_t* __restrict__ bias, void* __restrict__ out, int bias_f32)
 {
     skinny_tile<TM, C, WAVES, OUT_F32>(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, bias_f32,
-                                       (int)blockIdx.x * 32);
+                                       (int)blockIdx.x * 32, r);
 }
 
 // Several weight matrices against ONE packed activation in one launch (q/k/v, gate/up): the column tiles of the
@@ -846,7 +846,7 @@ struct SkinnyMember {
     const uint16_t* u;
     const uint16_t* bias;
     void* out;
-    int N, r, tile_end, bias_f32;
+    int N, r, tile_end, bias_f32, ldt;
 };
 struct SkinnyGroup {
     SkinnyMember m[kMaxGroupMembers];
@@ -869,7 +869,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nvfp4_skinny_grouped_kernel(
     for (int i = 1; i < kMaxGroupMembers; ++i)
         if (g == i) mm = grp.m[i];
     skinny_tile<TM, C, WAVES, OUT_F32>(a_codes, a_scales, a_unit, mm.b_codes, mm.b_scales, mm.b_unit, M, mm.N, K, mm.t, mm.u, mm.r,
-                                       mm.bias, mm.out, mm.bias_f32, (tile - start) * 32);
+                                       mm.bias, mm.out, mm.bias_f32, (tile - start) * 32, mm.ldt);
 }
 
 template <int TM, int C, int WAVES>
@@ -938,7 +938,7 @@ int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a
     for (int i = 0; i < count && skinny; ++i) {
         const GemmMember& g = members[i];
         if (!g.b_codes || !g.b_scales || !g.b_unit || !g.out || g.N <= 0 || g.N > INT32_MAX || g.N % 4 || g.r < 0 || g.r % 32 ||
-            (g.r > 0 && (!g.t || !g.u)) || ((uintptr_t)g.b_codes % 16) || ((uintptr_t)g.b_scales % 2) || ((uintptr_t)g.out % 16) ||
+            (g.r > 0 && (!g.t || !g.u)) || (g.ldt != 0 && (g.ldt < g.r || g.ldt % 8 || g.ldt > INT32_MAX)) || ((uintptr_t)g.b_codes % 16) || ((uintptr_t)g.b_scales % 2) || ((uintptr_t)g.out % 16) ||
             ((uintptr_t)g.t % 16) || ((uintptr_t)g.u % 16) || ((uintptr_t)g.bias % (g.bias_is_f32 ? 4 : 2)))
             skinny = false;
         al8 = al8 && ((uintptr_t)g.b_scales % 8) == 0;
@@ -947,6 +947,7 @@ int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a
     if (!skinny || tiles > INT32_MAX) {
         for (int i = 0; i < count; ++i) {
             const GemmMember& g = members[i];
+            if (g.ldt != 0 && g.ldt != g.r) return METIS_E_ARG;   // a strided t is only taken by the single-launch path
             const int rc = gemm_nvfp4(a_codes, a_scales, a_unit, g.b_codes, g.b_scales, g.b_unit, M, g.N, K, g.t, g.u, g.r, g.bias,
                                       g.out, out_dtype, st, nullptr, 0, g.bias_is_f32 != 0);
             if (rc != METIS_OK) return rc;
@@ -960,7 +961,8 @@ int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a
         const GemmMember& g = members[i];
         end += (int)((g.N + 31) / 32);
         grp.m[i] = SkinnyMember{(const uint8_t*)g.b_codes, (const uint8_t*)g.b_scales, g.b_unit, (const uint16_t*)g.t,
-                                (const uint16_t*)g.u, (const uint16_t*)g.bias, g.out, (int)g.N, (int)g.r, end, g.bias_is_f32 != 0};
+                                (const uint16_t*)g.u, (const uint16_t*)g.bias, g.out, (int)g.N, (int)g.r, end, g.bias_is_f32 != 0,
+                                (int)(g.ldt ? g.ldt : g.r)};
     }
     // same shape heuristics as gemm_skinny, on the joint column count
     const int c = (K % 256 == 0 && al8) ? 4 : 1;

@@ -78,6 +78,7 @@ struct GemmMember {
     void* out;
     int64_t N;
     int64_t bias_is_f32;
+    int64_t ldt;
 };
 int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a_unit, int64_t M, int64_t K,
                        const GemmMember* members, int count, int out_dtype, hipStream_t st);
@@ -88,6 +89,11 @@ size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 size_t column_mean_workspace_bytes(int64_t cols);
 int column_mean(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_f32, void* out, int out_bf16, void* workspace,
                 size_t workspace_bytes, hipStream_t st, bool sum_only = false);
+
+// xv[M, R] = x[M, K] . v[R, K]^T (bf16, binary32 accumulation) and t = bf16(xv * s) for M < 256; lowrank_small.hip
+size_t lowrank_small_workspace_bytes(int64_t M, int64_t R, int64_t K);
+int lowrank_small(const void* x, int64_t ldx, const void* v, int64_t M, int64_t R, int64_t K, const void* s, void* xv, void* t,
+                  void* workspace, size_t workspace_bytes, hipStream_t st);
 
 int expand_f16(const void* codes, const void* scales, int64_t rows, int64_t cols, void* out, hipStream_t st);
 int gemm_expanded(const void* a_exp, const float* a_unit, const void* b_exp, const float* b_unit, int64_t M, int64_t N,

@@ -16,7 +16,7 @@ class LinearMember(ctypes.Structure):
     """metis_linear_member of include/metis_hip.h: one weight matrix of a grouped GEMM."""
     _fields_ = [("b_codes", ctypes.c_void_p), ("b_scales", ctypes.c_void_p), ("b_unit", ctypes.c_void_p),
                 ("t", ctypes.c_void_p), ("u", ctypes.c_void_p), ("r", ctypes.c_int64), ("bias", ctypes.c_void_p),
-                ("out", ctypes.c_void_p), ("N", ctypes.c_int64), ("bias_is_f32", ctypes.c_int64)]
+                ("out", ctypes.c_void_p), ("N", ctypes.c_int64), ("bias_is_f32", ctypes.c_int64), ("ldt", ctypes.c_int64)]
 
 
 MODE_P32, MODE_PB16 = 0, 1
@@ -53,6 +53,8 @@ SIGNATURES = {
     "metis_column_sum": (_i32, [_vp, _i64, _i64, _i64, _i32, _vp, _i32, _vp, _sz, _vp]),
     "metis_nvfp4_matvec": (_i32, [_vp, _vp, _vp, _i64, _i64, _vp, _f32, _vp, _vp, _i64, _i32, _vp]),
     "metis_linear_fwd_f32bias": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _i32, _vp, _sz, _vp]),
+    "metis_lowrank_project_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "metis_lowrank_project": (_i32, [_vp, _i64, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _sz, _vp]),
     "metis_linear_fwd_grouped": (_i32, [_vp, _vp, _vp, _i64, _i64, _vp, _i32, _i32, _vp]),
     "metis_linear_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "metis_linear_fwd_ws": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _i32, _vp, _sz, _vp]),

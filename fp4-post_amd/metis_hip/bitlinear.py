@@ -501,8 +501,9 @@ class _MetisFusedFunction(torch.autograd.Function):
         F = LinearLowbitFunction
         cd = torch.bfloat16
         x2 = _flat2d(x).to(cd)
-        xv = torch.matmul(x2, v.to(cd).T)                      # [L, r] rank-r projection (library GEMM, bf16)
-        t = xv * s.to(cd)
+        # [L, r] rank-r projection and its product with s (bf16): own split-K kernel for decode-sized batches,
+        # the vendor library's GEMM otherwise
+        xv, t = ops.lowrank_project(x2, v.to(cd), s.to(cd))
         out_dtype = torch.float32 if F.compute_dtype == torch.float32 else torch.bfloat16
         ctx.center = None
         gemm_bias = None if bias is None else bias.to(cd)
@@ -708,7 +709,7 @@ class BitLinear(nn.Module):
             cached = (key, torch.cat([m.vlinear.weight.to(cd) for m in members], dim=0),
                       torch.cat([m.s.to(cd) for m in members], dim=0))
             group["stacked_v"] = cached
-        t_all = torch.matmul(x2, cached[1].T) * cached[2]
+        _, t_all = ops.lowrank_project(x2, cached[1], cached[2])
         centre = shared_input.mean if isinstance(shared_input, CenteredNVFP4) else None
         px = shared_input.residual if centre is not None else shared_input
         calls, c0 = [], 0
@@ -720,7 +721,7 @@ class BitLinear(nn.Module):
                 bias = w_mean if bias is None else w_mean + bias.float()
             elif bias is not None:
                 bias = bias.to(cd)
-            calls.append((p_res, t_all[:, c0:c0 + r].contiguous(), m.ulinear.weight.to(cd), bias))
+            calls.append((p_res, t_all[:, c0:c0 + r], m.ulinear.weight.to(cd), bias))      # a column slice: no copy
             c0 += r
         out_dtype = torch.float32 if F.compute_dtype == torch.float32 else torch.bfloat16
         outs = ops.linear_fwd_grouped(px, calls, out_dtype=out_dtype)

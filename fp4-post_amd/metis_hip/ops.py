@@ -356,6 +356,29 @@ def linear_fwd(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None,
     return out
 
 
+def lowrank_project(x2: torch.Tensor, v: torch.Tensor, s: torch.Tensor | None = None):
+    """Rank-r projection of the low-rank branch: xv = x2[M, K] . v[R, K]^T in bf16 (binary32 accumulation) and, with
+    `s` [R], t = bf16(xv * s): returns xv or (xv, t).  Decode-sized batches (M < 256, R <= 256) run on the library's
+    split-K kernel; everything else is a torch matmul (the vendor library serves those shapes well)."""
+    M, K = x2.shape
+    R = v.shape[0]
+    ok = (x2.is_cuda and x2.dtype == torch.bfloat16 and v.dtype == torch.bfloat16 and 0 < M < 256 and R % 32 == 0
+          and 0 < R <= 256 and K % 64 == 0 and v.shape[1] == K and x2.stride(1) == 1 and x2.stride(0) % 8 == 0
+          and (s is None or s.dtype == torch.bfloat16))
+    if not ok:
+        xv = torch.matmul(x2, v.T)
+        return xv if s is None else (xv, xv * s.to(xv.dtype))
+    v = v.contiguous()
+    L = load()
+    xv = torch.empty(M, R, dtype=torch.bfloat16, device=x2.device)
+    t = None if s is None else torch.empty_like(xv)
+    ws = torch.empty(L.metis_lowrank_project_workspace_bytes(M, R, K), dtype=torch.uint8, device=x2.device)
+    rc = L.metis_lowrank_project(x2.data_ptr(), x2.stride(0), v.data_ptr(), M, R, K, None if s is None else s.contiguous().data_ptr(),
+                                 xv.data_ptr(), None if t is None else t.data_ptr(), ws.data_ptr(), ws.numel(), _stream())
+    check(rc, "metis_lowrank_project", (M, R, K))
+    return xv if s is None else (xv, t)
+
+
 def linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.bfloat16) -> list[torch.Tensor]:
     """[linear_fwd(a, b, t=t, u=u, bias=bias) for (b, t, u, bias) in members] in one call: a projection group
     (q/k/v, gate/up) that shares one packed activation.  Decode-sized batches run as a single launch."""
@@ -367,12 +390,18 @@ def linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.b
     for i, (b, t, u, bias) in enumerate(members):
         if b.cols != K:
             raise ValueError(f"contraction mismatch: {K} vs {b.cols}")
-        r = 0
+        r = ldt = 0
         if t is not None:
-            t, u = t.to(torch.bfloat16).contiguous(), u.to(torch.bfloat16).contiguous()
+            t, u = t.to(torch.bfloat16), u.to(torch.bfloat16).contiguous()
             r = t.shape[1]
             if t.shape != (M, r) or u.shape != (b.rows, r):
                 raise ValueError("low-rank operands must be t[M, r], u[N, r]")
+            # a column slice of a stacked projection is taken as it is by the single-launch path
+            strided_ok = M < 256 and K % 64 == 0 and t.stride(1) == 1 and t.stride(0) % 8 == 0 and t.data_ptr() % 16 == 0
+            if t.is_contiguous() or not strided_ok:
+                t = t.contiguous()
+            else:
+                ldt = t.stride(0)
         bias_f32 = bias is not None and bias.dtype == torch.float32
         if bias is not None:
             bias = bias.contiguous() if bias_f32 else bias.to(torch.bfloat16).contiguous()
@@ -381,7 +410,7 @@ def linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.b
         outs.append(out)
         arr[i] = _lib.LinearMember(b.codes.data_ptr(), b.scales.data_ptr(), b.unit.data_ptr(),
                                    None if t is None else t.data_ptr(), None if u is None else u.data_ptr(), r,
-                                   None if bias is None else bias.data_ptr(), out.data_ptr(), b.rows, int(bias_f32))
+                                   None if bias is None else bias.data_ptr(), out.data_ptr(), b.rows, int(bias_f32), ldt)
     rc = load().metis_linear_fwd_grouped(a.codes.data_ptr(), a.scales.data_ptr(), a.unit.data_ptr(), M, K,
                                          ctypes.cast(arr, ctypes.c_void_p), len(members),
                                          DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16, _stream())

@@ -243,6 +243,23 @@ int metis_linear_wgrad_ws(const void *dyt_codes, const void *dyt_scales, const f
                           void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * Rank-r projection of the low-rank branch for decode-sized batches (M < 256):
+ *     xv[M, R] = x[M, K] . v[R, K]^T   bf16 operands and result, binary32 accumulation
+ *     t [M, R] = bf16(xv * s[R])       when t != NULL
+ * `vlinear(x)` and `torch.mul(self.s, y)` of BitLinear.forward with the bf16 V of the north-star formula
+ * (src/Metis/Metis/bitlinear.py:752-756).  The contraction is cut into up to 32 chunks that run as separate
+ * workgroups (the vendor library walks all of K in one or a few workgroups: 35 us at 64 x 64 x 18944) and a second
+ * kernel adds the chunks in order.  Larger batches are served well by the vendor library.
+ *   x  bf16 [M, K], row stride ldx (% 8 == 0), 16-byte aligned;  v bf16 [R, K] contiguous;  s bf16 [R]
+ *   R % 32 == 0, R <= 256, K % 64 == 0, M < 256 (METIS_E_SHAPE otherwise)
+ *   workspace  metis_lowrank_project_workspace_bytes(M, R, K) bytes, 16-byte aligned, no initialisation
+ */
+size_t metis_lowrank_project_workspace_bytes(int64_t M, int64_t R, int64_t K);
+int metis_lowrank_project(const void *x, int64_t ldx, const void *v, int64_t M, int64_t R, int64_t K,
+                          const void *s, void *xv, void *t, void *workspace, size_t workspace_bytes,
+                          void *stream);
+
+/*
  * One packed activation against several weight matrices in one call: the q/k/v (gate/up) projections of a
  * decoder layer, which the reference quantizes the activation once for (BitLinear._get_shared_quantized_input,
  * src/Metis/Metis/bitlinear.py:676-702) and then multiplies one by one.  Result i equals
@@ -260,6 +277,8 @@ typedef struct metis_linear_member {
     void *out;
     int64_t N;
     int64_t bias_is_f32; /* 0: bias is bf16 [N]; 1: binary32 [N] (metis_linear_fwd_f32bias) */
+    int64_t ldt;         /* row stride of t in elements; 0 = r.  A stride other than r (members reading their columns of
+                            one stacked [M, sum r] projection) needs M < 256 and K % 64 == 0, else METIS_E_ARG */
 } metis_linear_member;
 int metis_linear_fwd_grouped(const void *a_codes, const void *a_scales, const float *a_unit, int64_t M,
                              int64_t K, const metis_linear_member *members, int count, int out_dtype,

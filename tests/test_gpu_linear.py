@@ -312,3 +312,49 @@ def test_config4_full_size_dgrad_and_wgrad():
     # stochastic rounding keeps the gradients unbiased estimates of the dense ones: FP4 noise level, not a parity bar
     assert rel_fro(gx.cpu(), (dy.double() @ w.double()).cpu()) < 0.2
     assert rel_fro(gw.cpu(), (dy.double().T @ x.double()).cpu()) < 0.3
+
+
+@pytest.mark.parametrize("M,K,R", [(64, 3584, 64), (64, 18944, 64), (1, 64, 32), (100, 1536, 96), (255, 8960, 192), (33, 3584, 256)])
+def test_lowrank_projection_for_decode_sized_batches(M, K, R):
+    """x V^T (and its bf16 product with s) on the split-K kernel: one correct bf16 rounding of the double-precision sum;
+    t is the bf16 product of the stored bf16 projection and s, as torch.mul on bf16 tensors."""
+    from metis_hip import ops
+    g = torch.Generator().manual_seed(M + K + R)
+    x = synthetic_activation(70 + M, M, K).cuda()
+    v = (torch.randn(R, K, generator=g) / K ** 0.5).bfloat16().cuda()
+    s = (torch.rand(R, generator=g) * 4 + 0.1).bfloat16().cuda()
+    xv, t = ops.lowrank_project(x, v, s)
+    want = x.double() @ v.double().T
+    torch.cuda.synchronize()
+    assert xv.dtype == torch.bfloat16 and xv.shape == (M, R)
+    d = (xv.double() - want).abs()
+    assert bool((d <= want.abs() * 2.0 ** -8 + 1e-6 * float(want.abs().max())).all())
+    assert torch.equal(t, xv * s)
+    assert torch.equal(ops.lowrank_project(x, v), xv)
+    wide = torch.zeros(M, K + 64, dtype=torch.bfloat16, device="cuda")
+    wide[:, :K] = x
+    assert torch.equal(ops.lowrank_project(wide[:, :K], v), xv)
+    # large batches fall back to the vendor library with the same signature
+    big = torch.randn(300, 128, generator=g).bfloat16().cuda()
+    vb = torch.randn(32, 128, generator=g).bfloat16().cuda()
+    a, b = ops.lowrank_project(big, vb, s[:32])
+    assert torch.equal(a, big @ vb.T) and torch.equal(b, a * s[:32])
+
+
+def test_grouped_members_read_column_slices_of_a_stacked_projection():
+    """t operands that are column slices of one [M, sum r] tensor (row stride sum r) are read in place."""
+    from metis_hip import ops
+    g = torch.Generator().manual_seed(88)
+    M, K, Ns, rs = 64, 1024, (512, 96, 256), (64, 32, 32)
+    px = ops.quantize(synthetic_activation(89, M, K).cuda())
+    stacked = torch.randn(M, sum(rs), generator=g).bfloat16().cuda()
+    members, c0 = [], 0
+    for i, (N, r) in enumerate(zip(Ns, rs)):
+        pw = ops.quantize(_weights(90 + i, N, K).cuda())
+        u = torch.randn(N, r, generator=g).bfloat16().cuda()
+        members.append((pw, stacked[:, c0:c0 + r], u, None))
+        c0 += r
+    assert not members[1][1].is_contiguous()
+    got = ops.linear_fwd_grouped(px, members, out_dtype=torch.float32)
+    for (pw, t, u, _), y in zip(members, got):
+        assert torch.equal(y, ops.linear_fwd(px, pw, t=t.contiguous(), u=u, out_dtype=torch.float32))
