@@ -198,11 +198,17 @@ int metis_linear_fwd_f32bias(const void* a_codes, const void* a_scales, const fl
 }
 
 int metis_linear_fwd_grouped(const void* a_codes, const void* a_scales, const float* a_unit, int64_t M, int64_t K,
-                             const metis_linear_member* members, int count, int out_dtype, void* stream)
+                             const metis_linear_member* members, int count, int out_dtype, void* workspace,
+                             size_t workspace_bytes, void* stream)
 {
     static_assert(sizeof(metis_linear_member) == sizeof(GemmMember), "member layouts must agree");
     return gemm_nvfp4_grouped(a_codes, a_scales, a_unit, M, K, reinterpret_cast<const GemmMember*>(members), count, out_dtype,
-                              (hipStream_t)stream);
+                              (hipStream_t)stream, workspace, workspace_bytes);
+}
+
+size_t metis_linear_grouped_workspace_bytes(int64_t M, int64_t K, const metis_linear_member* members, int count)
+{
+    return gemm_grouped_workspace_bytes(M, K, reinterpret_cast<const GemmMember*>(members), count);
 }
 
 size_t metis_lowrank_project_workspace_bytes(int64_t M, int64_t R, int64_t K) { return lowrank_small_workspace_bytes(M, R, K); }

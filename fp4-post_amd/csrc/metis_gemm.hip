@@ -623,9 +623,15 @@ static int split_factor(int64_t M, int64_t N, int64_t K)
     return s < 1 ? 1 : (int)s;
 }
 
+size_t gemm_grouped_workspace_bytes(int64_t M, int64_t K, const GemmMember* members, int count);
+
 size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K)
 {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
+    if (M < 256) {                                            // skinny kernel
+        const GemmMember g = {nullptr, nullptr, nullptr, nullptr, nullptr, 0, nullptr, nullptr, N, 0, 0};
+        return gemm_grouped_workspace_bytes(M, K, &g, 1);
+    }
     const int s = split_factor(M, N, K);
     if (s <= 1) return 0;
     return (size_t)s * (size_t)(((M + L_BM - 1) / L_BM) * ((N + L_BN - 1) / L_BN)) * L_BM * L_BN * sizeof(float);
@@ -736,7 +742,8 @@ __device__ __forceinline__ void skinny_tile(
     const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const float* __restrict__ a_unit,
     const uint8_t* __restrict__ b_codes, const uint8_t* __restrict__ b_scales, const float* __restrict__ b_unit,
     int M, int N, int K, const uint16_t* __restrict__ t, const uint16_t* __restrict__ u, int r,
-    const uint16_t* __restrict__ bias, void* __restrict__ out, int bias_f32, int n0, int ldt)
+    const uint16_t* __restrict__ bias, void* __restrict__ out, int bias_f32, int n0, int ldt,
+    float* __restrict__ part, int nsplit)
 {
     __shared__ float red[WAVES][TM * 16][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, hi = lane >> 5;
@@ -758,9 +765,13 @@ __device__ __forceinline__ void skinny_tile(
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[i][e] = 0.0f;
 
-    const int iters = K / (64 * C);
-    const int it1 = (wave + 1) * iters / WAVES;
-    for (int it = wave * iters / WAVES; it < it1; ++it) {
+    // K slice of this workgroup (grid z; the whole of K when part == nullptr), dealt to the waves
+    const int iters_all = K / (64 * C);
+    const int slice = part ? (int)blockIdx.z : 0;
+    const int s0 = part ? slice * iters_all / nsplit : 0;
+    const int iters = (part ? (slice + 1) * iters_all / nsplit : iters_all) - s0;
+    const int it1 = s0 + (wave + 1) * iters / WAVES;
+    for (int it = s0 + wave * iters / WAVES; it < it1; ++it) {
         RunRegs<C> rb;
         load_run<C>(rb, bc + (int64_t)it * 32 * C, bs + it * 4 * C);
         RunRegs<C> ra[TM];
@@ -780,8 +791,8 @@ __device__ __forceinline__ void skinny_tile(
     for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[i][e] *= us;
-    // bf16 low-rank extension: slices of 32 columns dealt to the waves
-    for (int j0 = wave * 32; j0 < r; j0 += WAVES * 32) {
+    // bf16 low-rank extension: slices of 32 columns dealt to the waves (K slice 0 only)
+    for (int j0 = wave * 32; j0 < (slice == 0 ? r : 0); j0 += WAVES * 32) {
 #pragma unroll
         for (int q = 0; q < 2; ++q) {
             const int j = j0 + q * 16 + hi * 8;
@@ -809,6 +820,10 @@ __device__ __forceinline__ void skinny_tile(
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[e] += red[w][i * 16 + 4 * g + e][l];
         if (m >= M || n >= N) continue;                        // N % 4 == 0 is required
+        if (part) {                                            // binary32 partial [nsplit][M][N]; the bias waits for the sum
+            *reinterpret_cast<float4*>(part + ((int64_t)slice * M + m) * N + n) = make_float4(v[0], v[1], v[2], v[3]);
+            continue;
+        }
         if (bias)
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[e] += bias_value(bias, bias_f32, n + e);
@@ -823,17 +838,6 @@ __device__ __forceinline__ void skinny_tile(
     }
 }
 
-template <int TM, int C, int WAVES, int OUT_F32>
-__global__ __launch_bounds__(64 * WAVES) void gemm_nvfp4_skinny_kernel(
-    const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const float* __restrict__ a_unit,
-    const uint8_t* __restrict__ b_codes, const uint8_t* __restrict__ b_scales, const float* __restrict__ b_unit,
-    int M, int N, int K, const uint16_t* __restrict__ t, const uint16_t* __restrict__ u, int r,
-    const uint16_t* __restrict__ bias, void* __restrict__ out, int bias_f32)
-{
-    skinny_tile<TM, C, WAVES, OUT_F32>(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, bias_f32,
-                                       (int)blockIdx.x * 32, r);
-}
-
 // Several weight matrices against ONE packed activation in one launch (q/k/v, gate/up): the column tiles of the
 // members are laid end to end along grid x.  A decode-sized k or v projection alone is 16 workgroups and costs a
 // whole launch latency; next to q it is free.
@@ -846,11 +850,12 @@ struct SkinnyMember {
     const uint16_t* u;
     const uint16_t* bias;
     void* out;
+    float* part;                 // split-K partial sums of this member, nullptr when K is not split
     int N, r, tile_end, bias_f32, ldt;
 };
 struct SkinnyGroup {
     SkinnyMember m[kMaxGroupMembers];
-    int count;
+    int count, nsplit;
 };
 
 template <int TM, int C, int WAVES, int OUT_F32>
@@ -869,72 +874,106 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nvfp4_skinny_grouped_kernel(
     for (int i = 1; i < kMaxGroupMembers; ++i)
         if (g == i) mm = grp.m[i];
     skinny_tile<TM, C, WAVES, OUT_F32>(a_codes, a_scales, a_unit, mm.b_codes, mm.b_scales, mm.b_unit, M, mm.N, K, mm.t, mm.u, mm.r,
-                                       mm.bias, mm.out, mm.bias_f32, (tile - start) * 32, mm.ldt);
+                                       mm.bias, mm.out, mm.bias_f32, (tile - start) * 32, mm.ldt, mm.part, grp.nsplit);
 }
 
-template <int TM, int C, int WAVES>
-static int launch_skinny(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes,
-                         const void* b_scales, const float* b_unit, int64_t M, int64_t N, int64_t K, const void* t,
-                         const void* u, int64_t r, const void* bias, void* out, int out_dtype, hipStream_t st, int bias_f32)
+// Adds the K slices of the skinny kernel in ascending order, then bias and output conversion.
+// grid (column quads / 256, M, members).
+template <int OUT_F32>
+__global__ __launch_bounds__(256) void skinny_splitk_reduce_kernel(const SkinnyGroup grp, int M)
 {
-    const dim3 grid((unsigned)((N + 31) / 32), (unsigned)((M + 32 * TM - 1) / (32 * TM))), block(64 * WAVES);
-#define METIS_SK(F) hipLaunchKernelGGL((gemm_nvfp4_skinny_kernel<TM, C, WAVES, F>), grid, block, 0, st, (const uint8_t*)a_codes, \
-                                       (const uint8_t*)a_scales, a_unit, (const uint8_t*)b_codes, (const uint8_t*)b_scales,   \
-                                       b_unit, (int)M, (int)N, (int)K, (const uint16_t*)t, (const uint16_t*)u, (int)r,        \
-                                       (const uint16_t*)bias, out, bias_f32)
-    if (out_dtype == METIS_DTYPE_F32) METIS_SK(1); else METIS_SK(0);
-#undef METIS_SK
-    return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
-}
-
-// Shape heuristics from measurements at 3584/4608/18944-wide projections: wide runs whenever alignment
-// allows; two row tiles per wave when M > 32 unless that leaves fewer workgroups than half the CUs (then the
-// row tiles go to separate workgroups); four waves per workgroup only when there are plenty of
-// workgroups anyway.
-static int gemm_skinny(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes,
-                       const void* b_scales, const float* b_unit, int64_t M, int64_t N, int64_t K, const void* t,
-                       const void* u, int64_t r, const void* bias, void* out, int out_dtype, hipStream_t st, int bias_f32)
-{
-    const bool al8 = ((uintptr_t)a_scales % 8) == 0 && ((uintptr_t)b_scales % 8) == 0;
-    const int c = (K % 256 == 0 && al8) ? 4 : 1;
-    const int64_t tiles_n = (N + 31) / 32;
-    const int tm = (M <= 32 || tiles_n < device_cus() / 2) ? 1 : 2;
-    const int waves = (tm == 1 && M <= 32 && tiles_n >= 2 * device_cus()) ? 4 : 8;
-#define METIS_SKL(TM, C, W) return launch_skinny<TM, C, W>(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st, bias_f32)
-    if (tm == 1) {
-        if (waves == 4) { if (c == 4) METIS_SKL(1, 4, 4); else METIS_SKL(1, 1, 4); }
-        else { if (c == 4) METIS_SKL(1, 4, 8); else METIS_SKL(1, 1, 8); }
-    } else {
-        if (c == 4) METIS_SKL(2, 4, 8); else METIS_SKL(2, 1, 8);
+    SkinnyMember mm = grp.m[0];
+#pragma unroll
+    for (int i = 1; i < kMaxGroupMembers; ++i)
+        if ((int)blockIdx.z == i) mm = grp.m[i];
+    const int n = 4 * (int)(blockIdx.x * 256u + threadIdx.x), m = (int)blockIdx.y;
+    if (n >= mm.N) return;
+    const float* src = mm.part + (int64_t)m * mm.N + n;
+    float4 v = *reinterpret_cast<const float4*>(src);
+    for (int z = 1; z < grp.nsplit; ++z) {
+        const float4 p = *reinterpret_cast<const float4*>(src + (int64_t)z * M * mm.N);
+        v.x += p.x; v.y += p.y; v.z += p.z; v.w += p.w;
     }
-#undef METIS_SKL
+    if (mm.bias) {
+        v.x += bias_value(mm.bias, mm.bias_f32, n);     v.y += bias_value(mm.bias, mm.bias_f32, n + 1);
+        v.z += bias_value(mm.bias, mm.bias_f32, n + 2); v.w += bias_value(mm.bias, mm.bias_f32, n + 3);
+    }
+    if (OUT_F32) {
+        *reinterpret_cast<float4*>((float*)mm.out + (int64_t)m * mm.N + n) = v;
+    } else {
+        uint2 w;
+        w.x = bf16_bits(v.x) | (bf16_bits(v.y) << 16);
+        w.y = bf16_bits(v.z) | (bf16_bits(v.w) << 16);
+        *reinterpret_cast<uint2*>((uint16_t*)mm.out + (int64_t)m * mm.N + n) = w;
+    }
 }
 
 template <int TM, int C, int WAVES>
 static int launch_skinny_grouped(const void* a_codes, const void* a_scales, const float* a_unit, int64_t M, int64_t K,
                                  const SkinnyGroup& grp, int tiles, int out_dtype, hipStream_t st)
 {
-    const dim3 grid((unsigned)tiles, (unsigned)((M + 32 * TM - 1) / (32 * TM))), block(64 * WAVES);
+    const bool split = grp.nsplit > 1;
+    const dim3 grid((unsigned)tiles, (unsigned)((M + 32 * TM - 1) / (32 * TM)), (unsigned)(split ? grp.nsplit : 1)), block(64 * WAVES);
     if (out_dtype == METIS_DTYPE_F32)
         hipLaunchKernelGGL((gemm_nvfp4_skinny_grouped_kernel<TM, C, WAVES, 1>), grid, block, 0, st, (const uint8_t*)a_codes,
                            (const uint8_t*)a_scales, a_unit, (int)M, (int)K, grp);
     else
         hipLaunchKernelGGL((gemm_nvfp4_skinny_grouped_kernel<TM, C, WAVES, 0>), grid, block, 0, st, (const uint8_t*)a_codes,
                            (const uint8_t*)a_scales, a_unit, (int)M, (int)K, grp);
-    return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
+    if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
+    if (split) {
+        int nmax = 0;
+        for (int i = 0; i < grp.count; ++i) nmax = grp.m[i].N > nmax ? grp.m[i].N : nmax;
+        const dim3 rgrid((unsigned)((nmax / 4 + 255) / 256), (unsigned)M, (unsigned)grp.count);
+        if (out_dtype == METIS_DTYPE_F32)
+            hipLaunchKernelGGL(skinny_splitk_reduce_kernel<1>, rgrid, dim3(256), 0, st, grp, (int)M);
+        else
+            hipLaunchKernelGGL(skinny_splitk_reduce_kernel<0>, rgrid, dim3(256), 0, st, grp, (int)M);
+        if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
+    }
+    return METIS_OK;
+}
+
+// K slices for the skinny kernel when its column tiles would leave compute units idle: enough to put two
+// workgroups on every unit, every wave of every slice keeping at least two iterations, at most 8.  1 = no split.
+static int skinny_split_factor(int64_t tiles, int64_t K, int c)
+{
+    const int cus = device_cus();
+    if (cus <= 0 || tiles <= 0 || tiles >= cus) return 1;
+    int64_t s = 2 * (int64_t)cus / tiles;
+    const int64_t iters = K / (64 * c);
+    if (s > iters / 16) s = iters / 16;
+    if (s > 8) s = 8;
+    return s < 1 ? 1 : (int)s;
+}
+
+// Workspace for the partial sums of a grouped call ([slices][M][N] binary32 per member); 0 = K is not split.
+size_t gemm_grouped_workspace_bytes(int64_t M, int64_t K, const GemmMember* members, int count)
+{
+    if (!members || count < 1 || M <= 0 || M >= 256 || K <= 0 || K % 64) return 0;
+    int64_t tiles = 0, ntot = 0;
+    for (int i = 0; i < count; ++i) {
+        if (members[i].N <= 0) return 0;
+        tiles += (members[i].N + 31) / 32;
+        ntot += members[i].N;
+    }
+    const int s1 = skinny_split_factor(tiles, K, 1), s4 = K % 256 == 0 ? skinny_split_factor(tiles, K, 4) : 1;
+    const int s = s1 > s4 ? s1 : s4;                        // which run width applies depends on pointer alignment
+    return s <= 1 ? 0 : (size_t)s * (size_t)M * (size_t)ntot * sizeof(float);
 }
 
 // One activation against up to four weight matrices.  Shapes the skinny kernel does not take fall back to one
 // gemm_nvfp4 call per member (same results either way).
 int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a_unit, int64_t M, int64_t K,
-                       const GemmMember* members, int count, int out_dtype, hipStream_t st)
+                       const GemmMember* members, int count, int out_dtype, hipStream_t st, void* workspace,
+                       size_t workspace_bytes)
 {
     if (!members || count < 1) return METIS_E_ARG;
     bool skinny = M > 0 && M < 256 && K % 64 == 0 && count <= kMaxGroupMembers && !getenv("METIS_GEMM_SMALL") &&
                   a_codes && a_scales && a_unit && !((uintptr_t)a_codes % 16) && !((uintptr_t)a_scales % 2) && K <= INT32_MAX &&
                   (out_dtype == METIS_DTYPE_BF16 || out_dtype == METIS_DTYPE_F32);
     bool al8 = ((uintptr_t)a_scales % 8) == 0;
-    int64_t tiles = 0;
+    int64_t tiles = 0, ntot = 0;
     for (int i = 0; i < count && skinny; ++i) {
         const GemmMember& g = members[i];
         if (!g.b_codes || !g.b_scales || !g.b_unit || !g.out || g.N <= 0 || g.N > INT32_MAX || g.N % 4 || g.r < 0 || g.r % 32 ||
@@ -943,6 +982,7 @@ int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a
             skinny = false;
         al8 = al8 && ((uintptr_t)g.b_scales % 8) == 0;
         tiles += (g.N + 31) / 32;
+        ntot += g.N;
     }
     if (!skinny || tiles > INT32_MAX) {
         for (int i = 0; i < count; ++i) {
@@ -954,28 +994,55 @@ int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a
         }
         return METIS_OK;
     }
+    // Shape heuristics from measurements at 3584/4608/18944-wide projections: wide runs whenever alignment
+    // allows; two row tiles per wave when M > 32 unless that leaves fewer workgroups than half the CUs (then the
+    // row tiles go to separate workgroups); four waves per workgroup only when there are plenty of
+    // workgroups anyway.
+    int c = (K % 256 == 0 && al8) ? 4 : 1;
+    int nsplit = (workspace && !getenv("METIS_GEMM_NOSPLIT")) ? skinny_split_factor(tiles, K, c) : 1;
+    int tm = (M <= 32 || tiles * nsplit < device_cus() / 2) ? 1 : 2;
+    int waves = (tm == 1 && M <= 32 && tiles >= 2 * device_cus()) ? 4 : 8;
+    if (const char* f = getenv("METIS_SKINNY_SHAPE")) {        // measurement switch: "tm,c,waves,slices"
+        int ftm = 0, fc = 0, fw = 0, fs = 0;
+        if (sscanf(f, "%d,%d,%d,%d", &ftm, &fc, &fw, &fs) == 4 && (ftm == 1 || ftm == 2) && (fc == 1 || (fc == 4 && c == 4)) &&
+            (fw == 4 || fw == 8) && fs >= 1 && fs <= 8 && (fs == 1 || workspace) && K / (64 * fc) >= fs) {
+            tm = ftm; c = fc; waves = fw; nsplit = fs;
+        }
+    }
+    if (nsplit > 1 && (((uintptr_t)workspace % 16) || workspace_bytes < (size_t)nsplit * (size_t)M * (size_t)ntot * sizeof(float)))
+        return METIS_E_WORKSPACE;
     SkinnyGroup grp = {};
     grp.count = count;
+    grp.nsplit = nsplit;
     int end = 0;
+    float* part = (float*)workspace;
     for (int i = 0; i < count; ++i) {
         const GemmMember& g = members[i];
         end += (int)((g.N + 31) / 32);
         grp.m[i] = SkinnyMember{(const uint8_t*)g.b_codes, (const uint8_t*)g.b_scales, g.b_unit, (const uint16_t*)g.t,
-                                (const uint16_t*)g.u, (const uint16_t*)g.bias, g.out, (int)g.N, (int)g.r, end, g.bias_is_f32 != 0,
-                                (int)(g.ldt ? g.ldt : g.r)};
+                                (const uint16_t*)g.u, (const uint16_t*)g.bias, g.out, nsplit > 1 ? part : nullptr, (int)g.N,
+                                (int)g.r, end, g.bias_is_f32 != 0, (int)(g.ldt ? g.ldt : g.r)};
+        part += (size_t)nsplit * (size_t)M * (size_t)g.N;
     }
-    // same shape heuristics as gemm_skinny, on the joint column count
-    const int c = (K % 256 == 0 && al8) ? 4 : 1;
-    const int tm = (M <= 32 || tiles < device_cus() / 2) ? 1 : 2;
-    const int waves = (tm == 1 && M <= 32 && tiles >= 2 * device_cus()) ? 4 : 8;
 #define METIS_SKG(TM, C, W) return launch_skinny_grouped<TM, C, W>(a_codes, a_scales, a_unit, M, K, grp, (int)tiles, out_dtype, st)
     if (tm == 1) {
         if (waves == 4) { if (c == 4) METIS_SKG(1, 4, 4); else METIS_SKG(1, 1, 4); }
         else { if (c == 4) METIS_SKG(1, 4, 8); else METIS_SKG(1, 1, 8); }
     } else {
-        if (c == 4) METIS_SKG(2, 4, 8); else METIS_SKG(2, 1, 8);
+        if (waves == 4) { if (c == 4) METIS_SKG(2, 4, 4); else METIS_SKG(2, 1, 4); }
+        else { if (c == 4) METIS_SKG(2, 4, 8); else METIS_SKG(2, 1, 8); }
     }
 #undef METIS_SKG
+}
+
+// The single-matrix call is a group of one.
+static int gemm_skinny(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes,
+                       const void* b_scales, const float* b_unit, int64_t M, int64_t N, int64_t K, const void* t,
+                       const void* u, int64_t r, const void* bias, void* out, int out_dtype, hipStream_t st, int bias_f32,
+                       void* workspace, size_t workspace_bytes)
+{
+    const GemmMember g = {b_codes, b_scales, b_unit, t, u, r, bias, out, N, bias_f32, 0};
+    return gemm_nvfp4_grouped(a_codes, a_scales, a_unit, M, K, &g, 1, out_dtype, st, workspace, workspace_bytes);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1244,7 +1311,8 @@ int gemm_nvfp4(const void* a_codes, const void* a_scales, const float* a_unit, c
                                bias_f32, (float*)workspace, nsplit);
     }
     if (M < 256 && K % 64 == 0 && !getenv("METIS_GEMM_SMALL"))    // up to four 64-row passes over the weights beat a mostly empty 256-row tile
-        return gemm_skinny(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st, bias_f32);
+        return gemm_skinny(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st, bias_f32,
+                           workspace, workspace_bytes);
     constexpr int BM = 128, BN = 128;
     dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM));
     if (out_dtype == METIS_DTYPE_F32)

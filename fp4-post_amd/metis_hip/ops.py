@@ -293,7 +293,7 @@ def _gemm_workspace(M: int, N: int, K: int, device: torch.device) -> torch.Tenso
 
     Taken from torch's caching allocator per call (stream-ordered, so overlapping streams and captured
     graphs each get their own) rather than cached here."""
-    if M < 256 or N < 256:
+    if M >= 256 and N < 256:
         return None
     need = load().metis_linear_workspace_bytes(M, N, K)
     return torch.empty(need, dtype=torch.uint8, device=device) if need else None
@@ -411,9 +411,13 @@ def linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.b
         arr[i] = _lib.LinearMember(b.codes.data_ptr(), b.scales.data_ptr(), b.unit.data_ptr(),
                                    None if t is None else t.data_ptr(), None if u is None else u.data_ptr(), r,
                                    None if bias is None else bias.data_ptr(), out.data_ptr(), b.rows, int(bias_f32), ldt)
-    rc = load().metis_linear_fwd_grouped(a.codes.data_ptr(), a.scales.data_ptr(), a.unit.data_ptr(), M, K,
-                                         ctypes.cast(arr, ctypes.c_void_p), len(members),
-                                         DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16, _stream())
+    L = load()
+    ap = ctypes.cast(arr, ctypes.c_void_p)
+    need = L.metis_linear_grouped_workspace_bytes(M, K, ap, len(members))     # split-K scratch (long K, few columns)
+    ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
+    rc = L.metis_linear_fwd_grouped(a.codes.data_ptr(), a.scales.data_ptr(), a.unit.data_ptr(), M, K, ap, len(members),
+                                    DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16,
+                                    None if ws is None else ws.data_ptr(), need, _stream())
     check(rc, "metis_linear_fwd_grouped", (M, K, [m[0].rows for m in members]))
     return outs
 

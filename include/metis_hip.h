@@ -282,7 +282,12 @@ typedef struct metis_linear_member {
 } metis_linear_member;
 int metis_linear_fwd_grouped(const void *a_codes, const void *a_scales, const float *a_unit, int64_t M,
                              int64_t K, const metis_linear_member *members, int count, int out_dtype,
-                             void *stream);
+                             void *workspace, size_t workspace_bytes, void *stream);
+/* Scratch for the call above: with few output columns and a long K (a down projection at decode size) K is cut
+ * into slices that run as separate workgroups, their binary32 partial sums meet in the workspace and a second
+ * small kernel adds them in a fixed order.  Only the N fields of the members are read.  0 = the shape is not
+ * split; workspace = NULL in the call = never split.  16-byte aligned, contents need no initialisation. */
+size_t metis_linear_grouped_workspace_bytes(int64_t M, int64_t K, const metis_linear_member *members, int count);
 
 /*
  * Mean mode: X^ = 1 me^T + QDQ(X - me), the column mean over tokens kept in high precision and only the

@@ -262,6 +262,47 @@ def test_grouped_projections_equal_member_by_member_calls(M, K, Ns, r):
             assert torch.equal(y, want)
 
 
+@pytest.mark.parametrize("M,K,Ns,r", [(64, 18944, (3584,), 64), (1, 8192, (256,), 0), (200, 16384, (132, 64), 32),
+                                      (33, 8256, (96,), 32)])
+def test_decode_sized_products_with_a_long_contraction_split_k(M, K, Ns, r, monkeypatch):
+    """Few output columns and a long K (a down projection at decode size): K is cut into slices that run as separate
+    workgroups and a second kernel adds the binary32 partial sums.  Checked against the double-precision product of the
+    dequantized operands, against the unsplit kernel (summation order only), and that the shape really is split."""
+    from metis_hip import _lib, ops
+    import ctypes
+    g = torch.Generator().manual_seed(M + K)
+    px = ops.quantize(synthetic_activation(70 + M, M, K).cuda())
+    members = []
+    for i, N in enumerate(Ns):
+        pw = ops.quantize(_weights(71 + i, N, K).cuda())
+        t = u = None
+        if r:
+            t = torch.randn(M, r, generator=g).bfloat16().cuda()
+            u = (torch.randn(N, r, generator=g) * 0.1).bfloat16().cuda()
+        bias = torch.randn(N, generator=g).cuda() if i == 0 else (torch.randn(N, generator=g) * 0.1).bfloat16().cuda()
+        members.append((pw, t, u, bias))
+    arr = (_lib.LinearMember * len(Ns))()
+    for i, N in enumerate(Ns):
+        arr[i].N = N
+    assert _lib.load().metis_linear_grouped_workspace_bytes(M, K, ctypes.cast(arr, ctypes.c_void_p), len(Ns)) > 0
+    da = ops.dequantize(px, torch.float32).double()
+    for dt in (torch.float32, torch.bfloat16):
+        got = ops.linear_fwd_grouped(px, members, out_dtype=dt)
+        single = [ops.linear_fwd(px, pw, t=t, u=u, bias=b, out_dtype=dt) for pw, t, u, b in members]
+        monkeypatch.setenv("METIS_GEMM_NOSPLIT", "1")
+        unsplit = ops.linear_fwd_grouped(px, members, out_dtype=dt)
+        monkeypatch.delenv("METIS_GEMM_NOSPLIT")
+        for (pw, t, u, b), y, y1, y0 in zip(members, got, single, unsplit):
+            want = da @ ops.dequantize(pw, torch.float32).double().T + b.double()
+            if t is not None:
+                want = want + t.double() @ u.double().T
+            tol = 5e-5 if dt == torch.float32 else TOL
+            want = want.cpu().to(dt)                            # a bf16 result is compared after the same final rounding
+            assert rel_fro(y.cpu(), want) <= tol
+            assert rel_fro(y1.cpu(), want) <= tol
+            assert rel_fro(y.float().cpu(), y0.float().cpu()) <= (1e-5 if dt == torch.float32 else TOL)
+
+
 def test_config3_full_size_forward_on_row_and_column_slices():
     """8192 x 4096 x 14336 with r = 64 and bias: the full launch is checked on three row slabs and one column slab
     against the double-precision product of the dequantized operands (the slabs straddle tile and XCD boundaries),
