@@ -267,16 +267,18 @@ __device__ __forceinline__ void tile_origin(int logical, int tiles_m, int tiles_
     n0 = tn * L_BN;
 }
 
-// SPLIT: the grid holds nsplit workgroups per tile, each contracting its own range of K steps; workgroup
-// `logical_all` leaves its binary32 tile (units applied; low-rank term and bias in split 0 only) in
-// ws[logical_all][65536], ordered as the accumulator registers lie, for gemm_splitk_reduce_kernel.
+// SPLIT: tiles nfull .. total-1 have nsplit workgroups each, every one contracting its own range of K steps and
+// leaving its binary32 tile (units applied; low-rank term and bias in split 0 only) in
+// ws[split * (total - nfull) + tile - nfull][65536], ordered as the accumulator registers lie, for
+// gemm_splitk_reduce_kernel.  nfull = 0 splits every tile (shapes with few tiles); nfull > 0 splits only the
+// last, partial round of a shape whose tile count is a little over a multiple of the compute units.
 template <int OUT_F32, int WN_WAVES, int DBG = 0, int SPLIT = 0>
 __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_nvfp4_large_kernel(
     const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const float* __restrict__ a_unit,
     const uint8_t* __restrict__ b_codes, const uint8_t* __restrict__ b_scales, const float* __restrict__ b_unit,
     int M, int N, int K, const uint16_t* __restrict__ t, const uint16_t* __restrict__ u, int r,
     const uint16_t* __restrict__ bias, void* __restrict__ out, int tiles_m, int tiles_n, float* __restrict__ ws,
-    int nsplit, int bias_f32)
+    int nsplit, int bias_f32, int nfull)
 {
     extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
     constexpr int TM = 4;                            // 32-tall MFMA tiles per wave along m
@@ -288,18 +290,33 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_nvfp4_large_kernel(
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN_WAVES, wn = wave % WN_WAVES;
 
-    // ---- tile assignment (XCD-contiguous, grouped)
+    // ---- tile assignment (XCD-contiguous, grouped).  SPLIT: the first nfull tiles (a multiple of 8) run unsplit,
+    //      every XCD its share of them first; the remaining tiles have nsplit workgroups each.
     const int total = tiles_m * tiles_n;
-    const int total_all = SPLIT ? total * nsplit : total;
-    const int per_xcd = (total_all + 7) / 8;
-    const int logical_all = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if (logical_all >= total_all) return;
-    const int split = SPLIT ? logical_all / total : 0;           // consecutive workgroups of an XCD share a K range
+    int logical, split = 0;
+    bool partial = false;
+    if constexpr (SPLIT != 0) {
+        const int xcd = blockIdx.x & 7, li = blockIdx.x >> 3, full_x = nfull >> 3;
+        if (li < full_x) {
+            logical = xcd * full_x + li;
+        } else {
+            const int tail = total - nfull, tail_all = tail * nsplit, per_xcd = (tail_all + 7) / 8;
+            const int j = xcd * per_xcd + (li - full_x);
+            if (li - full_x >= per_xcd || j >= tail_all) return;
+            split = j / tail;                                    // consecutive workgroups of an XCD share a K range
+            logical = nfull + j % tail;
+            partial = true;
+        }
+    } else {
+        const int per_xcd = (total + 7) / 8;
+        logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+        if (logical >= total) return;
+    }
     int m0, n0;
-    tile_origin(SPLIT ? logical_all % total : logical_all, tiles_m, tiles_n, m0, n0);
+    tile_origin(logical, tiles_m, tiles_n, m0, n0);
     const int steps_all = K / BK;
-    const int step_begin = SPLIT ? (int)((int64_t)split * steps_all / nsplit) : 0;
-    const int step_end = SPLIT ? (int)((int64_t)(split + 1) * steps_all / nsplit) : steps_all;
+    const int step_begin = partial ? (int)((int64_t)split * steps_all / nsplit) : 0;
+    const int step_end = partial ? (int)((int64_t)(split + 1) * steps_all / nsplit) : steps_all;
 
     float16_t acc[TM][TN];
 #pragma unroll
@@ -446,8 +463,8 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_nvfp4_large_kernel(
         __syncthreads();
     }
 
-    if constexpr (SPLIT != 0) {
-        float* wt = ws + (size_t)logical_all * (L_BM * L_BN) + tid * 4;
+    if (SPLIT != 0 && partial) {
+        float* wt = ws + (size_t)(split * (total - nfull) + (logical - nfull)) * (L_BM * L_BN) + tid * 4;
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -538,16 +555,16 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_nvfp4_large_kernel(
 // the GEMM wrote, 1 KiB per instruction, and add the splits in ascending order.
 template <int OUT_F32>
 __global__ __launch_bounds__(64) void gemm_splitk_reduce_kernel(const float* __restrict__ ws, int nsplit, int M, int N,
-                                                                int tiles_m, int tiles_n, void* __restrict__ out)
+                                                                int tiles_m, int tiles_n, void* __restrict__ out, int nfull)
 {
     constexpr int TN = 2, WTN = 64, NTHREADS = 512, TILE = L_BM * L_BN;
     __shared__ __attribute__((aligned(16))) uint16_t cw[32 * 72];
-    const int total = tiles_m * tiles_n;
+    const int total = tiles_m * tiles_n - nfull;                 // split tiles
     const int tile = blockIdx.x >> 5, wave = (blockIdx.x >> 2) & 7, i = blockIdx.x & 3;
     const int lane = threadIdx.x, tid = wave * 64 + lane;
     const int wm = wave / 4, wn = wave % 4;
     int m0, n0;
-    tile_origin(tile, tiles_m, tiles_n, m0, n0);
+    tile_origin(nfull + tile, tiles_m, tiles_n, m0, n0);
     const int mbase = m0 + wm * 128 + i * 32, nbase = n0 + wn * WTN;
     if (mbase >= M || nbase >= N) return;
 
@@ -609,18 +626,33 @@ __global__ __launch_bounds__(64) void gemm_splitk_reduce_kernel(const float* __r
         }
 }
 
-// Splits of K for a tiled GEMM that would leave more than half of the compute units without a tile:
-// as many as fill the device once, at least 8 K steps (512 elements) each, at most 16.  1 = do not split.
-static int split_factor(int64_t M, int64_t N, int64_t K)
+// Splits of K for a tiled GEMM.  A shape that would leave more than half of the compute units without a tile is
+// split whole: as many workgroups per tile as fill the device once, at least 8 K steps (512 elements) each, at
+// most 16.  A shape whose last round of tiles covers at most half of the units has only those tiles split; the
+// full rounds before it run unsplit (up to four of them: measured gains 6-28 % at 1-4 full rounds, a loss of 2 % at
+// nine, where the rounds have drifted apart enough to hide the tail anyway).  nsplit = 1: do not split.
+struct SplitPlan {
+    int nsplit;
+    int nfull;                   // leading tiles that run unsplit (a multiple of the compute units)
+};
+static SplitPlan split_plan(int64_t M, int64_t N, int64_t K)
 {
-    if (M < L_BM || N < L_BN || K % BK) return 1;
+    const SplitPlan none = {1, 0};
+    if (M < L_BM || N < L_BN || K % BK) return none;
     const int64_t tiles = ((M + L_BM - 1) / L_BM) * ((N + L_BN - 1) / L_BN);
     const int cus = device_cus();
-    if (cus <= 0 || tiles * 2 > cus) return 1;
-    int64_t s = cus / tiles;
+    if (cus <= 0 || cus % 8 || tiles > INT32_MAX) return none;
+    int64_t part = tiles, nfull = 0;                            // tiles to split
+    if (tiles * 2 > cus) {
+        part = tiles % cus;
+        nfull = tiles - part;
+        if (tiles < cus || part == 0 || part * 2 > cus || nfull > 4 * (int64_t)cus || getenv("METIS_GEMM_NOTAIL")) return none;
+    }
+    int64_t s = cus / part;
     if (s > K / BK / 8) s = K / BK / 8;
     if (s > 16) s = 16;
-    return s < 1 ? 1 : (int)s;
+    if (s < 2) return none;
+    return SplitPlan{(int)s, (int)nfull};
 }
 
 size_t gemm_grouped_workspace_bytes(int64_t M, int64_t K, const GemmMember* members, int count);
@@ -632,9 +664,10 @@ size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K)
         const GemmMember g = {nullptr, nullptr, nullptr, nullptr, nullptr, 0, nullptr, nullptr, N, 0, 0};
         return gemm_grouped_workspace_bytes(M, K, &g, 1);
     }
-    const int s = split_factor(M, N, K);
-    if (s <= 1) return 0;
-    return (size_t)s * (size_t)(((M + L_BM - 1) / L_BM) * ((N + L_BN - 1) / L_BN)) * L_BM * L_BN * sizeof(float);
+    const SplitPlan p = split_plan(M, N, K);
+    if (p.nsplit <= 1) return 0;
+    const int64_t tiles = ((M + L_BM - 1) / L_BM) * ((N + L_BN - 1) / L_BN);
+    return (size_t)p.nsplit * (size_t)(tiles - p.nfull) * L_BM * L_BN * sizeof(float);
 }
 
 // Dynamic LDS above 64 KiB has to be allowed per kernel function and per device: done once for each pair.
@@ -653,13 +686,14 @@ template <int WN_WAVES>
 static int launch_large(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes,
                         const void* b_scales, const float* b_unit, int64_t M, int64_t N, int64_t K, const void* t,
                         const void* u, int64_t r, const void* bias, void* out, int out_dtype, hipStream_t st,
-                        int bias_f32 = 0, float* ws = nullptr, int nsplit = 1)
+                        int bias_f32 = 0, float* ws = nullptr, int nsplit = 1, int nfull = 0)
 {
-    static bool attr_set[3][64] = {};
+    static bool attr_set[4][64] = {};
     const size_t lds_bytes = 2 * (size_t)L_STAGE_HALVES * sizeof(uint16_t);
     const bool split = WN_WAVES == 4 && ws && nsplit > 1;
     const int f32 = out_dtype == METIS_DTYPE_F32;
-    const void* fn = split ? (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 0, WN_WAVES == 4>
+    const void* fn = split ? (f32 ? (const void*)gemm_nvfp4_large_kernel<1, WN_WAVES, 0, WN_WAVES == 4>
+                                  : (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 0, WN_WAVES == 4>)
                    : f32   ? (const void*)gemm_nvfp4_large_kernel<1, WN_WAVES>
                            : (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES>;
     const char* d = getenv("METIS_GEMM_DBG");                  // measurement switches, results are meaningless:
@@ -667,28 +701,30 @@ static int launch_large(const void* a_codes, const void* a_scales, const float* 
     if (v == 1 || v == 7) {
         fn = v == 1 ? (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 1> : (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 7>;
         if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess) return METIS_E_DEVICE;
-    } else if (const int rc = allow_dynamic_lds(fn, lds_bytes, attr_set[split ? 2 : f32])) {
+    } else if (const int rc = allow_dynamic_lds(fn, lds_bytes, attr_set[(split ? 2 : 0) + f32])) {
         return rc;
     }
     const int tiles_m = (int)((M + L_BM - 1) / L_BM), tiles_n = (int)((N + L_BN - 1) / L_BN);
     const int total = tiles_m * tiles_n;
-    if (!split) nsplit = 1;
-    const unsigned grid_x = (unsigned)(((total * nsplit + 7) / 8) * 8);
+    if (!split) { nsplit = 1; nfull = 0; }
+    // per XCD: its share of the unsplit tiles, then its share of the split ones
+    const unsigned grid_x = split ? 8u * (unsigned)(nfull / 8 + ((total - nfull) * nsplit + 7) / 8)
+                                  : (unsigned)(((total + 7) / 8) * 8);
     const uint8_t *ac = (const uint8_t*)a_codes, *as = (const uint8_t*)a_scales, *bc = (const uint8_t*)b_codes,
                   *bs = (const uint8_t*)b_scales;
     const uint16_t *tp = (const uint16_t*)t, *up = (const uint16_t*)u, *bp = (const uint16_t*)bias;
     int Mi = (int)M, Ni = (int)N, Ki = (int)K, ri = (int)r, tmi = tiles_m, tni = tiles_n;
-    void* args[] = {&ac, &as, &a_unit, &bc, &bs, &b_unit, &Mi, &Ni, &Ki, &tp, &up, &ri, &bp, &out, &tmi, &tni, &ws, &nsplit, &bias_f32};
+    void* args[] = {&ac, &as, &a_unit, &bc, &bs, &b_unit, &Mi, &Ni, &Ki, &tp, &up, &ri, &bp, &out, &tmi, &tni, &ws, &nsplit, &bias_f32, &nfull};
     if (hipLaunchKernel(fn, dim3(grid_x), dim3(128 * WN_WAVES), args, lds_bytes, st) != hipSuccess) {
         (void)hipGetLastError();
         return METIS_E_LAUNCH;
     }
     if (split) {
-        const dim3 rgrid((unsigned)total * 32u);
+        const dim3 rgrid((unsigned)(total - nfull) * 32u);
         if (f32)
-            hipLaunchKernelGGL(gemm_splitk_reduce_kernel<1>, rgrid, dim3(64), 0, st, ws, nsplit, Mi, Ni, tmi, tni, out);
+            hipLaunchKernelGGL(gemm_splitk_reduce_kernel<1>, rgrid, dim3(64), 0, st, ws, nsplit, Mi, Ni, tmi, tni, out, nfull);
         else
-            hipLaunchKernelGGL(gemm_splitk_reduce_kernel<0>, rgrid, dim3(64), 0, st, ws, nsplit, Mi, Ni, tmi, tni, out);
+            hipLaunchKernelGGL(gemm_splitk_reduce_kernel<0>, rgrid, dim3(64), 0, st, ws, nsplit, Mi, Ni, tmi, tni, out, nfull);
         if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
     }
     return METIS_OK;
@@ -1302,13 +1338,13 @@ int gemm_nvfp4(const void* a_codes, const void* a_scales, const float* a_unit, c
     if (M >= 256 && N >= 256 && K % BK == 0 && !getenv("METIS_GEMM_SMALL")) {
         if (getenv("METIS_GEMM_W4"))
             return launch_large<2>(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st, bias_f32);
-        int nsplit = 1;
+        SplitPlan plan = {1, 0};
         if (workspace && !getenv("METIS_GEMM_NOSPLIT")) {
-            nsplit = split_factor(M, N, K);
-            if (nsplit > 1 && (((uintptr_t)workspace % 16) || workspace_bytes < gemm_workspace_bytes(M, N, K))) return METIS_E_WORKSPACE;
+            plan = split_plan(M, N, K);
+            if (plan.nsplit > 1 && (((uintptr_t)workspace % 16) || workspace_bytes < gemm_workspace_bytes(M, N, K))) return METIS_E_WORKSPACE;
         }
         return launch_large<4>(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st,
-                               bias_f32, (float*)workspace, nsplit);
+                               bias_f32, (float*)workspace, plan.nsplit, plan.nfull);
     }
     if (M < 256 && K % 64 == 0 && !getenv("METIS_GEMM_SMALL"))    // up to four 64-row passes over the weights beat a mostly empty 256-row tile
         return gemm_skinny(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st, bias_f32,

@@ -185,6 +185,44 @@ def test_split_k_shapes(M, N, K, r, monkeypatch):
     assert rel_fro(got32.cpu(), whole32.cpu()) <= 1e-5
 
 
+@pytest.mark.parametrize("M,N,K,r", [(4096, 4352, 1024, 32), (4100, 4004, 2112, 0), (4096, 8960, 1536, 64)])
+def test_split_k_of_the_last_partial_round(M, N, K, r, monkeypatch):
+    """A tile count a little over a multiple of the compute units (272 or 560 tiles on 256 units): the full rounds
+    run unsplit and write the output directly, only the tiles of the last round are split through the workspace.
+    Both kinds of tile are checked against the double-precision product and against the unsplit kernel."""
+    from metis_hip import _lib, ops
+    tiles = ((M + 255) // 256) * ((N + 255) // 256)
+    need = _lib.load().metis_linear_workspace_bytes(M, N, K)
+    assert 0 < need < tiles * 256 * 256 * 4                    # fewer partial tiles than two per output tile
+    g = torch.Generator().manual_seed(95)
+    x = synthetic_activation(52 + M, M, K).cuda()
+    w = _weights(53 + N, N, K).cuda()
+    t = u = None
+    if r:
+        t = torch.randn(M, r, generator=g).bfloat16().cuda()
+        u = torch.randn(N, r, generator=g).bfloat16().cuda()
+    bias = (torch.randn(N, generator=g) * 0.1).bfloat16().cuda()
+    px, pw = ops.quantize(x), ops.quantize(w)
+    got = ops.linear_fwd(px, pw, t=t, u=u, bias=bias)
+    got32 = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, out_dtype=torch.float32)
+    want = ops.dequantize(px, torch.float32).double() @ ops.dequantize(pw, torch.float32).double().T
+    if r:
+        want = want + t.double() @ u.double().T
+    want = want + bias.double()
+    torch.cuda.synchronize()
+    assert rel_fro(got32.cpu(), want.cpu()) <= 1e-5
+    assert rel_fro(got.cpu(), want.cpu().bfloat16()) <= TOL
+    monkeypatch.setenv("METIS_GEMM_NOSPLIT", "1")
+    whole32 = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, out_dtype=torch.float32)
+    whole = ops.linear_fwd(px, pw, t=t, u=u, bias=bias)
+    torch.cuda.synchronize()
+    # the unsplit tiles are bit-identical to the unsplit kernel, the split ones differ in summation order only
+    same = (got32 == whole32).float().mean().item()
+    assert 0.5 < same < 1.0 or same == 1.0
+    assert rel_fro(got32.cpu(), whole32.cpu()) <= 1e-5
+    assert (got != whole).float().mean().item() < 0.01
+
+
 def test_split_k_dgrad_wgrad_and_workspace_errors():
     from metis_hip import _lib, ops
     L, N, K = 512, 2048, 512
