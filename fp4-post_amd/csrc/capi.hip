@@ -206,6 +206,20 @@ int metis_linear_fwd_grouped(const void* a_codes, const void* a_scales, const fl
                               (hipStream_t)stream, workspace, workspace_bytes);
 }
 
+int metis_linear_fwd_grouped_centered(const void* a_codes, const void* a_scales, const float* a_unit, int64_t M, int64_t K,
+                                      const metis_linear_member* members, int count, int out_dtype, const float* center,
+                                      void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (!center) return METIS_E_ARG;
+    return gemm_nvfp4_grouped(a_codes, a_scales, a_unit, M, K, reinterpret_cast<const GemmMember*>(members), count, out_dtype,
+                              (hipStream_t)stream, workspace, workspace_bytes, center);
+}
+
+int metis_linear_grouped_centered_supported(int64_t M, int64_t K, const metis_linear_member* members, int count, int have_workspace)
+{
+    return gemm_grouped_center_supported(M, K, reinterpret_cast<const GemmMember*>(members), count, have_workspace);
+}
+
 size_t metis_linear_grouped_workspace_bytes(int64_t M, int64_t K, const metis_linear_member* members, int count)
 {
     return gemm_grouped_workspace_bytes(M, K, reinterpret_cast<const GemmMember*>(members), count);

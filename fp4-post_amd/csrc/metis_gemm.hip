@@ -773,15 +773,19 @@ __device__ __forceinline__ half8_t run_operand(const RunRegs<C>& r, int m)
     return __builtin_bit_cast(half8_t, expand8(w, scale_pair(byte)));
 }
 
-template <int TM, int C, int WAVES, int OUT_F32>
+// CEN: the activation is a centred residual, X^ = 1 me^T + R (mean mode).  The workgroup's slice of the binary32
+// centre me is staged in LDS (in the reduction buffer, idle during the main loop) and every lane accumulates
+// sum_k B[n, k] me[k] for its weight row next to the MFMAs, from the operand it has just expanded: the packed
+// weight is read once for R W^T and for the rank-one term 1 (W^ me)^T.
+template <int TM, int C, int WAVES, int OUT_F32, int CEN = 0>
 __device__ __forceinline__ void skinny_tile(
     const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const float* __restrict__ a_unit,
     const uint8_t* __restrict__ b_codes, const uint8_t* __restrict__ b_scales, const float* __restrict__ b_unit,
     int M, int N, int K, const uint16_t* __restrict__ t, const uint16_t* __restrict__ u, int r,
     const uint16_t* __restrict__ bias, void* __restrict__ out, int bias_f32, int n0, int ldt,
-    float* __restrict__ part, int nsplit)
+    float* __restrict__ part, int nsplit, const float* __restrict__ center = nullptr)
 {
-    __shared__ float red[WAVES][TM * 16][64];
+    __shared__ __attribute__((aligned(16))) float red[WAVES][TM * 16][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, hi = lane >> 5;
     const int m0 = blockIdx.y * 32 * TM;
     const int kbytes = K / 2, kblocks = K / kBlock;
@@ -807,6 +811,15 @@ __device__ __forceinline__ void skinny_tile(
     const int s0 = part ? slice * iters_all / nsplit : 0;
     const int iters = (part ? (slice + 1) * iters_all / nsplit : iters_all) - s0;
     const int it1 = s0 + (wave + 1) * iters / WAVES;
+    float* mes = &red[0][0][0];
+    float ys[4] = {0.0f, 0.0f, 0.0f, 0.0f};                    // CEN: sum_k B[n, k] me[k] over this lane's share of K (four chains)
+    if constexpr (CEN != 0) {                                  // the host has checked that the slice fits
+        const int klen = iters * 64 * C;
+        const float* src = center + (int64_t)s0 * 64 * C;
+        for (int k = threadIdx.x * 4; k < klen; k += 64 * WAVES * 4)
+            *reinterpret_cast<float4*>(mes + k) = *reinterpret_cast<const float4*>(src + k);
+        __syncthreads();
+    }
     for (int it = s0 + wave * iters / WAVES; it < it1; ++it) {
         RunRegs<C> rb;
         load_run<C>(rb, bc + (int64_t)it * 32 * C, bs + it * 4 * C);
@@ -816,6 +829,14 @@ __device__ __forceinline__ void skinny_tile(
 #pragma unroll
         for (int m = 0; m < 4 * C; ++m) {
             const half8_t fb = run_operand<C>(rb, m);
+            if constexpr (CEN != 0) {                          // the lane's run starts at element hi * 32 C of the iteration
+                const float* mp = mes + (it - s0) * 64 * C + hi * 32 * C + 8 * m;
+                const float4 c0 = *reinterpret_cast<const float4*>(mp), c1 = *reinterpret_cast<const float4*>(mp + 4);
+                ys[0] = fmaf((float)fb[0], c0.x, ys[0]); ys[1] = fmaf((float)fb[1], c0.y, ys[1]);
+                ys[2] = fmaf((float)fb[2], c0.z, ys[2]); ys[3] = fmaf((float)fb[3], c0.w, ys[3]);
+                ys[0] = fmaf((float)fb[4], c1.x, ys[0]); ys[1] = fmaf((float)fb[5], c1.y, ys[1]);
+                ys[2] = fmaf((float)fb[6], c1.z, ys[2]); ys[3] = fmaf((float)fb[7], c1.w, ys[3]);
+            }
 #pragma unroll
             for (int i = 0; i < TM; ++i)
                 acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb, run_operand<C>(ra[i], m), acc[i], 0, 0, 0);
@@ -827,6 +848,21 @@ __device__ __forceinline__ void skinny_tile(
     for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[i][e] *= us;
+    if constexpr (CEN != 0) {
+        // the rank-one term: every output row gets W^ me.  Lane l holds the sum of weight row l % 32 over its half
+        // of each iteration; the expanded operand carries 2^-8 and lacks the tensor unit.  Each wave adds its own
+        // share of K to its partial accumulators, so the sum over waves (and K slices) completes it.
+        const float ysum = (ys[0] + ys[1]) + (ys[2] + ys[3]);
+        float yt = ysum + __shfl_xor(ysum, 32);
+        yt *= (*b_unit) * 256.0f;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const float yv = __shfl(yt, 8 * (e >> 2) + 4 * hi + (e & 3));
+#pragma unroll
+            for (int i = 0; i < TM; ++i) acc[i][e] += yv;
+        }
+        __syncthreads();                                       // all waves are done with the staged centre: red is free
+    }
     // bf16 low-rank extension: slices of 32 columns dealt to the waves (K slice 0 only)
     for (int j0 = wave * 32; j0 < (slice == 0 ? r : 0); j0 += WAVES * 32) {
 #pragma unroll
@@ -892,9 +928,10 @@ struct SkinnyMember {
 struct SkinnyGroup {
     SkinnyMember m[kMaxGroupMembers];
     int count, nsplit;
+    const float* center;         // mean mode: binary32 [K], see skinny_tile
 };
 
-template <int TM, int C, int WAVES, int OUT_F32>
+template <int TM, int C, int WAVES, int OUT_F32, int CEN = 0>
 __global__ __launch_bounds__(64 * WAVES) void gemm_nvfp4_skinny_grouped_kernel(
     const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const float* __restrict__ a_unit, int M, int K,
     const SkinnyGroup grp)
@@ -909,8 +946,9 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nvfp4_skinny_grouped_kernel(
 #pragma unroll
     for (int i = 1; i < kMaxGroupMembers; ++i)
         if (g == i) mm = grp.m[i];
-    skinny_tile<TM, C, WAVES, OUT_F32>(a_codes, a_scales, a_unit, mm.b_codes, mm.b_scales, mm.b_unit, M, mm.N, K, mm.t, mm.u, mm.r,
-                                       mm.bias, mm.out, mm.bias_f32, (tile - start) * 32, mm.ldt, mm.part, grp.nsplit);
+    skinny_tile<TM, C, WAVES, OUT_F32, CEN>(a_codes, a_scales, a_unit, mm.b_codes, mm.b_scales, mm.b_unit, M, mm.N, K, mm.t, mm.u,
+                                            mm.r, mm.bias, mm.out, mm.bias_f32, (tile - start) * 32, mm.ldt, mm.part, grp.nsplit,
+                                            grp.center);
 }
 
 // Adds the K slices of the skinny kernel in ascending order, then bias and output conversion.
@@ -944,12 +982,37 @@ __global__ __launch_bounds__(256) void skinny_splitk_reduce_kernel(const SkinnyG
     }
 }
 
+static int launch_skinny_reduce(const SkinnyGroup& grp, int64_t M, int out_dtype, hipStream_t st)
+{
+    int nmax = 0;
+    for (int i = 0; i < grp.count; ++i) nmax = grp.m[i].N > nmax ? grp.m[i].N : nmax;
+    const dim3 rgrid((unsigned)((nmax / 4 + 255) / 256), (unsigned)M, (unsigned)grp.count);
+    if (out_dtype == METIS_DTYPE_F32)
+        hipLaunchKernelGGL(skinny_splitk_reduce_kernel<1>, rgrid, dim3(256), 0, st, grp, (int)M);
+    else
+        hipLaunchKernelGGL(skinny_splitk_reduce_kernel<0>, rgrid, dim3(256), 0, st, grp, (int)M);
+    return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
+}
+
 template <int TM, int C, int WAVES>
 static int launch_skinny_grouped(const void* a_codes, const void* a_scales, const float* a_unit, int64_t M, int64_t K,
                                  const SkinnyGroup& grp, int tiles, int out_dtype, hipStream_t st)
 {
     const bool split = grp.nsplit > 1;
     const dim3 grid((unsigned)tiles, (unsigned)((M + 32 * TM - 1) / (32 * TM)), (unsigned)(split ? grp.nsplit : 1)), block(64 * WAVES);
+    if constexpr (C == 4) {
+        if (grp.center) {                                      // mean mode (wide runs only)
+            if (out_dtype == METIS_DTYPE_F32)
+                hipLaunchKernelGGL((gemm_nvfp4_skinny_grouped_kernel<TM, C, WAVES, 1, 1>), grid, block, 0, st, (const uint8_t*)a_codes,
+                                   (const uint8_t*)a_scales, a_unit, (int)M, (int)K, grp);
+            else
+                hipLaunchKernelGGL((gemm_nvfp4_skinny_grouped_kernel<TM, C, WAVES, 0, 1>), grid, block, 0, st, (const uint8_t*)a_codes,
+                                   (const uint8_t*)a_scales, a_unit, (int)M, (int)K, grp);
+            if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
+            return split ? launch_skinny_reduce(grp, M, out_dtype, st) : METIS_OK;
+        }
+    }
+    if (grp.center) return METIS_E_ARG;
     if (out_dtype == METIS_DTYPE_F32)
         hipLaunchKernelGGL((gemm_nvfp4_skinny_grouped_kernel<TM, C, WAVES, 1>), grid, block, 0, st, (const uint8_t*)a_codes,
                            (const uint8_t*)a_scales, a_unit, (int)M, (int)K, grp);
@@ -957,17 +1020,7 @@ static int launch_skinny_grouped(const void* a_codes, const void* a_scales, cons
         hipLaunchKernelGGL((gemm_nvfp4_skinny_grouped_kernel<TM, C, WAVES, 0>), grid, block, 0, st, (const uint8_t*)a_codes,
                            (const uint8_t*)a_scales, a_unit, (int)M, (int)K, grp);
     if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
-    if (split) {
-        int nmax = 0;
-        for (int i = 0; i < grp.count; ++i) nmax = grp.m[i].N > nmax ? grp.m[i].N : nmax;
-        const dim3 rgrid((unsigned)((nmax / 4 + 255) / 256), (unsigned)M, (unsigned)grp.count);
-        if (out_dtype == METIS_DTYPE_F32)
-            hipLaunchKernelGGL(skinny_splitk_reduce_kernel<1>, rgrid, dim3(256), 0, st, grp, (int)M);
-        else
-            hipLaunchKernelGGL(skinny_splitk_reduce_kernel<0>, rgrid, dim3(256), 0, st, grp, (int)M);
-        if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
-    }
-    return METIS_OK;
+    return split ? launch_skinny_reduce(grp, M, out_dtype, st) : METIS_OK;
 }
 
 // K slices for the skinny kernel when its column tiles would leave compute units idle: enough to put two
@@ -1000,11 +1053,49 @@ size_t gemm_grouped_workspace_bytes(int64_t M, int64_t K, const GemmMember* memb
 
 // One activation against up to four weight matrices.  Shapes the skinny kernel does not take fall back to one
 // gemm_nvfp4 call per member (same results either way).
+// Shape chosen for a grouped call on the skinny kernel: run width, row tiles per wave, waves, K slices.
+struct SkinnyShape {
+    int c, tm, waves, nsplit;
+};
+static SkinnyShape skinny_shape(int64_t M, int64_t K, int64_t tiles, bool al8, bool have_workspace)
+{
+    // Shape heuristics from measurements at 3584/4608/18944-wide projections: wide runs whenever alignment
+    // allows; two row tiles per wave when M > 32 unless that leaves fewer workgroups than half the CUs (then the
+    // row tiles go to separate workgroups); four waves per workgroup only when there are plenty of
+    // workgroups anyway.
+    SkinnyShape s;
+    s.c = (K % 256 == 0 && al8) ? 4 : 1;
+    s.nsplit = (have_workspace && !getenv("METIS_GEMM_NOSPLIT")) ? skinny_split_factor(tiles, K, s.c) : 1;
+    s.tm = (M <= 32 || tiles * s.nsplit < device_cus() / 2) ? 1 : 2;
+    s.waves = (s.tm == 1 && M <= 32 && tiles >= 2 * device_cus()) ? 4 : 8;
+    return s;
+}
+// mean mode inside the skinny kernel: wide runs, and the workgroup's slice of the centre must fit the LDS reduction buffer
+static bool skinny_center_fits(const SkinnyShape& s, int64_t K)
+{
+    const int64_t iters = K / (64 * s.c), slice = ((iters + s.nsplit - 1) / s.nsplit) * 64 * s.c;
+    return s.c == 4 && slice <= (int64_t)s.waves * s.tm * 16 * 64;
+}
+
+// 1 when a grouped call of this shape can take a centre (mean mode in one pass over the weights), else 0: the caller
+// then adds W^ me as a binary32 bias computed with packed_gemv.  Scale-byte pointers are assumed 8-byte aligned.
+int gemm_grouped_center_supported(int64_t M, int64_t K, const GemmMember* members, int count, int have_workspace)
+{
+    if (!members || count < 1 || count > 4 || M <= 0 || M >= 256 || K <= 0 || K % 64 || getenv("METIS_GEMM_SMALL")) return 0;
+    int64_t tiles = 0;
+    for (int i = 0; i < count; ++i) {
+        if (members[i].N <= 0 || members[i].N % 4) return 0;
+        tiles += (members[i].N + 31) / 32;
+    }
+    return skinny_center_fits(skinny_shape(M, K, tiles, true, have_workspace != 0), K) ? 1 : 0;
+}
+
 int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a_unit, int64_t M, int64_t K,
                        const GemmMember* members, int count, int out_dtype, hipStream_t st, void* workspace,
-                       size_t workspace_bytes)
+                       size_t workspace_bytes, const float* center)
 {
     if (!members || count < 1) return METIS_E_ARG;
+    if ((uintptr_t)center % 16) return METIS_E_ARG;
     bool skinny = M > 0 && M < 256 && K % 64 == 0 && count <= kMaxGroupMembers && !getenv("METIS_GEMM_SMALL") &&
                   a_codes && a_scales && a_unit && !((uintptr_t)a_codes % 16) && !((uintptr_t)a_scales % 2) && K <= INT32_MAX &&
                   (out_dtype == METIS_DTYPE_BF16 || out_dtype == METIS_DTYPE_F32);
@@ -1021,6 +1112,7 @@ int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a
         ntot += g.N;
     }
     if (!skinny || tiles > INT32_MAX) {
+        if (center) return METIS_E_ARG;                        // the centre is only taken by the single-launch path
         for (int i = 0; i < count; ++i) {
             const GemmMember& g = members[i];
             if (g.ldt != 0 && g.ldt != g.r) return METIS_E_ARG;   // a strided t is only taken by the single-launch path
@@ -1030,14 +1122,8 @@ int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a
         }
         return METIS_OK;
     }
-    // Shape heuristics from measurements at 3584/4608/18944-wide projections: wide runs whenever alignment
-    // allows; two row tiles per wave when M > 32 unless that leaves fewer workgroups than half the CUs (then the
-    // row tiles go to separate workgroups); four waves per workgroup only when there are plenty of
-    // workgroups anyway.
-    int c = (K % 256 == 0 && al8) ? 4 : 1;
-    int nsplit = (workspace && !getenv("METIS_GEMM_NOSPLIT")) ? skinny_split_factor(tiles, K, c) : 1;
-    int tm = (M <= 32 || tiles * nsplit < device_cus() / 2) ? 1 : 2;
-    int waves = (tm == 1 && M <= 32 && tiles >= 2 * device_cus()) ? 4 : 8;
+    const SkinnyShape shape = skinny_shape(M, K, tiles, al8, workspace != nullptr);
+    int c = shape.c, nsplit = shape.nsplit, tm = shape.tm, waves = shape.waves;
     if (const char* f = getenv("METIS_SKINNY_SHAPE")) {        // measurement switch: "tm,c,waves,slices"
         int ftm = 0, fc = 0, fw = 0, fs = 0;
         if (sscanf(f, "%d,%d,%d,%d", &ftm, &fc, &fw, &fs) == 4 && (ftm == 1 || ftm == 2) && (fc == 1 || (fc == 4 && c == 4)) &&
@@ -1047,9 +1133,11 @@ int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a
     }
     if (nsplit > 1 && (((uintptr_t)workspace % 16) || workspace_bytes < (size_t)nsplit * (size_t)M * (size_t)ntot * sizeof(float)))
         return METIS_E_WORKSPACE;
+    if (center && !skinny_center_fits(SkinnyShape{c, tm, waves, nsplit}, K)) return METIS_E_ARG;
     SkinnyGroup grp = {};
     grp.count = count;
     grp.nsplit = nsplit;
+    grp.center = center;
     int end = 0;
     float* part = (float*)workspace;
     for (int i = 0; i < count; ++i) {
@@ -1078,7 +1166,7 @@ static int gemm_skinny(const void* a_codes, const void* a_scales, const float* a
                        void* workspace, size_t workspace_bytes)
 {
     const GemmMember g = {b_codes, b_scales, b_unit, t, u, r, bias, out, N, bias_f32, 0};
-    return gemm_nvfp4_grouped(a_codes, a_scales, a_unit, M, K, &g, 1, out_dtype, st, workspace, workspace_bytes);
+    return gemm_nvfp4_grouped(a_codes, a_scales, a_unit, M, K, &g, 1, out_dtype, st, workspace, workspace_bytes, nullptr);
 }
 
 // ---------------------------------------------------------------------------------------------

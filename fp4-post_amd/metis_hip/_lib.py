@@ -57,6 +57,8 @@ SIGNATURES = {
     "metis_lowrank_project": (_i32, [_vp, _i64, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _sz, _vp]),
     "metis_linear_fwd_grouped": (_i32, [_vp, _vp, _vp, _i64, _i64, _vp, _i32, _i32, _vp, _sz, _vp]),
     "metis_linear_grouped_workspace_bytes": (_sz, [_i64, _i64, _vp, _i32]),
+    "metis_linear_fwd_grouped_centered": (_i32, [_vp, _vp, _vp, _i64, _i64, _vp, _i32, _i32, _vp, _vp, _sz, _vp]),
+    "metis_linear_grouped_centered_supported": (_i32, [_i64, _i64, _vp, _i32, _i32]),
     "metis_linear_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "metis_linear_fwd_ws": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _i32, _vp, _sz, _vp]),
     "metis_linear_dgrad_ws": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i32, _vp, _sz, _vp]),

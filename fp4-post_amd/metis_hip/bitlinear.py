@@ -716,15 +716,13 @@ class BitLinear(nn.Module):
         for m, p_res in zip(members, packed):
             r = m.args.forward_svd_rank
             bias = m.warmup_linear.bias
-            if centre is not None:                              # mean mode: bias + W^ me in binary32
-                w_mean = ops.matvec(p_res, centre)
-                bias = w_mean if bias is None else w_mean + bias.float()
-            elif bias is not None:
-                bias = bias.to(cd)
+            if bias is not None:
+                bias = bias.float() if centre is not None else bias.to(cd)
             calls.append((p_res, t_all[:, c0:c0 + r], m.ulinear.weight.to(cd), bias))      # a column slice: no copy
             c0 += r
         out_dtype = torch.float32 if F.compute_dtype == torch.float32 else torch.bfloat16
-        outs = ops.linear_fwd_grouped(px, calls, out_dtype=out_dtype)
+        # mean mode: every member also receives W^ me, inside the same launch (binary32)
+        outs = ops.linear_fwd_grouped(px, calls, out_dtype=out_dtype, center=centre)
         lead = x.shape[:-1]
         return {id(m): y.reshape(*lead, y.shape[-1]).to(F.compute_dtype) for m, y in zip(members, outs)}
 

@@ -379,9 +379,13 @@ def lowrank_project(x2: torch.Tensor, v: torch.Tensor, s: torch.Tensor | None = 
     return xv if s is None else (xv, t)
 
 
-def linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.bfloat16) -> list[torch.Tensor]:
+def linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.bfloat16,
+                       center: torch.Tensor | None = None) -> list[torch.Tensor]:
     """[linear_fwd(a, b, t=t, u=u, bias=bias) for (b, t, u, bias) in members] in one call: a projection group
-    (q/k/v, gate/up) that shares one packed activation.  Decode-sized batches run as a single launch."""
+    (q/k/v, gate/up) that shares one packed activation.  Decode-sized batches run as a single launch.
+
+    center (mean mode: `a` packs the centred residual X - center): every output row also receives deq(b) . center,
+    inside the same launch where the shape allows, else through matvec and a binary32 bias."""
     import ctypes
     M, K = a.rows, a.cols
     dev = a.codes.device
@@ -415,9 +419,26 @@ def linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.b
     ap = ctypes.cast(arr, ctypes.c_void_p)
     need = L.metis_linear_grouped_workspace_bytes(M, K, ap, len(members))     # split-K scratch (long K, few columns)
     ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
+    dt = DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16
+    if center is not None:
+        center = center.reshape(-1).to(device=dev, dtype=torch.float32).contiguous()
+        if center.numel() != K:
+            raise ValueError(f"center must have {K} values, got {center.numel()}")
+        aligned = center.data_ptr() % 16 == 0 and all(m[0].scales.data_ptr() % 8 == 0 for m in members) and a.scales.data_ptr() % 8 == 0
+        if aligned and L.metis_linear_grouped_centered_supported(M, K, ap, len(members), int(need > 0)):
+            rc = L.metis_linear_fwd_grouped_centered(a.codes.data_ptr(), a.scales.data_ptr(), a.unit.data_ptr(), M, K, ap,
+                                                     len(members), dt, center.data_ptr(),
+                                                     None if ws is None else ws.data_ptr(), need, _stream())
+            check(rc, "metis_linear_fwd_grouped_centered", (M, K, [m[0].rows for m in members]))
+            return outs
+        # two passes: W^ center as a binary32 bias per member
+        shifted = []
+        for b, t, u, bias in members:
+            w_mean = matvec(b, center)
+            shifted.append((b, t, u, w_mean if bias is None else w_mean + bias.float()))
+        return linear_fwd_grouped(a, shifted, out_dtype)
     rc = L.metis_linear_fwd_grouped(a.codes.data_ptr(), a.scales.data_ptr(), a.unit.data_ptr(), M, K, ap, len(members),
-                                    DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16,
-                                    None if ws is None else ws.data_ptr(), need, _stream())
+                                    dt, None if ws is None else ws.data_ptr(), need, _stream())
     check(rc, "metis_linear_fwd_grouped", (M, K, [m[0].rows for m in members]))
     return outs
 

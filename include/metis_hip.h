@@ -288,6 +288,20 @@ int metis_linear_fwd_grouped(const void *a_codes, const void *a_scales, const fl
  * small kernel adds them in a fixed order.  Only the N fields of the members are read.  0 = the shape is not
  * split; workspace = NULL in the call = never split.  16-byte aligned, contents need no initialisation. */
 size_t metis_linear_grouped_workspace_bytes(int64_t M, int64_t K, const metis_linear_member *members, int count);
+/* Mean mode for decode-sized batches in one pass over the weights (BitLinear.forward under the reference's default
+ * arguments, bitlinear.py:311-336 with the running mean of 316-323): the packed activation holds the centred
+ * residual R = Q(X - me) and every output row additionally receives W^ me, accumulated in binary32 inside the
+ * GEMM kernel from the weight operands it expands anyway (center: binary32 [K], 16-byte aligned):
+ *     out_g = R . W^_g^T + 1 (W^_g center)^T + t_g u_g^T + bias_g.
+ * Same result as metis_nvfp4_matvec + metis_linear_fwd_f32bias to binary32 summation order, without reading the
+ * packed weights a second time.  Shapes: those for which ..._supported returns 1 (M < 256, K % 256 == 0, at most
+ * four members, scale pointers 8-byte aligned, and the K range of a workgroup small enough for its LDS: K <= 8192
+ * unsplit, longer with the workspace); METIS_E_ARG otherwise. */
+int metis_linear_fwd_grouped_centered(const void *a_codes, const void *a_scales, const float *a_unit, int64_t M,
+                                      int64_t K, const metis_linear_member *members, int count, int out_dtype,
+                                      const float *center, void *workspace, size_t workspace_bytes, void *stream);
+int metis_linear_grouped_centered_supported(int64_t M, int64_t K, const metis_linear_member *members, int count,
+                                            int have_workspace);
 
 /*
  * Mean mode: X^ = 1 me^T + QDQ(X - me), the column mean over tokens kept in high precision and only the

@@ -124,6 +124,53 @@ def _oracle_mean_qdq(x32):
     return me + O.nvfp4_qdq(x32 - me)
 
 
+@pytest.mark.parametrize("M,K,Ns,r,one_pass", [(64, 3584, (3584, 512, 512), 64, True), (64, 18944, (3584,), 64, True),
+                                               (1, 1024, (256, 96), 0, True), (40, 8192, (100,), 32, True),
+                                               (200, 512, (260, 64), 32, True), (8, 8448, (8192,), 0, False),
+                                               (16, 320, (128,), 0, False)])
+def test_grouped_decode_gemm_with_the_centre_inside(M, K, Ns, r, one_pass):
+    """Mean mode at decode size: out = R W^T + 1 (W^ me)^T + t u^T + bias with W^ me accumulated inside the GEMM
+    launch.  Checked against double precision and against the two-pass form (packed matvec, then a binary32 bias);
+    shapes whose centre slice does not fit the kernel (or K % 256 != 0) take the two-pass form by themselves."""
+    import ctypes
+    from metis_hip import _lib, ops
+    g = torch.Generator().manual_seed(M + K)
+    x = _offset_activation(600 + M, M, K).cuda()
+    me = x.float().mean(dim=0) + 0.01 * torch.randn(K, generator=g).cuda()      # a running mean is not the batch mean
+    px = ops.quantize(x, 0, center=me)
+    members = []
+    for i, N in enumerate(Ns):
+        pw = ops.quantize((torch.randn(N, K, generator=g) * 0.05).bfloat16().cuda())
+        t = u = None
+        if r and i != 1:
+            t = torch.randn(M, r, generator=g).bfloat16().cuda()
+            u = (torch.randn(N, r, generator=g) * 0.1).bfloat16().cuda()
+        bias = torch.randn(N, generator=g).cuda() if i % 2 == 0 else None
+        members.append((pw, t, u, bias))
+    arr = (_lib.LinearMember * len(Ns))()
+    for i, N in enumerate(Ns):
+        arr[i].N = N
+    ap = ctypes.cast(arr, ctypes.c_void_p)
+    L = _lib.load()
+    has_ws = L.metis_linear_grouped_workspace_bytes(M, K, ap, len(Ns)) > 0
+    assert bool(L.metis_linear_grouped_centered_supported(M, K, ap, len(Ns), int(has_ws))) == one_pass
+    dr = ops.dequantize(px, torch.float32).double()
+    for dt in (torch.float32, torch.bfloat16):
+        got = ops.linear_fwd_grouped(px, members, out_dtype=dt, center=me)
+        for (pw, t, u, b), y in zip(members, got):
+            dw = ops.dequantize(pw, torch.float32).double()
+            want = (dr + me.double()) @ dw.T
+            if t is not None:
+                want = want + t.double() @ u.double().T
+            if b is not None:
+                want = want + b.double()
+            two_pass = ops.linear_fwd(px, pw, t=t, u=u, out_dtype=dt,
+                                      bias=ops.matvec(pw, me) if b is None else ops.matvec(pw, me) + b)
+            tol = 5e-5 if dt == torch.float32 else 2e-3
+            assert rel_fro(y.cpu(), want.cpu().to(dt)) <= tol
+            assert rel_fro(y.float().cpu(), two_pass.float().cpu()) <= (1e-5 if dt == torch.float32 else 2e-3)
+
+
 def test_linear_lowbit_mean_mode_forward_runs_packed_and_matches_oracle(monkeypatch):
     """LinearLowbit under the reference's default arguments: mean + QDQ(x - mean) against QDQ(W), on the
     packed kernels (no dequantized activation or weight is ever formed)."""
