@@ -160,6 +160,16 @@ int metis_column_mean(const void* x, int64_t rows, int64_t cols, int64_t ld, int
                        workspace_bytes, (hipStream_t)stream);
 }
 
+int metis_column_mean_running(const void* x, int64_t rows, int64_t cols, int64_t ld, int x_dtype, const void* cached,
+                              int64_t cached_count, void* out, float* out32, int out_dtype, void* workspace, size_t workspace_bytes,
+                              void* stream)
+{
+    if ((x_dtype != METIS_DTYPE_BF16 && x_dtype != METIS_DTYPE_F32) || (out_dtype != METIS_DTYPE_BF16 && out_dtype != METIS_DTYPE_F32))
+        return METIS_E_ARG;
+    return column_mean(x, rows, cols, ld, x_dtype == METIS_DTYPE_F32, out, out_dtype == METIS_DTYPE_BF16, workspace,
+                       workspace_bytes, (hipStream_t)stream, false, cached, cached_count, out32);
+}
+
 int metis_column_sum(const void* x, int64_t rows, int64_t cols, int64_t ld, int x_dtype, void* out, int out_dtype,
                      void* workspace, size_t workspace_bytes, void* stream)
 {

@@ -21,6 +21,7 @@
 namespace metis {
 
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
@@ -774,9 +775,11 @@ __device__ __forceinline__ half8_t run_operand(const RunRegs<C>& r, int m)
 }
 
 // CEN: the activation is a centred residual, X^ = 1 me^T + R (mean mode).  The workgroup's slice of the binary32
-// centre me is staged in LDS (in the reduction buffer, idle during the main loop) and every lane accumulates
-// sum_k B[n, k] me[k] for its weight row next to the MFMAs, from the operand it has just expanded: the packed
-// weight is read once for R W^T and for the rank-one term 1 (W^ me)^T.
+// centre me is staged in LDS (in the reduction buffer, idle during the main loop) as binary16 pairs hi + lo
+// (22 significant bits, prescaled by 2^-4: |me| < 2^20) and enters as one more MFMA per step against the weight
+// operand that has just been expanded: a pseudo activation tile whose even rows are hi and odd rows lo.  The packed
+// weight is read once for R W^T and for the rank-one term 1 (W^ me)^T, at the cost of half as many MFMAs again
+// on a kernel that is bound elsewhere.
 template <int TM, int C, int WAVES, int OUT_F32, int CEN = 0>
 __device__ __forceinline__ void skinny_tile(
     const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const float* __restrict__ a_unit,
@@ -812,12 +815,26 @@ __device__ __forceinline__ void skinny_tile(
     const int iters = (part ? (slice + 1) * iters_all / nsplit : iters_all) - s0;
     const int it1 = s0 + (wave + 1) * iters / WAVES;
     float* mes = &red[0][0][0];
-    float ys[4] = {0.0f, 0.0f, 0.0f, 0.0f};                    // CEN: sum_k B[n, k] me[k] over this lane's share of K (four chains)
+    float16_t accm;                                            // CEN: the pseudo tile (even lanes: B . hi, odd lanes: B . lo)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) accm[e] = 0.0f;
     if constexpr (CEN != 0) {                                  // the host has checked that the slice fits
+        // 32 bytes per 8 elements: [hi x 8 | lo x 8]
         const int klen = iters * 64 * C;
         const float* src = center + (int64_t)s0 * 64 * C;
-        for (int k = threadIdx.x * 4; k < klen; k += 64 * WAVES * 4)
-            *reinterpret_cast<float4*>(mes + k) = *reinterpret_cast<const float4*>(src + k);
+        for (int k = threadIdx.x * 4; k < klen; k += 64 * WAVES * 4) {
+            const float4 f = *reinterpret_cast<const float4*>(src + k);
+            const float v[4] = {f.x * 0.0625f, f.y * 0.0625f, f.z * 0.0625f, f.w * 0.0625f};
+            half4_t h, l;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                h[j] = (_Float16)v[j];
+                l[j] = (_Float16)(v[j] - (float)h[j]);
+            }
+            char* d = reinterpret_cast<char*>(mes) + (k >> 3) * 32 + ((k >> 2) & 1) * 8;
+            *reinterpret_cast<uint2*>(d) = __builtin_bit_cast(uint2, h);
+            *reinterpret_cast<uint2*>(d + 16) = __builtin_bit_cast(uint2, l);
+        }
         __syncthreads();
     }
     for (int it = s0 + wave * iters / WAVES; it < it1; ++it) {
@@ -830,12 +847,8 @@ __device__ __forceinline__ void skinny_tile(
         for (int m = 0; m < 4 * C; ++m) {
             const half8_t fb = run_operand<C>(rb, m);
             if constexpr (CEN != 0) {                          // the lane's run starts at element hi * 32 C of the iteration
-                const float* mp = mes + (it - s0) * 64 * C + hi * 32 * C + 8 * m;
-                const float4 c0 = *reinterpret_cast<const float4*>(mp), c1 = *reinterpret_cast<const float4*>(mp + 4);
-                ys[0] = fmaf((float)fb[0], c0.x, ys[0]); ys[1] = fmaf((float)fb[1], c0.y, ys[1]);
-                ys[2] = fmaf((float)fb[2], c0.z, ys[2]); ys[3] = fmaf((float)fb[3], c0.w, ys[3]);
-                ys[0] = fmaf((float)fb[4], c1.x, ys[0]); ys[1] = fmaf((float)fb[5], c1.y, ys[1]);
-                ys[2] = fmaf((float)fb[6], c1.z, ys[2]); ys[3] = fmaf((float)fb[7], c1.w, ys[3]);
+                const uint4* mp = reinterpret_cast<const uint4*>(mes) + ((((it - s0) * 64 * C + hi * 32 * C) >> 3) + m) * 2 + (lane & 1);
+                accm = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb, __builtin_bit_cast(half8_t, *mp), accm, 0, 0, 0);
             }
 #pragma unroll
             for (int i = 0; i < TM; ++i)
@@ -849,15 +862,14 @@ __device__ __forceinline__ void skinny_tile(
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[i][e] *= us;
     if constexpr (CEN != 0) {
-        // the rank-one term: every output row gets W^ me.  Lane l holds the sum of weight row l % 32 over its half
-        // of each iteration; the expanded operand carries 2^-8 and lacks the tensor unit.  Each wave adds its own
-        // share of K to its partial accumulators, so the sum over waves (and K slices) completes it.
-        const float ysum = (ys[0] + ys[1]) + (ys[2] + ys[3]);
-        float yt = ysum + __shfl_xor(ysum, 32);
-        yt *= (*b_unit) * 256.0f;
+        // the rank-one term: every output row gets W^ me.  accm[e] holds it for this lane's column n(e), split over
+        // the lane pair (hi part, lo part); the expanded operand carries 2^-8, the centre 2^-4, and the tensor unit
+        // is missing.  Each wave adds its own share of K to its partial accumulators, so the sum over waves (and
+        // K slices) completes it.
+        const float ys = (*b_unit) * 4096.0f;
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-            const float yv = __shfl(yt, 8 * (e >> 2) + 4 * hi + (e & 3));
+            const float yv = (accm[e] + __shfl_xor(accm[e], 1)) * ys;
 #pragma unroll
             for (int i = 0; i < TM; ++i) acc[i][e] += yv;
         }

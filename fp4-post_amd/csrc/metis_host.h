@@ -92,7 +92,8 @@ size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 // me[c] = mean over rows of x[:, c] (binary32 accumulation); nvfp4_gemv.hip
 size_t column_mean_workspace_bytes(int64_t cols);
 int column_mean(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_f32, void* out, int out_bf16, void* workspace,
-                size_t workspace_bytes, hipStream_t st, bool sum_only = false);
+                size_t workspace_bytes, hipStream_t st, bool sum_only = false, const void* cached = nullptr,
+                int64_t cached_count = 0, float* out32 = nullptr);
 
 // xv[M, R] = x[M, K] . v[R, K]^T (bf16, binary32 accumulation) and t = bf16(xv * s) for M < 256; lowrank_small.hip
 size_t lowrank_small_workspace_bytes(int64_t M, int64_t R, int64_t K);

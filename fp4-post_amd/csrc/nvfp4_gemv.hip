@@ -233,9 +233,14 @@ __global__ __launch_bounds__(256) void column_sum_kernel(const void* __restrict_
     }
 }
 
+// cached (optional, same type as out): the weighted running mean of single-token decode calls,
+//     me = (cached * cached_count + this_mean * rows) / (cached_count + rows)
+// with every operation rounded to the output type as the reference's tensor expression does
+// (src/Metis/Metis/bitlinear.py:316-323; true division, as on the CPU).  out32 (optional): the result once more as binary32.
 template <bool OUT_BF16>
 __global__ __launch_bounds__(64) void column_mean_finish_kernel(const float* __restrict__ partial, uint32_t slabs, uint32_t cols,
-                                                                 float count, void* __restrict__ out)
+                                                                 float count, void* __restrict__ out, const void* __restrict__ cached,
+                                                                 float cached_count, float rows_f, float* __restrict__ out32)
 {
     const uint32_t c = blockIdx.x * 64u + threadIdx.x;
     if (c >= cols) return;
@@ -246,16 +251,26 @@ __global__ __launch_bounds__(64) void column_mean_finish_kernel(const float* __r
     float s = 0.0f;
 #pragma unroll
     for (uint32_t k = 0; k < (uint32_t)kMeanMaxSlabs; ++k) s += v[k];
-    const float m = s / count;
+    auto rnd = [](float x) { return OUT_BF16 ? __uint_as_float(bf16_bits(x) << 16) : x; };
+    float m = rnd(s / count);
+    if (cached) {
+        const float cm = OUT_BF16 ? __uint_as_float((uint32_t)static_cast<const uint16_t*>(cached)[c] << 16)
+                                  : static_cast<const float*>(cached)[c];
+        const float a = rnd(cm * cached_count), b = rnd(m * rows_f);
+        m = rnd(rnd(a + b) / (cached_count + rows_f));
+    }
     if (OUT_BF16) static_cast<uint16_t*>(out)[c] = (uint16_t)bf16_bits(m);
     else static_cast<float*>(out)[c] = m;
+    if (out32) out32[c] = m;
 }
 
 size_t column_mean_workspace_bytes(int64_t cols) { return cols > 0 ? (size_t)kMeanMaxSlabs * (size_t)cols * sizeof(float) : 0; }
 
 int column_mean(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_f32, void* out, int out_bf16, void* workspace,
-                size_t workspace_bytes, hipStream_t st, bool sum_only)
+                size_t workspace_bytes, hipStream_t st, bool sum_only, const void* cached, int64_t cached_count, float* out32)
 {
+    if (cached && (sum_only || cached_count < 0 || cached_count > (1 << 24) || ((uintptr_t)cached % (out_bf16 ? 2 : 4)))) return METIS_E_ARG;
+    if ((uintptr_t)out32 % 4) return METIS_E_ARG;
     if (rows <= 0 || cols <= 0 || ld < cols) return METIS_E_ARG;
     if (cols % 4 || ld % 4) return METIS_E_SHAPE;
     if (!x || !out) return METIS_E_ARG;
@@ -278,9 +293,11 @@ int column_mean(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_f3
         hipLaunchKernelGGL(column_sum_kernel<false>, grid, dim3(256), 0, st, x, (uint32_t)rows, (uint32_t)cols, ld, partial, rows_per_slab);
     const dim3 g2((unsigned)((cols + 63) / 64));
     if (out_bf16)
-        hipLaunchKernelGGL(column_mean_finish_kernel<true>, g2, dim3(64), 0, st, partial, (uint32_t)slabs, (uint32_t)cols, sum_only ? 1.0f : (float)rows, out);
+        hipLaunchKernelGGL(column_mean_finish_kernel<true>, g2, dim3(64), 0, st, partial, (uint32_t)slabs, (uint32_t)cols,
+                           sum_only ? 1.0f : (float)rows, out, cached, (float)cached_count, (float)rows, out32);
     else
-        hipLaunchKernelGGL(column_mean_finish_kernel<false>, g2, dim3(64), 0, st, partial, (uint32_t)slabs, (uint32_t)cols, sum_only ? 1.0f : (float)rows, out);
+        hipLaunchKernelGGL(column_mean_finish_kernel<false>, g2, dim3(64), 0, st, partial, (uint32_t)slabs, (uint32_t)cols,
+                           sum_only ? 1.0f : (float)rows, out, cached, (float)cached_count, (float)rows, out32);
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 

@@ -50,6 +50,7 @@ SIGNATURES = {
     "metis_rank_one_operands": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp]),
     "metis_column_mean_workspace_bytes": (_sz, [_i64]),
     "metis_column_mean": (_i32, [_vp, _i64, _i64, _i64, _i32, _vp, _i32, _vp, _sz, _vp]),
+    "metis_column_mean_running": (_i32, [_vp, _i64, _i64, _i64, _i32, _vp, _i64, _vp, _vp, _i32, _vp, _sz, _vp]),
     "metis_column_sum": (_i32, [_vp, _i64, _i64, _i64, _i32, _vp, _i32, _vp, _sz, _vp]),
     "metis_nvfp4_matvec": (_i32, [_vp, _vp, _vp, _i64, _i64, _vp, _f32, _vp, _vp, _i64, _i32, _vp]),
     "metis_linear_fwd_f32bias": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _i32, _vp, _sz, _vp]),

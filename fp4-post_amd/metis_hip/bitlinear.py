@@ -234,21 +234,31 @@ class LinearLowbitFunction(torch.autograd.Function):
         """Column mean over tokens in the compute dtype ([C]); single-token decode calls update a weighted
         running mean per cache key instead (reference 311-329).  The cache holds ([1, C] mean, count) as the
         reference's does."""
+        return LinearLowbitFunction._token_mean2(input_, mean_cache, cache_key)[0]
+
+    @staticmethod
+    def _token_mean2(input_: torch.Tensor, mean_cache=None, cache_key="default"):
+        """(mean in the compute dtype, the same values as float32 or None).  On the device the reduction and the
+        running update are one reduction kernel and one small kernel."""
         cd = LinearLowbitFunction.compute_dtype
         flat = _flat2d(input_)
         rows = flat.shape[0]
+        seq_len = input_.shape[1] if input_.dim() == 3 else input_.shape[0]
+        running = seq_len == 1 and mean_cache is not None and cache_key in mean_cache
+        cached_mean, cached_count = mean_cache[cache_key] if running else (None, 0)
         if flat.is_cuda and flat.dtype in (torch.float32, torch.bfloat16) and flat.shape[1] % 4 == 0 and \
-                cd in (torch.float32, torch.bfloat16):
+                cd in (torch.float32, torch.bfloat16) and cached_count + rows <= 2 ** 24:
             # one pass over the tensor; a bf16 tensor is read as it is in either arithmetic
             src = flat if (cd == torch.float32 or flat.dtype == torch.bfloat16) else flat.to(cd)
-            this_mean = ops.column_mean(src, out_dtype=cd).unsqueeze(0)
-        elif cd == torch.float32:
+            me, me32 = ops.column_mean_running(src, cached_mean, cached_count, out_dtype=cd)
+            if mean_cache is not None:
+                mean_cache[cache_key] = (me.detach().unsqueeze(0), cached_count + rows)
+            return me, me32
+        if cd == torch.float32:
             this_mean = flat.mean(dim=0, keepdim=True, dtype=torch.float32)
         else:
             this_mean = flat.to(cd).mean(dim=0, keepdim=True)
-        seq_len = input_.shape[1] if input_.dim() == 3 else input_.shape[0]
-        if seq_len == 1 and mean_cache is not None and cache_key in mean_cache:
-            cached_mean, cached_count = mean_cache[cache_key]
+        if running:
             new_count = cached_count + rows
             me = (cached_mean * cached_count + this_mean * rows) / new_count
             mean_cache[cache_key] = (me.detach(), new_count)
@@ -256,7 +266,7 @@ class LinearLowbitFunction(torch.autograd.Function):
             me = this_mean
             if mean_cache is not None:
                 mean_cache[cache_key] = (me.detach(), rows)
-        return me.reshape(-1)
+        return me.reshape(-1), None
 
     @staticmethod
     def _mean_mode_packable() -> bool:
@@ -275,8 +285,8 @@ class LinearLowbitFunction(torch.autograd.Function):
             if F._mean_mode_packable():
                 # mean + QDQ(x - mean) (reference 311-336) without materialising either: the subtraction happens
                 # inside the quantizer and the mean's contribution to a matmul is a rank-one term
-                me = F._token_mean(input_, mean_cache=mean_cache, cache_key=cache_key)
-                return CenteredNVFP4(F.q_forward_input.pack(_flat2d(input_), arith=F.compute_dtype, center=me), me)
+                me, me32 = F._token_mean2(input_, mean_cache=mean_cache, cache_key=cache_key)
+                return CenteredNVFP4(F.q_forward_input.pack(_flat2d(input_), arith=F.compute_dtype, center=me), me, me32)
         return F.quantize_input(input_, mean_cache=mean_cache, cache_key=cache_key)
 
     @staticmethod
@@ -508,12 +518,19 @@ class _MetisFusedFunction(torch.autograd.Function):
         ctx.center = None
         gemm_bias = None if bias is None else bias.to(cd)
         if isinstance(px, CenteredNVFP4):
-            # mean mode: the residual branch sees 1 me^T + R, whose mean term rides in a binary32 bias
+            # mean mode: the residual branch sees 1 me^T + R
             ctx.center = px.mean
-            w_mean = ops.matvec(p_res, px.mean)
-            gemm_bias = w_mean if bias is None else w_mean + bias.float()
-            px = px.residual
-        y = ops.linear_fwd(px, p_res, t=t, u=u.to(cd), bias=gemm_bias, out_dtype=out_dtype)
+            if px.rows < 256:
+                # decode-sized: W^ me is accumulated inside the GEMM launch
+                y = ops.linear_fwd_grouped(px.residual, [(p_res, t, u.to(cd), None if bias is None else bias.float())],
+                                           out_dtype=out_dtype, center=px.center32)[0]
+            else:
+                # the mean term rides in a binary32 bias
+                w_mean = ops.matvec(p_res, px.center32)
+                y = ops.linear_fwd(px.residual, p_res, t=t, u=u.to(cd), bias=w_mean if bias is None else w_mean + bias.float(),
+                                   out_dtype=out_dtype)
+        else:
+            y = ops.linear_fwd(px, p_res, t=t, u=u.to(cd), bias=gemm_bias, out_dtype=out_dtype)
         ctx.save_for_backward(x, v, s, u, res, xv)
         ctx.p_res = p_res
         ctx.has_bias = bias is not None
@@ -710,14 +727,14 @@ class BitLinear(nn.Module):
                       torch.cat([m.s.to(cd) for m in members], dim=0))
             group["stacked_v"] = cached
         _, t_all = ops.lowrank_project(x2, cached[1], cached[2])
-        centre = shared_input.mean if isinstance(shared_input, CenteredNVFP4) else None
+        centre = shared_input.center32 if isinstance(shared_input, CenteredNVFP4) else None
         px = shared_input.residual if centre is not None else shared_input
         calls, c0 = [], 0
         for m, p_res in zip(members, packed):
             r = m.args.forward_svd_rank
             bias = m.warmup_linear.bias
             if bias is not None:
-                bias = bias.float() if centre is not None else bias.to(cd)
+                bias = m._bias_as(torch.float32 if centre is not None else cd)
             calls.append((p_res, t_all[:, c0:c0 + r], m.ulinear.weight.to(cd), bias))      # a column slice: no copy
             c0 += r
         out_dtype = torch.float32 if F.compute_dtype == torch.float32 else torch.bfloat16
@@ -725,6 +742,18 @@ class BitLinear(nn.Module):
         outs = ops.linear_fwd_grouped(px, calls, out_dtype=out_dtype, center=centre)
         lead = x.shape[:-1]
         return {id(m): y.reshape(*lead, y.shape[-1]).to(F.compute_dtype) for m, y in zip(members, outs)}
+
+    def _bias_as(self, dtype: torch.dtype) -> torch.Tensor:
+        """The residual branch's bias in `dtype`, converted once per parameter version (decode calls are launch-bound)."""
+        b = self.warmup_linear.bias
+        if b.dtype == dtype:
+            return b
+        key = (b._version, b.device, dtype)
+        cached = getattr(self, "_bias_cast_cache", None)
+        if cached is None or cached[0] != key:
+            cached = (key, b.detach().to(dtype))
+            self._bias_cast_cache = cached
+        return cached[1]
 
     # ------------------------------------------------------------------ forward (reference 736-769)
     def forward(self, x: torch.Tensor) -> torch.Tensor:

@@ -44,6 +44,11 @@ class CenteredNVFP4:
     bf16 [cols] in bf16 arithmetic."""
     residual: PackedNVFP4
     mean: torch.Tensor
+    mean32: torch.Tensor | None = None       # the same values as float32 when the producer had them at hand
+
+    @property
+    def center32(self) -> torch.Tensor:
+        return self.mean32 if self.mean32 is not None else self.mean
 
     @property
     def rows(self) -> int:
@@ -188,6 +193,35 @@ def column_mean(x: torch.Tensor, out_dtype: torch.dtype = torch.float32, _sum_on
             out.data_ptr(), DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16, ws.data_ptr(), ws.numel(), _stream())
     check(rc, "metis_column_sum" if _sum_only else "metis_column_mean", x.shape)
     return out
+
+
+def column_mean_running(x: torch.Tensor, cached: torch.Tensor | None, cached_count: int,
+                        out_dtype: torch.dtype = torch.float32) -> tuple[torch.Tensor, torch.Tensor]:
+    """(me, me as float32) with me = (cached * cached_count + mean(x) * rows) / (cached_count + rows), each operation
+    rounded to out_dtype (cached None: me = mean(x)).  One reduction and one small kernel; in float32 both results
+    are the same tensor."""
+    if not x.is_cuda:
+        raise _lib.MetisHipError("metis_hip ops need a ROCm device tensor; there is no CPU path")
+    if x.dtype not in (torch.bfloat16, torch.float32) or out_dtype not in (torch.bfloat16, torch.float32):
+        raise ValueError("column_mean_running: bfloat16 or float32 tensors only")
+    x2 = x.reshape(-1, x.shape[-1])
+    if not x2.is_contiguous():
+        x2 = x2.contiguous()
+    rows, cols = x2.shape
+    if cached is not None:
+        cached = cached.reshape(-1).to(device=x2.device, dtype=out_dtype).contiguous()
+        if cached.numel() != cols:
+            raise ValueError(f"cached mean has {cached.numel()} values, the tensor {cols} columns")
+    out = torch.empty(cols, dtype=out_dtype, device=x2.device)
+    out32 = out if out_dtype == torch.float32 else torch.empty(cols, dtype=torch.float32, device=x2.device)
+    L = load()
+    ws = torch.empty(L.metis_column_mean_workspace_bytes(cols), dtype=torch.uint8, device=x2.device)
+    rc = L.metis_column_mean_running(x2.data_ptr(), rows, cols, x2.stride(0), DTYPE_F32 if x2.dtype == torch.float32 else DTYPE_BF16,
+                                     None if cached is None else cached.data_ptr(), int(cached_count), out.data_ptr(),
+                                     None if out32 is out else out32.data_ptr(),
+                                     DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16, ws.data_ptr(), ws.numel(), _stream())
+    check(rc, "metis_column_mean_running", x.shape)
+    return out, out32
 
 
 def matvec(p: PackedNVFP4, v: torch.Tensor | None = None, alpha: float = 1.0, *, out: torch.Tensor | None = None,

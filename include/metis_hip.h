@@ -293,7 +293,8 @@ size_t metis_linear_grouped_workspace_bytes(int64_t M, int64_t K, const metis_li
  * residual R = Q(X - me) and every output row additionally receives W^ me, accumulated in binary32 inside the
  * GEMM kernel from the weight operands it expands anyway (center: binary32 [K], 16-byte aligned):
  *     out_g = R . W^_g^T + 1 (W^_g center)^T + t_g u_g^T + bias_g.
- * Same result as metis_nvfp4_matvec + metis_linear_fwd_f32bias to binary32 summation order, without reading the
+ * Same result as metis_nvfp4_matvec + metis_linear_fwd_f32bias to about 2^-22 of the centre's magnitude (it enters
+ * as a pair of binary16 values hi + lo through one more MFMA per step; |center| < 2^20), without reading the
  * packed weights a second time.  Shapes: those for which ..._supported returns 1 (M < 256, K % 256 == 0, at most
  * four members, scale pointers 8-byte aligned, and the K range of a workgroup small enough for its LDS: K <= 8192
  * unsplit, longer with the workspace); METIS_E_ARG otherwise. */
@@ -334,6 +335,16 @@ int metis_nvfp4_quant_centered(const void *x, int64_t rows, int64_t cols, int64_
 size_t metis_column_mean_workspace_bytes(int64_t cols);
 int metis_column_mean(const void *x, int64_t rows, int64_t cols, int64_t ld, int x_dtype, void *out,
                       int out_dtype, void *workspace, size_t workspace_bytes, void *stream);
+/* The column mean followed by the weighted running mean of single-token decode calls
+ * (src/Metis/Metis/bitlinear.py:316-323), in the same two launches:
+ *     me = (cached * cached_count + mean(x) * rows) / (cached_count + rows),
+ * every operation rounded to out_dtype as the reference's tensor expression rounds it (true division).
+ *   cached        [cols] of out_dtype: the mean so far, or NULL (then me = mean(x)); may be the same buffer as out
+ *   cached_count  rows that went into it (<= 2^24)
+ *   out32         optional float [cols]: me once more as binary32 (what metis_linear_fwd_grouped_centered takes) */
+int metis_column_mean_running(const void *x, int64_t rows, int64_t cols, int64_t ld, int x_dtype,
+                              const void *cached, int64_t cached_count, void *out, float *out32, int out_dtype,
+                              void *workspace, size_t workspace_bytes, void *stream);
 /* Same reduction without the division: out[c] = sum_r x[r, c], the bias gradient grad_output.sum(dim=(0, 1))
  * of LinearLowbitFunction.backward (src/Metis/Metis/bitlinear.py:455).  Same arguments and workspace. */
 int metis_column_sum(const void *x, int64_t rows, int64_t cols, int64_t ld, int x_dtype, void *out,

@@ -299,6 +299,26 @@ def test_column_mean(rows, cols, dtype):
         assert torch.equal(again, got32)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_running_mean_update_matches_the_tensor_expression_bit_for_bit(dtype):
+    """Decode calls: me = (cached * count + mean(x) * rows) / (count + rows) with every operation rounded to the
+    arithmetic's dtype (reference bitlinear.py:316-323, evaluated on the CPU: true division), fused behind the
+    column reduction; the float32 copy holds the same values."""
+    from metis_hip import ops
+    g = torch.Generator().manual_seed(77)
+    x = (torch.randn(64, 1, 3584, generator=g) + 0.5).to(dtype).cuda()
+    cached = (torch.randn(3584, generator=g) * 0.3 + 0.5).to(dtype)
+    this_mean = ops.column_mean(x, dtype).cpu()
+    for count in (64, 4096, 1_000_003):
+        me, me32 = ops.column_mean_running(x, cached.cuda(), count, dtype)
+        want = (cached * count + this_mean * 64) / (count + 64)
+        assert want.dtype == dtype
+        assert torch.equal(me.cpu(), want), count
+        assert me32.dtype == torch.float32 and torch.equal(me32.cpu(), want.float())
+    me, me32 = ops.column_mean_running(x, None, 0, dtype)
+    assert torch.equal(me.cpu(), this_mean) and torch.equal(me32.cpu(), this_mean.float())
+
+
 def test_rank_one_operands_reach_binary32_precision():
     from metis_hip import ops
     g = torch.Generator().manual_seed(700)
