@@ -3,11 +3,12 @@
 // the north-star formula (src/Metis/Metis/bitlinear.py:752-756), for M < 256.
 //
 // The output is tiny (M x R) and the contraction long (K up to 18944): the vendor library runs such a product as one
-// or a few workgroups walking all of K (35 us at 64 x 64 x 18944).  Here K is cut into up to 32 chunks, one workgroup
-// per chunk and 64 rows; wave w owns 32 columns of R (R / 32 waves, at most 8); a lane streams 64 contiguous bytes of its row per iteration
-// straight into MFMA operands (both operands with the same mapping, so K may be visited in that permuted order).
-// Partial sums go to a caller-supplied workspace [chunks][M][R] and a second small kernel adds them in chunk order,
-// rounds to bf16 and applies s.
+// or a few workgroups walking all of K (35 us at 64 x 64 x 18944).  Here K is cut into up to 128 chunks of one to three
+// 64-element steps (the product is latency-bound: a step is one round trip to memory), one workgroup per chunk and
+// 64 rows; wave w owns 32 columns of R (R / 32 waves, at most 8); a lane streams 64 contiguous bytes of its row per
+// step straight into MFMA operands (both operands with the same mapping, so K may be visited in that permuted order).
+// Partial sums go to a caller-supplied workspace [chunks][M][R] and a second small kernel adds them in chunk order
+// (four threads per output quad, each a quarter of the chunks, folded in order), rounds to bf16 and applies s.
 #include "metis_device.h"
 #include "metis_host.h"
 
@@ -16,7 +17,8 @@ namespace metis {
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 
-constexpr int kLrMaxChunks = 32;
+constexpr int kLrMaxChunks = 128;
+constexpr int kLrGroup = kLrMaxChunks / 4;     // chunks per thread of the finish kernel
 
 __global__ __launch_bounds__(512) void lowrank_small_partial_kernel(const uint16_t* __restrict__ x, int64_t ldx,
                                                                     const uint16_t* __restrict__ v, int M, int R, int K, int kc,
@@ -71,15 +73,24 @@ __global__ __launch_bounds__(256) void lowrank_small_finish_kernel(const float* 
                                                                    const uint16_t* __restrict__ s, uint16_t* __restrict__ xv,
                                                                    uint16_t* __restrict__ t)
 {
-    const int id = (blockIdx.x * 256 + threadIdx.x) * 4;       // four consecutive elements of [M, R]
-    if (id >= MR) return;
-    float4 p[kLrMaxChunks];
+    __shared__ float4 fold[3][64];
+    const int q = threadIdx.x & 63, g = threadIdx.x >> 6;      // output quad within the block, chunk group
+    const int id = (blockIdx.x * 64 + q) * 4;                  // four consecutive elements of [M, R]
+    const bool live = id < MR;
+    const int per = (chunks + 3) / 4, c0 = g * per;            // this thread's chunks: [c0, c0 + per), per <= kLrGroup
+    float4 p[kLrGroup];
 #pragma unroll
-    for (int c = 0; c < kLrMaxChunks; ++c)
-        p[c] = c < chunks ? *reinterpret_cast<const float4*>(ws + (size_t)c * MR + id) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    for (int c = 0; c < kLrGroup; ++c)
+        p[c] = (live && c < per && c0 + c < chunks) ? *reinterpret_cast<const float4*>(ws + (size_t)(c0 + c) * MR + id)
+                                                    : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     float4 a = p[0];
 #pragma unroll
-    for (int c = 1; c < kLrMaxChunks; ++c) { a.x += p[c].x; a.y += p[c].y; a.z += p[c].z; a.w += p[c].w; }
+    for (int c = 1; c < kLrGroup; ++c) { a.x += p[c].x; a.y += p[c].y; a.z += p[c].z; a.w += p[c].w; }
+    if (g > 0) fold[g - 1][q] = a;
+    __syncthreads();
+    if (g > 0 || !live) return;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) { const float4 b = fold[k][q]; a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w; }
     const uint32_t h[4] = {bf16_bits(a.x), bf16_bits(a.y), bf16_bits(a.z), bf16_bits(a.w)};
     *reinterpret_cast<uint2*>(xv + id) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
     if (t) {
@@ -93,7 +104,7 @@ __global__ __launch_bounds__(256) void lowrank_small_finish_kernel(const float* 
 
 static int lowrank_small_chunks(int64_t K, int* kc_out)
 {
-    int64_t kc = 256;
+    int64_t kc = 64;
     if ((K + kc - 1) / kc > kLrMaxChunks) kc = ((K + kLrMaxChunks - 1) / kLrMaxChunks + 63) / 64 * 64;
     *kc_out = (int)kc;
     return (int)((K + kc - 1) / kc);
@@ -120,7 +131,7 @@ int lowrank_small(const void* x, int64_t ldx, const void* v, int64_t M, int64_t 
     hipLaunchKernelGGL(lowrank_small_partial_kernel, dim3((unsigned)chunks, (unsigned)((M + 63) / 64)), dim3((unsigned)(2 * R)), 0, st,
                        (const uint16_t*)x, ldx, (const uint16_t*)v, (int)M, (int)R, (int)K, kc, (float*)workspace);
     const int MR = (int)(M * R);
-    hipLaunchKernelGGL(lowrank_small_finish_kernel, dim3((unsigned)((MR / 4 + 255) / 256)), dim3(256), 0, st, (const float*)workspace,
+    hipLaunchKernelGGL(lowrank_small_finish_kernel, dim3((unsigned)((MR / 4 + 63) / 64)), dim3(256), 0, st, (const float*)workspace,
                        chunks, MR, (int)R, (const uint16_t*)s, (uint16_t*)xv, (uint16_t*)t);
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
