@@ -235,11 +235,14 @@ __device__ __forceinline__ void expand_row(const RowRegs& r, uint16_t* dst)
 }
 
 // one expand8 (8 elements) of a row: p in 0..7
+template <bool STORE = true>
 __device__ __forceinline__ void expand_piece(const RowRegs& r, int p, uint16_t* d)
 {
     const uint32_t w = p == 0 ? r.c0.x : p == 1 ? r.c0.y : p == 2 ? r.c0.z : p == 3 ? r.c0.w
                      : p == 4 ? r.c1.x : p == 5 ? r.c1.y : p == 6 ? r.c1.z : r.c1.w;
-    reinterpret_cast<uint4*>(d)[p] = expand8(w, scale_pair((r.sc >> (8 * (p >> 1))) & 0xffu));
+    const uint4 e = expand8(w, scale_pair((r.sc >> (8 * (p >> 1))) & 0xffu));
+    if (STORE) reinterpret_cast<uint4*>(d)[p] = e;
+    else asm volatile("" ::"v"(e.x), "v"(e.y), "v"(e.z), "v"(e.w));      // measurement: the arithmetic without the LDS write
 }
 
 // MFMA : VALU : LDS interleave requested from the scheduler for one K=16 sub-step of N_MFMA MFMAs
@@ -390,7 +393,7 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_nvfp4_large_kernel(
         if (FETCH) fetch(r2, (s + 2) * BK);
         auto pieces = [&](int from, int to) {
 #pragma unroll
-            for (int p = from; p < to; ++p) expand_piece(r1[p / 8], p % 8, nxt + lds_row[p / 8]);
+            for (int p = from; p < to; ++p) expand_piece<!(DBG & 4)>(r1[p / 8], p % 8, nxt + lds_row[p / 8]);
         };
         load_frags(1, cur, 1);
         if (EXPAND) pieces(0, P0);
@@ -698,9 +701,10 @@ static int launch_large(const void* a_codes, const void* a_scales, const float* 
                    : f32   ? (const void*)gemm_nvfp4_large_kernel<1, WN_WAVES>
                            : (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES>;
     const char* d = getenv("METIS_GEMM_DBG");                  // measurement switches, results are meaningless:
-    const int v = d ? atoi(d) : 0;                             // 1 = no operand fetch/expansion, 7 = also no barriers
-    if (v == 1 || v == 7) {
-        fn = v == 1 ? (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 1> : (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 7>;
+    const int v = d ? atoi(d) : 0;                             // 1 = no operand fetch/expansion, 7 = also no barriers,
+                                                               // 4 = expansion arithmetic without its LDS writes
+    if (v == 1 || v == 7 || v == 4) {
+        fn = v == 1 ? (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 1> : v == 4 ? (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 4> : (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 7>;
         if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess) return METIS_E_DEVICE;
     } else if (const int rc = allow_dynamic_lds(fn, lds_bytes, attr_set[(split ? 2 : 0) + f32])) {
         return rc;
