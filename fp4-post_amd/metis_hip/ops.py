@@ -5,6 +5,7 @@ PyTorch is used only to own device memory and streams.
 """
 from __future__ import annotations
 
+import functools
 from dataclasses import dataclass
 
 import torch
@@ -322,6 +323,29 @@ def rmsnorm_quantize(x: torch.Tensor, gamma: torch.Tensor, eps: float, mode: int
     return normed, PackedNVFP4(codes, scales, unit, rows, cols, mode)
 
 
+@functools.lru_cache(maxsize=4096)
+def _linear_workspace_bytes(M: int, N: int, K: int, device_index: int) -> int:
+    return int(load().metis_linear_workspace_bytes(M, N, K))          # depends on the device's CU count only
+
+
+@functools.lru_cache(maxsize=4096)
+def _lowrank_workspace_bytes(M: int, R: int, K: int) -> int:
+    return int(load().metis_lowrank_project_workspace_bytes(M, R, K))
+
+
+@functools.lru_cache(maxsize=4096)
+def _grouped_plan(M: int, K: int, ns: tuple, device_index: int) -> tuple[int, bool]:
+    """(split-K scratch bytes, whether a centre can ride inside the launch) of a grouped call; shape-only queries."""
+    import ctypes
+    arr = (_lib.LinearMember * len(ns))()
+    for i, n in enumerate(ns):
+        arr[i].N = n
+    ap = ctypes.cast(arr, ctypes.c_void_p)
+    L = load()
+    need = int(L.metis_linear_grouped_workspace_bytes(M, K, ap, len(ns)))
+    return need, bool(L.metis_linear_grouped_centered_supported(M, K, ap, len(ns), int(need > 0)))
+
+
 def _gemm_workspace(M: int, N: int, K: int, device: torch.device) -> torch.Tensor | None:
     """Split-K scratch for an M x N output contracted over K, or None when the shape is not split.
 
@@ -329,7 +353,7 @@ def _gemm_workspace(M: int, N: int, K: int, device: torch.device) -> torch.Tenso
     graphs each get their own) rather than cached here."""
     if M >= 256 and N < 256:
         return None
-    need = load().metis_linear_workspace_bytes(M, N, K)
+    need = _linear_workspace_bytes(M, N, K, device.index or 0)
     return torch.empty(need, dtype=torch.uint8, device=device) if need else None
 
 
@@ -406,7 +430,7 @@ def lowrank_project(x2: torch.Tensor, v: torch.Tensor, s: torch.Tensor | None = 
     L = load()
     xv = torch.empty(M, R, dtype=torch.bfloat16, device=x2.device)
     t = None if s is None else torch.empty_like(xv)
-    ws = torch.empty(L.metis_lowrank_project_workspace_bytes(M, R, K), dtype=torch.uint8, device=x2.device)
+    ws = torch.empty(_lowrank_workspace_bytes(M, R, K), dtype=torch.uint8, device=x2.device)
     rc = L.metis_lowrank_project(x2.data_ptr(), x2.stride(0), v.data_ptr(), M, R, K, None if s is None else s.contiguous().data_ptr(),
                                  xv.data_ptr(), None if t is None else t.data_ptr(), ws.data_ptr(), ws.numel(), _stream())
     check(rc, "metis_lowrank_project", (M, R, K))
@@ -451,7 +475,8 @@ def linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.b
                                    None if bias is None else bias.data_ptr(), out.data_ptr(), b.rows, int(bias_f32), ldt)
     L = load()
     ap = ctypes.cast(arr, ctypes.c_void_p)
-    need = L.metis_linear_grouped_workspace_bytes(M, K, ap, len(members))     # split-K scratch (long K, few columns)
+    # split-K scratch (long K, few columns) and whether a centre fits the launch: functions of the shape alone
+    need, centre_ok = _grouped_plan(M, K, tuple(m[0].rows for m in members), dev.index or 0)
     ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
     dt = DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16
     if center is not None:
@@ -459,7 +484,7 @@ def linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.b
         if center.numel() != K:
             raise ValueError(f"center must have {K} values, got {center.numel()}")
         aligned = center.data_ptr() % 16 == 0 and all(m[0].scales.data_ptr() % 8 == 0 for m in members) and a.scales.data_ptr() % 8 == 0
-        if aligned and L.metis_linear_grouped_centered_supported(M, K, ap, len(members), int(need > 0)):
+        if aligned and centre_ok:
             rc = L.metis_linear_fwd_grouped_centered(a.codes.data_ptr(), a.scales.data_ptr(), a.unit.data_ptr(), M, K, ap,
                                                      len(members), dt, center.data_ptr(),
                                                      None if ws is None else ws.data_ptr(), need, _stream())
