@@ -8,6 +8,10 @@
 //   4. metis_linear_fwd (tiled and skinny shapes)  -> against a double-precision product of the
 //                                                     dequantized operands, rel. Frobenius error <= 2e-3
 //   5. error codes for bad arguments
+//   6. split-K through a caller workspace (metis_linear_fwd_ws: tiled and decode-sized shapes)
+//   7. metis_linear_fwd_grouped, and metis_linear_fwd_grouped_centered with the centre from
+//      metis_column_mean_running                    -> against double precision on the host
+//   8. metis_nvfp4_matvec                           -> against double precision on the host
 //
 // Built and run by tests/test_gpu_cabi_native.py; prints one line per check and exits non-zero on failure.
 #include <hip/hip_runtime.h>
@@ -127,7 +131,7 @@ static double rel_fro(const std::vector<double>& got, const std::vector<double>&
     return sqrt(num / (den > 0 ? den : 1));
 }
 
-static void check_linear(int64_t M, int64_t N, int64_t K, hipStream_t st, const char* what)
+static void check_linear(int64_t M, int64_t N, int64_t K, hipStream_t st, const char* what, bool with_workspace = false)
 {
     const std::vector<uint16_t> x = make_input(M, K, 11u + (unsigned)M, 1.0f), w = make_input(N, K, 12u + (unsigned)N, 0.02f);
     DeviceBuffer<uint8_t> ac((size_t)(M * K / 2)), as((size_t)(M * K / 16)), bc((size_t)(N * K / 2)), bs((size_t)(N * K / 16));
@@ -135,8 +139,20 @@ static void check_linear(int64_t M, int64_t N, int64_t K, hipStream_t st, const 
     const Packed pa = quantize_on_device(x, M, K, METIS_MODE_P32, st, &ac, &as, &au);
     const Packed pb = quantize_on_device(w, N, K, METIS_MODE_P32, st, &bc, &bs, &bu);
     DeviceBuffer<float> out((size_t)(M * N));
-    const int rc = metis_linear_fwd(ac.p, as.p, au.p, bc.p, bs.p, bu.p, M, N, K, nullptr, nullptr, 0, nullptr, out.p, METIS_DTYPE_F32, st);
-    HIP_OK(hipStreamSynchronize(st));
+    int rc;
+    if (with_workspace) {
+        const size_t need = metis_linear_workspace_bytes(M, N, K);
+        char l2[160];
+        snprintf(l2, sizeof l2, "%s: metis_linear_workspace_bytes = %zu (the shape is split)", what, need);
+        check(need > 0, l2);
+        DeviceBuffer<uint8_t> ws(need ? need : 16);              // no initialisation needed
+        rc = metis_linear_fwd_ws(ac.p, as.p, au.p, bc.p, bs.p, bu.p, M, N, K, nullptr, nullptr, 0, nullptr, out.p, METIS_DTYPE_F32,
+                                 ws.p, need, st);
+        HIP_OK(hipStreamSynchronize(st));
+    } else {
+        rc = metis_linear_fwd(ac.p, as.p, au.p, bc.p, bs.p, bu.p, M, N, K, nullptr, nullptr, 0, nullptr, out.p, METIS_DTYPE_F32, st);
+        HIP_OK(hipStreamSynchronize(st));
+    }
     std::vector<float> xa((size_t)(M * K)), wb((size_t)(N * K));
     metis_oracle_nvfp4_dequant(pa.codes.data(), pa.scales.data(), pa.unit, M, K, 0, nullptr, xa.data());
     metis_oracle_nvfp4_dequant(pb.codes.data(), pb.scales.data(), pb.unit, N, K, 0, nullptr, wb.data());
@@ -153,6 +169,127 @@ static void check_linear(int64_t M, int64_t N, int64_t K, hipStream_t st, const 
     char line[160];
     snprintf(line, sizeof line, "%s: metis_linear_fwd %ldx%ldx%ld rc=%d rel.err %.2e", what, (long)M, (long)N, (long)K, rc, err);
     check(rc == METIS_OK && err <= 2e-3, line);
+}
+
+// Mean mode at decode size: column mean (with the running update) -> centred quantizer -> grouped GEMM with the
+// centre inside, and the packed matrix-vector product, all against double precision on the host.
+static void check_mean_mode_decode(hipStream_t st)
+{
+    const int64_t M = 24, K = 512, N0 = 96, N1 = 36;
+    std::vector<uint16_t> x = make_input(M, K, 21u, 1.0f);
+    for (size_t i = 0; i < x.size(); ++i) x[i] = metis_oracle_f32_to_bf16(bf16_to_f32(x[i]) + 0.75f);      // an offset worth removing
+    const std::vector<uint16_t> w0 = make_input(N0, K, 22u, 0.05f), w1 = make_input(N1, K, 23u, 0.05f);
+    DeviceBuffer<uint16_t> dx(x.size());
+    dx.upload(x);
+    // running mean in binary32: cached = 0.5 for every column with weight 40 rows
+    std::vector<float> cached((size_t)K, 0.5f);
+    DeviceBuffer<float> dcached((size_t)K), dme((size_t)K);
+    dcached.upload(cached);
+    const size_t mws = metis_column_mean_workspace_bytes(K);
+    DeviceBuffer<uint8_t> ws_mean(mws);
+    int rc = metis_column_mean_running(dx.p, M, K, K, METIS_DTYPE_BF16, dcached.p, 40, dme.p, nullptr, METIS_DTYPE_F32, ws_mean.p, mws, st);
+    HIP_OK(hipStreamSynchronize(st));
+    const std::vector<float> me = dme.download();
+    double worst = 0;
+    for (int64_t c = 0; c < K; ++c) {
+        double sum = 0;
+        for (int64_t r = 0; r < M; ++r) sum += bf16_to_f32(x[(size_t)(r * K + c)]);
+        const double want = (0.5 * 40 + (sum / M) * M) / (40 + M);
+        worst = fmax(worst, fabs(me[(size_t)c] - want));
+    }
+    char line[200];
+    snprintf(line, sizeof line, "metis_column_mean_running rc=%d: weighted running mean, worst abs. error %.2e", rc, worst);
+    check(rc == METIS_OK && worst <= 1e-6, line);
+
+    // centred quantizer: the packed tensor is that of x - me (binary32 arithmetic)
+    DeviceBuffer<uint8_t> ac((size_t)(M * K / 2)), as((size_t)(M * K / 16));
+    DeviceBuffer<float> au(1);
+    const size_t qws = metis_nvfp4_workspace_bytes(M, K);
+    DeviceBuffer<uint8_t> ws_q(qws);
+    HIP_OK(hipMemset(ws_q.p, 0, qws));
+    rc = metis_nvfp4_quant_centered(dx.p, M, K, K, METIS_MODE_P32, dme.p, 0, 0, nullptr, 0, 0, ac.p, as.p, au.p, ws_q.p, qws, st);
+    HIP_OK(hipStreamSynchronize(st));
+    std::vector<float> res((size_t)(M * K));
+    for (int64_t r = 0; r < M; ++r)
+        for (int64_t c = 0; c < K; ++c) res[(size_t)(r * K + c)] = bf16_to_f32(x[(size_t)(r * K + c)]) - me[(size_t)c];
+    std::vector<uint8_t> wc((size_t)(M * K / 2)), wsc((size_t)(M * K / 16));
+    float wu = 0;
+    metis_oracle_nvfp4_pack(res.data(), M, K, K, 2, nullptr, wc.data(), wsc.data(), &wu, nullptr);      // mode 2: binary32 input
+    check(rc == METIS_OK && ac.download() == wc && as.download() == wsc && au.download()[0] == wu,
+          "metis_nvfp4_quant_centered: packed residual bit-equal to the oracle on x - me");
+    std::vector<float> rdq((size_t)(M * K));
+    metis_oracle_nvfp4_dequant(wc.data(), wsc.data(), wu, M, K, 0, nullptr, rdq.data());
+
+    // two weights, one launch, the centre inside
+    DeviceBuffer<uint8_t> b0c((size_t)(N0 * K / 2)), b0s((size_t)(N0 * K / 16)), b1c((size_t)(N1 * K / 2)), b1s((size_t)(N1 * K / 16));
+    DeviceBuffer<float> b0u(1), b1u(1), o0((size_t)(M * N0)), o1((size_t)(M * N1));
+    const Packed p0 = quantize_on_device(w0, N0, K, METIS_MODE_P32, st, &b0c, &b0s, &b0u);
+    const Packed p1 = quantize_on_device(w1, N1, K, METIS_MODE_P32, st, &b1c, &b1s, &b1u);
+    metis_linear_member mem[2] = {};
+    mem[0].b_codes = b0c.p; mem[0].b_scales = b0s.p; mem[0].b_unit = b0u.p; mem[0].out = o0.p; mem[0].N = N0;
+    mem[1].b_codes = b1c.p; mem[1].b_scales = b1s.p; mem[1].b_unit = b1u.p; mem[1].out = o1.p; mem[1].N = N1;
+    const size_t gneed = metis_linear_grouped_workspace_bytes(M, K, mem, 2);
+    DeviceBuffer<uint8_t> gws(gneed ? gneed : 16);
+    const int supported = metis_linear_grouped_centered_supported(M, K, mem, 2, gneed > 0);
+    check(supported == 1, "metis_linear_grouped_centered_supported for a decode-sized group");
+    rc = metis_linear_fwd_grouped_centered(ac.p, as.p, au.p, M, K, mem, 2, METIS_DTYPE_F32, dme.p, gneed ? gws.p : nullptr, gneed, st);
+    HIP_OK(hipStreamSynchronize(st));
+    const Packed* pw[2] = {&p0, &p1};
+    const int64_t Ns[2] = {N0, N1};
+    const std::vector<float> got_o[2] = {o0.download(), o1.download()};
+    for (int g = 0; g < 2; ++g) {
+        std::vector<float> wdq((size_t)(Ns[g] * K));
+        metis_oracle_nvfp4_dequant(pw[g]->codes.data(), pw[g]->scales.data(), pw[g]->unit, Ns[g], K, 0, nullptr, wdq.data());
+        std::vector<double> want((size_t)(M * Ns[g])), got((size_t)(M * Ns[g]));
+        for (int64_t m = 0; m < M; ++m)
+            for (int64_t n = 0; n < Ns[g]; ++n) {
+                double sacc = 0;
+                for (int64_t k = 0; k < K; ++k) sacc += ((double)rdq[(size_t)(m * K + k)] + me[(size_t)k]) * wdq[(size_t)(n * K + k)];
+                want[(size_t)(m * Ns[g] + n)] = sacc;
+                got[(size_t)(m * Ns[g] + n)] = got_o[g][(size_t)(m * Ns[g] + n)];
+            }
+        const double err = rel_fro(got, want);
+        snprintf(line, sizeof line, "metis_linear_fwd_grouped_centered member %d (%ldx%ldx%ld) rc=%d rel.err %.2e", g, (long)M, (long)Ns[g], (long)K, rc, err);
+        check(rc == METIS_OK && err <= 5e-5, line);
+    }
+    // the same group without the centre equals R W^T
+    rc = metis_linear_fwd_grouped(ac.p, as.p, au.p, M, K, mem, 2, METIS_DTYPE_F32, nullptr, 0, st);
+    HIP_OK(hipStreamSynchronize(st));
+    {
+        std::vector<float> wdq((size_t)(N1 * K));
+        metis_oracle_nvfp4_dequant(p1.codes.data(), p1.scales.data(), p1.unit, N1, K, 0, nullptr, wdq.data());
+        const std::vector<float> o = o1.download();
+        std::vector<double> want((size_t)(M * N1)), got((size_t)(M * N1));
+        for (int64_t m = 0; m < M; ++m)
+            for (int64_t n = 0; n < N1; ++n) {
+                double sacc = 0;
+                for (int64_t k = 0; k < K; ++k) sacc += (double)rdq[(size_t)(m * K + k)] * wdq[(size_t)(n * K + k)];
+                want[(size_t)(m * N1 + n)] = sacc;
+                got[(size_t)(m * N1 + n)] = o[(size_t)(m * N1 + n)];
+            }
+        const double err = rel_fro(got, want);
+        snprintf(line, sizeof line, "metis_linear_fwd_grouped member 1 rc=%d rel.err %.2e", rc, err);
+        check(rc == METIS_OK && err <= 5e-5, line);
+    }
+    // packed matrix-vector product: W^_0 me
+    DeviceBuffer<float> dy((size_t)N0);
+    rc = metis_nvfp4_matvec(b0c.p, b0s.p, b0u.p, N0, K, dme.p, 1.0f, dy.p, nullptr, 0, 0, st);
+    HIP_OK(hipStreamSynchronize(st));
+    {
+        std::vector<float> wdq((size_t)(N0 * K));
+        metis_oracle_nvfp4_dequant(p0.codes.data(), p0.scales.data(), p0.unit, N0, K, 0, nullptr, wdq.data());
+        const std::vector<float> y = dy.download();
+        std::vector<double> want((size_t)N0), got((size_t)N0);
+        for (int64_t n = 0; n < N0; ++n) {
+            double sacc = 0;
+            for (int64_t k = 0; k < K; ++k) sacc += (double)wdq[(size_t)(n * K + k)] * me[(size_t)k];
+            want[(size_t)n] = sacc;
+            got[(size_t)n] = y[(size_t)n];
+        }
+        const double err = rel_fro(got, want);
+        snprintf(line, sizeof line, "metis_nvfp4_matvec rc=%d rel.err %.2e", rc, err);
+        check(rc == METIS_OK && err <= 1e-5, line);
+    }
 }
 
 int main()
@@ -225,6 +362,13 @@ int main()
     check_linear(272, 320, 256, st, "tiled 256x256");
     check_linear(96, 132, 96, st, "tiled 128x128");
     check_linear(48, 160, 512, st, "skinny");
+
+    // ---- 6: split-K through a caller workspace
+    check_linear(256, 256, 2048, st, "tiled, K split", true);
+    check_linear(40, 64, 8192, st, "skinny, K split", true);
+
+    // ---- 7 + 8: mean mode at decode size
+    check_mean_mode_decode(st);
 
     // ---- 5: error codes
     {
