@@ -381,6 +381,20 @@ int main()
         check(metis_nvfp4_quant_row(nullptr, 32, 32, 32, 0, dc.p, ds.p, du.p, ws.p, ws.n, st) == METIS_E_ARG, "null input -> METIS_E_ARG");
         check(metis_nvfp4_quant_row(nullptr, 0, 32, 32, 0, nullptr, nullptr, nullptr, nullptr, 0, st) == METIS_OK, "empty tensor is a no-op");
         check(strlen(metis_error_string(METIS_E_SHAPE)) > 0, "metis_error_string");
+        // grouped entry: a split shape with a short workspace, a centre on a shape that cannot take one
+        metis_linear_member one = {};
+        DeviceBuffer<uint8_t> pa((size_t)(8 * 8192 / 2)), ps((size_t)(8 * 8192 / 16)), pb((size_t)(64 * 8192 / 2)), pbs((size_t)(64 * 8192 / 16));
+        DeviceBuffer<float> un(1), o((size_t)(8 * 64)), cen(8192);
+        one.b_codes = pb.p; one.b_scales = pbs.p; one.b_unit = un.p; one.out = o.p; one.N = 64;
+        const size_t need = metis_linear_grouped_workspace_bytes(8, 8192, &one, 1);
+        DeviceBuffer<uint8_t> gws(need + 16);
+        check(need > 0 && metis_linear_fwd_grouped(pa.p, ps.p, un.p, 8, 8192, &one, 1, METIS_DTYPE_BF16, gws.p, 1024, st) == METIS_E_WORKSPACE,
+              "grouped call, short split-K workspace -> METIS_E_WORKSPACE");
+        check(metis_linear_fwd_grouped_centered(pa.p, ps.p, un.p, 8, 8192, &one, 1, METIS_DTYPE_BF16, nullptr, gws.p, need, st) == METIS_E_ARG,
+              "centred call without a centre -> METIS_E_ARG");
+        check(metis_linear_grouped_centered_supported(300, 8192, &one, 1, 1) == 0 &&
+              metis_linear_fwd_grouped_centered(pa.p, ps.p, un.p, 300, 8192, &one, 1, METIS_DTYPE_BF16, cen.p, gws.p, need, st) == METIS_E_ARG,
+              "centred call at M >= 256 -> not supported, METIS_E_ARG");
     }
     HIP_OK(hipStreamDestroy(st));
     printf(failures ? "FAILED %d check(s)\n" : "all checks passed\n", failures);
