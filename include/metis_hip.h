@@ -285,7 +285,8 @@ int metis_linear_fwd_grouped(const void *a_codes, const void *a_scales, const fl
                              void *workspace, size_t workspace_bytes, void *stream);
 /* Scratch for the call above: with few output columns and a long K (a down projection at decode size) K is cut
  * into slices that run as separate workgroups, their binary32 partial sums meet in the workspace and a second
- * small kernel adds them in a fixed order.  Only the N fields of the members are read.  0 = the shape is not
+ * small kernel adds them in a fixed order.  Only the N fields of the members are read; the figure is an upper
+ * bound (the number of slices also depends on pointer alignment, known only at the call).  0 = the shape is not
  * split; workspace = NULL in the call = never split.  16-byte aligned, contents need no initialisation. */
 size_t metis_linear_grouped_workspace_bytes(int64_t M, int64_t K, const metis_linear_member *members, int count);
 /* Mean mode for decode-sized batches in one pass over the weights (BitLinear.forward under the reference's default
