@@ -368,6 +368,47 @@ def test_hot_path_replays_from_a_captured_graph():
         assert torch.equal(got, want), seed
 
 
+def test_decode_path_replays_from_a_captured_graph():
+    """The decode-sized chain (column mean with running update, centred quantizer, rank-r projection, grouped GEMM with
+    K split through scratch taken from the allocator inside the capture, centre inside the launch) captured once and
+    replayed on fresh inputs, with eager work between the replays: every replay equals the eager result bit for bit."""
+    from metis_hip import ops
+    g = torch.Generator().manual_seed(14)
+    M, K, r = 8, 8192, 32
+    pws = [ops.quantize((torch.randn(n, K, generator=g) * 0.02).bfloat16().cuda()) for n in (64, 36)]
+    us = [(torch.randn(n, r, generator=g) * 0.1).bfloat16().cuda() for n in (64, 36)]
+    v = (torch.randn(2 * r, K, generator=g) / K ** 0.5).bfloat16().cuda()
+    sv = torch.rand(2 * r, generator=g).bfloat16().cuda()
+    bias = torch.randn(64, generator=g).cuda()
+    cached = (torch.randn(K, generator=g) * 0.1).cuda()
+    x_static = torch.zeros(M, K, dtype=torch.bfloat16, device="cuda")
+
+    def chain(x):
+        me, me32 = ops.column_mean_running(x, cached, 40, torch.float32)
+        px = ops.quantize(x, 0, center=me)
+        _, t = ops.lowrank_project(x, v, sv)
+        members = [(pws[0], t[:, :r], us[0], bias), (pws[1], t[:, r:], us[1], None)]
+        return ops.linear_fwd_grouped(px, members, out_dtype=torch.float32, center=me32)
+
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        chain(x_static)                                          # warm-up allocates the stream's workspace
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            outs_static = chain(x_static)
+    for seed in (31, 32, 33):
+        x = (synthetic_activation(seed, M, K).float() + 0.5).bfloat16().cuda()
+        x_static.copy_(x)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [o.clone() for o in outs_static]
+        want = chain(x)                                          # eager work between replays
+        torch.cuda.synchronize()
+        for a, b in zip(got, want):
+            assert torch.equal(a, b), seed
+
+
 def test_compile_flag_is_accepted_and_changes_nothing():
     """Reference tests/test_metis_quant_cache.py:30-42: the flag that selects the torch.compile'd QDQ there
     selects the same kernel here; results are identical at atol 0 and the status helper says so."""
