@@ -48,6 +48,11 @@ def extra(reps: int = 5):
     w_up = ops.quantize((torch.randn(18944, 3584, generator=g) * 0.02).bfloat16().cuda())
     w_down = ops.quantize((torch.randn(3584, 18944, generator=g) * 0.02).bfloat16().cuda())
     p_dec_up, p_dec_down, p_pre = ops.quantize(dec[:, :3584].contiguous()), ops.quantize(dec), ops.quantize(pre)
+    me_cache = torch.zeros(3584, dtype=torch.bfloat16, device="cuda")
+    me_down = torch.full((18944,), 0.01, device="cuda")
+    v_up = (torch.randn(128, 3584, generator=g) / 60).bfloat16().cuda()   # the stacked V of gate and up, r = 64 each
+    s_up = torch.rand(128, generator=g).bfloat16().cuda()
+    u_up = (torch.randn(18944, 64, generator=g) * 0.1).bfloat16().cuda()
     for i in range(reps):
         ops.quantize(x, 1)                                              # bf16 arithmetic, round to nearest
         ops.quantize(x, 0, col=True)                                    # column-blocked
@@ -66,6 +71,13 @@ def extra(reps: int = 5):
         ops.quantize(xf, 0, sr=True, col=True, seed=i, center=me)
         wm = ops.matvec(w_up, me[:3584])
         ops.rank_one_operands(18944, 3584, (wm, me[:3584]), (wm, me[:3584]))
+        # mean mode at decode size: running mean, centred quantizer, rank-r projection, centre inside the grouped GEMM
+        xd = dec[:, :3584].contiguous()
+        me_d, me_d32 = ops.column_mean_running(xd, me_cache, 4096, torch.bfloat16)
+        p_res = ops.quantize(xd, 1, center=me_d)
+        _, t_d = ops.lowrank_project(xd, v_up, s_up)
+        ops.linear_fwd_grouped(p_res, [(w_up, t_d[:, :64], u_up, None), (w_up, t_d[:, 64:], u_up, None)], center=me_d32)
+        ops.linear_fwd_grouped(p_dec_down, [(w_down, None, None, None)], center=me_down)     # K in slices, centre inside
     torch.cuda.synchronize()
 
 
