@@ -684,6 +684,10 @@ class BitLinear(nn.Module):
 
     def _apply(self, fn, recurse=True):
         self._merged_rollout_weight_cache = None
+        self._bias_cast_cache = None
+        group = getattr(self, "activation_group", None)
+        if group is not None:
+            group.pop("stacked_v", None)                         # parameters are replaced: versions start over
         return super()._apply(fn, recurse=recurse)
 
     # ------------------------------------------------------------------ projection group in one launch (inference)
