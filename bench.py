@@ -189,12 +189,17 @@ def main():
     q_bytes = x1.numel() * QUANT_BYTES_PER_ELT
     q_gbs = q_bytes / (q_ms * 1e-3) / 1e9
 
-    # the opt-in single-launch variant (needs the device to itself: every workgroup must be resident), same call
-    os.environ["METIS_FUSED_QUANT"] = "1"
-    try:
-        _, q1_ms = time_region(torch, qstep, max(args.steps, 50), args.warmup)
-    finally:
-        os.environ.pop("METIS_FUSED_QUANT", None)
+    # the opt-in single-launch variant (needs the device to itself: every workgroup must be resident)
+    def q1step(ev):
+        if ev is not None:
+            ev[0].record()
+        rc = L.metis_nvfp4_quant_row_resident(x1.data_ptr(), 8192, 4096, 0, qc.data_ptr(), qs.data_ptr(), qu.data_ptr(),
+                                              qws.data_ptr(), qws.numel(), 0, st)
+        if ev is not None:
+            ev[1].record()
+        assert rc == 0
+
+    _, q1_ms = time_region(torch, q1step, max(args.steps, 50), args.warmup)
     q1_gbs = q_bytes / (q1_ms * 1e-3) / 1e9
 
     # ------------------------------------------------------------------ config 2: fused RMSNorm -> quant

@@ -48,6 +48,13 @@ int metis_nvfp4_quant_row(const void* x, int64_t rows, int64_t cols, int64_t ld,
                     workspace_bytes, (hipStream_t)stream);
 }
 
+int metis_nvfp4_quant_row_resident(const void* x, int64_t rows, int64_t cols, int mode, void* codes, void* scales,
+                                   float* unit, void* workspace, size_t workspace_bytes, uint32_t spin_limit, void* stream)
+{
+    return quantize(x, rows, cols, cols, mode, false, false, nullptr, 0, 0, codes, scales, unit, workspace,
+                    workspace_bytes, (hipStream_t)stream, nullptr, true, spin_limit);
+}
+
 int metis_nvfp4_quant_col(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, void* codes, void* scales,
                           float* unit, void* workspace, size_t workspace_bytes, void* stream)
 {

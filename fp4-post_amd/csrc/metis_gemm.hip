@@ -20,6 +20,14 @@
 
 namespace metis {
 
+// Measurement switches (kernel variants and shape overrides read from the environment) exist only in a
+// -DMETIS_MEASURE build of the library; the shipped library reads no environment variables.
+#ifdef METIS_MEASURE
+static inline const char* measure_env(const char* name) { return getenv(name); }
+#else
+static inline const char* measure_env(const char*) { return nullptr; }
+#endif
+
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
@@ -650,7 +658,7 @@ static SplitPlan split_plan(int64_t M, int64_t N, int64_t K)
     if (tiles * 2 > cus) {
         part = tiles % cus;
         nfull = tiles - part;
-        if (tiles < cus || part == 0 || part * 2 > cus || nfull > 4 * (int64_t)cus || getenv("METIS_GEMM_NOTAIL")) return none;
+        if (tiles < cus || part == 0 || part * 2 > cus || nfull > 4 * (int64_t)cus || measure_env("METIS_GEMM_NOTAIL")) return none;
     }
     int64_t s = cus / part;
     if (s > K / BK / 8) s = K / BK / 8;
@@ -700,13 +708,16 @@ static int launch_large(const void* a_codes, const void* a_scales, const float* 
                                   : (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 0, WN_WAVES == 4>)
                    : f32   ? (const void*)gemm_nvfp4_large_kernel<1, WN_WAVES>
                            : (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES>;
-    const char* d = getenv("METIS_GEMM_DBG");                  // measurement switches, results are meaningless:
+#ifdef METIS_MEASURE
+    const char* d = getenv("METIS_GEMM_DBG");                  // results are meaningless:
     const int v = d ? atoi(d) : 0;                             // 1 = no operand fetch/expansion, 7 = also no barriers,
                                                                // 4 = expansion arithmetic without its LDS writes
     if (v == 1 || v == 7 || v == 4) {
         fn = v == 1 ? (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 1> : v == 4 ? (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 4> : (const void*)gemm_nvfp4_large_kernel<0, WN_WAVES, 7>;
         if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess) return METIS_E_DEVICE;
-    } else if (const int rc = allow_dynamic_lds(fn, lds_bytes, attr_set[(split ? 2 : 0) + f32])) {
+    } else
+#endif
+    if (const int rc = allow_dynamic_lds(fn, lds_bytes, attr_set[(split ? 2 : 0) + f32])) {
         return rc;
     }
     const int tiles_m = (int)((M + L_BM - 1) / L_BM), tiles_n = (int)((N + L_BN - 1) / L_BN);
@@ -1081,7 +1092,7 @@ static SkinnyShape skinny_shape(int64_t M, int64_t K, int64_t tiles, bool al8, b
     // workgroups anyway.
     SkinnyShape s;
     s.c = (K % 256 == 0 && al8) ? 4 : 1;
-    s.nsplit = (have_workspace && !getenv("METIS_GEMM_NOSPLIT")) ? skinny_split_factor(tiles, K, s.c) : 1;
+    s.nsplit = (have_workspace && !measure_env("METIS_GEMM_NOSPLIT")) ? skinny_split_factor(tiles, K, s.c) : 1;
     s.tm = (M <= 32 || tiles * s.nsplit < device_cus() / 2) ? 1 : 2;
     s.waves = (s.tm == 1 && M <= 32 && tiles >= 2 * device_cus()) ? 4 : 8;
     return s;
@@ -1097,7 +1108,7 @@ static bool skinny_center_fits(const SkinnyShape& s, int64_t K)
 // then adds W^ me as a binary32 bias computed with packed_gemv.  Scale-byte pointers are assumed 8-byte aligned.
 int gemm_grouped_center_supported(int64_t M, int64_t K, const GemmMember* members, int count, int have_workspace)
 {
-    if (!members || count < 1 || count > 4 || M <= 0 || M >= 256 || K <= 0 || K % 64 || getenv("METIS_GEMM_SMALL")) return 0;
+    if (!members || count < 1 || count > 4 || M <= 0 || M >= 256 || K <= 0 || K % 64 || measure_env("METIS_GEMM_SMALL")) return 0;
     int64_t tiles = 0;
     for (int i = 0; i < count; ++i) {
         if (members[i].N <= 0 || members[i].N % 4) return 0;
@@ -1112,7 +1123,7 @@ int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a
 {
     if (!members || count < 1) return METIS_E_ARG;
     if ((uintptr_t)center % 16) return METIS_E_ARG;
-    bool skinny = M > 0 && M < 256 && K % 64 == 0 && count <= kMaxGroupMembers && !getenv("METIS_GEMM_SMALL") &&
+    bool skinny = M > 0 && M < 256 && K % 64 == 0 && count <= kMaxGroupMembers && !measure_env("METIS_GEMM_SMALL") &&
                   a_codes && a_scales && a_unit && !((uintptr_t)a_codes % 16) && !((uintptr_t)a_scales % 2) && K <= INT32_MAX &&
                   (out_dtype == METIS_DTYPE_BF16 || out_dtype == METIS_DTYPE_F32);
     bool al8 = ((uintptr_t)a_scales % 8) == 0;
@@ -1140,7 +1151,7 @@ int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a
     }
     const SkinnyShape shape = skinny_shape(M, K, tiles, al8, workspace != nullptr);
     int c = shape.c, nsplit = shape.nsplit, tm = shape.tm, waves = shape.waves;
-    if (const char* f = getenv("METIS_SKINNY_SHAPE")) {        // measurement switch: "tm,c,waves,slices"
+    if (const char* f = measure_env("METIS_SKINNY_SHAPE")) {        // measurement switch: "tm,c,waves,slices"
         int ftm = 0, fc = 0, fw = 0, fs = 0;
         if (sscanf(f, "%d,%d,%d,%d", &ftm, &fc, &fw, &fs) == 4 && (ftm == 1 || ftm == 2) && (fc == 1 || (fc == 4 && c == 4)) &&
             (fw == 4 || fw == 8) && fs >= 1 && fs <= 8 && (fs == 1 || workspace) && K / (64 * fc) >= fs) {
@@ -1439,18 +1450,20 @@ int gemm_nvfp4(const void* a_codes, const void* a_scales, const float* a_unit, c
         return METIS_E_ARG;
     if (K % 32) return METIS_E_ARG;                            // 16-byte code chunks: rows must stay 16-byte aligned
     if (M == 0 || N == 0) return METIS_OK;
-    if (M >= 256 && N >= 256 && K % BK == 0 && !getenv("METIS_GEMM_SMALL")) {
-        if (getenv("METIS_GEMM_W4"))
+    if (M >= 256 && N >= 256 && K % BK == 0 && !measure_env("METIS_GEMM_SMALL")) {
+#ifdef METIS_MEASURE
+        if (measure_env("METIS_GEMM_W4"))                      // 4 waves of 128 x 128: measured 15 % slower than 8 of 128 x 64
             return launch_large<2>(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st, bias_f32);
+#endif
         SplitPlan plan = {1, 0};
-        if (workspace && !getenv("METIS_GEMM_NOSPLIT")) {
+        if (workspace && !measure_env("METIS_GEMM_NOSPLIT")) {
             plan = split_plan(M, N, K);
             if (plan.nsplit > 1 && (((uintptr_t)workspace % 16) || workspace_bytes < gemm_workspace_bytes(M, N, K))) return METIS_E_WORKSPACE;
         }
         return launch_large<4>(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st,
                                bias_f32, (float*)workspace, plan.nsplit, plan.nfull);
     }
-    if (M < 256 && K % 64 == 0 && !getenv("METIS_GEMM_SMALL"))    // up to four 64-row passes over the weights beat a mostly empty 256-row tile
+    if (M < 256 && K % 64 == 0 && !measure_env("METIS_GEMM_SMALL"))    // up to four 64-row passes over the weights beat a mostly empty 256-row tile
         return gemm_skinny(a_codes, a_scales, a_unit, b_codes, b_scales, b_unit, M, N, K, t, u, r, bias, out, out_dtype, st, bias_f32,
                            workspace, workspace_bytes);
     constexpr int BM = 128, BN = 128;

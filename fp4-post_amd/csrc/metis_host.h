@@ -45,7 +45,8 @@ int launch_scales(int mode, const Workspace& ws, uint32_t ngroups, void* scales,
 
 int quantize(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, bool sr, bool col, const void* noise,
              uint64_t seed, uint64_t offset, void* codes, void* scales, float* unit, void* workspace,
-             size_t workspace_bytes, hipStream_t st, const void* center = nullptr);
+             size_t workspace_bytes, hipStream_t st, const void* center = nullptr, bool resident = false,
+             uint32_t spin_limit = 0);
 int dequantize(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, int mode, void* out,
                int out_dtype, hipStream_t st);
 int block_scalars(const void* x, int64_t rows, int64_t cols, int mode, void* s, hipStream_t st);

@@ -315,7 +315,9 @@ __global__ __launch_bounds__(256) void quant_scales_f32_kernel(const float* __re
 // loads and stores only, and no line is polled by more than one group's members.
 // Workgroup 0 advances the generation counter once its own wait is over, by which time every
 // workgroup has read it.  The words only need zero-filling once.  The wait is bounded: after
-// kSpinLimit polls a workgroup raises the time-out word and carries on, so every wave always exits.
+// spin_limit polls a workgroup gives up, so every wave always exits; it then raises the sticky
+// time-out word of the workspace and its result is NaN, which ends up in the tensor unit (and in the
+// unit of every later call on that workspace until the caller zero-fills it again).
 // ---------------------------------------------------------------------------------------------
 constexpr uint32_t kSpinLimit = 1u << 20;
 constexpr uint32_t kGroups = 64;                 // groups, and the most members a group can have
@@ -362,7 +364,8 @@ __device__ __forceinline__ void grid_max_arrive(float thread_max, uint64_t tag, 
 
 // Wave-wide: polls one word per lane (lanes >= count are idle) until all carry the tag; returns the
 // maximum of the bf16 payloads.
-__device__ __forceinline__ float poll_tagged_max(const uint64_t* words, uint32_t count, uint64_t tag, uint32_t* sync)
+__device__ __forceinline__ float poll_tagged_max(const uint64_t* words, uint32_t count, uint64_t tag, uint32_t* sync,
+                                                 uint32_t spin_limit)
 {
     const uint32_t lane = threadIdx.x & 63u;
     uint64_t w = tag << 16;
@@ -370,27 +373,32 @@ __device__ __forceinline__ float poll_tagged_max(const uint64_t* words, uint32_t
     for (;;) {
         if (lane < count) w = METIS_AT_LOAD(words + lane);
         if (__builtin_amdgcn_ballot_w64((w >> 16) != tag) == 0ull) break;
-        if (++polls > kSpinLimit) {
+        if (++polls > spin_limit) {
             if (lane == 0) METIS_AT_STORE(sync_timeout(sync), 1u);
-            break;
+            return __builtin_nanf("");
         }
         __builtin_amdgcn_s_sleep(1);
     }
+    // a payload of 0x7fc0 (bf16 NaN) marks a group whose own wait gave up; fmaxf would drop it
+    if (__builtin_amdgcn_ballot_w64(lane < count && ((uint32_t)w & 0xffffu) == 0x7fc0u) != 0ull) return __builtin_nanf("");
     return wave_max(__uint_as_float(((uint32_t)w & 0xffffu) << 16));
 }
 
 // Called by every thread after grid_max_arrive(); returns the tensor-wide maximum.
-__device__ __forceinline__ float grid_max_wait(uint64_t tag, uint32_t* sync, GridMaxState& sh)
+__device__ __forceinline__ float grid_max_wait(uint64_t tag, uint32_t* sync, GridMaxState& sh, uint32_t spin_limit)
 {
     if (threadIdx.x < 64) {
         const uint32_t j = blockIdx.x % kGroups;
         const uint32_t ngroups = gridDim.x < kGroups ? gridDim.x : kGroups;
         const uint32_t members = (gridDim.x + kGroups - 1u - j) / kGroups;
         if (blockIdx.x < kGroups) {                               // member 0 folds its group and tells every group
-            const float gm = poll_tagged_max(sync_member(sync, j, 0), members, tag, sync);
-            if (threadIdx.x < ngroups) METIS_AT_STORE(sync_copy(sync, threadIdx.x, j), (tag << 16) | (uint64_t)(__float_as_uint(gm) >> 16));
+            const float gm = poll_tagged_max(sync_member(sync, j, 0), members, tag, sync, spin_limit);
+            // a group that gave up is published as the bf16 NaN pattern, so every reader's result is NaN as well
+            const uint64_t payload = gm == gm ? (uint64_t)(__float_as_uint(gm) >> 16) : 0x7fc0ull;
+            if (threadIdx.x < ngroups) METIS_AT_STORE(sync_copy(sync, threadIdx.x, j), (tag << 16) | payload);
         }
-        const float all = poll_tagged_max(sync_copy(sync, j, 0), ngroups, tag, sync);
+        float all = poll_tagged_max(sync_copy(sync, j, 0), ngroups, tag, sync, spin_limit);
+        if (METIS_AT_LOAD(sync_timeout(sync)) != 0u) all = __builtin_nanf("");   // sticky: this call or an earlier one gave up
         if (threadIdx.x == 0) {
             sh.result = all;
             if (blockIdx.x == 0) METIS_AT_STORE(sync_generation(sync), tag);
@@ -406,7 +414,7 @@ __device__ __forceinline__ float grid_max_wait(uint64_t tag, uint32_t* sync, Gri
 template <int MODE, int NB>
 __global__ __launch_bounds__(256) void quant_fused_kernel(const uint16_t* __restrict__ x, uint2* __restrict__ codes,
                                                           uint8_t* __restrict__ scales, float* __restrict__ unit_out,
-                                                          uint32_t* __restrict__ sync, uint32_t nblocks)
+                                                          uint32_t* __restrict__ sync, uint32_t nblocks, uint32_t spin_limit)
 {
     __shared__ GridMaxState sh;
     const uint64_t tag = grid_max_begin(sync);
@@ -431,8 +439,8 @@ __global__ __launch_bounds__(256) void quant_fused_kernel(const uint16_t* __rest
         if (i < nblocks) codes[i] = encode_block<MODE, false>(v, block_scalar<MODE>(am[k]), none);
         c0 = n0; c1 = n1;
     }
-    const float amax = grid_max_wait(tag, sync, sh);
-    const float unit = rd<MODE>(block_scalar<MODE>(amax) / 448.0f);          // quant.py:21-22
+    const float amax = grid_max_wait(tag, sync, sh, spin_limit);
+    const float unit = rd<MODE>(block_scalar<MODE>(amax) / 448.0f);          // quant.py:21-22 (NaN after a time-out)
     if (i0 == 0) *unit_out = unit;
 #pragma unroll
     for (int k = 0; k < NB; ++k) {
@@ -521,25 +529,25 @@ static int fused_capacity()
 
 template <int MODE, int NB>
 static int try_fused(const void* x, void* codes, void* scales, float* unit, const Workspace& ws, uint32_t nblocks,
-                     hipStream_t st)
+                     hipStream_t st, uint32_t spin_limit)
 {
     int cap = fused_capacity<MODE, NB>();
     if (cap > kFusedMaxGrid) cap = kFusedMaxGrid;
     const int64_t need = ((int64_t)nblocks + 256 * NB - 1) / (256 * NB);
     if (cap <= 0 || need > cap) return 1;                      // does not fit: caller picks another path
     hipLaunchKernelGGL((quant_fused_kernel<MODE, NB>), dim3((unsigned)need), dim3(256), 0, st, (const uint16_t*)x,
-                       (uint2*)codes, (uint8_t*)scales, unit, ws.sync, nblocks);
+                       (uint2*)codes, (uint8_t*)scales, unit, ws.sync, nblocks, spin_limit);
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 
 template <int MODE>
 static int launch_fused(const void* x, void* codes, void* scales, float* unit, const Workspace& ws, uint32_t nblocks,
-                        hipStream_t st)
+                        hipStream_t st, uint32_t spin_limit)
 {
-    int rc = try_fused<MODE, 1>(x, codes, scales, unit, ws, nblocks, st);
-    if (rc == 1) rc = try_fused<MODE, 2>(x, codes, scales, unit, ws, nblocks, st);
-    if (rc == 1) rc = try_fused<MODE, 4>(x, codes, scales, unit, ws, nblocks, st);
-    if (rc == 1) rc = try_fused<MODE, 8>(x, codes, scales, unit, ws, nblocks, st);
+    int rc = try_fused<MODE, 1>(x, codes, scales, unit, ws, nblocks, st, spin_limit);
+    if (rc == 1) rc = try_fused<MODE, 2>(x, codes, scales, unit, ws, nblocks, st, spin_limit);
+    if (rc == 1) rc = try_fused<MODE, 4>(x, codes, scales, unit, ws, nblocks, st, spin_limit);
+    if (rc == 1) rc = try_fused<MODE, 8>(x, codes, scales, unit, ws, nblocks, st, spin_limit);
     return rc;
 }
 
@@ -571,7 +579,7 @@ static int launch_quant(const void* x, int64_t rows, int64_t cols, int64_t ld, c
 
 int quantize(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, bool sr, bool col, const void* noise,
              uint64_t seed, uint64_t offset, void* codes, void* scales, float* unit, void* workspace,
-             size_t workspace_bytes, hipStream_t st, const void* center)
+             size_t workspace_bytes, hipStream_t st, const void* center, bool resident, uint32_t spin_limit)
 {
     if (rows < 0 || cols < 0 || ld < cols) return METIS_E_ARG;
     if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16 && mode != METIS_MODE_P32_F32) return METIS_E_ARG;
@@ -588,10 +596,11 @@ int quantize(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, bo
     Workspace ws;
     int rc = carve_workspace(workspace, workspace_bytes, rows, cols, &ws);
     if (rc != METIS_OK) return rc;
-    if (!sr && !col && !wide && !center && ld == cols && getenv("METIS_FUSED_QUANT")) {   // opt-in single-launch path; falls through when it does not fit
+    if (resident && !sr && !col && !wide && !center && ld == cols) {   // opt-in single-launch path; falls through when it does not fit
         const uint32_t nblocks = (uint32_t)(rows * cols / kBlock);
-        rc = mode == 0 ? launch_fused<0>(x, codes, scales, unit, ws, nblocks, st)
-                       : launch_fused<1>(x, codes, scales, unit, ws, nblocks, st);
+        if (spin_limit == 0) spin_limit = kSpinLimit;
+        rc = mode == 0 ? launch_fused<0>(x, codes, scales, unit, ws, nblocks, st, spin_limit)
+                       : launch_fused<1>(x, codes, scales, unit, ws, nblocks, st, spin_limit);
         if (rc != 1) return rc;
     }
 #define METIS_Q(M, S, C) return launch_quant<M, S, C>(x, rows, cols, ld, noise, seed, offset, codes, scales, unit, ws, st, 0, center)

@@ -108,7 +108,7 @@ def _as_2d_for_quant(x: torch.Tensor, mode: int) -> tuple[torch.Tensor, int]:
 
 def quantize(x: torch.Tensor, mode: int = MODE_P32, *, col: bool = False, sr: bool = False,
              noise: torch.Tensor | None = None, seed: int = 0, offset: int = 0,
-             center: torch.Tensor | None = None) -> PackedNVFP4:
+             center: torch.Tensor | None = None, resident: bool = False, spin_limit: int = 0) -> PackedNVFP4:
     """NVFP4-quantize x (flattened to [R, C]).
 
     col=False: blocks of 16 along C -> PackedNVFP4 of shape (R, C).
@@ -117,6 +117,9 @@ def quantize(x: torch.Tensor, mode: int = MODE_P32, *, col: bool = False, sr: bo
                overrides the internal Philox stream keyed by (seed, offset).
     center   : [C] vector subtracted from every row first (the reference's mean mode), in the arithmetic's
                dtype: the packed tensor is that of x - center.
+    resident : round-to-nearest rows of a bf16 tensor as ONE launch (metis_nvfp4_quant_row_resident): the caller
+               guarantees that nothing else keeps the launch's workgroups from being resident together.  A wait
+               that gives up after `spin_limit` polls (0: library default) leaves a NaN unit.
     """
     x2, kmode = _as_2d_for_quant(x, mode)
     rows, cols = x2.shape
@@ -152,6 +155,9 @@ def quantize(x: torch.Tensor, mode: int = MODE_P32, *, col: bool = False, sr: bo
         rc = fn(x2.data_ptr(), rows, cols, x2.stride(0), kmode, None if nz is None else nz.data_ptr(),
                 seed & (2 ** 64 - 1), offset, codes.data_ptr(), scales.data_ptr(), unit.data_ptr(),
                 ws.data_ptr(), ws.numel(), _stream())
+    elif resident and not col and kmode in (MODE_P32, MODE_PB16) and x2.stride(0) == cols:
+        rc = L.metis_nvfp4_quant_row_resident(x2.data_ptr(), rows, cols, kmode, codes.data_ptr(), scales.data_ptr(),
+                                              unit.data_ptr(), ws.data_ptr(), ws.numel(), int(spin_limit), _stream())
     else:
         fn = L.metis_nvfp4_quant_col if col else L.metis_nvfp4_quant_row
         rc = fn(x2.data_ptr(), rows, cols, x2.stride(0), kmode, codes.data_ptr(), scales.data_ptr(),
@@ -359,8 +365,10 @@ def _gemm_workspace(M: int, N: int, K: int, device: torch.device) -> torch.Tenso
 
 def linear_fwd(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None, u: torch.Tensor | None = None,
                bias: torch.Tensor | None = None, out_dtype: torch.dtype = torch.bfloat16,
-               expanded: bool | None = None) -> torch.Tensor:
+               expanded: bool | None = None, split_k: bool = True) -> torch.Tensor:
     """out[M, N] = deq(a)[M, K] . deq(b)[N, K]^T (+ t[M, r] . u[N, r]^T) (+ bias[N]).
+
+    split_k=False withholds the split-K workspace: the contraction then runs unsplit in one launch.
 
     expanded=True runs on cached exact f16 expansions of a and b (2 B/element extra HBM, inner loop of
     MFMA + LDS reads only); the default works on the packed operands directly."""
@@ -395,7 +403,7 @@ def linear_fwd(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None,
                                               tp, up, r, bp, out.data_ptr(), dt, _stream())
         check(rc, "metis_linear_fwd_expanded", (M, N, K))
         return out
-    ws = _gemm_workspace(M, N, K, dev)
+    ws = _gemm_workspace(M, N, K, dev) if split_k else None
     if bias_f32:
         rc = load().metis_linear_fwd_f32bias(a.codes.data_ptr(), a.scales.data_ptr(), a.unit.data_ptr(), b.codes.data_ptr(),
                                              b.scales.data_ptr(), b.unit.data_ptr(), M, N, K, tp, up, r, bp, out.data_ptr(), dt,
@@ -438,7 +446,7 @@ def lowrank_project(x2: torch.Tensor, v: torch.Tensor, s: torch.Tensor | None = 
 
 
 def linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.bfloat16,
-                       center: torch.Tensor | None = None) -> list[torch.Tensor]:
+                       center: torch.Tensor | None = None, split_k: bool = True) -> list[torch.Tensor]:
     """[linear_fwd(a, b, t=t, u=u, bias=bias) for (b, t, u, bias) in members] in one call: a projection group
     (q/k/v, gate/up) that shares one packed activation.  Decode-sized batches run as a single launch.
 
@@ -477,6 +485,9 @@ def linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.b
     ap = ctypes.cast(arr, ctypes.c_void_p)
     # split-K scratch (long K, few columns) and whether a centre fits the launch: functions of the shape alone
     need, centre_ok = _grouped_plan(M, K, tuple(m[0].rows for m in members), dev.index or 0)
+    if not split_k:
+        need, centre_ok = 0, bool(load().metis_linear_grouped_centered_supported(
+            M, K, ctypes.cast(arr, ctypes.c_void_p), len(members), 0))
     ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
     dt = DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16
     if center is not None:

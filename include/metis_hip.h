@@ -82,6 +82,22 @@ int metis_nvfp4_quant_row(const void *x, int64_t rows, int64_t cols, int64_t ld,
                           size_t workspace_bytes, void *stream);
 
 /*
+ * metis_nvfp4_quant_row (contiguous rows) as ONE launch when every workgroup of that launch can be resident on
+ * the device at once: block maxima stay in registers across a grid-wide maximum taken through tagged words of
+ * the workspace, so neither the parked maxima nor the second kernel are needed.  Same bytes as
+ * metis_nvfp4_quant_row.  Tensors too large for one resident launch take the two-launch path.
+ * Opt-in because the caller has to guarantee what the library cannot see: for the duration of the call no
+ * other kernel may keep its workgroups from becoming resident (in particular no second call of this entry
+ * point on another stream).  The grid-wide wait is bounded: after `spin_limit` polls (0 = the default of 2^20,
+ * about a second) a workgroup gives up, every wave still exits, *unit is NaN (scale bytes 0x7F) and the
+ * workspace stays poisoned -- every later call on it also yields a NaN unit -- until the caller zero-fills
+ * it again.  Same arithmetic as quant.py:6-36; the reference has no counterpart for the launch structure.
+ */
+int metis_nvfp4_quant_row_resident(const void *x, int64_t rows, int64_t cols, int mode, void *codes,
+                                   void *scales, float *unit, void *workspace, size_t workspace_bytes,
+                                   uint32_t spin_limit, void *stream);
+
+/*
  * Same quantizer with blocks of 16 along dimension 0 (tokens), written transposed: the operand
  * layout of a GEMM that contracts over tokens.  Equals metis_nvfp4_quant_row applied to x^T.
  * The reference quantizes dY along its last dimension only (src/Metis/Metis/bitlinear.py:

@@ -104,11 +104,10 @@ def test_dgrad_and_wgrad():
     assert rel_fro(gw.cpu(), dy.double().T @ x.double()) < 0.25
 
 
-def test_expanded_path_is_bit_identical_to_packed_path(monkeypatch):
+def test_expanded_path_is_bit_identical_to_packed_path():
     """metis_linear_fwd_expanded on exact f16 expansions == metis_linear_fwd on packed operands
     (with K unsplit: splitting changes the order of the binary32 additions)."""
     from metis_hip import ops
-    monkeypatch.setenv("METIS_GEMM_NOSPLIT", "1")
     M, N, K, r = 512, 768, 1024, 64
     x = synthetic_activation(40, M, K)
     w = _weights(41, N, K)
@@ -154,7 +153,7 @@ def test_decode_shapes_with_lowrank_and_bias(M, N, K, r):
 
 @pytest.mark.parametrize("M,N,K,r", [(256, 512, 4096, 64), (300, 260, 4096, 0), (512, 3584, 2048, 32), (1024, 1536, 4160, 64),
                                      (260, 776, 18944, 0)])
-def test_split_k_shapes(M, N, K, r, monkeypatch):
+def test_split_k_shapes(M, N, K, r):
     """Few output tiles and a long contraction: up to 16 workgroups share a tile, partial tiles meet in a
     caller-supplied workspace.  Covers ragged M and N (N % 8 != 0 takes the plain stores), step counts that
     do not divide by the number of splits, the low-rank term and the bias (which must enter exactly once)."""
@@ -179,14 +178,13 @@ def test_split_k_shapes(M, N, K, r, monkeypatch):
     assert rel_fro(got32.cpu(), want.cpu()) <= 1e-5
     assert rel_fro(got.cpu(), want.cpu().bfloat16()) <= TOL
     # and against the unsplit kernel on the same operands
-    monkeypatch.setenv("METIS_GEMM_NOSPLIT", "1")
-    whole32 = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, out_dtype=torch.float32)
+    whole32 = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, out_dtype=torch.float32, split_k=False)
     torch.cuda.synchronize()
     assert rel_fro(got32.cpu(), whole32.cpu()) <= 1e-5
 
 
 @pytest.mark.parametrize("M,N,K,r", [(4096, 4352, 1024, 32), (4100, 4004, 2112, 0), (4096, 8960, 1536, 64)])
-def test_split_k_of_the_last_partial_round(M, N, K, r, monkeypatch):
+def test_split_k_of_the_last_partial_round(M, N, K, r):
     """A tile count a little over a multiple of the compute units (272 or 560 tiles on 256 units): the full rounds
     run unsplit and write the output directly, only the tiles of the last round are split through the workspace.
     Both kinds of tile are checked against the double-precision product and against the unsplit kernel."""
@@ -212,9 +210,8 @@ def test_split_k_of_the_last_partial_round(M, N, K, r, monkeypatch):
     torch.cuda.synchronize()
     assert rel_fro(got32.cpu(), want.cpu()) <= 1e-5
     assert rel_fro(got.cpu(), want.cpu().bfloat16()) <= TOL
-    monkeypatch.setenv("METIS_GEMM_NOSPLIT", "1")
-    whole32 = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, out_dtype=torch.float32)
-    whole = ops.linear_fwd(px, pw, t=t, u=u, bias=bias)
+    whole32 = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, out_dtype=torch.float32, split_k=False)
+    whole = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, split_k=False)
     torch.cuda.synchronize()
     # the unsplit tiles are bit-identical to the unsplit kernel, the split ones differ in summation order only
     same = (got32 == whole32).float().mean().item()
@@ -302,7 +299,7 @@ def test_grouped_projections_equal_member_by_member_calls(M, K, Ns, r):
 
 @pytest.mark.parametrize("M,K,Ns,r", [(64, 18944, (3584,), 64), (1, 8192, (256,), 0), (200, 16384, (132, 64), 32),
                                       (33, 8256, (96,), 32)])
-def test_decode_sized_products_with_a_long_contraction_split_k(M, K, Ns, r, monkeypatch):
+def test_decode_sized_products_with_a_long_contraction_split_k(M, K, Ns, r):
     """Few output columns and a long K (a down projection at decode size): K is cut into slices that run as separate
     workgroups and a second kernel adds the binary32 partial sums.  Checked against the double-precision product of the
     dequantized operands, against the unsplit kernel (summation order only), and that the shape really is split."""
@@ -327,9 +324,7 @@ def test_decode_sized_products_with_a_long_contraction_split_k(M, K, Ns, r, monk
     for dt in (torch.float32, torch.bfloat16):
         got = ops.linear_fwd_grouped(px, members, out_dtype=dt)
         single = [ops.linear_fwd(px, pw, t=t, u=u, bias=b, out_dtype=dt) for pw, t, u, b in members]
-        monkeypatch.setenv("METIS_GEMM_NOSPLIT", "1")
-        unsplit = ops.linear_fwd_grouped(px, members, out_dtype=dt)
-        monkeypatch.delenv("METIS_GEMM_NOSPLIT")
+        unsplit = ops.linear_fwd_grouped(px, members, out_dtype=dt, split_k=False)
         for (pw, t, u, b), y, y1, y0 in zip(members, got, single, unsplit):
             want = da @ ops.dequantize(pw, torch.float32).double().T + b.double()
             if t is not None:

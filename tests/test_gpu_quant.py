@@ -3,6 +3,8 @@
 Bar: bit-exact codes, E4M3 scale bytes and unit in both parity modes; dequantized output equal
 to the reference's own golden QDQ output.
 """
+import math
+
 import numpy as np
 import pytest
 import torch
@@ -287,20 +289,44 @@ def test_full_size_config1(ops, tag, mode):
 
 
 @pytest.mark.parametrize("tag,mode", MODES)
-def test_single_launch_variant_matches_two_launch_path(ops, monkeypatch, tag, mode):
+def test_single_launch_variant_matches_two_launch_path(ops, tag, mode):
     """The opt-in single-launch kernel (grid-wide reduction through tagged words) gives the same
     bytes as the default two-launch path, call after call on one workspace (the generation tag
     advances each time) and across sizes that change the number of groups and members."""
     shapes = [(8192, 4096), (16, 16), (64, 256), (4096, 1536), (16384, 4096), (1000, 48), (8192, 4096), (2, 32)]
     for k, (r, c) in enumerate(shapes):
         x = synthetic_activation(300 + k, r, c).cuda()
-        monkeypatch.delenv("METIS_FUSED_QUANT", raising=False)
         ref = ops.quantize(x, mode)
-        monkeypatch.setenv("METIS_FUSED_QUANT", "1")
         for rep in range(3):
-            got = ops.quantize(x, mode)
+            got = ops.quantize(x, mode, resident=True)
             _check_packed(got, ref.codes.cpu(), ref.scales.cpu(), ref.unit.cpu(), f"shape {r}x{c} rep {rep} {tag}")
-    monkeypatch.delenv("METIS_FUSED_QUANT", raising=False)
+
+
+def test_single_launch_wait_that_gives_up_is_visible(ops):
+    """The grid-wide wait is bounded.  With a spin limit of one poll the first workgroup cannot see two thousand
+    others arrive: every kernel still exits, the unit comes back NaN (not a plausible wrong number), the workspace
+    stays poisoned for later calls, and a zero-filled workspace works again."""
+    from metis_hip import _lib
+    L = _lib.load()
+    rows, cols = 16384, 4096
+    x = synthetic_activation(777, rows, cols).cuda()
+    ref = ops.quantize(x, 0)
+    codes, scales, unit = torch.empty_like(ref.codes), torch.empty_like(ref.scales), torch.zeros(1, device="cuda")
+    ws = torch.zeros(L.metis_nvfp4_workspace_bytes(rows, cols), dtype=torch.uint8, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+
+    def call(limit):
+        rc = L.metis_nvfp4_quant_row_resident(x.data_ptr(), rows, cols, 0, codes.data_ptr(), scales.data_ptr(), unit.data_ptr(),
+                                              ws.data_ptr(), ws.numel(), limit, st)
+        assert rc == 0
+        torch.cuda.synchronize()
+        return float(unit.cpu())
+    assert call(0) == float(ref.unit.cpu())
+    assert math.isnan(call(1))                       # gave up
+    assert math.isnan(call(0))                       # poisoned workspace: still NaN
+    ws.zero_()
+    assert call(0) == float(ref.unit.cpu())
+    assert torch.equal(codes, ref.codes) and torch.equal(scales, ref.scales)
 
 
 @pytest.mark.parametrize("tag,mode", MODES)
