@@ -116,7 +116,7 @@ def test_expanded_path_is_bit_identical_to_packed_path():
     u = torch.randn(N, r, generator=g).bfloat16().cuda()
     bias = torch.randn(N, generator=g).bfloat16().cuda()
     px, pw = ops.quantize(x.cuda()), ops.quantize(w.cuda())
-    a = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, out_dtype=torch.float32, expanded=False)
+    a = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, out_dtype=torch.float32, expanded=False, split_k=False)
     b = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, out_dtype=torch.float32, expanded=True)
     assert torch.equal(a, b)
     # the expansion itself: e2m1 * e4m3 * 2^-8, exact
