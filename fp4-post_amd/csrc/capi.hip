@@ -31,6 +31,7 @@ const char* metis_error_string(int code)
         case METIS_E_WORKSPACE: return "workspace missing, misaligned or too small";
         case METIS_E_LAUNCH: return "HIP runtime rejected a kernel launch";
         case METIS_E_DEVICE: return "unsupported device";
+        case METIS_E_TOO_LARGE: return "tensor exceeds the capacity of the library's static scratch (2^26 elements)";
         default: return "unknown error code";
     }
 }
@@ -46,6 +47,12 @@ int metis_nvfp4_quant_row(const void* x, int64_t rows, int64_t cols, int64_t ld,
 {
     return quantize(x, rows, cols, ld, mode, false, false, nullptr, 0, 0, codes, scales, unit, workspace,
                     workspace_bytes, (hipStream_t)stream);
+}
+
+int metis_nvfp4_quant_row_static(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, void* codes, void* scales,
+                                 float* unit, void* stream)
+{
+    return quantize_row_static(x, rows, cols, ld, mode, codes, scales, unit, (hipStream_t)stream);
 }
 
 int metis_nvfp4_quant_row_resident(const void* x, int64_t rows, int64_t cols, int mode, void* codes, void* scales,

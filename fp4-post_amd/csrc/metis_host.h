@@ -47,6 +47,9 @@ int quantize(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, bo
              uint64_t seed, uint64_t offset, void* codes, void* scales, float* unit, void* workspace,
              size_t workspace_bytes, hipStream_t st, const void* center = nullptr, bool resident = false,
              uint32_t spin_limit = 0);
+// the row quantizer on the library's own static scratch (no workspace argument); nvfp4_quant.hip
+int quantize_row_static(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, void* codes, void* scales,
+                        float* unit, hipStream_t st);
 int dequantize(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, int mode, void* out,
                int out_dtype, hipStream_t st);
 int block_scalars(const void* x, int64_t rows, int64_t cols, int mode, void* s, hipStream_t st);

@@ -12,6 +12,7 @@
 #include "metis_device.h"
 #include "metis_host.h"
 #include "nvfp4_encode.h"
+#include <atomic>
 #include <stdio.h>
 #include <stdlib.h>
 #include <type_traits>
@@ -618,6 +619,47 @@ int quantize(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, bo
         else { if (!col) METIS_Q(1, true, false); else METIS_Q(1, true, true); }
     }
 #undef METIS_Q
+}
+
+// ---------------------------------------------------------------------------------------------
+// Allocation-free variant of the row quantizer: the workspace (per-workgroup maxima, reduction words,
+// parked block maxima) is a file-scope device array instead of caller memory, for callers that cannot
+// allocate (HIP graph capture, serving loops).  Every device the library runs on holds its own copy of
+// the array at its own address until the process ends; the address is looked up once per device, with
+// that device current, and host code only ever uses that address, never the array's name.
+// ---------------------------------------------------------------------------------------------
+constexpr int64_t kStaticMaxElements = (int64_t)1 << 26;         // 64 Mi elements, e.g. [16384, 4096]
+constexpr size_t kStaticScratchBytes = kWsGmaxBytes + kWsSyncBytes + (size_t)(kStaticMaxElements / kBlock) * 4;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+static int static_scratch(void** out)
+{
+    static std::atomic<void*> ptrs[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return METIS_E_DEVICE;
+    void* p = ptrs[dev].load(std::memory_order_acquire);
+    if (!p) {
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) {
+            (void)hipGetLastError();
+            return METIS_E_DEVICE;
+        }
+        ptrs[dev].store(p, std::memory_order_release);         // two racing first calls store the same address
+    }
+    *out = p;
+    return METIS_OK;
+}
+
+int quantize_row_static(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, void* codes, void* scales,
+                        float* unit, hipStream_t st)
+{
+    if (rows < 0 || cols < 0) return METIS_E_ARG;
+    if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16 && mode != METIS_MODE_P32_F32) return METIS_E_ARG;
+    if (rows > 0 && cols > kStaticMaxElements / rows) return METIS_E_TOO_LARGE;
+    static_assert(kStaticScratchBytes >= kWsGmaxBytes + kWsSyncBytes + (size_t)(kStaticMaxElements / kBlock) * 4, "scratch too small");
+    void* ws = nullptr;
+    if (const int rc = static_scratch(&ws)) return rc;
+    // the two-launch path: nothing in the scratch has to start at zero (phase 1 rewrites every word phase 2 reads)
+    return quantize(x, rows, cols, ld, mode, false, false, nullptr, 0, 0, codes, scales, unit, ws, kStaticScratchBytes, st);
 }
 
 int dequantize(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, int mode, void* out,

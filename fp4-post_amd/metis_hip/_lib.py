@@ -11,7 +11,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmetis_hip.so")
 
-OK, E_ARG, E_SHAPE, E_WORKSPACE, E_LAUNCH, E_DEVICE = 0, -1, -2, -3, -4, -5
+OK, E_ARG, E_SHAPE, E_WORKSPACE, E_LAUNCH, E_DEVICE, E_TOO_LARGE = 0, -1, -2, -3, -4, -5, -6
 class LinearMember(ctypes.Structure):
     """metis_linear_member of include/metis_hip.h: one weight matrix of a grouped GEMM."""
     _fields_ = [("b_codes", ctypes.c_void_p), ("b_scales", ctypes.c_void_p), ("b_unit", ctypes.c_void_p),
@@ -32,6 +32,7 @@ SIGNATURES = {
     "metis_error_string": (ctypes.c_char_p, [_i32]),
     "metis_nvfp4_workspace_bytes": (_sz, [_i64, _i64]),
     "metis_nvfp4_quant_row": (_i32, [_vp, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "metis_nvfp4_quant_row_static": (_i32, [_vp, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _vp]),
     "metis_nvfp4_quant_row_resident": (_i32, [_vp, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _sz, ctypes.c_uint32, _vp]),
     "metis_nvfp4_quant_col": (_i32, [_vp, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _sz, _vp]),
     "metis_nvfp4_quant_sr_row": (_i32, [_vp, _i64, _i64, _i64, _i32, _vp, _u64, _u64, _vp, _vp, _vp, _vp, _sz, _vp]),

@@ -51,6 +51,7 @@ extern "C" {
 #define METIS_E_WORKSPACE (-3) /* workspace missing, misaligned or too small                   */
 #define METIS_E_LAUNCH (-4)    /* the HIP runtime rejected a launch                             */
 #define METIS_E_DEVICE (-5)    /* not a gfx950 device / required feature missing               */
+#define METIS_E_TOO_LARGE (-6) /* metis_nvfp4_quant_row_static: more elements than its scratch holds */
 
 #define METIS_MODE_P32 0
 #define METIS_MODE_PB16 1
@@ -80,6 +81,21 @@ size_t metis_nvfp4_workspace_bytes(int64_t rows, int64_t cols);
 int metis_nvfp4_quant_row(const void *x, int64_t rows, int64_t cols, int64_t ld, int mode,
                           void *codes, void *scales, float *unit, void *workspace,
                           size_t workspace_bytes, void *stream);
+
+/*
+ * metis_nvfp4_quant_row without a workspace argument and without any allocation: the scratch (per-workgroup
+ * maxima and the parked block maxima) is a static device array inside the library.  No counterpart in the
+ * reference; it exists for callers that cannot allocate device memory: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  Same kernels and same bytes as metis_nvfp4_quant_row.
+ *   limit   rows * cols <= 2^26 elements (METIS_E_TOO_LARGE beyond that; nothing is launched)
+ *   cost    every device the library runs on holds the 16.1 MiB array from first use until the process ends
+ *   sharing all calls on one device use that device's single array: calls that overlap in time on one
+ *           device (two streams, two host threads) race on it and must be ordered by the caller
+ * The call never calls hipMalloc/hipFree or any allocating routine; its first call on a device looks the
+ * array's address up once (hipGetSymbolAddress).
+ */
+int metis_nvfp4_quant_row_static(const void *x, int64_t rows, int64_t cols, int64_t ld, int mode,
+                                 void *codes, void *scales, float *unit, void *stream);
 
 /*
  * metis_nvfp4_quant_row (contiguous rows) as ONE launch when every workgroup of that launch can be resident on
