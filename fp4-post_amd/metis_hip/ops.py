@@ -32,6 +32,7 @@ class PackedNVFP4:
     cols: int
     mode: int = MODE_P32
     expanded: torch.Tensor | None = None      # cached exact f16 expansion e2m1 * e4m3 * 2^-8, see expand()
+    tiled: torch.Tensor | None = None         # the same expansion in the pipelined GEMM's tiled layout, see expand_tiled()
     transposed: "PackedNVFP4 | None" = None   # cached column-blocked packing of the same source tensor (dgrad operand)
 
     def dequantize(self, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
@@ -304,6 +305,48 @@ def expand(p: PackedNVFP4) -> torch.Tensor:
         check(rc, "metis_nvfp4_expand_f16", (p.rows, p.cols))
         p.expanded = out
     return p.expanded
+
+
+def expand_tiled(p: PackedNVFP4, cache: bool = True) -> torch.Tensor:
+    """Exact binary16 expansion of a packed tensor in the tiled layout of the pipelined GEMM (uint8 buffer).
+    cache=True keeps it on the packed tensor (weights); activations are expanded per call."""
+    if p.tiled is not None:
+        return p.tiled
+    L = load()
+    out = torch.empty(L.metis_nvfp4_expand_tiled_bytes(p.rows, p.cols), dtype=torch.uint8, device=p.codes.device)
+    rc = L.metis_nvfp4_expand_tiled(p.codes.data_ptr(), p.scales.data_ptr(), p.rows, p.cols, out.data_ptr(), _stream())
+    check(rc, "metis_nvfp4_expand_tiled", (p.rows, p.cols))
+    if cache:
+        p.tiled = out
+    return out
+
+
+def linear_fwd_tiled(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None, u: torch.Tensor | None = None,
+                     bias: torch.Tensor | None = None, out_dtype: torch.dtype = torch.bfloat16,
+                     a_tiled: torch.Tensor | None = None) -> torch.Tensor:
+    """linear_fwd on tiled binary16 expansions: b's is cached on b, a's is made here unless given."""
+    if a.cols != b.cols:
+        raise ValueError(f"contraction mismatch: {a.cols} vs {b.cols}")
+    M, N, K = a.rows, b.rows, a.cols
+    r = 0
+    if t is not None:
+        t = t.to(torch.bfloat16).contiguous()
+        u = u.to(torch.bfloat16).contiguous()
+        r = t.shape[1]
+        if t.shape != (M, r) or u.shape != (N, r):
+            raise ValueError("low-rank operands must be t[M, r], u[N, r]")
+    bias_f32 = bias is not None and bias.dtype == torch.float32
+    if bias is not None:
+        bias = bias.contiguous() if bias_f32 else bias.to(torch.bfloat16).contiguous()
+    bx = expand_tiled(b)
+    ax = a_tiled if a_tiled is not None else expand_tiled(a, cache=False)
+    out = torch.empty(M, N, dtype=out_dtype, device=a.codes.device)
+    rc = load().metis_linear_fwd_tiled(ax.data_ptr(), a.unit.data_ptr(), bx.data_ptr(), b.unit.data_ptr(), M, N, K,
+                                       None if t is None else t.data_ptr(), None if u is None else u.data_ptr(), r,
+                                       None if bias is None else bias.data_ptr(), int(bias_f32), out.data_ptr(),
+                                       DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16, _stream())
+    check(rc, "metis_linear_fwd_tiled", (M, N, K))
+    return out
 
 
 def rmsnorm_quantize(x: torch.Tensor, gamma: torch.Tensor, eps: float, mode: int = MODE_P32,

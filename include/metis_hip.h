@@ -225,6 +225,25 @@ int metis_linear_fwd_expanded(const void *a_exp, const float *a_unit, const void
                               const void *bias, void *out, int out_dtype, void *stream);
 
 /*
+ * The same expansion in the layout the pipelined GEMM streams from: tiles of 16 rows x 32 k (1 KiB each, tile
+ * (rb, kb) at byte ((rb * cols/32) + kb) * 1024, rows padded to a multiple of 16 with zeros), the 16-byte chunks of
+ * a tile permuted so that one direct-to-LDS load per tile leaves it free of bank conflicts for the MFMA fragment
+ * reads.  metis_linear_fwd_tiled then runs a main loop of MFMA and LDS reads only, its operand tiles arriving
+ * through a four-stage ring of direct loads; results equal metis_linear_fwd on the packed operands bit for bit
+ * (same exact products, same order of binary32 accumulation).  Derived data like the expansion above: callers
+ * cache a weight's tiled expansion next to its packed form and re-expand an activation per call (2 B/element).
+ *   metis_nvfp4_expand_tiled_bytes  size of `out` for a [rows, cols] packed tensor
+ *   limits  cols % 32 == 0; GEMM: K % 32 == 0, N % 4 == 0, r % 32 == 0; out, t, u 16-byte aligned
+ *   bias    bf16 [N], or float [N] when bias_is_f32 != 0, or NULL
+ */
+size_t metis_nvfp4_expand_tiled_bytes(int64_t rows, int64_t cols);
+int metis_nvfp4_expand_tiled(const void *codes, const void *scales, int64_t rows, int64_t cols, void *out,
+                             void *stream);
+int metis_linear_fwd_tiled(const void *a_xt, const float *a_unit, const void *b_xt, const float *b_unit,
+                           int64_t M, int64_t N, int64_t K, const void *t, const void *u, int64_t r,
+                           const void *bias, int bias_is_f32, void *out, int out_dtype, void *stream);
+
+/*
  * grad_input[L,K] = deq(dY)[L,N] . deq(W)[N,K]   (src/Metis/Metis/bitlinear.py:507-508)
  *   dy_* : dY packed with blocks along N (metis_nvfp4_quant_sr_row of dY [L,N])
  *   wt_* : W packed with blocks along N  (metis_nvfp4_quant_col of W [N,K] -> [K, N/2])

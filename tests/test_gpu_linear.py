@@ -124,6 +124,44 @@ def test_expanded_path_is_bit_identical_to_packed_path():
     assert rel_fro(e.cpu(), ops.dequantize(px, torch.float32).cpu()) < 1e-6
 
 
+@pytest.mark.parametrize("M,N,K,r,bias_f32", [(512, 768, 1024, 64, False), (300, 260, 32, 0, False), (256, 256, 96, 32, True),
+                                              (1000, 516, 2112, 64, True), (2048, 1024, 4096, 0, False)])
+def test_tiled_pipelined_path_is_bit_identical_to_packed_path(M, N, K, r, bias_f32):
+    """metis_linear_fwd_tiled (operands expanded once into the tiled binary16 layout, direct-to-LDS ring) against
+    metis_linear_fwd on the packed operands, unsplit: the same exact products summed in the same order.  Covers
+    ragged M and N (tile rows padded with zeros, rows clamped), K shorter than the ring, and both bias and output
+    types; and against the double-precision product of the dequantized operands."""
+    from metis_hip import ops
+    g = torch.Generator().manual_seed(4000 + M)
+    x = synthetic_activation(60 + M, M, K).cuda()
+    w = _weights(61 + N, N, K).cuda()
+    t = u = None
+    if r:
+        t = torch.randn(M, r, generator=g).bfloat16().cuda()
+        u = torch.randn(N, r, generator=g).bfloat16().cuda()
+    bias = torch.randn(N, generator=g)
+    bias = bias.cuda() if bias_f32 else bias.bfloat16().cuda()
+    px, pw = ops.quantize(x), ops.quantize(w)
+    want = ops.dequantize(px, torch.float32).double() @ ops.dequantize(pw, torch.float32).double().T + bias.double()
+    if r:
+        want = want + t.double() @ u.double().T
+    for dt in (torch.float32, torch.bfloat16):
+        a = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, out_dtype=dt, split_k=False)
+        b = ops.linear_fwd_tiled(px, pw, t=t, u=u, bias=bias, out_dtype=dt)
+        torch.cuda.synchronize()
+        assert rel_fro(b.cpu(), want.cpu().to(dt)) <= (1e-5 if dt == torch.float32 else TOL)
+        assert torch.equal(a, b), f"{(a != b).sum().item()} of {a.numel()} elements differ ({dt})"
+    # the tiled expansion holds exactly the values of the row-major one
+    e = ops.expand(px)
+    tiles = ops.expand_tiled(px, cache=False).view(torch.float16).reshape(-1, K // 32, 16, 4, 8)
+    rows = torch.arange(16, device="cuda")
+    swz = ((rows >> 2) & 1) | ((((rows >> 1) ^ (rows >> 3)) & 1) << 1)
+    slot = torch.arange(4, device="cuda")[None, :] ^ swz[:, None]                  # [16 rows, 4 chunks] -> slot
+    unswz = torch.gather(tiles, 3, slot[None, None, :, :, None].expand(tiles.shape[0], tiles.shape[1], 16, 4, 8))
+    flat = unswz.permute(0, 2, 1, 3, 4).reshape(-1, K)[:M]
+    assert torch.equal(flat, e)
+
+
 @pytest.mark.parametrize("M,N,K,r", [(64, 4736, 3584, 64), (17, 2052, 2048, 0), (1, 4608, 3584, 32), (40, 1536, 8960, 64),
                                      (64, 18944, 3584, 64)])
 def test_decode_shapes_with_lowrank_and_bias(M, N, K, r):
