@@ -132,6 +132,7 @@ def main():
     # ------------------------------------------------------------------ headline: config 3
     x, v, s, u, res = config3_inputs(torch, dev, M, K, N, r)
     pw = ops.quantize(res)                                     # cached packed residual weight
+    pw.persistent = True                                       # as LinearLowbit marks a cached weight: its tiled expansion is kept
     vt = v.T.contiguous()
 
     # parity gate before any timing (bf16 vs bf16, P32): a 256-row slice against the CPU oracle

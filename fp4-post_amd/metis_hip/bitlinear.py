@@ -495,6 +495,8 @@ class LinearLowbit(nn.Module):
         else:
             q = F.q_forward_weight.quantize_dequantize(weight_compute)
         if self.cache_quantized_weight:
+            if isinstance(q, PackedNVFP4):
+                q.persistent = True                  # reused until the parameter changes: derived layouts may be kept on it
             self._quantized_weight_cache = (key, q)
         return q
 

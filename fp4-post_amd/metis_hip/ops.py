@@ -34,6 +34,7 @@ class PackedNVFP4:
     expanded: torch.Tensor | None = None      # cached exact f16 expansion e2m1 * e4m3 * 2^-8, see expand()
     tiled: torch.Tensor | None = None         # the same expansion in the pipelined GEMM's tiled layout, see expand_tiled()
     transposed: "PackedNVFP4 | None" = None   # cached column-blocked packing of the same source tensor (dgrad operand)
+    persistent: bool = False                  # lives across calls (a cached weight): worth keeping its tiled expansion
 
     def dequantize(self, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
         return dequantize(self, dtype)
@@ -372,6 +373,25 @@ def rmsnorm_quantize(x: torch.Tensor, gamma: torch.Tensor, eps: float, mode: int
     return normed, PackedNVFP4(codes, scales, unit, rows, cols, mode)
 
 
+@functools.lru_cache(maxsize=16)
+def _device_cus(device_index: int) -> int:
+    return int(torch.cuda.get_device_properties(device_index).multi_processor_count)
+
+
+def _tiled_applies(a: PackedNVFP4, b: PackedNVFP4) -> bool:
+    """The pipelined GEMM on tiled binary16 expansions pays when the weight-side expansion is reused across calls
+    (a cached weight) and the shape fills the device at least once with 256 x 256 tiles; the activation side is
+    expanded per call (2.56 B/element, about 2 % of the GEMM's time at such shapes).  Shapes with fewer tiles than
+    compute units stay on the packed kernels, which can split K."""
+    if not (b.persistent or b.tiled is not None):
+        return False
+    M, N, K = a.rows, b.rows, a.cols
+    if M < 256 or N < 256 or K % 32 or K < 128:
+        return False
+    tiles = ((M + 255) // 256) * ((N + 255) // 256)
+    return tiles >= _device_cus(a.codes.device.index or 0)
+
+
 @functools.lru_cache(maxsize=4096)
 def _linear_workspace_bytes(M: int, N: int, K: int, device_index: int) -> int:
     return int(load().metis_linear_workspace_bytes(M, N, K))          # depends on the device's CU count only
@@ -408,8 +428,11 @@ def _gemm_workspace(M: int, N: int, K: int, device: torch.device) -> torch.Tenso
 
 def linear_fwd(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None, u: torch.Tensor | None = None,
                bias: torch.Tensor | None = None, out_dtype: torch.dtype = torch.bfloat16,
-               expanded: bool | None = None, split_k: bool = True) -> torch.Tensor:
+               expanded: bool | None = None, split_k: bool = True, tiled: bool | None = None) -> torch.Tensor:
     """out[M, N] = deq(a)[M, K] . deq(b)[N, K]^T (+ t[M, r] . u[N, r]^T) (+ bias[N]).
+
+    tiled=None picks the pipelined kernel on tiled binary16 expansions when b is a cached weight and the shape is
+    large (see _tiled_applies); True / False force the choice.  Same bits either way (unsplit).
 
     split_k=False withholds the split-K workspace: the contraction then runs unsplit in one launch.
 
@@ -417,6 +440,10 @@ def linear_fwd(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None,
     MFMA + LDS reads only); the default works on the packed operands directly."""
     if a.cols != b.cols:
         raise ValueError(f"contraction mismatch: {a.cols} vs {b.cols}")
+    if tiled is None:
+        tiled = not expanded and _tiled_applies(a, b)
+    if tiled:
+        return linear_fwd_tiled(a, b, t=t, u=u, bias=bias, out_dtype=out_dtype)
     M, N, K = a.rows, b.rows, a.cols
     dev = a.codes.device
     r = 0
