@@ -80,8 +80,8 @@ int expand_xt(const void* codes, const void* scales, int64_t rows, int64_t cols,
 // ---------------------------------------------------------------------------------------------
 // The GEMM.  256 x 256 per workgroup; WN_WAVES = 4: eight waves (2 x 4) of 128 x 64, two per SIMD;
 // WN_WAVES = 2: four waves (2 x 2) of 128 x 128, one per SIMD (a third less LDS read traffic).
-// A stage is 32 k of the A|B tile: 32 KiB = 32 operand tiles, one direct load each.  NS stages form a
-// ring.  Iteration s (stage s in slot s % NS):
+// A stage is 32 k of the A|B tile: 32 KiB = 32 operand tiles, one direct load each.  NS slots of KS stages form a
+// ring (shipped: three slots of one stage, 96 KiB).  Iteration s (stage s in slot s % NS):
 //     read fragments (s, k 16..31)            | MFMAs on fragments (s, k 0..15)
 //     wait: own fragment reads done, own loads of stage s+1 landed;  BARRIER
 //     issue loads of stage s+NS into slot s % NS (every wave holds what it needs of stage s in registers)
@@ -96,7 +96,7 @@ __host__ __device__ constexpr int waitcnt_imm(int vm, int lgkm)
 }
 #define METIS_WAIT(VM, LGKM) __builtin_amdgcn_s_waitcnt(waitcnt_imm(VM, LGKM))
 
-template <int OUT_F32, int WN_WAVES, int NS>
+template <int OUT_F32, int WN_WAVES, int NS, int KS = 1, int ILV = 0>
 __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_xt_kernel(
     const uint8_t* __restrict__ a_xt, const float* __restrict__ a_unit, const uint8_t* __restrict__ b_xt,
     const float* __restrict__ b_unit, int M, int N, int K, const uint16_t* __restrict__ t, const uint16_t* __restrict__ u,
@@ -140,14 +140,18 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_xt_kernel(
         src[j] = (is_a ? a_xt : b_xt) + (int64_t)rt * kt * 1024;
     }
     const uint32_t lane16 = lane * 16;
-    auto issue = [&](int slot, int kb) {
+    constexpr int SLOT = KS * XT_STAGE;                         // a ring slot holds the KS stages of one iteration
+    constexpr int LPS = LPW * KS;                               // direct loads per wave per slot
+    auto issue_one = [&](int slot, int it, int n) {             // load n (0 .. LPS-1) of iteration `it` into `slot`
+        const int sub = n / LPW, j = n % LPW;
+        const uint8_t* g = src[j] + ((int64_t)it * KS + sub) * 1024;
+        const uint32_t dst = (uint32_t)(slot * SLOT + sub * XT_STAGE + (j * NWAVES + wave) * 1024);   // LDS byte address of the tile
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                     :: "v"(lane16), "s"(g), "s"(dst) : "memory");
+    };
+    auto issue = [&](int slot, int it) {
 #pragma unroll
-        for (int j = 0; j < LPW; ++j) {
-            const uint8_t* g = src[j] + (int64_t)kb * 1024;
-            const uint32_t dst = (uint32_t)(slot * XT_STAGE + (j * NWAVES + wave) * 1024);   // LDS byte address of the tile
-            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                         :: "v"(lane16), "s"(g), "s"(dst) : "memory");
-        }
+        for (int n = 0; n < LPS; ++n) issue_one(slot, it, n);
     };
 
     // ---- fragment addressing: lane -> row lr of a 32-row MFMA tile, k half hi; chunk = 2 * ks + hi.
@@ -157,12 +161,12 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_xt_kernel(
     const int a_off[2] = {wm * 8 * 1024 + lane_off, wm * 8 * 1024 + (lane_off ^ 32)};
     const int b_off[2] = {(16 + wn * (WTN / 16)) * 1024 + lane_off, (16 + wn * (WTN / 16)) * 1024 + (lane_off ^ 32)};
     half8_t fa[2][TM], fb[2][TN];
-    auto load_frags = [&](int fbuf, int slot, int ks) {
-        const int x = slot * XT_STAGE;
+    auto load_frags = [&](int slot, int q) {                    // sub-step q of the slot: stage q / 2, k half q % 2; buffer q % 2
+        const int x = slot * SLOT + (q >> 1) * XT_STAGE;
 #pragma unroll
-        for (int i = 0; i < TM; ++i) fa[fbuf][i] = *reinterpret_cast<const half8_t*>(xlds + (a_off[ks] + x) + i * 2048);
+        for (int i = 0; i < TM; ++i) fa[q & 1][i] = *reinterpret_cast<const half8_t*>(xlds + (a_off[q & 1] + x) + i * 2048);
 #pragma unroll
-        for (int j = 0; j < TN; ++j) fb[fbuf][j] = *reinterpret_cast<const half8_t*>(xlds + (b_off[ks] + x) + j * 2048);
+        for (int j = 0; j < TN; ++j) fb[q & 1][j] = *reinterpret_cast<const half8_t*>(xlds + (b_off[q & 1] + x) + j * 2048);
     };
     auto mfmas = [&](int fbuf) {
 #pragma unroll
@@ -172,49 +176,67 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_xt_kernel(
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[fbuf][j], fa[fbuf][i], acc[i][j], 0, 0, 0);
     };
     constexpr int NM = TM * TN, NF = TM + TN;
+    constexpr int QL = 2 * KS - 1;                              // last sub-step of an iteration
 
-    const int steps = kt;
+    const int steps = kt / KS;                                  // iterations (the host picks KS = 1 unless KS divides K / 32)
     // prologue: fill the ring
 #pragma unroll
     for (int p = 0; p < NS; ++p)
         if (p < steps) issue(p, p);
-    if (steps >= NS) METIS_WAIT((NS - 1) * LPW, 15);
+    if (steps >= NS) METIS_WAIT((NS - 1) * LPS, 15);
     else METIS_WAIT(0, 15);
     __syncthreads();
-    load_frags(0, 0, 0);
+    load_frags(0, 0);
 
+    // the sub-steps before the barrier: fragments of sub-step q+1 are read while the MFMAs of sub-step q run
+    auto head = [&](int slot) {
+#pragma unroll
+        for (int q = 0; q < QL; ++q) {
+            load_frags(slot, q + 1);
+            mfmas(q & 1);
+            sched_substep<NM, 0, NF, 0>();
+        }
+    };
     int s = 0, slot = 0;
-    // steady state: the stage NS ahead exists, so every wait allows NS-2 stages in flight
+    // steady state: the iteration NS ahead exists, so every wait allows NS-2 slots in flight
     for (; s + NS < steps; ++s) {
         const int nslot = slot + 1 == NS ? 0 : slot + 1;
-        load_frags(1, slot, 1);
-        mfmas(0);
-        sched_substep<NM, 0, NF, 0>();
-        METIS_WAIT((NS - 2) * LPW, 0);                          // own loads of stage s+1 landed, own fragment reads of stage s done
+        head(slot);
+        METIS_WAIT((NS - 2) * LPS, 0);                          // own loads of iteration s+1 landed, own fragment reads of s done
         __syncthreads();
-        issue(slot, s + NS);
-        load_frags(0, nslot, 0);
-        mfmas(1);
-        sched_substep<NM, 0, NF, 0>();
+        if constexpr (ILV != 0) {
+            // the direct loads are spread between the MFMAs of the last sub-step instead of issued in one burst
+            load_frags(nslot, 0);
+            constexpr int PER = (NM + LPS - 1) / LPS;
+#pragma unroll
+            for (int m = 0; m < NM; ++m) {
+                if (m % PER == 0 && m / PER < LPS) issue_one(slot, s + NS, m / PER);
+                const int i = m / TN, j = m % TN;
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[1][j], fa[1][i], acc[i][j], 0, 0, 0);
+            }
+        } else {
+            issue(slot, s + NS);
+            load_frags(nslot, 0);
+            mfmas(1);
+            sched_substep<NM, 0, NF, 0>();
+        }
         slot = nslot;
     }
-    // drain: nothing left to issue; the loads still in flight are at most NS-1 stages
+    // drain: nothing left to issue; the loads still in flight are at most NS-1 slots
     for (; s < steps; ++s) {
         const int nslot = slot + 1 == NS ? 0 : slot + 1;
-        load_frags(1, slot, 1);
-        mfmas(0);
-        sched_substep<NM, 0, NF, 0>();
-        const int ahead = steps - 2 - s;                           // stages issued beyond s+1
+        head(slot);
+        const int ahead = steps - 2 - s;                           // iterations issued beyond s+1
         bool waited = false;
         if constexpr (NS > 3) {
-            if (ahead >= NS - 3) { METIS_WAIT((NS - 3) * LPW, 0); waited = true; }
+            if (ahead >= NS - 3) { METIS_WAIT((NS - 3) * LPS, 0); waited = true; }
         }
         if constexpr (NS > 4) {
-            if (!waited && ahead == NS - 4) { METIS_WAIT((NS - 4) * LPW, 0); waited = true; }
+            if (!waited && ahead == NS - 4) { METIS_WAIT((NS - 4) * LPS, 0); waited = true; }
         }
         if (!waited) METIS_WAIT(0, 0);
         __syncthreads();
-        if (s + 1 < steps) load_frags(0, nslot, 0);
+        if (s + 1 < steps) load_frags(nslot, 0);
         mfmas(1);
         sched_substep<NM, 0, NF, 0>();
         slot = nslot;
@@ -330,13 +352,13 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_xt_kernel(
     }
 }
 
-template <int OUT_F32, int WN_WAVES, int NS>
+template <int OUT_F32, int WN_WAVES, int NS, int KS = 1, int ILV = 0>
 static int launch_xt(const void* a_xt, const float* a_unit, const void* b_xt, const float* b_unit, int64_t M, int64_t N, int64_t K,
                      const void* t, const void* u, int64_t r, const void* bias, int bias_f32, void* out, hipStream_t st)
 {
     static bool attr_set[64] = {};
-    const void* fn = (const void*)gemm_xt_kernel<OUT_F32, WN_WAVES, NS>;
-    const size_t lds_bytes = (size_t)NS * XT_STAGE;
+    const void* fn = (const void*)gemm_xt_kernel<OUT_F32, WN_WAVES, NS, KS, ILV>;
+    const size_t lds_bytes = (size_t)NS * KS * XT_STAGE;
     if (const int rc = allow_dynamic_lds(fn, lds_bytes, attr_set)) return rc;
     const int tiles_m = (int)((M + L_BM - 1) / L_BM), tiles_n = (int)((N + L_BN - 1) / L_BN);
     const int total = tiles_m * tiles_n;
@@ -370,13 +392,24 @@ int gemm_xt(const void* a_xt, const float* a_unit, const void* b_xt, const float
 #define METIS_XT(W, S) (f32 ? launch_xt<1, W, S>(a_xt, a_unit, b_xt, b_unit, M, N, K, t, u, r, bias, bias_f32, out, st) \
                             : launch_xt<0, W, S>(a_xt, a_unit, b_xt, b_unit, M, N, K, t, u, r, bias, bias_f32, out, st))
 #ifdef METIS_MEASURE
+#define METIS_XTK(W, S, KS_, I) (f32 ? launch_xt<1, W, S, KS_, I>(a_xt, a_unit, b_xt, b_unit, M, N, K, t, u, r, bias, bias_f32, out, st) \
+                                     : launch_xt<0, W, S, KS_, I>(a_xt, a_unit, b_xt, b_unit, M, N, K, t, u, r, bias, bias_f32, out, st))
+    if (variant == 5 && K % 64 == 0) return METIS_XTK(4, 2, 2, 0);
+    if (variant == 6 && K % 64 == 0) return METIS_XTK(4, 2, 2, 1);
+    if (variant == 7) return METIS_XTK(4, 3, 1, 1);
+    if (variant == 8 && K % 64 == 0) return METIS_XTK(2, 2, 2, 0);
+#undef METIS_XTK
     if (variant == 1) return METIS_XT(4, 5);
     if (variant == 2) return METIS_XT(2, 4);
     if (variant == 3) return METIS_XT(2, 5);
     if (variant == 4) return METIS_XT(4, 3);
 #endif
     (void)variant;
-    return METIS_XT(4, 4);
+    // measured at 8192 x 14336 x 4096: ring depths 3, 4 and 5 are within 1 % of each other (latency is covered), so the
+    // smallest ring is used; spreading the direct loads between the MFMAs gains 1-2 %; two stages per barrier and
+    // four waves of 128 x 128 are slower (3 % and 17 %)
+    return f32 ? launch_xt<1, 4, 3, 1, 1>(a_xt, a_unit, b_xt, b_unit, M, N, K, t, u, r, bias, bias_f32, out, st)
+               : launch_xt<0, 4, 3, 1, 1>(a_xt, a_unit, b_xt, b_unit, M, N, K, t, u, r, bias, bias_f32, out, st);
 #undef METIS_XT
 }
 

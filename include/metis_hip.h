@@ -229,7 +229,7 @@ int metis_linear_fwd_expanded(const void *a_exp, const float *a_unit, const void
  * (rb, kb) at byte ((rb * cols/32) + kb) * 1024, rows padded to a multiple of 16 with zeros), the 16-byte chunks of
  * a tile permuted so that one direct-to-LDS load per tile leaves it free of bank conflicts for the MFMA fragment
  * reads.  metis_linear_fwd_tiled then runs a main loop of MFMA and LDS reads only, its operand tiles arriving
- * through a four-stage ring of direct loads; results equal metis_linear_fwd on the packed operands bit for bit
+ * through a ring of direct-to-LDS loads; results equal metis_linear_fwd on the packed operands bit for bit
  * (same exact products, same order of binary32 accumulation).  Derived data like the expansion above: callers
  * cache a weight's tiled expansion next to its packed form and re-expand an activation per call (2 B/element).
  *   metis_nvfp4_expand_tiled_bytes  size of `out` for a [rows, cols] packed tensor
