@@ -40,8 +40,28 @@ def _flat2d(x: torch.Tensor) -> torch.Tensor:
 
 
 def _packable(x: torch.Tensor, q) -> bool:
-    """Fast path available: kernel-backed quantizer, device tensor, shapes the GEMM accepts."""
-    return is_hip_nvfp4(q) and x.is_cuda and x.shape[-1] % 32 == 0 and x.dtype in (torch.float32, torch.bfloat16)
+    """Fast path available: kernel-backed quantizer, device tensor, shapes the GEMM accepts (the contraction a
+    multiple of 32).  A device tensor that misses it only by its shape or dtype is reported once."""
+    if not (is_hip_nvfp4(q) and x.is_cuda):
+        return False
+    ok = x.shape[-1] % 32 == 0 and x.dtype in (torch.float32, torch.bfloat16)
+    if not ok:
+        _warn_generic_path(f"a tensor of shape {tuple(x.shape)}, dtype {x.dtype}")
+    return ok
+
+
+_generic_path_warned: set = set()
+
+
+def _warn_generic_path(what: str) -> None:
+    """Said once per distinct situation: an NVFP4 call on a device tensor left the packed kernels for the generic
+    path (dequantized tensors and torch matmuls: same formula as the reference, several times slower, and in backward
+    quantized along the last dimension instead of the contraction)."""
+    if what not in _generic_path_warned:
+        _generic_path_warned.add(what)
+        import warnings
+        warnings.warn(f"metis_hip: {what} does not fit the packed NVFP4 kernels; using the generic path", RuntimeWarning,
+                      stacklevel=3)
 
 
 def _token_sum(flat: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
@@ -305,6 +325,21 @@ class LinearLowbitFunction(torch.autograd.Function):
         cd = F.compute_dtype
         qg, qi = F.q_backward_outputgrad, F.q_backward_input
         me_dy = F._token_mean(dy2) if F.enable_backward_svd else None
+        # The weight gradient contracts over tokens in steps of 32.  A ragged token count is padded, not sent down
+        # another code path: rows equal to the centre (zero rows in direct mode) have a zero residual, so they change
+        # no block maximum, no tensor unit and no sum; the padded rows of grad_input are dropped at the end.
+        L = dy2.shape[0]
+        pad = (-L) % 32
+        if pad:
+            def padded(v, centre):
+                if centre is None:
+                    return torch.cat((v, v.new_zeros(pad, v.shape[1])), dim=0)
+                if v.dtype != centre.dtype:
+                    v = v.to(centre.dtype)                     # the padding rows must equal the centre exactly
+                return torch.cat((v, centre.reshape(1, -1).expand(pad, -1)), dim=0)
+            dy2, x2 = padded(dy2, me_dy), padded(x2, center_x)
+            if gx_lowrank is not None:
+                gx_lowrank = (padded(gx_lowrank[0], None), gx_lowrank[1])
         p_dy = qg.pack(dy2, arith=cd, center=me_dy)
         if me_dy is None and gx_lowrank is None:
             gx = ops.linear_dgrad(p_dy, pw_col, out_dtype=gx_dtype)
@@ -312,6 +347,8 @@ class LinearLowbitFunction(torch.autograd.Function):
             lt, lu = gx_lowrank if gx_lowrank is not None else (None, None)
             gx = ops.linear_fwd(p_dy, pw_col, t=lt, u=lu, bias=None if me_dy is None else ops.matvec(pw_col, me_dy),
                                 out_dtype=gx_dtype)
+        if pad:
+            gx = gx[:L]
         p_dyt = qg.pack(dy2, col=True, arith=cd, center=me_dy)
         p_xt = qi.pack(x2, col=True, arith=cd, center=center_x)
         if me_dy is None and center_x is None:
@@ -322,20 +359,26 @@ class LinearLowbitFunction(torch.autograd.Function):
         if center_x is not None:
             first = (ops.matvec(p_dyt), center_x)
         if me_dy is not None:
-            tail = ops.matvec(p_xt) if center_x is None else ops.matvec(p_xt, z=center_x, beta=float(dy2.shape[0]))
+            tail = ops.matvec(p_xt) if center_x is None else ops.matvec(p_xt, z=center_x, beta=float(L))
             second = (me_dy, tail)
         t, u = ops.rank_one_operands(p_dyt.rows, p_xt.rows, first or second, second if first else None)
         return gx, ops.linear_fwd(p_dyt, p_xt, t=t, u=u, out_dtype=gw_dtype)
 
     @staticmethod
     def _packed_backward_applies(L: int, N: int, grad_output: torch.Tensor) -> bool:
+        """Backward on the packed kernels.  Any token count L qualifies (ragged counts are padded inside
+        _packed_grads); the output width N is the contraction of the input gradient and has to be a multiple of 32.
+        A device NVFP4 configuration that does not qualify takes the generic path and says so once."""
         F = LinearLowbitFunction
-        if not (L % 32 == 0 and N % 32 == 0 and is_hip_nvfp4(F.q_backward_outputgrad) and is_hip_nvfp4(F.q_backward_input)
-                and grad_output.dtype in (torch.float32, torch.bfloat16)):
+        if not (is_hip_nvfp4(F.q_backward_outputgrad) and is_hip_nvfp4(F.q_backward_input)):
             return False
-        if not F.enable_backward_svd:
-            return True
-        return F.backward_lowrank_svd > 0 and F._mean_mode_packable()
+        ok = N % 32 == 0 and L > 0 and grad_output.dtype in (torch.float32, torch.bfloat16)
+        if ok and F.enable_backward_svd:
+            ok = F.backward_lowrank_svd > 0 and F._mean_mode_packable()
+        if not ok and grad_output.is_cuda:
+            _warn_generic_path(f"backward with {L} tokens, {N} output features, dtype {grad_output.dtype}, "
+                               f"metis_mode={F.metis_mode!r}, nv_recipe={F.enable_nv_recipe}")
+        return ok
 
     @staticmethod
     def _quantize_wgrad_operand(value: torch.Tensor, quantizer) -> torch.Tensor:
