@@ -361,6 +361,46 @@ def main():
             if isinstance(qat, dict):
                 qat["mean_mode"] = {"error": f"{type(exc).__name__}: {exc}"[:300]}
 
+    # config 4 as named: gate, up and down projections of the 1.5B-class MLP, each a rank-32 BitLinear, forward + backward
+    if not args.no_decode and isinstance(qat, dict):
+        try:
+            from metis_hip import BitLinear
+            a4 = MetisArgs.direct_fp4(forward_svd_rank=32)
+            g4 = torch.Generator().manual_seed(1004)
+            projs = []
+            for (k_, n_) in ((1536, 8960), (1536, 8960), (8960, 1536)):
+                bl = BitLinear(k_, n_, args=a4, bias=False, dtype=torch.bfloat16, compute_dtype=torch.bfloat16).to(dev)
+                with torch.no_grad():
+                    bl.warmup_linear.weight.copy_((torch.randn(n_, k_, generator=g4) * 0.02).bfloat16())
+                bl.split()
+                projs.append(bl)
+            x_h = torch.randn(1, 4096, 1536, generator=g4).bfloat16().to(dev).requires_grad_(True)
+            x_i = torch.randn(1, 4096, 8960, generator=g4).bfloat16().to(dev).requires_grad_(True)
+            dy_i = (torch.randn(1, 4096, 8960, generator=g4) * 1e-3).bfloat16().to(dev)
+            dy_h = (torch.randn(1, 4096, 1536, generator=g4) * 1e-3).bfloat16().to(dev)
+
+            def mlp_step(ev):
+                if ev is not None:
+                    ev[0].record()
+                for bl, xx, dd in ((projs[0], x_h, dy_i), (projs[1], x_h, dy_i), (projs[2], x_i, dy_h)):
+                    bl(xx).backward(dd)
+                if ev is not None:
+                    ev[1].record()
+                for bl in projs:
+                    for p_ in bl.parameters():
+                        p_.grad = None
+                x_h.grad = None
+                x_i.grad = None
+            _, mlp_ms = time_region(torch, mlp_step, 10, 3)
+            qat["three_projections"] = {"workload": "gate, up, down as BitLinear r=32 (bf16 arithmetic, direct NVFP4 mode), L=4096: forward + "
+                                                    "dgrad + wgrad + rank-r gradients of each, through the modules",
+                                        "us_per_step": round(mlp_ms * 1e3, 1),
+                                        "tflops": round(3 * 3 * 2.0 * 4096 * 1536 * 8960 / (mlp_ms * 1e-3) / 1e12, 1)}
+            LinearLowbitFunction.compute_dtype = torch.float32
+            del projs
+        except Exception as exc:
+            qat["three_projections"] = {"error": f"{type(exc).__name__}: {exc}"[:300]}
+
     # ------------------------------------------------------------------ a tile-starved shape: 1024-token prefill
     # through the Qwen2.5-7B down projection (56 output tiles on 256 CUs; K split through a workspace)
     prefill = None
@@ -385,6 +425,67 @@ def main():
                        "tflops": round(2.0 * 1024 * 3584 * (18944 + 64) / (pf_ms * 1e-3) / 1e12, 1)}
         except Exception as exc:  # an optional leg must not cost the headline line
             prefill = {"workload": "short prefill projection", "error": f"{type(exc).__name__}: {exc}"[:300]}
+
+    # ------------------------------------------------------------------ config 5 through the modules: one
+    # Qwen2.5-7B-shaped decoder layer, every projection a rank-64 BitLinear, fused RMSNorm->quant in front of
+    # q/k/v and gate/up; prefill of 8 x 2048 tokens, then a decode step of 64 sequences against a 2048-token KV cache
+    layer_leg = None
+    if not args.no_decode:
+        try:
+            from transformers.models.qwen2.modeling_qwen2 import Qwen2Config, Qwen2DecoderLayer, Qwen2RotaryEmbedding
+            from metis_hip import MetisArgs, replace_model_with_metis
+            cfg = Qwen2Config(hidden_size=3584, intermediate_size=18944, num_attention_heads=28, num_key_value_heads=4,
+                              head_dim=128, num_hidden_layers=1, vocab_size=128, max_position_embeddings=4096)
+            cfg._attn_implementation = "sdpa"
+            lyr = Qwen2DecoderLayer(cfg, layer_idx=0).to(torch.bfloat16)
+            gl = torch.Generator().manual_seed(1005)
+            with torch.no_grad():
+                for name_, p_ in lyr.named_parameters():
+                    if p_.dim() == 2 or name_.endswith("bias"):
+                        p_.copy_((torch.randn(p_.shape, generator=gl) * 0.02).to(p_.dtype))
+            holder = torch.nn.ModuleDict({"layer": lyr.to(dev)})
+            replace_model_with_metis(holder, MetisArgs.direct_fp4(forward_svd_rank=64), fuse_norms=True)
+            rope = Qwen2RotaryEmbedding(cfg).to(dev)
+            xp_ = torch.randn(8, 2048, 3584, generator=gl).bfloat16().to(dev)
+            pos_p = torch.arange(2048, device=dev).unsqueeze(0).expand(8, -1)
+            pe_p = rope(xp_, pos_p)
+            xd_ = torch.randn(64, 1, 3584, generator=gl).bfloat16().to(dev)
+            pos_d = torch.full((64, 1), 2048, dtype=torch.long, device=dev)
+            pe_d = rope(xd_, pos_d)
+
+            def prefill_layer(ev):
+                if ev is not None:
+                    ev[0].record()
+                with torch.no_grad():
+                    holder["layer"](xp_, position_embeddings=pe_p, attention_mask=None, position_ids=pos_p)
+                if ev is not None:
+                    ev[1].record()
+            _, pl_ms = time_region(torch, prefill_layer, 10, 3)
+            lin_flops = 2.0 * 16384 * 233.05e6                       # 233.05 M linear parameters per layer
+            # the projections and norms alone (what this library provides): the layer minus attention
+            def decode_layer(ev=None):
+                if ev is not None:
+                    ev[0].record()
+                with torch.no_grad():
+                    holder["layer"](xd_, position_embeddings=pe_d, attention_mask=None, position_ids=pos_d)
+                if ev is not None:
+                    ev[1].record()
+            _, dl_ms = time_region(torch, decode_layer, 50, 10)
+            try:
+                dl_graph_us = replay_us(decode_layer)
+            except Exception as exc_:
+                dl_graph_us = None
+            dec_bytes = 233.05e6 * (0.5 + 1.0 / 16)
+            layer_leg = {"workload": "config 5: Qwen2.5-7B-shaped decoder layer through the patched modules (BitLinear r=64, fused "
+                                     "RMSNorm->NVFP4, bf16 arithmetic), no autograd: prefill 8x2048 tokens, then a 64x1 decode step "
+                                     "(attention by torch SDPA, causal, no KV history in the decode step)",
+                         "prefill_ms": round(pl_ms, 3), "prefill_linear_tflops": round(lin_flops / (pl_ms * 1e-3) / 1e12, 1),
+                         "decode_us_eager": round(dl_ms * 1e3, 1),
+                         "decode_us_graph_replay": None if dl_graph_us is None else round(dl_graph_us, 1),
+                         "decode_packed_weight_GBps": None if dl_graph_us is None else round(dec_bytes / dl_graph_us / 1e3, 1)}
+            del holder, lyr
+        except Exception as exc:  # an optional leg must not cost the headline line
+            layer_leg = {"workload": "config 5 decoder layer", "error": f"{type(exc).__name__}: {exc}"[:300]}
 
     line = {
         "metric": "Metis NVFP4 linear TFLOP/s at 8192x4096x14336 (rank 64)",
@@ -420,6 +521,8 @@ def main():
     }
     if dec is not None:
         line["decode_layer"] = dec
+    if layer_leg is not None:
+        line["decoder_layer_modules"] = layer_leg
     if qat is not None:
         line["qat_projection"] = qat
     if prefill is not None:
