@@ -34,6 +34,35 @@ namespace metis {
 // 330-333).  binary32 [cols] in binary32 arithmetic (always WIDE then), bf16 [cols] in bf16 arithmetic.
 __device__ __forceinline__ float block_scalar_ieee(float amax) { return amax / 6.0f + 1e-9f; }
 
+// Round-to-nearest rows of a contiguous bf16 tensor, the shape every activation and weight has: a kernel of its own
+// so that its loop carries no row/column arithmetic at all.  Software-pipelined: the next block's 32 bytes are in
+// flight while the current block is encoded.
+template <int MODE>
+__global__ __launch_bounds__(256) void quant_codes_contig_kernel(const uint4* __restrict__ x, uint2* __restrict__ codes,
+                                                                 uint16_t* __restrict__ ws_amax, uint32_t* __restrict__ ws_gmax,
+                                                                 uint32_t nblocks)
+{
+    float gmax = 0.0f;
+    const uint32_t step = gridDim.x * 256u;
+    uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    uint4 c0 = make_uint4(0u, 0u, 0u, 0u), c1 = c0;
+    if (i < nblocks) { c0 = x[2 * (size_t)i]; c1 = x[2 * (size_t)i + 1]; }
+    while (i < nblocks) {
+        const uint32_t nxt = i + step;
+        uint4 n0 = c0, n1 = c1;
+        if (nxt < nblocks) { n0 = x[2 * (size_t)nxt]; n1 = x[2 * (size_t)nxt + 1]; }
+        float v[kBlock];
+        const float none[kBlock] = {};
+        unpack16(c0, c1, v);
+        const float am = block_amax(v);
+        gmax = fmaxf(gmax, am);
+        ws_amax[i] = (uint16_t)(__float_as_uint(am) >> 16);
+        codes[i] = encode_block<MODE, false>(v, block_scalar<MODE>(am), none);
+        c0 = n0; c1 = n1; i = nxt;
+    }
+    publish_group_max(gmax, ws_gmax);
+}
+
 template <int MODE, bool SR, bool WIDE = false>
 __global__ __launch_bounds__(256) void quant_codes_kernel(
     const void* __restrict__ xv, uint32_t rows, uint32_t cols, int64_t ld, const void* __restrict__ noise,
@@ -45,37 +74,6 @@ __global__ __launch_bounds__(256) void quant_codes_kernel(
     uint16_t* __restrict__ ws_amax = static_cast<uint16_t*>(ws_amax_v);
     float gmax = 0.0f;
     const uint32_t nbpr = cols / kBlock;      // row layout: blocks per row
-    if constexpr (!SR && !WIDE) {
-      if (!center) {
-        // Round-to-nearest rows: software-pipelined, the next block's 32 bytes are in flight while the
-        // current block is encoded.
-        const uint32_t step = gridDim.x * 256u;
-        uint32_t i = blockIdx.x * 256u + threadIdx.x;
-        uint4 c0 = make_uint4(0u, 0u, 0u, 0u), c1 = c0;
-        const bool contiguous = ld == (int64_t)cols;            // uniform: no per-block integer division then
-        auto src = [&](uint32_t blk) {
-            if (contiguous) return reinterpret_cast<const uint4*>(x) + 2 * (size_t)blk;
-            const uint32_t row = blk / nbpr, cb = blk - row * nbpr;
-            return reinterpret_cast<const uint4*>(x + (int64_t)row * ld + (int64_t)cb * kBlock);
-        };
-        if (i < nblocks) { const uint4* p = src(i); c0 = p[0]; c1 = p[1]; }
-        while (i < nblocks) {
-            const uint32_t nxt = i + step;
-            uint4 n0 = c0, n1 = c1;
-            if (nxt < nblocks) { const uint4* p = src(nxt); n0 = p[0]; n1 = p[1]; }
-            float v[kBlock];
-            const float none[kBlock] = {};
-            unpack16(c0, c1, v);
-            const float am = block_amax(v);
-            gmax = fmaxf(gmax, am);
-            ws_amax[i] = (uint16_t)(__float_as_uint(am) >> 16);
-            codes[i] = encode_block<MODE, false>(v, block_scalar<MODE>(am), none);
-            c0 = n0; c1 = n1; i = nxt;
-        }
-        publish_group_max(gmax, ws_gmax);
-        return;
-      }
-    }
     for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < nblocks; i += gridDim.x * 256u) {
         float v[kBlock], u[kBlock] = {};
         const uint32_t row = i / nbpr, cb = i - row * nbpr;
@@ -572,6 +570,13 @@ static int launch_quant(const void* x, int64_t rows, int64_t cols, int64_t ld, c
         return launch_scales(WIDE ? METIS_MODE_P32_F32 : MODE, ws, (uint32_t)g, scales, unit, nblocks, st);
     } else {
         const int g1 = grid_for(nblocks);
+        if constexpr (!SR && !WIDE) {
+            if (!center && ld == cols) {
+                hipLaunchKernelGGL((quant_codes_contig_kernel<MODE>), dim3(g1), dim3(256), 0, st, (const uint4*)x, (uint2*)codes,
+                                   ws.amax, ws.gmax, nblocks);
+                return launch_scales(MODE, ws, (uint32_t)g1, scales, unit, nblocks, st);
+            }
+        }
         hipLaunchKernelGGL((quant_codes_kernel<MODE, SR, WIDE>), dim3(g1), dim3(256), 0, st, x, (uint32_t)rows,
                            (uint32_t)cols, ld, noise, seed, offset, (uint2*)codes, (void*)ws.amax, ws.gmax, nblocks, in_f32, center);
         return launch_scales(WIDE ? METIS_MODE_P32_F32 : MODE, ws, (uint32_t)g1, scales, unit, nblocks, st);
