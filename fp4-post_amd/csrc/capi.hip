@@ -138,26 +138,21 @@ int metis_linear_fwd_expanded(const void* a_exp, const float* a_unit, const void
 
 size_t metis_nvfp4_expand_tiled_bytes(int64_t rows, int64_t cols) { return expand_xt_bytes(rows, cols); }
 
-int metis_nvfp4_expand_tiled(const void* codes, const void* scales, int64_t rows, int64_t cols, void* out, void* stream)
+int metis_nvfp4_expand_tiled(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, int mode,
+                             void* out, void* stream)
 {
-    return expand_xt(codes, scales, rows, cols, out, (hipStream_t)stream);
+    return expand_xt(codes, scales, unit, rows, cols, mode, out, (hipStream_t)stream);
 }
+
+size_t metis_linear_tiled_workspace_bytes(int64_t M, int64_t N, int64_t K, int mode) { return gemm_xt_workspace_bytes(M, N, K, mode); }
 
 int metis_linear_fwd_tiled(const void* a_xt, const float* a_unit, const void* b_xt, const float* b_unit, int64_t M, int64_t N,
                            int64_t K, const void* t, const void* u, int64_t r, const void* bias, int bias_is_f32, void* out,
-                           int out_dtype, void* stream)
+                           int out_dtype, int mode, void* workspace, size_t workspace_bytes, void* stream)
 {
-    return gemm_xt(a_xt, a_unit, b_xt, b_unit, M, N, K, t, u, r, bias, bias_is_f32 != 0, out, out_dtype, (hipStream_t)stream);
+    return gemm_xt(a_xt, a_unit, b_xt, b_unit, M, N, K, t, u, r, bias, bias_is_f32 != 0, out, out_dtype, mode, workspace,
+                   workspace_bytes, (hipStream_t)stream);
 }
-
-#ifdef METIS_MEASURE
-int metis_measure_linear_fwd_tiled(const void* a_xt, const float* a_unit, const void* b_xt, const float* b_unit, int64_t M, int64_t N,
-                                   int64_t K, const void* t, const void* u, int64_t r, const void* bias, int bias_is_f32, void* out,
-                                   int out_dtype, void* stream, int variant)
-{
-    return gemm_xt(a_xt, a_unit, b_xt, b_unit, M, N, K, t, u, r, bias, bias_is_f32 != 0, out, out_dtype, (hipStream_t)stream, variant);
-}
-#endif
 
 int metis_linear_dgrad(const void* dy_codes, const void* dy_scales, const float* dy_unit, const void* wt_codes,
                        const void* wt_scales, const float* wt_unit, int64_t L, int64_t N, int64_t K, void* grad_input,

@@ -79,4 +79,132 @@ inline int allow_dynamic_lds(const void* fn, size_t bytes, bool (&done)[64])
     return METIS_OK;
 }
 
+// Sums the nsplit partial tiles of a split 256 x 256 GEMM (8 waves of 128 x 64) and writes the output.
+// One wave per 32 x 64 piece (tile, wave of the GEMM, 32-row slab i): its lanes read what the same lanes of
+// the GEMM wrote, 1 KiB per instruction, and add the splits in ascending order.
+// PB16 (every op of the reference rounded to bf16): the partial tiles hold the residual product only; their sum is
+// rounded to bf16 as the reference's bf16 matmul rounds it, the bias is added in bf16, and the low-rank term (a
+// further partial tile in slot nsplit when has_low is set) is added before the final rounding.
+template <int OUT_F32, int PB16 = 0>
+__global__ __launch_bounds__(64) void gemm_splitk_reduce_kernel(const float* __restrict__ ws, int nsplit, int M, int N,
+                                                                int tiles_m, int tiles_n, void* __restrict__ out, int nfull,
+                                                                const uint16_t* __restrict__ bias, int bias_f32, int has_low)
+{
+    constexpr int TN = 2, WTN = 64, NTHREADS = 512, TILE = L_BM * L_BN;
+    __shared__ __attribute__((aligned(16))) uint16_t cw[32 * 72];
+    const int total = tiles_m * tiles_n - nfull;                 // split tiles
+    const int tile = blockIdx.x >> 5, wave = (blockIdx.x >> 2) & 7, i = blockIdx.x & 3;
+    const int lane = threadIdx.x, tid = wave * 64 + lane;
+    const int wm = wave / 4, wn = wave % 4;
+    int m0, n0;
+    tile_origin(nfull + tile, tiles_m, tiles_n, m0, n0);
+    const int mbase = m0 + wm * 128 + i * 32, nbase = n0 + wn * WTN;
+    if (mbase >= M || nbase >= N) return;
+
+    float4 v[TN][4];
+    const float* src = ws + (size_t)tile * TILE + (size_t)(i * TN * 4) * (NTHREADS * 4) + tid * 4;
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) v[j][g] = *reinterpret_cast<const float4*>(src + (j * 4 + g) * (NTHREADS * 4));
+    for (int z = 1; z < nsplit; ++z) {
+        const float* sz = src + (size_t)z * total * TILE;
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const float4 p = *reinterpret_cast<const float4*>(sz + (j * 4 + g) * (NTHREADS * 4));
+                v[j][g].x += p.x; v[j][g].y += p.y; v[j][g].z += p.z; v[j][g].w += p.w;
+            }
+    }
+    if constexpr (PB16 != 0) {
+        const float* sl = src + (size_t)nsplit * total * TILE;
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int n = nbase + j * 32 + 8 * g + 4 * (lane >> 5);
+                float r[4] = {rb(v[j][g].x), rb(v[j][g].y), rb(v[j][g].z), rb(v[j][g].w)};
+                if (bias) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) r[e] = rb(r[e] + bias_value(bias, bias_f32, min(n + e, N - 1)));
+                }
+                if (has_low) {
+                    const float4 p = *reinterpret_cast<const float4*>(sl + (j * 4 + g) * (NTHREADS * 4));
+                    r[0] += p.x; r[1] += p.y; r[2] += p.z; r[3] += p.w;
+                }
+                v[j][g] = make_float4(rb(r[0]), rb(r[1]), rb(r[2]), rb(r[3]));
+            }
+    }
+
+    if (!OUT_F32 && (N & 7) == 0) {
+        // 32 x 64 bf16 through LDS: a store instruction then writes 8 rows x 128 contiguous bytes
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                uint2 w;
+                w.x = bf16_bits(v[j][g].x) | (bf16_bits(v[j][g].y) << 16);
+                w.y = bf16_bits(v[j][g].z) | (bf16_bits(v[j][g].w) << 16);
+                *reinterpret_cast<uint2*>(cw + (lane & 31) * 72 + j * 32 + 8 * g + 4 * (lane >> 5)) = w;
+            }
+        __syncthreads();
+        const int rsub = lane >> 3, chunk = lane & 7;
+        const int n = nbase + chunk * 8;
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            const int ml = it * 8 + rsub;
+            const uint4 w = *reinterpret_cast<const uint4*>(cw + ml * 72 + chunk * 8);
+            if (mbase + ml < M && n < N) *reinterpret_cast<uint4*>((uint16_t*)out + (int64_t)(mbase + ml) * N + n) = w;
+        }
+        return;
+    }
+    const int m = mbase + (lane & 31);
+    if (m >= M) return;
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int n = nbase + j * 32 + 8 * g + 4 * (lane >> 5);
+            if (n >= N) continue;                                  // N % 4 == 0
+            if (OUT_F32) {
+                *reinterpret_cast<float4*>((float*)out + (int64_t)m * N + n) = v[j][g];
+            } else {
+                uint2 w;
+                w.x = bf16_bits(v[j][g].x) | (bf16_bits(v[j][g].y) << 16);
+                w.y = bf16_bits(v[j][g].z) | (bf16_bits(v[j][g].w) << 16);
+                *reinterpret_cast<uint2*>((uint16_t*)out + (int64_t)m * N + n) = w;
+            }
+        }
+}
+
+// Splits of K for a tiled GEMM.  A shape that would leave more than half of the compute units without a tile is
+// split whole: as many workgroups per tile as fill the device once, at least 8 K steps (512 elements) each, at
+// most 16.  A shape whose last round of tiles covers at most half of the units has only those tiles split; the
+// full rounds before it run unsplit (up to four of them: measured gains 6-28 % at 1-4 full rounds, a loss of 2 % at
+// nine, where the rounds have drifted apart enough to hide the tail anyway).  nsplit = 1: do not split.
+struct SplitPlan {
+    int nsplit;
+    int nfull;                   // leading tiles that run unsplit (a multiple of the compute units)
+};
+inline SplitPlan split_plan(int64_t M, int64_t N, int64_t K)
+{
+    const SplitPlan none = {1, 0};
+    if (M < L_BM || N < L_BN || K % BK) return none;
+    const int64_t tiles = ((M + L_BM - 1) / L_BM) * ((N + L_BN - 1) / L_BN);
+    const int cus = device_cus();
+    if (cus <= 0 || cus % 8 || tiles > INT32_MAX) return none;
+    int64_t part = tiles, nfull = 0;                            // tiles to split
+    if (tiles * 2 > cus) {
+        part = tiles % cus;
+        nfull = tiles - part;
+        if (tiles < cus || part == 0 || part * 2 > cus || nfull > 4 * (int64_t)cus || false) return none;
+    }
+    int64_t s = cus / part;
+    if (s > K / BK / 8) s = K / BK / 8;
+    if (s > 16) s = 16;
+    if (s < 2) return none;
+    return SplitPlan{(int)s, (int)nfull};
+}
+
 }  // namespace metis

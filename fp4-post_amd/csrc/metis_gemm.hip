@@ -500,111 +500,6 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_nvfp4_large_kernel(
     }
 }
 
-// Sums the nsplit partial tiles of gemm_nvfp4_large_kernel<.., SPLIT = 1> (8 waves) and writes the output.
-// One wave per 32 x 64 piece (tile, wave of the GEMM, 32-row slab i): its lanes read what the same lanes of
-// the GEMM wrote, 1 KiB per instruction, and add the splits in ascending order.
-template <int OUT_F32>
-__global__ __launch_bounds__(64) void gemm_splitk_reduce_kernel(const float* __restrict__ ws, int nsplit, int M, int N,
-                                                                int tiles_m, int tiles_n, void* __restrict__ out, int nfull)
-{
-    constexpr int TN = 2, WTN = 64, NTHREADS = 512, TILE = L_BM * L_BN;
-    __shared__ __attribute__((aligned(16))) uint16_t cw[32 * 72];
-    const int total = tiles_m * tiles_n - nfull;                 // split tiles
-    const int tile = blockIdx.x >> 5, wave = (blockIdx.x >> 2) & 7, i = blockIdx.x & 3;
-    const int lane = threadIdx.x, tid = wave * 64 + lane;
-    const int wm = wave / 4, wn = wave % 4;
-    int m0, n0;
-    tile_origin(nfull + tile, tiles_m, tiles_n, m0, n0);
-    const int mbase = m0 + wm * 128 + i * 32, nbase = n0 + wn * WTN;
-    if (mbase >= M || nbase >= N) return;
-
-    float4 v[TN][4];
-    const float* src = ws + (size_t)tile * TILE + (size_t)(i * TN * 4) * (NTHREADS * 4) + tid * 4;
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) v[j][g] = *reinterpret_cast<const float4*>(src + (j * 4 + g) * (NTHREADS * 4));
-    for (int z = 1; z < nsplit; ++z) {
-        const float* sz = src + (size_t)z * total * TILE;
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const float4 p = *reinterpret_cast<const float4*>(sz + (j * 4 + g) * (NTHREADS * 4));
-                v[j][g].x += p.x; v[j][g].y += p.y; v[j][g].z += p.z; v[j][g].w += p.w;
-            }
-    }
-
-    if (!OUT_F32 && (N & 7) == 0) {
-        // 32 x 64 bf16 through LDS: a store instruction then writes 8 rows x 128 contiguous bytes
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                uint2 w;
-                w.x = bf16_bits(v[j][g].x) | (bf16_bits(v[j][g].y) << 16);
-                w.y = bf16_bits(v[j][g].z) | (bf16_bits(v[j][g].w) << 16);
-                *reinterpret_cast<uint2*>(cw + (lane & 31) * 72 + j * 32 + 8 * g + 4 * (lane >> 5)) = w;
-            }
-        __syncthreads();
-        const int rsub = lane >> 3, chunk = lane & 7;
-        const int n = nbase + chunk * 8;
-#pragma unroll
-        for (int it = 0; it < 4; ++it) {
-            const int ml = it * 8 + rsub;
-            const uint4 w = *reinterpret_cast<const uint4*>(cw + ml * 72 + chunk * 8);
-            if (mbase + ml < M && n < N) *reinterpret_cast<uint4*>((uint16_t*)out + (int64_t)(mbase + ml) * N + n) = w;
-        }
-        return;
-    }
-    const int m = mbase + (lane & 31);
-    if (m >= M) return;
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const int n = nbase + j * 32 + 8 * g + 4 * (lane >> 5);
-            if (n >= N) continue;                                  // N % 4 == 0
-            if (OUT_F32) {
-                *reinterpret_cast<float4*>((float*)out + (int64_t)m * N + n) = v[j][g];
-            } else {
-                uint2 w;
-                w.x = bf16_bits(v[j][g].x) | (bf16_bits(v[j][g].y) << 16);
-                w.y = bf16_bits(v[j][g].z) | (bf16_bits(v[j][g].w) << 16);
-                *reinterpret_cast<uint2*>((uint16_t*)out + (int64_t)m * N + n) = w;
-            }
-        }
-}
-
-// Splits of K for a tiled GEMM.  A shape that would leave more than half of the compute units without a tile is
-// split whole: as many workgroups per tile as fill the device once, at least 8 K steps (512 elements) each, at
-// most 16.  A shape whose last round of tiles covers at most half of the units has only those tiles split; the
-// full rounds before it run unsplit (up to four of them: measured gains 6-28 % at 1-4 full rounds, a loss of 2 % at
-// nine, where the rounds have drifted apart enough to hide the tail anyway).  nsplit = 1: do not split.
-struct SplitPlan {
-    int nsplit;
-    int nfull;                   // leading tiles that run unsplit (a multiple of the compute units)
-};
-static SplitPlan split_plan(int64_t M, int64_t N, int64_t K)
-{
-    const SplitPlan none = {1, 0};
-    if (M < L_BM || N < L_BN || K % BK) return none;
-    const int64_t tiles = ((M + L_BM - 1) / L_BM) * ((N + L_BN - 1) / L_BN);
-    const int cus = device_cus();
-    if (cus <= 0 || cus % 8 || tiles > INT32_MAX) return none;
-    int64_t part = tiles, nfull = 0;                            // tiles to split
-    if (tiles * 2 > cus) {
-        part = tiles % cus;
-        nfull = tiles - part;
-        if (tiles < cus || part == 0 || part * 2 > cus || nfull > 4 * (int64_t)cus || measure_env("METIS_GEMM_NOTAIL")) return none;
-    }
-    int64_t s = cus / part;
-    if (s > K / BK / 8) s = K / BK / 8;
-    if (s > 16) s = 16;
-    if (s < 2) return none;
-    return SplitPlan{(int)s, (int)nfull};
-}
-
 size_t gemm_grouped_workspace_bytes(int64_t M, int64_t K, const GemmMember* members, int count);
 
 size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K)
@@ -664,9 +559,9 @@ static int launch_large(const void* a_codes, const void* a_scales, const float* 
     if (split) {
         const dim3 rgrid((unsigned)(total - nfull) * 32u);
         if (f32)
-            hipLaunchKernelGGL(gemm_splitk_reduce_kernel<1>, rgrid, dim3(64), 0, st, ws, nsplit, Mi, Ni, tmi, tni, out, nfull);
+            hipLaunchKernelGGL((gemm_splitk_reduce_kernel<1, 0>), rgrid, dim3(64), 0, st, ws, nsplit, Mi, Ni, tmi, tni, out, nfull, (const uint16_t*)nullptr, 0, 0);
         else
-            hipLaunchKernelGGL(gemm_splitk_reduce_kernel<0>, rgrid, dim3(64), 0, st, ws, nsplit, Mi, Ni, tmi, tni, out, nfull);
+            hipLaunchKernelGGL((gemm_splitk_reduce_kernel<0, 0>), rgrid, dim3(64), 0, st, ws, nsplit, Mi, Ni, tmi, tni, out, nfull, (const uint16_t*)nullptr, 0, 0);
         if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
     }
     return METIS_OK;

@@ -27,29 +27,50 @@ namespace metis {
 __host__ __device__ __forceinline__ int xt_swz(int q) { return ((q >> 2) & 1) | ((((q >> 1) ^ (q >> 3)) & 1) << 1); }
 
 // ---------------------------------------------------------------------------------------------
-// packed NVFP4 -> tiled binary16.  One wave per tile: lane l writes slot l (row l / 4).  A wave walks
+// packed NVFP4 -> tiled 16-bit operands.  One wave per tile: lane l writes slot l (row l / 4).  A wave walks
 // eight consecutive k tiles of one tile row, so the 128-byte lines of codes it touches are used whole.
 // HBM-bound: 0.5625 B read, 2 B written per element.
+//   PB16 = 0: binary16, e2m1(code) * e4m3(scale) * 2^-8, exact (the tensor unit is applied by the GEMM)
+//   PB16 = 1: bf16, the reference's dequantized value with every op rounded to bf16
+//             (src/Metis/Metis/quant.py:23-24, 32-35: bf16(bf16(e4m3 * unit) * v / 2)), unit included
 // ---------------------------------------------------------------------------------------------
+template <int PB16>
 __global__ __launch_bounds__(256) void expand_xt_kernel(const uint32_t* __restrict__ codes, const uint8_t* __restrict__ scales,
-                                                        uint4* __restrict__ out, int rows, int K, int row_tiles)
+                                                        const float* __restrict__ unit_p, uint4* __restrict__ out, int rows,
+                                                        int K, int row_tiles)
 {
+    typedef float float2_t __attribute__((ext_vector_type(2)));
     const int lane = threadIdx.x & 63;
     const int kt = K / 32, kgroups = (kt + 7) / 8;
     const int q = lane >> 2, chunk = (lane & 3) ^ xt_swz(q);
     const int64_t nunits = (int64_t)row_tiles * kgroups;
-    for (int64_t unit = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); unit < nunits; unit += (int64_t)gridDim.x * 4) {
-        const int rb = (int)(unit / kgroups), kg = (int)(unit - (int64_t)rb * kgroups);
-        const int row = rb * 16 + q;
+    const float unit = PB16 ? *unit_p : 0.0f;
+    for (int64_t un = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); un < nunits; un += (int64_t)gridDim.x * 4) {
+        const int rb_ = (int)(un / kgroups), kg = (int)(un - (int64_t)rb_ * kgroups);
+        const int row = rb_ * 16 + q;
         const bool live = row < rows;
         const int kend = min(kt, kg * 8 + 8);
         for (int kb = kg * 8; kb < kend; ++kb) {
             uint4 v = make_uint4(0u, 0u, 0u, 0u);
             if (live) {
                 const int k8 = kb * 4 + chunk;                   // index of the 8-element chunk inside the row
-                v = expand8(codes[(int64_t)row * (K / 8) + k8], scale_pair(scales[(int64_t)row * (K / 16) + (k8 >> 1)]));
+                const uint32_t c = codes[(int64_t)row * (K / 8) + k8];
+                const uint32_t sb = scales[(int64_t)row * (K / 16) + (k8 >> 1)];
+                if constexpr (PB16 != 0) {
+                    const float dq = rb(e4m3_value(sb) * unit);
+                    const float2_t p0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c, 1.0f, 0);
+                    const float2_t p1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c, 1.0f, 1);
+                    const float2_t p2 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c, 1.0f, 2);
+                    const float2_t p3 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c, 1.0f, 3);
+                    v.x = rb_pair(p0[0] * dq, p0[1] * dq);
+                    v.y = rb_pair(p1[0] * dq, p1[1] * dq);
+                    v.z = rb_pair(p2[0] * dq, p2[1] * dq);
+                    v.w = rb_pair(p3[0] * dq, p3[1] * dq);
+                } else {
+                    v = expand8(c, scale_pair(sb));
+                }
             }
-            out[((int64_t)rb * kt + kb) * 64 + lane] = v;
+            out[((int64_t)rb_ * kt + kb) * 64 + lane] = v;
         }
     }
 }
@@ -60,35 +81,54 @@ size_t expand_xt_bytes(int64_t rows, int64_t cols)
     return (size_t)((rows + 15) / 16) * 16 * (size_t)cols * 2;
 }
 
-int expand_xt(const void* codes, const void* scales, int64_t rows, int64_t cols, void* out, hipStream_t st)
+int expand_xt(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, int mode, void* out,
+              hipStream_t st)
 {
     if (rows < 0 || cols < 0) return METIS_E_ARG;
+    if (mode == METIS_MODE_P32_F32) mode = METIS_MODE_P32;
+    if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) return METIS_E_ARG;
     if (cols % kBlock) return METIS_E_SHAPE;
     if (cols % 32 || rows > INT32_MAX - 16 || cols > INT32_MAX) return METIS_E_ARG;
     if (rows == 0 || cols == 0) return METIS_OK;
     if (!codes || !scales || !out || ((uintptr_t)codes % 4) || ((uintptr_t)out % 16)) return METIS_E_ARG;
+    if (mode == METIS_MODE_PB16 && !unit) return METIS_E_ARG;
     const int row_tiles = (int)((rows + 15) / 16);
     const int64_t units = (int64_t)row_tiles * ((cols / 32 + 7) / 8);
     int64_t g = (units + 3) / 4;
     const int64_t cap = (int64_t)device_cus() * 16;
     if (g > cap) g = cap;
-    hipLaunchKernelGGL(expand_xt_kernel, dim3((unsigned)g), dim3(256), 0, st, (const uint32_t*)codes, (const uint8_t*)scales,
-                       (uint4*)out, (int)rows, (int)cols, row_tiles);
+    if (mode == METIS_MODE_PB16)
+        hipLaunchKernelGGL(expand_xt_kernel<1>, dim3((unsigned)g), dim3(256), 0, st, (const uint32_t*)codes, (const uint8_t*)scales,
+                           unit, (uint4*)out, (int)rows, (int)cols, row_tiles);
+    else
+        hipLaunchKernelGGL(expand_xt_kernel<0>, dim3((unsigned)g), dim3(256), 0, st, (const uint32_t*)codes, (const uint8_t*)scales,
+                           unit, (uint4*)out, (int)rows, (int)cols, row_tiles);
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 
 // ---------------------------------------------------------------------------------------------
-// The GEMM.  256 x 256 per workgroup; WN_WAVES = 4: eight waves (2 x 4) of 128 x 64, two per SIMD;
-// WN_WAVES = 2: four waves (2 x 2) of 128 x 128, one per SIMD (a third less LDS read traffic).
-// A stage is 32 k of the A|B tile: 32 KiB = 32 operand tiles, one direct load each.  NS slots of KS stages form a
-// ring (shipped: three slots of one stage, 96 KiB).  Iteration s (stage s in slot s % NS):
+// The GEMM.  256 x 256 per workgroup, eight waves (2 x 4) of 128 x 64, two per SIMD.
+// A stage is 32 k of the A|B tile: 32 KiB = 32 operand tiles, one direct load each.  Three slots form a ring
+// (96 KiB).  Iteration s (stage s in slot s % 3):
 //     read fragments (s, k 16..31)            | MFMAs on fragments (s, k 0..15)
 //     wait: own fragment reads done, own loads of stage s+1 landed;  BARRIER
-//     issue loads of stage s+NS into slot s % NS (every wave holds what it needs of stage s in registers)
-//     read fragments (s+1, k 0..15)           | MFMAs on fragments (s, k 16..31)
-// so a stage's loads have NS-1 iterations to arrive and the waits never drain the queue.
+//     read fragments (s+1, k 0..15); loads of stage s+3 into slot s % 3, spread between the MFMAs on fragments
+//     (s, k 16..31): every wave holds what it needs of stage s in registers by then
+// so a stage's loads have two iterations to arrive and the waits never drain the queue.
+// Measured at 8192 x 14336 x 4096 before these choices were fixed: rings of 3, 4 and 5 slots within 1 % of each
+// other (latency is covered); loads spread between the MFMAs 1-2 % faster than issued in one burst; two stages
+// per barrier 3 % slower; four waves of 128 x 128 (a third less LDS read traffic, one wave per SIMD) 17 % slower.
+//
+// PB16: operands are the reference's bf16 dequantized values (bf16 MFMA, no unit factor), and the epilogue
+// rounds where the reference's all-bf16 evaluation rounds: the residual product to bf16 (its bf16 matmul), the
+// bias added in bf16, then the low-rank term and the final rounding (bitlinear.py:435-438 under compute_dtype =
+// bfloat16, src/grpo/grpo.py:204-205).
+// SPLIT: as in gemm_nvfp4_large_kernel -- tiles nfull .. total-1 have nsplit workgroups each, every one contracting
+// its own range of stages into a binary32 partial tile in ws (accumulator-register order) for
+// gemm_splitk_reduce_kernel.  Exact mode: units applied, low-rank term and bias in split 0.  PB16: residual only;
+// split 0 leaves the low-rank term as one more partial tile in slot nsplit, the reduction kernel rounds and adds.
 // ---------------------------------------------------------------------------------------------
-constexpr int XT_STAGE = 32 * 1024;
+constexpr int XT_STAGE = 32 * 1024, XT_NS = 3;
 
 __host__ __device__ constexpr int waitcnt_imm(int vm, int lgkm)
 {
@@ -96,27 +136,47 @@ __host__ __device__ constexpr int waitcnt_imm(int vm, int lgkm)
 }
 #define METIS_WAIT(VM, LGKM) __builtin_amdgcn_s_waitcnt(waitcnt_imm(VM, LGKM))
 
-template <int OUT_F32, int WN_WAVES, int NS, int KS = 1, int ILV = 0>
-__global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_xt_kernel(
+template <int OUT_F32, int PB16, int SPLIT>
+__global__ __launch_bounds__(512, 1) void gemm_xt_kernel(
     const uint8_t* __restrict__ a_xt, const float* __restrict__ a_unit, const uint8_t* __restrict__ b_xt,
     const float* __restrict__ b_unit, int M, int N, int K, const uint16_t* __restrict__ t, const uint16_t* __restrict__ u,
-    int r, const uint16_t* __restrict__ bias, void* __restrict__ out, int tiles_m, int tiles_n, int bias_f32)
+    int r, const uint16_t* __restrict__ bias, void* __restrict__ out, int tiles_m, int tiles_n, int bias_f32,
+    float* __restrict__ ws, int nsplit, int nfull)
 {
     extern __shared__ __attribute__((aligned(1024))) uint8_t xlds[];
-    constexpr int TM = 4, TN = 8 / WN_WAVES, WTN = 256 / WN_WAVES;
-    constexpr int NWAVES = 2 * WN_WAVES, NTHREADS = 64 * NWAVES;
-    constexpr int LPW = 32 / NWAVES;                            // direct loads per wave per stage: 4 or 8
+    constexpr int TM = 4, TN = 2, WTN = 64, NWAVES = 8, NTHREADS = 512, NS = XT_NS;
+    constexpr int LPW = 32 / NWAVES;                            // direct loads per wave per stage
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave / WN_WAVES, wn = wave % WN_WAVES;
+    const int wm = wave / 4, wn = wave % 4;
 
-    // tile assignment: contiguous range per XCD, groups of four tile rows (see tile_origin)
+    // ---- tile assignment: contiguous range per XCD, groups of four tile rows (see tile_origin).  SPLIT: the first
+    //      nfull tiles (a multiple of 8) run unsplit, every XCD its share of them first; the rest have nsplit workgroups each.
     const int total = tiles_m * tiles_n;
-    const int per_xcd = (total + 7) / 8;
-    const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if (logical >= total) return;
+    int logical, split = 0;
+    bool partial = false;
+    if constexpr (SPLIT != 0) {
+        const int xcd = blockIdx.x & 7, li = blockIdx.x >> 3, full_x = nfull >> 3;
+        if (li < full_x) {
+            logical = xcd * full_x + li;
+        } else {
+            const int tail = total - nfull, tail_all = tail * nsplit, per_xcd = (tail_all + 7) / 8;
+            const int j = xcd * per_xcd + (li - full_x);
+            if (li - full_x >= per_xcd || j >= tail_all) return;
+            split = j / tail;                                    // consecutive workgroups of an XCD share a K range
+            logical = nfull + j % tail;
+            partial = true;
+        }
+    } else {
+        const int per_xcd = (total + 7) / 8;
+        logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+        if (logical >= total) return;
+    }
     int m0, n0;
     tile_origin(logical, tiles_m, tiles_n, m0, n0);
+    const int kt = K / 32;
+    const int step_begin = partial ? (int)((int64_t)split * kt / nsplit) : 0;
+    const int steps = (partial ? (int)((int64_t)(split + 1) * kt / nsplit) : kt) - step_begin;   // >= 1: the host never asks for more splits than stages
 
     float16_t acc[TM][TN];
 #pragma unroll
@@ -126,32 +186,24 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_xt_kernel(
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-    // ---- direct loads: instruction j of wave w copies operand tile j * NWAVES + w of the stage (0..15 A, 16..31 B).
+    // ---- direct loads: instruction j of wave w copies operand tile j * 8 + w of the stage (0..15 A, 16..31 B).
     // Written as assembly: the compiler orders every later LDS read behind ALL outstanding direct loads (it cannot
     // tell the ring slots apart), which would drain the queue each iteration; the waits are placed by hand instead.
-    const int kt = K / 32;
     const int a_rt = (M + 15) / 16, b_rt = (N + 15) / 16;
-    const uint8_t* src[LPW];                                    // wave-uniform: first byte of the tile row (k tile 0)
+    const uint8_t* src[LPW];                                    // wave-uniform: the tile row at the first stage of this workgroup
 #pragma unroll
     for (int j = 0; j < LPW; ++j) {
         const int ot = j * NWAVES + wave;
         const bool is_a = ot < 16;
         const int rt = is_a ? min(m0 / 16 + ot, a_rt - 1) : min(n0 / 16 + ot - 16, b_rt - 1);
-        src[j] = (is_a ? a_xt : b_xt) + (int64_t)rt * kt * 1024;
+        src[j] = (is_a ? a_xt : b_xt) + ((int64_t)rt * kt + step_begin) * 1024;
     }
     const uint32_t lane16 = lane * 16;
-    constexpr int SLOT = KS * XT_STAGE;                         // a ring slot holds the KS stages of one iteration
-    constexpr int LPS = LPW * KS;                               // direct loads per wave per slot
-    auto issue_one = [&](int slot, int it, int n) {             // load n (0 .. LPS-1) of iteration `it` into `slot`
-        const int sub = n / LPW, j = n % LPW;
-        const uint8_t* g = src[j] + ((int64_t)it * KS + sub) * 1024;
-        const uint32_t dst = (uint32_t)(slot * SLOT + sub * XT_STAGE + (j * NWAVES + wave) * 1024);   // LDS byte address of the tile
+    auto issue_one = [&](int slot, int it, int j) {
+        const uint8_t* g = src[j] + (int64_t)it * 1024;
+        const uint32_t dst = (uint32_t)(slot * XT_STAGE + (j * NWAVES + wave) * 1024);   // LDS byte address of the tile
         asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                      :: "v"(lane16), "s"(g), "s"(dst) : "memory");
-    };
-    auto issue = [&](int slot, int it) {
-#pragma unroll
-        for (int n = 0; n < LPS; ++n) issue_one(slot, it, n);
     };
 
     // ---- fragment addressing: lane -> row lr of a 32-row MFMA tile, k half hi; chunk = 2 * ks + hi.
@@ -160,81 +212,67 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_xt_kernel(
     const int lane_off = (lr >> 4) * 1024 + (lr & 15) * 64 + ((hi ^ xt_swz(lr & 15)) * 16);
     const int a_off[2] = {wm * 8 * 1024 + lane_off, wm * 8 * 1024 + (lane_off ^ 32)};
     const int b_off[2] = {(16 + wn * (WTN / 16)) * 1024 + lane_off, (16 + wn * (WTN / 16)) * 1024 + (lane_off ^ 32)};
-    half8_t fa[2][TM], fb[2][TN];
-    auto load_frags = [&](int slot, int q) {                    // sub-step q of the slot: stage q / 2, k half q % 2; buffer q % 2
-        const int x = slot * SLOT + (q >> 1) * XT_STAGE;
+    uint4 fa[2][TM], fb[2][TN];                                 // 8 binary16 / bf16 values each
+    auto load_frags = [&](int slot, int ks) {
+        const int x = slot * XT_STAGE;
 #pragma unroll
-        for (int i = 0; i < TM; ++i) fa[q & 1][i] = *reinterpret_cast<const half8_t*>(xlds + (a_off[q & 1] + x) + i * 2048);
+        for (int i = 0; i < TM; ++i) fa[ks][i] = *reinterpret_cast<const uint4*>(xlds + (a_off[ks] + x) + i * 2048);
 #pragma unroll
-        for (int j = 0; j < TN; ++j) fb[q & 1][j] = *reinterpret_cast<const half8_t*>(xlds + (b_off[q & 1] + x) + j * 2048);
+        for (int j = 0; j < TN; ++j) fb[ks][j] = *reinterpret_cast<const uint4*>(xlds + (b_off[ks] + x) + j * 2048);
+    };
+    auto mfma_one = [&](int fbuf, int i, int j) {
+        if constexpr (PB16 != 0)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, fb[fbuf][j]),
+                                                                __builtin_bit_cast(bf16x8_t, fa[fbuf][i]), acc[i][j], 0, 0, 0);
+        else
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, fb[fbuf][j]),
+                                                               __builtin_bit_cast(half8_t, fa[fbuf][i]), acc[i][j], 0, 0, 0);
     };
     auto mfmas = [&](int fbuf) {
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[fbuf][j], fa[fbuf][i], acc[i][j], 0, 0, 0);
+            for (int j = 0; j < TN; ++j) mfma_one(fbuf, i, j);
     };
     constexpr int NM = TM * TN, NF = TM + TN;
-    constexpr int QL = 2 * KS - 1;                              // last sub-step of an iteration
 
-    const int steps = kt / KS;                                  // iterations (the host picks KS = 1 unless KS divides K / 32)
     // prologue: fill the ring
 #pragma unroll
     for (int p = 0; p < NS; ++p)
-        if (p < steps) issue(p, p);
-    if (steps >= NS) METIS_WAIT((NS - 1) * LPS, 15);
+        if (p < steps) {
+#pragma unroll
+            for (int j = 0; j < LPW; ++j) issue_one(p, p, j);
+        }
+    if (steps >= NS) METIS_WAIT((NS - 1) * LPW, 15);
     else METIS_WAIT(0, 15);
     __syncthreads();
     load_frags(0, 0);
 
-    // the sub-steps before the barrier: fragments of sub-step q+1 are read while the MFMAs of sub-step q run
-    auto head = [&](int slot) {
-#pragma unroll
-        for (int q = 0; q < QL; ++q) {
-            load_frags(slot, q + 1);
-            mfmas(q & 1);
-            sched_substep<NM, 0, NF, 0>();
-        }
-    };
     int s = 0, slot = 0;
-    // steady state: the iteration NS ahead exists, so every wait allows NS-2 slots in flight
+    // steady state: the stage NS ahead exists, so every wait allows NS-2 stages in flight
     for (; s + NS < steps; ++s) {
         const int nslot = slot + 1 == NS ? 0 : slot + 1;
-        head(slot);
-        METIS_WAIT((NS - 2) * LPS, 0);                          // own loads of iteration s+1 landed, own fragment reads of s done
+        load_frags(slot, 1);
+        mfmas(0);
+        sched_substep<NM, 0, NF, 0>();
+        METIS_WAIT((NS - 2) * LPW, 0);                          // own loads of stage s+1 landed, own fragment reads of stage s done
         __syncthreads();
-        if constexpr (ILV != 0) {
-            // the direct loads are spread between the MFMAs of the last sub-step instead of issued in one burst
-            load_frags(nslot, 0);
-            constexpr int PER = (NM + LPS - 1) / LPS;
+        load_frags(nslot, 0);
+        constexpr int PER = NM / LPW;                           // one direct load every PER MFMAs
 #pragma unroll
-            for (int m = 0; m < NM; ++m) {
-                if (m % PER == 0 && m / PER < LPS) issue_one(slot, s + NS, m / PER);
-                const int i = m / TN, j = m % TN;
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[1][j], fa[1][i], acc[i][j], 0, 0, 0);
-            }
-        } else {
-            issue(slot, s + NS);
-            load_frags(nslot, 0);
-            mfmas(1);
-            sched_substep<NM, 0, NF, 0>();
+        for (int m = 0; m < NM; ++m) {
+            if (m % PER == 0) issue_one(slot, s + NS, m / PER);
+            mfma_one(1, m / TN, m % TN);
         }
         slot = nslot;
     }
-    // drain: nothing left to issue; the loads still in flight are at most NS-1 slots
+    // drain: nothing left to issue; the loads still in flight are at most NS-1 stages
     for (; s < steps; ++s) {
         const int nslot = slot + 1 == NS ? 0 : slot + 1;
-        head(slot);
-        const int ahead = steps - 2 - s;                           // iterations issued beyond s+1
-        bool waited = false;
-        if constexpr (NS > 3) {
-            if (ahead >= NS - 3) { METIS_WAIT((NS - 3) * LPS, 0); waited = true; }
-        }
-        if constexpr (NS > 4) {
-            if (!waited && ahead == NS - 4) { METIS_WAIT((NS - 4) * LPS, 0); waited = true; }
-        }
-        if (!waited) METIS_WAIT(0, 0);
+        load_frags(slot, 1);
+        mfmas(0);
+        sched_substep<NM, 0, NF, 0>();
+        METIS_WAIT(0, 0);
         __syncthreads();
         if (s + 1 < steps) load_frags(nslot, 0);
         mfmas(1);
@@ -243,20 +281,72 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_xt_kernel(
     }
     __syncthreads();                                            // the ring is free for the epilogue
 
-    // ---- tensor units (and the 2^8 * 2^8 of the scale placement)
-    const float us = (*a_unit) * (*b_unit) * 65536.0f;
+    const bool first = !(SPLIT != 0 && partial && split != 0);  // this workgroup adds the low-rank term (and, exact mode, the bias)
+    float* wt = nullptr;
+    if (SPLIT != 0 && partial) wt = ws + (size_t)(split * (total - nfull) + (logical - nfull)) * (L_BM * L_BN) + tid * 4;
+    auto store_partial = [&](float* dst, bool with_bias) {      // accumulator-register order, 1 KiB per store instruction
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+            for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) acc[i][j][e] *= us;
+                for (int g = 0; g < 4; ++g) {
+                    const int n = n0 + wn * WTN + j * 32 + 8 * g + 4 * hi;
+                    float v[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        v[e] = acc[i][j][4 * g + e];
+                        if (with_bias && bias) v[e] += bias_value(bias, bias_f32, min(n + e, N - 1));
+                    }
+                    *reinterpret_cast<float4*>(dst + ((i * TN + j) * 4 + g) * (NTHREADS * 4)) = make_float4(v[0], v[1], v[2], v[3]);
+                }
+    };
+
+    if constexpr (PB16 != 0) {
+        if (SPLIT != 0 && partial) {
+            store_partial(wt, false);                           // the residual product of this K range
+            if (!first || r == 0) return;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+        } else {
+            // the reference's bf16 matmul result, then its bf16 bias add
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        float v = rb(acc[i][j][e]);
+                        if (bias) v = rb(v + bias_value(bias, bias_f32, min(n0 + wn * WTN + j * 32 + 8 * (e >> 2) + 4 * hi + (e & 3), N - 1)));
+                        acc[i][j][e] = v;
+                    }
+            bias = nullptr;
+        }
+    } else {
+        // tensor units (and the 2^8 * 2^8 of the scale placement)
+        const float us = (*a_unit) * (*b_unit) * 65536.0f;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[i][j][e] *= us;
+        if (!first) {
+            r = 0;
+            bias = nullptr;
+        }
+    }
 
     // ---- bf16 low-rank extension, 32 columns of T / U per step, staged in rows of 144 bytes
     uint16_t* plds = reinterpret_cast<uint16_t*>(xlds);
     const int frag_off = lr * L_STRIDE + hi * 8;
     for (int j0 = 0; j0 < r; j0 += 32) {
-        for (int trow = tid; trow < L_BM + L_BN; trow += NTHREADS) {
+        {
+            const int trow = tid;                               // 512 threads, 512 rows of the T|U tile
             const bool is_a = trow < L_BM;
             const int64_t grow = is_a ? min(m0 + trow, M - 1) : min(n0 + trow - L_BM, N - 1);
             const uint4* sp = reinterpret_cast<const uint4*>((is_a ? t : u) + grow * r + j0);
@@ -281,12 +371,27 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_xt_kernel(
         __syncthreads();
     }
 
+    if (SPLIT != 0 && partial) {
+        // exact mode: this split's share (split 0 with the low-rank term and the bias); PB16: the low-rank tile, slot nsplit
+        if constexpr (PB16 != 0) store_partial(ws + (size_t)(nsplit * (total - nfull) + (logical - nfull)) * (L_BM * L_BN) + tid * 4, false);
+        else store_partial(wt, true);
+        return;
+    }
+    if constexpr (PB16 != 0 && OUT_F32 != 0) {                  // a binary32 output buffer still holds bf16 values in this mode
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[i][j][e] = rb(acc[i][j][e]);
+    }
+
     // ---- epilogue.  acc[i][j][e] of lane l: m = 32 i + l % 32, n = 32 j + 8 (e / 4) + 4 (l / 32) + e % 4 in the wave tile.
     if constexpr (!OUT_F32) {
         if ((N & 7) == 0) {
             // bf16: each wave transposes its tile through its own slice of LDS, 64 rows at a time, so that a store
-            // instruction writes whole 16-byte pieces of rows (WTN * 2 contiguous bytes per row)
-            constexpr int CROW = WTN + 8;                       // halves per staged row: 144 or 272 bytes
+            // instruction writes 8 rows x 128 contiguous bytes
+            constexpr int CROW = WTN + 8;                       // halves per staged row: 144 bytes
             constexpr int LPR = WTN / 8, RPI = 64 / LPR;        // lanes per row, rows per store instruction
             uint16_t* cw = plds + wave * (64 * CROW);
             const int rsub = lane / LPR, chunk = lane % LPR;
@@ -352,64 +457,88 @@ __global__ __launch_bounds__(128 * WN_WAVES, 1) void gemm_xt_kernel(
     }
 }
 
-template <int OUT_F32, int WN_WAVES, int NS, int KS = 1, int ILV = 0>
+// K splits of the pipelined kernel: the plan of the packed kernel (same tiles), with a stage of 32 k as the unit.
+static SplitPlan xt_split_plan(int64_t M, int64_t N, int64_t K)
+{
+    SplitPlan p = split_plan(M, N, K);                          // needs K % 64 == 0, M and N >= 256
+    if (p.nsplit > K / 32) p.nsplit = (int)(K / 32);
+    return p.nsplit < 2 ? SplitPlan{1, 0} : p;
+}
+
+size_t gemm_xt_workspace_bytes(int64_t M, int64_t N, int64_t K, int mode)
+{
+    if (M <= 0 || N <= 0 || K <= 0 || K % 32) return 0;
+    const SplitPlan p = xt_split_plan(M, N, K);
+    if (p.nsplit <= 1) return 0;
+    const int64_t tiles = ((M + L_BM - 1) / L_BM) * ((N + L_BN - 1) / L_BN);
+    const int slots = p.nsplit + (mode == METIS_MODE_PB16 ? 1 : 0);
+    return (size_t)slots * (size_t)(tiles - p.nfull) * L_BM * L_BN * sizeof(float);
+}
+
+template <int OUT_F32, int PB16, int SPLIT>
 static int launch_xt(const void* a_xt, const float* a_unit, const void* b_xt, const float* b_unit, int64_t M, int64_t N, int64_t K,
-                     const void* t, const void* u, int64_t r, const void* bias, int bias_f32, void* out, hipStream_t st)
+                     const void* t, const void* u, int64_t r, const void* bias, int bias_f32, void* out, hipStream_t st, float* ws,
+                     int nsplit, int nfull)
 {
     static bool attr_set[64] = {};
-    const void* fn = (const void*)gemm_xt_kernel<OUT_F32, WN_WAVES, NS, KS, ILV>;
-    const size_t lds_bytes = (size_t)NS * KS * XT_STAGE;
+    const void* fn = (const void*)gemm_xt_kernel<OUT_F32, PB16, SPLIT>;
+    const size_t lds_bytes = (size_t)XT_NS * XT_STAGE;
     if (const int rc = allow_dynamic_lds(fn, lds_bytes, attr_set)) return rc;
     const int tiles_m = (int)((M + L_BM - 1) / L_BM), tiles_n = (int)((N + L_BN - 1) / L_BN);
     const int total = tiles_m * tiles_n;
-    const unsigned grid_x = (unsigned)(((total + 7) / 8) * 8);
+    const unsigned grid_x = SPLIT ? 8u * (unsigned)(nfull / 8 + ((total - nfull) * nsplit + 7) / 8) : (unsigned)(((total + 7) / 8) * 8);
     const uint8_t *ae = (const uint8_t*)a_xt, *be = (const uint8_t*)b_xt;
     const uint16_t *tp = (const uint16_t*)t, *up = (const uint16_t*)u, *bp = (const uint16_t*)bias;
     int Mi = (int)M, Ni = (int)N, Ki = (int)K, ri = (int)r, tmi = tiles_m, tni = tiles_n;
-    void* args[] = {&ae, &a_unit, &be, &b_unit, &Mi, &Ni, &Ki, &tp, &up, &ri, &bp, &out, &tmi, &tni, &bias_f32};
-    if (hipLaunchKernel(fn, dim3(grid_x), dim3(128 * WN_WAVES), args, lds_bytes, st) != hipSuccess) {
+    void* args[] = {&ae, &a_unit, &be, &b_unit, &Mi, &Ni, &Ki, &tp, &up, &ri, &bp, &out, &tmi, &tni, &bias_f32, &ws, &nsplit, &nfull};
+    if (hipLaunchKernel(fn, dim3(grid_x), dim3(512), args, lds_bytes, st) != hipSuccess) {
         (void)hipGetLastError();
         return METIS_E_LAUNCH;
+    }
+    if (SPLIT) {
+        const dim3 rgrid((unsigned)(total - nfull) * 32u);
+        const int has_low = r > 0;
+        hipLaunchKernelGGL((gemm_splitk_reduce_kernel<OUT_F32, PB16>), rgrid, dim3(64), 0, st, (const float*)ws, nsplit, Mi, Ni, tmi, tni, out,
+                           nfull, PB16 ? bp : (const uint16_t*)nullptr, bias_f32, PB16 ? has_low : 0);
+        if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
     }
     return METIS_OK;
 }
 
 int gemm_xt(const void* a_xt, const float* a_unit, const void* b_xt, const float* b_unit, int64_t M, int64_t N, int64_t K,
-            const void* t, const void* u, int64_t r, const void* bias, int bias_f32, void* out, int out_dtype, hipStream_t st,
-            int variant)
+            const void* t, const void* u, int64_t r, const void* bias, int bias_f32, void* out, int out_dtype, int mode,
+            void* workspace, size_t workspace_bytes, hipStream_t st)
 {
     if (M < 0 || N < 0 || K < 0 || r < 0) return METIS_E_ARG;
     if (out_dtype != METIS_DTYPE_BF16 && out_dtype != METIS_DTYPE_F32) return METIS_E_ARG;
+    if (mode == METIS_MODE_P32_F32) mode = METIS_MODE_P32;
+    if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) return METIS_E_ARG;
     if (K % kBlock) return METIS_E_SHAPE;
     if (K % 32 || K == 0 || N % 4 || r % 32 || (r > 0 && (!t || !u))) return METIS_E_ARG;
     if (M > INT32_MAX - 256 || N > INT32_MAX - 256 || K > INT32_MAX) return METIS_E_ARG;
     if (M == 0 || N == 0) return METIS_OK;
-    if (!a_xt || !a_unit || !b_xt || !b_unit || !out) return METIS_E_ARG;
+    if (!a_xt || !b_xt || !out || (mode == METIS_MODE_P32 && (!a_unit || !b_unit))) return METIS_E_ARG;
     if (((uintptr_t)a_xt % 16) || ((uintptr_t)b_xt % 16) || ((uintptr_t)out % 16) || ((uintptr_t)t % 16) || ((uintptr_t)u % 16) ||
         ((uintptr_t)bias % (bias_f32 ? 4 : 2)))
         return METIS_E_ARG;
-    const int f32 = out_dtype == METIS_DTYPE_F32;
-#define METIS_XT(W, S) (f32 ? launch_xt<1, W, S>(a_xt, a_unit, b_xt, b_unit, M, N, K, t, u, r, bias, bias_f32, out, st) \
-                            : launch_xt<0, W, S>(a_xt, a_unit, b_xt, b_unit, M, N, K, t, u, r, bias, bias_f32, out, st))
-#ifdef METIS_MEASURE
-#define METIS_XTK(W, S, KS_, I) (f32 ? launch_xt<1, W, S, KS_, I>(a_xt, a_unit, b_xt, b_unit, M, N, K, t, u, r, bias, bias_f32, out, st) \
-                                     : launch_xt<0, W, S, KS_, I>(a_xt, a_unit, b_xt, b_unit, M, N, K, t, u, r, bias, bias_f32, out, st))
-    if (variant == 5 && K % 64 == 0) return METIS_XTK(4, 2, 2, 0);
-    if (variant == 6 && K % 64 == 0) return METIS_XTK(4, 2, 2, 1);
-    if (variant == 7) return METIS_XTK(4, 3, 1, 1);
-    if (variant == 8 && K % 64 == 0) return METIS_XTK(2, 2, 2, 0);
-#undef METIS_XTK
-    if (variant == 1) return METIS_XT(4, 5);
-    if (variant == 2) return METIS_XT(2, 4);
-    if (variant == 3) return METIS_XT(2, 5);
-    if (variant == 4) return METIS_XT(4, 3);
-#endif
-    (void)variant;
-    // measured at 8192 x 14336 x 4096: ring depths 3, 4 and 5 are within 1 % of each other (latency is covered), so the
-    // smallest ring is used; spreading the direct loads between the MFMAs gains 1-2 %; two stages per barrier and
-    // four waves of 128 x 128 are slower (3 % and 17 %)
-    return f32 ? launch_xt<1, 4, 3, 1, 1>(a_xt, a_unit, b_xt, b_unit, M, N, K, t, u, r, bias, bias_f32, out, st)
-               : launch_xt<0, 4, 3, 1, 1>(a_xt, a_unit, b_xt, b_unit, M, N, K, t, u, r, bias, bias_f32, out, st);
+    SplitPlan plan = {1, 0};
+    if (workspace) {
+        plan = xt_split_plan(M, N, K);
+        if (plan.nsplit > 1 && (((uintptr_t)workspace % 16) || workspace_bytes < gemm_xt_workspace_bytes(M, N, K, mode))) return METIS_E_WORKSPACE;
+    }
+    const int f32 = out_dtype == METIS_DTYPE_F32, pb = mode == METIS_MODE_PB16, sp = plan.nsplit > 1;
+#define METIS_XT(F, P, S) launch_xt<F, P, S>(a_xt, a_unit, b_xt, b_unit, M, N, K, t, u, r, bias, bias_f32, out, st, (float*)workspace, \
+                                            plan.nsplit, plan.nfull)
+    switch (f32 * 4 + pb * 2 + sp) {
+        case 0: return METIS_XT(0, 0, 0);
+        case 1: return METIS_XT(0, 0, 1);
+        case 2: return METIS_XT(0, 1, 0);
+        case 3: return METIS_XT(0, 1, 1);
+        case 4: return METIS_XT(1, 0, 0);
+        case 5: return METIS_XT(1, 0, 1);
+        case 6: return METIS_XT(1, 1, 0);
+        default: return METIS_XT(1, 1, 1);
+    }
 #undef METIS_XT
 }
 

@@ -109,11 +109,13 @@ int gemm_expanded(const void* a_exp, const float* a_unit, const void* b_exp, con
                   int64_t K, const void* t, const void* u, int64_t r, const void* bias, void* out, int out_dtype,
                   hipStream_t st);
 
-// tiled binary16 expansion of a packed tensor and the GEMM that consumes it; metis_gemm_pipe.hip
+// tiled 16-bit expansion of a packed tensor and the pipelined GEMM that consumes it; metis_gemm_pipe.hip
 size_t expand_xt_bytes(int64_t rows, int64_t cols);
-int expand_xt(const void* codes, const void* scales, int64_t rows, int64_t cols, void* out, hipStream_t st);
+int expand_xt(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, int mode, void* out,
+              hipStream_t st);
+size_t gemm_xt_workspace_bytes(int64_t M, int64_t N, int64_t K, int mode);
 int gemm_xt(const void* a_xt, const float* a_unit, const void* b_xt, const float* b_unit, int64_t M, int64_t N, int64_t K,
-            const void* t, const void* u, int64_t r, const void* bias, int bias_f32, void* out, int out_dtype, hipStream_t st,
-            int variant = 0);
+            const void* t, const void* u, int64_t r, const void* bias, int bias_f32, void* out, int out_dtype, int mode,
+            void* workspace, size_t workspace_bytes, hipStream_t st);
 
 }  // namespace metis

@@ -104,6 +104,10 @@ class LinearLowbitFunction(torch.autograd.Function):
     tp_parts = 4
 
     compute_dtype = torch.float32
+    # bf16 arithmetic (compute_dtype = bfloat16): forward GEMMs of 256 rows or more follow the reference's all-bf16
+    # evaluation rounding for rounding (operands bf16(bf16(e4m3 * unit) * v / 2), residual product and bias add rounded
+    # to bf16).  False keeps exact products and one rounding at the end, as every smaller batch does.
+    reference_rounding = True
     metis_mode = "mean"
     mean_cache = None
     mean_cache_key = "default"
@@ -416,7 +420,8 @@ class LinearLowbitFunction(torch.autograd.Function):
                 bias = w_mean if bias is None else w_mean + bias.float()
                 quantized_input = quantized_input.residual
             out_dtype = torch.float32 if F.compute_dtype == torch.float32 else torch.bfloat16
-            out = ops.linear_fwd(quantized_input, quantized_weight, bias=bias, out_dtype=out_dtype)
+            out = ops.linear_fwd(quantized_input, quantized_weight, bias=bias, out_dtype=out_dtype,
+                                 reference_rounding=F.reference_rounding and ctx.center is None)
             return out.reshape(*lead, quantized_weight.rows).to(F.compute_dtype)
         if isinstance(quantized_input, (PackedNVFP4, CenteredNVFP4)):
             quantized_input = quantized_input.dequantize(F.compute_dtype).reshape(input_.shape)
@@ -575,7 +580,8 @@ class _MetisFusedFunction(torch.autograd.Function):
                 y = ops.linear_fwd(px.residual, p_res, t=t, u=u.to(cd), bias=w_mean if bias is None else w_mean + bias.float(),
                                    out_dtype=out_dtype)
         else:
-            y = ops.linear_fwd(px, p_res, t=t, u=u.to(cd), bias=gemm_bias, out_dtype=out_dtype)
+            y = ops.linear_fwd(px, p_res, t=t, u=u.to(cd), bias=gemm_bias, out_dtype=out_dtype,
+                               reference_rounding=F.reference_rounding)
         ctx.save_for_backward(x, v, s, u, res, xv)
         ctx.p_res = p_res
         ctx.has_bias = bias is not None

@@ -32,7 +32,8 @@ class PackedNVFP4:
     cols: int
     mode: int = MODE_P32
     expanded: torch.Tensor | None = None      # cached exact f16 expansion e2m1 * e4m3 * 2^-8, see expand()
-    tiled: torch.Tensor | None = None         # the same expansion in the pipelined GEMM's tiled layout, see expand_tiled()
+    tiled: torch.Tensor | None = None         # exact binary16 expansion in the pipelined GEMM's tiled layout, see expand_tiled()
+    tiled_pb16: torch.Tensor | None = None    # the reference's bf16 dequantized values in the same layout (bf16 arithmetic)
     transposed: "PackedNVFP4 | None" = None   # cached column-blocked packing of the same source tensor (dgrad operand)
     persistent: bool = False                  # lives across calls (a cached weight): worth keeping its tiled expansion
 
@@ -308,27 +309,48 @@ def expand(p: PackedNVFP4) -> torch.Tensor:
     return p.expanded
 
 
-def expand_tiled(p: PackedNVFP4, cache: bool = True) -> torch.Tensor:
-    """Exact binary16 expansion of a packed tensor in the tiled layout of the pipelined GEMM (uint8 buffer).
+def expand_tiled(p: PackedNVFP4, cache: bool = True, mode: int = MODE_P32) -> torch.Tensor:
+    """16-bit expansion of a packed tensor in the tiled layout of the pipelined GEMM (uint8 buffer): exact binary16
+    values e2m1 * e4m3 * 2^-8 (mode P32) or the reference's bf16 dequantized values, unit included (mode PB16).
     cache=True keeps it on the packed tensor (weights); activations are expanded per call."""
-    if p.tiled is not None:
-        return p.tiled
+    have = p.tiled_pb16 if mode == MODE_PB16 else p.tiled
+    if have is not None:
+        return have
     L = load()
     out = torch.empty(L.metis_nvfp4_expand_tiled_bytes(p.rows, p.cols), dtype=torch.uint8, device=p.codes.device)
-    rc = L.metis_nvfp4_expand_tiled(p.codes.data_ptr(), p.scales.data_ptr(), p.rows, p.cols, out.data_ptr(), _stream())
+    rc = L.metis_nvfp4_expand_tiled(p.codes.data_ptr(), p.scales.data_ptr(), p.unit.data_ptr(), p.rows, p.cols, mode,
+                                    out.data_ptr(), _stream())
     check(rc, "metis_nvfp4_expand_tiled", (p.rows, p.cols))
     if cache:
-        p.tiled = out
+        if mode == MODE_PB16:
+            p.tiled_pb16 = out
+        else:
+            p.tiled = out
     return out
+
+
+@functools.lru_cache(maxsize=4096)
+def _tiled_workspace_bytes(M: int, N: int, K: int, mode: int, device_index: int) -> int:
+    return int(load().metis_linear_tiled_workspace_bytes(M, N, K, mode))
 
 
 def linear_fwd_tiled(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None, u: torch.Tensor | None = None,
                      bias: torch.Tensor | None = None, out_dtype: torch.dtype = torch.bfloat16,
-                     a_tiled: torch.Tensor | None = None) -> torch.Tensor:
-    """linear_fwd on tiled binary16 expansions: b's is cached on b, a's is made here unless given."""
+                     a_tiled: torch.Tensor | None = None, reference_rounding: bool = False,
+                     split_k: bool = True) -> torch.Tensor:
+    """linear_fwd on tiled 16-bit expansions: b's is cached on b when b is persistent, a's is made here unless given.
+
+    reference_rounding (both operands packed in bf16 arithmetic): operands are the reference's bf16 dequantized
+    values and the epilogue rounds where the reference's all-bf16 forward rounds; otherwise exact products."""
     if a.cols != b.cols:
         raise ValueError(f"contraction mismatch: {a.cols} vs {b.cols}")
+    mode = MODE_P32
+    if reference_rounding:
+        if a.mode != MODE_PB16 or b.mode != MODE_PB16:
+            raise ValueError("reference_rounding needs both operands packed in bf16 arithmetic")
+        mode = MODE_PB16
     M, N, K = a.rows, b.rows, a.cols
+    dev = a.codes.device
     r = 0
     if t is not None:
         t = t.to(torch.bfloat16).contiguous()
@@ -339,13 +361,16 @@ def linear_fwd_tiled(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None =
     bias_f32 = bias is not None and bias.dtype == torch.float32
     if bias is not None:
         bias = bias.contiguous() if bias_f32 else bias.to(torch.bfloat16).contiguous()
-    bx = expand_tiled(b)
-    ax = a_tiled if a_tiled is not None else expand_tiled(a, cache=False)
-    out = torch.empty(M, N, dtype=out_dtype, device=a.codes.device)
+    bx = expand_tiled(b, cache=b.persistent, mode=mode)
+    ax = a_tiled if a_tiled is not None else expand_tiled(a, cache=False, mode=mode)
+    out = torch.empty(M, N, dtype=out_dtype, device=dev)
+    need = _tiled_workspace_bytes(M, N, K, mode, dev.index or 0) if split_k else 0
+    ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
     rc = load().metis_linear_fwd_tiled(ax.data_ptr(), a.unit.data_ptr(), bx.data_ptr(), b.unit.data_ptr(), M, N, K,
                                        None if t is None else t.data_ptr(), None if u is None else u.data_ptr(), r,
                                        None if bias is None else bias.data_ptr(), int(bias_f32), out.data_ptr(),
-                                       DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16, _stream())
+                                       DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16, mode,
+                                       None if ws is None else ws.data_ptr(), need, _stream())
     check(rc, "metis_linear_fwd_tiled", (M, N, K))
     return out
 
@@ -380,16 +405,12 @@ def _device_cus(device_index: int) -> int:
 
 def _tiled_applies(a: PackedNVFP4, b: PackedNVFP4) -> bool:
     """The pipelined GEMM on tiled binary16 expansions pays when the weight-side expansion is reused across calls
-    (a cached weight) and the shape fills the device at least once with 256 x 256 tiles; the activation side is
-    expanded per call (2.56 B/element, about 2 % of the GEMM's time at such shapes).  Shapes with fewer tiles than
-    compute units stay on the packed kernels, which can split K."""
+    (a cached weight) and the batch fills a 256-row tile; the activation side is expanded per call (2.56 B/element,
+    about 2 % of the GEMM's time at such shapes)."""
     if not (b.persistent or b.tiled is not None):
         return False
     M, N, K = a.rows, b.rows, a.cols
-    if M < 256 or N < 256 or K % 32 or K < 128:
-        return False
-    tiles = ((M + 255) // 256) * ((N + 255) // 256)
-    return tiles >= _device_cus(a.codes.device.index or 0)
+    return M >= 256 and N >= 256 and K % 32 == 0 and K >= 128
 
 
 @functools.lru_cache(maxsize=4096)
@@ -428,11 +449,15 @@ def _gemm_workspace(M: int, N: int, K: int, device: torch.device) -> torch.Tenso
 
 def linear_fwd(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None, u: torch.Tensor | None = None,
                bias: torch.Tensor | None = None, out_dtype: torch.dtype = torch.bfloat16,
-               expanded: bool | None = None, split_k: bool = True, tiled: bool | None = None) -> torch.Tensor:
+               expanded: bool | None = None, split_k: bool = True, tiled: bool | None = None,
+               reference_rounding: bool = False) -> torch.Tensor:
     """out[M, N] = deq(a)[M, K] . deq(b)[N, K]^T (+ t[M, r] . u[N, r]^T) (+ bias[N]).
 
     tiled=None picks the pipelined kernel on tiled binary16 expansions when b is a cached weight and the shape is
     large (see _tiled_applies); True / False force the choice.  Same bits either way (unsplit).
+    reference_rounding: the forward of a layer whose arithmetic is bf16 (both operands packed in that mode): follow the
+    reference's all-bf16 evaluation (twice-rounded bf16 operands, residual product and bias add rounded to bf16), which
+    only the pipelined kernel implements; requests for fewer than 256 rows are served with exact products.
 
     split_k=False withholds the split-K workspace: the contraction then runs unsplit in one launch.
 
@@ -440,10 +465,11 @@ def linear_fwd(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None,
     MFMA + LDS reads only); the default works on the packed operands directly."""
     if a.cols != b.cols:
         raise ValueError(f"contraction mismatch: {a.cols} vs {b.cols}")
+    faithful = reference_rounding and a.mode == MODE_PB16 and b.mode == MODE_PB16 and (a.rows >= 256 or tiled) and a.cols % 32 == 0
     if tiled is None:
-        tiled = not expanded and _tiled_applies(a, b)
+        tiled = faithful or (not expanded and _tiled_applies(a, b))
     if tiled:
-        return linear_fwd_tiled(a, b, t=t, u=u, bias=bias, out_dtype=out_dtype)
+        return linear_fwd_tiled(a, b, t=t, u=u, bias=bias, out_dtype=out_dtype, reference_rounding=faithful, split_k=split_k)
     M, N, K = a.rows, b.rows, a.cols
     dev = a.codes.device
     r = 0

@@ -225,23 +225,36 @@ int metis_linear_fwd_expanded(const void *a_exp, const float *a_unit, const void
                               const void *bias, void *out, int out_dtype, void *stream);
 
 /*
- * The same expansion in the layout the pipelined GEMM streams from: tiles of 16 rows x 32 k (1 KiB each, tile
- * (rb, kb) at byte ((rb * cols/32) + kb) * 1024, rows padded to a multiple of 16 with zeros), the 16-byte chunks of
- * a tile permuted so that one direct-to-LDS load per tile leaves it free of bank conflicts for the MFMA fragment
- * reads.  metis_linear_fwd_tiled then runs a main loop of MFMA and LDS reads only, its operand tiles arriving
- * through a ring of direct-to-LDS loads; results equal metis_linear_fwd on the packed operands bit for bit
- * (same exact products, same order of binary32 accumulation).  Derived data like the expansion above: callers
- * cache a weight's tiled expansion next to its packed form and re-expand an activation per call (2 B/element).
- *   metis_nvfp4_expand_tiled_bytes  size of `out` for a [rows, cols] packed tensor
+ * Expansion of a packed tensor into the layout the pipelined GEMM streams from, and that GEMM.
+ * Layout: tiles of 16 rows x 32 k (1 KiB each, tile (rb, kb) at byte ((rb * cols/32) + kb) * 1024, rows padded to a
+ * multiple of 16 with zeros), the 16-byte chunks of a tile permuted so that one direct-to-LDS load per tile leaves
+ * it free of bank conflicts for the MFMA fragment reads.  Element values by `mode`:
+ *   METIS_MODE_P32   binary16  e2m1(code) * e4m3(scale) * 2^-8, exact; the GEMM applies unit_a * unit_b * 2^16 to its
+ *                    accumulators.  Results equal metis_linear_fwd on the packed operands bit for bit when neither
+ *                    splits K (same exact products, same order of binary32 accumulation).
+ *   METIS_MODE_PB16  bf16, the value the reference's quantize_dequantize returns when every op rounds to bf16
+ *                    (src/Metis/Metis/quant.py:23-24, 32-35: bf16(bf16(e4m3 * unit) * v / 2), `unit` required), and the
+ *                    GEMM follows the reference's all-bf16 forward (src/Metis/Metis/bitlinear.py:435-438 with
+ *                    compute_dtype = bfloat16, as src/grpo/grpo.py:204-205 configures it): bf16 operands, binary32
+ *                    accumulation, the residual product rounded to bf16, the bias added in bf16, then the low-rank
+ *                    term t u^T (binary32) and one final rounding to bf16 (a binary32 `out` receives those bf16 values).
+ *                    Both operands must have been packed and expanded in this mode; the units are not read.
+ * metis_linear_fwd_tiled runs a main loop of MFMA and LDS reads only, its operand tiles arriving through a ring of
+ * direct-to-LDS loads.  Derived data like the expansion above: callers cache a weight's tiled expansion next to its
+ * packed form and re-expand an activation per call (2.56 B/element).  With a workspace
+ * (metis_linear_tiled_workspace_bytes, 16-byte aligned, no initialisation; 0 = the shape is not split; NULL = never
+ * split) shapes with few 256 x 256 output tiles split K as metis_linear_fwd_ws does.
  *   limits  cols % 32 == 0; GEMM: K % 32 == 0, N % 4 == 0, r % 32 == 0; out, t, u 16-byte aligned
  *   bias    bf16 [N], or float [N] when bias_is_f32 != 0, or NULL
  */
 size_t metis_nvfp4_expand_tiled_bytes(int64_t rows, int64_t cols);
-int metis_nvfp4_expand_tiled(const void *codes, const void *scales, int64_t rows, int64_t cols, void *out,
-                             void *stream);
+int metis_nvfp4_expand_tiled(const void *codes, const void *scales, const float *unit, int64_t rows,
+                             int64_t cols, int mode, void *out, void *stream);
+size_t metis_linear_tiled_workspace_bytes(int64_t M, int64_t N, int64_t K, int mode);
 int metis_linear_fwd_tiled(const void *a_xt, const float *a_unit, const void *b_xt, const float *b_unit,
                            int64_t M, int64_t N, int64_t K, const void *t, const void *u, int64_t r,
-                           const void *bias, int bias_is_f32, void *out, int out_dtype, void *stream);
+                           const void *bias, int bias_is_f32, void *out, int out_dtype, int mode,
+                           void *workspace, size_t workspace_bytes, void *stream);
 
 /*
  * grad_input[L,K] = deq(dY)[L,N] . deq(W)[N,K]   (src/Metis/Metis/bitlinear.py:507-508)

@@ -147,9 +147,11 @@ def test_tiled_pipelined_path_is_bit_identical_to_packed_path(M, N, K, r, bias_f
         want = want + t.double() @ u.double().T
     for dt in (torch.float32, torch.bfloat16):
         a = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, out_dtype=dt, split_k=False)
-        b = ops.linear_fwd_tiled(px, pw, t=t, u=u, bias=bias, out_dtype=dt)
+        b = ops.linear_fwd_tiled(px, pw, t=t, u=u, bias=bias, out_dtype=dt, split_k=False)
+        c = ops.linear_fwd_tiled(px, pw, t=t, u=u, bias=bias, out_dtype=dt)                # K split where the shape has few tiles
         torch.cuda.synchronize()
         assert rel_fro(b.cpu(), want.cpu().to(dt)) <= (1e-5 if dt == torch.float32 else TOL)
+        assert rel_fro(c.cpu(), want.cpu().to(dt)) <= (1e-5 if dt == torch.float32 else TOL)
         assert torch.equal(a, b), f"{(a != b).sum().item()} of {a.numel()} elements differ ({dt})"
     # the tiled expansion holds exactly the values of the row-major one
     e = ops.expand(px)
@@ -160,6 +162,48 @@ def test_tiled_pipelined_path_is_bit_identical_to_packed_path(M, N, K, r, bias_f
     unswz = torch.gather(tiles, 3, slot[None, None, :, :, None].expand(tiles.shape[0], tiles.shape[1], 16, 4, 8))
     flat = unswz.permute(0, 2, 1, 3, 4).reshape(-1, K)[:M]
     assert torch.equal(flat, e)
+
+
+@pytest.mark.parametrize("M,N,K,r,with_bias", [(512, 768, 1024, 64, True), (300, 260, 96, 0, True), (1024, 512, 8192, 32, False),
+                                               (2048, 3584, 2048, 64, True), (4096, 4352, 1024, 32, True)])
+def test_tiled_path_with_reference_rounding_in_bf16_arithmetic(M, N, K, r, with_bias):
+    """Both operands packed in bf16 arithmetic, reference_rounding: the pipelined kernel multiplies the reference's own
+    bf16 dequantized values and rounds where its all-bf16 forward rounds (matmul result, bias add, final sum).  Checked
+    against that evaluation carried out in double precision between the roundings: the kernel's binary32 accumulation
+    can only move a result that sits on a bf16 rounding boundary.  Shapes cover unsplit tiles, K split over the whole
+    grid (1024 x 512 x 8192), and a split last round (4096 x 4352)."""
+    from metis_hip import _lib, ops
+    g = torch.Generator().manual_seed(5000 + M)
+    x = synthetic_activation(70 + M, M, K).cuda()
+    w = _weights(71 + N, N, K).cuda()
+    t = u = None
+    if r:
+        t = torch.randn(M, r, generator=g).bfloat16().cuda()
+        u = (torch.randn(N, r, generator=g) * 0.05).bfloat16().cuda()
+    bias = (torch.randn(N, generator=g) * 0.1).bfloat16().cuda() if with_bias else None
+    px, pw = ops.quantize(x, 1), ops.quantize(w, 1)
+    xq, wq = ops.dequantize(px, torch.bfloat16).double(), ops.dequantize(pw, torch.bfloat16).double()   # the reference's QDQ values
+    want = (xq @ wq.T).bfloat16()
+    if bias is not None:
+        want = (want.float() + bias.float()).bfloat16()
+    want = want.double()
+    if r:
+        want = want + t.double() @ u.double().T
+    want = want.bfloat16()
+    if K >= 2048 or M * N >= 4096 * 4096:
+        assert _lib.load().metis_linear_tiled_workspace_bytes(M, N, K, 1) > 0
+    got = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, reference_rounding=True)
+    got32 = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, out_dtype=torch.float32, reference_rounding=True)
+    unsplit = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, reference_rounding=True, split_k=False)
+    torch.cuda.synchronize()
+    assert torch.equal(got32, got.float())                       # a binary32 buffer receives the same bf16 values
+    for y in (got, unsplit):
+        differ = (y != want).float().mean().item()
+        assert differ < 2e-3, f"{differ:.2e} of the outputs differ from the all-bf16 evaluation"
+        assert rel_fro(y.float().cpu(), want.float().cpu()) <= 2e-4
+    # and it is a different number from the exact-product result: the two modes are not interchangeable
+    exact = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, reference_rounding=False, tiled=True)
+    assert 5e-4 < rel_fro(exact.float().cpu(), want.float().cpu()) < 2e-2
 
 
 @pytest.mark.parametrize("M,N,K,r", [(64, 4736, 3584, 64), (17, 2052, 2048, 0), (1, 4608, 3584, 32), (40, 1536, 8960, 64),
