@@ -246,6 +246,55 @@ def golden_mean_mode(out: dict):
         F.enable_activation_svd, F.enable_backward_svd = False, False
 
 
+def golden_rollout(out: dict):
+    """Rollout shortcut of BitLinear.forward (rollout_merge_active, no autograd): one matmul of the quantized
+    activation against the cached merged weight (U diag s) Q(V) + Q(W_res), next to the three-GEMM forward of the
+    same layer.  binary32 arithmetic; the layer is assembled by hand as in golden_linear."""
+    g = torch.Generator().manual_seed(47)
+    B, T, K, N, r = 2, 24, 96, 64, 8
+    x = torch.randn(B, T, K, generator=g).bfloat16().float()
+    w = (torch.randn(N, K, generator=g) * 0.05).bfloat16().float()
+    b = (torch.randn(N, generator=g) * 0.1).bfloat16().float()
+    args = SimpleNamespace(device="cpu", cache_quantized_weight=True, forward_svd_rank=r)
+    _configure("nvfp4e2m1bnosr", "nvfp4e2m1bnosr", "nvfp4e2m1b", torch.float32)
+    bl = rb.BitLinear.__new__(rb.BitLinear)
+    torch.nn.Module.__init__(bl)
+    bl.args = args
+    bl.is_svd_quant = True
+    bl.mean_cache = {}
+    bl.activation_group = None
+    bl._merged_rollout_weight_cache = None
+    bl.layer_name = "golden.rollout"
+    bl.vlinear = rb.LinearLowbit(K, r, bias=False, args=args)
+    bl.ulinear = torch.nn.Linear(r, N, bias=False)
+    bl.warmup_linear = rb.LinearLowbit(K, N, bias=True, args=args)
+    U, S, Vh = torch.linalg.svd(w, full_matrices=False)
+    with torch.no_grad():
+        bl.vlinear.weight.copy_(Vh[:r].bfloat16().float())
+        bl.ulinear.weight.copy_(U[:, :r].bfloat16().float())
+        bl.s = torch.nn.Parameter(S[:r].bfloat16().float().clone())
+        bl.warmup_linear.weight.copy_((w - (U[:, :r] * S[:r]) @ Vh[:r]).bfloat16().float())
+        bl.warmup_linear.bias.copy_(b)
+    with torch.no_grad():
+        y_three = bl(x)
+        rb.BitLinear.rollout_merge_active = True
+        try:
+            y_merged = bl(x)
+            merged_w = bl._get_merged_rollout_weight(torch.float32)
+            again = bl._get_merged_rollout_weight(torch.float32)
+            assert again is merged_w                                  # cached on the parameter versions
+            bl.s.add_(0.0)                                            # bumps the version: the cache is dropped
+            assert bl._get_merged_rollout_weight(torch.float32) is not merged_w
+        finally:
+            rb.BitLinear.rollout_merge_active = False
+    out["ro_x"], out["ro_b"] = bits(x), bits(b)
+    out["ro_v"], out["ro_u"] = bits(bl.vlinear.weight.detach()), bits(bl.ulinear.weight.detach())
+    out["ro_s"], out["ro_res"] = bits(bl.s.detach()), bits(bl.warmup_linear.weight.detach())
+    out["ro_merged_weight"] = bits(merged_w)
+    out["ro_y_merged"] = bits(y_merged)
+    out["ro_y_three_gemm"] = bits(y_three)
+
+
 def main():
     torch.set_num_threads(1)
     out: dict = {}
@@ -260,6 +309,11 @@ def main():
     path = os.path.join(HERE, "metis_reference_hadamard.npz")
     np.savez_compressed(path, **had)
     print(f"wrote {path}: {len(had)} arrays, {os.path.getsize(path)} bytes")
+    ro: dict = {}
+    golden_rollout(ro)
+    path = os.path.join(HERE, "metis_reference_rollout.npz")
+    np.savez_compressed(path, **ro)
+    print(f"wrote {path}: {len(ro)} arrays, {os.path.getsize(path)} bytes")
     mm: dict = {}
     golden_mean_mode(mm)
     path = os.path.join(HERE, "metis_reference_mean_mode.npz")

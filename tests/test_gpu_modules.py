@@ -242,6 +242,93 @@ def test_rollout_switch_on_the_fused_path_and_merged_weight_helper():
     assert rel_fro(first.cpu(), want.cpu()) < 1e-6
 
 
+def test_rollout_merged_weight_against_reference_vectors():
+    """The merged rollout weight (U diag s) Q(V) + Q(W_res) and the one-matmul forward that uses it, against what the
+    reference computed for the same hand-assembled layer (binary32 arithmetic): the two quantized weights are bit-exact,
+    so only the order of the binary32 sums in the small products differs."""
+    import os
+    import numpy as np
+    from metis_hip import BitLinear, LinearLowbit, MetisArgs
+    z = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "metis_reference_rollout.npz"))
+    x, b = t(z["ro_x"]), t(z["ro_b"])
+    v, u, s, res = t(z["ro_v"]), t(z["ro_u"]), t(z["ro_s"]), t(z["ro_res"])
+    r, K = v.shape
+    N = u.shape[0]
+    args = MetisArgs.direct_fp4(forward_svd_rank=r)
+    layer = BitLinear(K, N, args=args, bias=True, dtype=torch.float32, compute_dtype=torch.float32).cuda()
+    layer.warmup_linear = LinearLowbit(K, N, bias=True, args=args, device="cuda")
+    layer.vlinear = LinearLowbit(K, r, bias=False, args=args, device="cuda")
+    layer.ulinear = torch.nn.Linear(r, N, bias=False, device="cuda")
+    with torch.no_grad():
+        layer.vlinear.weight.copy_(v)
+        layer.ulinear.weight.copy_(u)
+        layer.s = torch.nn.Parameter(s.clone().cuda())
+        layer.warmup_linear.weight.copy_(res)
+        layer.warmup_linear.bias.copy_(b)
+    layer.is_svd_quant = True
+    with torch.no_grad():
+        merged = layer._get_merged_rollout_weight(torch.float32)
+        assert rel_fro(merged.cpu(), t(z["ro_merged_weight"])) <= 1e-6
+        # the reference's current file feeds the rank-r branch the quantized activation and the quantized V; with that
+        # variant selected the rollout switch takes the merged-weight matmul exactly as the reference does
+        BitLinear.quantized_lowrank_branch = True
+        try:
+            three = layer(x.cuda())
+            BitLinear.rollout_merge_active = True
+            one = layer(x.cuda())
+        finally:
+            BitLinear.rollout_merge_active = False
+            BitLinear.quantized_lowrank_branch = False
+    assert rel_fro(one.cpu(), t(z["ro_y_merged"])) <= 1e-5
+    assert rel_fro(three.cpu(), t(z["ro_y_three_gemm"])) <= 1e-5
+
+
+def test_packed_weight_cache_reuses_then_invalidates_on_the_device():
+    """The weight cache holds the PACKED weight (and what hangs off it: the column-blocked packing for dgrad, the tiled
+    expansion of the pipelined GEMM), keyed on Parameter._version as the reference keys its dequantized cache
+    (reference test_weight_cache_reuses_then_invalidates): one quantization before an update, a second one after
+    `weight.add_`, with fresh derived layouts and a different result."""
+    from metis_hip import LinearLowbit, MetisArgs, ops, quant_func
+    from metis_hip.ops import PackedNVFP4
+    args = MetisArgs.direct_fp4()
+    lin = LinearLowbit(512, 512, bias=False, args=args, device="cuda", storage_dtype=torch.bfloat16, compute_dtype=torch.float32)
+    x = synthetic_activation(91, 512, 512).cuda().requires_grad_(True)
+    base = quant_func["nvfp4e2m1bnosr"]
+    orig = base.pack.__func__
+    packs = []
+
+    def spy(cls, t_, col=False, noise=None, arith=None, center=None):
+        packs.append((tuple(t_.shape), bool(col)))
+        return orig(cls, t_, col, noise, arith, center)
+
+    base.pack = classmethod(spy)
+    try:
+        y1 = lin(x)
+        first = lin._quantized_weight_cache[1]
+        assert isinstance(first, PackedNVFP4) and first.persistent
+        y1.sum().backward()
+        assert first.transposed is not None                       # dgrad packed the weight column-blocked, once
+        assert first.tiled is not None                            # 512 rows: the pipelined GEMM kept its expansion
+        n_weight_packs = sum(1 for shp, _ in packs if shp == (512, 512))
+        y2 = lin(x)
+        y2.sum().backward()
+        assert lin._quantized_weight_cache[1] is first
+        # the second step packed activations only: x row-wise, nothing of the weight (dgrad operands are not this class)
+        assert sum(1 for shp, _ in packs if shp == (512, 512)) == n_weight_packs + 1
+        assert torch.equal(y1, y2)
+        with torch.no_grad():
+            lin.weight.add_(0.01)
+        y3 = lin(x)
+        second = lin._quantized_weight_cache[1]
+        assert second is not first and second.transposed is None                 # no backward yet on the new packing
+        assert second.tiled is not None and second.tiled is not first.tiled       # this forward made its own expansion
+        assert not torch.equal(y3, y1)
+        want = ops.dequantize(ops.quantize(x.detach()), torch.float32).double() @ ops.dequantize(second, torch.float32).double().T
+        assert rel_fro(y3.detach().cpu(), want.cpu()) <= 1e-5
+    finally:
+        base.pack = classmethod(orig)
+
+
 def test_patch_qwen2_decoder_layer():
     """A randomly initialised Hugging Face Qwen2 decoder layer with every projection replaced."""
     transformers = pytest.importorskip("transformers")
