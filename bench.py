@@ -150,7 +150,7 @@ def main():
         # launch alone: quantize X, expand it into the tiled binary16 layout, rank-r projection, pipelined GEMM
         px = ops.quantize(x)
         ax = ops.expand_tiled(px, cache=False)
-        t = torch.matmul(x, vt) * s
+        _, t = ops.lowrank_project(x, v, s)                      # (X V^T) * s in bf16, one pass over X
         if ev is not None:
             ev[0].record()
         y = ops.linear_fwd_tiled(px, pw, t=t, u=u, a_tiled=ax)

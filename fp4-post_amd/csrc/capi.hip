@@ -275,6 +275,20 @@ int metis_lowrank_project(const void* x, int64_t ldx, const void* v, int64_t M, 
     return lowrank_small(x, ldx, v, M, R, K, s, xv, t, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
+int metis_lowrank_project_rows(const void* x, int64_t ldx, const void* v, int64_t M, int64_t R, int64_t K, const void* s, void* xv,
+                               void* t, void* stream)
+{
+    return lowrank_nt(x, ldx, v, M, R, K, s, xv, t, (hipStream_t)stream);
+}
+
+size_t metis_lowrank_tokens_workspace_bytes(int64_t L, int64_t C, int64_t R) { return lowrank_tn_workspace_bytes(L, C, R); }
+
+int metis_lowrank_contract_tokens(const void* a, int64_t lda, const void* b, int64_t L, int64_t C, int64_t R, void* out, int out_dtype,
+                                  int transpose, void* workspace, size_t workspace_bytes, void* stream)
+{
+    return lowrank_tn(a, lda, b, L, C, R, out, out_dtype, transpose, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
 size_t metis_linear_workspace_bytes(int64_t M, int64_t N, int64_t K) { return gemm_workspace_bytes(M, N, K); }
 
 int metis_linear_fwd_ws(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes,

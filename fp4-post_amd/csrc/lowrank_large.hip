@@ -1,0 +1,332 @@
+// Rank-r products of the low-rank branch at training / prefill sizes (256 rows and more), bf16 operands, binary32
+// accumulation on MFMA.  Both are bound by one pass over the tall operand in HBM.
+//
+//   lowrank_nt:  xv[M, R] = x[M, K] . v[R, K]^T,  t = bf16(xv * s)      `vlinear(x)` and `torch.mul(self.s, y)` of
+//                BitLinear.forward with the bf16 V of the north-star formula (src/Metis/Metis/bitlinear.py:752-756);
+//                with v = U^T also dY . U of the backward pass
+//   lowrank_tn:  out[C, R] = sum_l a[l, C] . b[l, R]                     the two products of the backward pass that
+//                contract over tokens: dY^T . (xv * s) -> grad of U, x^T . g_xv -> grad of V (written transposed)
+//
+// lowrank_nt: a workgroup owns 32 rows of x and walks K in steps of 256.  The x rows (32 x 512 B) and the R rows of v
+// (R x 512 B, from L2 after the first workgroup touched them) are fetched two steps ahead into registers, 16 bytes
+// per thread and load, and staged in LDS with 528-byte rows; wave w multiplies the w-th quarter (64 k) of the step
+// for all R columns, and the four partial sums meet in LDS at the end.
+//
+// lowrank_tn: the contraction runs down the rows of both operands, so each has to be turned: a workgroup owns 64
+// columns of a and one slice of the tokens; a step of 64 tokens is loaded row by row (coalesced) and written to LDS
+// transposed, element by element, so that the MFMA fragments (8 consecutive tokens of one column) are single
+// 16-byte reads.  Token slices give every compute unit work; their binary32 partial results go to a caller workspace
+// and a second kernel adds them in slice order.
+#include "metis_device.h"
+#include "metis_host.h"
+
+namespace metis {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+constexpr int LR_STRIDE = 72;                    // halves per staged row of 64: 144 bytes, conflict-free 16-byte reads
+constexpr int NT_STEP = 256;                     // k per step of lowrank_nt
+constexpr int NT_STRIDE = NT_STEP + 8;           // halves per staged row: 528 bytes, conflict-free 16-byte reads
+
+template <int RT>                                // R / 32 column tiles: 1, 2 or 4
+__global__ __launch_bounds__(256) void lowrank_nt_kernel(const uint16_t* __restrict__ x, int64_t ldx, const uint16_t* __restrict__ v,
+                                                         const uint16_t* __restrict__ s, uint16_t* __restrict__ xv,
+                                                         uint16_t* __restrict__ t, int M, int K)
+{
+    constexpr int R = RT * 32;
+    constexpr int TILE_BYTES = (32 + R) * NT_STRIDE * 2;        // one staged step: x rows, then v rows
+    constexpr int RED_BYTES = 4 * RT * 16 * 64 * 4;
+    constexpr int LDS_BYTES = TILE_BYTES > RED_BYTES ? TILE_BYTES : RED_BYTES;
+    __shared__ __attribute__((aligned(16))) unsigned char lds[LDS_BYTES];     // the staged step, then the four partial sums
+    uint16_t* tile = reinterpret_cast<uint16_t*>(lds);
+    float* red = reinterpret_cast<float*>(lds);                 // [wave][j][e][lane]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int m0 = blockIdx.x * 32;
+    // staging: 16-byte chunk id -> (row id / 32, chunk id % 32): a wave covers two rows x 512 contiguous bytes per load.
+    // A thread keeps two whole steps (each 4 chunks of x, 4 RT of v) in registers while the one before them is
+    // multiplied: with one workgroup per compute unit that is what keeps enough bytes in flight.
+    uint4 rx[2][4], rv[2][RT * 4];
+    auto fetch = [&](uint4 (&qx)[4], uint4 (&qv)[RT * 4], int k0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int id = i * 256 + tid, row = id >> 5, k = k0 + (id & 31) * 8;
+            qx[i] = k < K ? *reinterpret_cast<const uint4*>(x + (int64_t)min(m0 + row, M - 1) * ldx + k) : make_uint4(0u, 0u, 0u, 0u);
+        }
+#pragma unroll
+        for (int i = 0; i < RT * 4; ++i) {
+            const int id = i * 256 + tid, row = id >> 5, k = k0 + (id & 31) * 8;
+            qv[i] = k < K ? *reinterpret_cast<const uint4*>(v + (int64_t)row * K + k) : make_uint4(0u, 0u, 0u, 0u);
+        }
+    };
+    auto stage = [&](const uint4 (&qx)[4], const uint4 (&qv)[RT * 4]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int id = i * 256 + tid;
+            *reinterpret_cast<uint4*>(tile + (id >> 5) * NT_STRIDE + (id & 31) * 8) = qx[i];
+        }
+#pragma unroll
+        for (int i = 0; i < RT * 4; ++i) {
+            const int id = i * 256 + tid;
+            *reinterpret_cast<uint4*>(tile + (32 + (id >> 5)) * NT_STRIDE + (id & 31) * 8) = qv[i];
+        }
+    };
+    float16_t acc[RT];
+#pragma unroll
+    for (int j = 0; j < RT; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[j][e] = 0.0f;
+
+    const int steps = (K + NT_STEP - 1) / NT_STEP;              // K % 64 == 0; a short last step is padded with zeros
+    // wave w multiplies the quarter [64 w, 64 w + 64) of every step
+    const int foff = (lane & 31) * NT_STRIDE + wave * 64 + (lane >> 5) * 8;
+    auto multiply = [&]() {
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const bf16x8_t fa = *reinterpret_cast<const bf16x8_t*>(tile + foff + ks * 16);
+#pragma unroll
+            for (int j = 0; j < RT; ++j) {
+                const bf16x8_t fb = *reinterpret_cast<const bf16x8_t*>(tile + (32 + j * 32) * NT_STRIDE + foff + ks * 16);
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb, fa, acc[j], 0, 0, 0);
+            }
+        }
+    };
+    // two steps are in flight while a third is multiplied: the time of one step is then half the memory latency
+    fetch(rx[0], rv[0], 0);
+    if (steps > 1) fetch(rx[1], rv[1], NT_STEP);
+    for (int st = 0; st < steps; st += 2) {
+        stage(rx[0], rv[0]);
+        __syncthreads();
+        if (st + 2 < steps) fetch(rx[0], rv[0], (st + 2) * NT_STEP);
+        multiply();
+        __syncthreads();
+        if (st + 1 < steps) {
+            stage(rx[1], rv[1]);
+            __syncthreads();
+            if (st + 3 < steps) fetch(rx[1], rv[1], (st + 3) * NT_STEP);
+            multiply();
+            __syncthreads();
+        }
+    }
+    // acc[j][e] of lane l: row m0 + l % 32, column 32 j + 8 (e / 4) + 4 (l / 32) + e % 4.  The four waves hold the four
+    // quarters of every step of K: their sums meet in LDS (the staged tile is dead after the last barrier), and
+    // wave w finishes the quarter e / 4 == w of the columns, adding the waves' shares in the order 0, 1, 2, 3.
+#pragma unroll
+    for (int j = 0; j < RT; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) red[((wave * RT + j) * 16 + e) * 64 + lane] = acc[j][e];
+    __syncthreads();
+    const int m = m0 + (lane & 31);
+    if (m >= M) return;
+#pragma unroll
+    for (int j = 0; j < RT; ++j) {
+        const int col = j * 32 + 8 * wave + 4 * (lane >> 5);
+        uint32_t h[4], ts[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int ee = 4 * wave + e;
+            float sum = red[((0 * RT + j) * 16 + ee) * 64 + lane];
+#pragma unroll
+            for (int w = 1; w < 4; ++w) sum += red[((w * RT + j) * 16 + ee) * 64 + lane];
+            h[e] = bf16_bits(sum);
+            if (t) ts[e] = bf16_bits(__uint_as_float(h[e] << 16) * bf16_lo(s[col + e]));
+        }
+        *reinterpret_cast<uint2*>(xv + (int64_t)m * R + col) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+        if (t) *reinterpret_cast<uint2*>(t + (int64_t)m * R + col) = make_uint2(ts[0] | (ts[1] << 16), ts[2] | (ts[3] << 16));
+    }
+}
+
+int lowrank_nt(const void* x, int64_t ldx, const void* v, int64_t M, int64_t R, int64_t K, const void* s, void* xv, void* t,
+               hipStream_t st)
+{
+    if (M < 0 || R <= 0 || K <= 0 || ldx < K) return METIS_E_ARG;
+    if ((R != 32 && R != 64 && R != 128) || K % 64 || ldx % 8) return METIS_E_SHAPE;
+    if (M == 0) return METIS_OK;
+    if (M > INT32_MAX - 32 || K > INT32_MAX) return METIS_E_ARG;
+    if (!x || !v || !xv || (t && !s)) return METIS_E_ARG;
+    if (((uintptr_t)x % 16) || ((uintptr_t)v % 16) || ((uintptr_t)xv % 8) || ((uintptr_t)t % 8) || ((uintptr_t)s % 2)) return METIS_E_ARG;
+    const dim3 grid((unsigned)((M + 31) / 32));
+#define METIS_NT(RT) hipLaunchKernelGGL((lowrank_nt_kernel<RT>), grid, dim3(256), 0, st, (const uint16_t*)x, ldx, (const uint16_t*)v, \
+                                        (const uint16_t*)s, (uint16_t*)xv, (uint16_t*)t, (int)M, (int)K)
+    if (R == 32) METIS_NT(1);
+    else if (R == 64) METIS_NT(2);
+    else METIS_NT(4);
+#undef METIS_NT
+    return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
+}
+
+// ---------------------------------------------------------------------------------------------
+// out[C, R] = sum_l a[l, C] b[l, R]
+// ---------------------------------------------------------------------------------------------
+template <int RT>
+__global__ __launch_bounds__(256) void lowrank_tn_kernel(const uint16_t* __restrict__ a, int64_t lda, const uint16_t* __restrict__ b,
+                                                         int L, int C, int steps_per_slice, float* __restrict__ part)
+{
+    constexpr int R = RT * 32;
+    __shared__ __attribute__((aligned(16))) uint16_t at[64 * LR_STRIDE];      // [column][token]
+    __shared__ __attribute__((aligned(16))) uint16_t bt[R * LR_STRIDE];       // [r][token]
+    __shared__ __attribute__((aligned(16))) float red[2][RT][16][64];         // the two waves that take the second half of each step
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int c0 = blockIdx.x * 64, slice = blockIdx.y;
+    const int steps_all = (L + 63) / 64;
+    const int s0 = slice * steps_per_slice, s1 = min(s0 + steps_per_slice, steps_all);
+    // loading: thread -> token tid / 8 (+ 32), 16-byte chunk tid % 8 of the 64 columns; for b, R / 8 chunks per token
+    const int lrow = tid >> 3, lch = tid & 7;
+    const bool col_live = c0 + lch * 8 < C;                     // C % 8 == 0: a chunk is inside or outside
+    constexpr int BCH = R / 8;                                  // 16-byte chunks per token of b: 4, 8 or 16
+    constexpr int BPT = 64 * BCH / 256;                         // b chunks per thread: 1, 2 or 4
+    uint4 ra[2][2], rbv[2][BPT];
+    auto fetch = [&](uint4 (&ra)[2], uint4 (&rbv)[BPT], int st) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int l = st * 64 + i * 32 + lrow;
+            ra[i] = (l < L && col_live) ? *reinterpret_cast<const uint4*>(a + (int64_t)l * lda + c0 + lch * 8) : make_uint4(0u, 0u, 0u, 0u);
+        }
+#pragma unroll
+        for (int i = 0; i < BPT; ++i) {
+            const int id = i * 256 + tid, l = st * 64 + id / BCH, ch = id % BCH;
+            rbv[i] = l < L ? *reinterpret_cast<const uint4*>(b + (int64_t)l * R + ch * 8) : make_uint4(0u, 0u, 0u, 0u);
+        }
+    };
+    // Transposed tiles: row = column of the operand, 64 tokens in 8 chunks of 8; the chunk of tokens [8 q, 8 q + 8) of
+    // row n sits at chunk q ^ ((n >> 4) & 3), so that the eight column groups a wave scatters at once fall into
+    // different banks (unswizzled they share eight of them).
+    auto scatter = [&](uint16_t* dst, int row0, int tok, const uint4& q) {      // 8 elements of one token -> 8 rows of dst
+        const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+        const int pos = (((tok >> 3) ^ ((row0 >> 4) & 3)) << 3) | (tok & 7);    // rows row0 .. row0 + 7 share row >> 4
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            dst[(row0 + 2 * j) * LR_STRIDE + pos] = (uint16_t)(w[j] & 0xffffu);
+            dst[(row0 + 2 * j + 1) * LR_STRIDE + pos] = (uint16_t)(w[j] >> 16);
+        }
+    };
+    auto stage = [&](const uint4 (&ra)[2], const uint4 (&rbv)[BPT]) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) scatter(at, lch * 8, i * 32 + lrow, ra[i]);
+#pragma unroll
+        for (int i = 0; i < BPT; ++i) {
+            const int id = i * 256 + tid;
+            scatter(bt, (id % BCH) * 8, id / BCH, rbv[i]);
+        }
+    };
+    float16_t acc[RT];
+#pragma unroll
+    for (int j = 0; j < RT; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[j][e] = 0.0f;
+    // wave -> 32 columns (wave % 2) and the first or second half (wave / 2) of every 64-token step
+    const int ct = wave & 1, kh = wave >> 1;
+    const int frow = (lane & 31) * LR_STRIDE, fsw = ((lane & 31) >> 4) & 1;     // rows 32 j + n: (row >> 4) & 3 = 2 (j & 1) + fsw
+    auto multiply = [&]() {
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            const int q = kh * 4 + ks * 2 + (lane >> 5);
+            const bf16x8_t fa = *reinterpret_cast<const bf16x8_t*>(at + ct * 32 * LR_STRIDE + frow + ((q ^ (2 * ct + fsw)) << 3));
+#pragma unroll
+            for (int j = 0; j < RT; ++j) {
+                const bf16x8_t fb = *reinterpret_cast<const bf16x8_t*>(bt + j * 32 * LR_STRIDE + frow + ((q ^ (2 * (j & 1) + fsw)) << 3));
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb, fa, acc[j], 0, 0, 0);
+            }
+        }
+    };
+    // two steps in flight while a third is multiplied
+    if (s0 < s1) fetch(ra[0], rbv[0], s0);
+    if (s0 + 1 < s1) fetch(ra[1], rbv[1], s0 + 1);
+    for (int st = s0; st < s1; st += 2) {
+        stage(ra[0], rbv[0]);
+        __syncthreads();
+        if (st + 2 < s1) fetch(ra[0], rbv[0], st + 2);
+        multiply();
+        __syncthreads();
+        if (st + 1 < s1) {
+            stage(ra[1], rbv[1]);
+            __syncthreads();
+            if (st + 3 < s1) fetch(ra[1], rbv[1], st + 3);
+            multiply();
+            __syncthreads();
+        }
+    }
+    // acc[j][e] of lane l: column c0 + 32 ct + l % 32, r = 32 j + 8 (e / 4) + 4 (l / 32) + e % 4; halves of the steps add up
+    if (kh == 1) {
+#pragma unroll
+        for (int j = 0; j < RT; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) red[ct][j][e][lane] = acc[j][e];
+    }
+    __syncthreads();
+    if (kh == 1) return;
+    const int c = c0 + ct * 32 + (lane & 31);
+    if (c >= C) return;
+    float* dst = part + ((int64_t)slice * C + c) * R;
+#pragma unroll
+    for (int j = 0; j < RT; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            float4 o;
+            o.x = acc[j][4 * g] + red[ct][j][4 * g][lane];
+            o.y = acc[j][4 * g + 1] + red[ct][j][4 * g + 1][lane];
+            o.z = acc[j][4 * g + 2] + red[ct][j][4 * g + 2][lane];
+            o.w = acc[j][4 * g + 3] + red[ct][j][4 * g + 3][lane];
+            *reinterpret_cast<float4*>(dst + j * 32 + 8 * g + 4 * (lane >> 5)) = o;
+        }
+}
+
+// adds the token slices in order; out [C, R] or, transposed, [R, C]; bf16 or binary32
+__global__ __launch_bounds__(256) void lowrank_tn_finish_kernel(const float* __restrict__ part, int slices, int C, int R, void* __restrict__ out,
+                                                                int out_f32, int transpose)
+{
+    const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (id >= (int64_t)C * R) return;
+    float sum = part[id];
+    for (int z = 1; z < slices; ++z) sum += part[(int64_t)z * C * R + id];
+    const int c = (int)(id / R), r = (int)(id % R);
+    const int64_t o = transpose ? (int64_t)r * C + c : id;
+    if (out_f32) static_cast<float*>(out)[o] = sum;
+    else static_cast<uint16_t*>(out)[o] = (uint16_t)bf16_bits(sum);
+}
+
+static int tn_slices(int64_t L, int64_t C, int* steps_per_slice)
+{
+    const int64_t steps = (L + 63) / 64, groups = (C + 63) / 64;
+    int64_t want = (4 * (int64_t)device_cus() + groups - 1) / groups;       // four workgroups per compute unit
+    if (want > steps / 4) want = steps / 4;                                 // at least four steps per slice
+    if (want < 1) want = 1;
+    const int64_t per = (steps + want - 1) / want;
+    *steps_per_slice = (int)per;
+    return (int)((steps + per - 1) / per);
+}
+
+size_t lowrank_tn_workspace_bytes(int64_t L, int64_t C, int64_t R)
+{
+    if (L <= 0 || C <= 0 || R <= 0) return 0;
+    int per;
+    return (size_t)tn_slices(L, C, &per) * (size_t)C * (size_t)R * sizeof(float);
+}
+
+int lowrank_tn(const void* a, int64_t lda, const void* b, int64_t L, int64_t C, int64_t R, void* out, int out_dtype, int transpose,
+               void* workspace, size_t workspace_bytes, hipStream_t st)
+{
+    if (L < 0 || C <= 0 || R <= 0 || lda < C) return METIS_E_ARG;
+    if (out_dtype != METIS_DTYPE_BF16 && out_dtype != METIS_DTYPE_F32) return METIS_E_ARG;
+    if ((R != 32 && R != 64 && R != 128) || C % 8 || lda % 8) return METIS_E_SHAPE;
+    if (L > INT32_MAX - 64 || C > INT32_MAX - 64) return METIS_E_ARG;
+    if (!a || !b || !out) return METIS_E_ARG;
+    if (((uintptr_t)a % 16) || ((uintptr_t)b % 16) || ((uintptr_t)out % 4)) return METIS_E_ARG;
+    if (!workspace || ((uintptr_t)workspace % 16) || workspace_bytes < lowrank_tn_workspace_bytes(L, C, R)) return METIS_E_WORKSPACE;
+    int per;
+    const int slices = tn_slices(L, C, &per);
+    const dim3 grid((unsigned)((C + 63) / 64), (unsigned)slices);
+#define METIS_TN(RT) hipLaunchKernelGGL((lowrank_tn_kernel<RT>), grid, dim3(256), 0, st, (const uint16_t*)a, lda, (const uint16_t*)b, (int)L, \
+                                        (int)C, per, (float*)workspace)
+    if (R == 32) METIS_TN(1);
+    else if (R == 64) METIS_TN(2);
+    else METIS_TN(4);
+#undef METIS_TN
+    if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
+    const int64_t n = C * R;
+    hipLaunchKernelGGL(lowrank_tn_finish_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, (const float*)workspace, slices, (int)C,
+                       (int)R, out, out_dtype == METIS_DTYPE_F32, transpose);
+    return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
+}
+
+}  // namespace metis

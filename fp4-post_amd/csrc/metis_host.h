@@ -104,6 +104,13 @@ size_t lowrank_small_workspace_bytes(int64_t M, int64_t R, int64_t K);
 int lowrank_small(const void* x, int64_t ldx, const void* v, int64_t M, int64_t R, int64_t K, const void* s, void* xv, void* t,
                   void* workspace, size_t workspace_bytes, hipStream_t st);
 
+// rank-r products at training sizes (bf16, MFMA, one pass over the tall operand); lowrank_large.hip
+int lowrank_nt(const void* x, int64_t ldx, const void* v, int64_t M, int64_t R, int64_t K, const void* s, void* xv, void* t,
+               hipStream_t st);
+size_t lowrank_tn_workspace_bytes(int64_t L, int64_t C, int64_t R);
+int lowrank_tn(const void* a, int64_t lda, const void* b, int64_t L, int64_t C, int64_t R, void* out, int out_dtype, int transpose,
+               void* workspace, size_t workspace_bytes, hipStream_t st);
+
 int expand_f16(const void* codes, const void* scales, int64_t rows, int64_t cols, void* out, hipStream_t st);
 int gemm_expanded(const void* a_exp, const float* a_unit, const void* b_exp, const float* b_unit, int64_t M, int64_t N,
                   int64_t K, const void* t, const void* u, int64_t r, const void* bias, void* out, int out_dtype,

@@ -596,12 +596,12 @@ class _MetisFusedFunction(torch.autograd.Function):
         dy2 = _flat2d(dy).to(cd)
         x2 = _flat2d(x).to(cd)
         L, N = dy2.shape
-        # rank-r branch in bf16
-        g_t = torch.matmul(dy2, u.to(cd))                      # [L, r]
-        g_u = torch.matmul(dy2.T, xv * s.to(cd))               # [N, r]
+        # rank-r branch in bf16: one pass over dY for dY U, one for dY^T t, one over x for g_xv^T x
+        g_t = ops.lowrank_project(dy2, u.to(cd).T.contiguous())            # [L, r]
+        g_u = ops.lowrank_contract_tokens(dy2, xv * s.to(cd))               # [N, r]
         g_s = (g_t.float() * xv.float()).sum(dim=0)
         g_xv = g_t * s.to(cd)
-        g_v = torch.matmul(g_xv.T, x2)                         # [r, K]
+        g_v = ops.lowrank_contract_tokens(x2, g_xv, transpose=True)         # [r, K]
         # residual branch on re-quantized operands
         qg = F.q_backward_outputgrad
         if F._packed_backward_applies(L, N, dy2):

@@ -521,24 +521,56 @@ def linear_fwd(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None,
 def lowrank_project(x2: torch.Tensor, v: torch.Tensor, s: torch.Tensor | None = None):
     """Rank-r projection of the low-rank branch: xv = x2[M, K] . v[R, K]^T in bf16 (binary32 accumulation) and, with
     `s` [R], t = bf16(xv * s): returns xv or (xv, t).  Decode-sized batches (M < 256, R <= 256) run on the library's
-    split-K kernel; everything else is a torch matmul (the vendor library serves those shapes well)."""
+    split-K kernel, larger ones (R in 32 / 64 / 128) on its one-pass kernel; other shapes are a torch matmul."""
     M, K = x2.shape
     R = v.shape[0]
-    ok = (x2.is_cuda and x2.dtype == torch.bfloat16 and v.dtype == torch.bfloat16 and 0 < M < 256 and R % 32 == 0
-          and 0 < R <= 256 and K % 64 == 0 and v.shape[1] == K and x2.stride(1) == 1 and x2.stride(0) % 8 == 0
-          and (s is None or s.dtype == torch.bfloat16))
-    if not ok:
+    common = (x2.is_cuda and x2.dtype == torch.bfloat16 and v.dtype == torch.bfloat16 and M > 0 and K % 64 == 0 and v.shape[1] == K
+              and x2.stride(1) == 1 and x2.stride(0) % 8 == 0 and x2.data_ptr() % 16 == 0 and (s is None or s.dtype == torch.bfloat16))
+    small = common and M < 256 and R % 32 == 0 and 0 < R <= 256
+    large = common and M >= 256 and R in (32, 64, 128)
+    if not (small or large):
         xv = torch.matmul(x2, v.T)
         return xv if s is None else (xv, xv * s.to(xv.dtype))
     v = v.contiguous()
     L = load()
     xv = torch.empty(M, R, dtype=torch.bfloat16, device=x2.device)
     t = None if s is None else torch.empty_like(xv)
+    sp = None if s is None else s.contiguous().data_ptr()
+    if large:
+        rc = L.metis_lowrank_project_rows(x2.data_ptr(), x2.stride(0), v.data_ptr(), M, R, K, sp, xv.data_ptr(),
+                                          None if t is None else t.data_ptr(), _stream())
+        check(rc, "metis_lowrank_project_rows", (M, R, K))
+        return xv if s is None else (xv, t)
     ws = torch.empty(_lowrank_workspace_bytes(M, R, K), dtype=torch.uint8, device=x2.device)
-    rc = L.metis_lowrank_project(x2.data_ptr(), x2.stride(0), v.data_ptr(), M, R, K, None if s is None else s.contiguous().data_ptr(),
+    rc = L.metis_lowrank_project(x2.data_ptr(), x2.stride(0), v.data_ptr(), M, R, K, sp,
                                  xv.data_ptr(), None if t is None else t.data_ptr(), ws.data_ptr(), ws.numel(), _stream())
     check(rc, "metis_lowrank_project", (M, R, K))
     return xv if s is None else (xv, t)
+
+
+def lowrank_contract_tokens(a: torch.Tensor, b: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
+                            transpose: bool = False) -> torch.Tensor:
+    """sum_l a[l, C] b[l, R] -> [C, R] (or [R, C] with transpose): the rank-r products of the backward pass that
+    contract over tokens, bf16 operands, binary32 accumulation.  R in 32 / 64 / 128 on the library's kernel; other
+    shapes are a torch matmul."""
+    Lt, C = a.shape
+    R = b.shape[1]
+    ok = (a.is_cuda and a.dtype == torch.bfloat16 and b.dtype == torch.bfloat16 and b.shape[0] == Lt and Lt > 0 and R in (32, 64, 128)
+          and C % 8 == 0 and a.stride(1) == 1 and a.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0
+          and out_dtype in (torch.bfloat16, torch.float32))
+    if not ok:
+        out = torch.matmul(a.T, b).to(out_dtype)
+        return out.T.contiguous() if transpose else out
+    b = b.contiguous()
+    L = load()
+    out = torch.empty((R, C) if transpose else (C, R), dtype=out_dtype, device=a.device)
+    need = int(L.metis_lowrank_tokens_workspace_bytes(Lt, C, R))
+    ws = torch.empty(need, dtype=torch.uint8, device=a.device)
+    rc = L.metis_lowrank_contract_tokens(a.data_ptr(), a.stride(0), b.data_ptr(), Lt, C, R, out.data_ptr(),
+                                         DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16, int(transpose),
+                                         ws.data_ptr(), need, _stream())
+    check(rc, "metis_lowrank_contract_tokens", (Lt, C, R))
+    return out
 
 
 def linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.bfloat16,

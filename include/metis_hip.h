@@ -324,6 +324,31 @@ int metis_lowrank_project(const void *x, int64_t ldx, const void *v, int64_t M, 
                           void *stream);
 
 /*
+ * The same projection for training and prefill batches (any M; meant for M >= 256), one pass over x:
+ *     xv[M, R] = x[M, K] . v[R, K]^T,  t = bf16(xv * s) when t != NULL     (src/Metis/Metis/bitlinear.py:752-756)
+ * and, with v = U^T [r, N] and x = dY [L, N], the product dY . U of the backward pass.
+ *   R in {32, 64, 128}, K % 64 == 0, ldx % 8 == 0 (METIS_E_SHAPE otherwise); x, v 16-byte aligned; no workspace
+ */
+int metis_lowrank_project_rows(const void *x, int64_t ldx, const void *v, int64_t M, int64_t R, int64_t K,
+                               const void *s, void *xv, void *t, void *stream);
+
+/*
+ * The rank-r products of the backward pass that contract over tokens:
+ *     out[C, R] = sum_l a[l, C] * b[l, R]        bf16 operands, binary32 accumulation
+ * a = dY [L, N], b = (x V^T) * s  ->  gradient of U [N, r];   a = x [L, K], b = (dY U) * s, transpose = 1  ->
+ * gradient of V [r, K].  Replaces the torch matmuls autograd runs for ulinear / vlinear
+ * (src/Metis/Metis/bitlinear.py:752-757).  Tokens are cut into slices that run as separate workgroups; their
+ * binary32 partial results meet in the workspace and are added in slice order (deterministic).
+ *   R in {32, 64, 128}, C % 8 == 0, lda % 8 == 0 (METIS_E_SHAPE otherwise); a, b 16-byte aligned, b contiguous
+ *   out       [C, R], or [R, C] when transpose != 0, of out_dtype
+ *   workspace metis_lowrank_tokens_workspace_bytes(L, C, R) bytes, 16-byte aligned, no initialisation
+ */
+size_t metis_lowrank_tokens_workspace_bytes(int64_t L, int64_t C, int64_t R);
+int metis_lowrank_contract_tokens(const void *a, int64_t lda, const void *b, int64_t L, int64_t C, int64_t R,
+                                  void *out, int out_dtype, int transpose, void *workspace,
+                                  size_t workspace_bytes, void *stream);
+
+/*
  * One packed activation against several weight matrices in one call: the q/k/v (gate/up) projections of a
  * decoder layer, which the reference quantizes the activation once for (BitLinear._get_shared_quantized_input,
  * src/Metis/Metis/bitlinear.py:676-702) and then multiplies one by one.  Result i equals

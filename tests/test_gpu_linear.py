@@ -490,11 +490,11 @@ def test_lowrank_projection_for_decode_sized_batches(M, K, R):
     wide = torch.zeros(M, K + 64, dtype=torch.bfloat16, device="cuda")
     wide[:, :K] = x
     assert torch.equal(ops.lowrank_project(wide[:, :K], v), xv)
-    # large batches fall back to the vendor library with the same signature
+    # ranks that neither kernel takes fall back to the vendor library with the same signature
     big = torch.randn(300, 128, generator=g).bfloat16().cuda()
-    vb = torch.randn(32, 128, generator=g).bfloat16().cuda()
-    a, b = ops.lowrank_project(big, vb, s[:32])
-    assert torch.equal(a, big @ vb.T) and torch.equal(b, a * s[:32])
+    vb = torch.randn(16, 128, generator=g).bfloat16().cuda()
+    a, b = ops.lowrank_project(big, vb, s[:16])
+    assert torch.equal(a, big @ vb.T) and torch.equal(b, a * s[:16])
 
 
 def test_grouped_members_read_column_slices_of_a_stacked_projection():
@@ -514,3 +514,46 @@ def test_grouped_members_read_column_slices_of_a_stacked_projection():
     got = ops.linear_fwd_grouped(px, members, out_dtype=torch.float32)
     for (pw, t, u, _), y in zip(members, got):
         assert torch.equal(y, ops.linear_fwd(px, pw, t=t.contiguous(), u=u, out_dtype=torch.float32))
+
+
+@pytest.mark.parametrize("M,R,K", [(300, 32, 512), (4096, 64, 4096), (1000, 128, 1536), (8192, 64, 3584)])
+def test_rank_r_projection_at_training_sizes(M, R, K):
+    """xv = x V^T and t = bf16(xv * s) for 256 rows and more (one pass over x, MFMA): binary32 accumulation rounded once to
+    bf16, against double precision rounded the same way (only results on a rounding boundary can differ), and t exactly
+    the bf16 product of the kernel's own xv with s."""
+    from metis_hip import ops
+    g = torch.Generator().manual_seed(6000 + M)
+    x = synthetic_activation(80 + M, M, K).cuda()
+    v = (torch.randn(R, K, generator=g) / K ** 0.5).bfloat16().cuda()
+    s = (torch.rand(R, generator=g) * 4 + 0.1).bfloat16().cuda()
+    xv, t = ops.lowrank_project(x, v, s)
+    want = (x.double() @ v.double().T)
+    torch.cuda.synchronize()
+    assert xv.shape == (M, R) and xv.dtype == torch.bfloat16
+    assert rel_fro(xv.float().cpu(), want.bfloat16().float().cpu()) <= 5e-4
+    assert rel_fro(xv.float().cpu(), want.cpu()) <= 3e-3          # one bf16 rounding of the exact product
+    assert torch.equal(t, (xv.float() * s.float()).bfloat16())
+    only = ops.lowrank_project(x, v)
+    assert torch.equal(only, xv)
+    # a strided view (columns of a wider tensor) is read in place
+    wide = torch.cat((x, x), dim=1)
+    assert torch.equal(ops.lowrank_project(wide[:, :K], v), xv)
+
+
+@pytest.mark.parametrize("L,C,R", [(1000, 520, 32), (4096, 1536, 64), (4096, 8960, 32), (2048, 14336, 64), (777, 256, 128)])
+def test_rank_r_products_that_contract_over_tokens(L, C, R):
+    """out[C, R] = sum_l a[l, C] b[l, R] (gradients of U and, transposed, of V): token slices added in a fixed order,
+    against double precision; ragged token counts and column counts that are not multiples of the tile."""
+    from metis_hip import ops
+    g = torch.Generator().manual_seed(7000 + L)
+    a = (torch.randn(L, C, generator=g) * 1e-2).bfloat16().cuda()
+    b = torch.randn(L, R, generator=g).bfloat16().cuda()
+    want = a.double().T @ b.double()
+    got = ops.lowrank_contract_tokens(a, b, out_dtype=torch.float32)
+    got_t = ops.lowrank_contract_tokens(a, b, out_dtype=torch.bfloat16, transpose=True)
+    again = ops.lowrank_contract_tokens(a, b, out_dtype=torch.float32)
+    torch.cuda.synchronize()
+    assert got.shape == (C, R) and got_t.shape == (R, C)
+    assert rel_fro(got.cpu(), want.cpu()) <= 1e-5
+    assert torch.equal(got, again)                              # fixed summation order
+    assert torch.equal(got_t, got.bfloat16().T)
