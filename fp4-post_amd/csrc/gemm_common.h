@@ -39,6 +39,58 @@ __device__ __forceinline__ half2_t scale_pair(uint32_t byte)
     return __builtin_bit_cast(half2_t, h | (h << 16));
 }
 
+// Decode-sized GEMMs stream the packed weight rows straight from global memory into MFMA operands: lane l holds weight
+// row n0 + l % 32, and per step the two half-waves cover 64 C consecutive elements of K, lane group l / 32 taking a
+// contiguous run of 32 C elements (16 C bytes of codes, 2 C scale bytes).
+template <int C>
+struct RunRegs {
+    uint4 c[C];                  // 32*C codes
+    uint32_t sc[(C + 1) / 2];    // 2*C scale bytes
+};
+
+template <int C>
+__device__ __forceinline__ void load_run(RunRegs<C>& r, const uint8_t* codes, const uint8_t* scales)
+{
+#pragma unroll
+    for (int c = 0; c < C; ++c) r.c[c] = reinterpret_cast<const uint4*>(codes)[c];
+    if constexpr (C == 1) r.sc[0] = *reinterpret_cast<const uint16_t*>(scales);
+    else if constexpr (C == 2) r.sc[0] = *reinterpret_cast<const uint32_t*>(scales);
+    else {
+        const uint2 w = *reinterpret_cast<const uint2*>(scales);
+        r.sc[0] = w.x; r.sc[1] = w.y;
+    }
+}
+
+// MFMA operand m (8 elements) of a run
+template <int C>
+__device__ __forceinline__ half8_t run_operand(const RunRegs<C>& r, int m)
+{
+    const uint4 q = r.c[m >> 2];
+    const uint32_t w = (m & 3) == 0 ? q.x : (m & 3) == 1 ? q.y : (m & 3) == 2 ? q.z : q.w;
+    const uint32_t byte = (r.sc[m >> 3] >> (8 * ((m >> 1) & 3))) & 0xffu;
+    return __builtin_bit_cast(half8_t, expand8(w, scale_pair(byte)));
+}
+
+// One weight matrix of a grouped decode-sized call, and the group: the column tiles (32 columns each) of the members are
+// laid end to end.
+constexpr int kMaxGroupMembers = 4;
+struct SkinnyMember {
+    const uint8_t* b_codes;
+    const uint8_t* b_scales;
+    const float* b_unit;
+    const uint16_t* t;
+    const uint16_t* u;
+    const uint16_t* bias;
+    void* out;
+    float* part;                 // split-K partial sums of this member, nullptr when K is not split
+    int N, r, tile_end, bias_f32, ldt;
+};
+struct SkinnyGroup {
+    SkinnyMember m[kMaxGroupMembers];
+    int count, nsplit;
+    const float* center;         // mean mode: binary32 [K], see skinny_tile
+};
+
 constexpr int L_BM = 256, L_BN = 256, L_STRIDE = BK + LDS_PAD;   // large-tile kernels: 256 x 256 per workgroup
 
 // MFMA : VALU : LDS interleave requested from the scheduler for one K=16 sub-step of N_MFMA MFMAs

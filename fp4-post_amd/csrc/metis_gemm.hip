@@ -581,35 +581,6 @@ static int launch_large(const void* a_codes, const void* a_scales, const float* 
 // iteration multiplies elements [8m, 8m+8) of every lane's run, and the activation rows are
 // fetched with the same mapping.  Partial sums of the eight waves meet in LDS at the end.
 // ---------------------------------------------------------------------------------------------
-template <int C>
-struct RunRegs {
-    uint4 c[C];                  // 32*C codes
-    uint32_t sc[(C + 1) / 2];    // 2*C scale bytes
-};
-
-template <int C>
-__device__ __forceinline__ void load_run(RunRegs<C>& r, const uint8_t* codes, const uint8_t* scales)
-{
-#pragma unroll
-    for (int c = 0; c < C; ++c) r.c[c] = reinterpret_cast<const uint4*>(codes)[c];
-    if constexpr (C == 1) r.sc[0] = *reinterpret_cast<const uint16_t*>(scales);
-    else if constexpr (C == 2) r.sc[0] = *reinterpret_cast<const uint32_t*>(scales);
-    else {
-        const uint2 w = *reinterpret_cast<const uint2*>(scales);
-        r.sc[0] = w.x; r.sc[1] = w.y;
-    }
-}
-
-// MFMA operand m (8 elements) of a run
-template <int C>
-__device__ __forceinline__ half8_t run_operand(const RunRegs<C>& r, int m)
-{
-    const uint4 q = r.c[m >> 2];
-    const uint32_t w = (m & 3) == 0 ? q.x : (m & 3) == 1 ? q.y : (m & 3) == 2 ? q.z : q.w;
-    const uint32_t byte = (r.sc[m >> 3] >> (8 * ((m >> 1) & 3))) & 0xffu;
-    return __builtin_bit_cast(half8_t, expand8(w, scale_pair(byte)));
-}
-
 // CEN: the activation is a centred residual, X^ = 1 me^T + R (mean mode).  The workgroup's slice of the binary32
 // centre me is staged in LDS (in the reduction buffer, idle during the main loop) as binary16 pairs hi + lo
 // (22 significant bits, prescaled by 2^-4: |me| < 2^20) and enters as one more MFMA per step against the weight
@@ -761,24 +732,6 @@ __device__ __forceinline__ void skinny_tile(
 // Several weight matrices against ONE packed activation in one launch (q/k/v, gate/up): the column tiles of the
 // members are laid end to end along grid x.  A decode-sized k or v projection alone is 16 workgroups and costs a
 // whole launch latency; next to q it is free.
-constexpr int kMaxGroupMembers = 4;
-struct SkinnyMember {
-    const uint8_t* b_codes;
-    const uint8_t* b_scales;
-    const float* b_unit;
-    const uint16_t* t;
-    const uint16_t* u;
-    const uint16_t* bias;
-    void* out;
-    float* part;                 // split-K partial sums of this member, nullptr when K is not split
-    int N, r, tile_end, bias_f32, ldt;
-};
-struct SkinnyGroup {
-    SkinnyMember m[kMaxGroupMembers];
-    int count, nsplit;
-    const float* center;         // mean mode: binary32 [K], see skinny_tile
-};
-
 template <int TM, int C, int WAVES, int OUT_F32, int CEN = 0>
 __global__ __launch_bounds__(64 * WAVES) void gemm_nvfp4_skinny_grouped_kernel(
     const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const float* __restrict__ a_unit, int M, int K,
