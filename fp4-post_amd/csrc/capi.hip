@@ -144,6 +144,27 @@ int metis_nvfp4_expand_tiled(const void* codes, const void* scales, const float*
     return expand_xt(codes, scales, unit, rows, cols, mode, out, (hipStream_t)stream);
 }
 
+int metis_nvfp4_expand_tiled_rht(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, int mode,
+                                 uint32_t sign_mask, int rotate_back, int transpose, void* out, void* stream)
+{
+    if (transpose) return expand_xt_transposed(codes, scales, unit, rows, cols, mode, out, (hipStream_t)stream, rotate_back != 0, sign_mask);
+    return expand_xt(codes, scales, unit, rows, cols, mode, out, (hipStream_t)stream, rotate_back != 0, sign_mask);
+}
+
+int metis_nvfp4_quant_row_rht(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, uint32_t sign_mask, int sr, uint64_t seed,
+                              uint64_t offset, void* codes, void* scales, float* unit, void* workspace, size_t workspace_bytes,
+                              void* stream)
+{
+    return quantize_rht(x, rows, cols, ld, mode, sign_mask, sr != 0, seed, offset, codes, scales, unit, workspace, workspace_bytes,
+                        (hipStream_t)stream);
+}
+
+int metis_hadamard16(const void* x, int64_t rows, int64_t cols, int64_t ldx, int dtype, int inverse, uint32_t sign_mask, void* out,
+                     int64_t ldo, void* stream)
+{
+    return hadamard16(x, rows, cols, ldx, dtype, inverse, sign_mask, out, ldo, (hipStream_t)stream);
+}
+
 size_t metis_linear_tiled_workspace_bytes(int64_t M, int64_t N, int64_t K, int mode) { return gemm_xt_workspace_bytes(M, N, K, mode); }
 
 int metis_linear_fwd_tiled(const void* a_xt, const float* a_unit, const void* b_xt, const float* b_unit, int64_t M, int64_t N,

@@ -17,6 +17,7 @@
 // (eight whole cache lines), the LDS side is written linearly, and the swizzle that makes the MFMA fragment
 // reads (ds_read_b128, lane -> row) free of bank conflicts is already in the data.
 #include "gemm_common.h"
+#include "nvfp4_encode.h"
 #include <stdlib.h>
 
 namespace metis {
@@ -34,10 +35,16 @@ __host__ __device__ __forceinline__ int xt_swz(int q) { return ((q >> 2) & 1) | 
 //   PB16 = 1: bf16, the reference's dequantized value with every op rounded to bf16
 //             (src/Metis/Metis/quant.py:23-24, 32-35: bf16(bf16(e4m3 * unit) * v / 2)), unit included
 // ---------------------------------------------------------------------------------------------
-template <int PB16>
+//   RHT: the packed tensor is a rotated one (NV recipe); every block of 16 is rotated back after dequantization,
+//        (q H) / 16 * sign, as `_apply_hadamard_blocks(..., inverse=True)` does after the QDQ
+//        (src/Metis/Metis/bitlinear.py:395-405, 577-585).  The two lanes that hold the halves of a block exchange
+//        them and both run the 16-point butterflies.  PB16 = 0: the result is rounded to binary16 once (the sum of a
+//        block needs at most 12 significant bits); PB16 = 1: dequantized values and result rounded to bf16 as the
+//        reference's bf16 tensors are.
+template <int PB16, int RHT = 0>
 __global__ __launch_bounds__(256) void expand_xt_kernel(const uint32_t* __restrict__ codes, const uint8_t* __restrict__ scales,
                                                         const float* __restrict__ unit_p, uint4* __restrict__ out, int rows,
-                                                        int K, int row_tiles)
+                                                        int K, int row_tiles, uint32_t sign_mask)
 {
     typedef float float2_t __attribute__((ext_vector_type(2)));
     const int lane = threadIdx.x & 63;
@@ -52,11 +59,37 @@ __global__ __launch_bounds__(256) void expand_xt_kernel(const uint32_t* __restri
         const int kend = min(kt, kg * 8 + 8);
         for (int kb = kg * 8; kb < kend; ++kb) {
             uint4 v = make_uint4(0u, 0u, 0u, 0u);
-            if (live) {
+            if (live) {                                          // lane pairs (l, l ^ 1) share their row: both live or neither
                 const int k8 = kb * 4 + chunk;                   // index of the 8-element chunk inside the row
                 const uint32_t c = codes[(int64_t)row * (K / 8) + k8];
                 const uint32_t sb = scales[(int64_t)row * (K / 16) + (k8 >> 1)];
-                if constexpr (PB16 != 0) {
+                if constexpr (RHT != 0) {
+                    const float dq = PB16 ? rb(e4m3_value(sb) * unit) : e4m3_value(sb) * 0.00390625f;
+                    const float2_t p[4] = {__builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c, 1.0f, 0), __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c, 1.0f, 1),
+                                           __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c, 1.0f, 2), __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c, 1.0f, 3)};
+                    float mine[8], blk[kBlock];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) mine[j] = PB16 ? rb(p[j >> 1][j & 1] * dq) : p[j >> 1][j & 1] * dq;
+                    const int half = chunk & 1;                  // which half of the block this lane holds
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const float other = __shfl_xor(mine[j], 1);
+                        blk[j] = half ? other : mine[j];
+                        blk[8 + j] = half ? mine[j] : other;
+                    }
+                    hadamard16_inverse(blk, sign_mask);
+                    float o[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) o[j] = half ? blk[8 + j] : blk[j];
+                    if constexpr (PB16 != 0) {
+                        v.x = rb_pair(o[0], o[1]); v.y = rb_pair(o[2], o[3]); v.z = rb_pair(o[4], o[5]); v.w = rb_pair(o[6], o[7]);
+                    } else {
+                        const half2_t h0 = {(_Float16)o[0], (_Float16)o[1]}, h1 = {(_Float16)o[2], (_Float16)o[3]};
+                        const half2_t h2 = {(_Float16)o[4], (_Float16)o[5]}, h3 = {(_Float16)o[6], (_Float16)o[7]};
+                        v.x = __builtin_bit_cast(uint32_t, h0); v.y = __builtin_bit_cast(uint32_t, h1);
+                        v.z = __builtin_bit_cast(uint32_t, h2); v.w = __builtin_bit_cast(uint32_t, h3);
+                    }
+                } else if constexpr (PB16 != 0) {
                     const float dq = rb(e4m3_value(sb) * unit);
                     const float2_t p0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c, 1.0f, 0);
                     const float2_t p1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c, 1.0f, 1);
@@ -75,6 +108,61 @@ __global__ __launch_bounds__(256) void expand_xt_kernel(const uint32_t* __restri
     }
 }
 
+// Transposing variant: the packed [R, C] tensor (blocks along C) becomes the tiled operand [C, R], the layout a GEMM
+// that contracts over R (tokens) reads -- the wgrad operands dY^T and X^T and the dgrad operand W^T of
+// src/Metis/Metis/bitlinear.py:502-510.  An output tile (16 operand rows x 32 k) is one block of 16 from each of 32
+// source rows: lane l % 32 dequantizes (and, RHT, rotates back) one whole block in registers, the wave turns two
+// tiles through LDS and writes them as 2 x 1 KiB of consecutive bytes.  R % 32 == 0.
+template <int PB16, int RHT>
+__global__ __launch_bounds__(256) void expand_xt_t_kernel(const uint2* __restrict__ codes, const uint8_t* __restrict__ scales,
+                                                          const float* __restrict__ unit_p, uint4* __restrict__ out, int R, int C,
+                                                          uint32_t sign_mask)
+{
+    typedef float float2_t __attribute__((ext_vector_type(2)));
+    __shared__ __attribute__((aligned(16))) uint16_t turn[4][2][16][40];       // [wave][tile][operand row][k], 80-byte rows
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5, sl = lane & 31;
+    const int cb_n = C / 16, kt = R / 32, kpairs = (kt + 1) / 2;
+    const int64_t nunits = (int64_t)cb_n * kpairs;
+    const float unit = PB16 ? *unit_p : 0.0f;
+    for (int64_t un = (int64_t)blockIdx.x * 4 + wave; un < nunits; un += (int64_t)gridDim.x * 4) {
+        const int cb = (int)(un % cb_n), kp = (int)(un / cb_n);              // consecutive waves: consecutive blocks of a row
+        const int kb = kp * 2 + half;
+        if (kb < kt) {
+            const int r = kb * 32 + sl;
+            const uint2 c = codes[(int64_t)r * cb_n + cb];
+            const uint32_t sb = scales[(int64_t)r * cb_n + cb];
+            const float dq = PB16 ? rb(e4m3_value(sb) * unit) : e4m3_value(sb) * 0.00390625f;
+            float blk[kBlock];
+            const float2_t p[8] = {__builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 0), __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 1),
+                                   __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 2), __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 3),
+                                   __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 0), __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 1),
+                                   __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 2), __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 3)};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) { blk[2 * j] = p[j][0] * dq; blk[2 * j + 1] = p[j][1] * dq; }
+            if constexpr (PB16 != 0) {
+#pragma unroll
+                for (int j = 0; j < kBlock; ++j) blk[j] = rb(blk[j]);
+            }
+            if constexpr (RHT != 0) hadamard16_inverse(blk, sign_mask);
+#pragma unroll
+            for (int j = 0; j < kBlock; ++j)
+                turn[wave][half][j][sl] = PB16 ? (uint16_t)bf16_bits(blk[j]) : __builtin_bit_cast(uint16_t, (_Float16)blk[j]);
+        }
+        __builtin_amdgcn_s_waitcnt(0xc07f);                      // LDS writes of this wave are done (lgkmcnt 0)
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int tl = 0; tl < 2; ++tl) {
+            if (kp * 2 + tl < kt) {
+                const int q = lane >> 2, chunk = (lane & 3) ^ xt_swz(q);
+                const uint4 v = *reinterpret_cast<const uint4*>(&turn[wave][tl][q][chunk * 8]);
+                out[((int64_t)cb * kt + kp * 2 + tl) * 64 + lane] = v;
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
 size_t expand_xt_bytes(int64_t rows, int64_t cols)
 {
     if (rows <= 0 || cols <= 0) return 0;
@@ -82,9 +170,9 @@ size_t expand_xt_bytes(int64_t rows, int64_t cols)
 }
 
 int expand_xt(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, int mode, void* out,
-              hipStream_t st)
+              hipStream_t st, int rht, uint32_t sign_mask)
 {
-    if (rows < 0 || cols < 0) return METIS_E_ARG;
+    if (rows < 0 || cols < 0 || sign_mask > 0xffffu) return METIS_E_ARG;
     if (mode == METIS_MODE_P32_F32) mode = METIS_MODE_P32;
     if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) return METIS_E_ARG;
     if (cols % kBlock) return METIS_E_SHAPE;
@@ -97,12 +185,34 @@ int expand_xt(const void* codes, const void* scales, const float* unit, int64_t 
     int64_t g = (units + 3) / 4;
     const int64_t cap = (int64_t)device_cus() * 16;
     if (g > cap) g = cap;
-    if (mode == METIS_MODE_PB16)
-        hipLaunchKernelGGL(expand_xt_kernel<1>, dim3((unsigned)g), dim3(256), 0, st, (const uint32_t*)codes, (const uint8_t*)scales,
-                           unit, (uint4*)out, (int)rows, (int)cols, row_tiles);
-    else
-        hipLaunchKernelGGL(expand_xt_kernel<0>, dim3((unsigned)g), dim3(256), 0, st, (const uint32_t*)codes, (const uint8_t*)scales,
-                           unit, (uint4*)out, (int)rows, (int)cols, row_tiles);
+#define METIS_EX(P, R) hipLaunchKernelGGL((expand_xt_kernel<P, R>), dim3((unsigned)g), dim3(256), 0, st, (const uint32_t*)codes, \
+                                          (const uint8_t*)scales, unit, (uint4*)out, (int)rows, (int)cols, row_tiles, sign_mask)
+    if (mode == METIS_MODE_PB16) { if (rht) METIS_EX(1, 1); else METIS_EX(1, 0); }
+    else { if (rht) METIS_EX(0, 1); else METIS_EX(0, 0); }
+#undef METIS_EX
+    return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
+}
+
+int expand_xt_transposed(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, int mode, void* out,
+                         hipStream_t st, int rht, uint32_t sign_mask)
+{
+    if (rows < 0 || cols < 0 || sign_mask > 0xffffu) return METIS_E_ARG;
+    if (mode == METIS_MODE_P32_F32) mode = METIS_MODE_P32;
+    if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) return METIS_E_ARG;
+    if (cols % kBlock || rows % 32) return METIS_E_SHAPE;
+    if (rows > INT32_MAX - 32 || cols > INT32_MAX) return METIS_E_ARG;
+    if (rows == 0 || cols == 0) return METIS_OK;
+    if (!codes || !scales || !out || ((uintptr_t)codes % 8) || ((uintptr_t)out % 16)) return METIS_E_ARG;
+    if (mode == METIS_MODE_PB16 && !unit) return METIS_E_ARG;
+    const int64_t units = (cols / 16) * ((rows / 32 + 1) / 2);
+    int64_t g = (units + 3) / 4;
+    const int64_t cap = (int64_t)device_cus() * 16;
+    if (g > cap) g = cap;
+#define METIS_EXT(P, R) hipLaunchKernelGGL((expand_xt_t_kernel<P, R>), dim3((unsigned)g), dim3(256), 0, st, (const uint2*)codes, \
+                                           (const uint8_t*)scales, unit, (uint4*)out, (int)rows, (int)cols, sign_mask)
+    if (mode == METIS_MODE_PB16) { if (rht) METIS_EXT(1, 1); else METIS_EXT(1, 0); }
+    else { if (rht) METIS_EXT(0, 1); else METIS_EXT(0, 0); }
+#undef METIS_EXT
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 

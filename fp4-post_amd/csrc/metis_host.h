@@ -93,6 +93,12 @@ size_t gemm_grouped_workspace_bytes(int64_t M, int64_t K, const GemmMember* memb
 // bytes of split-K scratch gemm_nvfp4 can use for this shape on the current device (0: it would not split)
 size_t gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
+// NV recipe (nvfp4_quant.hip): rotate tiles of 16 along the last dimension and quantize the rotated tensor; the rotation alone
+int quantize_rht(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, uint32_t sign_mask, bool sr, uint64_t seed,
+                 uint64_t offset, void* codes, void* scales, float* unit, void* workspace, size_t workspace_bytes, hipStream_t st);
+int hadamard16(const void* x, int64_t rows, int64_t cols, int64_t ldx, int dtype, int inverse, uint32_t sign_mask, void* out,
+               int64_t ldo, hipStream_t st);
+
 // me[c] = mean over rows of x[:, c] (binary32 accumulation); nvfp4_gemv.hip
 size_t column_mean_workspace_bytes(int64_t cols);
 int column_mean(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_f32, void* out, int out_bf16, void* workspace,
@@ -119,7 +125,10 @@ int gemm_expanded(const void* a_exp, const float* a_unit, const void* b_exp, con
 // tiled 16-bit expansion of a packed tensor and the pipelined GEMM that consumes it; metis_gemm_pipe.hip
 size_t expand_xt_bytes(int64_t rows, int64_t cols);
 int expand_xt(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, int mode, void* out,
-              hipStream_t st);
+              hipStream_t st, int rht = 0, uint32_t sign_mask = 0);
+// the tiled operand [cols, rows] (contraction over the packed tensor's rows); rows % 32 == 0
+int expand_xt_transposed(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, int mode, void* out,
+                         hipStream_t st, int rht, uint32_t sign_mask);
 size_t gemm_xt_workspace_bytes(int64_t M, int64_t N, int64_t K, int mode);
 int gemm_xt(const void* a_xt, const float* a_unit, const void* b_xt, const float* b_unit, int64_t M, int64_t N, int64_t K,
             const void* t, const void* u, int64_t r, const void* bias, int bias_f32, void* out, int out_dtype, int mode,

@@ -245,6 +245,35 @@ __device__ __forceinline__ void unpack16(const uint4 a, const uint4 b, float (&v
     for (int j = 0; j < 8; ++j) { v[2 * j] = bf16_lo(w[j]); v[2 * j + 1] = bf16_hi(w[j]); }
 }
 
+// Tiled random Hadamard rotation of the NV recipe on one tile of 16 in registers (the tile is the scale block).
+// Forward: (v * sign) H, src/Metis/Metis/bitlinear.py:199-202; inverse: (v H) / 16 * sign, bitlinear.py:195-197, with H the
+// Sylvester matrix (75-96) and sign the shared vector of 126-137, here a bit mask (bit j set: sign[j] = -1).
+// binary32 sums in butterfly order; sums of bf16 values are exact whenever their exponents are within 12 of each other.
+__device__ __forceinline__ void hadamard16_butterflies(float (&v)[kBlock])
+{
+#pragma unroll
+    for (int h = 1; h < kBlock; h <<= 1)
+#pragma unroll
+        for (int j = 0; j < kBlock; ++j)
+            if ((j & h) == 0) {
+                const float a = v[j], b = v[j + h];
+                v[j] = a + b;
+                v[j + h] = a - b;
+            }
+}
+__device__ __forceinline__ void hadamard16_forward(float (&v)[kBlock], uint32_t sign_mask)
+{
+#pragma unroll
+    for (int j = 0; j < kBlock; ++j) v[j] = __uint_as_float(__float_as_uint(v[j]) ^ (((sign_mask >> j) & 1u) << 31));
+    hadamard16_butterflies(v);
+}
+__device__ __forceinline__ void hadamard16_inverse(float (&v)[kBlock], uint32_t sign_mask)
+{
+    hadamard16_butterflies(v);
+#pragma unroll
+    for (int j = 0; j < kBlock; ++j) v[j] = __uint_as_float(__float_as_uint(v[j] * 0.0625f) ^ (((sign_mask >> j) & 1u) << 31));
+}
+
 // publish the workgroup's maximum block-maximum (non-negative floats order like their bit patterns)
 __device__ __forceinline__ void publish_group_max(float m, uint32_t* ws_gmax)
 {

@@ -63,13 +63,18 @@ __global__ __launch_bounds__(256) void quant_codes_contig_kernel(const uint4* __
     publish_group_max(gmax, ws_gmax);
 }
 
-template <int MODE, bool SR, bool WIDE = false>
+// HAD: every block is rotated first (NV recipe, hadamard16_forward): the rotated tensor is what gets quantized, as in
+// `_quantize_wgrad_operand` and `_get_quantized_weight` of src/Metis/Metis/bitlinear.py:395-405, 577-585.  In bf16
+// arithmetic the rotated values are rounded to bf16 (the reference's rotation returns the input dtype); in binary32
+// arithmetic they are binary32 values that need not be bf16 values, hence WIDE.
+template <int MODE, bool SR, bool WIDE = false, bool HAD = false>
 __global__ __launch_bounds__(256) void quant_codes_kernel(
     const void* __restrict__ xv, uint32_t rows, uint32_t cols, int64_t ld, const void* __restrict__ noise,
     uint64_t seed, uint64_t offset, uint2* __restrict__ codes, void* __restrict__ ws_amax_v,
-    uint32_t* __restrict__ ws_gmax, uint32_t nblocks, int in_f32, const void* __restrict__ center)
+    uint32_t* __restrict__ ws_gmax, uint32_t nblocks, int in_f32, const void* __restrict__ center, uint32_t sign_mask)
 {
     static_assert(!WIDE || MODE == 0, "binary32 values imply binary32 arithmetic");
+    static_assert(!HAD || WIDE || MODE == 1, "rotated binary32 values are not bf16 values");
     const uint16_t* __restrict__ x = static_cast<const uint16_t*>(xv);
     uint16_t* __restrict__ ws_amax = static_cast<uint16_t*>(ws_amax_v);
     float gmax = 0.0f;
@@ -102,6 +107,13 @@ __global__ __launch_bounds__(256) void quant_codes_kernel(
                 unpack16(cp[0], cp[1], cv);
 #pragma unroll
                 for (int j = 0; j < kBlock; ++j) v[j] = rb(v[j] - cv[j]);
+            }
+        }
+        if constexpr (HAD) {
+            hadamard16_forward(v, sign_mask);
+            if constexpr (MODE == 1) {
+#pragma unroll
+                for (int j = 0; j < kBlock; ++j) v[j] = rb(v[j]);
             }
         }
         if (SR && noise) {
@@ -550,11 +562,12 @@ static int launch_fused(const void* x, void* codes, void* scales, float* unit, c
     return rc;
 }
 
-template <int MODE, bool SR, bool COL, bool WIDE = false>
+template <int MODE, bool SR, bool COL, bool WIDE = false, bool HAD = false>
 static int launch_quant(const void* x, int64_t rows, int64_t cols, int64_t ld, const void* noise, uint64_t seed,
                         uint64_t offset, void* codes, void* scales, float* unit, const Workspace& ws, hipStream_t st,
-                        int in_f32 = 0, const void* center = nullptr)
+                        int in_f32 = 0, const void* center = nullptr, uint32_t sign_mask = 0)
 {
+    static_assert(!HAD || !COL, "the rotation runs along the last dimension, as the row blocks do");
     const uint32_t nblocks = (uint32_t)(rows * cols / kBlock);
     if constexpr (COL) {
         const uint32_t tiles_r = (uint32_t)((rows / kBlock + kColTileBlocks - 1) / kColTileBlocks);
@@ -570,15 +583,16 @@ static int launch_quant(const void* x, int64_t rows, int64_t cols, int64_t ld, c
         return launch_scales(WIDE ? METIS_MODE_P32_F32 : MODE, ws, (uint32_t)g, scales, unit, nblocks, st);
     } else {
         const int g1 = grid_for(nblocks);
-        if constexpr (!SR && !WIDE) {
+        if constexpr (!SR && !WIDE && !HAD) {
             if (!center && ld == cols) {
                 hipLaunchKernelGGL((quant_codes_contig_kernel<MODE>), dim3(g1), dim3(256), 0, st, (const uint4*)x, (uint2*)codes,
                                    ws.amax, ws.gmax, nblocks);
                 return launch_scales(MODE, ws, (uint32_t)g1, scales, unit, nblocks, st);
             }
         }
-        hipLaunchKernelGGL((quant_codes_kernel<MODE, SR, WIDE>), dim3(g1), dim3(256), 0, st, x, (uint32_t)rows,
-                           (uint32_t)cols, ld, noise, seed, offset, (uint2*)codes, (void*)ws.amax, ws.gmax, nblocks, in_f32, center);
+        hipLaunchKernelGGL((quant_codes_kernel<MODE, SR, WIDE, HAD>), dim3(g1), dim3(256), 0, st, x, (uint32_t)rows,
+                           (uint32_t)cols, ld, noise, seed, offset, (uint2*)codes, (void*)ws.amax, ws.gmax, nblocks, in_f32, center,
+                           sign_mask);
         return launch_scales(WIDE ? METIS_MODE_P32_F32 : MODE, ws, (uint32_t)g1, scales, unit, nblocks, st);
     }
 }
@@ -624,6 +638,87 @@ int quantize(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, bo
         else { if (!col) METIS_Q(1, true, false); else METIS_Q(1, true, true); }
     }
 #undef METIS_Q
+}
+
+// ---------------------------------------------------------------------------------------------
+// NV recipe: rotate every tile of 16 along the last dimension, then quantize the rotated tensor (row blocks = tiles),
+// in one pass over x.  Round to nearest, or stochastic rounding on the library's own stream.
+// ---------------------------------------------------------------------------------------------
+int quantize_rht(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, uint32_t sign_mask, bool sr, uint64_t seed,
+                 uint64_t offset, void* codes, void* scales, float* unit, void* workspace, size_t workspace_bytes, hipStream_t st)
+{
+    if (rows < 0 || cols < 0 || ld < cols || sign_mask > 0xffffu) return METIS_E_ARG;
+    if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16 && mode != METIS_MODE_P32_F32) return METIS_E_ARG;
+    const bool f32in = mode == METIS_MODE_P32_F32;
+    if (cols % kBlock) return METIS_E_SHAPE;
+    if (rows == 0 || cols == 0) return METIS_OK;
+    if (!x || !codes || !scales || !unit) return METIS_E_ARG;
+    if (rows * cols / kBlock >= (int64_t)1 << 31) return METIS_E_ARG;
+    if ((ld % (f32in ? 4 : 8)) || ((uintptr_t)x % 16)) return METIS_E_ARG;
+    if (((uintptr_t)codes % 8) || ((uintptr_t)scales % 8)) return METIS_E_ARG;
+    Workspace ws;
+    if (const int rc = carve_workspace(workspace, workspace_bytes, rows, cols, &ws)) return rc;
+#define METIS_QH(M, S, W) return launch_quant<M, S, false, W, true>(x, rows, cols, ld, nullptr, seed, offset, codes, scales, unit, ws, st, \
+                                                                    f32in, nullptr, sign_mask)
+    if (mode == METIS_MODE_PB16) { if (sr) METIS_QH(1, true, false); else METIS_QH(1, false, false); }
+    if (sr) METIS_QH(0, true, true); else METIS_QH(0, false, true);
+#undef METIS_QH
+}
+
+// The rotation alone, bf16 or binary32 in and out (same dtype): out = rotate(x) or its inverse, tile by tile.
+template <int F32, int INVERSE>
+__global__ __launch_bounds__(256) void hadamard16_kernel(const void* __restrict__ xv, void* __restrict__ outv, int64_t ntiles,
+                                                         int64_t tiles_per_row, int64_t ldx, int64_t ldo, uint32_t sign_mask)
+{
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < ntiles; i += (int64_t)gridDim.x * 256) {
+        const int64_t row = i / tiles_per_row, cb = i - row * tiles_per_row;
+        float v[kBlock];
+        if (F32) {
+            const float4* p = reinterpret_cast<const float4*>(static_cast<const float*>(xv) + row * ldx + cb * kBlock);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const float4 f = p[c];
+                v[4 * c] = f.x; v[4 * c + 1] = f.y; v[4 * c + 2] = f.z; v[4 * c + 3] = f.w;
+            }
+        } else {
+            const uint4* p = reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(xv) + row * ldx + cb * kBlock);
+            unpack16(p[0], p[1], v);
+        }
+        if (INVERSE) hadamard16_inverse(v, sign_mask);
+        else hadamard16_forward(v, sign_mask);
+        if (F32) {
+            float4* o = reinterpret_cast<float4*>(static_cast<float*>(outv) + row * ldo + cb * kBlock);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) o[c] = make_float4(v[4 * c], v[4 * c + 1], v[4 * c + 2], v[4 * c + 3]);
+        } else {
+            uint32_t w[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) w[j] = bf16_bits(v[2 * j]) | (bf16_bits(v[2 * j + 1]) << 16);
+            uint4* o = reinterpret_cast<uint4*>(static_cast<uint16_t*>(outv) + row * ldo + cb * kBlock);
+            o[0] = make_uint4(w[0], w[1], w[2], w[3]);
+            o[1] = make_uint4(w[4], w[5], w[6], w[7]);
+        }
+    }
+}
+
+int hadamard16(const void* x, int64_t rows, int64_t cols, int64_t ldx, int dtype, int inverse, uint32_t sign_mask, void* out,
+               int64_t ldo, hipStream_t st)
+{
+    if (rows < 0 || cols < 0 || ldx < cols || ldo < cols || sign_mask > 0xffffu) return METIS_E_ARG;
+    if (dtype != METIS_DTYPE_BF16 && dtype != METIS_DTYPE_F32) return METIS_E_ARG;
+    if (cols % kBlock) return METIS_E_SHAPE;
+    if (rows == 0 || cols == 0) return METIS_OK;
+    const int al = dtype == METIS_DTYPE_F32 ? 4 : 8;
+    if (!x || !out || (ldx % al) || (ldo % al) || ((uintptr_t)x % 16) || ((uintptr_t)out % 16)) return METIS_E_ARG;
+    const int64_t tpr = cols / kBlock, ntiles = rows * tpr;
+    int64_t g = (ntiles + 255) / 256;
+    const int64_t cap = (int64_t)device_cus() * 16;
+    if (g > cap) g = cap;
+#define METIS_H(F, I) hipLaunchKernelGGL((hadamard16_kernel<F, I>), dim3((unsigned)g), dim3(256), 0, st, x, out, ntiles, tpr, ldx, ldo, sign_mask)
+    if (dtype == METIS_DTYPE_F32) { if (inverse) METIS_H(1, 1); else METIS_H(1, 0); }
+    else { if (inverse) METIS_H(0, 1); else METIS_H(0, 0); }
+#undef METIS_H
+    return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 
 // ---------------------------------------------------------------------------------------------

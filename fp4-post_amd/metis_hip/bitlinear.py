@@ -145,6 +145,20 @@ class LinearLowbitFunction(torch.autograd.Function):
         return F._hadamard_sign_cache[key]
 
     @staticmethod
+    def _hadamard_mask() -> int:
+        """The shared sign vector of the 16-wide rotation as a bit mask for the kernels: bit j set <=> sign[j] = -1."""
+        signs = LinearLowbitFunction._get_hadamard_sign(16, torch.device("cpu"), torch.float32)
+        return sum(1 << j for j in range(16) if float(signs[j]) < 0)
+
+    @staticmethod
+    def _nv_on_kernels() -> bool:
+        """NV recipe with the tile the scale blocks have: rotation, quantizer and GEMM operands stay on the library's
+        kernels (a rotated tile is one block of 16).  hadamard_backend "torch_gemm" asks for the reference's portable
+        formula instead: rotation as a small GEMM, dequantized tensors, torch matmuls."""
+        F = LinearLowbitFunction
+        return F.enable_nv_recipe and int(F.hadamard_tile_size) == 16 and F.hadamard_backend == "auto"
+
+    @staticmethod
     def _apply_hadamard_blocks(value: torch.Tensor, inverse: bool = False) -> torch.Tensor:
         """Rotate every tile of `hadamard_tile_size` consecutive elements of the last dimension:
         forward (x * S) H, inverse (y H) / d * S (reference 125-211).  All tiles go through one
@@ -165,6 +179,9 @@ class LinearLowbitFunction(torch.autograd.Function):
         if F.hadamard_backend == "dao_cuda":
             raise RuntimeError("Hadamard backend dao_cuda was requested but fast_hadamard_transform is unavailable "
                                "in this build; use 'auto' or 'torch_gemm'")
+        if tile == 16 and value.is_cuda and value.dtype in (torch.float32, torch.bfloat16) and F.hadamard_backend == "auto":
+            # in-register butterflies, one pass over the tensor; "torch_gemm" keeps the reference's fallback formula
+            return ops.hadamard16(value, F._hadamard_mask(), inverse=inverse)
         work_dtype = torch.float32 if value.dtype in (torch.float16, torch.bfloat16) else value.dtype
         h = F._get_hadamard(tile, value.device, work_dtype)
         signs = F._get_hadamard_sign(tile, value.device, work_dtype)
@@ -302,7 +319,7 @@ class LinearLowbitFunction(torch.autograd.Function):
         """Packed activation when a kernel path applies (direct: PackedNVFP4; mean mode: CenteredNVFP4), else
         the dequantized tensor."""
         F = LinearLowbitFunction
-        if not F.enable_nv_recipe and _packable(input_, F.q_forward_input):
+        if (not F.enable_nv_recipe or F._nv_on_kernels()) and _packable(input_, F.q_forward_input):
             if not F.enable_activation_svd:
                 # the kernels read bf16 values and take the arithmetic as a mode: no upcast copy of a bf16 tensor
                 return F.q_forward_input.pack(_flat2d(input_), arith=F.compute_dtype)
@@ -369,6 +386,38 @@ class LinearLowbitFunction(torch.autograd.Function):
         return gx, ops.linear_fwd(p_dyt, p_xt, t=t, u=u, out_dtype=gw_dtype)
 
     @staticmethod
+    def _packed_grads_nv(dy2, x2, pw, gx_dtype, gw_dtype):
+        """(grad_input, grad_weight) of the NV recipe (reference 443-513 with 395-405, 495-501) without leaving the
+        packed kernels.  The reference rotates dY and the saved (already quantized) input tile by tile along their
+        last dimension, quantizes, dequantizes and rotates back, and multiplies the results:
+            dY~ = rot^-1(QDQ(rot(dY))),  X~ = rot^-1(QDQ(rot(QDQ(x)))),  gW = dY~^T X~,  gX = dY~ W~
+        with W~ the forward weight (577-585).  Here rot + quantizer is one kernel, and every GEMM operand is the tiled
+        16-bit expansion of a packed tensor with the rotation back applied block by block on the way: dY~ [L, N] and
+        W~^T [K, N] for the input gradient (contraction over N), dY~^T [N, L] and X~^T [K, L] for the weight gradient
+        (contraction over tokens; the expansion transposes).  Quantization blocks run along the last dimension, as the
+        reference's do."""
+        F = LinearLowbitFunction
+        cd = F.compute_dtype
+        mask = pw.rht
+        gmode = ops.MODE_PB16 if (cd != torch.float32 and F.reference_rounding and pw.mode == ops.MODE_PB16) else ops.MODE_P32
+        L, N = dy2.shape
+        K = x2.shape[1]
+        pad = (-L) % 32                                        # the token contraction runs in steps of 32: zero rows add nothing
+        if pad:
+            dy2 = torch.cat((dy2, dy2.new_zeros(pad, N)), dim=0)
+            x2 = torch.cat((x2, x2.new_zeros(pad, K)), dim=0)
+        p_dy = F.q_backward_outputgrad.pack(dy2, arith=cd, rht=mask)
+        xq = F.q_forward_input.pack(x2, arith=cd).dequantize(torch.float32 if cd == torch.float32 else torch.bfloat16)
+        p_x = F.q_backward_input.pack(xq, arith=cd, rht=mask)
+        a_dy = ops.expand_tiled(p_dy, cache=False, mode=gmode)
+        b_wt = ops.expand_tiled_transposed(pw, cache=pw.persistent, mode=gmode)
+        gx = ops.gemm_tiled(a_dy, p_dy.unit, b_wt, pw.unit, L + pad, K, N, mode=gmode, out_dtype=gx_dtype)
+        a_dyt = ops.expand_tiled_transposed(p_dy, mode=gmode)
+        b_xt = ops.expand_tiled_transposed(p_x, mode=gmode)
+        gw = ops.gemm_tiled(a_dyt, p_dy.unit, b_xt, p_x.unit, N, K, L + pad, mode=gmode, out_dtype=gw_dtype)
+        return (gx[:L] if pad else gx), gw
+
+    @staticmethod
     def _packed_backward_applies(L: int, N: int, grad_output: torch.Tensor) -> bool:
         """Backward on the packed kernels.  Any token count L qualifies (ragged counts are padded inside
         _packed_grads); the output width N is the contraction of the input gradient and has to be a multiple of 32.
@@ -379,6 +428,8 @@ class LinearLowbitFunction(torch.autograd.Function):
         ok = N % 32 == 0 and L > 0 and grad_output.dtype in (torch.float32, torch.bfloat16)
         if ok and F.enable_backward_svd:
             ok = F.backward_lowrank_svd > 0 and F._mean_mode_packable()
+        if ok and F.enable_nv_recipe:
+            ok = F._nv_on_kernels()
         if not ok and grad_output.is_cuda:
             _warn_generic_path(f"backward with {L} tokens, {N} output features, dtype {grad_output.dtype}, "
                                f"metis_mode={F.metis_mode!r}, nv_recipe={F.enable_nv_recipe}")
@@ -452,11 +503,14 @@ class LinearLowbitFunction(torch.autograd.Function):
                 dy2, x2 = _flat2d(grad_output), _flat2d(input_)
                 if cd != torch.float32:
                     dy2, x2 = dy2.to(torch.bfloat16), x2.to(torch.bfloat16)
+                gx_dtype = input_.dtype if input_.dtype in (torch.float32, torch.bfloat16) else torch.float32
+                gw_dtype = torch.bfloat16 if ctx.weight_ref.dtype == torch.bfloat16 else torch.float32
+                if ctx.pw.rht is not None:
+                    gx, gw = F._packed_grads_nv(dy2, x2, ctx.pw, gx_dtype, gw_dtype)
+                    return gx.reshape(*ctx.lead, gx.shape[-1]), gw, grad_bias, None, None
                 pw_col = ctx.pw.transposed                    # lives as long as the (possibly cached) packed weight
                 if pw_col is None:
                     pw_col = ctx.pw.transposed = F.q_forward_weight.pack(ctx.weight_ref, col=True, arith=cd)
-                gx_dtype = input_.dtype if input_.dtype in (torch.float32, torch.bfloat16) else torch.float32
-                gw_dtype = torch.bfloat16 if ctx.weight_ref.dtype == torch.bfloat16 else torch.float32
                 gx, gw = F._packed_grads(dy2, x2, pw_col, ctx.center, gx_dtype, gw_dtype)
                 return gx.reshape(*ctx.lead, gx.shape[-1]), gw, grad_bias, None, None
             grad_output = grad_output.to(F.compute_dtype)
@@ -516,7 +570,7 @@ class LinearLowbit(nn.Module):
     def forward(self, input, quantized_input=None):
         F = LinearLowbitFunction
         bias_compute = self.bias.to(self.compute_dtype) if self.bias is not None else None
-        if not F.enable_nv_recipe and _packable(self.weight, F.q_forward_weight) and self.weight.shape[0] % 4 == 0:
+        if (not F.enable_nv_recipe or F._nv_on_kernels()) and _packable(self.weight, F.q_forward_weight) and self.weight.shape[0] % 4 == 0:
             # kernel path: packed straight from the stored parameter in compute_dtype arithmetic, so a cache hit
             # costs no pass over the weight at all
             quantized_weight = self._get_quantized_weight(self.weight, arith=self.compute_dtype)
@@ -535,7 +589,11 @@ class LinearLowbit(nn.Module):
             cached_key, cached = self._quantized_weight_cache
             if cached_key == key:
                 return cached
-        if F.enable_nv_recipe:                                             # reference 577-585
+        if F._nv_on_kernels() and arith is not None and _packable(weight_compute, F.q_forward_weight) and weight_compute.shape[0] % 4 == 0:
+            # reference 577-585 on the kernels: the packed tensor holds the ROTATED weight's codes, rotated in the
+            # quantizer's registers; whoever reads it (tiled GEMM operand, dequantize) rotates back
+            q = F.q_forward_weight.pack(weight_compute, arith=arith, rht=F._hadamard_mask())
+        elif F.enable_nv_recipe:                                           # reference 577-585
             q = F._apply_hadamard_blocks(weight_compute, inverse=False)
             q = F._apply_hadamard_blocks(F.q_forward_weight.quantize_dequantize(q), inverse=True)
         elif _packable(weight_compute, F.q_forward_weight) and weight_compute.shape[0] % 4 == 0:

@@ -36,6 +36,9 @@ class PackedNVFP4:
     tiled_pb16: torch.Tensor | None = None    # the reference's bf16 dequantized values in the same layout (bf16 arithmetic)
     transposed: "PackedNVFP4 | None" = None   # cached column-blocked packing of the same source tensor (dgrad operand)
     persistent: bool = False                  # lives across calls (a cached weight): worth keeping its tiled expansion
+    rht: int | None = None                    # NV recipe: the packed values are those of the ROTATED tensor (sign mask of the rotation)
+    tiled_t: torch.Tensor | None = None       # tiled expansion of the transposed tensor (contraction over this tensor's rows)
+    tiled_t_pb16: torch.Tensor | None = None
 
     def dequantize(self, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
         return dequantize(self, dtype)
@@ -177,7 +180,43 @@ def dequantize(p: PackedNVFP4, dtype: torch.dtype = torch.bfloat16) -> torch.Ten
                                     p.mode, out.data_ptr(), DTYPE_F32 if dtype == torch.float32 else DTYPE_BF16,
                                     _stream())
     check(rc, "metis_nvfp4_dequant", (p.rows, p.cols))
+    if p.rht is not None:                     # packed in the rotated domain: back to the tensor's own
+        out = hadamard16(out, p.rht, inverse=True)
     return out
+
+
+def hadamard16(x: torch.Tensor, sign_mask: int, inverse: bool = False) -> torch.Tensor:
+    """Tiled random Hadamard rotation along the last dimension, tiles of 16: (x * sign) H, or the rotation back
+    (x H) / 16 * sign (reference bitlinear.py:195-202).  bf16 or float32, same dtype out."""
+    if x.dtype not in (torch.bfloat16, torch.float32) or not x.is_cuda:
+        raise ValueError("hadamard16: bf16 or float32 device tensor")
+    cols = x.shape[-1]
+    x2 = x.reshape(-1, cols)
+    if not x2.is_contiguous():
+        x2 = x2.contiguous()
+    out = torch.empty_like(x2)
+    rc = load().metis_hadamard16(x2.data_ptr(), x2.shape[0], cols, cols, DTYPE_F32 if x.dtype == torch.float32 else DTYPE_BF16,
+                                 int(inverse), int(sign_mask), out.data_ptr(), cols, _stream())
+    check(rc, "metis_hadamard16", tuple(x.shape))
+    return out.reshape(x.shape)
+
+
+def quantize_rht(x: torch.Tensor, mode: int, sign_mask: int, *, sr: bool = False, seed: int = 0, offset: int = 0) -> PackedNVFP4:
+    """Row quantizer of the ROTATED tensor (NV recipe): rotation and quantization in one pass over x.  The result
+    carries `rht` = sign_mask; its dequantize() and tiled expansions rotate back."""
+    x2, kmode = _as_2d_for_quant(x, mode)
+    rows, cols = x2.shape
+    if cols % BLOCK:
+        raise ValueError(f"last dimension {cols} is not a multiple of {BLOCK}")
+    dev = x2.device
+    codes = torch.empty(rows, cols // 2, dtype=torch.uint8, device=dev)
+    scales = torch.empty(rows, cols // BLOCK, dtype=torch.uint8, device=dev)
+    unit = torch.empty(1, dtype=torch.float32, device=dev)
+    ws = _workspace(rows, cols, dev)
+    rc = load().metis_nvfp4_quant_row_rht(x2.data_ptr(), rows, cols, x2.stride(0), kmode, int(sign_mask), int(sr), int(seed), int(offset),
+                                          codes.data_ptr(), scales.data_ptr(), unit.data_ptr(), ws.data_ptr(), ws.numel(), _stream())
+    check(rc, "metis_nvfp4_quant_row_rht", (rows, cols))
+    return PackedNVFP4(codes, scales, unit, rows, cols, MODE_PB16 if mode == MODE_PB16 else MODE_P32, rht=int(sign_mask))
 
 
 def column_sum(x: torch.Tensor, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
@@ -318,8 +357,12 @@ def expand_tiled(p: PackedNVFP4, cache: bool = True, mode: int = MODE_P32) -> to
         return have
     L = load()
     out = torch.empty(L.metis_nvfp4_expand_tiled_bytes(p.rows, p.cols), dtype=torch.uint8, device=p.codes.device)
-    rc = L.metis_nvfp4_expand_tiled(p.codes.data_ptr(), p.scales.data_ptr(), p.unit.data_ptr(), p.rows, p.cols, mode,
-                                    out.data_ptr(), _stream())
+    if p.rht is not None:                     # NV recipe: the operand holds the values rotated back
+        rc = L.metis_nvfp4_expand_tiled_rht(p.codes.data_ptr(), p.scales.data_ptr(), p.unit.data_ptr(), p.rows, p.cols, mode,
+                                            p.rht, 1, 0, out.data_ptr(), _stream())
+    else:
+        rc = L.metis_nvfp4_expand_tiled(p.codes.data_ptr(), p.scales.data_ptr(), p.unit.data_ptr(), p.rows, p.cols, mode,
+                                        out.data_ptr(), _stream())
     check(rc, "metis_nvfp4_expand_tiled", (p.rows, p.cols))
     if cache:
         if mode == MODE_PB16:
@@ -329,9 +372,57 @@ def expand_tiled(p: PackedNVFP4, cache: bool = True, mode: int = MODE_P32) -> to
     return out
 
 
+def expand_tiled_transposed(p: PackedNVFP4, cache: bool = False, mode: int = MODE_P32) -> torch.Tensor:
+    """expand_tiled of the TRANSPOSED tensor: the operand [cols, rows] of a GEMM that contracts over this tensor's
+    rows (rows % 32 == 0); a rotated tensor (NV recipe) is rotated back block by block on the way."""
+    have = p.tiled_t_pb16 if mode == MODE_PB16 else p.tiled_t
+    if have is not None:
+        return have
+    L = load()
+    out = torch.empty(L.metis_nvfp4_expand_tiled_bytes(p.cols, p.rows), dtype=torch.uint8, device=p.codes.device)
+    rc = L.metis_nvfp4_expand_tiled_rht(p.codes.data_ptr(), p.scales.data_ptr(), p.unit.data_ptr(), p.rows, p.cols, mode,
+                                        p.rht or 0, int(p.rht is not None), 1, out.data_ptr(), _stream())
+    check(rc, "metis_nvfp4_expand_tiled_rht", (p.rows, p.cols))
+    if cache:
+        if mode == MODE_PB16:
+            p.tiled_t_pb16 = out
+        else:
+            p.tiled_t = out
+    return out
+
+
 @functools.lru_cache(maxsize=4096)
 def _tiled_workspace_bytes(M: int, N: int, K: int, mode: int, device_index: int) -> int:
     return int(load().metis_linear_tiled_workspace_bytes(M, N, K, mode))
+
+
+def gemm_tiled(ax: torch.Tensor, a_unit: torch.Tensor, bx: torch.Tensor, b_unit: torch.Tensor, M: int, N: int, K: int, *,
+               mode: int = MODE_P32, t: torch.Tensor | None = None, u: torch.Tensor | None = None,
+               bias: torch.Tensor | None = None, out_dtype: torch.dtype = torch.bfloat16, split_k: bool = True) -> torch.Tensor:
+    """out[M, N] = A B^T (+ t u^T + bias) on tiled 16-bit operands ax [M, K], bx [N, K] (see expand_tiled); mode P32:
+    binary16 operands, the product times a_unit * b_unit; mode PB16: bf16 operands that hold their units, the
+    reference's bf16 roundings in the epilogue."""
+    dev = ax.device
+    r = 0
+    if t is not None:
+        t = t.to(torch.bfloat16).contiguous()
+        u = u.to(torch.bfloat16).contiguous()
+        r = t.shape[1]
+        if t.shape != (M, r) or u.shape != (N, r):
+            raise ValueError("low-rank operands must be t[M, r], u[N, r]")
+    bias_f32 = bias is not None and bias.dtype == torch.float32
+    if bias is not None:
+        bias = bias.contiguous() if bias_f32 else bias.to(torch.bfloat16).contiguous()
+    out = torch.empty(M, N, dtype=out_dtype, device=dev)
+    need = _tiled_workspace_bytes(M, N, K, mode, dev.index or 0) if split_k else 0
+    ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
+    rc = load().metis_linear_fwd_tiled(ax.data_ptr(), a_unit.data_ptr(), bx.data_ptr(), b_unit.data_ptr(), M, N, K,
+                                       None if t is None else t.data_ptr(), None if u is None else u.data_ptr(), r,
+                                       None if bias is None else bias.data_ptr(), int(bias_f32), out.data_ptr(),
+                                       DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16, mode,
+                                       None if ws is None else ws.data_ptr(), need, _stream())
+    check(rc, "metis_linear_fwd_tiled", (M, N, K))
+    return out
 
 
 def linear_fwd_tiled(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None, u: torch.Tensor | None = None,
@@ -349,30 +440,10 @@ def linear_fwd_tiled(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None =
         if a.mode != MODE_PB16 or b.mode != MODE_PB16:
             raise ValueError("reference_rounding needs both operands packed in bf16 arithmetic")
         mode = MODE_PB16
-    M, N, K = a.rows, b.rows, a.cols
-    dev = a.codes.device
-    r = 0
-    if t is not None:
-        t = t.to(torch.bfloat16).contiguous()
-        u = u.to(torch.bfloat16).contiguous()
-        r = t.shape[1]
-        if t.shape != (M, r) or u.shape != (N, r):
-            raise ValueError("low-rank operands must be t[M, r], u[N, r]")
-    bias_f32 = bias is not None and bias.dtype == torch.float32
-    if bias is not None:
-        bias = bias.contiguous() if bias_f32 else bias.to(torch.bfloat16).contiguous()
     bx = expand_tiled(b, cache=b.persistent, mode=mode)
     ax = a_tiled if a_tiled is not None else expand_tiled(a, cache=False, mode=mode)
-    out = torch.empty(M, N, dtype=out_dtype, device=dev)
-    need = _tiled_workspace_bytes(M, N, K, mode, dev.index or 0) if split_k else 0
-    ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
-    rc = load().metis_linear_fwd_tiled(ax.data_ptr(), a.unit.data_ptr(), bx.data_ptr(), b.unit.data_ptr(), M, N, K,
-                                       None if t is None else t.data_ptr(), None if u is None else u.data_ptr(), r,
-                                       None if bias is None else bias.data_ptr(), int(bias_f32), out.data_ptr(),
-                                       DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16, mode,
-                                       None if ws is None else ws.data_ptr(), need, _stream())
-    check(rc, "metis_linear_fwd_tiled", (M, N, K))
-    return out
+    return gemm_tiled(ax, a.unit, bx, b.unit, a.rows, b.rows, a.cols, mode=mode, t=t, u=u, bias=bias, out_dtype=out_dtype,
+                      split_k=split_k)
 
 
 def rmsnorm_quantize(x: torch.Tensor, gamma: torch.Tensor, eps: float, mode: int = MODE_P32,
@@ -465,6 +536,11 @@ def linear_fwd(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None,
     MFMA + LDS reads only); the default works on the packed operands directly."""
     if a.cols != b.cols:
         raise ValueError(f"contraction mismatch: {a.cols} vs {b.cols}")
+    if a.rht is not None or b.rht is not None:
+        # NV recipe: only the tiled operands know how to rotate a block back
+        if a.cols % 32:
+            raise ValueError("a rotated operand needs a contraction that is a multiple of 32")
+        tiled = True
     faithful = reference_rounding and a.mode == MODE_PB16 and b.mode == MODE_PB16 and (a.rows >= 256 or tiled) and a.cols % 32 == 0
     if tiled is None:
         tiled = faithful or (not expanded and _tiled_applies(a, b))

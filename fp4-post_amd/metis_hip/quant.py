@@ -88,14 +88,22 @@ class _NVFP4Base(BlockQuantFunc):
     @classmethod
     @torch.no_grad()
     def pack(cls, x: torch.Tensor, col: bool = False, noise: torch.Tensor | None = None,
-             arith: torch.dtype | None = None, center: torch.Tensor | None = None) -> ops.PackedNVFP4:
+             arith: torch.dtype | None = None, center: torch.Tensor | None = None, rht: int | None = None) -> ops.PackedNVFP4:
         """Packed NVFP4 (codes, E4M3 scale bytes, unit) of x in the arithmetic of x's dtype, or of `arith`
         when given: a bf16 tensor packed with arith=float32 gives what x.float() would, without the copy.
-        center: per-column vector subtracted first (mean mode): the packed tensor is that of x - center."""
+        center: per-column vector subtracted first (mean mode): the packed tensor is that of x - center.
+        rht: sign mask of the NV recipe's rotation: the packed tensor is that of the rotated x (see ops.quantize_rht)."""
         _need_gpu(x)
         if not col:
             cls._check(x)
         mode = _mode_of(x) if arith is None else (MODE_P32 if arith == torch.float32 else MODE_PB16)
+        if rht is not None:
+            # NV recipe: the tensor is rotated tile by tile along its last dimension first (sign mask rht); row blocks only
+            if col or noise is not None or center is not None:
+                raise ValueError("a rotated tensor is packed along its last dimension, without caller noise or centre")
+            if cls.stochastic:
+                return ops.quantize_rht(x, mode, rht, sr=True, seed=_NVFP4Base.sr_seed, offset=cls._next_offset(x.numel()))
+            return ops.quantize_rht(x, mode, rht)
         if cls.stochastic:
             return ops.quantize(x, mode, col=col, sr=True, noise=noise, seed=_NVFP4Base.sr_seed,
                                 offset=cls._next_offset(x.numel()) if noise is None else 0, center=center)

@@ -251,6 +251,42 @@ size_t metis_nvfp4_expand_tiled_bytes(int64_t rows, int64_t cols);
 int metis_nvfp4_expand_tiled(const void *codes, const void *scales, const float *unit, int64_t rows,
                              int64_t cols, int mode, void *out, void *stream);
 size_t metis_linear_tiled_workspace_bytes(int64_t M, int64_t N, int64_t K, int mode);
+
+/*
+ * NV recipe (tiled random Hadamard rotation, tile = 16 = the scale block) on the packed kernels.
+ * The reference rotates a tensor tile by tile along its last dimension, (x * sign) H with the Sylvester matrix H_16 and
+ * one shared sign vector (src/Metis/Metis/bitlinear.py:75-137, 199-202), quantizes and dequantizes the rotated tensor,
+ * and rotates back, (q H) / 16 * sign (195-197): `_quantize_wgrad_operand` (395-405) for dY and X of the weight
+ * gradient (495-501) and `_get_quantized_weight` (577-585) for the forward weight.  `sign_mask` carries the sign
+ * vector: bit j set <=> sign[j] = -1 (the reference draws it with torch.randint under seed 1729 + 16; the Python host
+ * side reproduces that draw and passes the mask).
+ *   metis_hadamard16            the rotation (inverse != 0: the rotation back) of a bf16 or float tensor, same dtype out;
+ *                               binary32 sums in butterfly order, one rounding to the output dtype
+ *   metis_nvfp4_quant_row_rht   rotation and row quantizer in one pass over x: the packed tensor holds QDQ's codes of
+ *                               the ROTATED tensor.  mode as metis_nvfp4_quant_row (bf16 arithmetic rounds the rotated
+ *                               values to bf16 first, as the reference's bf16 tensor does); sr != 0: stochastic
+ *                               rounding on the library's own stream (seed, offset) as metis_nvfp4_quant_sr_row
+ *                               without caller noise
+ *   metis_nvfp4_expand_tiled_rht  metis_nvfp4_expand_tiled of such a packed tensor with the rotation back applied to
+ *                               every dequantized block (rotate_back != 0), so that the tiled operand holds the values
+ *                               the reference multiplies with; mode METIS_MODE_P32: one rounding to binary16 (a block's
+ *                               rotated sum needs at most 12 significant bits; relative error <= 2^-12), tensor unit
+ *                               left to the GEMM; METIS_MODE_PB16: dequantized values and result rounded to bf16.
+ *                               transpose != 0: the tiled operand of the TRANSPOSED tensor, [cols, rows] with the
+ *                               contraction over rows (rows % 32 == 0): what the weight-gradient GEMM (contraction over
+ *                               tokens) and the input-gradient GEMM (contraction over out_features) read;
+ *                               out holds metis_nvfp4_expand_tiled_bytes(cols, rows) bytes then
+ *   limits  cols % 16 == 0 (expand: cols % 32 == 0 when not transposed); 16-byte aligned x / out, ld % 8 == 0 (bf16)
+ */
+int metis_hadamard16(const void *x, int64_t rows, int64_t cols, int64_t ldx, int dtype, int inverse,
+                     uint32_t sign_mask, void *out, int64_t ldo, void *stream);
+int metis_nvfp4_quant_row_rht(const void *x, int64_t rows, int64_t cols, int64_t ld, int mode,
+                              uint32_t sign_mask, int sr, uint64_t seed, uint64_t offset, void *codes,
+                              void *scales, float *unit, void *workspace, size_t workspace_bytes,
+                              void *stream);
+int metis_nvfp4_expand_tiled_rht(const void *codes, const void *scales, const float *unit, int64_t rows,
+                                 int64_t cols, int mode, uint32_t sign_mask, int rotate_back,
+                                 int transpose, void *out, void *stream);
 int metis_linear_fwd_tiled(const void *a_xt, const float *a_unit, const void *b_xt, const float *b_unit,
                            int64_t M, int64_t N, int64_t K, const void *t, const void *u, int64_t r,
                            const void *bias, int bias_is_f32, void *out, int out_dtype, int mode,

@@ -3,6 +3,7 @@
 Run once, in the build container only (the reference checkout does not exist on GPU boxes):
 
     python tests/golden/make_golden.py [/root/reference]
+    python tests/golden/make_golden.py /root/reference hadamard_wide     (only metis_reference_hadamard_wide.npz)
 
 Why an import and not only closed forms: the results recorded here depend on the exact
 sequence of per-op roundings of eager PyTorch (bf16-per-op mode differs from an ideal
@@ -202,6 +203,41 @@ def golden_hadamard(out: dict):
         F.enable_nv_recipe = False
 
 
+def golden_hadamard_wide(out: dict):
+    """NV recipe through LinearLowbit at a shape whose backward contractions are multiples of 32 (64 tokens,
+    96 -> 64 features), round-to-nearest quantizers everywhere: once in binary32 arithmetic, once with bf16 tensors
+    and bf16 arithmetic (the GRPO / QAT configuration)."""
+    F = rb.LinearLowbitFunction
+    g = torch.Generator().manual_seed(43)
+    B, T, K, N = 2, 32, 96, 64
+    xl = torch.randn(B, T, K, generator=g).bfloat16()
+    w = (torch.randn(N, K, generator=g) * 0.05).bfloat16()
+    dy = (torch.randn(B, T, N, generator=g) * 1e-3).bfloat16()
+    out["hw_x"], out["hw_w"], out["hw_dy"] = bits(xl), bits(w), bits(dy)
+    F.hadamard_tile_size, F.hadamard_backend, F.hadamard_workspace_mb = 16, "torch_gemm", 128
+    for tag, dtype in (("p32", torch.float32), ("pb16", torch.bfloat16)):
+        _configure("nvfp4e2m1bnosr", "nvfp4e2m1bnosr", "nvfp4e2m1bnosr", dtype)
+        F.enable_nv_recipe = True
+        try:
+            layer = rb.LinearLowbit(K, N, bias=False, args=SimpleNamespace(device="cpu", cache_quantized_weight=False))
+            layer.weight.data = w.to(dtype).clone()
+            layer.compute_dtype = dtype
+            xr = xl.to(dtype).clone().requires_grad_(True)
+            y = layer(xr)
+            y.backward(dy.to(dtype))
+            out[f"hw_{tag}_wq"] = bits(layer._get_quantized_weight(layer.weight.detach().to(dtype)))
+            # the two weight-gradient operands as the backward pass forms them (495-501): rotated, quantized, rotated back
+            xq = F.quantize_input(xl.to(dtype).clone())
+            out[f"hw_{tag}_xq"] = bits(xq)
+            out[f"hw_{tag}_wgrad_x"] = bits(F._quantize_wgrad_operand(xq.clone(), F.q_backward_input))
+            out[f"hw_{tag}_wgrad_dy"] = bits(F._quantize_wgrad_operand(dy.to(dtype).clone(), F.q_backward_outputgrad))
+            out[f"hw_{tag}_y"], out[f"hw_{tag}_gx"] = bits(y.detach()), bits(xr.grad)
+            out[f"hw_{tag}_gw"] = bits(layer.weight.grad)
+        finally:
+            F.enable_nv_recipe = False
+            F.compute_dtype = torch.float32
+
+
 def golden_mean_mode(out: dict):
     """Mean mode (bitlinear.py:311-336): column mean over tokens kept, centred residual through the fused QDQ; a
     prefill call, then a single-token decode call on the same cache (weighted running mean), in binary32 and in
@@ -297,6 +333,13 @@ def golden_rollout(out: dict):
 
 def main():
     torch.set_num_threads(1)
+    if len(sys.argv) > 2 and sys.argv[2] == "hadamard_wide":    # only this file (the others are not touched)
+        hw: dict = {}
+        golden_hadamard_wide(hw)
+        path = os.path.join(HERE, "metis_reference_hadamard_wide.npz")
+        np.savez_compressed(path, **hw)
+        print(f"wrote {path}: {len(hw)} arrays, {os.path.getsize(path)} bytes")
+        return
     out: dict = {}
     golden_rne(out)
     golden_sr(out)

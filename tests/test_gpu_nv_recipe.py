@@ -1,0 +1,234 @@
+"""GPU tests of the NV recipe (tiled random Hadamard rotation, reference bitlinear.py:75-211, 395-405, 495-501,
+577-585) on the library's kernels: the rotation itself, rotation + quantizer in one pass, the tiled GEMM operands that
+rotate a packed block back (plain and transposed), and LinearLowbit forward + both gradients against vectors the
+reference wrote (tests/golden/metis_reference_hadamard*.npz)."""
+import os
+from types import SimpleNamespace
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import rel_fro, same_bits, synthetic_activation, t
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+@pytest.fixture(autouse=True)
+def _config():
+    from metis_hip import LinearLowbitFunction as F, quant_func
+    nosr = quant_func["nvfp4e2m1bnosr"]
+    F.q_forward_input = F.q_forward_weight = nosr
+    F.q_backward_input = F.q_backward_weight = F.q_backward_outputgrad = nosr
+    F.enable_activation_svd = False
+    F.enable_backward_svd = False
+    F.enable_nv_recipe = False
+    F.hadamard_tile_size, F.hadamard_backend = 16, "auto"
+    F.compute_dtype = torch.float32
+    keep = F.reference_rounding
+    yield
+    F.enable_nv_recipe = False
+    F.compute_dtype = torch.float32
+    F.reference_rounding = keep
+
+
+def _mask():
+    from metis_hip import LinearLowbitFunction as F
+    return F._hadamard_mask()
+
+
+def _signs():
+    m = _mask()
+    return torch.tensor([-1.0 if (m >> j) & 1 else 1.0 for j in range(16)], dtype=torch.float64)
+
+
+def _h16():
+    h = torch.ones(1, 1, dtype=torch.float64)
+    while h.shape[0] < 16:
+        h = torch.cat((torch.cat((h, h), 1), torch.cat((h, -h), 1)), 0)
+    return h
+
+
+def _rot(x64, inverse=False):
+    tiles = x64.reshape(-1, 16)
+    out = (tiles @ _h16()) / 16 * _signs() if inverse else (tiles * _signs()) @ _h16()
+    return out.reshape(x64.shape)
+
+
+def test_rotation_kernel_against_reference_vectors_and_closed_form():
+    from metis_hip import LinearLowbitFunction as F, ops
+    g = dict(np.load(os.path.join(GOLDEN, "metis_reference_hadamard.npz")))
+    assert torch.equal(F._get_hadamard_sign(16, torch.device("cpu"), torch.float32), t(g["had_sign16"]))
+    x = t(g["had_x"]).cuda()
+    torch.testing.assert_close(ops.hadamard16(x, _mask()).cpu(), t(g["had_fwd"]), rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(ops.hadamard16(x, _mask(), inverse=True).cpu(), t(g["had_inv"]), rtol=1e-6, atol=1e-6)
+    got = ops.hadamard16(x.bfloat16(), _mask()).cpu()
+    want = t(g["had_fwd_bf16"])
+    assert float((got.view(torch.int16).int() - want.view(torch.int16).int()).abs().max()) <= 1   # one rounding of a binary32 sum
+    # the module's rotation now runs on that kernel
+    F.hadamard_backend = "auto"
+    assert torch.equal(F._apply_hadamard_blocks(x), ops.hadamard16(x, _mask()))
+    # closed form on a larger tensor, and the round trip
+    big = synthetic_activation(5, 300, 1024).cuda()
+    rot = ops.hadamard16(big, _mask())
+    want = _rot(big.double().cpu())
+    assert float((rot.double().cpu() - want).abs().max()) <= float(want.abs().max()) * 2.0 ** -8
+    f = big.float()
+    back = ops.hadamard16(ops.hadamard16(f, _mask()), _mask(), inverse=True)
+    torch.testing.assert_close(back, f, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+def test_rotation_and_quantizer_in_one_pass_equal_the_two_steps(mode):
+    """quantize_rht(x) packs exactly what quantizing the rotated tensor packs: binary32 arithmetic quantizes the
+    binary32 rotated values, bf16 arithmetic their bf16 roundings."""
+    from metis_hip import ops
+    x = synthetic_activation(21 + mode, 512, 1024).cuda()
+    p = ops.quantize_rht(x, mode, _mask())
+    if mode == 0:
+        two = ops.quantize(ops.hadamard16(x.float(), _mask()), 0)          # binary32 input path
+    else:
+        two = ops.quantize(ops.hadamard16(x, _mask()), 1)
+    assert torch.equal(p.codes, two.codes) and torch.equal(p.scales, two.scales) and torch.equal(p.unit, two.unit)
+    assert p.rht == _mask()
+    # dequantize() returns to the tensor's own domain: close to x, and equal to rotating the plain dequantization back
+    plain = ops.PackedNVFP4(p.codes, p.scales, p.unit, p.rows, p.cols, p.mode)
+    want = ops.hadamard16(plain.dequantize(torch.float32), _mask(), inverse=True)
+    assert torch.equal(p.dequantize(torch.float32), want)
+    assert rel_fro(p.dequantize(torch.float32).cpu(), x.float().cpu()) < 0.15
+    # stochastic rounding on the library's stream: reproducible, and a different stream gives different codes
+    a = ops.quantize_rht(x, mode, _mask(), sr=True, seed=7, offset=0)
+    b = ops.quantize_rht(x, mode, _mask(), sr=True, seed=7, offset=0)
+    c = ops.quantize_rht(x, mode, _mask(), sr=True, seed=8, offset=0)
+    assert torch.equal(a.codes, b.codes) and not torch.equal(a.codes, c.codes)
+    assert torch.equal(a.scales, p.scales) and torch.equal(a.unit, p.unit)
+
+
+def test_wgrad_operand_against_reference_vector():
+    """rot -> QDQ -> rot^-1 of the reference's test tensor (binary32 arithmetic, round to nearest)."""
+    from metis_hip import ops
+    g = dict(np.load(os.path.join(GOLDEN, "metis_reference_hadamard.npz")))
+    x = t(g["had_x"]).cuda()
+    got = ops.quantize_rht(x, 0, _mask()).dequantize(torch.float32).cpu()
+    want = t(g["had_wgrad_operand_p32"])
+    assert rel_fro(got, want) <= 1e-6
+    assert float((got - want).abs().le(1e-6).float().mean()) == 1.0
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+def test_tiled_operands_rotate_a_packed_block_back(mode):
+    """GEMMs on the tiled expansions of a rotated packed tensor (plain and transposed) equal the product of its
+    dequantized, rotated-back values: within the one binary16 rounding per operand element (2^-12) in binary32
+    arithmetic, within the bf16 roundings of the reference's evaluation in bf16 arithmetic."""
+    from metis_hip import ops
+    L, N, K = 512, 384, 640
+    a = synthetic_activation(31, L, K).cuda()
+    w = (torch.randn(N, K, generator=torch.Generator().manual_seed(32)) * 0.05).bfloat16().cuda()
+    pa = ops.quantize(a, mode)                                  # plain activation
+    pw = ops.quantize_rht(w, mode, _mask())                     # rotated weight
+    # dense references in the arithmetic's own dtype: in bf16 arithmetic the rotated-back values are bf16 tensors, and
+    # the GEMM rounds its product to bf16 once more (2^-9 relative at worst)
+    dt = torch.float32 if mode == 0 else torch.bfloat16
+    da, dw = pa.dequantize(dt).double(), pw.dequantize(dt).double()
+    tol = 2e-4 if mode == 0 else 2.5e-3
+    # forward shape: A [L, K] . W~[N, K]^T
+    y = ops.gemm_tiled(ops.expand_tiled(pa, cache=False, mode=mode), pa.unit, ops.expand_tiled(pw, cache=False, mode=mode), pw.unit,
+                       L, N, K, mode=mode, out_dtype=torch.float32)
+    assert rel_fro(y.double().cpu(), (da @ dw.T).cpu()) <= tol
+    # the same through linear_fwd, which routes a rotated operand to the tiled kernel by itself
+    y2 = ops.linear_fwd(pa, pw, out_dtype=torch.float32, reference_rounding=mode == 1)
+    assert torch.equal(y2, y)
+    # transposed operands: contraction over the packed tensors' rows.  dY~ [L, N] rotated, against W~^T [K, N] and X~^T
+    dy = (torch.randn(L, N, generator=torch.Generator().manual_seed(33)) * 1e-3).bfloat16().cuda()
+    pdy = ops.quantize_rht(dy, mode, _mask())
+    px = ops.quantize_rht(a, mode, _mask())
+    ddy, dx = pdy.dequantize(dt).double(), px.dequantize(dt).double()
+    gx = ops.gemm_tiled(ops.expand_tiled(pdy, cache=False, mode=mode), pdy.unit, ops.expand_tiled_transposed(pw, mode=mode), pw.unit,
+                        L, K, N, mode=mode, out_dtype=torch.float32)
+    assert rel_fro(gx.double().cpu(), (ddy @ dw).cpu()) <= tol
+    gw = ops.gemm_tiled(ops.expand_tiled_transposed(pdy, mode=mode), pdy.unit, ops.expand_tiled_transposed(px, mode=mode), px.unit,
+                        N, K, L, mode=mode, out_dtype=torch.float32)
+    assert rel_fro(gw.double().cpu(), (ddy.T @ dx).cpu()) <= tol
+    # a transposed expansion without rotation: plain packed tensors
+    gw2 = ops.gemm_tiled(ops.expand_tiled_transposed(pa, mode=mode), pa.unit, ops.expand_tiled_transposed(pa, mode=mode), pa.unit,
+                         K, K, L, mode=mode, out_dtype=torch.float32)
+    assert rel_fro(gw2.double().cpu(), (da.T @ da).cpu()) <= tol
+
+
+@pytest.mark.parametrize("tag", ["p32", "pb16"])
+def test_linear_lowbit_nv_recipe_on_the_packed_kernels_against_reference_vectors(tag):
+    """LinearLowbit with enable_nv_recipe, 64 tokens, 96 -> 64 features: forward, grad_input and grad_weight against
+    what the reference computed, with no torch matmul on the way (the generic path would warn)."""
+    import warnings
+
+    from metis_hip import LinearLowbit, LinearLowbitFunction as F, bitlinear, ops
+    g = dict(np.load(os.path.join(GOLDEN, "metis_reference_hadamard_wide.npz")))
+    dtype = torch.float32 if tag == "p32" else torch.bfloat16
+    F.enable_nv_recipe = True
+    F.compute_dtype = dtype
+    layer = LinearLowbit(96, 64, bias=False, args=SimpleNamespace(device="cuda", cache_quantized_weight=True),
+                         storage_dtype=dtype, compute_dtype=dtype)
+    with torch.no_grad():
+        layer.weight.copy_(t(g["hw_w"]).to(dtype))
+    xr = t(g["hw_x"]).to(dtype).cuda().requires_grad_(True)
+    bitlinear._generic_path_warned.clear()
+    calls = []
+    real = ops.gemm_tiled
+    ops.gemm_tiled = lambda *a, **k: (calls.append(1), real(*a, **k))[1]
+    try:
+        with warnings.catch_warnings():
+            warnings.simplefilter("error")
+            y = layer(xr)
+            y.backward(t(g["hw_dy"]).to(dtype).cuda())
+    finally:
+        ops.gemm_tiled = real
+    assert len(calls) == 3                                      # forward, input gradient, weight gradient
+    pw = layer._get_quantized_weight(layer.weight, arith=dtype)
+    assert isinstance(pw, ops.PackedNVFP4) and pw.rht == F._hadamard_mask() and (pw.tiled_t is not None or pw.tiled_t_pb16 is not None)
+    # the quantized weight the reference multiplied with
+    wq = pw.dequantize(dtype).float().cpu()
+    assert rel_fro(wq, t(g[f"hw_{tag}_wq"]).float()) <= (1e-6 if tag == "p32" else 2e-3)
+    tol = 2e-3
+    assert rel_fro(y.detach().float().cpu(), t(g[f"hw_{tag}_y"]).float()) <= tol
+    assert rel_fro(xr.grad.float().cpu(), t(g[f"hw_{tag}_gx"]).float()) <= tol
+    # The weight gradient's second operand is the ALREADY quantized input, rotated and quantized again (495-501).  Its
+    # rotated values are small-integer combinations of one block scale, so their quotients by the new block scalar sit
+    # exactly on FP4 rounding boundaries far more often than those of ordinary data, and which side such a value lands
+    # on hangs on the last bit of a 16-term binary32 sum, i.e. on the summation order of whoever computes it (the
+    # reference's own CPU and GPU results differ the same way).  A flipped code spreads over its block of 16 on the way
+    # back: about 5 % of the operand's elements differ from the reference's CPU run, 2e-2 in the Frobenius norm.
+    x_op = F.q_backward_input.pack(t(g[f"hw_{tag}_xq"]).to(dtype).cuda().reshape(-1, 96), arith=dtype, rht=F._hadamard_mask())
+    got, want = x_op.dequantize(dtype).float().cpu(), t(g[f"hw_{tag}_wgrad_x"]).float().reshape(-1, 96)
+    assert rel_fro(got, want) <= 3e-2 and float((got - want).abs().le(1e-6 * float(want.abs().max())).float().mean()) > 0.9
+    dy_op = F.q_backward_outputgrad.pack(t(g["hw_dy"]).to(dtype).cuda().reshape(-1, 64), arith=dtype, rht=F._hadamard_mask())
+    assert rel_fro(dy_op.dequantize(dtype).float().cpu(), t(g[f"hw_{tag}_wgrad_dy"]).float().reshape(-1, 64)) <= (1e-6 if tag == "p32" else 2e-3)
+    assert rel_fro(layer.weight.grad.float().cpu(), t(g[f"hw_{tag}_gw"]).float()) <= 3e-2
+    # and against the product of the operands as this library formed them: the GEMM itself is exact to its tolerance
+    dense = dy_op.dequantize(dtype).double().T @ x_op.dequantize(dtype).double()
+    assert rel_fro(layer.weight.grad.double().cpu(), dense.cpu()) <= (2e-4 if tag == "p32" else 2.5e-3)
+
+
+def test_nv_recipe_at_a_training_shape_keeps_the_packed_kernels_and_matches_the_generic_path():
+    """4096 tokens, 1536 -> 8960 (the QAT projection): kernel path against the module's own generic path
+    (rotation kernel + three-call QDQ + torch matmuls, `hadamard_backend="torch_gemm"` switches the kernels off)."""
+    from metis_hip import LinearLowbit, LinearLowbitFunction as F
+    F.enable_nv_recipe = True
+    args = SimpleNamespace(device="cuda", cache_quantized_weight=True)
+    layer = LinearLowbit(1536, 8960, bias=False, args=args, storage_dtype=torch.bfloat16, compute_dtype=torch.float32)
+    x = synthetic_activation(41, 4096, 1536).cuda().reshape(2, 2048, 1536)
+    dy = (torch.randn(2, 2048, 8960, generator=torch.Generator().manual_seed(42)) * 1e-3).bfloat16().cuda()
+    outs = {}
+    for backend in ("auto", "torch_gemm"):
+        F.hadamard_backend = backend
+        layer._quantized_weight_cache = None
+        layer.weight.grad = None
+        xr = x.clone().requires_grad_(True)
+        y = layer(xr)
+        y.backward(dy.to(y.dtype))
+        outs[backend] = (y.detach().float(), xr.grad.float(), layer.weight.grad.float())
+    # output and input gradient agree to the GEMM tolerance; the weight gradient's re-quantized input operand is the one
+    # whose codes hang on the last bit of the rotation's sums (see the test above), and the two paths sum in different orders
+    for (a, b), tol in zip(zip(outs["auto"], outs["torch_gemm"]), (2e-3, 2e-3, 3e-2)):
+        assert rel_fro(a.cpu(), b.cpu()) <= tol
