@@ -361,6 +361,39 @@ def main():
             if isinstance(qat, dict):
                 qat["mean_mode"] = {"error": f"{type(exc).__name__}: {exc}"[:300]}
 
+    # the same projection under the NV recipe (tiled random Hadamard rotation around the weight QDQ and the two
+    # weight-gradient operands): on the packed kernels, and on the module's generic path (rotation kernel, three-call
+    # QDQ, dequantized tensors, torch matmuls) that hadamard_backend = "torch_gemm" selects
+    if not args.no_decode and isinstance(qat, dict):
+        try:
+            nv_args = MetisArgs.direct_fp4()
+            nv_args.cache_quantized_weight = True
+            nlin = LinearLowbit(1536, 8960, bias=False, args=nv_args, device=dev, storage_dtype=torch.bfloat16, compute_dtype=torch.float32)
+            LinearLowbitFunction.enable_nv_recipe = True
+
+            def nv_step(ev):
+                if ev is not None:
+                    ev[0].record()
+                y_ = nlin(xq_)
+                y_.backward(dy_.to(y_.dtype))
+                if ev is not None:
+                    ev[1].record()
+                nlin.weight.grad = None
+                xq_.grad = None
+            nv = {"workload": "same projection, enable_nv_recipe (rotation fused into the row quantizer, tiled GEMM operands rotated back "
+                              "block by block, quantization blocks along the last dimension as in the reference)"}
+            for backend, key in (("auto", "us_per_step"), ("torch_gemm", "us_per_step_generic_path")):
+                LinearLowbitFunction.hadamard_backend = backend
+                nlin._quantized_weight_cache = None
+                _, nv_ms = time_region(torch, nv_step, 10, 3)
+                nv[key] = round(nv_ms * 1e3, 1)
+            qat["nv_recipe"] = nv
+        except Exception as exc:
+            qat["nv_recipe"] = {"error": f"{type(exc).__name__}: {exc}"[:300]}
+        finally:
+            LinearLowbitFunction.enable_nv_recipe = False
+            LinearLowbitFunction.hadamard_backend = "auto"
+
     # config 4 as named: gate, up and down projections of the 1.5B-class MLP, each a rank-32 BitLinear, forward + backward
     if not args.no_decode and isinstance(qat, dict):
         try:

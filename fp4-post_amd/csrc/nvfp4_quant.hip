@@ -311,121 +311,103 @@ __global__ __launch_bounds__(256) void quant_scales_f32_kernel(const float* __re
 }
 
 // ---------------------------------------------------------------------------------------------
-// Single-launch variant for round-to-nearest row quantization (opt-in): both phases in one kernel
-// whose workgroups are all resident at once.  Each thread keeps the maxima of its (at most NB)
-// blocks in registers across a grid-wide reduction, so neither the parked maxima nor a second
-// launch are needed.
+// Single-launch variant for round-to-nearest rows of a contiguous bf16 tensor: both phases in one kernel.  Each thread
+// keeps the maxima of its (at most NB) blocks in registers across a grid-wide maximum, so in the ordinary case neither
+// the parked maxima nor a second launch are needed.
 //
-// Grid-wide maximum from tagged words, no read-modify-write traffic at all.  A call's tag is the
-// 48-bit generation counter of the workspace plus one.  Workgroup b belongs to group j = b % 64
-// as member b / 64 and publishes {tag, its maximum as bf16} as ONE 64-bit store to its own word.
-// Wave 0 of member 0 polls the (at most 64) words of its group with one load per lane until all
-// carry the tag, folds them and stores {tag, group maximum} into a private copy for each of the
-// 64 groups; wave 0 of every workgroup polls its group's copy of the 64 group maxima the same way.
-// Tag and value share a word, so no ordering between locations is needed: relaxed device-scope
-// loads and stores only, and no line is polled by more than one group's members.
-// Workgroup 0 advances the generation counter once its own wait is over, by which time every
-// workgroup has read it.  The words only need zero-filling once.  The wait is bounded: after
-// spin_limit polls a workgroup gives up, so every wave always exits; it then raises the sticky
-// time-out word of the workspace and its result is NaN, which ends up in the tensor unit (and in the
-// unit of every later call on that workspace until the caller zero-fills it again).
+// The grid-wide maximum does not assume that all workgroups are resident together.  Workgroups arrive through a
+// two-level tree (64 groups of up to 64 workgroups) whose nodes are a maximum and an arrival counter, each updated by one
+// read-modify-write, so exactly one workgroup learns that it is the LAST to arrive and what the tensor maximum is.  It
+// exchanges {call tag, result, maximum} into 64 words (one per group, a line each), writes the tensor unit, and cleans
+// the tree for the next call.  Every other workgroup polls its group's word a bounded number of times.  One that gives
+// up -- because part of the grid is still waiting for a compute unit, held by another kernel or by these very pollers
+// -- parks its block maxima in the workspace, raises its flag, swaps {call tag, "somebody left"} into its group's word
+// and exits WITHOUT its scale bytes: the last workgroup finds that marker in what its exchange returns and writes
+// those bytes itself.  If the exchange came first, the leaver's swap fails, it reads the result and finishes its own
+// bytes after all.  That decision hangs on one word, so relaxed device-scope atomics suffice on the ordinary path (an
+// acquire or release at device scope writes back or invalidates a whole L2 on this part); only a workgroup that leaves
+// and the last workgroup that cleans up after one pay for fences.  Every wave exits after a bounded time whatever else
+// runs on the device, and the result is always complete and always the same bytes as the two-launch path.
+// The area starts zero-filled; a call leaves the tree clean and only tagged words behind.
 // ---------------------------------------------------------------------------------------------
-constexpr uint32_t kSpinLimit = 1u << 20;
+constexpr uint32_t kSpinLimit = 4096;            // polls (roughly a microsecond each) before a workgroup leaves its scale bytes behind
 constexpr uint32_t kGroups = 64;                 // groups, and the most members a group can have
 constexpr int kFusedMaxGrid = kGroups * kGroups;
 // locations inside the synchronisation area (uint32 units)
 __device__ __forceinline__ uint64_t* sync_generation(uint32_t* s) { return reinterpret_cast<uint64_t*>(s); }
-__device__ __forceinline__ uint32_t* sync_timeout(uint32_t* s) { return s + 32; }
-__device__ __forceinline__ uint64_t* sync_member(uint32_t* s, uint32_t j, uint32_t m)
-{
-    return reinterpret_cast<uint64_t*>(s + 256) + j * kGroups + m;
-}
-// group maxima as seen by reader group g: a private copy per group so that no line has more than
-// a group's worth of pollers (device-scope accesses to one line are served one after another)
-__device__ __forceinline__ uint64_t* sync_copy(uint32_t* s, uint32_t g, uint32_t j)
-{
-    return reinterpret_cast<uint64_t*>(s + 256 + 2 * kGroups * kGroups) + g * kGroups + j;
-}
+__device__ __forceinline__ uint32_t* sync_top(uint32_t* s) { return s + 4; }                           // {maximum, arrivals}
+__device__ __forceinline__ uint32_t* sync_group(uint32_t* s, uint32_t j) { return s + 64 + j * 32; }     // {maximum, arrivals}, a line each
+__device__ __forceinline__ uint64_t* sync_result(uint32_t* s, uint32_t j) { return reinterpret_cast<uint64_t*>(s + 2176 + j * 32); }
+__device__ __forceinline__ uint32_t* sync_left_flag(uint32_t* s, uint32_t b) { return s + 4224 + b; }
+static_assert((4224 + kFusedMaxGrid) * 4 <= kWsSyncBytes, "synchronisation area too small");
 
 #define METIS_AT_LOAD(p) __hip_atomic_load((p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
 #define METIS_AT_STORE(p, v) __hip_atomic_store((p), (v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+#define METIS_AT_CAS(p, expected, desired) \
+    __hip_atomic_compare_exchange_strong((p), (expected), (desired), __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+#define METIS_AT_XCHG(p, v) __hip_atomic_exchange((p), (v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+
+// a group's result word: tag << 18 | kind << 16 | bf16 payload; kind 0: the tensor maximum, kind 1: a member has left
+__device__ __forceinline__ uint64_t result_word(uint64_t tag, uint32_t kind, uint32_t payload) { return (tag << 18) | ((uint64_t)kind << 16) | payload; }
+__device__ __forceinline__ bool is_result(uint64_t w, uint64_t tag) { return (w >> 16) == (tag << 2); }
+__device__ __forceinline__ bool is_left_marker(uint64_t w, uint64_t tag) { return (w >> 16) == ((tag << 2) | 1u); }
 
 struct GridMaxState {
     float wave_part[4];
+    uint32_t last;               // this workgroup was the last to arrive
+    uint32_t known;              // result holds the tensor maximum
     float result;
+    uint32_t nleft;
+    uint32_t left[256];          // workgroups of one slab of 256 flags that left their scale bytes behind
 };
 
-// Wave 0 of every workgroup, at kernel start: the tag of this call (other waves get 0, unused).
+// Every thread, at kernel start (before its workgroup arrives, so before the counter can move): the tag of this call.
 __device__ __forceinline__ uint64_t grid_max_begin(uint32_t* sync)
 {
-    return threadIdx.x < 64 ? METIS_AT_LOAD(sync_generation(sync)) + 1u : 0u;
+    return METIS_AT_LOAD(sync_generation(sync)) + 1u;
 }
 
-// Called by every thread of every workgroup, once: publishes the workgroup maximum (a bf16 value).
-__device__ __forceinline__ void grid_max_arrive(float thread_max, uint64_t tag, uint32_t* sync, GridMaxState& sh)
+// One more arrival with maximum `bits` at a tree node {maximum, arrivals}; true for the arrival that completes `expected`,
+// with the node's maximum.  Two relaxed read-modify-writes without retry: the counter's increment is made to depend on
+// the value the maximum's returns, so it is issued only after the maximum has been performed at the coherence point; the
+// arrival that sees the count complete therefore reads a maximum that every earlier arrival has folded in.
+__device__ __forceinline__ bool tree_arrive(uint32_t* node, uint32_t bits, uint32_t expected, uint32_t& folded)
+{
+    const uint32_t before = __hip_atomic_fetch_max(node, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const uint32_t one = 1u + (before >> 31);                      // bit 31 of a non-negative float's pattern: always 0
+    if (__hip_atomic_fetch_add(node + 1, one, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != expected - 1u) return false;
+    folded = METIS_AT_LOAD(node);
+    METIS_AT_STORE(node, 0u);                                      // nobody else touches the node before the next call
+    METIS_AT_STORE(node + 1, 0u);
+    return true;
+}
+
+// Called by every thread of every workgroup, once: folds the workgroup maximum (a bf16 value) into the tree.
+__device__ __forceinline__ void grid_max_arrive(float thread_max, uint32_t* sync, GridMaxState& sh)
 {
     const float m = wave_max(thread_max);
     if ((threadIdx.x & 63) == 0) sh.wave_part[threadIdx.x >> 6] = m;
     __syncthreads();
     if (threadIdx.x == 0) {
-        const float g = fmaxf(fmaxf(sh.wave_part[0], sh.wave_part[1]), fmaxf(sh.wave_part[2], sh.wave_part[3]));
-        METIS_AT_STORE(sync_member(sync, blockIdx.x % kGroups, blockIdx.x / kGroups), (tag << 16) | (uint64_t)(__float_as_uint(g) >> 16));
-    }
-}
-
-// Wave-wide: polls one word per lane (lanes >= count are idle) until all carry the tag; returns the
-// maximum of the bf16 payloads.
-__device__ __forceinline__ float poll_tagged_max(const uint64_t* words, uint32_t count, uint64_t tag, uint32_t* sync,
-                                                 uint32_t spin_limit)
-{
-    const uint32_t lane = threadIdx.x & 63u;
-    uint64_t w = tag << 16;
-    uint32_t polls = 0;
-    for (;;) {
-        if (lane < count) w = METIS_AT_LOAD(words + lane);
-        if (__builtin_amdgcn_ballot_w64((w >> 16) != tag) == 0ull) break;
-        if (++polls > spin_limit) {
-            if (lane == 0) METIS_AT_STORE(sync_timeout(sync), 1u);
-            return __builtin_nanf("");
-        }
-        __builtin_amdgcn_s_sleep(1);
-    }
-    // a payload of 0x7fc0 (bf16 NaN) marks a group whose own wait gave up; fmaxf would drop it
-    if (__builtin_amdgcn_ballot_w64(lane < count && ((uint32_t)w & 0xffffu) == 0x7fc0u) != 0ull) return __builtin_nanf("");
-    return wave_max(__uint_as_float(((uint32_t)w & 0xffffu) << 16));
-}
-
-// Called by every thread after grid_max_arrive(); returns the tensor-wide maximum.
-__device__ __forceinline__ float grid_max_wait(uint64_t tag, uint32_t* sync, GridMaxState& sh, uint32_t spin_limit)
-{
-    if (threadIdx.x < 64) {
+        const uint32_t bits = __float_as_uint(fmaxf(fmaxf(sh.wave_part[0], sh.wave_part[1]), fmaxf(sh.wave_part[2], sh.wave_part[3])));
         const uint32_t j = blockIdx.x % kGroups;
         const uint32_t ngroups = gridDim.x < kGroups ? gridDim.x : kGroups;
         const uint32_t members = (gridDim.x + kGroups - 1u - j) / kGroups;
-        if (blockIdx.x < kGroups) {                               // member 0 folds its group and tells every group
-            const float gm = poll_tagged_max(sync_member(sync, j, 0), members, tag, sync, spin_limit);
-            // a group that gave up is published as the bf16 NaN pattern, so every reader's result is NaN as well
-            const uint64_t payload = gm == gm ? (uint64_t)(__float_as_uint(gm) >> 16) : 0x7fc0ull;
-            if (threadIdx.x < ngroups) METIS_AT_STORE(sync_copy(sync, threadIdx.x, j), (tag << 16) | payload);
-        }
-        float all = poll_tagged_max(sync_copy(sync, j, 0), ngroups, tag, sync, spin_limit);
-        if (METIS_AT_LOAD(sync_timeout(sync)) != 0u) all = __builtin_nanf("");   // sticky: this call or an earlier one gave up
-        if (threadIdx.x == 0) {
-            sh.result = all;
-            if (blockIdx.x == 0) METIS_AT_STORE(sync_generation(sync), tag);
-        }
+        uint32_t gm = 0u, fin = 0u;
+        const bool last = tree_arrive(sync_group(sync, j), bits, members, gm) && tree_arrive(sync_top(sync), gm, ngroups, fin);
+        sh.last = last ? 1u : 0u;
+        sh.known = sh.last;
+        sh.result = __uint_as_float(fin);
     }
-    __syncthreads();
-    return sh.result;
 }
 
-// One block in flight ahead of the one being encoded (as in phase 1 of the two-launch path), block
-// maxima kept in registers, and the arrival placed before the encoding of the thread's last block
-// so that part of the reduction latency is covered.
+// One block in flight ahead of the one being encoded (as in phase 1 of the two-launch path), block maxima kept in
+// registers, and the arrival placed before the encoding of the thread's last block so that the tree's latency is covered.
 template <int MODE, int NB>
 __global__ __launch_bounds__(256) void quant_fused_kernel(const uint16_t* __restrict__ x, uint2* __restrict__ codes,
                                                           uint8_t* __restrict__ scales, float* __restrict__ unit_out,
-                                                          uint32_t* __restrict__ sync, uint32_t nblocks, uint32_t spin_limit)
+                                                          uint32_t* __restrict__ sync, uint16_t* __restrict__ parked,
+                                                          uint32_t nblocks, uint32_t spin_limit)
 {
     __shared__ GridMaxState sh;
     const uint64_t tag = grid_max_begin(sync);
@@ -436,28 +418,129 @@ __global__ __launch_bounds__(256) void quant_fused_kernel(const uint16_t* __rest
     if (i0 < nblocks) { c0 = xp[2 * (size_t)i0]; c1 = xp[2 * (size_t)i0 + 1]; }
     float am[NB];
     float gmax = 0.0f;
+    const float none[kBlock] = {};
+    constexpr int TAIL = NB >= 2 ? 2 : 1;                          // blocks encoded after the arrival
 #pragma unroll
-    for (int k = 0; k < NB; ++k) {
+    for (int k = 0; k < NB - TAIL; ++k) {
         const uint32_t i = i0 + k * stride;
         uint4 n0 = make_uint4(0u, 0u, 0u, 0u), n1 = n0;
-        if (k + 1 < NB && i + stride < nblocks) { n0 = xp[2 * (size_t)(i + stride)]; n1 = xp[2 * (size_t)(i + stride) + 1]; }
+        if (i + stride < nblocks) { n0 = xp[2 * (size_t)(i + stride)]; n1 = xp[2 * (size_t)(i + stride) + 1]; }
         float v[kBlock];
-        const float none[kBlock] = {};
         unpack16(c0, c1, v);
         am[k] = block_amax(v);
         gmax = fmaxf(gmax, am[k]);
-        if (k == NB - 1) grid_max_arrive(gmax, tag, sync, sh);
         if (i < nblocks) codes[i] = encode_block<MODE, false>(v, block_scalar<MODE>(am[k]), none);
         c0 = n0; c1 = n1;
     }
-    const float amax = grid_max_wait(tag, sync, sh, spin_limit);
-    const float unit = rd<MODE>(block_scalar<MODE>(amax) / 448.0f);          // quant.py:21-22 (NaN after a time-out)
-    if (i0 == 0) *unit_out = unit;
-#pragma unroll
-    for (int k = 0; k < NB; ++k) {
-        const uint32_t i = i0 + k * stride;
-        if (i < nblocks) scales[i] = (uint8_t)e4m3_byte(rd<MODE>(block_scalar<MODE>(am[k]) / unit));   // quant.py:23
+    {
+        // the last blocks: all their maxima first, then the arrival, then their encoding -- a few microseconds of vector
+        // work between the arrival and the wait, which is what the tree and the last workgroup's word need to get round
+        const uint32_t ia = i0 + (NB - TAIL) * stride, ib = ia + stride;
+        uint4 d0 = make_uint4(0u, 0u, 0u, 0u), d1 = d0;
+        if (TAIL == 2 && ib < nblocks) { d0 = xp[2 * (size_t)ib]; d1 = xp[2 * (size_t)ib + 1]; }
+        float va[kBlock], vb[kBlock];
+        unpack16(c0, c1, va);
+        am[NB - TAIL] = block_amax(va);
+        gmax = fmaxf(gmax, am[NB - TAIL]);
+        if (TAIL == 2) {
+            unpack16(d0, d1, vb);
+            am[NB - 1] = block_amax(vb);
+            gmax = fmaxf(gmax, am[NB - 1]);
+        }
+        grid_max_arrive(gmax, sync, sh);
+        if (ia < nblocks) codes[ia] = encode_block<MODE, false>(va, block_scalar<MODE>(am[NB - TAIL]), none);
+        if (TAIL == 2 && ib < nblocks) codes[ib] = encode_block<MODE, false>(vb, block_scalar<MODE>(am[NB - 1]), none);
     }
+    auto scale_bytes = [&](float amax) {
+        const float unit = rd<MODE>(block_scalar<MODE>(amax) / 448.0f);      // quant.py:21-22
+#pragma unroll
+        for (int k = 0; k < NB; ++k) {
+            const uint32_t i = i0 + k * stride;
+            if (i < nblocks) scales[i] = (uint8_t)e4m3_byte(rd<MODE>(block_scalar<MODE>(am[k]) / unit));   // quant.py:23
+        }
+        return unit;
+    };
+    __syncthreads();                                               // thread 0 is through the tree: sh.last, sh.result
+    const uint32_t j = blockIdx.x % kGroups;
+    if (!sh.last) {
+        // ---- wait for the last workgroup's word, a bounded number of polls
+        if (threadIdx.x < 64) {
+            uint64_t w = 0;
+            uint32_t polls = 0;
+            bool have = false;
+            for (;;) {
+                w = METIS_AT_LOAD(sync_result(sync, j));
+                have = is_result(w, tag);
+                if (have || ++polls > spin_limit) break;
+                __builtin_amdgcn_s_sleep(2);
+            }
+            if (threadIdx.x == 0) {
+                sh.known = have ? 1u : 0u;
+                sh.result = __uint_as_float(((uint32_t)w & 0xffffu) << 16);
+            }
+        }
+        __syncthreads();
+        if (!sh.known) {
+            // ---- leave: park the block maxima, raise the flag, tell the group's word -- unless the result is there by now
+#pragma unroll
+            for (int k = 0; k < NB; ++k) {
+                const uint32_t i = i0 + k * stride;
+                if (i < nblocks) parked[i] = (uint16_t)(__float_as_uint(am[k]) >> 16);
+            }
+            __threadfence();
+            __syncthreads();
+            if (threadIdx.x == 0) {
+                METIS_AT_STORE(sync_left_flag(sync, blockIdx.x), (uint32_t)tag);
+                __threadfence();                                   // maxima and flag are out before the marker can be seen
+                uint64_t w = METIS_AT_LOAD(sync_result(sync, j));
+                for (;;) {
+                    if (is_result(w, tag)) {
+                        sh.known = 1u;
+                        sh.result = __uint_as_float(((uint32_t)w & 0xffffu) << 16);
+                        break;
+                    }
+                    if (is_left_marker(w, tag) || METIS_AT_CAS(sync_result(sync, j), &w, result_word(tag, 1u, 0u))) break;
+                }
+            }
+            __syncthreads();
+            if (!sh.known) return;                                 // the last workgroup writes this workgroup's scale bytes
+        }
+        scale_bytes(sh.result);
+        return;
+    }
+    // ---- the last workgroup to arrive: publish, then look after workgroups that have left
+    const float amax = sh.result;
+    const uint32_t ngroups = gridDim.x < kGroups ? gridDim.x : kGroups;
+    bool somebody_left = false;
+    if (threadIdx.x < ngroups)
+        somebody_left = is_left_marker(METIS_AT_XCHG(sync_result(sync, threadIdx.x), result_word(tag, 0u, __float_as_uint(amax) >> 16)), tag);
+    if (threadIdx.x == 0) sh.nleft = 0u;
+    const float unit = scale_bytes(amax);
+    if (threadIdx.x == 0) *unit_out = unit;
+    if (__syncthreads_or(somebody_left)) {
+        __threadfence();                                           // their parked maxima and flags were out before their markers
+        for (uint32_t slab = 0; slab < gridDim.x; slab += 256u) {
+            const uint32_t b = slab + threadIdx.x;
+            if (b < gridDim.x && METIS_AT_LOAD(sync_left_flag(sync, b)) == (uint32_t)tag) sh.left[atomicAdd(&sh.nleft, 1u)] = b;
+            __syncthreads();
+            const uint32_t nd = sh.nleft;
+            for (uint32_t d = 0; d < nd; ++d) {
+                const uint32_t base = sh.left[d] * 256u + threadIdx.x;
+#pragma unroll
+                for (int k = 0; k < NB; ++k) {
+                    const uint32_t i = base + k * stride;
+                    if (i < nblocks) {
+                        const float a = __uint_as_float((uint32_t)parked[i] << 16);
+                        scales[i] = (uint8_t)e4m3_byte(rd<MODE>(block_scalar<MODE>(a) / unit));
+                    }
+                }
+            }
+            __syncthreads();
+            if (threadIdx.x == 0) sh.nleft = 0u;
+            __syncthreads();
+        }
+    }
+    if (threadIdx.x == 0) METIS_AT_STORE(sync_generation(sync), tag);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -547,7 +630,7 @@ static int try_fused(const void* x, void* codes, void* scales, float* unit, cons
     const int64_t need = ((int64_t)nblocks + 256 * NB - 1) / (256 * NB);
     if (cap <= 0 || need > cap) return 1;                      // does not fit: caller picks another path
     hipLaunchKernelGGL((quant_fused_kernel<MODE, NB>), dim3((unsigned)need), dim3(256), 0, st, (const uint16_t*)x,
-                       (uint2*)codes, (uint8_t*)scales, unit, ws.sync, nblocks, spin_limit);
+                       (uint2*)codes, (uint8_t*)scales, unit, ws.sync, ws.amax, nblocks, spin_limit);
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 

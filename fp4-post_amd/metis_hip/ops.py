@@ -123,9 +123,9 @@ def quantize(x: torch.Tensor, mode: int = MODE_P32, *, col: bool = False, sr: bo
                overrides the internal Philox stream keyed by (seed, offset).
     center   : [C] vector subtracted from every row first (the reference's mean mode), in the arithmetic's
                dtype: the packed tensor is that of x - center.
-    resident : round-to-nearest rows of a bf16 tensor as ONE launch (metis_nvfp4_quant_row_resident): the caller
-               guarantees that nothing else keeps the launch's workgroups from being resident together.  A wait
-               that gives up after `spin_limit` polls (0: library default) leaves a NaN unit.
+    resident : round-to-nearest rows of a bf16 tensor as ONE launch (metis_nvfp4_quant_row_resident), same bytes: a
+               workgroup that gives up waiting for the grid's maximum after `spin_limit` polls (0: library default)
+               leaves its scale bytes to the last workgroup.
     """
     x2, kmode = _as_2d_for_quant(x, mode)
     rows, cols = x2.shape

@@ -10,6 +10,11 @@ column-blocked and binary32-input quantizers, the skinny (decode) GEMM, the spli
 the kernels of the mean mode.
 
     rocprofv3 --kernel-trace --stats -- python3 fp4-post_amd/metis_hip/tools/profile_workload.py --extra
+
+`--decode` runs the four grouped GEMM calls of one 7B-class decoder layer at 64 tokens (q/k/v, o, gate/up, down) next to
+the same calibration copy: the decode leg of the benchmark.
+
+    rocprofv3 --pmc FETCH_SIZE       -- python3 fp4-post_amd/metis_hip/tools/profile_workload.py --decode
 """
 import os
 import sys
@@ -29,6 +34,9 @@ def main(reps: int = 5):
     w = (torch.randn(14336, 4096, generator=g) * 0.02).bfloat16().cuda()
     t = torch.randn(8192, 64, generator=g).bfloat16().cuda()
     u = torch.randn(14336, 64, generator=g).bfloat16().cuda()
+    v = (torch.randn(64, 4096, generator=g) / 64).bfloat16().cuda()
+    s = torch.rand(64, generator=g).bfloat16().cuda()
+    dy = (torch.randn(8192, 14336, generator=g) * 1e-3).bfloat16().cuda()
     y = torch.empty_like(x)
     pw = ops.quantize(w)
     pw.persistent = True                                                # a cached weight: the pipelined GEMM on tiled expansions
@@ -38,6 +46,8 @@ def main(reps: int = 5):
         ops.rmsnorm_quantize(h, gamma, 1e-6)
         ops.linear_fwd(px, pw, t=t, u=u)                                # expand_xt_kernel + gemm_xt_kernel
         ops.linear_fwd(px, pw, t=t, u=u, tiled=False, split_k=False)    # gemm_nvfp4_large_kernel (expansion inside the K loop)
+        _, t_ = ops.lowrank_project(x, v, s)                            # lowrank_nt_kernel: x V^T and (x V^T) * s
+        ops.lowrank_contract_tokens(dy, t_)                             # lowrank_tn_kernel + finish: dY^T t
     torch.cuda.synchronize()
     del px, pw, y
     torch.cuda.synchronize()
@@ -85,5 +95,29 @@ def extra(reps: int = 5):
     torch.cuda.synchronize()
 
 
+def decode(reps: int = 5):
+    g = torch.Generator().manual_seed(1005)
+    x = torch.randn(8192, 4096, generator=g).bfloat16().cuda()
+    y = torch.empty_like(x)
+    groups = []
+    for k, ns in ((3584, (3584, 512, 512)), (3584, (3584,)), (3584, (18944, 18944)), (18944, (3584,))):
+        a = ops.quantize(torch.randn(64, k, generator=g).bfloat16().cuda())
+        members = [(ops.quantize((torch.randn(n, k, generator=g) * 0.02).bfloat16().cuda()), torch.randn(64, 64, generator=g).bfloat16().cuda(),
+                    torch.randn(n, 64, generator=g).bfloat16().cuda(), None) for n in ns]
+        groups.append((a, members))
+    for _ in range(reps):
+        y.copy_(x)                                                      # calibration: 64 MiB read, 64 MiB written
+        for a, members in groups:
+            ops.linear_fwd_grouped(a, members)
+    torch.cuda.synchronize()
+    del groups, y
+    torch.cuda.synchronize()
+
+
 if __name__ == "__main__":
-    extra() if "--extra" in sys.argv[1:] else main()
+    if "--extra" in sys.argv[1:]:
+        extra()
+    elif "--decode" in sys.argv[1:]:
+        decode()
+    else:
+        main()

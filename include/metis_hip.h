@@ -98,16 +98,18 @@ int metis_nvfp4_quant_row_static(const void *x, int64_t rows, int64_t cols, int6
                                  void *codes, void *scales, float *unit, void *stream);
 
 /*
- * metis_nvfp4_quant_row (contiguous rows) as ONE launch when every workgroup of that launch can be resident on
- * the device at once: block maxima stay in registers across a grid-wide maximum taken through tagged words of
- * the workspace, so neither the parked maxima nor the second kernel are needed.  Same bytes as
- * metis_nvfp4_quant_row.  Tensors too large for one resident launch take the two-launch path.
- * Opt-in because the caller has to guarantee what the library cannot see: for the duration of the call no
- * other kernel may keep its workgroups from becoming resident (in particular no second call of this entry
- * point on another stream).  The grid-wide wait is bounded: after `spin_limit` polls (0 = the default of 2^20,
- * about a second) a workgroup gives up, every wave still exits, *unit is NaN (scale bytes 0x7F) and the
- * workspace stays poisoned -- every later call on it also yields a NaN unit -- until the caller zero-fills
- * it again.  Same arithmetic as quant.py:6-36; the reference has no counterpart for the launch structure.
+ * metis_nvfp4_quant_row (contiguous rows, round to nearest) as ONE launch: block maxima stay in registers across a
+ * grid-wide maximum taken through a small tree of device-scope atomics in the workspace, so in the ordinary case
+ * neither the parked maxima nor the second kernel are needed.  Same bytes as metis_nvfp4_quant_row, always: a
+ * workgroup that has polled for the grid's maximum `spin_limit` times (0 = the default of 4096, a few milliseconds)
+ * without seeing it -- because part of the grid still waits for a compute unit that another kernel, or these very
+ * pollers, hold -- parks its block maxima, leaves, and the last workgroup to arrive writes its scale bytes for it.
+ * Every wave exits after a bounded time whatever else runs on the device.  Tensors too large for one launch of at
+ * most 4096 workgroups with 8 blocks per thread take the two-launch path.
+ * The workspace's reduction area (see metis_nvfp4_workspace_bytes) must be zero when first used and must not be
+ * shared by calls that overlap in time; a call leaves it ready for the next one.  Measured on MI355X the single
+ * launch is as fast as the two launches, not faster (the atomics' round trips cost what the second launch costs), so
+ * it is not the default.  Same arithmetic as quant.py:6-36; the reference has no counterpart for the launch structure.
  */
 int metis_nvfp4_quant_row_resident(const void *x, int64_t rows, int64_t cols, int mode, void *codes,
                                    void *scales, float *unit, void *workspace, size_t workspace_bytes,
