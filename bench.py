@@ -29,11 +29,27 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_PEAK_TFLOPS = 2516.6      # dense bf16/fp16 MFMA: 256 CU x 4096 flop/clk x 2.4 GHz
 QUANT_BYTES_PER_ELT = 2.5625   # 2 B read + 0.5 B codes + 1/16 B scale
 NORMQ_BYTES_PER_ELT = 4.5625   # + 2 B normed
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this workload, scaled by what the
-# same counters read for a 64 MiB copy (x2.0 reads, x1.0 writes); summary in profiles/hbm_traffic_pmc_config1_2_3.md
-TRAFFIC_GEMM_C3 = 653.6e6
-TRAFFIC_QUANT_C1 = 94.8e6
-TRAFFIC_NORMQ_C2 = 324.0e6
+# HBM bytes per launch.  NOT measured in this run: constants from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# fp4-post_amd/metis_hip/tools/profile_workload.py on the same shapes, scaled by what the same counters read for a
+# 64 MiB copy (x2.0 KiB per FETCH_SIZE unit, x1.0 KiB per WRITE_SIZE unit); summary in profiles/hbm_traffic_pmc.md
+TRAFFIC_SOURCE = ("profiles/hbm_traffic_pmc.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE on profile_workload.py, "
+                  "calibrated by a 64 MiB copy); a constant, not measured in this run")
+TRAFFIC_GEMM_C3 = 1666.5e6      # gemm_xt_kernel: 1431.6 MB fetched (tiled f16 operands re-read below L2) + 234.9 MB written
+TRAFFIC_QUANT_C1 = 94.8e6       # quant_codes_contig_kernel 88.4 MB + quant_scales_kernel 6.4 MB
+TRAFFIC_NORMQ_C2 = 323.8e6      # rmsnorm_quant_kernel 311.1 MB + quant_scales_kernel 12.7 MB
+TRAFFIC_DECODE_C5 = 160.8e6     # the five launches of the decode layer: 150.8 MB fetched + 10.0 MB written
+
+
+def cpu_model() -> str:
+    try:
+        with open("/proc/cpuinfo") as f:
+            for ln in f:
+                if ln.lower().startswith("model name"):
+                    return ln.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    import platform
+    return platform.processor() or "unknown"
 
 
 def outlier_activation(torch, seed, rows, cols, device):
@@ -301,7 +317,7 @@ def main():
                    "us_per_layer": round(d_us, 1), "tflops": round(d_flops / d_us / 1e6, 1),
                    "roofline": {"bound": "hbm", "kernel": "gemm_nvfp4_skinny_grouped_kernel", "achieved": round(d_bytes / d_us / 1e3, 1),
                                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(d_bytes / d_us / 1e3 / HBM_PEAK_GBS, 4),
-                                "traffic": None},
+                                "traffic": TRAFFIC_DECODE_C5, "traffic_source": TRAFFIC_SOURCE},
                    "mean_mode_us_per_layer": round(d_mean_us, 1)}
         except Exception as exc:  # an optional leg must not cost the headline line
             dec = {"workload": "config 5 decode", "error": f"{type(exc).__name__}: {exc}"[:300]}
@@ -538,19 +554,20 @@ def main():
                    "parity_mode": "P32", "parity_rel_fro_256_rows": err},
         "roofline": {"bound": "mfma", "kernel": "gemm_xt_kernel", "achieved": round(gemm_tflops, 2),
                      "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(gemm_tflops / MFMA_PEAK_TFLOPS, 4),
-                     "traffic": TRAFFIC_GEMM_C3, "kernel_ms": round(gemm_ms, 4)},
+                     "traffic": TRAFFIC_GEMM_C3, "traffic_source": TRAFFIC_SOURCE, "kernel_ms": round(gemm_ms, 4)},
         "quant": {"workload": "config 1: NVFP4 RNE quantize bf16 [8192,4096] (P32), codes+scales+unit",
                   "value": round(q_gbs, 1), "unit": "GB/s", "us_per_call": round(q_ms * 1e3, 2),
-                  "roofline": {"bound": "hbm", "kernel": "quant_codes_kernel+quant_scales_kernel",
+                  "roofline": {"bound": "hbm", "kernel": "quant_codes_contig_kernel+quant_scales_kernel",
                                "achieved": round(q_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                               "frac": round(q_gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_QUANT_C1},
-                  "single_launch_opt_in": {"value": round(q1_gbs, 1), "unit": "GB/s", "us_per_call": round(q1_ms * 1e3, 2),
+                               "frac": round(q_gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_QUANT_C1, "traffic_source": TRAFFIC_SOURCE},
+                  "single_launch": {"value": round(q1_gbs, 1), "unit": "GB/s", "us_per_call": round(q1_ms * 1e3, 2),
                                            "frac": round(q1_gbs / HBM_PEAK_GBS, 4)}},
         "rmsnorm_quant": {"workload": "config 2: fused RMSNorm->NVFP4 bf16 [16384,4096] (P32), normed+codes+scales",
                           "value": round(n_gbs, 1), "unit": "GB/s", "us_per_call": round(n_ms * 1e3, 2),
                           "roofline": {"bound": "hbm", "kernel": "rmsnorm_quant_kernel+quant_scales_kernel",
                                        "achieved": round(n_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                                       "frac": round(n_gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_NORMQ_C2}},
+                                       "frac": round(n_gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_NORMQ_C2,
+                                       "traffic_source": TRAFFIC_SOURCE}},
     }
     if dec is not None:
         line["decode_layer"] = dec
@@ -565,7 +582,7 @@ def main():
         cpu_tflops, cpu_dt, cpu_reps = cpu_baseline_linear(torch, x, v, s, u, res)
         q_torch, q_c, c_threads = cpu_baseline_quant(torch, x1)
         line["cpu_baseline"] = {
-            "value": round(cpu_tflops, 4), "unit": "TFLOP/s", "cores": torch_threads, "kind": "port",
+            "value": round(cpu_tflops, 4), "unit": "TFLOP/s", "cores": torch_threads, "kind": "port", "cpu_model": cpu_model(),
             "sample": f"oracle metis_forward (PyTorch CPU eager restatement of the reference) on the first 2048 of "
                       f"8192 rows incl. QDQ of the full residual weight each pass, {cpu_reps} passes, {cpu_dt:.1f} s",
             "quant_GBps_torch_eager": round(q_torch, 2), "quant_GBps_c_port": round(q_c, 2),
