@@ -151,6 +151,12 @@ int metis_nvfp4_expand_tiled_rht(const void* codes, const void* scales, const fl
     return expand_xt(codes, scales, unit, rows, cols, mode, out, (hipStream_t)stream, rotate_back != 0, sign_mask);
 }
 
+int metis_dense_expand_tiled(const void* x, int64_t rows, int64_t cols, int64_t ld, int dtype, const void* col_scale, int mode, void* out,
+                             void* stream)
+{
+    return dense_xt(x, rows, cols, ld, dtype, col_scale, mode, out, (hipStream_t)stream);
+}
+
 int metis_nvfp4_quant_row_rht(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, uint32_t sign_mask, int sr, uint64_t seed,
                               uint64_t offset, void* codes, void* scales, float* unit, void* workspace, size_t workspace_bytes,
                               void* stream)

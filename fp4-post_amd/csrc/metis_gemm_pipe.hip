@@ -163,6 +163,77 @@ __global__ __launch_bounds__(256) void expand_xt_t_kernel(const uint2* __restric
     }
 }
 
+// A dense [R, K] tensor (bf16 or binary32, row stride ld) in the same tiled layout: binary16 (PB16 = 0: one rounding of
+// each value; no prescale, so the caller passes 2^-8 as this operand's unit to cancel the 2^8 the GEMM applies for an
+// exact expansion) or bf16 (PB16 = 1).  col_scale (optional, bf16 [K]) multiplies column
+// k first, rounded to the tensor's dtype as `weight * s.unsqueeze(0)` rounds (src/Metis/Metis/bitlinear.py:727).
+// The dense operand of the merged rollout forward (705-751): U diag(s) and the merged weight itself.
+template <int PB16, int F32>
+__global__ __launch_bounds__(256) void dense_xt_kernel(const void* __restrict__ xv, int64_t ld, const uint16_t* __restrict__ col_scale,
+                                                       uint4* __restrict__ out, int rows, int K, int row_tiles)
+{
+    const int lane = threadIdx.x & 63;
+    const int kt = K / 32;
+    const int q = lane >> 2, chunk = (lane & 3) ^ xt_swz(q);
+    const int64_t ntiles = (int64_t)row_tiles * kt;
+    for (int64_t tile = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); tile < ntiles; tile += (int64_t)gridDim.x * 4) {
+        const int rb_ = (int)(tile / kt), kb = (int)(tile - (int64_t)rb_ * kt);
+        const int row = rb_ * 16 + q, k0 = kb * 32 + chunk * 8;
+        uint4 v = make_uint4(0u, 0u, 0u, 0u);
+        if (row < rows) {
+            float f[8];
+            if (F32) {
+                const float4* p = reinterpret_cast<const float4*>(static_cast<const float*>(xv) + (int64_t)row * ld + k0);
+                const float4 a = p[0], b = p[1];
+                f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+            } else {
+                const uint4 w = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(xv) + (int64_t)row * ld + k0);
+                f[0] = bf16_lo(w.x); f[1] = bf16_hi(w.x); f[2] = bf16_lo(w.y); f[3] = bf16_hi(w.y);
+                f[4] = bf16_lo(w.z); f[5] = bf16_hi(w.z); f[6] = bf16_lo(w.w); f[7] = bf16_hi(w.w);
+            }
+            if (col_scale) {
+                const uint4 w = *reinterpret_cast<const uint4*>(col_scale + k0);
+                const float sc[8] = {bf16_lo(w.x), bf16_hi(w.x), bf16_lo(w.y), bf16_hi(w.y), bf16_lo(w.z), bf16_hi(w.z), bf16_lo(w.w), bf16_hi(w.w)};
+#pragma unroll
+                for (int j = 0; j < 8; ++j) f[j] = F32 ? f[j] * sc[j] : rb(f[j] * sc[j]);
+            }
+            if constexpr (PB16 != 0) {
+                v.x = rb_pair(f[0], f[1]); v.y = rb_pair(f[2], f[3]); v.z = rb_pair(f[4], f[5]); v.w = rb_pair(f[6], f[7]);
+            } else {
+                const half2_t h0 = {(_Float16)f[0], (_Float16)f[1]}, h1 = {(_Float16)f[2], (_Float16)f[3]};
+                const half2_t h2 = {(_Float16)f[4], (_Float16)f[5]}, h3 = {(_Float16)f[6], (_Float16)f[7]};
+                v.x = __builtin_bit_cast(uint32_t, h0); v.y = __builtin_bit_cast(uint32_t, h1);
+                v.z = __builtin_bit_cast(uint32_t, h2); v.w = __builtin_bit_cast(uint32_t, h3);
+            }
+        }
+        out[tile * 64 + lane] = v;
+    }
+}
+
+int dense_xt(const void* x, int64_t rows, int64_t cols, int64_t ld, int dtype, const void* col_scale, int mode, void* out, hipStream_t st)
+{
+    if (rows < 0 || cols < 0 || ld < cols) return METIS_E_ARG;
+    if (mode == METIS_MODE_P32_F32) mode = METIS_MODE_P32;
+    if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) return METIS_E_ARG;
+    if (dtype != METIS_DTYPE_BF16 && dtype != METIS_DTYPE_F32) return METIS_E_ARG;
+    if (cols % 32) return METIS_E_SHAPE;
+    if (rows > INT32_MAX - 16 || cols > INT32_MAX) return METIS_E_ARG;
+    if (rows == 0 || cols == 0) return METIS_OK;
+    const int al = dtype == METIS_DTYPE_F32 ? 4 : 8;
+    if (!x || !out || (ld % al) || ((uintptr_t)x % 16) || ((uintptr_t)out % 16) || ((uintptr_t)col_scale % 16)) return METIS_E_ARG;
+    const int row_tiles = (int)((rows + 15) / 16);
+    const int64_t ntiles = (int64_t)row_tiles * (cols / 32);
+    int64_t g = (ntiles + 3) / 4;
+    const int64_t cap = (int64_t)device_cus() * 16;
+    if (g > cap) g = cap;
+#define METIS_DX(P, F) hipLaunchKernelGGL((dense_xt_kernel<P, F>), dim3((unsigned)g), dim3(256), 0, st, x, ld, (const uint16_t*)col_scale, \
+                                          (uint4*)out, (int)rows, (int)cols, row_tiles)
+    if (mode == METIS_MODE_PB16) { if (dtype == METIS_DTYPE_F32) METIS_DX(1, 1); else METIS_DX(1, 0); }
+    else { if (dtype == METIS_DTYPE_F32) METIS_DX(0, 1); else METIS_DX(0, 0); }
+#undef METIS_DX
+    return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
+}
+
 size_t expand_xt_bytes(int64_t rows, int64_t cols)
 {
     if (rows <= 0 || cols <= 0) return 0;

@@ -126,6 +126,8 @@ int gemm_expanded(const void* a_exp, const float* a_unit, const void* b_exp, con
 size_t expand_xt_bytes(int64_t rows, int64_t cols);
 int expand_xt(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, int mode, void* out,
               hipStream_t st, int rht = 0, uint32_t sign_mask = 0);
+// a dense bf16 / binary32 tensor in the tiled layout (optional per-column bf16 scale first)
+int dense_xt(const void* x, int64_t rows, int64_t cols, int64_t ld, int dtype, const void* col_scale, int mode, void* out, hipStream_t st);
 // the tiled operand [cols, rows] (contraction over the packed tensor's rows); rows % 32 == 0
 int expand_xt_transposed(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, int mode, void* out,
                          hipStream_t st, int rht, uint32_t sign_mask);

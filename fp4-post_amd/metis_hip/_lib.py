@@ -48,6 +48,7 @@ SIGNATURES = {
     "metis_nvfp4_expand_tiled_bytes": (_sz, [_i64, _i64]),
     "metis_nvfp4_expand_tiled": (_i32, [_vp, _vp, _vp, _i64, _i64, _i32, _vp, _vp]),
     "metis_linear_tiled_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32]),
+    "metis_dense_expand_tiled": (_i32, [_vp, _i64, _i64, _i64, _i32, _vp, _i32, _vp, _vp]),
     "metis_hadamard16": (_i32, [_vp, _i64, _i64, _i64, _i32, _i32, ctypes.c_uint32, _vp, _i64, _vp]),
     "metis_nvfp4_quant_row_rht": (_i32, [_vp, _i64, _i64, _i64, _i32, ctypes.c_uint32, _i32, _u64, _u64, _vp, _vp, _vp, _vp, _sz, _vp]),
     "metis_nvfp4_expand_tiled_rht": (_i32, [_vp, _vp, _vp, _i64, _i64, _i32, ctypes.c_uint32, _i32, _i32, _vp, _vp]),

@@ -619,12 +619,13 @@ class _MetisFusedFunction(torch.autograd.Function):
         F = LinearLowbitFunction
         cd = torch.bfloat16
         x2 = _flat2d(x).to(cd)
-        # [L, r] rank-r projection and its product with s (bf16): own split-K kernel for decode-sized batches,
-        # the vendor library's GEMM otherwise
+        # [L, r] rank-r projection and its product with s (bf16) on the library's kernels (split-K below 256 rows,
+        # one pass over x from there on)
         xv, t = ops.lowrank_project(x2, v.to(cd), s.to(cd))
         out_dtype = torch.float32 if F.compute_dtype == torch.float32 else torch.bfloat16
         ctx.center = None
-        gemm_bias = None if bias is None else bias.to(cd)
+        # binary32 arithmetic keeps a binary32 bias (as LinearLowbit and the centred path do); bf16 arithmetic adds it in bf16
+        gemm_bias = None if bias is None else (bias.float() if F.compute_dtype == torch.float32 else bias.to(cd))
         if isinstance(px, CenteredNVFP4):
             # mean mode: the residual branch sees 1 me^T + R
             ctx.center = px.mean
@@ -749,6 +750,7 @@ class BitLinear(nn.Module):
         self.mean_cache = {}
         self.activation_group = None
         self._merged_rollout_weight_cache = None
+        self._merged_rollout_tiled = None
         self.layer_name = ""
 
     # ------------------------------------------------------------------ shared activation (reference 676-702)
@@ -785,14 +787,51 @@ class BitLinear(nn.Module):
         def deq(q):
             return q.dequantize(dtype) if isinstance(q, PackedNVFP4) else q
 
-        v_weight = deq(self.vlinear._get_quantized_weight(self.vlinear.weight.to(dtype)))
+        qv = self.vlinear._get_quantized_weight(self.vlinear.weight.to(dtype))
         residual = deq(self.warmup_linear._get_quantized_weight(self.warmup_linear.weight.to(dtype)))
-        merged = (self.ulinear.weight.to(dtype) * self.s.to(dtype).unsqueeze(0)) @ v_weight + residual
+        us = self.ulinear.weight.to(dtype) * self.s.to(dtype).unsqueeze(0)
+        r = us.shape[1]
+        if (dtype == torch.bfloat16 and isinstance(qv, PackedNVFP4) and qv.rht is None and qv.mode == ops.MODE_PB16 and r % 32 == 0
+                and qv.cols % 4 == 0):
+            # bf16 arithmetic (the rollout's own configuration): the rank-r product on the tiled GEMM, bf16 operands,
+            # binary32 accumulation, one rounding to bf16 -- what the reference's bf16 matmul computes; Q(V)^T [K, r] is
+            # the transposed tiled expansion of the packed V
+            low = ops.gemm_tiled(ops.dense_expand_tiled(us, ops.MODE_PB16), qv.unit, ops.expand_tiled_transposed(qv, mode=ops.MODE_PB16),
+                                 qv.unit, us.shape[0], qv.cols, r, mode=ops.MODE_PB16, out_dtype=torch.bfloat16)
+            merged = low + residual
+        else:
+            merged = us @ deq(qv) + residual
         self._merged_rollout_weight_cache = (key, merged)
+        self._merged_rollout_tiled = None
         return merged
+
+    def _rollout_forward(self, shared_input, x_shape):
+        """y = QDQ(x) . merged^T (+ bias), the reference's one-matmul rollout forward (752-757).  bf16 arithmetic with a
+        packed activation: the tiled GEMM on the activation's bf16 expansion and the merged weight as a dense tiled
+        operand (cached with it), rounding the product and the bias add to bf16 as the reference's bf16 ops do.
+        Otherwise the reference's formula on dequantized tensors."""
+        F = LinearLowbitFunction
+        bias = self.warmup_linear.bias
+        if (isinstance(shared_input, PackedNVFP4) and shared_input.mode == ops.MODE_PB16 and shared_input.rht is None
+                and F.compute_dtype == torch.bfloat16 and shared_input.cols % 32 == 0 and self.warmup_linear.weight.shape[0] % 4 == 0):
+            merged = self._get_merged_rollout_weight(torch.bfloat16)
+            if self._merged_rollout_tiled is None:
+                self._merged_rollout_tiled = ops.dense_expand_tiled(merged, ops.MODE_PB16)
+            y = ops.gemm_tiled(ops.expand_tiled(shared_input, cache=False, mode=ops.MODE_PB16), shared_input.unit, self._merged_rollout_tiled,
+                               shared_input.unit, shared_input.rows, merged.shape[0], shared_input.cols, mode=ops.MODE_PB16,
+                               bias=None if bias is None else bias.to(torch.bfloat16), out_dtype=torch.bfloat16)
+            return y.reshape(*x_shape[:-1], merged.shape[0])
+        if isinstance(shared_input, (PackedNVFP4, CenteredNVFP4)):
+            shared_input = shared_input.dequantize(F.compute_dtype).reshape(x_shape)
+        merged = self._get_merged_rollout_weight(shared_input.dtype)
+        y = torch.matmul(shared_input, merged.T)
+        if bias is not None:
+            y = y + bias.to(y.dtype)
+        return y
 
     def _apply(self, fn, recurse=True):
         self._merged_rollout_weight_cache = None
+        self._merged_rollout_tiled = None
         self._bias_cast_cache = None
         group = getattr(self, "activation_group", None)
         if group is not None:
@@ -905,13 +944,7 @@ class BitLinear(nn.Module):
                     return _MetisFusedFunction.apply(x, self.vlinear.weight, self.s, self.ulinear.weight,
                                                      self.warmup_linear.weight, self.warmup_linear.bias, shared_input, p_res)
             if BitLinear.rollout_merge_active and not torch.is_grad_enabled():
-                if isinstance(shared_input, (PackedNVFP4, CenteredNVFP4)):
-                    shared_input = shared_input.dequantize(F.compute_dtype).reshape(x.shape)
-                merged = self._get_merged_rollout_weight(shared_input.dtype)
-                y = torch.matmul(shared_input, merged.T)
-                if self.warmup_linear.bias is not None:
-                    y = y + self.warmup_linear.bias.to(y.dtype)
-                return y
+                return self._rollout_forward(shared_input, x.shape)
             y = self.vlinear(x, quantized_input=shared_input)
         else:
             F.mean_cache_key = f"{self.layer_name}.vlinear"

@@ -391,6 +391,24 @@ def expand_tiled_transposed(p: PackedNVFP4, cache: bool = False, mode: int = MOD
     return out
 
 
+def dense_expand_tiled(x: torch.Tensor, mode: int = MODE_P32, col_scale: torch.Tensor | None = None) -> torch.Tensor:
+    """A dense [rows, cols] bf16 or float32 tensor as a tiled GEMM operand (see expand_tiled): binary16 values in mode
+    P32 (pair it with a unit of 2^-8, see gemm_tiled), bf16 values in mode PB16.  col_scale (bf16 [cols]) multiplies
+    column k first."""
+    if x.dim() != 2 or x.dtype not in (torch.bfloat16, torch.float32) or not x.is_cuda:
+        raise ValueError("dense_expand_tiled: a 2-D bf16 or float32 device tensor")
+    if x.stride(1) != 1 or x.data_ptr() % 16 or x.stride(0) % (4 if x.dtype == torch.float32 else 8):
+        x = x.contiguous()
+    rows, cols = x.shape
+    L = load()
+    out = torch.empty(L.metis_nvfp4_expand_tiled_bytes(rows, cols), dtype=torch.uint8, device=x.device)
+    cs = None if col_scale is None else col_scale.to(torch.bfloat16).contiguous()
+    rc = L.metis_dense_expand_tiled(x.data_ptr(), rows, cols, x.stride(0), DTYPE_F32 if x.dtype == torch.float32 else DTYPE_BF16,
+                                    None if cs is None else cs.data_ptr(), mode, out.data_ptr(), _stream())
+    check(rc, "metis_dense_expand_tiled", (rows, cols))
+    return out
+
+
 @functools.lru_cache(maxsize=4096)
 def _tiled_workspace_bytes(M: int, N: int, K: int, mode: int, device_index: int) -> int:
     return int(load().metis_linear_tiled_workspace_bytes(M, N, K, mode))

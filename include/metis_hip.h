@@ -255,6 +255,20 @@ int metis_nvfp4_expand_tiled(const void *codes, const void *scales, const float 
 size_t metis_linear_tiled_workspace_bytes(int64_t M, int64_t N, int64_t K, int mode);
 
 /*
+ * A dense tensor as a tiled GEMM operand: x [rows, cols] bf16 or float (dtype METIS_DTYPE_*, row stride ld) in the layout
+ * of metis_nvfp4_expand_tiled, each value rounded once to binary16 (mode METIS_MODE_P32; pass a device float 2^-8 as this
+ * operand's unit to metis_linear_fwd_tiled, which multiplies by 2^16 for two exact expansions) or to bf16
+ * (METIS_MODE_PB16).  col_scale (bf16 [cols], 16-byte aligned, or NULL) multiplies column k first, rounded to x's dtype.
+ * For the merged rollout forward of src/Metis/Metis/bitlinear.py:705-751: the merged weight
+ * (U diag(s)) Q(V) + Q(W_res) is a dense matrix, and the rollout multiplies the dequantized activation by it --
+ * here metis_linear_fwd_tiled on the activation's tiled expansion and this operand.
+ *   limits  cols % 32 == 0; x and out 16-byte aligned; ld % 8 == 0 (bf16) or % 4 (float); out holds
+ *           metis_nvfp4_expand_tiled_bytes(rows, cols) bytes
+ */
+int metis_dense_expand_tiled(const void *x, int64_t rows, int64_t cols, int64_t ld, int dtype,
+                             const void *col_scale, int mode, void *out, void *stream);
+
+/*
  * NV recipe (tiled random Hadamard rotation, tile = 16 = the scale block) on the packed kernels.
  * The reference rotates a tensor tile by tile along its last dimension, (x * sign) H with the Sylvester matrix H_16 and
  * one shared sign vector (src/Metis/Metis/bitlinear.py:75-137, 199-202), quantizes and dequantizes the rotated tensor,

@@ -4,6 +4,7 @@ Run once, in the build container only (the reference checkout does not exist on 
 
     python tests/golden/make_golden.py [/root/reference]
     python tests/golden/make_golden.py /root/reference hadamard_wide     (only metis_reference_hadamard_wide.npz)
+    python tests/golden/make_golden.py /root/reference rollout_bf16      (only metis_reference_rollout_bf16.npz)
 
 Why an import and not only closed forms: the results recorded here depend on the exact
 sequence of per-op roundings of eager PyTorch (bf16-per-op mode differs from an ideal
@@ -331,8 +332,62 @@ def golden_rollout(out: dict):
     out["ro_y_three_gemm"] = bits(y_three)
 
 
+def golden_rollout_bf16(out: dict):
+    """The rollout shortcut with bf16 tensors and bf16 arithmetic (the GRPO configuration), rank 32, 256 tokens: merged
+    weight and the one-matmul forward, assembled by hand as in golden_rollout."""
+    g = torch.Generator().manual_seed(53)
+    B, T, K, N, r = 2, 128, 128, 96, 32
+    dt = torch.bfloat16
+    x = torch.randn(B, T, K, generator=g).bfloat16()
+    w = (torch.randn(N, K, generator=g) * 0.05).bfloat16().float()
+    b = (torch.randn(N, generator=g) * 0.1).bfloat16()
+    args = SimpleNamespace(device="cpu", cache_quantized_weight=True, forward_svd_rank=r)
+    _configure("nvfp4e2m1bnosr", "nvfp4e2m1bnosr", "nvfp4e2m1b", dt)
+    try:
+        bl = rb.BitLinear.__new__(rb.BitLinear)
+        torch.nn.Module.__init__(bl)
+        bl.args = args
+        bl.is_svd_quant = True
+        bl.mean_cache = {}
+        bl.activation_group = None
+        bl._merged_rollout_weight_cache = None
+        bl.layer_name = "golden.rollout16"
+        bl.vlinear = rb.LinearLowbit(K, r, bias=False, args=args, storage_dtype=dt, compute_dtype=dt)
+        bl.ulinear = torch.nn.Linear(r, N, bias=False, dtype=dt)
+        bl.warmup_linear = rb.LinearLowbit(K, N, bias=True, args=args, storage_dtype=dt, compute_dtype=dt)
+        U, S, Vh = torch.linalg.svd(w, full_matrices=False)
+        with torch.no_grad():
+            bl.vlinear.weight.copy_(Vh[:r].bfloat16())
+            bl.ulinear.weight.copy_(U[:, :r].bfloat16())
+            bl.s = torch.nn.Parameter(S[:r].bfloat16().clone())
+            bl.warmup_linear.weight.copy_((w - (U[:, :r] * S[:r]) @ Vh[:r]).bfloat16())
+            bl.warmup_linear.bias.copy_(b)
+        with torch.no_grad():
+            rb.BitLinear.rollout_merge_active = True
+            try:
+                y_merged = bl(x)
+                merged_w = bl._get_merged_rollout_weight(dt)
+            finally:
+                rb.BitLinear.rollout_merge_active = False
+        assert y_merged.dtype == dt and merged_w.dtype == dt
+        out["ro16_x"], out["ro16_b"] = bits(x), bits(b)
+        out["ro16_v"], out["ro16_u"] = bits(bl.vlinear.weight.detach()), bits(bl.ulinear.weight.detach())
+        out["ro16_s"], out["ro16_res"] = bits(bl.s.detach()), bits(bl.warmup_linear.weight.detach())
+        out["ro16_merged_weight"] = bits(merged_w)
+        out["ro16_y_merged"] = bits(y_merged)
+    finally:
+        rb.LinearLowbitFunction.compute_dtype = torch.float32
+
+
 def main():
     torch.set_num_threads(1)
+    if len(sys.argv) > 2 and sys.argv[2] == "rollout_bf16":     # only this file (the others are not touched)
+        ro16: dict = {}
+        golden_rollout_bf16(ro16)
+        path = os.path.join(HERE, "metis_reference_rollout_bf16.npz")
+        np.savez_compressed(path, **ro16)
+        print(f"wrote {path}: {len(ro16)} arrays, {os.path.getsize(path)} bytes")
+        return
     if len(sys.argv) > 2 and sys.argv[2] == "hadamard_wide":    # only this file (the others are not touched)
         hw: dict = {}
         golden_hadamard_wide(hw)

@@ -283,6 +283,61 @@ def test_rollout_merged_weight_against_reference_vectors():
     assert rel_fro(three.cpu(), t(z["ro_y_three_gemm"])) <= 1e-5
 
 
+def test_rollout_in_bf16_arithmetic_runs_on_the_tiled_gemm_against_reference_vectors():
+    """The rollout shortcut as GRPO runs it (bf16 tensors, bf16 arithmetic, rank 32, 256 tokens): the merged weight's
+    rank-r product and the one-matmul forward run on the tiled GEMM with bf16 operands (no torch matmul), rounding
+    where the reference's bf16 ops round.  Against vectors the reference wrote: the merged weight to a bf16 ulp of its
+    largest entries, the output within 2e-3."""
+    import os
+    import numpy as np
+    from metis_hip import BitLinear, LinearLowbit, LinearLowbitFunction as F, MetisArgs, ops
+    z = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "metis_reference_rollout_bf16.npz"))
+    x, b = t(z["ro16_x"]), t(z["ro16_b"])
+    v, u, s, res = t(z["ro16_v"]), t(z["ro16_u"]), t(z["ro16_s"]), t(z["ro16_res"])
+    r, K = v.shape
+    N = u.shape[0]
+    dt = torch.bfloat16
+    args = MetisArgs.direct_fp4(forward_svd_rank=r)
+    args.cache_quantized_weight = True
+    F.compute_dtype = dt
+    layer = BitLinear(K, N, args=args, bias=True, dtype=dt, compute_dtype=dt).cuda()
+    layer.warmup_linear = LinearLowbit(K, N, bias=True, args=args, device="cuda", storage_dtype=dt, compute_dtype=dt)
+    layer.vlinear = LinearLowbit(K, r, bias=False, args=args, device="cuda", storage_dtype=dt, compute_dtype=dt)
+    layer.ulinear = torch.nn.Linear(r, N, bias=False, device="cuda", dtype=dt)
+    with torch.no_grad():
+        layer.vlinear.weight.copy_(v)
+        layer.ulinear.weight.copy_(u)
+        layer.s = torch.nn.Parameter(s.clone().cuda())
+        layer.warmup_linear.weight.copy_(res)
+        layer.warmup_linear.bias.copy_(b)
+    layer.is_svd_quant = True
+    calls = []
+    real, real_mm = ops.gemm_tiled, torch.matmul
+    ops.gemm_tiled = lambda *a, **k: (calls.append("tiled"), real(*a, **k))[1]
+    torch.matmul = lambda *a, **k: (calls.append("torch"), real_mm(*a, **k))[1]
+    # the reference's current file feeds the rank-r branch the quantized activation and the quantized V; with that variant
+    # selected the rollout switch takes the merged-weight matmul exactly as the reference does
+    BitLinear.quantized_lowrank_branch = True
+    try:
+        with torch.no_grad():
+            BitLinear.rollout_merge_active = True
+            y = layer(x.cuda())
+            y2 = layer(x.cuda())
+            merged = layer._get_merged_rollout_weight(dt)
+    finally:
+        ops.gemm_tiled, torch.matmul = real, real_mm
+        BitLinear.rollout_merge_active = False
+        BitLinear.quantized_lowrank_branch = False
+        F.compute_dtype = torch.float32
+    assert layer._merged_rollout_tiled is not None
+    assert calls == ["tiled", "tiled", "tiled"]                 # merged weight once (cached), one GEMM per forward
+    want_w = t(z["ro16_merged_weight"]).float()
+    assert float((merged.float().cpu() - want_w).abs().max()) <= float(want_w.abs().max()) * 2.0 ** -8
+    assert rel_fro(merged.float().cpu(), want_w) <= 2e-3
+    assert y.dtype == dt and torch.equal(y, y2)
+    assert rel_fro(y.float().cpu(), t(z["ro16_y_merged"]).float()) <= 2e-3
+
+
 def test_packed_weight_cache_reuses_then_invalidates_on_the_device():
     """The weight cache holds the PACKED weight (and what hangs off it: the column-blocked packing for dgrad, the tiled
     expansion of the pipelined GEMM), keyed on Parameter._version as the reference keys its dequantized cache
