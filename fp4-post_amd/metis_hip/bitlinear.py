@@ -386,7 +386,7 @@ class LinearLowbitFunction(torch.autograd.Function):
         return gx, ops.linear_fwd(p_dyt, p_xt, t=t, u=u, out_dtype=gw_dtype)
 
     @staticmethod
-    def _packed_grads_nv(dy2, x2, pw, gx_dtype, gw_dtype):
+    def _packed_grads_nv(dy2, x2, pw, gx_dtype, gw_dtype, gx_lowrank=None):
         """(grad_input, grad_weight) of the NV recipe (reference 443-513 with 395-405, 495-501) without leaving the
         packed kernels.  The reference rotates dY and the saved (already quantized) input tile by tile along their
         last dimension, quantizes, dequantizes and rotates back, and multiplies the results:
@@ -395,7 +395,7 @@ class LinearLowbitFunction(torch.autograd.Function):
         16-bit expansion of a packed tensor with the rotation back applied block by block on the way: dY~ [L, N] and
         W~^T [K, N] for the input gradient (contraction over N), dY~^T [N, L] and X~^T [K, L] for the weight gradient
         (contraction over tokens; the expansion transposes).  Quantization blocks run along the last dimension, as the
-        reference's do."""
+        reference's do.  gx_lowrank = (t [L, r], u [K, r]) adds t u^T to grad_input inside the same launch."""
         F = LinearLowbitFunction
         cd = F.compute_dtype
         mask = pw.rht
@@ -403,15 +403,18 @@ class LinearLowbitFunction(torch.autograd.Function):
         L, N = dy2.shape
         K = x2.shape[1]
         pad = (-L) % 32                                        # the token contraction runs in steps of 32: zero rows add nothing
+        lt, lu = gx_lowrank if gx_lowrank is not None else (None, None)
         if pad:
             dy2 = torch.cat((dy2, dy2.new_zeros(pad, N)), dim=0)
             x2 = torch.cat((x2, x2.new_zeros(pad, K)), dim=0)
+            if lt is not None:
+                lt = torch.cat((lt, lt.new_zeros(pad, lt.shape[1])), dim=0)
         p_dy = F.q_backward_outputgrad.pack(dy2, arith=cd, rht=mask)
         xq = F.q_forward_input.pack(x2, arith=cd).dequantize(torch.float32 if cd == torch.float32 else torch.bfloat16)
         p_x = F.q_backward_input.pack(xq, arith=cd, rht=mask)
         a_dy = ops.expand_tiled(p_dy, cache=False, mode=gmode)
         b_wt = ops.expand_tiled_transposed(pw, cache=pw.persistent, mode=gmode)
-        gx = ops.gemm_tiled(a_dy, p_dy.unit, b_wt, pw.unit, L + pad, K, N, mode=gmode, out_dtype=gx_dtype)
+        gx = ops.gemm_tiled(a_dy, p_dy.unit, b_wt, pw.unit, L + pad, K, N, mode=gmode, t=lt, u=lu, out_dtype=gx_dtype)
         a_dyt = ops.expand_tiled_transposed(p_dy, mode=gmode)
         b_xt = ops.expand_tiled_transposed(p_x, mode=gmode)
         gw = ops.gemm_tiled(a_dyt, p_dy.unit, b_xt, p_x.unit, N, K, L + pad, mode=gmode, out_dtype=gw_dtype)
@@ -663,7 +666,13 @@ class _MetisFusedFunction(torch.autograd.Function):
         g_v = ops.lowrank_contract_tokens(x2, g_xv, transpose=True)         # [r, K]
         # residual branch on re-quantized operands
         qg = F.q_backward_outputgrad
-        if F._packed_backward_applies(L, N, dy2):
+        if F._packed_backward_applies(L, N, dy2) and ctx.p_res.rht is not None:
+            # NV recipe: rotated operands, blocks along the last dimension (see _packed_grads_nv)
+            ar = F.compute_dtype
+            dyq, xq_src = (_flat2d(dy), _flat2d(x)) if ar == torch.float32 else (dy2, x2)
+            gx, g_res = F._packed_grads_nv(dyq, xq_src, ctx.p_res, cd, torch.bfloat16 if res.dtype == torch.bfloat16 else torch.float32,
+                                           gx_lowrank=(g_xv, v.to(cd).T.contiguous()))
+        elif F._packed_backward_applies(L, N, dy2):
             ar = F.compute_dtype                               # arithmetic of the quantizers
             p_res_col = ctx.p_res.transposed                   # lives as long as the (cached) packed residual
             if p_res_col is None:
@@ -845,7 +854,7 @@ class BitLinear(nn.Module):
         """Packed residual weight for the fused launch, or None when the kernel path does not apply."""
         F = LinearLowbitFunction
         wl = self.warmup_linear
-        if not F.enable_nv_recipe and _packable(wl.weight, F.q_forward_weight) and wl.weight.shape[0] % 4 == 0:
+        if (not F.enable_nv_recipe or F._nv_on_kernels()) and _packable(wl.weight, F.q_forward_weight) and wl.weight.shape[0] % 4 == 0:
             p_res = wl._get_quantized_weight(wl.weight, arith=self.compute_dtype)       # cache hit: no pass over W
         else:
             p_res = wl._get_quantized_weight(wl.weight.to(self.compute_dtype))
@@ -867,7 +876,7 @@ class BitLinear(nn.Module):
         if rows >= 256 or not all(m._fusable() and m.compute_dtype == self.compute_dtype for m in members):
             return None
         packed = [m._packed_residual() for m in members]
-        if any(p is None for p in packed):
+        if any(p is None or p.rht is not None for p in packed):   # a rotated weight (NV recipe) needs the tiled GEMM's operands
             return None
         cd = torch.bfloat16
         x2 = _flat2d(x).to(cd)

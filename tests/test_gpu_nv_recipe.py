@@ -232,3 +232,46 @@ def test_nv_recipe_at_a_training_shape_keeps_the_packed_kernels_and_matches_the_
     # whose codes hang on the last bit of the rotation's sums (see the test above), and the two paths sum in different orders
     for (a, b), tol in zip(zip(outs["auto"], outs["torch_gemm"]), (2e-3, 2e-3, 3e-2)):
         assert rel_fro(a.cpu(), b.cpu()) <= tol
+
+
+def test_bitlinear_under_the_nv_recipe_is_the_rotated_residual_plus_the_rank_r_branch():
+    """BitLinear (rank 32) with enable_nv_recipe: the fused launch multiplies the quantized activation with the rotated,
+    quantized, rotated-back residual weight and adds the rank-r branch; its gradients are LinearLowbit's (pinned above
+    against the reference's vectors) plus the branch's share.  Checked against the pieces computed separately."""
+    from metis_hip import BitLinear, LinearLowbitFunction as F, MetisArgs, ops
+    F.enable_nv_recipe = True
+    K, N, r, L = 256, 192, 32, 320
+    args = MetisArgs.direct_fp4(forward_svd_rank=r)
+    args.enable_nv_recipe = True
+    args.q_backward_input = args.q_backward_weight = args.q_backward_outputgrad = "nvfp4e2m1bnosr"   # round to nearest: deterministic
+    layer = BitLinear(K, N, args=args, bias=False, dtype=torch.float32, compute_dtype=torch.float32).cuda()
+    with torch.no_grad():
+        layer.warmup_linear.weight.copy_(torch.randn(N, K, generator=torch.Generator().manual_seed(61)) * 0.05)
+    layer.split()
+    assert F.enable_nv_recipe and F._nv_on_kernels()
+    x = synthetic_activation(62, L, K).float().cuda().requires_grad_(True)
+    dy = (torch.randn(L, N, generator=torch.Generator().manual_seed(63)) * 1e-2).cuda()
+    calls = []
+    real = ops.gemm_tiled
+    ops.gemm_tiled = lambda *a, **k: (calls.append(1), real(*a, **k))[1]
+    try:
+        y = layer(x)
+        y.backward(dy)
+    finally:
+        ops.gemm_tiled = real
+    assert len(calls) == 3
+    mask = F._hadamard_mask()
+    v, u, s_ = layer.vlinear.weight.detach(), layer.ulinear.weight.detach(), layer.s.detach()
+    res = layer.warmup_linear.weight.detach()
+    pw = ops.quantize_rht(res, 0, mask)
+    w_back = pw.dequantize(torch.float32).double()
+    xq = ops.quantize(x.detach(), 0).dequantize(torch.float32).double()
+    tt = ((x.detach().bfloat16() @ v.bfloat16().T) * s_.bfloat16()).double()              # bf16 rank-r branch
+    want_y = xq @ w_back.T + tt @ u.bfloat16().double().T
+    assert rel_fro(y.detach().double().cpu(), want_y.cpu()) <= 2e-3
+    dy_back = ops.quantize_rht(dy, 0, mask).dequantize(torch.float32).double()
+    x_back = ops.quantize_rht(xq.float(), 0, mask).dequantize(torch.float32).double()
+    assert rel_fro(layer.warmup_linear.weight.grad.double().cpu(), (dy_back.T @ x_back).cpu()) <= 2e-3
+    g_xv = (dy.bfloat16() @ u.bfloat16()) * s_.bfloat16()                                   # [L, r]
+    want_gx = dy_back @ w_back + g_xv.double() @ v.bfloat16().double()
+    assert rel_fro(x.grad.double().cpu(), want_gx.cpu()) <= 2e-3
