@@ -171,6 +171,54 @@ static void check_linear(int64_t M, int64_t N, int64_t K, hipStream_t st, const 
     check(rc == METIS_OK && err <= 2e-3, line);
 }
 
+// The pipelined GEMM on tiled 16-bit expansions: metis_nvfp4_expand_tiled for both operands, metis_linear_fwd_tiled,
+// against the packed-operand GEMM on the same packed tensors (same products, binary32 sums in another order) and, with
+// the rotated quantizer, the NV recipe's round trip: quant_row_rht -> dequant -> hadamard16 (inverse) stays close to x.
+static void check_tiled(int64_t M, int64_t N, int64_t K, hipStream_t st)
+{
+    const std::vector<uint16_t> x = make_input(M, K, 21u, 1.0f), w = make_input(N, K, 22u, 0.02f);
+    DeviceBuffer<uint8_t> ac((size_t)(M * K / 2)), as((size_t)(M * K / 16)), bc((size_t)(N * K / 2)), bs((size_t)(N * K / 16));
+    DeviceBuffer<float> au(1), bu(1);
+    quantize_on_device(x, M, K, METIS_MODE_P32, st, &ac, &as, &au);
+    quantize_on_device(w, N, K, METIS_MODE_P32, st, &bc, &bs, &bu);
+    DeviceBuffer<uint8_t> ax(metis_nvfp4_expand_tiled_bytes(M, K)), bx(metis_nvfp4_expand_tiled_bytes(N, K));
+    int rc = metis_nvfp4_expand_tiled(ac.p, as.p, au.p, M, K, METIS_MODE_P32, ax.p, st);
+    if (rc == METIS_OK) rc = metis_nvfp4_expand_tiled(bc.p, bs.p, bu.p, N, K, METIS_MODE_P32, bx.p, st);
+    DeviceBuffer<float> out_t((size_t)(M * N)), out_p((size_t)(M * N));
+    const size_t need = metis_linear_tiled_workspace_bytes(M, N, K, METIS_MODE_P32);
+    DeviceBuffer<uint8_t> ws(need ? need : 16);
+    if (rc == METIS_OK)
+        rc = metis_linear_fwd_tiled(ax.p, au.p, bx.p, bu.p, M, N, K, nullptr, nullptr, 0, nullptr, 0, out_t.p, METIS_DTYPE_F32, METIS_MODE_P32,
+                                    need ? ws.p : nullptr, need, st);
+    if (rc == METIS_OK) rc = metis_linear_fwd(ac.p, as.p, au.p, bc.p, bs.p, bu.p, M, N, K, nullptr, nullptr, 0, nullptr, out_p.p, METIS_DTYPE_F32, st);
+    HIP_OK(hipStreamSynchronize(st));
+    const std::vector<float> t = out_t.download(), q = out_p.download();
+    std::vector<double> got(t.begin(), t.end()), want(q.begin(), q.end());
+    char line[200];
+    snprintf(line, sizeof line, "metis_nvfp4_expand_tiled + metis_linear_fwd_tiled %ldx%ldx%ld rc=%d vs metis_linear_fwd rel.err %.2e",
+             (long)M, (long)N, (long)K, rc, rel_fro(got, want));
+    check(rc == METIS_OK && rel_fro(got, want) <= 1e-6, line);
+
+    // NV recipe round trip on the activation (sign mask 0x5a3c: any mask is a valid rotation)
+    DeviceBuffer<uint16_t> dx(x.size()), deq(x.size()), back(x.size());
+    dx.upload(x);
+    const size_t wsb = metis_nvfp4_workspace_bytes(M, K);
+    DeviceBuffer<uint8_t> qws(wsb);
+    HIP_OK(hipMemset(qws.p, 0, wsb));
+    rc = metis_nvfp4_quant_row_rht(dx.p, M, K, K, METIS_MODE_PB16, 0x5a3cu, 0, 0, 0, ac.p, as.p, au.p, qws.p, wsb, st);
+    if (rc == METIS_OK) rc = metis_nvfp4_dequant(ac.p, as.p, au.p, M, K, METIS_MODE_PB16, deq.p, METIS_DTYPE_BF16, st);
+    if (rc == METIS_OK) rc = metis_hadamard16(deq.p, M, K, K, METIS_DTYPE_BF16, 1, 0x5a3cu, back.p, K, st);
+    HIP_OK(hipStreamSynchronize(st));
+    const std::vector<uint16_t> b = back.download();
+    std::vector<double> g2(b.size()), w2(b.size());
+    for (size_t i = 0; i < b.size(); ++i) { g2[i] = bf16_to_f32(b[i]); w2[i] = bf16_to_f32(x[i]); }
+    snprintf(line, sizeof line, "metis_nvfp4_quant_row_rht -> dequant -> metis_hadamard16 (inverse) rc=%d rel.err to x %.3f (FP4 level)", rc,
+             rel_fro(g2, w2));
+    check(rc == METIS_OK && rel_fro(g2, w2) < 0.2, line);
+    check(metis_nvfp4_quant_row_rht(dx.p, M, K, K, METIS_MODE_PB16, 0x10000u, 0, 0, 0, ac.p, as.p, au.p, qws.p, wsb, st) == METIS_E_ARG,
+          "a sign mask wider than 16 bits -> METIS_E_ARG");
+}
+
 // Mean mode at decode size: column mean (with the running update) -> centred quantizer -> grouped GEMM with the
 // centre inside, and the packed matrix-vector product, all against double precision on the host.
 static void check_mean_mode_decode(hipStream_t st)
@@ -362,6 +410,10 @@ int main()
     check_linear(272, 320, 256, st, "tiled 256x256");
     check_linear(96, 132, 96, st, "tiled 128x128");
     check_linear(48, 160, 512, st, "skinny");
+
+    // ---- 4b: the pipelined GEMM on tiled expansions, and the rotated quantizer
+    check_tiled(272, 320, 256, st);
+    check_tiled(512, 256, 2048, st);
 
     // ---- 6: split-K through a caller workspace
     check_linear(256, 256, 2048, st, "tiled, K split", true);
