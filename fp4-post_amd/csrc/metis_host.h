@@ -10,7 +10,7 @@ namespace metis {
 
 // Caller-supplied scratch, carved as:
 //   [0, 16 KiB)        one partial maximum (uint32 bit pattern) per workgroup of phase 1
-//   [16 KiB, +65 KiB)  grid-wide reduction words of the single-launch quantizer (zero when idle)
+//   [16 KiB, +65 KiB)  reduction area of the single-launch quantizer (zero when first used)
 //   [81 KiB, ..)       one block maximum per block of 16: bf16 for bf16 input, binary32 for binary32 input
 struct Workspace {
     uint32_t* gmax;
@@ -18,7 +18,7 @@ struct Workspace {
     uint16_t* amax;
 };
 constexpr size_t kWsGmaxBytes = 4096 * 4;
-constexpr size_t kWsSyncBytes = 260 * 256;     // 1 KiB header + 4096 member words + 64 x 64 group-maximum copies, 8 bytes each
+constexpr size_t kWsSyncBytes = 260 * 256;     // reduction area of the single-launch quantizer: header, 65 tree nodes and 64 result words on lines of their own, 4096 flags (33 KiB used)
 
 inline size_t workspace_bytes(int64_t rows, int64_t cols)
 {
