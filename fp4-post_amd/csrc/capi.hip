@@ -275,6 +275,14 @@ int metis_linear_fwd_grouped(const void* a_codes, const void* a_scales, const fl
                               (hipStream_t)stream, workspace, workspace_bytes);
 }
 
+int metis_linear_fwd_grouped_bf16(const void* a_codes, const void* a_scales, const float* a_unit, int64_t M, int64_t K,
+                                  const metis_linear_member* members, int count, int out_dtype, void* workspace,
+                                  size_t workspace_bytes, void* stream)
+{
+    return gemm_nvfp4_grouped(a_codes, a_scales, a_unit, M, K, reinterpret_cast<const GemmMember*>(members), count, out_dtype,
+                              (hipStream_t)stream, workspace, workspace_bytes, nullptr, true);
+}
+
 int metis_linear_fwd_grouped_centered(const void* a_codes, const void* a_scales, const float* a_unit, int64_t M, int64_t K,
                                       const metis_linear_member* members, int count, int out_dtype, const float* center,
                                       void* workspace, size_t workspace_bytes, void* stream)

@@ -71,6 +71,28 @@ __device__ __forceinline__ half8_t run_operand(const RunRegs<C>& r, int m)
     return __builtin_bit_cast(half8_t, expand8(w, scale_pair(byte)));
 }
 
+// The same operand as the reference's bf16 arithmetic dequantizes it: bf16(bf16(e4m3 * unit) * e2m1), eight bf16 values
+// (src/Metis/Metis/quant.py:33-36 evaluated in bf16, as under compute_dtype = bfloat16 in src/grpo/grpo.py:204-205).
+template <int C>
+__device__ __forceinline__ bf16x8_t run_operand_bf16(const RunRegs<C>& r, int m, float unit)
+{
+    typedef float float2_t __attribute__((ext_vector_type(2)));
+    const uint4 q = r.c[m >> 2];
+    const uint32_t w = (m & 3) == 0 ? q.x : (m & 3) == 1 ? q.y : (m & 3) == 2 ? q.z : q.w;
+    const uint32_t byte = (r.sc[m >> 3] >> (8 * ((m >> 1) & 3))) & 0xffu;
+    const float dq = rb(e4m3_value(byte) * unit);
+    const float2_t p0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 0);
+    const float2_t p1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 1);
+    const float2_t p2 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 2);
+    const float2_t p3 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 3);
+    uint4 o;
+    o.x = rb_pair(p0[0] * dq, p0[1] * dq);
+    o.y = rb_pair(p1[0] * dq, p1[1] * dq);
+    o.z = rb_pair(p2[0] * dq, p2[1] * dq);
+    o.w = rb_pair(p3[0] * dq, p3[1] * dq);
+    return __builtin_bit_cast(bf16x8_t, o);
+}
+
 // One weight matrix of a grouped decode-sized call, and the group: the column tiles (32 columns each) of the members are
 // laid end to end.
 constexpr int kMaxGroupMembers = 4;

@@ -587,7 +587,14 @@ static int launch_large(const void* a_codes, const void* a_scales, const float* 
 // operand that has just been expanded: a pseudo activation tile whose even rows are hi and odd rows lo.  The packed
 // weight is read once for R W^T and for the rank-one term 1 (W^ me)^T, at the cost of half as many MFMAs again
 // on a kernel that is bound elsewhere.
-template <int TM, int C, int WAVES, int OUT_F32, int CEN = 0>
+//
+// PB16: the layer's arithmetic is bf16 and the forward follows the reference's all-bf16 evaluation
+// (src/Metis/Metis/bitlinear.py:435-438 under compute_dtype = bfloat16, src/grpo/grpo.py:204-205): both operands are its
+// twice-rounded bf16 dequantized values (bf16 MFMA, no unit factor), the residual product is rounded to bf16 as its
+// bf16 matmul rounds it, the bias is added in bf16, then the low-rank term and one final rounding.  The low-rank
+// products therefore stay apart from the residual sums: they pass through the reduction buffer a second time (K slice 0
+// leaves them as one more partial in slot nsplit when K is split).
+template <int TM, int C, int WAVES, int OUT_F32, int CEN = 0, int PB16 = 0>
 __device__ __forceinline__ void skinny_tile(
     const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const float* __restrict__ a_unit,
     const uint8_t* __restrict__ b_codes, const uint8_t* __restrict__ b_scales, const float* __restrict__ b_unit,
@@ -644,15 +651,24 @@ __device__ __forceinline__ void skinny_tile(
         }
         __syncthreads();
     }
+    static_assert(!(PB16 != 0 && CEN != 0), "the centre rides on exact binary16 operands");
+    const float ua = PB16 ? *a_unit : 0.0f, ub = PB16 ? *b_unit : 0.0f;
     for (int it = s0 + wave * iters / WAVES; it < it1; ++it) {
-        RunRegs<C> rb;
-        load_run<C>(rb, bc + (int64_t)it * 32 * C, bs + it * 4 * C);
+        RunRegs<C> rw;
+        load_run<C>(rw, bc + (int64_t)it * 32 * C, bs + it * 4 * C);
         RunRegs<C> ra[TM];
 #pragma unroll
         for (int i = 0; i < TM; ++i) load_run<C>(ra[i], ac[i] + (int64_t)it * 32 * C, as[i] + it * 4 * C);
 #pragma unroll
         for (int m = 0; m < 4 * C; ++m) {
-            const half8_t fb = run_operand<C>(rb, m);
+            if constexpr (PB16 != 0) {
+                const bf16x8_t fw = run_operand_bf16<C>(rw, m, ub);
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+                    acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw, run_operand_bf16<C>(ra[i], m, ua), acc[i], 0, 0, 0);
+                continue;
+            }
+            const half8_t fb = run_operand<C>(rw, m);
             if constexpr (CEN != 0) {                          // the lane's run starts at element hi * 32 C of the iteration
                 const uint4* mp = reinterpret_cast<const uint4*>(mes) + ((((it - s0) * 64 * C + hi * 32 * C) >> 3) + m) * 2 + (lane & 1);
                 accm = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb, __builtin_bit_cast(half8_t, *mp), accm, 0, 0, 0);
@@ -662,12 +678,14 @@ __device__ __forceinline__ void skinny_tile(
                 acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb, run_operand<C>(ra[i], m), acc[i], 0, 0, 0);
         }
     }
-    // tensor units (and the 2^8 * 2^8 of the scale placement)
-    const float us = (*a_unit) * (*b_unit) * 65536.0f;
+    if constexpr (PB16 == 0) {
+        // tensor units (and the 2^8 * 2^8 of the scale placement)
+        const float us = (*a_unit) * (*b_unit) * 65536.0f;
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) acc[i][e] *= us;
+            for (int e = 0; e < 16; ++e) acc[i][e] *= us;
+    }
     if constexpr (CEN != 0) {
         // the rank-one term: every output row gets W^ me.  accm[e] holds it for this lane's column n(e), split over
         // the lane pair (hi part, lo part); the expanded operand carries 2^-8, the centre 2^-4, and the tensor unit
@@ -683,41 +701,30 @@ __device__ __forceinline__ void skinny_tile(
         __syncthreads();                                       // all waves are done with the staged centre: red is free
     }
     // bf16 low-rank extension: slices of 32 columns dealt to the waves (K slice 0 only)
-    for (int j0 = wave * 32; j0 < (slice == 0 ? r : 0); j0 += WAVES * 32) {
+    auto lowrank_into = [&](float16_t (&dst)[TM]) {
+        for (int j0 = wave * 32; j0 < (slice == 0 ? r : 0); j0 += WAVES * 32) {
 #pragma unroll
-        for (int q = 0; q < 2; ++q) {
-            const int j = j0 + q * 16 + hi * 8;
-            const bf16x8_t fu = *reinterpret_cast<const bf16x8_t*>(u + (int64_t)nrow * r + j);
+            for (int q = 0; q < 2; ++q) {
+                const int j = j0 + q * 16 + hi * 8;
+                const bf16x8_t fu = *reinterpret_cast<const bf16x8_t*>(u + (int64_t)nrow * r + j);
 #pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                const int mrow = min(m0 + i * 32 + (lane & 31), M - 1);
-                const bf16x8_t ft = *reinterpret_cast<const bf16x8_t*>(t + (int64_t)mrow * ldt + j);
-                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fu, ft, acc[i], 0, 0, 0);
+                for (int i = 0; i < TM; ++i) {
+                    const int mrow = min(m0 + i * 32 + (lane & 31), M - 1);
+                    const bf16x8_t ft = *reinterpret_cast<const bf16x8_t*>(t + (int64_t)mrow * ldt + j);
+                    dst[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fu, ft, dst[i], 0, 0, 0);
+                }
             }
         }
-    }
+    };
+    if constexpr (PB16 == 0) lowrank_into(acc);
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int e = 0; e < 16; ++e) red[wave][i * 16 + e][lane] = acc[i][e];
     __syncthreads();
-    // acc[i][e] of lane l: m = 32 i + l % 32, n = 8 (e / 4) + 4 (l / 32) + e % 4.  One (i, e / 4, l) per thread.
-    for (int id = threadIdx.x; id < TM * 256; id += 64 * WAVES) {
-        const int l = id & 63, g = (id >> 6) & 3, i = id >> 8;
-        const int m = m0 + i * 32 + (l & 31), n = n0 + 8 * g + 4 * (l >> 5);
-        float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-        for (int w = 0; w < WAVES; ++w)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] += red[w][i * 16 + 4 * g + e][l];
-        if (m >= M || n >= N) continue;                        // N % 4 == 0 is required
-        if (part) {                                            // binary32 partial [nsplit][M][N]; the bias waits for the sum
-            *reinterpret_cast<float4*>(part + ((int64_t)slice * M + m) * N + n) = make_float4(v[0], v[1], v[2], v[3]);
-            continue;
-        }
-        if (bias)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] += bias_value(bias, bias_f32, n + e);
+    // acc[i][e] of lane l: m = 32 i + l % 32, n = 8 (e / 4) + 4 (l / 32) + e % 4.  One (i, e / 4, l) per thread and pass.
+    constexpr int NID = (TM * 256 + 64 * WAVES - 1) / (64 * WAVES);
+    auto store4 = [&](int m, int n, const float (&v)[4]) {
         if (OUT_F32) {
             *reinterpret_cast<float4*>((float*)out + (int64_t)m * N + n) = make_float4(v[0], v[1], v[2], v[3]);
         } else {
@@ -726,13 +733,92 @@ __device__ __forceinline__ void skinny_tile(
             w.y = bf16_bits(v[2]) | (bf16_bits(v[3]) << 16);
             *reinterpret_cast<uint2*>((uint16_t*)out + (int64_t)m * N + n) = w;
         }
+    };
+    float keep[NID][4];                                        // PB16: the rounded residual (+ bias) while the low-rank term is summed
+#pragma unroll
+    for (int p = 0; p < NID; ++p) {
+        const int id = threadIdx.x + p * 64 * WAVES;
+        const int l = id & 63, g = (id >> 6) & 3, i = min(id >> 8, TM - 1);
+        const int m = m0 + i * 32 + (l & 31), n = n0 + 8 * g + 4 * (l >> 5);
+        float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] += red[w][i * 16 + 4 * g + e][l];
+        const bool live = id < TM * 256 && m < M && n < N;     // N % 4 == 0 is required
+        if constexpr (PB16 != 0) {
+            if (!part) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    v[e] = rb(v[e]);                           // the reference's bf16 matmul result, then its bf16 bias add
+                    if (bias && live) v[e] = rb(v[e] + bias_value(bias, bias_f32, n + e));
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) keep[p][e] = v[e];
+        }
+        if (!live) continue;
+        if (part) {                                            // binary32 partial [nsplit][M][N]; the bias waits for the sum
+            *reinterpret_cast<float4*>(part + ((int64_t)slice * M + m) * N + n) = make_float4(v[0], v[1], v[2], v[3]);
+            continue;
+        }
+        if constexpr (PB16 == 0) {
+            if (bias)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] += bias_value(bias, bias_f32, n + e);
+            store4(m, n, v);
+        }
+    }
+    if constexpr (PB16 != 0) {
+        const bool low = r > 0 && slice == 0;                  // uniform over the workgroup
+        const int nlw = min(WAVES, r / 32);                    // waves that hold low-rank products
+        if (low) {
+            __syncthreads();                                   // the residual sums have been read: red is free
+            float16_t accl[TM];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) accl[i][e] = 0.0f;
+            lowrank_into(accl);
+            if (wave < nlw) {
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) red[wave][i * 16 + e][lane] = accl[i][e];
+            }
+            __syncthreads();
+        }
+        if (part && !low) return;
+#pragma unroll
+        for (int p = 0; p < NID; ++p) {
+            const int id = threadIdx.x + p * 64 * WAVES;
+            const int l = id & 63, g = (id >> 6) & 3, i = min(id >> 8, TM - 1);
+            const int m = m0 + i * 32 + (l & 31), n = n0 + 8 * g + 4 * (l >> 5);
+            if (id >= TM * 256 || m >= M || n >= N) continue;
+            float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (low) {
+                for (int w = 0; w < nlw; ++w)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] += red[w][i * 16 + 4 * g + e][l];
+            }
+            if (part) {                                        // the low-rank term of this tile: one more partial, slot nsplit
+                *reinterpret_cast<float4*>(part + ((int64_t)nsplit * M + m) * N + n) = make_float4(v[0], v[1], v[2], v[3]);
+                continue;
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                v[e] += keep[p][e];
+                if (OUT_F32) v[e] = rb(v[e]);                  // a binary32 buffer still receives bf16 values in this mode
+            }
+            store4(m, n, v);
+        }
     }
 }
 
 // Several weight matrices against ONE packed activation in one launch (q/k/v, gate/up): the column tiles of the
 // members are laid end to end along grid x.  A decode-sized k or v projection alone is 16 workgroups and costs a
 // whole launch latency; next to q it is free.
-template <int TM, int C, int WAVES, int OUT_F32, int CEN = 0>
+template <int TM, int C, int WAVES, int OUT_F32, int CEN = 0, int PB16 = 0>
 __global__ __launch_bounds__(64 * WAVES) void gemm_nvfp4_skinny_grouped_kernel(
     const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const float* __restrict__ a_unit, int M, int K,
     const SkinnyGroup grp)
@@ -747,14 +833,16 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nvfp4_skinny_grouped_kernel(
 #pragma unroll
     for (int i = 1; i < kMaxGroupMembers; ++i)
         if (g == i) mm = grp.m[i];
-    skinny_tile<TM, C, WAVES, OUT_F32, CEN>(a_codes, a_scales, a_unit, mm.b_codes, mm.b_scales, mm.b_unit, M, mm.N, K, mm.t, mm.u,
+    skinny_tile<TM, C, WAVES, OUT_F32, CEN, PB16>(a_codes, a_scales, a_unit, mm.b_codes, mm.b_scales, mm.b_unit, M, mm.N, K, mm.t, mm.u,
                                             mm.r, mm.bias, mm.out, mm.bias_f32, (tile - start) * 32, mm.ldt, mm.part, grp.nsplit,
                                             grp.center);
 }
 
 // Adds the K slices of the skinny kernel in ascending order, then bias and output conversion.
 // grid (column quads / 256, M, members).
-template <int OUT_F32>
+// PB16: the slices hold the residual product only; their sum is rounded to bf16, the bias added in bf16, then the
+// low-rank term (slot nsplit, members with r > 0) and the final rounding.
+template <int OUT_F32, int PB16 = 0>
 __global__ __launch_bounds__(256) void skinny_splitk_reduce_kernel(const SkinnyGroup grp, int M)
 {
     SkinnyMember mm = grp.m[0];
@@ -769,7 +857,18 @@ __global__ __launch_bounds__(256) void skinny_splitk_reduce_kernel(const SkinnyG
         const float4 p = *reinterpret_cast<const float4*>(src + (int64_t)z * M * mm.N);
         v.x += p.x; v.y += p.y; v.z += p.z; v.w += p.w;
     }
-    if (mm.bias) {
+    if constexpr (PB16 != 0) {
+        v.x = rb(v.x); v.y = rb(v.y); v.z = rb(v.z); v.w = rb(v.w);
+        if (mm.bias) {
+            v.x = rb(v.x + bias_value(mm.bias, mm.bias_f32, n));     v.y = rb(v.y + bias_value(mm.bias, mm.bias_f32, n + 1));
+            v.z = rb(v.z + bias_value(mm.bias, mm.bias_f32, n + 2)); v.w = rb(v.w + bias_value(mm.bias, mm.bias_f32, n + 3));
+        }
+        if (mm.r > 0) {
+            const float4 p = *reinterpret_cast<const float4*>(src + (int64_t)grp.nsplit * M * mm.N);
+            v.x += p.x; v.y += p.y; v.z += p.z; v.w += p.w;
+        }
+        if (OUT_F32) { v.x = rb(v.x); v.y = rb(v.y); v.z = rb(v.z); v.w = rb(v.w); }
+    } else if (mm.bias) {
         v.x += bias_value(mm.bias, mm.bias_f32, n);     v.y += bias_value(mm.bias, mm.bias_f32, n + 1);
         v.z += bias_value(mm.bias, mm.bias_f32, n + 2); v.w += bias_value(mm.bias, mm.bias_f32, n + 3);
     }
@@ -783,12 +882,17 @@ __global__ __launch_bounds__(256) void skinny_splitk_reduce_kernel(const SkinnyG
     }
 }
 
-static int launch_skinny_reduce(const SkinnyGroup& grp, int64_t M, int out_dtype, hipStream_t st)
+static int launch_skinny_reduce(const SkinnyGroup& grp, int64_t M, int out_dtype, hipStream_t st, bool pb16 = false)
 {
     int nmax = 0;
     for (int i = 0; i < grp.count; ++i) nmax = grp.m[i].N > nmax ? grp.m[i].N : nmax;
     const dim3 rgrid((unsigned)((nmax / 4 + 255) / 256), (unsigned)M, (unsigned)grp.count);
-    if (out_dtype == METIS_DTYPE_F32)
+    if (pb16) {
+        if (out_dtype == METIS_DTYPE_F32)
+            hipLaunchKernelGGL((skinny_splitk_reduce_kernel<1, 1>), rgrid, dim3(256), 0, st, grp, (int)M);
+        else
+            hipLaunchKernelGGL((skinny_splitk_reduce_kernel<0, 1>), rgrid, dim3(256), 0, st, grp, (int)M);
+    } else if (out_dtype == METIS_DTYPE_F32)
         hipLaunchKernelGGL(skinny_splitk_reduce_kernel<1>, rgrid, dim3(256), 0, st, grp, (int)M);
     else
         hipLaunchKernelGGL(skinny_splitk_reduce_kernel<0>, rgrid, dim3(256), 0, st, grp, (int)M);
@@ -797,10 +901,21 @@ static int launch_skinny_reduce(const SkinnyGroup& grp, int64_t M, int out_dtype
 
 template <int TM, int C, int WAVES>
 static int launch_skinny_grouped(const void* a_codes, const void* a_scales, const float* a_unit, int64_t M, int64_t K,
-                                 const SkinnyGroup& grp, int tiles, int out_dtype, hipStream_t st)
+                                 const SkinnyGroup& grp, int tiles, int out_dtype, hipStream_t st, bool pb16)
 {
     const bool split = grp.nsplit > 1;
     const dim3 grid((unsigned)tiles, (unsigned)((M + 32 * TM - 1) / (32 * TM)), (unsigned)(split ? grp.nsplit : 1)), block(64 * WAVES);
+    if (pb16) {                                                // the reference's all-bf16 evaluation
+        if (grp.center) return METIS_E_ARG;
+        if (out_dtype == METIS_DTYPE_F32)
+            hipLaunchKernelGGL((gemm_nvfp4_skinny_grouped_kernel<TM, C, WAVES, 1, 0, 1>), grid, block, 0, st, (const uint8_t*)a_codes,
+                               (const uint8_t*)a_scales, a_unit, (int)M, (int)K, grp);
+        else
+            hipLaunchKernelGGL((gemm_nvfp4_skinny_grouped_kernel<TM, C, WAVES, 0, 0, 1>), grid, block, 0, st, (const uint8_t*)a_codes,
+                               (const uint8_t*)a_scales, a_unit, (int)M, (int)K, grp);
+        if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
+        return split ? launch_skinny_reduce(grp, M, out_dtype, st, true) : METIS_OK;
+    }
     if constexpr (C == 4) {
         if (grp.center) {                                      // mean mode (wide runs only)
             if (out_dtype == METIS_DTYPE_F32)
@@ -837,7 +952,8 @@ static int skinny_split_factor(int64_t tiles, int64_t K, int c)
     return s < 1 ? 1 : (int)s;
 }
 
-// Workspace for the partial sums of a grouped call ([slices][M][N] binary32 per member); 0 = K is not split.
+// Workspace for the partial sums of a grouped call ([slices + 1][M][N] binary32 per member: bf16 arithmetic keeps the
+// low-rank term in a slot of its own); 0 = K is not split.
 size_t gemm_grouped_workspace_bytes(int64_t M, int64_t K, const GemmMember* members, int count)
 {
     if (!members || count < 1 || M <= 0 || M >= 256 || K <= 0 || K % 64) return 0;
@@ -849,7 +965,7 @@ size_t gemm_grouped_workspace_bytes(int64_t M, int64_t K, const GemmMember* memb
     }
     const int s1 = skinny_split_factor(tiles, K, 1), s4 = K % 256 == 0 ? skinny_split_factor(tiles, K, 4) : 1;
     const int s = s1 > s4 ? s1 : s4;                        // which run width applies depends on pointer alignment
-    return s <= 1 ? 0 : (size_t)s * (size_t)M * (size_t)ntot * sizeof(float);
+    return s <= 1 ? 0 : (size_t)(s + 1) * (size_t)M * (size_t)ntot * sizeof(float);
 }
 
 // One activation against up to four weight matrices.  Shapes the skinny kernel does not take fall back to one
@@ -893,10 +1009,11 @@ int gemm_grouped_center_supported(int64_t M, int64_t K, const GemmMember* member
 
 int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a_unit, int64_t M, int64_t K,
                        const GemmMember* members, int count, int out_dtype, hipStream_t st, void* workspace,
-                       size_t workspace_bytes, const float* center)
+                       size_t workspace_bytes, const float* center, bool pb16)
 {
     if (!members || count < 1) return METIS_E_ARG;
     if ((uintptr_t)center % 16) return METIS_E_ARG;
+    if (pb16 && center) return METIS_E_ARG;
     bool skinny = M > 0 && M < 256 && K % 64 == 0 && count <= kMaxGroupMembers && !measure_env("METIS_GEMM_SMALL") &&
                   a_codes && a_scales && a_unit && !((uintptr_t)a_codes % 16) && !((uintptr_t)a_scales % 2) && K <= INT32_MAX &&
                   (out_dtype == METIS_DTYPE_BF16 || out_dtype == METIS_DTYPE_F32);
@@ -913,7 +1030,7 @@ int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a
         ntot += g.N;
     }
     if (!skinny || tiles > INT32_MAX) {
-        if (center) return METIS_E_ARG;                        // the centre is only taken by the single-launch path
+        if (center || pb16) return METIS_E_ARG;                // the centre and the bf16 evaluation are only taken by the single-launch path
         for (int i = 0; i < count; ++i) {
             const GemmMember& g = members[i];
             if (g.ldt != 0 && g.ldt != g.r) return METIS_E_ARG;   // a strided t is only taken by the single-launch path
@@ -932,7 +1049,8 @@ int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a
             tm = ftm; c = fc; waves = fw; nsplit = fs;
         }
     }
-    if (nsplit > 1 && (((uintptr_t)workspace % 16) || workspace_bytes < (size_t)nsplit * (size_t)M * (size_t)ntot * sizeof(float)))
+    const size_t slots = (size_t)nsplit + (pb16 ? 1 : 0);      // bf16 arithmetic: one more for the low-rank term
+    if (nsplit > 1 && (((uintptr_t)workspace % 16) || workspace_bytes < slots * (size_t)M * (size_t)ntot * sizeof(float)))
         return METIS_E_WORKSPACE;
     if (center && !skinny_center_fits(SkinnyShape{c, tm, waves, nsplit}, K)) return METIS_E_ARG;
     SkinnyGroup grp = {};
@@ -947,9 +1065,9 @@ int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a
         grp.m[i] = SkinnyMember{(const uint8_t*)g.b_codes, (const uint8_t*)g.b_scales, g.b_unit, (const uint16_t*)g.t,
                                 (const uint16_t*)g.u, (const uint16_t*)g.bias, g.out, nsplit > 1 ? part : nullptr, (int)g.N,
                                 (int)g.r, end, g.bias_is_f32 != 0, (int)(g.ldt ? g.ldt : g.r)};
-        part += (size_t)nsplit * (size_t)M * (size_t)g.N;
+        part += slots * (size_t)M * (size_t)g.N;
     }
-#define METIS_SKG(TM, C, W) return launch_skinny_grouped<TM, C, W>(a_codes, a_scales, a_unit, M, K, grp, (int)tiles, out_dtype, st)
+#define METIS_SKG(TM, C, W) return launch_skinny_grouped<TM, C, W>(a_codes, a_scales, a_unit, M, K, grp, (int)tiles, out_dtype, st, pb16)
     if (tm == 1) {
         if (waves == 4) { if (c == 4) METIS_SKG(1, 4, 4); else METIS_SKG(1, 1, 4); }
         else { if (c == 4) METIS_SKG(1, 4, 8); else METIS_SKG(1, 1, 8); }

@@ -86,7 +86,7 @@ struct GemmMember {
 };
 int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a_unit, int64_t M, int64_t K,
                        const GemmMember* members, int count, int out_dtype, hipStream_t st, void* workspace = nullptr,
-                       size_t workspace_bytes = 0, const float* center = nullptr);
+                       size_t workspace_bytes = 0, const float* center = nullptr, bool pb16 = false);
 int gemm_grouped_center_supported(int64_t M, int64_t K, const GemmMember* members, int count, int have_workspace);
 // bytes of split-K scratch a grouped call can use (only the N fields of the members are read; 0: it would not split)
 size_t gemm_grouped_workspace_bytes(int64_t M, int64_t K, const GemmMember* members, int count);

@@ -70,6 +70,7 @@ SIGNATURES = {
     "metis_lowrank_tokens_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "metis_lowrank_contract_tokens": (_i32, [_vp, _i64, _vp, _i64, _i64, _i64, _vp, _i32, _i32, _vp, _sz, _vp]),
     "metis_linear_fwd_grouped": (_i32, [_vp, _vp, _vp, _i64, _i64, _vp, _i32, _i32, _vp, _sz, _vp]),
+    "metis_linear_fwd_grouped_bf16": (_i32, [_vp, _vp, _vp, _i64, _i64, _vp, _i32, _i32, _vp, _sz, _vp]),
     "metis_linear_grouped_workspace_bytes": (_sz, [_i64, _i64, _vp, _i32]),
     "metis_linear_fwd_grouped_centered": (_i32, [_vp, _vp, _vp, _i64, _i64, _vp, _i32, _i32, _vp, _vp, _sz, _vp]),
     "metis_linear_grouped_centered_supported": (_i32, [_i64, _i64, _vp, _i32, _i32]),

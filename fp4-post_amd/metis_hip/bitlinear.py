@@ -900,7 +900,7 @@ class BitLinear(nn.Module):
             c0 += r
         out_dtype = torch.float32 if F.compute_dtype == torch.float32 else torch.bfloat16
         # mean mode: every member also receives W^ me, inside the same launch (binary32)
-        outs = ops.linear_fwd_grouped(px, calls, out_dtype=out_dtype, center=centre)
+        outs = ops.linear_fwd_grouped(px, calls, out_dtype=out_dtype, center=centre, reference_rounding=F.reference_rounding)
         lead = x.shape[:-1]
         return {id(m): y.reshape(*lead, y.shape[-1]).to(F.compute_dtype) for m, y in zip(members, outs)}
 

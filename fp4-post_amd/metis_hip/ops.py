@@ -536,6 +536,11 @@ def _gemm_workspace(M: int, N: int, K: int, device: torch.device) -> torch.Tenso
     return torch.empty(need, dtype=torch.uint8, device=device) if need else None
 
 
+def _decode_kernel_takes(M: int, N: int, K: int, r: int) -> bool:
+    """Shapes of the decode-sized kernel (waves split K over packed operands streamed from global memory)."""
+    return 0 < M < 256 and K % 64 == 0 and N % 4 == 0 and r % 32 == 0
+
+
 def linear_fwd(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None, u: torch.Tensor | None = None,
                bias: torch.Tensor | None = None, out_dtype: torch.dtype = torch.bfloat16,
                expanded: bool | None = None, split_k: bool = True, tiled: bool | None = None,
@@ -545,8 +550,8 @@ def linear_fwd(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None,
     tiled=None picks the pipelined kernel on tiled binary16 expansions when b is a cached weight and the shape is
     large (see _tiled_applies); True / False force the choice.  Same bits either way (unsplit).
     reference_rounding: the forward of a layer whose arithmetic is bf16 (both operands packed in that mode): follow the
-    reference's all-bf16 evaluation (twice-rounded bf16 operands, residual product and bias add rounded to bf16), which
-    only the pipelined kernel implements; requests for fewer than 256 rows are served with exact products.
+    reference's all-bf16 evaluation (twice-rounded bf16 operands, residual product and bias add rounded to bf16): the
+    pipelined kernel from 256 rows on, the decode-sized kernel below (shapes it does not take get exact products).
 
     split_k=False withholds the split-K workspace: the contraction then runs unsplit in one launch.
 
@@ -559,12 +564,15 @@ def linear_fwd(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None,
         if a.cols % 32:
             raise ValueError("a rotated operand needs a contraction that is a multiple of 32")
         tiled = True
-    faithful = reference_rounding and a.mode == MODE_PB16 and b.mode == MODE_PB16 and (a.rows >= 256 or tiled) and a.cols % 32 == 0
+    rounded = reference_rounding and a.mode == MODE_PB16 and b.mode == MODE_PB16
+    faithful = rounded and (a.rows >= 256 or tiled) and a.cols % 32 == 0
     if tiled is None:
         tiled = faithful or (not expanded and _tiled_applies(a, b))
     if tiled:
         return linear_fwd_tiled(a, b, t=t, u=u, bias=bias, out_dtype=out_dtype, reference_rounding=faithful, split_k=split_k)
     M, N, K = a.rows, b.rows, a.cols
+    if rounded and not expanded and _decode_kernel_takes(M, N, K, 0 if t is None else t.shape[1]):
+        return _linear_fwd_grouped(a, [(b, t, u, bias)], out_dtype=out_dtype, split_k=split_k, reference_rounding=True)[0]
     dev = a.codes.device
     r = 0
     if t is not None:
@@ -668,15 +676,30 @@ def lowrank_contract_tokens(a: torch.Tensor, b: torch.Tensor, out_dtype: torch.d
 
 
 def linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.bfloat16,
-                       center: torch.Tensor | None = None, split_k: bool = True) -> list[torch.Tensor]:
+                       center: torch.Tensor | None = None, split_k: bool = True,
+                       reference_rounding: bool = False) -> list[torch.Tensor]:
+    return _linear_fwd_grouped(a, members, out_dtype, center, split_k, reference_rounding)
+
+
+def _linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.bfloat16,
+                        center: torch.Tensor | None = None, split_k: bool = True,
+                        reference_rounding: bool = False) -> list[torch.Tensor]:
     """[linear_fwd(a, b, t=t, u=u, bias=bias) for (b, t, u, bias) in members] in one call: a projection group
     (q/k/v, gate/up) that shares one packed activation.  Decode-sized batches run as a single launch.
+
+    reference_rounding (every operand packed in bf16 arithmetic, no centre): the reference's all-bf16 evaluation, as in
+    linear_fwd; shapes the decode-sized kernel does not take are served member by member.
 
     center (mean mode: `a` packs the centred residual X - center): every output row also receives deq(b) . center,
     inside the same launch where the shape allows, else through matvec and a binary32 bias."""
     import ctypes
     M, K = a.rows, a.cols
     dev = a.codes.device
+    rounded = (reference_rounding and center is None and a.mode == MODE_PB16 and all(m[0].mode == MODE_PB16 for m in members))
+    if rounded and not (len(members) <= 4 and all(_decode_kernel_takes(M, m[0].rows, K, 0 if m[1] is None else m[1].shape[1])
+                                                  for m in members)):
+        return [linear_fwd(a, b, t=t, u=u, bias=bias, out_dtype=out_dtype, split_k=split_k, reference_rounding=True)
+                for b, t, u, bias in members]
     arr = (_lib.LinearMember * len(members))()
     outs, keep = [], []
     for i, (b, t, u, bias) in enumerate(members):
@@ -728,10 +751,11 @@ def linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.b
         for b, t, u, bias in members:
             w_mean = matvec(b, center)
             shifted.append((b, t, u, w_mean if bias is None else w_mean + bias.float()))
-        return linear_fwd_grouped(a, shifted, out_dtype)
-    rc = L.metis_linear_fwd_grouped(a.codes.data_ptr(), a.scales.data_ptr(), a.unit.data_ptr(), M, K, ap, len(members),
-                                    dt, None if ws is None else ws.data_ptr(), need, _stream())
-    check(rc, "metis_linear_fwd_grouped", (M, K, [m[0].rows for m in members]))
+        return _linear_fwd_grouped(a, shifted, out_dtype)
+    fn = L.metis_linear_fwd_grouped_bf16 if rounded else L.metis_linear_fwd_grouped
+    rc = fn(a.codes.data_ptr(), a.scales.data_ptr(), a.unit.data_ptr(), M, K, ap, len(members),
+            dt, None if ws is None else ws.data_ptr(), need, _stream())
+    check(rc, "metis_linear_fwd_grouped_bf16" if rounded else "metis_linear_fwd_grouped", (M, K, [m[0].rows for m in members]))
     return outs
 
 

@@ -424,7 +424,18 @@ typedef struct metis_linear_member {
 int metis_linear_fwd_grouped(const void *a_codes, const void *a_scales, const float *a_unit, int64_t M,
                              int64_t K, const metis_linear_member *members, int count, int out_dtype,
                              void *workspace, size_t workspace_bytes, void *stream);
-/* Scratch for the call above: with few output columns and a long K (a down projection at decode size) K is cut
+/* The same call for a layer whose arithmetic is bf16 (both operands packed with METIS_MODE_PB16; compute_dtype =
+ * bfloat16 as src/grpo/grpo.py:204-205 configures every patched layer): result i follows the reference's all-bf16
+ * evaluation of LinearLowbitFunction.forward / BitLinear.forward (src/Metis/Metis/bitlinear.py:435-438, 752-760) the way
+ * metis_linear_tiled_fwd does with mode = METIS_MODE_PB16 -- operands are its twice-rounded bf16 dequantized values,
+ * the residual product is rounded to bf16, the bias added in bf16, then the low-rank term and the final rounding (a
+ * binary32 `out` receives bf16 values).  Decode-sized shapes only (M < 256, K % 64 == 0, N % 4 == 0, r % 32 == 0,
+ * count <= 4, the alignments of the call above): METIS_E_ARG otherwise -- larger batches run on
+ * metis_linear_tiled_fwd.  Workspace as above. */
+int metis_linear_fwd_grouped_bf16(const void *a_codes, const void *a_scales, const float *a_unit, int64_t M,
+                                  int64_t K, const metis_linear_member *members, int count, int out_dtype,
+                                  void *workspace, size_t workspace_bytes, void *stream);
+/* Scratch for the two calls above: with few output columns and a long K (a down projection at decode size) K is cut
  * into slices that run as separate workgroups, their binary32 partial sums meet in the workspace and a second
  * small kernel adds them in a fixed order.  Only the N fields of the members are read; the figure is an upper
  * bound (the number of slices also depends on pointer alignment, known only at the call).  0 = the shape is not

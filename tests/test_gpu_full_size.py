@@ -31,7 +31,7 @@ def _config():
 def _slab_reference(mod, xin, rows, mode):
     """Double-precision value of BitLinear.forward on rows `rows` of its input: deq(Q(x)) deq(Q(W_res))^T + t u^T + b, with
     t = bf16(bf16(x V^T) * s) as the module forms it.  Q(x) is taken over the WHOLE input (the tensor unit is global).
-    In bf16 arithmetic with 256 rows or more the module follows the reference's all-bf16 forward: operands are its
+    In bf16 arithmetic the module follows the reference's all-bf16 forward at every batch size: operands are its
     bf16 dequantized values, the residual product and the bias add are rounded to bf16."""
     import dataclasses
     from metis_hip import ops
@@ -42,7 +42,7 @@ def _slab_reference(mod, xin, rows, mode):
         # binary32 dequantizer returns those values
         return ops.dequantize(dataclasses.replace(p, mode=0), torch.float32)
     x2 = xin.reshape(-1, xin.shape[-1])
-    faithful = mode == MODE_PB16 and x2.shape[0] >= 256
+    faithful = mode == MODE_PB16
     px = ops.quantize(x2, mode)
     p_res = mod._packed_residual()
     if faithful:

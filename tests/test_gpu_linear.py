@@ -206,6 +206,48 @@ def test_tiled_path_with_reference_rounding_in_bf16_arithmetic(M, N, K, r, with_
     assert 5e-4 < rel_fro(exact.float().cpu(), want.float().cpu()) < 2e-2
 
 
+@pytest.mark.parametrize("M,N,K,r,with_bias", [(64, 4736, 3584, 64, True), (17, 2052, 2048, 0, True), (1, 4608, 3584, 32, False),
+                                               (40, 1536, 8960, 64, True), (64, 3584, 18944, 64, True), (200, 512, 1024, 32, True),
+                                               (33, 260, 192, 96, False), (64, 3584, 18944, 0, True)])
+def test_decode_shapes_with_reference_rounding_in_bf16_arithmetic(M, N, K, r, with_bias):
+    """Below 256 rows the decode-sized kernel serves reference_rounding: it expands both packed operands to the
+    reference's twice-rounded bf16 dequantized values in registers and rounds where the all-bf16 forward rounds (residual
+    product, bias add, final sum), also when K is cut into slices that meet in a second kernel (the two 18944-long
+    contractions).  Same check as for the pipelined kernel: that evaluation in double precision between the roundings."""
+    from metis_hip import ops
+    g = torch.Generator().manual_seed(6000 + M + N)
+    x = synthetic_activation(80 + M, M, K).cuda()
+    w = _weights(81 + N, N, K).cuda()
+    t = u = None
+    if r:
+        t = torch.randn(M, r, generator=g).bfloat16().cuda()
+        u = (torch.randn(N, r, generator=g) * 0.05).bfloat16().cuda()
+    bias = (torch.randn(N, generator=g) * 0.1).bfloat16().cuda() if with_bias else None
+    px, pw = ops.quantize(x, 1), ops.quantize(w, 1)
+    xq, wq = ops.dequantize(px, torch.bfloat16).double(), ops.dequantize(pw, torch.bfloat16).double()   # the reference's QDQ values
+    want = (xq @ wq.T).bfloat16()
+    if bias is not None:
+        want = (want.float() + bias.float()).bfloat16()
+    want = want.double()
+    if r:
+        want = want + t.double() @ u.double().T
+    want = want.bfloat16()
+    got = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, reference_rounding=True)
+    got32 = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, out_dtype=torch.float32, reference_rounding=True)
+    unsplit = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, reference_rounding=True, split_k=False)
+    grouped = ops.linear_fwd_grouped(px, [(pw, t, u, bias), (pw, None, None, None)], reference_rounding=True)
+    torch.cuda.synchronize()
+    assert torch.equal(got32, got.float())                       # a binary32 buffer receives the same bf16 values
+    assert (grouped[1] != (xq @ wq.T).bfloat16()).float().mean().item() < 2e-3     # a member without bias or low-rank term
+    for y in (got, unsplit, grouped[0]):                         # (a group has more column tiles: K may be sliced differently)
+        differ = (y != want).float().mean().item()
+        assert differ < 2e-3, f"{differ:.2e} of the outputs differ from the all-bf16 evaluation"
+        assert rel_fro(y.float().cpu(), want.float().cpu()) <= 2e-4
+    # the exact-product result is a different number: the two modes are not interchangeable
+    exact = ops.linear_fwd(px, pw, t=t, u=u, bias=bias, reference_rounding=False)
+    assert 5e-4 < rel_fro(exact.float().cpu(), want.float().cpu()) < 2e-2
+
+
 @pytest.mark.parametrize("M,N,K,r", [(64, 4736, 3584, 64), (17, 2052, 2048, 0), (1, 4608, 3584, 32), (40, 1536, 8960, 64),
                                      (64, 18944, 3584, 64)])
 def test_decode_shapes_with_lowrank_and_bias(M, N, K, r):
