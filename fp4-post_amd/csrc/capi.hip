@@ -151,6 +151,13 @@ int metis_nvfp4_expand_tiled_rht(const void* codes, const void* scales, const fl
     return expand_xt(codes, scales, unit, rows, cols, mode, out, (hipStream_t)stream, rotate_back != 0, sign_mask);
 }
 
+int metis_nvfp4_expand_tiled_centered(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols,
+                                      const void* center, void* out, void* stream)
+{
+    if (!center) return METIS_E_ARG;
+    return expand_xt(codes, scales, unit, rows, cols, METIS_MODE_PB16, out, (hipStream_t)stream, 0, 0, center);
+}
+
 int metis_dense_expand_tiled(const void* x, int64_t rows, int64_t cols, int64_t ld, int dtype, const void* col_scale, int mode, void* out,
                              void* stream)
 {
@@ -281,6 +288,23 @@ int metis_linear_fwd_grouped_bf16(const void* a_codes, const void* a_scales, con
 {
     return gemm_nvfp4_grouped(a_codes, a_scales, a_unit, M, K, reinterpret_cast<const GemmMember*>(members), count, out_dtype,
                               (hipStream_t)stream, workspace, workspace_bytes, nullptr, true);
+}
+
+size_t metis_nvfp4_decode_operand_bytes(int64_t rows, int64_t cols) { return skinny_operand_bytes(rows, cols); }
+
+int metis_nvfp4_decode_operand(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, int mode,
+                               const void* center, void* out, void* stream)
+{
+    return skinny_operand(codes, scales, unit, rows, cols, mode, center, out, (hipStream_t)stream);
+}
+
+int metis_linear_fwd_grouped_operand(const void* a_operand, const float* a_unit, int64_t M, int64_t K,
+                                     const metis_linear_member* members, int count, int out_dtype, int mode, void* workspace,
+                                     size_t workspace_bytes, void* stream)
+{
+    if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) return METIS_E_ARG;
+    return gemm_nvfp4_grouped(a_operand, nullptr, a_unit, M, K, reinterpret_cast<const GemmMember*>(members), count, out_dtype,
+                              (hipStream_t)stream, workspace, workspace_bytes, nullptr, mode == METIS_MODE_PB16, true);
 }
 
 int metis_linear_fwd_grouped_centered(const void* a_codes, const void* a_scales, const float* a_unit, int64_t M, int64_t K,

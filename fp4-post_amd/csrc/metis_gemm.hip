@@ -594,7 +594,11 @@ static int launch_large(const void* a_codes, const void* a_scales, const float* 
 // bf16 matmul rounds it, the bias is added in bf16, then the low-rank term and one final rounding.  The low-rank
 // products therefore stay apart from the residual sums: they pass through the reduction buffer a second time (K slice 0
 // leaves them as one more partial in slot nsplit when K is split).
-template <int TM, int C, int WAVES, int OUT_F32, int CEN = 0, int PB16 = 0>
+//
+// ADENSE: the activation arrives as ready 16-bit MFMA operands (skinny_operand_kernel: one 16-byte piece per lane and
+// MFMA, a coalesced KiB per load instruction) instead of packed codes that every workgroup would expand again: the
+// vector unit is left with the weight operand alone.  a_codes then points at that buffer and a_scales is unused.
+template <int TM, int C, int WAVES, int OUT_F32, int CEN = 0, int PB16 = 0, int ADENSE = 0>
 __device__ __forceinline__ void skinny_tile(
     const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const float* __restrict__ a_unit,
     const uint8_t* __restrict__ b_codes, const uint8_t* __restrict__ b_scales, const float* __restrict__ b_unit,
@@ -609,12 +613,16 @@ __device__ __forceinline__ void skinny_tile(
     const int nrow = min(n0 + (lane & 31), N - 1);
     const uint8_t* bc = b_codes + (int64_t)nrow * kbytes + hi * 16 * C;
     const uint8_t* bs = b_scales + (int64_t)nrow * kblocks + hi * 2 * C;
+    static_assert(ADENSE == 0 || (C == 4 && CEN == 0), "ready operands come in the wide-run layout");
     const uint8_t *ac[TM], *as[TM];
+    const uint4* ap[TM];
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const int mrow = min(m0 + i * 32 + (lane & 31), M - 1);
         ac[i] = a_codes + (int64_t)mrow * kbytes + hi * 16 * C;
         as[i] = a_scales + (int64_t)mrow * kblocks + hi * 2 * C;
+        // operand (row tile, iteration, m): 64 lanes x 16 bytes
+        ap[i] = reinterpret_cast<const uint4*>(a_codes) + (int64_t)(m0 / 32 + i) * (K / (64 * C)) * (4 * C * 64) + lane;
     }
     float16_t acc[TM];
 #pragma unroll
@@ -656,6 +664,26 @@ __device__ __forceinline__ void skinny_tile(
     for (int it = s0 + wave * iters / WAVES; it < it1; ++it) {
         RunRegs<C> rw;
         load_run<C>(rw, bc + (int64_t)it * 32 * C, bs + it * 4 * C);
+        if constexpr (ADENSE != 0) {
+#pragma unroll
+            for (int m = 0; m < 4 * C; ++m) {
+                uint4 fa[TM];
+#pragma unroll
+                for (int i = 0; i < TM; ++i) fa[i] = ap[i][(int64_t)(it * 4 * C + m) * 64];
+                if constexpr (PB16 != 0) {
+                    const bf16x8_t fw = run_operand_bf16<C>(rw, m, ub);
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+                        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw, __builtin_bit_cast(bf16x8_t, fa[i]), acc[i], 0, 0, 0);
+                } else {
+                    const half8_t fw = run_operand<C>(rw, m);
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+                        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw, __builtin_bit_cast(half8_t, fa[i]), acc[i], 0, 0, 0);
+                }
+            }
+            continue;
+        }
         RunRegs<C> ra[TM];
 #pragma unroll
         for (int i = 0; i < TM; ++i) load_run<C>(ra[i], ac[i] + (int64_t)it * 32 * C, as[i] + it * 4 * C);
@@ -818,7 +846,7 @@ __device__ __forceinline__ void skinny_tile(
 // Several weight matrices against ONE packed activation in one launch (q/k/v, gate/up): the column tiles of the
 // members are laid end to end along grid x.  A decode-sized k or v projection alone is 16 workgroups and costs a
 // whole launch latency; next to q it is free.
-template <int TM, int C, int WAVES, int OUT_F32, int CEN = 0, int PB16 = 0>
+template <int TM, int C, int WAVES, int OUT_F32, int CEN = 0, int PB16 = 0, int ADENSE = 0>
 __global__ __launch_bounds__(64 * WAVES) void gemm_nvfp4_skinny_grouped_kernel(
     const uint8_t* __restrict__ a_codes, const uint8_t* __restrict__ a_scales, const float* __restrict__ a_unit, int M, int K,
     const SkinnyGroup grp)
@@ -833,9 +861,80 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nvfp4_skinny_grouped_kernel(
 #pragma unroll
     for (int i = 1; i < kMaxGroupMembers; ++i)
         if (g == i) mm = grp.m[i];
-    skinny_tile<TM, C, WAVES, OUT_F32, CEN, PB16>(a_codes, a_scales, a_unit, mm.b_codes, mm.b_scales, mm.b_unit, M, mm.N, K, mm.t, mm.u,
+    skinny_tile<TM, C, WAVES, OUT_F32, CEN, PB16, ADENSE>(a_codes, a_scales, a_unit, mm.b_codes, mm.b_scales, mm.b_unit, M, mm.N, K, mm.t, mm.u,
                                             mm.r, mm.bias, mm.out, mm.bias_f32, (tile - start) * 32, mm.ldt, mm.part, grp.nsplit,
                                             grp.center);
+}
+
+// The activation of a decode-sized call as ready MFMA operands for the wide-run layout of skinny_tile (K % 256 == 0):
+// piece ((row tile, iteration, m), lane) holds the 8 elements k = 256 it + 128 (lane / 32) + 8 m .. of row
+// 32 tile + lane % 32, rows past M zero.  Exact mode: e2m1 * e4m3 * 2^-8 in binary16 (the tensor unit stays outside).
+// PB16: the reference's bf16 value bf16(bf16(e4m3 * unit) * e2m1), and with a centre (mean mode, one bf16 value per
+// column) its me + QDQ(x - me) rounded to bf16 once more (src/Metis/Metis/bitlinear.py:330-333 in bf16 arithmetic).
+template <int PB16>
+__global__ __launch_bounds__(256) void skinny_operand_kernel(const uint32_t* __restrict__ codes, const uint8_t* __restrict__ scales,
+                                                             const float* __restrict__ unit_p, const uint16_t* __restrict__ center,
+                                                             int M, int K, int tiles, uint4* __restrict__ out)
+{
+    typedef float float2_t __attribute__((ext_vector_type(2)));
+    const int iters = K / 256;
+    const int64_t total = (int64_t)tiles * iters * 1024;
+    const float unit = PB16 ? *unit_p : 0.0f;
+    for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
+        const int lane = (int)(idx & 63), m = (int)((idx >> 6) & 15);
+        const int64_t ti = idx >> 10;
+        const int it = (int)(ti % iters), tile = (int)(ti / iters);
+        const int row = tile * 32 + (lane & 31), k0 = it * 256 + (lane >> 5) * 128 + 8 * m;
+        uint4 v = make_uint4(0u, 0u, 0u, 0u);
+        if (row < M) {
+            const uint32_t c = codes[(int64_t)row * (K / 8) + (k0 >> 3)];
+            const uint32_t sb = scales[(int64_t)row * (K / 16) + (k0 >> 4)];
+            if constexpr (PB16 != 0) {
+                const float dq = rb(e4m3_value(sb) * unit);
+                const float2_t p[4] = {__builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c, 1.0f, 0), __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c, 1.0f, 1),
+                                       __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c, 1.0f, 2), __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c, 1.0f, 3)};
+                float o[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) o[j] = p[j >> 1][j & 1] * dq;
+                if (center) {
+                    const uint4 cw = *reinterpret_cast<const uint4*>(center + k0);
+                    const uint32_t cws[4] = {cw.x, cw.y, cw.z, cw.w};
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) o[j] = ((j & 1) ? bf16_hi(cws[j >> 1]) : bf16_lo(cws[j >> 1])) + rb(o[j]);
+                }
+                v.x = rb_pair(o[0], o[1]); v.y = rb_pair(o[2], o[3]); v.z = rb_pair(o[4], o[5]); v.w = rb_pair(o[6], o[7]);
+            } else {
+                v = expand8(c, scale_pair(sb));
+            }
+        }
+        out[idx] = v;
+    }
+}
+
+size_t skinny_operand_bytes(int64_t M, int64_t K)
+{
+    if (M <= 0 || K <= 0) return 0;
+    return (size_t)((M + 63) / 64) * 64 * (size_t)K * 2;      // whole pairs of 32-row tiles
+}
+
+int skinny_operand(const void* codes, const void* scales, const float* unit, int64_t M, int64_t K, int mode, const void* center,
+                   void* out, hipStream_t st)
+{
+    if (mode == METIS_MODE_P32_F32) mode = METIS_MODE_P32;
+    if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) return METIS_E_ARG;
+    if (M <= 0 || M >= 256 || K <= 0 || K % 256 || K > INT32_MAX) return METIS_E_SHAPE;
+    if (!codes || !scales || !out || ((uintptr_t)codes % 4) || ((uintptr_t)out % 16) || ((uintptr_t)center % 16)) return METIS_E_ARG;
+    if (mode == METIS_MODE_PB16 ? !unit : center != nullptr) return METIS_E_ARG;   // a centre belongs to bf16 arithmetic
+    const int tiles = (int)((M + 63) / 64) * 2;
+    const int64_t total = (int64_t)tiles * (K / 256) * 1024;
+    const int g = (int)((total + 255) / 256);
+    if (mode == METIS_MODE_PB16)
+        hipLaunchKernelGGL(skinny_operand_kernel<1>, dim3(g), dim3(256), 0, st, (const uint32_t*)codes, (const uint8_t*)scales, unit,
+                           (const uint16_t*)center, (int)M, (int)K, tiles, (uint4*)out);
+    else
+        hipLaunchKernelGGL(skinny_operand_kernel<0>, dim3(g), dim3(256), 0, st, (const uint32_t*)codes, (const uint8_t*)scales, unit,
+                           (const uint16_t*)center, (int)M, (int)K, tiles, (uint4*)out);
+    return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 
 // Adds the K slices of the skinny kernel in ascending order, then bias and output conversion.
@@ -901,10 +1000,23 @@ static int launch_skinny_reduce(const SkinnyGroup& grp, int64_t M, int out_dtype
 
 template <int TM, int C, int WAVES>
 static int launch_skinny_grouped(const void* a_codes, const void* a_scales, const float* a_unit, int64_t M, int64_t K,
-                                 const SkinnyGroup& grp, int tiles, int out_dtype, hipStream_t st, bool pb16)
+                                 const SkinnyGroup& grp, int tiles, int out_dtype, hipStream_t st, bool pb16, bool adense)
 {
     const bool split = grp.nsplit > 1;
     const dim3 grid((unsigned)tiles, (unsigned)((M + 32 * TM - 1) / (32 * TM)), (unsigned)(split ? grp.nsplit : 1)), block(64 * WAVES);
+    if constexpr (C == 4) {
+        if (adense) {                                          // the activation as ready operands (skinny_operand)
+            if (grp.center) return METIS_E_ARG;
+#define METIS_SKD(O, P) hipLaunchKernelGGL((gemm_nvfp4_skinny_grouped_kernel<TM, C, WAVES, O, 0, P, 1>), grid, block, 0, st, \
+                                           (const uint8_t*)a_codes, (const uint8_t*)a_scales, a_unit, (int)M, (int)K, grp)
+            if (pb16) { if (out_dtype == METIS_DTYPE_F32) METIS_SKD(1, 1); else METIS_SKD(0, 1); }
+            else { if (out_dtype == METIS_DTYPE_F32) METIS_SKD(1, 0); else METIS_SKD(0, 0); }
+#undef METIS_SKD
+            if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
+            return split ? launch_skinny_reduce(grp, M, out_dtype, st, pb16) : METIS_OK;
+        }
+    }
+    if (adense) return METIS_E_ARG;
     if (pb16) {                                                // the reference's all-bf16 evaluation
         if (grp.center) return METIS_E_ARG;
         if (out_dtype == METIS_DTYPE_F32)
@@ -1009,11 +1121,13 @@ int gemm_grouped_center_supported(int64_t M, int64_t K, const GemmMember* member
 
 int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a_unit, int64_t M, int64_t K,
                        const GemmMember* members, int count, int out_dtype, hipStream_t st, void* workspace,
-                       size_t workspace_bytes, const float* center, bool pb16)
+                       size_t workspace_bytes, const float* center, bool pb16, bool a_dense)
 {
     if (!members || count < 1) return METIS_E_ARG;
     if ((uintptr_t)center % 16) return METIS_E_ARG;
-    if (pb16 && center) return METIS_E_ARG;
+    if ((pb16 || a_dense) && center) return METIS_E_ARG;
+    if (a_dense && (K % 256 || !a_unit)) return METIS_E_ARG;
+    if (a_dense) a_scales = a_codes;                          // unused by the kernel: the checks below see an aligned pointer
     bool skinny = M > 0 && M < 256 && K % 64 == 0 && count <= kMaxGroupMembers && !measure_env("METIS_GEMM_SMALL") &&
                   a_codes && a_scales && a_unit && !((uintptr_t)a_codes % 16) && !((uintptr_t)a_scales % 2) && K <= INT32_MAX &&
                   (out_dtype == METIS_DTYPE_BF16 || out_dtype == METIS_DTYPE_F32);
@@ -1030,7 +1144,7 @@ int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a
         ntot += g.N;
     }
     if (!skinny || tiles > INT32_MAX) {
-        if (center || pb16) return METIS_E_ARG;                // the centre and the bf16 evaluation are only taken by the single-launch path
+        if (center || pb16 || a_dense) return METIS_E_ARG;     // the centre, the bf16 evaluation and ready operands are only taken by the single-launch path
         for (int i = 0; i < count; ++i) {
             const GemmMember& g = members[i];
             if (g.ldt != 0 && g.ldt != g.r) return METIS_E_ARG;   // a strided t is only taken by the single-launch path
@@ -1049,6 +1163,7 @@ int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a
             tm = ftm; c = fc; waves = fw; nsplit = fs;
         }
     }
+    if (a_dense && c != 4) return METIS_E_ARG;                 // weight scale bytes must be 8-byte aligned for wide runs
     const size_t slots = (size_t)nsplit + (pb16 ? 1 : 0);      // bf16 arithmetic: one more for the low-rank term
     if (nsplit > 1 && (((uintptr_t)workspace % 16) || workspace_bytes < slots * (size_t)M * (size_t)ntot * sizeof(float)))
         return METIS_E_WORKSPACE;
@@ -1067,7 +1182,7 @@ int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a
                                 (int)g.r, end, g.bias_is_f32 != 0, (int)(g.ldt ? g.ldt : g.r)};
         part += slots * (size_t)M * (size_t)g.N;
     }
-#define METIS_SKG(TM, C, W) return launch_skinny_grouped<TM, C, W>(a_codes, a_scales, a_unit, M, K, grp, (int)tiles, out_dtype, st, pb16)
+#define METIS_SKG(TM, C, W) return launch_skinny_grouped<TM, C, W>(a_codes, a_scales, a_unit, M, K, grp, (int)tiles, out_dtype, st, pb16, a_dense)
     if (tm == 1) {
         if (waves == 4) { if (c == 4) METIS_SKG(1, 4, 4); else METIS_SKG(1, 1, 4); }
         else { if (c == 4) METIS_SKG(1, 4, 8); else METIS_SKG(1, 1, 8); }

@@ -41,10 +41,14 @@ __host__ __device__ __forceinline__ int xt_swz(int q) { return ((q >> 2) & 1) | 
 //        them and both run the 16-point butterflies.  PB16 = 0: the result is rounded to binary16 once (the sum of a
 //        block needs at most 12 significant bits); PB16 = 1: dequantized values and result rounded to bf16 as the
 //        reference's bf16 tensors are.
+//   center (PB16 without RHT): the packed tensor is the centred residual of the mean mode; the operand is the
+//        reference's me + QDQ(x - me) with the sum rounded to bf16 (src/Metis/Metis/bitlinear.py:330-333 in bf16
+//        arithmetic): one bf16 value per column.
 template <int PB16, int RHT = 0>
 __global__ __launch_bounds__(256) void expand_xt_kernel(const uint32_t* __restrict__ codes, const uint8_t* __restrict__ scales,
                                                         const float* __restrict__ unit_p, uint4* __restrict__ out, int rows,
-                                                        int K, int row_tiles, uint32_t sign_mask)
+                                                        int K, int row_tiles, uint32_t sign_mask,
+                                                        const uint16_t* __restrict__ center = nullptr)
 {
     typedef float float2_t __attribute__((ext_vector_type(2)));
     const int lane = threadIdx.x & 63;
@@ -99,6 +103,13 @@ __global__ __launch_bounds__(256) void expand_xt_kernel(const uint32_t* __restri
                     v.y = rb_pair(p1[0] * dq, p1[1] * dq);
                     v.z = rb_pair(p2[0] * dq, p2[1] * dq);
                     v.w = rb_pair(p3[0] * dq, p3[1] * dq);
+                    if (center) {
+                        const uint4 cw = *reinterpret_cast<const uint4*>(center + k8 * 8);
+                        v.x = rb_pair(bf16_lo(cw.x) + bf16_lo(v.x), bf16_hi(cw.x) + bf16_hi(v.x));
+                        v.y = rb_pair(bf16_lo(cw.y) + bf16_lo(v.y), bf16_hi(cw.y) + bf16_hi(v.y));
+                        v.z = rb_pair(bf16_lo(cw.z) + bf16_lo(v.z), bf16_hi(cw.z) + bf16_hi(v.z));
+                        v.w = rb_pair(bf16_lo(cw.w) + bf16_lo(v.w), bf16_hi(cw.w) + bf16_hi(v.w));
+                    }
                 } else {
                     v = expand8(c, scale_pair(sb));
                 }
@@ -241,9 +252,10 @@ size_t expand_xt_bytes(int64_t rows, int64_t cols)
 }
 
 int expand_xt(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, int mode, void* out,
-              hipStream_t st, int rht, uint32_t sign_mask)
+              hipStream_t st, int rht, uint32_t sign_mask, const void* center)
 {
     if (rows < 0 || cols < 0 || sign_mask > 0xffffu) return METIS_E_ARG;
+    if (center && (mode != METIS_MODE_PB16 || rht || ((uintptr_t)center % 16))) return METIS_E_ARG;   // a centre belongs to bf16 arithmetic
     if (mode == METIS_MODE_P32_F32) mode = METIS_MODE_P32;
     if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) return METIS_E_ARG;
     if (cols % kBlock) return METIS_E_SHAPE;
@@ -258,6 +270,11 @@ int expand_xt(const void* codes, const void* scales, const float* unit, int64_t 
     if (g > cap) g = cap;
 #define METIS_EX(P, R) hipLaunchKernelGGL((expand_xt_kernel<P, R>), dim3((unsigned)g), dim3(256), 0, st, (const uint32_t*)codes, \
                                           (const uint8_t*)scales, unit, (uint4*)out, (int)rows, (int)cols, row_tiles, sign_mask)
+    if (center) {
+        hipLaunchKernelGGL((expand_xt_kernel<1, 0>), dim3((unsigned)g), dim3(256), 0, st, (const uint32_t*)codes, (const uint8_t*)scales,
+                           unit, (uint4*)out, (int)rows, (int)cols, row_tiles, sign_mask, (const uint16_t*)center);
+        return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
+    }
     if (mode == METIS_MODE_PB16) { if (rht) METIS_EX(1, 1); else METIS_EX(1, 0); }
     else { if (rht) METIS_EX(0, 1); else METIS_EX(0, 0); }
 #undef METIS_EX

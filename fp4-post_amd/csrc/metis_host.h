@@ -86,7 +86,11 @@ struct GemmMember {
 };
 int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a_unit, int64_t M, int64_t K,
                        const GemmMember* members, int count, int out_dtype, hipStream_t st, void* workspace = nullptr,
-                       size_t workspace_bytes = 0, const float* center = nullptr, bool pb16 = false);
+                       size_t workspace_bytes = 0, const float* center = nullptr, bool pb16 = false, bool a_dense = false);
+// the activation of a decode-sized call as ready 16-bit MFMA operands (a_dense above: a_codes is this buffer); metis_gemm.hip
+size_t skinny_operand_bytes(int64_t M, int64_t K);
+int skinny_operand(const void* codes, const void* scales, const float* unit, int64_t M, int64_t K, int mode, const void* center,
+                   void* out, hipStream_t st);
 int gemm_grouped_center_supported(int64_t M, int64_t K, const GemmMember* members, int count, int have_workspace);
 // bytes of split-K scratch a grouped call can use (only the N fields of the members are read; 0: it would not split)
 size_t gemm_grouped_workspace_bytes(int64_t M, int64_t K, const GemmMember* members, int count);
@@ -125,7 +129,7 @@ int gemm_expanded(const void* a_exp, const float* a_unit, const void* b_exp, con
 // tiled 16-bit expansion of a packed tensor and the pipelined GEMM that consumes it; metis_gemm_pipe.hip
 size_t expand_xt_bytes(int64_t rows, int64_t cols);
 int expand_xt(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, int mode, void* out,
-              hipStream_t st, int rht = 0, uint32_t sign_mask = 0);
+              hipStream_t st, int rht = 0, uint32_t sign_mask = 0, const void* center = nullptr);
 // a dense bf16 / binary32 tensor in the tiled layout (optional per-column bf16 scale first)
 int dense_xt(const void* x, int64_t rows, int64_t cols, int64_t ld, int dtype, const void* col_scale, int mode, void* out, hipStream_t st);
 // the tiled operand [cols, rows] (contraction over the packed tensor's rows); rows % 32 == 0

@@ -452,6 +452,15 @@ class LinearLowbitFunction(torch.autograd.Function):
             value = F._apply_hadamard_blocks(value, inverse=True)
         return value
 
+    @staticmethod
+    def _mean_in_operand(px, pw) -> bool:
+        """Mean mode in bf16 arithmetic with reference_rounding: the GEMM's activation operand is the reference's own
+        bf16 tensor me + QDQ(x - me) (reference 330-333), so the forward follows its all-bf16 evaluation; otherwise the
+        mean's share is a separate binary32 term next to exact products of the packed residual."""
+        F = LinearLowbitFunction
+        return (F.reference_rounding and F.compute_dtype != torch.float32 and px.residual.mode == ops.MODE_PB16
+                and pw.mode == ops.MODE_PB16 and pw.rht is None and px.mean.dtype == torch.bfloat16 and px.cols % 32 == 0)
+
     # ------------------------------------------------------------------ autograd
     @staticmethod
     def forward(ctx, input_, weight, bias, quantized_weight, quantized_input):
@@ -467,13 +476,18 @@ class LinearLowbitFunction(torch.autograd.Function):
             ctx.weight_ref = weight
             ctx.save_for_backward(input_, bias if bias is not None else input_.new_empty(0))
             ctx.center = None
+            out_dtype = torch.float32 if F.compute_dtype == torch.float32 else torch.bfloat16
+            if isinstance(quantized_input, CenteredNVFP4) and F._mean_in_operand(quantized_input, quantized_weight):
+                ctx.center = quantized_input.mean
+                out = ops.linear_fwd_grouped(quantized_input.residual, [(quantized_weight, None, None, bias)], out_dtype=out_dtype,
+                                             center=quantized_input.mean, reference_rounding=True)[0]
+                return out.reshape(*lead, quantized_weight.rows).to(F.compute_dtype)
             if isinstance(quantized_input, CenteredNVFP4):
                 # (1 me^T + R) W^^T = R W^^T + 1 (W^ me)^T: the mean's term rides in a binary32 bias
                 ctx.center = quantized_input.mean
                 w_mean = ops.matvec(quantized_weight, quantized_input.mean)
                 bias = w_mean if bias is None else w_mean + bias.float()
                 quantized_input = quantized_input.residual
-            out_dtype = torch.float32 if F.compute_dtype == torch.float32 else torch.bfloat16
             out = ops.linear_fwd(quantized_input, quantized_weight, bias=bias, out_dtype=out_dtype,
                                  reference_rounding=F.reference_rounding and ctx.center is None)
             return out.reshape(*lead, quantized_weight.rows).to(F.compute_dtype)
@@ -632,7 +646,11 @@ class _MetisFusedFunction(torch.autograd.Function):
         if isinstance(px, CenteredNVFP4):
             # mean mode: the residual branch sees 1 me^T + R
             ctx.center = px.mean
-            if px.rows < 256:
+            if F._mean_in_operand(px, p_res):
+                # bf16 arithmetic: the activation operand is the reference's bf16 tensor me + QDQ(x - me)
+                y = ops.linear_fwd_grouped(px.residual, [(p_res, t, u.to(cd), gemm_bias)], out_dtype=out_dtype, center=px.mean,
+                                           reference_rounding=True)[0]
+            elif px.rows < 256:
                 # decode-sized: W^ me is accumulated inside the GEMM launch
                 y = ops.linear_fwd_grouped(px.residual, [(p_res, t, u.to(cd), None if bias is None else bias.float())],
                                            out_dtype=out_dtype, center=px.center32)[0]
@@ -890,12 +908,14 @@ class BitLinear(nn.Module):
         _, t_all = ops.lowrank_project(x2, cached[1], cached[2])
         centre = shared_input.center32 if isinstance(shared_input, CenteredNVFP4) else None
         px = shared_input.residual if centre is not None else shared_input
+        if centre is not None and all(F._mean_in_operand(shared_input, p) for p in packed):
+            centre = shared_input.mean                             # bf16: goes into the activation operand (reference's bf16 tensor)
         calls, c0 = [], 0
         for m, p_res in zip(members, packed):
             r = m.args.forward_svd_rank
             bias = m.warmup_linear.bias
             if bias is not None:
-                bias = m._bias_as(torch.float32 if centre is not None else cd)
+                bias = m._bias_as(torch.float32 if (centre is not None and centre.dtype == torch.float32) else cd)
             calls.append((p_res, t_all[:, c0:c0 + r], m.ulinear.weight.to(cd), bias))      # a column slice: no copy
             c0 += r
         out_dtype = torch.float32 if F.compute_dtype == torch.float32 else torch.bfloat16

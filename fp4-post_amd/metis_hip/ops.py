@@ -348,14 +348,27 @@ def expand(p: PackedNVFP4) -> torch.Tensor:
     return p.expanded
 
 
-def expand_tiled(p: PackedNVFP4, cache: bool = True, mode: int = MODE_P32) -> torch.Tensor:
+def expand_tiled(p: PackedNVFP4, cache: bool = True, mode: int = MODE_P32, center: torch.Tensor | None = None) -> torch.Tensor:
     """16-bit expansion of a packed tensor in the tiled layout of the pipelined GEMM (uint8 buffer): exact binary16
     values e2m1 * e4m3 * 2^-8 (mode P32) or the reference's bf16 dequantized values, unit included (mode PB16).
-    cache=True keeps it on the packed tensor (weights); activations are expanded per call."""
+    cache=True keeps it on the packed tensor (weights); activations are expanded per call.
+    center (bf16 [cols], mode PB16): p packs a centred residual; the operand is the mean mode's center + QDQ(x - center)
+    rounded to bf16, the tensor the reference multiplies with in bf16 arithmetic (never cached)."""
+    L = load()
+    if center is not None:
+        if mode != MODE_PB16 or p.rht is not None:
+            raise ValueError("a centre goes into the bf16-arithmetic operand of an unrotated tensor")
+        center = center.reshape(-1).to(torch.bfloat16).contiguous()
+        if center.numel() != p.cols:
+            raise ValueError(f"center must have {p.cols} values, got {center.numel()}")
+        out = torch.empty(L.metis_nvfp4_expand_tiled_bytes(p.rows, p.cols), dtype=torch.uint8, device=p.codes.device)
+        rc = L.metis_nvfp4_expand_tiled_centered(p.codes.data_ptr(), p.scales.data_ptr(), p.unit.data_ptr(), p.rows, p.cols,
+                                                 center.data_ptr(), out.data_ptr(), _stream())
+        check(rc, "metis_nvfp4_expand_tiled_centered", (p.rows, p.cols))
+        return out
     have = p.tiled_pb16 if mode == MODE_PB16 else p.tiled
     if have is not None:
         return have
-    L = load()
     out = torch.empty(L.metis_nvfp4_expand_tiled_bytes(p.rows, p.cols), dtype=torch.uint8, device=p.codes.device)
     if p.rht is not None:                     # NV recipe: the operand holds the values rotated back
         rc = L.metis_nvfp4_expand_tiled_rht(p.codes.data_ptr(), p.scales.data_ptr(), p.unit.data_ptr(), p.rows, p.cols, mode,
@@ -388,6 +401,22 @@ def expand_tiled_transposed(p: PackedNVFP4, cache: bool = False, mode: int = MOD
             p.tiled_t_pb16 = out
         else:
             p.tiled_t = out
+    return out
+
+
+def decode_operand(p: PackedNVFP4, mode: int = MODE_P32, center: torch.Tensor | None = None) -> torch.Tensor:
+    """The activation of a decode-sized call (rows < 256, cols % 256 == 0) as ready 16-bit MFMA operands for
+    metis_linear_fwd_grouped_operand: exact binary16 values (mode P32), the reference's bf16 dequantized values (mode
+    PB16), or with `center` (bf16 [cols], PB16) the mean mode's center + QDQ(x - center) rounded to bf16."""
+    L = load()
+    out = torch.empty(L.metis_nvfp4_decode_operand_bytes(p.rows, p.cols), dtype=torch.uint8, device=p.codes.device)
+    if center is not None:
+        center = center.reshape(-1).to(torch.bfloat16).contiguous()
+        if center.numel() != p.cols:
+            raise ValueError(f"center must have {p.cols} values, got {center.numel()}")
+    rc = L.metis_nvfp4_decode_operand(p.codes.data_ptr(), p.scales.data_ptr(), p.unit.data_ptr(), p.rows, p.cols, mode,
+                                      None if center is None else center.data_ptr(), out.data_ptr(), _stream())
+    check(rc, "metis_nvfp4_decode_operand", (p.rows, p.cols))
     return out
 
 
@@ -446,11 +475,13 @@ def gemm_tiled(ax: torch.Tensor, a_unit: torch.Tensor, bx: torch.Tensor, b_unit:
 def linear_fwd_tiled(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None, u: torch.Tensor | None = None,
                      bias: torch.Tensor | None = None, out_dtype: torch.dtype = torch.bfloat16,
                      a_tiled: torch.Tensor | None = None, reference_rounding: bool = False,
-                     split_k: bool = True) -> torch.Tensor:
+                     split_k: bool = True, center: torch.Tensor | None = None) -> torch.Tensor:
     """linear_fwd on tiled 16-bit expansions: b's is cached on b when b is persistent, a's is made here unless given.
 
     reference_rounding (both operands packed in bf16 arithmetic): operands are the reference's bf16 dequantized
-    values and the epilogue rounds where the reference's all-bf16 forward rounds; otherwise exact products."""
+    values and the epilogue rounds where the reference's all-bf16 forward rounds; otherwise exact products.
+    center (bf16 [K], with reference_rounding): `a` packs the centred residual of the mean mode and the activation
+    operand is the reference's bf16 tensor center + QDQ(x - center)."""
     if a.cols != b.cols:
         raise ValueError(f"contraction mismatch: {a.cols} vs {b.cols}")
     mode = MODE_P32
@@ -458,8 +489,10 @@ def linear_fwd_tiled(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None =
         if a.mode != MODE_PB16 or b.mode != MODE_PB16:
             raise ValueError("reference_rounding needs both operands packed in bf16 arithmetic")
         mode = MODE_PB16
+    elif center is not None:
+        raise ValueError("a centre inside the operand belongs to reference_rounding")
     bx = expand_tiled(b, cache=b.persistent, mode=mode)
-    ax = a_tiled if a_tiled is not None else expand_tiled(a, cache=False, mode=mode)
+    ax = a_tiled if a_tiled is not None else expand_tiled(a, cache=False, mode=mode, center=center)
     return gemm_tiled(ax, a.unit, bx, b.unit, a.rows, b.rows, a.cols, mode=mode, t=t, u=u, bias=bias, out_dtype=out_dtype,
                       split_k=split_k)
 
@@ -687,17 +720,28 @@ def _linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.
     """[linear_fwd(a, b, t=t, u=u, bias=bias) for (b, t, u, bias) in members] in one call: a projection group
     (q/k/v, gate/up) that shares one packed activation.  Decode-sized batches run as a single launch.
 
-    reference_rounding (every operand packed in bf16 arithmetic, no centre): the reference's all-bf16 evaluation, as in
-    linear_fwd; shapes the decode-sized kernel does not take are served member by member.
+    reference_rounding (every operand packed in bf16 arithmetic): the reference's all-bf16 evaluation, as in
+    linear_fwd; shapes the decode-sized kernel does not take are served member by member.  A bf16 `center` then goes
+    into the activation operand itself (the reference's bf16 tensor center + QDQ(x - center)); a float32 centre keeps
+    exact products with the centre's share accumulated in binary32.
 
     center (mean mode: `a` packs the centred residual X - center): every output row also receives deq(b) . center,
     inside the same launch where the shape allows, else through matvec and a binary32 bias."""
     import ctypes
     M, K = a.rows, a.cols
     dev = a.codes.device
-    rounded = (reference_rounding and center is None and a.mode == MODE_PB16 and all(m[0].mode == MODE_PB16 for m in members))
-    if rounded and not (len(members) <= 4 and all(_decode_kernel_takes(M, m[0].rows, K, 0 if m[1] is None else m[1].shape[1])
-                                                  for m in members)):
+    rounded = (reference_rounding and (center is None or center.dtype == torch.bfloat16) and a.mode == MODE_PB16
+               and all(m[0].mode == MODE_PB16 for m in members))
+    takes = len(members) <= 4 and all(_decode_kernel_takes(M, m[0].rows, K, 0 if m[1] is None else m[1].shape[1]) for m in members)
+    # ready operands (built once for the group): wide runs only
+    operand = rounded and takes and K % 256 == 0 and all(m[0].scales.data_ptr() % 8 == 0 for m in members)
+    if rounded and center is not None and not operand:
+        if M >= 256 and K % 32 == 0:
+            ax = expand_tiled(a, cache=False, mode=MODE_PB16, center=center)
+            return [linear_fwd_tiled(a, b, t=t, u=u, bias=bias, out_dtype=out_dtype, a_tiled=ax, reference_rounding=True, split_k=split_k)
+                    for b, t, u, bias in members]
+        rounded = False                                        # exact products, the centre's share in binary32
+    if rounded and not takes:
         return [linear_fwd(a, b, t=t, u=u, bias=bias, out_dtype=out_dtype, split_k=split_k, reference_rounding=True)
                 for b, t, u, bias in members]
     arr = (_lib.LinearMember * len(members))()
@@ -735,6 +779,12 @@ def _linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.
             M, K, ctypes.cast(arr, ctypes.c_void_p), len(members), 0))
     ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
     dt = DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16
+    if operand:
+        aop = decode_operand(a, MODE_PB16, center)
+        rc = L.metis_linear_fwd_grouped_operand(aop.data_ptr(), a.unit.data_ptr(), M, K, ap, len(members), dt, MODE_PB16,
+                                                None if ws is None else ws.data_ptr(), need, _stream())
+        check(rc, "metis_linear_fwd_grouped_operand", (M, K, [m[0].rows for m in members]))
+        return outs
     if center is not None:
         center = center.reshape(-1).to(device=dev, dtype=torch.float32).contiguous()
         if center.numel() != K:

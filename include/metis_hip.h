@@ -303,6 +303,17 @@ int metis_nvfp4_quant_row_rht(const void *x, int64_t rows, int64_t cols, int64_t
 int metis_nvfp4_expand_tiled_rht(const void *codes, const void *scales, const float *unit, int64_t rows,
                                  int64_t cols, int mode, uint32_t sign_mask, int rotate_back,
                                  int transpose, void *out, void *stream);
+/*
+ * Mean mode in bf16 arithmetic: the activation the reference multiplies with is X^ = me + QDQ(X - me) as ONE bf16
+ * tensor, the sum rounded to bf16 (LinearLowbitFunction.svd_quant with metis_mode = "mean",
+ * src/Metis/Metis/bitlinear.py:311-336, under compute_dtype = bfloat16).  This is metis_nvfp4_expand_tiled with
+ * mode = METIS_MODE_PB16 of the packed centred residual (metis_nvfp4_quant_centered) with that sum applied: the
+ * tiled operand holds X^ itself, and metis_linear_fwd_tiled with mode = METIS_MODE_PB16 then follows the reference's
+ * all-bf16 forward without a separate W^ me term.
+ *   center  bf16 [cols], 16-byte aligned (required)
+ */
+int metis_nvfp4_expand_tiled_centered(const void *codes, const void *scales, const float *unit, int64_t rows,
+                                      int64_t cols, const void *center, void *out, void *stream);
 int metis_linear_fwd_tiled(const void *a_xt, const float *a_unit, const void *b_xt, const float *b_unit,
                            int64_t M, int64_t N, int64_t K, const void *t, const void *u, int64_t r,
                            const void *bias, int bias_is_f32, void *out, int out_dtype, int mode,
@@ -435,7 +446,26 @@ int metis_linear_fwd_grouped(const void *a_codes, const void *a_scales, const fl
 int metis_linear_fwd_grouped_bf16(const void *a_codes, const void *a_scales, const float *a_unit, int64_t M,
                                   int64_t K, const metis_linear_member *members, int count, int out_dtype,
                                   void *workspace, size_t workspace_bytes, void *stream);
-/* Scratch for the two calls above: with few output columns and a long K (a down projection at decode size) K is cut
+/* The activation of a decode-sized call as ready 16-bit MFMA operands, built once per activation instead of being
+ * expanded from its codes by every workgroup of every projection that reads it (in bf16 arithmetic the expansion is
+ * two roundings per element; q/k/v or gate/up share one activation).
+ *   metis_nvfp4_decode_operand   mode METIS_MODE_P32: binary16 e2m1 * e4m3 * 2^-8 (exact, the tensor unit stays
+ *                                outside); METIS_MODE_PB16: the reference's bf16 dequantized values, and with `center`
+ *                                (bf16 [cols], 16-byte aligned, or NULL; PB16 only) the mean mode's me + QDQ(x - me)
+ *                                rounded to bf16 (src/Metis/Metis/bitlinear.py:330-333).  rows < 256, cols % 256 == 0;
+ *                                out: metis_nvfp4_decode_operand_bytes(rows, cols) bytes, 16-byte aligned
+ *   metis_linear_fwd_grouped_operand  metis_linear_fwd_grouped (mode METIS_MODE_P32, same bits) or
+ *                                metis_linear_fwd_grouped_bf16 (mode METIS_MODE_PB16, same bits when no centre went
+ *                                into the operand) reading that buffer; a_unit as for the packed activation (unused in
+ *                                mode PB16 but required); weight scale pointers 8-byte aligned; METIS_E_ARG for
+ *                                shapes the decode-sized kernel does not take */
+size_t metis_nvfp4_decode_operand_bytes(int64_t rows, int64_t cols);
+int metis_nvfp4_decode_operand(const void *codes, const void *scales, const float *unit, int64_t rows,
+                               int64_t cols, int mode, const void *center, void *out, void *stream);
+int metis_linear_fwd_grouped_operand(const void *a_operand, const float *a_unit, int64_t M, int64_t K,
+                                     const metis_linear_member *members, int count, int out_dtype, int mode,
+                                     void *workspace, size_t workspace_bytes, void *stream);
+/* Scratch for the calls above: with few output columns and a long K (a down projection at decode size) K is cut
  * into slices that run as separate workgroups, their binary32 partial sums meet in the workspace and a second
  * small kernel adds them in a fixed order.  Only the N fields of the members are read; the figure is an upper
  * bound (the number of slices also depends on pointer alignment, known only at the call).  0 = the shape is not

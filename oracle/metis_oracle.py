@@ -208,7 +208,7 @@ def linear_forward(xq: torch.Tensor, wq: torch.Tensor, bias: torch.Tensor | None
 
 def metis_forward(x: torch.Tensor, v: torch.Tensor, s: torch.Tensor, u: torch.Tensor,
                   w_res: torch.Tensor, bias: torch.Tensor | None, p32: bool = True,
-                  quantized_lowrank: bool = False) -> torch.Tensor:
+                  quantized_lowrank: bool = False, mean_mode: bool = False) -> torch.Tensor:
     """Low-rank-residual linear, bitlinear.py:736-769 with the sub-module layout of 863-879.
 
     y = ulinear(s * vlinear(x)) + warmup_linear(x)
@@ -219,10 +219,18 @@ def metis_forward(x: torch.Tensor, v: torch.Tensor, s: torch.Tensor, u: torch.Te
     the single rounding of the output to bf16.  With ``quantized_lowrank`` the rank-r branch
     consumes QDQ(x) and QDQ(v) in dtype D as the current reference file does
     (bitlinear.py:752, 863-871).  The residual branch is computed in fp32 (p32) or bf16.
+    ``mean_mode`` (bitlinear.py:311-336, metis_mode="mean", a first call without cached mean): the residual branch
+    sees X^ = me + QDQ(x - me) with me the column mean over tokens, every op in dtype D (the expression
+    tests/test_oracle_golden.py pins against the reference's own svd_quant outputs).
     Returns bf16 [M,N].
     """
     D = torch.float32 if p32 else torch.bfloat16
-    xq = nvfp4_qdq(x.to(D))
+    if mean_mode:
+        xd = x.to(D)
+        me = xd.mean(dim=0, keepdim=True)
+        xq = me + nvfp4_qdq(xd - me)
+    else:
+        xq = nvfp4_qdq(x.to(D))
     wq = nvfp4_qdq(w_res.to(D))
     res = linear_forward(xq, wq, None if bias is None else bias.to(D))
     if quantized_lowrank:

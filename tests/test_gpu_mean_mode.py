@@ -437,6 +437,74 @@ def test_mean_mode_against_reference_vectors(tag, cd):
         F.compute_dtype, F.enable_activation_svd, F.metis_mode, F.tp_simulate, F.enable_nv_recipe, F.q_forward_input = keep
 
 
+def test_mean_mode_operands_in_bf16_arithmetic_hold_the_reference_tensor():
+    """bf16 arithmetic: the reference multiplies with ONE bf16 tensor, me + QDQ(x - me) with the sum rounded to bf16.
+    The tiled operand (prefill) and the ready decode operand built from the packed centred residual and the bf16 mean
+    hold exactly that tensor: against the reference's own svd_quant output for the mean it computed, and bit for bit
+    against the sum formed by torch from the same packed residual on larger shapes."""
+    from helpers import from_decode_operand, t, untile
+    from metis_hip import ops
+    g = _mean_golden()
+    x = t(g["mean_x"]).cuda().reshape(-1, 64)
+    me = t(g["mean_cache_pb16"]).cuda().reshape(-1)                   # the reference's own bf16 mean of these tokens
+    assert me.dtype == torch.bfloat16
+    p = ops.quantize(x, 1, center=me)
+    got = untile(ops.expand_tiled(p, cache=False, mode=1, center=me), x.shape[0], 64, torch.bfloat16)
+    assert torch.equal(got.cpu(), t(g["mean_out_pb16"]).reshape(-1, 64))
+    gen = torch.Generator().manual_seed(77)
+    for rows, cols in ((300, 512), (64, 3584), (17, 256), (200, 1024)):
+        xx = _offset_activation(rows + cols, rows, cols).cuda()
+        mm = ops.column_mean(xx, torch.bfloat16)
+        pp = ops.quantize(xx, 1, center=mm)
+        want = mm.unsqueeze(0) + ops.dequantize(pp, torch.bfloat16)                  # bf16 add: the reference's expression
+        assert torch.equal(untile(ops.expand_tiled(pp, cache=False, mode=1, center=mm), rows, cols, torch.bfloat16), want)
+        if rows < 256:
+            assert torch.equal(from_decode_operand(ops.decode_operand(pp, 1, mm), rows, cols, torch.bfloat16), want)
+            assert torch.equal(from_decode_operand(ops.decode_operand(pp, 1), rows, cols, torch.bfloat16), ops.dequantize(pp, torch.bfloat16))
+            exact = from_decode_operand(ops.decode_operand(pp, 0), rows, cols, torch.float16)
+            assert torch.equal(exact, ops.expand(pp))
+
+
+@pytest.mark.parametrize("L", [64, 512])
+def test_mean_mode_forward_in_bf16_arithmetic_follows_the_all_bf16_evaluation(L):
+    """The reference's default arguments under the GRPO caller's dtypes (mean mode, bf16 storage and arithmetic): the
+    fused BitLinear forward against the oracle's evaluation in that arithmetic -- X^ = me + QDQ(x - me) as one bf16
+    tensor, the residual product and the bias add rounded to bf16, the rank-r branch added before the final rounding --
+    within the GEMM tolerance at decode and prefill sizes.  (Exact products with a separate binary32 mean term sit
+    2-5e-3 from it.)"""
+    from oracle import metis_oracle as O
+    from metis_hip import BitLinear, LinearLowbitFunction as F, MetisArgs
+    K, N, r = 1024, 768, 32
+    g = torch.Generator().manual_seed(9)
+    names = ("q_forward_input", "q_forward_weight", "q_backward_input", "q_backward_weight", "q_backward_outputgrad",
+             "enable_backward_svd", "enable_activation_svd", "enable_nv_recipe", "compute_dtype", "metis_mode", "backward_lowrank_svd")
+    saved = {k: getattr(F, k) for k in names}
+    try:
+        _mean_forward_bf16(L, K, N, r, g)
+    finally:
+        for k, val in saved.items():
+            setattr(F, k, val)
+
+
+def _mean_forward_bf16(L, K, N, r, g):
+    from oracle import metis_oracle as O
+    from metis_hip import BitLinear, LinearLowbitFunction as F, MetisArgs
+    layer = BitLinear(K, N, args=MetisArgs(forward_svd_rank=r), bias=True, dtype=torch.bfloat16, compute_dtype=torch.bfloat16).cuda()
+    with torch.no_grad():
+        w = torch.randn(N, K, generator=g) * 0.02 + (torch.linalg.qr(torch.randn(N, 8, generator=g))[0] * 3.0) @ torch.linalg.qr(torch.randn(K, 8, generator=g))[0].T
+        layer.warmup_linear.weight.copy_(w)
+        layer.warmup_linear.bias.copy_(torch.randn(N, generator=g) * 0.1)
+    layer.split()
+    assert F.metis_mode == "mean" and F.enable_activation_svd and F.compute_dtype == torch.bfloat16
+    x = _offset_activation(5, L, K)
+    with torch.no_grad():
+        y = layer(x.cuda().reshape(1, L, K)).reshape(L, N).cpu()
+    want = O.metis_forward(x, layer.vlinear.weight.detach().cpu(), layer.s.detach().cpu(), layer.ulinear.weight.detach().cpu(),
+                           layer.warmup_linear.weight.detach().cpu(), layer.warmup_linear.bias.detach().cpu(), p32=False, mean_mode=True)
+    err = rel_fro(y.float(), want.float())
+    assert err <= 3e-4, err                                         # tolerance of the task: 2e-3; measured 3e-5
+
+
 def test_mean_mode_linear_against_reference_vectors(monkeypatch):
     """LinearLowbit with the mean mode on for activations and output gradients, round-to-nearest quantizers everywhere:
     forward against the reference's output on both paths; backward of the generic path (which follows the reference's
