@@ -665,21 +665,32 @@ __device__ __forceinline__ void skinny_tile(
         RunRegs<C> rw;
         load_run<C>(rw, bc + (int64_t)it * 32 * C, bs + it * 4 * C);
         if constexpr (ADENSE != 0) {
+            // a ring of AHEAD operand pieces per row tile keeps the L2 round trips ahead of the MFMAs
+            constexpr int AHEAD = 4;
+            uint4 fa[AHEAD][TM];
+#pragma unroll
+            for (int m = 0; m < AHEAD; ++m)
+#pragma unroll
+                for (int i = 0; i < TM; ++i) fa[m][i] = ap[i][(int64_t)(it * 4 * C + m) * 64];
 #pragma unroll
             for (int m = 0; m < 4 * C; ++m) {
-                uint4 fa[TM];
+                uint4 cur[TM];
 #pragma unroll
-                for (int i = 0; i < TM; ++i) fa[i] = ap[i][(int64_t)(it * 4 * C + m) * 64];
+                for (int i = 0; i < TM; ++i) cur[i] = fa[m % AHEAD][i];
+                if (m + AHEAD < 4 * C) {
+#pragma unroll
+                    for (int i = 0; i < TM; ++i) fa[m % AHEAD][i] = ap[i][(int64_t)(it * 4 * C + m + AHEAD) * 64];
+                }
                 if constexpr (PB16 != 0) {
                     const bf16x8_t fw = run_operand_bf16<C>(rw, m, ub);
 #pragma unroll
                     for (int i = 0; i < TM; ++i)
-                        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw, __builtin_bit_cast(bf16x8_t, fa[i]), acc[i], 0, 0, 0);
+                        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw, __builtin_bit_cast(bf16x8_t, cur[i]), acc[i], 0, 0, 0);
                 } else {
                     const half8_t fw = run_operand<C>(rw, m);
 #pragma unroll
                     for (int i = 0; i < TM; ++i)
-                        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw, __builtin_bit_cast(half8_t, fa[i]), acc[i], 0, 0, 0);
+                        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw, __builtin_bit_cast(half8_t, cur[i]), acc[i], 0, 0, 0);
                 }
             }
             continue;
