@@ -219,6 +219,51 @@ static void check_tiled(int64_t M, int64_t N, int64_t K, hipStream_t st)
           "a sign mask wider than 16 bits -> METIS_E_ARG");
 }
 
+// bf16 arithmetic at decode size: metis_linear_fwd_grouped_bf16 on the packed activation and
+// metis_nvfp4_decode_operand + metis_linear_fwd_grouped_operand give the same bits, and both agree with the all-bf16
+// evaluation (bf16 dequantized operands from metis_nvfp4_dequant, product rounded to bf16) computed on the host.
+static void check_decode_bf16(int64_t M, int64_t N, int64_t K, hipStream_t st)
+{
+    const std::vector<uint16_t> x = make_input(M, K, 31u, 1.0f), w = make_input(N, K, 32u, 0.02f);
+    DeviceBuffer<uint8_t> ac((size_t)(M * K / 2)), as((size_t)(M * K / 16)), bc((size_t)(N * K / 2)), bs((size_t)(N * K / 16));
+    DeviceBuffer<float> au(1), bu(1);
+    quantize_on_device(x, M, K, METIS_MODE_PB16, st, &ac, &as, &au);
+    quantize_on_device(w, N, K, METIS_MODE_PB16, st, &bc, &bs, &bu);
+    DeviceBuffer<uint16_t> xa((size_t)(M * K)), wb((size_t)(N * K)), out_a((size_t)(M * N)), out_b((size_t)(M * N));
+    int rc = metis_nvfp4_dequant(ac.p, as.p, au.p, M, K, METIS_MODE_PB16, xa.p, METIS_DTYPE_BF16, st);
+    if (rc == METIS_OK) rc = metis_nvfp4_dequant(bc.p, bs.p, bu.p, N, K, METIS_MODE_PB16, wb.p, METIS_DTYPE_BF16, st);
+    metis_linear_member mem = {};
+    mem.b_codes = bc.p; mem.b_scales = bs.p; mem.b_unit = bu.p; mem.N = N;
+    const size_t need = metis_linear_grouped_workspace_bytes(M, K, &mem, 1);
+    DeviceBuffer<uint8_t> ws(need ? need : 16), aop(metis_nvfp4_decode_operand_bytes(M, K));
+    mem.out = out_a.p;
+    if (rc == METIS_OK) rc = metis_linear_fwd_grouped_bf16(ac.p, as.p, au.p, M, K, &mem, 1, METIS_DTYPE_BF16, need ? ws.p : nullptr, need, st);
+    mem.out = out_b.p;
+    if (rc == METIS_OK) rc = metis_nvfp4_decode_operand(ac.p, as.p, au.p, M, K, METIS_MODE_PB16, nullptr, aop.p, st);
+    if (rc == METIS_OK)
+        rc = metis_linear_fwd_grouped_operand(aop.p, au.p, M, K, &mem, 1, METIS_DTYPE_BF16, METIS_MODE_PB16, need ? ws.p : nullptr, need, st);
+    HIP_OK(hipStreamSynchronize(st));
+    const std::vector<uint16_t> a = out_a.download(), b = out_b.download(), xq = xa.download(), wq = wb.download();
+    size_t differ = 0, off = 0;
+    for (int64_t m = 0; m < M; ++m)
+        for (int64_t n = 0; n < N; ++n) {
+            double s = 0;
+            for (int64_t k = 0; k < K; ++k) s += (double)bf16_to_f32(xq[(size_t)(m * K + k)]) * (double)bf16_to_f32(wq[(size_t)(n * K + k)]);
+            const float f = (float)s;
+            uint32_t u;
+            memcpy(&u, &f, 4);
+            const uint16_t want = (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);      // round to nearest even
+            differ += a[(size_t)(m * N + n)] != b[(size_t)(m * N + n)];
+            off += a[(size_t)(m * N + n)] != want;
+        }
+    char line[240];
+    snprintf(line, sizeof line, "metis_linear_fwd_grouped_bf16 vs decode operand path %ldx%ldx%ld rc=%d: %zu differ; %zu of %ld off the all-bf16 "
+             "evaluation (sums on a rounding boundary)", (long)M, (long)N, (long)K, rc, differ, off, (long)(M * N));
+    check(rc == METIS_OK && differ == 0 && off * 500 <= (size_t)(M * N), line);
+    check(metis_linear_fwd_grouped_bf16(ac.p, as.p, au.p, 256, K, &mem, 1, METIS_DTYPE_BF16, nullptr, 0, st) == METIS_E_ARG,
+          "metis_linear_fwd_grouped_bf16 with 256 rows -> METIS_E_ARG (the pipelined kernel's size)");
+}
+
 // Mean mode at decode size: column mean (with the running update) -> centred quantizer -> grouped GEMM with the
 // centre inside, and the packed matrix-vector product, all against double precision on the host.
 static void check_mean_mode_decode(hipStream_t st)
@@ -421,6 +466,8 @@ int main()
 
     // ---- 7 + 8: mean mode at decode size
     check_mean_mode_decode(st);
+    check_decode_bf16(48, 160, 512, st);
+    check_decode_bf16(64, 96, 8192, st);
 
     // ---- 5: error codes
     {
