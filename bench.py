@@ -278,11 +278,24 @@ def main():
             # binary32 centre enters inside the same launches
             centres = {k_: (torch.randn(k_, generator=gd) * 0.1).to(dev) for k_ in acts}
 
-            def layer(centred=False):
+            # bf16 arithmetic (the reference's all-bf16 forward): the same kernel with bf16 operands and roundings, on the
+            # packed activation or on ready operands built once per activation
+            aops = {k_: torch.empty(L.metis_nvfp4_decode_operand_bytes(64, k_), dtype=torch.uint8, device=dev) for k_ in acts}
+
+            def layer(centred=False, bf16=0):
                 s_ = torch.cuda.current_stream().cuda_stream
                 for k_, arr in calls:
                     a_ = acts[k_]
-                    if centred:
+                    if bf16 == 1:
+                        rc = L.metis_linear_fwd_grouped_bf16(a_.codes.data_ptr(), a_.scales.data_ptr(), a_.unit.data_ptr(), 64, k_,
+                                                             ctypes.cast(arr, ctypes.c_void_p), len(arr), 0, gws.data_ptr(), gws.numel(), s_)
+                    elif bf16 == 2:
+                        rc = L.metis_nvfp4_decode_operand(a_.codes.data_ptr(), a_.scales.data_ptr(), a_.unit.data_ptr(), 64, k_, 1, None,
+                                                          aops[k_].data_ptr(), s_)
+                        assert rc == 0
+                        rc = L.metis_linear_fwd_grouped_operand(aops[k_].data_ptr(), a_.unit.data_ptr(), 64, k_,
+                                                                ctypes.cast(arr, ctypes.c_void_p), len(arr), 0, 1, gws.data_ptr(), gws.numel(), s_)
+                    elif centred:
                         rc = L.metis_linear_fwd_grouped_centered(a_.codes.data_ptr(), a_.scales.data_ptr(), a_.unit.data_ptr(), 64, k_,
                                                                  ctypes.cast(arr, ctypes.c_void_p), len(arr), 0, centres[k_].data_ptr(),
                                                                  gws.data_ptr(), gws.numel(), s_)
@@ -311,6 +324,8 @@ def main():
                 return e0.elapsed_time(e1) / 100 * 1e3
             d_us = replay_us(layer)
             d_mean_us = replay_us(lambda: layer(True))
+            d_bf16_us = replay_us(lambda: layer(bf16=1))
+            d_bf16_op_us = replay_us(lambda: layer(bf16=2))
             d_bytes = sum(n_ * k_ for n_, k_ in shapes) * (0.5 + 1.0 / 16)
             d_flops = sum(2.0 * 64 * n_ * k_ for n_, k_ in shapes)
             dec = {"workload": "config 5 decode: 7 projections of a Qwen2.5-7B layer, M=64, r=64, packed weights; q/k/v and gate/up as grouped calls (graph replay)",
@@ -318,7 +333,9 @@ def main():
                    "roofline": {"bound": "hbm", "kernel": "gemm_nvfp4_skinny_grouped_kernel", "achieved": round(d_bytes / d_us / 1e3, 1),
                                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(d_bytes / d_us / 1e3 / HBM_PEAK_GBS, 4),
                                 "traffic": TRAFFIC_DECODE_C5, "traffic_source": TRAFFIC_SOURCE},
-                   "mean_mode_us_per_layer": round(d_mean_us, 1)}
+                   "mean_mode_us_per_layer": round(d_mean_us, 1),
+                   "bf16_arithmetic_us_per_layer": {"packed_activation": round(d_bf16_us, 1),
+                                                    "ready_operands_incl_4_builds": round(d_bf16_op_us, 1)}}
         except Exception as exc:  # an optional leg must not cost the headline line
             dec = {"workload": "config 5 decode", "error": f"{type(exc).__name__}: {exc}"[:300]}
 

@@ -151,6 +151,32 @@ int metis_nvfp4_expand_tiled_rht(const void* codes, const void* scales, const fl
     return expand_xt(codes, scales, unit, rows, cols, mode, out, (hipStream_t)stream, rotate_back != 0, sign_mask);
 }
 
+size_t metis_nvfp4_deferred_bytes(int64_t rows, int64_t cols) { return deferred_bytes(rows, cols); }
+
+int metis_nvfp4_quant_row_deferred(const void* x, int64_t rows, int64_t cols, int mode, void* codes, void* deferred, size_t deferred_bytes,
+                                   void* stream)
+{
+    return quantize_row_deferred(x, rows, cols, mode, codes, deferred, deferred_bytes, (hipStream_t)stream);
+}
+
+int metis_rmsnorm_nvfp4_quant_deferred(const void* x, const void* gamma, float eps, int64_t rows, int64_t cols, int mode, void* normed,
+                                       void* codes, void* deferred, size_t deferred_bytes, void* stream)
+{
+    return rmsnorm_quantize(x, gamma, eps, rows, cols, mode, normed, codes, nullptr, nullptr, deferred, deferred_bytes, (hipStream_t)stream,
+                            true);
+}
+
+int metis_nvfp4_deferred_scales(const void* deferred, int64_t rows, int64_t cols, int mode, void* scales, float* unit, void* stream)
+{
+    return deferred_scales(deferred, rows, cols, mode, scales, unit, (hipStream_t)stream);
+}
+
+int metis_nvfp4_expand_tiled_deferred(const void* codes, const void* deferred, int64_t rows, int64_t cols, int quant_mode, int mode,
+                                      float* unit, void* out, void* stream)
+{
+    return expand_xt_deferred(codes, deferred, rows, cols, quant_mode, mode, unit, out, (hipStream_t)stream);
+}
+
 int metis_nvfp4_expand_tiled_centered(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols,
                                       const void* center, void* out, void* stream)
 {

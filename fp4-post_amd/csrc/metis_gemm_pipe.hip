@@ -44,18 +44,32 @@ __host__ __device__ __forceinline__ int xt_swz(int q) { return ((q >> 2) & 1) | 
 //   center (PB16 without RHT): the packed tensor is the centred residual of the mean mode; the operand is the
 //        reference's me + QDQ(x - me) with the sum rounded to bf16 (src/Metis/Metis/bitlinear.py:330-333 in bf16
 //        arithmetic): one bf16 value per column.
-template <int PB16, int RHT = 0>
+//   DEF: the quantizer stopped after its first phase (deferred scale bytes, nvfp4_quant.hip): `scales` holds one bf16
+//        block maximum per block instead of E4M3 bytes, `partials` the partial tensor maxima.  The kernel forms the
+//        tensor unit (written to unit_out by the first workgroup) and every scale byte itself, in the arithmetic the
+//        tensor was quantized in (QMODE) -- the expressions of quant_scales_kernel, so the bytes it would have written.
+template <int PB16, int RHT = 0, int DEF = 0, int QMODE = 0>
 __global__ __launch_bounds__(256) void expand_xt_kernel(const uint32_t* __restrict__ codes, const uint8_t* __restrict__ scales,
                                                         const float* __restrict__ unit_p, uint4* __restrict__ out, int rows,
                                                         int K, int row_tiles, uint32_t sign_mask,
-                                                        const uint16_t* __restrict__ center = nullptr)
+                                                        const uint16_t* __restrict__ center = nullptr,
+                                                        const uint32_t* __restrict__ partials = nullptr,
+                                                        float* __restrict__ unit_out = nullptr)
 {
     typedef float float2_t __attribute__((ext_vector_type(2)));
+    static_assert(DEF == 0 || RHT == 0, "deferred scale bytes: unrotated tensors");
     const int lane = threadIdx.x & 63;
     const int kt = K / 32, kgroups = (kt + 7) / 8;
     const int q = lane >> 2, chunk = (lane & 3) ^ xt_swz(q);
     const int64_t nunits = (int64_t)row_tiles * kgroups;
-    const float unit = PB16 ? *unit_p : 0.0f;
+    float unit = 0.0f;
+    if constexpr (DEF != 0) {
+        unit = tensor_unit_of<QMODE>(fold_partial_maxima(partials));
+        if (blockIdx.x == 0 && threadIdx.x == 0) *unit_out = unit;
+    } else if constexpr (PB16 != 0) {
+        unit = *unit_p;
+    }
+    const uint16_t* __restrict__ maxima = reinterpret_cast<const uint16_t*>(scales);
     for (int64_t un = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); un < nunits; un += (int64_t)gridDim.x * 4) {
         const int rb_ = (int)(un / kgroups), kg = (int)(un - (int64_t)rb_ * kgroups);
         const int row = rb_ * 16 + q;
@@ -66,7 +80,9 @@ __global__ __launch_bounds__(256) void expand_xt_kernel(const uint32_t* __restri
             if (live) {                                          // lane pairs (l, l ^ 1) share their row: both live or neither
                 const int k8 = kb * 4 + chunk;                   // index of the 8-element chunk inside the row
                 const uint32_t c = codes[(int64_t)row * (K / 8) + k8];
-                const uint32_t sb = scales[(int64_t)row * (K / 16) + (k8 >> 1)];
+                uint32_t sb;
+                if constexpr (DEF != 0) sb = scale_byte_of<QMODE>(maxima[(int64_t)row * (K / 16) + (k8 >> 1)], unit);
+                else sb = scales[(int64_t)row * (K / 16) + (k8 >> 1)];
                 if constexpr (RHT != 0) {
                     const float dq = PB16 ? rb(e4m3_value(sb) * unit) : e4m3_value(sb) * 0.00390625f;
                     const float2_t p[4] = {__builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c, 1.0f, 0), __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c, 1.0f, 1),
@@ -278,6 +294,32 @@ int expand_xt(const void* codes, const void* scales, const float* unit, int64_t 
     if (mode == METIS_MODE_PB16) { if (rht) METIS_EX(1, 1); else METIS_EX(1, 0); }
     else { if (rht) METIS_EX(0, 1); else METIS_EX(0, 0); }
 #undef METIS_EX
+    return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
+}
+
+int expand_xt_deferred(const void* codes, const void* deferred, int64_t rows, int64_t cols, int qmode, int mode, float* unit_out,
+                       void* out, hipStream_t st)
+{
+    if (rows < 0 || cols < 0) return METIS_E_ARG;
+    if (mode == METIS_MODE_P32_F32) mode = METIS_MODE_P32;
+    if ((mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) || (qmode != METIS_MODE_P32 && qmode != METIS_MODE_PB16)) return METIS_E_ARG;
+    if (cols % kBlock) return METIS_E_SHAPE;
+    if (cols % 32 || rows > INT32_MAX - 16 || cols > INT32_MAX) return METIS_E_ARG;
+    if (rows == 0 || cols == 0) return METIS_OK;
+    if (!codes || !unit_out || !out || ((uintptr_t)codes % 4) || ((uintptr_t)out % 16)) return METIS_E_ARG;
+    Workspace ws;
+    if (const int rc = carve_deferred(const_cast<void*>(deferred), deferred_bytes(rows, cols), rows, cols, &ws)) return rc;
+    const int row_tiles = (int)((rows + 15) / 16);
+    const int64_t units = (int64_t)row_tiles * ((cols / 32 + 7) / 8);
+    int64_t g = (units + 3) / 4;
+    const int64_t cap = (int64_t)device_cus() * 16;
+    if (g > cap) g = cap;
+#define METIS_EXD(P, Q) hipLaunchKernelGGL((expand_xt_kernel<P, 0, 1, Q>), dim3((unsigned)g), dim3(256), 0, st, (const uint32_t*)codes, \
+                                           (const uint8_t*)ws.amax, nullptr, (uint4*)out, (int)rows, (int)cols, row_tiles, 0u, nullptr, \
+                                           (const uint32_t*)ws.gmax, unit_out)
+    if (mode == METIS_MODE_PB16) { if (qmode) METIS_EXD(1, 1); else METIS_EXD(1, 0); }
+    else { if (qmode) METIS_EXD(0, 1); else METIS_EXD(0, 0); }
+#undef METIS_EXD
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 

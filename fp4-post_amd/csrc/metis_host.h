@@ -47,6 +47,12 @@ int quantize(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, bo
              uint64_t seed, uint64_t offset, void* codes, void* scales, float* unit, void* workspace,
              size_t workspace_bytes, hipStream_t st, const void* center = nullptr, bool resident = false,
              uint32_t spin_limit = 0);
+// deferred scale bytes (nvfp4_quant.hip): phase 1 alone into caller-owned parked data, phase 2 on it later or never
+size_t deferred_bytes(int64_t rows, int64_t cols);
+int carve_deferred(void* p, size_t bytes, int64_t rows, int64_t cols, Workspace* ws);
+int deferred_grid(uint32_t work_items);
+int quantize_row_deferred(const void* x, int64_t rows, int64_t cols, int mode, void* codes, void* deferred, size_t bytes, hipStream_t st);
+int deferred_scales(const void* deferred, int64_t rows, int64_t cols, int mode, void* scales, float* unit, hipStream_t st);
 // the row quantizer on the library's own static scratch (no workspace argument); nvfp4_quant.hip
 int quantize_row_static(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, void* codes, void* scales,
                         float* unit, hipStream_t st);
@@ -58,7 +64,8 @@ int quant_values(const void* x, const void* s, int64_t rows, int64_t cols, int m
 int rquant_values(const void* xq, void* s, int64_t rows, int64_t cols, int mode, void* out, float* scratch,
                   hipStream_t st);
 int rmsnorm_quantize(const void* x, const void* gamma, float eps, int64_t rows, int64_t cols, int mode, void* normed,
-                     void* codes, void* scales, float* unit, void* workspace, size_t workspace_bytes, hipStream_t st);
+                     void* codes, void* scales, float* unit, void* workspace, size_t workspace_bytes, hipStream_t st,
+                     bool deferred = false);
 int gemm_nvfp4(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes, const void* b_scales,
                const float* b_unit, int64_t M, int64_t N, int64_t K, const void* t, const void* u, int64_t r,
                const void* bias, void* out, int out_dtype, hipStream_t st, void* workspace = nullptr,
@@ -130,6 +137,9 @@ int gemm_expanded(const void* a_exp, const float* a_unit, const void* b_exp, con
 size_t expand_xt_bytes(int64_t rows, int64_t cols);
 int expand_xt(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, int mode, void* out,
               hipStream_t st, int rht = 0, uint32_t sign_mask = 0, const void* center = nullptr);
+// the same from a tensor whose quantizer call deferred its scale bytes (qmode: the arithmetic it was quantized in); writes the unit
+int expand_xt_deferred(const void* codes, const void* deferred, int64_t rows, int64_t cols, int qmode, int mode, float* unit_out,
+                       void* out, hipStream_t st);
 // a dense bf16 / binary32 tensor in the tiled layout (optional per-column bf16 scale first)
 int dense_xt(const void* x, int64_t rows, int64_t cols, int64_t ld, int dtype, const void* col_scale, int mode, void* out, hipStream_t st);
 // the tiled operand [cols, rows] (contraction over the packed tensor's rows); rows % 32 == 0

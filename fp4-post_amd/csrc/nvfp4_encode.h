@@ -274,14 +274,41 @@ __device__ __forceinline__ void hadamard16_inverse(float (&v)[kBlock], uint32_t 
     for (int j = 0; j < kBlock; ++j) v[j] = __uint_as_float(__float_as_uint(v[j] * 0.0625f) ^ (((sign_mask >> j) & 1u) << 31));
 }
 
-// publish the workgroup's maximum block-maximum (non-negative floats order like their bit patterns)
-__device__ __forceinline__ void publish_group_max(float m, uint32_t* ws_gmax)
+// publish the workgroup's maximum block-maximum (non-negative floats order like their bit patterns).
+// fill_to: entries gridDim.x .. fill_to-1 are cleared as well, for readers that always fold a fixed number of entries.
+__device__ __forceinline__ void publish_group_max(float m, uint32_t* ws_gmax, uint32_t fill_to = 0)
 {
     __shared__ float smax[4];
     m = wave_max(m);
     if ((threadIdx.x & 63) == 0) smax[threadIdx.x >> 6] = m;
     __syncthreads();
     if (threadIdx.x == 0) ws_gmax[blockIdx.x] = __float_as_uint(fmaxf(fmaxf(smax[0], smax[1]), fmaxf(smax[2], smax[3])));
+    for (uint32_t j = gridDim.x + blockIdx.x * 256u + threadIdx.x; j < fill_to; j += gridDim.x * 256u) ws_gmax[j] = 0u;
+}
+
+// Deferred scale bytes: a quantizer call may stop after phase 1 and hand its parked bf16 block maxima and its partial
+// maxima (always kDeferredPartials entries, unused ones zero) to the consumer, which forms the tensor unit and the E4M3
+// bytes itself (quant.py:21-23) -- the same expressions as quant_scales_kernel, so the same bits.
+constexpr uint32_t kDeferredPartials = 2048;
+// tensor maximum from the partial maxima: every thread of a 256-thread workgroup calls this
+__device__ __forceinline__ float fold_partial_maxima(const uint32_t* __restrict__ partials)
+{
+    __shared__ float fmax_s[4];
+    const uint4 a = reinterpret_cast<const uint4*>(partials)[threadIdx.x];
+    const uint4 b = reinterpret_cast<const uint4*>(partials)[threadIdx.x + 256];
+    float m = fmaxf(fmaxf(fmaxf(__uint_as_float(a.x), __uint_as_float(a.y)), fmaxf(__uint_as_float(a.z), __uint_as_float(a.w))),
+                    fmaxf(fmaxf(__uint_as_float(b.x), __uint_as_float(b.y)), fmaxf(__uint_as_float(b.z), __uint_as_float(b.w))));
+    m = wave_max(m);
+    if ((threadIdx.x & 63) == 0) fmax_s[threadIdx.x >> 6] = m;
+    __syncthreads();
+    return fmaxf(fmaxf(fmax_s[0], fmax_s[1]), fmaxf(fmax_s[2], fmax_s[3]));
+}
+template <int MODE>
+__device__ __forceinline__ float tensor_unit_of(float amax) { return rd<MODE>(block_scalar<MODE>(amax) / 448.0f); }
+template <int MODE>
+__device__ __forceinline__ uint32_t scale_byte_of(uint32_t amax_bf16, float unit)
+{
+    return e4m3_byte(rd<MODE>(block_scalar<MODE>(__uint_as_float(amax_bf16 << 16)) / unit));
 }
 
 }  // namespace metis

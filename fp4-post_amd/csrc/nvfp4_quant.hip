@@ -40,7 +40,7 @@ __device__ __forceinline__ float block_scalar_ieee(float amax) { return amax / 6
 template <int MODE>
 __global__ __launch_bounds__(256) void quant_codes_contig_kernel(const uint4* __restrict__ x, uint2* __restrict__ codes,
                                                                  uint16_t* __restrict__ ws_amax, uint32_t* __restrict__ ws_gmax,
-                                                                 uint32_t nblocks)
+                                                                 uint32_t nblocks, uint32_t fill_to)
 {
     float gmax = 0.0f;
     const uint32_t step = gridDim.x * 256u;
@@ -60,7 +60,7 @@ __global__ __launch_bounds__(256) void quant_codes_contig_kernel(const uint4* __
         codes[i] = encode_block<MODE, false>(v, block_scalar<MODE>(am), none);
         c0 = n0; c1 = n1; i = nxt;
     }
-    publish_group_max(gmax, ws_gmax);
+    publish_group_max(gmax, ws_gmax, fill_to);
 }
 
 // HAD: every block is rotated first (NV recipe, hadamard16_forward): the rotated tensor is what gets quantized, as in
@@ -256,7 +256,7 @@ __global__ __launch_bounds__(256) void quant_scales_kernel(const uint16_t* __res
     __syncthreads();
     const float amax = fmaxf(fmaxf(smax[0], smax[1]), fmaxf(smax[2], smax[3]));
     // max over blocks of scalar(amax_block) = scalar(max amax_block): the scalar map is monotone
-    const float unit = rd<MODE>(block_scalar<MODE>(amax) / 448.0f);
+    const float unit = tensor_unit_of<MODE>(amax);
     if (blockIdx.x == 0 && threadIdx.x == 0) *unit_out = unit;
 
     auto four_bytes = [&](uint32_t w0, uint32_t w1) {
@@ -669,7 +669,7 @@ static int launch_quant(const void* x, int64_t rows, int64_t cols, int64_t ld, c
         if constexpr (!SR && !WIDE && !HAD) {
             if (!center && ld == cols) {
                 hipLaunchKernelGGL((quant_codes_contig_kernel<MODE>), dim3(g1), dim3(256), 0, st, (const uint4*)x, (uint2*)codes,
-                                   ws.amax, ws.gmax, nblocks);
+                                   ws.amax, ws.gmax, nblocks, 0u);
                 return launch_scales(MODE, ws, (uint32_t)g1, scales, unit, nblocks, st);
             }
         }
@@ -721,6 +721,67 @@ int quantize(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, bo
         else { if (!col) METIS_Q(1, true, false); else METIS_Q(1, true, true); }
     }
 #undef METIS_Q
+}
+
+// ---------------------------------------------------------------------------------------------
+// Deferred scale bytes.  The codes of a block depend on the block alone, the scale bytes on the tensor maximum: a
+// consumer that runs after the quantizer anyway (the tiled expansion ahead of a GEMM) can form them from the parked
+// block maxima, and the quantizer is then ONE launch.  The caller owns the parked data: [0, 8 KiB) the partial maxima
+// (kDeferredPartials entries), then one bf16 maximum per block.  Round-to-nearest rows of a contiguous bf16 tensor.
+// ---------------------------------------------------------------------------------------------
+size_t deferred_bytes(int64_t rows, int64_t cols)
+{
+    if (rows <= 0 || cols <= 0) return 0;
+    const size_t nblocks = (size_t)((rows * cols + 15) / 16);
+    return kDeferredPartials * 4 + ((nblocks * 2 + 255) / 256) * 256;
+}
+
+int carve_deferred(void* p, size_t bytes, int64_t rows, int64_t cols, Workspace* ws)
+{
+    if (!p || ((uintptr_t)p % 256) || bytes < deferred_bytes(rows, cols)) return METIS_E_WORKSPACE;
+    ws->gmax = static_cast<uint32_t*>(p);
+    ws->sync = nullptr;
+    ws->amax = reinterpret_cast<uint16_t*>(static_cast<char*>(p) + kDeferredPartials * 4);
+    return METIS_OK;
+}
+
+int deferred_grid(uint32_t work_items)
+{
+    const int g = grid_for(work_items);
+    return g > (int)kDeferredPartials ? (int)kDeferredPartials : g;
+}
+
+int quantize_row_deferred(const void* x, int64_t rows, int64_t cols, int mode, void* codes, void* deferred, size_t bytes, hipStream_t st)
+{
+    if (rows < 0 || cols < 0) return METIS_E_ARG;
+    if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) return METIS_E_ARG;
+    if (cols % kBlock) return METIS_E_SHAPE;
+    if (rows == 0 || cols == 0) return METIS_OK;
+    if (!x || !codes || ((uintptr_t)x % 16) || ((uintptr_t)codes % 8)) return METIS_E_ARG;
+    if (rows * cols / kBlock >= (int64_t)1 << 31) return METIS_E_ARG;
+    Workspace ws;
+    if (const int rc = carve_deferred(deferred, bytes, rows, cols, &ws)) return rc;
+    const uint32_t nblocks = (uint32_t)(rows * cols / kBlock);
+    const int g1 = deferred_grid(nblocks);
+    if (mode == 0)
+        hipLaunchKernelGGL((quant_codes_contig_kernel<0>), dim3(g1), dim3(256), 0, st, (const uint4*)x, (uint2*)codes, ws.amax, ws.gmax,
+                           nblocks, kDeferredPartials);
+    else
+        hipLaunchKernelGGL((quant_codes_contig_kernel<1>), dim3(g1), dim3(256), 0, st, (const uint4*)x, (uint2*)codes, ws.amax, ws.gmax,
+                           nblocks, kDeferredPartials);
+    return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
+}
+
+// phase 2 on parked data, whenever somebody wants the bytes after all
+int deferred_scales(const void* deferred, int64_t rows, int64_t cols, int mode, void* scales, float* unit, hipStream_t st)
+{
+    if (rows < 0 || cols < 0 || (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16)) return METIS_E_ARG;
+    if (cols % kBlock) return METIS_E_SHAPE;
+    if (rows == 0 || cols == 0) return METIS_OK;
+    if (!scales || !unit || ((uintptr_t)scales % 8)) return METIS_E_ARG;
+    Workspace ws;
+    if (const int rc = carve_deferred(const_cast<void*>(deferred), deferred_bytes(rows, cols), rows, cols, &ws)) return rc;
+    return launch_scales(mode, ws, kDeferredPartials, scales, unit, (uint32_t)(rows * cols / kBlock), st);
 }
 
 // ---------------------------------------------------------------------------------------------

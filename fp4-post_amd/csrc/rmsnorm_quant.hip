@@ -19,7 +19,7 @@ __global__ __launch_bounds__(256) void rmsnorm_quant_kernel(const uint16_t* __re
                                                             const uint16_t* __restrict__ gamma, float eps,
                                                             uint32_t rows, uint32_t cols, uint16_t* __restrict__ normed,
                                                             uint2* __restrict__ codes, uint16_t* __restrict__ ws_amax,
-                                                            uint32_t* __restrict__ ws_gmax)
+                                                            uint32_t* __restrict__ ws_gmax, uint32_t fill_to)
 {
     __shared__ float part[2][4];
     const uint32_t nbpr = cols / kBlock;
@@ -99,39 +99,44 @@ __global__ __launch_bounds__(256) void rmsnorm_quant_kernel(const uint16_t* __re
             }
         }
     }
-    publish_group_max(gmax, ws_gmax);
+    publish_group_max(gmax, ws_gmax, fill_to);
 }
 
+// deferred: stop after the main kernel; `workspace` is then the caller-owned parked data of the deferred form
+// (nvfp4_quant.hip) and scales / unit are not written.
 int rmsnorm_quantize(const void* x, const void* gamma, float eps, int64_t rows, int64_t cols, int mode, void* normed,
-                     void* codes, void* scales, float* unit, void* workspace, size_t workspace_bytes, hipStream_t st)
+                     void* codes, void* scales, float* unit, void* workspace, size_t workspace_bytes, hipStream_t st, bool deferred)
 {
     if (rows < 0 || cols < 0) return METIS_E_ARG;
     if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) return METIS_E_ARG;
     if (cols % kBlock) return METIS_E_SHAPE;
     if (rows == 0 || cols == 0) return METIS_OK;
-    if (!x || !gamma || !codes || !scales || !unit) return METIS_E_ARG;
+    if (!x || !gamma || !codes || (!deferred && (!scales || !unit))) return METIS_E_ARG;
     if (cols > 256 * kBlock * 4) return METIS_E_ARG;          // a row is held in registers: at most 16384 columns
     if (rows * cols / kBlock >= (int64_t)1 << 31) return METIS_E_ARG;
     if (((uintptr_t)x % 16) || ((uintptr_t)gamma % 16) || ((uintptr_t)codes % 8) || ((uintptr_t)scales % 8) ||
         (normed && ((uintptr_t)normed % 16)))
         return METIS_E_ARG;
     Workspace ws;
-    int rc = carve_workspace(workspace, workspace_bytes, rows, cols, &ws);
+    int rc = deferred ? carve_deferred(workspace, workspace_bytes, rows, cols, &ws) : carve_workspace(workspace, workspace_bytes, rows, cols, &ws);
     if (rc != METIS_OK) return rc;
     int64_t g = rows;
     const int64_t cap = (int64_t)device_cus() * 8;
     if (g > cap) g = cap;
     if (g > kMaxGroups) g = kMaxGroups;
+    if (deferred && g > (int64_t)kDeferredPartials) g = kDeferredPartials;
+    const uint32_t fill_to = deferred ? kDeferredPartials : 0u;
     const int nbt = (int)((cols / kBlock + 255) / 256);
 #define METIS_R(M, NBT, W) hipLaunchKernelGGL((rmsnorm_quant_kernel<M, NBT, W>), dim3((int)g), dim3(256), 0, st, \
         (const uint16_t*)x, (const uint16_t*)gamma, eps, (uint32_t)rows, (uint32_t)cols, (uint16_t*)normed, (uint2*)codes, \
-        ws.amax, ws.gmax)
+        ws.amax, ws.gmax, fill_to)
 #define METIS_RN(M, W) do { if (nbt <= 1) METIS_R(M, 1, W); else if (nbt == 2) METIS_R(M, 2, W); else METIS_R(M, 4, W); } while (0)
     if (mode == 0) { if (normed) METIS_RN(0, true); else METIS_RN(0, false); }
     else { if (normed) METIS_RN(1, true); else METIS_RN(1, false); }
 #undef METIS_RN
 #undef METIS_R
     if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
+    if (deferred) return METIS_OK;
     return launch_scales(mode, ws, (uint32_t)g, scales, unit, (uint32_t)(rows * cols / kBlock), st);
 }
 

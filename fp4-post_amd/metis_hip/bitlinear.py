@@ -322,7 +322,10 @@ class LinearLowbitFunction(torch.autograd.Function):
         if (not F.enable_nv_recipe or F._nv_on_kernels()) and _packable(input_, F.q_forward_input):
             if not F.enable_activation_svd:
                 # the kernels read bf16 values and take the arithmetic as a mode: no upcast copy of a bf16 tensor
-                return F.q_forward_input.pack(_flat2d(input_), arith=F.compute_dtype)
+                # from 256 rows on the consumer is the tiled expansion, which forms the scale bytes itself
+                x2 = _flat2d(input_)
+                more = {"deferred": True} if x2.shape[0] >= 256 else {}
+                return F.q_forward_input.pack(x2, arith=F.compute_dtype, **more)
             if F._mean_mode_packable():
                 # mean + QDQ(x - mean) (reference 311-336) without materialising either: the subtraction happens
                 # inside the quantizer and the mean's contribution to a matmul is a rank-one term

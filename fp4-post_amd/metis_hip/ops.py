@@ -39,9 +39,39 @@ class PackedNVFP4:
     rht: int | None = None                    # NV recipe: the packed values are those of the ROTATED tensor (sign mask of the rotation)
     tiled_t: torch.Tensor | None = None       # tiled expansion of the transposed tensor (contraction over this tensor's rows)
     tiled_t_pb16: torch.Tensor | None = None
+    # deferred scale bytes: the quantizer stopped after its first launch and parked the block maxima here; `scales` and
+    # `unit` are produced on first access (one more launch), unless a consumer that forms the bytes itself
+    # (expand_tiled) got there first and wrote the unit
+    deferred: torch.Tensor | None = None
 
     def dequantize(self, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
         return dequantize(self, dtype)
+
+    def _materialize(self) -> None:
+        d = self.__dict__
+        scales = torch.empty(self.rows, self.cols // BLOCK, dtype=torch.uint8, device=self.codes.device)
+        rc = load().metis_nvfp4_deferred_scales(d["deferred"].data_ptr(), self.rows, self.cols, self.mode, scales.data_ptr(),
+                                                d["_unit"].data_ptr(), _stream())
+        check(rc, "metis_nvfp4_deferred_scales", (self.rows, self.cols))
+        d["_scales"], d["_unit_ready"] = scales, True
+
+
+def _packed_scales(self):
+    d = self.__dict__
+    if d.get("_scales") is None and d.get("deferred") is not None:
+        self._materialize()
+    return d.get("_scales")
+
+
+def _packed_unit(self):
+    d = self.__dict__
+    if d.get("deferred") is not None and not d.get("_unit_ready", False):
+        self._materialize()
+    return d.get("_unit")
+
+
+PackedNVFP4.scales = property(_packed_scales, lambda self, v: self.__dict__.__setitem__("_scales", v))
+PackedNVFP4.unit = property(_packed_unit, lambda self, v: self.__dict__.__setitem__("_unit", v))
 
 
 @dataclass
@@ -114,7 +144,8 @@ def _as_2d_for_quant(x: torch.Tensor, mode: int) -> tuple[torch.Tensor, int]:
 
 def quantize(x: torch.Tensor, mode: int = MODE_P32, *, col: bool = False, sr: bool = False,
              noise: torch.Tensor | None = None, seed: int = 0, offset: int = 0,
-             center: torch.Tensor | None = None, resident: bool = False, spin_limit: int = 0) -> PackedNVFP4:
+             center: torch.Tensor | None = None, resident: bool = False, spin_limit: int = 0,
+             deferred: bool = False) -> PackedNVFP4:
     """NVFP4-quantize x (flattened to [R, C]).
 
     col=False: blocks of 16 along C -> PackedNVFP4 of shape (R, C).
@@ -126,6 +157,9 @@ def quantize(x: torch.Tensor, mode: int = MODE_P32, *, col: bool = False, sr: bo
     resident : round-to-nearest rows of a bf16 tensor as ONE launch (metis_nvfp4_quant_row_resident), same bytes: a
                workgroup that gives up waiting for the grid's maximum after `spin_limit` polls (0: library default)
                leaves its scale bytes to the last workgroup.
+    deferred : round-to-nearest rows of a bf16 tensor: only the first of the two launches now (codes, parked block
+               maxima); `scales` and `unit` of the result appear on first access, or never if the only consumer is
+               expand_tiled, which forms the bytes itself.  Same bits either way.
     """
     x2, kmode = _as_2d_for_quant(x, mode)
     rows, cols = x2.shape
@@ -135,10 +169,17 @@ def quantize(x: torch.Tensor, mode: int = MODE_P32, *, col: bool = False, sr: bo
     prow, pcol = (cols, rows) if col else (rows, cols)
     dev = x2.device
     codes = torch.empty(prow, pcol // 2, dtype=torch.uint8, device=dev)
-    scales = torch.empty(prow, pcol // BLOCK, dtype=torch.uint8, device=dev)
     unit = torch.empty(1, dtype=torch.float32, device=dev)
-    ws = _workspace(rows, cols, dev)
     L = load()
+    if (deferred and not col and not sr and center is None and kmode in (MODE_P32, MODE_PB16) and x2.stride(0) == cols
+            and rows * cols > 0):
+        parked = torch.empty(L.metis_nvfp4_deferred_bytes(rows, cols), dtype=torch.uint8, device=dev)
+        rc = L.metis_nvfp4_quant_row_deferred(x2.data_ptr(), rows, cols, kmode, codes.data_ptr(), parked.data_ptr(), parked.numel(),
+                                              _stream())
+        check(rc, "metis_nvfp4_quant_row_deferred", x.shape)
+        return PackedNVFP4(codes, None, unit, prow, pcol, mode, deferred=parked)
+    scales = torch.empty(prow, pcol // BLOCK, dtype=torch.uint8, device=dev)
+    ws = _workspace(rows, cols, dev)
     if center is not None:
         cen = center.reshape(-1).to(device=dev, dtype=torch.bfloat16 if mode == MODE_PB16 else torch.float32).contiguous()
         if cen.numel() != cols:
@@ -370,7 +411,14 @@ def expand_tiled(p: PackedNVFP4, cache: bool = True, mode: int = MODE_P32, cente
     if have is not None:
         return have
     out = torch.empty(L.metis_nvfp4_expand_tiled_bytes(p.rows, p.cols), dtype=torch.uint8, device=p.codes.device)
-    if p.rht is not None:                     # NV recipe: the operand holds the values rotated back
+    d = p.__dict__
+    if d.get("deferred") is not None and d.get("_scales") is None and p.rht is None and p.cols % 32 == 0:
+        # the scale bytes were never written: this kernel forms them from the parked block maxima, and writes the unit
+        rc = L.metis_nvfp4_expand_tiled_deferred(p.codes.data_ptr(), d["deferred"].data_ptr(), p.rows, p.cols, p.mode, mode,
+                                                 d["_unit"].data_ptr(), out.data_ptr(), _stream())
+        check(rc, "metis_nvfp4_expand_tiled_deferred", (p.rows, p.cols))
+        d["_unit_ready"] = True
+    elif p.rht is not None:                   # NV recipe: the operand holds the values rotated back
         rc = L.metis_nvfp4_expand_tiled_rht(p.codes.data_ptr(), p.scales.data_ptr(), p.unit.data_ptr(), p.rows, p.cols, mode,
                                             p.rht, 1, 0, out.data_ptr(), _stream())
     else:
@@ -498,8 +546,9 @@ def linear_fwd_tiled(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None =
 
 
 def rmsnorm_quantize(x: torch.Tensor, gamma: torch.Tensor, eps: float, mode: int = MODE_P32,
-                     want_normed: bool = True):
-    """Fused RMSNorm -> NVFP4.  Returns (normed bf16 or None, PackedNVFP4)."""
+                     want_normed: bool = True, deferred: bool = False):
+    """Fused RMSNorm -> NVFP4.  Returns (normed bf16 or None, PackedNVFP4).  deferred: as in quantize (one launch; scale
+    bytes and unit on first access, or formed by expand_tiled)."""
     x2 = _as_2d_bf16(x)
     rows, cols = x2.shape
     if cols % BLOCK:
@@ -508,8 +557,18 @@ def rmsnorm_quantize(x: torch.Tensor, gamma: torch.Tensor, eps: float, mode: int
     dev = x2.device
     normed = torch.empty(rows, cols, dtype=torch.bfloat16, device=dev) if want_normed else None
     codes = torch.empty(rows, cols // 2, dtype=torch.uint8, device=dev)
-    scales = torch.empty(rows, cols // BLOCK, dtype=torch.uint8, device=dev)
     unit = torch.empty(1, dtype=torch.float32, device=dev)
+    if deferred and rows * cols > 0:
+        L = load()
+        parked = torch.empty(L.metis_nvfp4_deferred_bytes(rows, cols), dtype=torch.uint8, device=dev)
+        rc = L.metis_rmsnorm_nvfp4_quant_deferred(x2.data_ptr(), g.data_ptr(), float(eps), rows, cols, mode,
+                                                  None if normed is None else normed.data_ptr(), codes.data_ptr(),
+                                                  parked.data_ptr(), parked.numel(), _stream())
+        check(rc, "metis_rmsnorm_nvfp4_quant_deferred", x.shape)
+        if normed is not None:
+            normed = normed.reshape(x.shape)
+        return normed, PackedNVFP4(codes, None, unit, rows, cols, mode, deferred=parked)
+    scales = torch.empty(rows, cols // BLOCK, dtype=torch.uint8, device=dev)
     ws = _workspace(rows, cols, dev)
     rc = load().metis_rmsnorm_nvfp4_quant(x2.data_ptr(), g.data_ptr(), float(eps), rows, cols, mode,
                                           None if normed is None else normed.data_ptr(), codes.data_ptr(),

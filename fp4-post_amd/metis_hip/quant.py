@@ -88,11 +88,13 @@ class _NVFP4Base(BlockQuantFunc):
     @classmethod
     @torch.no_grad()
     def pack(cls, x: torch.Tensor, col: bool = False, noise: torch.Tensor | None = None,
-             arith: torch.dtype | None = None, center: torch.Tensor | None = None, rht: int | None = None) -> ops.PackedNVFP4:
+             arith: torch.dtype | None = None, center: torch.Tensor | None = None, rht: int | None = None,
+             deferred: bool = False) -> ops.PackedNVFP4:
         """Packed NVFP4 (codes, E4M3 scale bytes, unit) of x in the arithmetic of x's dtype, or of `arith`
         when given: a bf16 tensor packed with arith=float32 gives what x.float() would, without the copy.
         center: per-column vector subtracted first (mean mode): the packed tensor is that of x - center.
-        rht: sign mask of the NV recipe's rotation: the packed tensor is that of the rotated x (see ops.quantize_rht)."""
+        rht: sign mask of the NV recipe's rotation: the packed tensor is that of the rotated x (see ops.quantize_rht).
+        deferred: round-to-nearest rows only: one launch now, the scale bytes when (and if) somebody reads them (ops.quantize)."""
         _need_gpu(x)
         if not col:
             cls._check(x)
@@ -107,7 +109,7 @@ class _NVFP4Base(BlockQuantFunc):
         if cls.stochastic:
             return ops.quantize(x, mode, col=col, sr=True, noise=noise, seed=_NVFP4Base.sr_seed,
                                 offset=cls._next_offset(x.numel()) if noise is None else 0, center=center)
-        return ops.quantize(x, mode, col=col, center=center)
+        return ops.quantize(x, mode, col=col, center=center, deferred=deferred)
 
     @classmethod
     @torch.no_grad()

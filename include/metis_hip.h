@@ -304,6 +304,34 @@ int metis_nvfp4_expand_tiled_rht(const void *codes, const void *scales, const fl
                                  int64_t cols, int mode, uint32_t sign_mask, int rotate_back,
                                  int transpose, void *out, void *stream);
 /*
+ * Deferred scale bytes.  The codes of a block depend on the block alone (src/Metis/Metis/quant.py:27), the E4M3 bytes
+ * and the tensor unit on the maximum over the whole tensor (quant.py:21-23) -- which is why the quantizers above are two
+ * launches.  A consumer that runs after the quantizer anyway can form the bytes itself, so these entry points stop
+ * after the first launch and park what the second would have read in a buffer the CALLER owns (it travels with the
+ * codes): 2048 partial tensor maxima, then one bf16 block maximum per block.  Round-to-nearest rows of a contiguous
+ * bf16 tensor (ld == cols), mode METIS_MODE_P32 or METIS_MODE_PB16.
+ *   metis_nvfp4_deferred_bytes           size of that buffer; 256-byte aligned, contents need no initialisation
+ *   metis_nvfp4_quant_row_deferred       metis_nvfp4_quant_row without scales and unit
+ *   metis_rmsnorm_nvfp4_quant_deferred   metis_rmsnorm_nvfp4_quant likewise
+ *   metis_nvfp4_expand_tiled_deferred    metis_nvfp4_expand_tiled reading the parked data: quant_mode = the mode of the
+ *                                        quantizer call, mode = the operand format; also writes the tensor unit (float
+ *                                        [1], required), which metis_linear_fwd_tiled reads afterwards.  Same bits as
+ *                                        the two-launch quantizer followed by metis_nvfp4_expand_tiled
+ *   metis_nvfp4_deferred_scales          the second launch after all: scales and unit exactly as metis_nvfp4_quant_row
+ *                                        would have written them, for consumers that read E4M3 bytes
+ */
+size_t metis_nvfp4_deferred_bytes(int64_t rows, int64_t cols);
+int metis_nvfp4_quant_row_deferred(const void *x, int64_t rows, int64_t cols, int mode, void *codes,
+                                   void *deferred, size_t deferred_bytes, void *stream);
+int metis_rmsnorm_nvfp4_quant_deferred(const void *x, const void *gamma, float eps, int64_t rows, int64_t cols,
+                                       int mode, void *normed, void *codes, void *deferred,
+                                       size_t deferred_bytes, void *stream);
+int metis_nvfp4_expand_tiled_deferred(const void *codes, const void *deferred, int64_t rows, int64_t cols,
+                                      int quant_mode, int mode, float *unit, void *out, void *stream);
+int metis_nvfp4_deferred_scales(const void *deferred, int64_t rows, int64_t cols, int mode, void *scales,
+                                float *unit, void *stream);
+
+/*
  * Mean mode in bf16 arithmetic: the activation the reference multiplies with is X^ = me + QDQ(X - me) as ONE bf16
  * tensor, the sum rounded to bf16 (LinearLowbitFunction.svd_quant with metis_mode = "mean",
  * src/Metis/Metis/bitlinear.py:311-336, under compute_dtype = bfloat16).  This is metis_nvfp4_expand_tiled with

@@ -195,10 +195,10 @@ def test_shared_activation_is_quantized_once_per_group():
     base = quant_func["nvfp4e2m1bnosr"]
     orig = base.pack.__func__
 
-    def counting(cls, x, col=False, noise=None, arith=None):
+    def counting(cls, x, col=False, noise=None, arith=None, **more):
         if not col and tuple(x.shape) == (96, 256):      # the activation, not the [N, 256] weights
             calls["n"] += 1
-        return orig(cls, x, col, noise, arith)
+        return orig(cls, x, col, noise, arith, **more)
 
     base.pack = classmethod(counting)
     try:
@@ -351,9 +351,9 @@ def test_packed_weight_cache_reuses_then_invalidates_on_the_device():
     orig = base.pack.__func__
     packs = []
 
-    def spy(cls, t_, col=False, noise=None, arith=None, center=None):
+    def spy(cls, t_, col=False, noise=None, arith=None, center=None, **more):
         packs.append((tuple(t_.shape), bool(col)))
-        return orig(cls, t_, col, noise, arith, center)
+        return orig(cls, t_, col, noise, arith, center, **more)
 
     base.pack = classmethod(spy)
     try:
@@ -625,10 +625,10 @@ def test_fused_rmsnorm_feeds_the_projection_groups_of_a_qwen2_layer():
     orig = base.pack.__func__
     seen = []
 
-    def spy(cls, t_, col=False, noise=None, arith=None):
+    def spy(cls, t_, col=False, noise=None, arith=None, **more):
         if not col:
             seen.append(tuple(t_.shape))
-        return orig(cls, t_, col, noise, arith)
+        return orig(cls, t_, col, noise, arith, **more)
 
     base.pack = classmethod(spy)
     try:

@@ -289,6 +289,49 @@ def test_full_size_config1(ops, tag, mode):
 
 
 @pytest.mark.parametrize("tag,mode", MODES)
+def test_deferred_scale_bytes_give_the_same_packed_tensor(ops, tag, mode):
+    """deferred=True runs the first launch only and parks the block maxima with the packed tensor.  Whoever reads
+    `scales` / `unit` later gets the bytes of the two-launch path; the tiled expansion forms them itself (it never
+    materialises them) and is bit-equal to the expansion of the eager tensor, in both operand formats; and a parked
+    buffer that is all garbage beforehand changes nothing (every entry a reader folds is written by the call)."""
+    from helpers import untile
+    shapes = [(8192, 4096), (16, 32), (64, 256), (4096, 1536), (1000, 96), (3, 32), (16384, 4096), (300, 7168)]
+    for k, (r, c) in enumerate(shapes):
+        x = synthetic_activation(700 + k, r, c).cuda()
+        ref = ops.quantize(x, mode)
+        got = ops.quantize(x, mode, deferred=True)
+        assert got.deferred is not None and got.__dict__.get("_scales") is None
+        for fmt in (0, 1):
+            if fmt == 1 and mode == 0:
+                continue                                          # bf16 operands belong to tensors packed in bf16 arithmetic
+            lazy = ops.quantize(x, mode, deferred=True)
+            a = ops.expand_tiled(lazy, cache=False, mode=fmt)
+            b = ops.expand_tiled(ref, cache=False, mode=fmt)
+            assert torch.equal(a, b), f"tiled operand differs, shape {r}x{c} {tag} format {fmt}"
+            assert lazy.__dict__.get("_scales") is None and lazy.__dict__["_unit_ready"]
+            assert float(lazy.unit.cpu()) == float(ref.unit.cpu())
+            assert lazy.__dict__.get("_scales") is None               # reading the unit after the expansion launches nothing
+            _check_packed(lazy, ref.codes.cpu(), ref.scales.cpu(), ref.unit.cpu(), f"after expansion, shape {r}x{c} {tag}")
+        _check_packed(got, ref.codes.cpu(), ref.scales.cpu(), ref.unit.cpu(), f"shape {r}x{c} {tag}")
+        assert torch.equal(ops.dequantize(got, torch.bfloat16), ops.dequantize(ref, torch.bfloat16))
+    # through the C ABI with a poisoned parked buffer
+    from metis_hip import _lib
+    L = _lib.load()
+    x = synthetic_activation(777, 48, 64).cuda()
+    ref = ops.quantize(x, mode)
+    parked = torch.full((L.metis_nvfp4_deferred_bytes(48, 64),), 0x7f, dtype=torch.uint8, device="cuda")
+    codes = torch.empty(48, 32, dtype=torch.uint8, device="cuda")
+    scales = torch.empty(48, 4, dtype=torch.uint8, device="cuda")
+    unit = torch.empty(1, dtype=torch.float32, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    assert L.metis_nvfp4_quant_row_deferred(x.data_ptr(), 48, 64, mode, codes.data_ptr(), parked.data_ptr(), parked.numel(), st) == 0
+    assert L.metis_nvfp4_deferred_scales(parked.data_ptr(), 48, 64, mode, scales.data_ptr(), unit.data_ptr(), st) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(codes, ref.codes) and torch.equal(scales, ref.scales) and float(unit.cpu()) == float(ref.unit.cpu())
+    assert L.metis_nvfp4_quant_row_deferred(x.data_ptr(), 48, 64, mode, codes.data_ptr(), parked.data_ptr(), 16, st) == _lib.E_WORKSPACE
+
+
+@pytest.mark.parametrize("tag,mode", MODES)
 def test_single_launch_variant_matches_two_launch_path(ops, tag, mode):
     """The single-launch kernel (grid-wide maximum through a tree of device-scope atomics) gives the same
     bytes as the two-launch path, call after call on one workspace (the generation tag

@@ -44,6 +44,24 @@ def test_fused_rmsnorm_quant(rows, cols, mode):
     assert none is None and torch.equal(p2.codes, p.codes) and torch.equal(p2.scales, p.scales)
 
 
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("rows,cols", [(64, 512), (300, 3584), (16384, 4096), (7, 96)])
+def test_fused_rmsnorm_quant_with_deferred_scale_bytes(rows, cols, mode):
+    """deferred=True: the main kernel only.  Same normed tensor and codes; scale bytes and unit appear on first access
+    with the bytes of the two-launch call, and the tiled expansion forms them itself, bit-equal to the eager tensor's."""
+    from metis_hip import ops
+    x = synthetic_activation(1100 + rows, rows, cols).cuda()
+    gamma = _gamma(8, cols).cuda()
+    normed, ref = ops.rmsnorm_quantize(x, gamma, 1e-6, mode)
+    normed2, lazy = ops.rmsnorm_quantize(x, gamma, 1e-6, mode, deferred=True)
+    assert torch.equal(normed, normed2) and torch.equal(lazy.codes, ref.codes)
+    assert lazy.__dict__.get("_scales") is None
+    assert torch.equal(ops.expand_tiled(lazy, cache=False, mode=mode), ops.expand_tiled(ref, cache=False, mode=mode))
+    assert lazy.__dict__.get("_scales") is None and float(lazy.unit.cpu()) == float(ref.unit.cpu())
+    _, lazy2 = ops.rmsnorm_quantize(x, gamma, 1e-6, mode, want_normed=False, deferred=True)
+    assert torch.equal(lazy2.scales, ref.scales) and float(lazy2.unit.cpu()) == float(ref.unit.cpu())
+
+
 def test_fused_rmsnorm_quant_config2_full_size():
     """bf16 [16384, 4096], gamma = 1 + N(0, 0.1^2), eps = 1e-6 (P32)."""
     from metis_hip import ops
