@@ -44,6 +44,9 @@ def main(reps: int = 5):
         y.copy_(x)                                                      # calibration: 64 MiB read, 64 MiB written
         px = ops.quantize(x)
         ops.rmsnorm_quantize(h, gamma, 1e-6)
+        # deferred scale bytes: the quantizers' first launch alone, the expansion forms unit and bytes (expand_xt_kernel<0, 0, 1, 0>)
+        ops.expand_tiled(ops.quantize(x, deferred=True), cache=False)
+        ops.rmsnorm_quantize(h, gamma, 1e-6, deferred=True)
         ops.linear_fwd(px, pw, t=t, u=u)                                # expand_xt_kernel + gemm_xt_kernel
         ops.linear_fwd(px, pw, t=t, u=u, tiled=False, split_k=False)    # gemm_nvfp4_large_kernel (expansion inside the K loop)
         _, t_ = ops.lowrank_project(x, v, s)                            # lowrank_nt_kernel: x V^T and (x V^T) * s
@@ -67,7 +70,13 @@ def extra(reps: int = 5):
     v_up = (torch.randn(128, 3584, generator=g) / 60).bfloat16().cuda()   # the stacked V of gate and up, r = 64 each
     s_up = torch.rand(128, generator=g).bfloat16().cuda()
     u_up = (torch.randn(18944, 64, generator=g) * 0.1).bfloat16().cuda()
+    # bf16 arithmetic at decode size: operands packed in that arithmetic, the reference's roundings in the GEMM
+    w_up16 = ops.quantize((torch.randn(18944, 3584, generator=g) * 0.02).bfloat16().cuda(), 1)
+    p_dec16 = ops.quantize(dec[:, :3584].contiguous(), 1)
+    me16 = torch.full((3584,), 0.01, dtype=torch.bfloat16, device="cuda")
     for i in range(reps):
+        ops.linear_fwd_grouped(p_dec16, [(w_up16, None, None, None), (w_up16, None, None, None)], reference_rounding=True)
+        ops.linear_fwd_grouped(p_dec16, [(w_up16, None, None, None), (w_up16, None, None, None)], reference_rounding=True, center=me16)
         ops.quantize(x, 1)                                              # bf16 arithmetic, round to nearest
         ops.quantize(x, 0, col=True)                                    # column-blocked
         ops.quantize(x, 0, sr=True, seed=i)                             # stochastic rounding, own stream
