@@ -216,7 +216,7 @@ def main():
     def qdstep(ev):
         if ev is not None:
             ev[0].record()
-        rc = L.metis_nvfp4_quant_row_deferred(x1.data_ptr(), 8192, 4096, 0, qc.data_ptr(), qdef.data_ptr(), qdef.numel(), st)
+        rc = L.metis_nvfp4_quant_row_deferred(x1.data_ptr(), 8192, 4096, 0, None, qc.data_ptr(), qdef.data_ptr(), qdef.numel(), st)
         if ev is not None:
             ev[1].record()
         assert rc == 0

@@ -153,10 +153,10 @@ int metis_nvfp4_expand_tiled_rht(const void* codes, const void* scales, const fl
 
 size_t metis_nvfp4_deferred_bytes(int64_t rows, int64_t cols) { return deferred_bytes(rows, cols); }
 
-int metis_nvfp4_quant_row_deferred(const void* x, int64_t rows, int64_t cols, int mode, void* codes, void* deferred, size_t deferred_bytes,
-                                   void* stream)
+int metis_nvfp4_quant_row_deferred(const void* x, int64_t rows, int64_t cols, int mode, const void* center, void* codes, void* deferred,
+                                   size_t deferred_bytes, void* stream)
 {
-    return quantize_row_deferred(x, rows, cols, mode, codes, deferred, deferred_bytes, (hipStream_t)stream);
+    return quantize_row_deferred(x, rows, cols, mode, center, codes, deferred, deferred_bytes, (hipStream_t)stream);
 }
 
 int metis_rmsnorm_nvfp4_quant_deferred(const void* x, const void* gamma, float eps, int64_t rows, int64_t cols, int mode, void* normed,
@@ -172,9 +172,9 @@ int metis_nvfp4_deferred_scales(const void* deferred, int64_t rows, int64_t cols
 }
 
 int metis_nvfp4_expand_tiled_deferred(const void* codes, const void* deferred, int64_t rows, int64_t cols, int quant_mode, int mode,
-                                      float* unit, void* out, void* stream)
+                                      const void* center, float* unit, void* out, void* stream)
 {
-    return expand_xt_deferred(codes, deferred, rows, cols, quant_mode, mode, unit, out, (hipStream_t)stream);
+    return expand_xt_deferred(codes, deferred, rows, cols, quant_mode, mode, center, unit, out, (hipStream_t)stream);
 }
 
 int metis_nvfp4_expand_tiled_centered(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols,
@@ -322,6 +322,12 @@ int metis_nvfp4_decode_operand(const void* codes, const void* scales, const floa
                                const void* center, void* out, void* stream)
 {
     return skinny_operand(codes, scales, unit, rows, cols, mode, center, out, (hipStream_t)stream);
+}
+
+int metis_nvfp4_decode_operand_deferred(const void* codes, const void* deferred, int64_t rows, int64_t cols, int quant_mode, int mode,
+                                        const void* center, float* unit, void* out, void* stream)
+{
+    return skinny_operand_deferred(codes, deferred, rows, cols, quant_mode, mode, center, unit, out, (hipStream_t)stream);
 }
 
 int metis_linear_fwd_grouped_operand(const void* a_operand, const float* a_unit, int64_t M, int64_t K,

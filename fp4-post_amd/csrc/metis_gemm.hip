@@ -14,6 +14,7 @@
 // e4m3(b) * 2^-8 for normal and subnormal bytes alike; the 2^16 is folded into the unit product.
 // The low-rank operands stay bf16 and use v_mfma_f32_32x32x16_bf16 on the same accumulators.
 #include "gemm_common.h"
+#include "nvfp4_encode.h"
 #include <stdlib.h>
 #include <type_traits>
 
@@ -882,15 +883,26 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nvfp4_skinny_grouped_kernel(
 // 32 tile + lane % 32, rows past M zero.  Exact mode: e2m1 * e4m3 * 2^-8 in binary16 (the tensor unit stays outside).
 // PB16: the reference's bf16 value bf16(bf16(e4m3 * unit) * e2m1), and with a centre (mean mode, one bf16 value per
 // column) its me + QDQ(x - me) rounded to bf16 once more (src/Metis/Metis/bitlinear.py:330-333 in bf16 arithmetic).
-template <int PB16>
+// DEF: the quantizer call deferred its scale bytes (nvfp4_quant.hip): `scales` holds bf16 block maxima, `partials` the
+// partial tensor maxima; unit (written to unit_out) and E4M3 bytes are formed here, in the arithmetic of that call (QMODE).
+template <int PB16, int DEF = 0, int QMODE = 0>
 __global__ __launch_bounds__(256) void skinny_operand_kernel(const uint32_t* __restrict__ codes, const uint8_t* __restrict__ scales,
                                                              const float* __restrict__ unit_p, const uint16_t* __restrict__ center,
-                                                             int M, int K, int tiles, uint4* __restrict__ out)
+                                                             int M, int K, int tiles, uint4* __restrict__ out,
+                                                             const uint32_t* __restrict__ partials = nullptr,
+                                                             float* __restrict__ unit_out = nullptr)
 {
     typedef float float2_t __attribute__((ext_vector_type(2)));
     const int iters = K / 256;
     const int64_t total = (int64_t)tiles * iters * 1024;
-    const float unit = PB16 ? *unit_p : 0.0f;
+    float unit = 0.0f;
+    if constexpr (DEF != 0) {
+        unit = tensor_unit_of<QMODE>(fold_partial_maxima(partials));
+        if (blockIdx.x == 0 && threadIdx.x == 0) *unit_out = unit;
+    } else if constexpr (PB16 != 0) {
+        unit = *unit_p;
+    }
+    const uint16_t* __restrict__ maxima = reinterpret_cast<const uint16_t*>(scales);
     for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
         const int lane = (int)(idx & 63), m = (int)((idx >> 6) & 15);
         const int64_t ti = idx >> 10;
@@ -899,7 +911,9 @@ __global__ __launch_bounds__(256) void skinny_operand_kernel(const uint32_t* __r
         uint4 v = make_uint4(0u, 0u, 0u, 0u);
         if (row < M) {
             const uint32_t c = codes[(int64_t)row * (K / 8) + (k0 >> 3)];
-            const uint32_t sb = scales[(int64_t)row * (K / 16) + (k0 >> 4)];
+            uint32_t sb;
+            if constexpr (DEF != 0) sb = scale_byte_of<QMODE>(maxima[(int64_t)row * (K / 16) + (k0 >> 4)], unit);
+            else sb = scales[(int64_t)row * (K / 16) + (k0 >> 4)];
             if constexpr (PB16 != 0) {
                 const float dq = rb(e4m3_value(sb) * unit);
                 const float2_t p[4] = {__builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c, 1.0f, 0), __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c, 1.0f, 1),
@@ -945,6 +959,28 @@ int skinny_operand(const void* codes, const void* scales, const float* unit, int
     else
         hipLaunchKernelGGL(skinny_operand_kernel<0>, dim3(g), dim3(256), 0, st, (const uint32_t*)codes, (const uint8_t*)scales, unit,
                            (const uint16_t*)center, (int)M, (int)K, tiles, (uint4*)out);
+    return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
+}
+
+int skinny_operand_deferred(const void* codes, const void* deferred, int64_t M, int64_t K, int qmode, int mode, const void* center,
+                            float* unit_out, void* out, hipStream_t st)
+{
+    if (mode == METIS_MODE_P32_F32) mode = METIS_MODE_P32;
+    if ((mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) || (qmode != METIS_MODE_P32 && qmode != METIS_MODE_PB16)) return METIS_E_ARG;
+    if (M <= 0 || M >= 256 || K <= 0 || K % 256 || K > INT32_MAX) return METIS_E_SHAPE;
+    if (!codes || !unit_out || !out || ((uintptr_t)codes % 4) || ((uintptr_t)out % 16) || ((uintptr_t)center % 16)) return METIS_E_ARG;
+    if (center && mode != METIS_MODE_PB16) return METIS_E_ARG;
+    Workspace ws;
+    if (const int rc = carve_deferred(const_cast<void*>(deferred), deferred_bytes(M, K), M, K, &ws)) return rc;
+    const int tiles = (int)((M + 63) / 64) * 2;
+    const int64_t total = (int64_t)tiles * (K / 256) * 1024;
+    const int g = (int)((total + 255) / 256);
+#define METIS_SOD(P, Q) hipLaunchKernelGGL((skinny_operand_kernel<P, 1, Q>), dim3(g), dim3(256), 0, st, (const uint32_t*)codes, \
+                                           (const uint8_t*)ws.amax, nullptr, (const uint16_t*)center, (int)M, (int)K, tiles, (uint4*)out, \
+                                           (const uint32_t*)ws.gmax, unit_out)
+    if (mode == METIS_MODE_PB16) { if (qmode) METIS_SOD(1, 1); else METIS_SOD(1, 0); }
+    else { if (qmode) METIS_SOD(0, 1); else METIS_SOD(0, 0); }
+#undef METIS_SOD
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 

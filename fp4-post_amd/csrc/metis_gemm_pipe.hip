@@ -297,10 +297,11 @@ int expand_xt(const void* codes, const void* scales, const float* unit, int64_t 
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 
-int expand_xt_deferred(const void* codes, const void* deferred, int64_t rows, int64_t cols, int qmode, int mode, float* unit_out,
-                       void* out, hipStream_t st)
+int expand_xt_deferred(const void* codes, const void* deferred, int64_t rows, int64_t cols, int qmode, int mode, const void* center,
+                       float* unit_out, void* out, hipStream_t st)
 {
     if (rows < 0 || cols < 0) return METIS_E_ARG;
+    if (center && (mode != METIS_MODE_PB16 || ((uintptr_t)center % 16))) return METIS_E_ARG;   // a centre belongs to bf16 arithmetic
     if (mode == METIS_MODE_P32_F32) mode = METIS_MODE_P32;
     if ((mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) || (qmode != METIS_MODE_P32 && qmode != METIS_MODE_PB16)) return METIS_E_ARG;
     if (cols % kBlock) return METIS_E_SHAPE;
@@ -315,8 +316,8 @@ int expand_xt_deferred(const void* codes, const void* deferred, int64_t rows, in
     const int64_t cap = (int64_t)device_cus() * 16;
     if (g > cap) g = cap;
 #define METIS_EXD(P, Q) hipLaunchKernelGGL((expand_xt_kernel<P, 0, 1, Q>), dim3((unsigned)g), dim3(256), 0, st, (const uint32_t*)codes, \
-                                           (const uint8_t*)ws.amax, nullptr, (uint4*)out, (int)rows, (int)cols, row_tiles, 0u, nullptr, \
-                                           (const uint32_t*)ws.gmax, unit_out)
+                                           (const uint8_t*)ws.amax, nullptr, (uint4*)out, (int)rows, (int)cols, row_tiles, 0u, \
+                                           (const uint16_t*)center, (const uint32_t*)ws.gmax, unit_out)
     if (mode == METIS_MODE_PB16) { if (qmode) METIS_EXD(1, 1); else METIS_EXD(1, 0); }
     else { if (qmode) METIS_EXD(0, 1); else METIS_EXD(0, 0); }
 #undef METIS_EXD

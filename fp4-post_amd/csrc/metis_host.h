@@ -51,7 +51,8 @@ int quantize(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, bo
 size_t deferred_bytes(int64_t rows, int64_t cols);
 int carve_deferred(void* p, size_t bytes, int64_t rows, int64_t cols, Workspace* ws);
 int deferred_grid(uint32_t work_items);
-int quantize_row_deferred(const void* x, int64_t rows, int64_t cols, int mode, void* codes, void* deferred, size_t bytes, hipStream_t st);
+int quantize_row_deferred(const void* x, int64_t rows, int64_t cols, int mode, const void* center, void* codes, void* deferred,
+                          size_t bytes, hipStream_t st);
 int deferred_scales(const void* deferred, int64_t rows, int64_t cols, int mode, void* scales, float* unit, hipStream_t st);
 // the row quantizer on the library's own static scratch (no workspace argument); nvfp4_quant.hip
 int quantize_row_static(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, void* codes, void* scales,
@@ -98,6 +99,9 @@ int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a
 size_t skinny_operand_bytes(int64_t M, int64_t K);
 int skinny_operand(const void* codes, const void* scales, const float* unit, int64_t M, int64_t K, int mode, const void* center,
                    void* out, hipStream_t st);
+// the same from a tensor whose quantizer call deferred its scale bytes; writes the unit
+int skinny_operand_deferred(const void* codes, const void* deferred, int64_t M, int64_t K, int qmode, int mode, const void* center,
+                            float* unit_out, void* out, hipStream_t st);
 int gemm_grouped_center_supported(int64_t M, int64_t K, const GemmMember* members, int count, int have_workspace);
 // bytes of split-K scratch a grouped call can use (only the N fields of the members are read; 0: it would not split)
 size_t gemm_grouped_workspace_bytes(int64_t M, int64_t K, const GemmMember* members, int count);
@@ -138,8 +142,8 @@ size_t expand_xt_bytes(int64_t rows, int64_t cols);
 int expand_xt(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, int mode, void* out,
               hipStream_t st, int rht = 0, uint32_t sign_mask = 0, const void* center = nullptr);
 // the same from a tensor whose quantizer call deferred its scale bytes (qmode: the arithmetic it was quantized in); writes the unit
-int expand_xt_deferred(const void* codes, const void* deferred, int64_t rows, int64_t cols, int qmode, int mode, float* unit_out,
-                       void* out, hipStream_t st);
+int expand_xt_deferred(const void* codes, const void* deferred, int64_t rows, int64_t cols, int qmode, int mode, const void* center,
+                       float* unit_out, void* out, hipStream_t st);
 // a dense bf16 / binary32 tensor in the tiled layout (optional per-column bf16 scale first)
 int dense_xt(const void* x, int64_t rows, int64_t cols, int64_t ld, int dtype, const void* col_scale, int mode, void* out, hipStream_t st);
 // the tiled operand [cols, rows] (contraction over the packed tensor's rows); rows % 32 == 0

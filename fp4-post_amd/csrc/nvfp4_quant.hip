@@ -71,7 +71,8 @@ template <int MODE, bool SR, bool WIDE = false, bool HAD = false>
 __global__ __launch_bounds__(256) void quant_codes_kernel(
     const void* __restrict__ xv, uint32_t rows, uint32_t cols, int64_t ld, const void* __restrict__ noise,
     uint64_t seed, uint64_t offset, uint2* __restrict__ codes, void* __restrict__ ws_amax_v,
-    uint32_t* __restrict__ ws_gmax, uint32_t nblocks, int in_f32, const void* __restrict__ center, uint32_t sign_mask)
+    uint32_t* __restrict__ ws_gmax, uint32_t nblocks, int in_f32, const void* __restrict__ center, uint32_t sign_mask,
+    uint32_t fill_to)
 {
     static_assert(!WIDE || MODE == 0, "binary32 values imply binary32 arithmetic");
     static_assert(!HAD || WIDE || MODE == 1, "rotated binary32 values are not bf16 values");
@@ -137,7 +138,7 @@ __global__ __launch_bounds__(256) void quant_codes_kernel(
                                       : encode_block<MODE, SR>(v, block_scalar<MODE>(am), u);
         }
     }
-    publish_group_max(gmax, ws_gmax);
+    publish_group_max(gmax, ws_gmax, fill_to);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -675,7 +676,7 @@ static int launch_quant(const void* x, int64_t rows, int64_t cols, int64_t ld, c
         }
         hipLaunchKernelGGL((quant_codes_kernel<MODE, SR, WIDE, HAD>), dim3(g1), dim3(256), 0, st, x, (uint32_t)rows,
                            (uint32_t)cols, ld, noise, seed, offset, (uint2*)codes, (void*)ws.amax, ws.gmax, nblocks, in_f32, center,
-                           sign_mask);
+                           sign_mask, 0u);
         return launch_scales(WIDE ? METIS_MODE_P32_F32 : MODE, ws, (uint32_t)g1, scales, unit, nblocks, st);
     }
 }
@@ -751,10 +752,14 @@ int deferred_grid(uint32_t work_items)
     return g > (int)kDeferredPartials ? (int)kDeferredPartials : g;
 }
 
-int quantize_row_deferred(const void* x, int64_t rows, int64_t cols, int mode, void* codes, void* deferred, size_t bytes, hipStream_t st)
+// center (bf16 arithmetic only: a binary32 centre leaves residuals whose maxima are not bf16 values): one bf16 value per
+// column subtracted first, as quantize() does for the mean mode.
+int quantize_row_deferred(const void* x, int64_t rows, int64_t cols, int mode, const void* center, void* codes, void* deferred,
+                          size_t bytes, hipStream_t st)
 {
     if (rows < 0 || cols < 0) return METIS_E_ARG;
     if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) return METIS_E_ARG;
+    if (center && (mode != METIS_MODE_PB16 || ((uintptr_t)center % 16))) return METIS_E_ARG;
     if (cols % kBlock) return METIS_E_SHAPE;
     if (rows == 0 || cols == 0) return METIS_OK;
     if (!x || !codes || ((uintptr_t)x % 16) || ((uintptr_t)codes % 8)) return METIS_E_ARG;
@@ -763,7 +768,11 @@ int quantize_row_deferred(const void* x, int64_t rows, int64_t cols, int mode, v
     if (const int rc = carve_deferred(deferred, bytes, rows, cols, &ws)) return rc;
     const uint32_t nblocks = (uint32_t)(rows * cols / kBlock);
     const int g1 = deferred_grid(nblocks);
-    if (mode == 0)
+    if (center)
+        hipLaunchKernelGGL((quant_codes_kernel<1, false, false, false>), dim3(g1), dim3(256), 0, st, x, (uint32_t)rows, (uint32_t)cols,
+                           cols, nullptr, (uint64_t)0, (uint64_t)0, (uint2*)codes, (void*)ws.amax, ws.gmax, nblocks, 0, center, 0u,
+                           kDeferredPartials);
+    else if (mode == 0)
         hipLaunchKernelGGL((quant_codes_contig_kernel<0>), dim3(g1), dim3(256), 0, st, (const uint4*)x, (uint2*)codes, ws.amax, ws.gmax,
                            nblocks, kDeferredPartials);
     else

@@ -53,10 +53,10 @@ SIGNATURES = {
     "metis_nvfp4_quant_row_rht": (_i32, [_vp, _i64, _i64, _i64, _i32, ctypes.c_uint32, _i32, _u64, _u64, _vp, _vp, _vp, _vp, _sz, _vp]),
     "metis_nvfp4_expand_tiled_rht": (_i32, [_vp, _vp, _vp, _i64, _i64, _i32, ctypes.c_uint32, _i32, _i32, _vp, _vp]),
     "metis_nvfp4_deferred_bytes": (_sz, [_i64, _i64]),
-    "metis_nvfp4_quant_row_deferred": (_i32, [_vp, _i64, _i64, _i32, _vp, _vp, _sz, _vp]),
+    "metis_nvfp4_quant_row_deferred": (_i32, [_vp, _i64, _i64, _i32, _vp, _vp, _vp, _sz, _vp]),
     "metis_rmsnorm_nvfp4_quant_deferred": (_i32, [_vp, _vp, _f32, _i64, _i64, _i32, _vp, _vp, _vp, _sz, _vp]),
     "metis_nvfp4_deferred_scales": (_i32, [_vp, _i64, _i64, _i32, _vp, _vp, _vp]),
-    "metis_nvfp4_expand_tiled_deferred": (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _vp, _vp, _vp]),
+    "metis_nvfp4_expand_tiled_deferred": (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _vp, _vp, _vp, _vp]),
     "metis_nvfp4_expand_tiled_centered": (_i32, [_vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp]),
     "metis_linear_fwd_tiled": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _i32, _vp, _i32, _i32, _vp, _sz, _vp]),
     "metis_linear_dgrad": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i32, _vp]),
@@ -79,6 +79,7 @@ SIGNATURES = {
     "metis_linear_fwd_grouped_bf16": (_i32, [_vp, _vp, _vp, _i64, _i64, _vp, _i32, _i32, _vp, _sz, _vp]),
     "metis_nvfp4_decode_operand_bytes": (_sz, [_i64, _i64]),
     "metis_nvfp4_decode_operand": (_i32, [_vp, _vp, _vp, _i64, _i64, _i32, _vp, _vp, _vp]),
+    "metis_nvfp4_decode_operand_deferred": (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _vp, _vp, _vp, _vp]),
     "metis_linear_fwd_grouped_operand": (_i32, [_vp, _vp, _i64, _i64, _vp, _i32, _i32, _i32, _vp, _sz, _vp]),
     "metis_linear_grouped_workspace_bytes": (_sz, [_i64, _i64, _vp, _i32]),
     "metis_linear_fwd_grouped_centered": (_i32, [_vp, _vp, _vp, _i64, _i64, _vp, _i32, _i32, _vp, _vp, _sz, _vp]),

@@ -324,13 +324,14 @@ class LinearLowbitFunction(torch.autograd.Function):
                 # the kernels read bf16 values and take the arithmetic as a mode: no upcast copy of a bf16 tensor
                 # from 256 rows on the consumer is the tiled expansion, which forms the scale bytes itself
                 x2 = _flat2d(input_)
-                more = {"deferred": True} if x2.shape[0] >= 256 else {}
+                more = {"deferred": True} if (x2.shape[0] >= 256 or F._bf16_rounding()) else {}
                 return F.q_forward_input.pack(x2, arith=F.compute_dtype, **more)
             if F._mean_mode_packable():
                 # mean + QDQ(x - mean) (reference 311-336) without materialising either: the subtraction happens
                 # inside the quantizer and the mean's contribution to a matmul is a rank-one term
                 me, me32 = F._token_mean2(input_, mean_cache=mean_cache, cache_key=cache_key)
-                return CenteredNVFP4(F.q_forward_input.pack(_flat2d(input_), arith=F.compute_dtype, center=me), me, me32)
+                more = {"deferred": True} if (F._bf16_rounding() and me.dtype == torch.bfloat16) else {}
+                return CenteredNVFP4(F.q_forward_input.pack(_flat2d(input_), arith=F.compute_dtype, center=me, **more), me, me32)
         return F.quantize_input(input_, mean_cache=mean_cache, cache_key=cache_key)
 
     @staticmethod
@@ -454,6 +455,13 @@ class LinearLowbitFunction(torch.autograd.Function):
         if F.enable_nv_recipe:
             value = F._apply_hadamard_blocks(value, inverse=True)
         return value
+
+    @staticmethod
+    def _bf16_rounding() -> bool:
+        """bf16 arithmetic with the reference's roundings: every consumer of a packed activation (tiled expansion, ready
+        decode operands) forms the scale bytes itself, so the quantizer may always defer them."""
+        F = LinearLowbitFunction
+        return F.reference_rounding and F.compute_dtype != torch.float32
 
     @staticmethod
     def _mean_in_operand(px, pw) -> bool:

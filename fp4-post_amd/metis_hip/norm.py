@@ -82,9 +82,10 @@ class FusedRMSNormQuant(nn.Module):
             return self._plain(x)
         mode = MODE_P32 if F.compute_dtype == torch.float32 else MODE_PB16
         with torch.no_grad():
-            # from 256 rows on the consumer is the tiled expansion, which forms the scale bytes itself
+            # the tiled expansion (256 rows or more) and the ready decode operands of bf16 arithmetic form the scale bytes
+            # themselves
             normed, packed = ops.rmsnorm_quantize(x, self.weight, self.variance_epsilon, mode,
-                                                  deferred=x.numel() // cols >= 256)
+                                                  deferred=x.numel() // cols >= 256 or F._bf16_rounding())
         normed = normed.reshape(x.shape)
         out = _NormedWithGrad.apply(x, self.weight, normed, self.variance_epsilon) if torch.is_grad_enabled() and (
             x.requires_grad or self.weight.requires_grad) else normed

@@ -171,11 +171,16 @@ def quantize(x: torch.Tensor, mode: int = MODE_P32, *, col: bool = False, sr: bo
     codes = torch.empty(prow, pcol // 2, dtype=torch.uint8, device=dev)
     unit = torch.empty(1, dtype=torch.float32, device=dev)
     L = load()
-    if (deferred and not col and not sr and center is None and kmode in (MODE_P32, MODE_PB16) and x2.stride(0) == cols
-            and rows * cols > 0):
+    if (deferred and not col and not sr and (center is None or kmode == MODE_PB16) and kmode in (MODE_P32, MODE_PB16)
+            and x2.stride(0) == cols and rows * cols > 0):
+        cen = None
+        if center is not None:
+            cen = center.reshape(-1).to(device=dev, dtype=torch.bfloat16).contiguous()
+            if cen.numel() != cols:
+                raise ValueError(f"center must have one value per column ({cols}), got {cen.numel()}")
         parked = torch.empty(L.metis_nvfp4_deferred_bytes(rows, cols), dtype=torch.uint8, device=dev)
-        rc = L.metis_nvfp4_quant_row_deferred(x2.data_ptr(), rows, cols, kmode, codes.data_ptr(), parked.data_ptr(), parked.numel(),
-                                              _stream())
+        rc = L.metis_nvfp4_quant_row_deferred(x2.data_ptr(), rows, cols, kmode, None if cen is None else cen.data_ptr(),
+                                              codes.data_ptr(), parked.data_ptr(), parked.numel(), _stream())
         check(rc, "metis_nvfp4_quant_row_deferred", x.shape)
         return PackedNVFP4(codes, None, unit, prow, pcol, mode, deferred=parked)
     scales = torch.empty(prow, pcol // BLOCK, dtype=torch.uint8, device=dev)
@@ -396,6 +401,8 @@ def expand_tiled(p: PackedNVFP4, cache: bool = True, mode: int = MODE_P32, cente
     center (bf16 [cols], mode PB16): p packs a centred residual; the operand is the mean mode's center + QDQ(x - center)
     rounded to bf16, the tensor the reference multiplies with in bf16 arithmetic (never cached)."""
     L = load()
+    d = p.__dict__
+    lazy = d.get("deferred") is not None and d.get("_scales") is None and p.rht is None and p.cols % 32 == 0
     if center is not None:
         if mode != MODE_PB16 or p.rht is not None:
             raise ValueError("a centre goes into the bf16-arithmetic operand of an unrotated tensor")
@@ -403,19 +410,23 @@ def expand_tiled(p: PackedNVFP4, cache: bool = True, mode: int = MODE_P32, cente
         if center.numel() != p.cols:
             raise ValueError(f"center must have {p.cols} values, got {center.numel()}")
         out = torch.empty(L.metis_nvfp4_expand_tiled_bytes(p.rows, p.cols), dtype=torch.uint8, device=p.codes.device)
-        rc = L.metis_nvfp4_expand_tiled_centered(p.codes.data_ptr(), p.scales.data_ptr(), p.unit.data_ptr(), p.rows, p.cols,
-                                                 center.data_ptr(), out.data_ptr(), _stream())
+        if lazy:
+            rc = L.metis_nvfp4_expand_tiled_deferred(p.codes.data_ptr(), d["deferred"].data_ptr(), p.rows, p.cols, p.mode, mode,
+                                                     center.data_ptr(), d["_unit"].data_ptr(), out.data_ptr(), _stream())
+            d["_unit_ready"] = True
+        else:
+            rc = L.metis_nvfp4_expand_tiled_centered(p.codes.data_ptr(), p.scales.data_ptr(), p.unit.data_ptr(), p.rows, p.cols,
+                                                     center.data_ptr(), out.data_ptr(), _stream())
         check(rc, "metis_nvfp4_expand_tiled_centered", (p.rows, p.cols))
         return out
     have = p.tiled_pb16 if mode == MODE_PB16 else p.tiled
     if have is not None:
         return have
     out = torch.empty(L.metis_nvfp4_expand_tiled_bytes(p.rows, p.cols), dtype=torch.uint8, device=p.codes.device)
-    d = p.__dict__
-    if d.get("deferred") is not None and d.get("_scales") is None and p.rht is None and p.cols % 32 == 0:
+    if lazy:
         # the scale bytes were never written: this kernel forms them from the parked block maxima, and writes the unit
         rc = L.metis_nvfp4_expand_tiled_deferred(p.codes.data_ptr(), d["deferred"].data_ptr(), p.rows, p.cols, p.mode, mode,
-                                                 d["_unit"].data_ptr(), out.data_ptr(), _stream())
+                                                 None, d["_unit"].data_ptr(), out.data_ptr(), _stream())
         check(rc, "metis_nvfp4_expand_tiled_deferred", (p.rows, p.cols))
         d["_unit_ready"] = True
     elif p.rht is not None:                   # NV recipe: the operand holds the values rotated back
@@ -462,6 +473,15 @@ def decode_operand(p: PackedNVFP4, mode: int = MODE_P32, center: torch.Tensor | 
         center = center.reshape(-1).to(torch.bfloat16).contiguous()
         if center.numel() != p.cols:
             raise ValueError(f"center must have {p.cols} values, got {center.numel()}")
+    d = p.__dict__
+    if d.get("deferred") is not None and d.get("_scales") is None:
+        # the scale bytes were never written: this kernel forms them from the parked block maxima, and writes the unit
+        rc = L.metis_nvfp4_decode_operand_deferred(p.codes.data_ptr(), d["deferred"].data_ptr(), p.rows, p.cols, p.mode, mode,
+                                                   None if center is None else center.data_ptr(), d["_unit"].data_ptr(),
+                                                   out.data_ptr(), _stream())
+        check(rc, "metis_nvfp4_decode_operand_deferred", (p.rows, p.cols))
+        d["_unit_ready"] = True
+        return out
     rc = L.metis_nvfp4_decode_operand(p.codes.data_ptr(), p.scales.data_ptr(), p.unit.data_ptr(), p.rows, p.cols, mode,
                                       None if center is None else center.data_ptr(), out.data_ptr(), _stream())
     check(rc, "metis_nvfp4_decode_operand", (p.rows, p.cols))

@@ -311,23 +311,28 @@ int metis_nvfp4_expand_tiled_rht(const void *codes, const void *scales, const fl
  * codes): 2048 partial tensor maxima, then one bf16 block maximum per block.  Round-to-nearest rows of a contiguous
  * bf16 tensor (ld == cols), mode METIS_MODE_P32 or METIS_MODE_PB16.
  *   metis_nvfp4_deferred_bytes           size of that buffer; 256-byte aligned, contents need no initialisation
- *   metis_nvfp4_quant_row_deferred       metis_nvfp4_quant_row without scales and unit
+ *   metis_nvfp4_quant_row_deferred       metis_nvfp4_quant_row without scales and unit; center: NULL, or in mode
+ *                                        METIS_MODE_PB16 one bf16 value per column subtracted first (16-byte aligned), as
+ *                                        metis_nvfp4_quant_centered does for the mean mode
  *   metis_rmsnorm_nvfp4_quant_deferred   metis_rmsnorm_nvfp4_quant likewise
  *   metis_nvfp4_expand_tiled_deferred    metis_nvfp4_expand_tiled reading the parked data: quant_mode = the mode of the
- *                                        quantizer call, mode = the operand format; also writes the tensor unit (float
- *                                        [1], required), which metis_linear_fwd_tiled reads afterwards.  Same bits as
+ *                                        quantizer call, mode = the operand format; center: NULL, or (mode
+ *                                        METIS_MODE_PB16) the bf16 centre as in metis_nvfp4_expand_tiled_centered; also
+ *                                        writes the tensor unit (float [1], required), which metis_linear_fwd_tiled
+ *                                        reads afterwards.  Same bits as
  *                                        the two-launch quantizer followed by metis_nvfp4_expand_tiled
  *   metis_nvfp4_deferred_scales          the second launch after all: scales and unit exactly as metis_nvfp4_quant_row
  *                                        would have written them, for consumers that read E4M3 bytes
  */
 size_t metis_nvfp4_deferred_bytes(int64_t rows, int64_t cols);
-int metis_nvfp4_quant_row_deferred(const void *x, int64_t rows, int64_t cols, int mode, void *codes,
-                                   void *deferred, size_t deferred_bytes, void *stream);
+int metis_nvfp4_quant_row_deferred(const void *x, int64_t rows, int64_t cols, int mode, const void *center,
+                                   void *codes, void *deferred, size_t deferred_bytes, void *stream);
 int metis_rmsnorm_nvfp4_quant_deferred(const void *x, const void *gamma, float eps, int64_t rows, int64_t cols,
                                        int mode, void *normed, void *codes, void *deferred,
                                        size_t deferred_bytes, void *stream);
 int metis_nvfp4_expand_tiled_deferred(const void *codes, const void *deferred, int64_t rows, int64_t cols,
-                                      int quant_mode, int mode, float *unit, void *out, void *stream);
+                                      int quant_mode, int mode, const void *center, float *unit, void *out,
+                                      void *stream);
 int metis_nvfp4_deferred_scales(const void *deferred, int64_t rows, int64_t cols, int mode, void *scales,
                                 float *unit, void *stream);
 
@@ -486,10 +491,17 @@ int metis_linear_fwd_grouped_bf16(const void *a_codes, const void *a_scales, con
  *                                metis_linear_fwd_grouped_bf16 (mode METIS_MODE_PB16, same bits when no centre went
  *                                into the operand) reading that buffer; a_unit as for the packed activation (unused in
  *                                mode PB16 but required); weight scale pointers 8-byte aligned; METIS_E_ARG for
- *                                shapes the decode-sized kernel does not take */
+ *                                shapes the decode-sized kernel does not take
+ *   metis_nvfp4_decode_operand_deferred  the same from a tensor whose quantizer call deferred its scale bytes
+ *                                (metis_nvfp4_quant_row_deferred: quant_mode = its mode): forms the E4M3 bytes itself and
+ *                                writes the tensor unit (float [1], required), so a decode-sized activation costs two
+ *                                launches ahead of its GEMMs instead of three */
 size_t metis_nvfp4_decode_operand_bytes(int64_t rows, int64_t cols);
 int metis_nvfp4_decode_operand(const void *codes, const void *scales, const float *unit, int64_t rows,
                                int64_t cols, int mode, const void *center, void *out, void *stream);
+int metis_nvfp4_decode_operand_deferred(const void *codes, const void *deferred, int64_t rows, int64_t cols,
+                                        int quant_mode, int mode, const void *center, float *unit, void *out,
+                                        void *stream);
 int metis_linear_fwd_grouped_operand(const void *a_operand, const float *a_unit, int64_t M, int64_t K,
                                      const metis_linear_member *members, int count, int out_dtype, int mode,
                                      void *workspace, size_t workspace_bytes, void *stream);

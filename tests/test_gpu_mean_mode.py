@@ -458,7 +458,18 @@ def test_mean_mode_operands_in_bf16_arithmetic_hold_the_reference_tensor():
         pp = ops.quantize(xx, 1, center=mm)
         want = mm.unsqueeze(0) + ops.dequantize(pp, torch.bfloat16)                  # bf16 add: the reference's expression
         assert torch.equal(untile(ops.expand_tiled(pp, cache=False, mode=1, center=mm), rows, cols, torch.bfloat16), want)
+        # the same operands from a quantizer call that deferred its scale bytes (the consumers form them)
+        lazy = ops.quantize(xx, 1, center=mm, deferred=True)
+        assert lazy.deferred is not None and torch.equal(lazy.codes, pp.codes)
+        assert torch.equal(untile(ops.expand_tiled(lazy, cache=False, mode=1, center=mm), rows, cols, torch.bfloat16), want)
+        assert lazy.__dict__.get("_scales") is None and float(lazy.unit.cpu()) == float(pp.unit.cpu())
         if rows < 256:
+            lazy = ops.quantize(xx, 1, center=mm, deferred=True)
+            assert torch.equal(from_decode_operand(ops.decode_operand(lazy, 1, mm), rows, cols, torch.bfloat16), want)
+            assert lazy.__dict__.get("_scales") is None and float(lazy.unit.cpu()) == float(pp.unit.cpu())
+            assert torch.equal(lazy.scales, pp.scales)
+            lazy0 = ops.quantize(xx, 0, deferred=True)
+            assert torch.equal(from_decode_operand(ops.decode_operand(lazy0, 0), rows, cols, torch.float16), ops.expand(ops.quantize(xx, 0)))
             assert torch.equal(from_decode_operand(ops.decode_operand(pp, 1, mm), rows, cols, torch.bfloat16), want)
             assert torch.equal(from_decode_operand(ops.decode_operand(pp, 1), rows, cols, torch.bfloat16), ops.dequantize(pp, torch.bfloat16))
             exact = from_decode_operand(ops.decode_operand(pp, 0), rows, cols, torch.float16)

@@ -324,11 +324,11 @@ def test_deferred_scale_bytes_give_the_same_packed_tensor(ops, tag, mode):
     scales = torch.empty(48, 4, dtype=torch.uint8, device="cuda")
     unit = torch.empty(1, dtype=torch.float32, device="cuda")
     st = torch.cuda.current_stream().cuda_stream
-    assert L.metis_nvfp4_quant_row_deferred(x.data_ptr(), 48, 64, mode, codes.data_ptr(), parked.data_ptr(), parked.numel(), st) == 0
+    assert L.metis_nvfp4_quant_row_deferred(x.data_ptr(), 48, 64, mode, None, codes.data_ptr(), parked.data_ptr(), parked.numel(), st) == 0
     assert L.metis_nvfp4_deferred_scales(parked.data_ptr(), 48, 64, mode, scales.data_ptr(), unit.data_ptr(), st) == 0
     torch.cuda.synchronize()
     assert torch.equal(codes, ref.codes) and torch.equal(scales, ref.scales) and float(unit.cpu()) == float(ref.unit.cpu())
-    assert L.metis_nvfp4_quant_row_deferred(x.data_ptr(), 48, 64, mode, codes.data_ptr(), parked.data_ptr(), 16, st) == _lib.E_WORKSPACE
+    assert L.metis_nvfp4_quant_row_deferred(x.data_ptr(), 48, 64, mode, None, codes.data_ptr(), parked.data_ptr(), 16, st) == _lib.E_WORKSPACE
 
 
 @pytest.mark.parametrize("tag,mode", MODES)
