@@ -293,6 +293,7 @@ constexpr uint32_t kDeferredPartials = 2048;
 // tensor maximum from the partial maxima: every thread of a 256-thread workgroup calls this
 __device__ __forceinline__ float fold_partial_maxima(const uint32_t* __restrict__ partials)
 {
+    static_assert(kDeferredPartials == 256 * 8, "256 threads fold eight entries each");
     __shared__ float fmax_s[4];
     const uint4 a = reinterpret_cast<const uint4*>(partials)[threadIdx.x];
     const uint4 b = reinterpret_cast<const uint4*>(partials)[threadIdx.x + 256];
