@@ -156,13 +156,16 @@ inline int allow_dynamic_lds(const void* fn, size_t bytes, bool (&done)[64])
 // Sums the nsplit partial tiles of a split 256 x 256 GEMM (8 waves of 128 x 64) and writes the output.
 // One wave per 32 x 64 piece (tile, wave of the GEMM, 32-row slab i): its lanes read what the same lanes of
 // the GEMM wrote, 1 KiB per instruction, and add the splits in ascending order.
-// PB16 (every op of the reference rounded to bf16): the partial tiles hold the residual product only; their sum is
-// rounded to bf16 as the reference's bf16 matmul rounds it, the bias is added in bf16, and the low-rank term (a
-// further partial tile in slot nsplit when has_low is set) is added before the final rounding.
+// The partial tiles hold the residual product only; the low-rank term t u^T (r > 0) is formed here, two 32 x 32 MFMA tiles
+// per wave in ascending steps of 16 columns, and added with the bias.
+// PB16 (every op of the reference rounded to bf16): the sum of the partial tiles is rounded to bf16 as the reference's
+// bf16 matmul rounds it, the bias is added in bf16, then the low-rank term and the final rounding.
 template <int OUT_F32, int PB16 = 0>
 __global__ __launch_bounds__(64) void gemm_splitk_reduce_kernel(const float* __restrict__ ws, int nsplit, int M, int N,
                                                                 int tiles_m, int tiles_n, void* __restrict__ out, int nfull,
-                                                                const uint16_t* __restrict__ bias, int bias_f32, int has_low)
+                                                                const uint16_t* __restrict__ bias, int bias_f32,
+                                                                const uint16_t* __restrict__ t = nullptr,
+                                                                const uint16_t* __restrict__ u = nullptr, int r = 0)
 {
     constexpr int TN = 2, WTN = 64, NTHREADS = 512, TILE = L_BM * L_BN;
     __shared__ __attribute__((aligned(16))) uint16_t cw[32 * 72];
@@ -191,23 +194,53 @@ __global__ __launch_bounds__(64) void gemm_splitk_reduce_kernel(const float* __r
                 v[j][g].x += p.x; v[j][g].y += p.y; v[j][g].z += p.z; v[j][g].w += p.w;
             }
     }
-    if constexpr (PB16 != 0) {
-        const float* sl = src + (size_t)nsplit * total * TILE;
+    float16_t low[TN];                                           // the low-rank term t u^T of this piece
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) low[j][e] = 0.0f;
+    {
+        if (r > 0) {                                             // lane l: row l % 32 of its operand, columns 8 (l / 32) .. of the step
+            const uint16_t* tp = t + (int64_t)min(mbase + (lane & 31), M - 1) * r + 8 * (lane >> 5);
+            const uint16_t* up[TN];
+#pragma unroll
+            for (int j = 0; j < TN; ++j) up[j] = u + (int64_t)min(nbase + j * 32 + (lane & 31), N - 1) * r + 8 * (lane >> 5);
+            for (int k0 = 0; k0 < r; k0 += 16) {
+                const bf16x8_t ga = *reinterpret_cast<const bf16x8_t*>(tp + k0);
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    low[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8_t*>(up[j] + k0), ga, low[j], 0, 0, 0);
+            }
+        }
+    }
+    if constexpr (PB16 == 0) {
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 const int n = nbase + j * 32 + 8 * g + 4 * (lane >> 5);
-                float r[4] = {rb(v[j][g].x), rb(v[j][g].y), rb(v[j][g].z), rb(v[j][g].w)};
+                float q[4] = {v[j][g].x, v[j][g].y, v[j][g].z, v[j][g].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    q[e] += low[j][4 * g + e];
+                    if (bias) q[e] += bias_value(bias, bias_f32, min(n + e, N - 1));
+                }
+                v[j][g] = make_float4(q[0], q[1], q[2], q[3]);
+            }
+    } else {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int n = nbase + j * 32 + 8 * g + 4 * (lane >> 5);
+                float q[4] = {rb(v[j][g].x), rb(v[j][g].y), rb(v[j][g].z), rb(v[j][g].w)};
                 if (bias) {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) r[e] = rb(r[e] + bias_value(bias, bias_f32, min(n + e, N - 1)));
+                    for (int e = 0; e < 4; ++e) q[e] = rb(q[e] + bias_value(bias, bias_f32, min(n + e, N - 1)));
                 }
-                if (has_low) {
-                    const float4 p = *reinterpret_cast<const float4*>(sl + (j * 4 + g) * (NTHREADS * 4));
-                    r[0] += p.x; r[1] += p.y; r[2] += p.z; r[3] += p.w;
-                }
-                v[j][g] = make_float4(rb(r[0]), rb(r[1]), rb(r[2]), rb(r[3]));
+#pragma unroll
+                for (int e = 0; e < 4; ++e) q[e] += low[j][4 * g + e];
+                v[j][g] = make_float4(rb(q[0]), rb(q[1]), rb(q[2]), rb(q[3]));
             }
     }
 

@@ -560,9 +560,9 @@ static int launch_large(const void* a_codes, const void* a_scales, const float* 
     if (split) {
         const dim3 rgrid((unsigned)(total - nfull) * 32u);
         if (f32)
-            hipLaunchKernelGGL((gemm_splitk_reduce_kernel<1, 0>), rgrid, dim3(64), 0, st, ws, nsplit, Mi, Ni, tmi, tni, out, nfull, (const uint16_t*)nullptr, 0, 0);
+            hipLaunchKernelGGL((gemm_splitk_reduce_kernel<1, 0>), rgrid, dim3(64), 0, st, ws, nsplit, Mi, Ni, tmi, tni, out, nfull, (const uint16_t*)nullptr, 0);
         else
-            hipLaunchKernelGGL((gemm_splitk_reduce_kernel<0, 0>), rgrid, dim3(64), 0, st, ws, nsplit, Mi, Ni, tmi, tni, out, nfull, (const uint16_t*)nullptr, 0, 0);
+            hipLaunchKernelGGL((gemm_splitk_reduce_kernel<0, 0>), rgrid, dim3(64), 0, st, ws, nsplit, Mi, Ni, tmi, tni, out, nfull, (const uint16_t*)nullptr, 0);
         if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
     }
     return METIS_OK;

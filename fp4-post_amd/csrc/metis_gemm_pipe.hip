@@ -366,8 +366,8 @@ int expand_xt_transposed(const void* codes, const void* scales, const float* uni
 // bfloat16, src/grpo/grpo.py:204-205).
 // SPLIT: as in gemm_nvfp4_large_kernel -- tiles nfull .. total-1 have nsplit workgroups each, every one contracting
 // its own range of stages into a binary32 partial tile in ws (accumulator-register order) for
-// gemm_splitk_reduce_kernel.  Exact mode: units applied, low-rank term and bias in split 0.  PB16: residual only;
-// split 0 leaves the low-rank term as one more partial tile in slot nsplit, the reduction kernel rounds and adds.
+// gemm_splitk_reduce_kernel, which also forms the low-rank term of the tile and adds the bias.  Exact mode: units
+// applied; PB16: the reduction kernel rounds the sum and adds the bias in bf16, as the reference's bf16 forward does.
 // ---------------------------------------------------------------------------------------------
 constexpr int XT_STAGE = 32 * 1024, XT_NS = 3;
 
@@ -522,7 +522,6 @@ __global__ __launch_bounds__(512, 1) void gemm_xt_kernel(
     }
     __syncthreads();                                            // the ring is free for the epilogue
 
-    const bool first = !(SPLIT != 0 && partial && split != 0);  // this workgroup adds the low-rank term (and, exact mode, the bias)
     float* wt = nullptr;
     if (SPLIT != 0 && partial) wt = ws + (size_t)(split * (total - nfull) + (logical - nfull)) * (L_BM * L_BN) + tid * 4;
     auto store_partial = [&](float* dst, bool with_bias) {      // accumulator-register order, 1 KiB per store instruction
@@ -545,14 +544,8 @@ __global__ __launch_bounds__(512, 1) void gemm_xt_kernel(
 
     if constexpr (PB16 != 0) {
         if (SPLIT != 0 && partial) {
-            store_partial(wt, false);                           // the residual product of this K range
-            if (!first || r == 0) return;
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+            store_partial(wt, false);                           // the residual product of this K range; the reduction kernel
+            return;                                             // rounds the sum and adds bias and low-rank term
         } else {
             // the reference's bf16 matmul result, then its bf16 bias add
 #pragma unroll
@@ -576,9 +569,9 @@ __global__ __launch_bounds__(512, 1) void gemm_xt_kernel(
             for (int j = 0; j < TN; ++j)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) acc[i][j][e] *= us;
-        if (!first) {
-            r = 0;
-            bias = nullptr;
+        if (SPLIT != 0 && partial) {
+            store_partial(wt, false);                           // this split's share; low-rank term and bias wait for the sum
+            return;
         }
     }
 
@@ -612,12 +605,6 @@ __global__ __launch_bounds__(512, 1) void gemm_xt_kernel(
         __syncthreads();
     }
 
-    if (SPLIT != 0 && partial) {
-        // exact mode: this split's share (split 0 with the low-rank term and the bias); PB16: the low-rank tile, slot nsplit
-        if constexpr (PB16 != 0) store_partial(ws + (size_t)(nsplit * (total - nfull) + (logical - nfull)) * (L_BM * L_BN) + tid * 4, false);
-        else store_partial(wt, true);
-        return;
-    }
     if constexpr (PB16 != 0 && OUT_F32 != 0) {                  // a binary32 output buffer still holds bf16 values in this mode
 #pragma unroll
         for (int i = 0; i < TM; ++i)
@@ -738,9 +725,8 @@ static int launch_xt(const void* a_xt, const float* a_unit, const void* b_xt, co
     }
     if (SPLIT) {
         const dim3 rgrid((unsigned)(total - nfull) * 32u);
-        const int has_low = r > 0;
         hipLaunchKernelGGL((gemm_splitk_reduce_kernel<OUT_F32, PB16>), rgrid, dim3(64), 0, st, (const float*)ws, nsplit, Mi, Ni, tmi, tni, out,
-                           nfull, PB16 ? bp : (const uint16_t*)nullptr, bias_f32, PB16 ? has_low : 0);
+                           nfull, bp, bias_f32, tp, up, ri);
         if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
     }
     return METIS_OK;
