@@ -673,24 +673,38 @@ class _MetisFusedFunction(torch.autograd.Function):
         else:
             y = ops.linear_fwd(px, p_res, t=t, u=u.to(cd), bias=gemm_bias, out_dtype=out_dtype,
                                reference_rounding=F.reference_rounding)
-        ctx.save_for_backward(x, v, s, u, res, xv)
+        ctx.save_for_backward(x, v, s, u, res, xv, t)               # t = bf16(xv * s): [L, r], kept for the gradient of U
         ctx.p_res = p_res
         ctx.has_bias = bias is not None
         ctx.lead = x.shape[:-1]
         return y.reshape(*ctx.lead, y.shape[-1]).to(F.compute_dtype)
 
     @staticmethod
+    def _transposed_bf16(w: torch.Tensor) -> torch.Tensor:
+        """w^T in bf16, contiguous, cached on the tensor until it is modified in place (the rank-r kernels read both
+        factors with the rank as the slow dimension)."""
+        key = (w._version, w.device, w.dtype)
+        hit = getattr(w, "_metis_transposed", None)
+        if hit is None or hit[0] != key:
+            hit = (key, w.detach().to(torch.bfloat16).T.contiguous())
+            try:
+                w._metis_transposed = hit
+            except AttributeError:                                   # a tensor subclass without a dict: no cache
+                pass
+        return hit[1]
+
+    @staticmethod
     def backward(ctx, dy):
         F = LinearLowbitFunction
-        x, v, s, u, res, xv = ctx.saved_tensors
+        x, v, s, u, res, xv, t = ctx.saved_tensors
         cd = torch.bfloat16
         dy2 = _flat2d(dy).to(cd)
         x2 = _flat2d(x).to(cd)
         L, N = dy2.shape
         # rank-r branch in bf16: one pass over dY for dY U, one for dY^T t, one over x for g_xv^T x
-        g_t = ops.lowrank_project(dy2, u.to(cd).T.contiguous())            # [L, r]
-        g_u = ops.lowrank_contract_tokens(dy2, xv * s.to(cd))               # [N, r]
-        g_s = (g_t.float() * xv.float()).sum(dim=0)
+        g_t = ops.lowrank_project(dy2, _MetisFusedFunction._transposed_bf16(u))    # [L, r]
+        g_u = ops.lowrank_contract_tokens(dy2, t)                           # [N, r]
+        g_s = (g_t * xv).sum(dim=0, dtype=torch.float32)                    # the product in bf16, as autograd forms it for torch.mul(s, y)
         g_xv = g_t * s.to(cd)
         g_v = ops.lowrank_contract_tokens(x2, g_xv, transpose=True)         # [r, K]
         # residual branch on re-quantized operands
@@ -700,7 +714,7 @@ class _MetisFusedFunction(torch.autograd.Function):
             ar = F.compute_dtype
             dyq, xq_src = (_flat2d(dy), _flat2d(x)) if ar == torch.float32 else (dy2, x2)
             gx, g_res = F._packed_grads_nv(dyq, xq_src, ctx.p_res, cd, torch.bfloat16 if res.dtype == torch.bfloat16 else torch.float32,
-                                           gx_lowrank=(g_xv, v.to(cd).T.contiguous()))
+                                           gx_lowrank=(g_xv, _MetisFusedFunction._transposed_bf16(v)))
         elif F._packed_backward_applies(L, N, dy2):
             ar = F.compute_dtype                               # arithmetic of the quantizers
             p_res_col = ctx.p_res.transposed                   # lives as long as the (cached) packed residual
@@ -711,7 +725,7 @@ class _MetisFusedFunction(torch.autograd.Function):
             # the rank-r branch's share of grad_input, g_xv V, rides in the dgrad launch as its low-rank extension
             gx, g_res = F._packed_grads(dyq, xq_src, p_res_col, ctx.center, cd,
                                         torch.bfloat16 if res.dtype == torch.bfloat16 else torch.float32,
-                                        gx_lowrank=(g_xv, v.to(cd).T.contiguous()))
+                                        gx_lowrank=(g_xv, _MetisFusedFunction._transposed_bf16(v)))
         else:
             gx = torch.matmul(g_xv, v.to(cd))                  # [L, K]
             cdt = F.compute_dtype
