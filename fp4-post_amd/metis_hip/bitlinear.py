@@ -823,6 +823,10 @@ class BitLinear(nn.Module):
 
         group["input_ref"] = weakref.ref(x, clear_cached_input)
         group["quantized_input"] = quantized_input
+        # every member's GEMM reads this activation: its tiled expansion is made once and kept while it lives
+        packed = quantized_input.residual if isinstance(quantized_input, CenteredNVFP4) else quantized_input
+        if isinstance(packed, PackedNVFP4):
+            packed.shared = True
         return quantized_input
 
     @torch.no_grad()

@@ -96,6 +96,7 @@ class FusedRMSNormQuant(nn.Module):
                 group["input_ref"] = None
                 group["quantized_input"] = None
 
+        packed.shared = True                     # read by every member of the group: its tiled expansion is kept while it lives
         group["input_ref"] = weakref.ref(out, clear)
         group["quantized_input"] = packed
         return out

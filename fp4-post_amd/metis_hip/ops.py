@@ -36,6 +36,7 @@ class PackedNVFP4:
     tiled_pb16: torch.Tensor | None = None    # the reference's bf16 dequantized values in the same layout (bf16 arithmetic)
     transposed: "PackedNVFP4 | None" = None   # cached column-blocked packing of the same source tensor (dgrad operand)
     persistent: bool = False                  # lives across calls (a cached weight): worth keeping its tiled expansion
+    shared: bool = False                      # an activation read by several GEMMs (a q/k/v or gate/up group): likewise, while it lives
     rht: int | None = None                    # NV recipe: the packed values are those of the ROTATED tensor (sign mask of the rotation)
     tiled_t: torch.Tensor | None = None       # tiled expansion of the transposed tensor (contraction over this tensor's rows)
     tiled_t_pb16: torch.Tensor | None = None
@@ -399,7 +400,7 @@ def expand_tiled(p: PackedNVFP4, cache: bool = True, mode: int = MODE_P32, cente
     values e2m1 * e4m3 * 2^-8 (mode P32) or the reference's bf16 dequantized values, unit included (mode PB16).
     cache=True keeps it on the packed tensor (weights); activations are expanded per call.
     center (bf16 [cols], mode PB16): p packs a centred residual; the operand is the mean mode's center + QDQ(x - center)
-    rounded to bf16, the tensor the reference multiplies with in bf16 arithmetic (never cached)."""
+    rounded to bf16, the tensor the reference multiplies with in bf16 arithmetic."""
     L = load()
     d = p.__dict__
     lazy = d.get("deferred") is not None and d.get("_scales") is None and p.rht is None and p.cols % 32 == 0
@@ -409,7 +410,13 @@ def expand_tiled(p: PackedNVFP4, cache: bool = True, mode: int = MODE_P32, cente
         center = center.reshape(-1).to(torch.bfloat16).contiguous()
         if center.numel() != p.cols:
             raise ValueError(f"center must have {p.cols} values, got {center.numel()}")
+        key = (center.data_ptr(), center._version)
+        kept = d.get("_tiled_centered")
+        if cache and kept is not None and kept[0] == key:
+            return kept[1]
         out = torch.empty(L.metis_nvfp4_expand_tiled_bytes(p.rows, p.cols), dtype=torch.uint8, device=p.codes.device)
+        if cache:
+            d["_tiled_centered"] = (key, out, center)                 # (the centre is kept alive with its address)
         if lazy:
             rc = L.metis_nvfp4_expand_tiled_deferred(p.codes.data_ptr(), d["deferred"].data_ptr(), p.rows, p.cols, p.mode, mode,
                                                      center.data_ptr(), d["_unit"].data_ptr(), out.data_ptr(), _stream())
@@ -560,7 +567,7 @@ def linear_fwd_tiled(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None =
     elif center is not None:
         raise ValueError("a centre inside the operand belongs to reference_rounding")
     bx = expand_tiled(b, cache=b.persistent, mode=mode)
-    ax = a_tiled if a_tiled is not None else expand_tiled(a, cache=False, mode=mode, center=center)
+    ax = a_tiled if a_tiled is not None else expand_tiled(a, cache=a.shared, mode=mode, center=center)
     return gemm_tiled(ax, a.unit, bx, b.unit, a.rows, b.rows, a.cols, mode=mode, t=t, u=u, bias=bias, out_dtype=out_dtype,
                       split_k=split_k)
 
@@ -816,7 +823,7 @@ def _linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.
     operand = rounded and takes and K % 256 == 0 and all(m[0].scales.data_ptr() % 8 == 0 for m in members)
     if rounded and center is not None and not operand:
         if M >= 256 and K % 32 == 0:
-            ax = expand_tiled(a, cache=False, mode=MODE_PB16, center=center)
+            ax = expand_tiled(a, cache=a.shared, mode=MODE_PB16, center=center)
             return [linear_fwd_tiled(a, b, t=t, u=u, bias=bias, out_dtype=out_dtype, a_tiled=ax, reference_rounding=True, split_k=split_k)
                     for b, t, u, bias in members]
         rounded = False                                        # exact products, the centre's share in binary32
