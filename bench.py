@@ -381,12 +381,13 @@ def main():
                                compute_dtype=torch.float32)
             xq_ = torch.randn(1, 4096, 1536, generator=torch.Generator().manual_seed(1004)).bfloat16().to(dev).requires_grad_(True)
             dy_ = (torch.randn(1, 4096, 8960, generator=torch.Generator().manual_seed(2004)) * 1e-3).bfloat16().to(dev)
+            dy_ = dy_.float()        # the layer's output is binary32 in this arithmetic: the upstream gradient arrives in that dtype
 
             def qat_step(ev):
                 if ev is not None:
                     ev[0].record()
                 y_ = lin(xq_)
-                y_.backward(dy_.to(y_.dtype))
+                y_.backward(dy_)
                 if ev is not None:
                     ev[1].record()
                 lin.weight.grad = None
@@ -408,7 +409,7 @@ def main():
                 if ev is not None:
                     ev[0].record()
                 y_ = mlin(xq_)
-                y_.backward(dy_.to(y_.dtype))
+                y_.backward(dy_)
                 if ev is not None:
                     ev[1].record()
                 mlin.weight.grad = None
@@ -437,7 +438,7 @@ def main():
                 if ev is not None:
                     ev[0].record()
                 y_ = nlin(xq_)
-                y_.backward(dy_.to(y_.dtype))
+                y_.backward(dy_)
                 if ev is not None:
                     ev[1].record()
                 nlin.weight.grad = None
