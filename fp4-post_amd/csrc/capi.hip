@@ -151,6 +151,14 @@ int metis_nvfp4_expand_tiled_rht(const void* codes, const void* scales, const fl
     return expand_xt(codes, scales, unit, rows, cols, mode, out, (hipStream_t)stream, rotate_back != 0, sign_mask);
 }
 
+int metis_nvfp4_quant_sr_both(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, uint64_t seed, uint64_t offset_row,
+                              uint64_t offset_col, void* codes_row, void* scales_row, float* unit_row, void* codes_col,
+                              void* scales_col, float* unit_col, void* workspace, size_t workspace_bytes, void* stream)
+{
+    return quantize_both_sr(x, rows, cols, ld, mode, seed, offset_row, offset_col, codes_row, scales_row, unit_row, codes_col, scales_col,
+                            unit_col, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
 size_t metis_nvfp4_deferred_bytes(int64_t rows, int64_t cols) { return deferred_bytes(rows, cols); }
 
 int metis_nvfp4_quant_row_deferred(const void* x, int64_t rows, int64_t cols, int mode, const void* center, void* codes, void* deferred,

@@ -47,6 +47,10 @@ int quantize(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, bo
              uint64_t seed, uint64_t offset, void* codes, void* scales, float* unit, void* workspace,
              size_t workspace_bytes, hipStream_t st, const void* center = nullptr, bool resident = false,
              uint32_t spin_limit = 0);
+// both packings (blocks along rows, blocks down columns) of one tensor with stochastic rounding in one pass; nvfp4_quant.hip
+int quantize_both_sr(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, uint64_t seed, uint64_t offset_row,
+                     uint64_t offset_col, void* codes_row, void* scales_row, float* unit_row, void* codes_col, void* scales_col,
+                     float* unit_col, void* workspace, size_t bytes, hipStream_t st);
 // deferred scale bytes (nvfp4_quant.hip): phase 1 alone into caller-owned parked data, phase 2 on it later or never
 size_t deferred_bytes(int64_t rows, int64_t cols);
 int carve_deferred(void* p, size_t bytes, int64_t rows, int64_t cols, Workspace* ws);

@@ -234,6 +234,131 @@ __global__ __launch_bounds__(256) void quant_codes_col_kernel(
 }
 
 // ---------------------------------------------------------------------------------------------
+// Phase 1 of BOTH packings of one tensor in one pass: the weight-gradient and input-gradient GEMMs of the backward
+// pass contract the output gradient over different dimensions, so dY is packed twice -- blocks along its last
+// dimension (rows) and blocks down its columns (src/Metis/Metis/bitlinear.py:488-510 re-quantizes grad_output for
+// each product).  Stochastic rounding on the library's own stream; the two packings draw from their own offsets, so the
+// results are those of quant_codes_kernel<.., SR> and quant_codes_col_kernel<.., SR> called one after the other.
+// Same tile as the column kernel (256 rows x 64 columns per workgroup, wave g takes 16-row slabs 4g .. 4g+3): a lane
+// holds one column of a slab; the slab also goes through LDS (68-word rows) and comes back as row blocks, lane l
+// taking row l / 4, block l % 4.  Both packings share the tensor maximum, hence one partial maximum per workgroup.
+// ---------------------------------------------------------------------------------------------
+constexpr uint32_t kBothRun = 16;
+template <int MODE, bool WIDE = false>
+__global__ __launch_bounds__(256) void quant_codes_both_kernel(
+    const void* __restrict__ xv, uint32_t rows, uint32_t cols, int64_t ld, uint64_t seed, uint64_t offset_row, uint64_t offset_col,
+    uint2* __restrict__ codes_row, void* __restrict__ amax_row_v, uint2* __restrict__ codes_col, void* __restrict__ amax_col_v,
+    uint32_t* __restrict__ ws_gmax, uint32_t tiles_c, uint32_t tiles_total)
+{
+    static_assert(!WIDE || MODE == 0, "binary32 values imply binary32 arithmetic");
+    using amax_t = typename std::conditional<WIDE, float, uint16_t>::type;
+    amax_t* __restrict__ amax_row = static_cast<amax_t*>(amax_row_v);
+    amax_t* __restrict__ amax_col = static_cast<amax_t*>(amax_col_v);
+    __shared__ uint2 s_codes[kColTileCols][kColTileBlocks + 1];
+    __shared__ amax_t s_amax[kColTileCols][kColTileBlocks + 2];
+    // one 16 x 64 slab per wave, in the input's own width: binary32 words, or bf16 pairs as loaded
+    constexpr int kSlabWords = WIDE ? kColTileCols + 4 : kColTileCols / 2 + 4;
+    __shared__ __attribute__((aligned(16))) uint32_t slab[4][kBlock][kSlabWords];
+    const uint32_t nbc = rows / kBlock, nbpr = cols / kBlock;
+    const uint32_t lane = threadIdx.x & 63u, g = threadIdx.x >> 6;
+    const uint32_t rr = lane >> 2, cb = lane & 3u;            // as a row block: row rr of the slab, block cb of its 64 columns
+    float gmax = 0.0f;
+    auto parked = [](float am) -> amax_t {
+        if constexpr (WIDE) return am;
+        else return (uint16_t)(__float_as_uint(am) >> 16);
+    };
+    // A tile's row blocks are 32 bytes of a row of codes, and 8 bytes of a row of maxima: kBothRun tiles side by side
+    // complete whole 128-byte lines.  Workgroups go round the eight dies in turn, each die with an L2 of its own that
+    // merges partial lines; so the workgroups of one die take a run of kBothRun neighbouring tiles at a time.
+    const uint32_t span = 8u * kBothRun, padded = (tiles_total + span - 1) / span * span;
+    for (uint32_t wid = blockIdx.x; wid < padded; wid += gridDim.x) {
+        const uint32_t tile = wid / span * span + (wid % 8u) * kBothRun + (wid / 8u) % kBothRun;
+        if (tile >= tiles_total) continue;
+        const uint32_t tr = tile / tiles_c, tc = tile - tr * tiles_c;
+        const uint32_t c = tc * kColTileCols + lane;
+        const uint32_t cbg = tc * 4u + cb;
+#pragma unroll 1
+        for (uint32_t k = 0; k < 4u; ++k) {
+            const uint32_t bl = g * 4u + k, b = tr * kColTileBlocks + bl;
+            // the row block: 16 consecutive values of one row, 16-byte loads; to this wave's slab in LDS as loaded, and
+            // back as columns.  A wave's LDS operations complete in the order issued, so no wait lies between its own
+            // writes and reads: the barriers only keep the compiler from moving them.
+            float w[kBlock] = {}, v[kBlock];
+            const bool have_row = b < nbc && cbg < nbpr;
+            if constexpr (WIDE) {
+                float4 f[4] = {};
+                if (have_row) {
+                    const float4* src = reinterpret_cast<const float4*>(static_cast<const float*>(xv) + (int64_t)(b * kBlock + rr) * ld + (int64_t)cbg * kBlock);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) f[q] = src[q];
+                }
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    w[4 * q] = f[q].x; w[4 * q + 1] = f[q].y; w[4 * q + 2] = f[q].z; w[4 * q + 3] = f[q].w;
+                    *reinterpret_cast<float4*>(&slab[g][rr][cb * kBlock + 4 * q]) = f[q];
+                }
+                __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                for (int j = 0; j < kBlock; ++j) v[j] = __uint_as_float(slab[g][j][lane]);
+            } else {
+                uint4 lo = make_uint4(0u, 0u, 0u, 0u), hi = lo;
+                if (have_row) {
+                    const uint4* src = reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(xv) + (int64_t)(b * kBlock + rr) * ld + (int64_t)cbg * kBlock);
+                    lo = src[0];
+                    hi = src[1];
+                }
+                const uint32_t u[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+                for (int q = 0; q < 8; ++q) { w[2 * q] = bf16_lo(u[q]); w[2 * q + 1] = bf16_hi(u[q]); }
+                *reinterpret_cast<uint4*>(&slab[g][rr][cb * 8u]) = lo;
+                *reinterpret_cast<uint4*>(&slab[g][rr][cb * 8u + 4u]) = hi;
+                __builtin_amdgcn_wave_barrier();
+                const uint32_t shift = (lane & 1u) ? 0u : 16u;  // a bf16 is the upper half of its binary32 value
+#pragma unroll
+                for (int j = 0; j < kBlock; ++j) v[j] = __uint_as_float((slab[g][j][lane >> 1] << shift) & 0xffff0000u);
+            }
+            __builtin_amdgcn_wave_barrier();
+            if (have_row) {
+                const float amr = block_amax(w);
+                gmax = fmaxf(gmax, amr);
+                const int64_t ir = (int64_t)(b * kBlock + rr) * nbpr + cbg;
+                uint2 pr;
+                if constexpr (WIDE) pr = encode_sr_hardware<0, true>(w, block_scalar_ieee(amr), seed, offset_row, ir);
+                else pr = encode_sr_hardware<MODE>(w, block_scalar<MODE>(amr), seed, offset_row, ir);
+                codes_row[ir] = pr;
+                amax_row[ir] = parked(amr);
+            }
+            uint2 packed = make_uint2(0u, 0u);
+            float am = 0.0f;
+            if (c < cols && b < nbc) {
+                am = block_amax(v);
+                if constexpr (WIDE) packed = encode_sr_hardware<0, true>(v, block_scalar_ieee(am), seed, offset_col, (int64_t)c * nbc + b);
+                else packed = encode_sr_hardware<MODE>(v, block_scalar<MODE>(am), seed, offset_col, (int64_t)c * nbc + b);
+            }
+            s_codes[lane][bl] = packed;
+            s_amax[lane][bl] = parked(am);
+        }
+        __syncthreads();
+        {   // column t / 4, blocks 4 (t % 4) .. +3 of the tile: 32 contiguous bytes of codes, 8 of maxima
+            const uint32_t oc = threadIdx.x >> 2, part = threadIdx.x & 3u;
+            const uint32_t c2 = tc * kColTileCols + oc, b0 = tr * kColTileBlocks + part * 4u;
+            if (c2 < cols) {
+#pragma unroll
+                for (uint32_t i = 0; i < 4u; ++i) {
+                    if (b0 + i < nbc) {
+                        const int64_t ob = (int64_t)c2 * nbc + b0 + i;
+                        codes_col[ob] = s_codes[oc][part * 4u + i];
+                        amax_col[ob] = s_amax[oc][part * 4u + i];
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+    publish_group_max(gmax, ws_gmax);
+}
+
+// ---------------------------------------------------------------------------------------------
 // Phase 2: tensor unit and E4M3 scale bytes (quant.py:21-23), four blocks per thread.
 // Every workgroup folds the published partial maxima itself (a few KB from L2).
 // ---------------------------------------------------------------------------------------------
@@ -722,6 +847,66 @@ int quantize(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, bo
         else { if (!col) METIS_Q(1, true, false); else METIS_Q(1, true, true); }
     }
 #undef METIS_Q
+}
+
+// Workgroups of quant_codes_both_kernel that the current device holds at once (its LDS slabs bound them): the grid is
+// no larger, so that every workgroup starts at once and walks the same number of tiles, give or take one.
+template <int MODE, bool WIDE>
+static int both_capacity()
+{
+    static int cached[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    if (cached[dev] == 0) {
+        int per_cu = 0;
+        const hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, quant_codes_both_kernel<MODE, WIDE>, 256, 0);
+        cached[dev] = (e != hipSuccess || per_cu <= 0) ? -1 : per_cu * device_cus();
+    }
+    return cached[dev] < 0 ? device_cus() * 4 : cached[dev];
+}
+
+// ---------------------------------------------------------------------------------------------
+// Both packings of one tensor (rows and columns) with stochastic rounding, one pass over x; then phase 2 for each.
+// The workspace holds two areas of parked maxima: 2 x workspace_bytes(rows, cols).
+// ---------------------------------------------------------------------------------------------
+int quantize_both_sr(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, uint64_t seed, uint64_t offset_row,
+                     uint64_t offset_col, void* codes_row, void* scales_row, float* unit_row, void* codes_col, void* scales_col,
+                     float* unit_col, void* workspace, size_t bytes, hipStream_t st)
+{
+    if (rows < 0 || cols < 0 || ld < cols) return METIS_E_ARG;
+    if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16 && mode != METIS_MODE_P32_F32) return METIS_E_ARG;
+    const bool f32in = mode == METIS_MODE_P32_F32;
+    if (rows % kBlock || cols % kBlock) return METIS_E_SHAPE;
+    if (rows == 0 || cols == 0) return METIS_OK;
+    if (!x || !codes_row || !scales_row || !unit_row || !codes_col || !scales_col || !unit_col) return METIS_E_ARG;
+    if (rows * cols / kBlock >= (int64_t)1 << 31) return METIS_E_ARG;
+    if ((ld % (f32in ? 4 : 8)) || ((uintptr_t)x % 16)) return METIS_E_ARG;                 // 16-byte vector loads
+    if (((uintptr_t)codes_row % 8) || ((uintptr_t)scales_row % 8) || ((uintptr_t)codes_col % 8) || ((uintptr_t)scales_col % 8)) return METIS_E_ARG;
+    const size_t one = workspace_bytes(rows, cols);
+    if (!workspace || ((uintptr_t)workspace % 256) || bytes < 2 * one) return METIS_E_WORKSPACE;
+    Workspace wr, wc;
+    if (const int rc = carve_workspace(workspace, one, rows, cols, &wr)) return rc;
+    if (const int rc = carve_workspace(static_cast<char*>(workspace) + one, one, rows, cols, &wc)) return rc;
+    wc.gmax = wr.gmax;                                         // one tensor, one maximum: both packings fold the same partials
+    const uint32_t nblocks = (uint32_t)(rows * cols / kBlock);
+    const uint32_t tiles_r = (uint32_t)((rows / kBlock + kColTileBlocks - 1) / kColTileBlocks);
+    const uint32_t tiles_c = (uint32_t)((cols + kColTileCols - 1) / kColTileCols);
+    const int64_t tiles = (int64_t)tiles_r * tiles_c;
+    int64_t g = tiles;
+    const int64_t cap = f32in ? both_capacity<0, true>() : mode == 0 ? both_capacity<0, false>() : both_capacity<1, false>();
+    if (g > cap) g = cap;
+    if (g > kMaxGroups) g = kMaxGroups;
+#define METIS_QB(M, W) hipLaunchKernelGGL((quant_codes_both_kernel<M, W>), dim3((unsigned)g), dim3(256), 0, st, x, (uint32_t)rows, \
+                                          (uint32_t)cols, ld, seed, offset_row, offset_col, (uint2*)codes_row, (void*)wr.amax, (uint2*)codes_col, \
+                                          (void*)wc.amax, wr.gmax, tiles_c, (uint32_t)tiles)
+    if (f32in) METIS_QB(0, true);
+    else if (mode == 0) METIS_QB(0, false);
+    else METIS_QB(1, false);
+#undef METIS_QB
+    if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
+    const int pm = f32in ? METIS_MODE_P32_F32 : mode;
+    if (const int rc = launch_scales(pm, wr, (uint32_t)g, scales_row, unit_row, nblocks, st)) return rc;
+    return launch_scales(pm, wc, (uint32_t)g, scales_col, unit_col, nblocks, st);
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -52,6 +52,8 @@ SIGNATURES = {
     "metis_hadamard16": (_i32, [_vp, _i64, _i64, _i64, _i32, _i32, ctypes.c_uint32, _vp, _i64, _vp]),
     "metis_nvfp4_quant_row_rht": (_i32, [_vp, _i64, _i64, _i64, _i32, ctypes.c_uint32, _i32, _u64, _u64, _vp, _vp, _vp, _vp, _sz, _vp]),
     "metis_nvfp4_expand_tiled_rht": (_i32, [_vp, _vp, _vp, _i64, _i64, _i32, ctypes.c_uint32, _i32, _i32, _vp, _vp]),
+    "metis_nvfp4_quant_sr_both": (_i32, [_vp, _i64, _i64, _i64, _i32, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64, _vp, _vp, _vp, _vp, _vp,
+                                  _vp, _vp, _sz, _vp]),
     "metis_nvfp4_deferred_bytes": (_sz, [_i64, _i64]),
     "metis_nvfp4_quant_row_deferred": (_i32, [_vp, _i64, _i64, _i32, _vp, _vp, _vp, _sz, _vp]),
     "metis_rmsnorm_nvfp4_quant_deferred": (_i32, [_vp, _vp, _f32, _i64, _i64, _i32, _vp, _vp, _vp, _sz, _vp]),

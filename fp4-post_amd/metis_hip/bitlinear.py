@@ -365,7 +365,10 @@ class LinearLowbitFunction(torch.autograd.Function):
             dy2, x2 = padded(dy2, me_dy), padded(x2, center_x)
             if gx_lowrank is not None:
                 gx_lowrank = (padded(gx_lowrank[0], None), gx_lowrank[1])
-        p_dy = qg.pack(dy2, arith=cd, center=me_dy)
+        if me_dy is None and hasattr(qg, "pack_both"):
+            p_dy, p_dyt = qg.pack_both(dy2, arith=cd)          # one pass over dY for both products
+        else:
+            p_dy, p_dyt = qg.pack(dy2, arith=cd, center=me_dy), None
         if me_dy is None and gx_lowrank is None:
             gx = ops.linear_dgrad(p_dy, pw_col, out_dtype=gx_dtype)
         else:
@@ -374,7 +377,8 @@ class LinearLowbitFunction(torch.autograd.Function):
                                 out_dtype=gx_dtype)
         if pad:
             gx = gx[:L]
-        p_dyt = qg.pack(dy2, col=True, arith=cd, center=me_dy)
+        if p_dyt is None:
+            p_dyt = qg.pack(dy2, col=True, arith=cd, center=me_dy)
         p_xt = qi.pack(x2, col=True, arith=cd, center=center_x)
         if me_dy is None and center_x is None:
             # autograd rounds the gradient to the parameter's dtype anyway: let the GEMM epilogue do that rounding

@@ -219,6 +219,37 @@ def quantize(x: torch.Tensor, mode: int = MODE_P32, *, col: bool = False, sr: bo
     return PackedNVFP4(codes, scales, unit, prow, pcol, mode)
 
 
+def quantize_both_sr(x: torch.Tensor, mode: int = MODE_P32, *, seed: int = 0, offset_row: int = 0,
+                     offset_col: int = 0) -> tuple[PackedNVFP4, PackedNVFP4]:
+    """(quantize(x, sr=True, offset=offset_row), quantize(x, col=True, sr=True, offset=offset_col)) from ONE pass over x:
+    the two packings of an output gradient that the input-gradient and weight-gradient products contract.  Same
+    bytes as the two calls.  Both dimensions of x flattened to [R, C] have to be multiples of 16."""
+    x2, kmode = _as_2d_for_quant(x, mode)
+    rows, cols = x2.shape
+    if rows % BLOCK or cols % BLOCK:
+        raise ValueError(f"NVFP4 block shape (1, 16) does not divide tensor shape {tuple(x.shape)} both ways")
+    dev = x2.device
+    L = load()
+    packs = []
+    for prow, pcol in ((rows, cols), (cols, rows)):
+        packs.append((torch.empty(prow, pcol // 2, dtype=torch.uint8, device=dev),
+                      torch.empty(prow, pcol // BLOCK, dtype=torch.uint8, device=dev),
+                      torch.empty(1, dtype=torch.float32, device=dev)))
+    need = 2 * L.metis_nvfp4_workspace_bytes(rows, cols)
+    key = (dev.index, _stream(), "both")
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < need:
+        ws = torch.empty(max(need, 1 << 20), dtype=torch.uint8, device=dev).fill_(0)
+        _workspaces[key] = ws
+    (cr, sr_, ur), (cc, sc, uc) = packs
+    if rows * cols:
+        rc = L.metis_nvfp4_quant_sr_both(x2.data_ptr(), rows, cols, x2.stride(0), kmode, seed & (2 ** 64 - 1), offset_row, offset_col,
+                                         cr.data_ptr(), sr_.data_ptr(), ur.data_ptr(), cc.data_ptr(), sc.data_ptr(), uc.data_ptr(),
+                                         ws.data_ptr(), ws.numel(), _stream())
+        check(rc, "metis_nvfp4_quant_sr_both", x.shape)
+    return PackedNVFP4(cr, sr_, ur, rows, cols, mode), PackedNVFP4(cc, sc, uc, cols, rows, mode)
+
+
 def dequantize(p: PackedNVFP4, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     if dtype not in (torch.bfloat16, torch.float32):
         raise ValueError("dequantize: dtype must be bfloat16 or float32")

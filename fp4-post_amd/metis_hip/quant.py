@@ -113,6 +113,21 @@ class _NVFP4Base(BlockQuantFunc):
 
     @classmethod
     @torch.no_grad()
+    def pack_both(cls, x: torch.Tensor, arith: torch.dtype | None = None) -> tuple[ops.PackedNVFP4, ops.PackedNVFP4]:
+        """(pack(x), pack(x, col=True)): the same two tensors, and under stochastic rounding the same draws in the same
+        order, from one pass over x where the kernels have one (stochastic rounding, both dimensions multiples of 16)."""
+        _need_gpu(x)
+        cls._check(x)
+        rows = x.numel() // x.shape[-1] if x.numel() else 0
+        if cls.stochastic and rows and rows % 16 == 0 and x.dtype in (torch.bfloat16, torch.float32):
+            mode = _mode_of(x) if arith is None else (MODE_P32 if arith == torch.float32 else MODE_PB16)
+            first = cls._next_offset(x.numel())
+            second = cls._next_offset(x.numel())
+            return ops.quantize_both_sr(x, mode, seed=_NVFP4Base.sr_seed, offset_row=first, offset_col=second)
+        return cls.pack(x, arith=arith), cls.pack(x, col=True, arith=arith)
+
+    @classmethod
+    @torch.no_grad()
     def quantize_dequantize(cls, x: torch.Tensor):
         """Fused QDQ (quant.py:6-36 / 392-433): same shape and dtype as x."""
         cls._check(x)

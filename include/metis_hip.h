@@ -157,6 +157,22 @@ int metis_nvfp4_quant_sr_col(const void *x, int64_t rows, int64_t cols, int64_t 
                              void *stream);
 
 /*
+ * Both packings of one tensor with stochastic rounding on the library's own stream, in one pass over x: the
+ * backward pass needs dY blocked along its last dimension for dX = dY W and blocked down its columns for
+ * dW = dY^T X (src/Metis/Metis/bitlinear.py:488-510 quantizes grad_output for each product).  The results are
+ * those of metis_nvfp4_quant_sr_row(.., noise = NULL, seed, offset_row, ..) and metis_nvfp4_quant_sr_col(.., noise =
+ * NULL, seed, offset_col, ..), byte for byte; each consumes rows * cols / 16 counters from its own offset.
+ *   x          bf16 [rows, cols] (binary32 in METIS_MODE_P32_F32), row stride ld (ld % 8 == 0, ld % 4 in binary32),
+ *              16-byte aligned; rows % 16 == 0 and cols % 16 == 0, else METIS_E_SHAPE
+ *   workspace  2 * metis_nvfp4_workspace_bytes(rows, cols) bytes
+ */
+int metis_nvfp4_quant_sr_both(const void *x, int64_t rows, int64_t cols, int64_t ld, int mode,
+                              uint64_t seed, uint64_t offset_row, uint64_t offset_col,
+                              void *codes_row, void *scales_row, float *unit_row, void *codes_col,
+                              void *scales_col, float *unit_col, void *workspace,
+                              size_t workspace_bytes, void *stream);
+
+/*
  * The reference's three-call form on dequantized tensors of dtype D (float32 in METIS_MODE_P32, bf16 in
  * METIS_MODE_PB16), for callers that use the quantizer classes directly.  All tensors contiguous [rows, cols].
  *   metis_nvfp4_get_scalar : Cast2NVFp4e2m1Block[NOSR].get_scalar (src/Metis/Metis/quant.py:435-455)

@@ -560,3 +560,65 @@ def test_col_quant_large_ragged_tensors(ops, tag, mode):
     a = ops.quantize(xin.cuda(), 1 if mode == 1 else 0, col=True, sr=True, seed=5, offset=9)
     b = ops.quantize(xin.cuda().t().contiguous(), 1 if mode == 1 else 0, sr=True, seed=5, offset=9)
     assert torch.equal(a.codes, b.codes) and torch.equal(a.scales, b.scales)
+
+
+@pytest.mark.parametrize("tag,mode", MODES + [("f32", 2)])
+@pytest.mark.parametrize("shape", [(16, 16), (48, 80), (256, 64), (1008, 1552), (4096 + 48, 2048 + 16)])
+def test_both_packings_in_one_pass_equal_the_two_calls(ops, tag, mode, shape):
+    """Row-blocked and column-blocked stochastic packings of one tensor from one kernel: the same bytes as the row call
+    and the column call with the same seed and offsets (tiles ragged in both directions, single block, one tile)."""
+    rows, cols = shape
+    g = torch.Generator().manual_seed(1234 + rows)
+    x = torch.randn(rows, cols, generator=g) * torch.exp(torch.randn(rows, 1, generator=g))
+    x.view(-1)[::53] = 0
+    xin = (x if mode == 2 else x.bfloat16()).cuda()
+    km = 1 if mode == 1 else 0
+    seed, o_row, o_col = 0x9E3779B97F4A7C15, (1 << 33) + 7, 12345
+    pr, pc = ops.quantize_both_sr(xin, km, seed=seed, offset_row=o_row, offset_col=o_col)
+    want_r = ops.quantize(xin, km, sr=True, seed=seed, offset=o_row)
+    want_c = ops.quantize(xin, km, col=True, sr=True, seed=seed, offset=o_col)
+    torch.cuda.synchronize()
+    for got, want, what in ((pr, want_r, "rows"), (pc, want_c, "columns")):
+        assert (got.rows, got.cols) == (want.rows, want.cols)
+        assert torch.equal(got.codes, want.codes), f"{what} codes {tag} {shape}: {(got.codes != want.codes).sum().item()} bytes"
+        assert torch.equal(got.scales, want.scales), f"{what} scale bytes {tag} {shape}"
+        assert torch.equal(got.unit, want.unit), f"{what} unit {tag} {shape}"
+    # a strided view (row stride larger than the width) reads the same values
+    if cols >= 32:
+        wide = torch.zeros(rows, cols + 64, dtype=xin.dtype, device="cuda")
+        wide[:, :cols] = xin
+        x2, kmode = wide[:, :cols], (2 if mode == 2 else km)
+        from metis_hip import _lib
+        L = _lib.load()
+        outs = [torch.empty_like(t_) for t_ in (pr.codes, pr.scales, pr.unit, pc.codes, pc.scales, pc.unit)]
+        ws = torch.zeros(2 * L.metis_nvfp4_workspace_bytes(rows, cols), dtype=torch.uint8, device="cuda")
+        rc = L.metis_nvfp4_quant_sr_both(x2.data_ptr(), rows, cols, x2.stride(0), kmode, seed, o_row, o_col, *[o.data_ptr() for o in outs],
+                                         ws.data_ptr(), ws.numel(), None)
+        assert rc == 0
+        torch.cuda.synchronize()
+        for o, w in zip(outs, (pr.codes, pr.scales, pr.unit, pc.codes, pc.scales, pc.unit)):
+            assert torch.equal(o, w)
+
+
+def test_both_packings_argument_checks(ops):
+    from metis_hip import _lib
+    L = _lib.load()
+    x = torch.zeros(64, 64, dtype=torch.bfloat16, device="cuda")
+    o = torch.zeros(1 << 16, dtype=torch.uint8, device="cuda")
+    u = torch.zeros(2, dtype=torch.float32, device="cuda")
+    ws = torch.zeros(2 * L.metis_nvfp4_workspace_bytes(64, 64), dtype=torch.uint8, device="cuda")
+
+    def call(rows, cols, ld, mode=0, ptr=None, wsn=None):
+        return L.metis_nvfp4_quant_sr_both(x.data_ptr() if ptr is None else ptr, rows, cols, ld, mode, 1, 0, 0, o.data_ptr(), o.data_ptr() + 8192,
+                                           u.data_ptr(), o.data_ptr() + 16384, o.data_ptr() + 32768, u.data_ptr() + 4, ws.data_ptr(),
+                                           ws.numel() if wsn is None else wsn, None)
+
+    assert call(64, 64, 64) == 0
+    assert call(0, 64, 64) == 0 and call(64, 0, 64) == 0           # nothing to do
+    assert call(40, 64, 64) == _lib.E_SHAPE and call(64, 40, 64) == _lib.E_SHAPE
+    assert call(64, 64, 60) == _lib.E_ARG                          # row stride below the width
+    assert call(32, 32, 36) == _lib.E_ARG                          # rows not 16-byte aligned
+    assert call(64, 64, 64, ptr=x.data_ptr() + 2) == _lib.E_ARG
+    assert call(64, 64, 64, mode=7) == _lib.E_ARG
+    assert call(64, 64, 64, wsn=ws.numel() // 2) == _lib.E_WORKSPACE  # one workspace is not enough for two sets of maxima
+    torch.cuda.synchronize()
