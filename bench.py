@@ -162,12 +162,11 @@ def main():
         sys.exit(1)
 
     def step(ev):
-        # what ops.linear_fwd does for a cached weight of this size, spelled out so that the events bracket the GEMM
-        # launch alone: quantize X (codes and parked block maxima: the expansion forms unit and scale bytes itself),
-        # expand it into the tiled binary16 layout, rank-r projection, pipelined GEMM
-        px = ops.quantize(x, deferred=True)
+        # what BitLinear.forward does for a cached weight of this size, spelled out so that the events bracket the GEMM
+        # launch alone: one pass over X that quantizes it (codes and parked block maxima: the expansion forms unit and
+        # scale bytes itself) and forms (X V^T) * s in bf16; the expansion into the tiled binary16 layout; the pipelined GEMM
+        px, _, t = ops.quantize_project(x, v, s)
         ax = ops.expand_tiled(px, cache=False)
-        _, t = ops.lowrank_project(x, v, s)                      # (X V^T) * s in bf16, one pass over X
         if ev is not None:
             ev[0].record()
         y = ops.linear_fwd_tiled(px, pw, t=t, u=u, a_tiled=ax)
@@ -597,7 +596,7 @@ def main():
         "dtype": "nvfp4 (e2m1 x e4m3) expanded exactly to f16, f32 accumulate; low-rank bf16",
         "data": "synthetic",
         "config": {"workload": "config 3: Metis low-rank-residual linear forward, X[8192,4096] W[14336,4096] r=64; "
-                               "step = quantize X (codes + block maxima) + expand X to tiled f16 (forms unit and scale bytes) + X.V^T*s + fused pipelined GEMM (packed W and its tiled f16 expansion cached)",
+                               "step = one pass over X (NVFP4 codes + block maxima, and X.V^T*s) + expand X to tiled f16 (forms unit and scale bytes) + fused pipelined GEMM (packed W and its tiled f16 expansion cached)",
                    "parity_mode": "P32", "parity_rel_fro_256_rows": err},
         "roofline": {"bound": "mfma", "kernel": "gemm_xt_kernel", "achieved": round(gemm_tflops, 2),
                      "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(gemm_tflops / MFMA_PEAK_TFLOPS, 4),

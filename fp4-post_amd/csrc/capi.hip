@@ -380,6 +380,23 @@ int metis_lowrank_project_rows(const void* x, int64_t ldx, const void* v, int64_
     return lowrank_nt(x, ldx, v, M, R, K, s, xv, t, (hipStream_t)stream);
 }
 
+size_t metis_lowrank_project_rows_workspace_bytes(int64_t M, int64_t R, int64_t K) { return lowrank_nt_workspace_bytes(M, R, K); }
+
+int metis_lowrank_project_rows_ws(const void* x, int64_t ldx, const void* v, int64_t M, int64_t R, int64_t K, const void* s, void* xv,
+                                  void* t, void* workspace, size_t workspace_bytes, void* stream)
+{
+    return lowrank_nt(x, ldx, v, M, R, K, s, xv, t, (hipStream_t)stream, workspace, workspace_bytes);
+}
+
+int metis_nvfp4_quant_project_deferred(const void* x, int64_t rows, int64_t cols, int mode, const void* v, int64_t R, const void* s,
+                                       void* xv, void* t, void* codes, void* deferred, size_t deferred_bytes, void* workspace,
+                                       size_t workspace_bytes, void* stream)
+{
+    if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) return METIS_E_ARG;
+    return lowrank_nt(x, cols, v, rows, R, cols, s, xv, t, (hipStream_t)stream, workspace, workspace_bytes, mode, codes, deferred,
+                      deferred_bytes);
+}
+
 size_t metis_lowrank_tokens_workspace_bytes(int64_t L, int64_t C, int64_t R) { return lowrank_tn_workspace_bytes(L, C, R); }
 
 int metis_lowrank_contract_tokens(const void* a, int64_t lda, const void* b, int64_t L, int64_t C, int64_t R, void* out, int out_dtype,

@@ -19,6 +19,7 @@
 // and a second kernel adds them in slice order.
 #include "metis_device.h"
 #include "metis_host.h"
+#include "nvfp4_encode.h"
 
 namespace metis {
 
@@ -29,10 +30,20 @@ constexpr int LR_STRIDE = 72;                    // halves per staged row of 64:
 constexpr int NT_STEP = 256;                     // k per step of lowrank_nt
 constexpr int NT_STRIDE = NT_STEP + 8;           // halves per staged row: 528 bytes, conflict-free 16-byte reads
 
-template <int RT>                                // R / 32 column tiles: 1, 2 or 4
+// K slices: with 32 rows per workgroup a tensor of a few thousand rows gives one workgroup per compute unit, too few
+// bytes in flight to cover the memory latency.  gridDim.y workgroups then share a row tile, each walking its own range
+// of steps; their binary32 partial sums go to a caller workspace ([slice][row][R]) and lowrank_nt_finish_kernel adds
+// them in slice order.  One slice: the result is written directly.
+//
+// QMODE >= 0: the same pass also quantizes x (round to nearest, rows; METIS_MODE_P32 or _PB16 arithmetic): the thread that
+// fetched a block of 16 encodes it while it stages it -- E2M1 codes, the block maximum parked as bf16, one partial
+// tensor maximum per workgroup: what quant_codes_contig_kernel leaves for a consumer that forms the scale bytes itself.
+template <int RT, int QMODE = -1>                // R / 32 column tiles: 1, 2 or 4
 __global__ __launch_bounds__(256) void lowrank_nt_kernel(const uint16_t* __restrict__ x, int64_t ldx, const uint16_t* __restrict__ v,
                                                          const uint16_t* __restrict__ s, uint16_t* __restrict__ xv,
-                                                         uint16_t* __restrict__ t, int M, int K)
+                                                         uint16_t* __restrict__ t, int M, int K, float* __restrict__ part,
+                                                         uint2* __restrict__ codes, uint16_t* __restrict__ q_amax,
+                                                         uint32_t* __restrict__ q_gmax, uint32_t fill_to)
 {
     constexpr int R = RT * 32;
     constexpr int TILE_BYTES = (32 + R) * NT_STRIDE * 2;        // one staged step: x rows, then v rows
@@ -43,15 +54,17 @@ __global__ __launch_bounds__(256) void lowrank_nt_kernel(const uint16_t* __restr
     float* red = reinterpret_cast<float*>(lds);                 // [wave][j][e][lane]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int m0 = blockIdx.x * 32;
-    // staging: 16-byte chunk id -> (row id / 32, chunk id % 32): a wave covers two rows x 512 contiguous bytes per load.
-    // A thread keeps two whole steps (each 4 chunks of x, 4 RT of v) in registers while the one before them is
-    // multiplied: with one workgroup per compute unit that is what keeps enough bytes in flight.
+    // staging: a thread fetches two blocks of 16 of x per step (32 contiguous bytes each; 16 threads cover the 512
+    // bytes of a row) and 4 RT 16-byte chunks of v (a wave covers two rows x 512 contiguous bytes per load).
+    // It keeps two whole steps in registers while the one before them is multiplied: that is what keeps bytes in flight.
     uint4 rx[2][4], rv[2][RT * 4];
     auto fetch = [&](uint4 (&qx)[4], uint4 (&qv)[RT * 4], int k0) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int id = i * 256 + tid, row = id >> 5, k = k0 + (id & 31) * 8;
-            qx[i] = k < K ? *reinterpret_cast<const uint4*>(x + (int64_t)min(m0 + row, M - 1) * ldx + k) : make_uint4(0u, 0u, 0u, 0u);
+        for (int i = 0; i < 2; ++i) {
+            const int id = i * 256 + tid, row = id >> 4, k = k0 + (id & 15) * 16;
+            const uint4* src = reinterpret_cast<const uint4*>(x + (int64_t)min(m0 + row, M - 1) * ldx + k);
+            qx[2 * i] = k < K ? src[0] : make_uint4(0u, 0u, 0u, 0u);
+            qx[2 * i + 1] = k < K ? src[1] : make_uint4(0u, 0u, 0u, 0u);
         }
 #pragma unroll
         for (int i = 0; i < RT * 4; ++i) {
@@ -59,16 +72,43 @@ __global__ __launch_bounds__(256) void lowrank_nt_kernel(const uint16_t* __restr
             qv[i] = k < K ? *reinterpret_cast<const uint4*>(v + (int64_t)row * K + k) : make_uint4(0u, 0u, 0u, 0u);
         }
     };
+    float gmax = 0.0f;
+    // QMODE >= 0: the step just staged stays in px and is encoded after the next loads have been issued and the MFMAs
+    // queued, so the encoder's vector arithmetic runs while the memory system works, not between a wait and a barrier
+    uint4 px[QMODE >= 0 ? 4 : 1];
     auto stage = [&](const uint4 (&qx)[4], const uint4 (&qv)[RT * 4]) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int id = i * 256 + tid;
-            *reinterpret_cast<uint4*>(tile + (id >> 5) * NT_STRIDE + (id & 31) * 8) = qx[i];
+        for (int i = 0; i < 2; ++i) {
+            const int id = i * 256 + tid, row = id >> 4, blk = id & 15;
+            *reinterpret_cast<uint4*>(tile + row * NT_STRIDE + blk * 16) = qx[2 * i];
+            *reinterpret_cast<uint4*>(tile + row * NT_STRIDE + blk * 16 + 8) = qx[2 * i + 1];
+        }
+        if constexpr (QMODE >= 0) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) px[i] = qx[i];
         }
 #pragma unroll
         for (int i = 0; i < RT * 4; ++i) {
             const int id = i * 256 + tid;
             *reinterpret_cast<uint4*>(tile + (32 + (id >> 5)) * NT_STRIDE + (id & 31) * 8) = qv[i];
+        }
+    };
+    auto encode = [&](int k0) {
+        if constexpr (QMODE >= 0) {
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const int id = i * 256 + tid, row = id >> 4, k = k0 + (id & 15) * 16;
+                if (m0 + row < M && k < K) {
+                    float val[kBlock];
+                    const float none[kBlock] = {};
+                    unpack16(px[2 * i], px[2 * i + 1], val);
+                    const float am = block_amax(val);
+                    gmax = fmaxf(gmax, am);
+                    const int64_t ib = (int64_t)(m0 + row) * (K / kBlock) + k / kBlock;
+                    q_amax[ib] = (uint16_t)(__float_as_uint(am) >> 16);
+                    codes[ib] = encode_block<QMODE < 0 ? 0 : QMODE, false>(val, block_scalar<QMODE < 0 ? 0 : QMODE>(am), none);
+                }
+            }
         }
     };
     float16_t acc[RT];
@@ -77,7 +117,9 @@ __global__ __launch_bounds__(256) void lowrank_nt_kernel(const uint16_t* __restr
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[j][e] = 0.0f;
 
-    const int steps = (K + NT_STEP - 1) / NT_STEP;              // K % 64 == 0; a short last step is padded with zeros
+    const int steps_all = (K + NT_STEP - 1) / NT_STEP;          // K % 64 == 0; a short last step is padded with zeros
+    const int per = (steps_all + (int)gridDim.y - 1) / (int)gridDim.y;
+    const int first = (int)blockIdx.y * per, steps = max(0, min(steps_all, first + per) - first);
     // wave w multiplies the quarter [64 w, 64 w + 64) of every step
     const int foff = (lane & 31) * NT_STRIDE + wave * 64 + (lane >> 5) * 8;
     auto multiply = [&]() {
@@ -92,21 +134,33 @@ __global__ __launch_bounds__(256) void lowrank_nt_kernel(const uint16_t* __restr
         }
     };
     // two steps are in flight while a third is multiplied: the time of one step is then half the memory latency
-    fetch(rx[0], rv[0], 0);
-    if (steps > 1) fetch(rx[1], rv[1], NT_STEP);
+    if (steps > 0) fetch(rx[0], rv[0], first * NT_STEP);
+    if (steps > 1) fetch(rx[1], rv[1], (first + 1) * NT_STEP);
     for (int st = 0; st < steps; st += 2) {
         stage(rx[0], rv[0]);
         __syncthreads();
-        if (st + 2 < steps) fetch(rx[0], rv[0], (st + 2) * NT_STEP);
+        if (st + 2 < steps) fetch(rx[0], rv[0], (first + st + 2) * NT_STEP);
         multiply();
+        encode((first + st) * NT_STEP);
         __syncthreads();
         if (st + 1 < steps) {
             stage(rx[1], rv[1]);
             __syncthreads();
-            if (st + 3 < steps) fetch(rx[1], rv[1], (st + 3) * NT_STEP);
+            if (st + 3 < steps) fetch(rx[1], rv[1], (first + st + 3) * NT_STEP);
             multiply();
+            encode((first + st + 1) * NT_STEP);
             __syncthreads();
         }
+    }
+    if constexpr (QMODE >= 0) {
+        // one partial maximum per workgroup, indexed over the whole grid; unused entries cleared for the folding reader
+        __shared__ float smax[4];
+        const float wm = wave_max(gmax);
+        if (lane == 0) smax[wave] = wm;
+        __syncthreads();
+        const uint32_t gid = blockIdx.y * gridDim.x + blockIdx.x, gsize = gridDim.x * gridDim.y;
+        if (tid == 0) q_gmax[gid] = __float_as_uint(fmaxf(fmaxf(smax[0], smax[1]), fmaxf(smax[2], smax[3])));
+        for (uint32_t j = gsize + gid * 256u + tid; j < fill_to; j += gsize * 256u) q_gmax[j] = 0u;
     }
     // acc[j][e] of lane l: row m0 + l % 32, column 32 j + 8 (e / 4) + 4 (l / 32) + e % 4.  The four waves hold the four
     // quarters of every step of K: their sums meet in LDS (the staged tile is dead after the last barrier), and
@@ -121,6 +175,7 @@ __global__ __launch_bounds__(256) void lowrank_nt_kernel(const uint16_t* __restr
 #pragma unroll
     for (int j = 0; j < RT; ++j) {
         const int col = j * 32 + 8 * wave + 4 * (lane >> 5);
+        float sum4[4];
         uint32_t h[4], ts[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -128,7 +183,15 @@ __global__ __launch_bounds__(256) void lowrank_nt_kernel(const uint16_t* __restr
             float sum = red[((0 * RT + j) * 16 + ee) * 64 + lane];
 #pragma unroll
             for (int w = 1; w < 4; ++w) sum += red[((w * RT + j) * 16 + ee) * 64 + lane];
-            h[e] = bf16_bits(sum);
+            sum4[e] = sum;
+        }
+        if (part) {                                             // one of several slices: the finishing kernel rounds
+            *reinterpret_cast<float4*>(part + ((int64_t)blockIdx.y * M + m) * R + col) = make_float4(sum4[0], sum4[1], sum4[2], sum4[3]);
+            continue;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            h[e] = bf16_bits(sum4[e]);
             if (t) ts[e] = bf16_bits(__uint_as_float(h[e] << 16) * bf16_lo(s[col + e]));
         }
         *reinterpret_cast<uint2*>(xv + (int64_t)m * R + col) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
@@ -136,8 +199,55 @@ __global__ __launch_bounds__(256) void lowrank_nt_kernel(const uint16_t* __restr
     }
 }
 
+// xv = bf16(sum over slices, ascending), t = bf16(xv * s): four columns per thread
+__global__ __launch_bounds__(256) void lowrank_nt_finish_kernel(const float* __restrict__ part, int slices, int64_t MR, int R,
+                                                                const uint16_t* __restrict__ s, uint16_t* __restrict__ xv,
+                                                                uint16_t* __restrict__ t)
+{
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= MR) return;
+    float4 a = *reinterpret_cast<const float4*>(part + i);
+    for (int k = 1; k < slices; ++k) {
+        const float4 b = *reinterpret_cast<const float4*>(part + (int64_t)k * MR + i);
+        a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+    }
+    const uint32_t h[4] = {bf16_bits(a.x), bf16_bits(a.y), bf16_bits(a.z), bf16_bits(a.w)};
+    *reinterpret_cast<uint2*>(xv + i) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+    if (t) {
+        const int col = (int)(i % R);
+        uint32_t ts[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) ts[e] = bf16_bits(__uint_as_float(h[e] << 16) * bf16_lo(s[col + e]));
+        *reinterpret_cast<uint2*>(t + i) = make_uint2(ts[0] | (ts[1] << 16), ts[2] | (ts[3] << 16));
+    }
+}
+
+// K slices for M rows: none when the row tiles alone give every compute unit a workgroup (measured: slices then cost
+// what the second launch costs); otherwise about two workgroups per compute unit, at least four steps per slice, and
+// never more workgroups than the quantizer's partial maxima have room for.
+static int nt_slices(int64_t M, int64_t K, size_t workspace_bytes, int64_t R)
+{
+    const int64_t tiles = (M + 31) / 32, steps = (K + NT_STEP - 1) / NT_STEP, cus = device_cus();
+    if (tiles >= cus) return 1;
+    int64_t sl = (2 * cus + tiles - 1) / tiles;
+    if (sl > steps / 4) sl = steps / 4;
+    if (sl * tiles > (int64_t)kDeferredPartials) sl = (int64_t)kDeferredPartials / tiles;
+    if (sl > 16) sl = 16;
+    while (sl > 1 && (size_t)(sl * M * R * 4) > workspace_bytes) --sl;
+    return sl < 1 ? 1 : (int)sl;
+}
+
+size_t lowrank_nt_workspace_bytes(int64_t M, int64_t R, int64_t K)
+{
+    if (M <= 0 || R <= 0 || K <= 0) return 0;
+    const int sl = nt_slices(M, K, (size_t)-1, R);
+    return sl > 1 ? (size_t)sl * M * R * 4 : 0;
+}
+
+// qmode < 0: the product alone.  qmode = METIS_MODE_P32 / _PB16: x (contiguous rows, ldx == K) is quantized on the way,
+// codes and the deferred data (partial maxima, parked block maxima) as quantize_row_deferred leaves them.
 int lowrank_nt(const void* x, int64_t ldx, const void* v, int64_t M, int64_t R, int64_t K, const void* s, void* xv, void* t,
-               hipStream_t st)
+               hipStream_t st, void* workspace, size_t workspace_bytes, int qmode, void* codes, void* deferred, size_t deferred_size)
 {
     if (M < 0 || R <= 0 || K <= 0 || ldx < K) return METIS_E_ARG;
     if ((R != 32 && R != 64 && R != 128) || K % 64 || ldx % 8) return METIS_E_SHAPE;
@@ -145,14 +255,35 @@ int lowrank_nt(const void* x, int64_t ldx, const void* v, int64_t M, int64_t R, 
     if (M > INT32_MAX - 32 || K > INT32_MAX) return METIS_E_ARG;
     if (!x || !v || !xv || (t && !s)) return METIS_E_ARG;
     if (((uintptr_t)x % 16) || ((uintptr_t)v % 16) || ((uintptr_t)xv % 8) || ((uintptr_t)t % 8) || ((uintptr_t)s % 2)) return METIS_E_ARG;
-    const dim3 grid((unsigned)((M + 31) / 32));
-#define METIS_NT(RT) hipLaunchKernelGGL((lowrank_nt_kernel<RT>), grid, dim3(256), 0, st, (const uint16_t*)x, ldx, (const uint16_t*)v, \
-                                        (const uint16_t*)s, (uint16_t*)xv, (uint16_t*)t, (int)M, (int)K)
-    if (R == 32) METIS_NT(1);
-    else if (R == 64) METIS_NT(2);
-    else METIS_NT(4);
+    if (workspace && ((uintptr_t)workspace % 16)) return METIS_E_WORKSPACE;
+    Workspace q = {nullptr, nullptr, nullptr};
+    if (qmode >= 0) {
+        if (qmode != METIS_MODE_P32 && qmode != METIS_MODE_PB16) return METIS_E_ARG;
+        if (ldx != K || !codes || ((uintptr_t)codes % 8)) return METIS_E_ARG;
+        if ((M + 31) / 32 > (int64_t)kDeferredPartials) return METIS_E_TOO_LARGE;
+        if (M * K / kBlock >= (int64_t)1 << 31) return METIS_E_ARG;
+        if (const int rc = carve_deferred(deferred, deferred_size, M, K, &q)) return rc;
+    }
+    const int slices = workspace ? nt_slices(M, K, workspace_bytes, R) : 1;
+    float* part = slices > 1 ? static_cast<float*>(workspace) : nullptr;
+    const dim3 grid((unsigned)((M + 31) / 32), (unsigned)slices);
+#define METIS_NT(RT, Q) hipLaunchKernelGGL((lowrank_nt_kernel<RT, Q>), grid, dim3(256), 0, st, (const uint16_t*)x, ldx, (const uint16_t*)v, \
+                                           (const uint16_t*)s, (uint16_t*)xv, (uint16_t*)t, (int)M, (int)K, part, (uint2*)codes, q.amax, \
+                                           q.gmax, (uint32_t)kDeferredPartials)
+#define METIS_NTQ(RT) do { if (qmode < 0) METIS_NT(RT, -1); else if (qmode == 0) METIS_NT(RT, 0); else METIS_NT(RT, 1); } while (0)
+    if (R == 32) METIS_NTQ(1);
+    else if (R == 64) METIS_NTQ(2);
+    else METIS_NTQ(4);
+#undef METIS_NTQ
 #undef METIS_NT
-    return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
+    if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
+    if (slices > 1) {
+        const int64_t MR = M * R;
+        hipLaunchKernelGGL(lowrank_nt_finish_kernel, dim3((unsigned)((MR / 4 + 255) / 256)), dim3(256), 0, st, part, slices, MR, (int)R,
+                           (const uint16_t*)s, (uint16_t*)xv, (uint16_t*)t);
+        if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
+    }
+    return METIS_OK;
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -130,8 +130,11 @@ int lowrank_small(const void* x, int64_t ldx, const void* v, int64_t M, int64_t 
                   void* workspace, size_t workspace_bytes, hipStream_t st);
 
 // rank-r products at training sizes (bf16, MFMA, one pass over the tall operand); lowrank_large.hip
+// workspace (optional): K slices for more workgroups; qmode >= 0: x is quantized in the same pass (deferred scale bytes)
 int lowrank_nt(const void* x, int64_t ldx, const void* v, int64_t M, int64_t R, int64_t K, const void* s, void* xv, void* t,
-               hipStream_t st);
+               hipStream_t st, void* workspace = nullptr, size_t workspace_bytes = 0, int qmode = -1, void* codes = nullptr,
+               void* deferred = nullptr, size_t deferred_size = 0);
+size_t lowrank_nt_workspace_bytes(int64_t M, int64_t R, int64_t K);
 size_t lowrank_tn_workspace_bytes(int64_t L, int64_t C, int64_t R);
 int lowrank_tn(const void* a, int64_t lda, const void* b, int64_t L, int64_t C, int64_t R, void* out, int out_dtype, int transpose,
                void* workspace, size_t workspace_bytes, hipStream_t st);

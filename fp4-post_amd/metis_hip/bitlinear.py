@@ -647,13 +647,13 @@ class _MetisFusedFunction(torch.autograd.Function):
     """y = ((x V^T) * s) U^T + deq(Q(x)) deq(Q(R))^T + b in one GEMM launch, with its gradients."""
 
     @staticmethod
-    def forward(ctx, x, v, s, u, res, bias, px, p_res):
+    def forward(ctx, x, v, s, u, res, bias, px, p_res, xv=None, t=None):
         F = LinearLowbitFunction
         cd = torch.bfloat16
-        x2 = _flat2d(x).to(cd)
-        # [L, r] rank-r projection and its product with s (bf16) on the library's kernels (split-K below 256 rows,
-        # one pass over x from there on)
-        xv, t = ops.lowrank_project(x2, v.to(cd), s.to(cd))
+        if xv is None:
+            # [L, r] rank-r projection and its product with s (bf16) on the library's kernels (split-K below 256 rows,
+            # one pass over x from there on); the caller has it already when the quantizer's pass produced it
+            xv, t = ops.lowrank_project(_flat2d(x).to(cd), v.to(cd), s.to(cd))
         out_dtype = torch.float32 if F.compute_dtype == torch.float32 else torch.bfloat16
         ctx.center = None
         # binary32 arithmetic keeps a binary32 bias (as LinearLowbit and the centred path do); bf16 arithmetic adds it in bf16
@@ -748,7 +748,7 @@ class _MetisFusedFunction(torch.autograd.Function):
             g_res = torch.matmul(dyq.T, xq).to(torch.float32)
         g_b = _token_sum(dy2, torch.float32) if ctx.has_bias else None
         return (gx.reshape(x.shape).to(x.dtype), g_v.to(v.dtype), g_s.to(s.dtype), g_u.to(u.dtype),
-                g_res, g_b, None, None)
+                g_res, g_b, None, None, None, None)
 
 
 class BitLinear(nn.Module):
@@ -916,6 +916,23 @@ class BitLinear(nn.Module):
         return (self.is_svd_quant and isinstance(self.vlinear, LinearLowbit) and isinstance(self.warmup_linear, LinearLowbit)
                 and r > 0 and r % 32 == 0 and self.ulinear.bias is None and not BitLinear.quantized_lowrank_branch)
 
+    def _quantize_and_project(self, x: torch.Tensor):
+        """(packed activation, x V^T, bf16((x V^T) s)) from one pass over an activation that no sibling shares (direct
+        mode, round to nearest, bf16 tensor of 256 rows or more), or None: both branches of the layer read x, the
+        residual branch through the quantizer and the rank-r branch as it is."""
+        F = LinearLowbitFunction
+        if (F.enable_activation_svd or F.enable_nv_recipe or F.q_forward_input is not Cast2NVFp4e2m1BlockNOSR
+                or not x.is_cuda or x.dtype != torch.bfloat16 or F.compute_dtype not in (torch.float32, torch.bfloat16)):
+            return None
+        x2 = _flat2d(x)
+        v = self.vlinear.weight
+        if v.dtype != torch.bfloat16 or self._packed_residual() is None:
+            return None
+        mode = ops.MODE_P32 if F.compute_dtype == torch.float32 else ops.MODE_PB16
+        if not ops.quantize_project_applies(x2, v, mode):
+            return None
+        return ops.quantize_project(x2, v.detach(), self.s.detach(), mode)
+
     def _forward_group(self, x: torch.Tensor, shared_input):
         """All members of this layer's projection group on the shared activation in one call (no autograd):
         {id(member): output}, or None when the group does not qualify.  The siblings pick their result up when they
@@ -995,16 +1012,18 @@ class BitLinear(nn.Module):
         share_activation = (isinstance(self.vlinear, LinearLowbit) and isinstance(self.warmup_linear, LinearLowbit)
                             and self.args.forward_svd_rank > 0)
         if share_activation:
-            shared_input = self._get_shared_quantized_input(x)
             r = self.args.forward_svd_rank
+            fused = self._quantize_and_project(x) if (group is None and self._fusable()) else None
+            shared_input = fused[0] if fused is not None else self._get_shared_quantized_input(x)
             if (isinstance(shared_input, (PackedNVFP4, CenteredNVFP4)) and r % 32 == 0 and self.ulinear.bias is None
                     and not BitLinear.quantized_lowrank_branch):
                 # one fused launch for both branches; it already is the "merged" evaluation, so the
                 # rollout switch changes nothing on this path
                 p_res = self._packed_residual()
                 if p_res is not None:
+                    more = () if fused is None else fused[1:]
                     return _MetisFusedFunction.apply(x, self.vlinear.weight, self.s, self.ulinear.weight,
-                                                     self.warmup_linear.weight, self.warmup_linear.bias, shared_input, p_res)
+                                                     self.warmup_linear.weight, self.warmup_linear.bias, shared_input, p_res, *more)
             if BitLinear.rollout_merge_active and not torch.is_grad_enabled():
                 return self._rollout_forward(shared_input, x.shape)
             y = self.vlinear(x, quantized_input=shared_input)

@@ -789,15 +789,52 @@ def lowrank_project(x2: torch.Tensor, v: torch.Tensor, s: torch.Tensor | None = 
     t = None if s is None else torch.empty_like(xv)
     sp = None if s is None else s.contiguous().data_ptr()
     if large:
-        rc = L.metis_lowrank_project_rows(x2.data_ptr(), x2.stride(0), v.data_ptr(), M, R, K, sp, xv.data_ptr(),
-                                          None if t is None else t.data_ptr(), _stream())
-        check(rc, "metis_lowrank_project_rows", (M, R, K))
+        need = L.metis_lowrank_project_rows_workspace_bytes(M, R, K)
+        ws = torch.empty(need, dtype=torch.uint8, device=x2.device) if need else None
+        rc = L.metis_lowrank_project_rows_ws(x2.data_ptr(), x2.stride(0), v.data_ptr(), M, R, K, sp, xv.data_ptr(),
+                                             None if t is None else t.data_ptr(), None if ws is None else ws.data_ptr(), need, _stream())
+        check(rc, "metis_lowrank_project_rows_ws", (M, R, K))
         return xv if s is None else (xv, t)
     ws = torch.empty(_lowrank_workspace_bytes(M, R, K), dtype=torch.uint8, device=x2.device)
     rc = L.metis_lowrank_project(x2.data_ptr(), x2.stride(0), v.data_ptr(), M, R, K, sp,
                                  xv.data_ptr(), None if t is None else t.data_ptr(), ws.data_ptr(), ws.numel(), _stream())
     check(rc, "metis_lowrank_project", (M, R, K))
     return xv if s is None else (xv, t)
+
+
+def quantize_project_applies(x2: torch.Tensor, v: torch.Tensor, mode: int) -> bool:
+    """quantize_project takes this activation: a contiguous bf16 [M, K] from 256 to 65536 rows, K a multiple of 64, a bf16
+    V of 32, 64 or 128 rows."""
+    M, K = x2.shape
+    return (x2.is_cuda and x2.dtype == torch.bfloat16 and v.dtype == torch.bfloat16 and 256 <= M <= 65536 and K % 64 == 0
+            and v.shape[0] in (32, 64, 128) and v.shape[1] == K and x2.is_contiguous() and x2.data_ptr() % 16 == 0
+            and mode in (MODE_P32, MODE_PB16))
+
+
+def quantize_project(x2: torch.Tensor, v: torch.Tensor, s: torch.Tensor, mode: int = MODE_P32):
+    """(quantize(x2, mode, deferred=True), xv, t) from ONE pass over the activation: the packed tensor that feeds the
+    residual branch and the rank-r projection xv = x2 . v^T, t = bf16(xv * s) of the low-rank branch (lowrank_project).
+    The packed tensor has the bytes of quantize(); xv is the K-sliced sum of lowrank_project."""
+    if not quantize_project_applies(x2, v, mode):
+        raise ValueError("quantize_project: shape or dtype outside the kernel's domain (see quantize_project_applies)")
+    M, K = x2.shape
+    R = v.shape[0]
+    dev = x2.device
+    L = load()
+    v = v.contiguous()
+    s = s.to(torch.bfloat16).contiguous()
+    xv = torch.empty(M, R, dtype=torch.bfloat16, device=dev)
+    t = torch.empty_like(xv)
+    codes = torch.empty(M, K // 2, dtype=torch.uint8, device=dev)
+    unit = torch.empty(1, dtype=torch.float32, device=dev)
+    parked = torch.empty(L.metis_nvfp4_deferred_bytes(M, K), dtype=torch.uint8, device=dev)
+    need = L.metis_lowrank_project_rows_workspace_bytes(M, R, K)
+    ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
+    rc = L.metis_nvfp4_quant_project_deferred(x2.data_ptr(), M, K, mode, v.data_ptr(), R, s.data_ptr(), xv.data_ptr(), t.data_ptr(),
+                                              codes.data_ptr(), parked.data_ptr(), parked.numel(),
+                                              None if ws is None else ws.data_ptr(), need, _stream())
+    check(rc, "metis_nvfp4_quant_project_deferred", (M, K, R))
+    return PackedNVFP4(codes, None, unit, M, K, mode, deferred=parked), xv, t
 
 
 def lowrank_contract_tokens(a: torch.Tensor, b: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,

@@ -445,6 +445,34 @@ int metis_lowrank_project_rows(const void *x, int64_t ldx, const void *v, int64_
                                const void *s, void *xv, void *t, void *stream);
 
 /*
+ * metis_lowrank_project_rows with K slices: a tensor of a few thousand rows gives one workgroup of 32 rows per compute
+ * unit, too few bytes in flight; with a workspace several workgroups share a row tile, each over its own range of K,
+ * and a second small launch adds their binary32 partial sums in slice order (deterministic; the sums are grouped
+ * differently from the one-slice call, so the last bit of xv may differ from it).
+ *   workspace  metis_lowrank_project_rows_workspace_bytes(M, R, K) bytes (0: one slice is enough), 16-byte aligned;
+ *              NULL or a smaller buffer: fewer slices, down to the call above
+ */
+size_t metis_lowrank_project_rows_workspace_bytes(int64_t M, int64_t R, int64_t K);
+int metis_lowrank_project_rows_ws(const void *x, int64_t ldx, const void *v, int64_t M, int64_t R, int64_t K,
+                                  const void *s, void *xv, void *t, void *workspace, size_t workspace_bytes,
+                                  void *stream);
+
+/*
+ * Both things BitLinear.forward does with its activation, in one pass over it: the NVFP4 quantization that feeds the
+ * residual branch (src/Metis/Metis/bitlinear.py:566-576 via quant.py:6-36) and the rank-r projection of the low-rank
+ * branch (bitlinear.py:752-756).  Results: xv / t as metis_lowrank_project_rows_ws, codes / deferred as
+ * metis_nvfp4_quant_row_deferred (same bytes), i.e. round to nearest, rows, scale bytes left to the consumer
+ * (metis_nvfp4_expand_tiled_deferred, metis_nvfp4_deferred_scales).
+ *   x  bf16 [rows, cols] contiguous, 16-byte aligned; cols % 64 == 0; R in {32, 64, 128}; rows <= 65536
+ *      (METIS_E_TOO_LARGE beyond: call the two functions separately)
+ *   mode  METIS_MODE_P32 or METIS_MODE_PB16 (arithmetic of the quantizer; the projection is bf16 x bf16 -> binary32)
+ */
+int metis_nvfp4_quant_project_deferred(const void *x, int64_t rows, int64_t cols, int mode, const void *v,
+                                       int64_t R, const void *s, void *xv, void *t, void *codes,
+                                       void *deferred, size_t deferred_bytes, void *workspace,
+                                       size_t workspace_bytes, void *stream);
+
+/*
  * The rank-r products of the backward pass that contract over tokens:
  *     out[C, R] = sum_l a[l, C] * b[l, R]        bf16 operands, binary32 accumulation
  * a = dY [L, N], b = (x V^T) * s  ->  gradient of U [N, r];   a = x [L, K], b = (dY U) * s, transpose = 1  ->

@@ -558,11 +558,13 @@ def test_grouped_members_read_column_slices_of_a_stacked_projection():
         assert torch.equal(y, ops.linear_fwd(px, pw, t=t.contiguous(), u=u, out_dtype=torch.float32))
 
 
-@pytest.mark.parametrize("M,R,K", [(300, 32, 512), (4096, 64, 4096), (1000, 128, 1536), (8192, 64, 3584)])
+@pytest.mark.parametrize("M,R,K", [(300, 32, 512), (4096, 64, 4096), (1000, 128, 1536), (8192, 64, 3584), (1024, 64, 18944),
+                                   (2048, 32, 4096), (260, 128, 2112)])
 def test_rank_r_projection_at_training_sizes(M, R, K):
     """xv = x V^T and t = bf16(xv * s) for 256 rows and more (one pass over x, MFMA): binary32 accumulation rounded once to
     bf16, against double precision rounded the same way (only results on a rounding boundary can differ), and t exactly
-    the bf16 product of the kernel's own xv with s."""
+    the bf16 product of the kernel's own xv with s.  Few rows against a long contraction run as K slices whose partial
+    sums a second launch adds (the last three shapes: 16, 4 and 2 slices on a 256-CU device)."""
     from metis_hip import ops
     g = torch.Generator().manual_seed(6000 + M)
     x = synthetic_activation(80 + M, M, K).cuda()
@@ -599,3 +601,59 @@ def test_rank_r_products_that_contract_over_tokens(L, C, R):
     assert rel_fro(got.cpu(), want.cpu()) <= 1e-5
     assert torch.equal(got, again)                              # fixed summation order
     assert torch.equal(got_t, got.bfloat16().T)
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("M,R,K", [(256, 32, 64), (300, 64, 192), (1024, 64, 4096), (4100, 128, 1536), (8192, 64, 4096)])
+def test_quantizer_and_rank_r_projection_in_one_pass(M, R, K, mode):
+    """metis_nvfp4_quant_project_deferred: the packed activation has the bytes of the quantizer (codes, parked block maxima,
+    and the scale bytes and unit formed from them), the projection is that of the projection call; ragged rows, a short
+    last step of K, K slices (1024 rows), every rank the kernel takes, both arithmetics."""
+    from metis_hip import ops
+    g = torch.Generator().manual_seed(9000 + M + mode)
+    x = synthetic_activation(90 + M, M, K).cuda()
+    v = (torch.randn(R, K, generator=g) / K ** 0.5).bfloat16().cuda()
+    s = (torch.rand(R, generator=g) * 4 + 0.1).bfloat16().cuda()
+    assert ops.quantize_project_applies(x, v, mode)
+    p, xv, t = ops.quantize_project(x, v, s, mode)
+    want = ops.quantize(x, mode)
+    lazy = ops.quantize(x, mode, deferred=True)
+    xv0, t0 = ops.lowrank_project(x, v, s)
+    torch.cuda.synchronize()
+    nb = M * K // 16
+    assert torch.equal(p.codes, want.codes)
+    assert torch.equal(p.deferred[8192:8192 + 2 * nb], lazy.deferred[8192:8192 + 2 * nb])       # parked bf16 block maxima
+    assert torch.equal(p.scales, want.scales) and torch.equal(p.unit, want.unit)
+    assert torch.equal(xv, xv0) and torch.equal(t, t0)
+    assert rel_fro(xv.float().cpu(), (x.double() @ v.double().T).cpu()) <= 3e-3
+    # the consumer of the parked data: the tiled expansion forms the same operand from either packing
+    if K % 32 == 0:
+        fresh = ops.quantize_project(x, v, s, mode)[0]
+        assert torch.equal(ops.expand_tiled(fresh, cache=False, mode=mode), ops.expand_tiled(want, cache=False, mode=mode))
+
+
+def test_quantizer_and_projection_argument_checks():
+    from metis_hip import _lib, ops
+    L = _lib.load()
+    x = torch.zeros(256, 64, dtype=torch.bfloat16, device="cuda")
+    v = torch.zeros(32, 64, dtype=torch.bfloat16, device="cuda")
+    s = torch.zeros(32, dtype=torch.bfloat16, device="cuda")
+    out = torch.zeros(256, 32, dtype=torch.bfloat16, device="cuda")
+    codes = torch.zeros(256, 32, dtype=torch.uint8, device="cuda")
+    parked = torch.zeros(L.metis_nvfp4_deferred_bytes(256, 64), dtype=torch.uint8, device="cuda")
+
+    def call(rows=256, cols=64, mode=0, R=32, parked_bytes=None, xp=None):
+        return L.metis_nvfp4_quant_project_deferred(x.data_ptr() if xp is None else xp, rows, cols, mode, v.data_ptr(), R, s.data_ptr(),
+                                                    out.data_ptr(), out.data_ptr(), codes.data_ptr(), parked.data_ptr(),
+                                                    parked.numel() if parked_bytes is None else parked_bytes, None, 0, None)
+
+    assert call() == 0
+    assert call(rows=0) == 0
+    assert call(mode=2) == _lib.E_ARG                               # binary32 input has no fused form
+    assert call(R=48) == _lib.E_SHAPE and call(cols=48) == _lib.E_SHAPE
+    assert call(rows=70000) == _lib.E_TOO_LARGE                     # more row tiles than partial maxima: call the two functions
+    assert call(parked_bytes=1024) == _lib.E_WORKSPACE
+    assert call(xp=x.data_ptr() + 2) == _lib.E_ARG
+    assert not ops.quantize_project_applies(x[:, :32], v[:, :32], 0)       # a strided view
+    assert not ops.quantize_project_applies(x[:128], v, 0)                 # decode-sized batches have their own kernels
+    torch.cuda.synchronize()

@@ -700,3 +700,46 @@ def test_projection_groups_run_as_one_launch_without_autograd(mean_mode, monkeyp
     calls.update(grouped=0, plain=0)
     out = holder["layer"](x.clone().requires_grad_(True), position_embeddings=pe, attention_mask=None, position_ids=pos)
     assert calls["grouped"] == 0
+
+
+@pytest.mark.parametrize("compute", [torch.bfloat16, torch.float32])
+def test_an_unshared_activation_is_quantized_and_projected_in_one_pass(compute, monkeypatch):
+    """A BitLinear whose activation no sibling shares (o_proj, down_proj) quantizes it and forms x V^T in one kernel from
+    256 rows on: same output and gradients as with the two separate passes, bit for bit in the forward (the packed
+    activation and the projection are the same bytes)."""
+    from metis_hip import BitLinear, ops
+    layer, _ = _make_bitlinear(512, 384, 64, True, torch.bfloat16, compute, seed=41)
+    x = synthetic_activation(77, 512, 512).reshape(4, 128, 512).cuda()
+    calls = {"n": 0}
+    orig = ops.quantize_project
+
+    def counting(*a, **k):
+        calls["n"] += 1
+        return orig(*a, **k)
+
+    monkeypatch.setattr(ops, "quantize_project", counting)
+
+    def run():
+        xi = x.clone().requires_grad_(True)
+        for p_ in layer.parameters():
+            p_.grad = None
+        from metis_hip.quant import _NVFP4Base
+        _NVFP4Base.sr_offset = 0                                      # the same stochastic draws in both runs
+        y = layer(xi)
+        y.backward(torch.ones_like(y) * 1e-2)
+        return y.detach(), xi.grad, layer.vlinear.weight.grad.clone(), layer.warmup_linear.weight.grad.clone()
+
+    fused = run()
+    assert calls["n"] == 1
+    monkeypatch.setattr(BitLinear, "_quantize_and_project", lambda self, x_: None)
+    plain = run()
+    assert calls["n"] == 1
+    torch.cuda.synchronize()
+    for a, b in zip(fused, plain):
+        assert torch.equal(a, b)
+    # fewer than 256 rows: the decode-sized kernels, no fused pass
+    monkeypatch.undo()
+    monkeypatch.setattr(ops, "quantize_project", counting)
+    with torch.no_grad():
+        layer(x[:1])
+    assert calls["n"] == 1
