@@ -35,15 +35,20 @@ constexpr int NT_STRIDE = NT_STEP + 8;           // halves per staged row: 528 b
 // of steps; their binary32 partial sums go to a caller workspace ([slice][row][R]) and lowrank_nt_finish_kernel adds
 // them in slice order.  One slice: the result is written directly.
 //
-// QMODE >= 0: the same pass also quantizes x (round to nearest, rows; METIS_MODE_P32 or _PB16 arithmetic): the thread that
-// fetched a block of 16 encodes it while it stages it -- E2M1 codes, the block maximum parked as bf16, one partial
-// tensor maximum per workgroup: what quant_codes_contig_kernel leaves for a consumer that forms the scale bytes itself.
-template <int RT, int QMODE = -1>                // R / 32 column tiles: 1, 2 or 4
-__global__ __launch_bounds__(256) void lowrank_nt_kernel(const uint16_t* __restrict__ x, int64_t ldx, const uint16_t* __restrict__ v,
-                                                         const uint16_t* __restrict__ s, uint16_t* __restrict__ xv,
-                                                         uint16_t* __restrict__ t, int M, int K, float* __restrict__ part,
-                                                         uint2* __restrict__ codes, uint16_t* __restrict__ q_amax,
-                                                         uint32_t* __restrict__ q_gmax, uint32_t fill_to)
+// QMODE >= 0: the same pass also quantizes x (round to nearest, rows; METIS_MODE_P32 or _PB16 arithmetic).  The workgroup
+// then has four more waves that take no part in the product: after the barrier that publishes a staged step they read
+// the x rows back from LDS, two blocks of 16 per thread, and encode them while the first four waves wait for the next
+// loads -- E2M1 codes, the block maximum parked as bf16, one partial tensor maximum per workgroup: what
+// quant_codes_contig_kernel leaves for a consumer that forms the scale bytes itself.  (Encoding in the loading waves
+// themselves put the encoder's ~250 vector instructions per step between their wait and their barrier.)
+// EW = false: the loading waves encode the block they fetched themselves, one step later (kept in px), after the next
+// loads are issued: 256 threads and fewer registers per workgroup, so two workgroups fit a compute unit -- the better
+// form when there are more row tiles than compute units (16384 rows: 41 against 46 us; 8192 rows: 38 against 30 us).
+template <int RT, int QMODE = -1, bool EW = false>  // R / 32 column tiles: 1, 2 or 4
+__global__ __launch_bounds__((QMODE >= 0 && EW) ? 512 : 256) void lowrank_nt_kernel(
+    const uint16_t* __restrict__ x, int64_t ldx, const uint16_t* __restrict__ v, const uint16_t* __restrict__ s,
+    uint16_t* __restrict__ xv, uint16_t* __restrict__ t, int M, int K, float* __restrict__ part, uint2* __restrict__ codes,
+    uint16_t* __restrict__ q_amax, uint32_t* __restrict__ q_gmax, uint32_t fill_to)
 {
     constexpr int R = RT * 32;
     constexpr int TILE_BYTES = (32 + R) * NT_STRIDE * 2;        // one staged step: x rows, then v rows
@@ -54,6 +59,50 @@ __global__ __launch_bounds__(256) void lowrank_nt_kernel(const uint16_t* __restr
     float* red = reinterpret_cast<float*>(lds);                 // [wave][j][e][lane]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int m0 = blockIdx.x * 32;
+    const int steps_all = (K + NT_STEP - 1) / NT_STEP;          // K % 64 == 0; a short last step is padded with zeros
+    const int per = (steps_all + (int)gridDim.y - 1) / (int)gridDim.y;
+    const int first = (int)blockIdx.y * per, steps = max(0, min(steps_all, first + per) - first);
+    __shared__ float smax[4];
+    if constexpr (QMODE >= 0 && EW) {
+        if (tid >= 256) {                                       // the encoding waves: same barriers as the others, nothing else shared
+            const int et = tid - 256;
+            float gmax = 0.0f;
+            for (int st = 0; st < steps; ++st) {
+                __syncthreads();                                // the step is staged
+                uint4 b[2][2];
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    const int id = i * 256 + et, row = id >> 4, blk = id & 15;
+                    b[i][0] = *reinterpret_cast<const uint4*>(tile + row * NT_STRIDE + blk * 16);
+                    b[i][1] = *reinterpret_cast<const uint4*>(tile + row * NT_STRIDE + blk * 16 + 8);
+                }
+                __syncthreads();                                // the tile may be overwritten: the blocks are in registers
+                const int k0 = (first + st) * NT_STEP;
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    const int id = i * 256 + et, row = id >> 4, k = k0 + (id & 15) * 16;
+                    if (m0 + row < M && k < K) {
+                        float val[kBlock];
+                        const float none[kBlock] = {};
+                        unpack16(b[i][0], b[i][1], val);
+                        const float am = block_amax(val);
+                        gmax = fmaxf(gmax, am);
+                        const int64_t ib = (int64_t)(m0 + row) * (K / kBlock) + k / kBlock;
+                        q_amax[ib] = (uint16_t)(__float_as_uint(am) >> 16);
+                        codes[ib] = encode_block<QMODE < 0 ? 0 : QMODE, false>(val, block_scalar<QMODE < 0 ? 0 : QMODE>(am), none);
+                    }
+                }
+            }
+            // one partial maximum per workgroup, indexed over the whole grid; unused entries cleared for the folding reader
+            const float wm = wave_max(gmax);
+            if (lane == 0) smax[wave - 4] = wm;
+            __syncthreads();                                    // the barrier the other waves pass after parking their sums
+            const uint32_t gid = blockIdx.y * gridDim.x + blockIdx.x, gsize = gridDim.x * gridDim.y;
+            if (et == 0) q_gmax[gid] = __float_as_uint(fmaxf(fmaxf(smax[0], smax[1]), fmaxf(smax[2], smax[3])));
+            for (uint32_t j = gsize + gid * 256u + et; j < fill_to; j += gsize * 256u) q_gmax[j] = 0u;
+            return;
+        }
+    }
     // staging: a thread fetches two blocks of 16 of x per step (32 contiguous bytes each; 16 threads cover the 512
     // bytes of a row) and 4 RT 16-byte chunks of v (a wave covers two rows x 512 contiguous bytes per load).
     // It keeps two whole steps in registers while the one before them is multiplied: that is what keeps bytes in flight.
@@ -73,9 +122,7 @@ __global__ __launch_bounds__(256) void lowrank_nt_kernel(const uint16_t* __restr
         }
     };
     float gmax = 0.0f;
-    // QMODE >= 0: the step just staged stays in px and is encoded after the next loads have been issued and the MFMAs
-    // queued, so the encoder's vector arithmetic runs while the memory system works, not between a wait and a barrier
-    uint4 px[QMODE >= 0 ? 4 : 1];
+    uint4 px[(QMODE >= 0 && !EW) ? 4 : 1];
     auto stage = [&](const uint4 (&qx)[4], const uint4 (&qv)[RT * 4]) {
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
@@ -83,7 +130,7 @@ __global__ __launch_bounds__(256) void lowrank_nt_kernel(const uint16_t* __restr
             *reinterpret_cast<uint4*>(tile + row * NT_STRIDE + blk * 16) = qx[2 * i];
             *reinterpret_cast<uint4*>(tile + row * NT_STRIDE + blk * 16 + 8) = qx[2 * i + 1];
         }
-        if constexpr (QMODE >= 0) {
+        if constexpr (QMODE >= 0 && !EW) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) px[i] = qx[i];
         }
@@ -94,7 +141,7 @@ __global__ __launch_bounds__(256) void lowrank_nt_kernel(const uint16_t* __restr
         }
     };
     auto encode = [&](int k0) {
-        if constexpr (QMODE >= 0) {
+        if constexpr (QMODE >= 0 && !EW) {
 #pragma unroll
             for (int i = 0; i < 2; ++i) {
                 const int id = i * 256 + tid, row = id >> 4, k = k0 + (id & 15) * 16;
@@ -117,9 +164,6 @@ __global__ __launch_bounds__(256) void lowrank_nt_kernel(const uint16_t* __restr
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[j][e] = 0.0f;
 
-    const int steps_all = (K + NT_STEP - 1) / NT_STEP;          // K % 64 == 0; a short last step is padded with zeros
-    const int per = (steps_all + (int)gridDim.y - 1) / (int)gridDim.y;
-    const int first = (int)blockIdx.y * per, steps = max(0, min(steps_all, first + per) - first);
     // wave w multiplies the quarter [64 w, 64 w + 64) of every step
     const int foff = (lane & 31) * NT_STRIDE + wave * 64 + (lane >> 5) * 8;
     auto multiply = [&]() {
@@ -152,9 +196,7 @@ __global__ __launch_bounds__(256) void lowrank_nt_kernel(const uint16_t* __restr
             __syncthreads();
         }
     }
-    if constexpr (QMODE >= 0) {
-        // one partial maximum per workgroup, indexed over the whole grid; unused entries cleared for the folding reader
-        __shared__ float smax[4];
+    if constexpr (QMODE >= 0 && !EW) {
         const float wm = wave_max(gmax);
         if (lane == 0) smax[wave] = wm;
         __syncthreads();
@@ -259,6 +301,7 @@ int lowrank_nt(const void* x, int64_t ldx, const void* v, int64_t M, int64_t R, 
     Workspace q = {nullptr, nullptr, nullptr};
     if (qmode >= 0) {
         if (qmode != METIS_MODE_P32 && qmode != METIS_MODE_PB16) return METIS_E_ARG;
+        if (R == 128) return METIS_E_SHAPE;
         if (ldx != K || !codes || ((uintptr_t)codes % 8)) return METIS_E_ARG;
         if ((M + 31) / 32 > (int64_t)kDeferredPartials) return METIS_E_TOO_LARGE;
         if (M * K / kBlock >= (int64_t)1 << 31) return METIS_E_ARG;
@@ -267,14 +310,19 @@ int lowrank_nt(const void* x, int64_t ldx, const void* v, int64_t M, int64_t R, 
     const int slices = workspace ? nt_slices(M, K, workspace_bytes, R) : 1;
     float* part = slices > 1 ? static_cast<float*>(workspace) : nullptr;
     const dim3 grid((unsigned)((M + 31) / 32), (unsigned)slices);
-#define METIS_NT(RT, Q) hipLaunchKernelGGL((lowrank_nt_kernel<RT, Q>), grid, dim3(256), 0, st, (const uint16_t*)x, ldx, (const uint16_t*)v, \
+    // encoding waves of their own when a compute unit gets one workgroup anyway
+    const bool ew = (int64_t)grid.x * grid.y <= (int64_t)device_cus();
+#define METIS_NT(RT, Q) METIS_NT2(RT, Q, false)
+#define METIS_NT2(RT, Q, E) hipLaunchKernelGGL((lowrank_nt_kernel<RT, Q, E>), grid, dim3((Q >= 0 && E) ? 512 : 256), 0, st, (const uint16_t*)x, ldx, (const uint16_t*)v, \
                                            (const uint16_t*)s, (uint16_t*)xv, (uint16_t*)t, (int)M, (int)K, part, (uint2*)codes, q.amax, \
                                            q.gmax, (uint32_t)kDeferredPartials)
-#define METIS_NTQ(RT) do { if (qmode < 0) METIS_NT(RT, -1); else if (qmode == 0) METIS_NT(RT, 0); else METIS_NT(RT, 1); } while (0)
+#define METIS_NTQ(RT) do { if (qmode < 0) METIS_NT(RT, -1); else if (qmode == 0) { if (ew) METIS_NT2(RT, 0, true); else METIS_NT(RT, 0); } \
+                           else { if (ew) METIS_NT2(RT, 1, true); else METIS_NT(RT, 1); } } while (0)
     if (R == 32) METIS_NTQ(1);
     else if (R == 64) METIS_NTQ(2);
-    else METIS_NTQ(4);
+    else METIS_NT(4, -1);                                      // R = 128 fills the register file with the product alone
 #undef METIS_NTQ
+#undef METIS_NT2
 #undef METIS_NT
     if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
     if (slices > 1) {

@@ -804,10 +804,10 @@ def lowrank_project(x2: torch.Tensor, v: torch.Tensor, s: torch.Tensor | None = 
 
 def quantize_project_applies(x2: torch.Tensor, v: torch.Tensor, mode: int) -> bool:
     """quantize_project takes this activation: a contiguous bf16 [M, K] from 256 to 65536 rows, K a multiple of 64, a bf16
-    V of 32, 64 or 128 rows."""
+    V of 32 or 64 rows."""
     M, K = x2.shape
     return (x2.is_cuda and x2.dtype == torch.bfloat16 and v.dtype == torch.bfloat16 and 256 <= M <= 65536 and K % 64 == 0
-            and v.shape[0] in (32, 64, 128) and v.shape[1] == K and x2.is_contiguous() and x2.data_ptr() % 16 == 0
+            and v.shape[0] in (32, 64) and v.shape[1] == K and x2.is_contiguous() and x2.data_ptr() % 16 == 0
             and mode in (MODE_P32, MODE_PB16))
 
 

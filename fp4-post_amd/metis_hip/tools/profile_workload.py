@@ -6,7 +6,7 @@ device-to-device copy of known size that calibrates the FETCH_SIZE / WRITE_SIZE 
     rocprofv3 --pmc WRITE_SIZE       -- python3 fp4-post_amd/metis_hip/tools/profile_workload.py
 
 `--extra` adds the other kernels of the library at representative shapes: bf16-arithmetic, stochastic-rounding,
-column-blocked and binary32-input quantizers, the skinny (decode) GEMM, the split-K GEMM with its reduction and
+column-blocked, binary32-input and two-packings-in-one-pass quantizers, the K-sliced rank-r projection, the skinny (decode) GEMM, the split-K GEMM with its reduction and
 the kernels of the mean mode.
 
     rocprofv3 --kernel-trace --stats -- python3 fp4-post_amd/metis_hip/tools/profile_workload.py --extra
@@ -49,7 +49,8 @@ def main(reps: int = 5):
         ops.rmsnorm_quantize(h, gamma, 1e-6, deferred=True)
         ops.linear_fwd(px, pw, t=t, u=u)                                # expand_xt_kernel + gemm_xt_kernel
         ops.linear_fwd(px, pw, t=t, u=u, tiled=False, split_k=False)    # gemm_nvfp4_large_kernel (expansion inside the K loop)
-        _, t_ = ops.lowrank_project(x, v, s)                            # lowrank_nt_kernel: x V^T and (x V^T) * s
+        _, t_ = ops.lowrank_project(x, v, s)                            # lowrank_nt_kernel<2, -1>: x V^T and (x V^T) * s
+        ops.quantize_project(x, v, s)                                   # lowrank_nt_kernel<2, 0>: the same pass also quantizes x
         ops.lowrank_contract_tokens(dy, t_)                             # lowrank_tn_kernel + finish: dY^T t
     torch.cuda.synchronize()
     del px, pw, y
@@ -74,6 +75,8 @@ def extra(reps: int = 5):
     w_up16 = ops.quantize((torch.randn(18944, 3584, generator=g) * 0.02).bfloat16().cuda(), 1)
     p_dec16 = ops.quantize(dec[:, :3584].contiguous(), 1)
     me16 = torch.full((3584,), 0.01, dtype=torch.bfloat16, device="cuda")
+    v_pre = (torch.randn(64, 18944, generator=g) / 130).bfloat16().cuda()
+    s_pre = torch.rand(64, generator=g).bfloat16().cuda()
     for i in range(reps):
         ops.linear_fwd_grouped(p_dec16, [(w_up16, None, None, None), (w_up16, None, None, None)], reference_rounding=True)
         ops.linear_fwd_grouped(p_dec16, [(w_up16, None, None, None), (w_up16, None, None, None)], reference_rounding=True, center=me16)
@@ -83,6 +86,9 @@ def extra(reps: int = 5):
         ops.quantize(x, 0, sr=True, col=True, seed=i)
         ops.quantize(xf, 0)                                             # binary32 input
         ops.quantize(xf, 0, sr=True, col=True, seed=i)
+        ops.quantize_both_sr(x, 0, seed=i, offset_row=0, offset_col=1 << 24)     # row and column packings of one tensor in one pass
+        ops.quantize_both_sr(xf, 0, seed=i, offset_row=0, offset_col=1 << 24)
+        ops.lowrank_project(pre, v_pre, s_pre)                          # 1024 x 18944, r 64: 16 K slices + finish
         ops.linear_fwd(p_dec_up, w_up)                                  # skinny: 64 x 18944 x 3584
         ops.linear_fwd(p_dec_down, w_down)                              # skinny: 64 x 3584 x 18944
         ops.linear_fwd(p_pre, w_down)                                   # split-K: 1024 x 3584 x 18944

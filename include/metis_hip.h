@@ -463,7 +463,7 @@ int metis_lowrank_project_rows_ws(const void *x, int64_t ldx, const void *v, int
  * branch (bitlinear.py:752-756).  Results: xv / t as metis_lowrank_project_rows_ws, codes / deferred as
  * metis_nvfp4_quant_row_deferred (same bytes), i.e. round to nearest, rows, scale bytes left to the consumer
  * (metis_nvfp4_expand_tiled_deferred, metis_nvfp4_deferred_scales).
- *   x  bf16 [rows, cols] contiguous, 16-byte aligned; cols % 64 == 0; R in {32, 64, 128}; rows <= 65536
+ *   x  bf16 [rows, cols] contiguous, 16-byte aligned; cols % 64 == 0; R in {32, 64}; rows <= 65536
  *      (METIS_E_TOO_LARGE beyond: call the two functions separately)
  *   mode  METIS_MODE_P32 or METIS_MODE_PB16 (arithmetic of the quantizer; the projection is bf16 x bf16 -> binary32)
  */
