@@ -385,6 +385,63 @@ static void check_mean_mode_decode(hipStream_t st)
     }
 }
 
+// One pass over an activation: NVFP4 codes + parked maxima (scale bytes formed afterwards) and the rank-r projection.
+static void check_quant_project(int64_t M, int64_t K, int64_t R, int mode, hipStream_t st)
+{
+    const std::vector<uint16_t> x = make_input(M, K, 7u + (unsigned)M, 1.0f), v = make_input(R, K, 8u, 0.05f), s = make_input(1, R, 9u, 1.0f);
+    DeviceBuffer<uint16_t> dx(x.size()), dv(v.size()), dsv(s.size()), dxv((size_t)(M * R)), dt((size_t)(M * R));
+    dx.upload(x); dv.upload(v); dsv.upload(s);
+    DeviceBuffer<uint8_t> dc((size_t)(M * K / 2)), dsc((size_t)(M * K / 16));
+    DeviceBuffer<float> du(1);
+    const size_t pb = metis_nvfp4_deferred_bytes(M, K), wb = metis_lowrank_project_rows_workspace_bytes(M, R, K);
+    DeviceBuffer<uint8_t> parked(pb), ws(wb + 16);
+    int rc = metis_nvfp4_quant_project_deferred(dx.p, M, K, mode, dv.p, R, dsv.p, dxv.p, dt.p, dc.p, parked.p, pb, wb ? ws.p : nullptr, wb, st);
+    if (rc == METIS_OK) rc = metis_nvfp4_deferred_scales(parked.p, M, K, mode, dsc.p, du.p, st);
+    HIP_OK(hipStreamSynchronize(st));
+    std::vector<uint8_t> wc((size_t)(M * K / 2)), wsc((size_t)(M * K / 16));
+    float wu = 0;
+    metis_oracle_nvfp4_pack(x.data(), M, K, K, mode, nullptr, wc.data(), wsc.data(), &wu, nullptr);
+    char line[200];
+    snprintf(line, sizeof line, "metis_nvfp4_quant_project_deferred %lldx%lld r=%lld mode %d rc=%d: codes, scale bytes, unit bit-equal to the oracle",
+             (long long)M, (long long)K, (long long)R, mode, rc);
+    check(rc == METIS_OK && dc.download() == wc && dsc.download() == wsc && du.download()[0] == wu, line);
+    const std::vector<uint16_t> gxv = dxv.download(), gt = dt.download();
+    std::vector<double> got((size_t)(M * R)), want((size_t)(M * R));
+    bool t_exact = true;
+    for (int64_t m = 0; m < M; ++m)
+        for (int64_t r = 0; r < R; ++r) {
+            double acc = 0;
+            for (int64_t k = 0; k < K; ++k) acc += (double)bf16_to_f32(x[(size_t)(m * K + k)]) * (double)bf16_to_f32(v[(size_t)(r * K + k)]);
+            want[(size_t)(m * R + r)] = acc;
+            got[(size_t)(m * R + r)] = bf16_to_f32(gxv[(size_t)(m * R + r)]);
+            t_exact = t_exact && gt[(size_t)(m * R + r)] == metis_oracle_f32_to_bf16(bf16_to_f32(gxv[(size_t)(m * R + r)]) * bf16_to_f32(s[(size_t)r]));
+        }
+    snprintf(line, sizeof line, "  x V^T within one bf16 rounding of the double-precision product (%.2e), t = bf16(xv * s) exactly", rel_fro(got, want));
+    check(rel_fro(got, want) <= 3e-3 && t_exact, line);
+}
+
+// Row- and column-blocked stochastic packings of one tensor from one pass: the bytes of the two separate calls.
+static void check_sr_both(int64_t rows, int64_t cols, int mode, hipStream_t st)
+{
+    const std::vector<uint16_t> x = make_input(rows, cols, 11u, 1e-3f);
+    DeviceBuffer<uint16_t> dx(x.size());
+    dx.upload(x);
+    const size_t nb = (size_t)(rows * cols / 16), wsb = metis_nvfp4_workspace_bytes(rows, cols);
+    DeviceBuffer<uint8_t> cr(nb * 8), sr(nb), cc(nb * 8), sc(nb), cr2(nb * 8), sr2(nb), cc2(nb * 8), sc2(nb), ws(2 * wsb);
+    DeviceBuffer<float> ur(1), uc(1), ur2(1), uc2(1);
+    HIP_OK(hipMemset(ws.p, 0, 2 * wsb));
+    const uint64_t seed = 0x1234567887654321ull, o_row = 17, o_col = (1ull << 35) + 3;
+    int rc = metis_nvfp4_quant_sr_both(dx.p, rows, cols, cols, mode, seed, o_row, o_col, cr.p, sr.p, ur.p, cc.p, sc.p, uc.p, ws.p, 2 * wsb, st);
+    if (rc == METIS_OK) rc = metis_nvfp4_quant_sr_row(dx.p, rows, cols, cols, mode, nullptr, seed, o_row, cr2.p, sr2.p, ur2.p, ws.p, wsb, st);
+    if (rc == METIS_OK) rc = metis_nvfp4_quant_sr_col(dx.p, rows, cols, cols, mode, nullptr, seed, o_col, cc2.p, sc2.p, uc2.p, ws.p, wsb, st);
+    HIP_OK(hipStreamSynchronize(st));
+    char line[160];
+    snprintf(line, sizeof line, "metis_nvfp4_quant_sr_both %lldx%lld mode %d rc=%d: both packings equal the separate calls", (long long)rows,
+             (long long)cols, mode, rc);
+    check(rc == METIS_OK && cr.download() == cr2.download() && sr.download() == sr2.download() && ur.download()[0] == ur2.download()[0] &&
+              cc.download() == cc2.download() && sc.download() == sc2.download() && uc.download()[0] == uc2.download()[0], line);
+}
+
 int main()
 {
     hipStream_t st;
@@ -468,6 +525,13 @@ int main()
     check_mean_mode_decode(st);
     check_decode_bf16(48, 160, 512, st);
     check_decode_bf16(64, 96, 8192, st);
+
+    // ---- 4b: one pass over an activation (quantizer + rank-r projection; K slices at 256 rows against a long K), and
+    //          both stochastic packings of a gradient
+    check_quant_project(288, 448, 32, METIS_MODE_P32, st);
+    check_quant_project(256, 4096, 64, METIS_MODE_PB16, st);
+    check_sr_both(272, 336, METIS_MODE_P32, st);
+    check_sr_both(64, 1024, METIS_MODE_PB16, st);
 
     // ---- 5: error codes
     {
