@@ -271,73 +271,89 @@ __global__ __launch_bounds__(256) void quant_codes_both_kernel(
     // complete whole 128-byte lines.  Workgroups go round the eight dies in turn, each die with an L2 of its own that
     // merges partial lines; so the workgroups of one die take a run of kBothRun neighbouring tiles at a time.
     const uint32_t span = 8u * kBothRun, padded = (tiles_total + span - 1) / span * span;
+    auto tile_of = [&](uint32_t wid) { return wid / span * span + (wid % 8u) * kBothRun + (wid / 8u) % kBothRun; };
+    // the row block of slab k of workgroup item wid: 16 consecutive values of one row, 16-byte loads; zeros beyond the tensor.
+    // The next slab's loads are issued before the current one is encoded (one slab ahead, across tiles).
+    constexpr int NQ = WIDE ? 4 : 2;
+    auto fetch = [&](uint32_t wid, uint32_t k, uint4 (&q)[NQ]) {
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) q[i] = make_uint4(0u, 0u, 0u, 0u);
+        if (wid >= padded) return;
+        const uint32_t tile = tile_of(wid);
+        if (tile >= tiles_total) return;
+        const uint32_t tr = tile / tiles_c, tc = tile - tr * tiles_c;
+        const uint32_t b = tr * kColTileBlocks + g * 4u + k, cbg = tc * 4u + cb;
+        if (b < nbc && cbg < nbpr) {
+            const int64_t at = (int64_t)(b * kBlock + rr) * ld + (int64_t)cbg * kBlock;
+            const uint4* src = WIDE ? reinterpret_cast<const uint4*>(static_cast<const float*>(xv) + at)
+                                    : reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(xv) + at);
+#pragma unroll
+            for (int i = 0; i < NQ; ++i) q[i] = src[i];
+        }
+    };
+    uint4 cur[NQ], nxt[NQ];
+    fetch(blockIdx.x, 0u, cur);
     for (uint32_t wid = blockIdx.x; wid < padded; wid += gridDim.x) {
-        const uint32_t tile = wid / span * span + (wid % 8u) * kBothRun + (wid / 8u) % kBothRun;
-        if (tile >= tiles_total) continue;
+        const uint32_t tile = tile_of(wid);
+        const bool live = tile < tiles_total;                  // the same for the whole workgroup
         const uint32_t tr = tile / tiles_c, tc = tile - tr * tiles_c;
         const uint32_t c = tc * kColTileCols + lane;
         const uint32_t cbg = tc * 4u + cb;
 #pragma unroll 1
         for (uint32_t k = 0; k < 4u; ++k) {
-            const uint32_t bl = g * 4u + k, b = tr * kColTileBlocks + bl;
-            // the row block: 16 consecutive values of one row, 16-byte loads; to this wave's slab in LDS as loaded, and
-            // back as columns.  A wave's LDS operations complete in the order issued, so no wait lies between its own
-            // writes and reads: the barriers only keep the compiler from moving them.
-            float w[kBlock] = {}, v[kBlock];
-            const bool have_row = b < nbc && cbg < nbpr;
-            if constexpr (WIDE) {
-                float4 f[4] = {};
-                if (have_row) {
-                    const float4* src = reinterpret_cast<const float4*>(static_cast<const float*>(xv) + (int64_t)(b * kBlock + rr) * ld + (int64_t)cbg * kBlock);
+            if (k < 3u) fetch(wid, k + 1u, nxt);
+            else fetch(wid + gridDim.x, 0u, nxt);
+            if (live) {
+                const uint32_t bl = g * 4u + k, b = tr * kColTileBlocks + bl;
+                // to this wave's slab in LDS as loaded, and back as columns.  A wave's LDS operations complete in the
+                // order issued, so no wait lies between its own writes and reads: the barriers only keep the compiler
+                // from moving them.
+                float w[kBlock], v[kBlock];
+                const bool have_row = b < nbc && cbg < nbpr;
+                if constexpr (WIDE) {
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) f[q] = src[q];
-                }
+                    for (int q = 0; q < 4; ++q) {
+                        w[4 * q] = __uint_as_float(cur[q].x); w[4 * q + 1] = __uint_as_float(cur[q].y);
+                        w[4 * q + 2] = __uint_as_float(cur[q].z); w[4 * q + 3] = __uint_as_float(cur[q].w);
+                        *reinterpret_cast<uint4*>(&slab[g][rr][cb * kBlock + 4 * q]) = cur[q];
+                    }
+                    __builtin_amdgcn_wave_barrier();
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    w[4 * q] = f[q].x; w[4 * q + 1] = f[q].y; w[4 * q + 2] = f[q].z; w[4 * q + 3] = f[q].w;
-                    *reinterpret_cast<float4*>(&slab[g][rr][cb * kBlock + 4 * q]) = f[q];
+                    for (int j = 0; j < kBlock; ++j) v[j] = __uint_as_float(slab[g][j][lane]);
+                } else {
+                    unpack16(cur[0], cur[1], w);
+                    *reinterpret_cast<uint4*>(&slab[g][rr][cb * 8u]) = cur[0];
+                    *reinterpret_cast<uint4*>(&slab[g][rr][cb * 8u + 4u]) = cur[1];
+                    __builtin_amdgcn_wave_barrier();
+                    const uint32_t shift = (lane & 1u) ? 0u : 16u;  // a bf16 is the upper half of its binary32 value
+#pragma unroll
+                    for (int j = 0; j < kBlock; ++j) v[j] = __uint_as_float((slab[g][j][lane >> 1] << shift) & 0xffff0000u);
                 }
                 __builtin_amdgcn_wave_barrier();
-#pragma unroll
-                for (int j = 0; j < kBlock; ++j) v[j] = __uint_as_float(slab[g][j][lane]);
-            } else {
-                uint4 lo = make_uint4(0u, 0u, 0u, 0u), hi = lo;
                 if (have_row) {
-                    const uint4* src = reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(xv) + (int64_t)(b * kBlock + rr) * ld + (int64_t)cbg * kBlock);
-                    lo = src[0];
-                    hi = src[1];
+                    const float amr = block_amax(w);
+                    gmax = fmaxf(gmax, amr);
+                    const int64_t ir = (int64_t)(b * kBlock + rr) * nbpr + cbg;
+                    uint2 pr;
+                    if constexpr (WIDE) pr = encode_sr_hardware<0, true>(w, block_scalar_ieee(amr), seed, offset_row, ir);
+                    else pr = encode_sr_hardware<MODE>(w, block_scalar<MODE>(amr), seed, offset_row, ir);
+                    codes_row[ir] = pr;
+                    amax_row[ir] = parked(amr);
                 }
-                const uint32_t u[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+                uint2 packed = make_uint2(0u, 0u);
+                float am = 0.0f;
+                if (c < cols && b < nbc) {
+                    am = block_amax(v);
+                    if constexpr (WIDE) packed = encode_sr_hardware<0, true>(v, block_scalar_ieee(am), seed, offset_col, (int64_t)c * nbc + b);
+                    else packed = encode_sr_hardware<MODE>(v, block_scalar<MODE>(am), seed, offset_col, (int64_t)c * nbc + b);
+                }
+                s_codes[lane][bl] = packed;
+                s_amax[lane][bl] = parked(am);
+            }
 #pragma unroll
-                for (int q = 0; q < 8; ++q) { w[2 * q] = bf16_lo(u[q]); w[2 * q + 1] = bf16_hi(u[q]); }
-                *reinterpret_cast<uint4*>(&slab[g][rr][cb * 8u]) = lo;
-                *reinterpret_cast<uint4*>(&slab[g][rr][cb * 8u + 4u]) = hi;
-                __builtin_amdgcn_wave_barrier();
-                const uint32_t shift = (lane & 1u) ? 0u : 16u;  // a bf16 is the upper half of its binary32 value
-#pragma unroll
-                for (int j = 0; j < kBlock; ++j) v[j] = __uint_as_float((slab[g][j][lane >> 1] << shift) & 0xffff0000u);
-            }
-            __builtin_amdgcn_wave_barrier();
-            if (have_row) {
-                const float amr = block_amax(w);
-                gmax = fmaxf(gmax, amr);
-                const int64_t ir = (int64_t)(b * kBlock + rr) * nbpr + cbg;
-                uint2 pr;
-                if constexpr (WIDE) pr = encode_sr_hardware<0, true>(w, block_scalar_ieee(amr), seed, offset_row, ir);
-                else pr = encode_sr_hardware<MODE>(w, block_scalar<MODE>(amr), seed, offset_row, ir);
-                codes_row[ir] = pr;
-                amax_row[ir] = parked(amr);
-            }
-            uint2 packed = make_uint2(0u, 0u);
-            float am = 0.0f;
-            if (c < cols && b < nbc) {
-                am = block_amax(v);
-                if constexpr (WIDE) packed = encode_sr_hardware<0, true>(v, block_scalar_ieee(am), seed, offset_col, (int64_t)c * nbc + b);
-                else packed = encode_sr_hardware<MODE>(v, block_scalar<MODE>(am), seed, offset_col, (int64_t)c * nbc + b);
-            }
-            s_codes[lane][bl] = packed;
-            s_amax[lane][bl] = parked(am);
+            for (int i = 0; i < NQ; ++i) cur[i] = nxt[i];
         }
+        if (!live) continue;
         __syncthreads();
         {   // column t / 4, blocks 4 (t % 4) .. +3 of the tile: 32 contiguous bytes of codes, 8 of maxima
             const uint32_t oc = threadIdx.x >> 2, part = threadIdx.x & 3u;
