@@ -370,6 +370,10 @@ int expand_xt_transposed(const void* codes, const void* scales, const float* uni
 // applied; PB16: the reduction kernel rounds the sum and adds the bias in bf16, as the reference's bf16 forward does.
 // ---------------------------------------------------------------------------------------------
 constexpr int XT_STAGE = 32 * 1024, XT_NS = 3;
+// Beyond the ring: the first two 32-column steps of the rank-r factors T | U of the tile (512 rows x 32 columns each, in the
+// operand tile format), requested by direct loads before the first operand stage, so that the low-rank extension at the
+// end of the tile finds them in LDS instead of waiting for two dependent memory round trips.
+constexpr int XT_LR_STEPS = 2, XT_LDS = (XT_NS + XT_LR_STEPS) * XT_STAGE;     // 160 KiB: all of a compute unit's LDS
 
 __host__ __device__ constexpr int waitcnt_imm(int vm, int lgkm)
 {
@@ -446,6 +450,26 @@ __global__ __launch_bounds__(512, 1) void gemm_xt_kernel(
         asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                      :: "v"(lane16), "s"(g), "s"(dst) : "memory");
     };
+
+    // ---- rank-r factors ahead of everything else: instruction j of wave w gathers the 16 rows x 32 columns piece
+    //      j * 8 + w of T | U (0..15 rows of T, 16..31 rows of U) for step p, every lane its 16 bytes, into the slot
+    //      order of an operand tile.  They are the oldest loads of the wave: whatever wait covers an operand stage covers them.
+    // (Kernels with split tiles keep the staged form for all steps: their register budget has no room for both.)
+    const int lr_ahead = (SPLIT == 0 && t != nullptr) ? min(r / 32, XT_LR_STEPS) : 0;
+    if constexpr (SPLIT == 0) {
+        const int q = lane >> 2, chunk = (lane & 3) ^ xt_swz(q);
+        for (int p = 0; p < lr_ahead; ++p) {
+#pragma unroll
+            for (int j = 0; j < LPW; ++j) {
+                const int ot = j * NWAVES + wave;
+                const bool is_a = ot < 16;
+                const int64_t row = is_a ? min(m0 + ot * 16 + q, M - 1) : min(n0 + (ot - 16) * 16 + q, N - 1);
+                const uint16_t* g = (is_a ? t : u) + row * r + p * 32 + chunk * 8;
+                const uint32_t dst = (uint32_t)((NS + p) * XT_STAGE + ot * 1024);
+                asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(g), "s"(dst) : "memory");
+            }
+        }
+    }
 
     // ---- fragment addressing: lane -> row lr of a 32-row MFMA tile, k half hi; chunk = 2 * ks + hi.
     // ks = 1 flips bit 1 of the chunk index, which flips bit 1 of the slot: byte offset ^ 32.
@@ -575,10 +599,28 @@ __global__ __launch_bounds__(512, 1) void gemm_xt_kernel(
         }
     }
 
-    // ---- bf16 low-rank extension, 32 columns of T / U per step, staged in rows of 144 bytes
+    // ---- bf16 low-rank extension: the steps that were requested ahead are one more operand stage each
+    if constexpr (SPLIT == 0)
+    for (int p = 0; p < lr_ahead; ++p) {
+        const int x = (NS + p) * XT_STAGE;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            bf16x8_t ga[TM], gb[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) ga[i] = *reinterpret_cast<const bf16x8_t*>(xlds + (a_off[ks] + x) + i * 2048);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) gb[j] = *reinterpret_cast<const bf16x8_t*>(xlds + (b_off[ks] + x) + j * 2048);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gb[j], ga[i], acc[i][j], 0, 0, 0);
+        }
+    }
+    // ---- further steps (r > 64): 32 columns of T / U per step, staged in rows of 144 bytes
     uint16_t* plds = reinterpret_cast<uint16_t*>(xlds);
     const int frag_off = lr * L_STRIDE + hi * 8;
-    for (int j0 = 0; j0 < r; j0 += 32) {
+    for (int j0 = lr_ahead * 32; j0 < r; j0 += 32) {
         {
             const int trow = tid;                               // 512 threads, 512 rows of the T|U tile
             const bool is_a = trow < L_BM;
@@ -710,7 +752,7 @@ static int launch_xt(const void* a_xt, const float* a_unit, const void* b_xt, co
 {
     static bool attr_set[64] = {};
     const void* fn = (const void*)gemm_xt_kernel<OUT_F32, PB16, SPLIT>;
-    const size_t lds_bytes = (size_t)XT_NS * XT_STAGE;
+    const size_t lds_bytes = (size_t)XT_LDS;
     if (const int rc = allow_dynamic_lds(fn, lds_bytes, attr_set)) return rc;
     const int tiles_m = (int)((M + L_BM - 1) / L_BM), tiles_n = (int)((N + L_BN - 1) / L_BN);
     const int total = tiles_m * tiles_n;
