@@ -563,10 +563,11 @@ def test_col_quant_large_ragged_tensors(ops, tag, mode):
 
 
 @pytest.mark.parametrize("tag,mode", MODES + [("f32", 2)])
-@pytest.mark.parametrize("shape", [(16, 16), (48, 80), (256, 64), (1008, 1552), (4096 + 48, 2048 + 16)])
+@pytest.mark.parametrize("shape", [(16, 16), (48, 80), (256, 64), (1008, 1552), (4096 + 48, 2048 + 16), (4096, 8960)])
 def test_both_packings_in_one_pass_equal_the_two_calls(ops, tag, mode, shape):
     """Row-blocked and column-blocked stochastic packings of one tensor from one kernel: the same bytes as the row call
-    and the column call with the same seed and offsets (tiles ragged in both directions, single block, one tile)."""
+    and the column call with the same seed and offsets (tiles ragged in both directions, single block, one tile, and the
+    output gradient of the config-4 projection at full size)."""
     rows, cols = shape
     g = torch.Generator().manual_seed(1234 + rows)
     x = torch.randn(rows, cols, generator=g) * torch.exp(torch.randn(rows, 1, generator=g))
