@@ -207,3 +207,44 @@ def test_rank_r_kernels_and_dense_operands_on_random_shapes(seed):
                                out_dtype=torch.bfloat16)
             ref = (qx.dequantize(torch.bfloat16).double() @ v.double().T).float().bfloat16()
             assert rel_fro(y.float().cpu(), ref.float().cpu()) <= 3e-4, what
+
+
+@pytest.mark.parametrize("seed", [51, 52])
+def test_one_pass_kernels_on_random_cases(seed):
+    """The two kernels that serve two consumers from one pass, on 40 random shapes and value ranges per seed (zeros,
+    all-zero blocks, outliers, tiny and huge magnitudes, exact ties): both stochastic packings of a tensor against the row
+    and the column call (same seed and offsets: same bytes), and the quantizer inside the rank-r projection's pass against
+    the quantizer's own kernels (same bytes) and double precision (the projection)."""
+    from metis_hip import ops
+    rng = random.Random(seed)
+    for case in range(40):
+        kind = rng.choice(["plain", "plain", "ties", "tiny", "huge"])
+        mode = rng.choice([0, 1])
+        # both packings: every shape with both dimensions multiples of 16
+        rows, cols = 16 * rng.randint(1, 40), 16 * rng.randint(1, 40)
+        x, _ = _values(rng, rows, cols, kind)
+        wide = mode == 0 and rng.random() < 0.3
+        xin = (x if wide else x.bfloat16()).cuda()
+        sd, o1, o2 = rng.randrange(1 << 62), rng.randrange(1 << 40), rng.randrange(1 << 40)
+        pr, pc = ops.quantize_both_sr(xin, mode, seed=sd, offset_row=o1, offset_col=o2)
+        wr = ops.quantize(xin, mode, sr=True, seed=sd, offset=o1)
+        wc = ops.quantize(xin, mode, col=True, sr=True, seed=sd, offset=o2)
+        torch.cuda.synchronize()
+        what = f"seed {seed} case {case}: {rows}x{cols} {kind} mode {mode} wide {wide}"
+        assert torch.equal(pr.codes, wr.codes) and torch.equal(pr.scales, wr.scales) and torch.equal(pr.unit, wr.unit), what
+        assert torch.equal(pc.codes, wc.codes) and torch.equal(pc.scales, wc.scales) and torch.equal(pc.unit, wc.unit), what
+        # quantizer + projection: 256 rows and more, K a multiple of 64, rank 32 or 64
+        M, K, R = rng.randint(256, 700), 64 * rng.randint(1, 24), rng.choice([32, 64])
+        a, g = _values(rng, M, K, kind)
+        a = a.bfloat16().cuda()
+        v = (torch.randn(R, K, generator=g) / K ** 0.5).bfloat16().cuda()
+        s = (torch.rand(R, generator=g) + 0.5).bfloat16().cuda()
+        p, xv, t = ops.quantize_project(a, v, s, mode)
+        want = ops.quantize(a, mode)
+        torch.cuda.synchronize()
+        what = f"seed {seed} case {case}: {M}x{K} r{R} {kind} mode {mode}"
+        assert torch.equal(p.codes, want.codes) and torch.equal(p.scales, want.scales) and torch.equal(p.unit, want.unit), what
+        ref = a.double() @ v.double().T
+        if kind != "huge":                                        # bf16 sums of 1e20-sized terms overflow nothing, but the bound is relative anyway
+            assert rel_fro(xv.float().cpu(), ref.cpu()) <= 4e-3, what
+        assert torch.equal(t, (xv.float() * s.float()).bfloat16()), what
