@@ -41,7 +41,7 @@ int device_cus();
 
 // phase 2 of the quantizer (tensor unit + E4M3 bytes from parked block maxima); nvfp4_quant.hip
 int launch_scales(int mode, const Workspace& ws, uint32_t ngroups, void* scales, float* unit, uint32_t nblocks,
-                  hipStream_t st);
+                  hipStream_t st, const void* amax2 = nullptr, void* scales2 = nullptr, float* unit2 = nullptr);
 
 int quantize(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, bool sr, bool col, const void* noise,
              uint64_t seed, uint64_t offset, void* codes, void* scales, float* unit, void* workspace,

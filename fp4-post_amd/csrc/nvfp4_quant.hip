@@ -382,8 +382,11 @@ template <int MODE>
 __global__ __launch_bounds__(256) void quant_scales_kernel(const uint16_t* __restrict__ ws_amax,
                                                            const uint32_t* __restrict__ ws_gmax, uint32_t ngroups,
                                                            uint8_t* __restrict__ scales, float* __restrict__ unit_out,
-                                                           uint32_t nblocks)
+                                                           uint32_t nblocks, const uint16_t* __restrict__ ws_amax2 = nullptr,
+                                                           uint8_t* __restrict__ scales2 = nullptr, float* __restrict__ unit_out2 = nullptr)
 {
+    // grid row 1 (if launched): a second packing of the same tensor (same partial maxima, its own parked block maxima)
+    if (blockIdx.y) { ws_amax = ws_amax2; scales = scales2; unit_out = unit_out2; }
     __shared__ float smax[4];
     const uint32_t nocts = nblocks / 8u;
     const uint32_t step = gridDim.x * 256u;
@@ -430,8 +433,10 @@ __global__ __launch_bounds__(256) void quant_scales_kernel(const uint16_t* __res
 __global__ __launch_bounds__(256) void quant_scales_f32_kernel(const float* __restrict__ ws_amax,
                                                                const uint32_t* __restrict__ ws_gmax, uint32_t ngroups,
                                                                uint8_t* __restrict__ scales, float* __restrict__ unit_out,
-                                                               uint32_t nblocks)
+                                                               uint32_t nblocks, const float* __restrict__ ws_amax2 = nullptr,
+                                                               uint8_t* __restrict__ scales2 = nullptr, float* __restrict__ unit_out2 = nullptr)
 {
+    if (blockIdx.y) { ws_amax = ws_amax2; scales = scales2; unit_out = unit_out2; }
     __shared__ float smax[4];
     float m = 0.0f;
     for (uint32_t g = threadIdx.x; g < ngroups; g += 256u) m = fmaxf(m, __uint_as_float(ws_gmax[g]));
@@ -733,18 +738,19 @@ static int grid_for(uint32_t work_items)
 }
 
 int launch_scales(int mode, const Workspace& ws, uint32_t ngroups, void* scales, float* unit, uint32_t nblocks,
-                  hipStream_t st)
+                  hipStream_t st, const void* amax2, void* scales2, float* unit2)
 {
     const int g2 = grid_for((nblocks + 7) / 8);
+    const dim3 grid((unsigned)g2, amax2 ? 2u : 1u);            // a second packing of the same tensor rides in grid row 1
     if (mode == METIS_MODE_P32_F32)
-        hipLaunchKernelGGL(quant_scales_f32_kernel, dim3(g2), dim3(256), 0, st, (const float*)ws.amax, ws.gmax, ngroups,
-                           (uint8_t*)scales, unit, nblocks);
+        hipLaunchKernelGGL(quant_scales_f32_kernel, grid, dim3(256), 0, st, (const float*)ws.amax, ws.gmax, ngroups,
+                           (uint8_t*)scales, unit, nblocks, (const float*)amax2, (uint8_t*)scales2, unit2);
     else if (mode == 0)
-        hipLaunchKernelGGL((quant_scales_kernel<0>), dim3(g2), dim3(256), 0, st, ws.amax, ws.gmax, ngroups,
-                           (uint8_t*)scales, unit, nblocks);
+        hipLaunchKernelGGL((quant_scales_kernel<0>), grid, dim3(256), 0, st, ws.amax, ws.gmax, ngroups,
+                           (uint8_t*)scales, unit, nblocks, (const uint16_t*)amax2, (uint8_t*)scales2, unit2);
     else
-        hipLaunchKernelGGL((quant_scales_kernel<1>), dim3(g2), dim3(256), 0, st, ws.amax, ws.gmax, ngroups,
-                           (uint8_t*)scales, unit, nblocks);
+        hipLaunchKernelGGL((quant_scales_kernel<1>), grid, dim3(256), 0, st, ws.amax, ws.gmax, ngroups,
+                           (uint8_t*)scales, unit, nblocks, (const uint16_t*)amax2, (uint8_t*)scales2, unit2);
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 
@@ -921,8 +927,7 @@ int quantize_both_sr(const void* x, int64_t rows, int64_t cols, int64_t ld, int 
 #undef METIS_QB
     if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
     const int pm = f32in ? METIS_MODE_P32_F32 : mode;
-    if (const int rc = launch_scales(pm, wr, (uint32_t)g, scales_row, unit_row, nblocks, st)) return rc;
-    return launch_scales(pm, wc, (uint32_t)g, scales_col, unit_col, nblocks, st);
+    return launch_scales(pm, wr, (uint32_t)g, scales_row, unit_row, nblocks, st, wc.amax, scales_col, unit_col);   // one launch for both
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -706,10 +706,10 @@ class _MetisFusedFunction(torch.autograd.Function):
         x2 = _flat2d(x).to(cd)
         L, N = dy2.shape
         # rank-r branch in bf16: one pass over dY for dY U, one for dY^T t, one over x for g_xv^T x
-        g_t = ops.lowrank_project(dy2, _MetisFusedFunction._transposed_bf16(u))    # [L, r]
+        # dY U [L, r] and its product with s (the gradient with respect to x V^T) from the same launch
+        g_t, g_xv = ops.lowrank_project(dy2, _MetisFusedFunction._transposed_bf16(u), s.to(cd))
         g_u = ops.lowrank_contract_tokens(dy2, t)                           # [N, r]
         g_s = (g_t * xv).sum(dim=0, dtype=torch.float32)                    # the product in bf16, as autograd forms it for torch.mul(s, y)
-        g_xv = g_t * s.to(cd)
         g_v = ops.lowrank_contract_tokens(x2, g_xv, transpose=True)         # [r, K]
         # residual branch on re-quantized operands
         qg = F.q_backward_outputgrad
