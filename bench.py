@@ -270,6 +270,36 @@ def main():
     _, nd_ms = time_region(torch, ndstep, max(args.steps, 50), args.warmup)
     nd_gbs = n_bytes / (nd_ms * 1e-3) / 1e9
 
+    # ------------------------------------------------------------------ the kernels that serve two consumers from one pass
+    # (config-3 activation: quantizer + rank-r projection; config-4 output gradient: row- and column-blocked packing),
+    # each beside the two calls it replaces
+    one_pass = None
+    try:
+        def us_of(fn, n=40, w=10):
+            for _ in range(w):
+                fn()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(n):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            return round(e0.elapsed_time(e1) / n * 1e3, 1)
+        dy4 = (torch.randn(4096, 8960, generator=torch.Generator().manual_seed(2004)) * 1e-3).bfloat16().to(dev)
+        one_pass = {
+            "quantize_and_project": {
+                "workload": "config-3 activation bf16 [8192,4096], r = 64: NVFP4 codes + parked block maxima and (x V^T) * s",
+                "two_calls_us": us_of(lambda: (ops.quantize(x, deferred=True), ops.lowrank_project(x, v, s))),
+                "one_pass_us": us_of(lambda: ops.quantize_project(x, v, s))},
+            "both_packings_of_dY": {
+                "workload": "config-4 output gradient bf16 [4096,8960]: stochastic row-blocked and column-blocked NVFP4 packing incl. scale bytes",
+                "two_calls_us": us_of(lambda: (ops.quantize(dy4, sr=True, seed=1), ops.quantize(dy4, col=True, sr=True, seed=1, offset=1 << 24))),
+                "one_pass_us": us_of(lambda: ops.quantize_both_sr(dy4, seed=1, offset_row=0, offset_col=1 << 24))}}
+        del dy4
+    except Exception as exc:  # an optional leg must not cost the headline line
+        one_pass = {"error": f"{type(exc).__name__}: {exc}"[:300]}
+
     # ------------------------------------------------------------------ config 5, decode step: the seven
     # projections of one Qwen2.5-7B decoder layer at M = 64 rows (rank 64), packed weights streamed once
     dec = None
@@ -626,6 +656,8 @@ def main():
                                                    "value": round(nd_gbs, 1), "unit": "GB/s", "us_per_call": round(nd_ms * 1e3, 2),
                                                    "frac": round(nd_gbs / HBM_PEAK_GBS, 4)}},
     }
+    if one_pass is not None:
+        line["one_pass_kernels"] = one_pass
     if dec is not None:
         line["decode_layer"] = dec
     if layer_leg is not None:
