@@ -272,9 +272,12 @@ __global__ __launch_bounds__(256) void quant_codes_both_kernel(
     // merges partial lines; so the workgroups of one die take a run of kBothRun neighbouring tiles at a time.
     const uint32_t span = 8u * kBothRun, padded = (tiles_total + span - 1) / span * span;
     auto tile_of = [&](uint32_t wid) { return wid / span * span + (wid % 8u) * kBothRun + (wid / 8u) % kBothRun; };
-    // the row block of slab k of workgroup item wid: 16 consecutive values of one row, 16-byte loads; zeros beyond the tensor.
-    // The next slab's loads are issued before the current one is encoded (one slab ahead, across tiles).
-    constexpr int NQ = WIDE ? 4 : 2;
+    // slab k of workgroup item wid, as the wave loads it: instruction i covers RPI whole rows of the slab, consecutive lanes
+    // consecutive 16-byte chunks (every instruction reads whole lines); zeros beyond the tensor.  The next slab's loads are
+    // issued before the current one is encoded (one slab ahead, across tiles).
+    constexpr int NQ = WIDE ? 4 : 2, CPR = WIDE ? 16 : 8, RPI = 64 / CPR;   // loads per lane, 16-byte chunks per slab row, rows per load
+    static_assert(NQ * RPI == kBlock, "the instructions of a wave cover the 16 rows of a slab");
+    const uint32_t lrow = lane / CPR, lch = lane % CPR;        // row within an instruction's rows, 16-byte chunk of the row
     auto fetch = [&](uint32_t wid, uint32_t k, uint4 (&q)[NQ]) {
 #pragma unroll
         for (int i = 0; i < NQ; ++i) q[i] = make_uint4(0u, 0u, 0u, 0u);
@@ -282,13 +285,15 @@ __global__ __launch_bounds__(256) void quant_codes_both_kernel(
         const uint32_t tile = tile_of(wid);
         if (tile >= tiles_total) return;
         const uint32_t tr = tile / tiles_c, tc = tile - tr * tiles_c;
-        const uint32_t b = tr * kColTileBlocks + g * 4u + k, cbg = tc * 4u + cb;
-        if (b < nbc && cbg < nbpr) {
-            const int64_t at = (int64_t)(b * kBlock + rr) * ld + (int64_t)cbg * kBlock;
-            const uint4* src = WIDE ? reinterpret_cast<const uint4*>(static_cast<const float*>(xv) + at)
-                                    : reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(xv) + at);
+        const uint32_t b = tr * kColTileBlocks + g * 4u + k;
+        const uint32_t col = tc * kColTileCols + lch * (WIDE ? 4u : 8u);
+        if (b < nbc && col < cols) {
 #pragma unroll
-            for (int i = 0; i < NQ; ++i) q[i] = src[i];
+            for (int i = 0; i < NQ; ++i) {
+                const int64_t at = (int64_t)(b * kBlock + i * RPI + lrow) * ld + col;
+                q[i] = WIDE ? *reinterpret_cast<const uint4*>(static_cast<const float*>(xv) + at)
+                            : *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(xv) + at);
+            }
         }
     };
     uint4 cur[NQ], nxt[NQ];
@@ -310,21 +315,20 @@ __global__ __launch_bounds__(256) void quant_codes_both_kernel(
                 // from moving them.
                 float w[kBlock], v[kBlock];
                 const bool have_row = b < nbc && cbg < nbpr;
+#pragma unroll
+                for (int i = 0; i < NQ; ++i) *reinterpret_cast<uint4*>(&slab[g][i * RPI + lrow][lch * 4u]) = cur[i];
+                __builtin_amdgcn_wave_barrier();
                 if constexpr (WIDE) {
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
-                        w[4 * q] = __uint_as_float(cur[q].x); w[4 * q + 1] = __uint_as_float(cur[q].y);
-                        w[4 * q + 2] = __uint_as_float(cur[q].z); w[4 * q + 3] = __uint_as_float(cur[q].w);
-                        *reinterpret_cast<uint4*>(&slab[g][rr][cb * kBlock + 4 * q]) = cur[q];
+                        const uint4 f = *reinterpret_cast<const uint4*>(&slab[g][rr][cb * kBlock + 4 * q]);
+                        w[4 * q] = __uint_as_float(f.x); w[4 * q + 1] = __uint_as_float(f.y);
+                        w[4 * q + 2] = __uint_as_float(f.z); w[4 * q + 3] = __uint_as_float(f.w);
                     }
-                    __builtin_amdgcn_wave_barrier();
 #pragma unroll
                     for (int j = 0; j < kBlock; ++j) v[j] = __uint_as_float(slab[g][j][lane]);
                 } else {
-                    unpack16(cur[0], cur[1], w);
-                    *reinterpret_cast<uint4*>(&slab[g][rr][cb * 8u]) = cur[0];
-                    *reinterpret_cast<uint4*>(&slab[g][rr][cb * 8u + 4u]) = cur[1];
-                    __builtin_amdgcn_wave_barrier();
+                    unpack16(*reinterpret_cast<const uint4*>(&slab[g][rr][cb * 8u]), *reinterpret_cast<const uint4*>(&slab[g][rr][cb * 8u + 4u]), w);
                     const uint32_t shift = (lane & 1u) ? 0u : 16u;  // a bf16 is the upper half of its binary32 value
 #pragma unroll
                     for (int j = 0; j < kBlock; ++j) v[j] = __uint_as_float((slab[g][j][lane >> 1] << shift) & 0xffff0000u);
