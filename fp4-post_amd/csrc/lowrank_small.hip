@@ -136,4 +136,48 @@ int lowrank_small(const void* x, int64_t ldx, const void* v, int64_t M, int64_t 
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Gradient of s in y = s * (x V^T): g_s[c] = sum_l bf16(g[l, c] * xv[l, c]), the product rounded to bf16 as autograd
+// forms it for torch.mul on bf16 tensors (src/Metis/Metis/bitlinear.py:755), the sum in binary32.  Two [L, R] bf16
+// tensors, a few hundred KB: one workgroup per 8 columns walks all rows (a thread takes every 256th row, 16 bytes of
+// each tensor per row), and the 256 per-thread sums of a column are added in thread order -- a fixed order, one launch.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void scale_grad_kernel(const uint16_t* __restrict__ g, const uint16_t* __restrict__ xv, int L, int R,
+                                                         float* __restrict__ out)
+{
+    __shared__ float part[256][9];
+    const int c0 = blockIdx.x * 8, tid = threadIdx.x;
+    float acc[8] = {};
+    for (int l = tid; l < L; l += 256) {
+        const uint4 a = *reinterpret_cast<const uint4*>(g + (int64_t)l * R + c0);
+        const uint4 b = *reinterpret_cast<const uint4*>(xv + (int64_t)l * R + c0);
+        const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, bw[4] = {b.x, b.y, b.z, b.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            acc[2 * j] += rb(bf16_lo(aw[j]) * bf16_lo(bw[j]));
+            acc[2 * j + 1] += rb(bf16_hi(aw[j]) * bf16_hi(bw[j]));
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) part[tid][j] = acc[j];
+    __syncthreads();
+    if (tid < 8) {
+        float sum = 0.0f;
+        for (int t = 0; t < 256; ++t) sum += part[t][tid];
+        out[c0 + tid] = sum;
+    }
+}
+
+int scale_grad(const void* g, const void* xv, int64_t L, int64_t R, float* out, hipStream_t st)
+{
+    if (L < 0 || R <= 0) return METIS_E_ARG;
+    if (R % 8) return METIS_E_SHAPE;
+    if (L > INT32_MAX || R > INT32_MAX) return METIS_E_ARG;
+    if (!out || ((uintptr_t)out % 4)) return METIS_E_ARG;
+    if (L > 0 && (!g || !xv || ((uintptr_t)g % 16) || ((uintptr_t)xv % 16))) return METIS_E_ARG;
+    hipLaunchKernelGGL(scale_grad_kernel, dim3((unsigned)(R / 8)), dim3(256), 0, st, (const uint16_t*)g, (const uint16_t*)xv, (int)L, (int)R,
+                       out);
+    return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
+}
+
 }  // namespace metis

@@ -129,6 +129,9 @@ size_t lowrank_small_workspace_bytes(int64_t M, int64_t R, int64_t K);
 int lowrank_small(const void* x, int64_t ldx, const void* v, int64_t M, int64_t R, int64_t K, const void* s, void* xv, void* t,
                   void* workspace, size_t workspace_bytes, hipStream_t st);
 
+// gradient of the rank-r scale vector: column sums of the bf16 products of two [L, R] tensors; lowrank_small.hip
+int scale_grad(const void* g, const void* xv, int64_t L, int64_t R, float* out, hipStream_t st);
+
 // rank-r products at training sizes (bf16, MFMA, one pass over the tall operand); lowrank_large.hip
 // workspace (optional): K slices for more workgroups; qmode >= 0: x is quantized in the same pass (deferred scale bytes)
 int lowrank_nt(const void* x, int64_t ldx, const void* v, int64_t M, int64_t R, int64_t K, const void* s, void* xv, void* t,

@@ -657,3 +657,25 @@ def test_quantizer_and_projection_argument_checks():
     assert not ops.quantize_project_applies(x[:, :32], v[:, :32], 0)       # a strided view
     assert not ops.quantize_project_applies(x[:128], v, 0)                 # decode-sized batches have their own kernels
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("L,R", [(4096, 32), (1000, 64), (16384, 128), (1, 8), (255, 40)])
+def test_gradient_of_the_rank_r_scale_vector(L, R):
+    """g_s = sum over tokens of the bf16 products g * xv (what autograd computes for torch.mul(s, y) on bf16 tensors) in one
+    launch: the products rounded to bf16 exactly as torch rounds them, summed in binary32 in a fixed order."""
+    from metis_hip import ops
+    g_ = torch.Generator().manual_seed(8000 + L)
+    g = torch.randn(L, R, generator=g_).bfloat16().cuda()
+    xv = (torch.randn(L, R, generator=g_) * 3).bfloat16().cuda()
+    got = ops.lowrank_scale_grad(g, xv)
+    again = ops.lowrank_scale_grad(g, xv)
+    want = (g * xv).double().sum(dim=0)                          # torch's bf16 products, summed exactly
+    torch.cuda.synchronize()
+    assert got.shape == (R,) and got.dtype == torch.float32
+    assert torch.equal(got, again)
+    scale = (g * xv).double().abs().sum(dim=0).clamp_min(1e-30)
+    assert float(((got.double() - want).abs() / scale).max()) <= 1e-6
+    # a view that the kernel does not take (strided) falls back to torch's own ops
+    wide = torch.cat((g, g), dim=1)
+    torch.testing.assert_close(ops.lowrank_scale_grad(wide[:, :R], xv), got, rtol=1e-4, atol=1e-4)
+    assert torch.equal(ops.lowrank_scale_grad(g[:0], xv[:0]), torch.zeros(R, device="cuda"))
