@@ -380,9 +380,9 @@ int metis_lowrank_project_rows(const void* x, int64_t ldx, const void* v, int64_
     return lowrank_nt(x, ldx, v, M, R, K, s, xv, t, (hipStream_t)stream);
 }
 
-int metis_lowrank_scale_grad(const void* g, const void* xv, int64_t L, int64_t R, float* out, void* stream)
+int metis_lowrank_scale_grad(const void* g, const void* xv, int64_t L, int64_t R, void* out, int out_dtype, void* stream)
 {
-    return scale_grad(g, xv, L, R, out, (hipStream_t)stream);
+    return scale_grad(g, xv, L, R, out, out_dtype, (hipStream_t)stream);
 }
 
 size_t metis_lowrank_project_rows_workspace_bytes(int64_t M, int64_t R, int64_t K) { return lowrank_nt_workspace_bytes(M, R, K); }

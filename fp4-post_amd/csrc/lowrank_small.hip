@@ -143,7 +143,7 @@ int lowrank_small(const void* x, int64_t ldx, const void* v, int64_t M, int64_t 
 // each tensor per row), and the 256 per-thread sums of a column are added in thread order -- a fixed order, one launch.
 // ---------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void scale_grad_kernel(const uint16_t* __restrict__ g, const uint16_t* __restrict__ xv, int L, int R,
-                                                         float* __restrict__ out)
+                                                         void* __restrict__ out, int out_f32)
 {
     __shared__ float part[256][9];
     const int c0 = blockIdx.x * 8, tid = threadIdx.x;
@@ -164,19 +164,20 @@ __global__ __launch_bounds__(256) void scale_grad_kernel(const uint16_t* __restr
     if (tid < 8) {
         float sum = 0.0f;
         for (int t = 0; t < 256; ++t) sum += part[t][tid];
-        out[c0 + tid] = sum;
+        if (out_f32) static_cast<float*>(out)[c0 + tid] = sum;
+        else static_cast<uint16_t*>(out)[c0 + tid] = (uint16_t)bf16_bits(sum);
     }
 }
 
-int scale_grad(const void* g, const void* xv, int64_t L, int64_t R, float* out, hipStream_t st)
+int scale_grad(const void* g, const void* xv, int64_t L, int64_t R, void* out, int out_dtype, hipStream_t st)
 {
-    if (L < 0 || R <= 0) return METIS_E_ARG;
+    if (L < 0 || R <= 0 || (out_dtype != METIS_DTYPE_BF16 && out_dtype != METIS_DTYPE_F32)) return METIS_E_ARG;
     if (R % 8) return METIS_E_SHAPE;
     if (L > INT32_MAX || R > INT32_MAX) return METIS_E_ARG;
     if (!out || ((uintptr_t)out % 4)) return METIS_E_ARG;
     if (L > 0 && (!g || !xv || ((uintptr_t)g % 16) || ((uintptr_t)xv % 16))) return METIS_E_ARG;
     hipLaunchKernelGGL(scale_grad_kernel, dim3((unsigned)(R / 8)), dim3(256), 0, st, (const uint16_t*)g, (const uint16_t*)xv, (int)L, (int)R,
-                       out);
+                       out, (int)(out_dtype == METIS_DTYPE_F32));
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 

@@ -130,7 +130,7 @@ int lowrank_small(const void* x, int64_t ldx, const void* v, int64_t M, int64_t 
                   void* workspace, size_t workspace_bytes, hipStream_t st);
 
 // gradient of the rank-r scale vector: column sums of the bf16 products of two [L, R] tensors; lowrank_small.hip
-int scale_grad(const void* g, const void* xv, int64_t L, int64_t R, float* out, hipStream_t st);
+int scale_grad(const void* g, const void* xv, int64_t L, int64_t R, void* out, int out_dtype, hipStream_t st);
 
 // rank-r products at training sizes (bf16, MFMA, one pass over the tall operand); lowrank_large.hip
 // workspace (optional): K slices for more workgroups; qmode >= 0: x is quantized in the same pass (deferred scale bytes)

@@ -75,7 +75,7 @@ SIGNATURES = {
     "metis_lowrank_project_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "metis_lowrank_project": (_i32, [_vp, _i64, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _sz, _vp]),
     "metis_lowrank_project_rows": (_i32, [_vp, _i64, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp]),
-    "metis_lowrank_scale_grad": (_i32, [_vp, _vp, _i64, _i64, _vp, _vp]),
+    "metis_lowrank_scale_grad": (_i32, [_vp, _vp, _i64, _i64, _vp, _i32, _vp]),
     "metis_lowrank_project_rows_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "metis_lowrank_project_rows_ws": (_i32, [_vp, _i64, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _sz, _vp]),
     "metis_nvfp4_quant_project_deferred": (_i32, [_vp, _i64, _i64, _i32, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _sz, _vp, _sz, _vp]),

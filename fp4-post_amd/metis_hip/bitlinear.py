@@ -709,7 +709,8 @@ class _MetisFusedFunction(torch.autograd.Function):
         # dY U [L, r] and its product with s (the gradient with respect to x V^T) from the same launch
         g_t, g_xv = ops.lowrank_project(dy2, _MetisFusedFunction._transposed_bf16(u), s.to(cd))
         g_u = ops.lowrank_contract_tokens(dy2, t)                           # [N, r]
-        g_s = ops.lowrank_scale_grad(g_t, xv)                               # sum of the bf16 products, as autograd forms it for torch.mul(s, y)
+        # sum of the bf16 products, as autograd forms it for torch.mul(s, y); rounded once to the parameter's dtype
+        g_s = ops.lowrank_scale_grad(g_t, xv, out_dtype=s.dtype if s.dtype in (torch.float32, torch.bfloat16) else torch.float32)
         g_v = ops.lowrank_contract_tokens(x2, g_xv, transpose=True)         # [r, K]
         # residual branch on re-quantized operands
         qg = F.q_backward_outputgrad

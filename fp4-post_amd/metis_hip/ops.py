@@ -862,15 +862,18 @@ def lowrank_contract_tokens(a: torch.Tensor, b: torch.Tensor, out_dtype: torch.d
     return out
 
 
-def lowrank_scale_grad(g: torch.Tensor, xv: torch.Tensor) -> torch.Tensor:
-    """sum_l bf16(g[l, :] * xv[l, :]) -> float32 [R]: the gradient of s in y = s * (x V^T), as (g * xv).sum(0, dtype=float32)
-    on bf16 tensors computes it (the product rounded to bf16), in one launch and a fixed summation order."""
+def lowrank_scale_grad(g: torch.Tensor, xv: torch.Tensor, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """sum_l bf16(g[l, :] * xv[l, :]) -> [R]: the gradient of s in y = s * (x V^T), as (g * xv).sum(0, dtype=float32) on bf16
+    tensors computes it (the product rounded to bf16), in one launch and a fixed summation order; out_dtype bfloat16
+    rounds the binary32 sum once, as .to(bfloat16) would."""
     R = g.shape[-1]
     if not (g.is_cuda and g.dtype == torch.bfloat16 and xv.dtype == torch.bfloat16 and g.shape == xv.shape and g.dim() == 2
-            and R % 8 == 0 and g.is_contiguous() and xv.is_contiguous() and g.data_ptr() % 16 == 0 and xv.data_ptr() % 16 == 0):
-        return (g * xv).sum(dim=0, dtype=torch.float32)
-    out = torch.empty(R, dtype=torch.float32, device=g.device)
-    rc = load().metis_lowrank_scale_grad(g.data_ptr(), xv.data_ptr(), g.shape[0], R, out.data_ptr(), _stream())
+            and R % 8 == 0 and g.is_contiguous() and xv.is_contiguous() and g.data_ptr() % 16 == 0 and xv.data_ptr() % 16 == 0
+            and out_dtype in (torch.float32, torch.bfloat16)):
+        return (g * xv).sum(dim=0, dtype=torch.float32).to(out_dtype)
+    out = torch.empty(R, dtype=out_dtype, device=g.device)
+    rc = load().metis_lowrank_scale_grad(g.data_ptr(), xv.data_ptr(), g.shape[0], R, out.data_ptr(),
+                                         DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16, _stream())
     check(rc, "metis_lowrank_scale_grad", tuple(g.shape))
     return out
 

@@ -474,12 +474,14 @@ int metis_nvfp4_quant_project_deferred(const void *x, int64_t rows, int64_t cols
 
 /*
  * Gradient of the scale vector s of the low-rank branch, y = s * (x V^T) (src/Metis/Metis/bitlinear.py:755):
- *     out[c] = sum_l bf16(g[l, c] * xv[l, c])      g = dY U, xv = x V^T, both bf16 [L, R] contiguous, out float[R]
+ *     out[c] = sum_l bf16(g[l, c] * xv[l, c])      g = dY U, xv = x V^T, both bf16 [L, R] contiguous; out [R] of
+ *                                                  out_dtype (METIS_DTYPE_F32, or _BF16: the sum rounded once)
  * the product rounded to bf16 as autograd forms it for torch.mul on bf16 tensors, the sum in binary32 in a fixed order.
  * One launch in place of the multiply, fill, reduction and cast that torch runs.  R % 8 == 0 (METIS_E_SHAPE otherwise);
  * g and xv 16-byte aligned; L == 0 writes zeros.
  */
-int metis_lowrank_scale_grad(const void *g, const void *xv, int64_t L, int64_t R, float *out, void *stream);
+int metis_lowrank_scale_grad(const void *g, const void *xv, int64_t L, int64_t R, void *out, int out_dtype,
+                             void *stream);
 
 /*
  * The rank-r products of the backward pass that contract over tokens:

@@ -679,3 +679,4 @@ def test_gradient_of_the_rank_r_scale_vector(L, R):
     wide = torch.cat((g, g), dim=1)
     torch.testing.assert_close(ops.lowrank_scale_grad(wide[:, :R], xv), got, rtol=1e-4, atol=1e-4)
     assert torch.equal(ops.lowrank_scale_grad(g[:0], xv[:0]), torch.zeros(R, device="cuda"))
+    assert torch.equal(ops.lowrank_scale_grad(g, xv, out_dtype=torch.bfloat16), got.bfloat16())
