@@ -150,12 +150,15 @@ __global__ __launch_bounds__(256) void quant_codes_kernel(
 // column owns in the tile, instead of one scattered 8-byte and 2-byte store per lane.
 // ---------------------------------------------------------------------------------------------
 constexpr int kColTileBlocks = 16, kColTileCols = 64;
-template <int MODE, bool SR, bool WIDE = false>
+// F32IN (WIDE only): the input tensor itself is binary32; a compile-time choice, so that the sixteen loads of a block are
+// issued back to back (decided at run time, element by element, the bf16 input of a centred call took twice as long).
+template <int MODE, bool SR, bool WIDE = false, bool F32IN = false>
 __global__ __launch_bounds__(256) void quant_codes_col_kernel(
     const void* __restrict__ xv, uint32_t rows, uint32_t cols, int64_t ld, const void* __restrict__ noise,
     uint64_t seed, uint64_t offset, uint2* __restrict__ codes, void* __restrict__ ws_amax_v,
-    uint32_t* __restrict__ ws_gmax, uint32_t tiles_c, uint32_t tiles_total, int in_f32, const void* __restrict__ center)
+    uint32_t* __restrict__ ws_gmax, uint32_t tiles_c, uint32_t tiles_total, const void* __restrict__ center)
 {
+    static_assert(!F32IN || WIDE, "binary32 input implies binary32 values");
     static_assert(!WIDE || MODE == 0, "binary32 values imply binary32 arithmetic");
     using amax_t = typename std::conditional<WIDE, float, uint16_t>::type;   // parked block maximum
     const uint16_t* __restrict__ x = static_cast<const uint16_t*>(xv);
@@ -176,9 +179,10 @@ __global__ __launch_bounds__(256) void quant_codes_col_kernel(
             if (c < cols && b < nbc) {
                 float v[kBlock], u[kBlock] = {};
 #pragma unroll
-                for (int j = 0; j < kBlock; ++j)
-                    v[j] = (WIDE && in_f32) ? static_cast<const float*>(xv)[(int64_t)(b * kBlock + j) * ld + c]
-                                            : bf16_lo(x[(int64_t)(b * kBlock + j) * ld + c]);
+                for (int j = 0; j < kBlock; ++j) {
+                    if constexpr (F32IN) v[j] = static_cast<const float*>(xv)[(int64_t)(b * kBlock + j) * ld + c];
+                    else v[j] = bf16_lo(x[(int64_t)(b * kBlock + j) * ld + c]);
+                }
                 if (center) {                                  // one centre per column: the same for the whole block
                     if constexpr (MODE == 0) {
                         const float cen = static_cast<const float*>(center)[c];
@@ -812,9 +816,14 @@ static int launch_quant(const void* x, int64_t rows, int64_t cols, int64_t ld, c
         const int64_t cap = (int64_t)device_cus() * 8;
         if (g > cap) g = cap;
         if (g > kMaxGroups) g = kMaxGroups;
-        hipLaunchKernelGGL((quant_codes_col_kernel<MODE, SR, WIDE>), dim3((unsigned)g), dim3(256), 0, st, x,
-                           (uint32_t)rows, (uint32_t)cols, ld, noise, seed, offset, (uint2*)codes, (void*)ws.amax, ws.gmax, tiles_c,
-                           (uint32_t)tiles, in_f32, center);
+        if (WIDE && in_f32)
+            hipLaunchKernelGGL((quant_codes_col_kernel<MODE, SR, WIDE, WIDE>), dim3((unsigned)g), dim3(256), 0, st, x,
+                               (uint32_t)rows, (uint32_t)cols, ld, noise, seed, offset, (uint2*)codes, (void*)ws.amax, ws.gmax, tiles_c,
+                               (uint32_t)tiles, center);
+        else
+            hipLaunchKernelGGL((quant_codes_col_kernel<MODE, SR, WIDE, false>), dim3((unsigned)g), dim3(256), 0, st, x,
+                               (uint32_t)rows, (uint32_t)cols, ld, noise, seed, offset, (uint2*)codes, (void*)ws.amax, ws.gmax, tiles_c,
+                               (uint32_t)tiles, center);
         return launch_scales(WIDE ? METIS_MODE_P32_F32 : MODE, ws, (uint32_t)g, scales, unit, nblocks, st);
     } else {
         const int g1 = grid_for(nblocks);
