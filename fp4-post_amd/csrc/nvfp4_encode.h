@@ -100,9 +100,27 @@ __device__ __forceinline__ uint2 encode_rne_wide(const float (&v)[kBlock], float
     hi = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(hi, quot(14), quot(15), 1.0f, 3);
     const bool flagged = least == 0u;
     if (__builtin_amdgcn_ballot_w64(flagged) != 0ull) {        // wave-uniform: a real branch around the long sequence
-        const float none[kBlock] = {};
-        const uint2 lit = encode_literal<0, false>(v, s, none);
-        if (flagged) { lo = lit.x; hi = lit.y; }
+        // Element by element: the literal rule only for the positions at which some lane of the wave holds a flagged
+        // quotient (tensors with short mantissas flag a few quotients in most waves: redoing whole blocks cost 40 %).
+        const float h = rd<0>(s / 2.0f);
+        uint32_t w[2] = {lo, hi};
+#pragma unroll
+        for (int j = 0; j < kBlock; ++j) {
+            const float q = div3(v[j], s, rs);
+            uint32_t a = __float_as_uint(q) & 0x7fffffffu;
+            a = a < 0x3e000010u ? 0x3e000010u : a;
+            a = a > 0x40b00010u ? 0x40b00010u : a;
+            const bool fj = (((a + 4u) >> 3) & 0x1ffffu) == 0u;
+            if (__builtin_amdgcn_ballot_w64(fj) != 0ull) {
+                const float r = code_literal<0, false>(fabsf(v[j]), h, 0.0f);
+                uint32_t code = (uint32_t)fminf(fmaxf(r, 0.0f), 7.0f);
+                code |= (v[j] < 0.0f) ? 8u : 0u;
+                const uint32_t sh = 4u * (uint32_t)(j & 7);
+                if (fj) w[j >> 3] = (w[j >> 3] & ~(0xFu << sh)) | (code << sh);
+            }
+        }
+        lo = w[0];
+        hi = w[1];
     }
     return make_uint2(lo, hi);
 }
