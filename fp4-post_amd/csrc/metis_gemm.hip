@@ -20,13 +20,7 @@
 
 namespace metis {
 
-// Measurement switches (kernel variants and shape overrides read from the environment) exist only in a
-// -DMETIS_MEASURE build of the library; the shipped library reads no environment variables.
-#ifdef METIS_MEASURE
-static inline const char* measure_env(const char* name) { return getenv(name); }
-#else
-static inline const char* measure_env(const char*) { return nullptr; }
-#endif
+// (measure_env(), metis_host.h: kernel variants and shape overrides of a -DMETIS_MEASURE build)
 
 // Workgroup tile BM x BN, 256 threads = 4 waves in a 2 x 2 arrangement, each wave (BM/2) x (BN/2).
 template <int BM, int BN, int OUT_F32>

@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 #include <stddef.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include "../../include/metis_hip.h"
 
@@ -38,6 +39,16 @@ inline int carve_workspace(void* p, size_t bytes, int64_t rows, int64_t cols, Wo
 
 // compute units of the current device (cached per device ordinal)
 int device_cus();
+
+// Measurement switches (kernel variants and shape overrides read from the environment) exist only in a
+// -DMETIS_MEASURE build of the library; the shipped library reads no environment variables.
+#ifdef METIS_MEASURE
+static inline const char* measure_env(const char* name) { return getenv(name); }
+static inline int measure_int(const char* name, int dflt) { const char* v = getenv(name); return v ? atoi(v) : dflt; }
+#else
+static inline const char* measure_env(const char*) { return nullptr; }
+static inline int measure_int(const char*, int dflt) { return dflt; }
+#endif
 
 // phase 2 of the quantizer (tensor unit + E4M3 bytes from parked block maxima); nvfp4_quant.hip
 int launch_scales(int mode, const Workspace& ws, uint32_t ngroups, void* scales, float* unit, uint32_t nblocks,

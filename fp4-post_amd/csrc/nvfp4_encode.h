@@ -1,6 +1,7 @@
 // Per-block NVFP4 encoding shared by the quantizer kernels (plain and RMSNorm-fused).
 #pragma once
 #include "metis_device.h"
+#include "quotient_table.h"
 
 namespace metis {
 
@@ -62,6 +63,74 @@ __device__ __forceinline__ uint2 encode_rne_p32(const float (&v)[kBlock], float 
     hi = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(hi, div3(v[12], s, rs), div3(v[13], s, rs), 1.0f, 2);
     hi = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(hi, div3(v[14], s, rs), div3(v[15], s, rs), 1.0f, 3);
     return make_uint2(lo, hi);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Round-to-nearest, binary32 arithmetic on bf16 values, two operations per quotient.  The block scalar is a function
+// of the block maximum alone, a bf16 value, so there are only 32 640 of them: quotient_table.h (written by
+// gen_quotient_table.c, which walks every block maximum, every bf16 element below it and every reciprocal the
+// hardware may return) has one bit per maximum that says whether
+//     q = fma(x, rh, fma(x, rl, 0)),   rh = rcp(s),   rl = fma(-s, rh, 1) * rh        (rh + rl = 1/s to 2^-46)
+// followed by the hardware conversion gives the reference's code for EVERY element such a block can hold.  All but 26
+// maxima below 2^64 qualify; a block with any other maximum takes the literal sequence.  The inner fma adds +0 so that
+// an input of -0.0 yields the quotient +0.0 (the reference's sign(-0.0) is 0).
+// A workgroup stages the 4 KiB table in LDS once; N = 16 encodes a block, N = 8 one half of it (one packed word).
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ void stage_quotient_table(uint32_t* lds)      // every thread of the workgroup; ends with a barrier
+{
+    for (uint32_t i = threadIdx.x; i < (uint32_t)kQuotientTableWords / 4u; i += blockDim.x)
+        reinterpret_cast<uint4*>(lds)[i] = reinterpret_cast<const uint4*>(kQuotientSafe)[i];
+    __syncthreads();
+}
+__device__ __forceinline__ bool quotient_safe(const uint32_t* lds, float amax)   // amax >= 0, a bf16 value
+{
+    const uint32_t p = __float_as_uint(amax) >> 16;
+    return ((lds[p >> 5] >> (p & 31u)) & 1u) != 0u;
+}
+struct SplitReciprocal { float hi, lo; };
+__device__ __forceinline__ SplitReciprocal split_reciprocal(float s)
+{
+    SplitReciprocal r;
+    r.hi = __builtin_amdgcn_rcpf(s);                          // 1 ulp
+    r.lo = fmaf(-s, r.hi, 1.0f) * r.hi;
+    return r;
+}
+__device__ __forceinline__ float quot2(float x, const SplitReciprocal r) { return fmaf(x, r.hi, fmaf(x, r.lo, 0.0f)); }
+
+template <int N>
+__device__ __forceinline__ void encode_p32_fast_n(const float (&v)[N], const SplitReciprocal r, uint32_t (&w)[N / 8])
+{
+#pragma unroll
+    for (int k = 0; k < N / 8; ++k) {
+        uint32_t c = 0u;
+        // code = E2M1(x / s): x/s = (|x| / (s/2)) / 2 exactly, sign carried by the quotient
+        c = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(c, quot2(v[8 * k], r), quot2(v[8 * k + 1], r), 1.0f, 0);
+        c = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(c, quot2(v[8 * k + 2], r), quot2(v[8 * k + 3], r), 1.0f, 1);
+        c = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(c, quot2(v[8 * k + 4], r), quot2(v[8 * k + 5], r), 1.0f, 2);
+        c = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(c, quot2(v[8 * k + 6], r), quot2(v[8 * k + 7], r), 1.0f, 3);
+        w[k] = c;
+    }
+}
+template <int MODE, int N>
+__device__ __forceinline__ void encode_literal_n(const float (&v)[N], float s, uint32_t (&w)[N / 8])
+{
+    const float h = rd<MODE>(s / 2.0f);
+#pragma unroll
+    for (int k = 0; k < N / 8; ++k) w[k] = 0u;
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+        const float r = code_literal<MODE, false>(fabsf(v[j]), h, 0.0f);
+        uint32_t code = (uint32_t)fminf(fmaxf(r, 0.0f), 7.0f);
+        code |= (v[j] < 0.0f) ? 8u : 0u;
+        w[j >> 3] |= code << (4 * (j & 7));
+    }
+}
+// N elements of a block whose maximum is amax and whose scalar is s (binary32 arithmetic, bf16 values)
+template <int N>
+__device__ __forceinline__ void encode_rne_p32_tbl(const float (&v)[N], float amax, float s, const uint32_t* table, uint32_t (&w)[N / 8])
+{
+    if (quotient_safe(table, amax)) encode_p32_fast_n<N>(v, split_reciprocal(s), w);
+    else encode_literal_n<0, N>(v, s, w);
 }
 
 // Round-to-nearest, binary32 arithmetic, on binary32 VALUES (inputs that are not bf16 values: a binary32
@@ -159,6 +228,31 @@ __device__ __forceinline__ uint2 encode_rne_pb16(const float (&v)[kBlock], float
         }
     }
     return make_uint2(w[0] | sg[0], w[1] | sg[1]);
+}
+
+// the same for N elements (8: half a block, one packed word)
+template <int N>
+__device__ __forceinline__ void encode_rne_pb16_n(const float (&v)[N], float s, uint32_t (&out)[N / 8])
+{
+    const float h = 0.5f * s;
+    const float rh = __builtin_amdgcn_rcpf(h);
+#pragma unroll
+    for (int k = 0; k < N / 8; ++k) {
+        uint32_t w = 0u, sg = 0u;
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) {
+            const uint32_t qq = rb_pair(div3(v[8 * k + j], h, rh), div3(v[8 * k + j + 1], h, rh));
+            const float q0 = nudge_pb16(fabsf(bf16_lo(qq))), q1 = nudge_pb16(fabsf(bf16_hi(qq)));
+            sg |= (((qq >> 12) & 0x8u) | ((qq >> 24) & 0x80u)) << (4 * j);
+            switch (j >> 1) {
+            case 0: w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, q0, q1, 2.0f, 0); break;
+            case 1: w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, q0, q1, 2.0f, 1); break;
+            case 2: w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, q0, q1, 2.0f, 2); break;
+            default: w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, q0, q1, 2.0f, 3); break;
+            }
+        }
+        out[k] = w | sg;
+    }
 }
 
 // One v_cvt_scalef32_sr_pk_fp4_f32: converts (q0, q1) / 2^MODE with stochastic rounding into byte `byte` of w

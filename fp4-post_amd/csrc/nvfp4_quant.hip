@@ -35,30 +35,50 @@ namespace metis {
 __device__ __forceinline__ float block_scalar_ieee(float amax) { return amax / 6.0f + 1e-9f; }
 
 // Round-to-nearest rows of a contiguous bf16 tensor, the shape every activation and weight has: a kernel of its own
-// so that its loop carries no row/column arithmetic at all.  Software-pipelined: the next block's 32 bytes are in
-// flight while the current block is encoded.
-template <int MODE>
+// so that its loop carries no row/column arithmetic at all.  Software-pipelined: the next DEPTH blocks' bytes are in
+// flight while the current block is encoded.  Binary32 arithmetic takes the two-operation quotient for every block
+// maximum the staged table clears (nvfp4_encode.h).
+template <int MODE> __device__ __forceinline__ uint2 encode_row_block(const float (&v)[kBlock], float am, const uint32_t* table)
+{
+    if constexpr (MODE == 0) {
+        uint32_t w[2];
+        encode_rne_p32_tbl<kBlock>(v, am, block_scalar<0>(am), table, w);
+        return make_uint2(w[0], w[1]);
+    } else {
+        return encode_rne_pb16(v, block_scalar<1>(am));
+    }
+}
+
+template <int MODE, int DEPTH = 1>
 __global__ __launch_bounds__(256) void quant_codes_contig_kernel(const uint4* __restrict__ x, uint2* __restrict__ codes,
                                                                  uint16_t* __restrict__ ws_amax, uint32_t* __restrict__ ws_gmax,
                                                                  uint32_t nblocks, uint32_t fill_to)
 {
+    __shared__ uint32_t table[MODE == 0 ? kQuotientTableWords : 4];
     float gmax = 0.0f;
     const uint32_t step = gridDim.x * 256u;
     uint32_t i = blockIdx.x * 256u + threadIdx.x;
-    uint4 c0 = make_uint4(0u, 0u, 0u, 0u), c1 = c0;
-    if (i < nblocks) { c0 = x[2 * (size_t)i]; c1 = x[2 * (size_t)i + 1]; }
+    uint4 c0[DEPTH], c1[DEPTH];
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+        const uint32_t j = i + d * step;
+        c0[d] = c1[d] = make_uint4(0u, 0u, 0u, 0u);
+        if (j < nblocks) { c0[d] = x[2 * (size_t)j]; c1[d] = x[2 * (size_t)j + 1]; }
+    }
+    if constexpr (MODE == 0) stage_quotient_table(table);
     while (i < nblocks) {
-        const uint32_t nxt = i + step;
-        uint4 n0 = c0, n1 = c1;
-        if (nxt < nblocks) { n0 = x[2 * (size_t)nxt]; n1 = x[2 * (size_t)nxt + 1]; }
+        const uint4 a0 = c0[0], a1 = c1[0];
+#pragma unroll
+        for (int d = 0; d + 1 < DEPTH; ++d) { c0[d] = c0[d + 1]; c1[d] = c1[d + 1]; }
+        const uint32_t nxt = i + DEPTH * step;
+        if (nxt < nblocks) { c0[DEPTH - 1] = x[2 * (size_t)nxt]; c1[DEPTH - 1] = x[2 * (size_t)nxt + 1]; }
         float v[kBlock];
-        const float none[kBlock] = {};
-        unpack16(c0, c1, v);
+        unpack16(a0, a1, v);
         const float am = block_amax(v);
         gmax = fmaxf(gmax, am);
         ws_amax[i] = (uint16_t)(__float_as_uint(am) >> 16);
-        codes[i] = encode_block<MODE, false>(v, block_scalar<MODE>(am), none);
-        c0 = n0; c1 = n1; i = nxt;
+        codes[i] = encode_row_block<MODE>(v, am, table);
+        i += step;
     }
     publish_group_max(gmax, ws_gmax, fill_to);
 }
@@ -739,7 +759,7 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint32_t* __restrict
 static int grid_for(uint32_t work_items)
 {
     int64_t g = ((int64_t)work_items + 255) / 256;
-    const int64_t cap = (int64_t)device_cus() * 8;           // 8 workgroups of 256 per CU are resident
+    const int64_t cap = (int64_t)device_cus() * measure_int("METIS_Q_WGPC", 8);   // 8 workgroups of 256 per CU are resident
     if (g > cap) g = cap;
     if (g > kMaxGroups) g = kMaxGroups;
     return g < 1 ? 1 : (int)g;
@@ -801,6 +821,17 @@ static int launch_fused(const void* x, void* codes, void* scales, float* unit, c
     return rc;
 }
 
+template <int MODE>
+static void launch_contig(const void* x, void* codes, const Workspace& ws, uint32_t nblocks, uint32_t fill_to, int grid, hipStream_t st)
+{
+    if (measure_int("METIS_Q_DEPTH", 1) == 2)
+        hipLaunchKernelGGL((quant_codes_contig_kernel<MODE, 2>), dim3(grid), dim3(256), 0, st, (const uint4*)x, (uint2*)codes, ws.amax,
+                           ws.gmax, nblocks, fill_to);
+    else
+        hipLaunchKernelGGL((quant_codes_contig_kernel<MODE, 1>), dim3(grid), dim3(256), 0, st, (const uint4*)x, (uint2*)codes, ws.amax,
+                           ws.gmax, nblocks, fill_to);
+}
+
 template <int MODE, bool SR, bool COL, bool WIDE = false, bool HAD = false>
 static int launch_quant(const void* x, int64_t rows, int64_t cols, int64_t ld, const void* noise, uint64_t seed,
                         uint64_t offset, void* codes, void* scales, float* unit, const Workspace& ws, hipStream_t st,
@@ -829,8 +860,7 @@ static int launch_quant(const void* x, int64_t rows, int64_t cols, int64_t ld, c
         const int g1 = grid_for(nblocks);
         if constexpr (!SR && !WIDE && !HAD) {
             if (!center && ld == cols) {
-                hipLaunchKernelGGL((quant_codes_contig_kernel<MODE>), dim3(g1), dim3(256), 0, st, (const uint4*)x, (uint2*)codes,
-                                   ws.amax, ws.gmax, nblocks, 0u);
+                launch_contig<MODE>(x, codes, ws, nblocks, 0u, g1, st);
                 return launch_scales(MODE, ws, (uint32_t)g1, scales, unit, nblocks, st);
             }
         }
@@ -992,11 +1022,9 @@ int quantize_row_deferred(const void* x, int64_t rows, int64_t cols, int mode, c
                            cols, nullptr, (uint64_t)0, (uint64_t)0, (uint2*)codes, (void*)ws.amax, ws.gmax, nblocks, 0, center, 0u,
                            kDeferredPartials);
     else if (mode == 0)
-        hipLaunchKernelGGL((quant_codes_contig_kernel<0>), dim3(g1), dim3(256), 0, st, (const uint4*)x, (uint2*)codes, ws.amax, ws.gmax,
-                           nblocks, kDeferredPartials);
+        launch_contig<0>(x, codes, ws, nblocks, kDeferredPartials, g1, st);
     else
-        hipLaunchKernelGGL((quant_codes_contig_kernel<1>), dim3(g1), dim3(256), 0, st, (const uint4*)x, (uint2*)codes, ws.amax, ws.gmax,
-                           nblocks, kDeferredPartials);
+        launch_contig<1>(x, codes, ws, nblocks, kDeferredPartials, g1, st);
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 

@@ -102,6 +102,124 @@ __global__ __launch_bounds__(256) void rmsnorm_quant_kernel(const uint16_t* __re
     publish_group_max(gmax, ws_gmax, fill_to);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Rows of at most 4096 columns: one WAVE per row, no barrier and no LDS traffic for the reduction.  Lane l holds the
+// 16-byte chunks l, l + 64, ... of the row (8 elements: half a scale block; lanes 2m and 2m + 1 share a block), so
+// every load and store instruction of the wave covers consecutive bytes: a KiB of the row in, a KiB of the normed
+// row out, 256 bytes of codes.  (Thread-per-block stores of the normed row, 16 bytes at a 32-byte lane stride, held
+// this kernel's byte mix to 5.2 TB/s; whole lines written with the non-temporal hint reach 7.)  The sum of squares is
+// taken on the packed pairs (v_dot2_f32_bf16) and folded across the wave with DPP moves; the product with gamma is a
+// v_dot2_f32_bf16 of the packed bf16(x * rstd) pair against gamma with the other half masked off -- the exact product
+// of the two bf16 values, no unpacking (subnormal products are rounded differently by that instruction and a zero
+// product comes out as +0.0: both below anything the normed tensor's consumers can tell apart).  gamma is staged in
+// LDS once per workgroup in that masked form; the block maximum is one DPP exchange between the two lanes of a block.
+// ---------------------------------------------------------------------------------------------
+typedef __bf16 metis_bf16pair_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c)
+{
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(metis_bf16pair_t, a), __builtin_bit_cast(metis_bf16pair_t, b), c, false);
+}
+template <int CTRL> __device__ __forceinline__ float dpp_f32(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+// sum over the 64 lanes, the same value in every lane
+__device__ __forceinline__ float wave_sum_dpp(float v)
+{
+    v += dpp_f32<0xB1>(v);           // quad_perm [1,0,3,2]
+    v += dpp_f32<0x4E>(v);           // quad_perm [2,3,0,1]
+    v += dpp_f32<0x141>(v);          // row_half_mirror
+    v += dpp_f32<0x140>(v);          // row_mirror: every lane of a row of 16 holds the row's sum
+    const int b = __builtin_bit_cast(int, v);                 // (the builtin takes an integer: pass the bits, not the value)
+    const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0)), r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16));
+    const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32)), r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
+    return (r0 + r1) + (r2 + r3);
+}
+typedef uint32_t metis_u32x4_t __attribute__((ext_vector_type(4)));
+
+template <int MODE, int NL, bool WRITE_NORMED>
+__global__ __launch_bounds__(256) void rmsnorm_quant_rows_kernel(const uint4* __restrict__ x, const uint4* __restrict__ gamma, float eps,
+                                                                 uint32_t rows, uint32_t cols, metis_u32x4_t* __restrict__ normed,
+                                                                 uint32_t* __restrict__ codes, uint16_t* __restrict__ ws_amax,
+                                                                 uint32_t* __restrict__ ws_gmax, uint32_t fill_to)
+{
+    __shared__ uint4 g_a[NL * 64], g_b[NL * 64];              // gamma pairs 0, 1 and 2, 3 of every chunk, each as {low only, high only}
+    __shared__ uint32_t table[MODE == 0 ? kQuotientTableWords : 4];
+    const uint32_t cpr = cols / 8u;                           // 16-byte chunks per row (even: cols % 16 == 0)
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const float fcols = (float)cols;
+    const uint32_t wstep = gridDim.x * 4u;
+    uint32_t row = blockIdx.x * 4u + wave;
+    uint4 raw[NL];
+    auto request = [&](uint32_t r) {
+#pragma unroll
+        for (int i = 0; i < NL; ++i) {
+            const uint32_t c = i * 64u + lane;
+            if (c < cpr) raw[i] = x[(size_t)r * cpr + c];
+        }
+    };
+#pragma unroll
+    for (int i = 0; i < NL; ++i) raw[i] = make_uint4(0u, 0u, 0u, 0u);
+    if (row < rows) request(row);
+    for (uint32_t c = threadIdx.x; c < cpr; c += 256u) {
+        const uint4 g = gamma[c];
+        g_a[c] = make_uint4(g.x & 0xffffu, g.x & 0xffff0000u, g.y & 0xffffu, g.y & 0xffff0000u);
+        g_b[c] = make_uint4(g.z & 0xffffu, g.z & 0xffff0000u, g.w & 0xffffu, g.w & 0xffff0000u);
+    }
+    if constexpr (MODE == 0) stage_quotient_table(table);
+    else __syncthreads();
+    float gmax = 0.0f;
+    for (; row < rows; row += wstep) {
+        uint4 cur[NL];
+        float ss = 0.0f;
+#pragma unroll
+        for (int i = 0; i < NL; ++i) {
+            cur[i] = raw[i];
+            ss = dot2_bf16(cur[i].x, cur[i].x, ss);
+            ss = dot2_bf16(cur[i].y, cur[i].y, ss);
+            ss = dot2_bf16(cur[i].z, cur[i].z, ss);
+            ss = dot2_bf16(cur[i].w, cur[i].w, ss);
+        }
+        if (row + wstep < rows) request(row + wstep);           // the next row is in flight while this one is encoded
+        const float total = wave_sum_dpp(ss);
+        const float rstd = 1.0f / sqrtf(total / fcols + eps);
+#pragma unroll
+        for (int i = 0; i < NL; ++i) {
+            const uint32_t c = i * 64u + lane;
+            if (i * 64u >= cpr) break;                         // wave-uniform: chunks beyond the row
+            if (c < cpr) {
+                const uint32_t in[4] = {cur[i].x, cur[i].y, cur[i].z, cur[i].w};
+                const uint4 ga = g_a[c], gb = g_b[c];
+                const uint32_t gl[4] = {ga.x, ga.z, gb.x, gb.z}, gh[4] = {ga.y, ga.w, gb.y, gb.w};
+                uint32_t w[4];
+                float n[8];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    // bf16(bf16(x * rstd) * gamma), two elements per conversion; the packed pairs are the normed output
+                    const uint32_t h = rb_pair(bf16_lo(in[j]) * rstd, bf16_hi(in[j]) * rstd);
+                    w[j] = rb_pair(dot2_bf16(h, gl[j], 0.0f), dot2_bf16(h, gh[j], 0.0f));
+                    n[2 * j] = bf16_lo(w[j]);
+                    n[2 * j + 1] = bf16_hi(w[j]);
+                }
+                const size_t at = (size_t)row * cpr + c;
+                if (WRITE_NORMED) __builtin_nontemporal_store((metis_u32x4_t){w[0], w[1], w[2], w[3]}, normed + at);
+                float hm = amax3(0.0f, n[0], n[1]);
+                hm = amax3(hm, n[2], n[3]);
+                hm = amax3(hm, n[4], n[5]);
+                hm = amax3(hm, n[6], n[7]);
+                const float am = fmaxf(hm, dpp_f32<0xB1>(hm));  // the other half of the block sits in the neighbouring lane
+                gmax = fmaxf(gmax, am);
+                if ((lane & 1u) == 0u) ws_amax[at >> 1] = (uint16_t)(__float_as_uint(am) >> 16);
+                uint32_t cw[1];
+                if constexpr (MODE == 0) encode_rne_p32_tbl<8>(n, am, block_scalar<0>(am), table, cw);
+                else encode_rne_pb16_n<8>(n, block_scalar<1>(am), cw);
+                codes[at] = cw[0];
+            }
+        }
+    }
+    publish_group_max(gmax, ws_gmax, fill_to);
+}
+
 // deferred: stop after the main kernel; `workspace` is then the caller-owned parked data of the deferred form
 // (nvfp4_quant.hip) and scales / unit are not written.
 int rmsnorm_quantize(const void* x, const void* gamma, float eps, int64_t rows, int64_t cols, int mode, void* normed,
@@ -120,6 +238,26 @@ int rmsnorm_quantize(const void* x, const void* gamma, float eps, int64_t rows, 
     Workspace ws;
     int rc = deferred ? carve_deferred(workspace, workspace_bytes, rows, cols, &ws) : carve_workspace(workspace, workspace_bytes, rows, cols, &ws);
     if (rc != METIS_OK) return rc;
+    if (cols <= 4096) {
+        // one wave per row
+        int64_t g = (rows + 3) / 4;
+        const int64_t cap = (int64_t)device_cus() * measure_int("METIS_N_WGPC", 4);
+        if (g > cap) g = cap;
+        if (g > kMaxGroups) g = kMaxGroups;
+        if (deferred && g > (int64_t)kDeferredPartials) g = kDeferredPartials;
+        const uint32_t fill_to = deferred ? kDeferredPartials : 0u;
+        const int nl = (int)((cols / 8 + 63) / 64);
+#define METIS_RW(M, NL, W) hipLaunchKernelGGL((rmsnorm_quant_rows_kernel<M, NL, W>), dim3((int)g), dim3(256), 0, st, (const uint4*)x, \
+        (const uint4*)gamma, eps, (uint32_t)rows, (uint32_t)cols, (metis_u32x4_t*)normed, (uint32_t*)codes, ws.amax, ws.gmax, fill_to)
+#define METIS_RWN(M, W) do { if (nl <= 2) METIS_RW(M, 2, W); else if (nl <= 4) METIS_RW(M, 4, W); else METIS_RW(M, 8, W); } while (0)
+        if (mode == 0) { if (normed) METIS_RWN(0, true); else METIS_RWN(0, false); }
+        else { if (normed) METIS_RWN(1, true); else METIS_RWN(1, false); }
+#undef METIS_RWN
+#undef METIS_RW
+        if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
+        if (deferred) return METIS_OK;
+        return launch_scales(mode, ws, (uint32_t)g, scales, unit, (uint32_t)(rows * cols / kBlock), st);
+    }
     int64_t g = rows;
     const int64_t cap = (int64_t)device_cus() * 8;
     if (g > cap) g = cap;
