@@ -65,7 +65,7 @@ int quantize_both_sr(const void* x, int64_t rows, int64_t cols, int64_t ld, int 
 // deferred scale bytes (nvfp4_quant.hip): phase 1 alone into caller-owned parked data, phase 2 on it later or never
 size_t deferred_bytes(int64_t rows, int64_t cols);
 int carve_deferred(void* p, size_t bytes, int64_t rows, int64_t cols, Workspace* ws);
-int deferred_grid(uint32_t work_items);
+int deferred_grid(uint32_t work_items, int per_cu = 8);
 int quantize_row_deferred(const void* x, int64_t rows, int64_t cols, int mode, const void* center, void* codes, void* deferred,
                           size_t bytes, hipStream_t st);
 int deferred_scales(const void* deferred, int64_t rows, int64_t cols, int mode, void* scales, float* unit, hipStream_t st);

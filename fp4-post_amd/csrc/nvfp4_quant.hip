@@ -38,6 +38,7 @@ __device__ __forceinline__ float block_scalar_ieee(float amax) { return amax / 6
 // so that its loop carries no row/column arithmetic at all.  Software-pipelined: the next DEPTH blocks' bytes are in
 // flight while the current block is encoded.  Binary32 arithmetic takes the two-operation quotient for every block
 // maximum the staged table clears (nvfp4_encode.h).
+typedef uint32_t metis_u32x2_t __attribute__((ext_vector_type(2)));
 template <int MODE> __device__ __forceinline__ uint2 encode_row_block(const float (&v)[kBlock], float am, const uint32_t* table)
 {
     if constexpr (MODE == 0) {
@@ -76,8 +77,9 @@ __global__ __launch_bounds__(256) void quant_codes_contig_kernel(const uint4* __
         unpack16(a0, a1, v);
         const float am = block_amax(v);
         gmax = fmaxf(gmax, am);
-        ws_amax[i] = (uint16_t)(__float_as_uint(am) >> 16);
-        codes[i] = encode_row_block<MODE>(v, am, table);
+        ws_amax[i] = (uint16_t)(__float_as_uint(am) >> 16);        // read again soon by whoever forms the scale bytes
+        const uint2 cw = encode_row_block<MODE>(v, am, table);
+        __builtin_nontemporal_store((metis_u32x2_t){cw.x, cw.y}, reinterpret_cast<metis_u32x2_t*>(codes) + i);
         i += step;
     }
     publish_group_max(gmax, ws_gmax, fill_to);
@@ -756,10 +758,10 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint32_t* __restrict
 // ---------------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------------
-static int grid_for(uint32_t work_items)
+static int grid_for(uint32_t work_items, int per_cu = 8)           // 8 workgroups of 256 per CU are resident
 {
     int64_t g = ((int64_t)work_items + 255) / 256;
-    const int64_t cap = (int64_t)device_cus() * measure_int("METIS_Q_WGPC", 8);   // 8 workgroups of 256 per CU are resident
+    const int64_t cap = (int64_t)device_cus() * per_cu;
     if (g > cap) g = cap;
     if (g > kMaxGroups) g = kMaxGroups;
     return g < 1 ? 1 : (int)g;
@@ -781,6 +783,11 @@ int launch_scales(int mode, const Workspace& ws, uint32_t ngroups, void* scales,
                            (uint8_t*)scales, unit, nblocks, (const uint16_t*)amax2, (uint8_t*)scales2, unit2);
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
+
+// Workgroups per compute unit of the contiguous row quantizer: four waves per SIMD hide the memory latency as well as eight
+// do, the last round of blocks (encoded with nothing left to overlap) is half as long, and half as many partial maxima
+// are folded later.
+constexpr int kContigPerCu = 4;
 
 // Co-resident workgroups of the single-launch kernel on the current device (0 = unknown).
 template <int MODE, int NB>
@@ -857,13 +864,14 @@ static int launch_quant(const void* x, int64_t rows, int64_t cols, int64_t ld, c
                                (uint32_t)tiles, center);
         return launch_scales(WIDE ? METIS_MODE_P32_F32 : MODE, ws, (uint32_t)g, scales, unit, nblocks, st);
     } else {
-        const int g1 = grid_for(nblocks);
         if constexpr (!SR && !WIDE && !HAD) {
             if (!center && ld == cols) {
-                launch_contig<MODE>(x, codes, ws, nblocks, 0u, g1, st);
-                return launch_scales(MODE, ws, (uint32_t)g1, scales, unit, nblocks, st);
+                const int gc = grid_for(nblocks, measure_int("METIS_Q_WGPC", kContigPerCu));
+                launch_contig<MODE>(x, codes, ws, nblocks, 0u, gc, st);
+                return launch_scales(MODE, ws, (uint32_t)gc, scales, unit, nblocks, st);
             }
         }
+        const int g1 = grid_for(nblocks);
         hipLaunchKernelGGL((quant_codes_kernel<MODE, SR, WIDE, HAD>), dim3(g1), dim3(256), 0, st, x, (uint32_t)rows,
                            (uint32_t)cols, ld, noise, seed, offset, (uint2*)codes, (void*)ws.amax, ws.gmax, nblocks, in_f32, center,
                            sign_mask, 0u);
@@ -995,9 +1003,9 @@ int carve_deferred(void* p, size_t bytes, int64_t rows, int64_t cols, Workspace*
     return METIS_OK;
 }
 
-int deferred_grid(uint32_t work_items)
+int deferred_grid(uint32_t work_items, int per_cu)
 {
-    const int g = grid_for(work_items);
+    const int g = grid_for(work_items, per_cu);
     return g > (int)kDeferredPartials ? (int)kDeferredPartials : g;
 }
 
@@ -1016,7 +1024,7 @@ int quantize_row_deferred(const void* x, int64_t rows, int64_t cols, int mode, c
     Workspace ws;
     if (const int rc = carve_deferred(deferred, bytes, rows, cols, &ws)) return rc;
     const uint32_t nblocks = (uint32_t)(rows * cols / kBlock);
-    const int g1 = deferred_grid(nblocks);
+    const int g1 = deferred_grid(nblocks, center ? 8 : measure_int("METIS_Q_WGPC", kContigPerCu));
     if (center)
         hipLaunchKernelGGL((quant_codes_kernel<1, false, false, false>), dim3(g1), dim3(256), 0, st, x, (uint32_t)rows, (uint32_t)cols,
                            cols, nullptr, (uint64_t)0, (uint64_t)0, (uint2*)codes, (void*)ws.amax, ws.gmax, nblocks, 0, center, 0u,

@@ -241,7 +241,7 @@ int rmsnorm_quantize(const void* x, const void* gamma, float eps, int64_t rows, 
     if (cols <= 4096) {
         // one wave per row
         int64_t g = (rows + 3) / 4;
-        const int64_t cap = (int64_t)device_cus() * measure_int("METIS_N_WGPC", 4);
+        const int64_t cap = (int64_t)device_cus() * measure_int("METIS_N_WGPC", 3);
         if (g > cap) g = cap;
         if (g > kMaxGroups) g = kMaxGroups;
         if (deferred && g > (int64_t)kDeferredPartials) g = kDeferredPartials;
