@@ -94,6 +94,88 @@ def time_region(torch, fn, steps, warmup):
     return t1 - t0, ev_ms
 
 
+def region_us(torch, fn, steps, warmup):
+    """Average duration of one call in microseconds: ONE pair of events around `steps` back-to-back calls on the launch
+    stream (what a kernel trace of the same region adds up to, launch gaps included)."""
+    for _ in range(warmup):
+        fn(None)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        fn(None)
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps * 1e3
+
+
+def settle(torch, fn, seconds=1.0):
+    """Untimed launches of the headline step until `seconds` have passed: the part's clock needs about a second under
+    load to settle, whatever --warmup says.  Returns the seconds spent."""
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while True:
+        for _ in range(10):
+            fn(None)
+        torch.cuda.synchronize()
+        if time.perf_counter() - t0 >= seconds:
+            return time.perf_counter() - t0
+
+
+def ceilings_leg(torch, dev, st):
+    """Byte-only and MFMA-only kernels (fp4-post_amd/csrc/ceilings.hip, built beside the library) on this device, now."""
+    import ctypes
+    path = os.path.join(ROOT, "fp4-post_amd", "metis_hip", "libmetis_ceilings.so")
+    C = ctypes.CDLL(path)
+    vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+    C.metis_ceiling_stream.restype, C.metis_ceiling_stream.argtypes = i32, [vp, vp, vp, vp, i64, i32, i32, vp]
+    C.metis_ceiling_mfma.restype, C.metis_ceiling_mfma.argtypes = i32, [vp, vp, i32, i32, vp]
+    out = {"source": "fp4-post_amd/csrc/ceilings.hip: kernels that only move the hot kernels' bytes, or only issue their MFMAs, "
+                     "in this process on this device (events around 50 back-to-back launches)"}
+    n2 = 16384 * 4096
+    xb = torch.randn(n2, device=dev).bfloat16()
+    nb = torch.empty(n2, dtype=torch.bfloat16, device=dev)
+    cb = torch.empty(n2 // 2, dtype=torch.uint8, device=dev)
+    ab = torch.empty(n2 // 16, dtype=torch.int16, device=dev)
+
+    def us_of(fn, n=50, w=10):
+        for _ in range(w):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n * 1e3
+    for name, elems, mix, bpe in (("quantizer_bytes_config1", n2 // 2, 0, QUANT_BYTES_PER_ELT), ("fused_norm_bytes_config2", n2, 1, NORMQ_BYTES_PER_ELT)):
+        best = None
+        for grid in (768, 1024, 2048):
+            def run():
+                assert C.metis_ceiling_stream(xb.data_ptr(), nb.data_ptr(), cb.data_ptr(), ab.data_ptr(), elems, mix, grid, st) == 0
+            us = us_of(run)
+            if best is None or us < best[0]:
+                best = (us, grid)
+        out[name] = {"us": round(best[0], 2), "GBps_on_algorithmic_bytes": round(elems * bpe / best[0] / 1e3, 1),
+                     "frac_of_hbm_peak": round(elems * bpe / best[0] / 1e3 / HBM_PEAK_GBS, 4), "grid": best[1]}
+    del xb, nb, cb, ab
+    res_ = torch.empty(512 * 256, dtype=torch.float32, device=dev)
+    iters = 4000
+    for name, src in (("mfma_f16_loop_constant_operands", torch.ones(32768, dtype=torch.float16, device=dev)),
+                      ("mfma_f16_loop_normal_operands", torch.randn(32768, generator=torch.Generator().manual_seed(1)).to(torch.float16).to(dev))):
+        best = 0.0
+        for per_cu in (1, 2):
+            grid = 256 * per_cu
+
+            def run():
+                assert C.metis_ceiling_mfma(src.data_ptr(), res_.data_ptr(), iters, grid, st) == 0
+            us = us_of(run, n=5, w=2)
+            best = max(best, grid * 4 * iters * 16 * 32768.0 / us / 1e6)
+        out[name] = {"tflops": round(best, 1), "frac_of_mfma_peak": round(best / MFMA_PEAK_TFLOPS, 4)}
+    return out
+
+
 def cpu_baseline_linear(torch, x, v, s, u, res, budget_rows=2048):
     """Oracle (port of the reference arithmetic, PyTorch CPU eager) on the first rows of config 3."""
     from oracle import metis_oracle as O
@@ -174,6 +256,7 @@ def main():
             ev[1].record()
         return y
 
+    settle_s = settle(torch, step, 1.0)
     wall, gemm_ms = time_region(torch, step, args.steps, args.warmup)
     flops_step = 2.0 * M * N * K + 2.0 * M * K * r + 2.0 * M * r * N
     gemm_flops = 2.0 * M * N * K + 2.0 * M * r * N             # what the fused GEMM launch computes
@@ -205,7 +288,9 @@ def main():
             ev[1].record()
         assert rc == 0
 
-    qwall, q_ms = time_region(torch, qstep, max(args.steps, 50), args.warmup)
+    qsteps = max(args.steps, 100)
+    _, q_pair_ms = time_region(torch, qstep, qsteps, args.warmup)
+    q_ms = region_us(torch, qstep, qsteps, args.warmup) * 1e-3
     q_bytes = x1.numel() * QUANT_BYTES_PER_ELT
     q_gbs = q_bytes / (q_ms * 1e-3) / 1e9
 
@@ -220,7 +305,7 @@ def main():
             ev[1].record()
         assert rc == 0
 
-    _, qd_ms = time_region(torch, qdstep, max(args.steps, 50), args.warmup)
+    qd_ms = region_us(torch, qdstep, qsteps, args.warmup) * 1e-3
     qd_gbs = q_bytes / (qd_ms * 1e-3) / 1e9
 
     # the opt-in single-launch variant (needs the device to itself: every workgroup must be resident)
@@ -233,8 +318,21 @@ def main():
             ev[1].record()
         assert rc == 0
 
-    _, q1_ms = time_region(torch, q1step, max(args.steps, 50), args.warmup)
+    q1_ms = region_us(torch, q1step, qsteps, args.warmup) * 1e-3
     q1_gbs = q_bytes / (q1_ms * 1e-3) / 1e9
+
+    # the round trip as config 1 states it: codes, scale bytes AND the dequantized bf16 tensor from one call
+    qdq = torch.empty(8192, 4096, dtype=torch.bfloat16, device=dev)
+
+    def qrstep(ev):
+        rc = L.metis_nvfp4_quant_dequant_row(x1.data_ptr(), 8192, 4096, 0, qc.data_ptr(), qs.data_ptr(), qu.data_ptr(), qdq.data_ptr(),
+                                             qws.data_ptr(), qws.numel(), st)
+        assert rc == 0
+
+    qr_ms = region_us(torch, qrstep, qsteps, args.warmup) * 1e-3
+    qr_bytes = x1.numel() * NORMQ_BYTES_PER_ELT                 # 2 B read + 0.5625 B packed + 2 B dequantized
+    qr_gbs = qr_bytes / (qr_ms * 1e-3) / 1e9
+    del qdq
 
     # ------------------------------------------------------------------ config 2: fused RMSNorm -> quant
     h = outlier_activation(torch, 1002, 16384, 4096, dev)
@@ -252,7 +350,8 @@ def main():
             ev[1].record()
         assert rc == 0
 
-    nwall, n_ms = time_region(torch, nstep, max(args.steps, 50), args.warmup)
+    _, n_pair_ms = time_region(torch, nstep, qsteps, args.warmup)
+    n_ms = region_us(torch, nstep, qsteps, args.warmup) * 1e-3
     n_bytes = h.numel() * NORMQ_BYTES_PER_ELT
     n_gbs = n_bytes / (n_ms * 1e-3) / 1e9
 
@@ -267,7 +366,7 @@ def main():
             ev[1].record()
         assert rc == 0
 
-    _, nd_ms = time_region(torch, ndstep, max(args.steps, 50), args.warmup)
+    nd_ms = region_us(torch, ndstep, qsteps, args.warmup) * 1e-3
     nd_gbs = n_bytes / (nd_ms * 1e-3) / 1e9
 
     # ------------------------------------------------------------------ the kernels that serve two consumers from one pass
@@ -625,6 +724,7 @@ def main():
         "vs_baseline": None,
         "dtype": "nvfp4 (e2m1 x e4m3) expanded exactly to f16, f32 accumulate; low-rank bf16",
         "data": "synthetic",
+        "settle_s": round(settle_s, 2),
         "config": {"workload": "config 3: Metis low-rank-residual linear forward, X[8192,4096] W[14336,4096] r=64; "
                                "step = one pass over X (NVFP4 codes + block maxima, and X.V^T*s) + expand X to tiled f16 (forms unit and scale bytes) + fused pipelined GEMM (packed W and its tiled f16 expansion cached)",
                    "parity_mode": "P32", "parity_rel_fro_256_rows": err},
@@ -633,6 +733,12 @@ def main():
                      "traffic": TRAFFIC_GEMM_C3, "traffic_source": TRAFFIC_SOURCE, "kernel_ms": round(gemm_ms, 4)},
         "quant": {"workload": "config 1: NVFP4 RNE quantize bf16 [8192,4096] (P32), codes+scales+unit",
                   "value": round(q_gbs, 1), "unit": "GB/s", "us_per_call": round(q_ms * 1e3, 2),
+                  "timing": "events around the region of back-to-back calls on the launch stream; us_per_call_event_pairs brackets every call with its own pair",
+                  "us_per_call_event_pairs": round(q_pair_ms * 1e3, 2),
+                  "round_trip": {"workload": "the same tensor through metis_nvfp4_quant_dequant_row: codes + scale bytes + unit + the dequantized bf16 "
+                                             "tensor (config 1's three outputs) from one call of two launches; 4.5625 B/element = 153.09 MB",
+                                 "value": round(qr_gbs, 1), "unit": "GB/s", "us_per_call": round(qr_ms * 1e3, 2),
+                                 "frac": round(qr_gbs / HBM_PEAK_GBS, 4)},
                   "roofline": {"bound": "hbm", "kernel": "quant_codes_contig_kernel+quant_scales_kernel",
                                "achieved": round(q_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                "frac": round(q_gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_QUANT_C1, "traffic_source": TRAFFIC_SOURCE},
@@ -646,7 +752,8 @@ def main():
                                            "frac": round(qd_gbs / HBM_PEAK_GBS, 4)}},
         "rmsnorm_quant": {"workload": "config 2: fused RMSNorm->NVFP4 bf16 [16384,4096] (P32), normed+codes+scales",
                           "value": round(n_gbs, 1), "unit": "GB/s", "us_per_call": round(n_ms * 1e3, 2),
-                          "roofline": {"bound": "hbm", "kernel": "rmsnorm_quant_kernel+quant_scales_kernel",
+                          "us_per_call_event_pairs": round(n_pair_ms * 1e3, 2),
+                          "roofline": {"bound": "hbm", "kernel": "rmsnorm_quant_rows_kernel+quant_scales_kernel",
                                        "achieved": round(n_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                        "frac": round(n_gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_NORMQ_C2,
                                        "traffic_source": TRAFFIC_SOURCE},
@@ -656,6 +763,10 @@ def main():
                                                    "value": round(nd_gbs, 1), "unit": "GB/s", "us_per_call": round(nd_ms * 1e3, 2),
                                                    "frac": round(nd_gbs / HBM_PEAK_GBS, 4)}},
     }
+    try:
+        line["ceilings"] = ceilings_leg(torch, dev, st)
+    except Exception as exc:  # an optional leg must not cost the headline line
+        line["ceilings"] = {"error": f"{type(exc).__name__}: {exc}"[:300]}
     if one_pass is not None:
         line["one_pass_kernels"] = one_pass
     if dec is not None:

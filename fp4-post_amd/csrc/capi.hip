@@ -49,6 +49,12 @@ int metis_nvfp4_quant_row(const void* x, int64_t rows, int64_t cols, int64_t ld,
                     workspace_bytes, (hipStream_t)stream);
 }
 
+int metis_nvfp4_quant_dequant_row(const void* x, int64_t rows, int64_t cols, int mode, void* codes, void* scales, float* unit,
+                                  void* out, void* workspace, size_t workspace_bytes, void* stream)
+{
+    return quantize_dequantize_row(x, rows, cols, mode, codes, scales, unit, out, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
 int metis_nvfp4_quant_row_static(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, void* codes, void* scales,
                                  float* unit, void* stream)
 {

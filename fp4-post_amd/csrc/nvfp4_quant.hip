@@ -39,6 +39,7 @@ __device__ __forceinline__ float block_scalar_ieee(float amax) { return amax / 6
 // flight while the current block is encoded.  Binary32 arithmetic takes the two-operation quotient for every block
 // maximum the staged table clears (nvfp4_encode.h).
 typedef uint32_t metis_u32x2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t metis_u32x4_t __attribute__((ext_vector_type(4)));
 template <int MODE> __device__ __forceinline__ uint2 encode_row_block(const float (&v)[kBlock], float am, const uint32_t* table)
 {
     if constexpr (MODE == 0) {
@@ -756,6 +757,62 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint32_t* __restrict
 }
 
 // ---------------------------------------------------------------------------------------------
+// Phase 2 with the dequantized tensor (the round trip of quant.py:6-36: codes, scale bytes AND the dequantized values
+// from one call): tensor unit, E4M3 bytes and out = ((v * sign) / 2) * (e4m3 * unit) in one pass over the codes and the
+// parked maxima.  A lane owns half a block (one word of codes, 16 bytes of output), so every load and store instruction
+// of a wave covers consecutive bytes; the hardware converter turns two codes into their binary32 values (E2M1 = v / 2
+// with its sign).  The scale bytes of a wave's 32 blocks leave as eight dwords.
+// ---------------------------------------------------------------------------------------------
+typedef float metis_f32x2_t __attribute__((ext_vector_type(2)));
+template <int MODE>
+__global__ __launch_bounds__(256) void quant_scales_dequant_kernel(const uint32_t* __restrict__ codes, const uint16_t* __restrict__ ws_amax,
+                                                                   const uint32_t* __restrict__ ws_gmax, uint32_t ngroups,
+                                                                   uint8_t* __restrict__ scales, float* __restrict__ unit_out,
+                                                                   metis_u32x4_t* __restrict__ out, uint32_t nhalves)
+{
+    __shared__ float smax[4];
+    const uint32_t step = gridDim.x * 256u;
+    uint32_t i = blockIdx.x * 256u + threadIdx.x;               // half-block index
+    uint32_t cw = 0u, aw = 0u;
+    if (i < nhalves) { cw = codes[i]; aw = ws_amax[i >> 1]; }
+    float m = 0.0f;
+    for (uint32_t g = threadIdx.x; g < ngroups; g += 256u) m = fmaxf(m, __uint_as_float(ws_gmax[g]));
+    m = wave_max(m);
+    if ((threadIdx.x & 63) == 0) smax[threadIdx.x >> 6] = m;
+    __syncthreads();
+    const float unit = tensor_unit_of<MODE>(fmaxf(fmaxf(smax[0], smax[1]), fmaxf(smax[2], smax[3])));
+    if (blockIdx.x == 0 && threadIdx.x == 0) *unit_out = unit;
+    const uint32_t lane = threadIdx.x & 63u;
+    while (i < nhalves) {
+        const uint32_t nxt = i + step;
+        uint32_t ncw = 0u, naw = 0u;
+        if (nxt < nhalves) { ncw = codes[nxt]; naw = ws_amax[nxt >> 1]; }
+        const uint32_t byte = scale_byte_of<MODE>(aw, unit);
+        const float dq = rd<MODE>(e4m3_value(byte) * unit);
+        uint32_t w[4];
+#define METIS_DQ_PAIR(J)                                                                                  \
+        {                                                                                                 \
+            const metis_f32x2_t v = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(cw, 1.0f, J);                \
+            w[J] = rb_pair(rd<MODE>(v.x * dq), rd<MODE>(v.y * dq));                                       \
+        }
+        METIS_DQ_PAIR(0) METIS_DQ_PAIR(1) METIS_DQ_PAIR(2) METIS_DQ_PAIR(3)
+#undef METIS_DQ_PAIR
+        __builtin_nontemporal_store((metis_u32x4_t){w[0], w[1], w[2], w[3]}, out + i);
+        // scale bytes: the wave's 32 blocks; lane 8 j + {0, 2, 4, 6} hold the bytes of dword j
+        const uint32_t b1 = __shfl(byte, (lane & ~7u) + 2u, 64), b2 = __shfl(byte, (lane & ~7u) + 4u, 64), b3 = __shfl(byte, (lane & ~7u) + 6u, 64);
+        if ((lane & 7u) == 0u) {
+            const uint32_t blk = i >> 1;                          // first of four consecutive blocks
+            if (2u * (blk + 3u) < nhalves) *reinterpret_cast<uint32_t*>(scales + blk) = byte | (b1 << 8) | (b2 << 16) | (b3 << 24);
+            else {
+                const uint32_t bs[4] = {byte, b1, b2, b3};
+                for (uint32_t j = 0; j < 4u && 2u * (blk + j) < nhalves; ++j) scales[blk + j] = (uint8_t)bs[j];
+            }
+        }
+        cw = ncw; aw = naw; i = nxt;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------------
 static int grid_for(uint32_t work_items, int per_cu = 8)           // 8 workgroups of 256 per CU are resident
@@ -920,6 +977,37 @@ int quantize(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, bo
         else { if (!col) METIS_Q(1, true, false); else METIS_Q(1, true, true); }
     }
 #undef METIS_Q
+}
+
+// The round trip of quant.py:6-36 from one call: codes, scale bytes, unit and the dequantized bf16 tensor, two launches
+// (phase 1 as in quantize(); phase 2 forms bytes and dequantized values together).  Contiguous bf16 rows, round to nearest.
+int quantize_dequantize_row(const void* x, int64_t rows, int64_t cols, int mode, void* codes, void* scales, float* unit, void* out,
+                            void* workspace, size_t workspace_bytes, hipStream_t st)
+{
+    if (rows < 0 || cols < 0) return METIS_E_ARG;
+    if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) return METIS_E_ARG;
+    if (cols % kBlock) return METIS_E_SHAPE;
+    if (rows == 0 || cols == 0) return METIS_OK;
+    if (!x || !codes || !scales || !unit || !out) return METIS_E_ARG;
+    if (rows * cols / kBlock >= (int64_t)1 << 30) return METIS_E_ARG;
+    if (((uintptr_t)x % 16) || ((uintptr_t)out % 16) || ((uintptr_t)codes % 8) || ((uintptr_t)scales % 8)) return METIS_E_ARG;
+    Workspace ws;
+    if (const int rc = carve_workspace(workspace, workspace_bytes, rows, cols, &ws)) return rc;
+    const uint32_t nblocks = (uint32_t)(rows * cols / kBlock);
+    const int g1 = grid_for(nblocks, kContigPerCu);
+    if (mode == 0) launch_contig<0>(x, codes, ws, nblocks, 0u, g1, st);
+    else launch_contig<1>(x, codes, ws, nblocks, 0u, g1, st);
+    if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
+    const uint32_t nhalves = nblocks * 2u;
+    // whole waves of 32 blocks per iteration: the stride is a multiple of 64 halves by construction (256 threads)
+    const int g2 = grid_for((nhalves + 3) / 4);                 // four halves per thread
+    if (mode == 0)
+        hipLaunchKernelGGL((quant_scales_dequant_kernel<0>), dim3(g2), dim3(256), 0, st, (const uint32_t*)codes, ws.amax, ws.gmax, (uint32_t)g1,
+                           (uint8_t*)scales, unit, (metis_u32x4_t*)out, nhalves);
+    else
+        hipLaunchKernelGGL((quant_scales_dequant_kernel<1>), dim3(g2), dim3(256), 0, st, (const uint32_t*)codes, ws.amax, ws.gmax, (uint32_t)g1,
+                           (uint8_t*)scales, unit, (metis_u32x4_t*)out, nhalves);
+    return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 
 // Workgroups of quant_codes_both_kernel that the current device holds at once (its LDS slabs bound them): the grid is

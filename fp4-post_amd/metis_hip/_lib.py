@@ -32,6 +32,7 @@ SIGNATURES = {
     "metis_error_string": (ctypes.c_char_p, [_i32]),
     "metis_nvfp4_workspace_bytes": (_sz, [_i64, _i64]),
     "metis_nvfp4_quant_row": (_i32, [_vp, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "metis_nvfp4_quant_dequant_row": (_i32, [_vp, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "metis_nvfp4_quant_row_static": (_i32, [_vp, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _vp]),
     "metis_nvfp4_quant_row_resident": (_i32, [_vp, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _sz, ctypes.c_uint32, _vp]),
     "metis_nvfp4_quant_col": (_i32, [_vp, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _sz, _vp]),

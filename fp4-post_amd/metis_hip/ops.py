@@ -219,6 +219,29 @@ def quantize(x: torch.Tensor, mode: int = MODE_P32, *, col: bool = False, sr: bo
     return PackedNVFP4(codes, scales, unit, prow, pcol, mode)
 
 
+def quantize_dequantize(x: torch.Tensor, mode: int = MODE_P32) -> tuple[PackedNVFP4, torch.Tensor]:
+    """(quantize(x, mode), its dequantized bf16 tensor) of a bf16 tensor with round to nearest, from one call of two
+    launches: the second forms scale bytes and dequantized values in one pass over the codes.  Same bytes as
+    quantize() followed by dequantize()."""
+    if x.dtype != torch.bfloat16 or mode not in (MODE_P32, MODE_PB16):
+        p = quantize(x, mode)
+        return p, dequantize(p, torch.bfloat16)
+    x2 = _as_2d_bf16(x)
+    rows, cols = x2.shape
+    if cols % BLOCK:
+        raise ValueError(f"NVFP4 block shape (1, 16) does not divide tensor shape {tuple(x.shape)}")
+    dev = x2.device
+    codes = torch.empty(rows, cols // 2, dtype=torch.uint8, device=dev)
+    scales = torch.empty(rows, cols // BLOCK, dtype=torch.uint8, device=dev)
+    unit = torch.empty(1, dtype=torch.float32, device=dev)
+    out = torch.empty(rows, cols, dtype=torch.bfloat16, device=dev)
+    ws = _workspace(rows, cols, dev)
+    rc = load().metis_nvfp4_quant_dequant_row(x2.data_ptr(), rows, cols, mode, codes.data_ptr(), scales.data_ptr(), unit.data_ptr(),
+                                              out.data_ptr(), ws.data_ptr(), ws.numel(), _stream())
+    check(rc, "metis_nvfp4_quant_dequant_row", x.shape)
+    return PackedNVFP4(codes, scales, unit, rows, cols, mode), out
+
+
 def quantize_both_sr(x: torch.Tensor, mode: int = MODE_P32, *, seed: int = 0, offset_row: int = 0,
                      offset_col: int = 0) -> tuple[PackedNVFP4, PackedNVFP4]:
     """(quantize(x, sr=True, offset=offset_row), quantize(x, col=True, sr=True, offset=offset_col)) from ONE pass over x:

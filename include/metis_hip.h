@@ -83,6 +83,20 @@ int metis_nvfp4_quant_row(const void *x, int64_t rows, int64_t cols, int64_t ld,
                           size_t workspace_bytes, void *stream);
 
 /*
+ * The quantize -> dequantize round trip of _nvfp4_nosr_quantize_dequantize (src/Metis/Metis/quant.py:6-36) with all
+ * three of its results from one call: packed codes, E4M3 scale bytes + unit, and the dequantized tensor
+ * out = ((v * sign) / 2) * (e4m3 * unit) (quant.py:23-26, 32-35) in bf16.  Two launches: phase 1 of
+ * metis_nvfp4_quant_row, then one pass over the codes and the parked block maxima that forms scale bytes and
+ * dequantized values together.  Same bytes as metis_nvfp4_quant_row followed by metis_nvfp4_dequant.
+ *   x      bf16 [rows, cols], contiguous
+ *   out    bf16 [rows, cols]
+ *   mode   METIS_MODE_P32 or METIS_MODE_PB16
+ */
+int metis_nvfp4_quant_dequant_row(const void *x, int64_t rows, int64_t cols, int mode, void *codes,
+                                  void *scales, float *unit, void *out, void *workspace,
+                                  size_t workspace_bytes, void *stream);
+
+/*
  * metis_nvfp4_quant_row without a workspace argument and without any allocation: the scratch (per-workgroup
  * maxima and the parked block maxima) is a static device array inside the library.  No counterpart in the
  * reference; it exists for callers that cannot allocate device memory: code under HIP graph capture, tight

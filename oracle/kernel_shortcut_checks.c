@@ -20,6 +20,10 @@
  *               threshold: literal sequence  vs  round-to-nearest-even of div3(x, s), for quotients the
  *               kernel's per-element test does not send to the literal path.
  *
+ *   table FILE  binary32 arithmetic on bf16 values with the two-operation quotient q = fma(x, rh, fma(x, rl, 0)): for every
+ *               block maximum that the table in FILE (the kernels' quotient_table.h) clears, every bf16 element of such
+ *               a block: literal sequence  vs  round-to-nearest-even of q.
+ *
  * Exit status 0 and a final line "mismatches 0" mean the shortcut is exact on the domain covered.
  */
 #include <math.h>
@@ -215,6 +219,48 @@ static long check_wide(long iters)
     return bad;
 }
 
+/* ---- binary32 arithmetic on bf16 values, two operations per quotient: the table of block maxima the kernels consult
+ * (fp4-post_amd/csrc/quotient_table.h, one bit per bf16 pattern of the maximum).  For every maximum whose bit is set: every
+ * bf16 element of such a block and the three reciprocals the hardware may return, against the literal sequence. */
+static long check_table(const char* path)
+{
+    static uint32_t words[1024];
+    FILE* f = fopen(path, "r");
+    if (!f) { printf("table: cannot open %s\n", path); return 1; }
+    char line[512];
+    int nw = 0;
+    while (fgets(line, sizeof line, f)) {
+        if (strncmp(line, "0x", 2) != 0) continue;
+        for (char* p = line; (p = strstr(p, "0x")) != NULL && nw < 1024; p += 2) words[nw++] = (uint32_t)strtoul(p, NULL, 16);
+    }
+    fclose(f);
+    if (nw != 1024) { printf("table: %d words instead of 1024\n", nw); return 1; }
+    long n = 0, bad = 0, set = 0;
+#pragma omp parallel for reduction(+ : n, bad, set) schedule(dynamic, 64)
+    for (uint32_t p = 0; p < 0x8000; ++p) {
+        if (!((words[p >> 5] >> (p & 31)) & 1u)) continue;
+        set++;
+        if (p >= 0x7f80) { bad++; continue; }                   /* infinities and NaNs must never be cleared */
+        const float amax = bits_f(p << 16);
+        volatile float s0 = amax / 6.0f;
+        volatile float s = s0 + 1e-9f;
+        const float r0 = 1.0f / s;
+        for (uint32_t xp = 0; xp <= p; ++xp) {
+            const float x = bits_f(xp << 16);
+            const int want = literal_p32(x, s);
+            for (int pert = -1; pert <= 1; ++pert) {
+                const float rh = bits_f(f_bits(r0) + pert);
+                const float rl = fmaf(-s, rh, 1.0f) * rh;
+                const float q = fmaf(x, rh, fmaf(x, rl, 0.0f));  /* x / s: half of the reference's quotient */
+                n++;
+                if (rne_grid(2.0f * q) != want) bad++;
+            }
+        }
+    }
+    printf("table: maxima cleared %ld, cases %ld mismatches %ld\n", set, n, bad);
+    return bad;
+}
+
 static long check_div6(void)
 {
     long n = 0, bad = 0;
@@ -235,6 +281,7 @@ int main(int argc, char** argv)
     if (argc >= 2 && !strcmp(argv[1], "pb16")) return check_pb16() ? 1 : 0;
     if (argc >= 3 && !strcmp(argv[1], "p32")) return check_p32(atol(argv[2])) ? 1 : 0;
     if (argc >= 3 && !strcmp(argv[1], "wide")) return check_wide(atol(argv[2])) ? 1 : 0;
-    fprintf(stderr, "usage: %s div6 | pb16 | p32 ITERS | wide ITERS\n", argv[0]);
+    if (argc >= 3 && !strcmp(argv[1], "table")) return check_table(argv[2]) ? 1 : 0;
+    fprintf(stderr, "usage: %s div6 | pb16 | p32 ITERS | wide ITERS | table QUOTIENT_TABLE_H\n", argv[0]);
     return 2;
 }

@@ -289,6 +289,39 @@ def test_full_size_config1(ops, tag, mode):
 
 
 @pytest.mark.parametrize("tag,mode", MODES)
+def test_round_trip_from_one_call(ops, tag, mode):
+    """metis_nvfp4_quant_dequant_row: codes, scale bytes, unit and the dequantized bf16 tensor of quant.py:6-36 from one
+    call whose second launch forms bytes and dequantized values together.  Config 1 at full size bit for bit against
+    the C restatement; ragged and tiny shapes against the separate calls (block counts that are not multiples of four,
+    signed zeros, an all-zero tensor)."""
+    from oracle import c_oracle as C
+    x = synthetic_activation(1001, 8192, 4096)
+    p, deq = ops.quantize_dequantize(x.cuda(), mode)
+    cc, cs, cu, _ = C.nvfp4_pack(x, mode)
+    _check_packed(p, cc, cs, cu, "config 1 round trip")
+    ob, _ = C.nvfp4_dequant(cc, cs, cu, mode)
+    assert same_bits(deq.cpu(), ob)
+    for k, (r, c) in enumerate([(1, 16), (3, 48), (7, 80), (64, 256), (1000, 96), (300, 7168), (5, 16)]):
+        y = synthetic_activation(4100 + k, r, c)
+        y[0, ::5] = -0.0
+        y[-1, 1::3] = -1e-5
+        if k == 6:
+            y.zero_()
+        y = y.cuda()
+        ref = ops.quantize(y, mode)
+        want = ops.dequantize(ref, torch.bfloat16)
+        got_p, got = ops.quantize_dequantize(y, mode)
+        _check_packed(got_p, ref.codes.cpu(), ref.scales.cpu(), ref.unit.cpu(), f"round trip {r}x{c} {tag}")
+        assert same_bits(got.cpu(), want.cpu()), (r, c, tag)
+    # the quantizer class takes this path for bf16 tensors
+    from metis_hip import quant_func
+    if mode == 1:
+        z = synthetic_activation(4200, 24, 64).reshape(8, 3, 64).cuda()
+        q = quant_func["nvfp4e2m1bnosr"].quantize_dequantize(z)
+        assert q.shape == z.shape and same_bits(q.reshape(24, 64).cpu(), ops.dequantize(ops.quantize(z, 1), torch.bfloat16).cpu())
+
+
+@pytest.mark.parametrize("tag,mode", MODES)
 def test_deferred_scale_bytes_give_the_same_packed_tensor(ops, tag, mode):
     """deferred=True runs the first launch only and parks the block maxima with the packed tensor.  Whoever reads
     `scales` / `unit` later gets the bytes of the two-launch path; the tiled expansion forms them itself (it never

@@ -42,6 +42,16 @@ def test_binary32_mode_shortcut_is_exact_outside_its_guards():
     assert 0 < guarded < 2_000_000 // 4            # the guards fire, but mostly on the adversarial families
 
 
+def test_two_operation_quotient_is_exact_for_every_block_maximum_its_table_clears():
+    """The row quantizer's fast path in binary32 arithmetic: a bit per bf16 block maximum says whether the quotient
+    fma(x, rh, fma(x, rl, 0)) + hardware conversion reproduces the literal sequence for every bf16 element of such a
+    block.  Every cleared maximum is walked here against this file's own restatement of the literal sequence
+    (9e8 cases), and the table must clear all but a handful of the maxima below 2^64."""
+    text = _run("table", os.path.join(ROOT, "fp4-post_amd", "csrc", "quotient_table.h"))
+    assert int(text.split("cleared")[1].split(",")[0]) >= 0x5f80 - 64
+    assert int(text.split("cases")[1].split()[0]) > 800_000_000
+
+
 def test_binary32_values_shortcut_is_exact_outside_its_per_quotient_test():
     """Inputs that are not bf16 values (binary32 tensors, centred residuals): div3 + round-to-nearest-even
     against the literal sequence for every quotient the kernel's low-bits test does not flag."""
