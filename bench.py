@@ -369,6 +369,24 @@ def main():
     nd_ms = region_us(torch, ndstep, qsteps, args.warmup) * 1e-3
     nd_gbs = n_bytes / (nd_ms * 1e-3) / 1e9
 
+    # the same under the reference's default arguments (mean mode): RMSNorm that leaves the column mean of its output, then
+    # the centred quantizer on the normed tensor (mean + QDQ(x - mean), bitlinear.py:311-336)
+    nm_ms = None
+    try:
+        nmean = torch.empty(4096, dtype=torch.float32, device=dev)
+        nmws = torch.empty(max(L.metis_rmsnorm_colmean_workspace_bytes(16384, 4096), 16), dtype=torch.uint8, device=dev)
+
+        def nmstep(ev):
+            rc = L.metis_rmsnorm_colmean(h.data_ptr(), gamma.data_ptr(), 1e-6, 16384, 4096, normed.data_ptr(), nmean.data_ptr(), 1, None, 0,
+                                         None, nmws.data_ptr(), nmws.numel(), st)
+            assert rc == 0
+            rc = L.metis_nvfp4_quant_centered(normed.data_ptr(), 16384, 4096, 4096, 0, nmean.data_ptr(), 0, 0, None, 0, 0, nc.data_ptr(),
+                                              ns.data_ptr(), nu.data_ptr(), nws.data_ptr(), nws.numel(), st)
+            assert rc == 0
+        nm_ms = region_us(torch, nmstep, qsteps, args.warmup) * 1e-3
+    except Exception as exc:  # an optional leg must not cost the headline line
+        nm_err = f"{type(exc).__name__}: {exc}"[:300]
+
     # ------------------------------------------------------------------ the kernels that serve two consumers from one pass
     # (config-3 activation: quantizer + rank-r projection; config-4 output gradient: row- and column-blocked packing),
     # each beside the two calls it replaces
@@ -757,6 +775,12 @@ def main():
                                        "achieved": round(n_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                        "frac": round(n_gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_NORMQ_C2,
                                        "traffic_source": TRAFFIC_SOURCE},
+                          "mean_mode": ({"workload": "the reference's default arguments: metis_rmsnorm_colmean (normed + column mean over tokens "
+                                                     "from one pass) + metis_nvfp4_quant_centered on the normed tensor (binary32 centre); four "
+                                                     "launches, priced on the same 4.5625 B/element (the quantizer's re-read of the normed "
+                                                     "tensor is not algorithmic)",
+                                         "value": round(n_bytes / (nm_ms * 1e-3) / 1e9, 1), "unit": "GB/s", "us_per_call": round(nm_ms * 1e3, 2),
+                                         "frac": round(n_bytes / (nm_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)} if nm_ms is not None else {"error": nm_err}),
                           "deferred_scale_bytes": {"workload": "the same through metis_rmsnorm_nvfp4_quant_deferred (normed + codes + parked "
                                                                "block maxima; unit and E4M3 bytes formed by the consumer); priced on the "
                                                                "same 4.5625 B/element",

@@ -49,6 +49,16 @@ int metis_nvfp4_quant_row(const void* x, int64_t rows, int64_t cols, int64_t ld,
                     workspace_bytes, (hipStream_t)stream);
 }
 
+size_t metis_rmsnorm_colmean_workspace_bytes(int64_t rows, int64_t cols) { return rmsnorm_colmean_workspace_bytes(rows, cols); }
+
+int metis_rmsnorm_colmean(const void* x, const void* gamma, float eps, int64_t rows, int64_t cols, void* normed, void* mean, int mean_dtype,
+                          const void* cached, int64_t cached_count, float* mean32, void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (mean_dtype != METIS_DTYPE_BF16 && mean_dtype != METIS_DTYPE_F32) return METIS_E_ARG;
+    return rmsnorm_colmean(x, gamma, eps, rows, cols, normed, mean, mean_dtype == METIS_DTYPE_BF16, cached, cached_count, mean32, workspace,
+                           workspace_bytes, (hipStream_t)stream);
+}
+
 int metis_nvfp4_quant_dequant_row(const void* x, int64_t rows, int64_t cols, int mode, void* codes, void* scales, float* unit,
                                   void* out, void* workspace, size_t workspace_bytes, void* stream)
 {

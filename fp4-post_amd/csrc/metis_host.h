@@ -85,6 +85,10 @@ int rquant_values(const void* xq, void* s, int64_t rows, int64_t cols, int mode,
 int rmsnorm_quantize(const void* x, const void* gamma, float eps, int64_t rows, int64_t cols, int mode, void* normed,
                      void* codes, void* scales, float* unit, void* workspace, size_t workspace_bytes, hipStream_t st,
                      bool deferred = false);
+// RMSNorm that also leaves the column mean of its output (mean mode); rmsnorm_quant.hip
+size_t rmsnorm_colmean_workspace_bytes(int64_t rows, int64_t cols);
+int rmsnorm_colmean(const void* x, const void* gamma, float eps, int64_t rows, int64_t cols, void* normed, void* mean, int mean_bf16,
+                    const void* cached, int64_t cached_count, float* mean32, void* workspace, size_t workspace_bytes, hipStream_t st);
 int gemm_nvfp4(const void* a_codes, const void* a_scales, const float* a_unit, const void* b_codes, const void* b_scales,
                const float* b_unit, int64_t M, int64_t N, int64_t K, const void* t, const void* u, int64_t r,
                const void* bias, void* out, int out_dtype, hipStream_t st, void* workspace = nullptr,

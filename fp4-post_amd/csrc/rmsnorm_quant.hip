@@ -220,6 +220,190 @@ __global__ __launch_bounds__(256) void rmsnorm_quant_rows_kernel(const uint4* __
     publish_group_max(gmax, ws_gmax, fill_to);
 }
 
+// ---------------------------------------------------------------------------------------------
+// RMSNorm with the column sums of its output, for the mean mode (the reference's default arguments,
+// src/grpo/grpo.py:66-69): there the activation is quantized as mean + QDQ(x - mean) with the column mean over tokens
+// (src/Metis/Metis/bitlinear.py:311-336), so the quantizer needs the mean of the WHOLE normed tensor before it can
+// start.  This kernel is the norm of rmsnorm_quant_rows_kernel (one wave per row, whole-line accesses) and leaves, per
+// workgroup, the sums of the normed bf16 values of its rows, column by column, in a fixed order: rows in order within
+// a wave, then the four waves in order.  rmsnorm_colmean_finish_kernel adds the workgroups' partial rows in order and
+// applies the mean's division and rounding (and the running mean of decode calls) as column_mean_finish_kernel does.
+// ---------------------------------------------------------------------------------------------
+template <int NL>
+__global__ __launch_bounds__(256) void rmsnorm_colsum_rows_kernel(const uint4* __restrict__ x, const uint4* __restrict__ gamma, float eps,
+                                                                  uint32_t rows, uint32_t cols, metis_u32x4_t* __restrict__ normed,
+                                                                  float* __restrict__ partial)
+{
+    __shared__ uint4 g_a[NL * 64], g_b[NL * 64];
+    __shared__ float4 sums[NL * 64][2];                        // column sums of the workgroup, chunk by chunk
+    const uint32_t cpr = cols / 8u;
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const float fcols = (float)cols;
+    const uint32_t wstep = gridDim.x * 4u;
+    uint32_t row = blockIdx.x * 4u + wave;
+    uint4 raw[NL];
+    auto request = [&](uint32_t r) {
+#pragma unroll
+        for (int i = 0; i < NL; ++i) {
+            const uint32_t c = i * 64u + lane;
+            if (c < cpr) raw[i] = x[(size_t)r * cpr + c];
+        }
+    };
+#pragma unroll
+    for (int i = 0; i < NL; ++i) raw[i] = make_uint4(0u, 0u, 0u, 0u);
+    if (row < rows) request(row);
+    for (uint32_t c = threadIdx.x; c < cpr; c += 256u) {
+        const uint4 g = gamma[c];
+        g_a[c] = make_uint4(g.x & 0xffffu, g.x & 0xffff0000u, g.y & 0xffffu, g.y & 0xffff0000u);
+        g_b[c] = make_uint4(g.z & 0xffffu, g.z & 0xffff0000u, g.w & 0xffffu, g.w & 0xffff0000u);
+    }
+    __syncthreads();
+    float acc[NL][8];
+#pragma unroll
+    for (int i = 0; i < NL; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[i][j] = 0.0f;
+    for (; row < rows; row += wstep) {
+        uint4 cur[NL];
+        float ss = 0.0f;
+#pragma unroll
+        for (int i = 0; i < NL; ++i) {
+            cur[i] = raw[i];
+            ss = dot2_bf16(cur[i].x, cur[i].x, ss);
+            ss = dot2_bf16(cur[i].y, cur[i].y, ss);
+            ss = dot2_bf16(cur[i].z, cur[i].z, ss);
+            ss = dot2_bf16(cur[i].w, cur[i].w, ss);
+        }
+        if (row + wstep < rows) request(row + wstep);
+        const float total = wave_sum_dpp(ss);
+        const float rstd = 1.0f / sqrtf(total / fcols + eps);
+#pragma unroll
+        for (int i = 0; i < NL; ++i) {
+            const uint32_t c = i * 64u + lane;
+            if (i * 64u >= cpr) break;
+            if (c < cpr) {
+                const uint32_t in[4] = {cur[i].x, cur[i].y, cur[i].z, cur[i].w};
+                const uint4 ga = g_a[c], gb = g_b[c];
+                const uint32_t gl[4] = {ga.x, ga.z, gb.x, gb.z}, gh[4] = {ga.y, ga.w, gb.y, gb.w};
+                uint32_t w[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t h = rb_pair(bf16_lo(in[j]) * rstd, bf16_hi(in[j]) * rstd);
+                    w[j] = rb_pair(dot2_bf16(h, gl[j], 0.0f), dot2_bf16(h, gh[j], 0.0f));
+                    acc[i][2 * j] += bf16_lo(w[j]);
+                    acc[i][2 * j + 1] += bf16_hi(w[j]);
+                }
+                __builtin_nontemporal_store((metis_u32x4_t){w[0], w[1], w[2], w[3]}, normed + (size_t)row * cpr + c);
+            }
+        }
+    }
+    // the four waves' sums, added in wave order
+#pragma unroll 1
+    for (uint32_t v = 0; v < 4u; ++v) {
+        if (wave == v) {
+#pragma unroll
+            for (int i = 0; i < NL; ++i) {
+                const uint32_t c = i * 64u + lane;
+                if (c < cpr) {
+                    float4 lo = make_float4(acc[i][0], acc[i][1], acc[i][2], acc[i][3]), hi = make_float4(acc[i][4], acc[i][5], acc[i][6], acc[i][7]);
+                    if (v) {
+                        const float4 pl = sums[c][0], ph = sums[c][1];
+                        lo = make_float4(pl.x + lo.x, pl.y + lo.y, pl.z + lo.z, pl.w + lo.w);
+                        hi = make_float4(ph.x + hi.x, ph.y + hi.y, ph.z + hi.z, ph.w + hi.w);
+                    }
+                    sums[c][0] = lo;
+                    sums[c][1] = hi;
+                }
+            }
+        }
+        __syncthreads();
+    }
+    float4* out = reinterpret_cast<float4*>(partial + (size_t)blockIdx.x * cols);
+    for (uint32_t q = threadIdx.x; q < cpr * 2u; q += 256u) out[q] = sums[q >> 1][q & 1u];
+}
+
+constexpr int kColmeanBatch = 8;
+template <bool OUT_BF16>
+__global__ __launch_bounds__(256) void rmsnorm_colmean_finish_kernel(const float* __restrict__ partial, uint32_t slabs, uint32_t cols,
+                                                                     float count, void* __restrict__ out, const void* __restrict__ cached,
+                                                                     float cached_count, float rows_f, float* __restrict__ out32)
+{
+    __shared__ float part[4][64];
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t c = blockIdx.x * 64u + lane;
+    float s = 0.0f;
+    if (c < cols) {
+        // wave w adds the partial rows w, w + 4, ... in order, kColmeanBatch loads in flight at a time
+        for (uint32_t k0 = wave; k0 < slabs; k0 += 4u * kColmeanBatch) {
+            float v[kColmeanBatch];
+#pragma unroll
+            for (int b = 0; b < kColmeanBatch; ++b) {
+                const uint32_t k = k0 + 4u * b;
+                v[b] = k < slabs ? partial[(size_t)k * cols + c] : 0.0f;
+            }
+#pragma unroll
+            for (int b = 0; b < kColmeanBatch; ++b) s += v[b];
+        }
+    }
+    part[wave][lane] = s;
+    __syncthreads();
+    if (wave != 0 || c >= cols) return;
+    s = (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]);
+    auto rnd = [](float x) { return OUT_BF16 ? __uint_as_float(bf16_bits(x) << 16) : x; };
+    float m = rnd(s / count);
+    if (cached) {                                              // weighted running mean of decode calls, bitlinear.py:316-323
+        const float cm = OUT_BF16 ? __uint_as_float((uint32_t)static_cast<const uint16_t*>(cached)[c] << 16)
+                                  : static_cast<const float*>(cached)[c];
+        const float a = rnd(cm * cached_count), b = rnd(m * rows_f);
+        m = rnd(rnd(a + b) / (cached_count + rows_f));
+    }
+    if (OUT_BF16) static_cast<uint16_t*>(out)[c] = (uint16_t)bf16_bits(m);
+    else static_cast<float*>(out)[c] = m;
+    if (out32) out32[c] = m;
+}
+
+static int colmean_grid(int64_t rows)
+{
+    int64_t g = (rows + 3) / 4;
+    const int64_t cap = (int64_t)device_cus() * 2;           // the column sums cost registers: two waves per SIMD
+    if (g > cap) g = cap;
+    return g < 1 ? 1 : (int)g;
+}
+
+size_t rmsnorm_colmean_workspace_bytes(int64_t rows, int64_t cols)
+{
+    if (rows <= 0 || cols <= 0) return 0;
+    return (size_t)colmean_grid(rows) * (size_t)cols * sizeof(float);
+}
+
+int rmsnorm_colmean(const void* x, const void* gamma, float eps, int64_t rows, int64_t cols, void* normed, void* mean, int mean_bf16,
+                    const void* cached, int64_t cached_count, float* mean32, void* workspace, size_t workspace_bytes, hipStream_t st)
+{
+    if (rows <= 0 || cols <= 0) return METIS_E_ARG;
+    if (cols % kBlock) return METIS_E_SHAPE;
+    if (cols > 4096) return METIS_E_ARG;                      // one wave per row
+    if (!x || !gamma || !normed || !mean) return METIS_E_ARG;
+    if (cached && (cached_count < 0 || cached_count > (1 << 24) || ((uintptr_t)cached % (mean_bf16 ? 2 : 4)))) return METIS_E_ARG;
+    if (((uintptr_t)x % 16) || ((uintptr_t)gamma % 16) || ((uintptr_t)normed % 16) || ((uintptr_t)mean % 4) || ((uintptr_t)mean32 % 4)) return METIS_E_ARG;
+    if (!workspace || ((uintptr_t)workspace % 16) || workspace_bytes < rmsnorm_colmean_workspace_bytes(rows, cols)) return METIS_E_WORKSPACE;
+    const int g = colmean_grid(rows);
+    const int nl = (int)((cols / 8 + 63) / 64);
+    float* partial = static_cast<float*>(workspace);
+#define METIS_RC(NL) hipLaunchKernelGGL((rmsnorm_colsum_rows_kernel<NL>), dim3(g), dim3(256), 0, st, (const uint4*)x, (const uint4*)gamma, eps, \
+        (uint32_t)rows, (uint32_t)cols, (metis_u32x4_t*)normed, partial)
+    if (nl <= 2) METIS_RC(2); else if (nl <= 4) METIS_RC(4); else METIS_RC(8);
+#undef METIS_RC
+    if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
+    const dim3 g2((unsigned)((cols + 63) / 64));
+    if (mean_bf16)
+        hipLaunchKernelGGL(rmsnorm_colmean_finish_kernel<true>, g2, dim3(256), 0, st, partial, (uint32_t)g, (uint32_t)cols, (float)rows, mean, cached,
+                           (float)cached_count, (float)rows, mean32);
+    else
+        hipLaunchKernelGGL(rmsnorm_colmean_finish_kernel<false>, g2, dim3(256), 0, st, partial, (uint32_t)g, (uint32_t)cols, (float)rows, mean, cached,
+                           (float)cached_count, (float)rows, mean32);
+    return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
+}
+
 // deferred: stop after the main kernel; `workspace` is then the caller-owned parked data of the deferred form
 // (nvfp4_quant.hip) and scales / unit are not written.
 int rmsnorm_quantize(const void* x, const void* gamma, float eps, int64_t rows, int64_t cols, int mode, void* normed,

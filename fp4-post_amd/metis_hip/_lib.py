@@ -43,6 +43,8 @@ SIGNATURES = {
     "metis_nvfp4_rquant": (_i32, [_vp, _vp, _i64, _i64, _i32, _vp, _vp, _vp]),
     "metis_nvfp4_dequant": (_i32, [_vp, _vp, _vp, _i64, _i64, _i32, _vp, _i32, _vp]),
     "metis_rmsnorm_nvfp4_quant": (_i32, [_vp, _vp, _f32, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "metis_rmsnorm_colmean_workspace_bytes": (_sz, [_i64, _i64]),
+    "metis_rmsnorm_colmean": (_i32, [_vp, _vp, _f32, _i64, _i64, _vp, _vp, _i32, _vp, _i64, _vp, _vp, _sz, _vp]),
     "metis_linear_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _i32, _vp]),
     "metis_nvfp4_expand_f16": (_i32, [_vp, _vp, _i64, _i64, _vp, _vp]),
     "metis_linear_fwd_expanded": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _i32, _vp]),

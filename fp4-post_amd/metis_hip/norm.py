@@ -17,6 +17,7 @@ from torch import nn
 
 from . import ops
 from ._lib import MODE_P32, MODE_PB16
+from .ops import CenteredNVFP4
 from .bitlinear import BitLinear, LinearLowbitFunction
 from .quant import is_hip_nvfp4
 
@@ -72,20 +73,53 @@ class FusedRMSNormQuant(nn.Module):
         h = h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + self.variance_epsilon)
         return self.weight * h.to(dtype)
 
+    def _mean_mode(self, x: torch.Tensor):
+        """The reference's default arguments (mean mode, src/grpo/grpo.py:66-69): the group's activation is
+        mean + QDQ(normed - mean) with the column mean over tokens (src/Metis/Metis/bitlinear.py:311-336).  One pass
+        over x writes the normed tensor and leaves its column sums; the centred quantizer then reads the normed tensor.
+        The running mean of single-token decode calls is kept in the group's cache exactly as the first projection of
+        the group would keep it."""
+        F = LinearLowbitFunction
+        cd = F.compute_dtype
+        cols = x.shape[-1]
+        rows = x.numel() // cols
+        group = self.group
+        cache, key = group["mean_cache"], f"{group['name']}.shared"
+        seq_len = x.shape[1] if x.dim() == 3 else x.shape[0]
+        running = seq_len == 1 and key in cache
+        cached_mean, cached_count = cache[key] if running else (None, 0)
+        if cached_count + rows > 2 ** 24:
+            return None
+        normed, me, me32 = ops.rmsnorm_colmean(x, self.weight, self.variance_epsilon, cd, cached_mean, cached_count)
+        cache[key] = (me.detach().unsqueeze(0), cached_count + rows)
+        more = {"deferred": True} if (F._bf16_rounding() and me.dtype == torch.bfloat16) else {}
+        packed = CenteredNVFP4(F.q_forward_input.pack(normed, arith=cd, center=me, **more), me, me32)
+        return normed, packed
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         F = LinearLowbitFunction
         cols = x.shape[-1]
         fused = (x.is_cuda and x.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16 and cols % 32 == 0
-                 and cols <= 16384 and is_hip_nvfp4(F.q_forward_input) and not F.enable_activation_svd
-                 and not F.enable_nv_recipe)
+                 and cols <= 16384 and is_hip_nvfp4(F.q_forward_input) and not F.enable_nv_recipe and x.numel() > 0)
+        mean_mode = fused and F.enable_activation_svd
+        if mean_mode:
+            fused = (F._mean_mode_packable() and cols <= 4096 and F.compute_dtype in (torch.float32, torch.bfloat16)
+                     and self.group.get("mean_cache") is not None)
         if not fused:
             return self._plain(x)
         mode = MODE_P32 if F.compute_dtype == torch.float32 else MODE_PB16
         with torch.no_grad():
-            # the tiled expansion (256 rows or more) and the ready decode operands of bf16 arithmetic form the scale bytes
-            # themselves
-            normed, packed = ops.rmsnorm_quantize(x, self.weight, self.variance_epsilon, mode,
-                                                  deferred=x.numel() // cols >= 256 or F._bf16_rounding())
+            if mean_mode:
+                got = self._mean_mode(x)
+                if got is None:
+                    return self._plain(x)
+                normed, packed = got
+                packed.residual.shared = True
+            else:
+                # the tiled expansion (256 rows or more) and the ready decode operands of bf16 arithmetic form the scale
+                # bytes themselves
+                normed, packed = ops.rmsnorm_quantize(x, self.weight, self.variance_epsilon, mode,
+                                                      deferred=x.numel() // cols >= 256 or F._bf16_rounding())
         normed = normed.reshape(x.shape)
         out = _NormedWithGrad.apply(x, self.weight, normed, self.variance_epsilon) if torch.is_grad_enabled() and (
             x.requires_grad or self.weight.requires_grad) else normed
@@ -96,7 +130,8 @@ class FusedRMSNormQuant(nn.Module):
                 group["input_ref"] = None
                 group["quantized_input"] = None
 
-        packed.shared = True                     # read by every member of the group: its tiled expansion is kept while it lives
+        if not mean_mode:
+            packed.shared = True                 # read by every member of the group: its tiled expansion is kept while it lives
         group["input_ref"] = weakref.ref(out, clear)
         group["quantized_input"] = packed
         return out

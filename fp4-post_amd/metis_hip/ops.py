@@ -661,6 +661,37 @@ def rmsnorm_quantize(x: torch.Tensor, gamma: torch.Tensor, eps: float, mode: int
 
 
 @functools.lru_cache(maxsize=16)
+def rmsnorm_colmean(x: torch.Tensor, gamma: torch.Tensor, eps: float, mean_dtype: torch.dtype = torch.float32,
+                    cached: torch.Tensor | None = None, cached_count: int = 0):
+    """RMSNorm for the mean mode: (normed bf16 [R, C], column mean of normed over its rows in mean_dtype, the same as
+    float32) from one pass over x plus one small kernel.  cached / cached_count: the weighted running mean of
+    single-token decode calls, as column_mean_running.  C <= 4096."""
+    x2 = _as_2d_bf16(x)
+    rows, cols = x2.shape
+    if cols % BLOCK:
+        raise ValueError(f"NVFP4 block shape (1, 16) does not divide tensor shape {tuple(x.shape)}")
+    if mean_dtype not in (torch.bfloat16, torch.float32):
+        raise ValueError("rmsnorm_colmean: the mean is bfloat16 or float32")
+    dev = x2.device
+    g = gamma.to(device=dev, dtype=torch.bfloat16).contiguous()
+    normed = torch.empty(rows, cols, dtype=torch.bfloat16, device=dev)
+    me = torch.empty(cols, dtype=mean_dtype, device=dev)
+    me32 = me if mean_dtype == torch.float32 else torch.empty(cols, dtype=torch.float32, device=dev)
+    L = load()
+    ws = torch.empty(max(L.metis_rmsnorm_colmean_workspace_bytes(rows, cols), 16), dtype=torch.uint8, device=dev)
+    cp = None
+    if cached is not None:
+        cached = cached.reshape(-1).to(device=dev, dtype=mean_dtype).contiguous()
+        if cached.numel() != cols:
+            raise ValueError(f"cached mean must have one value per column ({cols}), got {cached.numel()}")
+        cp = cached.data_ptr()
+    rc = L.metis_rmsnorm_colmean(x2.data_ptr(), g.data_ptr(), float(eps), rows, cols, normed.data_ptr(), me.data_ptr(),
+                                 DTYPE_F32 if mean_dtype == torch.float32 else DTYPE_BF16, cp, int(cached_count),
+                                 None if me32 is me else me32.data_ptr(), ws.data_ptr(), ws.numel(), _stream())
+    check(rc, "metis_rmsnorm_colmean", x.shape)
+    return normed, me, me32
+
+
 def _device_cus(device_index: int) -> int:
     return int(torch.cuda.get_device_properties(device_index).multi_processor_count)
 

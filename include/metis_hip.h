@@ -225,6 +225,28 @@ int metis_rmsnorm_nvfp4_quant(const void *x, const void *gamma, float eps, int64
                               float *unit, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * RMSNorm for the mean mode, the reference's default arguments (src/grpo/grpo.py:66-69): there the activation that
+ * enters a projection group is quantized as mean + QDQ(x - mean) with the column mean over tokens
+ * (src/Metis/Metis/bitlinear.py:311-336), so the quantizer cannot start before the whole normed tensor's mean is
+ * known.  This call is the norm of metis_rmsnorm_nvfp4_quant (same arithmetic, src/Metis/models/llama.py:23-31) and
+ * hands back the normed bf16 tensor together with its column mean -- `input_flat.mean(dim=0)` of bitlinear.py:326,
+ * binary32 sums in a fixed order -- from one pass over x; metis_nvfp4_quant_centered then takes normed and mean.
+ *   x       bf16 [rows, cols], cols <= 4096 and a multiple of 16; gamma bf16 [cols]
+ *   normed  bf16 [rows, cols]
+ *   mean    [cols] in mean_dtype (METIS_DTYPE_F32 for binary32 arithmetic, METIS_DTYPE_BF16 for bf16 arithmetic: the
+ *           division by rows and every later operation are rounded to it)
+ *   cached, cached_count   (optional) the weighted running mean of single-token decode calls, bitlinear.py:316-323:
+ *           mean = (cached * cached_count + this_mean * rows) / (cached_count + rows)
+ *   mean32  (optional) the same values once more as binary32
+ *   workspace   metis_rmsnorm_colmean_workspace_bytes(rows, cols) bytes, 16-byte aligned, no initialisation needed
+ */
+size_t metis_rmsnorm_colmean_workspace_bytes(int64_t rows, int64_t cols);
+int metis_rmsnorm_colmean(const void *x, const void *gamma, float eps, int64_t rows, int64_t cols,
+                          void *normed, void *mean, int mean_dtype, const void *cached,
+                          int64_t cached_count, float *mean32, void *workspace, size_t workspace_bytes,
+                          void *stream);
+
+/*
  * Block-scaled NVFP4 GEMM with an optional bf16 low-rank extension and bias:
  *   out[M,N] = ua*ub * sum_k deq(A)[m,k] * deq(B)[n,k]  +  sum_j T[m,j] * U[n,j]  +  bias[n]
  * A (M x K) and B (N x K) are packed NVFP4 with blocks of 16 along K; *ua, *ub are their units.

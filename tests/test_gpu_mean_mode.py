@@ -394,6 +394,110 @@ def test_qwen2_decoder_layer_under_the_reference_default_arguments(monkeypatch):
     assert rel_fro(gx_packed, xg.grad.detach().float().cpu()) < 0.2      # both carry independent stochastic rounding
 
 
+@pytest.mark.parametrize("rows,cols", [(64, 512), (333, 1536), (4096, 3584), (16384, 4096), (7, 48), (1, 256)])
+def test_rmsnorm_with_column_mean(rows, cols):
+    """metis_rmsnorm_colmean: the normed tensor is that of the fused RMSNorm -> NVFP4 kernel, bit for bit; its column
+    mean over tokens agrees with a double-precision mean of that tensor to binary32 / bf16 rounding; the running mean of
+    decode calls follows the reference's tensor expression bit for bit given this call's mean; and the whole chain
+    against the oracle: O.rmsnorm within the norm's tolerance, then me + QDQ(x - me) with codes and scale bytes
+    bit-exact on the kernel's own normed tensor and mean."""
+    from metis_hip import ops
+    from oracle import metis_oracle as O
+    x = _offset_activation(900 + rows, rows, cols)
+    gamma = (1 + 0.1 * torch.randn(cols, generator=torch.Generator().manual_seed(9))).bfloat16()
+    ref_normed, _ = ops.rmsnorm_quantize(x.cuda(), gamma.cuda(), 1e-6, 0)
+    normed, me, me32 = ops.rmsnorm_colmean(x.cuda(), gamma.cuda(), 1e-6, torch.float32)
+    assert torch.equal(normed, ref_normed) and me32 is me
+    assert rel_fro(normed.cpu(), O.rmsnorm(x, gamma, 1e-6)) <= 2e-3
+    want = normed.cpu().double().mean(dim=0)
+    assert float((me.cpu().double() - want).abs().max()) <= 1e-6 * float(want.abs().max() + 1)
+    again = ops.rmsnorm_colmean(x.cuda(), gamma.cuda(), 1e-6, torch.float32)[1]
+    assert torch.equal(again, me)                                  # fixed summation order: the same bits call after call
+    # centred quantizer on the kernel's own outputs, against the oracle formula
+    p = ops.quantize(normed, 0, center=me)
+    codes, scales, unit, _ = O.nvfp4_pack(normed.cpu().float() - me.cpu())
+    _check(p, codes, scales, unit, f"fused norm, mean mode {rows}x{cols}")
+    # bf16 arithmetic: every operation of the mean rounded to bf16
+    n16, me16, me16_32 = ops.rmsnorm_colmean(x.cuda(), gamma.cuda(), 1e-6, torch.bfloat16)
+    assert torch.equal(n16, normed) and me16.dtype == torch.bfloat16 and torch.equal(me16_32, me16.float())
+    assert float((me16.cpu().double() - want).abs().max()) <= 2 ** -8 * float(want.abs().max() + 1)
+    p16 = ops.quantize(normed, 1, center=me16)
+    codes, scales, unit, _ = O.nvfp4_pack(normed.cpu() - me16.cpu())
+    _check(p16, codes, scales, unit, f"fused norm, mean mode, bf16 arithmetic {rows}x{cols}")
+    # running mean (decode calls)
+    for dtype, this_mean in ((torch.float32, me.cpu()), (torch.bfloat16, me16.cpu())):
+        cached = (torch.randn(cols, generator=torch.Generator().manual_seed(11)) * 0.3).to(dtype)
+        for count in (64, 1_000_003):
+            _, run, run32 = ops.rmsnorm_colmean(x.cuda(), gamma.cuda(), 1e-6, dtype, cached.cuda(), count)
+            wantr = (cached * count + this_mean * rows) / (count + rows)
+            assert wantr.dtype == dtype and torch.equal(run.cpu(), wantr) and torch.equal(run32.cpu(), wantr.float())
+
+
+@pytest.mark.parametrize("compute", [torch.float32, torch.bfloat16])
+def test_fused_norm_feeds_the_projection_groups_under_the_reference_default_arguments(monkeypatch, compute):
+    """MetisArgs() as the reference constructs it (mean mode) with the norms fused into the q/k/v and gate/up groups:
+    no torch RMSNorm runs (the module's eager fallback is made to raise), the group's activation arrives as a
+    CenteredNVFP4 whose mean is the column mean of the normed tensor, the running mean of decode calls lands in the
+    group's cache, and the layer's output agrees with the same layer with unfused norms."""
+    pytest.importorskip("transformers")
+    from transformers.models.qwen2.modeling_qwen2 import Qwen2Config, Qwen2DecoderLayer, Qwen2RotaryEmbedding
+    from metis_hip import BitLinear, LinearLowbitFunction as F, MetisArgs, replace_linear_with_metis
+    from metis_hip.norm import FusedRMSNormQuant, fuse_rmsnorm_into_groups
+    from metis_hip.ops import CenteredNVFP4
+    torch.manual_seed(0)
+    cfg = Qwen2Config(hidden_size=256, intermediate_size=512, num_attention_heads=4, num_key_value_heads=2,
+                      num_hidden_layers=1, vocab_size=128, max_position_embeddings=256)
+    cfg._attn_implementation = "eager"
+
+    def build(fuse):
+        torch.manual_seed(1)
+        layer = Qwen2DecoderLayer(cfg, layer_idx=0).to(torch.bfloat16).cuda()
+        for p in layer.parameters():
+            if p.dim() == 2:
+                torch.nn.init.normal_(p, std=0.02)
+        holder = torch.nn.ModuleDict({"layer": layer})
+        args = MetisArgs(forward_svd_rank=32)
+        replace_linear_with_metis(holder, torch.bfloat16, args, compute_dtype=compute)
+        if fuse:
+            assert fuse_rmsnorm_into_groups(holder) == 2
+        return holder
+
+    x = (torch.randn(2, 64, 256, device="cuda") + 1.5 * torch.randn(1, 1, 256, device="cuda")).bfloat16()
+    pos = torch.arange(64, device="cuda").unsqueeze(0).expand(2, -1)
+    pe = Qwen2RotaryEmbedding(cfg).cuda()(x, pos)
+    plain, fused = build(False), build(True)
+    assert sum(isinstance(m, FusedRMSNormQuant) for m in fused.modules()) == 2
+    real_plain = FusedRMSNormQuant._plain
+
+    def plain_only_for_binary32(self, t):
+        # with compute_dtype=float32 the residual stream after the first block is binary32 (the reference's forward returns
+        # its compute dtype): that input keeps the eager norm; a bf16 input must never reach it
+        assert t.dtype != torch.bfloat16, "eager RMSNorm ran on a bf16 tensor"
+        return real_plain(self, t)
+    monkeypatch.setattr(FusedRMSNormQuant, "_plain", plain_only_for_binary32)
+    seen = []
+    real = BitLinear._get_shared_quantized_input
+    monkeypatch.setattr(BitLinear, "_get_shared_quantized_input", lambda self, t: (seen.append(real(self, t)), seen[-1])[1])
+    with torch.no_grad():
+        want = plain["layer"](x, position_embeddings=pe, attention_mask=None, position_ids=pos)
+        seen.clear()
+        got = fused["layer"](x, position_embeddings=pe, attention_mask=None, position_ids=pos)
+    want, got = (t[0] if isinstance(t, tuple) else t for t in (want, got))
+    assert all(isinstance(q, CenteredNVFP4) for q in seen) and len(seen) == 4     # q/k/v as one group call, o, gate/up, down
+    # the rows' sums of squares are taken in another order than torch's: single roundings of the normed tensor may differ
+    assert rel_fro(got.float().cpu(), want.float().cpu()) <= 2e-3
+    group = fused["layer"].self_attn.q_proj.activation_group
+    key = f"{group['name']}.shared"
+    assert key in group["mean_cache"] and group["mean_cache"][key][1] == 128
+    # a decode call updates the running mean through the same kernel
+    xd = x[:, :1].contiguous()
+    with torch.no_grad():
+        fused["layer"](xd, position_embeddings=tuple(t[:, :1] for t in pe), attention_mask=None, position_ids=pos[:, :1])
+    assert group["mean_cache"][key][1] == 130
+    F.enable_activation_svd = False
+    F.enable_backward_svd = False
+
+
 def _mean_golden():
     import os
     import numpy as np
