@@ -438,9 +438,10 @@ def main():
             def member_array(idx):
                 arr = (_ml.LinearMember * len(idx))()
                 for j, i_ in enumerate(idx):
+                    # cached weights: packed, plus the same bytes in the decode layout that the decode-sized kernel streams as whole lines
                     arr[j] = _ml.LinearMember(ws_[i_].codes.data_ptr(), ws_[i_].scales.data_ptr(), ws_[i_].unit.data_ptr(),
                                               lows[i_][0].data_ptr(), lows[i_][1].data_ptr(), 64, None, outs[i_].data_ptr(),
-                                              shapes[i_][0], 0, 0)
+                                              shapes[i_][0], 0, 0, ops.decode_weight(ws_[i_]).data_ptr())
                 return arr
             # projection groups share their activation: q/k/v in one call, o, gate/up in one call, down
             calls = [(3584, member_array([0, 1, 2])), (3584, member_array([3])), (3584, member_array([4, 5])),
@@ -503,7 +504,7 @@ def main():
             d_bf16_op_us = replay_us(lambda: layer(bf16=2))
             d_bytes = sum(n_ * k_ for n_, k_ in shapes) * (0.5 + 1.0 / 16)
             d_flops = sum(2.0 * 64 * n_ * k_ for n_, k_ in shapes)
-            dec = {"workload": "config 5 decode: 7 projections of a Qwen2.5-7B layer, M=64, r=64, packed weights; q/k/v and gate/up as grouped calls (graph replay)",
+            dec = {"workload": "config 5 decode: 7 projections of a Qwen2.5-7B layer, M=64, r=64, packed weights cached in the decode layout; q/k/v and gate/up as grouped calls (graph replay)",
                    "us_per_layer": round(d_us, 1), "tflops": round(d_flops / d_us / 1e6, 1),
                    "roofline": {"bound": "hbm", "kernel": "gemm_nvfp4_skinny_grouped_kernel", "achieved": round(d_bytes / d_us / 1e3, 1),
                                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(d_bytes / d_us / 1e3 / HBM_PEAK_GBS, 4),

@@ -49,6 +49,15 @@ int metis_nvfp4_quant_row(const void* x, int64_t rows, int64_t cols, int64_t ld,
                     workspace_bytes, (hipStream_t)stream);
 }
 
+size_t metis_linear_member_size(void) { return sizeof(metis_linear_member); }
+
+size_t metis_nvfp4_decode_weight_bytes(int64_t N, int64_t K) { return decode_weight_bytes(N, K); }
+
+int metis_nvfp4_decode_weight(const void* codes, const void* scales, int64_t N, int64_t K, void* out, void* stream)
+{
+    return decode_weight(codes, scales, N, K, out, (hipStream_t)stream);
+}
+
 size_t metis_rmsnorm_colmean_workspace_bytes(int64_t rows, int64_t cols) { return rmsnorm_colmean_workspace_bytes(rows, cols); }
 
 int metis_rmsnorm_colmean(const void* x, const void* gamma, float eps, int64_t rows, int64_t cols, void* normed, void* mean, int mean_dtype,

@@ -61,6 +61,28 @@ __device__ __forceinline__ void load_run(RunRegs<C>& r, const uint8_t* codes, co
     }
 }
 
+// The same with the distance between a run's 16-byte pieces as a run-time value: 16 for a row-major packed tensor, 1024
+// for the decode layout of a weight (decode_weight_kernel: the pieces of the 64 lanes of a wave lie side by side, so one
+// load instruction reads a KiB of consecutive bytes instead of 16 bytes from each of 64 rows).
+template <int C>
+__device__ __forceinline__ void load_run_strided(RunRegs<C>& r, const uint8_t* codes, int piece_stride, const uint8_t* scales)
+{
+#pragma unroll
+    for (int c = 0; c < C; ++c) r.c[c] = *reinterpret_cast<const uint4*>(codes + (int64_t)c * piece_stride);
+    if constexpr (C == 1) r.sc[0] = *reinterpret_cast<const uint16_t*>(scales);
+    else if constexpr (C == 2) r.sc[0] = *reinterpret_cast<const uint32_t*>(scales);
+    else {
+        const uint2 w = *reinterpret_cast<const uint2*>(scales);
+        r.sc[0] = w.x; r.sc[1] = w.y;
+    }
+}
+
+// Decode layout of a packed weight [N, K], K % 256 == 0: for column tile T (rows 32 T .. 32 T + 31) and step `it`
+// (256 elements of K) one block of kDecodeBlock bytes: four KiB of codes -- piece j of lane l = (h << 5 | row) at
+// j * 1024 + l * 16 holds the row's code bytes [it * 128 + h * 64 + 16 j, + 16) -- then 512 bytes of scale bytes, lane l
+// at 4096 + l * 8 holding the row's bytes [it * 16 + h * 8, + 8).  Rows past N are zero.  0.5625 B per element, as packed.
+constexpr int kDecodeBlock = 4096 + 512;
+
 // MFMA operand m (8 elements) of a run
 template <int C>
 __device__ __forceinline__ half8_t run_operand(const RunRegs<C>& r, int m)
@@ -106,6 +128,7 @@ struct SkinnyMember {
     void* out;
     float* part;                 // split-K partial sums of this member, nullptr when K is not split
     int N, r, tile_end, bias_f32, ldt;
+    int decode;                  // b_codes is the weight in the decode layout (b_scales unused)
 };
 struct SkinnyGroup {
     SkinnyMember m[kMaxGroupMembers];

@@ -599,15 +599,23 @@ __device__ __forceinline__ void skinny_tile(
     const uint8_t* __restrict__ b_codes, const uint8_t* __restrict__ b_scales, const float* __restrict__ b_unit,
     int M, int N, int K, const uint16_t* __restrict__ t, const uint16_t* __restrict__ u, int r,
     const uint16_t* __restrict__ bias, void* __restrict__ out, int bias_f32, int n0, int ldt,
-    float* __restrict__ part, int nsplit, const float* __restrict__ center = nullptr)
+    float* __restrict__ part, int nsplit, const float* __restrict__ center = nullptr, int decode = 0)
 {
     __shared__ __attribute__((aligned(16))) float red[WAVES][TM * 16][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, hi = lane >> 5;
     const int m0 = blockIdx.y * 32 * TM;
     const int kbytes = K / 2, kblocks = K / kBlock;
     const int nrow = min(n0 + (lane & 31), N - 1);
+    // the weight: row-major packed (a lane walks its row), or the decode layout (a wave walks the blocks of its column tile)
     const uint8_t* bc = b_codes + (int64_t)nrow * kbytes + hi * 16 * C;
     const uint8_t* bs = b_scales + (int64_t)nrow * kblocks + hi * 2 * C;
+    int w_step = 32 * C, w_piece = 16, ws_step = 4 * C;
+    if (C == 4 && decode) {
+        const uint8_t* tile0 = b_codes + (int64_t)(n0 / 32) * (K / 256) * kDecodeBlock;
+        bc = tile0 + lane * 16;
+        bs = tile0 + 4096 + lane * 8;
+        w_step = kDecodeBlock; w_piece = 1024; ws_step = kDecodeBlock;
+    }
     static_assert(ADENSE == 0 || (C == 4 && CEN == 0), "ready operands come in the wide-run layout");
     const uint8_t *ac[TM], *as[TM];
     const uint4* ap[TM];
@@ -658,7 +666,7 @@ __device__ __forceinline__ void skinny_tile(
     const float ua = PB16 ? *a_unit : 0.0f, ub = PB16 ? *b_unit : 0.0f;
     for (int it = s0 + wave * iters / WAVES; it < it1; ++it) {
         RunRegs<C> rw;
-        load_run<C>(rw, bc + (int64_t)it * 32 * C, bs + it * 4 * C);
+        load_run_strided<C>(rw, bc + (int64_t)it * w_step, w_piece, bs + (int64_t)it * ws_step);
         if constexpr (ADENSE != 0) {
             // a ring of AHEAD operand pieces per row tile keeps the L2 round trips ahead of the MFMAs
             constexpr int AHEAD = 4;
@@ -869,7 +877,49 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_nvfp4_skinny_grouped_kernel(
         if (g == i) mm = grp.m[i];
     skinny_tile<TM, C, WAVES, OUT_F32, CEN, PB16, ADENSE>(a_codes, a_scales, a_unit, mm.b_codes, mm.b_scales, mm.b_unit, M, mm.N, K, mm.t, mm.u,
                                             mm.r, mm.bias, mm.out, mm.bias_f32, (tile - start) * 32, mm.ldt, mm.part, grp.nsplit,
-                                            grp.center);
+                                            grp.center, mm.decode);
+}
+
+// A packed weight in the decode layout (gemm_common.h): one thread per 16-byte piece of codes, then the scale bytes.
+// Derived data, built once per weight update and cached beside the packed form like the tiled expansion.
+__global__ __launch_bounds__(256) void decode_weight_kernel(const uint8_t* __restrict__ codes, const uint8_t* __restrict__ scales,
+                                                            int N, int K, uint8_t* __restrict__ out, int64_t blocks)
+{
+    const int iters = K / 256;
+    for (int64_t b = blockIdx.x; b < blocks; b += gridDim.x) {
+        const int tile = (int)(b / iters), it = (int)(b % iters);
+        uint8_t* dst = out + b * kDecodeBlock;
+        const int l = threadIdx.x & 63, j = threadIdx.x >> 6;              // lane, piece
+        const int row = tile * 32 + (l & 31), h = l >> 5;
+        uint4 v = make_uint4(0u, 0u, 0u, 0u);
+        if (row < N) v = *reinterpret_cast<const uint4*>(codes + (int64_t)row * (K / 2) + it * 128 + h * 64 + 16 * j);
+        *reinterpret_cast<uint4*>(dst + j * 1024 + l * 16) = v;
+        if (j == 0) {
+            uint2 sc = make_uint2(0u, 0u);
+            if (row < N) sc = *reinterpret_cast<const uint2*>(scales + (int64_t)row * (K / 16) + it * 16 + h * 8);
+            *reinterpret_cast<uint2*>(dst + 4096 + l * 8) = sc;
+        }
+    }
+}
+
+size_t decode_weight_bytes(int64_t N, int64_t K)
+{
+    if (N <= 0 || K <= 0 || K % 256) return 0;
+    return (size_t)((N + 31) / 32) * (size_t)(K / 256) * kDecodeBlock;
+}
+
+int decode_weight(const void* codes, const void* scales, int64_t N, int64_t K, void* out, hipStream_t st)
+{
+    if (N <= 0 || K <= 0 || N > INT32_MAX || K > INT32_MAX) return METIS_E_ARG;
+    if (K % 256) return METIS_E_SHAPE;
+    if (!codes || !scales || !out || ((uintptr_t)codes % 16) || ((uintptr_t)scales % 8) || ((uintptr_t)out % 16)) return METIS_E_ARG;
+    const int64_t blocks = ((N + 31) / 32) * (K / 256);
+    int64_t g = blocks;
+    const int64_t cap = (int64_t)device_cus() * 16;
+    if (g > cap) g = cap;
+    hipLaunchKernelGGL(decode_weight_kernel, dim3((unsigned)g), dim3(256), 0, st, (const uint8_t*)codes, (const uint8_t*)scales, (int)N, (int)K,
+                       (uint8_t*)out, blocks);
+    return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 
 // The activation of a decode-sized call as ready MFMA operands for the wide-run layout of skinny_tile (K % 256 == 0):
@@ -1176,15 +1226,17 @@ int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a
     int64_t tiles = 0, ntot = 0;
     for (int i = 0; i < count && skinny; ++i) {
         const GemmMember& g = members[i];
-        if (!g.b_codes || !g.b_scales || !g.b_unit || !g.out || g.N <= 0 || g.N > INT32_MAX || g.N % 4 || g.r < 0 || g.r % 32 ||
+        if ((!g.b_decode && (!g.b_codes || !g.b_scales)) || ((uintptr_t)g.b_decode % 16) || (g.b_decode && K % 256) || !g.b_unit || !g.out || g.N <= 0 || g.N > INT32_MAX || g.N % 4 || g.r < 0 || g.r % 32 ||
             (g.r > 0 && (!g.t || !g.u)) || (g.ldt != 0 && (g.ldt < g.r || g.ldt % 8 || g.ldt > INT32_MAX)) || ((uintptr_t)g.b_codes % 16) || ((uintptr_t)g.b_scales % 2) || ((uintptr_t)g.out % 16) ||
             ((uintptr_t)g.t % 16) || ((uintptr_t)g.u % 16) || ((uintptr_t)g.bias % (g.bias_is_f32 ? 4 : 2)))
             skinny = false;
-        al8 = al8 && ((uintptr_t)g.b_scales % 8) == 0;
+        al8 = al8 && (g.b_decode || ((uintptr_t)g.b_scales % 8) == 0);
         tiles += (g.N + 31) / 32;
         ntot += g.N;
     }
     if (!skinny || tiles > INT32_MAX) {
+        for (int i = 0; i < count; ++i)
+            if (!members[i].b_codes || !members[i].b_scales) return METIS_E_ARG;   // only the decode-sized kernel reads the decode layout
         if (center || pb16 || a_dense) return METIS_E_ARG;     // the centre, the bf16 evaluation and ready operands are only taken by the single-launch path
         for (int i = 0; i < count; ++i) {
             const GemmMember& g = members[i];
@@ -1218,9 +1270,11 @@ int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a
     for (int i = 0; i < count; ++i) {
         const GemmMember& g = members[i];
         end += (int)((g.N + 31) / 32);
-        grp.m[i] = SkinnyMember{(const uint8_t*)g.b_codes, (const uint8_t*)g.b_scales, g.b_unit, (const uint16_t*)g.t,
+        const bool dec = g.b_decode && c == 4;
+        if (!dec && (!g.b_codes || !g.b_scales)) return METIS_E_ARG;
+        grp.m[i] = SkinnyMember{(const uint8_t*)(dec ? g.b_decode : g.b_codes), (const uint8_t*)g.b_scales, g.b_unit, (const uint16_t*)g.t,
                                 (const uint16_t*)g.u, (const uint16_t*)g.bias, g.out, nsplit > 1 ? part : nullptr, (int)g.N,
-                                (int)g.r, end, g.bias_is_f32 != 0, (int)(g.ldt ? g.ldt : g.r)};
+                                (int)g.r, end, g.bias_is_f32 != 0, (int)(g.ldt ? g.ldt : g.r), dec ? 1 : 0};
         part += slots * (size_t)M * (size_t)g.N;
     }
 #define METIS_SKG(TM, C, W) return launch_skinny_grouped<TM, C, W>(a_codes, a_scales, a_unit, M, K, grp, (int)tiles, out_dtype, st, pb16, a_dense)
@@ -1240,7 +1294,7 @@ static int gemm_skinny(const void* a_codes, const void* a_scales, const float* a
                        const void* u, int64_t r, const void* bias, void* out, int out_dtype, hipStream_t st, int bias_f32,
                        void* workspace, size_t workspace_bytes)
 {
-    const GemmMember g = {b_codes, b_scales, b_unit, t, u, r, bias, out, N, bias_f32, 0};
+    const GemmMember g = {b_codes, b_scales, b_unit, t, u, r, bias, out, N, bias_f32, 0, nullptr};
     return gemm_nvfp4_grouped(a_codes, a_scales, a_unit, M, K, &g, 1, out_dtype, st, workspace, workspace_bytes, nullptr);
 }
 

@@ -113,7 +113,11 @@ struct GemmMember {
     int64_t N;
     int64_t bias_is_f32;
     int64_t ldt;
+    const void* b_decode;        // the weight in the decode layout (decode_weight), or nullptr
 };
+// a packed weight [N, K], K % 256 == 0, in the layout the decode-sized kernel streams as whole lines; metis_gemm.hip
+size_t decode_weight_bytes(int64_t N, int64_t K);
+int decode_weight(const void* codes, const void* scales, int64_t N, int64_t K, void* out, hipStream_t st);
 int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a_unit, int64_t M, int64_t K,
                        const GemmMember* members, int count, int out_dtype, hipStream_t st, void* workspace = nullptr,
                        size_t workspace_bytes = 0, const float* center = nullptr, bool pb16 = false, bool a_dense = false);

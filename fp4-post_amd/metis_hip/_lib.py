@@ -16,7 +16,8 @@ class LinearMember(ctypes.Structure):
     """metis_linear_member of include/metis_hip.h: one weight matrix of a grouped GEMM."""
     _fields_ = [("b_codes", ctypes.c_void_p), ("b_scales", ctypes.c_void_p), ("b_unit", ctypes.c_void_p),
                 ("t", ctypes.c_void_p), ("u", ctypes.c_void_p), ("r", ctypes.c_int64), ("bias", ctypes.c_void_p),
-                ("out", ctypes.c_void_p), ("N", ctypes.c_int64), ("bias_is_f32", ctypes.c_int64), ("ldt", ctypes.c_int64)]
+                ("out", ctypes.c_void_p), ("N", ctypes.c_int64), ("bias_is_f32", ctypes.c_int64), ("ldt", ctypes.c_int64),
+                ("b_decode", ctypes.c_void_p)]
 
 
 MODE_P32, MODE_PB16 = 0, 1
@@ -43,6 +44,9 @@ SIGNATURES = {
     "metis_nvfp4_rquant": (_i32, [_vp, _vp, _i64, _i64, _i32, _vp, _vp, _vp]),
     "metis_nvfp4_dequant": (_i32, [_vp, _vp, _vp, _i64, _i64, _i32, _vp, _i32, _vp]),
     "metis_rmsnorm_nvfp4_quant": (_i32, [_vp, _vp, _f32, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "metis_linear_member_size": (_sz, []),
+    "metis_nvfp4_decode_weight_bytes": (_sz, [_i64, _i64]),
+    "metis_nvfp4_decode_weight": (_i32, [_vp, _vp, _i64, _i64, _vp, _vp]),
     "metis_rmsnorm_colmean_workspace_bytes": (_sz, [_i64, _i64]),
     "metis_rmsnorm_colmean": (_i32, [_vp, _vp, _f32, _i64, _i64, _vp, _vp, _i32, _vp, _i64, _vp, _vp, _sz, _vp]),
     "metis_linear_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _i32, _vp]),
@@ -119,6 +123,9 @@ def load():
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(lib, name)
             fn.restype, fn.argtypes = res, args
+        if lib.metis_linear_member_size() != ctypes.sizeof(LinearMember):
+            raise MetisHipError(f"{LIB_PATH} was built from another revision of include/metis_hip.h: metis_linear_member is "
+                                f"{lib.metis_linear_member_size()} bytes there, {ctypes.sizeof(LinearMember)} here; rebuild it")
         _lib = lib
     return _lib
 

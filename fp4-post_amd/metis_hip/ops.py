@@ -15,6 +15,8 @@ from ._lib import DTYPE_BF16, DTYPE_F32, MODE_P32, MODE_PB16, check, load
 
 BLOCK = 16
 _workspaces: dict = {}
+# Derived copies of a cached weight that cost memory: the decode layout (0.5625 B per parameter) for decode-sized batches
+decode_layout_weights = True
 
 
 @dataclass
@@ -44,6 +46,7 @@ class PackedNVFP4:
     # `unit` are produced on first access (one more launch), unless a consumer that forms the bytes itself
     # (expand_tiled) got there first and wrote the unit
     deferred: torch.Tensor | None = None
+    decode_layout: torch.Tensor | None = None  # a persistent weight in the layout the decode-sized kernel streams as whole lines
 
     def dequantize(self, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
         return dequantize(self, dtype)
@@ -549,6 +552,23 @@ def decode_operand(p: PackedNVFP4, mode: int = MODE_P32, center: torch.Tensor | 
     return out
 
 
+def decode_weight(p: PackedNVFP4, cache: bool = True) -> torch.Tensor | None:
+    """The packed weight in the decode layout (same 0.5625 B per element): rows in tiles of 32, K in steps of 256, the
+    pieces of a wave's 64 lanes side by side, so that the decode-sized kernel's loads cover whole lines.  None when
+    K % 256 != 0.  Kept on a persistent (cached) weight."""
+    if p.decode_layout is not None:
+        return p.decode_layout
+    if p.cols % 256 or p.rht is not None:
+        return None
+    L = load()
+    out = torch.empty(L.metis_nvfp4_decode_weight_bytes(p.rows, p.cols), dtype=torch.uint8, device=p.codes.device)
+    rc = L.metis_nvfp4_decode_weight(p.codes.data_ptr(), p.scales.data_ptr(), p.rows, p.cols, out.data_ptr(), _stream())
+    check(rc, "metis_nvfp4_decode_weight", (p.rows, p.cols))
+    if cache:
+        p.decode_layout = out
+    return out
+
+
 def dense_expand_tiled(x: torch.Tensor, mode: int = MODE_P32, col_scale: torch.Tensor | None = None) -> torch.Tensor:
     """A dense [rows, cols] bf16 or float32 tensor as a tiled GEMM operand (see expand_tiled): binary16 values in mode
     P32 (pair it with a unit of 2^-8, see gemm_tiled), bf16 values in mode PB16.  col_scale (bf16 [cols]) multiplies
@@ -991,9 +1011,12 @@ def _linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.
         out = torch.empty(M, b.rows, dtype=out_dtype, device=dev)
         keep += [t, u, bias]
         outs.append(out)
+        # a cached weight is streamed in its decode layout (whole lines per load instruction) by the decode-sized kernel
+        dec = decode_weight(b) if (b.persistent and takes and M < 256 and decode_layout_weights) else None
         arr[i] = _lib.LinearMember(b.codes.data_ptr(), b.scales.data_ptr(), b.unit.data_ptr(),
                                    None if t is None else t.data_ptr(), None if u is None else u.data_ptr(), r,
-                                   None if bias is None else bias.data_ptr(), out.data_ptr(), b.rows, int(bias_f32), ldt)
+                                   None if bias is None else bias.data_ptr(), out.data_ptr(), b.rows, int(bias_f32), ldt,
+                                   None if dec is None else dec.data_ptr())
     L = load()
     ap = ctypes.cast(arr, ctypes.c_void_p)
     # split-K scratch (long K, few columns) and whether a centre fits the launch: functions of the shape alone

@@ -555,7 +555,20 @@ typedef struct metis_linear_member {
     int64_t bias_is_f32; /* 0: bias is bf16 [N]; 1: binary32 [N] (metis_linear_fwd_f32bias) */
     int64_t ldt;         /* row stride of t in elements; 0 = r.  A stride other than r (members reading their columns of
                             one stacked [M, sum r] projection) needs M < 256 and K % 64 == 0, else METIS_E_ARG */
+    const void *b_decode; /* NULL, or the same packed weight in the decode layout (metis_nvfp4_decode_weight; K % 256 == 0,
+                            16-byte aligned): the decode-sized kernel then streams it as whole lines and b_codes /
+                            b_scales may be NULL.  Calls that do not run on the decode-sized kernel need b_codes / b_scales */
 } metis_linear_member;
+/* sizeof(metis_linear_member) as the library was built: a caller compiled against another revision of this header
+ * compares it with its own before passing member arrays (a mismatch would make the library read past the caller's array). */
+size_t metis_linear_member_size(void);
+/* A packed weight [N, K] in the decode layout, derived data to be cached beside the packed form (the reference caches
+ * its dequantized weight the same way, src/Metis/Metis/bitlinear.py:563-589): 0.5625 B per element as packed, rows
+ * grouped in tiles of 32 and K in steps of 256 so that every load instruction of a wave of the decode-sized kernel
+ * reads a KiB of consecutive bytes instead of 16 bytes from each of 64 rows.  K % 256 == 0 (METIS_E_SHAPE otherwise).
+ *   out   metis_nvfp4_decode_weight_bytes(N, K) bytes, 16-byte aligned */
+size_t metis_nvfp4_decode_weight_bytes(int64_t N, int64_t K);
+int metis_nvfp4_decode_weight(const void *codes, const void *scales, int64_t N, int64_t K, void *out, void *stream);
 int metis_linear_fwd_grouped(const void *a_codes, const void *a_scales, const float *a_unit, int64_t M,
                              int64_t K, const metis_linear_member *members, int count, int out_dtype,
                              void *workspace, size_t workspace_bytes, void *stream);

@@ -444,6 +444,12 @@ static void check_sr_both(int64_t rows, int64_t cols, int mode, hipStream_t st)
 
 int main()
 {
+    // before anything touches the GPU: this program and the library must agree on the layout of the member descriptors
+    if (metis_linear_member_size() != sizeof(metis_linear_member)) {
+        printf("FAIL: libmetis_hip.so was built with a metis_linear_member of %zu bytes, this program with %zu: rebuild it (make native-check)\n",
+               metis_linear_member_size(), sizeof(metis_linear_member));
+        return 1;
+    }
     hipStream_t st;
     HIP_OK(hipStreamCreate(&st));                                // a caller-owned stream, default priority
     printf("library version %d\n", metis_version());

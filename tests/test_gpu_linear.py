@@ -421,6 +421,54 @@ def test_grouped_projections_equal_member_by_member_calls(M, K, Ns, r):
             assert torch.equal(y, want)
 
 
+@pytest.mark.parametrize("M,K,Ns,r", [(64, 3584, (3584, 512, 512), 64), (1, 1024, (256, 100), 0), (40, 3584, (18944, 18944), 32),
+                                      (64, 18944, (3584,), 64), (200, 2048, (132, 64, 36), 32), (17, 256, (4,), 0)])
+def test_cached_weights_in_the_decode_layout_give_the_same_bits(M, K, Ns, r):
+    """A persistent (cached) weight is also kept in the decode layout -- rows in tiles of 32, K in steps of 256, the 16-byte
+    pieces of a wave's lanes side by side -- and decode-sized calls stream that copy.  Same kernel, same order of
+    operations: bit-identical outputs with and without it, in exact arithmetic, with the reference's bf16 roundings, with
+    a centre inside the launch, with K split into slices, for ragged last tiles (N % 32 != 0); the layout itself is
+    checked against its definition."""
+    from metis_hip import ops
+    g = torch.Generator().manual_seed(M + K)
+    x = synthetic_activation(160 + M, M, K).cuda()
+    centre = (torch.randn(K, generator=g) * 0.2).cuda()
+    for mode in (0, 1):
+        px = ops.quantize(x, mode)
+        plain, cached = [], []
+        for i, N in enumerate(Ns):
+            w = _weights(161 + i, N, K).cuda()
+            t = u = None
+            if r and i != 1:
+                t = torch.randn(M, r, generator=g).bfloat16().cuda()
+                u = (torch.randn(N, r, generator=g) * 0.1).bfloat16().cuda()
+            bias = (torch.randn(N, generator=g) * 0.1).bfloat16().cuda() if i % 2 == 0 else None
+            pw, pc = ops.quantize(w, mode), ops.quantize(w, mode)
+            pc.persistent = True
+            plain.append((pw, t, u, bias))
+            cached.append((pc, t, u, bias))
+        for kw in ({}, {"reference_rounding": True} if mode == 1 else {"center": centre}, {"split_k": False}):
+            want = ops.linear_fwd_grouped(px, plain, **kw)
+            got = ops.linear_fwd_grouped(px, cached, **kw)
+            assert all(m[0].decode_layout is not None for m in cached) and all(m[0].decode_layout is None for m in plain)
+            for a, b in zip(got, want):
+                assert torch.equal(a, b), (mode, kw.keys())
+    # the layout: block (tile, step) = 4 KiB of codes (piece j of lane l at j * 1024 + l * 16) + 512 scale bytes (lane l at 4096 + l * 8)
+    pc = cached[0][0]
+    N = Ns[0]
+    lay = pc.decode_layout.cpu().reshape((N + 31) // 32, K // 256, 4608)
+    codes, scales = pc.codes.cpu(), pc.scales.cpu()
+    for tile, step, lane, j in ((0, 0, 0, 0), ((N - 1) // 32, K // 256 - 1, 37, 3), (0, K // 256 - 1, 63, 1)):
+        row, h = tile * 32 + (lane & 31), lane >> 5
+        got_c = lay[tile, step, j * 1024 + lane * 16: j * 1024 + lane * 16 + 16]
+        got_s = lay[tile, step, 4096 + lane * 8: 4096 + lane * 8 + 8]
+        if row < N:
+            assert torch.equal(got_c, codes[row, step * 128 + h * 64 + 16 * j: step * 128 + h * 64 + 16 * j + 16])
+            assert torch.equal(got_s, scales[row, step * 16 + h * 8: step * 16 + h * 8 + 8])
+        else:
+            assert int(got_c.sum()) == 0 and int(got_s.sum()) == 0
+
+
 @pytest.mark.parametrize("M,K,Ns,r", [(64, 18944, (3584,), 64), (1, 8192, (256,), 0), (200, 16384, (132, 64), 32),
                                       (33, 8256, (96,), 32)])
 def test_decode_sized_products_with_a_long_contraction_split_k(M, K, Ns, r):
