@@ -360,28 +360,35 @@ __device__ __forceinline__ void unpack16(const uint4 a, const uint4 b, float (&v
 // Tiled random Hadamard rotation of the NV recipe on one tile of 16 in registers (the tile is the scale block).
 // Forward: (v * sign) H, src/Metis/Metis/bitlinear.py:199-202; inverse: (v H) / 16 * sign, bitlinear.py:195-197, with H the
 // Sylvester matrix (75-96) and sign the shared vector of 126-137, here a bit mask (bit j set: sign[j] = -1).
-// binary32 sums in butterfly order; sums of bf16 values are exact whenever their exponents are within 12 of each other.
-__device__ __forceinline__ void hadamard16_butterflies(float (&v)[kBlock])
+// The reference forms v H as a binary32 matrix product (torch.mm on the CPU): every output is the sum of its sixteen
+// terms +-v[k] taken in the order k = 0 .. 15.  The order matters: the weight gradient's second operand is the already
+// quantized input rotated and quantized AGAIN, its rotated values sit on FP4 rounding boundaries far more often than
+// ordinary data, and which side they land on hangs on the last bit of these sums.  Summed in this order the kernels
+// reproduce the reference's operand bit for bit (a butterfly network, or a double-precision sum rounded once, each
+// leave 5 % of that operand's elements different: 2e-2 in the Frobenius norm).  240 additions instead of the
+// network's 64; H[k][n] = (-1)^popcount(k & n) is folded at compile time.
+__device__ __forceinline__ void hadamard16_product(float (&v)[kBlock])
 {
+    float o[kBlock];
 #pragma unroll
-    for (int h = 1; h < kBlock; h <<= 1)
+    for (int n = 0; n < kBlock; ++n) {
+        float acc = v[0];                                     // H[0][n] = +1, and 0 + v[0] = v[0]
 #pragma unroll
-        for (int j = 0; j < kBlock; ++j)
-            if ((j & h) == 0) {
-                const float a = v[j], b = v[j + h];
-                v[j] = a + b;
-                v[j + h] = a - b;
-            }
+        for (int k = 1; k < kBlock; ++k) acc = (__builtin_popcount(k & n) & 1) ? acc - v[k] : acc + v[k];
+        o[n] = acc;
+    }
+#pragma unroll
+    for (int n = 0; n < kBlock; ++n) v[n] = o[n];
 }
 __device__ __forceinline__ void hadamard16_forward(float (&v)[kBlock], uint32_t sign_mask)
 {
 #pragma unroll
     for (int j = 0; j < kBlock; ++j) v[j] = __uint_as_float(__float_as_uint(v[j]) ^ (((sign_mask >> j) & 1u) << 31));
-    hadamard16_butterflies(v);
+    hadamard16_product(v);
 }
 __device__ __forceinline__ void hadamard16_inverse(float (&v)[kBlock], uint32_t sign_mask)
 {
-    hadamard16_butterflies(v);
+    hadamard16_product(v);
 #pragma unroll
     for (int j = 0; j < kBlock; ++j) v[j] = __uint_as_float(__float_as_uint(v[j] * 0.0625f) ^ (((sign_mask >> j) & 1u) << 31));
 }

@@ -196,15 +196,16 @@ def test_linear_lowbit_nv_recipe_on_the_packed_kernels_against_reference_vectors
     # The weight gradient's second operand is the ALREADY quantized input, rotated and quantized again (495-501).  Its
     # rotated values are small-integer combinations of one block scale, so their quotients by the new block scalar sit
     # exactly on FP4 rounding boundaries far more often than those of ordinary data, and which side such a value lands
-    # on hangs on the last bit of a 16-term binary32 sum, i.e. on the summation order of whoever computes it (the
-    # reference's own CPU and GPU results differ the same way).  A flipped code spreads over its block of 16 on the way
-    # back: about 5 % of the operand's elements differ from the reference's CPU run, 2e-2 in the Frobenius norm.
+    # on hangs on the last bit of a 16-term binary32 sum.  The kernels add the sixteen terms in the order the reference's
+    # matrix product adds them (k = 0 .. 15), which reproduces its operand bit for bit (test_oracle_pins.py shows on the
+    # CPU that a butterfly network or a double-precision sum would each leave 5 % of the elements different).
     x_op = F.q_backward_input.pack(t(g[f"hw_{tag}_xq"]).to(dtype).cuda().reshape(-1, 96), arith=dtype, rht=F._hadamard_mask())
     got, want = x_op.dequantize(dtype).float().cpu(), t(g[f"hw_{tag}_wgrad_x"]).float().reshape(-1, 96)
-    assert rel_fro(got, want) <= 3e-2 and float((got - want).abs().le(1e-6 * float(want.abs().max())).float().mean()) > 0.9
+    assert rel_fro(got, want) <= (1e-6 if tag == "p32" else 2e-3)
+    assert float((got - want).abs().le(1e-6 * float(want.abs().max())).float().mean()) > (0.9999 if tag == "p32" else 0.99)
     dy_op = F.q_backward_outputgrad.pack(t(g["hw_dy"]).to(dtype).cuda().reshape(-1, 64), arith=dtype, rht=F._hadamard_mask())
     assert rel_fro(dy_op.dequantize(dtype).float().cpu(), t(g[f"hw_{tag}_wgrad_dy"]).float().reshape(-1, 64)) <= (1e-6 if tag == "p32" else 2e-3)
-    assert rel_fro(layer.weight.grad.float().cpu(), t(g[f"hw_{tag}_gw"]).float()) <= 3e-2
+    assert rel_fro(layer.weight.grad.float().cpu(), t(g[f"hw_{tag}_gw"]).float()) <= tol
     # and against the product of the operands as this library formed them: the GEMM itself is exact to its tolerance
     dense = dy_op.dequantize(dtype).double().T @ x_op.dequantize(dtype).double()
     assert rel_fro(layer.weight.grad.double().cpu(), dense.cpu()) <= (2e-4 if tag == "p32" else 2.5e-3)

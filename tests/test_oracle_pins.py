@@ -154,3 +154,51 @@ def test_rmsnorm_against_library_and_fp64():
 def test_value_error_on_non_divisible_last_dim():
     with pytest.raises(ValueError):
         O.nvfp4_qdq(torch.zeros(4, 24))
+
+
+def test_rotation_of_the_nv_recipe_is_summed_in_the_order_of_the_reference_matrix_product():
+    """The NV recipe rotates a tile of 16 with a binary32 matrix product (src/Metis/Metis/bitlinear.py:195-202, torch.mm on
+    the CPU).  For the weight gradient's second operand -- the already quantized input, rotated and quantized AGAIN
+    (495-501) -- the summation order of those 16-term sums decides codes: rotated values of quantized data sit on FP4
+    rounding boundaries far more often than ordinary data.  On the reference's own vectors: adding the terms in the order
+    k = 0 .. 15 (what the kernels do) reproduces the reference's operand bit for bit, while a butterfly network and a
+    double-precision sum rounded once each leave about 5 % of its elements different, 2e-2 in the Frobenius norm."""
+    import os
+    import numpy as np
+    from helpers import rel_fro, t
+    from oracle import metis_oracle as O
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    g = dict(np.load(os.path.join(here, "metis_reference_hadamard_wide.npz")))
+    sign = t(dict(np.load(os.path.join(here, "metis_reference_hadamard.npz")))["had_sign16"]).float()
+    H = torch.tensor([[1.0]])
+    while H.shape[0] < 16:
+        H = torch.cat([torch.cat([H, H], 1), torch.cat([H, -H], 1)], 0)
+    xq = t(g["hw_p32_xq"]).float().reshape(-1, 16)
+    want = t(g["hw_p32_wgrad_x"]).float().reshape(-1, 16)
+
+    def sequential(v):
+        acc = torch.zeros_like(v)
+        for k in range(16):
+            acc = acc + v[:, k:k + 1] * H[k:k + 1, :]
+        return acc
+
+    def butterfly(v):
+        w = v.clone()
+        h = 1
+        while h < 16:
+            for j in range(16):
+                if (j & h) == 0:
+                    a, b = w[:, j].clone(), w[:, j + h].clone()
+                    w[:, j], w[:, j + h] = a + b, a - b
+            h <<= 1
+        return w
+
+    def operand(product):
+        rotated = product(xq * sign).reshape(-1, 96)
+        q = O.nvfp4_qdq(rotated).reshape(-1, 16)
+        return sequential(q) * (1.0 / 16) * sign
+
+    assert torch.equal(operand(sequential), want)
+    for other in (butterfly, lambda v: (v.double() @ H.double()).float()):
+        got = operand(other)
+        assert 5e-3 < rel_fro(got, want) < 5e-2 and 0.9 < float((got == want).float().mean()) < 0.99
