@@ -35,6 +35,13 @@ from .quant import (Cast2Fp32, Cast2NVFp4e2m1Block, Cast2NVFp4e2m1BlockNOSR, Qua
 __all__ = ["LinearLowbitFunction", "LinearLowbit", "BitLinear"]
 
 
+def _pkey(p: torch.Tensor) -> tuple:
+    """Cache key of a parameter: its identity and storage as well as its version counter, so that a Parameter that is
+    REPLACED (load_state_dict(assign=True), `m.s = nn.Parameter(...)`) is seen although a fresh one starts at the same
+    version.  (A write through `.data`, which moves neither, stays invisible, as it does to the reference's own cache.)"""
+    return (id(p), p.data_ptr(), p._version)
+
+
 def _flat2d(x: torch.Tensor) -> torch.Tensor:
     return x.reshape(-1, x.shape[-1])
 
@@ -429,6 +436,16 @@ class LinearLowbitFunction(torch.autograd.Function):
         return (gx[:L] if pad else gx), gw
 
     @staticmethod
+    def _check_backward_config() -> None:
+        F = LinearLowbitFunction
+        if F.enable_backward_svd and F.backward_lowrank_svd <= 0:
+            # the reference takes a full SVD of the output gradient here (bitlinear.py:476-486); neither path of this
+            # library implements that branch, and the low-rank / mean-residual QDQ it would silently get instead is
+            # another method
+            raise NotImplementedError("enable_backward_svd with backward_lowrank_svd <= 0 (the reference's full-SVD branch, "
+                                      "bitlinear.py:476-486) is not implemented; use a positive rank")
+
+    @staticmethod
     def _packed_backward_applies(L: int, N: int, grad_output: torch.Tensor) -> bool:
         """Backward on the packed kernels.  Any token count L qualifies (ragged counts are padded inside
         _packed_grads); the output width N is the contraction of the input gradient and has to be a multiple of 32.
@@ -519,6 +536,7 @@ class LinearLowbitFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output):
         F = LinearLowbitFunction
+        F._check_backward_config()
         grad_bias = None
         if ctx.has_bias:
             grad_bias = _token_sum(_flat2d(grad_output), F.compute_dtype).to(torch.float32)
@@ -616,7 +634,7 @@ class LinearLowbit(nn.Module):
         """Quantized weight, cached on Parameter._version when enabled (reference 563-589).  Returns a
         PackedNVFP4 when the kernel path applies, otherwise the dequantized tensor."""
         F = LinearLowbitFunction
-        key = (self.weight._version, weight_compute.device, arith or weight_compute.dtype, F.q_forward_weight, F.enable_nv_recipe)
+        key = (_pkey(self.weight), weight_compute.device, arith or weight_compute.dtype, F.q_forward_weight, F.enable_nv_recipe)
         if self.cache_quantized_weight and self._quantized_weight_cache is not None:
             cached_key, cached = self._quantized_weight_cache
             if cached_key == key:
@@ -700,6 +718,7 @@ class _MetisFusedFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dy):
         F = LinearLowbitFunction
+        F._check_backward_config()
         x, v, s, u, res, xv, t = ctx.saved_tensors
         cd = torch.bfloat16
         dy2 = _flat2d(dy).to(cd)
@@ -838,8 +857,8 @@ class BitLinear(nn.Module):
     def _get_merged_rollout_weight(self, dtype: torch.dtype) -> torch.Tensor:
         """(U diag s) Q(V) + Q(W_res), cached on the parameters' versions (reference 704-730)."""
         F = LinearLowbitFunction
-        key = (self.vlinear.weight._version, self.ulinear.weight._version, self.s._version,
-               self.warmup_linear.weight._version, self.vlinear.weight.device, dtype, F.q_forward_weight, F.enable_nv_recipe)
+        key = (_pkey(self.vlinear.weight), _pkey(self.ulinear.weight), _pkey(self.s),
+               _pkey(self.warmup_linear.weight), self.vlinear.weight.device, dtype, F.q_forward_weight, F.enable_nv_recipe)
         if self._merged_rollout_weight_cache is not None:
             cached_key, cached = self._merged_rollout_weight_cache
             if cached_key == key:
@@ -950,7 +969,7 @@ class BitLinear(nn.Module):
         cd = torch.bfloat16
         x2 = _flat2d(x).to(cd)
         # one product for every member's rank-r projection: V of all members stacked, cached on their versions
-        key = tuple((m.vlinear.weight._version, m.s._version) for m in members) + (x2.device,)
+        key = tuple((_pkey(m.vlinear.weight), _pkey(m.s)) for m in members) + (x2.device,)
         cached = group.get("stacked_v")
         if cached is None or cached[0] != key:
             cached = (key, torch.cat([m.vlinear.weight.to(cd) for m in members], dim=0),
@@ -980,7 +999,7 @@ class BitLinear(nn.Module):
         b = self.warmup_linear.bias
         if b.dtype == dtype:
             return b
-        key = (b._version, b.device, dtype)
+        key = (_pkey(b), b.device, dtype)
         cached = getattr(self, "_bias_cast_cache", None)
         if cached is None or cached[0] != key:
             cached = (key, b.detach().to(dtype))

@@ -15,8 +15,13 @@ from ._lib import DTYPE_BF16, DTYPE_F32, MODE_P32, MODE_PB16, check, load
 
 BLOCK = 16
 _workspaces: dict = {}
-# Derived copies of a cached weight that cost memory: the decode layout (0.5625 B per parameter) for decode-sized batches
+# Derived copies of a cached weight cost memory beside its packed form (0.5625 B per parameter): the decode layout
+# (0.5625 B) for decode-sized batches, and the tiled binary16 expansions (2 B each: one per arithmetic the layer runs in,
+# one more per arithmetic for the transposed operand of the NV recipe).  Memory-bound deployments switch them off:
+# without the tiled copies, binary32-arithmetic GEMMs run on the packed operands, and bf16-arithmetic GEMMs expand the
+# weight on every call instead of once.  Same bits either way.
 decode_layout_weights = True
+tiled_weight_copies = True
 
 
 @dataclass
@@ -50,6 +55,18 @@ class PackedNVFP4:
 
     def dequantize(self, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
         return dequantize(self, dtype)
+
+    def held_bytes(self) -> dict:
+        """Device bytes this tensor holds right now, by part: the packed form and every derived copy built so far."""
+        d = self.__dict__
+        parts = {"packed": self.codes.numel() + (d["_scales"].numel() if d.get("_scales") is not None else 0)}
+        for name in ("expanded", "tiled", "tiled_pb16", "tiled_t", "tiled_t_pb16", "decode_layout", "deferred"):
+            t = d.get(name)
+            if t is not None:
+                parts[name] = t.numel() * t.element_size()
+        if self.transposed is not None:
+            parts["transposed"] = sum(self.transposed.held_bytes().values())
+        return parts
 
     def _materialize(self) -> None:
         d = self.__dict__
@@ -500,7 +517,7 @@ def expand_tiled(p: PackedNVFP4, cache: bool = True, mode: int = MODE_P32, cente
         rc = L.metis_nvfp4_expand_tiled(p.codes.data_ptr(), p.scales.data_ptr(), p.unit.data_ptr(), p.rows, p.cols, mode,
                                         out.data_ptr(), _stream())
     check(rc, "metis_nvfp4_expand_tiled", (p.rows, p.cols))
-    if cache:
+    if cache and (tiled_weight_copies or not p.persistent):
         if mode == MODE_PB16:
             p.tiled_pb16 = out
         else:
@@ -519,7 +536,7 @@ def expand_tiled_transposed(p: PackedNVFP4, cache: bool = False, mode: int = MOD
     rc = L.metis_nvfp4_expand_tiled_rht(p.codes.data_ptr(), p.scales.data_ptr(), p.unit.data_ptr(), p.rows, p.cols, mode,
                                         p.rht or 0, int(p.rht is not None), 1, out.data_ptr(), _stream())
     check(rc, "metis_nvfp4_expand_tiled_rht", (p.rows, p.cols))
-    if cache:
+    if cache and (tiled_weight_copies or not p.persistent):
         if mode == MODE_PB16:
             p.tiled_t_pb16 = out
         else:
@@ -720,7 +737,7 @@ def _tiled_applies(a: PackedNVFP4, b: PackedNVFP4) -> bool:
     """The pipelined GEMM on tiled binary16 expansions pays when the weight-side expansion is reused across calls
     (a cached weight) and the batch fills a 256-row tile; the activation side is expanded per call (2.56 B/element,
     about 2 % of the GEMM's time at such shapes)."""
-    if not (b.persistent or b.tiled is not None):
+    if not ((b.persistent and tiled_weight_copies) or b.tiled is not None):
         return False
     M, N, K = a.rows, b.rows, a.cols
     return M >= 256 and N >= 256 and K % 32 == 0 and K >= 128

@@ -106,7 +106,9 @@ int metis_nvfp4_quant_dequant_row(const void *x, int64_t rows, int64_t cols, int
  *   sharing all calls on one device use that device's single array: calls that overlap in time on one
  *           device (two streams, two host threads) race on it and must be ordered by the caller
  * The call never calls hipMalloc/hipFree or any allocating routine; its first call on a device looks the
- * array's address up once (hipGetSymbolAddress).
+ * array's address up once (hipGetSymbolAddress, which may load the code object and place the array) and reads a few
+ * device properties: make that FIRST call per device outside stream capture (any size, e.g. at start-up).  Every later
+ * call only launches two kernels and may be captured into a HIP graph (no memset node is recorded).
  */
 int metis_nvfp4_quant_row_static(const void *x, int64_t rows, int64_t cols, int64_t ld, int mode,
                                  void *codes, void *scales, float *unit, void *stream);

@@ -728,3 +728,36 @@ def test_gradient_of_the_rank_r_scale_vector(L, R):
     torch.testing.assert_close(ops.lowrank_scale_grad(wide[:, :R], xv), got, rtol=1e-4, atol=1e-4)
     assert torch.equal(ops.lowrank_scale_grad(g[:0], xv[:0]), torch.zeros(R, device="cuda"))
     assert torch.equal(ops.lowrank_scale_grad(g, xv, out_dtype=torch.bfloat16), got.bfloat16())
+
+def test_memory_bound_deployments_can_drop_the_derived_weight_copies(monkeypatch):
+    """A cached weight holds 0.5625 B per parameter packed; the tiled binary16 expansion (2 B, one per arithmetic) and
+    the decode layout (0.5625 B) are built on first use.  With both switches off nothing but the packed form stays,
+    and the outputs keep their bits: prefill on the packed operands (binary32 arithmetic) or on an expansion made per
+    call (bf16 arithmetic), decode on the row-major packing."""
+    from metis_hip import ops
+    N, K = 512, 1024
+    w = _weights(171, N, K).cuda()
+    for mode in (0, 1):
+        kw = {"reference_rounding": True, "split_k": False} if mode == 1 else {"split_k": False}   # one order of additions
+        outs = {}
+        for keep in (True, False):
+            monkeypatch.setattr(ops, "tiled_weight_copies", keep)
+            monkeypatch.setattr(ops, "decode_layout_weights", keep)
+            pw = ops.quantize(w, mode)
+            pw.persistent = True
+            ys = []
+            for M in (512, 48):
+                px = ops.quantize(synthetic_activation(172 + M, M, K).cuda(), mode)
+                ys.append(ops.linear_fwd_grouped(px, [(pw, None, None, None)], **kw)[0])
+                ys.append(ops.linear_fwd(px, pw, **kw))
+            held = pw.held_bytes()
+            packed = N * K // 2 + N * K // 16
+            assert held["packed"] == packed
+            if keep:
+                assert held["tiled_pb16" if mode == 1 else "tiled"] >= 2 * N * K and held["decode_layout"] >= packed
+                assert sum(held.values()) >= 3.1 * N * K
+            else:
+                assert set(held) == {"packed"}
+            outs[keep] = ys
+        for a, b in zip(outs[True], outs[False]):
+            assert torch.equal(a, b), mode

@@ -702,6 +702,58 @@ def test_projection_groups_run_as_one_launch_without_autograd(mean_mode, monkeyp
     assert calls["grouped"] == 0
 
 
+def test_grouped_decode_sees_replaced_parameters():
+    """The per-group caches of the decode path (stacked V and s of the members, converted biases, packed weights) key on
+    the parameters' identity as well as their version: a member whose `s`, `vlinear.weight` or residual weight is
+    REPLACED by a fresh Parameter with the same version counter changes the grouped result exactly as it changes the
+    member-by-member evaluation."""
+    pytest.importorskip("transformers")
+    from transformers.models.qwen2.modeling_qwen2 import Qwen2Config, Qwen2DecoderLayer, Qwen2RotaryEmbedding
+    from metis_hip import BitLinear, MetisArgs, replace_model_with_metis
+    torch.manual_seed(0)
+    cfg = Qwen2Config(hidden_size=256, intermediate_size=512, num_attention_heads=4, num_key_value_heads=2,
+                      num_hidden_layers=1, vocab_size=128, max_position_embeddings=256)
+    cfg._attn_implementation = "eager"
+    layer = Qwen2DecoderLayer(cfg, layer_idx=0).to(torch.bfloat16).cuda()
+    for p in layer.parameters():
+        if p.dim() == 2:
+            torch.nn.init.normal_(p, std=0.02)
+    holder = torch.nn.ModuleDict({"layer": layer})
+    replace_model_with_metis(holder, MetisArgs.direct_fp4(forward_svd_rank=32))
+    x = (torch.randn(64, 1, 256, device="cuda") + 0.5).bfloat16()
+    pos = torch.zeros(64, 1, dtype=torch.long, device="cuda")
+    pe = Qwen2RotaryEmbedding(cfg).cuda()(x, pos)
+
+    def run():
+        with torch.no_grad():
+            out = holder["layer"](x, position_embeddings=pe, attention_mask=None, position_ids=pos)
+        return (out[0] if isinstance(out, tuple) else out).float().cpu()
+
+    def same_version(old, new):
+        with torch.no_grad():
+            while new._version < old._version:
+                new.add_(0.0)
+        assert new._version == old._version
+        return new
+
+    base = run()
+    gate = holder["layer"].mlp.gate_proj
+    assert isinstance(gate, BitLinear)
+    for name, owner in (("s", gate), ("weight", gate.vlinear), ("weight", gate.warmup_linear)):
+        old = getattr(owner, name)
+        fresh = same_version(old, torch.nn.Parameter((old.detach() * 1.5 + 0.01).clone()))
+        setattr(owner, name, fresh)
+        grouped = run()
+        BitLinear.grouped_inference = False
+        try:
+            single = run()
+        finally:
+            BitLinear.grouped_inference = True
+        assert not torch.equal(grouped, base), name
+        assert rel_fro(grouped, single) <= 2e-3, name
+        base = grouped
+
+
 @pytest.mark.parametrize("compute", [torch.bfloat16, torch.float32])
 def test_an_unshared_activation_is_quantized_and_projected_in_one_pass(compute, monkeypatch):
     """A BitLinear whose activation no sibling shares (o_proj, down_proj) quantizes it and forms x V^T in one kernel from

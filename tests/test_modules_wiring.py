@@ -261,6 +261,52 @@ def test_rollout_merged_weight_cache_reuses_and_invalidates():
     assert first is second and updated is not first
 
 
+def test_weight_cache_sees_a_replaced_parameter():
+    """A Parameter that is replaced by a fresh one (load_state_dict(assign=True), `layer.weight = nn.Parameter(...)`) starts
+    at the same version counter as the one it replaces: the caches key on the parameter's identity and storage as well."""
+    class CountingQuant(Cast2Fp32):
+        calls = 0
+
+        @classmethod
+        def quantize_dequantize(cls, value):
+            cls.calls += 1
+            return value.detach().clone()
+
+    layer = LinearLowbit(16, 8, bias=False, args=SimpleNamespace(device="cpu", cache_quantized_weight=True))
+    _identity_config()
+    LinearLowbitFunction.q_forward_weight = CountingQuant
+    x = torch.randn(2, 3, 16)
+    first = layer(x)
+    layer(x)
+    assert CountingQuant.calls == 1
+    fresh = torch.nn.Parameter(torch.randn(8, 16))
+    with torch.no_grad():
+        while fresh._version < layer.weight._version:            # the same version counter as the parameter it replaces
+            fresh.add_(0.0)
+    assert fresh._version == layer.weight._version
+    layer.weight = fresh
+    second = layer(x)
+    assert CountingQuant.calls == 2 and not torch.equal(first, second)
+    layer.load_state_dict({"weight": torch.randn(8, 16)}, assign=True)
+    third = layer(x)
+    assert CountingQuant.calls == 3 and not torch.equal(second, third)
+
+
+def test_full_svd_backward_branch_is_refused():
+    """enable_backward_svd with backward_lowrank_svd <= 0 is the reference's full-SVD branch (bitlinear.py:476-486), which
+    this library does not implement: it says so instead of quantizing the gradient with another method."""
+    layer = LinearLowbit(16, 8, bias=False, args=SimpleNamespace(device="cpu", cache_quantized_weight=False))
+    _identity_config()
+    F = LinearLowbitFunction
+    F.enable_backward_svd, F.backward_lowrank_svd = True, 0
+    try:
+        y = layer(torch.randn(2, 3, 16, requires_grad=True))
+        with pytest.raises(NotImplementedError):
+            y.sum().backward()
+    finally:
+        F.enable_backward_svd, F.backward_lowrank_svd = False, 32
+
+
 def test_unsupported_options_fail_loudly():
     args = MetisArgs()
     args.device = "cpu"

@@ -93,6 +93,9 @@ def test_bitlinear_forward_matches_reference(golden):
     y = torch.matmul(y, u.T)
     y = y + O.linear_forward(xq, O.nvfp4_qdq(res), b)
     assert same_bits(y, t(golden["bl_y"]))
+    # and the oracle's own composite, the function the GPU tests compare against: the same sum, rounded to bf16 once
+    got = O.metis_forward(x, v, s, u, res, b, p32=True, quantized_lowrank=True)
+    assert got.dtype == torch.bfloat16 and same_bits(got, t(golden["bl_y"]).bfloat16())
 
 
 def test_c_oracle_binary32_input_mode_matches_torch_restatement():
