@@ -274,6 +274,15 @@ int metis_nvfp4_quant_centered(const void* x, int64_t rows, int64_t cols, int64_
                     workspace, workspace_bytes, (hipStream_t)stream, center);
 }
 
+int metis_nvfp4_quant_lowrank_residual(const void* x, int x_dtype, const void* us, const void* vt, int64_t rows, int64_t cols,
+                                       int rank, int mode, void* codes, void* scales, float* unit, void* dense, void* workspace,
+                                       size_t workspace_bytes, void* stream)
+{
+    if (x_dtype != METIS_DTYPE_BF16 && x_dtype != METIS_DTYPE_F32) return METIS_E_ARG;
+    return quantize_lowrank_residual(x, x_dtype == METIS_DTYPE_F32, us, vt, rows, cols, rank, mode, codes, scales, unit, dense,
+                                     workspace, workspace_bytes, (hipStream_t)stream);
+}
+
 size_t metis_column_mean_workspace_bytes(int64_t cols) { return column_mean_workspace_bytes(cols); }
 
 int metis_column_mean(const void* x, int64_t rows, int64_t cols, int64_t ld, int x_dtype, void* out, int out_dtype,

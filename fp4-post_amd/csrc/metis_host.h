@@ -73,6 +73,9 @@ int deferred_scales(const void* deferred, int64_t rows, int64_t cols, int mode, 
 int quantize_row_static(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, void* codes, void* scales,
                         float* unit, hipStream_t st);
 // codes, scale bytes, unit and the dequantized bf16 tensor of contiguous bf16 rows from one call (two launches); nvfp4_quant.hip
+int quantize_lowrank_residual(const void* x, bool x_f32, const void* us, const void* vt, int64_t rows, int64_t cols, int rank, int mode,
+                              void* codes, void* scales, float* unit, void* dense, void* workspace, size_t workspace_bytes,
+                              hipStream_t st);
 int quantize_dequantize_row(const void* x, int64_t rows, int64_t cols, int mode, void* codes, void* scales, float* unit, void* out,
                             void* workspace, size_t workspace_bytes, hipStream_t st);
 int dequantize(const void* codes, const void* scales, const float* unit, int64_t rows, int64_t cols, int mode, void* out,

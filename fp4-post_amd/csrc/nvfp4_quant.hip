@@ -1137,6 +1137,229 @@ int deferred_scales(const void* deferred, int64_t rows, int64_t cols, int mode, 
 }
 
 // ---------------------------------------------------------------------------------------------
+// "svd" mode of the activation / output-gradient decomposition (src/Metis/Metis/bitlinear.py:283-303): the tensor that is
+// quantized is x - ker with ker = (U diag(s)) V of rank r, and the caller goes on with ker + QDQ(x - ker).  ker is formed
+// in registers: a workgroup owns tiles of 64 rows x 256 columns, a thread one block of 16 columns in four rows, and the
+// factors pass through LDS sixteen ranks at a time.  Every element of ker is the chain
+//     acc = 0;  acc = fma(us[i][k], v[k][j], acc)  for k = 0 .. r-1 in that order, in binary32
+// (bf16 arithmetic: exact products of bf16 factors, the sum rounded to bf16 once, as a bf16 matrix product with
+// binary32 accumulation does) -- a fixed order, so that a CPU restatement reproduces the bits.  Then the residual
+// x - ker (rounded to the arithmetic's type) is encoded like any other block; the codes and the parked block maxima go
+// where the row quantizer puts them, and ker is written out only when the caller wants the dense result.
+// ---------------------------------------------------------------------------------------------
+constexpr int kLrRows = 64, kLrCols = 256, kLrRanks = 16;
+
+template <int MODE, bool F32IN>
+__global__ __launch_bounds__(256) void quant_lowrank_residual_kernel(
+    const void* __restrict__ xv, const void* __restrict__ usv, const void* __restrict__ vtv, uint32_t rows, uint32_t cols,
+    uint32_t rank, uint2* __restrict__ codes, void* __restrict__ ws_amax_v, uint32_t* __restrict__ ws_gmax,
+    void* __restrict__ ker_out, uint32_t tiles_c, uint32_t tiles)
+{
+    static_assert(MODE == 0 || !F32IN, "bf16 arithmetic reads bf16 tensors");
+    __shared__ __align__(16) float s_v[kLrRanks][kLrCols];
+    __shared__ __align__(16) float s_u[kLrRows][kLrRanks];
+    const uint32_t t = threadIdx.x, cb = t & 15u, rg = t >> 4;
+    const uint32_t nbpr = cols / kBlock;
+    float gmax = 0.0f;
+    for (uint32_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+        const uint32_t tr = tile / tiles_c, tc = tile - tr * tiles_c;
+        const uint32_t row0 = tr * kLrRows, col0 = tc * kLrCols;
+        float acc[4][kBlock];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < kBlock; ++j) acc[i][j] = 0.0f;
+        for (uint32_t k0 = 0; k0 < rank; k0 += kLrRanks) {
+            __syncthreads();                                   // the previous chunk (or tile) has been read
+            {   // V: rank k0 + t / 16, columns col0 + 16 (t % 16) ..; zeros beyond the tensor
+                const uint32_t k = k0 + rg, c = col0 + cb * kBlock;
+                float v[kBlock];
+#pragma unroll
+                for (int j = 0; j < kBlock; ++j) v[j] = 0.0f;
+                if (c < cols) {
+                    if constexpr (MODE == 0) {
+                        const float4* p = reinterpret_cast<const float4*>(static_cast<const float*>(vtv) + (size_t)k * cols + c);
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) { const float4 f = p[q]; v[4 * q] = f.x; v[4 * q + 1] = f.y; v[4 * q + 2] = f.z; v[4 * q + 3] = f.w; }
+                    } else {
+                        const uint4* p = reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(vtv) + (size_t)k * cols + c);
+                        unpack16(p[0], p[1], v);
+                    }
+                }
+                float4* d = reinterpret_cast<float4*>(&s_v[rg][cb * kBlock]);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) d[q] = make_float4(v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]);
+            }
+            {   // U diag(s): row row0 + t / 4, ranks k0 + 4 (t % 4) ..
+                const uint32_t r = row0 + (t >> 2), k = k0 + (t & 3u) * 4u;
+                float4 f = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                if (r < rows) {
+                    if constexpr (MODE == 0) f = *reinterpret_cast<const float4*>(static_cast<const float*>(usv) + (size_t)r * rank + k);
+                    else {
+                        const uint2 w = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(usv) + (size_t)r * rank + k);
+                        f = make_float4(bf16_lo(w.x), bf16_hi(w.x), bf16_lo(w.y), bf16_hi(w.y));
+                    }
+                }
+                *reinterpret_cast<float4*>(&s_u[t >> 2][(t & 3u) * 4u]) = f;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int kq = 0; kq < kLrRanks / 4; ++kq) {
+                float4 u4[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) u4[i] = *reinterpret_cast<const float4*>(&s_u[rg * 4 + i][kq * 4]);
+#pragma unroll
+                for (int kk = 0; kk < 4; ++kk) {
+                    float vv[kBlock];
+                    const float4* sp = reinterpret_cast<const float4*>(&s_v[kq * 4 + kk][cb * kBlock]);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) { const float4 f = sp[q]; vv[4 * q] = f.x; vv[4 * q + 1] = f.y; vv[4 * q + 2] = f.z; vv[4 * q + 3] = f.w; }
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float uu = kk == 0 ? u4[i].x : kk == 1 ? u4[i].y : kk == 2 ? u4[i].z : u4[i].w;
+#pragma unroll
+                        for (int j = 0; j < kBlock; ++j) acc[i][j] = fmaf(uu, vv[j], acc[i][j]);
+                    }
+                }
+            }
+        }
+        const uint32_t cbg = tc * (kLrCols / kBlock) + cb;      // block column in the tensor
+        if (cbg < nbpr) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t row = row0 + rg * 4u + (uint32_t)i;
+                if (row >= rows) break;
+                const size_t e0 = (size_t)row * cols + (size_t)cbg * kBlock;
+                float v[kBlock];
+                if constexpr (F32IN) {
+                    const float4* p = reinterpret_cast<const float4*>(static_cast<const float*>(xv) + e0);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) { const float4 f = p[q]; v[4 * q] = f.x; v[4 * q + 1] = f.y; v[4 * q + 2] = f.z; v[4 * q + 3] = f.w; }
+                } else {
+                    const uint4* p = reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(xv) + e0);
+                    unpack16(p[0], p[1], v);
+                }
+                if constexpr (MODE == 0) {
+                    if (ker_out) {
+                        float4* o = reinterpret_cast<float4*>(static_cast<float*>(ker_out) + e0);
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) o[q] = make_float4(acc[i][4 * q], acc[i][4 * q + 1], acc[i][4 * q + 2], acc[i][4 * q + 3]);
+                    }
+#pragma unroll
+                    for (int j = 0; j < kBlock; ++j) v[j] -= acc[i][j];
+                } else {
+                    uint32_t kw[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) kw[j] = bf16_bits(acc[i][2 * j]) | (bf16_bits(acc[i][2 * j + 1]) << 16);
+                    if (ker_out) {
+                        uint4* o = reinterpret_cast<uint4*>(static_cast<uint16_t*>(ker_out) + e0);
+                        o[0] = make_uint4(kw[0], kw[1], kw[2], kw[3]);
+                        o[1] = make_uint4(kw[4], kw[5], kw[6], kw[7]);
+                    }
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        v[2 * j] = rb(v[2 * j] - bf16_lo(kw[j]));
+                        v[2 * j + 1] = rb(v[2 * j + 1] - bf16_hi(kw[j]));
+                    }
+                }
+                const float am = block_amax(v);
+                gmax = fmaxf(gmax, am);
+                const uint32_t blk = row * nbpr + cbg;
+                if constexpr (MODE == 0) {
+                    static_cast<float*>(ws_amax_v)[blk] = am;
+                    codes[blk] = encode_rne_wide(v, block_scalar_ieee(am));
+                } else {
+                    const float none[kBlock] = {};
+                    static_cast<uint16_t*>(ws_amax_v)[blk] = (uint16_t)(__float_as_uint(am) >> 16);
+                    codes[blk] = encode_block<1, false>(v, block_scalar<1>(am), none);
+                }
+            }
+        }
+    }
+    publish_group_max(gmax, ws_gmax, 0u);
+}
+
+// out = ker + QDQ(x - ker), in place on the buffer that holds ker (bitlinear.py:301-303): eight elements per thread
+template <int MODE>
+__global__ __launch_bounds__(256) void lowrank_add_dequant_kernel(const uint32_t* __restrict__ codes, const uint8_t* __restrict__ scales,
+                                                                  const float* __restrict__ unit_p, void* __restrict__ out, int64_t noct)
+{
+    const float unit = *unit_p;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < noct; i += (int64_t)gridDim.x * 256) {
+        const uint32_t c = codes[i];
+        const float dq = rd<MODE>(e4m3_value(scales[i >> 1]) * unit);
+        float o[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t nib = (c >> (4 * j)) & 0xfu, r = nib & 7u;
+            float v = (float)(r + (r > 4u ? r - 4u : 0u) + (r > 6u ? 2u * (r - 6u) : 0u));
+            v = (nib & 8u) ? -v : v;
+            o[j] = rd<MODE>((v * 0.5f) * dq);
+        }
+        if constexpr (MODE == 0) {
+            float4* p = reinterpret_cast<float4*>(out) + i * 2;
+            const float4 a = p[0], b = p[1];
+            p[0] = make_float4(a.x + o[0], a.y + o[1], a.z + o[2], a.w + o[3]);
+            p[1] = make_float4(b.x + o[4], b.y + o[5], b.z + o[6], b.w + o[7]);
+        } else {
+            uint4* p = reinterpret_cast<uint4*>(out) + i;
+            const uint4 k = *p;
+            uint4 w;
+            w.x = rb_pair(bf16_lo(k.x) + o[0], bf16_hi(k.x) + o[1]);
+            w.y = rb_pair(bf16_lo(k.y) + o[2], bf16_hi(k.y) + o[3]);
+            w.z = rb_pair(bf16_lo(k.z) + o[4], bf16_hi(k.z) + o[5]);
+            w.w = rb_pair(bf16_lo(k.w) + o[6], bf16_hi(k.w) + o[7]);
+            *p = w;
+        }
+    }
+}
+
+int quantize_lowrank_residual(const void* x, bool x_f32, const void* us, const void* vt, int64_t rows, int64_t cols, int rank, int mode,
+                              void* codes, void* scales, float* unit, void* dense, void* workspace, size_t workspace_bytes,
+                              hipStream_t st)
+{
+    if (rows < 0 || cols < 0 || rank <= 0) return METIS_E_ARG;
+    if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) return METIS_E_ARG;
+    if (x_f32 && mode != METIS_MODE_P32) return METIS_E_ARG;
+    if (cols % kBlock || rank % kLrRanks) return METIS_E_SHAPE;
+    if (rows == 0 || cols == 0) return METIS_OK;
+    if (!x || !us || !vt || !codes || !scales || !unit) return METIS_E_ARG;
+    if (((uintptr_t)x % 16) || ((uintptr_t)us % 16) || ((uintptr_t)vt % 16) || ((uintptr_t)dense % 16) || ((uintptr_t)codes % 8) ||
+        ((uintptr_t)scales % 8))
+        return METIS_E_ARG;
+    if (rows * cols / kBlock >= (int64_t)1 << 31) return METIS_E_ARG;
+    Workspace ws;
+    if (const int rc = carve_workspace(workspace, workspace_bytes, rows, cols, &ws)) return rc;
+    const uint32_t tiles_c = (uint32_t)((cols + kLrCols - 1) / kLrCols);
+    const int64_t tiles = (int64_t)((rows + kLrRows - 1) / kLrRows) * tiles_c;
+    int64_t g = tiles;
+    if (g > (int64_t)device_cus() * 3) g = (int64_t)device_cus() * 3;          // three workgroups per CU are resident (139 VGPRs)
+    if (g > kMaxGroups) g = kMaxGroups;
+    const uint32_t nblocks = (uint32_t)(rows * cols / kBlock);
+#define METIS_LR(M, F)                                                                                                          \
+    hipLaunchKernelGGL((quant_lowrank_residual_kernel<M, F>), dim3((unsigned)g), dim3(256), 0, st, x, us, vt, (uint32_t)rows,      \
+                       (uint32_t)cols, (uint32_t)rank, (uint2*)codes, (void*)ws.amax, ws.gmax, dense, tiles_c, (uint32_t)tiles)
+    if (mode == METIS_MODE_PB16) METIS_LR(1, false);
+    else if (x_f32) METIS_LR(0, true);
+    else METIS_LR(0, false);
+#undef METIS_LR
+    if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
+    if (const int rc = launch_scales(mode == METIS_MODE_P32 ? METIS_MODE_P32_F32 : METIS_MODE_PB16, ws, (uint32_t)g, scales, unit, nblocks, st,
+                                     nullptr, nullptr, nullptr))
+        return rc;
+    if (dense) {
+        const int64_t noct = rows * cols / 8;
+        const int g3 = grid_for((uint32_t)noct);                 // noct < 2^32: nblocks < 2^31
+        if (mode == METIS_MODE_P32)
+            hipLaunchKernelGGL((lowrank_add_dequant_kernel<0>), dim3(g3), dim3(256), 0, st, (const uint32_t*)codes, (const uint8_t*)scales, unit, dense, noct);
+        else
+            hipLaunchKernelGGL((lowrank_add_dequant_kernel<1>), dim3(g3), dim3(256), 0, st, (const uint32_t*)codes, (const uint8_t*)scales, unit, dense, noct);
+        if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
+    }
+    return METIS_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
 // NV recipe: rotate every tile of 16 along the last dimension, then quantize the rotated tensor (row blocks = tiles),
 // in one pass over x.  Round to nearest, or stochastic rounding on the library's own stream.
 // ---------------------------------------------------------------------------------------------

@@ -29,7 +29,7 @@ import torch.nn as nn
 import torch.nn.init as init
 
 from . import ops
-from .ops import CenteredNVFP4, PackedNVFP4
+from .ops import CenteredNVFP4, LowRankNVFP4, PackedNVFP4
 from .quant import (Cast2Fp32, Cast2NVFp4e2m1Block, Cast2NVFp4e2m1BlockNOSR, QuantFunc, is_hip_nvfp4, quant_func)
 
 __all__ = ["LinearLowbitFunction", "LinearLowbit", "BitLinear"]
@@ -220,6 +220,8 @@ class LinearLowbitFunction(torch.autograd.Function):
         F = LinearLowbitFunction
 
         def lowrank_single(chunk):
+            if broadcast_dim < 0 and F._svd_mode_on_kernels(chunk, quant_func, rank):
+                return F._lowrank_decompose(chunk, quant_func, rank, niter, dense=True).dense.view(chunk.shape)
             picked = broadcast_dim >= 0
             rep = chunk.select(broadcast_dim, 0) if picked else chunk
             shape = rep.shape
@@ -322,17 +324,64 @@ class LinearLowbitFunction(torch.autograd.Function):
         return F.metis_mode == "mean" and not F.tp_simulate and not F.enable_nv_recipe
 
     @staticmethod
-    def _prepare_input(input_: torch.Tensor, mean_cache=None, cache_key="default"):
-        """Packed activation when a kernel path applies (direct: PackedNVFP4; mean mode: CenteredNVFP4), else
-        the dequantized tensor."""
+    def _svd_mode_on_kernels(x: torch.Tensor, q, rank: int) -> bool:
+        """The fused kernel of the "svd" mode takes this tensor: round-to-nearest NVFP4 on a device tensor in binary32 or
+        bf16 arithmetic, rank and width multiples of the block."""
+        return (q is Cast2NVFp4e2m1BlockNOSR and x.is_cuda and x.dtype in (torch.float32, torch.bfloat16) and x.numel() > 0
+                and rank > 0 and rank % 16 == 0 and x.shape[-1] % 16 == 0 and x.dim() in (2, 3))
+
+    @staticmethod
+    def _lowrank_decompose(x: torch.Tensor, q, rank: int, niter: int, dense: bool, arith: torch.dtype | None = None) -> LowRankNVFP4:
+        """Reference 262-303 with the factors from torch.svd_lowrank (randomized, as there): U and V through the
+        quantizer (V stays packed: its three-call QDQ is the packed tensor's dequantization, bit for bit), then ONE
+        fused kernel forms ker = U diag(s) V in registers, encodes x - ker and, with dense, writes ker + QDQ(x - ker).
+        arith: the arithmetic's type when it is not x's own (a bf16 tensor under binary32 arithmetic is widened in the
+        kernel's registers, not copied)."""
+        x2 = _flat2d(x)
+        dt = x2.dtype if arith is None else arith
+        if dt != torch.float32:
+            x2 = x2.to(torch.bfloat16)
+        with torch.amp.autocast(x2.device.type, enabled=False):
+            ug, sg, vg = torch.svd_lowrank(x2.to(torch.float32), q=rank, niter=niter)
+        ug, sg, vt = ug.to(dt), sg.to(dt), vg.to(dt).T.contiguous()
+        s_u = q.get_scalar(ug)
+        us = q.rquant(q.quant(ug, s_u), s_u) * sg              # == ugq @ diag(sg): one nonzero term per sum
+        p_vt = q.pack(vt)
+        mode = ops.MODE_P32 if dt == torch.float32 else ops.MODE_PB16
+        residual, out = ops.quantize_lowrank_residual(x2, us, ops.dequantize(p_vt, dt), mode, dense=dense)
+        return LowRankNVFP4(residual, us, p_vt, out)
+
+    @staticmethod
+    def _scales_formed_by_consumer(rows: int, weights_cached: bool) -> bool:
+        """Whether the GEMM that will read a packed activation forms its scale bytes itself, so that the quantizer may
+        stop after its first launch: the tiled expansion does (it is chosen from 256 rows on when the weight side's
+        expansion is kept, i.e. for cached weights with ops.tiled_weight_copies), and so does every consumer under bf16
+        arithmetic with the reference's roundings.  The packed-operand kernels read the bytes: deferring there only
+        moves the second launch."""
+        F = LinearLowbitFunction
+        return F._bf16_rounding() or (rows >= 256 and weights_cached and ops.tiled_weight_copies)
+
+    @staticmethod
+    def _prepare_input(input_: torch.Tensor, mean_cache=None, cache_key="default", weights_cached: bool = True,
+                       keep_dense: bool | None = None):
+        """Packed activation when a kernel path applies (direct: PackedNVFP4; mean mode: CenteredNVFP4; svd mode:
+        LowRankNVFP4), else the dequantized tensor.  weights_cached: the layers that will read it keep their packed
+        weights across calls.  keep_dense (svd mode): a backward pass will follow; default: autograd is recording."""
         F = LinearLowbitFunction
         if (not F.enable_nv_recipe or F._nv_on_kernels()) and _packable(input_, F.q_forward_input):
             if not F.enable_activation_svd:
                 # the kernels read bf16 values and take the arithmetic as a mode: no upcast copy of a bf16 tensor
-                # from 256 rows on the consumer is the tiled expansion, which forms the scale bytes itself
                 x2 = _flat2d(input_)
-                more = {"deferred": True} if (x2.shape[0] >= 256 or F._bf16_rounding()) else {}
+                more = {"deferred": True} if F._scales_formed_by_consumer(x2.shape[0], weights_cached) else {}
                 return F.q_forward_input.pack(x2, arith=F.compute_dtype, **more)
+            if (F.metis_mode == "svd" and not F.tp_simulate and not F.enable_nv_recipe and F.activation_broadcast_dim < 0
+                    and F._svd_mode_on_kernels(input_, F.q_forward_input, F.activation_lowrank_svd)
+                    and F.compute_dtype in (torch.float32, torch.bfloat16)):
+                # ker + QDQ(x - ker) (reference 243-309): packed residual + the factors; the dense tensor as well when
+                # a backward pass will want it (the factors are randomized: it cannot be derived again)
+                return F._lowrank_decompose(input_, F.q_forward_input, F.activation_lowrank_svd, F.activation_lowrank_niter,
+                                            dense=torch.is_grad_enabled() if keep_dense is None else keep_dense,
+                                            arith=F.compute_dtype)
             if F._mean_mode_packable():
                 # mean + QDQ(x - mean) (reference 311-336) without materialising either: the subtraction happens
                 # inside the quantizer and the mean's contribution to a matmul is a rank-one term
@@ -498,11 +547,29 @@ class LinearLowbitFunction(torch.autograd.Function):
     def forward(ctx, input_, weight, bias, quantized_weight, quantized_input):
         F = LinearLowbitFunction
         if quantized_input is None:
-            quantized_input = F._prepare_input(input_, mean_cache=F.mean_cache, cache_key=F.mean_cache_key)
+            quantized_input = F._prepare_input(input_, mean_cache=F.mean_cache, cache_key=F.mean_cache_key,
+                                               weights_cached=bool(getattr(quantized_weight, "persistent", False)),
+                                               keep_dense=any(ctx.needs_input_grad[:3]))
         lead = input_.shape[:-1]
         ctx.lead = lead
         ctx.has_bias = bias is not None
-        ctx.packed = isinstance(quantized_input, (PackedNVFP4, CenteredNVFP4)) and isinstance(quantized_weight, PackedNVFP4)
+        ctx.packed = (isinstance(quantized_input, (PackedNVFP4, CenteredNVFP4, LowRankNVFP4))
+                      and isinstance(quantized_weight, PackedNVFP4))
+        ctx.lowrank = False
+        if ctx.packed and isinstance(quantized_input, LowRankNVFP4):
+            # "svd" mode: (us V^ + R^) W^^T = R^ W^^T + us (V^ W^^T) -- both products on packed operands, the rank-r
+            # correction a library product in binary32.  The backward pass multiplies with the reference's dense
+            # activation (its factors are randomized and cannot be derived again), kept only when autograd will ask.
+            ctx.pw = quantized_weight
+            ctx.weight_ref = weight
+            ctx.center = None
+            ctx.lowrank = True
+            saved = quantized_input.dense if quantized_input.dense is not None else input_.new_empty(0)
+            ctx.save_for_backward(saved, bias if bias is not None else input_.new_empty(0))
+            vw = ops.linear_fwd(quantized_input.vt, quantized_weight, out_dtype=torch.float32)            # [r, N]
+            out = ops.linear_fwd(quantized_input.residual, quantized_weight, bias=bias, out_dtype=torch.float32)
+            out.addmm_(quantized_input.us.float(), vw)
+            return out.reshape(*lead, quantized_weight.rows).to(F.compute_dtype)
         if ctx.packed:
             ctx.pw = quantized_weight
             ctx.weight_ref = weight
@@ -523,7 +590,7 @@ class LinearLowbitFunction(torch.autograd.Function):
             out = ops.linear_fwd(quantized_input, quantized_weight, bias=bias, out_dtype=out_dtype,
                                  reference_rounding=F.reference_rounding and ctx.center is None)
             return out.reshape(*lead, quantized_weight.rows).to(F.compute_dtype)
-        if isinstance(quantized_input, (PackedNVFP4, CenteredNVFP4)):
+        if isinstance(quantized_input, (PackedNVFP4, CenteredNVFP4, LowRankNVFP4)):
             quantized_input = quantized_input.dequantize(F.compute_dtype).reshape(input_.shape)
         if isinstance(quantized_weight, PackedNVFP4):
             quantized_weight = quantized_weight.dequantize(F.compute_dtype)
@@ -543,7 +610,7 @@ class LinearLowbitFunction(torch.autograd.Function):
         if ctx.packed:
             input_, _ = ctx.saved_tensors
             L, N = _flat2d(grad_output).shape
-            if F._packed_backward_applies(L, N, grad_output):
+            if not ctx.lowrank and F._packed_backward_applies(L, N, grad_output):
                 # dgrad: contraction over N; wgrad: contraction over tokens.  Operands are packed straight from the
                 # tensors autograd hands over, in compute_dtype arithmetic (no upcast copies of bf16 tensors).
                 cd = F.compute_dtype
@@ -566,7 +633,12 @@ class LinearLowbitFunction(torch.autograd.Function):
             grad_output = grad_output.to(F.compute_dtype)
             dy2 = _flat2d(grad_output)
             x2 = _flat2d(input_.to(F.compute_dtype))
-            if ctx.center is not None:
+            if ctx.lowrank:
+                if x2.numel() == 0:
+                    raise RuntimeError("the svd-mode activation was prepared without autograd (no dense tensor kept) but a "
+                                       "backward pass asks for it")
+                xq = x2                                          # the reference's saved activation ker + QDQ(x - ker) itself
+            elif ctx.center is not None:
                 xq = ctx.center.to(F.compute_dtype) + F.q_forward_input.quantize_dequantize(x2 - ctx.center.to(F.compute_dtype))
             else:
                 xq = F.q_forward_input.quantize_dequantize(x2)
@@ -620,6 +692,11 @@ class LinearLowbit(nn.Module):
     def forward(self, input, quantized_input=None):
         F = LinearLowbitFunction
         bias_compute = self.bias.to(self.compute_dtype) if self.bias is not None else None
+        if quantized_input is None and F.enable_activation_svd and F.metis_mode == "svd":
+            # decomposed here, where autograd's recording state is visible (inside the Function it never is): the dense
+            # activation is written only when a backward pass can follow
+            quantized_input = F._prepare_input(input, mean_cache=F.mean_cache, cache_key=F.mean_cache_key,
+                                               weights_cached=self.cache_quantized_weight)
         if (not F.enable_nv_recipe or F._nv_on_kernels()) and _packable(self.weight, F.q_forward_weight) and self.weight.shape[0] % 4 == 0:
             # kernel path: packed straight from the stored parameter in compute_dtype arithmetic, so a cache hit
             # costs no pass over the weight at all
@@ -829,16 +906,22 @@ class BitLinear(nn.Module):
         self._merged_rollout_tiled = None
         self.layer_name = ""
 
+    def _weights_cached(self) -> bool:
+        """The packed weights of this layer's quantized branches live across calls (cache_quantized_weight)."""
+        return bool(getattr(self.args, "cache_quantized_weight", False))
+
     # ------------------------------------------------------------------ shared activation (reference 676-702)
     def _get_shared_quantized_input(self, x: torch.Tensor):
         F = LinearLowbitFunction
         group = getattr(self, "activation_group", None)
         if group is None:
-            return F._prepare_input(x, mean_cache=self.mean_cache, cache_key=f"{self.layer_name}.shared")
+            return F._prepare_input(x, mean_cache=self.mean_cache, cache_key=f"{self.layer_name}.shared",
+                                    weights_cached=self._weights_cached())
         input_ref = group.get("input_ref")
         if input_ref is not None and input_ref() is x:
             return group["quantized_input"]
-        quantized_input = F._prepare_input(x, mean_cache=group["mean_cache"], cache_key=f"{group['name']}.shared")
+        quantized_input = F._prepare_input(x, mean_cache=group["mean_cache"], cache_key=f"{group['name']}.shared",
+                                           weights_cached=all(m._weights_cached() for m in group.get("members", ())))
 
         def clear_cached_input(ref):
             if group.get("input_ref") is ref:
@@ -901,7 +984,7 @@ class BitLinear(nn.Module):
                                shared_input.unit, shared_input.rows, merged.shape[0], shared_input.cols, mode=ops.MODE_PB16,
                                bias=None if bias is None else bias.to(torch.bfloat16), out_dtype=torch.bfloat16)
             return y.reshape(*x_shape[:-1], merged.shape[0])
-        if isinstance(shared_input, (PackedNVFP4, CenteredNVFP4)):
+        if isinstance(shared_input, (PackedNVFP4, CenteredNVFP4, LowRankNVFP4)):
             shared_input = shared_input.dequantize(F.compute_dtype).reshape(x_shape)
         merged = self._get_merged_rollout_weight(shared_input.dtype)
         y = torch.matmul(shared_input, merged.T)

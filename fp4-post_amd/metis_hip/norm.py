@@ -116,10 +116,9 @@ class FusedRMSNormQuant(nn.Module):
                 normed, packed = got
                 packed.residual.shared = True
             else:
-                # the tiled expansion (256 rows or more) and the ready decode operands of bf16 arithmetic form the scale
-                # bytes themselves
+                cached = all(m._weights_cached() for m in self.group.get("members", ()))
                 normed, packed = ops.rmsnorm_quantize(x, self.weight, self.variance_epsilon, mode,
-                                                      deferred=x.numel() // cols >= 256 or F._bf16_rounding())
+                                                      deferred=F._scales_formed_by_consumer(x.numel() // cols, cached))
         normed = normed.reshape(x.shape)
         out = _NormedWithGrad.apply(x, self.weight, normed, self.variance_epsilon) if torch.is_grad_enabled() and (
             x.requires_grad or self.weight.requires_grad) else normed

@@ -120,6 +120,32 @@ class CenteredNVFP4:
         return self.mean.to(dtype).unsqueeze(0) + dequantize(self.residual, dtype)
 
 
+@dataclass
+class LowRankNVFP4:
+    """"svd"-mode activation: value = us @ deq(vt) + deq(residual) (reference src/Metis/Metis/bitlinear.py:296-303).
+    `us` [rows, r] is U (after its QDQ) times diag(s), in the arithmetic's type; `vt` is V after its QDQ, kept packed
+    (its QDQ is the packed tensor's dequantization), so that products with a packed weight run on the packed GEMM;
+    `residual` packs x - ker.  `dense` (when the producer wrote it) is the reference's own tensor ker + QDQ(x - ker)."""
+    residual: PackedNVFP4
+    us: torch.Tensor
+    vt: PackedNVFP4
+    dense: torch.Tensor | None = None
+
+    @property
+    def rows(self) -> int:
+        return self.residual.rows
+
+    @property
+    def cols(self) -> int:
+        return self.residual.cols
+
+    def dequantize(self, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+        if self.dense is not None:
+            return self.dense.to(dtype)
+        # without the dense tensor: a library product in the arithmetic's type (agrees with the kernel's ker to rounding)
+        return (self.us @ dequantize(self.vt, self.us.dtype)).to(dtype) + dequantize(self.residual, dtype)
+
+
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
 
@@ -259,6 +285,41 @@ def quantize_dequantize(x: torch.Tensor, mode: int = MODE_P32) -> tuple[PackedNV
     rc = load().metis_nvfp4_quant_dequant_row(x2.data_ptr(), rows, cols, mode, codes.data_ptr(), scales.data_ptr(), unit.data_ptr(),
                                               out.data_ptr(), ws.data_ptr(), ws.numel(), _stream())
     check(rc, "metis_nvfp4_quant_dequant_row", x.shape)
+    return PackedNVFP4(codes, scales, unit, rows, cols, mode), out
+
+
+def quantize_lowrank_residual(x: torch.Tensor, us: torch.Tensor, vt: torch.Tensor, mode: int = MODE_P32,
+                              dense: bool = False) -> tuple[PackedNVFP4, torch.Tensor | None]:
+    """The packed residual QDQ(x - ker) with ker = us @ vt formed in registers (the "svd" mode of the activation
+    decomposition, src/Metis/Metis/bitlinear.py:296-303), and with dense=True also ker + QDQ(x - ker).
+    MODE_P32: us, vt binary32, x bf16 or binary32, dense binary32; MODE_PB16: all bf16.  x [rows, cols], us [rows, r],
+    vt [r, cols], r a multiple of 16.  ker sums its r products in the order k = 0 .. r-1 with fused multiply-adds."""
+    if not x.is_cuda:
+        raise RuntimeError("metis_hip kernels need tensors on the GPU")
+    x2 = x.reshape(-1, x.shape[-1]).contiguous()
+    rows, cols = x2.shape
+    r = us.shape[-1]
+    want = torch.float32 if mode == MODE_P32 else torch.bfloat16
+    if mode not in (MODE_P32, MODE_PB16) or us.dtype != want or vt.dtype != want:
+        raise ValueError("the factors come in the arithmetic's type: binary32 for MODE_P32, bf16 for MODE_PB16")
+    if x2.dtype != torch.bfloat16 and not (mode == MODE_P32 and x2.dtype == torch.float32):
+        raise ValueError(f"unsupported tensor type {x2.dtype} for this arithmetic")
+    if tuple(us.shape) != (rows, r) or tuple(vt.shape) != (r, cols):
+        raise ValueError(f"factors {tuple(us.shape)} x {tuple(vt.shape)} do not give {tuple(x2.shape)}")
+    if cols % BLOCK or r % BLOCK or r == 0:
+        raise ValueError(f"NVFP4 block shape (1, 16) does not divide {tuple(x.shape)} or the rank {r}")
+    us, vt = us.contiguous(), vt.contiguous()
+    dev = x2.device
+    codes = torch.empty(rows, cols // 2, dtype=torch.uint8, device=dev)
+    scales = torch.empty(rows, cols // BLOCK, dtype=torch.uint8, device=dev)
+    unit = torch.empty(1, dtype=torch.float32, device=dev)
+    out = torch.empty(rows, cols, dtype=want, device=dev) if dense else None
+    ws = _workspace(rows, cols, dev)
+    rc = load().metis_nvfp4_quant_lowrank_residual(x2.data_ptr(), DTYPE_F32 if x2.dtype == torch.float32 else DTYPE_BF16, us.data_ptr(),
+                                                   vt.data_ptr(), rows, cols, r, mode, codes.data_ptr(), scales.data_ptr(),
+                                                   unit.data_ptr(), None if out is None else out.data_ptr(), ws.data_ptr(),
+                                                   ws.numel(), _stream())
+    check(rc, "metis_nvfp4_quant_lowrank_residual", (rows, cols, r))
     return PackedNVFP4(codes, scales, unit, rows, cols, mode), out
 
 

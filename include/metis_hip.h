@@ -391,6 +391,29 @@ int metis_nvfp4_deferred_scales(const void *deferred, int64_t rows, int64_t cols
                                 float *unit, void *stream);
 
 /*
+ * "svd" mode of the activation / output-gradient decomposition (LinearLowbitFunction.svd_quant with metis_mode = "svd",
+ * src/Metis/Metis/bitlinear.py:243-309): with the factors of a rank-r approximation in hand (torch.svd_lowrank, U and V
+ * through the three-call QDQ, :270-293), the reference forms ker = U diag(s) V (:296), quantizes x - ker (:300-301) and
+ * goes on with ker + QDQ(x - ker) (:303).  This call does the three steps without storing ker or the residual: ker is
+ * formed tile by tile in registers, the residual is encoded there, and the dense sum is written only when asked for.
+ *   x        [rows, cols] contiguous: bf16, or (mode METIS_MODE_P32 only) binary32 with x_dtype = METIS_DTYPE_F32
+ *   us       [rows, rank]  U diag(s), i.e. `ug @ torch.diag(sg)`: binary32 (METIS_MODE_P32) or bf16 (METIS_MODE_PB16)
+ *   vt       [rank, cols]  V after `vg = vg.T`, same type as us
+ *   mode     METIS_MODE_P32: everything in binary32 (compute_dtype = float32); METIS_MODE_PB16: ker rounded to bf16 once
+ *            after binary32 accumulation, the subtraction and the quantizer in bf16 arithmetic
+ *   codes, scales, unit   the packed residual QDQ(x - ker), as metis_nvfp4_quant_row writes them
+ *   dense    NULL, or [rows, cols] in the arithmetic's type (binary32 / bf16): receives ker + QDQ(x - ker)
+ *   workspace  metis_nvfp4_workspace_bytes(rows, cols)
+ * Every element of ker is the chain acc = fma(us[i][k], vt[k][j], acc) over k = 0 .. rank-1 in that order in binary32
+ * (a library matrix product sums in an order of its own: results agree to rounding, not to the bit).
+ * Limits: cols % 16 == 0, rank % 16 == 0, 16-byte aligned tensors.  Two launches, three with dense.
+ */
+int metis_nvfp4_quant_lowrank_residual(const void *x, int x_dtype, const void *us, const void *vt,
+                                       int64_t rows, int64_t cols, int rank, int mode, void *codes,
+                                       void *scales, float *unit, void *dense, void *workspace,
+                                       size_t workspace_bytes, void *stream);
+
+/*
  * Mean mode in bf16 arithmetic: the activation the reference multiplies with is X^ = me + QDQ(X - me) as ONE bf16
  * tensor, the sum rounded to bf16 (LinearLowbitFunction.svd_quant with metis_mode = "mean",
  * src/Metis/Metis/bitlinear.py:311-336, under compute_dtype = bfloat16).  This is metis_nvfp4_expand_tiled with

@@ -42,6 +42,8 @@ def lib():
         L.metis_oracle_f32_to_bf16.argtypes = [f32]
         L.metis_oracle_f32_to_bf16.restype = ctypes.c_uint16
         L.metis_oracle_threads.restype = i32
+        L.metis_oracle_lowrank_product.argtypes = [vp, vp, i64, i64, i64, vp]
+        L.metis_oracle_lowrank_product.restype = i32
         _lib = L
     return _lib
 
@@ -104,3 +106,13 @@ def e4m3_decode(b: int) -> float:
 
 def threads() -> int:
     return int(lib().metis_oracle_threads())
+
+
+def lowrank_product(us: torch.Tensor, vt: torch.Tensor) -> torch.Tensor:
+    """us [rows, r] @ vt [r, cols] in binary32 with the additions in the order k = 0 .. r-1, one fused multiply-add each."""
+    assert us.dtype == torch.float32 and vt.dtype == torch.float32 and us.shape[1] == vt.shape[0]
+    us, vt = us.contiguous(), vt.contiguous()
+    ker = torch.empty(us.shape[0], vt.shape[1], dtype=torch.float32)
+    rc = lib().metis_oracle_lowrank_product(_p(us), _p(vt), us.shape[0], vt.shape[1], us.shape[1], _p(ker))
+    assert rc == 0
+    return ker

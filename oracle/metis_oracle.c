@@ -15,6 +15,8 @@
  *   src/Metis/Metis/quant.py:137-147   stochastic rounding: += rand - 0.5 before round
  *   src/Metis/Metis/quant.py:435-477   get_scalar / quant / rquant
  *   src/Metis/models/llama.py:23-31    RMSNorm
+ *   src/Metis/Metis/bitlinear.py:296   ker = ug @ diag(sg) @ vg, with the summation order FIXED here (see
+ *                                      metis_oracle_lowrank_product; the reference leaves it to its BLAS)
  * Third-party arithmetic restated from its published definition (absent from the reference
  * tree): the float8_e4m3fn cast of PyTorch (OCP FP8 E4M3: bias 7, 3 mantissa bits, no
  * infinities, 0x7F/0xFF = NaN, round-to-nearest-even, values that round above 448 -> NaN).
@@ -239,6 +241,24 @@ int metis_oracle_rmsnorm_nvfp4(const uint16_t *x, const uint16_t *gamma, float e
     if (cols % BLK) return -1;
     metis_oracle_rmsnorm(x, gamma, eps, rows, cols, normed);
     return metis_oracle_nvfp4_pack(normed, rows, cols, cols, mode, NULL, codes, scales, unit, NULL);
+}
+
+/*
+ * ker = us @ vt (src/Metis/Metis/bitlinear.py:296 after `ug @ torch.diag(sg)`), binary32, [rows, rank] x [rank, cols].
+ * The reference calls a library matrix product, whose order of additions is the library's own.  This restatement fixes
+ * one: acc = 0; acc = fma(us[i][k], vt[k][j], acc) for k = 0 .. rank-1.  It is the order the HIP kernel uses, so the two
+ * agree bit for bit; against the reference's product it agrees to rounding (checked on the reference's own vectors).
+ */
+int metis_oracle_lowrank_product(const float *us, const float *vt, int64_t rows, int64_t cols, int64_t rank, float *ker)
+{
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < rows; ++i)
+        for (int64_t j = 0; j < cols; ++j) {
+            float acc = 0.0f;
+            for (int64_t k = 0; k < rank; ++k) acc = fmaf(us[i * rank + k], vt[k * cols + j], acc);
+            ker[i * cols + j] = acc;
+        }
+    return 0;
 }
 
 int metis_oracle_threads(void)

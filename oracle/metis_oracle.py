@@ -21,6 +21,7 @@ Reference files followed (paths relative to the reference checkout):
   src/Metis/Metis/bitlinear.py:407-441   LinearLowbitFunction.forward
   src/Metis/Metis/bitlinear.py:443-513   LinearLowbitFunction.backward
   src/Metis/Metis/bitlinear.py:736-769   BitLinear.forward
+  src/Metis/Metis/bitlinear.py:243-309   svd_quant, metis_mode="svd" (factors given)
 
 Pinning status (which independent evidence fixes each function) is listed in
 ``tests/test_oracle_pins.py`` and in the design notes; nothing here is "parity
@@ -132,6 +133,27 @@ def rquant(xq: torch.Tensor, s: torch.Tensor) -> torch.Tensor:
     s2 = s.to(torch.float8_e4m3fn).to(s.dtype)
     s2 *= smax / 448
     return (b * s2.reshape(b.shape[0], b.shape[1], 1)).reshape(xq.shape)
+
+
+# ----------------------------------------------------------------------------- "svd" mode, factors given
+def svd_mode_recompose(x: torch.Tensor, ug: torch.Tensor, sg: torch.Tensor, vg: torch.Tensor, ker: torch.Tensor | None = None):
+    """bitlinear.py:276-303 from the point where the factors exist: x [L, D], ug [L, r], sg [r], vg [r, D] (already
+    `vg.T`), all in the dtype D of the arithmetic.  U and V go through the three calls, ker = ug @ diag(sg) @ vg, the
+    residual through the fused QDQ.  Returns (ker, residual QDQ, ker + residual QDQ).
+
+    ker: the reference's matrix product leaves the order of its additions to the BLAS; this restatement takes
+    `ug @ diag(sg)` as the elementwise product it is (one nonzero term per sum) and sums the second product in the
+    order k = 0 .. r-1 with fused multiply-adds in binary32 (oracle/metis_oracle.c), rounding to bf16 once in bf16
+    arithmetic.  A caller may pass another ker (the reference's own) to check everything behind it bit for bit."""
+    from . import c_oracle
+    s_u, s_v = get_scalar(ug), get_scalar(vg)
+    ugq = rquant(quant(ug, s_u), s_u)
+    vgq = rquant(quant(vg, s_v), s_v)
+    if ker is None:
+        us = ugq * sg                                  # == ugq @ diag(sg): every other term of the sums is an exact zero
+        ker = c_oracle.lowrank_product(us.float(), vgq.float()).to(x.dtype)
+    res = nvfp4_qdq(x - ker)
+    return ker, res, ker + res
 
 
 # ----------------------------------------------------------------------------- packed view

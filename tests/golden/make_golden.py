@@ -5,6 +5,7 @@ Run once, in the build container only (the reference checkout does not exist on 
     python tests/golden/make_golden.py [/root/reference]
     python tests/golden/make_golden.py /root/reference hadamard_wide     (only metis_reference_hadamard_wide.npz)
     python tests/golden/make_golden.py /root/reference rollout_bf16      (only metis_reference_rollout_bf16.npz)
+    python tests/golden/make_golden.py /root/reference svd_mode          (only metis_reference_svd_mode.npz)
 
 Why an import and not only closed forms: the results recorded here depend on the exact
 sequence of per-op roundings of eager PyTorch (bf16-per-op mode differs from an ideal
@@ -379,8 +380,57 @@ def golden_rollout_bf16(out: dict):
         rb.LinearLowbitFunction.compute_dtype = torch.float32
 
 
+def golden_svd_mode(out: dict):
+    """LinearLowbitFunction.svd_quant with metis_mode="svd" (bitlinear.py:243-309) on a [2, 64, 256] activation, rank 32,
+    in binary32 and in bf16 arithmetic.  The factors come from torch.svd_lowrank, which draws from torch's random
+    stream: a recording wrapper around it keeps what it returned, so that a consumer of this file starts from the same
+    factors.  ker is not returned by the reference; it is recomputed here by the reference's own expressions
+    (:276-296) on the reference's quantizer, for the comparison of summation orders."""
+    q = rq.Cast2NVFp4e2m1BlockNOSR
+    g = torch.Generator().manual_seed(71)
+    B, T, D, r = 2, 64, 256, 32
+    low = torch.randn(B * T, 6, generator=g) @ torch.randn(6, D, generator=g)
+    x = (low + 0.3 * torch.randn(B * T, D, generator=g)).reshape(B, T, D)
+    x[..., 7] *= 12.0
+    for tag, dt in (("f32", torch.float32), ("bf16", torch.bfloat16)):
+        xin = x.bfloat16().to(dt)                     # bf16 values in both cases
+        kept = {}
+        real = torch.svd_lowrank
+
+        def recording(a, q=6, niter=2, M=None):
+            u, s, v = real(a, q=q, niter=niter, M=M)
+            kept["u"], kept["s"], kept["v"] = u.clone(), s.clone(), v.clone()
+            return u, s, v
+
+        torch.manual_seed(1000 + len(tag))
+        torch.svd_lowrank = recording
+        try:
+            y = rb.LinearLowbitFunction.svd_quant(xin.clone(), quant_func=q, rank=r, niter=2, broadcast_dim=-1, metis_mode="svd")
+        finally:
+            torch.svd_lowrank = real
+        ug, sg, vg = kept["u"].to(dt), kept["s"].to(dt), kept["v"].to(dt).T
+        us_, vs_ = q.get_scalar(ug), q.get_scalar(vg)
+        ugq = q.rquant(q.quant(ug, us_), us_)
+        vgq = q.rquant(q.quant(vg, vs_), vs_)
+        ker = ugq @ torch.diag(sg) @ vgq
+        again = ker + q.quantize_dequantize(xin.reshape(-1, D) - ker)
+        assert torch.equal(again.view(B, T, D), y)    # the recomputation follows the reference's path
+        out[f"svd_{tag}_x"] = bits(xin.bfloat16())    # bf16 values in both cases
+        out[f"svd_{tag}_u"], out[f"svd_{tag}_s"], out[f"svd_{tag}_v"] = bits(kept["u"]), bits(kept["s"]), bits(kept["v"])
+        out[f"svd_{tag}_uq"], out[f"svd_{tag}_vq"] = bits(ugq), bits(vgq)
+        out[f"svd_{tag}_ker"] = bits(ker)
+        out[f"svd_{tag}_y"] = bits(y)
+
+
 def main():
     torch.set_num_threads(1)
+    if len(sys.argv) > 2 and sys.argv[2] == "svd_mode":         # only this file (the others are not touched)
+        sv: dict = {}
+        golden_svd_mode(sv)
+        path = os.path.join(HERE, "metis_reference_svd_mode.npz")
+        np.savez_compressed(path, **sv)
+        print(f"wrote {path}: {len(sv)} arrays, {os.path.getsize(path)} bytes")
+        return
     if len(sys.argv) > 2 and sys.argv[2] == "rollout_bf16":     # only this file (the others are not touched)
         ro16: dict = {}
         golden_rollout_bf16(ro16)

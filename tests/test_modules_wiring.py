@@ -431,3 +431,21 @@ def test_merge_tool_restores_plain_linear_weights(tmp_path):
     merge_main([str(src), str(dst), "--dtype", "bf16"])
     back = load_file(str(dst))
     assert set(back) == set(reference_weights) and all(t.dtype == torch.bfloat16 for t in back.values())
+
+
+def test_scale_bytes_are_deferred_only_when_the_consumer_forms_them(monkeypatch):
+    """The quantizer may stop after its first launch when the GEMM that follows forms the scale bytes itself: the tiled
+    expansion (256 rows or more, cached weights, tiled copies kept) or any consumer under bf16 arithmetic with the
+    reference's roundings.  Row count alone does not decide."""
+    from metis_hip import ops
+    from metis_hip.bitlinear import LinearLowbitFunction as F
+    monkeypatch.setattr(F, "compute_dtype", torch.float32)
+    monkeypatch.setattr(F, "reference_rounding", True)
+    assert F._scales_formed_by_consumer(4096, True) and not F._scales_formed_by_consumer(4096, False)
+    assert not F._scales_formed_by_consumer(64, True)
+    monkeypatch.setattr(ops, "tiled_weight_copies", False)
+    assert not F._scales_formed_by_consumer(4096, True)
+    monkeypatch.setattr(F, "compute_dtype", torch.bfloat16)
+    assert F._scales_formed_by_consumer(4096, False) and F._scales_formed_by_consumer(1, False)
+    monkeypatch.setattr(F, "reference_rounding", False)
+    assert not F._scales_formed_by_consumer(1, False)

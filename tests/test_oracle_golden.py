@@ -137,3 +137,31 @@ def test_mean_mode_formula_matches_reference(tag, dt):
     assert int(g[f"mean_step_count_{tag}"][0]) == count + step.shape[0]
     assert same_bits(me2, t(g[f"mean_step_cache_{tag}"]))
     assert same_bits((me2 + O.nvfp4_qdq(step - me2)).reshape(4, 1, 64), t(g[f"mean_step_out_{tag}"]))
+
+
+@pytest.mark.parametrize("tag,dt", [("f32", "float32"), ("bf16", "bfloat16")])
+def test_svd_mode_recomposition_matches_reference(tag, dt):
+    """svd_quant(metis_mode="svd") of the reference (bitlinear.py:243-309), restated from the point where the factors of
+    its torch.svd_lowrank call exist (they are recorded in the fixture).  The restatement fixes the order in which ker's
+    rank products are added (k ascending, one fused multiply-add each); on the reference's vectors that order
+    reproduces its library product bit for bit -- ker and the final tensor -- and with the reference's own ker handed
+    in, everything behind it (residual, QDQ, sum) is bit-exact by construction of the same op sequence.  A transposed
+    factor, a dropped diag(s) or a quantizer applied to the wrong operand changes every element."""
+    import os
+    import numpy as np
+    g = dict(np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "metis_reference_svd_mode.npz")))
+    D = getattr(torch, dt)
+    x = t(g[f"svd_{tag}_x"]).to(D).reshape(-1, 256)
+    u, s, v = (t(g[f"svd_{tag}_{n}"]) for n in "usv")
+    ug, sg, vg = u.to(D), s.to(D), v.to(D).T.contiguous()
+    ker, res, y = O.svd_mode_recompose(x, ug.clone(), sg, vg.clone())
+    assert same_bits(ker, t(g[f"svd_{tag}_ker"]))
+    assert same_bits(y.reshape(2, 64, 256), t(g[f"svd_{tag}_y"]))
+    _, _, y2 = O.svd_mode_recompose(x, ug.clone(), sg, vg.clone(), ker=t(g[f"svd_{tag}_ker"]))
+    assert same_bits(y2.reshape(2, 64, 256), t(g[f"svd_{tag}_y"]))
+    # the fixed order is one valid evaluation of the product: against torch's own matmul it agrees to rounding
+    uq, vq = t(g[f"svd_{tag}_uq"]), t(g[f"svd_{tag}_vq"])
+    lib = (uq @ torch.diag(sg) @ vq).float()
+    assert float((ker.float() - lib).abs().max()) <= (1e-5 if dt == "float32" else 2 ** -7) * float(lib.abs().max())
+    # and a wrong order of factors is nowhere near
+    assert not same_bits(C.lowrank_product((uq.float() * sg.float()).contiguous(), vq.float().flip(0).contiguous()).to(D), ker)
