@@ -644,6 +644,35 @@ def main():
         except Exception as exc:
             qat["three_projections"] = {"error": f"{type(exc).__name__}: {exc}"[:300]}
 
+    # ------------------------------------------------------------------ the "svd" mode of the activation decomposition:
+    # ker = U diag(s) V formed in registers, x - ker encoded, packed residual (and the dense sum) written
+    svd_leg = None
+    if not args.no_decode:
+        try:
+            gs = torch.Generator().manual_seed(1007)
+            Ls, Ds, rs = 4096, 3584, 64
+            xs_ = outlier_activation(torch, 1008, Ls, Ds, dev)
+            us32 = (torch.randn(Ls, rs, generator=gs) * 0.3).to(dev)
+            vt32 = (torch.randn(rs, Ds, generator=gs) / Ds ** 0.5).to(dev)
+            flops_s = 2.0 * Ls * Ds * rs
+            svd_leg = {"workload": f"metis_nvfp4_quant_lowrank_residual on bf16 [{Ls},{Ds}], rank {rs}: binary32 fused multiply-adds on the "
+                                   "vector units in a fixed order (bit parity with the CPU restatement), 2 r flops and 2.5625 B per element",
+                       "bound": "valu_f32", "peak": 157.3, "unit": "TFLOP/s"}
+            for tag, mode_, u_, v_ in (("binary32", ops.MODE_P32, us32, vt32), ("bf16", ops.MODE_PB16, us32.bfloat16(), vt32.bfloat16())):
+                for dense_ in (False, True):
+                    us_t = region_us(torch, lambda ev: ops.quantize_lowrank_residual(xs_, u_, v_, mode_, dense=dense_), 20, 5)
+                    svd_leg[f"{tag}_{'dense' if dense_ else 'packed'}_us"] = round(us_t, 2)
+                    if not dense_:
+                        svd_leg[f"{tag}_frac"] = round(flops_s / (us_t * 1e-6) / 1e12 / 157.3, 4)
+            from metis_hip.quant import Cast2NVFp4e2m1BlockNOSR as Qn
+
+            def op_by_op(ev=None):
+                ker = us32 @ vt32
+                return ker + Qn.quantize_dequantize(xs_.float() - ker)
+            svd_leg["binary32_op_by_op_us"] = round(region_us(torch, op_by_op, 10, 3), 2)
+        except Exception as exc:  # an optional leg must not cost the headline line
+            svd_leg = {"error": f"{type(exc).__name__}: {exc}"[:300]}
+
     # ------------------------------------------------------------------ a tile-starved shape: 1024-token prefill
     # through the Qwen2.5-7B down projection (56 output tiles on 256 CUs; K split through a workspace)
     prefill = None
@@ -802,6 +831,8 @@ def main():
         line["qat_projection"] = qat
     if prefill is not None:
         line["short_prefill_projection"] = prefill
+    if svd_leg is not None:
+        line["svd_mode_residual_quant"] = svd_leg
     if not args.no_cpu_baseline:
         torch_threads = torch.get_num_threads()
         cpu_tflops, cpu_dt, cpu_reps = cpu_baseline_linear(torch, x, v, s, u, res)

@@ -758,7 +758,6 @@ def rmsnorm_quantize(x: torch.Tensor, gamma: torch.Tensor, eps: float, mode: int
     return normed, PackedNVFP4(codes, scales, unit, rows, cols, mode)
 
 
-@functools.lru_cache(maxsize=16)
 def rmsnorm_colmean(x: torch.Tensor, gamma: torch.Tensor, eps: float, mean_dtype: torch.dtype = torch.float32,
                     cached: torch.Tensor | None = None, cached_count: int = 0):
     """RMSNorm for the mean mode: (normed bf16 [R, C], column mean of normed over its rows in mean_dtype, the same as
@@ -790,6 +789,7 @@ def rmsnorm_colmean(x: torch.Tensor, gamma: torch.Tensor, eps: float, mean_dtype
     return normed, me, me32
 
 
+@functools.lru_cache(maxsize=16)
 def _device_cus(device_index: int) -> int:
     return int(torch.cuda.get_device_properties(device_index).multi_processor_count)
 

@@ -38,6 +38,9 @@ def main(reps: int = 5):
     s = torch.rand(64, generator=g).bfloat16().cuda()
     dy = (torch.randn(8192, 14336, generator=g) * 1e-3).bfloat16().cuda()
     y = torch.empty_like(x)
+    xs = x[:4096, :3584].contiguous()                                   # svd mode: [4096, 3584], rank 64
+    us = (torch.randn(4096, 64, generator=g) * 0.3).cuda()
+    vt = (torch.randn(64, 3584, generator=g) / 60).cuda()
     pw = ops.quantize(w)
     pw.persistent = True                                                # a cached weight: the pipelined GEMM on tiled expansions
     for _ in range(reps):
@@ -47,6 +50,11 @@ def main(reps: int = 5):
         # deferred scale bytes: the quantizers' first launch alone, the expansion forms unit and bytes (expand_xt_kernel<0, 0, 1, 0>)
         ops.expand_tiled(ops.quantize(x, deferred=True), cache=False)
         ops.rmsnorm_quantize(h, gamma, 1e-6, deferred=True)
+        ops.quantize_dequantize(x)                                      # round trip: quant_codes_contig_kernel + quant_scales_dequant_kernel
+        normed, me, _ = ops.rmsnorm_colmean(h, gamma, 1e-6, torch.float32)   # mean mode: rmsnorm_colsum_rows_kernel + finish
+        ops.quantize(normed, 0, center=me)                              # ... and the centred quantizer on the normed tensor
+        ops.quantize_lowrank_residual(xs, us, vt, 0)                    # svd mode: quant_lowrank_residual_kernel + scales
+        ops.quantize_lowrank_residual(xs, us, vt, 0, dense=True)        # ... + lowrank_add_dequant_kernel
         ops.linear_fwd(px, pw, t=t, u=u)                                # expand_xt_kernel + gemm_xt_kernel
         ops.linear_fwd(px, pw, t=t, u=u, tiled=False, split_k=False)    # gemm_nvfp4_large_kernel (expansion inside the K loop)
         _, t_ = ops.lowrank_project(x, v, s)                            # lowrank_nt_kernel<2, -1>: x V^T and (x V^T) * s
@@ -119,6 +127,8 @@ def decode(reps: int = 5):
         a = ops.quantize(torch.randn(64, k, generator=g).bfloat16().cuda())
         members = [(ops.quantize((torch.randn(n, k, generator=g) * 0.02).bfloat16().cuda()), torch.randn(64, 64, generator=g).bfloat16().cuda(),
                     torch.randn(n, 64, generator=g).bfloat16().cuda(), None) for n in ns]
+        for m in members:
+            m[0].persistent = True                                      # cached weights: streamed from the decode layout
         groups.append((a, members))
     for _ in range(reps):
         y.copy_(x)                                                      # calibration: 64 MiB read, 64 MiB written

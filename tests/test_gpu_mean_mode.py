@@ -413,6 +413,14 @@ def test_rmsnorm_with_column_mean(rows, cols):
     assert float((me.cpu().double() - want).abs().max()) <= 1e-6 * float(want.abs().max() + 1)
     again = ops.rmsnorm_colmean(x.cuda(), gamma.cuda(), 1e-6, torch.float32)[1]
     assert torch.equal(again, me)                                  # fixed summation order: the same bits call after call
+    # the same tensor OBJECTS with new contents (a serving loop's buffers): every call reads them afresh
+    buf, gd = x.cuda(), gamma.cuda()
+    first = ops.rmsnorm_colmean(buf, gd, 1e-6, torch.float32)
+    buf.mul_(-0.5)
+    buf[:, 0] += 3.0
+    second = ops.rmsnorm_colmean(buf, gd, 1e-6, torch.float32)
+    assert second[0].data_ptr() != first[0].data_ptr() and not torch.equal(second[1], first[1])
+    assert torch.equal(second[0], ops.rmsnorm_quantize(buf, gd, 1e-6, 0)[0])
     # centred quantizer on the kernel's own outputs, against the oracle formula
     p = ops.quantize(normed, 0, center=me)
     codes, scales, unit, _ = O.nvfp4_pack(normed.cpu().float() - me.cpu())
