@@ -49,6 +49,23 @@ int metis_nvfp4_quant_row(const void* x, int64_t rows, int64_t cols, int64_t ld,
                     workspace_bytes, (hipStream_t)stream);
 }
 
+int metis_nvfp4_quant_row_decode(const void* x, int64_t rows, int64_t cols, int mode, void* codes, void* scales, float* unit,
+                                 void* decode, void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (!decode) return METIS_E_ARG;
+    return quantize(x, rows, cols, cols, mode, false, false, nullptr, 0, 0, codes, scales, unit, workspace, workspace_bytes,
+                    (hipStream_t)stream, nullptr, false, 0, decode);
+}
+
+int metis_rmsnorm_nvfp4_quant_decode(const void* x, const void* gamma, float eps, int64_t rows, int64_t cols, int mode, void* normed,
+                                     void* codes, void* scales, float* unit, void* decode, void* workspace, size_t workspace_bytes,
+                                     void* stream)
+{
+    if (!decode) return METIS_E_ARG;
+    return rmsnorm_quantize(x, gamma, eps, rows, cols, mode, normed, codes, scales, unit, workspace, workspace_bytes,
+                            (hipStream_t)stream, false, decode);
+}
+
 size_t metis_linear_member_size(void) { return sizeof(metis_linear_member); }
 
 size_t metis_nvfp4_decode_weight_bytes(int64_t N, int64_t K) { return decode_weight_bytes(N, K); }

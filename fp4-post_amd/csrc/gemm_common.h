@@ -81,7 +81,6 @@ __device__ __forceinline__ void load_run_strided(RunRegs<C>& r, const uint8_t* c
 // (256 elements of K) one block of kDecodeBlock bytes: four KiB of codes -- piece j of lane l = (h << 5 | row) at
 // j * 1024 + l * 16 holds the row's code bytes [it * 128 + h * 64 + 16 j, + 16) -- then 512 bytes of scale bytes, lane l
 // at 4096 + l * 8 holding the row's bytes [it * 16 + h * 8, + 8).  Rows past N are zero.  0.5625 B per element, as packed.
-constexpr int kDecodeBlock = 4096 + 512;
 
 // MFMA operand m (8 elements) of a run
 template <int C>
@@ -134,6 +133,7 @@ struct SkinnyGroup {
     SkinnyMember m[kMaxGroupMembers];
     int count, nsplit;
     const float* center;         // mean mode: binary32 [K], see skinny_tile
+    int a_decode;                // the activation comes in the decode layout too (a_codes points at it, a_scales unused)
 };
 
 constexpr int L_BM = 256, L_BN = 256, L_STRIDE = BK + LDS_PAD;   // large-tile kernels: 256 x 256 per workgroup

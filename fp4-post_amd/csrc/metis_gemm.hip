@@ -590,7 +590,8 @@ static int launch_large(const void* a_codes, const void* a_scales, const float* 
 // products therefore stay apart from the residual sums: they pass through the reduction buffer a second time (K slice 0
 // leaves them as one more partial in slot nsplit when K is split).
 //
-// ADENSE: the activation arrives as ready 16-bit MFMA operands (skinny_operand_kernel: one 16-byte piece per lane and
+// ADENSE = 2: the packed activation comes in the decode layout, like a cached weight.
+// ADENSE = 1: the activation arrives as ready 16-bit MFMA operands (skinny_operand_kernel: one 16-byte piece per lane and
 // MFMA, a coalesced KiB per load instruction) instead of packed codes that every workgroup would expand again: the
 // vector unit is left with the weight operand alone.  a_codes then points at that buffer and a_scales is unused.
 template <int TM, int C, int WAVES, int OUT_F32, int CEN = 0, int PB16 = 0, int ADENSE = 0>
@@ -616,14 +617,24 @@ __device__ __forceinline__ void skinny_tile(
         bs = tile0 + 4096 + lane * 8;
         w_step = kDecodeBlock; w_piece = 1024; ws_step = kDecodeBlock;
     }
-    static_assert(ADENSE == 0 || (C == 4 && CEN == 0), "ready operands come in the wide-run layout");
+    static_assert(ADENSE != 1 || CEN == 0, "ready operands carry no centre");
+    static_assert(ADENSE == 0 || C == 4, "ready operands and the decode layout come in the wide-run layout");
     const uint8_t *ac[TM], *as[TM];
     const uint4* ap[TM];
+    // the activation likewise: row-major packed (64 lanes read 64 different lines per load instruction), or its decode
+    // layout (one KiB of consecutive bytes per load instruction; rows past M are zero there)
+    constexpr bool a_dec = ADENSE == 2;
+    constexpr int a_step = a_dec ? kDecodeBlock : 32 * C, a_piece = a_dec ? 1024 : 16, as_step = a_dec ? kDecodeBlock : 4 * C;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const int mrow = min(m0 + i * 32 + (lane & 31), M - 1);
         ac[i] = a_codes + (int64_t)mrow * kbytes + hi * 16 * C;
         as[i] = a_scales + (int64_t)mrow * kblocks + hi * 2 * C;
+        if constexpr (a_dec) {
+            const uint8_t* tile0 = a_codes + (int64_t)(m0 / 32 + i) * (K / 256) * kDecodeBlock;
+            ac[i] = tile0 + lane * 16;
+            as[i] = tile0 + 4096 + lane * 8;
+        }
         // operand (row tile, iteration, m): 64 lanes x 16 bytes
         ap[i] = reinterpret_cast<const uint4*>(a_codes) + (int64_t)(m0 / 32 + i) * (K / (64 * C)) * (4 * C * 64) + lane;
     }
@@ -667,7 +678,7 @@ __device__ __forceinline__ void skinny_tile(
     for (int it = s0 + wave * iters / WAVES; it < it1; ++it) {
         RunRegs<C> rw;
         load_run_strided<C>(rw, bc + (int64_t)it * w_step, w_piece, bs + (int64_t)it * ws_step);
-        if constexpr (ADENSE != 0) {
+        if constexpr (ADENSE == 1) {
             // a ring of AHEAD operand pieces per row tile keeps the L2 round trips ahead of the MFMAs
             constexpr int AHEAD = 4;
             uint4 fa[AHEAD][TM];
@@ -700,7 +711,7 @@ __device__ __forceinline__ void skinny_tile(
         }
         RunRegs<C> ra[TM];
 #pragma unroll
-        for (int i = 0; i < TM; ++i) load_run<C>(ra[i], ac[i] + (int64_t)it * 32 * C, as[i] + it * 4 * C);
+        for (int i = 0; i < TM; ++i) load_run_strided<C>(ra[i], ac[i] + (int64_t)it * a_step, a_piece, as[i] + (int64_t)it * as_step);
 #pragma unroll
         for (int m = 0; m < 4 * C; ++m) {
             if constexpr (PB16 != 0) {
@@ -1108,6 +1119,20 @@ static int launch_skinny_grouped(const void* a_codes, const void* a_scales, cons
         }
     }
     if (adense) return METIS_E_ARG;
+    if constexpr (C == 4) {
+        if (grp.a_decode) {                                    // the packed activation in the decode layout: exact, centred or bf16 evaluation
+#define METIS_SKA(O, CE, P) hipLaunchKernelGGL((gemm_nvfp4_skinny_grouped_kernel<TM, C, WAVES, O, CE, P, 2>), grid, block, 0, st, \
+                                               (const uint8_t*)a_codes, (const uint8_t*)a_scales, a_unit, (int)M, (int)K, grp)
+            const bool f32 = out_dtype == METIS_DTYPE_F32;
+            if (pb16) { if (grp.center) return METIS_E_ARG; if (f32) METIS_SKA(1, 0, 1); else METIS_SKA(0, 0, 1); }
+            else if (grp.center) { if (f32) METIS_SKA(1, 1, 0); else METIS_SKA(0, 1, 0); }
+            else { if (f32) METIS_SKA(1, 0, 0); else METIS_SKA(0, 0, 0); }
+#undef METIS_SKA
+            if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
+            return split ? launch_skinny_reduce(grp, M, out_dtype, st, pb16) : METIS_OK;
+        }
+    }
+    if (grp.a_decode) return METIS_E_ARG;
     if (pb16) {                                                // the reference's all-bf16 evaluation
         if (grp.center) return METIS_E_ARG;
         if (out_dtype == METIS_DTYPE_F32)
@@ -1218,7 +1243,10 @@ int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a
     if ((uintptr_t)center % 16) return METIS_E_ARG;
     if ((pb16 || a_dense) && center) return METIS_E_ARG;
     if (a_dense && (K % 256 || !a_unit)) return METIS_E_ARG;
-    if (a_dense) a_scales = a_codes;                          // unused by the kernel: the checks below see an aligned pointer
+    // no scale-byte pointer: a_codes is the packed activation in the decode layout (decode_weight applied to it)
+    const bool a_decode = !a_dense && a_codes && !a_scales;
+    if (a_decode && (K % 256 || M >= 256)) return METIS_E_ARG;
+    if (a_dense || a_decode) a_scales = a_codes;              // unused by the kernel: the checks below see an aligned pointer
     bool skinny = M > 0 && M < 256 && K % 64 == 0 && count <= kMaxGroupMembers && !measure_env("METIS_GEMM_SMALL") &&
                   a_codes && a_scales && a_unit && !((uintptr_t)a_codes % 16) && !((uintptr_t)a_scales % 2) && K <= INT32_MAX &&
                   (out_dtype == METIS_DTYPE_BF16 || out_dtype == METIS_DTYPE_F32);
@@ -1237,7 +1265,7 @@ int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a
     if (!skinny || tiles > INT32_MAX) {
         for (int i = 0; i < count; ++i)
             if (!members[i].b_codes || !members[i].b_scales) return METIS_E_ARG;   // only the decode-sized kernel reads the decode layout
-        if (center || pb16 || a_dense) return METIS_E_ARG;     // the centre, the bf16 evaluation and ready operands are only taken by the single-launch path
+        if (center || pb16 || a_dense || a_decode) return METIS_E_ARG;     // the centre, the bf16 evaluation, ready operands and the decode layout are only taken by the single-launch path
         for (int i = 0; i < count; ++i) {
             const GemmMember& g = members[i];
             if (g.ldt != 0 && g.ldt != g.r) return METIS_E_ARG;   // a strided t is only taken by the single-launch path
@@ -1256,7 +1284,7 @@ int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a
             tm = ftm; c = fc; waves = fw; nsplit = fs;
         }
     }
-    if (a_dense && c != 4) return METIS_E_ARG;                 // weight scale bytes must be 8-byte aligned for wide runs
+    if ((a_dense || a_decode) && c != 4) return METIS_E_ARG;   // weight scale bytes must be 8-byte aligned for wide runs
     const size_t slots = (size_t)nsplit + (pb16 ? 1 : 0);      // bf16 arithmetic: one more for the low-rank term
     if (nsplit > 1 && (((uintptr_t)workspace % 16) || workspace_bytes < slots * (size_t)M * (size_t)ntot * sizeof(float)))
         return METIS_E_WORKSPACE;
@@ -1265,6 +1293,7 @@ int gemm_nvfp4_grouped(const void* a_codes, const void* a_scales, const float* a
     grp.count = count;
     grp.nsplit = nsplit;
     grp.center = center;
+    grp.a_decode = a_decode ? 1 : 0;
     int end = 0;
     float* part = (float*)workspace;
     for (int i = 0; i < count; ++i) {

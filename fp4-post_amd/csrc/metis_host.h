@@ -51,13 +51,19 @@ static inline int measure_int(const char*, int dflt) { return dflt; }
 #endif
 
 // phase 2 of the quantizer (tensor unit + E4M3 bytes from parked block maxima); nvfp4_quant.hip
+// bytes of one block of the decode layout (32 rows x 256 elements of K: four KiB of codes, 512 scale bytes), see gemm_common.h
+constexpr int kDecodeBlock = 4096 + 512;
+// phase 2 of a quantizer call on a decode-sized tensor (rows < 256, cols % 256 == 0, bf16 block maxima parked): scale bytes
+// and unit as launch_scales writes them, and the packed tensor in the decode layout; nvfp4_quant.hip
+int launch_scales_decode(int mode, const Workspace& ws, uint32_t ngroups, const void* codes, void* scales, float* unit, int64_t rows,
+                         int64_t cols, void* decode, hipStream_t st);
 int launch_scales(int mode, const Workspace& ws, uint32_t ngroups, void* scales, float* unit, uint32_t nblocks,
                   hipStream_t st, const void* amax2 = nullptr, void* scales2 = nullptr, float* unit2 = nullptr);
 
 int quantize(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, bool sr, bool col, const void* noise,
              uint64_t seed, uint64_t offset, void* codes, void* scales, float* unit, void* workspace,
              size_t workspace_bytes, hipStream_t st, const void* center = nullptr, bool resident = false,
-             uint32_t spin_limit = 0);
+             uint32_t spin_limit = 0, void* decode = nullptr);
 // both packings (blocks along rows, blocks down columns) of one tensor with stochastic rounding in one pass; nvfp4_quant.hip
 int quantize_both_sr(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, uint64_t seed, uint64_t offset_row,
                      uint64_t offset_col, void* codes_row, void* scales_row, float* unit_row, void* codes_col, void* scales_col,
@@ -87,7 +93,7 @@ int rquant_values(const void* xq, void* s, int64_t rows, int64_t cols, int mode,
                   hipStream_t st);
 int rmsnorm_quantize(const void* x, const void* gamma, float eps, int64_t rows, int64_t cols, int mode, void* normed,
                      void* codes, void* scales, float* unit, void* workspace, size_t workspace_bytes, hipStream_t st,
-                     bool deferred = false);
+                     bool deferred = false, void* decode = nullptr);
 // RMSNorm that also leaves the column mean of its output (mean mode); rmsnorm_quant.hip
 size_t rmsnorm_colmean_workspace_bytes(int64_t rows, int64_t cols);
 int rmsnorm_colmean(const void* x, const void* gamma, float eps, int64_t rows, int64_t cols, void* normed, void* mean, int mean_bf16,

@@ -460,6 +460,54 @@ __global__ __launch_bounds__(256) void quant_scales_kernel(const uint16_t* __res
     }
 }
 
+// Phase 2 for a decode-sized activation (fewer than 256 rows, cols % 256 == 0): unit and scale bytes as above, and the
+// packed tensor once more in the decode layout that the decode-sized GEMM streams as whole lines (gemm_common.h): block
+// (tile of 32 rows, step of 256 elements) = four KiB of codes, piece j of lane l = (h << 5 | row) at j * 1024 + l * 16,
+// then 512 scale bytes, lane l at 4096 + l * 8.  One workgroup per block at a time: thread (j, l) moves a piece, and the
+// threads with j == 0 form the eight scale bytes of their lane.  Rows past the tensor are zero.
+template <int MODE>
+__global__ __launch_bounds__(256) void quant_scales_decode_kernel(const uint16_t* __restrict__ ws_amax, const uint32_t* __restrict__ ws_gmax,
+                                                                  uint32_t ngroups, const uint8_t* __restrict__ codes,
+                                                                  uint8_t* __restrict__ scales, float* __restrict__ unit_out,
+                                                                  uint8_t* __restrict__ decode, int rows, int cols, int blocks)
+{
+    __shared__ float smax[4];
+    float m = 0.0f;
+    for (uint32_t g = threadIdx.x; g < ngroups; g += 256u) m = fmaxf(m, __uint_as_float(ws_gmax[g]));
+    m = wave_max(m);
+    if ((threadIdx.x & 63) == 0) smax[threadIdx.x >> 6] = m;
+    __syncthreads();
+    const float unit = tensor_unit_of<MODE>(fmaxf(fmaxf(smax[0], smax[1]), fmaxf(smax[2], smax[3])));
+    if (blockIdx.x == 0 && threadIdx.x == 0) *unit_out = unit;
+    const int iters = cols / 256, l = threadIdx.x & 63, j = threadIdx.x >> 6, h = l >> 5;
+    for (int b = blockIdx.x; b < blocks; b += gridDim.x) {
+        const int tile = b / iters, it = b - tile * iters;
+        const int row = tile * 32 + (l & 31);
+        uint8_t* dst = decode + (int64_t)b * kDecodeBlock;
+        uint4 v = make_uint4(0u, 0u, 0u, 0u);
+        if (row < rows) v = *reinterpret_cast<const uint4*>(codes + (int64_t)row * (cols / 2) + it * 128 + h * 64 + 16 * j);
+        *reinterpret_cast<uint4*>(dst + j * 1024 + l * 16) = v;
+        if (j == 0) {
+            uint2 o = make_uint2(0u, 0u);
+            if (row < rows) {
+                const int64_t kb = (int64_t)row * (cols / kBlock) + it * 16 + h * 8;
+                const uint4 a = *reinterpret_cast<const uint4*>(ws_amax + kb);
+                uint32_t by[8];
+                const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    by[2 * q] = scale_byte_of<MODE>(w[q] & 0xffffu, unit);
+                    by[2 * q + 1] = scale_byte_of<MODE>(w[q] >> 16, unit);
+                }
+                o.x = by[0] | (by[1] << 8) | (by[2] << 16) | (by[3] << 24);
+                o.y = by[4] | (by[5] << 8) | (by[6] << 16) | (by[7] << 24);
+                *reinterpret_cast<uint2*>(scales + kb) = o;
+            }
+            *reinterpret_cast<uint2*>(dst + 4096 + l * 8) = o;
+        }
+    }
+}
+
 // Phase 2 for parked binary32 maxima (binary32 input): IEEE divisions, four blocks per thread.
 __global__ __launch_bounds__(256) void quant_scales_f32_kernel(const float* __restrict__ ws_amax,
                                                                const uint32_t* __restrict__ ws_gmax, uint32_t ngroups,
@@ -824,6 +872,23 @@ static int grid_for(uint32_t work_items, int per_cu = 8)           // 8 workgrou
     return g < 1 ? 1 : (int)g;
 }
 
+int launch_scales_decode(int mode, const Workspace& ws, uint32_t ngroups, const void* codes, void* scales, float* unit, int64_t rows,
+                         int64_t cols, void* decode, hipStream_t st)
+{
+    if (rows <= 0 || rows >= 256 || cols <= 0 || cols % 256 || (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16)) return METIS_E_ARG;
+    if (!decode || ((uintptr_t)decode % 16) || ((uintptr_t)scales % 8) || ((uintptr_t)codes % 16)) return METIS_E_ARG;
+    const int blocks = (int)(((rows + 31) / 32) * (cols / 256));
+    const int cap = device_cus() * 8;
+    const dim3 grid((unsigned)(blocks < cap ? blocks : cap));
+    if (mode == 0)
+        hipLaunchKernelGGL((quant_scales_decode_kernel<0>), grid, dim3(256), 0, st, ws.amax, ws.gmax, ngroups, (const uint8_t*)codes,
+                           (uint8_t*)scales, unit, (uint8_t*)decode, (int)rows, (int)cols, blocks);
+    else
+        hipLaunchKernelGGL((quant_scales_decode_kernel<1>), grid, dim3(256), 0, st, ws.amax, ws.gmax, ngroups, (const uint8_t*)codes,
+                           (uint8_t*)scales, unit, (uint8_t*)decode, (int)rows, (int)cols, blocks);
+    return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
+}
+
 int launch_scales(int mode, const Workspace& ws, uint32_t ngroups, void* scales, float* unit, uint32_t nblocks,
                   hipStream_t st, const void* amax2, void* scales2, float* unit2)
 {
@@ -899,7 +964,7 @@ static void launch_contig(const void* x, void* codes, const Workspace& ws, uint3
 template <int MODE, bool SR, bool COL, bool WIDE = false, bool HAD = false>
 static int launch_quant(const void* x, int64_t rows, int64_t cols, int64_t ld, const void* noise, uint64_t seed,
                         uint64_t offset, void* codes, void* scales, float* unit, const Workspace& ws, hipStream_t st,
-                        int in_f32 = 0, const void* center = nullptr, uint32_t sign_mask = 0)
+                        int in_f32 = 0, const void* center = nullptr, uint32_t sign_mask = 0, void* decode = nullptr)
 {
     static_assert(!HAD || !COL, "the rotation runs along the last dimension, as the row blocks do");
     const uint32_t nblocks = (uint32_t)(rows * cols / kBlock);
@@ -925,9 +990,11 @@ static int launch_quant(const void* x, int64_t rows, int64_t cols, int64_t ld, c
             if (!center && ld == cols) {
                 const int gc = grid_for(nblocks, measure_int("METIS_Q_WGPC", kContigPerCu));
                 launch_contig<MODE>(x, codes, ws, nblocks, 0u, gc, st);
+                if (decode) return launch_scales_decode(MODE, ws, (uint32_t)gc, codes, scales, unit, rows, cols, decode, st);
                 return launch_scales(MODE, ws, (uint32_t)gc, scales, unit, nblocks, st);
             }
         }
+        if (decode) return METIS_E_ARG;                         // only contiguous bf16 rows, round to nearest, come with the decode layout
         const int g1 = grid_for(nblocks);
         hipLaunchKernelGGL((quant_codes_kernel<MODE, SR, WIDE, HAD>), dim3(g1), dim3(256), 0, st, x, (uint32_t)rows,
                            (uint32_t)cols, ld, noise, seed, offset, (uint2*)codes, (void*)ws.amax, ws.gmax, nblocks, in_f32, center,
@@ -938,7 +1005,7 @@ static int launch_quant(const void* x, int64_t rows, int64_t cols, int64_t ld, c
 
 int quantize(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, bool sr, bool col, const void* noise,
              uint64_t seed, uint64_t offset, void* codes, void* scales, float* unit, void* workspace,
-             size_t workspace_bytes, hipStream_t st, const void* center, bool resident, uint32_t spin_limit)
+             size_t workspace_bytes, hipStream_t st, const void* center, bool resident, uint32_t spin_limit, void* decode)
 {
     if (rows < 0 || cols < 0 || ld < cols) return METIS_E_ARG;
     if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16 && mode != METIS_MODE_P32_F32) return METIS_E_ARG;
@@ -955,14 +1022,15 @@ int quantize(const void* x, int64_t rows, int64_t cols, int64_t ld, int mode, bo
     Workspace ws;
     int rc = carve_workspace(workspace, workspace_bytes, rows, cols, &ws);
     if (rc != METIS_OK) return rc;
-    if (resident && !sr && !col && !wide && !center && ld == cols) {   // opt-in single-launch path; falls through when it does not fit
+    if (decode && (sr || col || wide || center || ld != cols || rows >= 256 || cols % 256)) return METIS_E_ARG;
+    if (resident && !decode && !sr && !col && !wide && !center && ld == cols) {   // opt-in single-launch path; falls through when it does not fit
         const uint32_t nblocks = (uint32_t)(rows * cols / kBlock);
         if (spin_limit == 0) spin_limit = kSpinLimit;
         rc = mode == 0 ? launch_fused<0>(x, codes, scales, unit, ws, nblocks, st, spin_limit)
                        : launch_fused<1>(x, codes, scales, unit, ws, nblocks, st, spin_limit);
         if (rc != 1) return rc;
     }
-#define METIS_Q(M, S, C) return launch_quant<M, S, C>(x, rows, cols, ld, noise, seed, offset, codes, scales, unit, ws, st, 0, center)
+#define METIS_Q(M, S, C) return launch_quant<M, S, C>(x, rows, cols, ld, noise, seed, offset, codes, scales, unit, ws, st, 0, center, 0u, decode)
 #define METIS_QF(S, C) return launch_quant<0, S, C, true>(x, rows, cols, ld, noise, seed, offset, codes, scales, unit, ws, st, f32in, center)
     if (wide) {
         if (!sr) { if (!col) METIS_QF(false, false); else METIS_QF(false, true); }

@@ -407,8 +407,10 @@ int rmsnorm_colmean(const void* x, const void* gamma, float eps, int64_t rows, i
 // deferred: stop after the main kernel; `workspace` is then the caller-owned parked data of the deferred form
 // (nvfp4_quant.hip) and scales / unit are not written.
 int rmsnorm_quantize(const void* x, const void* gamma, float eps, int64_t rows, int64_t cols, int mode, void* normed,
-                     void* codes, void* scales, float* unit, void* workspace, size_t workspace_bytes, hipStream_t st, bool deferred)
+                     void* codes, void* scales, float* unit, void* workspace, size_t workspace_bytes, hipStream_t st, bool deferred,
+                     void* decode)
 {
+    if (decode && (deferred || rows >= 256 || cols % 256)) return METIS_E_ARG;
     if (rows < 0 || cols < 0) return METIS_E_ARG;
     if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) return METIS_E_ARG;
     if (cols % kBlock) return METIS_E_SHAPE;
@@ -440,6 +442,7 @@ int rmsnorm_quantize(const void* x, const void* gamma, float eps, int64_t rows, 
 #undef METIS_RW
         if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
         if (deferred) return METIS_OK;
+        if (decode) return launch_scales_decode(mode, ws, (uint32_t)g, codes, scales, unit, rows, cols, decode, st);
         return launch_scales(mode, ws, (uint32_t)g, scales, unit, (uint32_t)(rows * cols / kBlock), st);
     }
     int64_t g = rows;
@@ -459,6 +462,7 @@ int rmsnorm_quantize(const void* x, const void* gamma, float eps, int64_t rows, 
 #undef METIS_R
     if (hipGetLastError() != hipSuccess) return METIS_E_LAUNCH;
     if (deferred) return METIS_OK;
+    if (decode) return launch_scales_decode(mode, ws, (uint32_t)g, codes, scales, unit, rows, cols, decode, st);
     return launch_scales(mode, ws, (uint32_t)g, scales, unit, (uint32_t)(rows * cols / kBlock), st);
 }
 

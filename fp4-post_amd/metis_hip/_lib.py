@@ -71,6 +71,8 @@ SIGNATURES = {
     "metis_linear_dgrad": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i32, _vp]),
     "metis_linear_wgrad": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i32, _vp]),
     "metis_nvfp4_quant_centered": (_i32, [_vp, _i64, _i64, _i64, _i32, _vp, _i32, _i32, _vp, _u64, _u64, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "metis_nvfp4_quant_row_decode": (_i32, [_vp, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "metis_rmsnorm_nvfp4_quant_decode": (_i32, [_vp, _vp, _f32, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "metis_nvfp4_quant_lowrank_residual": (_i32, [_vp, _i32, _vp, _vp, _i64, _i64, _i32, _i32, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "metis_nvfp4_matvec_affine": (_i32, [_vp, _vp, _vp, _i64, _i64, _vp, _f32, _vp, _f32, _vp, _vp]),
     "metis_rank_one_operands": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp]),

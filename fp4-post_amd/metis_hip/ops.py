@@ -22,6 +22,9 @@ _workspaces: dict = {}
 # weight on every call instead of once.  Same bits either way.
 decode_layout_weights = True
 tiled_weight_copies = True
+# Decode-sized activations (fewer than 256 rows, a multiple of 256 columns) leave the round-to-nearest quantizers in the
+# decode layout as well: written by the quantizer's second launch, read by the decode-sized GEMM as whole lines.
+decode_layout_activations = True
 
 
 @dataclass
@@ -257,6 +260,13 @@ def quantize(x: torch.Tensor, mode: int = MODE_P32, *, col: bool = False, sr: bo
     elif resident and not col and kmode in (MODE_P32, MODE_PB16) and x2.stride(0) == cols:
         rc = L.metis_nvfp4_quant_row_resident(x2.data_ptr(), rows, cols, kmode, codes.data_ptr(), scales.data_ptr(),
                                               unit.data_ptr(), ws.data_ptr(), ws.numel(), int(spin_limit), _stream())
+    elif (decode_layout_activations and not col and kmode in (MODE_P32, MODE_PB16) and 0 < rows < 256 and cols % 256 == 0
+          and x2.stride(0) == cols):
+        dec = torch.empty(L.metis_nvfp4_decode_weight_bytes(rows, cols), dtype=torch.uint8, device=dev)
+        rc = L.metis_nvfp4_quant_row_decode(x2.data_ptr(), rows, cols, kmode, codes.data_ptr(), scales.data_ptr(), unit.data_ptr(),
+                                            dec.data_ptr(), ws.data_ptr(), ws.numel(), _stream())
+        check(rc, "metis_nvfp4_quant_row_decode", x.shape)
+        return PackedNVFP4(codes, scales, unit, prow, pcol, mode, decode_layout=dec)
     else:
         fn = L.metis_nvfp4_quant_col if col else L.metis_nvfp4_quant_row
         rc = fn(x2.data_ptr(), rows, cols, x2.stride(0), kmode, codes.data_ptr(), scales.data_ptr(),
@@ -749,13 +759,22 @@ def rmsnorm_quantize(x: torch.Tensor, gamma: torch.Tensor, eps: float, mode: int
         return normed, PackedNVFP4(codes, None, unit, rows, cols, mode, deferred=parked)
     scales = torch.empty(rows, cols // BLOCK, dtype=torch.uint8, device=dev)
     ws = _workspace(rows, cols, dev)
-    rc = load().metis_rmsnorm_nvfp4_quant(x2.data_ptr(), g.data_ptr(), float(eps), rows, cols, mode,
-                                          None if normed is None else normed.data_ptr(), codes.data_ptr(),
-                                          scales.data_ptr(), unit.data_ptr(), ws.data_ptr(), ws.numel(), _stream())
+    dec = None
+    if decode_layout_activations and 0 < rows < 256 and cols % 256 == 0:
+        L = load()
+        dec = torch.empty(L.metis_nvfp4_decode_weight_bytes(rows, cols), dtype=torch.uint8, device=dev)
+        rc = L.metis_rmsnorm_nvfp4_quant_decode(x2.data_ptr(), g.data_ptr(), float(eps), rows, cols, mode,
+                                                None if normed is None else normed.data_ptr(), codes.data_ptr(),
+                                                scales.data_ptr(), unit.data_ptr(), dec.data_ptr(), ws.data_ptr(), ws.numel(),
+                                                _stream())
+    else:
+        rc = load().metis_rmsnorm_nvfp4_quant(x2.data_ptr(), g.data_ptr(), float(eps), rows, cols, mode,
+                                              None if normed is None else normed.data_ptr(), codes.data_ptr(),
+                                              scales.data_ptr(), unit.data_ptr(), ws.data_ptr(), ws.numel(), _stream())
     check(rc, "metis_rmsnorm_nvfp4_quant", x.shape)
     if normed is not None:
         normed = normed.reshape(x.shape)
-    return normed, PackedNVFP4(codes, scales, unit, rows, cols, mode)
+    return normed, PackedNVFP4(codes, scales, unit, rows, cols, mode, decode_layout=dec)
 
 
 def rmsnorm_colmean(x: torch.Tensor, gamma: torch.Tensor, eps: float, mean_dtype: torch.dtype = torch.float32,
@@ -1104,6 +1123,9 @@ def _linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.
             M, K, ctypes.cast(arr, ctypes.c_void_p), len(members), 0))
     ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
     dt = DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16
+    # the activation's decode layout (written by its quantizer) in place of the row-major packing: wide runs only
+    a_dec = a.decode_layout if (takes and K % 256 == 0 and all(m[0].scales.data_ptr() % 8 == 0 for m in members)) else None
+    a_codes, a_scales = (a_dec.data_ptr(), None) if a_dec is not None else (a.codes.data_ptr(), a.scales.data_ptr())
     if operand:
         aop = decode_operand(a, MODE_PB16, center)
         rc = L.metis_linear_fwd_grouped_operand(aop.data_ptr(), a.unit.data_ptr(), M, K, ap, len(members), dt, MODE_PB16,
@@ -1116,7 +1138,7 @@ def _linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.
             raise ValueError(f"center must have {K} values, got {center.numel()}")
         aligned = center.data_ptr() % 16 == 0 and all(m[0].scales.data_ptr() % 8 == 0 for m in members) and a.scales.data_ptr() % 8 == 0
         if aligned and centre_ok:
-            rc = L.metis_linear_fwd_grouped_centered(a.codes.data_ptr(), a.scales.data_ptr(), a.unit.data_ptr(), M, K, ap,
+            rc = L.metis_linear_fwd_grouped_centered(a_codes, a_scales, a.unit.data_ptr(), M, K, ap,
                                                      len(members), dt, center.data_ptr(),
                                                      None if ws is None else ws.data_ptr(), need, _stream())
             check(rc, "metis_linear_fwd_grouped_centered", (M, K, [m[0].rows for m in members]))
@@ -1128,7 +1150,7 @@ def _linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.
             shifted.append((b, t, u, w_mean if bias is None else w_mean + bias.float()))
         return _linear_fwd_grouped(a, shifted, out_dtype)
     fn = L.metis_linear_fwd_grouped_bf16 if rounded else L.metis_linear_fwd_grouped
-    rc = fn(a.codes.data_ptr(), a.scales.data_ptr(), a.unit.data_ptr(), M, K, ap, len(members),
+    rc = fn(a_codes, a_scales, a.unit.data_ptr(), M, K, ap, len(members),
             dt, None if ws is None else ws.data_ptr(), need, _stream())
     check(rc, "metis_linear_fwd_grouped_bf16" if rounded else "metis_linear_fwd_grouped", (M, K, [m[0].rows for m in members]))
     return outs

@@ -594,6 +594,28 @@ size_t metis_linear_member_size(void);
  *   out   metis_nvfp4_decode_weight_bytes(N, K) bytes, 16-byte aligned */
 size_t metis_nvfp4_decode_weight_bytes(int64_t N, int64_t K);
 int metis_nvfp4_decode_weight(const void *codes, const void *scales, int64_t N, int64_t K, void *out, void *stream);
+
+/*
+ * Decode-sized activations in the decode layout as well.  Against a row-major packed activation, a load instruction of the
+ * decode-sized kernel touches 64 different lines (one per activation row), and every workgroup reads the whole
+ * activation: the layout above turns that into one KiB of consecutive bytes per instruction (66 instead of 73 us for the
+ * four calls of a Qwen2.5-7B layer at 64 tokens).  The quantizer writes it in its second launch, next to the ordinary
+ * scale bytes (no additional launch):
+ *   metis_nvfp4_quant_row_decode        metis_nvfp4_quant_row of a contiguous bf16 tensor with rows < 256 and
+ *                                       cols % 256 == 0 (mode METIS_MODE_P32 or METIS_MODE_PB16), and `decode`
+ *                                       (metis_nvfp4_decode_weight_bytes(rows, cols) bytes, 16-byte aligned)
+ *   metis_rmsnorm_nvfp4_quant_decode    metis_rmsnorm_nvfp4_quant likewise
+ * and metis_linear_fwd_grouped, metis_linear_fwd_grouped_bf16 and metis_linear_fwd_grouped_centered take it in place of
+ * the packed activation: pass the buffer as a_codes and NULL as a_scales (M < 256, K % 256 == 0, weight scale bytes
+ * 8-byte aligned; METIS_E_ARG otherwise).  Same kernel, same order of operations: the same bits.
+ */
+int metis_nvfp4_quant_row_decode(const void *x, int64_t rows, int64_t cols, int mode, void *codes,
+                                 void *scales, float *unit, void *decode, void *workspace,
+                                 size_t workspace_bytes, void *stream);
+int metis_rmsnorm_nvfp4_quant_decode(const void *x, const void *gamma, float eps, int64_t rows,
+                                     int64_t cols, int mode, void *normed, void *codes, void *scales,
+                                     float *unit, void *decode, void *workspace,
+                                     size_t workspace_bytes, void *stream);
 int metis_linear_fwd_grouped(const void *a_codes, const void *a_scales, const float *a_unit, int64_t M,
                              int64_t K, const metis_linear_member *members, int count, int out_dtype,
                              void *workspace, size_t workspace_bytes, void *stream);

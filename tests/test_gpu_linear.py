@@ -444,6 +444,7 @@ def test_cached_weights_in_the_decode_layout_give_the_same_bits(M, K, Ns, r):
                 u = (torch.randn(N, r, generator=g) * 0.1).bfloat16().cuda()
             bias = (torch.randn(N, generator=g) * 0.1).bfloat16().cuda() if i % 2 == 0 else None
             pw, pc = ops.quantize(w, mode), ops.quantize(w, mode)
+            pw.decode_layout = pc.decode_layout = None          # (a tensor of fewer than 256 rows leaves the quantizer with one)
             pc.persistent = True
             plain.append((pw, t, u, bias))
             cached.append((pc, t, u, bias))
@@ -761,3 +762,48 @@ def test_memory_bound_deployments_can_drop_the_derived_weight_copies(monkeypatch
             outs[keep] = ys
         for a, b in zip(outs[True], outs[False]):
             assert torch.equal(a, b), mode
+
+
+@pytest.mark.parametrize("M,K,Ns,r", [(64, 3584, (3584, 512, 512), 64), (1, 1024, (256, 100), 0), (40, 3584, (18944,), 32),
+                                      (64, 18944, (3584,), 64), (200, 2048, (132, 64), 32), (17, 256, (4,), 0)])
+def test_decode_sized_activations_leave_the_quantizer_in_the_decode_layout(M, K, Ns, r, monkeypatch):
+    """The quantizer's second launch writes a decode-sized activation (fewer than 256 rows, K % 256 == 0) once more in
+    the layout the decode-sized kernel streams as whole lines, and the grouped GEMM reads that instead of the row-major
+    packing: the same kernel in the same order, so the same bits -- exact products, the reference's bf16 roundings, a
+    centre inside the launch, K in slices, ragged M and N -- and the same codes, scale bytes and unit as the plain
+    quantizer.  The fused RMSNorm -> NVFP4 call does the same."""
+    from metis_hip import ops
+    g = torch.Generator().manual_seed(M * 3 + K)
+    x = synthetic_activation(260 + M, M, K).cuda()
+    gamma = (1 + 0.1 * torch.randn(K, generator=g)).bfloat16().cuda()
+    centre = (torch.randn(K, generator=g) * 0.2).cuda()
+    for mode in (0, 1):
+        members = []
+        for i, N in enumerate(Ns):
+            pw = ops.quantize(_weights(261 + i, N, K).cuda(), mode)
+            pw.persistent = i % 2 == 0                          # with and without the weight's own decode layout
+            t = u = None
+            if r:
+                t = torch.randn(M, r, generator=g).bfloat16().cuda()
+                u = (torch.randn(N, r, generator=g) * 0.1).bfloat16().cuda()
+            members.append((pw, t, u, (torch.randn(N, generator=g) * 0.1).bfloat16().cuda() if i == 0 else None))
+        packs = {}
+        for on in (False, True):
+            monkeypatch.setattr(ops, "decode_layout_activations", on)
+            packs[on] = (ops.quantize(x, mode), ops.rmsnorm_quantize(x, gamma, 1e-6, mode) if K <= 16384 else None)   # the norm holds a row in registers
+        plain, dec = packs[False][0], packs[True][0]
+        assert plain.decode_layout is None and dec.decode_layout is not None
+        pairs = [(plain, dec)]
+        if K <= 16384:
+            (normed_plain, fused_plain), (normed_dec, fused_dec) = packs[False][1], packs[True][1]
+            assert torch.equal(normed_plain, normed_dec) and fused_plain.decode_layout is None
+            pairs.append((fused_plain, fused_dec))
+        for a, b in pairs:
+            assert torch.equal(a.codes, b.codes) and torch.equal(a.scales, b.scales) and torch.equal(a.unit, b.unit)
+            # the layout against its definition (the weight's re-tiling kernel applied to the packed activation)
+            assert torch.equal(b.decode_layout, ops.decode_weight(a, cache=False))
+        for kw in ({}, {"reference_rounding": True} if mode == 1 else {"center": centre}, {"split_k": False}):
+            want = ops.linear_fwd_grouped(plain, members, **kw)
+            got = ops.linear_fwd_grouped(dec, members, **kw)
+            for a, b in zip(got, want):
+                assert torch.equal(a, b), (mode, kw.keys())
