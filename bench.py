@@ -35,9 +35,9 @@ NORMQ_BYTES_PER_ELT = 4.5625   # + 2 B normed
 TRAFFIC_SOURCE = ("profiles/hbm_traffic_pmc.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE on profile_workload.py, "
                   "calibrated by a 64 MiB copy); a constant, not measured in this run")
 TRAFFIC_GEMM_C3 = 1666.5e6      # gemm_xt_kernel: 1431.6 MB fetched (tiled f16 operands re-read below L2) + 234.9 MB written
-TRAFFIC_QUANT_C1 = 94.8e6       # quant_codes_contig_kernel 88.4 MB + quant_scales_kernel 6.4 MB
-TRAFFIC_NORMQ_C2 = 323.8e6      # rmsnorm_quant_kernel 311.1 MB + quant_scales_kernel 12.7 MB
-TRAFFIC_DECODE_C5 = 160.8e6     # the five launches of the decode layer: 150.8 MB fetched + 10.0 MB written
+TRAFFIC_QUANT_C1 = 94.6e6       # quant_codes_contig_kernel 88.2 MB + quant_scales_kernel 6.4 MB
+TRAFFIC_NORMQ_C2 = 323.5e6      # rmsnorm_quant_rows_kernel 310.8 MB + quant_scales_kernel 12.7 MB
+TRAFFIC_DECODE_C5 = 160.8e6     # the five launches of the decode layer: 150.7 MB fetched + 10.0 MB written
 
 
 def cpu_model() -> str:
