@@ -86,6 +86,64 @@ __global__ __launch_bounds__(256) void quant_codes_contig_kernel(const uint4* __
     publish_group_max(gmax, ws_gmax, fill_to);
 }
 
+// The same loop with a centre subtracted first (mean mode, src/Metis/Metis/bitlinear.py:311-336: the tensor that is
+// quantized is x - me with the column mean me): contiguous bf16 rows of at most 4096 columns, the centre staged once per
+// workgroup in LDS (binary32 [cols] in binary32 arithmetic, bf16 values widened in bf16 arithmetic).  In binary32 arithmetic
+// the residuals are binary32 values that need not be bf16 values: the per-quotient encoder and binary32 block maxima, as
+// quant_codes_kernel<0, false, true>; in bf16 arithmetic the residual is rounded to bf16 and encoded as any bf16 block.
+// A block's column position advances by a fixed amount modulo the row length: no division in the loop.
+constexpr int kCentreMaxCols = 4096;
+template <int MODE>
+__global__ __launch_bounds__(256) void quant_codes_contig_centered_kernel(const uint4* __restrict__ x, const void* __restrict__ center,
+                                                                          uint2* __restrict__ codes, void* __restrict__ ws_amax_v,
+                                                                          uint32_t* __restrict__ ws_gmax, uint32_t nblocks,
+                                                                          uint32_t nbpr, uint32_t fill_to)
+{
+    __shared__ __align__(16) float cen[kCentreMaxCols];
+    for (uint32_t c = threadIdx.x; c < nbpr * kBlock; c += 256u)
+        cen[c] = MODE == 0 ? static_cast<const float*>(center)[c] : bf16_lo(static_cast<const uint16_t*>(center)[c]);
+    __syncthreads();
+    float gmax = 0.0f;
+    const uint32_t step = gridDim.x * 256u, step_mod = step % nbpr;
+    uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    uint32_t cb = i % nbpr;
+    uint4 c0 = make_uint4(0u, 0u, 0u, 0u), c1 = c0;
+    if (i < nblocks) { c0 = x[2 * (size_t)i]; c1 = x[2 * (size_t)i + 1]; }
+    while (i < nblocks) {
+        const uint4 a0 = c0, a1 = c1;
+        const uint32_t nxt = i + step;
+        if (nxt < nblocks) { c0 = x[2 * (size_t)nxt]; c1 = x[2 * (size_t)nxt + 1]; }
+        float v[kBlock];
+        unpack16(a0, a1, v);
+        const float4* cp = reinterpret_cast<const float4*>(cen + cb * kBlock);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const float4 f = cp[q];
+            if constexpr (MODE == 0) {
+                v[4 * q] -= f.x; v[4 * q + 1] -= f.y; v[4 * q + 2] -= f.z; v[4 * q + 3] -= f.w;
+            } else {
+                v[4 * q] = rb(v[4 * q] - f.x); v[4 * q + 1] = rb(v[4 * q + 1] - f.y);
+                v[4 * q + 2] = rb(v[4 * q + 2] - f.z); v[4 * q + 3] = rb(v[4 * q + 3] - f.w);
+            }
+        }
+        const float am = block_amax(v);
+        gmax = fmaxf(gmax, am);
+        uint2 cw;
+        if constexpr (MODE == 0) {
+            static_cast<float*>(ws_amax_v)[i] = am;
+            cw = encode_rne_wide(v, block_scalar_ieee(am));
+        } else {
+            static_cast<uint16_t*>(ws_amax_v)[i] = (uint16_t)(__float_as_uint(am) >> 16);
+            cw = encode_rne_pb16(v, block_scalar<1>(am));
+        }
+        __builtin_nontemporal_store((metis_u32x2_t){cw.x, cw.y}, reinterpret_cast<metis_u32x2_t*>(codes) + i);
+        i = nxt;
+        cb += step_mod;
+        cb = cb >= nbpr ? cb - nbpr : cb;
+    }
+    publish_group_max(gmax, ws_gmax, fill_to);
+}
+
 // HAD: every block is rotated first (NV recipe, hadamard16_forward): the rotated tensor is what gets quantized, as in
 // `_quantize_wgrad_operand` and `_get_quantized_weight` of src/Metis/Metis/bitlinear.py:395-405, 577-585.  In bf16
 // arithmetic the rotated values are rounded to bf16 (the reference's rotation returns the input dtype); in binary32
@@ -986,6 +1044,15 @@ static int launch_quant(const void* x, int64_t rows, int64_t cols, int64_t ld, c
                                (uint32_t)tiles, center);
         return launch_scales(WIDE ? METIS_MODE_P32_F32 : MODE, ws, (uint32_t)g, scales, unit, nblocks, st);
     } else {
+        if constexpr (!SR && !HAD && (WIDE ? MODE == 0 : MODE == 1)) {
+            if (center && !in_f32 && ld == cols && cols <= kCentreMaxCols) {   // mean mode on contiguous bf16 rows
+                if (decode) return METIS_E_ARG;
+                const int gc = grid_for(nblocks, kContigPerCu);
+                hipLaunchKernelGGL((quant_codes_contig_centered_kernel<MODE>), dim3(gc), dim3(256), 0, st, (const uint4*)x, center,
+                                   (uint2*)codes, (void*)ws.amax, ws.gmax, nblocks, (uint32_t)(cols / kBlock), 0u);
+                return launch_scales(WIDE ? METIS_MODE_P32_F32 : MODE, ws, (uint32_t)gc, scales, unit, nblocks, st);
+            }
+        }
         if constexpr (!SR && !WIDE && !HAD) {
             if (!center && ld == cols) {
                 const int gc = grid_for(nblocks, measure_int("METIS_Q_WGPC", kContigPerCu));
@@ -1181,7 +1248,10 @@ int quantize_row_deferred(const void* x, int64_t rows, int64_t cols, int mode, c
     if (const int rc = carve_deferred(deferred, bytes, rows, cols, &ws)) return rc;
     const uint32_t nblocks = (uint32_t)(rows * cols / kBlock);
     const int g1 = deferred_grid(nblocks, center ? 8 : measure_int("METIS_Q_WGPC", kContigPerCu));
-    if (center)
+    if (center && cols <= kCentreMaxCols)
+        hipLaunchKernelGGL((quant_codes_contig_centered_kernel<1>), dim3(g1), dim3(256), 0, st, (const uint4*)x, center, (uint2*)codes,
+                           (void*)ws.amax, ws.gmax, nblocks, (uint32_t)(cols / kBlock), kDeferredPartials);
+    else if (center)
         hipLaunchKernelGGL((quant_codes_kernel<1, false, false, false>), dim3(g1), dim3(256), 0, st, x, (uint32_t)rows, (uint32_t)cols,
                            cols, nullptr, (uint64_t)0, (uint64_t)0, (uint2*)codes, (void*)ws.amax, ws.gmax, nblocks, 0, center, 0u,
                            kDeferredPartials);
