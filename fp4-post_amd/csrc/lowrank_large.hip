@@ -48,7 +48,7 @@ template <int RT, int QMODE = -1, bool EW = false>  // R / 32 column tiles: 1, 2
 __global__ __launch_bounds__((QMODE >= 0 && EW) ? 512 : 256) void lowrank_nt_kernel(
     const uint16_t* __restrict__ x, int64_t ldx, const uint16_t* __restrict__ v, const uint16_t* __restrict__ s,
     uint16_t* __restrict__ xv, uint16_t* __restrict__ t, int M, int K, float* __restrict__ part, uint2* __restrict__ codes,
-    uint16_t* __restrict__ q_amax, uint32_t* __restrict__ q_gmax, uint32_t fill_to)
+    uint16_t* __restrict__ q_amax, uint32_t* __restrict__ q_gmax, uint32_t fill_to, int rotate)
 {
     constexpr int R = RT * 32;
     constexpr int TILE_BYTES = (32 + R) * NT_STRIDE * 2;        // one staged step: x rows, then v rows
@@ -63,6 +63,13 @@ __global__ __launch_bounds__((QMODE >= 0 && EW) ? 512 : 256) void lowrank_nt_ker
     const int per = (steps_all + (int)gridDim.y - 1) / (int)gridDim.y;
     const int first = (int)blockIdx.y * per, steps = max(0, min(steps_all, first + per) - first);
     __shared__ float smax[4];
+    // Every row tile starts at a different step of its K range and wraps around: at any moment the workgroups then read
+    // different column stripes of x instead of the same one.  With rows a multiple of 4 KiB long, 512-byte pieces at the
+    // same offset of every row fall on the same few memory channels (flushed caches, 8192 x 4096: 39 -> 31 us; 8192 x 14336:
+    // 146 -> 104 us; row lengths like 7168 or 17920 bytes are indifferent).  The binary32 sums of a tile are therefore added
+    // in an order that depends on the tile, the same for every call and for both forms of the kernel.
+    const int rot = (rotate && steps > 0) ? (int)((blockIdx.x * 5u) % (unsigned)steps) : 0;
+    auto kof = [&](int st) { int q = st + rot; if (q >= steps) q -= steps; return (first + q) * NT_STEP; };
     if constexpr (QMODE >= 0 && EW) {
         if (tid >= 256) {                                       // the encoding waves: same barriers as the others, nothing else shared
             const int et = tid - 256;
@@ -77,7 +84,7 @@ __global__ __launch_bounds__((QMODE >= 0 && EW) ? 512 : 256) void lowrank_nt_ker
                     b[i][1] = *reinterpret_cast<const uint4*>(tile + row * NT_STRIDE + blk * 16 + 8);
                 }
                 __syncthreads();                                // the tile may be overwritten: the blocks are in registers
-                const int k0 = (first + st) * NT_STEP;
+                const int k0 = kof(st);
 #pragma unroll
                 for (int i = 0; i < 2; ++i) {
                     const int id = i * 256 + et, row = id >> 4, k = k0 + (id & 15) * 16;
@@ -178,21 +185,21 @@ __global__ __launch_bounds__((QMODE >= 0 && EW) ? 512 : 256) void lowrank_nt_ker
         }
     };
     // two steps are in flight while a third is multiplied: the time of one step is then half the memory latency
-    if (steps > 0) fetch(rx[0], rv[0], first * NT_STEP);
-    if (steps > 1) fetch(rx[1], rv[1], (first + 1) * NT_STEP);
+    if (steps > 0) fetch(rx[0], rv[0], kof(0));
+    if (steps > 1) fetch(rx[1], rv[1], kof(1));
     for (int st = 0; st < steps; st += 2) {
         stage(rx[0], rv[0]);
         __syncthreads();
-        if (st + 2 < steps) fetch(rx[0], rv[0], (first + st + 2) * NT_STEP);
+        if (st + 2 < steps) fetch(rx[0], rv[0], kof(st + 2));
         multiply();
-        encode((first + st) * NT_STEP);
+        encode(kof(st));
         __syncthreads();
         if (st + 1 < steps) {
             stage(rx[1], rv[1]);
             __syncthreads();
-            if (st + 3 < steps) fetch(rx[1], rv[1], (first + st + 3) * NT_STEP);
+            if (st + 3 < steps) fetch(rx[1], rv[1], kof(st + 3));
             multiply();
-            encode((first + st + 1) * NT_STEP);
+            encode(kof(st + 1));
             __syncthreads();
         }
     }
@@ -315,7 +322,7 @@ int lowrank_nt(const void* x, int64_t ldx, const void* v, int64_t M, int64_t R, 
 #define METIS_NT(RT, Q) METIS_NT2(RT, Q, false)
 #define METIS_NT2(RT, Q, E) hipLaunchKernelGGL((lowrank_nt_kernel<RT, Q, E>), grid, dim3((Q >= 0 && E) ? 512 : 256), 0, st, (const uint16_t*)x, ldx, (const uint16_t*)v, \
                                            (const uint16_t*)s, (uint16_t*)xv, (uint16_t*)t, (int)M, (int)K, part, (uint2*)codes, q.amax, \
-                                           q.gmax, (uint32_t)kDeferredPartials)
+                                           q.gmax, (uint32_t)kDeferredPartials, measure_env("METIS_NT_NOROT") ? 0 : 1)
 #define METIS_NTQ(RT) do { if (qmode < 0) METIS_NT(RT, -1); else if (qmode == 0) { if (ew) METIS_NT2(RT, 0, true); else METIS_NT(RT, 0); } \
                            else { if (ew) METIS_NT2(RT, 1, true); else METIS_NT(RT, 1); } } while (0)
     if (R == 32) METIS_NTQ(1);
