@@ -68,7 +68,7 @@ __global__ __launch_bounds__((QMODE >= 0 && EW) ? 512 : 256) void lowrank_nt_ker
     // same offset of every row fall on the same few memory channels (flushed caches, 8192 x 4096: 39 -> 31 us; 8192 x 14336:
     // 146 -> 104 us; row lengths like 7168 or 17920 bytes are indifferent).  The binary32 sums of a tile are therefore added
     // in an order that depends on the tile, the same for every call and for both forms of the kernel.
-    const int rot = (rotate && steps > 0) ? (int)((blockIdx.x * 5u) % (unsigned)steps) : 0;
+    const int rot = (rotate && steps > 0) ? (int)((blockIdx.x * (unsigned)rotate) % (unsigned)steps) : 0;
     auto kof = [&](int st) { int q = st + rot; if (q >= steps) q -= steps; return (first + q) * NT_STEP; };
     if constexpr (QMODE >= 0 && EW) {
         if (tid >= 256) {                                       // the encoding waves: same barriers as the others, nothing else shared
@@ -322,7 +322,7 @@ int lowrank_nt(const void* x, int64_t ldx, const void* v, int64_t M, int64_t R, 
 #define METIS_NT(RT, Q) METIS_NT2(RT, Q, false)
 #define METIS_NT2(RT, Q, E) hipLaunchKernelGGL((lowrank_nt_kernel<RT, Q, E>), grid, dim3((Q >= 0 && E) ? 512 : 256), 0, st, (const uint16_t*)x, ldx, (const uint16_t*)v, \
                                            (const uint16_t*)s, (uint16_t*)xv, (uint16_t*)t, (int)M, (int)K, part, (uint2*)codes, q.amax, \
-                                           q.gmax, (uint32_t)kDeferredPartials, measure_env("METIS_NT_NOROT") ? 0 : 1)
+                                           q.gmax, (uint32_t)kDeferredPartials, measure_int("METIS_NT_ROT", 5))
 #define METIS_NTQ(RT) do { if (qmode < 0) METIS_NT(RT, -1); else if (qmode == 0) { if (ew) METIS_NT2(RT, 0, true); else METIS_NT(RT, 0); } \
                            else { if (ew) METIS_NT2(RT, 1, true); else METIS_NT(RT, 1); } } while (0)
     if (R == 32) METIS_NTQ(1);
