@@ -1123,15 +1123,16 @@ def _linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.
             M, K, ctypes.cast(arr, ctypes.c_void_p), len(members), 0))
     ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
     dt = DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16
-    # the activation's decode layout (written by its quantizer) in place of the row-major packing: wide runs only
-    a_dec = a.decode_layout if (takes and K % 256 == 0 and all(m[0].scales.data_ptr() % 8 == 0 for m in members)) else None
-    a_codes, a_scales = (a_dec.data_ptr(), None) if a_dec is not None else (a.codes.data_ptr(), a.scales.data_ptr())
     if operand:
+        # (a quantizer call that deferred its scale bytes never gets them: the operand kernel forms them on the way)
         aop = decode_operand(a, MODE_PB16, center)
         rc = L.metis_linear_fwd_grouped_operand(aop.data_ptr(), a.unit.data_ptr(), M, K, ap, len(members), dt, MODE_PB16,
                                                 None if ws is None else ws.data_ptr(), need, _stream())
         check(rc, "metis_linear_fwd_grouped_operand", (M, K, [m[0].rows for m in members]))
         return outs
+    # the activation's decode layout (written by its quantizer) in place of the row-major packing: wide runs only
+    a_dec = a.decode_layout if (takes and K % 256 == 0 and all(m[0].scales.data_ptr() % 8 == 0 for m in members)) else None
+    a_codes, a_scales = (a_dec.data_ptr(), None) if a_dec is not None else (a.codes.data_ptr(), a.scales.data_ptr())
     if center is not None:
         center = center.reshape(-1).to(device=dev, dtype=torch.float32).contiguous()
         if center.numel() != K:

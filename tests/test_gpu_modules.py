@@ -795,3 +795,26 @@ def test_an_unshared_activation_is_quantized_and_projected_in_one_pass(compute, 
     with torch.no_grad():
         layer(x[:1])
     assert calls["n"] == 1
+
+
+def test_decode_step_in_bf16_arithmetic_never_writes_the_activation_scale_bytes(monkeypatch):
+    """A decode-sized forward in bf16 arithmetic feeds the GEMM ready operands built straight from the codes and the parked
+    block maxima: the quantizer's second launch (scale bytes of the row-major packing) must not run at all."""
+    from metis_hip import ops
+    layer, _ = _make_bitlinear(512, 768, 64, True, torch.bfloat16, torch.bfloat16, seed=43)
+    x = synthetic_activation(78, 64, 512).reshape(64, 1, 512).cuda()
+    calls = {"n": 0}
+    orig = ops.PackedNVFP4._materialize
+
+    def counting(self):
+        calls["n"] += 1
+        return orig(self)
+
+    with torch.no_grad():
+        want = layer(x)
+    monkeypatch.setattr(ops.PackedNVFP4, "_materialize", counting)
+    with torch.no_grad():
+        got = layer(x)
+    torch.cuda.synchronize()
+    assert calls["n"] == 0
+    assert torch.equal(got, want)
