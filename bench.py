@@ -109,6 +109,23 @@ def region_us(torch, fn, steps, warmup):
     return e0.elapsed_time(e1) / steps * 1e3
 
 
+def flushed_us(torch, fn, flush, n=15):
+    """Median duration of one call (events on the launch stream) when a read of `flush` (larger than the caches and the
+    256 MB memory-side cache together) runs before every call: inputs come from HBM itself, not from what the previous
+    iteration of a timing loop left in a cache.  A read, not a fill: dirty lines would have to be written back while the
+    timed call runs."""
+    ts = []
+    words = flush.view(torch.int32)
+    for _ in range(n):
+        words.sum()
+        pair = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+        fn(pair)
+        torch.cuda.synchronize()
+        ts.append(pair[0].elapsed_time(pair[1]) * 1e3)
+    ts.sort()
+    return ts[len(ts) // 2]
+
+
 def settle(torch, fn, seconds=1.0):
     """Untimed launches of the headline step until `seconds` have passed: the part's clock needs about a second under
     load to settle, whatever --warmup says.  Returns the seconds spent."""
@@ -293,6 +310,8 @@ def main():
     q_ms = region_us(torch, qstep, qsteps, args.warmup) * 1e-3
     q_bytes = x1.numel() * QUANT_BYTES_PER_ELT
     q_gbs = q_bytes / (q_ms * 1e-3) / 1e9
+    flush_buf = torch.zeros(512 << 20, dtype=torch.uint8, device=dev)
+    q_cold_us = flushed_us(torch, qstep, flush_buf)
 
     # deferred scale bytes: the first launch alone (codes + parked block maxima); the consumer forms unit and bytes
     qdef = torch.empty(L.metis_nvfp4_deferred_bytes(8192, 4096), dtype=torch.uint8, device=dev)
@@ -354,6 +373,8 @@ def main():
     n_ms = region_us(torch, nstep, qsteps, args.warmup) * 1e-3
     n_bytes = h.numel() * NORMQ_BYTES_PER_ELT
     n_gbs = n_bytes / (n_ms * 1e-3) / 1e9
+    n_cold_us = flushed_us(torch, nstep, flush_buf)
+    del flush_buf
 
     ndef = torch.empty(L.metis_nvfp4_deferred_bytes(16384, 4096), dtype=torch.uint8, device=dev)
 
@@ -788,6 +809,9 @@ def main():
                   "value": round(q_gbs, 1), "unit": "GB/s", "us_per_call": round(q_ms * 1e3, 2),
                   "timing": "events around the region of back-to-back calls on the launch stream; us_per_call_event_pairs brackets every call with its own pair",
                   "us_per_call_event_pairs": round(q_pair_ms * 1e3, 2),
+                  "us_per_call_caches_flushed": round(q_cold_us, 2),
+                  "caches_flushed": "a read of 512 MiB before every call (own event pair, median of 15): nothing is served from the 256 MB "
+                                    "memory-side cache, which in the back-to-back loop still holds the 67 MB input of the previous call",
                   "round_trip": {"workload": "the same tensor through metis_nvfp4_quant_dequant_row: codes + scale bytes + unit + the dequantized bf16 "
                                              "tensor (config 1's three outputs) from one call of two launches; 4.5625 B/element = 153.09 MB",
                                  "value": round(qr_gbs, 1), "unit": "GB/s", "us_per_call": round(qr_ms * 1e3, 2),
@@ -806,6 +830,7 @@ def main():
         "rmsnorm_quant": {"workload": "config 2: fused RMSNorm->NVFP4 bf16 [16384,4096] (P32), normed+codes+scales",
                           "value": round(n_gbs, 1), "unit": "GB/s", "us_per_call": round(n_ms * 1e3, 2),
                           "us_per_call_event_pairs": round(n_pair_ms * 1e3, 2),
+                          "us_per_call_caches_flushed": round(n_cold_us, 2),
                           "roofline": {"bound": "hbm", "kernel": "rmsnorm_quant_rows_kernel+quant_scales_kernel",
                                        "achieved": round(n_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                        "frac": round(n_gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_NORMQ_C2,
