@@ -65,9 +65,10 @@ __global__ __launch_bounds__((QMODE >= 0 && EW) ? 512 : 256) void lowrank_nt_ker
     __shared__ float smax[4];
     // Every row tile starts at a different step of its K range and wraps around: at any moment the workgroups then read
     // different column stripes of x instead of the same one.  With rows a multiple of 4 KiB long, 512-byte pieces at the
-    // same offset of every row fall on the same few memory channels (flushed caches, 8192 x 4096: 39 -> 31 us; 8192 x 14336:
-    // 146 -> 104 us; row lengths like 7168 or 17920 bytes are indifferent).  The binary32 sums of a tile are therefore added
-    // in an order that depends on the tile, the same for every call and for both forms of the kernel.
+    // same offset of every row can fall on the same few memory channels (flushed caches, 8192 x 14336: 146 -> 104 us on one
+    // machine, 126 -> 107 us on another; 8192 x 4096: 39 -> 31 us on the first, no change on the second; row lengths like
+    // 7168 or 17920 bytes are indifferent).  The binary32 sums of a tile are therefore added in an order that depends on
+    // the tile, the same for every call and for both forms of the kernel.
     const int rot = (rotate && steps > 0) ? (int)((blockIdx.x * (unsigned)rotate) % (unsigned)steps) : 0;
     auto kof = [&](int st) { int q = st + rot; if (q >= steps) q -= steps; return (first + q) * NT_STEP; };
     if constexpr (QMODE >= 0 && EW) {
