@@ -1294,8 +1294,11 @@ __global__ __launch_bounds__(256) void quant_lowrank_residual_kernel(
     void* __restrict__ ker_out, uint32_t tiles_c, uint32_t tiles)
 {
     static_assert(MODE == 0 || !F32IN, "bf16 arithmetic reads bf16 tensors");
-    __shared__ __align__(16) float s_v[kLrRanks][kLrCols];
-    __shared__ __align__(16) float s_u[kLrRows][kLrRanks];
+    // LDS layouts without bank conflicts: of V, quarter q of every thread's block of 16 lies side by side with the same
+    // quarter of the fifteen other blocks (a 16-byte read of sixteen lanes covers 256 contiguous bytes); the rows of
+    // U diag(s) are 80 bytes apart, so that the four row groups of a wave read from different banks.
+    __shared__ float4 s_v[kLrRanks][4][kLrCols / kBlock];
+    __shared__ __align__(16) float s_u[kLrRows][kLrRanks + 4];
     const uint32_t t = threadIdx.x, cb = t & 15u, rg = t >> 4;
     const uint32_t nbpr = cols / kBlock;
     float gmax = 0.0f;
@@ -1307,40 +1310,48 @@ __global__ __launch_bounds__(256) void quant_lowrank_residual_kernel(
         for (int i = 0; i < 4; ++i)
 #pragma unroll
             for (int j = 0; j < kBlock; ++j) acc[i][j] = 0.0f;
-        for (uint32_t k0 = 0; k0 < rank; k0 += kLrRanks) {
-            __syncthreads();                                   // the previous chunk (or tile) has been read
+        // The factors of the next sixteen ranks are fetched into registers while the current ones are multiplied, and go to
+        // LDS between two barriers afterwards: their memory latency is off the critical path.
+        float pv[kBlock];
+        float4 pu;
+        auto fetch_chunk = [&](uint32_t k0) {
             {   // V: rank k0 + t / 16, columns col0 + 16 (t % 16) ..; zeros beyond the tensor
                 const uint32_t k = k0 + rg, c = col0 + cb * kBlock;
-                float v[kBlock];
 #pragma unroll
-                for (int j = 0; j < kBlock; ++j) v[j] = 0.0f;
+                for (int j = 0; j < kBlock; ++j) pv[j] = 0.0f;
                 if (c < cols) {
                     if constexpr (MODE == 0) {
                         const float4* p = reinterpret_cast<const float4*>(static_cast<const float*>(vtv) + (size_t)k * cols + c);
 #pragma unroll
-                        for (int q = 0; q < 4; ++q) { const float4 f = p[q]; v[4 * q] = f.x; v[4 * q + 1] = f.y; v[4 * q + 2] = f.z; v[4 * q + 3] = f.w; }
+                        for (int q = 0; q < 4; ++q) { const float4 f = p[q]; pv[4 * q] = f.x; pv[4 * q + 1] = f.y; pv[4 * q + 2] = f.z; pv[4 * q + 3] = f.w; }
                     } else {
                         const uint4* p = reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(vtv) + (size_t)k * cols + c);
-                        unpack16(p[0], p[1], v);
+                        unpack16(p[0], p[1], pv);
                     }
                 }
-                float4* d = reinterpret_cast<float4*>(&s_v[rg][cb * kBlock]);
-#pragma unroll
-                for (int q = 0; q < 4; ++q) d[q] = make_float4(v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]);
             }
             {   // U diag(s): row row0 + t / 4, ranks k0 + 4 (t % 4) ..
                 const uint32_t r = row0 + (t >> 2), k = k0 + (t & 3u) * 4u;
-                float4 f = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                pu = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
                 if (r < rows) {
-                    if constexpr (MODE == 0) f = *reinterpret_cast<const float4*>(static_cast<const float*>(usv) + (size_t)r * rank + k);
+                    if constexpr (MODE == 0) pu = *reinterpret_cast<const float4*>(static_cast<const float*>(usv) + (size_t)r * rank + k);
                     else {
                         const uint2 w = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(usv) + (size_t)r * rank + k);
-                        f = make_float4(bf16_lo(w.x), bf16_hi(w.x), bf16_lo(w.y), bf16_hi(w.y));
+                        pu = make_float4(bf16_lo(w.x), bf16_hi(w.x), bf16_lo(w.y), bf16_hi(w.y));
                     }
                 }
-                *reinterpret_cast<float4*>(&s_u[t >> 2][(t & 3u) * 4u]) = f;
+            }
+        };
+        fetch_chunk(0);
+        for (uint32_t k0 = 0; k0 < rank; k0 += kLrRanks) {
+            __syncthreads();                                   // the previous chunk (or tile) has been read
+            {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) s_v[rg][q][cb] = make_float4(pv[4 * q], pv[4 * q + 1], pv[4 * q + 2], pv[4 * q + 3]);
+                *reinterpret_cast<float4*>(&s_u[t >> 2][(t & 3u) * 4u]) = pu;
             }
             __syncthreads();
+            if (k0 + kLrRanks < rank) fetch_chunk(k0 + kLrRanks);
 #pragma unroll
             for (int kq = 0; kq < kLrRanks / 4; ++kq) {
                 float4 u4[4];
@@ -1349,9 +1360,8 @@ __global__ __launch_bounds__(256) void quant_lowrank_residual_kernel(
 #pragma unroll
                 for (int kk = 0; kk < 4; ++kk) {
                     float vv[kBlock];
-                    const float4* sp = reinterpret_cast<const float4*>(&s_v[kq * 4 + kk][cb * kBlock]);
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) { const float4 f = sp[q]; vv[4 * q] = f.x; vv[4 * q + 1] = f.y; vv[4 * q + 2] = f.z; vv[4 * q + 3] = f.w; }
+                    for (int q = 0; q < 4; ++q) { const float4 f = s_v[kq * 4 + kk][q][cb]; vv[4 * q] = f.x; vv[4 * q + 1] = f.y; vv[4 * q + 2] = f.z; vv[4 * q + 3] = f.w; }
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         const float uu = kk == 0 ? u4[i].x : kk == 1 ? u4[i].y : kk == 2 ? u4[i].z : u4[i].w;
