@@ -99,9 +99,12 @@ __global__ __launch_bounds__(256) void quant_codes_contig_centered_kernel(const 
                                                                           uint32_t* __restrict__ ws_gmax, uint32_t nblocks,
                                                                           uint32_t nbpr, uint32_t fill_to)
 {
-    __shared__ __align__(16) float cen[kCentreMaxCols];
+    // quarter q of block b at cen[q][b]: the 16-byte reads of consecutive lanes (consecutive blocks) are consecutive in LDS
+    // (block after block, a lane's four reads would be 64 bytes apart from its neighbour's: four lanes per bank)
+    __shared__ float4 cen[4][kCentreMaxCols / kBlock];
     for (uint32_t c = threadIdx.x; c < nbpr * kBlock; c += 256u)
-        cen[c] = MODE == 0 ? static_cast<const float*>(center)[c] : bf16_lo(static_cast<const uint16_t*>(center)[c]);
+        reinterpret_cast<float*>(&cen[(c % kBlock) / 4u][c / kBlock])[c % 4u] =
+            MODE == 0 ? static_cast<const float*>(center)[c] : bf16_lo(static_cast<const uint16_t*>(center)[c]);
     __syncthreads();
     float gmax = 0.0f;
     const uint32_t step = gridDim.x * 256u, step_mod = step % nbpr;
@@ -115,10 +118,9 @@ __global__ __launch_bounds__(256) void quant_codes_contig_centered_kernel(const 
         if (nxt < nblocks) { c0 = x[2 * (size_t)nxt]; c1 = x[2 * (size_t)nxt + 1]; }
         float v[kBlock];
         unpack16(a0, a1, v);
-        const float4* cp = reinterpret_cast<const float4*>(cen + cb * kBlock);
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            const float4 f = cp[q];
+            const float4 f = cen[q][cb];
             if constexpr (MODE == 0) {
                 v[4 * q] -= f.x; v[4 * q + 1] -= f.y; v[4 * q + 2] -= f.z; v[4 * q + 3] -= f.w;
             } else {
