@@ -13,10 +13,10 @@
 // for all R columns, and the four partial sums meet in LDS at the end.
 //
 // lowrank_tn: the contraction runs down the rows of both operands, so each has to be turned: a workgroup owns 64
-// columns of a and one slice of the tokens; a step of 64 tokens is loaded row by row (coalesced) and written to LDS
-// transposed, element by element, so that the MFMA fragments (8 consecutive tokens of one column) are single
-// 16-byte reads.  Token slices give every compute unit work; their binary32 partial results go to a caller workspace
-// and a second kernel adds them in slice order.
+// columns of a and one slice of the tokens; a step of 64 tokens is loaded row by row (coalesced) and staged in LDS as it
+// is; the MFMA fragments (8 consecutive tokens of one column) are read with the transposing LDS read of gfx950.  Token
+// slices give every compute unit work; their binary32 partial results go to a caller workspace and a second kernel adds
+// them in slice order.
 #include "metis_device.h"
 #include "metis_host.h"
 #include "nvfp4_encode.h"
@@ -26,7 +26,6 @@ namespace metis {
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 
-constexpr int LR_STRIDE = 72;                    // halves per staged row of 64: 144 bytes, conflict-free 16-byte reads
 constexpr int NT_STEP = 256;                     // k per step of lowrank_nt
 constexpr int NT_STRIDE = NT_STEP + 8;           // halves per staged row: 528 bytes, conflict-free 16-byte reads
 
@@ -350,8 +349,14 @@ __global__ __launch_bounds__(256) void lowrank_tn_kernel(const uint16_t* __restr
                                                          int L, int C, int steps_per_slice, float* __restrict__ part)
 {
     constexpr int R = RT * 32;
-    __shared__ __attribute__((aligned(16))) uint16_t at[64 * LR_STRIDE];      // [column][token]
-    __shared__ __attribute__((aligned(16))) uint16_t bt[R * LR_STRIDE];       // [r][token]
+    // Staged as loaded, token by token, in slabs of 32 columns: [slab][token][32], 64 bytes per token and slab.  The MFMA
+    // fragments (8 consecutive tokens of one column) come out of LDS through the transposing read of gfx950
+    // (ds_read_b64_tr_b16: the sixteen lanes of a group hand in sixteen addresses of 4 halves each, lane i the piece
+    // (row i / 4, columns 4 (i % 4) ..), and lane l receives element l % 4 ... of column l: four consecutive tokens of its own
+    // column), so nothing is scattered element by element.  Rows of 64 bytes keep both the 16-byte writes and the
+    // transposing reads free of bank conflicts (rows r .. r + 3 and the two 32-byte halves of a row fall on different banks).
+    __shared__ __attribute__((aligned(16))) uint16_t at[2][64 * 32];          // [column slab][token][column]
+    __shared__ __attribute__((aligned(16))) uint16_t bt[RT][64 * 32];         // [r slab][token][r]
     __shared__ __attribute__((aligned(16))) float red[2][RT][16][64];         // the two waves that take the second half of each step
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int c0 = blockIdx.x * 64, slice = blockIdx.y;
@@ -375,25 +380,14 @@ __global__ __launch_bounds__(256) void lowrank_tn_kernel(const uint16_t* __restr
             rbv[i] = l < L ? *reinterpret_cast<const uint4*>(b + (int64_t)l * R + ch * 8) : make_uint4(0u, 0u, 0u, 0u);
         }
     };
-    // Transposed tiles: row = column of the operand, 64 tokens in 8 chunks of 8; the chunk of tokens [8 q, 8 q + 8) of
-    // row n sits at chunk q ^ ((n >> 4) & 3), so that the eight column groups a wave scatters at once fall into
-    // different banks (unswizzled they share eight of them).
-    auto scatter = [&](uint16_t* dst, int row0, int tok, const uint4& q) {      // 8 elements of one token -> 8 rows of dst
-        const uint32_t w[4] = {q.x, q.y, q.z, q.w};
-        const int pos = (((tok >> 3) ^ ((row0 >> 4) & 3)) << 3) | (tok & 7);    // rows row0 .. row0 + 7 share row >> 4
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            dst[(row0 + 2 * j) * LR_STRIDE + pos] = (uint16_t)(w[j] & 0xffffu);
-            dst[(row0 + 2 * j + 1) * LR_STRIDE + pos] = (uint16_t)(w[j] >> 16);
-        }
-    };
     auto stage = [&](const uint4 (&ra)[2], const uint4 (&rbv)[BPT]) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) scatter(at, lch * 8, i * 32 + lrow, ra[i]);
+        for (int i = 0; i < 2; ++i)
+            *reinterpret_cast<uint4*>(&at[lch >> 2][(i * 32 + lrow) * 32 + (lch & 3) * 8]) = ra[i];
 #pragma unroll
         for (int i = 0; i < BPT; ++i) {
-            const int id = i * 256 + tid;
-            scatter(bt, (id % BCH) * 8, id / BCH, rbv[i]);
+            const int id = i * 256 + tid, tok = id / BCH, ch = id % BCH;
+            *reinterpret_cast<uint4*>(&bt[ch >> 2][tok * 32 + (ch & 3) * 8]) = rbv[i];
         }
     };
     float16_t acc[RT];
@@ -403,15 +397,27 @@ __global__ __launch_bounds__(256) void lowrank_tn_kernel(const uint16_t* __restr
         for (int e = 0; e < 16; ++e) acc[j][e] = 0.0f;
     // wave -> 32 columns (wave % 2) and the first or second half (wave / 2) of every 64-token step
     const int ct = wave & 1, kh = wave >> 1;
-    const int frow = (lane & 31) * LR_STRIDE, fsw = ((lane & 31) >> 4) & 1;     // rows 32 j + n: (row >> 4) & 3 = 2 (j & 1) + fsw
+    // lane l of the MFMA holds column l % 32 and the tokens 8 (l / 32) .. + 7 of a 16-token step; in its group of sixteen
+    // lanes it hands in the piece (token i / 4, columns 16 (l / 16 % 2) + 4 (i % 4) ..), i = l % 16
+    typedef short short4_t __attribute__((ext_vector_type(4)));
+    typedef short short8_t __attribute__((ext_vector_type(8)));
+    const int piece = ((lane & 15) >> 2) * 32 + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
+    auto fragment = [&](const uint16_t* slab, int tok0) -> bf16x8_t {
+        typedef short4_t __attribute__((address_space(3))) * lds_ptr_t;
+        const uint16_t* p = slab + tok0 * 32 + piece;
+        const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)p);
+        const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(p + 4 * 32));
+        const short8_t v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        return __builtin_bit_cast(bf16x8_t, v);
+    };
     auto multiply = [&]() {
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
-            const int q = kh * 4 + ks * 2 + (lane >> 5);
-            const bf16x8_t fa = *reinterpret_cast<const bf16x8_t*>(at + ct * 32 * LR_STRIDE + frow + ((q ^ (2 * ct + fsw)) << 3));
+            const int tok0 = (kh * 4 + ks * 2 + (lane >> 5)) * 8;
+            const bf16x8_t fa = fragment(at[ct], tok0);
 #pragma unroll
             for (int j = 0; j < RT; ++j) {
-                const bf16x8_t fb = *reinterpret_cast<const bf16x8_t*>(bt + j * 32 * LR_STRIDE + frow + ((q ^ (2 * (j & 1) + fsw)) << 3));
+                const bf16x8_t fb = fragment(bt[j], tok0);
                 acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb, fa, acc[j], 0, 0, 0);
             }
         }
