@@ -93,14 +93,26 @@ __global__ __launch_bounds__(256) void expand_xt_kernel(const uint32_t* __restri
                     const int half = chunk & 1;                  // which half of the block this lane holds
 #pragma unroll
                     for (int j = 0; j < 8; ++j) {
-                        const float other = __shfl_xor(mine[j], 1);
+                        // the neighbouring lane's value through DPP (quad_perm 1,0,3,2): no trip through the LDS crossbar
+                        const float other = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, mine[j]), 0xB1, 0xf, 0xf, false));
                         blk[j] = half ? other : mine[j];
                         blk[8 + j] = half ? mine[j] : other;
                     }
-                    hadamard16_inverse(blk, sign_mask);
+                    // This lane's half of the rotated block alone, n = 8 half + j: H[k][n] = H[k][j] for k < 8 and
+                    // H[k][j] (-1)^half for k >= 8, so the second half of the inputs changes sign with `half` and the sums run
+                    // in the order of hadamard16_inverse (a - b and a + (-b) are the same operation).  No array is indexed
+                    // by a run-time value: such an array would be moved to LDS.
+                    const uint32_t flip = (uint32_t)half << 31;
+#pragma unroll
+                    for (int k = 8; k < kBlock; ++k) blk[k] = __uint_as_float(__float_as_uint(blk[k]) ^ flip);
                     float o[8];
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) o[j] = half ? blk[8 + j] : blk[j];
+                    for (int j = 0; j < 8; ++j) {
+                        float acc = blk[0];
+#pragma unroll
+                        for (int k = 1; k < kBlock; ++k) acc = (__builtin_popcount(k & j) & 1) ? acc - blk[k] : acc + blk[k];
+                        o[j] = __uint_as_float(__float_as_uint(acc * 0.0625f) ^ (((sign_mask >> (8 * half + j)) & 1u) << 31));
+                    }
                     if constexpr (PB16 != 0) {
                         v.x = rb_pair(o[0], o[1]); v.y = rb_pair(o[2], o[3]); v.z = rb_pair(o[4], o[5]); v.w = rb_pair(o[6], o[7]);
                     } else {
