@@ -351,9 +351,10 @@ __global__ __launch_bounds__(256) void lowrank_tn_kernel(const uint16_t* __restr
     constexpr int R = RT * 32;
     // Staged as loaded, token by token, in slabs of 32 columns: [slab][token][32], 64 bytes per token and slab.  The MFMA
     // fragments (8 consecutive tokens of one column) come out of LDS through the transposing read of gfx950
-    // (ds_read_b64_tr_b16: the sixteen lanes of a group hand in sixteen addresses of 4 halves each, lane i the piece
-    // (row i / 4, columns 4 (i % 4) ..), and lane l receives element l % 4 ... of column l: four consecutive tokens of its own
-    // column), so nothing is scattered element by element.  Rows of 64 bytes keep both the 16-byte writes and the
+    // (ds_read_b64_tr_b16: the sixteen lanes of a group hand in sixteen addresses of 4 halves each and lane l receives
+    // element l % 4 of the pieces of lanes l / 4, l / 4 + 4, l / 4 + 8, l / 4 + 12 -- established with a probe on the
+    // device.  With lane i handing in the piece (token i / 4, columns 4 (i % 4) ..), lane l gets column l of four
+    // consecutive tokens), so nothing is scattered element by element.  Rows of 64 bytes keep both the 16-byte writes and the
     // transposing reads free of bank conflicts (rows r .. r + 3 and the two 32-byte halves of a row fall on different banks).
     __shared__ __attribute__((aligned(16))) uint16_t at[2][64 * 32];          // [column slab][token][column]
     __shared__ __attribute__((aligned(16))) uint16_t bt[RT][64 * 32];         // [r slab][token][r]
