@@ -20,7 +20,7 @@ def _gamma(seed, cols):
 
 
 @pytest.mark.parametrize("mode", [0, 1])
-@pytest.mark.parametrize("rows,cols", [(64, 512), (33, 1536), (16, 4096), (5, 8192), (7, 48), (3, 12288)])
+@pytest.mark.parametrize("rows,cols", [(64, 512), (33, 1536), (16, 4096), (5, 8192), (7, 48), (3, 12288), (256, 512), (300, 3584), (257, 4096)])
 def test_fused_rmsnorm_quant(rows, cols, mode):
     from metis_hip import ops
     from oracle import metis_oracle as O
