@@ -1157,11 +1157,23 @@ def _linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.
     return outs
 
 
+def _tiled_backward_pays(M: int, N: int, K: int, device_index: int) -> bool:
+    """Whether a backward product out[M, N] over a contraction of K goes to the pipelined kernel on tiled expansions made
+    for this one call: from about 2e11 flop on, with at least one 256 x 256 tile per compute unit, the faster GEMM more
+    than pays for writing the expansions (8192 x 4096 x 14336: input gradient 858 -> 749 us with the weight's
+    expansion cached, weight gradient 915 -> 835 us with both operands expanded; 4096 x 1536 x 8960: 134 -> 149 and
+    117 -> 141 us, so small products stay on the packed kernel).  Same bits either way."""
+    return (tiled_weight_copies and M >= 256 and N >= 256 and K % 32 == 0 and 2.0 * M * N * K >= 2e11
+            and (M // 256) * (N // 256) >= _device_cus(device_index))
+
+
 def linear_dgrad(dy: PackedNVFP4, wt: PackedNVFP4, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     """grad_input[L, K] from dY packed along N [L, N] and W packed along N (column-blocked) [K, N]."""
     if dy.cols != wt.cols:
         raise ValueError(f"contraction mismatch: {dy.cols} vs {wt.cols}")
     L, N, K = dy.rows, dy.cols, wt.rows
+    if dy.mode == wt.mode and _tiled_backward_pays(L, K, N, dy.codes.device.index or 0):
+        return linear_fwd(dy, wt, out_dtype=out_dtype, tiled=True)          # out = deq(dy) . deq(wt)^T: the same product
     out = torch.empty(L, K, dtype=out_dtype, device=dy.codes.device)
     dt = DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16
     ws = _gemm_workspace(L, K, N, out.device)
@@ -1182,6 +1194,8 @@ def linear_wgrad(dyt: PackedNVFP4, xt: PackedNVFP4, out_dtype: torch.dtype = tor
     if dyt.cols != xt.cols:
         raise ValueError(f"contraction mismatch: {dyt.cols} vs {xt.cols}")
     N, L, K = dyt.rows, dyt.cols, xt.rows
+    if dyt.mode == xt.mode and _tiled_backward_pays(N, K, L, dyt.codes.device.index or 0):
+        return linear_fwd(dyt, xt, out_dtype=out_dtype, tiled=True)
     out = torch.empty(N, K, dtype=out_dtype, device=dyt.codes.device)
     dt = DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16
     ws = _gemm_workspace(N, K, L, out.device)

@@ -807,3 +807,30 @@ def test_decode_sized_activations_leave_the_quantizer_in_the_decode_layout(M, K,
             got = ops.linear_fwd_grouped(dec, members, **kw)
             for a, b in zip(got, want):
                 assert torch.equal(a, b), (mode, kw.keys())
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+def test_large_backward_products_take_the_pipelined_kernel_with_the_same_bits(mode):
+    """From about 2e11 flop on, linear_dgrad and linear_wgrad expand their operands for the one call and run on the
+    pipelined kernel (ops._tiled_backward_pays); the products are the packed kernels', bit for bit."""
+    from metis_hip import ops
+    g = torch.Generator().manual_seed(4242 + mode)
+    N, K, L = 4096, 4352, 8192
+    assert ops._tiled_backward_pays(L, K, N, 0) and ops._tiled_backward_pays(N, K, L, 0)
+    assert not ops._tiled_backward_pays(4096, 1536, 8960, 0)               # the config-4 projection stays packed
+    dy = (torch.randn(L, N, generator=g) * 1e-3).bfloat16().cuda()
+    x = torch.randn(L, K, generator=g).bfloat16().cuda()
+    w = (torch.randn(N, K, generator=g) * 0.02).bfloat16().cuda()
+    p_dy, p_dyt, p_xt = ops.quantize(dy, mode), ops.quantize(dy, mode, col=True), ops.quantize(x, mode, col=True)
+    p_wt = ops.quantize(w, mode, col=True)
+    p_wt.persistent = True
+    gx, gw = ops.linear_dgrad(p_dy, p_wt), ops.linear_wgrad(p_dyt, p_xt)
+    ops.tiled_weight_copies = False
+    try:
+        gx_p, gw_p = ops.linear_dgrad(p_dy, p_wt), ops.linear_wgrad(p_dyt, p_xt)
+    finally:
+        ops.tiled_weight_copies = True
+    torch.cuda.synchronize()
+    assert torch.equal(gx, gx_p) and torch.equal(gw, gw_p)
+    ref = dy.double() @ w.double()
+    assert rel_fro(gx.double().cpu(), ref.cpu()) <= 0.2                     # FP4 operands: a coarse sanity bound on the product itself
