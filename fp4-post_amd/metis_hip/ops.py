@@ -869,7 +869,8 @@ def linear_fwd(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None,
     """out[M, N] = deq(a)[M, K] . deq(b)[N, K]^T (+ t[M, r] . u[N, r]^T) (+ bias[N]).
 
     tiled=None picks the pipelined kernel on tiled binary16 expansions when b is a cached weight and the shape is
-    large (see _tiled_applies); True / False force the choice.  Same bits either way (unsplit).
+    large (see _tiled_applies), or when the product is large enough to pay for expansions made for this one call
+    (_tiled_backward_pays); True / False force the choice.  Same bits either way (unsplit).
     reference_rounding: the forward of a layer whose arithmetic is bf16 (both operands packed in that mode): follow the
     reference's all-bf16 evaluation (twice-rounded bf16 operands, residual product and bias add rounded to bf16): the
     pipelined kernel from 256 rows on, the decode-sized kernel below (shapes it does not take get exact products).
@@ -888,7 +889,7 @@ def linear_fwd(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None,
     rounded = reference_rounding and a.mode == MODE_PB16 and b.mode == MODE_PB16
     faithful = rounded and (a.rows >= 256 or tiled) and a.cols % 32 == 0
     if tiled is None:
-        tiled = faithful or (not expanded and _tiled_applies(a, b))
+        tiled = faithful or (not expanded and (_tiled_applies(a, b) or _tiled_backward_pays(a.rows, b.rows, a.cols, a.codes.device.index or 0)))
     if tiled:
         return linear_fwd_tiled(a, b, t=t, u=u, bias=bias, out_dtype=out_dtype, reference_rounding=faithful, split_k=split_k)
     M, N, K = a.rows, b.rows, a.cols
