@@ -19,7 +19,8 @@ _workspaces: dict = {}
 # (0.5625 B) for decode-sized batches, and the tiled binary16 expansions (2 B each: one per arithmetic the layer runs in,
 # one more per arithmetic for the transposed operand of the NV recipe).  Memory-bound deployments switch them off:
 # without the tiled copies, binary32-arithmetic GEMMs run on the packed operands, and bf16-arithmetic GEMMs expand the
-# weight on every call instead of once.  Same bits either way.
+# weight on every call instead of once.  A plain unsplit product has the same bits either way; a low-rank term joins
+# the binary32 sum at another point on the pipelined kernel than on the packed one (1e-6 relative in binary32).
 decode_layout_weights = True
 tiled_weight_copies = True
 # Decode-sized activations (fewer than 256 rows, a multiple of 256 columns) leave the round-to-nearest quantizers in the
@@ -870,7 +871,8 @@ def linear_fwd(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None,
 
     tiled=None picks the pipelined kernel on tiled binary16 expansions when b is a cached weight and the shape is
     large (see _tiled_applies), or when the product is large enough to pay for expansions made for this one call
-    (_tiled_backward_pays); True / False force the choice.  Same bits either way (unsplit).
+    (_tiled_backward_pays); True / False force the choice.  Same products either way; a plain unsplit product has the
+    same bits, a low-rank term joins the binary32 sum at another point (1e-6 relative in binary32).
     reference_rounding: the forward of a layer whose arithmetic is bf16 (both operands packed in that mode): follow the
     reference's all-bf16 evaluation (twice-rounded bf16 operands, residual product and bias add rounded to bf16): the
     pipelined kernel from 256 rows on, the decode-sized kernel below (shapes it does not take get exact products).
@@ -1163,7 +1165,8 @@ def _tiled_backward_pays(M: int, N: int, K: int, device_index: int) -> bool:
     for this one call: from about 2e11 flop on, with at least one 256 x 256 tile per compute unit, the faster GEMM more
     than pays for writing the expansions (8192 x 4096 x 14336: input gradient 858 -> 749 us with the weight's
     expansion cached, weight gradient 915 -> 835 us with both operands expanded; 4096 x 1536 x 8960: 134 -> 149 and
-    117 -> 141 us, so small products stay on the packed kernel).  Same bits either way."""
+    117 -> 141 us, so small products stay on the packed kernel).  Plain products keep their bits; with a low-rank term
+    the binary32 sums are taken in another order."""
     return (tiled_weight_copies and M >= 256 and N >= 256 and K % 32 == 0 and 2.0 * M * N * K >= 2e11
             and (M // 256) * (N // 256) >= _device_cus(device_index))
 

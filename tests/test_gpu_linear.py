@@ -834,3 +834,26 @@ def test_large_backward_products_take_the_pipelined_kernel_with_the_same_bits(mo
     assert torch.equal(gx, gx_p) and torch.equal(gw, gw_p)
     ref = dy.double() @ w.double()
     assert rel_fro(gx.double().cpu(), ref.cpu()) <= 0.2                     # FP4 operands: a coarse sanity bound on the product itself
+
+
+def test_large_products_with_rank_r_operands_and_binary32_bias_on_either_kernel():
+    """The size criterion also sends gradient products that carry a low-rank term (t, u) and the mean mode's binary32
+    bias to the pipelined kernel.  Same products as the packed kernel; the low-rank term joins the binary32 sum at
+    another point, so the results agree to binary32 rounding of the sums rather than bit for bit."""
+    from metis_hip import ops
+    g = torch.Generator().manual_seed(77)
+    M, N, K, r = 4096, 4352, 8192, 32
+    a = ops.quantize(torch.randn(M, K, generator=g).bfloat16().cuda())
+    b = ops.quantize((torch.randn(N, K, generator=g) * 0.02).bfloat16().cuda())
+    t = torch.randn(M, r, generator=g).bfloat16().cuda()
+    u = torch.randn(N, r, generator=g).bfloat16().cuda()
+    bias = torch.randn(N, generator=g).cuda()
+    assert ops._tiled_backward_pays(M, N, K, 0)
+    for out_dtype, tol in ((torch.float32, 1e-6), (torch.bfloat16, 2e-4)):
+        auto = ops.linear_fwd(a, b, t=t, u=u, bias=bias, out_dtype=out_dtype)
+        packed = ops.linear_fwd(a, b, t=t, u=u, bias=bias, out_dtype=out_dtype, tiled=False)
+        forced = ops.linear_fwd(a, b, t=t, u=u, bias=bias, out_dtype=out_dtype, tiled=True)
+        torch.cuda.synchronize()
+        assert torch.equal(auto, forced), out_dtype                   # the criterion picked the pipelined kernel
+        err = (auto.float() - packed.float()).norm() / packed.float().norm()
+        assert err <= tol, (out_dtype, float(err))
