@@ -389,6 +389,22 @@ int metis_nvfp4_decode_operand_deferred(const void* codes, const void* deferred,
     return skinny_operand_deferred(codes, deferred, rows, cols, quant_mode, mode, center, unit, out, (hipStream_t)stream);
 }
 
+int metis_decode_quant_project_deferred(const void* x, int64_t rows, int64_t cols, int mode, void* codes, void* deferred,
+                                        size_t deferred_bytes, const void* v, int64_t R, void* workspace, size_t workspace_bytes,
+                                        void* stream)
+{
+    return quantize_row_deferred_partial(x, rows, cols, mode, codes, deferred, deferred_bytes, v, R, workspace, workspace_bytes,
+                                         (hipStream_t)stream);
+}
+
+int metis_decode_prepare_deferred(const void* x, int64_t ldx, const void* v, int64_t R, const void* s, void* xv, void* t,
+                                  void* workspace, size_t workspace_bytes, const void* codes, const void* deferred, int64_t rows,
+                                  int64_t cols, int quant_mode, int mode, const void* center, float* unit, void* out, void* stream)
+{
+    return decode_prepare_deferred(x, ldx, v, R, s, xv, t, workspace, workspace_bytes, codes, deferred, rows, cols, quant_mode, mode,
+                                   center, unit, out, (hipStream_t)stream);
+}
+
 int metis_linear_fwd_grouped_operand(const void* a_operand, const float* a_unit, int64_t M, int64_t K,
                                      const metis_linear_member* members, int count, int out_dtype, int mode, void* workspace,
                                      size_t workspace_bytes, void* stream)

@@ -15,6 +15,7 @@
 // The low-rank operands stay bf16 and use v_mfma_f32_32x32x16_bf16 on the same accumulators.
 #include "gemm_common.h"
 #include "nvfp4_encode.h"
+#include "lowrank_small_steps.h"
 #include <stdlib.h>
 #include <type_traits>
 
@@ -940,12 +941,13 @@ int decode_weight(const void* codes, const void* scales, int64_t N, int64_t K, v
 // column) its me + QDQ(x - me) rounded to bf16 once more (src/Metis/Metis/bitlinear.py:330-333 in bf16 arithmetic).
 // DEF: the quantizer call deferred its scale bytes (nvfp4_quant.hip): `scales` holds bf16 block maxima, `partials` the
 // partial tensor maxima; unit (written to unit_out) and E4M3 bytes are formed here, in the arithmetic of that call (QMODE).
-template <int PB16, int DEF = 0, int QMODE = 0>
-__global__ __launch_bounds__(256) void skinny_operand_kernel(const uint32_t* __restrict__ codes, const uint8_t* __restrict__ scales,
-                                                             const float* __restrict__ unit_p, const uint16_t* __restrict__ center,
-                                                             int M, int K, int tiles, uint4* __restrict__ out,
-                                                             const uint32_t* __restrict__ partials = nullptr,
-                                                             float* __restrict__ unit_out = nullptr)
+// (block `block` of `nblocks`: a launch may give its first blocks to other work)
+template <int PB16, int DEF, int QMODE>
+__device__ __forceinline__ void skinny_operand_block(int block, int nblocks, const uint32_t* __restrict__ codes,
+                                                     const uint8_t* __restrict__ scales, const float* __restrict__ unit_p,
+                                                     const uint16_t* __restrict__ center, int M, int K, int tiles,
+                                                     uint4* __restrict__ out, const uint32_t* __restrict__ partials,
+                                                     float* __restrict__ unit_out)
 {
     typedef float float2_t __attribute__((ext_vector_type(2)));
     const int iters = K / 256;
@@ -953,12 +955,12 @@ __global__ __launch_bounds__(256) void skinny_operand_kernel(const uint32_t* __r
     float unit = 0.0f;
     if constexpr (DEF != 0) {
         unit = tensor_unit_of<QMODE>(fold_partial_maxima(partials));
-        if (blockIdx.x == 0 && threadIdx.x == 0) *unit_out = unit;
+        if (block == 0 && threadIdx.x == 0) *unit_out = unit;
     } else if constexpr (PB16 != 0) {
         unit = *unit_p;
     }
     const uint16_t* __restrict__ maxima = reinterpret_cast<const uint16_t*>(scales);
-    for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
+    for (int64_t idx = (int64_t)block * 256 + threadIdx.x; idx < total; idx += (int64_t)nblocks * 256) {
         const int lane = (int)(idx & 63), m = (int)((idx >> 6) & 15);
         const int64_t ti = idx >> 10;
         const int it = (int)(ti % iters), tile = (int)(ti / iters);
@@ -989,6 +991,36 @@ __global__ __launch_bounds__(256) void skinny_operand_kernel(const uint32_t* __r
         }
         out[idx] = v;
     }
+}
+
+template <int PB16, int DEF = 0, int QMODE = 0>
+__global__ __launch_bounds__(256) void skinny_operand_kernel(const uint32_t* __restrict__ codes, const uint8_t* __restrict__ scales,
+                                                             const float* __restrict__ unit_p, const uint16_t* __restrict__ center,
+                                                             int M, int K, int tiles, uint4* __restrict__ out,
+                                                             const uint32_t* __restrict__ partials = nullptr,
+                                                             float* __restrict__ unit_out = nullptr)
+{
+    skinny_operand_block<PB16, DEF, QMODE>((int)blockIdx.x, (int)gridDim.x, codes, scales, unit_p, center, M, K, tiles, out, partials,
+                                           unit_out);
+}
+
+// One launch for the two small independent steps between a decode-sized layer's quantizer and its GEMM: the first
+// `finish_blocks` blocks finish the rank-r projection (lowrank_small_steps.h), the others build the activation's
+// operands from a tensor whose quantizer call deferred its scale bytes.
+template <int PB16, int QMODE>
+__global__ __launch_bounds__(256) void decode_prepare_kernel(int finish_blocks, const float* __restrict__ lr_ws, int chunks, int MR, int R,
+                                                             const uint16_t* __restrict__ s, uint16_t* __restrict__ xv,
+                                                             uint16_t* __restrict__ t, const uint32_t* __restrict__ codes,
+                                                             const uint8_t* __restrict__ maxima, const uint16_t* __restrict__ center,
+                                                             int M, int K, int tiles, uint4* __restrict__ out,
+                                                             const uint32_t* __restrict__ partials, float* __restrict__ unit_out)
+{
+    if ((int)blockIdx.x < finish_blocks) {
+        lowrank_small_finish_block((int)blockIdx.x, lr_ws, chunks, MR, R, s, xv, t);
+        return;
+    }
+    skinny_operand_block<PB16, 1, QMODE>((int)blockIdx.x - finish_blocks, (int)gridDim.x - finish_blocks, codes, maxima, nullptr, center,
+                                         M, K, tiles, out, partials, unit_out);
 }
 
 size_t skinny_operand_bytes(int64_t M, int64_t K)
@@ -1036,6 +1068,45 @@ int skinny_operand_deferred(const void* codes, const void* deferred, int64_t M, 
     if (mode == METIS_MODE_PB16) { if (qmode) METIS_SOD(1, 1); else METIS_SOD(1, 0); }
     else { if (qmode) METIS_SOD(0, 1); else METIS_SOD(0, 0); }
 #undef METIS_SOD
+    return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
+}
+
+// lowrank_small + skinny_operand_deferred on the same activation (x [M, K] bf16 and its packed form) in two launches
+// instead of three: partial sums of the projection, then one launch that finishes it and builds the operands.
+// x = nullptr: the first of the two already ran beside the quantizer (quantize_row_deferred_partial): one launch.
+int decode_prepare_deferred(const void* x, int64_t ldx, const void* v, int64_t R, const void* s, void* xv, void* t, void* workspace,
+                            size_t workspace_bytes, const void* codes, const void* deferred, int64_t M, int64_t K, int qmode, int mode,
+                            const void* center, float* unit_out, void* out, hipStream_t st)
+{
+    if (mode == METIS_MODE_P32_F32) mode = METIS_MODE_P32;
+    if ((mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) || (qmode != METIS_MODE_P32 && qmode != METIS_MODE_PB16)) return METIS_E_ARG;
+    if (M <= 0 || M >= 256 || K <= 0 || K % 256 || K > INT32_MAX) return METIS_E_SHAPE;
+    if (!codes || !unit_out || !out || ((uintptr_t)codes % 4) || ((uintptr_t)out % 16) || ((uintptr_t)center % 16)) return METIS_E_ARG;
+    if (center && mode != METIS_MODE_PB16) return METIS_E_ARG;
+    Workspace ws;
+    if (const int rc = carve_deferred(const_cast<void*>(deferred), deferred_bytes(M, K), M, K, &ws)) return rc;
+    int chunks = 0;
+    if (x) {
+        if (const int rc = lowrank_small_partial(x, ldx, v, M, R, K, s, xv, t, workspace, workspace_bytes, st, &chunks)) return rc;
+    } else {
+        // the partial sums are in the workspace already (quantize_row_deferred_partial on the same shapes)
+        if (R <= 0 || R % 32 || R > 128) return METIS_E_SHAPE;
+        if (!xv || (t && !s) || ((uintptr_t)xv % 8) || ((uintptr_t)t % 8) || ((uintptr_t)s % 2)) return METIS_E_ARG;
+        if (!workspace || ((uintptr_t)workspace % 16) || workspace_bytes < lowrank_small_workspace_bytes(M, R, K)) return METIS_E_WORKSPACE;
+        int kc;
+        chunks = lowrank_small_chunks(K, &kc);
+    }
+    const int fb = lowrank_small_finish_blocks(M, R);
+    const int tiles = (int)((M + 63) / 64) * 2;
+    const int64_t total = (int64_t)tiles * (K / 256) * 1024;
+    const int g = fb + (int)((total + 255) / 256);
+#define METIS_DP(P, Q) hipLaunchKernelGGL((decode_prepare_kernel<P, Q>), dim3(g), dim3(256), 0, st, fb, (const float*)workspace, chunks, \
+                                          (int)(M * R), (int)R, (const uint16_t*)s, (uint16_t*)xv, (uint16_t*)t, (const uint32_t*)codes, \
+                                          (const uint8_t*)ws.amax, (const uint16_t*)center, (int)M, (int)K, tiles, (uint4*)out, \
+                                          (const uint32_t*)ws.gmax, unit_out)
+    if (mode == METIS_MODE_PB16) { if (qmode) METIS_DP(1, 1); else METIS_DP(1, 0); }
+    else { if (qmode) METIS_DP(0, 1); else METIS_DP(0, 0); }
+#undef METIS_DP
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 

@@ -137,6 +137,14 @@ int skinny_operand(const void* codes, const void* scales, const float* unit, int
 // the same from a tensor whose quantizer call deferred its scale bytes; writes the unit
 int skinny_operand_deferred(const void* codes, const void* deferred, int64_t M, int64_t K, int qmode, int mode, const void* center,
                             float* unit_out, void* out, hipStream_t st);
+// quantize_row_deferred of a decode-sized activation with the projection's first step in the same launch; nvfp4_quant.hip
+int quantize_row_deferred_partial(const void* x, int64_t rows, int64_t cols, int mode, void* codes, void* deferred, size_t bytes,
+                                  const void* v, int64_t R, void* lr_workspace, size_t lr_workspace_bytes, hipStream_t st);
+// the decode-sized rank-r projection (lowrank_small) and skinny_operand_deferred of the same activation, the
+// projection's finishing step inside the operand launch
+int decode_prepare_deferred(const void* x, int64_t ldx, const void* v, int64_t R, const void* s, void* xv, void* t, void* workspace,
+                            size_t workspace_bytes, const void* codes, const void* deferred, int64_t M, int64_t K, int qmode, int mode,
+                            const void* center, float* unit_out, void* out, hipStream_t st);
 int gemm_grouped_center_supported(int64_t M, int64_t K, const GemmMember* members, int count, int have_workspace);
 // bytes of split-K scratch a grouped call can use (only the N fields of the members are read; 0: it would not split)
 size_t gemm_grouped_workspace_bytes(int64_t M, int64_t K, const GemmMember* members, int count);
@@ -159,6 +167,12 @@ int column_mean(const void* x, int64_t rows, int64_t cols, int64_t ld, int in_f3
 size_t lowrank_small_workspace_bytes(int64_t M, int64_t R, int64_t K);
 int lowrank_small(const void* x, int64_t ldx, const void* v, int64_t M, int64_t R, int64_t K, const void* s, void* xv, void* t,
                   void* workspace, size_t workspace_bytes, hipStream_t st);
+
+// the same in two steps, for a caller whose next launch carries the finishing step in its first
+// lowrank_small_finish_blocks(M, R) blocks (lowrank_small_steps.h)
+int lowrank_small_partial(const void* x, int64_t ldx, const void* v, int64_t M, int64_t R, int64_t K, const void* s, void* xv, void* t,
+                          void* workspace, size_t workspace_bytes, hipStream_t st, int* chunks_out);
+inline int lowrank_small_finish_blocks(int64_t M, int64_t R) { return (int)((M * R / 4 + 63) / 64); }
 
 // gradient of the rank-r scale vector: column sums of the bf16 products of two [L, R] tensors; lowrank_small.hip
 int scale_grad(const void* g, const void* xv, int64_t L, int64_t R, void* out, int out_dtype, hipStream_t st);

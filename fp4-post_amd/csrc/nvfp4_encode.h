@@ -395,14 +395,19 @@ __device__ __forceinline__ void hadamard16_inverse(float (&v)[kBlock], uint32_t 
 
 // publish the workgroup's maximum block-maximum (non-negative floats order like their bit patterns).
 // fill_to: entries gridDim.x .. fill_to-1 are cleared as well, for readers that always fold a fixed number of entries.
-__device__ __forceinline__ void publish_group_max(float m, uint32_t* ws_gmax, uint32_t fill_to = 0)
+// (block, grid: the workgroup's index among the `grid` workgroups that publish, when that is not the whole launch)
+__device__ __forceinline__ void publish_group_max(float m, uint32_t* ws_gmax, uint32_t fill_to, uint32_t block, uint32_t grid)
 {
     __shared__ float smax[4];
     m = wave_max(m);
     if ((threadIdx.x & 63) == 0) smax[threadIdx.x >> 6] = m;
     __syncthreads();
-    if (threadIdx.x == 0) ws_gmax[blockIdx.x] = __float_as_uint(fmaxf(fmaxf(smax[0], smax[1]), fmaxf(smax[2], smax[3])));
-    for (uint32_t j = gridDim.x + blockIdx.x * 256u + threadIdx.x; j < fill_to; j += gridDim.x * 256u) ws_gmax[j] = 0u;
+    if (threadIdx.x == 0) ws_gmax[block] = __float_as_uint(fmaxf(fmaxf(smax[0], smax[1]), fmaxf(smax[2], smax[3])));
+    for (uint32_t j = grid + block * 256u + threadIdx.x; j < fill_to; j += grid * 256u) ws_gmax[j] = 0u;
+}
+__device__ __forceinline__ void publish_group_max(float m, uint32_t* ws_gmax, uint32_t fill_to = 0)
+{
+    publish_group_max(m, ws_gmax, fill_to, blockIdx.x, gridDim.x);
 }
 
 // Deferred scale bytes: a quantizer call may stop after phase 1 and hand its parked bf16 block maxima and its partial

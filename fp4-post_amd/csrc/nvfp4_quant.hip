@@ -12,6 +12,7 @@
 #include "metis_device.h"
 #include "metis_host.h"
 #include "nvfp4_encode.h"
+#include "lowrank_small_steps.h"
 #include <atomic>
 #include <stdio.h>
 #include <stdlib.h>
@@ -51,15 +52,16 @@ template <int MODE> __device__ __forceinline__ uint2 encode_row_block(const floa
     }
 }
 
-template <int MODE, int DEPTH = 1>
-__global__ __launch_bounds__(256) void quant_codes_contig_kernel(const uint4* __restrict__ x, uint2* __restrict__ codes,
-                                                                 uint16_t* __restrict__ ws_amax, uint32_t* __restrict__ ws_gmax,
-                                                                 uint32_t nblocks, uint32_t fill_to)
+// (workgroup `block` of `grid`: a launch may give other blocks to other work)
+template <int MODE, int DEPTH>
+__device__ __forceinline__ void quant_codes_contig_block(uint32_t block, uint32_t grid, const uint4* __restrict__ x,
+                                                         uint2* __restrict__ codes, uint16_t* __restrict__ ws_amax,
+                                                         uint32_t* __restrict__ ws_gmax, uint32_t nblocks, uint32_t fill_to)
 {
     __shared__ uint32_t table[MODE == 0 ? kQuotientTableWords : 4];
     float gmax = 0.0f;
-    const uint32_t step = gridDim.x * 256u;
-    uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t step = grid * 256u;
+    uint32_t i = block * 256u + threadIdx.x;
     uint4 c0[DEPTH], c1[DEPTH];
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
@@ -83,7 +85,33 @@ __global__ __launch_bounds__(256) void quant_codes_contig_kernel(const uint4* __
         __builtin_nontemporal_store((metis_u32x2_t){cw.x, cw.y}, reinterpret_cast<metis_u32x2_t*>(codes) + i);
         i += step;
     }
-    publish_group_max(gmax, ws_gmax, fill_to);
+    publish_group_max(gmax, ws_gmax, fill_to, block, grid);
+}
+
+template <int MODE, int DEPTH = 1>
+__global__ __launch_bounds__(256) void quant_codes_contig_kernel(const uint4* __restrict__ x, uint2* __restrict__ codes,
+                                                                 uint16_t* __restrict__ ws_amax, uint32_t* __restrict__ ws_gmax,
+                                                                 uint32_t nblocks, uint32_t fill_to)
+{
+    quant_codes_contig_block<MODE, DEPTH>(blockIdx.x, gridDim.x, x, codes, ws_amax, ws_gmax, nblocks, fill_to);
+}
+
+// A decode-sized activation's quantizer (scale bytes deferred) and the first step of its rank-r projection
+// (lowrank_small_steps.h) in one launch: both only read x.  Blocks 0 .. qgrid-1 quantize, the others take one K chunk of
+// 64 rows each (R <= 128: four waves cover the columns).
+template <int MODE>
+__global__ __launch_bounds__(256) void decode_quant_partial_kernel(uint32_t qgrid, const uint4* __restrict__ x, uint2* __restrict__ codes,
+                                                                   uint16_t* __restrict__ ws_amax, uint32_t* __restrict__ ws_gmax,
+                                                                   uint32_t nblocks, uint32_t fill_to, int64_t ldx,
+                                                                   const uint16_t* __restrict__ v, int M, int R, int K, int kc, int chunks,
+                                                                   float* __restrict__ lr_ws)
+{
+    if (blockIdx.x < qgrid) {
+        quant_codes_contig_block<MODE, 1>(blockIdx.x, qgrid, x, codes, ws_amax, ws_gmax, nblocks, fill_to);
+        return;
+    }
+    const int b = (int)(blockIdx.x - qgrid);
+    lowrank_small_partial_block(b % chunks, b / chunks, reinterpret_cast<const uint16_t*>(x), ldx, v, M, R, K, kc, lr_ws);
 }
 
 // The same loop with a centre subtracted first (mean mode, src/Metis/Metis/bitlinear.py:311-336: the tensor that is
@@ -1261,6 +1289,33 @@ int quantize_row_deferred(const void* x, int64_t rows, int64_t cols, int mode, c
         launch_contig<0>(x, codes, ws, nblocks, kDeferredPartials, g1, st);
     else
         launch_contig<1>(x, codes, ws, nblocks, kDeferredPartials, g1, st);
+    return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
+}
+
+// quantize_row_deferred of a decode-sized contiguous bf16 activation and, in the same launch, the first step of its
+// rank-r projection onto v [R, cols]: partial sums per K chunk into lr_workspace (lowrank_small's workspace), for a
+// finishing step that runs later (decode_prepare_deferred with x = nullptr).
+int quantize_row_deferred_partial(const void* x, int64_t rows, int64_t cols, int mode, void* codes, void* deferred, size_t bytes,
+                                  const void* v, int64_t R, void* lr_workspace, size_t lr_workspace_bytes, hipStream_t st)
+{
+    if (rows < 0 || cols < 0 || R <= 0) return METIS_E_ARG;
+    if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) return METIS_E_ARG;
+    if (rows == 0 || rows >= 256 || cols == 0 || cols % 64 || R % 32 || R > 128) return METIS_E_SHAPE;
+    if (!x || !codes || !v || ((uintptr_t)x % 16) || ((uintptr_t)codes % 8) || ((uintptr_t)v % 16)) return METIS_E_ARG;
+    if (!lr_workspace || ((uintptr_t)lr_workspace % 16) || lr_workspace_bytes < lowrank_small_workspace_bytes(rows, R, cols))
+        return METIS_E_WORKSPACE;
+    Workspace ws;
+    if (const int rc = carve_deferred(deferred, bytes, rows, cols, &ws)) return rc;
+    const uint32_t nblocks = (uint32_t)(rows * cols / kBlock);
+    const int g1 = deferred_grid(nblocks, kContigPerCu);
+    int kc;
+    const int chunks = lowrank_small_chunks(cols, &kc);
+    const int g = g1 + chunks * (int)((rows + 63) / 64);
+#define METIS_QP(MODE) hipLaunchKernelGGL((decode_quant_partial_kernel<MODE>), dim3(g), dim3(256), 0, st, (uint32_t)g1, (const uint4*)x, \
+                                          (uint2*)codes, ws.amax, ws.gmax, nblocks, kDeferredPartials, cols, (const uint16_t*)v, \
+                                          (int)rows, (int)R, (int)cols, kc, chunks, (float*)lr_workspace)
+    if (mode == 0) METIS_QP(0); else METIS_QP(1);
+#undef METIS_QP
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 

@@ -742,13 +742,27 @@ class _MetisFusedFunction(torch.autograd.Function):
     """y = ((x V^T) * s) U^T + deq(Q(x)) deq(Q(R))^T + b in one GEMM launch, with its gradients."""
 
     @staticmethod
-    def forward(ctx, x, v, s, u, res, bias, px, p_res, xv=None, t=None):
+    def forward(ctx, x, v, s, u, res, bias, px, p_res, xv=None, t=None, pending=None):
         F = LinearLowbitFunction
         cd = torch.bfloat16
-        if xv is None:
+        aop = None
+        if pending is not None:
+            # the quantizer's launch left the projection's partial sums (BitLinear._quantize_and_project)
+            xv, t, aop = ops.project_and_operand(_flat2d(x).to(cd), v.to(cd), s.to(cd), px, ops.MODE_PB16, None, pending=pending)
+        elif xv is None:
             # [L, r] rank-r projection and its product with s (bf16) on the library's kernels (split-K below 256 rows,
             # one pass over x from there on); the caller has it already when the quantizer's pass produced it
-            xv, t = ops.lowrank_project(_flat2d(x).to(cd), v.to(cd), s.to(cd))
+            x2, vb, sb = _flat2d(x).to(cd), v.to(cd), s.to(cd)
+            in_operand = isinstance(px, CenteredNVFP4) and F._mean_in_operand(px, p_res)
+            target = px.residual if in_operand else px
+            if ((in_operand or (isinstance(px, PackedNVFP4) and F.reference_rounding)) and p_res.rht is None
+                    and ops.grouped_operand_applies(target, [p_res], [vb.shape[0]], px.mean if in_operand else None, True)
+                    and ops.project_and_operand_applies(x2, vb, sb, target)):
+                # decode-sized call in bf16 arithmetic: the projection's finishing step and the activation's GEMM
+                # operands in one launch
+                xv, t, aop = ops.project_and_operand(x2, vb, sb, target, ops.MODE_PB16, px.mean if in_operand else None)
+            else:
+                xv, t = ops.lowrank_project(x2, vb, sb)
         out_dtype = torch.float32 if F.compute_dtype == torch.float32 else torch.bfloat16
         ctx.center = None
         # binary32 arithmetic keeps a binary32 bias (as LinearLowbit and the centred path do); bf16 arithmetic adds it in bf16
@@ -759,7 +773,7 @@ class _MetisFusedFunction(torch.autograd.Function):
             if F._mean_in_operand(px, p_res):
                 # bf16 arithmetic: the activation operand is the reference's bf16 tensor me + QDQ(x - me)
                 y = ops.linear_fwd_grouped(px.residual, [(p_res, t, u.to(cd), gemm_bias)], out_dtype=out_dtype, center=px.mean,
-                                           reference_rounding=True)[0]
+                                           reference_rounding=True, a_operand=aop)[0]
             elif px.rows < 256:
                 # decode-sized: W^ me is accumulated inside the GEMM launch
                 y = ops.linear_fwd_grouped(px.residual, [(p_res, t, u.to(cd), None if bias is None else bias.float())],
@@ -771,7 +785,7 @@ class _MetisFusedFunction(torch.autograd.Function):
                                    out_dtype=out_dtype)
         else:
             y = ops.linear_fwd(px, p_res, t=t, u=u.to(cd), bias=gemm_bias, out_dtype=out_dtype,
-                               reference_rounding=F.reference_rounding)
+                               reference_rounding=F.reference_rounding, a_operand=aop)
         ctx.save_for_backward(x, v, s, u, res, xv, t)               # t = bf16(xv * s): [L, r], kept for the gradient of U
         ctx.p_res = p_res
         ctx.has_bias = bias is not None
@@ -845,7 +859,7 @@ class _MetisFusedFunction(torch.autograd.Function):
             g_res = torch.matmul(dyq.T, xq).to(torch.float32)
         g_b = _token_sum(dy2, torch.float32) if ctx.has_bias else None
         return (gx.reshape(x.shape).to(x.dtype), g_v.to(v.dtype), g_s.to(s.dtype), g_u.to(u.dtype),
-                g_res, g_b, None, None, None, None)
+                g_res, g_b, None, None, None, None, None)
 
 
 class BitLinear(nn.Module):
@@ -1022,7 +1036,8 @@ class BitLinear(nn.Module):
     def _quantize_and_project(self, x: torch.Tensor):
         """(packed activation, x V^T, bf16((x V^T) s)) from one pass over an activation that no sibling shares (direct
         mode, round to nearest, bf16 tensor of 256 rows or more), or None: both branches of the layer read x, the
-        residual branch through the quantizer and the rank-r branch as it is."""
+        residual branch through the quantizer and the rank-r branch as it is.  A decode-sized activation in bf16
+        arithmetic gives (packed activation, None, None, pending partial sums of the projection)."""
         F = LinearLowbitFunction
         if (F.enable_activation_svd or F.enable_nv_recipe or F.q_forward_input is not Cast2NVFp4e2m1BlockNOSR
                 or not x.is_cuda or x.dtype != torch.bfloat16 or F.compute_dtype not in (torch.float32, torch.bfloat16)):
@@ -1032,9 +1047,21 @@ class BitLinear(nn.Module):
         if v.dtype != torch.bfloat16 or self._packed_residual() is None:
             return None
         mode = ops.MODE_P32 if F.compute_dtype == torch.float32 else ops.MODE_PB16
-        if not ops.quantize_project_applies(x2, v, mode):
-            return None
-        return ops.quantize_project(x2, v.detach(), self.s.detach(), mode)
+        if ops.quantize_project_applies(x2, v, mode):
+            return ops.quantize_project(x2, v.detach(), self.s.detach(), mode)
+        # decode-sized call in bf16 arithmetic: the quantizer's launch carries the projection's first step, and the launch
+        # that builds the GEMM's activation operands its finishing step
+        p_res = self._packed_residual()
+        if (mode == ops.MODE_PB16 and F.reference_rounding and p_res.rht is None
+                and self.s.dtype == torch.bfloat16 and ops.quantize_project_decode_applies(x2, v, mode)
+                and x2.shape[0] * x2.shape[1] > 0):
+            px, pending = ops.quantize_project_decode(x2, v.detach(), mode)
+            if ops.grouped_operand_applies(px, [p_res], [v.shape[0]], None, True):
+                return px, None, None, pending
+            # (a weight the decode-sized kernel does not take: finish the projection on its own)
+            xv, t, _ = ops.project_and_operand(x2, v.detach(), self.s.detach(), px, mode, None, pending=pending)
+            return px, xv, t
+        return None
 
     def _forward_group(self, x: torch.Tensor, shared_input):
         """All members of this layer's projection group on the shared activation in one call (no autograd):
@@ -1058,11 +1085,17 @@ class BitLinear(nn.Module):
             cached = (key, torch.cat([m.vlinear.weight.to(cd) for m in members], dim=0),
                       torch.cat([m.s.to(cd) for m in members], dim=0))
             group["stacked_v"] = cached
-        _, t_all = ops.lowrank_project(x2, cached[1], cached[2])
         centre = shared_input.center32 if isinstance(shared_input, CenteredNVFP4) else None
         px = shared_input.residual if centre is not None else shared_input
         if centre is not None and all(F._mean_in_operand(shared_input, p) for p in packed):
             centre = shared_input.mean                             # bf16: goes into the activation operand (reference's bf16 tensor)
+        aop = None
+        if (ops.grouped_operand_applies(px, packed, [m.args.forward_svd_rank for m in members], centre, F.reference_rounding)
+                and ops.project_and_operand_applies(x2, cached[1], cached[2], px)):
+            # the projection's finishing step and the activation's GEMM operands in one launch
+            _, t_all, aop = ops.project_and_operand(x2, cached[1], cached[2], px, ops.MODE_PB16, centre)
+        else:
+            _, t_all = ops.lowrank_project(x2, cached[1], cached[2])
         calls, c0 = [], 0
         for m, p_res in zip(members, packed):
             r = m.args.forward_svd_rank
@@ -1073,7 +1106,8 @@ class BitLinear(nn.Module):
             c0 += r
         out_dtype = torch.float32 if F.compute_dtype == torch.float32 else torch.bfloat16
         # mean mode: every member also receives W^ me, inside the same launch (binary32)
-        outs = ops.linear_fwd_grouped(px, calls, out_dtype=out_dtype, center=centre, reference_rounding=F.reference_rounding)
+        outs = ops.linear_fwd_grouped(px, calls, out_dtype=out_dtype, center=centre, reference_rounding=F.reference_rounding,
+                                      a_operand=aop)
         lead = x.shape[:-1]
         return {id(m): y.reshape(*lead, y.shape[-1]).to(F.compute_dtype) for m, y in zip(members, outs)}
 

@@ -641,6 +641,66 @@ def decode_operand(p: PackedNVFP4, mode: int = MODE_P32, center: torch.Tensor | 
     return out
 
 
+def grouped_operand_applies(a: PackedNVFP4, weights, ranks, center: torch.Tensor | None, reference_rounding: bool) -> bool:
+    """Whether linear_fwd_grouped(a, members, center=center, reference_rounding=...) reads the activation as ready
+    operands (decode_operand): bf16 arithmetic on every tensor, decode-sized shapes in wide runs.  weights: the
+    members' packed weights, ranks: the widths of their low-rank terms (0 without)."""
+    M, K = a.rows, a.cols
+    return bool(reference_rounding and (center is None or center.dtype == torch.bfloat16) and a.mode == MODE_PB16
+                and all(b.mode == MODE_PB16 for b in weights) and len(weights) <= 4 and K % 256 == 0
+                and all(_decode_kernel_takes(M, b.rows, K, r) for b, r in zip(weights, ranks))
+                and all(b.scales.data_ptr() % 8 == 0 for b in weights))
+
+
+def project_and_operand_applies(x2: torch.Tensor, v: torch.Tensor, s: torch.Tensor, p: PackedNVFP4) -> bool:
+    """project_and_operand takes these: the decode-sized domain of lowrank_project (with s), and a packed form of the
+    same shape whose quantizer call deferred its scale bytes, never materialized since."""
+    M, K = x2.shape
+    R = v.shape[0]
+    d = p.__dict__
+    return bool(x2.is_cuda and x2.dtype == torch.bfloat16 and v.dtype == torch.bfloat16 and s.dtype == torch.bfloat16
+                and 0 < M < 256 and K % 256 == 0 and v.shape[1] == K and R % 32 == 0 and 0 < R <= 256 and s.numel() == R
+                and x2.stride(1) == 1 and x2.stride(0) % 8 == 0 and x2.data_ptr() % 16 == 0
+                and p.rows == M and p.cols == K and p.rht is None
+                and d.get("deferred") is not None and d.get("_scales") is None)
+
+
+def project_and_operand(x2: torch.Tensor, v: torch.Tensor, s: torch.Tensor, p: PackedNVFP4, mode: int = MODE_PB16,
+                        center: torch.Tensor | None = None, pending: torch.Tensor | None = None):
+    """(xv, t, operand) = lowrank_project(x2, v, s) and decode_operand(p, mode, center) of one decode-sized activation
+    in two launches instead of three: the projection's finishing step rides in the operand launch.  Same bits.
+    pending: the projection's partial sums as quantize_project_decode left them (the first of the two launches already
+    ran beside the quantizer): one launch."""
+    if not project_and_operand_applies(x2, v, s, p):
+        raise ValueError("project_and_operand: outside the call's domain (see project_and_operand_applies)")
+    M, K = x2.shape
+    R = v.shape[0]
+    L = load()
+    dev = x2.device
+    v = v.contiguous()
+    s = s.contiguous()
+    if center is not None:
+        center = center.reshape(-1).to(torch.bfloat16).contiguous()
+        if center.numel() != K:
+            raise ValueError(f"center must have {K} values, got {center.numel()}")
+    xv = torch.empty(M, R, dtype=torch.bfloat16, device=dev)
+    t = torch.empty_like(xv)
+    out = torch.empty(L.metis_nvfp4_decode_operand_bytes(M, K), dtype=torch.uint8, device=dev)
+    need = L.metis_lowrank_project_workspace_bytes(M, R, K)
+    if pending is not None and (pending.numel() < need or pending.device != dev or R > 128):
+        raise ValueError("project_and_operand: `pending` is not what quantize_project_decode returns for these shapes")
+    ws = pending if pending is not None else torch.empty(need, dtype=torch.uint8, device=dev)
+    d = p.__dict__
+    rc = L.metis_decode_prepare_deferred(None if pending is not None else x2.data_ptr(), x2.stride(0), v.data_ptr(), R, s.data_ptr(),
+                                         xv.data_ptr(), t.data_ptr(),
+                                         ws.data_ptr(), need, p.codes.data_ptr(), d["deferred"].data_ptr(), M, K, p.mode, mode,
+                                         None if center is None else center.data_ptr(), d["_unit"].data_ptr(), out.data_ptr(),
+                                         _stream())
+    check(rc, "metis_decode_prepare_deferred", (M, K, R))
+    d["_unit_ready"] = True
+    return xv, t, out
+
+
 def decode_weight(p: PackedNVFP4, cache: bool = True) -> torch.Tensor | None:
     """The packed weight in the decode layout (same 0.5625 B per element): rows in tiles of 32, K in steps of 256, the
     pieces of a wave's 64 lanes side by side, so that the decode-sized kernel's loads cover whole lines.  None when
@@ -866,7 +926,7 @@ def _decode_kernel_takes(M: int, N: int, K: int, r: int) -> bool:
 def linear_fwd(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None, u: torch.Tensor | None = None,
                bias: torch.Tensor | None = None, out_dtype: torch.dtype = torch.bfloat16,
                expanded: bool | None = None, split_k: bool = True, tiled: bool | None = None,
-               reference_rounding: bool = False) -> torch.Tensor:
+               reference_rounding: bool = False, a_operand: torch.Tensor | None = None) -> torch.Tensor:
     """out[M, N] = deq(a)[M, K] . deq(b)[N, K]^T (+ t[M, r] . u[N, r]^T) (+ bias[N]).
 
     tiled=None picks the pipelined kernel on tiled binary16 expansions when b is a cached weight and the shape is
@@ -880,7 +940,8 @@ def linear_fwd(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None,
     split_k=False withholds the split-K workspace: the contraction then runs unsplit in one launch.
 
     expanded=True runs on cached exact f16 expansions of a and b (2 B/element extra HBM, inner loop of
-    MFMA + LDS reads only); the default works on the packed operands directly."""
+    MFMA + LDS reads only); the default works on the packed operands directly.
+    a_operand: as in linear_fwd_grouped (a decode-sized call in bf16 arithmetic)."""
     if a.cols != b.cols:
         raise ValueError(f"contraction mismatch: {a.cols} vs {b.cols}")
     if a.rht is not None or b.rht is not None:
@@ -896,7 +957,8 @@ def linear_fwd(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None,
         return linear_fwd_tiled(a, b, t=t, u=u, bias=bias, out_dtype=out_dtype, reference_rounding=faithful, split_k=split_k)
     M, N, K = a.rows, b.rows, a.cols
     if rounded and not expanded and _decode_kernel_takes(M, N, K, 0 if t is None else t.shape[1]):
-        return _linear_fwd_grouped(a, [(b, t, u, bias)], out_dtype=out_dtype, split_k=split_k, reference_rounding=True)[0]
+        return _linear_fwd_grouped(a, [(b, t, u, bias)], out_dtype=out_dtype, split_k=split_k, reference_rounding=True,
+                                   a_operand=a_operand)[0]
     dev = a.codes.device
     r = 0
     if t is not None:
@@ -1011,6 +1073,37 @@ def quantize_project(x2: torch.Tensor, v: torch.Tensor, s: torch.Tensor, mode: i
     return PackedNVFP4(codes, None, unit, M, K, mode, deferred=parked), xv, t
 
 
+def quantize_project_decode_applies(x2: torch.Tensor, v: torch.Tensor, mode: int) -> bool:
+    """quantize_project_decode takes this activation: a contiguous bf16 [M, K] of fewer than 256 rows, K a multiple of
+    256 (what the consumer of the pending sums, project_and_operand, needs), a bf16 V of 32 to 128 rows."""
+    M, K = x2.shape
+    return bool(x2.is_cuda and x2.dtype == torch.bfloat16 and v.dtype == torch.bfloat16 and 0 < M < 256 and K % 256 == 0
+                and v.shape[0] % 32 == 0 and 0 < v.shape[0] <= 128 and v.shape[1] == K and x2.is_contiguous()
+                and x2.data_ptr() % 16 == 0 and mode in (MODE_P32, MODE_PB16))
+
+
+def quantize_project_decode(x2: torch.Tensor, v: torch.Tensor, mode: int = MODE_PB16):
+    """(quantize(x2, mode, deferred=True), pending) from ONE launch over a decode-sized activation: the packed tensor and
+    the partial sums of its rank-r projection x2 . v^T, which project_and_operand(..., pending=pending) finishes in the
+    launch that also builds the GEMM operands.  Same bits as the separate calls."""
+    if not quantize_project_decode_applies(x2, v, mode):
+        raise ValueError("quantize_project_decode: outside the call's domain (see quantize_project_decode_applies)")
+    M, K = x2.shape
+    R = v.shape[0]
+    dev = x2.device
+    L = load()
+    v = v.contiguous()
+    codes = torch.empty(M, K // 2, dtype=torch.uint8, device=dev)
+    unit = torch.empty(1, dtype=torch.float32, device=dev)
+    parked = torch.empty(L.metis_nvfp4_deferred_bytes(M, K), dtype=torch.uint8, device=dev)
+    need = L.metis_lowrank_project_workspace_bytes(M, R, K)
+    pending = torch.empty(need, dtype=torch.uint8, device=dev)
+    rc = L.metis_decode_quant_project_deferred(x2.data_ptr(), M, K, mode, codes.data_ptr(), parked.data_ptr(), parked.numel(),
+                                               v.data_ptr(), R, pending.data_ptr(), need, _stream())
+    check(rc, "metis_decode_quant_project_deferred", (M, K, R))
+    return PackedNVFP4(codes, None, unit, M, K, mode, deferred=parked), pending
+
+
 def lowrank_contract_tokens(a: torch.Tensor, b: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
                             transpose: bool = False) -> torch.Tensor:
     """sum_l a[l, C] b[l, R] -> [C, R] (or [R, C] with transpose): the rank-r products of the backward pass that
@@ -1054,13 +1147,13 @@ def lowrank_scale_grad(g: torch.Tensor, xv: torch.Tensor, out_dtype: torch.dtype
 
 def linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.bfloat16,
                        center: torch.Tensor | None = None, split_k: bool = True,
-                       reference_rounding: bool = False) -> list[torch.Tensor]:
-    return _linear_fwd_grouped(a, members, out_dtype, center, split_k, reference_rounding)
+                       reference_rounding: bool = False, a_operand: torch.Tensor | None = None) -> list[torch.Tensor]:
+    return _linear_fwd_grouped(a, members, out_dtype, center, split_k, reference_rounding, a_operand)
 
 
 def _linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.bfloat16,
                         center: torch.Tensor | None = None, split_k: bool = True,
-                        reference_rounding: bool = False) -> list[torch.Tensor]:
+                        reference_rounding: bool = False, a_operand: torch.Tensor | None = None) -> list[torch.Tensor]:
     """[linear_fwd(a, b, t=t, u=u, bias=bias) for (b, t, u, bias) in members] in one call: a projection group
     (q/k/v, gate/up) that shares one packed activation.  Decode-sized batches run as a single launch.
 
@@ -1070,7 +1163,10 @@ def _linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.
     exact products with the centre's share accumulated in binary32.
 
     center (mean mode: `a` packs the centred residual X - center): every output row also receives deq(b) . center,
-    inside the same launch where the shape allows, else through matvec and a binary32 bias."""
+    inside the same launch where the shape allows, else through matvec and a binary32 bias.
+
+    a_operand: decode_operand(a, MODE_PB16, center) when the caller has it already (project_and_operand); read only
+    where grouped_operand_applies says the call reads ready operands."""
     import ctypes
     M, K = a.rows, a.cols
     dev = a.codes.device
@@ -1078,7 +1174,8 @@ def _linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.
                and all(m[0].mode == MODE_PB16 for m in members))
     takes = len(members) <= 4 and all(_decode_kernel_takes(M, m[0].rows, K, 0 if m[1] is None else m[1].shape[1]) for m in members)
     # ready operands (built once for the group): wide runs only
-    operand = rounded and takes and K % 256 == 0 and all(m[0].scales.data_ptr() % 8 == 0 for m in members)
+    operand = grouped_operand_applies(a, [m[0] for m in members], [0 if m[1] is None else m[1].shape[1] for m in members],
+                                      center, reference_rounding)
     if rounded and center is not None and not operand:
         if M >= 256 and K % 32 == 0:
             ax = expand_tiled(a, cache=a.shared, mode=MODE_PB16, center=center)
@@ -1128,7 +1225,7 @@ def _linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.
     dt = DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16
     if operand:
         # (a quantizer call that deferred its scale bytes never gets them: the operand kernel forms them on the way)
-        aop = decode_operand(a, MODE_PB16, center)
+        aop = a_operand if a_operand is not None else decode_operand(a, MODE_PB16, center)
         rc = L.metis_linear_fwd_grouped_operand(aop.data_ptr(), a.unit.data_ptr(), M, K, ap, len(members), dt, MODE_PB16,
                                                 None if ws is None else ws.data_ptr(), need, _stream())
         check(rc, "metis_linear_fwd_grouped_operand", (M, K, [m[0].rows for m in members]))

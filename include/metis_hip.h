@@ -646,13 +646,36 @@ int metis_linear_fwd_grouped_bf16(const void *a_codes, const void *a_scales, con
  *   metis_nvfp4_decode_operand_deferred  the same from a tensor whose quantizer call deferred its scale bytes
  *                                (metis_nvfp4_quant_row_deferred: quant_mode = its mode): forms the E4M3 bytes itself and
  *                                writes the tensor unit (float [1], required), so a decode-sized activation costs two
- *                                launches ahead of its GEMMs instead of three */
+ *                                launches ahead of its GEMMs instead of three
+ *   metis_decode_prepare_deferred  metis_lowrank_project (x [rows, cols] bf16 with row stride ldx, v [R, cols], s, xv,
+ *                                t, workspace: its arguments and limits) and metis_nvfp4_decode_operand_deferred of
+ *                                the same activation (codes, deferred, quant_mode, mode, center, unit, out: its
+ *                                arguments and limits) in two launches instead of three: the projection's finishing
+ *                                step rides in the first blocks of the operand launch.  Same bits as the two calls
+ *                                (`vlinear(x)`, `torch.mul(self.s, y)` and the quantized input of BitLinear.forward,
+ *                                src/Metis/Metis/bitlinear.py:752-760).  x = NULL: the workspace already holds the
+ *                                projection's partial sums, left there by metis_decode_quant_project_deferred on the
+ *                                same rows, cols and R (R <= 128 then): one launch
+ *   metis_decode_quant_project_deferred  metis_nvfp4_quant_row_deferred (no centre; x contiguous bf16 [rows, cols],
+ *                                rows < 256, cols % 64 == 0) and, in the same launch, the first step of
+ *                                metis_lowrank_project on v [R, cols] (R % 32 == 0, R <= 128; METIS_E_SHAPE otherwise):
+ *                                its partial sums go to `workspace` (metis_lowrank_project_workspace_bytes(rows, R,
+ *                                cols) bytes, 16-byte aligned) and wait there for metis_decode_prepare_deferred with
+ *                                x = NULL.  Same bits as the separate calls: a decode-sized BitLinear.forward is then
+ *                                three launches (this, the prepare call, the GEMM) instead of five */
 size_t metis_nvfp4_decode_operand_bytes(int64_t rows, int64_t cols);
 int metis_nvfp4_decode_operand(const void *codes, const void *scales, const float *unit, int64_t rows,
                                int64_t cols, int mode, const void *center, void *out, void *stream);
 int metis_nvfp4_decode_operand_deferred(const void *codes, const void *deferred, int64_t rows, int64_t cols,
                                         int quant_mode, int mode, const void *center, float *unit, void *out,
                                         void *stream);
+int metis_decode_quant_project_deferred(const void *x, int64_t rows, int64_t cols, int mode, void *codes,
+                                        void *deferred, size_t deferred_bytes, const void *v, int64_t R,
+                                        void *workspace, size_t workspace_bytes, void *stream);
+int metis_decode_prepare_deferred(const void *x, int64_t ldx, const void *v, int64_t R, const void *s, void *xv,
+                                  void *t, void *workspace, size_t workspace_bytes, const void *codes,
+                                  const void *deferred, int64_t rows, int64_t cols, int quant_mode, int mode,
+                                  const void *center, float *unit, void *out, void *stream);
 int metis_linear_fwd_grouped_operand(const void *a_operand, const float *a_unit, int64_t M, int64_t K,
                                      const metis_linear_member *members, int count, int out_dtype, int mode,
                                      void *workspace, size_t workspace_bytes, void *stream);

@@ -857,3 +857,110 @@ def test_large_products_with_rank_r_operands_and_binary32_bias_on_either_kernel(
         assert torch.equal(auto, forced), out_dtype                   # the criterion picked the pipelined kernel
         err = (auto.float() - packed.float()).norm() / packed.float().norm()
         assert err <= tol, (out_dtype, float(err))
+
+
+@pytest.mark.parametrize("M,K,R", [(64, 3584, 192), (1, 256, 32), (200, 2048, 64), (255, 18944, 64), (33, 512, 256)])
+@pytest.mark.parametrize("mode,centred", [(1, False), (1, True), (0, False)])
+def test_projection_finish_and_operand_build_in_one_launch(M, K, R, mode, centred):
+    """metis_decode_prepare_deferred against metis_lowrank_project + metis_nvfp4_decode_operand_deferred on the same
+    activation: the same xv, t, operand bytes and tensor unit, bit for bit; and its argument checks."""
+    from metis_hip import ops
+    g = torch.Generator().manual_seed(M + K + R)
+    x = (torch.randn(M, K, generator=g) * 3).bfloat16().cuda()
+    v = (torch.randn(R, K, generator=g) * 0.05).bfloat16().cuda()
+    s = torch.rand(R, generator=g).bfloat16().cuda()
+    centre = (torch.randn(K, generator=g) * 0.1).bfloat16().cuda() if centred else None
+    want_xv, want_t = ops.lowrank_project(x, v, s)
+    p1 = ops.quantize(x, mode, deferred=True)
+    want_op = ops.decode_operand(p1, mode, centre)
+    p2 = ops.quantize(x, mode, deferred=True)
+    assert ops.project_and_operand_applies(x, v, s, p2)
+    xv, t, op = ops.project_and_operand(x, v, s, p2, mode, centre)
+    torch.cuda.synchronize()
+    assert torch.equal(xv, want_xv) and torch.equal(t, want_t)
+    assert torch.equal(op, want_op)
+    assert torch.equal(p2.unit, p1.unit)
+    # once its scale bytes exist the tensor no longer qualifies (the operand call for written bytes is another one)
+    p1.scales
+    assert not ops.project_and_operand_applies(x, v, s, p1)
+    with pytest.raises(ValueError):
+        ops.project_and_operand(x, v, s, p1, mode, centre)
+
+
+def test_decode_prepare_rejects_what_its_two_halves_reject():
+    from metis_hip import _lib, ops
+    L = _lib.load()
+    M, K, R = 64, 512, 64
+    x = torch.randn(M, K).bfloat16().cuda()
+    v = torch.randn(R, K).bfloat16().cuda()
+    s = torch.rand(R).bfloat16().cuda()
+    p = ops.quantize(x, 1, deferred=True)
+    xv = torch.empty(M, R, dtype=torch.bfloat16, device="cuda")
+    t = torch.empty_like(xv)
+    out = torch.empty(L.metis_nvfp4_decode_operand_bytes(M, K), dtype=torch.uint8, device="cuda")
+    need = L.metis_lowrank_project_workspace_bytes(M, R, K)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    unit = torch.zeros(1, device="cuda")
+
+    def call(rows=M, cols=K, r=R, wsb=need, mode=1, centre=None, xp=x.data_ptr(), up=unit.data_ptr()):
+        return L.metis_decode_prepare_deferred(xp, cols, v.data_ptr(), r, s.data_ptr(), xv.data_ptr(), t.data_ptr(), ws.data_ptr(), wsb,
+                                               p.codes.data_ptr(), p.deferred.data_ptr(), rows, cols, 1, mode, centre, up, out.data_ptr(), None)
+    assert call() == 0
+    assert call(rows=256) != 0 and call(rows=0) != 0          # decode-sized only
+    assert call(cols=320) != 0                                # wide runs: K % 256 == 0
+    assert call(r=48) != 0                                    # rank a multiple of 32
+    assert call(wsb=need - 1) != 0                            # workspace too small
+    assert call(mode=7) != 0
+    assert call(mode=0, centre=x.data_ptr()) != 0             # a centre belongs to bf16 arithmetic
+    assert call(up=None) != 0
+    assert call(xp=None) == 0                                 # x = NULL: the partial sums are taken from the workspace
+    assert call(xp=None, r=160) != 0                          # ... which the quantizer's launch fills for R <= 128 only
+    torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("M,K,R", [(64, 3584, 64), (1, 256, 32), (200, 2048, 128), (255, 18944, 64), (33, 512, 96)])
+@pytest.mark.parametrize("mode", [1, 0])
+def test_quantizer_launch_carries_the_projections_first_step(M, K, R, mode):
+    """metis_decode_quant_project_deferred + metis_decode_prepare_deferred(x = NULL) against the separate quantizer,
+    projection and operand calls: codes, parked maxima, unit, xv, t and operand bytes, bit for bit."""
+    from metis_hip import ops
+    g = torch.Generator().manual_seed(3 * M + K + R)
+    x = (torch.randn(M, K, generator=g) * 2).bfloat16().cuda()
+    v = (torch.randn(R, K, generator=g) * 0.05).bfloat16().cuda()
+    s = torch.rand(R, generator=g).bfloat16().cuda()
+    want_xv, want_t = ops.lowrank_project(x, v, s)
+    p1 = ops.quantize(x, mode, deferred=True)
+    assert ops.quantize_project_decode_applies(x, v, mode)
+    p2, pending = ops.quantize_project_decode(x, v, mode)
+    nb = M * K // 16
+    assert torch.equal(p2.codes, p1.codes)
+    assert torch.equal(p2.deferred[:8192 + 2 * nb], p1.deferred[:8192 + 2 * nb])     # partial maxima, parked block maxima
+    xv, t, op = ops.project_and_operand(x, v, s, p2, mode, None, pending=pending)
+    want_op = ops.decode_operand(p1, mode)
+    torch.cuda.synchronize()
+    assert torch.equal(xv, want_xv) and torch.equal(t, want_t)
+    assert torch.equal(op, want_op) and torch.equal(p2.unit, p1.unit)
+
+
+def test_decode_quant_project_rejects_shapes_outside_its_domain():
+    from metis_hip import _lib
+    L = _lib.load()
+    M, K, R = 64, 512, 64
+    x = torch.randn(M, K).bfloat16().cuda()
+    v = torch.randn(R, K).bfloat16().cuda()
+    codes = torch.empty(M, K // 2, dtype=torch.uint8, device="cuda")
+    parked = torch.empty(L.metis_nvfp4_deferred_bytes(M, K), dtype=torch.uint8, device="cuda")
+    need = L.metis_lowrank_project_workspace_bytes(M, R, K)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+
+    def call(rows=M, cols=K, r=R, mode=1, wsb=need, pb=parked.numel(), xp=x.data_ptr()):
+        return L.metis_decode_quant_project_deferred(xp, rows, cols, mode, codes.data_ptr(), parked.data_ptr(), pb, v.data_ptr(), r,
+                                                     ws.data_ptr(), wsb, None)
+    assert call() == 0
+    assert call(rows=256) != 0 and call(rows=0) != 0
+    assert call(cols=48) != 0
+    assert call(r=160) != 0 and call(r=40) != 0
+    assert call(mode=2) != 0
+    assert call(wsb=need - 1) != 0 and call(pb=16) != 0
+    assert call(xp=None) != 0
+    torch.cuda.synchronize()

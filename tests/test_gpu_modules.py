@@ -630,12 +630,22 @@ def test_fused_rmsnorm_feeds_the_projection_groups_of_a_qwen2_layer():
             seen.append(tuple(t_.shape))
         return orig(cls, t_, col, noise, arith, **more)
 
+    # (a decode-sized activation that no sibling shares is quantized by the launch that also starts its projection)
+    from metis_hip import ops
+    orig_qpd = ops.quantize_project_decode
+
+    def spy_qpd(x2, *a, **k):
+        seen.append(tuple(x2.shape))
+        return orig_qpd(x2, *a, **k)
+
     base.pack = classmethod(spy)
+    ops.quantize_project_decode = spy_qpd
     try:
         with torch.no_grad():
             run(x)
     finally:
         base.pack = classmethod(orig)
+        ops.quantize_project_decode = orig_qpd
     # q/k/v and gate/up inputs came packed from the norms: the only row quantizations left are o_proj's input
     # (attention output, also [128, 256]) and down_proj's (the MLP activation)
     assert sorted(seen) == [(128, 256), (128, 512)], seen
