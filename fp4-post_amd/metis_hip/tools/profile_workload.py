@@ -115,6 +115,12 @@ def extra(reps: int = 5):
         _, t_d = ops.lowrank_project(xd, v_up, s_up)
         ops.linear_fwd_grouped(p_res, [(w_up, t_d[:, :64], u_up, None), (w_up, t_d[:, 64:], u_up, None)], center=me_d32)
         ops.linear_fwd_grouped(p_dec_down, [(w_down, None, None, None)], center=me_down)     # K in slices, centre inside
+        # decode-sized layer call in bf16 arithmetic, small steps merged: quantizer || projection's partial sums, then
+        # finishing step || operand build (gate/up's stacked V on a quantized activation; down's own V)
+        p_up16 = ops.quantize(xd, 1, deferred=True)
+        ops.project_and_operand(xd, v_up, s_up, p_up16, 1)
+        p_dn16, pending = ops.quantize_project_decode(dec, v_pre, 1)
+        ops.project_and_operand(dec, v_pre, s_pre, p_dn16, 1, pending=pending)
     torch.cuda.synchronize()
 
 
