@@ -264,6 +264,79 @@ static void check_decode_bf16(int64_t M, int64_t N, int64_t K, hipStream_t st)
           "metis_linear_fwd_grouped_bf16 with 256 rows -> METIS_E_ARG (the pipelined kernel's size)");
 }
 
+// A decode-sized BitLinear.forward in bf16 arithmetic as three launches: quantizer + the projection's first step,
+// its finishing step + the activation's GEMM operands, the GEMM.  The quantizer's half against the C oracle, the
+// projection against double precision on the host, the output against the same forward through the separate calls.
+static void check_decode_three_launches(int64_t M, int64_t N, int64_t K, int64_t R, hipStream_t st)
+{
+    const std::vector<uint16_t> x = make_input(M, K, 41u, 1.0f), w = make_input(N, K, 42u, 0.02f), v = make_input(R, K, 43u, 0.02f);
+    std::vector<uint16_t> sv((size_t)R), u = make_input(N, R, 44u, 0.1f);
+    for (int64_t j = 0; j < R; ++j) sv[(size_t)j] = metis_oracle_f32_to_bf16(0.5f + 0.01f * (float)j);
+    DeviceBuffer<uint16_t> dx(x.size()), dv(v.size()), ds(sv.size()), du(u.size());
+    dx.upload(x); dv.upload(v); ds.upload(sv); du.upload(u);
+    DeviceBuffer<uint8_t> bc((size_t)(N * K / 2)), bs((size_t)(N * K / 16));
+    DeviceBuffer<float> bu(1);
+    quantize_on_device(w, N, K, METIS_MODE_PB16, st, &bc, &bs, &bu);
+    // merged launches
+    DeviceBuffer<uint8_t> codes((size_t)(M * K / 2)), parked(metis_nvfp4_deferred_bytes(M, K) + 256);
+    uint8_t* parked_p = (uint8_t*)(((uintptr_t)parked.p + 255) & ~(uintptr_t)255);
+    const size_t lws = metis_lowrank_project_workspace_bytes(M, R, K);
+    DeviceBuffer<uint8_t> lr_ws(lws), aop(metis_nvfp4_decode_operand_bytes(M, K));
+    DeviceBuffer<uint16_t> xv((size_t)(M * R)), t((size_t)(M * R)), out_a((size_t)(M * N)), out_b((size_t)(M * N));
+    DeviceBuffer<float> unit(1);
+    int rc = metis_decode_quant_project_deferred(dx.p, M, K, METIS_MODE_PB16, codes.p, parked_p, metis_nvfp4_deferred_bytes(M, K), dv.p, R,
+                                                 lr_ws.p, lws, st);
+    if (rc == METIS_OK)
+        rc = metis_decode_prepare_deferred(nullptr, K, dv.p, R, ds.p, xv.p, t.p, lr_ws.p, lws, codes.p, parked_p, M, K, METIS_MODE_PB16,
+                                           METIS_MODE_PB16, nullptr, unit.p, aop.p, st);
+    metis_linear_member mem = {};
+    mem.b_codes = bc.p; mem.b_scales = bs.p; mem.b_unit = bu.p; mem.N = N; mem.t = t.p; mem.u = du.p; mem.r = (int)R;
+    const size_t need = metis_linear_grouped_workspace_bytes(M, K, &mem, 1);
+    DeviceBuffer<uint8_t> gws(need ? need : 16);
+    mem.out = out_a.p;
+    if (rc == METIS_OK)
+        rc = metis_linear_fwd_grouped_operand(aop.p, unit.p, M, K, &mem, 1, METIS_DTYPE_BF16, METIS_MODE_PB16, need ? gws.p : nullptr, need, st);
+    HIP_OK(hipStreamSynchronize(st));
+    // the quantizer's half against the oracle (codes and tensor unit; the scale bytes are never written on this path)
+    std::vector<uint8_t> wc((size_t)(M * K / 2)), wsc((size_t)(M * K / 16));
+    float wu = 0.0f;
+    metis_oracle_nvfp4_pack(x.data(), M, K, K, METIS_MODE_PB16, nullptr, wc.data(), wsc.data(), &wu, nullptr);
+    char line[260];
+    snprintf(line, sizeof line, "metis_decode_quant_project_deferred %ldx%ld r=%ld rc=%d: codes and unit equal the oracle's", (long)M, (long)K, (long)R, rc);
+    check(rc == METIS_OK && codes.download() == wc && unit.download()[0] == wu, line);
+    // the projection against double precision: one bf16 rounding of the exact sum, t = bf16(xv * s)
+    const std::vector<uint16_t> gxv = xv.download(), gt = t.download();
+    double worst = 0.0, scale = 0.0;
+    size_t t_off = 0;
+    for (int64_t m = 0; m < M; ++m)
+        for (int64_t j = 0; j < R; ++j) {
+            double sum = 0;
+            for (int64_t k = 0; k < K; ++k) sum += (double)bf16_to_f32(x[(size_t)(m * K + k)]) * (double)bf16_to_f32(v[(size_t)(j * K + k)]);
+            worst = fmax(worst, fabs((double)bf16_to_f32(gxv[(size_t)(m * R + j)]) - sum));
+            scale = fmax(scale, fabs(sum));
+            t_off += gt[(size_t)(m * R + j)] != metis_oracle_f32_to_bf16(bf16_to_f32(gxv[(size_t)(m * R + j)]) * bf16_to_f32(sv[(size_t)j]));
+        }
+    snprintf(line, sizeof line, "metis_decode_prepare_deferred: x V^T within a bf16 ulp of the exact sums (%.3g of max %.3g), t = bf16(xv * s) (%zu off)",
+             worst, scale, t_off);
+    check(worst <= scale / 128.0 && t_off == 0, line);
+    // the same forward through the separate calls
+    DeviceBuffer<uint8_t> ac((size_t)(M * K / 2)), as((size_t)(M * K / 16)), aop2(metis_nvfp4_decode_operand_bytes(M, K)), lr_ws2(lws);
+    DeviceBuffer<float> au(1);
+    DeviceBuffer<uint16_t> xv2((size_t)(M * R)), t2((size_t)(M * R));
+    quantize_on_device(x, M, K, METIS_MODE_PB16, st, &ac, &as, &au);
+    int rc2 = metis_lowrank_project(dx.p, K, dv.p, M, R, K, ds.p, xv2.p, t2.p, lr_ws2.p, lws, st);
+    if (rc2 == METIS_OK) rc2 = metis_nvfp4_decode_operand(ac.p, as.p, au.p, M, K, METIS_MODE_PB16, nullptr, aop2.p, st);
+    mem.t = t2.p; mem.out = out_b.p;
+    if (rc2 == METIS_OK)
+        rc2 = metis_linear_fwd_grouped_operand(aop2.p, au.p, M, K, &mem, 1, METIS_DTYPE_BF16, METIS_MODE_PB16, need ? gws.p : nullptr, need, st);
+    HIP_OK(hipStreamSynchronize(st));
+    snprintf(line, sizeof line, "decode-sized forward %ldx%ldx%ld r=%ld in three launches equals the separate calls bit for bit (rc %d, %d)",
+             (long)M, (long)N, (long)K, (long)R, rc, rc2);
+    check(rc == METIS_OK && rc2 == METIS_OK && out_a.download() == out_b.download() && xv2.download() == gxv && aop2.download() == aop.download(), line);
+    check(metis_decode_quant_project_deferred(dx.p, 256, K, METIS_MODE_PB16, codes.p, parked_p, metis_nvfp4_deferred_bytes(M, K), dv.p, R, lr_ws.p,
+                                              lws, st) == METIS_E_SHAPE, "metis_decode_quant_project_deferred with 256 rows -> METIS_E_SHAPE");
+}
+
 // Mean mode at decode size: column mean (with the running update) -> centred quantizer -> grouped GEMM with the
 // centre inside, and the packed matrix-vector product, all against double precision on the host.
 static void check_mean_mode_decode(hipStream_t st)
@@ -531,6 +604,8 @@ int main()
     check_mean_mode_decode(st);
     check_decode_bf16(48, 160, 512, st);
     check_decode_bf16(64, 96, 8192, st);
+    check_decode_three_launches(48, 160, 512, 32, st);
+    check_decode_three_launches(64, 96, 4096, 64, st);
 
     // ---- 4b: one pass over an activation (quantizer + rank-r projection; K slices at 256 rows against a long K), and
     //          both stochastic packings of a gradient
