@@ -828,3 +828,52 @@ def test_decode_step_in_bf16_arithmetic_never_writes_the_activation_scale_bytes(
     torch.cuda.synchronize()
     assert calls["n"] == 0
     assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("mean_mode,fuse_norms,rows", [(False, True, 64), (False, False, 48), (True, False, 64), (False, True, 1)])
+def test_merged_decode_launches_leave_the_layer_output_unchanged(mean_mode, fuse_norms, rows, monkeypatch):
+    """The decode step of a patched Qwen2 layer with the small launches merged (the projection's finishing step inside
+    the operand build, the projection's first step inside an unshared activation's quantizer launch) against the same
+    step with the merged calls switched off: the same bits, and the merged calls are the ones that ran."""
+    pytest.importorskip("transformers")
+    from transformers.models.qwen2.modeling_qwen2 import Qwen2Config, Qwen2DecoderLayer, Qwen2RotaryEmbedding
+    from metis_hip import BitLinear, MetisArgs, ops, replace_model_with_metis
+    torch.manual_seed(3)
+    cfg = Qwen2Config(hidden_size=256, intermediate_size=512, num_attention_heads=4, num_key_value_heads=2,
+                      num_hidden_layers=1, vocab_size=128, max_position_embeddings=256)
+    cfg._attn_implementation = "eager"
+    layer = Qwen2DecoderLayer(cfg, layer_idx=0).to(torch.bfloat16).cuda()
+    for p in layer.parameters():
+        if p.dim() == 2:
+            torch.nn.init.normal_(p, std=0.02)
+    holder = torch.nn.ModuleDict({"layer": layer})
+    args = MetisArgs(forward_svd_rank=32, cache_quantized_weight=True) if mean_mode else MetisArgs.direct_fp4(forward_svd_rank=32)
+    replace_model_with_metis(holder, args, fuse_norms=fuse_norms)
+    x = (torch.randn(rows, 1, 256, device="cuda") + 0.5).bfloat16()
+    pos = torch.zeros(rows, 1, dtype=torch.long, device="cuda")
+    pe = Qwen2RotaryEmbedding(cfg).cuda()(x, pos)
+
+    def run():
+        for m in holder.modules():
+            if isinstance(m, BitLinear):
+                m.mean_cache.clear()
+                if m.activation_group is not None:
+                    m.activation_group["mean_cache"].clear()
+        with torch.no_grad():
+            out = holder["layer"](x, position_embeddings=pe, attention_mask=None, position_ids=pos)
+        return out[0] if isinstance(out, tuple) else out
+
+    seen = {"prepare": 0, "quant_project": 0}
+    real_pao, real_qpd = ops.project_and_operand, ops.quantize_project_decode
+    monkeypatch.setattr(ops, "project_and_operand", lambda *a, **k: (seen.__setitem__("prepare", seen["prepare"] + 1), real_pao(*a, **k))[1])
+    monkeypatch.setattr(ops, "quantize_project_decode",
+                        lambda *a, **k: (seen.__setitem__("quant_project", seen["quant_project"] + 1), real_qpd(*a, **k))[1])
+    merged = run()
+    # q/k/v, o, gate/up, down each prepare once; o and down quantize their own activation (direct mode only)
+    assert seen == {"prepare": 4, "quant_project": 0 if mean_mode else 2}, seen
+    monkeypatch.setattr(ops, "project_and_operand_applies", lambda *a, **k: False)
+    monkeypatch.setattr(ops, "quantize_project_decode_applies", lambda *a, **k: False)
+    seen.update(prepare=0, quant_project=0)
+    separate = run()
+    assert seen == {"prepare": 0, "quant_project": 0}
+    assert torch.equal(merged, separate)
