@@ -389,6 +389,12 @@ int metis_nvfp4_decode_operand_deferred(const void* codes, const void* deferred,
     return skinny_operand_deferred(codes, deferred, rows, cols, quant_mode, mode, center, unit, out, (hipStream_t)stream);
 }
 
+int metis_nvfp4_decode_operand_rht(const void* codes, const void* scales, float* unit, const void* deferred, int64_t rows, int64_t cols,
+                                   int quant_mode, int mode, uint32_t sign_mask, void* out, void* stream)
+{
+    return skinny_operand_rht(codes, scales, unit, deferred, rows, cols, quant_mode, mode, sign_mask, out, (hipStream_t)stream);
+}
+
 int metis_decode_quant_project_deferred(const void* x, int64_t rows, int64_t cols, int mode, void* codes, void* deferred,
                                         size_t deferred_bytes, const void* v, int64_t R, void* workspace, size_t workspace_bytes,
                                         void* stream)

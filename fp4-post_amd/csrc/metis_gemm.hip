@@ -1004,6 +1004,77 @@ __global__ __launch_bounds__(256) void skinny_operand_kernel(const uint32_t* __r
                                            unit_out);
 }
 
+// NV recipe at decode size.  The cached weight holds the codes of the ROTATED weight, and the forward multiplies with
+// W~ = rotate_back(QDQ(rotate(W))) (src/Metis/Metis/bitlinear.py:577-585, 395-405): per block of 16 along K,
+// W~[n] = sign[n] / 16 * sum_k H[k][n] q[k] with q the dequantized rotated block.  The decode-sized kernel streams the
+// packed weight as it is, so the rotation goes to the other operand:
+//     sum_n x^[n] W~[n] = sum_k q[k] a'[k],   a'[k] = 1/16 * sum_n H[n][k] (sign[n] x^[n])
+// -- the activation's dequantized block rotated forward and scaled by 1/16.  The sums are exact in binary32 (sixteen
+// values of one block: at most 16 significant bits), a' is rounded once to the operand's 16-bit format (the tiled
+// path rounds W~ once instead).  A thread forms the eight values of its piece from the whole block (both code words).
+template <int PB16, int DEF, int QMODE>
+__global__ __launch_bounds__(256) void skinny_operand_rht_kernel(const uint2* __restrict__ codes, const uint8_t* __restrict__ scales,
+                                                                 const float* __restrict__ unit_p, int M, int K, int tiles,
+                                                                 uint4* __restrict__ out, const uint32_t* __restrict__ partials,
+                                                                 float* __restrict__ unit_out, uint32_t sign_mask)
+{
+    typedef float float2_t __attribute__((ext_vector_type(2)));
+    const int iters = K / 256;
+    const int64_t total = (int64_t)tiles * iters * 1024;
+    float unit = 0.0f;
+    if constexpr (DEF != 0) {
+        unit = tensor_unit_of<QMODE>(fold_partial_maxima(partials));
+        if (blockIdx.x == 0 && threadIdx.x == 0) *unit_out = unit;
+    } else if constexpr (PB16 != 0) {
+        unit = *unit_p;
+    }
+    const uint16_t* __restrict__ maxima = reinterpret_cast<const uint16_t*>(scales);
+    for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
+        const int lane = (int)(idx & 63), m = (int)((idx >> 6) & 15);
+        const int64_t ti = idx >> 10;
+        const int it = (int)(ti % iters), tile = (int)(ti / iters);
+        const int row = tile * 32 + (lane & 31), k0 = it * 256 + (lane >> 5) * 128 + 8 * m;
+        uint4 v = make_uint4(0u, 0u, 0u, 0u);
+        if (row < M) {
+            const int half = m & 1;                              // which eight of the block's sixteen outputs are this thread's
+            const uint2 c = codes[(int64_t)row * (K / 16) + (k0 >> 4)];
+            uint32_t sb;
+            if constexpr (DEF != 0) sb = scale_byte_of<QMODE>(maxima[(int64_t)row * (K / 16) + (k0 >> 4)], unit);
+            else sb = scales[(int64_t)row * (K / 16) + (k0 >> 4)];
+            const float dq = PB16 ? rb(e4m3_value(sb) * unit) : e4m3_value(sb) * 0.00390625f;
+            const float2_t p[8] = {__builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 0), __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 1),
+                                   __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 2), __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 3),
+                                   __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 0), __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 1),
+                                   __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 2), __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 3)};
+            float blk[kBlock];
+#pragma unroll
+            for (int n = 0; n < kBlock; ++n) {
+                const float x = PB16 ? rb(p[n >> 1][n & 1] * dq) : p[n >> 1][n & 1] * dq;
+                // sign[n] of the rotation; inputs 8..15 change sign for the outputs 8..15 (H[n][8 + j] = -H[n][j] there)
+                const uint32_t flip = (((sign_mask >> n) & 1u) ^ (n >= 8 ? (uint32_t)half : 0u)) << 31;
+                blk[n] = __uint_as_float(__float_as_uint(x) ^ flip);
+            }
+            float o[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                float acc = blk[0];
+#pragma unroll
+                for (int n = 1; n < kBlock; ++n) acc = (__builtin_popcount(n & j) & 1) ? acc - blk[n] : acc + blk[n];
+                o[j] = acc * 0.0625f;
+            }
+            if constexpr (PB16 != 0) {
+                v.x = rb_pair(o[0], o[1]); v.y = rb_pair(o[2], o[3]); v.z = rb_pair(o[4], o[5]); v.w = rb_pair(o[6], o[7]);
+            } else {
+                const half2_t h0 = {(_Float16)o[0], (_Float16)o[1]}, h1 = {(_Float16)o[2], (_Float16)o[3]};
+                const half2_t h2 = {(_Float16)o[4], (_Float16)o[5]}, h3 = {(_Float16)o[6], (_Float16)o[7]};
+                v.x = __builtin_bit_cast(uint32_t, h0); v.y = __builtin_bit_cast(uint32_t, h1);
+                v.z = __builtin_bit_cast(uint32_t, h2); v.w = __builtin_bit_cast(uint32_t, h3);
+            }
+        }
+        out[idx] = v;
+    }
+}
+
 // One launch for the two small independent steps between a decode-sized layer's quantizer and its GEMM: the first
 // `finish_blocks` blocks finish the rank-r projection (lowrank_small_steps.h), the others build the activation's
 // operands from a tensor whose quantizer call deferred its scale bytes.
@@ -1068,6 +1139,42 @@ int skinny_operand_deferred(const void* codes, const void* deferred, int64_t M, 
     if (mode == METIS_MODE_PB16) { if (qmode) METIS_SOD(1, 1); else METIS_SOD(1, 0); }
     else { if (qmode) METIS_SOD(0, 1); else METIS_SOD(0, 0); }
 #undef METIS_SOD
+    return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
+}
+
+// The operand of a decode-sized call against a ROTATED packed weight (NV recipe): the activation's dequantized blocks
+// rotated forward and scaled by 1/16 (skinny_operand_rht_kernel).  deferred = nullptr: scale bytes and unit as given;
+// otherwise the quantizer call deferred them (qmode = its arithmetic) and unit receives the tensor unit.
+int skinny_operand_rht(const void* codes, const void* scales, float* unit, const void* deferred, int64_t M, int64_t K, int qmode, int mode,
+                       uint32_t sign_mask, void* out, hipStream_t st)
+{
+    if (mode == METIS_MODE_P32_F32) mode = METIS_MODE_P32;
+    if (mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) return METIS_E_ARG;
+    if (sign_mask > 0xffffu) return METIS_E_ARG;
+    if (M <= 0 || M >= 256 || K <= 0 || K % 256 || K > INT32_MAX) return METIS_E_SHAPE;
+    if (!codes || !out || ((uintptr_t)codes % 8) || ((uintptr_t)out % 16)) return METIS_E_ARG;
+    const int tiles = (int)((M + 63) / 64) * 2;
+    const int64_t total = (int64_t)tiles * (K / 256) * 1024;
+    const int g = (int)((total + 255) / 256);
+    if (deferred) {
+        if ((qmode != METIS_MODE_P32 && qmode != METIS_MODE_PB16) || !unit) return METIS_E_ARG;
+        Workspace ws;
+        if (const int rc = carve_deferred(const_cast<void*>(deferred), deferred_bytes(M, K), M, K, &ws)) return rc;
+#define METIS_SOR(P, Q) hipLaunchKernelGGL((skinny_operand_rht_kernel<P, 1, Q>), dim3(g), dim3(256), 0, st, (const uint2*)codes, \
+                                           (const uint8_t*)ws.amax, nullptr, (int)M, (int)K, tiles, (uint4*)out, (const uint32_t*)ws.gmax, \
+                                           unit, sign_mask)
+        if (mode == METIS_MODE_PB16) { if (qmode) METIS_SOR(1, 1); else METIS_SOR(1, 0); }
+        else { if (qmode) METIS_SOR(0, 1); else METIS_SOR(0, 0); }
+#undef METIS_SOR
+        return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
+    }
+    if (!scales || (mode == METIS_MODE_PB16 && !unit)) return METIS_E_ARG;
+    if (mode == METIS_MODE_PB16)
+        hipLaunchKernelGGL((skinny_operand_rht_kernel<1, 0, 0>), dim3(g), dim3(256), 0, st, (const uint2*)codes, (const uint8_t*)scales, unit,
+                           (int)M, (int)K, tiles, (uint4*)out, nullptr, nullptr, sign_mask);
+    else
+        hipLaunchKernelGGL((skinny_operand_rht_kernel<0, 0, 0>), dim3(g), dim3(256), 0, st, (const uint2*)codes, (const uint8_t*)scales, unit,
+                           (int)M, (int)K, tiles, (uint4*)out, nullptr, nullptr, sign_mask);
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }
 

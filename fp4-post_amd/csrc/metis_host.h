@@ -137,6 +137,9 @@ int skinny_operand(const void* codes, const void* scales, const float* unit, int
 // the same from a tensor whose quantizer call deferred its scale bytes; writes the unit
 int skinny_operand_deferred(const void* codes, const void* deferred, int64_t M, int64_t K, int qmode, int mode, const void* center,
                             float* unit_out, void* out, hipStream_t st);
+// the same operand for a call against a ROTATED packed weight (NV recipe): activation blocks rotated forward / 16
+int skinny_operand_rht(const void* codes, const void* scales, float* unit, const void* deferred, int64_t M, int64_t K, int qmode, int mode,
+                       uint32_t sign_mask, void* out, hipStream_t st);
 // quantize_row_deferred of a decode-sized activation with the projection's first step in the same launch; nvfp4_quant.hip
 int quantize_row_deferred_partial(const void* x, int64_t rows, int64_t cols, int mode, void* codes, void* deferred, size_t bytes,
                                   const void* v, int64_t R, void* lr_workspace, size_t lr_workspace_bytes, hipStream_t st);

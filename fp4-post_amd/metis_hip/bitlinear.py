@@ -1074,8 +1074,9 @@ class BitLinear(nn.Module):
         if rows >= 256 or not all(m._fusable() and m.compute_dtype == self.compute_dtype for m in members):
             return None
         packed = [m._packed_residual() for m in members]
-        if any(p is None or p.rht is not None for p in packed):   # a rotated weight (NV recipe) needs the tiled GEMM's operands
+        if any(p is None for p in packed):
             return None
+        rotated = any(p.rht is not None for p in packed)          # NV recipe: the activation's operand carries the rotation
         cd = torch.bfloat16
         x2 = _flat2d(x).to(cd)
         # one product for every member's rank-r projection: V of all members stacked, cached on their versions
@@ -1089,6 +1090,8 @@ class BitLinear(nn.Module):
         px = shared_input.residual if centre is not None else shared_input
         if centre is not None and all(F._mean_in_operand(shared_input, p) for p in packed):
             centre = shared_input.mean                             # bf16: goes into the activation operand (reference's bf16 tensor)
+        if rotated and (centre is not None or not ops.nv_decode_applies(px, packed, [m.args.forward_svd_rank for m in members])):
+            return None                                            # member by member on the tiled GEMM
         aop = None
         if (ops.grouped_operand_applies(px, packed, [m.args.forward_svd_rank for m in members], centre, F.reference_rounding)
                 and ops.project_and_operand_applies(x2, cached[1], cached[2], px)):

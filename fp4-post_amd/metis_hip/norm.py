@@ -100,7 +100,8 @@ class FusedRMSNormQuant(nn.Module):
         F = LinearLowbitFunction
         cols = x.shape[-1]
         fused = (x.is_cuda and x.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16 and cols % 32 == 0
-                 and cols <= 16384 and is_hip_nvfp4(F.q_forward_input) and not F.enable_nv_recipe and x.numel() > 0)
+                 and cols <= 16384 and is_hip_nvfp4(F.q_forward_input) and (not F.enable_nv_recipe or F._nv_on_kernels())
+                 and x.numel() > 0)     # (NV recipe: the forward quantizes its activation unrotated, like any other)
         mean_mode = fused and F.enable_activation_svd
         if mean_mode:
             fused = (F._mean_mode_packable() and cols <= 4096 and F.compute_dtype in (torch.float32, torch.bfloat16)

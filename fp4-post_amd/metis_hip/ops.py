@@ -616,12 +616,28 @@ def expand_tiled_transposed(p: PackedNVFP4, cache: bool = False, mode: int = MOD
     return out
 
 
-def decode_operand(p: PackedNVFP4, mode: int = MODE_P32, center: torch.Tensor | None = None) -> torch.Tensor:
+def decode_operand(p: PackedNVFP4, mode: int = MODE_P32, center: torch.Tensor | None = None, rotate: int | None = None) -> torch.Tensor:
     """The activation of a decode-sized call (rows < 256, cols % 256 == 0) as ready 16-bit MFMA operands for
     metis_linear_fwd_grouped_operand: exact binary16 values (mode P32), the reference's bf16 dequantized values (mode
-    PB16), or with `center` (bf16 [cols], PB16) the mean mode's center + QDQ(x - center) rounded to bf16."""
+    PB16), or with `center` (bf16 [cols], PB16) the mean mode's center + QDQ(x - center) rounded to bf16.
+    rotate (sign mask): the call multiplies with a weight packed in the rotated domain (NV recipe); the operand then
+    holds the activation's dequantized blocks rotated forward and scaled by 1/16, which gives the product with the
+    weight rotated back."""
     L = load()
     out = torch.empty(L.metis_nvfp4_decode_operand_bytes(p.rows, p.cols), dtype=torch.uint8, device=p.codes.device)
+    if rotate is not None:
+        if center is not None or p.rht is not None:
+            raise ValueError("a rotated operand is built from an unrotated, uncentred activation")
+        d = p.__dict__
+        lazy = d.get("deferred") is not None and d.get("_scales") is None
+        rc = L.metis_nvfp4_decode_operand_rht(p.codes.data_ptr(), None if lazy else p.scales.data_ptr(),
+                                              d["_unit"].data_ptr() if lazy else p.unit.data_ptr(),
+                                              d["deferred"].data_ptr() if lazy else None, p.rows, p.cols, p.mode, mode, int(rotate),
+                                              out.data_ptr(), _stream())
+        check(rc, "metis_nvfp4_decode_operand_rht", (p.rows, p.cols))
+        if lazy:
+            d["_unit_ready"] = True
+        return out
     if center is not None:
         center = center.reshape(-1).to(torch.bfloat16).contiguous()
         if center.numel() != p.cols:
@@ -647,7 +663,7 @@ def grouped_operand_applies(a: PackedNVFP4, weights, ranks, center: torch.Tensor
     members' packed weights, ranks: the widths of their low-rank terms (0 without)."""
     M, K = a.rows, a.cols
     return bool(reference_rounding and (center is None or center.dtype == torch.bfloat16) and a.mode == MODE_PB16
-                and all(b.mode == MODE_PB16 for b in weights) and len(weights) <= 4 and K % 256 == 0
+                and all(b.mode == MODE_PB16 and b.rht is None for b in weights) and len(weights) <= 4 and K % 256 == 0
                 and all(_decode_kernel_takes(M, b.rows, K, r) for b, r in zip(weights, ranks))
                 and all(b.scales.data_ptr() % 8 == 0 for b in weights))
 
@@ -707,7 +723,7 @@ def decode_weight(p: PackedNVFP4, cache: bool = True) -> torch.Tensor | None:
     K % 256 != 0.  Kept on a persistent (cached) weight."""
     if p.decode_layout is not None:
         return p.decode_layout
-    if p.cols % 256 or p.rht is not None:
+    if p.cols % 256:
         return None
     L = load()
     out = torch.empty(L.metis_nvfp4_decode_weight_bytes(p.rows, p.cols), dtype=torch.uint8, device=p.codes.device)
@@ -918,6 +934,16 @@ def _gemm_workspace(M: int, N: int, K: int, device: torch.device) -> torch.Tenso
     return torch.empty(need, dtype=torch.uint8, device=device) if need else None
 
 
+def nv_decode_applies(a: PackedNVFP4, weights, ranks) -> bool:
+    """A decode-sized call against weights packed in the rotated domain (NV recipe) runs on the decode-sized kernel,
+    the rotation carried by the activation's operand: one rotation for all members, an unrotated activation, the
+    kernel's shapes in wide runs."""
+    masks = {b.rht for b in weights}
+    return bool(len(masks) == 1 and None not in masks and a.rht is None and len(weights) <= 4 and a.cols % 256 == 0
+                and all(_decode_kernel_takes(a.rows, b.rows, a.cols, r) for b, r in zip(weights, ranks))
+                and all(b.scales.data_ptr() % 8 == 0 for b in weights))
+
+
 def _decode_kernel_takes(M: int, N: int, K: int, r: int) -> bool:
     """Shapes of the decode-sized kernel (waves split K over packed operands streamed from global memory)."""
     return 0 < M < 256 and K % 64 == 0 and N % 4 == 0 and r % 32 == 0
@@ -944,6 +970,11 @@ def linear_fwd(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None,
     a_operand: as in linear_fwd_grouped (a decode-sized call in bf16 arithmetic)."""
     if a.cols != b.cols:
         raise ValueError(f"contraction mismatch: {a.cols} vs {b.cols}")
+    if (tiled is None and not expanded and b.rht is not None
+            and nv_decode_applies(a, [b], [0 if t is None else t.shape[1]])):
+        # NV recipe at decode size: the packed rotated weight is streamed as it is, the activation's operand is rotated
+        return _linear_fwd_grouped(a, [(b, t, u, bias)], out_dtype=out_dtype, split_k=split_k,
+                                   reference_rounding=reference_rounding)[0]
     if a.rht is not None or b.rht is not None:
         # NV recipe: only the tiled operands know how to rotate a block back
         if a.cols % 32:
@@ -1173,6 +1204,16 @@ def _linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.
     rounded = (reference_rounding and (center is None or center.dtype == torch.bfloat16) and a.mode == MODE_PB16
                and all(m[0].mode == MODE_PB16 for m in members))
     takes = len(members) <= 4 and all(_decode_kernel_takes(M, m[0].rows, K, 0 if m[1] is None else m[1].shape[1]) for m in members)
+    # NV recipe: weights packed in the rotated domain.  The decode-sized kernel streams them as they are and the
+    # activation's operand carries the rotation (decode_operand(rotate=...)); callers check nv_decode_applies first
+    rotate = None
+    masks = {m[0].rht for m in members}
+    if masks != {None}:
+        if len(masks) != 1 or a.rht is not None or center is not None or not takes or K % 256 \
+                or any(m[0].scales.data_ptr() % 8 for m in members):
+            raise ValueError("rotated weights: one rotation for all members of a decode-sized call on an unrotated, uncentred "
+                             "activation (see nv_decode_applies); other calls take the tiled GEMM")
+        rotate = masks.pop()
     # ready operands (built once for the group): wide runs only
     operand = grouped_operand_applies(a, [m[0] for m in members], [0 if m[1] is None else m[1].shape[1] for m in members],
                                       center, reference_rounding)
@@ -1223,6 +1264,13 @@ def _linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.
             M, K, ctypes.cast(arr, ctypes.c_void_p), len(members), 0))
     ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
     dt = DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16
+    if rotate is not None:
+        op_mode = MODE_PB16 if rounded else MODE_P32
+        aop = decode_operand(a, op_mode, None, rotate=rotate)
+        rc = L.metis_linear_fwd_grouped_operand(aop.data_ptr(), a.unit.data_ptr(), M, K, ap, len(members), dt, op_mode,
+                                                None if ws is None else ws.data_ptr(), need, _stream())
+        check(rc, "metis_linear_fwd_grouped_operand", (M, K, [m[0].rows for m in members]))
+        return outs
     if operand:
         # (a quantizer call that deferred its scale bytes never gets them: the operand kernel forms them on the way)
         aop = a_operand if a_operand is not None else decode_operand(a, MODE_PB16, center)

@@ -121,6 +121,8 @@ def extra(reps: int = 5):
         ops.project_and_operand(xd, v_up, s_up, p_up16, 1)
         p_dn16, pending = ops.quantize_project_decode(dec, v_pre, 1)
         ops.project_and_operand(dec, v_pre, s_pre, p_dn16, 1, pending=pending)
+        # NV recipe at decode size: the activation's operand rotated for a weight packed in the rotated domain
+        ops.decode_operand(ops.quantize(dec, 1, deferred=True), 1, rotate=0x5a3c)
     torch.cuda.synchronize()
 
 

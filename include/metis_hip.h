@@ -656,6 +656,16 @@ int metis_linear_fwd_grouped_bf16(const void *a_codes, const void *a_scales, con
  *                                src/Metis/Metis/bitlinear.py:752-760).  x = NULL: the workspace already holds the
  *                                projection's partial sums, left there by metis_decode_quant_project_deferred on the
  *                                same rows, cols and R (R <= 128 then): one launch
+ *   metis_nvfp4_decode_operand_rht  the operand for a call against a weight packed in the ROTATED domain (NV recipe:
+ *                                metis_nvfp4_quant_row_rht with sign_mask; the forward multiplies with
+ *                                rotate_back(QDQ(rotate(W))), src/Metis/Metis/bitlinear.py:577-585, 395-405).  The
+ *                                decode-sized kernel streams that packed weight as it is, so the rotation is applied
+ *                                to the activation instead: every dequantized block of 16 rotated forward with the same
+ *                                sign_mask and scaled by 1/16 (sums exact, one rounding to the 16-bit operand format),
+ *                                which gives the same product.  deferred = NULL: scales / unit as written by the
+ *                                quantizer (unit needed in mode PB16 only); otherwise scales is ignored, the parked
+ *                                data of metis_nvfp4_quant_row_deferred is read (quant_mode = its mode) and unit
+ *                                receives the tensor unit.  Shapes and `out` as metis_nvfp4_decode_operand
  *   metis_decode_quant_project_deferred  metis_nvfp4_quant_row_deferred (no centre; x contiguous bf16 [rows, cols],
  *                                rows < 256, cols % 64 == 0) and, in the same launch, the first step of
  *                                metis_lowrank_project on v [R, cols] (R % 32 == 0, R <= 128; METIS_E_SHAPE otherwise):
@@ -669,6 +679,9 @@ int metis_nvfp4_decode_operand(const void *codes, const void *scales, const floa
 int metis_nvfp4_decode_operand_deferred(const void *codes, const void *deferred, int64_t rows, int64_t cols,
                                         int quant_mode, int mode, const void *center, float *unit, void *out,
                                         void *stream);
+int metis_nvfp4_decode_operand_rht(const void *codes, const void *scales, float *unit, const void *deferred,
+                                   int64_t rows, int64_t cols, int quant_mode, int mode, uint32_t sign_mask,
+                                   void *out, void *stream);
 int metis_decode_quant_project_deferred(const void *x, int64_t rows, int64_t cols, int mode, void *codes,
                                         void *deferred, size_t deferred_bytes, const void *v, int64_t R,
                                         void *workspace, size_t workspace_bytes, void *stream);

@@ -264,6 +264,53 @@ static void check_decode_bf16(int64_t M, int64_t N, int64_t K, hipStream_t st)
           "metis_linear_fwd_grouped_bf16 with 256 rows -> METIS_E_ARG (the pipelined kernel's size)");
 }
 
+// NV recipe at decode size: a weight packed in the rotated domain is streamed as it is by the decode-sized kernel and
+// the activation's operand carries the rotation (metis_nvfp4_decode_operand_rht).  Against the double-precision product
+// of the activation's dequantized values (oracle) with the weight dequantized and rotated back
+// (metis_nvfp4_dequant + metis_hadamard16, binary32), in binary32 arithmetic: one binary16 rounding of the rotated operand.
+static void check_decode_rotated_weight(int64_t M, int64_t N, int64_t K, hipStream_t st)
+{
+    const uint32_t mask = 0x5a3cu;
+    const std::vector<uint16_t> x = make_input(M, K, 51u, 1.0f), w = make_input(N, K, 52u, 0.02f);
+    DeviceBuffer<uint16_t> dw(w.size());
+    dw.upload(w);
+    DeviceBuffer<uint8_t> ac((size_t)(M * K / 2)), as((size_t)(M * K / 16)), bc((size_t)(N * K / 2)), bs((size_t)(N * K / 16));
+    DeviceBuffer<float> au(1), bu(1), wdeq((size_t)(N * K)), wback((size_t)(N * K)), out((size_t)(M * N));
+    const Packed pa = quantize_on_device(x, M, K, METIS_MODE_P32, st, &ac, &as, &au);
+    const size_t wsb = metis_nvfp4_workspace_bytes(N, K);
+    DeviceBuffer<uint8_t> qws(wsb), aop(metis_nvfp4_decode_operand_bytes(M, K));
+    HIP_OK(hipMemset(qws.p, 0, wsb));
+    int rc = metis_nvfp4_quant_row_rht(dw.p, N, K, K, METIS_MODE_P32, mask, 0, 0, 0, bc.p, bs.p, bu.p, qws.p, wsb, st);
+    if (rc == METIS_OK) rc = metis_nvfp4_dequant(bc.p, bs.p, bu.p, N, K, METIS_MODE_P32, wdeq.p, METIS_DTYPE_F32, st);
+    if (rc == METIS_OK) rc = metis_hadamard16(wdeq.p, N, K, K, METIS_DTYPE_F32, 1, mask, wback.p, K, st);
+    if (rc == METIS_OK) rc = metis_nvfp4_decode_operand_rht(ac.p, as.p, au.p, nullptr, M, K, METIS_MODE_P32, METIS_MODE_P32, mask, aop.p, st);
+    metis_linear_member mem = {};
+    mem.b_codes = bc.p; mem.b_scales = bs.p; mem.b_unit = bu.p; mem.N = N; mem.out = out.p;
+    const size_t need = metis_linear_grouped_workspace_bytes(M, K, &mem, 1);
+    DeviceBuffer<uint8_t> gws(need ? need : 16);
+    if (rc == METIS_OK)
+        rc = metis_linear_fwd_grouped_operand(aop.p, au.p, M, K, &mem, 1, METIS_DTYPE_F32, METIS_MODE_P32, need ? gws.p : nullptr, need, st);
+    HIP_OK(hipStreamSynchronize(st));
+    std::vector<float> xa((size_t)(M * K));
+    metis_oracle_nvfp4_dequant(pa.codes.data(), pa.scales.data(), pa.unit, M, K, 0, nullptr, xa.data());
+    const std::vector<float> wb = wback.download(), got_f = out.download();
+    std::vector<double> got(got_f.begin(), got_f.end()), want((size_t)(M * N));
+    for (int64_t m = 0; m < M; ++m)
+        for (int64_t n = 0; n < N; ++n) {
+            double sum = 0;
+            for (int64_t k = 0; k < K; ++k) sum += (double)xa[(size_t)(m * K + k)] * (double)wb[(size_t)(n * K + k)];
+            want[(size_t)(m * N + n)] = sum;
+        }
+    char line[240];
+    snprintf(line, sizeof line, "metis_nvfp4_decode_operand_rht + grouped operand call %ldx%ldx%ld rc=%d vs x^ . rotate_back(Q)^T rel.err %.2e",
+             (long)M, (long)N, (long)K, rc, rel_fro(got, want));
+    check(rc == METIS_OK && rel_fro(got, want) <= 5e-4, line);
+    check(metis_nvfp4_decode_operand_rht(ac.p, as.p, au.p, nullptr, M, K, METIS_MODE_P32, METIS_MODE_P32, 0x10000u, aop.p, st) == METIS_E_ARG,
+          "metis_nvfp4_decode_operand_rht with a sign mask wider than 16 bits -> METIS_E_ARG");
+    check(metis_nvfp4_decode_operand_rht(ac.p, as.p, au.p, nullptr, 256, K, METIS_MODE_P32, METIS_MODE_P32, mask, aop.p, st) == METIS_E_SHAPE,
+          "metis_nvfp4_decode_operand_rht with 256 rows -> METIS_E_SHAPE");
+}
+
 // A decode-sized BitLinear.forward in bf16 arithmetic as three launches: quantizer + the projection's first step,
 // its finishing step + the activation's GEMM operands, the GEMM.  The quantizer's half against the C oracle, the
 // projection against double precision on the host, the output against the same forward through the separate calls.
@@ -604,6 +651,7 @@ int main()
     check_mean_mode_decode(st);
     check_decode_bf16(48, 160, 512, st);
     check_decode_bf16(64, 96, 8192, st);
+    check_decode_rotated_weight(40, 96, 512, st);
     check_decode_three_launches(48, 160, 512, 32, st);
     check_decode_three_launches(64, 96, 4096, 64, st);
 

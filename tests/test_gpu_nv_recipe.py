@@ -276,3 +276,141 @@ def test_bitlinear_under_the_nv_recipe_is_the_rotated_residual_plus_the_rank_r_b
     g_xv = (dy.bfloat16() @ u.bfloat16()) * s_.bfloat16()                                   # [L, r]
     want_gx = dy_back @ w_back + g_xv.double() @ v.bfloat16().double()
     assert rel_fro(x.grad.double().cpu(), want_gx.cpu()) <= 2e-3
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("M,N,K,r", [(64, 384, 1024, 32), (1, 132, 256, 0), (200, 64, 2048, 64), (48, 512, 18944, 0)])
+@pytest.mark.parametrize("deferred", [False, True])
+def test_decode_sized_call_against_a_rotated_weight_rotates_the_activation(mode, M, N, K, r, deferred, monkeypatch):
+    """NV recipe at decode size: the packed rotated weight is streamed as it is by the decode-sized kernel and the
+    activation's operand carries the rotation (every dequantized block rotated forward, / 16): x^ W~^T = a' Q^T.
+    Against the product of the dequantized tensors (the weight rotated back) in double precision, within the one
+    rounding of the rotated operand to its 16-bit format; the tiled GEMM (which rounds the rotated-back weight
+    instead) gives the same to that accuracy; and no tiled expansion is built."""
+    from metis_hip import ops
+    g = torch.Generator().manual_seed(M + N + K)
+    x = synthetic_activation(41 + M, M, K).cuda()
+    w = (torch.randn(N, K, generator=g) * 0.05).bfloat16().cuda()
+    tt = uu = None
+    if r:
+        tt, uu = (torch.randn(M, r, generator=g) * 0.1).bfloat16().cuda(), (torch.randn(N, r, generator=g) * 0.1).bfloat16().cuda()
+    bias = torch.randn(N, generator=g).bfloat16().cuda()
+    pw = ops.quantize_rht(w, mode, _mask())
+    pw.persistent = True
+    px = ops.quantize(x, mode, deferred=deferred)
+    tiled = ops.linear_fwd(ops.quantize(x, mode), pw, t=tt, u=uu, bias=bias, out_dtype=torch.float32, reference_rounding=mode == 1, tiled=True)
+    assert ops.nv_decode_applies(px, [pw], [r])
+    monkeypatch.setattr(ops, "expand_tiled", lambda *a, **k: (_ for _ in ()).throw(AssertionError("the tiled expansion ran")))
+    got = ops.linear_fwd(px, pw, t=tt, u=uu, bias=bias, out_dtype=torch.float32, reference_rounding=mode == 1)
+    monkeypatch.undo()
+    dt = torch.float32 if mode == 0 else torch.bfloat16
+    want = ops.quantize(x, mode).dequantize(dt).double() @ pw.dequantize(dt).double().T + bias.double()
+    if r:
+        want = want + tt.double() @ uu.double().T
+    tol = 4e-4 if mode == 0 else 4e-3                     # binary16 / bf16 rounding of one operand (and of the bf16 product)
+    assert rel_fro(got.double().cpu(), want.cpu()) <= tol
+    assert rel_fro(tiled.double().cpu(), want.cpu()) <= tol
+    assert torch.equal(px.unit, ops.quantize(x, mode).unit)
+    # grouped: two rotated members on one activation, one launch
+    outs = ops.linear_fwd_grouped(ops.quantize(x, mode, deferred=deferred), [(pw, tt, uu, bias), (pw, None, None, None)],
+                                  out_dtype=torch.float32, reference_rounding=mode == 1)
+    assert torch.equal(outs[0], got)
+    # a rotated activation, or mixed rotations, are not this call's business
+    assert not ops.nv_decode_applies(ops.quantize_rht(x, mode, _mask()), [pw], [r])
+    assert not ops.nv_decode_applies(px, [pw, ops.quantize(w, mode)], [r, r])
+
+
+@pytest.mark.parametrize("compute,fuse_norms", [(torch.bfloat16, False), (torch.float32, False), (torch.bfloat16, True)])
+def test_decode_step_of_a_layer_under_the_nv_recipe_stays_on_the_decode_sized_kernel(compute, fuse_norms, monkeypatch):
+    """A patched Qwen2 decoder layer under the NV recipe, 64 sequences x 1 token, no autograd: every projection runs on the
+    decode-sized kernel against its packed rotated weight (q/k/v and gate/up as grouped launches), no tiled expansion
+    and no tiled GEMM; the output agrees with the member-by-member evaluation on the tiled GEMM."""
+    pytest.importorskip("transformers")
+    from transformers.models.qwen2.modeling_qwen2 import Qwen2Config, Qwen2DecoderLayer, Qwen2RotaryEmbedding
+    from metis_hip import BitLinear, LinearLowbitFunction as F, MetisArgs, ops, replace_model_with_metis
+    torch.manual_seed(0)
+    cfg = Qwen2Config(hidden_size=256, intermediate_size=512, num_attention_heads=4, num_key_value_heads=2,
+                      num_hidden_layers=1, vocab_size=128, max_position_embeddings=256)
+    cfg._attn_implementation = "eager"
+    layer = Qwen2DecoderLayer(cfg, layer_idx=0).to(torch.bfloat16).cuda()
+    for p in layer.parameters():
+        if p.dim() == 2:
+            torch.nn.init.normal_(p, std=0.02)
+    holder = torch.nn.ModuleDict({"layer": layer})
+    args = MetisArgs.direct_fp4(forward_svd_rank=32)
+    args.enable_nv_recipe = True
+    if compute == torch.float32:
+        from metis_hip.patch import DEFAULT_TARGETS, replace_linear_with_metis
+        replace_linear_with_metis(model=holder, dtype=torch.bfloat16, metis_args=args, target_modules=list(DEFAULT_TARGETS),
+                                  compute_dtype=torch.float32)
+    else:
+        replace_model_with_metis(holder, args, fuse_norms=fuse_norms)
+    assert F.enable_nv_recipe and F._nv_on_kernels()
+    if fuse_norms:
+        from metis_hip import FusedRMSNormQuant
+        fused_calls = []
+        real_rq = ops.rmsnorm_quantize
+        monkeypatch.setattr(ops, "rmsnorm_quantize", lambda *a, **k: (fused_calls.append(1), real_rq(*a, **k))[1])
+        assert isinstance(layer.input_layernorm, FusedRMSNormQuant)
+    x = (torch.randn(64, 1, 256, device="cuda") + 0.5).bfloat16()
+    pos = torch.zeros(64, 1, dtype=torch.long, device="cuda")
+    pe = Qwen2RotaryEmbedding(cfg).cuda()(x, pos)
+
+    def run():
+        with torch.no_grad():
+            out = holder["layer"](x, position_embeddings=pe, attention_mask=None, position_ids=pos)
+        return (out[0] if isinstance(out, tuple) else out).float()
+
+    seen = {"rotated_operand": 0, "tiled": 0}
+    real_do, real_gt = ops.decode_operand, ops.gemm_tiled
+    monkeypatch.setattr(ops, "decode_operand", lambda p, mode=0, center=None, rotate=None:
+                        (seen.__setitem__("rotated_operand", seen["rotated_operand"] + (rotate is not None)), real_do(p, mode, center, rotate))[1])
+    monkeypatch.setattr(ops, "gemm_tiled", lambda *a, **k: (seen.__setitem__("tiled", seen["tiled"] + 1), real_gt(*a, **k))[1])
+    got = run()
+    assert seen == {"rotated_operand": 4, "tiled": 0}, seen          # q/k/v, o, gate/up, down
+    if fuse_norms:
+        assert len(fused_calls) == 2                                 # both norms quantize for their groups under the recipe too
+    monkeypatch.setattr(ops, "nv_decode_applies", lambda *a, **k: False)
+    seen.update(rotated_operand=0, tiled=0)
+    want = run()
+    assert seen == {"rotated_operand": 0, "tiled": 7}, seen
+    assert rel_fro(got.cpu(), want.cpu()) <= 1e-2
+
+
+def test_fused_norm_feeds_the_groups_under_the_nv_recipe_with_autograd():
+    """Training step of a patched Qwen2 layer under the NV recipe (round-to-nearest backward quantizers, so that two
+    runs can be compared): with the norms fused into the groups' quantizer the output and every gradient agree with
+    the unfused layer up to a bf16 ulp of the normed tensor here and there."""
+    pytest.importorskip("transformers")
+    from transformers.models.qwen2.modeling_qwen2 import Qwen2Config, Qwen2DecoderLayer, Qwen2RotaryEmbedding
+    from metis_hip import FusedRMSNormQuant, LinearLowbitFunction as F, MetisArgs, replace_model_with_metis
+    cfg = Qwen2Config(hidden_size=256, intermediate_size=512, num_attention_heads=4, num_key_value_heads=2,
+                      num_hidden_layers=1, vocab_size=128, max_position_embeddings=256)
+    cfg._attn_implementation = "eager"
+    results = {}
+    for fuse in (False, True):
+        torch.manual_seed(0)
+        layer = Qwen2DecoderLayer(cfg, layer_idx=0).to(torch.bfloat16).cuda()
+        for p in layer.parameters():
+            if p.dim() == 2:
+                torch.nn.init.normal_(p, std=0.02)
+        holder = torch.nn.ModuleDict({"layer": layer})
+        args = MetisArgs.direct_fp4(forward_svd_rank=32)
+        args.enable_nv_recipe = True
+        args.q_backward_input = args.q_backward_weight = args.q_backward_outputgrad = "nvfp4e2m1bnosr"
+        replace_model_with_metis(holder, args, fuse_norms=fuse)
+        assert F.enable_nv_recipe and F._nv_on_kernels() and isinstance(layer.input_layernorm, FusedRMSNormQuant) == fuse
+        g = torch.Generator().manual_seed(5)
+        x = (torch.randn(2, 160, 256, generator=g) + 0.5).bfloat16().cuda().requires_grad_(True)
+        pos = torch.arange(160, device="cuda").unsqueeze(0).expand(2, -1)
+        pe = Qwen2RotaryEmbedding(cfg).cuda()(x, pos)
+        out = holder["layer"](x, position_embeddings=pe, attention_mask=None, position_ids=pos)
+        out = out[0] if isinstance(out, tuple) else out
+        dy = (torch.randn(out.shape, generator=g) * 1e-2).bfloat16().cuda()
+        out.backward(dy)
+        results[fuse] = (out.detach().float().cpu(), x.grad.float().cpu(),
+                         layer.mlp.down_proj.warmup_linear.weight.grad.float().cpu(),
+                         layer.self_attn.q_proj.warmup_linear.weight.grad.float().cpu(),
+                         layer.input_layernorm.weight.grad.float().cpu())
+    for a, b in zip(results[True], results[False]):
+        assert rel_fro(a, b) <= 3e-2
