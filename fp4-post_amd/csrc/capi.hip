@@ -405,10 +405,11 @@ int metis_decode_quant_project_deferred(const void* x, int64_t rows, int64_t col
 
 int metis_decode_prepare_deferred(const void* x, int64_t ldx, const void* v, int64_t R, const void* s, void* xv, void* t,
                                   void* workspace, size_t workspace_bytes, const void* codes, const void* deferred, int64_t rows,
-                                  int64_t cols, int quant_mode, int mode, const void* center, float* unit, void* out, void* stream)
+                                  int64_t cols, int quant_mode, int mode, const void* center, float* unit, void* out, int rotate,
+                                  uint32_t sign_mask, void* stream)
 {
     return decode_prepare_deferred(x, ldx, v, R, s, xv, t, workspace, workspace_bytes, codes, deferred, rows, cols, quant_mode, mode,
-                                   center, unit, out, (hipStream_t)stream);
+                                   center, unit, out, (hipStream_t)stream, rotate, sign_mask);
 }
 
 int metis_linear_fwd_grouped_operand(const void* a_operand, const float* a_unit, int64_t M, int64_t K,

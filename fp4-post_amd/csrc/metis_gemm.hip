@@ -942,12 +942,52 @@ int decode_weight(const void* codes, const void* scales, int64_t N, int64_t K, v
 // DEF: the quantizer call deferred its scale bytes (nvfp4_quant.hip): `scales` holds bf16 block maxima, `partials` the
 // partial tensor maxima; unit (written to unit_out) and E4M3 bytes are formed here, in the arithmetic of that call (QMODE).
 // (block `block` of `nblocks`: a launch may give its first blocks to other work)
-template <int PB16, int DEF, int QMODE>
+// The eight values of one piece of the rotated operand: the block's two code words c, its scale byte sb, the tensor
+// unit (bf16 arithmetic), half = which eight of the block's sixteen outputs, sign_mask = the rotation's signs.
+template <int PB16>
+__device__ __forceinline__ uint4 rotated_operand_piece(const uint2 c, const uint32_t sb, const float unit, const int half, const uint32_t sign_mask)
+{
+    typedef float float2_t __attribute__((ext_vector_type(2)));
+    const float dq = PB16 ? rb(e4m3_value(sb) * unit) : e4m3_value(sb) * 0.00390625f;
+    const float2_t p[8] = {__builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 0), __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 1),
+                           __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 2), __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 3),
+                           __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 0), __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 1),
+                           __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 2), __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 3)};
+    float blk[kBlock];
+#pragma unroll
+    for (int n = 0; n < kBlock; ++n) {
+        const float x = PB16 ? rb(p[n >> 1][n & 1] * dq) : p[n >> 1][n & 1] * dq;
+        // sign[n] of the rotation; inputs 8..15 change sign for the outputs 8..15 (H[n][8 + j] = -H[n][j] there)
+        const uint32_t flip = (((sign_mask >> n) & 1u) ^ (n >= 8 ? (uint32_t)half : 0u)) << 31;
+        blk[n] = __uint_as_float(__float_as_uint(x) ^ flip);
+    }
+    float o[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        float acc = blk[0];
+#pragma unroll
+        for (int n = 1; n < kBlock; ++n) acc = (__builtin_popcount(n & j) & 1) ? acc - blk[n] : acc + blk[n];
+        o[j] = acc * 0.0625f;
+    }
+    uint4 v;
+    if constexpr (PB16 != 0) {
+        v.x = rb_pair(o[0], o[1]); v.y = rb_pair(o[2], o[3]); v.z = rb_pair(o[4], o[5]); v.w = rb_pair(o[6], o[7]);
+    } else {
+        const half2_t h0 = {(_Float16)o[0], (_Float16)o[1]}, h1 = {(_Float16)o[2], (_Float16)o[3]};
+        const half2_t h2 = {(_Float16)o[4], (_Float16)o[5]}, h3 = {(_Float16)o[6], (_Float16)o[7]};
+        v.x = __builtin_bit_cast(uint32_t, h0); v.y = __builtin_bit_cast(uint32_t, h1);
+        v.z = __builtin_bit_cast(uint32_t, h2); v.w = __builtin_bit_cast(uint32_t, h3);
+    }
+    return v;
+}
+
+// RHT (sign_mask): the call multiplies with a weight packed in the rotated domain; see skinny_operand_rht_kernel.
+template <int PB16, int DEF, int QMODE, int RHT = 0>
 __device__ __forceinline__ void skinny_operand_block(int block, int nblocks, const uint32_t* __restrict__ codes,
                                                      const uint8_t* __restrict__ scales, const float* __restrict__ unit_p,
                                                      const uint16_t* __restrict__ center, int M, int K, int tiles,
                                                      uint4* __restrict__ out, const uint32_t* __restrict__ partials,
-                                                     float* __restrict__ unit_out)
+                                                     float* __restrict__ unit_out, uint32_t sign_mask = 0u)
 {
     typedef float float2_t __attribute__((ext_vector_type(2)));
     const int iters = K / 256;
@@ -967,10 +1007,16 @@ __device__ __forceinline__ void skinny_operand_block(int block, int nblocks, con
         const int row = tile * 32 + (lane & 31), k0 = it * 256 + (lane >> 5) * 128 + 8 * m;
         uint4 v = make_uint4(0u, 0u, 0u, 0u);
         if (row < M) {
-            const uint32_t c = codes[(int64_t)row * (K / 8) + (k0 >> 3)];
             uint32_t sb;
             if constexpr (DEF != 0) sb = scale_byte_of<QMODE>(maxima[(int64_t)row * (K / 16) + (k0 >> 4)], unit);
             else sb = scales[(int64_t)row * (K / 16) + (k0 >> 4)];
+            if constexpr (RHT != 0) {
+                v = rotated_operand_piece<PB16>(reinterpret_cast<const uint2*>(codes)[(int64_t)row * (K / 16) + (k0 >> 4)], sb, unit, m & 1,
+                                                sign_mask);
+                out[idx] = v;
+                continue;
+            }
+            const uint32_t c = codes[(int64_t)row * (K / 8) + (k0 >> 3)];
             if constexpr (PB16 != 0) {
                 const float dq = rb(e4m3_value(sb) * unit);
                 const float2_t p[4] = {__builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c, 1.0f, 0), __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c, 1.0f, 1),
@@ -1018,80 +1064,28 @@ __global__ __launch_bounds__(256) void skinny_operand_rht_kernel(const uint2* __
                                                                  uint4* __restrict__ out, const uint32_t* __restrict__ partials,
                                                                  float* __restrict__ unit_out, uint32_t sign_mask)
 {
-    typedef float float2_t __attribute__((ext_vector_type(2)));
-    const int iters = K / 256;
-    const int64_t total = (int64_t)tiles * iters * 1024;
-    float unit = 0.0f;
-    if constexpr (DEF != 0) {
-        unit = tensor_unit_of<QMODE>(fold_partial_maxima(partials));
-        if (blockIdx.x == 0 && threadIdx.x == 0) *unit_out = unit;
-    } else if constexpr (PB16 != 0) {
-        unit = *unit_p;
-    }
-    const uint16_t* __restrict__ maxima = reinterpret_cast<const uint16_t*>(scales);
-    for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
-        const int lane = (int)(idx & 63), m = (int)((idx >> 6) & 15);
-        const int64_t ti = idx >> 10;
-        const int it = (int)(ti % iters), tile = (int)(ti / iters);
-        const int row = tile * 32 + (lane & 31), k0 = it * 256 + (lane >> 5) * 128 + 8 * m;
-        uint4 v = make_uint4(0u, 0u, 0u, 0u);
-        if (row < M) {
-            const int half = m & 1;                              // which eight of the block's sixteen outputs are this thread's
-            const uint2 c = codes[(int64_t)row * (K / 16) + (k0 >> 4)];
-            uint32_t sb;
-            if constexpr (DEF != 0) sb = scale_byte_of<QMODE>(maxima[(int64_t)row * (K / 16) + (k0 >> 4)], unit);
-            else sb = scales[(int64_t)row * (K / 16) + (k0 >> 4)];
-            const float dq = PB16 ? rb(e4m3_value(sb) * unit) : e4m3_value(sb) * 0.00390625f;
-            const float2_t p[8] = {__builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 0), __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 1),
-                                   __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 2), __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.x, 1.0f, 3),
-                                   __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 0), __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 1),
-                                   __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 2), __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c.y, 1.0f, 3)};
-            float blk[kBlock];
-#pragma unroll
-            for (int n = 0; n < kBlock; ++n) {
-                const float x = PB16 ? rb(p[n >> 1][n & 1] * dq) : p[n >> 1][n & 1] * dq;
-                // sign[n] of the rotation; inputs 8..15 change sign for the outputs 8..15 (H[n][8 + j] = -H[n][j] there)
-                const uint32_t flip = (((sign_mask >> n) & 1u) ^ (n >= 8 ? (uint32_t)half : 0u)) << 31;
-                blk[n] = __uint_as_float(__float_as_uint(x) ^ flip);
-            }
-            float o[8];
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                float acc = blk[0];
-#pragma unroll
-                for (int n = 1; n < kBlock; ++n) acc = (__builtin_popcount(n & j) & 1) ? acc - blk[n] : acc + blk[n];
-                o[j] = acc * 0.0625f;
-            }
-            if constexpr (PB16 != 0) {
-                v.x = rb_pair(o[0], o[1]); v.y = rb_pair(o[2], o[3]); v.z = rb_pair(o[4], o[5]); v.w = rb_pair(o[6], o[7]);
-            } else {
-                const half2_t h0 = {(_Float16)o[0], (_Float16)o[1]}, h1 = {(_Float16)o[2], (_Float16)o[3]};
-                const half2_t h2 = {(_Float16)o[4], (_Float16)o[5]}, h3 = {(_Float16)o[6], (_Float16)o[7]};
-                v.x = __builtin_bit_cast(uint32_t, h0); v.y = __builtin_bit_cast(uint32_t, h1);
-                v.z = __builtin_bit_cast(uint32_t, h2); v.w = __builtin_bit_cast(uint32_t, h3);
-            }
-        }
-        out[idx] = v;
-    }
+    skinny_operand_block<PB16, DEF, QMODE, 1>((int)blockIdx.x, (int)gridDim.x, reinterpret_cast<const uint32_t*>(codes), scales, unit_p,
+                                              nullptr, M, K, tiles, out, partials, unit_out, sign_mask);
 }
 
 // One launch for the two small independent steps between a decode-sized layer's quantizer and its GEMM: the first
 // `finish_blocks` blocks finish the rank-r projection (lowrank_small_steps.h), the others build the activation's
 // operands from a tensor whose quantizer call deferred its scale bytes.
-template <int PB16, int QMODE>
+template <int PB16, int QMODE, int RHT = 0>
 __global__ __launch_bounds__(256) void decode_prepare_kernel(int finish_blocks, const float* __restrict__ lr_ws, int chunks, int MR, int R,
                                                              const uint16_t* __restrict__ s, uint16_t* __restrict__ xv,
                                                              uint16_t* __restrict__ t, const uint32_t* __restrict__ codes,
                                                              const uint8_t* __restrict__ maxima, const uint16_t* __restrict__ center,
                                                              int M, int K, int tiles, uint4* __restrict__ out,
-                                                             const uint32_t* __restrict__ partials, float* __restrict__ unit_out)
+                                                             const uint32_t* __restrict__ partials, float* __restrict__ unit_out,
+                                                             uint32_t sign_mask)
 {
     if ((int)blockIdx.x < finish_blocks) {
         lowrank_small_finish_block((int)blockIdx.x, lr_ws, chunks, MR, R, s, xv, t);
         return;
     }
-    skinny_operand_block<PB16, 1, QMODE>((int)blockIdx.x - finish_blocks, (int)gridDim.x - finish_blocks, codes, maxima, nullptr, center,
-                                         M, K, tiles, out, partials, unit_out);
+    skinny_operand_block<PB16, 1, QMODE, RHT>((int)blockIdx.x - finish_blocks, (int)gridDim.x - finish_blocks, codes, maxima, nullptr, center,
+                                              M, K, tiles, out, partials, unit_out, sign_mask);
 }
 
 size_t skinny_operand_bytes(int64_t M, int64_t K)
@@ -1183,9 +1177,10 @@ int skinny_operand_rht(const void* codes, const void* scales, float* unit, const
 // x = nullptr: the first of the two already ran beside the quantizer (quantize_row_deferred_partial): one launch.
 int decode_prepare_deferred(const void* x, int64_t ldx, const void* v, int64_t R, const void* s, void* xv, void* t, void* workspace,
                             size_t workspace_bytes, const void* codes, const void* deferred, int64_t M, int64_t K, int qmode, int mode,
-                            const void* center, float* unit_out, void* out, hipStream_t st)
+                            const void* center, float* unit_out, void* out, hipStream_t st, int rotate, uint32_t sign_mask)
 {
     if (mode == METIS_MODE_P32_F32) mode = METIS_MODE_P32;
+    if (rotate && (center || sign_mask > 0xffffu || ((uintptr_t)codes % 8))) return METIS_E_ARG;   // a rotated operand: uncentred, whole blocks per load
     if ((mode != METIS_MODE_P32 && mode != METIS_MODE_PB16) || (qmode != METIS_MODE_P32 && qmode != METIS_MODE_PB16)) return METIS_E_ARG;
     if (M <= 0 || M >= 256 || K <= 0 || K % 256 || K > INT32_MAX) return METIS_E_SHAPE;
     if (!codes || !unit_out || !out || ((uintptr_t)codes % 4) || ((uintptr_t)out % 16) || ((uintptr_t)center % 16)) return METIS_E_ARG;
@@ -1207,12 +1202,14 @@ int decode_prepare_deferred(const void* x, int64_t ldx, const void* v, int64_t R
     const int tiles = (int)((M + 63) / 64) * 2;
     const int64_t total = (int64_t)tiles * (K / 256) * 1024;
     const int g = fb + (int)((total + 255) / 256);
-#define METIS_DP(P, Q) hipLaunchKernelGGL((decode_prepare_kernel<P, Q>), dim3(g), dim3(256), 0, st, fb, (const float*)workspace, chunks, \
-                                          (int)(M * R), (int)R, (const uint16_t*)s, (uint16_t*)xv, (uint16_t*)t, (const uint32_t*)codes, \
-                                          (const uint8_t*)ws.amax, (const uint16_t*)center, (int)M, (int)K, tiles, (uint4*)out, \
-                                          (const uint32_t*)ws.gmax, unit_out)
-    if (mode == METIS_MODE_PB16) { if (qmode) METIS_DP(1, 1); else METIS_DP(1, 0); }
-    else { if (qmode) METIS_DP(0, 1); else METIS_DP(0, 0); }
+#define METIS_DP(P, Q, H) hipLaunchKernelGGL((decode_prepare_kernel<P, Q, H>), dim3(g), dim3(256), 0, st, fb, (const float*)workspace, chunks, \
+                                             (int)(M * R), (int)R, (const uint16_t*)s, (uint16_t*)xv, (uint16_t*)t, (const uint32_t*)codes, \
+                                             (const uint8_t*)ws.amax, (const uint16_t*)center, (int)M, (int)K, tiles, (uint4*)out, \
+                                             (const uint32_t*)ws.gmax, unit_out, sign_mask)
+#define METIS_DPH(P, Q) do { if (rotate) METIS_DP(P, Q, 1); else METIS_DP(P, Q, 0); } while (0)
+    if (mode == METIS_MODE_PB16) { if (qmode) METIS_DPH(1, 1); else METIS_DPH(1, 0); }
+    else { if (qmode) METIS_DPH(0, 1); else METIS_DPH(0, 0); }
+#undef METIS_DPH
 #undef METIS_DP
     return hipGetLastError() == hipSuccess ? METIS_OK : METIS_E_LAUNCH;
 }

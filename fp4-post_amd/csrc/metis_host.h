@@ -147,7 +147,7 @@ int quantize_row_deferred_partial(const void* x, int64_t rows, int64_t cols, int
 // projection's finishing step inside the operand launch
 int decode_prepare_deferred(const void* x, int64_t ldx, const void* v, int64_t R, const void* s, void* xv, void* t, void* workspace,
                             size_t workspace_bytes, const void* codes, const void* deferred, int64_t M, int64_t K, int qmode, int mode,
-                            const void* center, float* unit_out, void* out, hipStream_t st);
+                            const void* center, float* unit_out, void* out, hipStream_t st, int rotate = 0, uint32_t sign_mask = 0);
 int gemm_grouped_center_supported(int64_t M, int64_t K, const GemmMember* members, int count, int have_workspace);
 // bytes of split-K scratch a grouped call can use (only the N fields of the members are read; 0: it would not split)
 size_t gemm_grouped_workspace_bytes(int64_t M, int64_t K, const GemmMember* members, int count);

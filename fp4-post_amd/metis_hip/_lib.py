@@ -98,7 +98,8 @@ SIGNATURES = {
     "metis_nvfp4_decode_operand_deferred": (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _vp, _vp, _vp, _vp]),
     "metis_nvfp4_decode_operand_rht": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, ctypes.c_uint32, _vp, _vp]),
     "metis_decode_quant_project_deferred": (_i32, [_vp, _i64, _i64, _i32, _vp, _vp, _sz, _vp, _i64, _vp, _sz, _vp]),
-    "metis_decode_prepare_deferred": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _i64, _i64, _i32, _i32, _vp, _vp, _vp, _vp]),
+    "metis_decode_prepare_deferred": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _i64, _i64, _i32, _i32, _vp, _vp, _vp, _i32,
+                                             ctypes.c_uint32, _vp]),
     "metis_linear_fwd_grouped_operand": (_i32, [_vp, _vp, _i64, _i64, _vp, _i32, _i32, _i32, _vp, _sz, _vp]),
     "metis_linear_grouped_workspace_bytes": (_sz, [_i64, _i64, _vp, _i32]),
     "metis_linear_fwd_grouped_centered": (_i32, [_vp, _vp, _vp, _i64, _i64, _vp, _i32, _i32, _vp, _vp, _sz, _vp]),

@@ -23,6 +23,7 @@ from __future__ import annotations
 
 import math
 import weakref
+from types import SimpleNamespace
 
 import torch
 import torch.nn as nn
@@ -748,14 +749,22 @@ class _MetisFusedFunction(torch.autograd.Function):
         aop = None
         if pending is not None:
             # the quantizer's launch left the projection's partial sums (BitLinear._quantize_and_project)
-            xv, t, aop = ops.project_and_operand(_flat2d(x).to(cd), v.to(cd), s.to(cd), px, ops.MODE_PB16, None, pending=pending)
+            if p_res.rht is not None:
+                xv, t, aop = ops.project_and_operand(_flat2d(x).to(cd), v.to(cd), s.to(cd), px,
+                                                     ops.nv_operand_mode(px, [p_res], F.reference_rounding), pending=pending, rotate=p_res.rht)
+            else:
+                xv, t, aop = ops.project_and_operand(_flat2d(x).to(cd), v.to(cd), s.to(cd), px, ops.MODE_PB16, None, pending=pending)
         elif xv is None:
             # [L, r] rank-r projection and its product with s (bf16) on the library's kernels (split-K below 256 rows,
             # one pass over x from there on); the caller has it already when the quantizer's pass produced it
             x2, vb, sb = _flat2d(x).to(cd), v.to(cd), s.to(cd)
             in_operand = isinstance(px, CenteredNVFP4) and F._mean_in_operand(px, p_res)
             target = px.residual if in_operand else px
-            if ((in_operand or (isinstance(px, PackedNVFP4) and F.reference_rounding)) and p_res.rht is None
+            if (isinstance(px, PackedNVFP4) and p_res.rht is not None and ops.nv_decode_applies(px, [p_res], [vb.shape[0]])
+                    and ops.project_and_operand_applies(x2, vb, sb, px)):
+                # NV recipe at decode size: the same merged launch, the operand rotated for the weight's domain
+                xv, t, aop = ops.project_and_operand(x2, vb, sb, px, ops.nv_operand_mode(px, [p_res], F.reference_rounding), rotate=p_res.rht)
+            elif ((in_operand or (isinstance(px, PackedNVFP4) and F.reference_rounding)) and p_res.rht is None
                     and ops.grouped_operand_applies(target, [p_res], [vb.shape[0]], px.mean if in_operand else None, True)
                     and ops.project_and_operand_applies(x2, vb, sb, target)):
                 # decode-sized call in bf16 arithmetic: the projection's finishing step and the activation's GEMM
@@ -1039,7 +1048,7 @@ class BitLinear(nn.Module):
         residual branch through the quantizer and the rank-r branch as it is.  A decode-sized activation in bf16
         arithmetic gives (packed activation, None, None, pending partial sums of the projection)."""
         F = LinearLowbitFunction
-        if (F.enable_activation_svd or F.enable_nv_recipe or F.q_forward_input is not Cast2NVFp4e2m1BlockNOSR
+        if (F.enable_activation_svd or (F.enable_nv_recipe and not F._nv_on_kernels()) or F.q_forward_input is not Cast2NVFp4e2m1BlockNOSR
                 or not x.is_cuda or x.dtype != torch.bfloat16 or F.compute_dtype not in (torch.float32, torch.bfloat16)):
             return None
         x2 = _flat2d(x)
@@ -1047,20 +1056,20 @@ class BitLinear(nn.Module):
         if v.dtype != torch.bfloat16 or self._packed_residual() is None:
             return None
         mode = ops.MODE_P32 if F.compute_dtype == torch.float32 else ops.MODE_PB16
-        if ops.quantize_project_applies(x2, v, mode):
+        if not F.enable_nv_recipe and ops.quantize_project_applies(x2, v, mode):
             return ops.quantize_project(x2, v.detach(), self.s.detach(), mode)
-        # decode-sized call in bf16 arithmetic: the quantizer's launch carries the projection's first step, and the launch
-        # that builds the GEMM's activation operands its finishing step
+        # decode-sized call: the quantizer's launch carries the projection's first step, and the launch that builds the
+        # GEMM's activation operands its finishing step (bf16 arithmetic; under the NV recipe either arithmetic, the
+        # operand rotated for the weight's domain)
         p_res = self._packed_residual()
-        if (mode == ops.MODE_PB16 and F.reference_rounding and p_res.rht is None
-                and self.s.dtype == torch.bfloat16 and ops.quantize_project_decode_applies(x2, v, mode)
-                and x2.shape[0] * x2.shape[1] > 0):
-            px, pending = ops.quantize_project_decode(x2, v.detach(), mode)
-            if ops.grouped_operand_applies(px, [p_res], [v.shape[0]], None, True):
+        if (self.s.dtype == torch.bfloat16 and ops.quantize_project_decode_applies(x2, v, mode) and x2.shape[0] * x2.shape[1] > 0
+                and (p_res.rht is not None or (mode == ops.MODE_PB16 and F.reference_rounding))):
+            probe = SimpleNamespace(rows=x2.shape[0], cols=x2.shape[1], mode=mode, rht=None)   # what the packed activation will be
+            takes = (ops.nv_decode_applies(probe, [p_res], [v.shape[0]]) if p_res.rht is not None
+                     else ops.grouped_operand_applies(probe, [p_res], [v.shape[0]], None, True))
+            if takes:
+                px, pending = ops.quantize_project_decode(x2, v.detach(), mode)
                 return px, None, None, pending
-            # (a weight the decode-sized kernel does not take: finish the projection on its own)
-            xv, t, _ = ops.project_and_operand(x2, v.detach(), self.s.detach(), px, mode, None, pending=pending)
-            return px, xv, t
         return None
 
     def _forward_group(self, x: torch.Tensor, shared_input):
@@ -1093,7 +1102,11 @@ class BitLinear(nn.Module):
         if rotated and (centre is not None or not ops.nv_decode_applies(px, packed, [m.args.forward_svd_rank for m in members])):
             return None                                            # member by member on the tiled GEMM
         aop = None
-        if (ops.grouped_operand_applies(px, packed, [m.args.forward_svd_rank for m in members], centre, F.reference_rounding)
+        if rotated and ops.project_and_operand_applies(x2, cached[1], cached[2], px):
+            # (the same launch with the operand rotated for the weights' domain)
+            _, t_all, aop = ops.project_and_operand(x2, cached[1], cached[2], px, ops.nv_operand_mode(px, packed, F.reference_rounding),
+                                                    rotate=packed[0].rht)
+        elif (ops.grouped_operand_applies(px, packed, [m.args.forward_svd_rank for m in members], centre, F.reference_rounding)
                 and ops.project_and_operand_applies(x2, cached[1], cached[2], px)):
             # the projection's finishing step and the activation's GEMM operands in one launch
             _, t_all, aop = ops.project_and_operand(x2, cached[1], cached[2], px, ops.MODE_PB16, centre)

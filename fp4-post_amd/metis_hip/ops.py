@@ -682,11 +682,13 @@ def project_and_operand_applies(x2: torch.Tensor, v: torch.Tensor, s: torch.Tens
 
 
 def project_and_operand(x2: torch.Tensor, v: torch.Tensor, s: torch.Tensor, p: PackedNVFP4, mode: int = MODE_PB16,
-                        center: torch.Tensor | None = None, pending: torch.Tensor | None = None):
+                        center: torch.Tensor | None = None, pending: torch.Tensor | None = None, rotate: int | None = None):
     """(xv, t, operand) = lowrank_project(x2, v, s) and decode_operand(p, mode, center) of one decode-sized activation
     in two launches instead of three: the projection's finishing step rides in the operand launch.  Same bits.
     pending: the projection's partial sums as quantize_project_decode left them (the first of the two launches already
-    ran beside the quantizer): one launch."""
+    ran beside the quantizer): one launch.  rotate (sign mask): the operand of decode_operand(p, mode, rotate=...)."""
+    if rotate is not None and center is not None:
+        raise ValueError("a rotated operand takes no centre")
     if not project_and_operand_applies(x2, v, s, p):
         raise ValueError("project_and_operand: outside the call's domain (see project_and_operand_applies)")
     M, K = x2.shape
@@ -711,7 +713,7 @@ def project_and_operand(x2: torch.Tensor, v: torch.Tensor, s: torch.Tensor, p: P
                                          xv.data_ptr(), t.data_ptr(),
                                          ws.data_ptr(), need, p.codes.data_ptr(), d["deferred"].data_ptr(), M, K, p.mode, mode,
                                          None if center is None else center.data_ptr(), d["_unit"].data_ptr(), out.data_ptr(),
-                                         _stream())
+                                         int(rotate is not None), int(rotate or 0), _stream())
     check(rc, "metis_decode_prepare_deferred", (M, K, R))
     d["_unit_ready"] = True
     return xv, t, out
@@ -944,6 +946,12 @@ def nv_decode_applies(a: PackedNVFP4, weights, ranks) -> bool:
                 and all(b.scales.data_ptr() % 8 == 0 for b in weights))
 
 
+def nv_operand_mode(a: PackedNVFP4, weights, reference_rounding: bool) -> int:
+    """The format of the rotated operand of a decode-sized NV-recipe call: the reference's bf16 values when the call
+    follows its all-bf16 evaluation (every tensor packed in bf16 arithmetic), exact binary16 otherwise."""
+    return MODE_PB16 if (reference_rounding and a.mode == MODE_PB16 and all(b.mode == MODE_PB16 for b in weights)) else MODE_P32
+
+
 def _decode_kernel_takes(M: int, N: int, K: int, r: int) -> bool:
     """Shapes of the decode-sized kernel (waves split K over packed operands streamed from global memory)."""
     return 0 < M < 256 and K % 64 == 0 and N % 4 == 0 and r % 32 == 0
@@ -974,7 +982,7 @@ def linear_fwd(a: PackedNVFP4, b: PackedNVFP4, *, t: torch.Tensor | None = None,
             and nv_decode_applies(a, [b], [0 if t is None else t.shape[1]])):
         # NV recipe at decode size: the packed rotated weight is streamed as it is, the activation's operand is rotated
         return _linear_fwd_grouped(a, [(b, t, u, bias)], out_dtype=out_dtype, split_k=split_k,
-                                   reference_rounding=reference_rounding)[0]
+                                   reference_rounding=reference_rounding, a_operand=a_operand)[0]
     if a.rht is not None or b.rht is not None:
         # NV recipe: only the tiled operands know how to rotate a block back
         if a.cols % 32:
@@ -1265,8 +1273,8 @@ def _linear_fwd_grouped(a: PackedNVFP4, members, out_dtype: torch.dtype = torch.
     ws = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
     dt = DTYPE_F32 if out_dtype == torch.float32 else DTYPE_BF16
     if rotate is not None:
-        op_mode = MODE_PB16 if rounded else MODE_P32
-        aop = decode_operand(a, op_mode, None, rotate=rotate)
+        op_mode = MODE_PB16 if rounded else MODE_P32          # (nv_operand_mode: what a caller that brings a_operand built it in)
+        aop = a_operand if a_operand is not None else decode_operand(a, op_mode, None, rotate=rotate)
         rc = L.metis_linear_fwd_grouped_operand(aop.data_ptr(), a.unit.data_ptr(), M, K, ap, len(members), dt, op_mode,
                                                 None if ws is None else ws.data_ptr(), need, _stream())
         check(rc, "metis_linear_fwd_grouped_operand", (M, K, [m[0].rows for m in members]))

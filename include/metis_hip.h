@@ -655,7 +655,8 @@ int metis_linear_fwd_grouped_bf16(const void *a_codes, const void *a_scales, con
  *                                (`vlinear(x)`, `torch.mul(self.s, y)` and the quantized input of BitLinear.forward,
  *                                src/Metis/Metis/bitlinear.py:752-760).  x = NULL: the workspace already holds the
  *                                projection's partial sums, left there by metis_decode_quant_project_deferred on the
- *                                same rows, cols and R (R <= 128 then): one launch
+ *                                same rows, cols and R (R <= 128 then): one launch.  rotate != 0: the operand half is
+ *                                metis_nvfp4_decode_operand_rht with sign_mask (no centre then; codes 8-byte aligned)
  *   metis_nvfp4_decode_operand_rht  the operand for a call against a weight packed in the ROTATED domain (NV recipe:
  *                                metis_nvfp4_quant_row_rht with sign_mask; the forward multiplies with
  *                                rotate_back(QDQ(rotate(W))), src/Metis/Metis/bitlinear.py:577-585, 395-405).  The
@@ -688,7 +689,8 @@ int metis_decode_quant_project_deferred(const void *x, int64_t rows, int64_t col
 int metis_decode_prepare_deferred(const void *x, int64_t ldx, const void *v, int64_t R, const void *s, void *xv,
                                   void *t, void *workspace, size_t workspace_bytes, const void *codes,
                                   const void *deferred, int64_t rows, int64_t cols, int quant_mode, int mode,
-                                  const void *center, float *unit, void *out, void *stream);
+                                  const void *center, float *unit, void *out, int rotate, uint32_t sign_mask,
+                                  void *stream);
 int metis_linear_fwd_grouped_operand(const void *a_operand, const float *a_unit, int64_t M, int64_t K,
                                      const metis_linear_member *members, int count, int out_dtype, int mode,
                                      void *workspace, size_t workspace_bytes, void *stream);

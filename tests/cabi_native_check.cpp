@@ -335,7 +335,7 @@ static void check_decode_three_launches(int64_t M, int64_t N, int64_t K, int64_t
                                                  lr_ws.p, lws, st);
     if (rc == METIS_OK)
         rc = metis_decode_prepare_deferred(nullptr, K, dv.p, R, ds.p, xv.p, t.p, lr_ws.p, lws, codes.p, parked_p, M, K, METIS_MODE_PB16,
-                                           METIS_MODE_PB16, nullptr, unit.p, aop.p, st);
+                                           METIS_MODE_PB16, nullptr, unit.p, aop.p, 0, 0u, st);
     metis_linear_member mem = {};
     mem.b_codes = bc.p; mem.b_scales = bs.p; mem.b_unit = bu.p; mem.N = N; mem.t = t.p; mem.u = du.p; mem.r = (int)R;
     const size_t need = metis_linear_grouped_workspace_bytes(M, K, &mem, 1);

@@ -902,9 +902,10 @@ def test_decode_prepare_rejects_what_its_two_halves_reject():
     ws = torch.empty(need, dtype=torch.uint8, device="cuda")
     unit = torch.zeros(1, device="cuda")
 
-    def call(rows=M, cols=K, r=R, wsb=need, mode=1, centre=None, xp=x.data_ptr(), up=unit.data_ptr()):
+    def call(rows=M, cols=K, r=R, wsb=need, mode=1, centre=None, xp=x.data_ptr(), up=unit.data_ptr(), rotate=0):
         return L.metis_decode_prepare_deferred(xp, cols, v.data_ptr(), r, s.data_ptr(), xv.data_ptr(), t.data_ptr(), ws.data_ptr(), wsb,
-                                               p.codes.data_ptr(), p.deferred.data_ptr(), rows, cols, 1, mode, centre, up, out.data_ptr(), None)
+                                               p.codes.data_ptr(), p.deferred.data_ptr(), rows, cols, 1, mode, centre, up, out.data_ptr(),
+                                               rotate, 0x5a3c, None)
     assert call() == 0
     assert call(rows=256) != 0 and call(rows=0) != 0          # decode-sized only
     assert call(cols=320) != 0                                # wide runs: K % 256 == 0
@@ -915,6 +916,9 @@ def test_decode_prepare_rejects_what_its_two_halves_reject():
     assert call(up=None) != 0
     assert call(xp=None) == 0                                 # x = NULL: the partial sums are taken from the workspace
     assert call(xp=None, r=160) != 0                          # ... which the quantizer's launch fills for R <= 128 only
+    assert call(rotate=1) == 0                                # the operand rotated for a weight packed in the rotated domain
+    centre16 = torch.zeros(K, dtype=torch.bfloat16, device="cuda")
+    assert call(rotate=1, centre=centre16.data_ptr()) != 0    # ... which takes no centre
     torch.cuda.synchronize()
 
 

@@ -366,6 +366,10 @@ def test_decode_step_of_a_layer_under_the_nv_recipe_stays_on_the_decode_sized_ke
     monkeypatch.setattr(ops, "decode_operand", lambda p, mode=0, center=None, rotate=None:
                         (seen.__setitem__("rotated_operand", seen["rotated_operand"] + (rotate is not None)), real_do(p, mode, center, rotate))[1])
     monkeypatch.setattr(ops, "gemm_tiled", lambda *a, **k: (seen.__setitem__("tiled", seen["tiled"] + 1), real_gt(*a, **k))[1])
+    # (the rotated operand usually comes from the launch that also finishes the rank-r projection)
+    real_pao = ops.project_and_operand
+    monkeypatch.setattr(ops, "project_and_operand", lambda *a, **k:
+                        (seen.__setitem__("rotated_operand", seen["rotated_operand"] + (k.get("rotate") is not None)), real_pao(*a, **k))[1])
     got = run()
     assert seen == {"rotated_operand": 4, "tiled": 0}, seen          # q/k/v, o, gate/up, down
     if fuse_norms:
@@ -414,3 +418,28 @@ def test_fused_norm_feeds_the_groups_under_the_nv_recipe_with_autograd():
                          layer.input_layernorm.weight.grad.float().cpu())
     for a, b in zip(results[True], results[False]):
         assert rel_fro(a, b) <= 3e-2
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("M,K,R", [(64, 3584, 192), (1, 256, 32), (200, 2048, 64)])
+def test_merged_prepare_launch_builds_the_rotated_operand_too(mode, M, K, R):
+    """metis_decode_prepare_deferred with rotate: the projection's finishing step and the rotated operand in one launch
+    equal metis_lowrank_project and metis_nvfp4_decode_operand_rht bit for bit, also after the quantizer's launch has
+    carried the projection's first step."""
+    from metis_hip import ops
+    g = torch.Generator().manual_seed(M + K + R)
+    x = (torch.randn(M, K, generator=g) * 2).bfloat16().cuda()
+    v = (torch.randn(R, K, generator=g) * 0.05).bfloat16().cuda()
+    s = torch.rand(R, generator=g).bfloat16().cuda()
+    want_xv, want_t = ops.lowrank_project(x, v, s)
+    p1 = ops.quantize(x, mode, deferred=True)
+    want_op = ops.decode_operand(p1, mode, rotate=_mask())
+    plain_op = ops.decode_operand(ops.quantize(x, mode, deferred=True), mode)
+    assert not torch.equal(want_op, plain_op)
+    p2 = ops.quantize(x, mode, deferred=True)
+    xv, t, op = ops.project_and_operand(x, v, s, p2, mode, rotate=_mask())
+    assert torch.equal(xv, want_xv) and torch.equal(t, want_t) and torch.equal(op, want_op) and torch.equal(p2.unit, p1.unit)
+    if R <= 128:
+        p3, pending = ops.quantize_project_decode(x, v, mode)
+        xv3, t3, op3 = ops.project_and_operand(x, v, s, p3, mode, pending=pending, rotate=_mask())
+        assert torch.equal(xv3, want_xv) and torch.equal(t3, want_t) and torch.equal(op3, want_op)
