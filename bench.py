@@ -782,6 +782,26 @@ def main():
                          "decode_us_graph_replay": None if dl_graph_us is None else round(dl_graph_us, 1),
                          "decode_packed_weight_GBps": None if dl_graph_us is None else round(dec_bytes / dl_graph_us / 1e3, 1)}
             del holder, lyr
+            # the same decode step under the NV recipe (weights packed in the rotated domain; the activation's operand
+            # carries the rotation, so the decode-sized kernel still streams the packed weights)
+            try:
+                from metis_hip import LinearLowbitFunction as F_
+                lyr = Qwen2DecoderLayer(cfg, layer_idx=0).to(torch.bfloat16)
+                gl = torch.Generator().manual_seed(1005)
+                with torch.no_grad():
+                    for name_, p_ in lyr.named_parameters():
+                        if p_.dim() == 2 or name_.endswith("bias"):
+                            p_.copy_((torch.randn(p_.shape, generator=gl) * 0.02).to(p_.dtype))
+                holder = torch.nn.ModuleDict({"layer": lyr.to(dev)})
+                nv_args = MetisArgs.direct_fp4(forward_svd_rank=64)
+                nv_args.enable_nv_recipe = True
+                replace_model_with_metis(holder, nv_args, fuse_norms=True)
+                layer_leg["decode_us_graph_replay_nv_recipe"] = round(replay_us(decode_layer), 1)
+                del holder, lyr
+            except Exception as exc_:
+                layer_leg["decode_us_graph_replay_nv_recipe"] = f"{type(exc_).__name__}: {exc_}"[:200]
+            finally:
+                F_.enable_nv_recipe = False
         except Exception as exc:  # an optional leg must not cost the headline line
             layer_leg = {"workload": "config 5 decoder layer", "error": f"{type(exc).__name__}: {exc}"[:300]}
 
